@@ -1,0 +1,165 @@
+"""Independent fp64 PyTorch-CPU formulations used to pin the oracle.
+
+`per_sample_*`  : textbook recursive evaluation of each sample on its own -- no
+                  scheduler, no batching, no message pool.  This is what a
+                  correct batched execution must equal (row-id pairing, serial
+                  scheduling, or any batch whose roots come last in their round).
+`round_based`   : executes the rounds of a scheduler trace with torch index ops
+                  using the reference's pairing (b-th list entry <-> b-th slab
+                  row) and lets autograd derive the backward, which pins the
+                  oracle's hand-written backward as the transpose of its forward.
+"""
+import numpy as np
+import torch
+
+D = torch.float64
+
+
+def _adj(graph):
+    parents, off = [], 0
+    for row in graph:
+        n = int(np.argmax(row == -1)) + 1
+        parents += [off + int(p) if p >= 0 else -1 for p in row[:n]]
+        off += n
+    children = [[] for _ in parents]
+    for v, p in enumerate(parents):
+        if p >= 0:
+            children[p].append(v)
+    return parents, children
+
+
+def tparams(params):
+    return {k: torch.tensor(np.asarray(v), dtype=D, requires_grad=True) for k, v in params.items()}
+
+
+def _head(GO, P, labels, loss, parents):
+    if loss == "softmax":
+        logits = GO @ P["Wfc"].T + P["bfc"]
+        rows = torch.nn.functional.cross_entropy(
+            logits, torch.tensor(np.asarray(labels), dtype=torch.long), reduction="none")
+        return rows, rows.mean()
+    if loss == "root_sq":
+        roots = [v for v, p in enumerate(parents) if p < 0]
+        t = (GO[roots] ** 2).sum()
+        return t.reshape(1), t
+    t = GO.abs().sum()
+    return t.reshape(1), t
+
+
+def _treelstm_cell(P, H, xid, hl, cl, hr, cr):
+    W, U, Bv = P["W"], P["U"], P["Bv"]
+    U_iou = U[: 3 * H * H].reshape(H, 3 * H)
+    U_f = U[3 * H * H :].reshape(H, H)
+    e = P["Emb"][xid]
+    xW = e @ W
+    hU = (hl + hr) @ U_iou
+    i = torch.sigmoid(xW[..., 0:H] + hU[..., 0:H] + Bv[0:H])
+    o = torch.sigmoid(xW[..., H : 2 * H] + hU[..., H : 2 * H] + Bv[3 * H :])
+    u = torch.tanh(xW[..., 2 * H : 3 * H] + hU[..., 2 * H :] + Bv[2 * H : 3 * H])
+    fl = torch.sigmoid(xW[..., 3 * H :] + hl @ U_f + Bv[H : 2 * H])
+    fr = torch.sigmoid(xW[..., 3 * H :] + hr @ U_f + Bv[H : 2 * H])
+    c = i * u + fl * cl + fr * cr
+    return o * torch.tanh(c), c
+
+
+def _lstm_cell(P, H, xid, hp, cp):
+    Wf = P["W"]
+    Ux = Wf[: 4 * H * H].reshape(H, 4 * H)
+    Wh = Wf[4 * H * H :].reshape(H, 4 * H)
+    a = P["Emb"][xid] @ Ux + hp @ Wh + P["Bv"]
+    i, f = torch.sigmoid(a[..., 0:H]), torch.sigmoid(a[..., H : 2 * H])
+    u, o = torch.tanh(a[..., 2 * H : 3 * H]), torch.sigmoid(a[..., 3 * H :])
+    c = i * u + f * cp
+    return o * torch.tanh(c), c
+
+
+def _fc_cell(P, hl, hr, xin, act, use_bias):
+    z = torch.cat([hl, hr], -1) @ P["W"]
+    if use_bias:
+        z = z + P["Bv"]
+    if xin is not None:
+        z = z + xin
+    return torch.tanh(z) if act else torch.relu(z)
+
+
+def per_sample(model, graph, x, labels, params, H, loss="softmax", act=0, use_bias=False,
+               use_x=False):
+    P = tparams(params)
+    parents, children = _adj(graph)
+    n = len(parents)
+    xs = torch.tensor(np.asarray(x), dtype=D)
+    zero = torch.zeros(H, dtype=D)
+    h, c = [None] * n, [None] * n
+    order, indeg = [], [len(ch) for ch in children]
+    stack = [v for v in range(n) if indeg[v] == 0]
+    while stack:  # any topological order
+        v = stack.pop()
+        order.append(v)
+        p = parents[v]
+        if p >= 0:
+            indeg[p] -= 1
+            if indeg[p] == 0:
+                stack.append(p)
+    for v in order:
+        ch = sorted(children[v])
+        if model == "treelstm":
+            hl, cl = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
+            hr, cr = (h[ch[1]], c[ch[1]]) if ch else (zero, zero)
+            h[v], c[v] = _treelstm_cell(P, H, int(xs[v]), hl, cl, hr, cr)
+        elif model == "lstm":
+            hp, cp = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
+            h[v], c[v] = _lstm_cell(P, H, int(xs[v]), hp, cp)
+        else:
+            hl = h[ch[0]] if ch else zero
+            hr = h[ch[1]] if ch else zero
+            h[v] = _fc_cell(P, hl, hr, xs[v] if use_x else None, act, use_bias)
+    GO = torch.stack(h)
+    GO.retain_grad()
+    rows, total = _head(GO, P, labels, loss, parents)
+    total.backward()
+    grads = {"d" + k: (v.grad.numpy() if v.grad is not None else np.zeros(v.shape)) for k, v in P.items()}
+    return dict(loss=rows.detach().numpy(), graph_out=GO.detach().numpy(),
+                dgraph_out=GO.grad.numpy(), grads=grads)
+
+
+def round_based(model, graph, trace, x, labels, params, H, loss="softmax", act=0,
+                use_bias=False, use_x=False, pairing="reference"):
+    P = tparams(params)
+    parents, _ = _adj(graph)
+    N = trace["N"]
+    mw = H if model == "treefc" else 2 * H
+    xs = torch.tensor(np.asarray(x), dtype=D)
+    pool = torch.zeros(N + 1, mw, dtype=D)
+    ret = [None] * N
+    for rd in trace["fwd"]:
+        jobs, off, n = rd["exec"], rd["offset"], len(rd["exec"])
+        G = []
+        for cidx in range(2):
+            lst = rd["gather"][cidx]
+            g = torch.zeros(n, mw, dtype=D)
+            if lst:
+                g = torch.cat([pool[lst], g[len(lst):]], 0)
+            G.append(g)
+        if model == "treelstm":
+            hh, cc = _treelstm_cell(P, H, xs[jobs].long(), G[0][:, :H], G[0][:, H:], G[1][:, :H],
+                                    G[1][:, H:])
+            msg = torch.cat([hh, cc], 1)
+        elif model == "lstm":
+            hh, cc = _lstm_cell(P, H, xs[jobs].long(), G[0][:, :H], G[0][:, H:])
+            msg = torch.cat([hh, cc], 1)
+        else:
+            hh = _fc_cell(P, G[0], G[1], xs[jobs] if use_x else None, act, use_bias)
+            msg = hh
+        lst = rd["scatter"][0]
+        if lst:
+            src = msg[: len(lst)] if pairing == "reference" else msg[[t - off for t in lst]]
+            pool = pool.index_copy(0, torch.tensor(lst), src)
+        for b, v in enumerate(jobs):
+            ret[v] = hh[b]
+    GO = torch.stack(ret)
+    GO.retain_grad()
+    rows, total = _head(GO, P, labels, loss, parents)
+    total.backward()
+    grads = {"d" + k: (v.grad.numpy() if v.grad is not None else np.zeros(v.shape)) for k, v in P.items()}
+    return dict(loss=rows.detach().numpy(), graph_out=GO.detach().numpy(),
+                dgraph_out=GO.grad.numpy(), grads=grads)
