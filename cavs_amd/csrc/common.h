@@ -1,0 +1,42 @@
+// Shared helpers of the HIP backend: error capture, stream cast, launch checks.
+#ifndef CAVS_CSRC_COMMON_H_
+#define CAVS_CSRC_COMMON_H_
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+
+#include "cavs_hip.h"
+
+namespace cavs {
+
+int set_error(int code, const char *fmt, ...);
+
+inline hipStream_t as_stream(void *s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+constexpr int kWave = 64;
+int num_cus();  // compute units of the current device (256 on MI355X)
+
+}  // namespace cavs
+
+#define CAVS_HIP_TRY(expr)                                                          \
+  do {                                                                              \
+    hipError_t _e = (expr);                                                         \
+    if (_e != hipSuccess)                                                           \
+      return cavs::set_error(CAVS_EHIP, "%s failed: %s (%s:%d)", #expr,             \
+                             hipGetErrorString(_e), __FILE__, __LINE__);            \
+  } while (0)
+
+#define CAVS_REQUIRE(cond, ...)                                   \
+  do {                                                            \
+    if (!(cond)) return cavs::set_error(CAVS_EINVAL, __VA_ARGS__); \
+  } while (0)
+
+// after a kernel launch
+#define CAVS_LAUNCH_CHECK() CAVS_HIP_TRY(hipGetLastError())
+
+#endif

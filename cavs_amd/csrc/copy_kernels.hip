@@ -1,0 +1,189 @@
+// Level-wise row movement: gather / scatter / zero / copy of [n, w] slabs through
+// int32 row lists.  HBM-bound: every payload byte is read once and written once
+// with 16-byte lane accesses (a wave moves 1 KiB per instruction), several
+// independent rows in flight per lane, and the row id read once per workgroup.
+#include "common.h"
+
+namespace cavs {
+
+template <typename V>
+__device__ inline V vzero();
+template <>
+__device__ inline float4 vzero<float4>() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+template <>
+__device__ inline float vzero<float>() { return 0.f; }
+
+__device__ inline float4 vadd(float4 a, float4 b) {
+  return make_float4(a.x + b.x, a.y + b.y, a.z + b.z, a.w + b.w);
+}
+__device__ inline float vadd(float a, float b) { return a + b; }
+
+constexpr int kRowsPerBlock = 4;
+
+// out[b] = ids[b] >= 0 ? src[ids[b]] : 0.  ids == nullptr copies row b (copy_rows);
+// src == nullptr zero-fills (zero_rows).  Strides and widths in units of V.
+template <typename V>
+__global__ void gather_rows_kernel(V *__restrict__ out, long ld_out, const V *__restrict__ src,
+                                   long ld_src, const int *__restrict__ ids, int n, int wv) {
+  const int row0 = blockIdx.x * kRowsPerBlock;
+  long srow[kRowsPerBlock];
+#pragma unroll
+  for (int r = 0; r < kRowsPerBlock; r++) {
+    int row = row0 + r;
+    long id = -1;
+    if (row < n && src) id = ids ? ids[row] : row;
+    srow[r] = id;
+  }
+  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+    V v[kRowsPerBlock];
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++)
+      v[r] = srow[r] >= 0 ? src[srow[r] * ld_src + c] : vzero<V>();
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++)
+      if (row0 + r < n) out[(long)(row0 + r) * ld_out + c] = v[r];
+  }
+}
+
+// dst[ids[b]] = inp[b] for ids[b] >= 0
+template <typename V>
+__global__ void scatter_rows_kernel(V *__restrict__ dst, long ld_dst, const int *__restrict__ ids,
+                                    const V *__restrict__ inp, long ld_inp, int n, int wv) {
+  const int row0 = blockIdx.x * kRowsPerBlock;
+  long drow[kRowsPerBlock];
+#pragma unroll
+  for (int r = 0; r < kRowsPerBlock; r++) {
+    int row = row0 + r;
+    drow[r] = row < n ? (long)ids[row] : -1;
+  }
+  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+    V v[kRowsPerBlock];
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++)
+      if (drow[r] >= 0) v[r] = inp[(long)(row0 + r) * ld_inp + c];
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++)
+      if (drow[r] >= 0) dst[drow[r] * ld_dst + c] = v[r];
+  }
+}
+
+// Two vertices per workgroup: G[2b+i] = pool[ids[2b+i]] (or 0), hsum[b] = G[2b] + G[2b+1]
+// over the first hv vector columns.
+template <typename V>
+__global__ void gather_children_kernel(V *__restrict__ G, V *__restrict__ hsum,
+                                       const V *__restrict__ pool, const int *__restrict__ ids,
+                                       int n, int wv, int hv) {
+  constexpr int kNodes = 2;
+  const int b0 = blockIdx.x * kNodes;
+  long srow[2 * kNodes];
+#pragma unroll
+  for (int r = 0; r < 2 * kNodes; r++) {
+    int row = 2 * b0 + r;
+    srow[r] = row < 2 * n ? (long)ids[row] : -1;
+  }
+  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+    V v[2 * kNodes];
+#pragma unroll
+    for (int r = 0; r < 2 * kNodes; r++)
+      v[r] = srow[r] >= 0 ? pool[srow[r] * wv + c] : vzero<V>();
+#pragma unroll
+    for (int r = 0; r < 2 * kNodes; r++)
+      if (2 * b0 + r < 2 * n) G[(long)(2 * b0 + r) * wv + c] = v[r];
+    if (hsum && c < hv) {
+#pragma unroll
+      for (int k = 0; k < kNodes; k++)
+        if (b0 + k < n) hsum[(long)(b0 + k) * hv + c] = vadd(v[2 * k], v[2 * k + 1]);
+    }
+  }
+}
+
+inline int block_for(int wv) { return wv >= 256 ? 256 : (wv > 128 ? 256 : (wv > 64 ? 128 : 64)); }
+
+inline bool vec_ok(const void *a, long lda, const void *b, long ldb, int w) {
+  return (w % 4 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (!a || aligned16(a)) &&
+         (!b || aligned16(b));
+}
+
+static int launch_gather(float *out, int ld_out, const float *src, int ld_src, const int *ids,
+                         int n, int w, hipStream_t st) {
+  if (n == 0 || w == 0) return CAVS_OK;
+  int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (vec_ok(out, ld_out, src, ld_src, w)) {
+    int wv = w / 4;
+    gather_rows_kernel<float4><<<grid, block_for(wv), 0, st>>>(
+        reinterpret_cast<float4 *>(out), ld_out / 4, reinterpret_cast<const float4 *>(src),
+        ld_src / 4, ids, n, wv);
+  } else {
+    gather_rows_kernel<float><<<grid, block_for(w), 0, st>>>(out, ld_out, src, ld_src, ids, n, w);
+  }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // namespace cavs
+
+using namespace cavs;
+
+extern "C" {
+
+int cavs_gather_rows(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n,
+                     int w, void *stream) {
+  CAVS_REQUIRE(n >= 0 && w >= 0 && ld_out >= w && ld_src >= w, "cavs_gather_rows: bad shape n=%d w=%d ld_out=%d ld_src=%d", n, w, ld_out, ld_src);
+  if (n == 0 || w == 0) return CAVS_OK;
+  CAVS_REQUIRE(out && src && ids, "cavs_gather_rows: null pointer");
+  return launch_gather(out, ld_out, src, ld_src, ids, n, w, as_stream(stream));
+}
+
+int cavs_copy_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w,
+                   void *stream) {
+  CAVS_REQUIRE(n >= 0 && w >= 0 && ld_out >= w && ld_inp >= w, "cavs_copy_rows: bad shape n=%d w=%d", n, w);
+  if (n == 0 || w == 0) return CAVS_OK;
+  CAVS_REQUIRE(out && inp, "cavs_copy_rows: null pointer");
+  return launch_gather(out, ld_out, inp, ld_inp, nullptr, n, w, as_stream(stream));
+}
+
+int cavs_zero_rows(float *out, int ld_out, int n, int w, void *stream) {
+  CAVS_REQUIRE(n >= 0 && w >= 0 && ld_out >= w, "cavs_zero_rows: bad shape n=%d w=%d", n, w);
+  if (n == 0 || w == 0) return CAVS_OK;
+  CAVS_REQUIRE(out, "cavs_zero_rows: null pointer");
+  return launch_gather(out, ld_out, nullptr, ld_out, nullptr, n, w, as_stream(stream));
+}
+
+int cavs_scatter_rows(float *dst, int ld_dst, const int *ids, const float *inp, int ld_inp, int n,
+                      int w, void *stream) {
+  CAVS_REQUIRE(n >= 0 && w >= 0 && ld_dst >= w && ld_inp >= w, "cavs_scatter_rows: bad shape n=%d w=%d", n, w);
+  if (n == 0 || w == 0) return CAVS_OK;
+  CAVS_REQUIRE(dst && ids && inp, "cavs_scatter_rows: null pointer");
+  hipStream_t st = as_stream(stream);
+  int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (vec_ok(dst, ld_dst, inp, ld_inp, w)) {
+    int wv = w / 4;
+    scatter_rows_kernel<float4><<<grid, block_for(wv), 0, st>>>(
+        reinterpret_cast<float4 *>(dst), ld_dst / 4, ids, reinterpret_cast<const float4 *>(inp),
+        ld_inp / 4, n, wv);
+  } else {
+    scatter_rows_kernel<float><<<grid, block_for(w), 0, st>>>(dst, ld_dst, ids, inp, ld_inp, n, w);
+  }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_gather_children(float *G, float *hsum, const float *pool, const int *ids, int n, int w,
+                         int hw, void *stream) {
+  CAVS_REQUIRE(n >= 0 && w > 0 && hw >= 0 && hw <= w, "cavs_gather_children: bad shape n=%d w=%d hw=%d", n, w, hw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(G && pool && ids, "cavs_gather_children: null pointer");
+  hipStream_t st = as_stream(stream);
+  int grid = (n + 1) / 2;
+  if (w % 4 == 0 && hw % 4 == 0 && aligned16(G) && aligned16(pool) && (!hsum || aligned16(hsum))) {
+    gather_children_kernel<float4><<<grid, block_for(w / 4), 0, st>>>(
+        reinterpret_cast<float4 *>(G), reinterpret_cast<float4 *>(hsum),
+        reinterpret_cast<const float4 *>(pool), ids, n, w / 4, hw / 4);
+  } else {
+    gather_children_kernel<float><<<grid, block_for(w), 0, st>>>(G, hsum, pool, ids, n, w, hw);
+  }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // extern "C"

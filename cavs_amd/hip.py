@@ -1,0 +1,117 @@
+"""ctypes binding of the C ABI declared in include/cavs_hip.h.
+
+The library is loaded from cavs_amd/lib; there is no CPU fallback: if the shared
+object is missing, loading raises.  Device buffers are plain integers (device
+addresses), typically `torch.Tensor.data_ptr()`; streams are raw hipStream_t
+handles (`torch.cuda.current_stream().cuda_stream`).
+"""
+import ctypes as C
+import os
+import re
+
+_PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_PKG, "lib", "libcavs_hip.so")
+HEADER = os.path.join(os.path.dirname(_PKG), "include", "cavs_hip.h")
+
+
+class CavsError(RuntimeError):
+    pass
+
+
+_lib = None
+
+_P, _I, _F, _Z = C.c_void_p, C.c_int, C.c_float, C.c_size_t
+
+# name -> argtypes (every function returns int unless listed in _RESTYPE)
+_SIGS = {
+    "cavs_init": [_I],
+    "cavs_device_name": [C.c_char_p, _Z],
+    "cavs_malloc": [C.POINTER(_P), _Z],
+    "cavs_free": [_P],
+    "cavs_host_alloc": [C.POINTER(_P), _Z],
+    "cavs_host_free": [_P],
+    "cavs_memcpy_h2d": [_P, _P, _Z, _P],
+    "cavs_memcpy_d2h": [_P, _P, _Z, _P],
+    "cavs_memcpy_d2d": [_P, _P, _Z, _P],
+    "cavs_zero": [_P, _Z, _P],
+    "cavs_fill": [_P, _F, _Z, _P],
+    "cavs_stream_create": [C.POINTER(_P)],
+    "cavs_stream_destroy": [_P],
+    "cavs_stream_sync": [_P],
+    "cavs_event_create": [C.POINTER(_P)],
+    "cavs_event_destroy": [_P],
+    "cavs_event_record": [_P, _P],
+    "cavs_event_elapsed_ms": [C.POINTER(_F), _P, _P],
+    "cavs_gather_rows": [_P, _I, _P, _I, _P, _I, _I, _P],
+    "cavs_scatter_rows": [_P, _I, _P, _P, _I, _I, _I, _P],
+    "cavs_zero_rows": [_P, _I, _I, _I, _P],
+    "cavs_copy_rows": [_P, _I, _P, _I, _I, _I, _P],
+    "cavs_gather_children": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "cavs_sgemm": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
+    "cavs_sgemm_addrows": [_I, _I, _I, _I, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P],
+    "cavs_sgemm_splitk": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _Z, _P],
+    "cavs_colsum": [_P, _P, _I, _I, _I, _I, _P],
+    "cavs_embed_fwd": [_P, _I, _P, _P, _I, _I, _P],
+    "cavs_embed_bwd": [_P, _P, _P, _I, _I, _I, _P],
+    "cavs_bias_add_rows": [_P, _P, _P, _I, _I, _P],
+    "cavs_softmax_xent": [_P, _P, _P, _P, _I, _I, _P],
+    "cavs_sgd": [_P, _P, _F, _Z, _P],
+    "cavs_ew_binary": [_I, _P, _P, _Z, _P, _Z, _Z, _I, _P],
+    "cavs_ew_unary": [_I, _P, _P, _Z, _I, _P],
+    "cavs_scale": [_P, _P, _F, _Z, _P],
+    "cavs_treelstm_gates_fwd": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
+    "cavs_lstm_gates_fwd": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_lstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
+    "cavs_treefc_fwd": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "cavs_treefc_bwd": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "cavs_fused_compile": [C.c_char_p, C.c_char_p, C.POINTER(_P)],
+    "cavs_fused_launch": [_P, C.POINTER(_P), _I, C.POINTER(_P), _I, C.POINTER(_I), C.POINTER(_I), _I, _P],
+    "cavs_fused_release": [_P],
+    "cavs_schedule_frontier": [_P, _I, _P, _P, _P, _P, _P, _P, _P],
+}
+_RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z}
+_NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I]}
+
+EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)
+EW_UNARY = dict(assign=0, neg=1, abs=2, square=3, sigmoid=4, tanh=5, relu=6)
+
+
+def declared_symbols():
+    """extern "C" function names declared in include/cavs_hip.h"""
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(cavs_[a-z0-9_]+)\s*\(", text)))
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise CavsError(f"{LIB_PATH} is missing: build it with `python -m cavs_amd.build` "
+                            "(there is no CPU fallback)")
+        l = C.CDLL(LIB_PATH)
+        for name, args in _SIGS.items():
+            fn = getattr(l, name)
+            fn.argtypes, fn.restype = args, _I
+        for name, args in _NOCHECK.items():
+            fn = getattr(l, name)
+            fn.argtypes, fn.restype = args, _RESTYPE[name]
+        _lib = l
+    return _lib
+
+
+def call(name, *args):
+    """Calls an int-returning entry point and raises CavsError on failure."""
+    rc = getattr(lib(), name)(*args)
+    if rc != 0:
+        raise CavsError(f"{name} -> {rc}: {lib().cavs_last_error().decode()}")
+
+
+def ptr(t):
+    """device address of a torch tensor (or None / int passthrough)"""
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    return t.data_ptr()

@@ -1,0 +1,229 @@
+/*
+ * cavs_hip.h -- C ABI of the MI355X (gfx950) backend for Cavs's batched execution
+ * of a vertex function F over an instance graph G.
+ *
+ * This is the boundary the reference's op plug-ins would bind: every entry point
+ * replaces the body of one backend::OpImpl::Compute (cavs/backend/op_impl.h:14-28)
+ * or one piece of the batching memory manager, and takes what that Compute reads
+ * from its OpContext (cavs/midend/op_context.h:14-62) as plain device pointers,
+ * row counts, widths and leading dimensions.  No C++ types cross it.
+ *
+ * Conventions
+ *   - every function returns 0 on success or a negative CAVS_E* code and never
+ *     aborts (the reference CHECK-aborts, cavs/util/macros_gpu.h:10-45);
+ *     cavs_last_error() gives the message of the calling thread's last failure;
+ *   - all matrices are row-major fp32; `ld*` is the row stride in elements;
+ *   - index lists are device int32 arrays;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ *     every compute entry point is asynchronous with respect to the device;
+ *   - single caller thread per stream, like the reference's session loop.
+ */
+#ifndef CAVS_HIP_H_
+#define CAVS_HIP_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  CAVS_OK = 0,
+  CAVS_EINVAL = -1,  /* bad argument (shape, alignment, null pointer) */
+  CAVS_EHIP = -2,    /* a HIP runtime call failed                      */
+  CAVS_ENOMEM = -3,
+  CAVS_EUNSUPPORTED = -4
+};
+
+const char *cavs_last_error(void);
+/* ABI version of this header; bumped on any signature change. */
+int cavs_abi_version(void);
+
+/* ------------------------------------------------------------------ runtime
+ * Replaces GPUAllocator (cavs/midend/allocator.cu:9-27), the H2D/D2H copies of
+ * Tensor feeds (cavs/midend/tensor.cc:324-351), the handle/stream pool
+ * (cavs/util/stream_event_handle_pool.h:8-65) and Timing (cavs/util/timing.h:10-67). */
+int cavs_init(int device);
+int cavs_device_name(char *buf, size_t len);
+int cavs_malloc(void **ptr, size_t bytes);
+int cavs_free(void *ptr);
+int cavs_host_alloc(void **ptr, size_t bytes); /* pinned host memory */
+int cavs_host_free(void *ptr);
+int cavs_memcpy_h2d(void *dst, const void *src, size_t bytes, void *stream);
+int cavs_memcpy_d2h(void *dst, const void *src, size_t bytes, void *stream);
+int cavs_memcpy_d2d(void *dst, const void *src, size_t bytes, void *stream);
+/* Tensor::InitWithZero (cavs/midend/tensor.cc:283-300); a fill kernel, safe to
+ * capture in a graph. */
+int cavs_zero(void *ptr, size_t bytes, void *stream);
+int cavs_fill(float *ptr, float value, size_t n, void *stream); /* ConstOp / Fill */
+int cavs_stream_create(void **stream);
+int cavs_stream_destroy(void *stream);
+int cavs_stream_sync(void *stream);
+int cavs_event_create(void **event);
+int cavs_event_destroy(void *event);
+int cavs_event_record(void *event, void *stream);
+int cavs_event_elapsed_ms(float *ms, void *start, void *stop); /* waits for `stop` */
+
+/* ------------------------------------------------------------------ graph ops
+ * Replace GraphGatherOp / GraphScatterOp / GraphPushOp / GraphPullOp /
+ * FunctionPopRetOp (cavs/backend/op_impl_graphop.cu:17-327) and their kernels
+ * (cavs/backend/functor_batched_memcpy.cuh:18-75).  An id of -1 means "no row":
+ * gather writes zeros for it (the reference's separate zero-fill kernel), scatter
+ * skips it. */
+
+/* out[b, 0:w] = ids[b] >= 0 ? src[ids[b], 0:w] : 0        b in [0,n) */
+int cavs_gather_rows(float *out, int ld_out, const float *src, int ld_src, const int *ids,
+                     int n, int w, void *stream);
+/* dst[ids[b], 0:w] = inp[b, 0:w]   for ids[b] >= 0 */
+int cavs_scatter_rows(float *dst, int ld_dst, const int *ids, const float *inp, int ld_inp,
+                      int n, int w, void *stream);
+/* out[b, 0:w] = 0 */
+int cavs_zero_rows(float *out, int ld_out, int n, int w, void *stream);
+/* out[b, 0:w] = inp[b, 0:w]  (Push, Slice, Concat: column blocks via ld) */
+int cavs_copy_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w,
+                   void *stream);
+/* Both child gathers of a binary vertex function in one pass, plus h_l + h_r:
+ *   G[2b+i, 0:w] = ids[2b+i] >= 0 ? pool[ids[2b+i], 0:w] : 0      i in {0,1}
+ *   hsum[b, 0:hw] = G[2b, 0:hw] + G[2b+1, 0:hw]   (hsum may be NULL)
+ * Replaces the two Gather ops and the Add of apps/paper/tree-lstm-cavs.cc:132-137. */
+int cavs_gather_children(float *G, float *hsum, const float *pool, const int *ids, int n,
+                         int w, int hw, void *stream);
+
+/* ------------------------------------------------------------------ dense math */
+/* Row-major C[M,N] = alpha*op(A)*op(B) + beta*C on the FP32 MFMA pipe.  Replaces
+ * MatMulMatCublasWrapper (cavs/backend/cublas_wrapper.cc:12-28) as used by
+ * MatMulMatOpCublas (cavs/backend/op_impl_blas3_cublas.cc:34-70) and its
+ * gradients (cavs/backend/op_decl_matmul.cc:18-69).  op(A) is M x K. */
+int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+               int lda, const float *B, int ldb, float beta, float *C, int ldc, void *stream);
+/* C[r,:] = op(A)*op(B) + D[r >> d_shift, :]: the GEMM and the Accumulate that
+ * follows it in the backward of a Mirror'ed operand
+ * (cavs/backend/op_decl_slice_join.cc:173-182) in one pass. */
+int cavs_sgemm_addrows(int transA, int transB, int M, int N, int K, const float *A, int lda,
+                       const float *B, int ldb, const float *D, int ldd, int d_shift, float *C,
+                       int ldc, void *stream);
+/* Bytes of device workspace cavs_sgemm_splitk needs for this shape. */
+size_t cavs_sgemm_splitk_workspace(int M, int N, int K);
+/* Same contract as cavs_sgemm for tall-K products (the deferred weight-gradient
+ * GEMMs of cavs/midend/batch_weight_updater.h:12-84): K is split over workgroups,
+ * partials go to `workspace` and are reduced in a fixed order (deterministic). */
+int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                      int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                      void *workspace, size_t workspace_bytes, void *stream);
+/* out[j] (+)= sum_r inp[r, j], j in [0,w): UnaryBroadcastingKernel
+ * (cavs/backend/op_impl_elementwise.cuh:24-34) used for bias gradients. */
+int cavs_colsum(float *out, const float *inp, int ld, int n, int w, int accumulate,
+                void *stream);
+/* EmbeddingLookupOp / GradOp (cavs/backend/op_impl_embedding_lookup.cu:37-148);
+ * ids are floats, the row offset is int(id * E) as in the reference. */
+int cavs_embed_fwd(float *out, int ld_out, const float *ids, const float *table, int n, int E,
+                   void *stream);
+int cavs_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, int n, int E,
+                   void *stream);
+/* out[r, :] = inp[r, :] + bias[:]  (BinaryBroadcastingKernel,
+ * cavs/backend/op_impl_elementwise.cuh:128-139; also the ones-vector bias GEMM of
+ * cavs/backend/op_impl_fullyconnected_cublas.cc:74-76) */
+int cavs_bias_add_rows(float *out, const float *inp, const float *bias, int n, int w,
+                       void *stream);
+/* SoftmaxEntropyLossOpCudnn / ...Grad
+ * (cavs/backend/op_impl_softmax_entropy_logits_loss.cu:94-140, 212-250):
+ * loss[r] = -log softmax(logits[r])[label[r]], dlogits = (softmax - onehot)/n.
+ * Either output may be NULL. */
+int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const float *labels,
+                      int n, int C, void *stream);
+/* SGD (cavs/backend/op_impl_sgd.cu): w -= lr * g */
+int cavs_sgd(float *w, const float *g, float lr, size_t n, void *stream);
+
+/* ------------------------------------------------------------------ elementwise
+ * The un-fused elementwise family (cavs/backend/op_impl_elementwise.{cu,cuh},
+ * functor_elementwise.h, op_impl_activation_cudnn.cu).  Operands are read as
+ * x[i % count], which covers same-shape, scalar and row-broadcast forms
+ * (BinaryKernel / BinaryScalarKernel / BinaryBroadcastingKernel). */
+enum {
+  CAVS_EW_ADD = 0, CAVS_EW_SUB = 1, CAVS_EW_MUL = 2, CAVS_EW_DIV = 3,
+  CAVS_EW_SIGMOID_GRAD = 4, /* a = dy, b = y : dy * y * (1-y)  */
+  CAVS_EW_TANH_GRAD = 5,    /* a = dy, b = y : dy * (1 - y*y)  */
+  CAVS_EW_RELU_GRAD = 6,    /* a = dy, b = y : y > 0 ? dy : 0  */
+  CAVS_EW_EQUAL = 7
+};
+enum {
+  CAVS_EW_ASSIGN = 0, CAVS_EW_NEG = 1, CAVS_EW_ABS = 2, CAVS_EW_SQUARE = 3,
+  CAVS_EW_SIGMOID = 4, CAVS_EW_TANH = 5, CAVS_EW_RELU = 6
+};
+int cavs_ew_binary(int op, float *out, const float *a, size_t na, const float *b, size_t nb,
+                   size_t n, int accumulate, void *stream);
+int cavs_ew_unary(int op, float *out, const float *a, size_t n, int accumulate, void *stream);
+int cavs_scale(float *out, const float *a, float s, size_t n, void *stream); /* Scal */
+
+/* ------------------------------------------------------------------ fused gates
+ * The fused-op interface for the three vertex functions the benchmarks use: one
+ * kernel replaces the Slice / Add / Sigmoid / Tanh / Mul / Concat chain of F
+ * (what the reference's runtime fusion compiler emits as FusedKernel nodes,
+ * cavs/midend/runtime_compiler/code_generator.cc:104-185, launched by
+ * cavs/backend/op_impl_fused_kernel.cu:34-64) and the chain of F's gradient.
+ * Row r of every operand is slab row r of the current round.
+ *
+ * Tree-LSTM (apps/paper/tree-lstm-cavs.cc:132-171):
+ *   xW  [n,4H] (ld_xw) column blocks [i|o|u|f]
+ *   hU  [n,3H] blocks [i|o|u], hUf [2n,H] rows (2r: f_l, 2r+1: f_r);
+ *        both NULL for a round of leaves (their gathered children are zero)
+ *   G   [2n,2H] gathered children, row 2r+i = child i as [h|c]; NULL for leaves
+ *   bias [4H] blocks [i|f|u|o]
+ *   gates [n,6H] = [i|o|u|f_l|f_r|tanh c] saved for backward; msg [n,2H] = [h|c] */
+int cavs_treelstm_gates_fwd(const float *xW, int ld_xw, const float *hU, const float *hUf,
+                            const float *G, const float *bias, float *gates, float *msg,
+                            int n, int H, void *stream);
+/* dmsg [n,2H] gathered-back message gradient, dret [n,H] pulled d GraphOutput.
+ * Writes dxW [n,4H] (ld_dxw) = [d_i|d_o|d_u|d_fl+d_fr]; for internal rounds also
+ * dF [2n,H] = rows (d_fl, d_fr) and the c half of dG [2n,2H] (dc_l, dc_r); pass
+ * G = dF = dG = NULL for a round of leaves. */
+int cavs_treelstm_gates_bwd(const float *dmsg, const float *dret, const float *gates,
+                            const float *G, float *dxW, int ld_dxw, float *dF, float *dG,
+                            int n, int H, void *stream);
+/* Chain LSTM (apps/paper/seq-lstm-cavs.cc:62-86): a [n,4H] = x*U' (+ h_p*W'),
+ * blocks [i|f|u|o]; a2 (optional, may be NULL) is added to a (the h_p*W' term
+ * kept in its own buffer); G [n,2H] = [h_p|c_p] or NULL for the first round;
+ * gates [n,5H] = [i|f|u|o|tanh c]. */
+int cavs_lstm_gates_fwd(const float *a, int ld_a, const float *a2, const float *G,
+                        const float *bias, float *gates, float *msg, int n, int H,
+                        void *stream);
+int cavs_lstm_gates_bwd(const float *dmsg, const float *dret, const float *gates,
+                        const float *G, float *da, int ld_da, float *dG, int n, int H,
+                        void *stream);
+/* Tree-FC (apps/paper/tree-fc-cavs.cc:28-36): h = act(z + bias + x); z, bias, x may
+ * each be NULL (z is NULL for a round of leaves).  act: 0 relu, 1 tanh. */
+int cavs_treefc_fwd(const float *z, const float *bias, const float *x, float *h, int n, int H,
+                    int act, void *stream);
+int cavs_treefc_bwd(const float *dh_m, const float *dret, const float *h, float *dz, int n,
+                    int H, int act, void *stream);
+
+/* ------------------------------------------------------------------ generic fused op
+ * FusedKernelOpImpl (cavs/backend/op_impl_fused_kernel.cu:17-71): compiles the
+ * source the fusion pass generated (runtime_compiler/code_generator.cc:20-100;
+ * signature: outputs, const inputs, output counts, input counts, n_elements) with
+ * the runtime compiler for gfx950, FMA contraction off like the reference's
+ * --fmad=false (cavs/backend/cudaRTC_wrapper.h:47-50), and launches it over a 1-D
+ * grid. */
+int cavs_fused_compile(const char *kernel_name, const char *source, void **handle);
+int cavs_fused_launch(void *handle, float *const *outs, int nouts, const float *const *ins,
+                      int nins, const int *out_counts, const int *in_counts, int n_elements,
+                      void *stream);
+int cavs_fused_release(void *handle);
+
+/* ------------------------------------------------------------------ device schedule
+ * The level-wise ready frontier of BatchGraphScheduler::Initialize/ActivateNext
+ * (cavs/midend/graph_scheduler.cc:169-245) computed on the GPU from the global
+ * parent array.  Inputs: parent[N] (global parent id or -1), N.  Outputs (device,
+ * each sized N unless noted): tids_to_jobids, jobids_to_tids, round_of_tid,
+ * round2offset [N+2] (entries past R+1 undefined), n_rounds [1]; `scratch` is 4*N
+ * ints of device memory the call may overwrite.  Vertices have at most two
+ * children, like the reference's two gather lists (graph_scheduler.h:16-18).
+ * The backward schedule is these rounds replayed last to first. */
+int cavs_schedule_frontier(const int *parent, int N, int *tids_to_jobids, int *jobids_to_tids,
+                           int *round_of_tid, int *round2offset, int *n_rounds, int *scratch,
+                           void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

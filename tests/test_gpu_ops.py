@@ -1,0 +1,434 @@
+"""GPU parity of every op-level entry point of the C ABI against the oracle.
+Bit-exact for row movement and index work, fp32 tolerance (1e-4 rel / 1e-5 abs,
+the bar of the path) for arithmetic."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from cavs_amd import hip, synth
+
+pytestmark = pytest.mark.gpu
+
+RTOL, ATOL = 1e-4, 1e-5
+
+
+@pytest.fixture(scope="module")
+def g():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import gpuutil
+
+    hip.call("cavs_init", 0)
+    return gpuutil
+
+
+@pytest.fixture(autouse=True)
+def _release_device_temporaries(g):
+    yield
+    g.release()
+
+
+def rng(seed):
+    return synth.SplitMix64(seed)
+
+
+def close(got, want, what="", rtol=RTOL, atol=ATOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    scale = max(1.0, float(np.abs(want).max())) if want.size else 1.0
+    np.testing.assert_allclose(got, want, rtol=rtol, atol=atol * scale, err_msg=what)
+
+
+# ---------------------------------------------------------------- row movement
+@pytest.mark.parametrize("n,w,ld_extra", [(1, 4, 0), (7, 1024, 0), (33, 256, 0), (130, 36, 4),
+                                           (50, 37, 3), (5, 2048, 0), (1000, 512, 0)])
+def test_gather_scatter_zero_copy_rows_bit_exact(g, oracle, n, w, ld_extra):
+    r = rng(n * 131 + w)
+    rows = 2 * n + 3
+    ld = w + ld_extra
+    src = r.bulk_normal(rows * ld).reshape(rows, ld)
+    ids = (np.floor(r.bulk_uniform(n) * rows)).astype(np.int32)
+    ids[::5] = -1  # "no row"
+    want = np.zeros((n, w), np.float32)
+    ok = ids >= 0
+    want[ok] = oracle.gather_rows(src, ids[ok], w=w)
+    out = g.zeros(n, w, fill=7.0)
+    g.call("cavs_gather_rows", g.P(out), w, g.P(g.devf(src)), ld, g.P(g.devi(ids)), n, w, g.stream())
+    np.testing.assert_array_equal(g.host(out), want)
+
+    # scatter: unique destinations so the result is order independent
+    perm = np.argsort(r.bulk_uniform(rows))[:n].astype(np.int32)
+    perm[1::4] = -1
+    inp = r.bulk_normal(n * ld).reshape(n, ld)
+    dst0 = r.bulk_normal(rows * w).reshape(rows, w)
+    want = dst0.copy()
+    ok = perm >= 0
+    tmp = np.ascontiguousarray(inp[ok][:, :w])
+    oracle.scatter_rows(want, perm[ok], tmp)
+    dst = g.devf(dst0)
+    g.call("cavs_scatter_rows", g.P(dst), w, g.P(g.devi(perm)), g.P(g.devf(inp)), ld, n, w, g.stream())
+    np.testing.assert_array_equal(g.host(dst), want)
+
+    # zero / copy through a leading dimension touch only the [n, w] block
+    buf0 = r.bulk_normal(n * ld).reshape(n, ld)
+    buf = g.devf(buf0)
+    g.call("cavs_zero_rows", g.P(buf), ld, n, w, g.stream())
+    want = buf0.copy()
+    want[:, :w] = 0
+    np.testing.assert_array_equal(g.host(buf), want)
+    buf = g.devf(buf0)
+    g.call("cavs_copy_rows", g.P(buf), ld, g.P(g.devf(src)), ld, n, w, g.stream())
+    want = buf0.copy()
+    want[:, :w] = src[:n, :w]
+    np.testing.assert_array_equal(g.host(buf), want)
+
+
+def test_row_ops_accept_empty_and_reject_bad_shapes(g):
+    out = g.zeros(4, 8)
+    hip.call("cavs_gather_rows", g.P(out), 8, None, 8, None, 0, 8, g.stream())  # n == 0 is a no-op
+    hip.call("cavs_scatter_rows", g.P(out), 8, None, None, 8, 0, 8, g.stream())
+    with pytest.raises(hip.CavsError, match="bad shape"):
+        hip.call("cavs_gather_rows", g.P(out), 4, g.P(out), 8, g.P(out), 2, 8, g.stream())
+    with pytest.raises(hip.CavsError, match="null pointer"):
+        hip.call("cavs_gather_rows", g.P(out), 8, None, 8, g.P(out), 2, 8, g.stream())
+
+
+@pytest.mark.parametrize("n,w,hw", [(1, 8, 4), (9, 1024, 512), (64, 20, 8), (31, 6, 3)])
+def test_gather_children(g, oracle, n, w, hw):
+    r = rng(n + w)
+    rows = 3 * n + 2
+    pool = r.bulk_normal(rows * w).reshape(rows, w)
+    ids = np.floor(r.bulk_uniform(2 * n) * rows).astype(np.int32)
+    if n > 2:
+        ids[2:4] = -1
+    G = g.zeros(2 * n, w, fill=3.0)
+    hs = g.zeros(n, hw, fill=3.0)
+    g.call("cavs_gather_children", g.P(G), g.P(hs), g.P(g.devf(pool)), g.P(g.devi(ids)), n, w, hw, g.stream())
+    want = np.zeros((2 * n, w), np.float32)
+    ok = ids >= 0
+    want[ok] = oracle.gather_rows(pool, ids[ok])
+    np.testing.assert_array_equal(g.host(G), want)
+    np.testing.assert_array_equal(g.host(hs), want[0::2, :hw] + want[1::2, :hw])
+
+
+# ---------------------------------------------------------------- GEMM
+SHAPES = [(13, 17, 29), (1, 64, 64), (200, 256, 64), (128, 128, 16), (129, 131, 300), (77, 2048, 300),
+          (300, 1536, 512), (5, 512, 40), (640, 5, 512), (512, 384, 2052)]
+
+
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_sgemm_matches_oracle(g, oracle, tA, tB, M, N, K):
+    r = rng(M * 7 + N * 3 + K + 2 * tA + tB)
+    A = r.bulk_uniform(M * K, -1, 1).reshape((K, M) if tA else (M, K))
+    B = r.bulk_uniform(N * K, -1, 1).reshape((N, K) if tB else (K, N))
+    C0 = r.bulk_uniform(M * N, -1, 1).reshape(M, N)
+    want = oracle.sgemm(tA, tB, A, B, alpha=0.5, beta=2.0, Cin=C0)
+    Cd = g.devf(C0)
+    g.call("cavs_sgemm", tA, tB, M, N, K, 0.5, g.P(g.devf(A)), A.shape[1], g.P(g.devf(B)), B.shape[1],
+           2.0, g.P(Cd), N, g.stream())
+    close(g.host(Cd), want, "sgemm alpha/beta")
+    # beta = 0 must not read C (NaNs in C stay out of the result)
+    Cd = g.zeros(M, N, fill=float("nan"))
+    g.call("cavs_sgemm", tA, tB, M, N, K, 1.0, g.P(g.devf(A)), A.shape[1], g.P(g.devf(B)), B.shape[1],
+           0.0, g.P(Cd), N, g.stream())
+    exact = (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64)
+    close(g.host(Cd), exact, "sgemm vs fp64")
+
+
+def test_sgemm_strided_operands_and_addrows(g, oracle):
+    """The shapes the Tree-LSTM backward uses: A is a column block of a wider slab,
+    C a column block of the child-gradient slab, plus the per-vertex addend."""
+    r = rng(5)
+    n, H = 37, 64
+    dF = r.bulk_normal(2 * n * H).reshape(2 * n, H)
+    Uf = r.bulk_uniform(H * H, -0.3, 0.3).reshape(H, H)
+    dhlr = r.bulk_normal(n * H).reshape(n, H)
+    dG0 = r.bulk_normal(2 * n * 2 * H).reshape(2 * n, 2 * H)
+    dG = g.devf(dG0)
+    g.call("cavs_sgemm_addrows", 0, 1, 2 * n, H, H, g.P(g.devf(dF)), H, g.P(g.devf(Uf)), H,
+           g.P(g.devf(dhlr)), H, 1, g.P(dG), 2 * H, g.stream())
+    want = dG0.copy()
+    want[:, :H] = oracle.sgemm(0, 1, dF, Uf) + np.repeat(dhlr, 2, axis=0)
+    close(g.host(dG), want)
+    np.testing.assert_array_equal(g.host(dG)[:, H:], dG0[:, H:])  # c half untouched
+    # A = first 3H columns of a [n,4H] slab (lda = 4H)
+    dxW = r.bulk_normal(n * 4 * H).reshape(n, 4 * H)
+    U = r.bulk_uniform(H * 3 * H, -0.3, 0.3).reshape(H, 3 * H)
+    out = g.zeros(n, H)
+    g.call("cavs_sgemm", 0, 1, n, H, 3 * H, 1.0, g.P(g.devf(dxW)), 4 * H, g.P(g.devf(U)), 3 * H, 0.0,
+           g.P(out), H, g.stream())
+    close(g.host(out), oracle.sgemm(0, 1, np.ascontiguousarray(dxW[:, :3 * H]), U))
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 96, 3000), (300, 2048, 2482), (12, 20, 777), (512, 1536, 64)])
+def test_sgemm_splitk_is_deterministic_and_correct(g, oracle, M, N, K):
+    import torch
+
+    r = rng(M + N + K)
+    A = r.bulk_uniform(K * M, -1, 1).reshape(K, M)  # TN: the weight-gradient form
+    B = r.bulk_uniform(K * N, -1, 1).reshape(K, N)
+    C0 = r.bulk_uniform(M * N, -1, 1).reshape(M, N)
+    nbytes = hip.lib().cavs_sgemm_splitk_workspace(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    outs = []
+    for _ in range(2):
+        Cd = g.devf(C0)
+        g.call("cavs_sgemm_splitk", 1, 0, M, N, K, 1.0, g.P(g.devf(A)), M, g.P(g.devf(B)), N, 1.0,
+               g.P(Cd), N, g.P(ws), nbytes, g.stream())
+        outs.append(g.host(Cd))
+    np.testing.assert_array_equal(outs[0], outs[1])
+    exact = A.T.astype(np.float64) @ B.astype(np.float64) + C0
+    close(outs[0], exact)
+    close(outs[0], oracle.sgemm(1, 0, A, B, beta=1.0, Cin=C0))
+
+
+# ---------------------------------------------------------------- gates
+@pytest.mark.parametrize("n,H", [(1, 4), (9, 8), (33, 512), (7, 6)])
+def test_treelstm_gates(g, oracle, n, H):
+    r = rng(n * H)
+    xW = r.bulk_normal(n * 4 * H).reshape(n, 4 * H)
+    hU = r.bulk_normal(n * 3 * H).reshape(n, 3 * H)
+    hUf = r.bulk_normal(2 * n * H).reshape(2 * n, H)
+    G = r.bulk_normal(2 * n * 2 * H).reshape(2 * n, 2 * H)
+    bias = r.bulk_normal(4 * H)
+    gates_w, msg_w = oracle.treelstm_gates_fwd(xW, hU, hUf, G, bias)
+    gates, msg = g.zeros(n, 6 * H), g.zeros(n, 2 * H)
+    dG_ = g.devf(G)
+    g.call("cavs_treelstm_gates_fwd", g.P(g.devf(xW)), 4 * H, g.P(g.devf(hU)), g.P(g.devf(hUf)), g.P(dG_),
+           g.P(g.devf(bias)), g.P(gates), g.P(msg), n, H, g.stream())
+    close(g.host(gates), gates_w, "gates")
+    close(g.host(msg), msg_w, "msg")
+    # a round of leaves: children are zero
+    gates_l, msg_l = oracle.treelstm_gates_fwd(xW, 0 * hU, 0 * hUf, 0 * G, bias)
+    g.call("cavs_treelstm_gates_fwd", g.P(g.devf(xW)), 4 * H, None, None, None, g.P(g.devf(bias)),
+           g.P(gates), g.P(msg), n, H, g.stream())
+    close(g.host(gates), gates_l, "leaf gates")
+    close(g.host(msg), msg_l, "leaf msg")
+
+    dmsg = r.bulk_normal(n * 2 * H).reshape(n, 2 * H)
+    dret = r.bulk_normal(n * H).reshape(n, H)
+    dxW_w, dF_w, dG_w = oracle.treelstm_gates_bwd(dmsg, dret, gates_w, G)
+    dxW, dF, dG = g.zeros(n, 4 * H), g.zeros(2 * n, H), g.zeros(2 * n, 2 * H)
+    g.call("cavs_treelstm_gates_bwd", g.P(g.devf(dmsg)), g.P(g.devf(dret)), g.P(g.devf(gates_w)), g.P(dG_),
+           g.P(dxW), 4 * H, g.P(dF), g.P(dG), n, H, g.stream())
+    close(g.host(dxW), dxW_w, "dxW")
+    close(g.host(dF), dF_w, "dF")
+    close(g.host(dG), dG_w, "dG")
+    dxW_l, _, _ = oracle.treelstm_gates_bwd(dmsg, dret, gates_l, 0 * G)
+    g.call("cavs_treelstm_gates_bwd", g.P(g.devf(dmsg)), g.P(g.devf(dret)), g.P(g.devf(gates_l)), None,
+           g.P(dxW), 4 * H, None, None, n, H, g.stream())
+    close(g.host(dxW), dxW_l, "leaf dxW")
+
+
+@pytest.mark.parametrize("n,H", [(1, 4), (19, 128), (5, 6)])
+def test_lstm_and_treefc_gates(g, oracle, n, H):
+    r = rng(3 * n + H)
+    a = r.bulk_normal(n * 4 * H).reshape(n, 4 * H)
+    a2 = r.bulk_normal(n * 4 * H).reshape(n, 4 * H)
+    G = r.bulk_normal(n * 2 * H).reshape(n, 2 * H)
+    bias = r.bulk_normal(4 * H)
+    gates_w, msg_w = oracle.lstm_gates_fwd(a + a2, G, bias)
+    gates, msg = g.zeros(n, 5 * H), g.zeros(n, 2 * H)
+    g.call("cavs_lstm_gates_fwd", g.P(g.devf(a)), 4 * H, g.P(g.devf(a2)), g.P(g.devf(G)), g.P(g.devf(bias)),
+           g.P(gates), g.P(msg), n, H, g.stream())
+    close(g.host(gates), gates_w)
+    close(g.host(msg), msg_w)
+    gates_0, msg_0 = oracle.lstm_gates_fwd(a, 0 * G, bias)
+    g.call("cavs_lstm_gates_fwd", g.P(g.devf(a)), 4 * H, None, None, g.P(g.devf(bias)), g.P(gates), g.P(msg),
+           n, H, g.stream())
+    close(g.host(msg), msg_0)
+    dmsg, dret = r.bulk_normal(n * 2 * H).reshape(n, 2 * H), r.bulk_normal(n * H).reshape(n, H)
+    da_w, dG_w = oracle.lstm_gates_bwd(dmsg, dret, gates_w, G)
+    da, dG = g.zeros(n, 4 * H), g.zeros(n, 2 * H)
+    g.call("cavs_lstm_gates_bwd", g.P(g.devf(dmsg)), g.P(g.devf(dret)), g.P(g.devf(gates_w)), g.P(g.devf(G)),
+           g.P(da), 4 * H, g.P(dG), n, H, g.stream())
+    close(g.host(da), da_w)
+    close(g.host(dG), dG_w)
+
+    for act in (0, 1):
+        z, b, x = r.bulk_normal(n * H).reshape(n, H), r.bulk_normal(H), r.bulk_normal(n * H).reshape(n, H)
+        h = g.zeros(n, H)
+        g.call("cavs_treefc_fwd", g.P(g.devf(z)), g.P(g.devf(b)), g.P(g.devf(x)), g.P(h), n, H, act, g.stream())
+        hw = oracle.treefc_fwd(z, b, x, act)
+        close(g.host(h), hw)
+        g.call("cavs_treefc_fwd", None, g.P(g.devf(b)), g.P(g.devf(x)), g.P(h), n, H, act, g.stream())
+        close(g.host(h), oracle.treefc_fwd(0 * z, b, x, act))
+        d1, d2 = r.bulk_normal(n * H).reshape(n, H), r.bulk_normal(n * H).reshape(n, H)
+        dz = g.zeros(n, H)
+        g.call("cavs_treefc_bwd", g.P(g.devf(d1)), g.P(g.devf(d2)), g.P(g.devf(hw)), g.P(dz), n, H, act, g.stream())
+        close(g.host(dz), oracle.treefc_bwd(d1, d2, hw, act))
+
+
+# ---------------------------------------------------------------- the rest
+@pytest.mark.parametrize("n,w", [(1, 1), (50, 7), (2482, 2048), (5000, 100), (3, 4096)])
+def test_colsum(g, oracle, n, w):
+    r = rng(n + w)
+    X = r.bulk_normal(n * w).reshape(n, w)
+    exact = X.astype(np.float64).sum(0)
+    out = g.zeros(w, fill=float("nan"))
+    g.call("cavs_colsum", g.P(out), g.P(g.devf(X)), w, n, w, 0, g.stream())
+    close(g.host(out), exact, rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    acc0 = r.bulk_normal(w)
+    out = g.devf(acc0)
+    g.call("cavs_colsum", g.P(out), g.P(g.devf(X)), w, n, w, 1, g.stream())
+    close(g.host(out), exact + acc0, rtol=1e-4, atol=1e-5 * np.sqrt(n))
+
+
+@pytest.mark.parametrize("V,E,n", [(23, 6, 31), (21701, 300, 500), (1000, 128, 64)])
+def test_embedding(g, oracle, V, E, n):
+    r = rng(V + E)
+    table = r.bulk_normal(V * E).reshape(V, E)
+    ids = np.floor(r.bulk_uniform(n) * V).astype(np.float32)
+    ids[: n // 3] = ids[0]  # duplicates exercise the atomic accumulation
+    out = g.zeros(n, E)
+    g.call("cavs_embed_fwd", g.P(out), E, g.P(g.devf(ids)), g.P(g.devf(table)), n, E, g.stream())
+    np.testing.assert_array_equal(g.host(out), oracle.embed_fwd(ids, table))
+    dy = r.bulk_normal(n * E).reshape(n, E)
+    d0 = r.bulk_normal(V * E).reshape(V, E)
+    want = oracle.embed_bwd(d0.copy(), ids, dy)
+    dt = g.devf(d0)
+    g.call("cavs_embed_bwd", g.P(dt), g.P(g.devf(ids)), g.P(g.devf(dy)), E, n, E, g.stream())
+    close(g.host(dt), want, atol=1e-5 * np.sqrt(n))
+
+
+@pytest.mark.parametrize("n,C_", [(19, 5), (300, 1000), (1, 2), (64, 10000)])
+def test_softmax_xent_bias_sgd(g, oracle, n, C_):
+    r = rng(n + C_)
+    logits = 3 * r.bulk_normal(n * C_).reshape(n, C_)
+    labels = np.floor(r.bulk_uniform(n) * C_).astype(np.float32)
+    loss_w, d_w = oracle.softmax_xent(logits, labels)
+    loss, d = g.zeros(n), g.zeros(n, C_)
+    g.call("cavs_softmax_xent", g.P(loss), g.P(d), g.P(g.devf(logits)), g.P(g.devf(labels)), n, C_, g.stream())
+    close(g.host(loss), loss_w)
+    close(g.host(d), d_w, atol=1e-7)
+    bias = r.bulk_normal(C_)
+    out = g.zeros(n, C_)
+    g.call("cavs_bias_add_rows", g.P(out), g.P(g.devf(logits)), g.P(g.devf(bias)), n, C_, g.stream())
+    np.testing.assert_array_equal(g.host(out), logits + bias[None, :])
+    w = g.devf(logits)
+    g.call("cavs_sgd", g.P(w), g.P(g.devf(d_w)), 0.5, n * C_, g.stream())
+    np.testing.assert_array_equal(g.host(w), logits - np.float32(0.5) * d_w)
+
+
+def test_elementwise_family(g):
+    r = rng(3)
+    n, w = 37, 20
+    a, b = r.bulk_normal(n * w), r.bulk_normal(n * w)
+    row = r.bulk_normal(w)
+    sig = lambda x: 1.0 / (1.0 + np.exp(-x.astype(np.float64)))
+    cases = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b,
+             "sigmoid_grad": a * (b * (1 - b)), "tanh_grad": a * (1 - b * b),
+             "relu_grad": np.where(b > 0, a, 0), "equal": (a == b).astype(np.float32)}
+    for name, want in cases.items():
+        out = g.zeros(n * w)
+        g.call("cavs_ew_binary", hip.EW_BINARY[name], g.P(out), g.P(g.devf(a)), n * w, g.P(g.devf(b)), n * w,
+               n * w, 0, g.stream())
+        close(g.host(out), want, name)
+    out = g.zeros(n * w)  # row broadcast (bias add) and scalar
+    g.call("cavs_ew_binary", 0, g.P(out), g.P(g.devf(a)), n * w, g.P(g.devf(row)), w, n * w, 0, g.stream())
+    np.testing.assert_array_equal(g.host(out), (a.reshape(n, w) + row).ravel())
+    out = g.devf(a)  # accumulate form
+    g.call("cavs_ew_binary", 2, g.P(out), g.P(g.devf(a)), n * w, g.P(g.devf(row[:1])), 1, n * w, 1, g.stream())
+    close(g.host(out), a + a * row[0])
+    un = {"assign": a, "neg": -a, "abs": np.abs(a), "square": a * a, "sigmoid": sig(a), "tanh": np.tanh(a.astype(np.float64)),
+          "relu": np.maximum(a, 0)}
+    for name, want in un.items():
+        out = g.zeros(n * w)
+        g.call("cavs_ew_unary", hip.EW_UNARY[name], g.P(out), g.P(g.devf(a)), n * w, 0, g.stream())
+        close(g.host(out), want, name)
+    out = g.zeros(n * w)
+    g.call("cavs_scale", g.P(out), g.P(g.devf(a)), 0.25, n * w, g.stream())
+    np.testing.assert_array_equal(g.host(out), np.float32(0.25) * a)
+    with pytest.raises(hip.CavsError, match="unknown op"):
+        hip.call("cavs_ew_unary", 99, g.P(out), g.P(out), 4, 0, g.stream())
+
+
+def test_fill_zero_and_copies(g):
+    import torch
+
+    t = torch.full((1003,), 5.0, device="cuda")
+    g.call("cavs_zero", g.P(t) + 4, 4 * 1001, g.stream())  # unaligned start
+    want = np.zeros(1003, np.float32)
+    want[0] = want[-1] = 5
+    np.testing.assert_array_equal(g.host(t), want)
+    g.call("cavs_fill", g.P(t), 2.5, 1003, g.stream())
+    assert (g.host(t) == 2.5).all()
+    src = np.arange(100, dtype=np.float32)
+    d = g.zeros(100)
+    g.call("cavs_memcpy_h2d", g.P(d), src.ctypes.data, 400, g.stream())
+    back = np.zeros(100, np.float32)
+    g.call("cavs_memcpy_d2h", back.ctypes.data, g.P(d), 400, g.stream())
+    g.call("cavs_stream_sync", g.stream())
+    np.testing.assert_array_equal(back, src)
+
+
+def test_fused_kernel_interface(g):
+    """The two fused groups of the reference's fusion smoke test
+    (cavs/frontend/cxx/fusion_session_test.cc): E = C + (A + B) and YY = (X + Y) + Z,
+    in the generator's dialect (idx % count reads, atomicAdd for narrower outputs)."""
+    src = r'''
+extern "C" __global__ void FusedKernel_0(float *E, const float *A, const float *B, const float *C,
+    const int E_count, const int A_count, const int B_count, const int C_count, const int n_elements)
+{
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < n_elements) {
+    float tmp_A = A[idx%A_count];
+    float tmp_B = B[idx%B_count];
+    float tmp_C = C[idx%C_count];
+    float tmp_D = tmp_A + tmp_B;
+    float tmp_E = tmp_C + tmp_D;
+    if (E_count < n_elements) {
+      float ori_E = E[idx%E_count];
+      atomicAdd(&E[idx%E_count], (tmp_E - ori_E));
+    } else {
+      E[idx%E_count] = tmp_E;
+    }
+  }
+}'''
+    h = C.c_void_p()
+    hip.call("cavs_fused_compile", b"FusedKernel_0", src.encode(), C.byref(h))
+    A = np.array([1, 2, 3, 4, 5, 6], np.float32)
+    B = np.array([6, 5, 4, 3, 2, 1], np.float32)
+    Cc = np.array([0.1, 0.2, 0.3, 0.4, 0.5, 0.6], np.float32)
+    out = g.zeros(6)
+    dA, dB, dC = g.devf(A), g.devf(B), g.devf(Cc)
+    outs = (C.c_void_p * 1)(g.P(out))
+    ins = (C.c_void_p * 3)(g.P(dA), g.P(dB), g.P(dC))
+    oc = (C.c_int * 1)(6)
+    ic = (C.c_int * 3)(6, 6, 6)
+    hip.call("cavs_fused_launch", h, outs, 1, ins, 3, oc, ic, 6, g.stream())
+    np.testing.assert_allclose(g.host(out), [7.1, 7.2, 7.3, 7.4, 7.5, 7.6], rtol=1e-6)
+    hip.call("cavs_fused_release", h)
+    bad = C.c_void_p()
+    with pytest.raises(hip.CavsError, match="compile"):
+        hip.call("cavs_fused_compile", b"k", b"this is not a kernel", C.byref(bad))
+
+
+@pytest.mark.parametrize("kind,seed,B,lo,hi", [("tree", 1, 1, 2, 2), ("tree", 2, 7, 2, 30), ("tree", 3, 64, 2, 56),
+                                               ("chain", 4, 9, 2, 40), ("tree", 5, 40, 32, 256)])
+def test_device_frontier_matches_host_schedule_bit_exact(g, oracle, kind, seed, B, lo, hi):
+    import torch
+
+    graph = (synth.tree_batch if kind == "tree" else synth.chain_batch)(seed, B, lo, hi)[0]
+    tr = oracle.sched_trace(graph)
+    N = tr["N"]
+    parent, off = [], 0
+    for row in graph:
+        n = int(np.argmax(row == -1)) + 1
+        parent += [off + int(p) if p >= 0 else -1 for p in row[:n]]
+        off += n
+    I = lambda k: torch.full((k,), -7, dtype=torch.int32, device="cuda")
+    t2j, j2t, rot, r2o, nr, scratch = I(N), I(N), I(N), I(N + 2), I(1), I(4 * N)
+    g.call("cavs_schedule_frontier", g.P(g.devi(parent)), N, g.P(t2j), g.P(j2t), g.P(rot), g.P(r2o), g.P(nr),
+           g.P(scratch), g.stream())
+    R = int(g.host(nr)[0])
+    assert R == len(tr["fwd"])
+    assert g.host(r2o)[: R + 1].tolist() == tr["round2offset"]
+    assert g.host(t2j).tolist() == tr["tids_to_jobids"]
+    inv = np.empty(N, np.int64)
+    inv[np.array(tr["tids_to_jobids"])] = np.arange(N)
+    assert g.host(j2t).tolist() == inv.tolist()
+    want_round = np.concatenate([[r] * len(rd["exec"]) for r, rd in enumerate(tr["fwd"])])
+    assert g.host(rot).tolist() == want_round.tolist()
