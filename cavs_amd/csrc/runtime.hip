@@ -186,6 +186,12 @@ int cavs_event_record(void *event, void *stream) {
   return CAVS_OK;
 }
 
+int cavs_event_sync(void *event) {
+  CAVS_REQUIRE(event, "cavs_event_sync: null event");
+  CAVS_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));
+  return CAVS_OK;
+}
+
 int cavs_event_elapsed_ms(float *ms, void *start, void *stop) {
   CAVS_REQUIRE(ms && start && stop, "cavs_event_elapsed_ms: null argument");
   CAVS_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));

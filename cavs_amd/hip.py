@@ -41,6 +41,7 @@ _SIGS = {
     "cavs_event_create": [C.POINTER(_P)],
     "cavs_event_destroy": [_P],
     "cavs_event_record": [_P, _P],
+    "cavs_event_sync": [_P],
     "cavs_event_elapsed_ms": [C.POINTER(_F), _P, _P],
     "cavs_gather_rows": [_P, _I, _P, _I, _P, _I, _I, _P],
     "cavs_scatter_rows": [_P, _I, _P, _P, _I, _I, _I, _P],

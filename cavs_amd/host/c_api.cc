@@ -1,0 +1,129 @@
+// extern "C" surface of the host runtime (cavs_session.h): exceptions end here.
+#include <cstdio>
+#include <cstring>
+#include <string>
+
+#include "cavs_session.h"
+#include "engine.h"
+
+struct cavs_session {
+  cavs::Engine engine;
+  explicit cavs_session(const cavs_session_config &c) : engine(c) {}
+};
+
+namespace {
+thread_local std::string g_error;
+
+template <typename F>
+int guarded(F &&f) {
+  try {
+    f();
+    return CAVS_OK;
+  } catch (const cavs::Error &e) {
+    g_error = e.what();
+    return e.code;
+  } catch (const std::bad_alloc &) {
+    g_error = "host allocation failed";
+    return CAVS_ENOMEM;
+  } catch (const std::exception &e) {
+    g_error = e.what();
+    return CAVS_EINVAL;
+  }
+}
+
+int need(const void *p, const char *what) {
+  if (p) return CAVS_OK;
+  g_error = std::string("null ") + what;
+  return CAVS_EINVAL;
+}
+
+int emit(const std::vector<int> &t, int *out, int cap) {
+  if ((int)t.size() > cap || !out) return -(int)t.size();
+  std::memcpy(out, t.data(), sizeof(int) * t.size());
+  return (int)t.size();
+}
+}  // namespace
+
+extern "C" {
+
+const char *cavs_session_error(void) { return g_error.c_str(); }
+
+int cavs_session_create(const cavs_session_config *cfg, cavs_session **out) {
+  if (int rc = need(cfg, "config")) return rc;
+  if (int rc = need(out, "out pointer")) return rc;
+  *out = nullptr;
+  return guarded([&] { *out = new cavs_session(*cfg); });
+}
+
+int cavs_session_destroy(cavs_session *s) {
+  return guarded([&] { delete s; });
+}
+
+int cavs_session_set_param(cavs_session *s, const char *name, const float *host, size_t n) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(name, "parameter name")) return rc;
+  return guarded([&] { s->engine.set_param(name, host, n); });
+}
+
+int cavs_session_get_param(cavs_session *s, const char *name, float *host, size_t n) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(name, "parameter name")) return rc;
+  return guarded([&] { s->engine.get_param(name, host, n, false); });
+}
+
+int cavs_session_get_grad(cavs_session *s, const char *name, float *host, size_t n) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(name, "parameter name")) return rc;
+  return guarded([&] { s->engine.get_param(name, host, n, true); });
+}
+
+int cavs_session_step(cavs_session *s, const int *graph, int B, int maxlen, const void *x,
+                      const void *labels, int inputs_on_device, int backward, float lr) {
+  if (int rc = need(s, "session")) return rc;
+  return guarded([&] { s->engine.step(graph, B, maxlen, x, labels, inputs_on_device != 0, backward != 0, lr); });
+}
+
+int cavs_session_sync(cavs_session *s) {
+  if (int rc = need(s, "session")) return rc;
+  return guarded([&] { s->engine.sync(); });
+}
+
+int cavs_session_fetch(cavs_session *s, const char *what, float *host, size_t n) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(what, "result name")) return rc;
+  return guarded([&] { s->engine.fetch(what, host, n); });
+}
+
+int cavs_session_total_length(cavs_session *s) { return s ? s->engine.total_length() : CAVS_EINVAL; }
+
+int cavs_session_schedule_trace(cavs_session *s, int *out, int cap) {
+  if (!s) return 0;
+  return emit(s->engine.schedule().trace(true), out, cap);
+}
+
+int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int with_backward, int *out,
+                        int cap) {
+  cavs::Schedule sch;
+  std::string err = cavs::build_schedule(graph, B, maxlen, batching != 0, &sch);
+  if (!err.empty()) {
+    g_error = err;
+    return 0;
+  }
+  return emit(sch.trace(with_backward != 0), out, cap);
+}
+
+int cavs_session_timing(cavs_session *s, const char *name, float *ms) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(ms, "output")) return rc;
+  return guarded([&] { *ms = s->engine.timing(name ? name : ""); });
+}
+
+void *cavs_session_stream(cavs_session *s) { return s ? s->engine.stream() : nullptr; }
+
+int cavs_session_counter(cavs_session *s, const char *key, double *value) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(value, "output")) return rc;
+  return guarded([&] { *value = s->engine.counter(key ? key : ""); });
+}
+
+}  // extern "C"

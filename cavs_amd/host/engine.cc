@@ -1,0 +1,619 @@
+#include "engine.h"
+
+#include <algorithm>
+#include <chrono>
+#include <cstring>
+
+namespace cavs {
+
+namespace {
+inline size_t grow(size_t need, size_t have) {
+  if (need <= have) return have;
+  size_t g = have + have / 4;
+  return std::max(need, g);
+}
+}  // namespace
+
+Engine::Engine(const cavs_session_config &cfg) : cfg_(cfg) {
+  if (cfg.model < 0 || cfg.model > 2) fail(CAVS_EINVAL, "unknown model " + std::to_string(cfg.model));
+  if (cfg.loss < 0 || cfg.loss > 2) fail(CAVS_EINVAL, "unknown loss " + std::to_string(cfg.loss));
+  if (cfg.pairing < 0 || cfg.pairing > 1) fail(CAVS_EINVAL, "unknown pairing");
+  if (cfg.H <= 0) fail(CAVS_EINVAL, "hidden size must be positive");
+  const size_t H = cfg.H;
+  E_ = cfg.model == CAVS_MODEL_LSTM ? cfg.H : cfg.E;  // the chain LSTM requires E == H
+  mw_ = cfg.model == CAVS_MODEL_TREEFC ? cfg.H : 2 * cfg.H;
+  nch_ = cfg.model == CAVS_MODEL_LSTM ? 1 : 2;
+  if (cfg.model != CAVS_MODEL_TREEFC && (cfg.V <= 0 || E_ <= 0))
+    fail(CAVS_EINVAL, "vocabulary and embedding sizes must be positive");
+  if (cfg.loss == CAVS_LOSS_SOFTMAX && cfg.C <= 0) fail(CAVS_EINVAL, "class count must be positive");
+  check(cavs_init(cfg.device));
+  check(cavs_stream_create(&stream_));
+  for (auto &e : ev_) check(cavs_event_create(&e));
+  for (auto &e : idx_copied_) check(cavs_event_create(&e));
+  switch (cfg.model) {
+    case CAVS_MODEL_TREELSTM:
+      add_param("Emb", (size_t)cfg.V * E_);
+      add_param("W", (size_t)E_ * 4 * H);
+      add_param("U", 4 * H * H);
+      add_param("Bv", 4 * H);
+      break;
+    case CAVS_MODEL_LSTM:
+      add_param("Emb", (size_t)cfg.V * H);
+      add_param("W", 8 * H * H);
+      add_param("Bv", 4 * H);
+      break;
+    default:
+      add_param("W", 2 * H * H);
+      if (cfg.use_bias) add_param("Bv", H);
+  }
+  if (cfg.loss == CAVS_LOSS_SOFTMAX) {
+    add_param("Wfc", (size_t)cfg.C * H);
+    add_param("bfc", cfg.C);
+  }
+}
+
+Engine::~Engine() {
+  cavs_stream_sync(stream_);
+  for (auto &e : ev_) cavs_event_destroy(e);
+  for (auto &e : idx_copied_) cavs_event_destroy(e);
+  cavs_stream_destroy(stream_);
+}
+
+void Engine::add_param(const std::string &name, size_t n) {
+  auto p = std::make_unique<Param>();
+  p->n = n;
+  p->w.reserve(n);
+  p->g.reserve(n);
+  check(cavs_zero(p->w.get(), n * 4, stream_));
+  check(cavs_zero(p->g.get(), n * 4, stream_));
+  params_[name] = std::move(p);
+}
+
+Param &Engine::param(const std::string &name) {
+  auto it = params_.find(name);
+  if (it == params_.end()) fail(CAVS_EINVAL, "this model has no parameter named '" + name + "'");
+  return *it->second;
+}
+
+void Engine::set_param(const std::string &name, const float *host, size_t n) {
+  Param &p = param(name);
+  if (n != p.n || !host)
+    fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
+  check(cavs_memcpy_h2d(p.w.get(), host, n * 4, stream_));
+  check(cavs_stream_sync(stream_));
+}
+
+void Engine::get_param(const std::string &name, float *host, size_t n, bool grad) {
+  Param &p = param(name);
+  if (n != p.n || !host)
+    fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
+  check(cavs_memcpy_d2h(host, grad ? p.g.get() : p.w.get(), n * 4, stream_));
+  check(cavs_stream_sync(stream_));
+}
+
+// ------------------------------------------------------------------ counted wrappers
+void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
+                  int ldb, float beta, float *C, int ldc) {
+  check(cavs_sgemm(tA, tB, M, N, K, 1.f, A, lda, B, ldb, beta, C, ldc, stream_));
+  c_gemm_flops_ += 2.0 * M * N * K;
+  c_launches_ += 1;
+}
+
+void Engine::gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda,
+                         const float *B, int ldb, float *C, int ldc) {
+  size_t need = cavs_sgemm_splitk_workspace(M, N, K);
+  if (ws_.capacity() * 4 < need) {
+    // the workspace may still be in use by an enqueued GEMM
+    check(cavs_stream_sync(stream_));
+    ws_.reserve(need / 4 + 1);
+  }
+  check(cavs_sgemm_splitk(tA, tB, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, ws_.get(),
+                          ws_.capacity() * 4, stream_));
+  c_gemm_flops_ += 2.0 * M * N * K;
+  c_launches_ += need ? 2 : 1;
+}
+
+void Engine::gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n,
+                    int w) {
+  check(cavs_gather_rows(out, ld_out, src, ld_src, ids, n, w, stream_));
+  c_gather_rows_ += n;
+  c_gather_bytes_ += (8.0 * w + 4.0) * n;
+  c_launches_ += 1;
+}
+
+void Engine::scatter(float *dst, int ld_dst, const int *ids, const float *inp, int ld_inp, int n,
+                     int w) {
+  check(cavs_scatter_rows(dst, ld_dst, ids, inp, ld_inp, n, w, stream_));
+  c_scatter_rows_ += n;
+  c_scatter_bytes_ += (8.0 * w + 4.0) * n;
+  c_launches_ += 1;
+}
+
+// Growing a buffer frees the old storage, which enqueued kernels may still read.
+void Engine::ensure(DeviceArray<float> &a, size_t n) {
+  if (n <= a.capacity()) return;
+  check(cavs_stream_sync(stream_));
+  a.reserve(n);
+}
+
+// ------------------------------------------------------------------ memory manager
+// Every edge of F is a [rows, width] buffer in which round r lives at rows
+// [offset_r, offset_r + n_r): row index == tensor id for every edge, and forward
+// activations persist for the backward pass (cavs/midend/op_context.cc:13-40,
+// cavs/midend/tensor.cc:311-321).  The reference sizes each edge for MAX_NODE = B*maxlen
+// rows (cavs/frontend/cxx/graphsupport.cc:34-35); here rows follow the batch's actual
+// total length, and the edges that live for one round only are sized by the widest round.
+void Engine::reserve_edges() {
+  const size_t H = cfg_.H, N = N_;
+  if ((size_t)cap_ < N) cap_ = (int)grow(N, cap_);
+  if (rcap_ < sched_.max_round) rcap_ = (int)grow(sched_.max_round, rcap_);
+  const size_t cap = cap_, rc = rcap_, mw = mw_;
+  auto R = [&](DeviceArray<float> &a, size_t n) { ensure(a, n); };
+  R(msg_, cap * mw);
+  R(pool_, cap * mw);
+  R(dpool_, cap * mw);
+  R(GO_, cap * H);
+  R(dGO_, cap * H);
+  R(dret_, cap * H);
+  R(G_, cap * nch_ * mw);
+  R(r_dmsg_, rc * mw);
+  R(r_dG_, rc * nch_ * mw);
+  if (cfg_.model != CAVS_MODEL_TREEFC) {
+    R(xs_, cap);
+    R(e_, cap * E_);
+    R(de_, cap * E_);
+    R(xW_, cap * 4 * H);
+    R(dxW_, cap * 4 * H);
+    R(gates_, cap * 6 * H);
+  } else {
+    if (cfg_.use_x) R(xs_, cap * H);
+    R(dxW_, cap * H);
+    R(r_z_, rc * H);
+  }
+  if (cfg_.model == CAVS_MODEL_TREELSTM) {
+    R(hlr_, cap * H);
+    R(dF_, cap * 2 * H);
+    R(r_hU_, rc * 3 * H);
+    R(r_hUf_, rc * 2 * H);
+    R(r_dhlr_, rc * H);
+  }
+  if (cfg_.loss == CAVS_LOSS_SOFTMAX) {
+    R(logits_, cap * cfg_.C);
+    R(dlogits_, cap * cfg_.C);
+    R(loss_, cap);
+  } else {
+    R(loss_, std::max<size_t>(cap, 2 * H + 2));
+    R(logits_, (size_t)sched_.B * H + 1);   // root rows / |h| scratch
+    R(dlogits_, std::max<size_t>((size_t)sched_.B * H, cap * H));
+  }
+}
+
+// One upload per step (the reference copies a list from pageable memory before every
+// Gather / Scatter / Pull, cavs/backend/op_impl_graphop.cu:68,149,241,308):
+//   t2j   [N]      tensor id -> global vertex id (Pull, FunctionPopRet)
+//   pair  [N]      per slab row: pool row the forward Scatter writes and the backward
+//                  Gather reads, or -1 (root, or past the end of the compacted list)
+//   child [nch*N]  per slab row and child: pool row the forward Gather reads and the
+//                  backward Scatter writes
+//   roots [B]      vertex ids of the roots (sum-of-squares loss)
+void Engine::upload_index_arena() {
+  const Schedule &s = sched_;
+  const int N = N_;
+  const size_t total = (size_t)N * (2 + nch_) + s.B;
+  // two pinned staging buffers alternate, so the host can build the lists of the next
+  // step while the device still runs this one; a buffer is rewritten only after the
+  // upload that last read it has finished
+  const int slot = idx_slot_;
+  idx_slot_ ^= 1;
+  if (idx_pending_[slot]) check(cavs_event_sync(idx_copied_[slot]));
+  idx_pending_[slot] = false;
+  idx_host_[slot].reserve(total);
+  if (idx_dev_.capacity() < total) {
+    check(cavs_stream_sync(stream_));
+    idx_dev_.reserve(grow(total, idx_dev_.capacity()));
+  }
+  int *t2j = idx_host_[slot].get(), *pair = t2j + N, *child = pair + N, *roots = child + (size_t)nch_ * N;
+  std::memcpy(t2j, s.tids_to_jobids.data(), sizeof(int) * N);
+  std::fill(pair, pair + N, -1);
+  std::fill(child, child + (size_t)nch_ * N, -1);
+  for (const Round &r : s.rounds) {
+    const int m = r.scatter_end - r.scatter_begin;
+    if (cfg_.pairing == CAVS_PAIR_REFERENCE) {
+      // b-th list entry <-> b-th slab row (op_impl_graphop.cu:148-157)
+      for (int b = 0; b < m; b++) pair[r.offset + b] = s.scatter_ids[r.scatter_begin + b];
+    } else {
+      for (int b = 0; b < m; b++) pair[s.scatter_ids[r.scatter_begin + b]] = s.scatter_ids[r.scatter_begin + b];
+    }
+    if (leaf_round(r)) continue;
+    for (int c = 0; c < nch_; c++) {
+      const int len = r.gather_end[c] - r.gather_begin[c];
+      if (len != r.n)
+        fail(CAVS_EUNSUPPORTED, "round at tensor id " + std::to_string(r.offset) + " mixes vertices with and without child " +
+                                    std::to_string(c) + " (the reference's gather lists misalign there too)");
+      for (int b = 0; b < len; b++) child[(size_t)nch_ * (r.offset + b) + c] = s.gather_ids[c][r.gather_begin[c] + b];
+    }
+    if (nch_ == 1 && r.gather_end[1] != r.gather_begin[1])
+      fail(CAVS_EUNSUPPORTED, "a chain vertex function got a vertex with two children");
+  }
+  int nr = 0;
+  for (int v = 0; v < N; v++)
+    if (s.parent[v] < 0) roots[nr++] = v;
+  check(cavs_memcpy_h2d(idx_dev_.get(), idx_host_[slot].get(), total * sizeof(int), stream_));
+  check(cavs_event_record(idx_copied_[slot], stream_));
+  idx_pending_[slot] = true;
+  d_t2j_ = idx_dev_.get();
+  d_pair_ = d_t2j_ + N;
+  d_child_ = d_pair_ + N;
+  d_roots_ = d_child_ + (size_t)nch_ * N;
+}
+
+// ------------------------------------------------------------------ step
+void Engine::step(const int *graph, int B, int maxlen, const void *x, const void *labels,
+                  bool on_device, bool backward, float lr) {
+  auto t0 = std::chrono::steady_clock::now();
+  std::string err = build_schedule(graph, B, maxlen, (cfg_.opt & CAVS_OPT_BATCHING) != 0, &sched_);
+  if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
+  if (sched_.executed != sched_.N)
+    fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample; the reference never executes such a vertex "
+                            "(graph_scheduler.cc:180) and leaves its rows undefined");
+  N_ = sched_.N;
+  const int N = N_, H = cfg_.H;
+  c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
+  reserve_edges();
+  upload_index_arena();
+  parse_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+
+  const bool needs_x = cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x;
+  const size_t xw = cfg_.model == CAVS_MODEL_TREEFC ? H : 1;
+  if (needs_x && !x) fail(CAVS_EINVAL, "vertex input feed is null");
+  if (cfg_.loss == CAVS_LOSS_SOFTMAX && !labels) fail(CAVS_EINVAL, "label feed is null");
+  if (on_device) {
+    d_x_ = static_cast<const float *>(x);
+    d_labels_ = static_cast<const float *>(labels);
+  } else {
+    if (needs_x) {
+      ensure(x_in_, grow((size_t)N * xw, x_in_.capacity()));
+      check(cavs_memcpy_h2d(x_in_.get(), x, (size_t)N * xw * 4, stream_));
+      d_x_ = x_in_.get();
+    }
+    if (cfg_.loss == CAVS_LOSS_SOFTMAX) {
+      ensure(labels_in_, grow(N, labels_in_.capacity()));
+      check(cavs_memcpy_h2d(labels_in_.get(), labels, (size_t)N * 4, stream_));
+      d_labels_ = labels_in_.get();
+    }
+    // pageable sources: make sure the copies are done before the caller reuses them
+    check(cavs_stream_sync(stream_));
+  }
+
+  check(cavs_event_record(ev_[0], stream_));
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
+    case CAVS_MODEL_LSTM: lstm_forward(); break;
+    default: treefc_forward();
+  }
+  pop_ret();
+  check(cavs_event_record(ev_[1], stream_));
+  ev_valid_ = true;
+  head_forward_backward(backward);
+  did_backward_ = backward;
+  ev_bwd_valid_ = false;
+  if (backward) {
+    check(cavs_event_record(ev_[2], stream_));
+    switch (cfg_.model) {
+      case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
+      case CAVS_MODEL_LSTM: lstm_backward(); break;
+      default: treefc_backward();
+    }
+    check(cavs_event_record(ev_[3], stream_));
+    ev_bwd_valid_ = true;
+    if (lr != 0.f)
+      for (auto &kv : params_) {
+        check(cavs_sgd(kv.second->w.get(), kv.second->g.get(), lr, kv.second->n, stream_));
+        c_launches_ += 1;
+      }
+  }
+}
+
+// FunctionPopRet (cavs/backend/op_impl_graphop.cu:304-318): GraphOutput[tids_to_jobids[t]] =
+// ret[t].  Push's slab copy is folded in: the h half of the message slab is the return value.
+void Engine::pop_ret() { scatter(GO_.get(), cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H); }
+
+// ------------------------------------------------------------------ Tree-LSTM
+// apps/paper/tree-lstm-cavs.cc:129-172.  Everything that does not depend on the children
+// (Pull, EmbeddingLookup, x*W) is hoisted out of the round loop and done once for all N
+// vertices in tensor-id order; rounds of leaves skip the child GEMMs because their
+// gathered rows are zero.
+void Engine::treelstm_forward() {
+  const int N = N_, H = cfg_.H, E = E_;
+  const float *W = param("W").w.get(), *U = param("U").w.get(), *Bv = param("Bv").w.get();
+  gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
+  check(cavs_embed_fwd(e_.get(), E, xs_.get(), param("Emb").w.get(), N, E, stream_));
+  c_launches_ += 1;
+  gemm(0, 0, N, 4 * H, E, e_.get(), E, W, 4 * H, 0.f, xW_.get(), 4 * H);
+  if (!sched_.batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
+    check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
+    check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
+  }
+  for (const Round &r : sched_.rounds) {
+    const size_t off = r.offset;
+    float *msg = msg_.at(off * 2 * H);
+    if (leaf_round(r)) {
+      check(cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, nullptr, nullptr, nullptr, Bv,
+                                    gates_.at(off * 6 * H), msg, r.n, H, stream_));
+    } else {
+      float *G = G_.at(2 * off * 2 * H), *hlr = hlr_.at(off * H);
+      check(cavs_gather_children(G, hlr, pool_.get(), d_child_ + 2 * off, r.n, 2 * H, H, stream_));
+      c_gather_rows_ += 2.0 * r.n;
+      c_gather_bytes_ += 2.0 * r.n * (16.0 * H + 4) + 4.0 * r.n * H;
+      c_launches_ += 1;
+      gemm(0, 0, r.n, 3 * H, H, hlr, H, U, 3 * H, 0.f, r_hU_.get(), 3 * H);
+      gemm(0, 0, 2 * r.n, H, H, G, 2 * H, U + (size_t)3 * H * H, H, 0.f, r_hUf_.get(), H);
+      check(cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, r_hU_.get(), r_hUf_.get(), G, Bv,
+                                    gates_.at(off * 6 * H), msg, r.n, H, stream_));
+    }
+    c_launches_ += 1;
+    scatter(pool_.get(), 2 * H, d_pair_ + off, msg, 2 * H, r.n, 2 * H);
+  }
+}
+
+void Engine::treelstm_backward() {
+  const int N = N_, H = cfg_.H, E = E_;
+  const float *W = param("W").w.get(), *U = param("U").w.get();
+  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);  // grad of Push is Pull
+  if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
+  for (int k : sched_.bwd_rounds) {
+    const Round &r = sched_.rounds[k];
+    const size_t off = r.offset;
+    // grad of Scatter is Gather on the recorded scatter list; rows without an entry read zero
+    gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
+    if (leaf_round(r)) {
+      check(cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H), nullptr,
+                                    dxW_.at(off * 4 * H), 4 * H, nullptr, nullptr, r.n, H, stream_));
+      c_launches_ += 1;
+      continue;
+    }
+    float *dxW = dxW_.at(off * 4 * H), *dF = dF_.at(2 * off * H);
+    check(cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H),
+                                  G_.at(2 * off * 2 * H), dxW, 4 * H, dF, r_dG_.get(), r.n, H, stream_));
+    c_launches_ += 1;
+    // dh_lr = [d_i|d_o|d_u] * U_iou^T ;  dh_{l,r} = dh_lr + d_f{l,r} * U_f^T
+    gemm(0, 1, r.n, H, 3 * H, dxW, 4 * H, U, 3 * H, 0.f, r_dhlr_.get(), H);
+    check(cavs_sgemm_addrows(0, 1, 2 * r.n, H, H, dF, H, U + (size_t)3 * H * H, H, r_dhlr_.get(), H, 1,
+                             r_dG_.get(), 2 * H, stream_));
+    c_gemm_flops_ += 2.0 * 2 * r.n * H * H;
+    c_launches_ += 1;
+    // grad of Gather(child) is Scatter on the recorded gather lists
+    scatter(dpool_.get(), 2 * H, d_child_ + 2 * off, r_dG_.get(), 2 * H, 2 * r.n, 2 * H);
+  }
+  // weight gradients once over all rows (OPT_BATCHING semantics; without it the reference
+  // accumulates the same sums round by round)
+  const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
+  gemm(0, 1, N, E, 4 * H, dxW_.get(), 4 * H, W, 4 * H, 0.f, de_.get(), E);
+  Param &emb = param("Emb");
+  check(cavs_zero(emb.g.get(), emb.n * 4, stream_));
+  check(cavs_embed_bwd(emb.g.get(), xs_.get(), de_.get(), E, N, E, stream_));
+  c_launches_ += 2;
+  gemm_splitk(1, 0, E, 4 * H, N, e_.get(), E, dxW_.get(), 4 * H, param("W").g.get(), 4 * H);
+  float *dU = param("U").g.get();
+  gemm_splitk(1, 0, H, 3 * H, N - lp, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H);
+  gemm_splitk(1, 0, H, H, 2 * (N - lp), G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
+              dU + (size_t)3 * H * H, H);
+  // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
+  float *dB = param("Bv").g.get();
+  const int src_block[4] = {0, 3, 2, 1};
+  for (int k = 0; k < 4; k++)
+    check(cavs_colsum(dB + (size_t)k * H, dxW_.get() + (size_t)src_block[k] * H, 4 * H, N, H, 0, stream_));
+  c_launches_ += 4;
+}
+
+// ------------------------------------------------------------------ chain LSTM
+// apps/paper/seq-lstm-cavs.cc:62-86
+void Engine::lstm_forward() {
+  const int N = N_, H = cfg_.H;
+  const float *Wx = param("W").w.get(), *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w.get();
+  gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
+  check(cavs_embed_fwd(e_.get(), H, xs_.get(), param("Emb").w.get(), N, H, stream_));
+  c_launches_ += 1;
+  gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
+  if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  for (const Round &r : sched_.rounds) {
+    const size_t off = r.offset;
+    float *a = xW_.at(off * 4 * H), *msg = msg_.at(off * 2 * H), *G = nullptr;
+    if (!leaf_round(r)) {
+      G = G_.at(off * 2 * H);
+      gather(G, 2 * H, pool_.get(), 2 * H, d_child_ + off, r.n, 2 * H);
+      gemm(0, 0, r.n, 4 * H, H, G, 2 * H, Wh, 4 * H, 1.f, a, 4 * H);  // a += h_p * W'
+    }
+    check(cavs_lstm_gates_fwd(a, 4 * H, nullptr, G, Bv, gates_.at(off * 5 * H), msg, r.n, H, stream_));
+    c_launches_ += 1;
+    scatter(pool_.get(), 2 * H, d_pair_ + off, msg, 2 * H, r.n, 2 * H);
+  }
+}
+
+void Engine::lstm_backward() {
+  const int N = N_, H = cfg_.H;
+  const float *Wx = param("W").w.get(), *Wh = Wx + (size_t)4 * H * H;
+  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);
+  for (int k : sched_.bwd_rounds) {
+    const Round &r = sched_.rounds[k];
+    const size_t off = r.offset;
+    gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
+    float *da = dxW_.at(off * 4 * H);
+    if (leaf_round(r)) {
+      check(cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), nullptr, da, 4 * H,
+                                nullptr, r.n, H, stream_));
+      c_launches_ += 1;
+      continue;
+    }
+    check(cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), G_.at(off * 2 * H), da,
+                              4 * H, r_dG_.get(), r.n, H, stream_));
+    c_launches_ += 1;
+    gemm(0, 1, r.n, H, 4 * H, da, 4 * H, Wh, 4 * H, 0.f, r_dG_.get(), 2 * H);  // dh_p = da * W'^T
+    scatter(dpool_.get(), 2 * H, d_child_ + off, r_dG_.get(), 2 * H, r.n, 2 * H);
+  }
+  const int lp = sched_.leaf_prefix;
+  gemm(0, 1, N, H, 4 * H, dxW_.get(), 4 * H, Wx, 4 * H, 0.f, de_.get(), H);
+  Param &emb = param("Emb");
+  check(cavs_zero(emb.g.get(), emb.n * 4, stream_));
+  check(cavs_embed_bwd(emb.g.get(), xs_.get(), de_.get(), H, N, H, stream_));
+  c_launches_ += 2;
+  float *dW = param("W").g.get();
+  gemm_splitk(1, 0, H, 4 * H, N, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H);
+  gemm_splitk(1, 0, H, 4 * H, N - lp, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
+              dW + (size_t)4 * H * H, 4 * H);
+  check(cavs_colsum(param("Bv").g.get(), dxW_.get(), 4 * H, N, 4 * H, 0, stream_));
+  c_launches_ += 1;
+}
+
+// ------------------------------------------------------------------ Tree-FC
+// apps/paper/tree-fc-cavs.cc:28-36 (optionally with a bias and a Pull'ed input row)
+void Engine::treefc_forward() {
+  const int N = N_, H = cfg_.H;
+  const float *W = param("W").w.get();
+  const float *Bv = cfg_.use_bias ? param("Bv").w.get() : nullptr;
+  if (cfg_.use_x) gather(xs_.get(), H, d_x_, H, d_t2j_, N, H);
+  if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  for (const Round &r : sched_.rounds) {
+    const size_t off = r.offset;
+    const float *xin = cfg_.use_x ? xs_.at(off * H) : nullptr;
+    float *msg = msg_.at(off * H);
+    if (leaf_round(r)) {
+      check(cavs_treefc_fwd(nullptr, Bv, xin, msg, r.n, H, cfg_.act, stream_));
+    } else {
+      float *G = G_.at(2 * off * H);  // row b = [G0 | G1] of vertex b
+      check(cavs_gather_children(G, nullptr, pool_.get(), d_child_ + 2 * off, r.n, H, 0, stream_));
+      c_gather_rows_ += 2.0 * r.n;
+      c_gather_bytes_ += 2.0 * r.n * (8.0 * H + 4);
+      c_launches_ += 1;
+      gemm(0, 0, r.n, H, 2 * H, G, 2 * H, W, H, 0.f, r_z_.get(), H);
+      check(cavs_treefc_fwd(r_z_.get(), Bv, xin, msg, r.n, H, cfg_.act, stream_));
+    }
+    c_launches_ += 1;
+    scatter(pool_.get(), H, d_pair_ + off, msg, H, r.n, H);
+  }
+}
+
+void Engine::treefc_backward() {
+  const int N = N_, H = cfg_.H;
+  const float *W = param("W").w.get();
+  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);
+  for (int k : sched_.bwd_rounds) {
+    const Round &r = sched_.rounds[k];
+    const size_t off = r.offset;
+    gather(r_dmsg_.get(), H, dpool_.get(), H, d_pair_ + off, r.n, H);
+    float *dz = dxW_.at(off * H);
+    check(cavs_treefc_bwd(r_dmsg_.get(), dret_.at(off * H), msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));
+    c_launches_ += 1;
+    if (leaf_round(r)) continue;
+    gemm(0, 1, r.n, 2 * H, H, dz, H, W, H, 0.f, r_dG_.get(), 2 * H);
+    scatter(dpool_.get(), H, d_child_ + 2 * off, r_dG_.get(), H, 2 * r.n, H);
+  }
+  const int lp = sched_.leaf_prefix;
+  gemm_splitk(1, 0, 2 * H, H, N - lp, G_.at((size_t)2 * lp * H), 2 * H, dxW_.at((size_t)lp * H), H,
+              param("W").g.get(), H);
+  if (cfg_.use_bias) {
+    check(cavs_colsum(param("Bv").g.get(), dxW_.get(), H, N, H, 0, stream_));
+    c_launches_ += 1;
+  }
+}
+
+// ------------------------------------------------------------------ loss head
+void Engine::head_forward_backward(bool backward) {
+  const int N = N_, H = cfg_.H, C = cfg_.C, B = sched_.B;
+  if (cfg_.loss == CAVS_LOSS_SOFTMAX) {
+    // FullyConnected + SoftmaxEntropyLoss (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79,
+    // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
+    Param &Wfc = param("Wfc"), &bfc = param("bfc");
+    gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w.get(), H, 0.f, logits_.get(), C);
+    check(cavs_bias_add_rows(logits_.get(), logits_.get(), bfc.w.get(), N, C, stream_));
+    check(cavs_softmax_xent(loss_.get(), backward ? dlogits_.get() : nullptr, logits_.get(), d_labels_, N, C, stream_));
+    c_launches_ += 2;
+    if (backward) {
+      gemm_splitk(1, 0, C, H, N, dlogits_.get(), C, GO_.get(), H, Wfc.g.get(), H);
+      check(cavs_colsum(bfc.g.get(), dlogits_.get(), C, N, C, 0, stream_));
+      c_launches_ += 1;
+      gemm(0, 0, N, H, C, dlogits_.get(), C, Wfc.w.get(), H, 0.f, dGO_.get(), H);
+    }
+    return;
+  }
+  float *tmp = logits_.get(), *colacc = loss_.get() + 1;
+  if (cfg_.loss == CAVS_LOSS_ROOT_SQ) {
+    // sum over roots of h^2; gradient 2h on root rows, zero elsewhere
+    gather(tmp, H, GO_.get(), H, d_roots_, B, H);
+    check(cavs_ew_unary(CAVS_EW_SQUARE, dlogits_.get(), tmp, (size_t)B * H, 0, stream_));
+    check(cavs_colsum(colacc, dlogits_.get(), H, B, H, 0, stream_));
+    check(cavs_colsum(loss_.get(), colacc, 1, H, 1, 0, stream_));
+    c_launches_ += 3;
+    if (backward) {
+      check(cavs_zero(dGO_.get(), (size_t)N * H * 4, stream_));
+      check(cavs_scale(dlogits_.get(), tmp, 2.f, (size_t)B * H, stream_));
+      c_launches_ += 2;
+      scatter(dGO_.get(), H, d_roots_, dlogits_.get(), H, B, H);
+    }
+  } else {
+    // Reduce_sum is a sum of absolute values whose gradient op is a constant fill
+    // (cavs/backend/op_impl_blas1_cublas.cc:62-77, cavs/backend/op_decl_reduction.cc:19-28)
+    check(cavs_ew_unary(CAVS_EW_ABS, dlogits_.get(), GO_.get(), (size_t)N * H, 0, stream_));
+    check(cavs_colsum(colacc, dlogits_.get(), H, N, H, 0, stream_));
+    check(cavs_colsum(loss_.get(), colacc, 1, H, 1, 0, stream_));
+    c_launches_ += 3;
+    if (backward) {
+      check(cavs_fill(dGO_.get(), 1.f, (size_t)N * H, stream_));
+      c_launches_ += 1;
+    }
+  }
+}
+
+void Engine::sync() { check(cavs_stream_sync(stream_)); }
+
+void Engine::fetch(const std::string &what, float *host, size_t n) {
+  const size_t N = N_, H = cfg_.H;
+  const float *src = nullptr;
+  size_t want = 0;
+  if (what == "loss") {
+    src = loss_.get();
+    want = cfg_.loss == CAVS_LOSS_SOFTMAX ? N : 1;
+  } else if (what == "graph_out") {
+    src = GO_.get();
+    want = N * H;
+  } else if (what == "dgraph_out") {
+    src = dGO_.get();
+    want = N * H;
+  } else if (what == "msg_pool") {
+    src = pool_.get();
+    want = N * mw_;
+  } else {
+    fail(CAVS_EINVAL, "unknown result '" + what + "'");
+  }
+  if (N == 0) fail(CAVS_EINVAL, "no step has run yet");
+  if (n != want || !host) fail(CAVS_EINVAL, "'" + what + "' holds " + std::to_string(want) + " floats, got " + std::to_string(n));
+  check(cavs_memcpy_d2h(host, src, want * 4, stream_));
+  check(cavs_stream_sync(stream_));
+}
+
+float Engine::timing(const std::string &name) {
+  float ms = 0.f;
+  if (name == "GraphParsing") return parse_ms_;
+  if (name == "RNNForward" && ev_valid_) {
+    check(cavs_event_elapsed_ms(&ms, ev_[0], ev_[1]));
+    return ms;
+  }
+  if (name == "RNNBackward" && ev_bwd_valid_) {
+    check(cavs_event_elapsed_ms(&ms, ev_[2], ev_[3]));
+    return ms;
+  }
+  fail(CAVS_EINVAL, "no timing named '" + name + "' for the last step");
+}
+
+double Engine::counter(const std::string &key) const {
+  if (key == "gather_rows") return c_gather_rows_;
+  if (key == "scatter_rows") return c_scatter_rows_;
+  if (key == "gather_bytes") return c_gather_bytes_;
+  if (key == "scatter_bytes") return c_scatter_bytes_;
+  if (key == "gemm_flops") return c_gemm_flops_;
+  if (key == "launches") return c_launches_;
+  if (key == "rounds") return (double)sched_.rounds.size();
+  fail(CAVS_EINVAL, "unknown counter '" + key + "'");
+}
+
+}  // namespace cavs

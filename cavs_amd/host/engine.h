@@ -1,0 +1,103 @@
+// The forward / backward round loops over a batch of instance graphs for the three
+// vertex functions, on top of the C ABI of the HIP backend.  Restates, for these F,
+// what the reference spreads over GraphStatement::Run / GraphGradStatement::Run
+// (cavs/midend/statement.cc:43-123), GraphSession's memory layout
+// (cavs/midend/graph_session.cc:45-206) and BatchingWeightUpdater
+// (cavs/midend/batch_weight_updater.h:12-84).
+#ifndef CAVS_HOST_ENGINE_H_
+#define CAVS_HOST_ENGINE_H_
+
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "cavs_session.h"
+#include "device.h"
+#include "scheduler.h"
+
+namespace cavs {
+
+struct Param {
+  DeviceArray<float> w, g;
+  size_t n = 0;
+};
+
+class Engine {
+ public:
+  explicit Engine(const cavs_session_config &cfg);
+  ~Engine();
+
+  void set_param(const std::string &name, const float *host, size_t n);
+  void get_param(const std::string &name, float *host, size_t n, bool grad);
+  void step(const int *graph, int B, int maxlen, const void *x, const void *labels,
+            bool on_device, bool backward, float lr);
+  void sync();
+  void fetch(const std::string &what, float *host, size_t n);
+  float timing(const std::string &name);
+  double counter(const std::string &key) const;
+  const Schedule &schedule() const { return sched_; }
+  void *stream() const { return stream_; }
+  int total_length() const { return sched_.N; }
+
+ private:
+  Param &param(const std::string &name);
+  void add_param(const std::string &name, size_t n);
+  void reserve_edges();
+  void ensure(DeviceArray<float> &a, size_t n);  // grow after draining the stream
+  void upload_index_arena();
+  // one model each: forward rounds, backward rounds + deferred weight gradients
+  void treelstm_forward();
+  void treelstm_backward();
+  void lstm_forward();
+  void lstm_backward();
+  void treefc_forward();
+  void treefc_backward();
+  void pop_ret();
+  void head_forward_backward(bool backward);
+  // counted wrappers
+  void gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B, int ldb,
+            float beta, float *C, int ldc);
+  void gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
+                   int ldb, float *C, int ldc);
+  void gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n, int w);
+  void scatter(float *dst, int ld_dst, const int *ids, const float *inp, int ld_inp, int n, int w);
+  bool leaf_round(const Round &r) const {
+    return r.gather_begin[0] == r.gather_end[0] && r.gather_begin[1] == r.gather_end[1];
+  }
+
+  cavs_session_config cfg_;
+  void *stream_ = nullptr;
+  void *ev_[4] = {nullptr, nullptr, nullptr, nullptr};  // fwd begin/end, bwd begin/end
+  bool ev_valid_ = false, ev_bwd_valid_ = false;
+  float parse_ms_ = 0.f;
+  std::map<std::string, std::unique_ptr<Param>> params_;
+
+  Schedule sched_;
+  bool did_backward_ = false;
+  int N_ = 0, cap_ = 0, rcap_ = 0, E_ = 0, mw_ = 0, nch_ = 1;
+
+  // per-step device index arena: [t2j | pair | child | roots]
+  PinnedArray<int> idx_host_[2];
+  void *idx_copied_[2] = {nullptr, nullptr};  // events: upload out of idx_host_[k] finished
+  bool idx_pending_[2] = {false, false};
+  int idx_slot_ = 0;
+  DeviceArray<int> idx_dev_;
+  const int *d_t2j_ = nullptr, *d_pair_ = nullptr, *d_child_ = nullptr, *d_roots_ = nullptr;
+
+  // feeds
+  DeviceArray<float> x_in_, labels_in_;
+  const float *d_x_ = nullptr, *d_labels_ = nullptr;
+
+  // edges (rows = tensor ids unless marked round-local)
+  DeviceArray<float> xs_, e_, xW_, G_, hlr_, gates_, msg_, pool_, GO_, dGO_, dret_, dpool_, dxW_,
+      dF_, de_, logits_, dlogits_, loss_, ws_;
+  DeviceArray<float> r_hU_, r_hUf_, r_dmsg_, r_dG_, r_dhlr_, r_z_;  // round-local
+
+  // counters of the last step
+  double c_gather_rows_ = 0, c_scatter_rows_ = 0, c_gemm_flops_ = 0, c_launches_ = 0,
+         c_gather_bytes_ = 0, c_scatter_bytes_ = 0;
+};
+
+}  // namespace cavs
+#endif

@@ -1,0 +1,226 @@
+#include "scheduler.h"
+
+#include <algorithm>
+
+namespace cavs {
+
+// LoadGraph, cavs/midend/graph_scheduler.cc:12-71.
+static std::string load_graph(const int32_t *g, int B, int maxlen, Schedule *s) {
+  s->B = B;
+  s->maxlen = maxlen;
+  s->sample_offset.assign(B, 0);
+  s->parent.clear();
+  int off = 0;
+  for (int i = 0; i < B; i++) {
+    const int32_t *row = g + (size_t)i * maxlen;
+    int k = 0;
+    while (k < maxlen && row[k] != -1) k++;
+    if (k == maxlen) return "sample " + std::to_string(i) + " has no -1 terminator within maxlen";
+    int len = k + 1;
+    s->sample_offset[i] = off;
+    for (int j = 0; j < len - 1; j++) {
+      if (row[j] < 0 || row[j] >= len)
+        return "sample " + std::to_string(i) + ": parent id out of range at vertex " + std::to_string(j);
+      s->parent.push_back(off + row[j]);
+    }
+    s->parent.push_back(-1);
+    off += len;
+  }
+  const int N = s->N = off;
+  // children in ascending vertex id (graph_scheduler.cc:52-58 appends in vertex order)
+  s->child_begin.assign(N + 1, 0);
+  for (int v = 0; v < N; v++)
+    if (s->parent[v] >= 0) s->child_begin[s->parent[v] + 1]++;
+  for (int v = 0; v < N; v++) s->child_begin[v + 1] += s->child_begin[v];
+  s->child.assign(s->child_begin[N], 0);
+  std::vector<int> fill(s->child_begin.begin(), s->child_begin.end() - 1);
+  for (int v = 0; v < N; v++)
+    if (s->parent[v] >= 0) s->child[fill[s->parent[v]]++] = v;
+  return "";
+}
+
+static inline int nchild(const Schedule &s, int v) { return s.child_begin[v + 1] - s.child_begin[v]; }
+
+// BatchGraphScheduler::Initialize / ActivateNext, forward branch
+// (cavs/midend/graph_scheduler.cc:169-193, 202-245).
+static void batch_rounds(Schedule *s) {
+  const int N = s->N;
+  s->tids_to_jobids.assign(N, 0);
+  s->jobids_to_tids.assign(N, 0);
+  s->round2offset.assign(1, 0);
+  std::vector<int> activated(N, 0);
+  int begin = 0, end = 0;  // current round = tids [begin, end)
+  for (int v = 0; v < N; v++)
+    if (nchild(*s, v) == 0 && s->parent[v] >= 0) {
+      s->tids_to_jobids[end] = v;
+      s->jobids_to_tids[v] = end;
+      end++;
+    }
+  s->leaf_prefix = end;
+  while (end > begin) {
+    Round r;
+    r.offset = begin;
+    r.n = end - begin;
+    // lists this round exposes: gather lists were appended while the round was being
+    // formed (below); the scatter list holds the non-root jobs in job order
+    for (int c = 0; c < 2; c++) r.gather_end[c] = (int)s->gather_ids[c].size();
+    r.scatter_begin = (int)s->scatter_ids.size();
+    for (int t = begin; t < end; t++)
+      if (s->parent[s->tids_to_jobids[t]] >= 0) s->scatter_ids.push_back(t);
+    r.scatter_end = (int)s->scatter_ids.size();
+    for (int c = 0; c < 2; c++)
+      r.gather_begin[c] = s->rounds.empty() ? r.gather_end[c] : s->rounds.back().gather_end[c];
+    s->rounds.push_back(r);
+    s->max_round = std::max(s->max_round, r.n);
+    s->round2offset.push_back(end);
+    int next = end;
+    for (int t = begin; t < end; t++) {
+      int p = s->parent[s->tids_to_jobids[t]];
+      if (p < 0) continue;
+      if (++activated[p] == nchild(*s, p)) {
+        s->tids_to_jobids[next] = p;
+        s->jobids_to_tids[p] = next;
+        for (int i = 0; i < nchild(*s, p) && i < 2; i++)
+          s->gather_ids[i].push_back(s->jobids_to_tids[s->child[s->child_begin[p] + i]]);
+        if (s->parent[p] < 0) s->root_tids.push_back(next);
+        next++;
+      }
+    }
+    begin = end;
+    end = next;
+  }
+  s->executed = end;
+  for (int k = (int)s->rounds.size() - 1; k >= 0; k--) s->bwd_rounds.push_back(k);
+}
+
+// SerialGraphScheduler (cavs/midend/graph_scheduler.cc:83-167): one vertex per round,
+// tensor id == vertex id, samples one after the other, FIFO activation order.
+static void serial_rounds(Schedule *s) {
+  const int N = s->N;
+  s->tids_to_jobids.assign(N, 0);
+  s->jobids_to_tids.assign(N, 0);
+  for (int v = 0; v < N; v++) s->tids_to_jobids[v] = s->jobids_to_tids[v] = v;
+  std::vector<int> activated(N, 0), fifo;
+  fifo.reserve(N);
+  for (int i = 0; i < s->B; i++) {
+    int lo = s->sample_offset[i], hi = i + 1 < s->B ? s->sample_offset[i + 1] : N;
+    size_t head = fifo.size();
+    for (int v = lo; v < hi; v++)
+      if (nchild(*s, v) == 0 && s->parent[v] >= 0) fifo.push_back(v);
+    for (; head < fifo.size(); head++) {
+      int v = fifo[head], p = s->parent[v];
+      if (p >= 0 && ++activated[p] == nchild(*s, p)) fifo.push_back(p);
+    }
+  }
+  for (int v : fifo) {
+    Round r;
+    r.offset = v;
+    r.n = 1;
+    for (int c = 0; c < 2; c++) {
+      r.gather_begin[c] = (int)s->gather_ids[c].size();
+      if (nchild(*s, v) > c) s->gather_ids[c].push_back(s->child[s->child_begin[v] + c]);
+      r.gather_end[c] = (int)s->gather_ids[c].size();
+    }
+    r.scatter_begin = (int)s->scatter_ids.size();
+    if (s->parent[v] >= 0) s->scatter_ids.push_back(v); else s->root_tids.push_back(v);
+    r.scatter_end = (int)s->scatter_ids.size();
+    s->rounds.push_back(r);
+  }
+  s->executed = (int)fifo.size();
+  s->max_round = fifo.empty() ? 0 : 1;
+  s->leaf_prefix = 0;
+  // Backward order (ReverseGraph + the same FIFO, graph_scheduler.cc:73-81,110-140): roots
+  // first, children after their parent.  The reference starts the next sample whenever
+  // the vertex it pops has no forward children, i.e. at every leaf, not only at the end
+  // of a sample; the order below reproduces that.
+  std::vector<int> round_of(N, -1);
+  for (size_t k = 0; k < s->rounds.size(); k++) round_of[s->rounds[k].offset] = (int)k;
+  std::vector<int> bf;
+  bf.reserve(N);
+  auto init_sample = [&](int i) {
+    int lo = s->sample_offset[i], hi = i + 1 < s->B ? s->sample_offset[i + 1] : N;
+    for (int v = lo; v < hi; v++)
+      if (s->parent[v] < 0 && nchild(*s, v) > 0) bf.push_back(v);
+  };
+  int sample_id = 0;
+  init_sample(0);
+  for (size_t head = 0; head < bf.size(); head++) {
+    int v = bf[head];
+    if (nchild(*s, v) > 0) {
+      for (int k = s->child_begin[v]; k < s->child_begin[v + 1]; k++) bf.push_back(s->child[k]);
+    } else if (++sample_id < s->B) {
+      init_sample(sample_id);
+    }
+  }
+  for (int v : bf) s->bwd_rounds.push_back(round_of[v]);
+}
+
+std::string build_schedule(const int32_t *graph, int B, int maxlen, bool batching, Schedule *out) {
+  *out = Schedule();
+  out->batching = batching;
+  if (!graph || B <= 0 || maxlen <= 0) return "empty graph feed";
+  std::string err = load_graph(graph, B, maxlen, out);
+  if (!err.empty()) return err;
+  if (batching) batch_rounds(out); else serial_rounds(out);
+  return "";
+}
+
+// trace_format: [N, R_fwd, R_bwd, then per round: offset, n_exec, exec..., n_g0, g0...,
+// n_g1, g1..., n_s0, s0..., n_s1, s1..., n_init, init..., then tids_to_jobids (N),
+// n_r2o, round2offset...].  Backward rounds are the forward rounds last to first with
+// gather := recorded scatter lists and scatter := recorded gather lists
+// (cavs/midend/graph_scheduler.cc:194-199, 246-257).
+std::vector<int> Schedule::trace(bool with_backward) const {
+  std::vector<int> o;
+  auto put_list = [&](const int *p, int n) {
+    o.push_back(n);
+    o.insert(o.end(), p, p + n);
+  };
+  const int R = (int)rounds.size();
+  o.push_back(N);
+  o.push_back(R);
+  o.push_back(with_backward ? (int)bwd_rounds.size() : 0);
+  // forward gather_init list: the leaves of round 0 (batch) / the current leaf (serial)
+  std::vector<int> init_fwd;
+  if (batching && R) init_fwd.assign(tids_to_jobids.begin(), tids_to_jobids.begin() + rounds[0].n);
+  for (int k = 0; k < R; k++) {
+    const Round &r = rounds[k];
+    o.push_back(r.offset);
+    if (batching) put_list(&tids_to_jobids[r.offset], r.n); else put_list(&r.offset, 1);
+    for (int c = 0; c < 2; c++) put_list(gather_ids[c].data() + r.gather_begin[c], r.gather_end[c] - r.gather_begin[c]);
+    put_list(scatter_ids.data() + r.scatter_begin, r.scatter_end - r.scatter_begin);
+    o.push_back(0);
+    if (!batching && r.gather_end[0] == r.gather_begin[0]) init_fwd.assign(1, r.offset);
+    put_list(init_fwd.data(), (int)init_fwd.size());
+  }
+  if (with_backward) {
+    std::vector<int> init_bwd = batching ? root_tids : std::vector<int>();
+    bool first = true;
+    for (int k : bwd_rounds) {
+      const Round &r = rounds[k];
+      o.push_back(r.offset);
+      if (batching) put_list(&tids_to_jobids[r.offset], r.n); else put_list(&r.offset, 1);
+      if (batching) {
+        put_list(scatter_ids.data() + r.scatter_begin, r.scatter_end - r.scatter_begin);
+        o.push_back(0);
+      } else {
+        // serial backward: the gather list is one copy of the vertex per forward parent
+        // (graph_scheduler.cc:158-161); the first round is set up by Initialize, which
+        // fills no gather list (:100-107)
+        int v = r.offset;
+        int has_parent = parent[v] >= 0;
+        if (first) o.push_back(0); else put_list(&v, has_parent);
+        o.push_back(0);
+        if (!has_parent) init_bwd.assign(1, v);
+      }
+      for (int c = 0; c < 2; c++) put_list(gather_ids[c].data() + r.gather_begin[c], r.gather_end[c] - r.gather_begin[c]);
+      put_list(init_bwd.data(), (int)init_bwd.size());
+      first = false;
+    }
+  }
+  o.insert(o.end(), tids_to_jobids.begin(), tids_to_jobids.end());
+  put_list(round2offset.data(), (int)round2offset.size());
+  return o;
+}
+
+}  // namespace cavs

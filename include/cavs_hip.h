@@ -62,6 +62,7 @@ int cavs_stream_sync(void *stream);
 int cavs_event_create(void **event);
 int cavs_event_destroy(void *event);
 int cavs_event_record(void *event, void *stream);
+int cavs_event_sync(void *event); /* host waits until the event has happened */
 int cavs_event_elapsed_ms(float *ms, void *start, void *stop); /* waits for `stop` */
 
 /* ------------------------------------------------------------------ graph ops

@@ -1,0 +1,96 @@
+/*
+ * cavs_session.h -- C ABI of the host runtime (libcavs_host.so): the part of the
+ * reference's midend that sits on the hot path -- graph scheduler, batching memory
+ * manager and the forward / backward round loops -- re-stated in C++ on top of
+ * cavs_hip.h.  It plays the role of the reference's outer C API
+ * (cavs/frontend/c_api.h:20-36: C_NewSession / C_Run) for the vertex functions the
+ * benchmarks use; the Sym/GraphSupport front end (cavs_amd/host/frontend) lowers
+ * onto it.
+ *
+ * Feeds follow the reference's wire format: `graph` is a host int32 [B, maxlen]
+ * parent array (cavs/midend/graph_scheduler.cc:35-43; the reference requires the
+ * graph placeholder on the CPU, graph_scheduler.cc:15), vertex inputs and labels are
+ * fp32 packed by global vertex id (apps/paper/seq-lstm-cavs-varLength.cc:38-56).
+ *
+ * All functions return 0 or a negative CAVS_E* code (cavs_hip.h);
+ * cavs_session_error() holds the message.
+ */
+#ifndef CAVS_SESSION_H_
+#define CAVS_SESSION_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cavs_session cavs_session;
+
+enum { CAVS_MODEL_TREELSTM = 0, CAVS_MODEL_LSTM = 1, CAVS_MODEL_TREEFC = 2 };
+enum { CAVS_LOSS_SOFTMAX = 0, CAVS_LOSS_ROOT_SQ = 1, CAVS_LOSS_SUM_ABS = 2 };
+/* How the forward Scatter / backward Gather pair list entries with slab rows:
+ * REFERENCE = b-th list entry with b-th slab row, exactly what the reference's
+ * kernels do (cavs/backend/op_impl_graphop.cu:67-76,148-157) -- rows shift after a
+ * root that is not last in its round; ROWID = the row the tensor id names. */
+enum { CAVS_PAIR_REFERENCE = 0, CAVS_PAIR_ROWID = 1 };
+/* cavs/proto/opt.proto:3-8 */
+enum { CAVS_OPT_FUSION = 1, CAVS_OPT_BATCHING = 2, CAVS_OPT_STREAMMING = 4 };
+
+typedef struct {
+  int model, loss, pairing;
+  int opt;            /* OPT_* bitmask; without OPT_BATCHING the serial scheduler runs */
+  int V, E, H, C;     /* vocabulary, embedding, hidden, classes */
+  int act;            /* Tree-FC activation: 0 relu, 1 tanh */
+  int use_bias;       /* Tree-FC */
+  int use_x;          /* Tree-FC: add the Pull'ed [H] input row */
+  int device;
+} cavs_session_config;
+
+const char *cavs_session_error(void);
+int cavs_session_create(const cavs_session_config *cfg, cavs_session **out);
+int cavs_session_destroy(cavs_session *s);
+
+/* Parameters and their gradients by name: "Emb" "W" "U" "Bv" "Wfc" "bfc"
+ * (shapes: apps/paper/tree-lstm-cavs.cc:110-126, seq-lstm-cavs.cc:49-59,
+ * tree-fc-cavs.cc:24). `n` is the element count and must match. */
+int cavs_session_set_param(cavs_session *s, const char *name, const float *host, size_t n);
+int cavs_session_get_param(cavs_session *s, const char *name, float *host, size_t n);
+int cavs_session_get_grad(cavs_session *s, const char *name, float *host, size_t n);
+
+/* One pass of F over the batch (C_Run of the train op, cavs/frontend/c_api.cc:149-172):
+ * schedule, forward rounds, loss head, and if `backward` the gradient rounds and the
+ * deferred weight gradients; if lr != 0 also the SGD update (cavs/backend/op_impl_sgd.cu).
+ * x and labels are host pointers unless inputs_on_device is set, in which case they
+ * are device pointers to buffers already resident in HBM.  The call only enqueues
+ * work; cavs_session_sync() waits for it. */
+int cavs_session_step(cavs_session *s, const int *graph, int B, int maxlen, const void *x,
+                      const void *labels, int inputs_on_device, int backward, float lr);
+int cavs_session_sync(cavs_session *s);
+
+/* Results of the last step, copied to host (synchronises):
+ *   "loss" [N] (softmax) or [1]; "graph_out" [N,H] in vertex order; "dgraph_out" [N,H];
+ *   "msg_pool" [N, 2H | H] by tensor id. */
+int cavs_session_fetch(cavs_session *s, const char *what, float *host, size_t n);
+int cavs_session_total_length(cavs_session *s); /* N of the last step */
+
+/* The last step's schedule in the serialisation of Schedule::trace (forward rounds,
+ * backward rounds, tids_to_jobids, round2offset).  Returns the number of ints, or the
+ * negative of the needed capacity. */
+int cavs_session_schedule_trace(cavs_session *s, int *out, int cap);
+/* Pure host call (no device): schedule of a graph feed, same serialisation. */
+int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int with_backward,
+                        int *out, int cap);
+
+/* Timers of the last step in ms, by the reference's names (cavs/midend/statement.cc:
+ * 53,65,68,84,102,122): "GraphParsing" (host), "RNNForward", "RNNBackward" (device). */
+int cavs_session_timing(cavs_session *s, const char *name, float *ms);
+/* Raw stream the session enqueues on (for callers that want to bracket it with events). */
+void *cavs_session_stream(cavs_session *s);
+/* Per-step counts for roofline accounting: rows moved by indexed copies and GEMM flops
+ * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" "rounds" "launches". */
+int cavs_session_counter(cavs_session *s, const char *key, double *value);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
