@@ -1,0 +1,173 @@
+#!/usr/bin/env python3
+"""Headline benchmark: train samples/sec (forward + backward + SGD) of the binary
+Tree-LSTM (hidden 512, embedding 300, batch 64, sentence-shaped random trees) through
+the batched F-over-G path on one MI355X, with the roofline fraction of the dominant
+kernel (the FP32-MFMA gate GEMM) and a CPU baseline (the CPU restatement of the
+reference's semantics -- the reference ships no CPU kernels) timed on this host.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3|C2|C4|C5]
+
+A step = host scheduling of a fresh batch structure (a pool of 16 pre-generated seeded
+batches is cycled, so graph parsing is inside the timed region, as in the reference's
+GraphStatement::Run) + forward rounds + loss head + backward rounds + deferred weight
+gradients + SGD.  Vertex inputs and labels are resident in HBM before timing starts;
+the graph placeholder is a host tensor by contract.
+Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
+
+
+def model_kwargs(w):
+    if w["model"] == "treefc":
+        return dict(loss="root_sq", act=1, use_bias=True, use_x=True)
+    return dict(loss="softmax")
+
+
+def make_pool(name, n_batches):
+    from cavs_amd import synth
+
+    base = synth.make_workload(name)
+    pool = [base]
+    for i in range(1, n_batches):
+        w = synth.make_workload(name, seed=base["seed"] + 7919 * i)
+        w["params"] = base["params"]
+        pool.append(w)
+    return pool
+
+
+def cpu_baseline(w, budget_s=20.0):
+    """Times the CPU checker on this host on a bounded sample of the same workload."""
+    sys.path.insert(0, os.path.join(ROOT, "oracle"))
+    import pyoracle
+
+    threads = min(16, len(os.sched_getaffinity(0)))
+    kw = model_kwargs(w)
+    args = dict(H=w["H"], E=w["E"], V=w["V"], Cc=w["C"], threads=threads, **kw)
+    t0 = time.perf_counter()
+    steps = 0
+    while True:
+        pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **args)
+        steps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or steps >= 8 or el + el / steps > 1.5 * budget_s:
+            break
+    return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port",
+                sample=f"{steps} full fwd+bwd step(s) of the {w['name']} batch (B={w['B']}, N={w['N']}) "
+                       f"in {el:.1f} s with {threads} OpenMP threads; CPU restatement of the reference's "
+                       "semantics (the reference has no CPU kernels)")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--pool", type=int, default=16)
+    ap.add_argument("--lr", type=float, default=1e-3)
+    ap.add_argument("--pairing", default="reference", choices=["reference", "rowid"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs the F-over-G path on one GPU; instance graphs shard by sample "
+                 "across GPUs (see DESIGN.md) but no multi-GPU path is built -- run with --gpus 1")
+
+    import torch
+
+    from cavs_amd import session
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    pool = make_pool(a.workload, a.pool)
+    w0 = pool[0]
+    kw = model_kwargs(w0)
+    s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
+                        opt=session.OPT_BATCHING, **kw)
+    s.set_params(w0["params"])
+    feeds = []
+    for w in pool:  # inputs resident in HBM before the timed region
+        feeds.append((w["graph"], torch.from_numpy(np.ascontiguousarray(w["x"])).cuda(),
+                      torch.from_numpy(w["labels"]).cuda()))
+    torch.cuda.synchronize()
+
+    def run(k0, k):
+        for i in range(k0, k0 + k):
+            g, x, lab = feeds[i % len(feeds)]
+            s.step(g, x, lab, backward=True, lr=a.lr)
+
+    run(0, a.warmup)
+    s.sync()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run(a.warmup, a.steps)
+    s.sync()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / a.steps
+    value = w0["B"] * a.steps / elapsed
+
+    # Roofline of the dominant kernel: the same K steps again with every launch of the
+    # session bracketed by HIP events on the session's own stream (the bracketing costs a
+    # little launch throughput, so it is kept out of the throughput figure above).
+    s.profile(True)
+    flops = rows = gbytes = sbytes = 0.0
+    for i in range(a.warmup, a.warmup + a.steps):
+        g, x, lab = feeds[i % len(feeds)]
+        s.step(g, x, lab, backward=True, lr=a.lr)
+        flops += s.counter("gemm_flops")
+        gbytes += s.counter("gather_bytes")
+        sbytes += s.counter("scatter_bytes")
+    gemm_ms, gemm_n = s.profile_read("gemm")
+    gat_ms, gat_n = s.profile_read("gather")
+    sca_ms, sca_n = s.profile_read("scatter")
+    gates_ms, gates_n = s.profile_read("gates")
+    s.profile(False)
+    achieved_tf = flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else 0.0
+    rounds = s.counter("rounds")
+    launches = s.counter("launches")
+
+    out = {
+        "metric": "train samples/sec (fwd+bwd) Tree-LSTM h=512 bs=64; % HBM/MFMA peak",
+        "value": round(value, 2), "unit": "samples/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{a.workload}: {w0['model']} V={w0['V']} E={w0['E']} H={w0['H']} B={w0['B']} "
+                               f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
+                   "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing, "rounds_last_batch": rounds,
+                   "launches_last_batch": launches},
+        "roofline": {"bound": "mfma", "achieved": round(achieved_tf, 3), "peak": FP32_MFMA_PEAK_TF,
+                     "unit": "TFLOP/s", "frac": round(achieved_tf / FP32_MFMA_PEAK_TF, 5), "traffic": None,
+                     "kernel": "sgemm_mfma_kernel (all gate / weight-gradient / head GEMMs of a step)",
+                     "avg_launch_us": round(1e3 * gemm_ms / gemm_n, 3) if gemm_n else None,
+                     "flops_per_launch": round(flops / gemm_n, 1) if gemm_n else None},
+        "kernels": {
+            "gather": {"bound": "hbm", "achieved": round(gbytes / (gat_ms * 1e-3) / 1e9, 2) if gat_ms else None,
+                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * gat_ms / max(gat_n, 1), 3)},
+            "scatter": {"bound": "hbm", "achieved": round(sbytes / (sca_ms * 1e-3) / 1e9, 2) if sca_ms else None,
+                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * sca_ms / max(sca_n, 1), 3)},
+            "gates": {"avg_launch_us": round(1e3 * gates_ms / max(gates_n, 1), 3)},
+            "device_ms_per_step": {"gemm": round(gemm_ms / a.steps, 4), "gather": round(gat_ms / a.steps, 4),
+                                   "scatter": round(sca_ms / a.steps, 4), "gates": round(gates_ms / a.steps, 4)},
+        },
+        "timers_ms": {"GraphParsing": round(s.timing("GraphParsing"), 4), "RNNForward": round(s.timing("RNNForward"), 4),
+                      "RNNBackward": round(s.timing("RNNBackward"), 4)},
+    }
+    if not a.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(w0)
+    s.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -118,6 +118,26 @@ int cavs_session_timing(cavs_session *s, const char *name, float *ms) {
   return guarded([&] { *ms = s->engine.timing(name ? name : ""); });
 }
 
+int cavs_session_profile(cavs_session *s, int enable) {
+  if (int rc = need(s, "session")) return rc;
+  return guarded([&] { s->engine.profile_enable(enable != 0); });
+}
+
+int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double *total_ms, double *launches) {
+  if (int rc = need(s, "session")) return rc;
+  if (int rc = need(total_ms, "output")) return rc;
+  if (int rc = need(launches, "output")) return rc;
+  static const char *names[] = {"gemm", "gather", "scatter", "gates", "other"};
+  int cls = -1;
+  for (int i = 0; i < 5; i++)
+    if (kernel_class && !std::strcmp(kernel_class, names[i])) cls = i;
+  if (cls < 0) {
+    g_error = "unknown kernel class";
+    return CAVS_EINVAL;
+  }
+  return guarded([&] { s->engine.profile_read(cls, total_ms, launches); });
+}
+
 void *cavs_session_stream(cavs_session *s) { return s ? s->engine.stream() : nullptr; }
 
 int cavs_session_counter(cavs_session *s, const char *key, double *value) {

@@ -4,6 +4,13 @@
 #include <chrono>
 #include <cstring>
 
+// runs one backend call inside a profiling bracket of the given kernel class
+#define CAVS_TIMED(cls, call)   \
+  do {                          \
+    ProfScope _ps(this, cls);   \
+    check(call);                \
+  } while (0)
+
 namespace cavs {
 
 namespace {
@@ -56,6 +63,7 @@ Engine::~Engine() {
   cavs_stream_sync(stream_);
   for (auto &e : ev_) cavs_event_destroy(e);
   for (auto &e : idx_copied_) cavs_event_destroy(e);
+  for (auto &e : prof_events_) cavs_event_destroy(e);
   cavs_stream_destroy(stream_);
 }
 
@@ -91,9 +99,53 @@ void Engine::get_param(const std::string &name, float *host, size_t n, bool grad
   check(cavs_stream_sync(stream_));
 }
 
+// ------------------------------------------------------------------ profiling
+void *Engine::prof_event() {
+  if (prof_used_ == prof_events_.size()) {
+    void *e = nullptr;
+    check(cavs_event_create(&e));
+    prof_events_.push_back(e);
+  }
+  return prof_events_[prof_used_++];
+}
+
+Engine::ProfScope::ProfScope(Engine *eng, int cls) : e(eng), s{cls, nullptr, nullptr}, on(eng->profile_) {
+  if (!on) return;
+  s.a = e->prof_event();
+  s.b = e->prof_event();
+  check(cavs_event_record(s.a, e->stream_));
+}
+
+Engine::ProfScope::~ProfScope() {
+  if (!on) return;
+  if (cavs_event_record(s.b, e->stream_) == CAVS_OK) e->spans_.push_back(s);
+}
+
+void Engine::profile_enable(bool on) {
+  check(cavs_stream_sync(stream_));
+  profile_ = on;
+  spans_.clear();
+  prof_used_ = 0;
+}
+
+void Engine::profile_read(int cls, double *total_ms, double *launches) {
+  check(cavs_stream_sync(stream_));
+  double t = 0, n = 0;
+  for (const Span &sp : spans_) {
+    if (sp.cls != cls) continue;
+    float ms = 0.f;
+    check(cavs_event_elapsed_ms(&ms, sp.a, sp.b));
+    t += ms;
+    n += 1;
+  }
+  *total_ms = t;
+  *launches = n;
+}
+
 // ------------------------------------------------------------------ counted wrappers
 void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
                   int ldb, float beta, float *C, int ldc) {
+  ProfScope ps(this, K_GEMM);
   check(cavs_sgemm(tA, tB, M, N, K, 1.f, A, lda, B, ldb, beta, C, ldc, stream_));
   c_gemm_flops_ += 2.0 * M * N * K;
   c_launches_ += 1;
@@ -102,6 +154,7 @@ void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, 
 void Engine::gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda,
                          const float *B, int ldb, float *C, int ldc) {
   size_t need = cavs_sgemm_splitk_workspace(M, N, K);
+  ProfScope ps(this, K_GEMM);
   if (ws_.capacity() * 4 < need) {
     // the workspace may still be in use by an enqueued GEMM
     check(cavs_stream_sync(stream_));
@@ -115,6 +168,7 @@ void Engine::gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, in
 
 void Engine::gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n,
                     int w) {
+  ProfScope ps(this, K_GATHER);
   check(cavs_gather_rows(out, ld_out, src, ld_src, ids, n, w, stream_));
   c_gather_rows_ += n;
   c_gather_bytes_ += (8.0 * w + 4.0) * n;
@@ -123,6 +177,7 @@ void Engine::gather(float *out, int ld_out, const float *src, int ld_src, const 
 
 void Engine::scatter(float *dst, int ld_dst, const int *ids, const float *inp, int ld_inp, int n,
                      int w) {
+  ProfScope ps(this, K_SCATTER);
   check(cavs_scatter_rows(dst, ld_dst, ids, inp, ld_inp, n, w, stream_));
   c_scatter_rows_ += n;
   c_scatter_bytes_ += (8.0 * w + 4.0) * n;
@@ -338,17 +393,20 @@ void Engine::treelstm_forward() {
     const size_t off = r.offset;
     float *msg = msg_.at(off * 2 * H);
     if (leaf_round(r)) {
-      check(cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, nullptr, nullptr, nullptr, Bv,
+      CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, nullptr, nullptr, nullptr, Bv,
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
     } else {
       float *G = G_.at(2 * off * 2 * H), *hlr = hlr_.at(off * H);
-      check(cavs_gather_children(G, hlr, pool_.get(), d_child_ + 2 * off, r.n, 2 * H, H, stream_));
+      {
+        ProfScope ps(this, K_GATHER);
+        check(cavs_gather_children(G, hlr, pool_.get(), d_child_ + 2 * off, r.n, 2 * H, H, stream_));
+      }
       c_gather_rows_ += 2.0 * r.n;
       c_gather_bytes_ += 2.0 * r.n * (16.0 * H + 4) + 4.0 * r.n * H;
       c_launches_ += 1;
       gemm(0, 0, r.n, 3 * H, H, hlr, H, U, 3 * H, 0.f, r_hU_.get(), 3 * H);
       gemm(0, 0, 2 * r.n, H, H, G, 2 * H, U + (size_t)3 * H * H, H, 0.f, r_hUf_.get(), H);
-      check(cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, r_hU_.get(), r_hUf_.get(), G, Bv,
+      CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, r_hU_.get(), r_hUf_.get(), G, Bv,
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
     }
     c_launches_ += 1;
@@ -367,19 +425,22 @@ void Engine::treelstm_backward() {
     // grad of Scatter is Gather on the recorded scatter list; rows without an entry read zero
     gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
     if (leaf_round(r)) {
-      check(cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H), nullptr,
+      CAVS_TIMED(K_GATES, cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H), nullptr,
                                     dxW_.at(off * 4 * H), 4 * H, nullptr, nullptr, r.n, H, stream_));
       c_launches_ += 1;
       continue;
     }
     float *dxW = dxW_.at(off * 4 * H), *dF = dF_.at(2 * off * H);
-    check(cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H),
+    CAVS_TIMED(K_GATES, cavs_treelstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 6 * H),
                                   G_.at(2 * off * 2 * H), dxW, 4 * H, dF, r_dG_.get(), r.n, H, stream_));
     c_launches_ += 1;
     // dh_lr = [d_i|d_o|d_u] * U_iou^T ;  dh_{l,r} = dh_lr + d_f{l,r} * U_f^T
     gemm(0, 1, r.n, H, 3 * H, dxW, 4 * H, U, 3 * H, 0.f, r_dhlr_.get(), H);
-    check(cavs_sgemm_addrows(0, 1, 2 * r.n, H, H, dF, H, U + (size_t)3 * H * H, H, r_dhlr_.get(), H, 1,
-                             r_dG_.get(), 2 * H, stream_));
+    {
+      ProfScope ps(this, K_GEMM);
+      check(cavs_sgemm_addrows(0, 1, 2 * r.n, H, H, dF, H, U + (size_t)3 * H * H, H, r_dhlr_.get(), H, 1,
+                               r_dG_.get(), 2 * H, stream_));
+    }
     c_gemm_flops_ += 2.0 * 2 * r.n * H * H;
     c_launches_ += 1;
     // grad of Gather(child) is Scatter on the recorded gather lists
@@ -424,7 +485,7 @@ void Engine::lstm_forward() {
       gather(G, 2 * H, pool_.get(), 2 * H, d_child_ + off, r.n, 2 * H);
       gemm(0, 0, r.n, 4 * H, H, G, 2 * H, Wh, 4 * H, 1.f, a, 4 * H);  // a += h_p * W'
     }
-    check(cavs_lstm_gates_fwd(a, 4 * H, nullptr, G, Bv, gates_.at(off * 5 * H), msg, r.n, H, stream_));
+    CAVS_TIMED(K_GATES, cavs_lstm_gates_fwd(a, 4 * H, nullptr, G, Bv, gates_.at(off * 5 * H), msg, r.n, H, stream_));
     c_launches_ += 1;
     scatter(pool_.get(), 2 * H, d_pair_ + off, msg, 2 * H, r.n, 2 * H);
   }
@@ -440,12 +501,12 @@ void Engine::lstm_backward() {
     gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
     float *da = dxW_.at(off * 4 * H);
     if (leaf_round(r)) {
-      check(cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), nullptr, da, 4 * H,
+      CAVS_TIMED(K_GATES, cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), nullptr, da, 4 * H,
                                 nullptr, r.n, H, stream_));
       c_launches_ += 1;
       continue;
     }
-    check(cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), G_.at(off * 2 * H), da,
+    CAVS_TIMED(K_GATES, cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), G_.at(off * 2 * H), da,
                               4 * H, r_dG_.get(), r.n, H, stream_));
     c_launches_ += 1;
     gemm(0, 1, r.n, H, 4 * H, da, 4 * H, Wh, 4 * H, 0.f, r_dG_.get(), 2 * H);  // dh_p = da * W'^T
@@ -478,15 +539,18 @@ void Engine::treefc_forward() {
     const float *xin = cfg_.use_x ? xs_.at(off * H) : nullptr;
     float *msg = msg_.at(off * H);
     if (leaf_round(r)) {
-      check(cavs_treefc_fwd(nullptr, Bv, xin, msg, r.n, H, cfg_.act, stream_));
+      CAVS_TIMED(K_GATES, cavs_treefc_fwd(nullptr, Bv, xin, msg, r.n, H, cfg_.act, stream_));
     } else {
       float *G = G_.at(2 * off * H);  // row b = [G0 | G1] of vertex b
-      check(cavs_gather_children(G, nullptr, pool_.get(), d_child_ + 2 * off, r.n, H, 0, stream_));
+      {
+        ProfScope ps(this, K_GATHER);
+        check(cavs_gather_children(G, nullptr, pool_.get(), d_child_ + 2 * off, r.n, H, 0, stream_));
+      }
       c_gather_rows_ += 2.0 * r.n;
       c_gather_bytes_ += 2.0 * r.n * (8.0 * H + 4);
       c_launches_ += 1;
       gemm(0, 0, r.n, H, 2 * H, G, 2 * H, W, H, 0.f, r_z_.get(), H);
-      check(cavs_treefc_fwd(r_z_.get(), Bv, xin, msg, r.n, H, cfg_.act, stream_));
+      CAVS_TIMED(K_GATES, cavs_treefc_fwd(r_z_.get(), Bv, xin, msg, r.n, H, cfg_.act, stream_));
     }
     c_launches_ += 1;
     scatter(pool_.get(), H, d_pair_ + off, msg, H, r.n, H);
@@ -502,7 +566,7 @@ void Engine::treefc_backward() {
     const size_t off = r.offset;
     gather(r_dmsg_.get(), H, dpool_.get(), H, d_pair_ + off, r.n, H);
     float *dz = dxW_.at(off * H);
-    check(cavs_treefc_bwd(r_dmsg_.get(), dret_.at(off * H), msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));
+    CAVS_TIMED(K_GATES, cavs_treefc_bwd(r_dmsg_.get(), dret_.at(off * H), msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));
     c_launches_ += 1;
     if (leaf_round(r)) continue;
     gemm(0, 1, r.n, 2 * H, H, dz, H, W, H, 0.f, r_dG_.get(), 2 * H);

@@ -36,6 +36,11 @@ class Engine {
   void fetch(const std::string &what, float *host, size_t n);
   float timing(const std::string &name);
   double counter(const std::string &key) const;
+  // Per-kernel-class device time: when enabled every launch is bracketed by a pair of
+  // events on the session's stream; read() waits for the stream and sums them.
+  enum KernelClass { K_GEMM = 0, K_GATHER, K_SCATTER, K_GATES, K_OTHER, K_CLASSES };
+  void profile_enable(bool on);
+  void profile_read(int cls, double *total_ms, double *launches);
   const Schedule &schedule() const { return sched_; }
   void *stream() const { return stream_; }
   int total_length() const { return sched_.N; }
@@ -65,6 +70,23 @@ class Engine {
   bool leaf_round(const Round &r) const {
     return r.gather_begin[0] == r.gather_end[0] && r.gather_begin[1] == r.gather_end[1];
   }
+
+  struct Span {
+    int cls;
+    void *a, *b;
+  };
+  struct ProfScope {  // brackets the launches made during its lifetime
+    Engine *e;
+    Span s;
+    bool on;
+    ProfScope(Engine *eng, int cls);
+    ~ProfScope();
+  };
+  void *prof_event();
+  bool profile_ = false;
+  std::vector<Span> spans_;
+  std::vector<void *> prof_events_;
+  size_t prof_used_ = 0;
 
   cavs_session_config cfg_;
   void *stream_ = nullptr;

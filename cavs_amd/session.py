@@ -53,6 +53,8 @@ def lib():
             "cavs_schedule_trace": [P, I, I, I, I, P, I],
             "cavs_session_timing": [P, C.c_char_p, C.POINTER(F)],
             "cavs_session_counter": [P, C.c_char_p, C.POINTER(C.c_double)],
+            "cavs_session_profile": [P, I],
+            "cavs_session_profile_read": [P, C.c_char_p, C.POINTER(C.c_double), C.POINTER(C.c_double)],
         }
         for k, a in sigs.items():
             fn = getattr(l, k)
@@ -218,6 +220,16 @@ class Session:
         v = C.c_double()
         _check(lib().cavs_session_counter(self._h, key.encode(), C.byref(v)), f"counter({key})")
         return v.value
+
+    def profile(self, enable):
+        _check(lib().cavs_session_profile(self._h, int(enable)), "cavs_session_profile")
+
+    def profile_read(self, kernel_class):
+        """(total device ms, launches) of a kernel class since profile(True)"""
+        t, n = C.c_double(), C.c_double()
+        _check(lib().cavs_session_profile_read(self._h, kernel_class.encode(), C.byref(t), C.byref(n)),
+               "cavs_session_profile_read")
+        return t.value, n.value
 
     @property
     def stream(self):

@@ -84,6 +84,13 @@ int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int w
 /* Timers of the last step in ms, by the reference's names (cavs/midend/statement.cc:
  * 53,65,68,84,102,122): "GraphParsing" (host), "RNNForward", "RNNBackward" (device). */
 int cavs_session_timing(cavs_session *s, const char *name, float *ms);
+/* Device time per kernel class.  While enabled, every launch of the session is
+ * bracketed by a pair of events on the session's stream; profile_read waits for the
+ * stream and returns the summed elapsed time and launch count since profiling was
+ * enabled.  Classes: "gemm" "gather" "scatter" "gates". */
+int cavs_session_profile(cavs_session *s, int enable);
+int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double *total_ms,
+                              double *launches);
 /* Raw stream the session enqueues on (for callers that want to bracket it with events). */
 void *cavs_session_stream(cavs_session *s);
 /* Per-step counts for roofline accounting: rows moved by indexed copies and GEMM flops
