@@ -1,20 +1,24 @@
 // FP32 GEMM on the CDNA4 matrix cores (v_mfma_f32_32x32x2_f32), row-major, for the
 // gate products of the vertex functions: NN (X*W), NT (dY*W^T) and TN (X^T*dY).
 //
-// Workgroup = 4 wavefronts (2x2) over a BM x BN tile of C, BK = 16 deep.  A and B
+// Workgroup = 4 wavefronts (2x2) over a BM x BN tile of C, BK deep (128x128x16 for
+// problems that fill the chip, 64x64x32 otherwise).  A and B
 // tiles are staged through LDS as [k][m] / [k][n] panels (double buffered, one
 // barrier per k-tile), so each MFMA operand read is a conflict-free ds_read_b32 of
 // 32 consecutive floats per half-wave.  Global loads are 16-byte per lane; the
 // k-contiguous operand (A of NN/NT, B of NT) is transposed on its way into LDS.
 // Workgroup ids are remapped so that consecutive tiles (which share an A row panel)
-// run on the same XCD and hit the same L2.
+// run on the same XCD and hit the same L2.  Products with too few tiles to fill the
+// chip take one of two other routes: skinny ones (the tail rounds of a batch) a
+// kernel whose wavefronts split K inside the workgroup, tall-K ones (the deferred
+// weight gradients) split K over workgroups with the partials reduced in a fixed
+// order by a second kernel.
 #include "common.h"
 
 namespace cavs {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
-constexpr int BK = 16;
 constexpr int PAD = 4;
 constexpr int kThreads = 256;
 
@@ -31,14 +35,16 @@ struct GemmArgs {
   long ldd;
   int dshift;
   int kchunk;      // K range per blockIdx.y (multiple of BK); == K when not split
-  float *ws;       // split-K partials [splits][M][N] or nullptr
+  float *ws;       // split-K workspace (counters + partial tiles) or nullptr
 };
 
 // Loader of one BX x BK operand tile.  KC: the operand's k index is the contiguous
 // one in memory (element (x,k) at P[x*ld + k]); otherwise element at P[k*ld + x].
-template <int BX, bool KC, bool VEC>
+template <int BX, int BK, bool KC, bool VEC>
 struct TileLoader {
   static constexpr int NV = BX * BK / 4 / kThreads;  // float4 per thread
+  static constexpr int KQ = BK / 4;                  // float4 per row of a k-contiguous tile
+  static constexpr int PER = BX / 4;                 // float4 per k row otherwise
   float4 reg[NV];
 
   __device__ inline void load(const float *__restrict__ P, long ld, int x0, int k0, int X,
@@ -46,21 +52,18 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       int gx, gk;
-      long off, step;
+      long off;
       bool xin[4], kin[4];
       if constexpr (KC) {
-        gx = x0 + tid / 4 + 64 * i;
-        gk = k0 + 4 * (tid % 4);
+        gx = x0 + tid / KQ + (kThreads / KQ) * i;
+        gk = k0 + 4 * (tid % KQ);
         off = (long)gx * ld + gk;
-        step = 1;
 #pragma unroll
         for (int c = 0; c < 4; c++) { xin[c] = gx < X; kin[c] = gk + c < Kend; }
       } else {
-        constexpr int PER = BX / 4;  // float4 per k row
         gk = k0 + tid / PER + (kThreads / PER) * i;
         gx = x0 + 4 * (tid % PER);
         off = (long)gk * ld + gx;
-        step = 1;
 #pragma unroll
         for (int c = 0; c < 4; c++) { xin[c] = gx + c < X; kin[c] = gk < Kend; }
       }
@@ -70,9 +73,9 @@ struct TileLoader {
         if (xin[0] && kin[0]) v = *reinterpret_cast<const float4 *>(P + off);
       } else {
         if (xin[0] && kin[0]) v.x = P[off];
-        if (xin[1] && kin[1]) v.y = P[off + step];
-        if (xin[2] && kin[2]) v.z = P[off + 2 * step];
-        if (xin[3] && kin[3]) v.w = P[off + 3 * step];
+        if (xin[1] && kin[1]) v.y = P[off + 1];
+        if (xin[2] && kin[2]) v.z = P[off + 2];
+        if (xin[3] && kin[3]) v.w = P[off + 3];
       }
       reg[i] = v;
     }
@@ -83,13 +86,12 @@ struct TileLoader {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       if constexpr (KC) {
-        int x = tid / 4 + 64 * i, k = 4 * (tid % 4);
+        int x = tid / KQ + (kThreads / KQ) * i, k = 4 * (tid % KQ);
         S[(k + 0) * LD + x] = reg[i].x;
         S[(k + 1) * LD + x] = reg[i].y;
         S[(k + 2) * LD + x] = reg[i].z;
         S[(k + 3) * LD + x] = reg[i].w;
       } else {
-        constexpr int PER = BX / 4;
         int k = tid / PER + (kThreads / PER) * i, x = 4 * (tid % PER);
         *reinterpret_cast<float4 *>(S + k * LD + x) = reg[i];
       }
@@ -106,7 +108,7 @@ __device__ inline int xcd_remap(int l, int total) {
   return xcd * per + (xcd < rem ? xcd : rem) + local;
 }
 
-template <int BM, int BN, bool TA, bool TB, bool VEC>
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
 __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int LDA = BM + PAD, LDB = BN + PAD;
@@ -121,8 +123,8 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
   const int kbeg = blockIdx.y * g.kchunk;
   const int kend = min(g.K, kbeg + g.kchunk);
 
-  TileLoader<BM, !TA, VEC> la;
-  TileLoader<BN, TB, VEC> lb;
+  TileLoader<BM, BK, !TA, VEC> la;
+  TileLoader<BN, BK, TB, VEC> lb;
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -170,8 +172,6 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
 
   // C layout of the 32x32 accumulator: element r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32.
-  float *out = g.ws ? g.ws + (long)blockIdx.y * g.M * g.N : g.C;
-  const long ldo = g.ws ? g.N : g.ldc;
 #pragma unroll
   for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -182,45 +182,184 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
       for (int r = 0; r < 16; r++) {
         const int row = m0 + wm * WM + 32 * i + 8 * (r / 4) + 4 * khalf + (r % 4);
         if (row >= g.M) continue;
-        float v = acc[i][j][r];
-        if (!g.ws) {
-          v *= g.alpha;
-          if (g.beta != 0.f) v += g.beta * out[row * ldo + col];
-          if (g.D) v += g.D[(long)(row >> g.dshift) * g.ldd + col];
+        if (g.ws) {  // split K: park the partial sum, the reduce kernel finishes the job
+          g.ws[((long)blockIdx.y * g.M + row) * g.N + col] = acc[i][j][r];
+          continue;
         }
-        out[row * ldo + col] = v;
+        float v = g.alpha * acc[i][j][r];
+        if (g.beta != 0.f) v += g.beta * g.C[row * g.ldc + col];
+        if (g.D) v += g.D[(long)(row >> g.dshift) * g.ldd + col];
+        g.C[row * g.ldc + col] = v;
       }
     }
 }
 
-// C = alpha * sum_z ws[z] + beta * C, z ascending (fixed order: deterministic)
-__global__ void splitk_reduce_kernel(const float *__restrict__ ws, int splits, int M, int N,
-                                     float alpha, float beta, float *__restrict__ C, long ldc) {
+
+// C = alpha * sum_z ws[z] + beta * C (+ D rows), z ascending: a fixed order, so the
+// result does not depend on how the workgroups were scheduled.
+__global__ void splitk_reduce_kernel(GemmArgs g, int splits) {
   long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  long total = (long)M * N;
+  long total = (long)g.M * g.N;
   if (idx >= total) return;
   float acc = 0.f;
-  for (int z = 0; z < splits; z++) acc += ws[(long)z * total + idx];
-  int r = (int)(idx / N), c = (int)(idx % N);
-  float v = alpha * acc;
-  if (beta != 0.f) v += beta * C[r * ldc + c];
-  C[r * ldc + c] = v;
+  for (int z = 0; z < splits; z++) acc += g.ws[(long)z * total + idx];
+  int r = (int)(idx / g.N), c = (int)(idx % g.N);
+  float v = g.alpha * acc;
+  if (g.beta != 0.f) v += g.beta * g.C[r * g.ldc + c];
+  if (g.D) v += g.D[(long)(r >> g.dshift) * g.ldd + c];
+  g.C[r * g.ldc + c] = v;
 }
 
-template <int BM, int BN>
-static void launch_tile(const GemmArgs &g, int tA, int tB, bool vec, int splits, hipStream_t st) {
-  int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-  dim3 grid(tiles, splits), block(kThreads);
-#define CAVS_GEMM_CASE(TA, TB)                                                                   \
-  if (vec)                                                                                       \
-    sgemm_mfma_kernel<BM, BN, TA, TB, true><<<grid, block, 0, st>>>(g);                           \
-  else                                                                                           \
-    sgemm_mfma_kernel<BM, BN, TA, TB, false><<<grid, block, 0, st>>>(g)
-  if (!tA && !tB) { CAVS_GEMM_CASE(false, false); }
-  else if (!tA && tB) { CAVS_GEMM_CASE(false, true); }
-  else if (tA && !tB) { CAVS_GEMM_CASE(true, false); }
-  else { CAVS_GEMM_CASE(true, true); }
-#undef CAVS_GEMM_CASE
+// Skinny products (few rows: the tail rounds of a batch).  Such a product is a
+// latency chain, not a throughput problem: the weights must stream past a handful of
+// rows.  One workgroup owns a (32*TM) x 32 tile of C and its W wavefronts split K
+// between them; every wavefront feeds the MFMA straight from global memory (the B
+// operand of a 32x32x2 step is 32 consecutive floats per half-wave, so no LDS staging
+// is needed) with several k-groups in flight, and the W partial tiles are summed
+// through LDS in wavefront order (deterministic).  A is [M,K] row-major; B is [K,N]
+// (TB = false) or [N,K] (TB = true).  Needs K, lda (and ldb when TB) multiples of 4.
+template <int TM, bool TB, int W>
+__global__ __launch_bounds__(W * 64) void sgemm_skinny_kernel(GemmArgs g) {
+  constexpr int U = 4;  // k-groups of 8 in flight
+  __shared__ float red[TM * 16 * 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j = lane & 31, h = lane >> 5;
+  const int n0 = blockIdx.x * 32, m0 = blockIdx.y * 32 * TM;
+  const int kper = ((g.K + W - 1) / W + 7) / 8 * 8;
+  const int kb = wave * kper, ke = min(g.K, kb + kper);
+  const bool col_ok = n0 + j < g.N;
+
+  floatx16 acc[TM];
+#pragma unroll
+  for (int t = 0; t < TM; t++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+
+  // one stage = U groups of 8 k values; the next stage's operands are fetched before
+  // the MFMAs of the current one are issued, so memory latency overlaps the matrix pipe
+  auto fetch = [&](int k0, float4 (&a)[U][TM], float (&b)[U][4]) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+      const int kk = k0 + 8 * u + 4 * h;
+      const bool kin = kk < ke;
+#pragma unroll
+      for (int t = 0; t < TM; t++) {
+        const int row = m0 + 32 * t + j;
+        a[u][t] = (kin && row < g.M) ? *reinterpret_cast<const float4 *>(g.A + (long)row * g.lda + kk)
+                                     : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+      if constexpr (TB) {
+        float4 q = (kin && col_ok) ? *reinterpret_cast<const float4 *>(g.B + (long)(n0 + j) * g.ldb + kk)
+                                   : make_float4(0.f, 0.f, 0.f, 0.f);
+        b[u][0] = q.x; b[u][1] = q.y; b[u][2] = q.z; b[u][3] = q.w;
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          b[u][c] = (col_ok && kk + c < ke) ? g.B[(long)(kk + c) * g.ldb + n0 + j] : 0.f;
+      }
+    }
+  };
+  auto multiply = [&](const float4 (&a)[U][TM], const float (&b)[U][4]) {
+#pragma unroll
+    for (int u = 0; u < U; u++)
+#pragma unroll
+      for (int t = 0; t < TM; t++) {
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t].x, b[u][0], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t].y, b[u][1], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t].z, b[u][2], acc[t], 0, 0, 0);
+        acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[u][t].w, b[u][3], acc[t], 0, 0, 0);
+      }
+  };
+  float4 a0[U][TM], a1[U][TM];
+  float b0[U][4], b1[U][4];
+  constexpr int S = 8 * U;
+  if (kb < ke) fetch(kb, a0, b0);
+  for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+    if (k0 + S < ke) fetch(k0 + S, a1, b1);
+    multiply(a0, b0);
+    if (k0 + S < ke) {
+      if (k0 + 2 * S < ke) fetch(k0 + 2 * S, a0, b0);
+      multiply(a1, b1);
+    }
+  }
+
+  // sum the W partial tiles in wavefront order
+  for (int w = 0; w < W; w++) {
+    if (wave == w) {
+#pragma unroll
+      for (int t = 0; t < TM; t++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float *p = red + (t * 16 + r) * 64 + lane;
+          *p = (w == 0) ? acc[t][r] : *p + acc[t][r];
+        }
+    }
+    __syncthreads();
+  }
+  // epilogue: the W*64 threads share the TM*1024 outputs; element (t, r, lane') sits at
+  // row 32t + 8(r/4) + 4(lane'/32) + r%4, column lane'%32
+  for (int e = tid; e < TM * 1024; e += W * 64) {
+    const int l2 = e & 63, r = (e >> 6) & 15, t = e >> 10;
+    const int row = m0 + 32 * t + 8 * (r / 4) + 4 * (l2 >> 5) + (r % 4), col = n0 + (l2 & 31);
+    if (row >= g.M || col >= g.N) continue;
+    float v = g.alpha * red[e];
+    if (g.beta != 0.f) v += g.beta * g.C[row * g.ldc + col];
+    if (g.D) v += g.D[(long)(row >> g.dshift) * g.ldd + col];
+    g.C[row * g.ldc + col] = v;
+  }
+}
+
+struct GemmPlan {
+  enum Kind { TILE128, TILE64, SKINNY } kind;
+  int splits;   // > 1: partial tiles to the workspace + reduce kernel (TILE64 only)
+  int kchunk;
+  long tiles;
+};
+
+static bool skinny_ok(int tA, int tB, int K, const float *A, int lda, const float *B, int ldb) {
+  if (tA || K % 4 || lda % 4 || !aligned16(A)) return false;
+  if (tB && (ldb % 4 || !aligned16(B))) return false;
+  return true;
+}
+
+static GemmPlan plan_gemm(int tA, int tB, int M, int N, int K, bool skinny_allowed, bool allow_split) {
+  GemmPlan p;
+  const long cus = num_cus();
+  const long t128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const long t64 = (long)((M + 63) / 64) * ((N + 63) / 64);
+  p.splits = 1;
+  p.kchunk = K > 0 ? K : 1;
+  if (t128 >= cus) {
+    p.kind = GemmPlan::TILE128;
+    p.tiles = t128;
+    return p;
+  }
+  p.kind = GemmPlan::TILE64;
+  p.tiles = t64;
+  if (t64 >= 2 * cus || K < 64) return p;
+  if (skinny_allowed) {
+    p.kind = GemmPlan::SKINNY;
+    return p;
+  }
+  if (allow_split && K >= 256) {
+    long want = (3 * cus + t64 - 1) / t64;
+    long maxs = K / 128;  // at least four k-tiles per split
+    long s = want < maxs ? want : maxs;
+    if (s > 32) s = 32;
+    if (s > 1) {
+      int kchunk = (int)(((K + s - 1) / s + 31) / 32 * 32);
+      int splits = (K + kchunk - 1) / kchunk;
+      if (splits > 1) {
+        p.splits = splits;
+        p.kchunk = kchunk;
+      }
+    }
+  }
+  return p;
+}
+
+static size_t plan_workspace(const GemmPlan &p, int M, int N) {
+  return p.splits > 1 ? sizeof(float) * (size_t)p.splits * M * N : 0;
 }
 
 static bool vec_path_ok(const GemmArgs &g, int tA, int tB) {
@@ -231,13 +370,19 @@ static bool vec_path_ok(const GemmArgs &g, int tA, int tB) {
   return true;
 }
 
-static void launch_gemm(const GemmArgs &g, int tA, int tB, int splits, hipStream_t st) {
-  bool vec = vec_path_ok(g, tA, tB);
-  long big_tiles = (long)((g.M + 127) / 128) * ((g.N + 127) / 128) * splits;
-  if (big_tiles >= num_cus())
-    launch_tile<128, 128>(g, tA, tB, vec, splits, st);
-  else
-    launch_tile<64, 64>(g, tA, tB, vec, splits, st);
+template <int BM, int BN, int BK>
+static void launch_tile(const GemmArgs &g, int tA, int tB, bool vec, const GemmPlan &p, hipStream_t st) {
+  dim3 grid((unsigned)p.tiles, p.splits), block(kThreads);
+#define CAVS_GEMM_CASE(TA, TB)                                                  \
+  if (vec)                                                                      \
+    sgemm_mfma_kernel<BM, BN, BK, TA, TB, true><<<grid, block, 0, st>>>(g);      \
+  else                                                                          \
+    sgemm_mfma_kernel<BM, BN, BK, TA, TB, false><<<grid, block, 0, st>>>(g)
+  if (!tA && !tB) { CAVS_GEMM_CASE(false, false); }
+  else if (!tA && tB) { CAVS_GEMM_CASE(false, true); }
+  else if (tA && !tB) { CAVS_GEMM_CASE(true, false); }
+  else { CAVS_GEMM_CASE(true, true); }
+#undef CAVS_GEMM_CASE
 }
 
 static int check_gemm(const char *who, int tA, int tB, int M, int N, int K, const float *A, int lda,
@@ -253,15 +398,48 @@ static int check_gemm(const char *who, int tA, int tB, int M, int N, int K, cons
   return CAVS_OK;
 }
 
-static int choose_splits(int M, int N, int K) {
-  long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  int cus = num_cus();
-  if (tiles >= cus || K < 4 * BK) return 1;
-  long want = (2L * cus + tiles - 1) / tiles;
-  long maxs = K / (2 * BK);
-  long s = want < maxs ? want : maxs;
-  if (s > 64) s = 64;
-  return s < 1 ? 1 : (int)s;
+template <bool TB>
+static void launch_skinny(const GemmArgs &g, hipStream_t st) {
+  constexpr int W = 8;
+  if (g.M <= 32) {
+    dim3 grid((g.N + 31) / 32, 1);
+    sgemm_skinny_kernel<1, TB, W><<<grid, W * 64, 0, st>>>(g);
+  } else {
+    dim3 grid((g.N + 31) / 32, (g.M + 63) / 64);
+    sgemm_skinny_kernel<2, TB, W><<<grid, W * 64, 0, st>>>(g);
+  }
+}
+
+static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float alpha, const float *A,
+                    int lda, const float *B, int ldb, float beta, float *C, int ldc, const float *D,
+                    int ldd, int dshift, void *ws, size_t ws_bytes, void *stream) {
+  int rc = check_gemm(who, tA, tB, M, N, K, A, lda, B, ldb, C, ldc);
+  if (rc || M == 0 || N == 0) return rc;
+  GemmPlan p = plan_gemm(tA, tB, M, N, K, skinny_ok(tA, tB, K, A, lda, B, ldb), ws != nullptr);
+  hipStream_t st = as_stream(stream);
+  GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, D, ldd, dshift, p.kchunk, nullptr};
+  if (p.kind == GemmPlan::SKINNY) {
+    if (tB) launch_skinny<true>(g, st); else launch_skinny<false>(g, st);
+    CAVS_LAUNCH_CHECK();
+    return CAVS_OK;
+  }
+  if (p.splits > 1) {
+    size_t need = plan_workspace(p, M, N);
+    CAVS_REQUIRE(ws_bytes >= need && aligned16(ws), "%s: workspace of %zu bytes needed, %zu given", who, need, ws_bytes);
+    g.ws = static_cast<float *>(ws);
+  }
+  bool vec = vec_path_ok(g, tA, tB);
+  if (p.kind == GemmPlan::TILE128)
+    launch_tile<128, 128, 16>(g, tA, tB, vec, p, st);
+  else
+    launch_tile<64, 64, 32>(g, tA, tB, vec, p, st);
+  CAVS_LAUNCH_CHECK();
+  if (p.splits > 1) {
+    long total = (long)M * N;
+    splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(g, p.splits);
+    CAVS_LAUNCH_CHECK();
+  }
+  return CAVS_OK;
 }
 
 }  // namespace cavs
@@ -272,59 +450,30 @@ extern "C" {
 
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                const float *B, int ldb, float beta, float *C, int ldc, void *stream) {
-  int rc = check_gemm("cavs_sgemm", transA, transB, M, N, K, A, lda, B, ldb, C, ldc);
-  if (rc || M == 0 || N == 0) return rc;
-  GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, 0, K > 0 ? K : 1, nullptr};
-  launch_gemm(g, transA, transB, 1, as_stream(stream));
-  CAVS_LAUNCH_CHECK();
-  return CAVS_OK;
+  return run_gemm("cavs_sgemm", transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc, nullptr, 0,
+                  0, nullptr, 0, stream);
 }
 
 int cavs_sgemm_addrows(int transA, int transB, int M, int N, int K, const float *A, int lda,
                        const float *B, int ldb, const float *D, int ldd, int d_shift, float *C,
-                       int ldc, void *stream) {
-  int rc = check_gemm("cavs_sgemm_addrows", transA, transB, M, N, K, A, lda, B, ldb, C, ldc);
-  if (rc || M == 0 || N == 0) return rc;
-  CAVS_REQUIRE(D && ldd >= N && d_shift >= 0 && d_shift < 31, "cavs_sgemm_addrows: bad addend (ldd=%d shift=%d)", ldd, d_shift);
-  GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, 1.f, 0.f, D, ldd, d_shift, K > 0 ? K : 1, nullptr};
-  launch_gemm(g, transA, transB, 1, as_stream(stream));
-  CAVS_LAUNCH_CHECK();
-  return CAVS_OK;
+                       int ldc, void *workspace, size_t workspace_bytes, void *stream) {
+  if (M > 0 && N > 0)
+    CAVS_REQUIRE(D && ldd >= N && d_shift >= 0 && d_shift < 31, "cavs_sgemm_addrows: bad addend (ldd=%d shift=%d)", ldd, d_shift);
+  return run_gemm("cavs_sgemm_addrows", transA, transB, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, D, ldd,
+                  d_shift, workspace, workspace_bytes, stream);
 }
 
 size_t cavs_sgemm_splitk_workspace(int M, int N, int K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  int s = choose_splits(M, N, K);
-  return s > 1 ? (size_t)s * M * N * sizeof(float) : 0;
+  // sized for the split plan whether or not a given call ends up taking the skinny path
+  return plan_workspace(plan_gemm(0, 0, M, N, K, false, true), M, N);
 }
 
 int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                       int lda, const float *B, int ldb, float beta, float *C, int ldc,
                       void *workspace, size_t workspace_bytes, void *stream) {
-  int rc = check_gemm("cavs_sgemm_splitk", transA, transB, M, N, K, A, lda, B, ldb, C, ldc);
-  if (rc || M == 0 || N == 0) return rc;
-  int splits = K > 0 ? choose_splits(M, N, K) : 1;
-  hipStream_t st = as_stream(stream);
-  if (splits <= 1) {
-    GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, 0, K > 0 ? K : 1, nullptr};
-    launch_gemm(g, transA, transB, 1, st);
-    CAVS_LAUNCH_CHECK();
-    return CAVS_OK;
-  }
-  size_t need = (size_t)splits * M * N * sizeof(float);
-  CAVS_REQUIRE(workspace && workspace_bytes >= need && aligned16(workspace),
-               "cavs_sgemm_splitk: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
-  int kchunk = ((K + splits - 1) / splits + BK - 1) / BK * BK;
-  splits = (K + kchunk - 1) / kchunk;
-  GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, nullptr, 0, 0, kchunk,
-             static_cast<float *>(workspace)};
-  launch_gemm(g, transA, transB, splits, st);
-  CAVS_LAUNCH_CHECK();
-  long total = (long)M * N;
-  splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(
-      static_cast<const float *>(workspace), splits, M, N, alpha, beta, C, ldc);
-  CAVS_LAUNCH_CHECK();
-  return CAVS_OK;
+  return run_gemm("cavs_sgemm_splitk", transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc,
+                  nullptr, 0, 0, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -143,27 +143,28 @@ void Engine::profile_read(int cls, double *total_ms, double *launches) {
 }
 
 // ------------------------------------------------------------------ counted wrappers
+// All GEMMs go through the workspace-assisted entry point, which picks the kernel by
+// shape (full tiles, skinny, or split K through the workspace).
+float *Engine::workspace(size_t bytes) {
+  if (ws_.capacity() * 4 < bytes) {
+    check(cavs_stream_sync(stream_));  // the old workspace may still be in use
+    ws_.reserve(std::max<size_t>(bytes / 4 + 1, (size_t)8 << 20));
+  }
+  return ws_.get();
+}
+
 void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
                   int ldb, float beta, float *C, int ldc) {
+  float *ws = workspace(cavs_sgemm_splitk_workspace(M, N, K));
   ProfScope ps(this, K_GEMM);
-  check(cavs_sgemm(tA, tB, M, N, K, 1.f, A, lda, B, ldb, beta, C, ldc, stream_));
+  check(cavs_sgemm_splitk(tA, tB, M, N, K, 1.f, A, lda, B, ldb, beta, C, ldc, ws, ws_.capacity() * 4, stream_));
   c_gemm_flops_ += 2.0 * M * N * K;
   c_launches_ += 1;
 }
 
 void Engine::gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda,
                          const float *B, int ldb, float *C, int ldc) {
-  size_t need = cavs_sgemm_splitk_workspace(M, N, K);
-  ProfScope ps(this, K_GEMM);
-  if (ws_.capacity() * 4 < need) {
-    // the workspace may still be in use by an enqueued GEMM
-    check(cavs_stream_sync(stream_));
-    ws_.reserve(need / 4 + 1);
-  }
-  check(cavs_sgemm_splitk(tA, tB, M, N, K, 1.f, A, lda, B, ldb, 0.f, C, ldc, ws_.get(),
-                          ws_.capacity() * 4, stream_));
-  c_gemm_flops_ += 2.0 * M * N * K;
-  c_launches_ += need ? 2 : 1;
+  gemm(tA, tB, M, N, K, A, lda, B, ldb, 0.f, C, ldc);
 }
 
 void Engine::gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n,
@@ -437,9 +438,10 @@ void Engine::treelstm_backward() {
     // dh_lr = [d_i|d_o|d_u] * U_iou^T ;  dh_{l,r} = dh_lr + d_f{l,r} * U_f^T
     gemm(0, 1, r.n, H, 3 * H, dxW, 4 * H, U, 3 * H, 0.f, r_dhlr_.get(), H);
     {
+      float *ws = workspace(cavs_sgemm_splitk_workspace(2 * r.n, H, H));
       ProfScope ps(this, K_GEMM);
       check(cavs_sgemm_addrows(0, 1, 2 * r.n, H, H, dF, H, U + (size_t)3 * H * H, H, r_dhlr_.get(), H, 1,
-                               r_dG_.get(), 2 * H, stream_));
+                               r_dG_.get(), 2 * H, ws, ws_.capacity() * 4, stream_));
     }
     c_gemm_flops_ += 2.0 * 2 * r.n * H * H;
     c_launches_ += 1;

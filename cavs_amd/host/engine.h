@@ -61,6 +61,7 @@ class Engine {
   void pop_ret();
   void head_forward_backward(bool backward);
   // counted wrappers
+  float *workspace(size_t bytes);
   void gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B, int ldb,
             float beta, float *C, int ldc);
   void gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,

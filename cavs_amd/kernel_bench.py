@@ -1,0 +1,148 @@
+#!/usr/bin/env python3
+"""Per-kernel roofline measurements through the C ABI (no model around the kernels).
+
+    python -m cavs_amd.kernel_bench [--set copies|gemm|gates|all] [--iters 50]
+
+For each case: launches the entry point `iters` times back to back on one stream between two
+HIP events and reports the average duration per launch, the algorithmic bytes / flops
+per launch and the fraction of the MI355X roofline (HBM 8 TB/s, FP32 MFMA 157.3 TFLOP/s).
+Shapes are the ones the benchmark configurations produce (C3: H=512, C5: H=1024).
+One JSON object per line.
+"""
+import argparse
+import ctypes as C
+import json
+
+import torch
+
+from . import hip
+
+HBM_GBS = 8000.0
+MFMA_TF = 157.3
+
+
+def _time(fn, iters, stream):
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    hip.call("cavs_event_create", C.byref(e0))
+    hip.call("cavs_event_create", C.byref(e1))
+    for _ in range(3):
+        fn()
+    hip.call("cavs_stream_sync", stream)
+    hip.call("cavs_event_record", e0, stream)
+    for _ in range(iters):
+        fn()
+    hip.call("cavs_event_record", e1, stream)
+    ms = C.c_float()
+    hip.call("cavs_event_elapsed_ms", C.byref(ms), e0, e1)
+    hip.call("cavs_event_destroy", e0)
+    hip.call("cavs_event_destroy", e1)
+    return ms.value * 1e3 / iters  # us per launch
+
+
+def _emit(kernel, shape, us, nbytes=None, flops=None):
+    rec = dict(kernel=kernel, shape=shape, us_per_launch=round(us, 3))
+    if nbytes is not None:
+        gbs = nbytes / us / 1e3
+        rec.update(bound="hbm", bytes_per_launch=int(nbytes), achieved_GBs=round(gbs, 1),
+                   frac=round(gbs / HBM_GBS, 4))
+    if flops is not None:
+        tf = flops / us / 1e6
+        rec.update(bound="mfma", flops_per_launch=int(flops), achieved_TFLOPs=round(tf, 2),
+                   frac=round(tf / MFMA_TF, 4))
+    print(json.dumps(rec), flush=True)
+
+
+def copies(iters, st):
+    f32 = dict(dtype=torch.float32, device="cuda")
+    for n, w, tag in [(600, 1024, "C3 round"), (2482, 1024, "C3 all rows"), (16384, 2048, "C5 round"),
+                      (65536, 2048, "C5 leaf round"), (131072, 1024, "wide batch")]:
+        rows = 2 * n
+        src = torch.randn(rows, w, **f32)
+        out = torch.empty(n, w, **f32)
+        g = torch.Generator(device="cpu").manual_seed(n)
+        ids = torch.randperm(rows, generator=g)[:n].to(torch.int32).cuda()
+        nbytes = n * (8 * w + 4)
+        us = _time(lambda: hip.call("cavs_gather_rows", out.data_ptr(), w, src.data_ptr(), w, ids.data_ptr(),
+                                    n, w, st), iters, st)
+        _emit("gather_rows", f"{tag}: n={n} w={w}", us, nbytes=nbytes)
+        dst = torch.empty(rows, w, **f32)
+        us = _time(lambda: hip.call("cavs_scatter_rows", dst.data_ptr(), w, ids.data_ptr(), out.data_ptr(), w,
+                                    n, w, st), iters, st)
+        _emit("scatter_rows", f"{tag}: n={n} w={w}", us, nbytes=nbytes)
+        us = _time(lambda: hip.call("cavs_copy_rows", out.data_ptr(), w, src.data_ptr(), w, n, w, st), iters, st)
+        _emit("copy_rows", f"{tag}: n={n} w={w}", us, nbytes=n * 8 * w)
+        if n % 2 == 0:
+            m = n // 2
+            G = torch.empty(2 * m, w, **f32)
+            hs = torch.empty(m, w // 2, **f32)
+            us = _time(lambda: hip.call("cavs_gather_children", G.data_ptr(), hs.data_ptr(), src.data_ptr(),
+                                        ids.data_ptr(), m, w, w // 2, st), iters, st)
+            _emit("gather_children", f"{tag}: vertices={m} w={w}", us, nbytes=2 * m * (8 * w + 4) + 4 * m * (w // 2))
+
+
+def gemm(iters, st):
+    f32 = dict(dtype=torch.float32, device="cuda")
+    cases = []
+    for H, E, N, tag in [(512, 300, 2482, "C3"), (1024, 1024, 73000, "C5")]:
+        n = 600 if H == 512 else 16384
+        cases += [
+            (0, 0, N, 4 * H, E, f"{tag} x*W all rows"),
+            (0, 0, n, 3 * H, H, f"{tag} round h_lr*U_iou"),
+            (0, 0, 2 * n, H, H, f"{tag} round [h_l;h_r]*U_f"),
+            (0, 1, n, H, 3 * H, f"{tag} round d(hU)*U_iou^T"),
+            (0, 1, 2 * n, H, H, f"{tag} round dF*U_f^T"),
+            (0, 1, N, E, 4 * H, f"{tag} de = dxW*W^T"),
+            (1, 0, E, 4 * H, N, f"{tag} dW = e^T*dxW"),
+            (1, 0, H, 3 * H, N // 2, f"{tag} dU_iou = h_lr^T*d(hU)"),
+        ]
+    cases += [(0, 0, 32, 1536, 512, "C3 tail round (32 rows)"), (0, 0, 8192, 8192, 8192, "square 8192")]
+    for tA, tB, M, Nn, K, tag in cases:
+        A = torch.randn((K, M) if tA else (M, K), **f32)
+        B = torch.randn((Nn, K) if tB else (K, Nn), **f32)
+        Cm = torch.empty(M, Nn, **f32)
+        nb = hip.lib().cavs_sgemm_splitk_workspace(M, Nn, K)
+        ws = torch.empty(max(nb // 4, 4), **f32)
+        us = _time(lambda: hip.call("cavs_sgemm_splitk", tA, tB, M, Nn, K, 1.0, A.data_ptr(), A.shape[1],
+                                    B.data_ptr(), B.shape[1], 0.0, Cm.data_ptr(), Nn, ws.data_ptr(), nb, st),
+                   max(5, iters // 5) if M * Nn * K > 1e11 else iters, st)
+        _emit("sgemm", f"{tag}: {'T' if tA else 'N'}{'T' if tB else 'N'} M={M} N={Nn} K={K}", us,
+              flops=2.0 * M * Nn * K)
+        del A, B, Cm, ws
+
+
+def gates(iters, st):
+    f32 = dict(dtype=torch.float32, device="cuda")
+    for n, H, tag in [(600, 512, "C3 round"), (16384, 1024, "C5 round")]:
+        xW, hU, hUf = torch.randn(n, 4 * H, **f32), torch.randn(n, 3 * H, **f32), torch.randn(2 * n, H, **f32)
+        G, bias = torch.randn(2 * n, 2 * H, **f32), torch.randn(4 * H, **f32)
+        gt, msg = torch.empty(n, 6 * H, **f32), torch.empty(n, 2 * H, **f32)
+        us = _time(lambda: hip.call("cavs_treelstm_gates_fwd", xW.data_ptr(), 4 * H, hU.data_ptr(), hUf.data_ptr(),
+                                    G.data_ptr(), bias.data_ptr(), gt.data_ptr(), msg.data_ptr(), n, H, st), iters, st)
+        _emit("treelstm_gates_fwd", f"{tag}: n={n} H={H}", us, nbytes=4 * n * H * 21 + 16 * H)
+        dmsg, dret = torch.randn(n, 2 * H, **f32), torch.randn(n, H, **f32)
+        dxW, dF, dG = torch.empty(n, 4 * H, **f32), torch.empty(2 * n, H, **f32), torch.empty(2 * n, 2 * H, **f32)
+        us = _time(lambda: hip.call("cavs_treelstm_gates_bwd", dmsg.data_ptr(), dret.data_ptr(), gt.data_ptr(),
+                                    G.data_ptr(), dxW.data_ptr(), 4 * H, dF.data_ptr(), dG.data_ptr(), n, H, st),
+                   iters, st)
+        # reads dmsg 2H, dret H, gates 6H, c_l c_r 2H; writes dxW 4H, dF 2H, dc_l dc_r 2H
+        _emit("treelstm_gates_bwd", f"{tag}: n={n} H={H}", us, nbytes=4 * n * H * 19)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--set", default="all", choices=["copies", "gemm", "gates", "all"])
+    ap.add_argument("--iters", type=int, default=50)
+    a = ap.parse_args()
+    assert torch.cuda.is_available(), "kernel_bench needs the MI355X"
+    hip.call("cavs_init", 0)
+    st = torch.cuda.current_stream().cuda_stream
+    if a.set in ("copies", "all"):
+        copies(a.iters, st)
+    if a.set in ("gemm", "all"):
+        gemm(a.iters, st)
+    if a.set in ("gates", "all"):
+        gates(a.iters, st)
+
+
+if __name__ == "__main__":
+    main()

@@ -97,20 +97,23 @@ int cavs_gather_children(float *G, float *hsum, const float *pool, const int *id
  * gradients (cavs/backend/op_decl_matmul.cc:18-69).  op(A) is M x K. */
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                int lda, const float *B, int ldb, float beta, float *C, int ldc, void *stream);
-/* C[r,:] = op(A)*op(B) + D[r >> d_shift, :]: the GEMM and the Accumulate that
- * follows it in the backward of a Mirror'ed operand
- * (cavs/backend/op_decl_slice_join.cc:173-182) in one pass. */
-int cavs_sgemm_addrows(int transA, int transB, int M, int N, int K, const float *A, int lda,
-                       const float *B, int ldb, const float *D, int ldd, int d_shift, float *C,
-                       int ldc, void *stream);
-/* Bytes of device workspace cavs_sgemm_splitk needs for this shape. */
+/* Bytes of device workspace the two workspace-assisted forms below need for this
+ * shape (0 when K is not split). */
 size_t cavs_sgemm_splitk_workspace(int M, int N, int K);
-/* Same contract as cavs_sgemm for tall-K products (the deferred weight-gradient
- * GEMMs of cavs/midend/batch_weight_updater.h:12-84): K is split over workgroups,
- * partials go to `workspace` and are reduced in a fixed order (deterministic). */
+/* Same contract as cavs_sgemm for tall-K products with too few output tiles to fill
+ * the chip (the deferred weight-gradient GEMMs of
+ * cavs/midend/batch_weight_updater.h:12-84): K is split over workgroups, partials go
+ * to `workspace` and a second kernel adds them in split order (deterministic).  One
+ * call at a time per workspace.  workspace may be NULL (then K is never split). */
 int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                       int lda, const float *B, int ldb, float beta, float *C, int ldc,
                       void *workspace, size_t workspace_bytes, void *stream);
+/* C[r,:] = op(A)*op(B) + D[r >> d_shift, :]: the GEMM and the Accumulate that
+ * follows it in the backward of a Mirror'ed operand
+ * (cavs/backend/op_decl_slice_join.cc:173-182) in one pass.  Workspace as above. */
+int cavs_sgemm_addrows(int transA, int transB, int M, int N, int K, const float *A, int lda,
+                       const float *B, int ldb, const float *D, int ldd, int d_shift, float *C,
+                       int ldc, void *workspace, size_t workspace_bytes, void *stream);
 /* out[j] (+)= sum_r inp[r, j], j in [0,w): UnaryBroadcastingKernel
  * (cavs/backend/op_impl_elementwise.cuh:24-34) used for bias gradients. */
 int cavs_colsum(float *out, const float *inp, int ld, int n, int w, int accumulate,

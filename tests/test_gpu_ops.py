@@ -148,7 +148,7 @@ def test_sgemm_strided_operands_and_addrows(g, oracle):
     dG0 = r.bulk_normal(2 * n * 2 * H).reshape(2 * n, 2 * H)
     dG = g.devf(dG0)
     g.call("cavs_sgemm_addrows", 0, 1, 2 * n, H, H, g.P(g.devf(dF)), H, g.P(g.devf(Uf)), H,
-           g.P(g.devf(dhlr)), H, 1, g.P(dG), 2 * H, g.stream())
+           g.P(g.devf(dhlr)), H, 1, g.P(dG), 2 * H, None, 0, g.stream())
     want = dG0.copy()
     want[:, :H] = oracle.sgemm(0, 1, dF, Uf) + np.repeat(dhlr, 2, axis=0)
     close(g.host(dG), want)
@@ -182,6 +182,38 @@ def test_sgemm_splitk_is_deterministic_and_correct(g, oracle, M, N, K):
     exact = A.T.astype(np.float64) @ B.astype(np.float64) + C0
     close(outs[0], exact)
     close(outs[0], oracle.sgemm(1, 0, A, B, beta=1.0, Cin=C0))
+
+
+@pytest.mark.parametrize("tA,tB,M,N,K", [(0, 0, 30, 1536, 512), (0, 1, 8, 512, 1536), (0, 1, 130, 512, 512),
+                                          (0, 0, 1, 64, 4096), (1, 1, 40, 72, 640), (0, 0, 33, 40, 300),
+                                          (0, 1, 65, 33, 68), (0, 0, 600, 1536, 512), (0, 1, 1200, 512, 1536),
+                                          (0, 1, 2482, 5, 512), (1, 0, 5, 512, 2482)])
+def test_small_products(g, oracle, tA, tB, M, N, K):
+    """Tail-round shapes (skinny kernel or split K through the workspace): correct and
+    bit-identical when repeated."""
+    import torch
+
+    r = rng(M * 3 + N + K)
+    A = r.bulk_uniform(M * K, -1, 1).reshape((K, M) if tA else (M, K))
+    B = r.bulk_uniform(N * K, -1, 1).reshape((N, K) if tB else (K, N))
+    nbytes = hip.lib().cavs_sgemm_splitk_workspace(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    exact = (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64)
+    outs = []
+    for _ in range(3):
+        Cd = g.zeros(M, N, fill=float("nan"))
+        g.call("cavs_sgemm_splitk", tA, tB, M, N, K, 1.0, g.P(g.devf(A)), A.shape[1], g.P(g.devf(B)), B.shape[1],
+               0.0, g.P(Cd), N, g.P(ws), nbytes, g.stream())
+        outs.append(g.host(Cd))
+    close(outs[0], exact)
+    np.testing.assert_array_equal(outs[0], outs[1])
+    np.testing.assert_array_equal(outs[0], outs[2])
+    if not tA and tB:  # with the per-vertex addend of the Tree-LSTM backward
+        D = r.bulk_normal(((M + 1) // 2) * N).reshape((M + 1) // 2, N)
+        Cd = g.zeros(M, N)
+        g.call("cavs_sgemm_addrows", tA, tB, M, N, K, g.P(g.devf(A)), K, g.P(g.devf(B)), K, g.P(g.devf(D)), N, 1,
+               g.P(Cd), N, g.P(ws), nbytes, g.stream())
+        close(g.host(Cd), exact + np.repeat(D, 2, axis=0)[:M])
 
 
 # ---------------------------------------------------------------- gates
