@@ -18,6 +18,12 @@ __device__ inline float4 vadd(float4 a, float4 b) {
 }
 __device__ inline float vadd(float a, float b) { return a + b; }
 
+// Pins a loaded value in registers at this point of the program, which keeps the
+// compiler from sinking the load into the predicated store that consumes it (that
+// would leave one load in flight per lane instead of four).
+__device__ inline void pin(float4 &v) { asm volatile("" : "+v"(v.x), "+v"(v.y), "+v"(v.z), "+v"(v.w)); }
+__device__ inline void pin(float &v) { asm volatile("" : "+v"(v)); }
+
 constexpr int kRowsPerBlock = 4;
 
 // out[b] = ids[b] >= 0 ? src[ids[b]] : 0.  ids == nullptr copies row b (copy_rows);
@@ -56,11 +62,14 @@ __global__ void scatter_rows_kernel(V *__restrict__ dst, long ld_dst, const int 
     int row = row0 + r;
     drow[r] = row < n ? (long)ids[row] : -1;
   }
+  // loads are unconditional (rows past the end re-read the last row) so that all four are
+  // in flight before the first store; only the stores are predicated
   for (int c = threadIdx.x; c < wv; c += blockDim.x) {
     V v[kRowsPerBlock];
 #pragma unroll
-    for (int r = 0; r < kRowsPerBlock; r++)
-      if (drow[r] >= 0) v[r] = inp[(long)(row0 + r) * ld_inp + c];
+    for (int r = 0; r < kRowsPerBlock; r++) v[r] = inp[(long)min(row0 + r, n - 1) * ld_inp + c];
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++) pin(v[r]);
 #pragma unroll
     for (int r = 0; r < kRowsPerBlock; r++)
       if (drow[r] >= 0) dst[drow[r] * ld_dst + c] = v[r];
