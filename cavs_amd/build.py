@@ -14,6 +14,7 @@ LIB = os.path.join(PKG, "lib")
 OBJ = os.path.join(PKG, "build")
 HIP_SO = os.path.join(LIB, "libcavs_hip.so")
 HOST_SO = os.path.join(LIB, "libcavs_host.so")
+APPS_SO = os.path.join(LIB, "libcavs_apps.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 HIP_FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-I", os.path.join(ROOT, "include"),
@@ -47,11 +48,20 @@ def build_hip(jobs=8):
 
 
 def build_host():
-    srcs = sorted(glob.glob(os.path.join(HOST, "*.cc")))
+    srcs = sorted(glob.glob(os.path.join(HOST, "*.cc")) + glob.glob(os.path.join(HOST, "frontend", "*.cc")) +
+                  glob.glob(os.path.join(HOST, "midend", "*.cc")))
     if not srcs:
         return None
-    _run([CXX] + CXX_FLAGS + ["-shared", "-o", HOST_SO] + srcs +
-         ["-L", LIB, "-lcavs_hip", "-Wl,-rpath,$ORIGIN"])
+    os.makedirs(OBJ, exist_ok=True)
+    objs = [os.path.join(OBJ, "host_" + os.path.relpath(s, HOST).replace(os.sep, "_")[:-3] + ".o") for s in srcs]
+    with ThreadPoolExecutor(max_workers=8) as ex:
+        list(ex.map(lambda so: _run([CXX] + CXX_FLAGS + ["-c", so[0], "-o", so[1]]), zip(srcs, objs)))
+    _run([CXX, "-shared", "-o", HOST_SO] + objs + ["-L", LIB, "-lcavs_hip", "-Wl,-rpath,$ORIGIN"])
+    # the benchmark applications written against the front end (a user-side program)
+    apps = sorted(glob.glob(os.path.join(HOST, "apps", "*.cc")))
+    if apps:
+        _run([CXX] + CXX_FLAGS + ["-shared", "-o", APPS_SO] + apps +
+             ["-L", LIB, "-lcavs_host", "-lcavs_hip", "-Wl,-rpath,$ORIGIN"])
     return HOST_SO
 
 

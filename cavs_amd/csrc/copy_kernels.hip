@@ -51,6 +51,21 @@ __global__ void gather_rows_kernel(V *__restrict__ out, long ld_out, const V *__
   }
 }
 
+// out[b] += inp[b] over a [n, wv] block (PartialAccumulate: a column block of a wider slab)
+template <typename V>
+__global__ void add_rows_kernel(V *__restrict__ out, long ld_out, const V *__restrict__ inp, long ld_inp,
+                                int n, int wv) {
+  const int row0 = blockIdx.x * kRowsPerBlock;
+  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+#pragma unroll
+    for (int r = 0; r < kRowsPerBlock; r++)
+      if (row0 + r < n) {
+        V *o = out + (long)(row0 + r) * ld_out + c;
+        *o = vadd(*o, inp[(long)(row0 + r) * ld_inp + c]);
+      }
+  }
+}
+
 // dst[ids[b]] = inp[b] for ids[b] >= 0
 template <typename V>
 __global__ void scatter_rows_kernel(V *__restrict__ dst, long ld_dst, const int *__restrict__ ids,
@@ -149,6 +164,21 @@ int cavs_copy_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, 
   if (n == 0 || w == 0) return CAVS_OK;
   CAVS_REQUIRE(out && inp, "cavs_copy_rows: null pointer");
   return launch_gather(out, ld_out, inp, ld_inp, nullptr, n, w, as_stream(stream));
+}
+
+int cavs_add_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w, void *stream) {
+  CAVS_REQUIRE(n >= 0 && w >= 0 && ld_out >= w && ld_inp >= w, "cavs_add_rows: bad shape n=%d w=%d", n, w);
+  if (n == 0 || w == 0) return CAVS_OK;
+  CAVS_REQUIRE(out && inp, "cavs_add_rows: null pointer");
+  hipStream_t st = as_stream(stream);
+  int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
+  if (vec_ok(out, ld_out, inp, ld_inp, w))
+    add_rows_kernel<float4><<<grid, block_for(w / 4), 0, st>>>(reinterpret_cast<float4 *>(out), ld_out / 4,
+                                                               reinterpret_cast<const float4 *>(inp), ld_inp / 4, n, w / 4);
+  else
+    add_rows_kernel<float><<<grid, block_for(w), 0, st>>>(out, ld_out, inp, ld_inp, n, w);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
 }
 
 int cavs_zero_rows(float *out, int ld_out, int n, int w, void *stream) {

@@ -47,6 +47,7 @@ _SIGS = {
     "cavs_scatter_rows": [_P, _I, _P, _P, _I, _I, _I, _P],
     "cavs_zero_rows": [_P, _I, _I, _I, _P],
     "cavs_copy_rows": [_P, _I, _P, _I, _I, _I, _P],
+    "cavs_add_rows": [_P, _I, _P, _I, _I, _I, _P],
     "cavs_gather_children": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_sgemm": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "cavs_sgemm_addrows": [_I, _I, _I, _I, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _Z, _P],

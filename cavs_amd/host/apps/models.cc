@@ -1,0 +1,304 @@
+// The three vertex functions of the reference's benchmark applications, written against
+// the front end exactly as a user would (apps/paper/tree-lstm-cavs.cc:106-184,
+// seq-lstm-cavs.cc:43-95, tree-fc-cavs.cc:21-40), plus an extern "C" harness so that the
+// tests and the benchmark can drive them from Python.  Every tensor that is consumed
+// more than once inside F goes through Mirror(), which is what makes the reference's own
+// gradient rules accumulate instead of overwrite.
+#include <cstring>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "cavs/frontend/cxx/graphsupport.h"
+#include "cavs/frontend/cxx/session.h"
+#include "cavs/frontend/cxx/sym.h"
+
+using std::tie;
+using std::vector;
+
+namespace {
+
+struct Dims {
+  int B, maxlen, V, E, H, C;
+};
+
+class TreeLSTM : public GraphSupport {
+ public:
+  TreeLSTM(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {4 * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    U = Sym::Variable(DT_FLOAT, {4 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {4 * H}, Sym::Zeros());
+    b_i = B.Slice(0, H);
+    b_f = B.Slice(H, H);
+    b_u = B.Slice(2 * H, H);
+    b_o = B.Slice(3 * H, H);
+    U_iou = U.Slice(0, 3 * H * H).Reshape({H, 3 * H});
+    U_f = U.Slice(3 * H * H, H * H).Reshape({H, H});
+  }
+  void Node() override {
+    Sym left = Gather(0, {2 * H});
+    Sym right = Gather(1, {2 * H});
+    Sym h_l, c_l, h_r, c_r;
+    tie(h_l, c_l) = left.Split2();
+    tie(h_r, c_r) = right.Split2();
+    Sym h_lr = h_l.Mirror() + h_r.Mirror();
+
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, 4 * H}).Mirror()).Reshape({H * 4});
+    Sym xW_i, xW_o, xW_u, xW_f;
+    tie(xW_i, xW_o, xW_u, xW_f) = xW.Split4();
+
+    Sym hU_iou = Sym::MatMul(h_lr.Reshape({1, H}), U_iou.Mirror()).Reshape({H * 3});
+    Sym hU_i, hU_o, hU_u;
+    tie(hU_i, hU_o, hU_u) = hU_iou.Split3();
+    Sym hU_fl = Sym::MatMul(h_l.Mirror().Reshape({1, H}), U_f.Mirror()).Reshape({H});
+    Sym hU_fr = Sym::MatMul(h_r.Mirror().Reshape({1, H}), U_f.Mirror()).Reshape({H});
+
+    Sym i = (xW_i + hU_i + b_i.Mirror()).Sigmoid();
+    Sym o = (xW_o + hU_o + b_o.Mirror()).Sigmoid();
+    Sym u = (xW_u + hU_u + b_u.Mirror()).Tanh();
+    Sym f_l = (xW_f.Mirror() + hU_fl + b_f.Mirror()).Sigmoid();
+    Sym f_r = (xW_f.Mirror() + hU_fr + b_f.Mirror()).Sigmoid();
+
+    Sym c = i * u + f_l * c_l + f_r * c_r;
+    Sym h = o * Sym::Tanh(c.Mirror());
+    Scatter(Sym::Concat({h.Mirror(), c.Mirror()}));
+    Push(h.Mirror());
+  }
+  Sym embedding, W, U, B;
+
+ private:
+  int E, H;
+  Sym b_i, b_f, b_u, b_o, U_iou, U_f;
+};
+
+class SeqLSTM : public GraphSupport {
+ public:
+  SeqLSTM(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, H}, Sym::Uniform(-0.1f, 0.1f));
+    LSTM_w = Sym::Variable(DT_FLOAT, {8 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    LSTM_b = Sym::Variable(DT_FLOAT, {4 * H}, Sym::Zeros());
+    Ux = LSTM_w.Slice(0, 4 * H * H);
+    Wh = LSTM_w.Slice(4 * H * H, 4 * H * H);
+    bi = LSTM_b.Slice(0, H);
+    bf = LSTM_b.Slice(H, H);
+    bu = LSTM_b.Slice(2 * H, H);
+    bo = LSTM_b.Slice(3 * H, H);
+  }
+  void Node() override {
+    Sym child = Gather(0, {2 * H});
+    Sym child_h, child_c;
+    tie(child_h, child_c) = child.Split2();
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding);
+    Sym tmp = Sym::MatMul(x, Ux.Mirror().Reshape({H, 4 * H})) +
+              Sym::MatMul(child_h.Expand_dims(0), Wh.Mirror().Reshape({H, 4 * H}));
+    Sym i, f, u, o;
+    tie(i, f, u, o) = tmp.Split4();
+    i = (i + bi.Mirror()).Sigmoid();
+    f = (f + bf.Mirror()).Sigmoid();
+    u = (u + bu.Mirror()).Tanh();
+    o = (o + bo.Mirror()).Sigmoid();
+    Sym c = i * u + f * child_c;
+    Sym h = o * Sym::Tanh(c.Mirror());
+    Scatter(Sym::Concat({h.Mirror(), c.Mirror()}));
+    Push(h.Mirror());
+  }
+  Sym embedding, LSTM_w, LSTM_b;
+
+ private:
+  int H;
+  Sym Ux, Wh, bi, bf, bu, bo;
+};
+
+class TreeFC : public GraphSupport {
+ public:
+  // variant 0: the reference app (relu, no bias, no vertex input); variant 1: tanh + bias + Pull'ed input
+  TreeFC(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d, int variant)
+      : GraphSupport(graph_ph, vertex_ph), H(d.H), variant_(variant) {
+    W = Sym::Variable(DT_FLOAT, {2 * H, H}, Sym::Uniform(-0.1f, 0.1f));
+    if (variant_) Bv = Sym::Variable(DT_FLOAT, {H}, Sym::Zeros());
+  }
+  void Node() override {
+    Sym left = Gather(0, {H});
+    Sym right = Gather(1, {H});
+    Sym fc = Sym::MatMul(Sym::Concat({left, right}).Reshape({1, 2 * H}), W.Mirror()).Reshape({H});
+    Sym res;
+    if (variant_) {
+      Sym x = Pull(0, {H});
+      res = (fc + Bv.Mirror() + x).Tanh();
+    } else {
+      res = fc.Relu();
+    }
+    Scatter(res.Mirror());
+    Push(res.Mirror());
+  }
+  Sym W, Bv;
+
+ private:
+  int H, variant_;
+};
+
+struct App {
+  Dims d{};
+  std::string model;
+  std::unique_ptr<GraphSupport> gs;
+  Sym graph, vertex, label, mask, weight, bias, graph_output, loss, train, total;
+  vector<std::pair<std::string, Sym>> vars;  // oracle name -> Variable
+  std::unique_ptr<Session> sess;
+};
+
+App *g_app = nullptr;
+
+}  // namespace
+
+extern "C" {
+
+// model: "treelstm" | "lstm" | "treefc" (reference app) | "treefc_x" (tanh + bias + input, sum of
+// squares at the roots).  Declares the program and opens a session.  One app per process at a time.
+int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, int C, int opt, float lr) {
+  try {
+    delete g_app;
+    g_app = nullptr;
+    C_ResetGraph();
+    auto app = std::make_unique<App>();
+    app->d = Dims{B, maxlen, V, E, H, C};
+    app->model = model;
+    const Dims &d = app->d;
+    app->graph = Sym::Placeholder(DT_FLOAT, {B, maxlen}, "CPU");
+    bool fc = app->model == "treefc" || app->model == "treefc_x";
+    app->vertex = Sym::Placeholder(DT_FLOAT, app->model == "treefc_x" ? vector<int>{B * maxlen, H} : vector<int>{B, maxlen});
+    if (!fc) {
+      app->label = Sym::Placeholder(DT_FLOAT, {B, maxlen});
+      app->weight = Sym::Variable(DT_FLOAT, {C, H}, Sym::Uniform(-0.1f, 0.1f));
+      app->bias = Sym::Variable(DT_FLOAT, {1, C}, Sym::Zeros());
+    }
+    if (app->model == "treelstm") {
+      auto *m = new TreeLSTM(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model == "lstm") {
+      auto *m = new SeqLSTM(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->LSTM_w}, {"Bv", m->LSTM_b}};
+    } else if (fc) {
+      auto *m = new TreeFC(app->graph, app->vertex, d, app->model == "treefc_x");
+      app->gs.reset(m);
+      app->vars = {{"W", m->W}};
+      if (app->model == "treefc_x") app->vars.push_back({"Bv", m->Bv});
+    } else {
+      return -1;
+    }
+    app->graph_output = app->gs->Output();
+    if (!fc) {
+      app->vars.push_back({"Wfc", app->weight});
+      app->vars.push_back({"bfc", app->bias});
+      Sym label_reshape = app->label.Reshape({-1, 1});
+      label_reshape.ControlDependency(app->graph_output);
+      app->loss = app->graph_output.FullyConnected(app->weight, app->bias).SoftmaxEntropyLoss(label_reshape);
+      app->total = app->loss.Reduce_mean();
+    } else if (app->model == "treefc_x") {
+      app->mask = Sym::Placeholder(DT_FLOAT, {B * maxlen, H});
+      Sym mask_rows = app->mask.Reshape({-1, H});
+      mask_rows.ControlDependency(app->graph_output);
+      app->loss = (app->graph_output.Square() * mask_rows).Reduce_sum();
+      app->total = app->loss;
+    } else {
+      app->loss = app->graph_output.Reduce_sum();  // tree-fc-cavs.cc:96
+      app->total = app->loss;
+    }
+    app->train = app->loss.Optimizer({}, lr);
+    if (opt >= 0) app->sess = std::make_unique<Session>(opt);  // opt < 0: declare only (no device needed)
+    g_app = app.release();
+    return 0;
+  } catch (const std::exception &e) {
+    std::fprintf(stderr, "cavs_app_create: %s\n", e.what());
+    return -2;
+  }
+}
+
+int cavs_app_set_param(const char *name, const float *data, size_t n) {
+  if (!g_app) return -1;
+  for (auto &v : g_app->vars)
+    if (v.first == name) {
+      try {
+        g_app->sess->SetVariable(v.second, data, n);
+        return 0;
+      } catch (const std::exception &e) {
+        std::fprintf(stderr, "cavs_app_set_param: %s\n", e.what());
+        return -2;
+      }
+    }
+  return -3;
+}
+
+void cavs_app_configure(int pairing, int allow_fused) {
+  if (!g_app) return;
+  g_app->sess->SetPairing(pairing);
+  g_app->sess->AllowFusedPath(allow_fused != 0);
+}
+
+// One Session::Run of {train, loss, graph_output} (or without train).  graph is the
+// [B, maxlen] parent array; x and labels are full placeholder buffers (packed by vertex id).
+// Outputs: loss rows (N, or 1 for the Tree-FC losses) and graph_out [N, H]; returns N or < 0.
+long cavs_app_step(const int *graph, const float *x, const float *labels, const float *mask, int train,
+                   float *loss_out, size_t loss_cap, float *go_out, size_t go_cap) {
+  if (!g_app) return -1;
+  try {
+    App &a = *g_app;
+    vector<std::pair<Sym, void *>> feeds = {{a.graph, (void *)graph}};
+    bool fc = a.model == "treefc" || a.model == "treefc_x";
+    if (!fc || a.model == "treefc_x") feeds.push_back({a.vertex, (void *)x});
+    if (!fc) feeds.push_back({a.label, (void *)labels});
+    if (a.model == "treefc_x") feeds.push_back({a.mask, (void *)mask});
+    vector<Sym> outs;
+    if (train) outs.push_back(a.train);
+    outs.push_back(a.loss);
+    outs.push_back(a.graph_output);
+    a.sess->Run(outs, feeds);
+    vector<float> go = a.sess->Read(a.graph_output.output(0));
+    vector<float> loss = a.sess->Read(a.loss.output(0));
+    if (loss.size() > loss_cap || go.size() > go_cap) return -4;
+    std::memcpy(loss_out, loss.data(), loss.size() * 4);
+    std::memcpy(go_out, go.data(), go.size() * 4);
+    return (long)(go.size() / a.d.H);
+  } catch (const std::exception &e) {
+    std::fprintf(stderr, "cavs_app_step: %s\n", e.what());
+    return -2;
+  }
+}
+
+// gradient (grad != 0) or current value of a parameter by oracle name
+long cavs_app_read_param(const char *name, int grad, float *out, size_t cap) {
+  if (!g_app) return -1;
+  for (auto &v : g_app->vars)
+    if (v.first == name) {
+      try {
+        vector<float> t = g_app->sess->Read(v.second.output(0) + (grad ? "_grad" : ""));
+        if (t.size() > cap) return -(long)t.size();
+        std::memcpy(out, t.data(), t.size() * 4);
+        return (long)t.size();
+      } catch (const std::exception &e) {
+        std::fprintf(stderr, "cavs_app_read_param: %s\n", e.what());
+        return -2;
+      }
+    }
+  return -3;
+}
+
+long cavs_app_read(const char *edge, float *out, size_t cap) {
+  if (!g_app) return -1;
+  return C_ReadTensor(g_app->sess->handle(), edge, out, cap);
+}
+
+int cavs_app_uses_fused_path(void) { return g_app && g_app->sess->UsesFusedPath(); }
+
+void cavs_app_destroy(void) {
+  delete g_app;
+  g_app = nullptr;
+  C_ResetGraph();
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+// Session of the front end: owns the device tensors of a program, interprets the
+// main-scope operators, and runs the vertex function over the rounds of a batch
+// (cavs/midend/session_simple.cc:56-108, statement.cc:8-123, graph_session.cc:45-206).
+// Two ways to run F: op by op through the backend's C ABI (the reference's execution
+// model), or -- when F is recognised as one of the vertex functions the fused round
+// kernels implement -- lowered onto cavs::Engine.
+#ifndef CAVS_HOST_MIDEND_EXECUTOR_H_
+#define CAVS_HOST_MIDEND_EXECUTOR_H_
+
+#include <map>
+#include <memory>
+#include <string>
+#include <vector>
+
+#include "../device.h"
+#include "../engine.h"
+#include "../scheduler.h"
+#include "graph.h"
+
+namespace cavs {
+namespace mid {
+
+struct Tensor {
+  DeviceArray<float> own;
+  float *base = nullptr;   // own.get() or a view into another tensor
+  long width = 1;          // elements per row (per-vertex tensors) or total (static)
+  bool per_vertex = false; // rows follow the batch: [rows, width]
+  long rows = 1;           // current row count of a per-vertex tensor
+  size_t count() const { return (size_t)(per_vertex ? rows * width : width); }
+};
+
+struct HostTensor {  // C_Tensor of the C API
+  std::string name;
+  std::vector<int> shape;
+  std::vector<char> data;
+};
+
+struct Lowering;  // recognised vertex function bound to Engine parameters
+
+class Executor {
+ public:
+  Executor(int opt, const std::string &name);
+  ~Executor();
+  void run(const std::vector<std::string> &outputs, std::vector<HostTensor *> *results,
+           const std::vector<std::pair<std::string, const HostTensor *>> &feeds);
+  void set_variable(const std::string &name, const float *data, size_t n);
+  long read_tensor(const std::string &name, float *out, size_t cap);
+  bool uses_fused_path() const { return lowered_; }
+  void allow_fused_path(bool a) { allow_fused_ = a; compiled_version_ = -1; }
+  void set_pairing(int p) { pairing_ = p; compiled_version_ = -1; }
+
+ private:
+  struct RoundCtx {
+    long off = 0, n = 0;
+    bool in_function = false;
+  };
+  void compile();
+  void init_variables();
+  Tensor &tensor(const std::string &name);
+  Tensor *find_tensor(const std::string &name);
+  float *view(const std::string &name, const RoundCtx &c, long *count, long *width);
+  void exec(const OpDef &d, const RoundCtx &c);
+  void run_graph_output(const Node *n);
+  void run_graph_output_grad(const OpDef &d);
+  void upload_lists();
+  void lowered_forward(const int32_t *graph, int B, int maxlen, float *graph_out);
+  void lowered_backward(const OpDef &d);
+  void forward_needed(const std::vector<std::string> &targets, std::vector<const Node *> *order);
+  const Edge *edge(const std::string &name) const;
+  float *workspace(size_t bytes);
+
+  int opt_;
+  std::string name_;
+  void *stream_ = nullptr;
+  int compiled_version_ = -1;
+  bool allow_fused_ = true, lowered_ = false;
+  int pairing_ = 0;
+  std::map<std::string, std::unique_ptr<Tensor>> tensors_;
+  std::map<std::string, std::vector<float>> pending_vars_;  // SetVariable before compile
+  bool vars_initialised_ = false;
+
+  // per-step state of the vertex function
+  Schedule sched_;
+  long N_ = 0;
+  int nch_ = 0;          // Gather children used by F
+  long pool_w_ = 0, ret_w_ = 0, arg_w_ = 0;
+  DeviceArray<float> pool_, dpool_, ret_, ws_;
+  PinnedArray<int> idx_host_;
+  DeviceArray<int> idx_dev_;
+  const int *d_t2j_ = nullptr, *d_pair_ = nullptr, *d_child_[2] = {nullptr, nullptr};
+  const float *func_arg_ = nullptr;   // vertex placeholder on the device
+  const float *dgo_ = nullptr;        // d GraphOutput during the backward function
+  std::unique_ptr<Engine> engine_;
+  std::unique_ptr<Lowering> lowering_;
+};
+
+}  // namespace mid
+}  // namespace cavs
+#endif

@@ -83,6 +83,10 @@ int cavs_zero_rows(float *out, int ld_out, int n, int w, void *stream);
 /* out[b, 0:w] = inp[b, 0:w]  (Push, Slice, Concat: column blocks via ld) */
 int cavs_copy_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w,
                    void *stream);
+/* out[b, 0:w] += inp[b, 0:w]: PartialAccumulate, the gradient of Slice
+ * (BinaryStridedKernel, cavs/backend/op_impl_elementwise.cuh:141-150;
+ * cavs/backend/op_impl_elementwise_common.h:97-122) */
+int cavs_add_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w, void *stream);
 /* Both child gathers of a binary vertex function in one pass, plus h_l + h_r:
  *   G[2b+i, 0:w] = ids[2b+i] >= 0 ? pool[ids[2b+i], 0:w] : 0      i in {0,1}
  *   hsum[b, 0:hw] = G[2b, 0:hw] + G[2b+1, 0:hw]   (hsum may be NULL)

@@ -82,6 +82,9 @@ def test_gather_scatter_zero_copy_rows_bit_exact(g, oracle, n, w, ld_extra):
     want = buf0.copy()
     want[:, :w] = src[:n, :w]
     np.testing.assert_array_equal(g.host(buf), want)
+    g.call("cavs_add_rows", g.P(buf), ld, g.P(g.devf(src)), ld, n, w, g.stream())
+    want[:, :w] += src[:n, :w]
+    np.testing.assert_array_equal(g.host(buf), want)
 
 
 def test_row_ops_accept_empty_and_reject_bad_shapes(g):
