@@ -21,7 +21,7 @@ inline size_t grow(size_t need, size_t have) {
 }
 }  // namespace
 
-Engine::Engine(const cavs_session_config &cfg) : cfg_(cfg) {
+Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg) {
   if (cfg.model < 0 || cfg.model > 2) fail(CAVS_EINVAL, "unknown model " + std::to_string(cfg.model));
   if (cfg.loss < 0 || cfg.loss > 2) fail(CAVS_EINVAL, "unknown loss " + std::to_string(cfg.loss));
   if (cfg.pairing < 0 || cfg.pairing > 1) fail(CAVS_EINVAL, "unknown pairing");
@@ -34,7 +34,12 @@ Engine::Engine(const cavs_session_config &cfg) : cfg_(cfg) {
     fail(CAVS_EINVAL, "vocabulary and embedding sizes must be positive");
   if (cfg.loss == CAVS_LOSS_SOFTMAX && cfg.C <= 0) fail(CAVS_EINVAL, "class count must be positive");
   check(cavs_init(cfg.device));
-  check(cavs_stream_create(&stream_));
+  if (external_stream) {
+    stream_ = external_stream;
+    own_stream_ = false;
+  } else {
+    check(cavs_stream_create(&stream_));
+  }
   for (auto &e : ev_) check(cavs_event_create(&e));
   for (auto &e : idx_copied_) check(cavs_event_create(&e));
   switch (cfg.model) {
@@ -64,16 +69,18 @@ Engine::~Engine() {
   for (auto &e : ev_) cavs_event_destroy(e);
   for (auto &e : idx_copied_) cavs_event_destroy(e);
   for (auto &e : prof_events_) cavs_event_destroy(e);
-  cavs_stream_destroy(stream_);
+  if (own_stream_) cavs_stream_destroy(stream_);
 }
 
 void Engine::add_param(const std::string &name, size_t n) {
   auto p = std::make_unique<Param>();
   p->n = n;
-  p->w.reserve(n);
-  p->g.reserve(n);
-  check(cavs_zero(p->w.get(), n * 4, stream_));
-  check(cavs_zero(p->g.get(), n * 4, stream_));
+  p->own_w.reserve(n);
+  p->own_g.reserve(n);
+  p->w = p->own_w.get();
+  p->g = p->own_g.get();
+  check(cavs_zero(p->w, n * 4, stream_));
+  check(cavs_zero(p->g, n * 4, stream_));
   params_[name] = std::move(p);
 }
 
@@ -83,11 +90,18 @@ Param &Engine::param(const std::string &name) {
   return *it->second;
 }
 
+void Engine::bind_param(const std::string &name, float *w, float *g) {
+  Param &p = param(name);
+  if (!w) fail(CAVS_EINVAL, "bind_param('" + name + "'): null weight pointer");
+  p.w = w;
+  p.g = g ? g : p.own_g.get();
+}
+
 void Engine::set_param(const std::string &name, const float *host, size_t n) {
   Param &p = param(name);
   if (n != p.n || !host)
     fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
-  check(cavs_memcpy_h2d(p.w.get(), host, n * 4, stream_));
+  check(cavs_memcpy_h2d(p.w, host, n * 4, stream_));
   check(cavs_stream_sync(stream_));
 }
 
@@ -95,7 +109,7 @@ void Engine::get_param(const std::string &name, float *host, size_t n, bool grad
   Param &p = param(name);
   if (n != p.n || !host)
     fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
-  check(cavs_memcpy_d2h(host, grad ? p.g.get() : p.w.get(), n * 4, stream_));
+  check(cavs_memcpy_d2h(host, grad ? p.g : p.w, n * 4, stream_));
   check(cavs_stream_sync(stream_));
 }
 
@@ -304,8 +318,7 @@ void Engine::upload_index_arena() {
 }
 
 // ------------------------------------------------------------------ step
-void Engine::step(const int *graph, int B, int maxlen, const void *x, const void *labels,
-                  bool on_device, bool backward, float lr) {
+void Engine::begin_step(const int *graph, int B, int maxlen) {
   auto t0 = std::chrono::steady_clock::now();
   std::string err = build_schedule(graph, B, maxlen, (cfg_.opt & CAVS_OPT_BATCHING) != 0, &sched_);
   if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
@@ -313,12 +326,45 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample; the reference never executes such a vertex "
                             "(graph_scheduler.cc:180) and leaves its rows undefined");
   N_ = sched_.N;
-  const int N = N_, H = cfg_.H;
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   reserve_edges();
   upload_index_arena();
   parse_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+}
 
+void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out) {
+  begin_step(graph, B, maxlen);
+  if ((cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x) && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
+  d_x_ = x_dev;
+  check(cavs_event_record(ev_[0], stream_));
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
+    case CAVS_MODEL_LSTM: lstm_forward(); break;
+    default: treefc_forward();
+  }
+  pop_ret(graph_out ? graph_out : GO_.get());
+  check(cavs_event_record(ev_[1], stream_));
+  ev_valid_ = true;
+  ev_bwd_valid_ = false;
+}
+
+void Engine::backward_only(const float *dgraph_out) {
+  if (!dgraph_out || N_ == 0) fail(CAVS_EINVAL, "backward_only needs d graph_out of a forward pass");
+  d_dgo_ = dgraph_out;
+  check(cavs_event_record(ev_[2], stream_));
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
+    case CAVS_MODEL_LSTM: lstm_backward(); break;
+    default: treefc_backward();
+  }
+  check(cavs_event_record(ev_[3], stream_));
+  ev_bwd_valid_ = true;
+}
+
+void Engine::step(const int *graph, int B, int maxlen, const void *x, const void *labels,
+                  bool on_device, bool backward, float lr) {
+  begin_step(graph, B, maxlen);
+  const int N = N_, H = cfg_.H;
   const bool needs_x = cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x;
   const size_t xw = cfg_.model == CAVS_MODEL_TREEFC ? H : 1;
   if (needs_x && !x) fail(CAVS_EINVAL, "vertex input feed is null");
@@ -347,10 +393,11 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     case CAVS_MODEL_LSTM: lstm_forward(); break;
     default: treefc_forward();
   }
-  pop_ret();
+  pop_ret(GO_.get());
   check(cavs_event_record(ev_[1], stream_));
   ev_valid_ = true;
   head_forward_backward(backward);
+  d_dgo_ = dGO_.get();
   did_backward_ = backward;
   ev_bwd_valid_ = false;
   if (backward) {
@@ -364,7 +411,7 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     ev_bwd_valid_ = true;
     if (lr != 0.f)
       for (auto &kv : params_) {
-        check(cavs_sgd(kv.second->w.get(), kv.second->g.get(), lr, kv.second->n, stream_));
+        check(cavs_sgd(kv.second->w, kv.second->g, lr, kv.second->n, stream_));
         c_launches_ += 1;
       }
   }
@@ -372,7 +419,7 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
 
 // FunctionPopRet (cavs/backend/op_impl_graphop.cu:304-318): GraphOutput[tids_to_jobids[t]] =
 // ret[t].  Push's slab copy is folded in: the h half of the message slab is the return value.
-void Engine::pop_ret() { scatter(GO_.get(), cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H); }
+void Engine::pop_ret(float *graph_out) { scatter(graph_out, cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H); }
 
 // ------------------------------------------------------------------ Tree-LSTM
 // apps/paper/tree-lstm-cavs.cc:129-172.  Everything that does not depend on the children
@@ -381,9 +428,9 @@ void Engine::pop_ret() { scatter(GO_.get(), cfg_.H, d_t2j_, msg_.get(), mw_, N_,
 // gathered rows are zero.
 void Engine::treelstm_forward() {
   const int N = N_, H = cfg_.H, E = E_;
-  const float *W = param("W").w.get(), *U = param("U").w.get(), *Bv = param("Bv").w.get();
+  const float *W = param("W").w, *U = param("U").w, *Bv = param("Bv").w;
   gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
-  check(cavs_embed_fwd(e_.get(), E, xs_.get(), param("Emb").w.get(), N, E, stream_));
+  check(cavs_embed_fwd(e_.get(), E, xs_.get(), param("Emb").w, N, E, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, E, e_.get(), E, W, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
@@ -417,8 +464,8 @@ void Engine::treelstm_forward() {
 
 void Engine::treelstm_backward() {
   const int N = N_, H = cfg_.H, E = E_;
-  const float *W = param("W").w.get(), *U = param("U").w.get();
-  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);  // grad of Push is Pull
+  const float *W = param("W").w, *U = param("U").w;
+  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);  // grad of Push is Pull
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -453,16 +500,16 @@ void Engine::treelstm_backward() {
   const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
   gemm(0, 1, N, E, 4 * H, dxW_.get(), 4 * H, W, 4 * H, 0.f, de_.get(), E);
   Param &emb = param("Emb");
-  check(cavs_zero(emb.g.get(), emb.n * 4, stream_));
-  check(cavs_embed_bwd(emb.g.get(), xs_.get(), de_.get(), E, N, E, stream_));
+  check(cavs_zero(emb.g, emb.n * 4, stream_));
+  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), E, N, E, stream_));
   c_launches_ += 2;
-  gemm_splitk(1, 0, E, 4 * H, N, e_.get(), E, dxW_.get(), 4 * H, param("W").g.get(), 4 * H);
-  float *dU = param("U").g.get();
+  gemm_splitk(1, 0, E, 4 * H, N, e_.get(), E, dxW_.get(), 4 * H, param("W").g, 4 * H);
+  float *dU = param("U").g;
   gemm_splitk(1, 0, H, 3 * H, N - lp, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H);
   gemm_splitk(1, 0, H, H, 2 * (N - lp), G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
               dU + (size_t)3 * H * H, H);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
-  float *dB = param("Bv").g.get();
+  float *dB = param("Bv").g;
   const int src_block[4] = {0, 3, 2, 1};
   for (int k = 0; k < 4; k++)
     check(cavs_colsum(dB + (size_t)k * H, dxW_.get() + (size_t)src_block[k] * H, 4 * H, N, H, 0, stream_));
@@ -473,9 +520,9 @@ void Engine::treelstm_backward() {
 // apps/paper/seq-lstm-cavs.cc:62-86
 void Engine::lstm_forward() {
   const int N = N_, H = cfg_.H;
-  const float *Wx = param("W").w.get(), *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w.get();
+  const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w;
   gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
-  check(cavs_embed_fwd(e_.get(), H, xs_.get(), param("Emb").w.get(), N, H, stream_));
+  check(cavs_embed_fwd(e_.get(), H, xs_.get(), param("Emb").w, N, H, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
@@ -495,8 +542,8 @@ void Engine::lstm_forward() {
 
 void Engine::lstm_backward() {
   const int N = N_, H = cfg_.H;
-  const float *Wx = param("W").w.get(), *Wh = Wx + (size_t)4 * H * H;
-  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);
+  const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H;
+  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
@@ -517,14 +564,14 @@ void Engine::lstm_backward() {
   const int lp = sched_.leaf_prefix;
   gemm(0, 1, N, H, 4 * H, dxW_.get(), 4 * H, Wx, 4 * H, 0.f, de_.get(), H);
   Param &emb = param("Emb");
-  check(cavs_zero(emb.g.get(), emb.n * 4, stream_));
-  check(cavs_embed_bwd(emb.g.get(), xs_.get(), de_.get(), H, N, H, stream_));
+  check(cavs_zero(emb.g, emb.n * 4, stream_));
+  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), H, N, H, stream_));
   c_launches_ += 2;
-  float *dW = param("W").g.get();
+  float *dW = param("W").g;
   gemm_splitk(1, 0, H, 4 * H, N, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H);
   gemm_splitk(1, 0, H, 4 * H, N - lp, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
               dW + (size_t)4 * H * H, 4 * H);
-  check(cavs_colsum(param("Bv").g.get(), dxW_.get(), 4 * H, N, 4 * H, 0, stream_));
+  check(cavs_colsum(param("Bv").g, dxW_.get(), 4 * H, N, 4 * H, 0, stream_));
   c_launches_ += 1;
 }
 
@@ -532,8 +579,8 @@ void Engine::lstm_backward() {
 // apps/paper/tree-fc-cavs.cc:28-36 (optionally with a bias and a Pull'ed input row)
 void Engine::treefc_forward() {
   const int N = N_, H = cfg_.H;
-  const float *W = param("W").w.get();
-  const float *Bv = cfg_.use_bias ? param("Bv").w.get() : nullptr;
+  const float *W = param("W").w;
+  const float *Bv = cfg_.use_bias ? param("Bv").w : nullptr;
   if (cfg_.use_x) gather(xs_.get(), H, d_x_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
   for (const Round &r : sched_.rounds) {
@@ -561,8 +608,8 @@ void Engine::treefc_forward() {
 
 void Engine::treefc_backward() {
   const int N = N_, H = cfg_.H;
-  const float *W = param("W").w.get();
-  gather(dret_.get(), H, dGO_.get(), H, d_t2j_, N, H);
+  const float *W = param("W").w;
+  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
@@ -576,9 +623,9 @@ void Engine::treefc_backward() {
   }
   const int lp = sched_.leaf_prefix;
   gemm_splitk(1, 0, 2 * H, H, N - lp, G_.at((size_t)2 * lp * H), 2 * H, dxW_.at((size_t)lp * H), H,
-              param("W").g.get(), H);
+              param("W").g, H);
   if (cfg_.use_bias) {
-    check(cavs_colsum(param("Bv").g.get(), dxW_.get(), H, N, H, 0, stream_));
+    check(cavs_colsum(param("Bv").g, dxW_.get(), H, N, H, 0, stream_));
     c_launches_ += 1;
   }
 }
@@ -590,15 +637,15 @@ void Engine::head_forward_backward(bool backward) {
     // FullyConnected + SoftmaxEntropyLoss (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79,
     // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
     Param &Wfc = param("Wfc"), &bfc = param("bfc");
-    gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w.get(), H, 0.f, logits_.get(), C);
-    check(cavs_bias_add_rows(logits_.get(), logits_.get(), bfc.w.get(), N, C, stream_));
+    gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w, H, 0.f, logits_.get(), C);
+    check(cavs_bias_add_rows(logits_.get(), logits_.get(), bfc.w, N, C, stream_));
     check(cavs_softmax_xent(loss_.get(), backward ? dlogits_.get() : nullptr, logits_.get(), d_labels_, N, C, stream_));
     c_launches_ += 2;
     if (backward) {
-      gemm_splitk(1, 0, C, H, N, dlogits_.get(), C, GO_.get(), H, Wfc.g.get(), H);
-      check(cavs_colsum(bfc.g.get(), dlogits_.get(), C, N, C, 0, stream_));
+      gemm_splitk(1, 0, C, H, N, dlogits_.get(), C, GO_.get(), H, Wfc.g, H);
+      check(cavs_colsum(bfc.g, dlogits_.get(), C, N, C, 0, stream_));
       c_launches_ += 1;
-      gemm(0, 0, N, H, C, dlogits_.get(), C, Wfc.w.get(), H, 0.f, dGO_.get(), H);
+      gemm(0, 0, N, H, C, dlogits_.get(), C, Wfc.w, H, 0.f, dGO_.get(), H);
     }
     return;
   }

@@ -19,15 +19,28 @@
 namespace cavs {
 
 struct Param {
-  DeviceArray<float> w, g;
+  float *w = nullptr, *g = nullptr;  // owned storage below, or bound to a caller's tensors
+  DeviceArray<float> own_w, own_g;
   size_t n = 0;
 };
 
 class Engine {
  public:
-  explicit Engine(const cavs_session_config &cfg);
+  // external_stream: enqueue on the caller's stream instead of creating one
+  explicit Engine(const cavs_session_config &cfg, void *external_stream = nullptr);
   ~Engine();
 
+  // Points a parameter and its gradient at device memory owned by the caller (the front
+  // end's Variable tensors) instead of the engine's own copies.  g may be null: then the
+  // engine keeps the gradient in its own buffer (read it with grad_ptr()).
+  void bind_param(const std::string &name, float *w, float *g);
+  const float *grad_ptr(const std::string &name) { return param(name).g; }
+  float *graph_out_ptr() const { return GO_.get(); }
+  // The two halves of step() for a caller that runs the loss head itself: forward F into
+  // graph_out [N,H] (vertex order), then backward F from d graph_out.
+  void forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out);
+  void backward_only(const float *dgraph_out);
+  void set_pairing(int pairing) { cfg_.pairing = pairing; }
   void set_param(const std::string &name, const float *host, size_t n);
   void get_param(const std::string &name, float *host, size_t n, bool grad);
   void step(const int *graph, int B, int maxlen, const void *x, const void *labels,
@@ -58,7 +71,8 @@ class Engine {
   void lstm_backward();
   void treefc_forward();
   void treefc_backward();
-  void pop_ret();
+  void pop_ret(float *graph_out);
+  void begin_step(const int *graph, int B, int maxlen);
   void head_forward_backward(bool backward);
   // counted wrappers
   float *workspace(size_t bytes);
@@ -91,6 +105,7 @@ class Engine {
 
   cavs_session_config cfg_;
   void *stream_ = nullptr;
+  bool own_stream_ = true;
   void *ev_[4] = {nullptr, nullptr, nullptr, nullptr};  // fwd begin/end, bwd begin/end
   bool ev_valid_ = false, ev_bwd_valid_ = false;
   float parse_ms_ = 0.f;
@@ -110,7 +125,7 @@ class Engine {
 
   // feeds
   DeviceArray<float> x_in_, labels_in_;
-  const float *d_x_ = nullptr, *d_labels_ = nullptr;
+  const float *d_x_ = nullptr, *d_labels_ = nullptr, *d_dgo_ = nullptr;
 
   // edges (rows = tensor ids unless marked round-local)
   DeviceArray<float> xs_, e_, xW_, G_, hlr_, gates_, msg_, pool_, GO_, dGO_, dret_, dpool_, dxW_,

@@ -532,31 +532,29 @@ void Executor::run_graph_output(const Node *n) {
   const Edge *ge = n->in[0];
   if (ge->shape.size() != 2) fail(CAVS_EINVAL, "the graph placeholder must be [batch, max vertices]");
   const int32_t *graph = reinterpret_cast<const int32_t *>(gt.base);
-  std::string err = build_schedule(graph, ge->shape[0], ge->shape[1], (opt_ & OPT_BATCHING) != 0, &sched_);
-  if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
-  if (sched_.executed != sched_.N)
-    fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample, which the reference never executes");
-  N_ = sched_.N;
-  // the vertex placeholder may be left unfed when F never Pulls (apps/paper/tree-fc-cavs.cc:104)
-  Tensor *arg = find_tensor(n->in[1]->name);
-  func_arg_ = arg ? arg->base : nullptr;
-
   auto &slot = tensors_[n->out[0]->name];
   if (!slot) slot = std::make_unique<Tensor>();
   Tensor &go = *slot;
   go.width = ret_w_;
   go.per_vertex = true;
+  // the vertex placeholder may be left unfed when F never Pulls (apps/paper/tree-fc-cavs.cc:104)
+  Tensor *arg = find_tensor(n->in[1]->name);
+  func_arg_ = arg ? arg->base : nullptr;
+  if (lowered_) {  // the engine schedules, runs the fused rounds and owns GraphOutput
+    lowered_forward(graph, ge->shape[0], ge->shape[1], nullptr);
+    return;
+  }
+  std::string err = build_schedule(graph, ge->shape[0], ge->shape[1], (opt_ & OPT_BATCHING) != 0, &sched_);
+  if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
+  if (sched_.executed != sched_.N)
+    fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample, which the reference never executes");
+  N_ = sched_.N;
   go.rows = N_;
   if (go.own.capacity() < go.count()) {
     check(cavs_stream_sync(stream_));
     go.own.reserve(go.count() + go.count() / 4);
   }
   go.base = go.own.get();
-
-  if (lowered_) {
-    lowered_forward(graph, ge->shape[0], ge->shape[1], go.base);
-    return;
-  }
   size_t need_pool = (size_t)N_ * pool_w_, need_ret = (size_t)N_ * ret_w_;
   if (pool_.capacity() < need_pool || ret_.capacity() < need_ret) {
     check(cavs_stream_sync(stream_));

@@ -33,6 +33,11 @@ Graph &global_graph() {
   if (!g_graph) g_graph = new Graph();
   return *g_graph;
 }
+Graph *swap_global_graph(Graph *g) {
+  Graph *old = g_graph;
+  g_graph = g;
+  return old;
+}
 void reset_global_graph() {
   delete g_graph;
   g_graph = nullptr;

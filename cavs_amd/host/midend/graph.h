@@ -88,6 +88,9 @@ struct Graph {
 
 Graph &global_graph();
 void reset_global_graph();
+// installs `g` as the process-wide graph and returns the previous one (used to declare
+// template programs without disturbing the user's)
+Graph *swap_global_graph(Graph *g);
 
 // shape inference for one op; inputs are the input edges in order
 std::vector<std::vector<int>> infer_shapes(const OpDef &def, const std::vector<const Edge *> &in);

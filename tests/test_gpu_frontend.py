@@ -77,3 +77,55 @@ def test_tree_fc_apps_op_by_op(oracle, pairing):
     close(loss, want["loss"], "loss")
     close(grads["dW"], want["grads"]["dW"], "dW")
     close(grads["dBv"], want["grads"]["dBv"], "dBv")
+
+
+@pytest.mark.parametrize("model", ["treelstm", "lstm", "treefc", "treefc_x"])
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_recognised_vertex_functions_run_on_the_fused_round_kernels(oracle, model, pairing):
+    """Session(OPT_BATCHING) on the benchmark apps: F is recognised and lowered onto the
+    fused kernels; results must equal the oracle (and hence the op-by-op path)."""
+    base = {"treefc_x": "treefc"}.get(model, model)
+    w = small_workload(base, 83, B=6, H=16, E=12, V=29, C=5)
+    mask, kw = None, {}
+    if model == "treefc":
+        kw = dict(loss="sum_abs", act=0)
+    elif model == "treefc_x":
+        kw = dict(loss="root_sq", act=1, use_bias=True, use_x=True)
+        mask = np.zeros((w["N"], w["H"]), np.float32)
+        off = 0
+        for row in w["graph"]:
+            n = int(np.argmax(row == -1)) + 1
+            mask[off + n - 1] = 1
+            off += n
+    want = oracle_step(oracle, w, base, pairing=pairing, **kw)
+    loss, go, grads, fused = run_app(model, w, opt=session.OPT_BATCHING, pairing=pairing, allow_fused=True, root_mask=mask)
+    assert fused, "the vertex function was not recognised"
+    close(go, want["graph_out"], "graph_out")
+    close(loss, want["loss"], "loss")
+    for k, v in grads.items():
+        close(v, want["grads"][k], k)
+
+
+def test_serial_sessions_are_never_lowered(oracle):
+    w = small_workload("lstm", 84, B=3, H=8)
+    _, _, _, fused = run_app("lstm", w, opt=0, pairing="reference", allow_fused=True)
+    assert not fused
+
+
+def test_training_steps_update_variables_like_the_oracle(oracle):
+    """Three SGD steps through Session::Run({train}) on the fused path."""
+    w = small_workload("treelstm", 85, B=4, H=8, E=6, V=19, C=3)
+    B, maxlen = w["graph"].shape
+    lr = 0.5
+    a = apps.App("treelstm", B=B, maxlen=maxlen, H=8, E=6, V=19, C_=3, opt=session.OPT_BATCHING, lr=lr)
+    a.set_params(w["params"])
+    p = {k: np.array(v, np.float32) for k, v in w["params"].items()}
+    for step in range(3):
+        print(f"[case] sgd step {step}", flush=True)
+        want = oracle_step(oracle, dict(w, params=p), "treelstm")
+        loss, _ = a.step(w["graph"], w["x"], w["labels"], train=True)
+        close(loss, want["loss"], f"loss at step {step}", rtol=2e-4, atol=2e-5)
+        for k in ("Emb", "W", "U", "Bv", "Wfc", "bfc"):
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    close(a.grad("W", (6, 32), grad=False), p["W"], "W after 3 steps", rtol=2e-4, atol=2e-5)
+    a.close()
