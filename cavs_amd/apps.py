@@ -33,6 +33,8 @@ def libs():
         a.cavs_app_read.restype = C.c_long
         _host.C_DumpGraph.restype = C.c_size_t
         _host.C_DumpGraph.argtypes = [C.c_char_p, C.c_size_t]
+        _host.C_DumpFusedGraph.restype = C.c_size_t
+        _host.C_DumpFusedGraph.argtypes = [C.c_char_p, C.c_size_t]
         _host.C_LastError.restype = C.c_char_p
         _apps = a
     return _apps, _host
@@ -57,6 +59,14 @@ class App:
         n = h.C_DumpGraph(None, 0)
         buf = C.create_string_buffer(n)
         h.C_DumpGraph(buf, n)
+        return buf.value.decode()
+
+    def dump_fused(self):
+        """The programs after the OPT_FUSION pass, with the generated kernel sources."""
+        _, h = libs()
+        n = h.C_DumpFusedGraph(None, 0)
+        buf = C.create_string_buffer(n)
+        h.C_DumpFusedGraph(buf, n)
         return buf.value.decode()
 
     def set_params(self, params):
@@ -114,6 +124,12 @@ class App:
     def fused(self):
         a, _ = libs()
         return bool(a.cavs_app_uses_fused_path())
+
+    @property
+    def generated_kernels(self):
+        """Kernels the OPT_FUSION pass generated for the programs compiled so far."""
+        a, _ = libs()
+        return int(a.cavs_app_generated_kernels())
 
     def close(self):
         a, _ = libs()

@@ -294,6 +294,7 @@ long cavs_app_read(const char *edge, float *out, size_t cap) {
 }
 
 int cavs_app_uses_fused_path(void) { return g_app && g_app->sess->UsesFusedPath(); }
+int cavs_app_generated_kernels(void) { return g_app ? g_app->sess->GeneratedKernels() : 0; }
 
 void cavs_app_destroy(void) {
   delete g_app;

@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "../midend/executor.h"
+#include "../midend/fusion.h"
 #include "../midend/graph.h"
 
 using cavs::mid::Executor;
@@ -146,6 +147,16 @@ size_t C_DumpGraph(char *buf, size_t cap) {
   return d.size() + 1;
 }
 
+size_t C_DumpFusedGraph(char *buf, size_t cap) {
+  std::string d = cavs::mid::dump_fused(cavs::mid::global_graph());
+  if (buf && cap) {
+    size_t n = std::min(cap - 1, d.size());
+    std::memcpy(buf, d.data(), n);
+    buf[n] = 0;
+  }
+  return d.size() + 1;
+}
+
 void C_ResetGraph(void) { cavs::mid::reset_global_graph(); }
 
 int C_SetVariable(C_Session *s, const char *name, const float *data, size_t n) {
@@ -159,6 +170,7 @@ long C_ReadTensor(C_Session *s, const char *name, float *out, size_t cap) {
 }
 
 int C_SessionUsesFusedPath(C_Session *s) { return s->exec.uses_fused_path() ? 1 : 0; }
+int C_SessionGeneratedKernels(C_Session *s) { return s->exec.fused_kernel_count(); }
 void C_SessionAllowFusedPath(C_Session *s, int allow) { s->exec.allow_fused_path(allow != 0); }
 void C_SessionSetPairing(C_Session *s, int pairing) { s->exec.set_pairing(pairing); }
 

@@ -4,6 +4,7 @@
 #include <cmath>
 #include <cstring>
 
+#include "fusion.h"
 #include "lowering.h"
 
 namespace cavs {
@@ -40,6 +41,8 @@ Executor::Executor(int opt, const std::string &name) : opt_(opt), name_(name) {
 Executor::~Executor() {
   cavs_stream_sync(stream_);
   engine_.reset();
+  for (auto &kv : fused_handles_)
+    if (kv.second) cavs_fused_release(kv.second);
   tensors_.clear();
   cavs_stream_destroy(stream_);
 }
@@ -159,6 +162,75 @@ void Executor::compile() {
       lowered_ = lowering_ != nullptr;
     }
   }
+  // programs as executed; with OPT_FUSION connected elementwise operators become generated kernels
+  func_fwd_.clear();
+  func_bwd_ = g.func_backward;
+  func_def_ = g.func_deferred;
+  main_all_.clear();
+  main_cache_.clear();
+  fused_groups_ = 0;
+  for (auto &n : g.main.nodes) main_all_.push_back(n->def);
+  if (g.func)
+    for (auto &n : g.func->nodes) func_fwd_.push_back(n->def);
+  if ((opt_ & OPT_FUSION) && g.func && !lowered_) {
+    std::vector<OpDef> fwd = fused(func_fwd_, {&func_bwd_, &func_def_, &main_all_, &g.opt.backward}, {});
+    std::vector<OpDef> bwd = fused(func_bwd_, {&func_fwd_, &func_def_, &main_all_, &g.opt.backward}, {});
+    func_fwd_.swap(fwd);
+    func_bwd_.swap(bwd);
+  }
+}
+
+std::vector<OpDef> Executor::fused(const std::vector<OpDef> &prog, const std::vector<const std::vector<OpDef> *> &others,
+                                   const std::vector<std::string> &extra_live) {
+  Graph &g = global_graph();
+  FusionEnv env = graph_env(g);
+  for (auto *o : others)
+    for (auto &d : *o)
+      for (int k = 0; k < operands_read(d); k++) env.live.insert(d.input(k));
+  for (auto &v : g.opt.vars) env.live.insert(GetGradientName(v));
+  for (auto &x : extra_live) env.live.insert(x);
+  int made = 0;
+  std::vector<OpDef> out = fuse_program(prog, env, &made);
+  fused_groups_ += made;
+  return out;
+}
+
+// FusedKernel: the generated kernel reads x[idx % x_count], so per-round slabs and
+// broadcast rows go in with their own element counts (cavs/backend/op_impl_fusedkernel.cu)
+void Executor::exec_fused(const OpDef &d, const RoundCtx &c) {
+  const std::string kname = GetSingleArg<std::string>(d, "KernelName", "");
+  void *&h = fused_handles_[kname];
+  if (!h) check(cavs_fused_compile(kname.c_str(), GetSingleArg<std::string>(d, "KernelSource", "").c_str(), &h));
+  std::vector<float *> outs;
+  std::vector<const float *> ins;
+  std::vector<int> oc, ic;
+  long cnt, w, n_elements = 0;
+  for (auto &x : d.input()) {
+    ins.push_back(view(x, c, &cnt, &w));
+    ic.push_back((int)cnt);
+  }
+  for (int i = 0; i < d.output_size(); i++) {
+    const std::string &name = d.output(i);
+    const Edge *e = edge(name);
+    if (!e) fail(CAVS_EINVAL, "no edge for fused output '" + name + "'");
+    auto &slot = tensors_[name];
+    if (!slot) slot = std::make_unique<Tensor>();
+    Tensor &t = *slot;
+    t.width = e->width();
+    t.per_vertex = e->per_vertex();
+    if (t.per_vertex) t.rows = N_;
+    if (t.own.capacity() < t.count()) {
+      check(cavs_stream_sync(stream_));
+      t.own.reserve(t.count() + t.count() / 4);
+    }
+    t.base = t.own.get();
+    outs.push_back(view(name, c, &cnt, &w));
+    oc.push_back((int)cnt);
+    n_elements = std::max(n_elements, cnt);
+  }
+  if (n_elements == 0) return;
+  check(cavs_fused_launch(h, outs.data(), (int)outs.size(), ins.data(), (int)ins.size(), oc.data(), ic.data(),
+                          (int)n_elements, stream_));
 }
 
 // Pointer, element count and row width of an edge as seen by an op running in `c`.
@@ -255,6 +327,7 @@ void Executor::exec(const OpDef &d, const RoundCtx &c) {
 
   long n0, w0, n1, w1, no, wo;
   if (op == "Variable" || op == "Placeholder" || op == "ControlDependency") return;
+  if (op == "FusedKernel") return exec_fused(d, c);
   if (op == "Mirror" || op == "Reshape" || op == "Flatten" || op == "Expand_dims") {
     alias(d.input(0), 0);  // ShareMemory: no copy (cavs/backend/op_impl_reshape.cc)
     return;
@@ -525,20 +598,19 @@ void Executor::upload_lists() {
 }
 
 // GraphStatement::Run, cavs/midend/statement.cc:43-85
-void Executor::run_graph_output(const Node *n) {
-  Graph &g = global_graph();
+void Executor::run_graph_output(const OpDef &d) {
   // the graph placeholder stays on the host (graph_scheduler.cc:15)
-  Tensor &gt = tensor(n->in[0]->name);
-  const Edge *ge = n->in[0];
+  Tensor &gt = tensor(d.input(0));
+  const Edge *ge = edge(d.input(0));
   if (ge->shape.size() != 2) fail(CAVS_EINVAL, "the graph placeholder must be [batch, max vertices]");
   const int32_t *graph = reinterpret_cast<const int32_t *>(gt.base);
-  auto &slot = tensors_[n->out[0]->name];
+  auto &slot = tensors_[d.output(0)];
   if (!slot) slot = std::make_unique<Tensor>();
   Tensor &go = *slot;
   go.width = ret_w_;
   go.per_vertex = true;
   // the vertex placeholder may be left unfed when F never Pulls (apps/paper/tree-fc-cavs.cc:104)
-  Tensor *arg = find_tensor(n->in[1]->name);
+  Tensor *arg = find_tensor(d.input(1));
   func_arg_ = arg ? arg->base : nullptr;
   if (lowered_) {  // the engine schedules, runs the fused rounds and owns GraphOutput
     lowered_forward(graph, ge->shape[0], ge->shape[1], nullptr);
@@ -565,7 +637,7 @@ void Executor::run_graph_output(const Node *n) {
   upload_lists();
   for (const Round &r : sched_.rounds) {
     RoundCtx c{r.offset, r.n, true};
-    for (auto &fn : g.func->nodes) exec(fn->def, c);
+    for (const OpDef &fd : func_fwd_) exec(fd, c);
   }
   // FunctionPopRet: GraphOutput[tids_to_jobids[t]] = ret[t]
   check(cavs_scatter_rows(go.base, (int)ret_w_, d_t2j_, ret_.get(), (int)ret_w_, (int)N_, (int)ret_w_, stream_));
@@ -573,7 +645,6 @@ void Executor::run_graph_output(const Node *n) {
 
 // GraphGradStatement::Run, cavs/midend/statement.cc:87-123
 void Executor::run_graph_output_grad(const OpDef &d) {
-  Graph &g = global_graph();
   dgo_ = tensor(d.input(0)).base;
   if (lowered_) {
     lowered_backward(d);
@@ -582,10 +653,10 @@ void Executor::run_graph_output_grad(const OpDef &d) {
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     RoundCtx c{r.offset, r.n, true};
-    for (const OpDef &gd : g.func_backward) exec(gd, c);
+    for (const OpDef &gd : func_bwd_) exec(gd, c);
   }
   RoundCtx all{0, N_, true};
-  for (const OpDef &gd : g.func_deferred) exec(gd, all);
+  for (const OpDef &gd : func_def_) exec(gd, all);
 }
 
 // ------------------------------------------------------------------ Session::Run
@@ -627,11 +698,27 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
   std::vector<const Node *> order;
   forward_needed(targets, &order);
   RoundCtx mainctx{0, 0, false};
-  for (const Node *n : order) {
-    if (n->def.name() == "GraphOutput") run_graph_output(n); else exec(n->def, mainctx);
+  std::string key = train ? "T" : "F";
+  for (auto &t : targets) key += "|" + t;
+  auto it = main_cache_.find(key);
+  if (it == main_cache_.end()) {
+    MainProgram mp;
+    for (const Node *n : order) mp.fwd.push_back(n->def);
+    if (train) mp.bwd = g.opt.backward;
+    if (opt_ & OPT_FUSION) {
+      std::vector<OpDef> none, fwd, bwd;
+      fwd = fused(mp.fwd, {&func_fwd_, &func_bwd_, &func_def_, train ? &g.opt.backward : &none}, targets);
+      if (train) bwd = fused(mp.bwd, {&func_fwd_, &func_bwd_, &func_def_}, targets);
+      mp.fwd.swap(fwd);
+      mp.bwd.swap(bwd);
+    }
+    it = main_cache_.emplace(key, std::move(mp)).first;
+  }
+  for (const OpDef &d : it->second.fwd) {
+    if (d.name() == "GraphOutput") run_graph_output(d); else exec(d, mainctx);
   }
   if (train) {
-    for (const OpDef &d : g.opt.backward) {
+    for (const OpDef &d : it->second.bwd) {
       if (d.name() == "GraphOutput_grad") run_graph_output_grad(d); else exec(d, mainctx);
     }
     // SGD: w -= lr * g (cavs/backend/op_impl_sgd.cu); clipping is not on the measured path

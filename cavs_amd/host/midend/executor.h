@@ -46,6 +46,7 @@ class Executor {
   void set_variable(const std::string &name, const float *data, size_t n);
   long read_tensor(const std::string &name, float *out, size_t cap);
   bool uses_fused_path() const { return lowered_; }
+  int fused_kernel_count() const { return fused_groups_; }
   void allow_fused_path(bool a) { allow_fused_ = a; compiled_version_ = -1; }
   void set_pairing(int p) { pairing_ = p; compiled_version_ = -1; }
 
@@ -60,7 +61,10 @@ class Executor {
   Tensor *find_tensor(const std::string &name);
   float *view(const std::string &name, const RoundCtx &c, long *count, long *width);
   void exec(const OpDef &d, const RoundCtx &c);
-  void run_graph_output(const Node *n);
+  void run_graph_output(const OpDef &d);
+  void exec_fused(const OpDef &d, const RoundCtx &c);
+  std::vector<OpDef> fused(const std::vector<OpDef> &prog, const std::vector<const std::vector<OpDef> *> &others,
+                           const std::vector<std::string> &extra_live);
   void run_graph_output_grad(const OpDef &d);
   void upload_lists();
   void lowered_forward(const int32_t *graph, int B, int maxlen, float *graph_out);
@@ -90,6 +94,13 @@ class Executor {
   const int *d_t2j_ = nullptr, *d_pair_ = nullptr, *d_child_[2] = {nullptr, nullptr};
   const float *func_arg_ = nullptr;   // vertex placeholder on the device
   const float *dgo_ = nullptr;        // d GraphOutput during the backward function
+  // programs of the vertex function as executed (after the fusion pass when OPT_FUSION is set)
+  std::vector<OpDef> func_fwd_, func_bwd_, func_def_;
+  std::vector<OpDef> main_all_;
+  struct MainProgram { std::vector<OpDef> fwd, bwd; };
+  std::map<std::string, MainProgram> main_cache_;  // keyed by the requested targets
+  std::map<std::string, void *> fused_handles_;    // kernel name -> compiled module
+  int fused_groups_ = 0;
   std::unique_ptr<Engine> engine_;
   std::unique_ptr<Lowering> lowering_;
 };

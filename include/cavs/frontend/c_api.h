@@ -50,6 +50,8 @@ int C_SetVariable(C_Session *s, const char *name, const float *data, size_t n);
 long C_ReadTensor(C_Session *s, const char *name, float *out, size_t cap);
 /* 1 if the vertex function was recognised and lowered onto the fused round kernels. */
 int C_SessionUsesFusedPath(C_Session *s);
+/* Number of kernels the OPT_FUSION pass generated for the programs compiled so far. */
+int C_SessionGeneratedKernels(C_Session *s);
 /* 0 forbids that lowering (op-by-op execution of F, for A/B tests); default 1. */
 void C_SessionAllowFusedPath(C_Session *s, int allow);
 void C_SessionSetPairing(C_Session *s, int pairing); /* CAVS_PAIR_* of cavs_session.h */
@@ -57,6 +59,8 @@ const char *C_LastError(void);
 /* Text dump of the declared program: forward ops, the vertex function, and the backward
  * programs the autograd pass derived.  Returns the length needed (including the NUL). */
 size_t C_DumpGraph(char *buf, size_t cap);
+/* The same programs after the OPT_FUSION pass, with the generated kernel sources. */
+size_t C_DumpFusedGraph(char *buf, size_t cap);
 
 #ifdef __cplusplus
 }

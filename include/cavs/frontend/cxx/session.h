@@ -32,6 +32,7 @@ class Session {
   void SetVariable(const Sym &var, const float *data, size_t n);
   std::vector<float> Read(const std::string &edge_name);
   bool UsesFusedPath() const { return C_SessionUsesFusedPath(s_) != 0; }
+  int GeneratedKernels() const { return C_SessionGeneratedKernels(s_); }
   void AllowFusedPath(bool allow) { C_SessionAllowFusedPath(s_, allow ? 1 : 0); }
   void SetPairing(int pairing) { C_SessionSetPairing(s_, pairing); }
   C_Session *handle() const { return s_; }

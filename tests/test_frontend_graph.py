@@ -60,3 +60,50 @@ def test_seq_lstm_and_tree_fc_programs(declare):
     c = declare("treefc_x", B=2, maxlen=7, H=4)
     d = c.dump()
     assert "Tanh_grad(" in d and "Square(" in d
+
+
+def test_fusion_pass_groups_the_gate_arithmetic_of_tree_lstm():
+    """OPT_FUSION's pass on the Tree-LSTM app, no device needed: the gate arithmetic of F
+    becomes one generated kernel, that of the backward function another; the kernel sits
+    before the Concat/Scatter that read its results, and broadcast operands wrap."""
+    import re
+    from cavs_amd import apps
+
+    a = apps.App("treelstm", B=2, maxlen=5, H=8, E=8, V=10, C_=3, opt=-1, lr=0.1)
+    try:
+        plain, d = a.dump(), a.dump_fused()
+    finally:
+        a.close()
+    assert "FusedKernel" not in plain
+    fn = d[d.index("function:"):d.index("function_grad:")]
+    bw = d[d.index("function_grad:"):d.index("backward:")]
+    assert fn.count("FusedKernel(") == 1 and bw.count("FusedKernel(") == 1
+    # every Sigmoid/Tanh/Add/Mul of the gates is inside the kernel, none left as an op
+    assert not re.search(r"^  (Sigmoid|Tanh|Mul)\(", fn, re.M)
+    assert fn.count("expf(") == 4 and fn.count("tanhf(") == 2
+    assert fn.index("FusedKernel(") < fn.index("  Concat(") < fn.index("  Scatter(")
+    # the kernel keeps the reference's signature: outputs, const inputs, counts, n_elements
+    sig = re.search(r'extern "C" __global__ void (FusedKernel_\d+)\((.*?)\)\n', fn, re.S).group(2)
+    kinds = [("out" if p.startswith("float *") else "in" if p.startswith("const float *") else "count")
+             for p in sig.split(", ")]
+    assert kinds[-1] == "count" and sig.endswith("const int n_elements")
+    assert kinds == sorted(kinds, key=["out", "in", "count"].index)
+    assert kinds.count("count") == kinds.count("out") + kinds.count("in") + 1
+    # a bias row is a broadcast operand; a per-vertex slab is indexed directly
+    assert re.search(r"tmp_Mirror_\d+ = Mirror_\d+\[idx % Mirror_\d+_count\]", fn)
+    assert re.search(r"tmp_Slice_\d+ = Slice_\d+\[idx\]", fn)
+    # the backward kernel accumulates onto gradients that an earlier op already wrote
+    assert re.search(r"float tmp_(\w+_grad) = \1\[idx\] \+ \(", bw)
+
+
+def test_fusion_pass_keeps_small_groups_unfused():
+    """A group pays only with two or more arithmetic members (cavs/midend/runtime_compiler/parser.cc:118-131)."""
+    from cavs_amd import apps
+
+    a = apps.App("treefc", B=2, maxlen=5, H=8, opt=-1, lr=0.1)
+    try:
+        d = a.dump_fused()
+    finally:
+        a.close()
+    fn = d[d.index("function:"):d.index("function_grad:")]
+    assert "FusedKernel(" not in fn  # forward F has a single Relu

@@ -22,7 +22,7 @@ def oracle_step(oracle, w, model, **kw):
                              Cc=w["C"], **kw)
 
 
-def run_app(model, w, *, opt, pairing, allow_fused, root_mask=None):
+def run_app(model, w, *, opt, pairing, allow_fused, root_mask=None, want_generated=False):
     B, maxlen = w["graph"].shape
     a = apps.App(model, B=B, maxlen=maxlen, H=w["H"], E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=0.0,
                  pairing=pairing, allow_fused=allow_fused)
@@ -36,7 +36,10 @@ def run_app(model, w, *, opt, pairing, allow_fused, root_mask=None):
               "U": (4 * H * H,), "Bv": (H,) if model.startswith("treefc") else (4 * H,), "Wfc": (C, H), "bfc": (C,)}
     grads = {"d" + k: a.grad(k, shapes[k]) for k in names}
     fused = a.fused
+    generated = a.generated_kernels
     a.close()
+    if want_generated:
+        return loss, go, grads, fused, generated
     return loss, go, grads, fused
 
 
@@ -129,3 +132,56 @@ def test_training_steps_update_variables_like_the_oracle(oracle):
             p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
     close(a.grad("W", (6, 32), grad=False), p["W"], "W after 3 steps", rtol=2e-4, atol=2e-5)
     a.close()
+
+
+def _root_mask(w):
+    mask = np.zeros((w["N"], w["H"]), np.float32)
+    off = 0
+    for row in w["graph"]:
+        n = int(np.argmax(row == -1)) + 1
+        mask[off + n - 1] = 1
+        off += n
+    return mask
+
+
+@pytest.mark.parametrize("model", ["treelstm", "lstm", "treefc", "treefc_x"])
+@pytest.mark.parametrize("opt", [session.OPT_BATCHING | session.OPT_FUSION, session.OPT_FUSION])
+def test_generated_kernels_of_the_fusion_pass_match_oracle(oracle, model, opt):
+    """OPT_FUSION on the op-by-op path: the elementwise groups of F and of its backward
+    function run as kernels generated and compiled at run time; values must not move."""
+    base = {"treefc_x": "treefc"}.get(model, model)
+    w = small_workload(base, 86, B=5, H=8, E=6, V=23, C=4)
+    mask, kw = None, {}
+    if model == "treefc":
+        kw = dict(loss="sum_abs", act=0)
+    elif model == "treefc_x":
+        kw = dict(loss="root_sq", act=1, use_bias=True, use_x=True)
+        mask = _root_mask(w)
+    want = oracle_step(oracle, w, base, batching=bool(opt & session.OPT_BATCHING), **kw)
+    loss, go, grads, fused, generated = run_app(model, w, opt=opt, pairing="reference", allow_fused=False,
+                                                root_mask=mask, want_generated=True)
+    assert not fused
+    assert generated >= 1
+    close(go, want["graph_out"], "graph_out")
+    close(loss, want["loss"], "loss")
+    for k, v in grads.items():
+        close(v, want["grads"][k], k)
+
+
+def test_reference_smoke_programs_print_their_known_values():
+    """session_test.cc and fusion_session_test.cc of the reference, same programs, same feeds."""
+    import ctypes as C
+    import json
+    import os
+
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "smoke_kats.json")))
+    lib, _ = apps.libs()
+    out = (C.c_float * 6)()
+    assert lib.cavs_smoke_session_add(out) == 0
+    np.testing.assert_array_equal(np.array(out[:]), np.array(kat["session_add"]["expect"], np.float32))
+    for opt, expect_kernels in ((session.OPT_FUSION, 2), (0, 0)):
+        e, yy, n = (C.c_float * 6)(), (C.c_float * 4)(), C.c_int(-1)
+        assert lib.cavs_smoke_fusion(opt, e, yy, C.byref(n)) == 0
+        np.testing.assert_allclose(np.array(e[:]), np.array(kat["fusion_E"]["expect"], np.float32), rtol=1e-6)
+        np.testing.assert_allclose(np.array(yy[:]), np.array(kat["fusion_YY"]["expect"], np.float32), rtol=1e-6)
+        assert n.value == expect_kernels

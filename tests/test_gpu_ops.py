@@ -467,3 +467,15 @@ def test_device_frontier_matches_host_schedule_bit_exact(g, oracle, kind, seed, 
     assert g.host(j2t).tolist() == inv.tolist()
     want_round = np.concatenate([[r] * len(rd["exec"]) for r, rd in enumerate(tr["fwd"])])
     assert g.host(rot).tolist() == want_round.tolist()
+
+
+def test_reference_elementwise_smoke_values(g):
+    """The Add the reference's op_impl_elementwise_test.cc prints: {1..6} + {0..5}."""
+    import json
+    import os
+
+    kat = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "smoke_kats.json")))["elementwise_add"]
+    a, b = np.array(kat["a"], np.float32), np.array(kat["b"], np.float32)
+    out = g.zeros(6)
+    g.call("cavs_ew_binary", hip.EW_BINARY["add"], g.P(out), g.P(g.devf(a)), 6, g.P(g.devf(b)), 6, 6, 0, g.stream())
+    np.testing.assert_array_equal(g.host(out), np.array(kat["expect"], np.float32))
