@@ -47,7 +47,7 @@ def make_pool(name, n_batches):
     return pool
 
 
-def cpu_baseline(w, budget_s=20.0):
+def cpu_baseline(w, budget_s=12.0):
     """Times the CPU checker on this host on a bounded sample of the same workload."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import pyoracle
@@ -61,7 +61,7 @@ def cpu_baseline(w, budget_s=20.0):
         pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **args)
         steps += 1
         el = time.perf_counter() - t0
-        if el > budget_s or steps >= 8 or el + el / steps > 1.5 * budget_s:
+        if el > budget_s or steps >= 400 or el + el / steps > 1.5 * budget_s:
             break
     return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port",
                 sample=f"{steps} full fwd+bwd step(s) of the {w['name']} batch (B={w['B']}, N={w['N']}) "
