@@ -1,0 +1,528 @@
+// One round of the Tree-LSTM vertex function in one launch (forward) or two (backward).
+//
+// A round of n vertices is n rows times five products against slices of the recurrent
+// weights (h_l+h_r with the i, o, u blocks of U_iou; h_l and h_r with U_f), the gate
+// arithmetic, and row movement through the child and scatter lists.  As separate kernels
+// that is a chain of five launches whose intermediates make a round trip through HBM; for
+// the rounds of a batch of parse trees (a few hundred rows down to one) the chain is
+// bound by launch latency, not by the matrix cores.  Here one workgroup owns a
+// (RT*TILE rows) x (TILE columns of H) piece of the round's output:
+//   * its eight wavefronts split the K range of the products between them and feed the
+//     MFMA straight from global memory -- the A operand rows are read through the child
+//     list (the gather is the operand fetch), B is TILE consecutive floats per k, so
+//     neither needs staging through LDS;
+//   * the five partial tiles are summed through LDS in wavefront order (deterministic),
+//     which leaves all five pre-activations of an output element in one thread;
+//   * the epilogue applies the gates and writes the message into the pool row named by
+//     the scatter list, plus everything the backward pass reads again (gates, gathered
+//     children, h_l+h_r).
+// TILE is 32 (v_mfma_f32_32x32x2_f32) or, for rounds of a few rows near the roots, 16
+// (v_mfma_f32_16x16x4_f32), which spreads a tiny round over four times as many CUs.
+#include "common.h"
+
+namespace cavs {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <int TILE>
+struct Mma;
+
+// 32x32x2: lane l supplies A[row l%32][k l/32] and B[k l/32][col l%32]; accumulator
+// element r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+template <>
+struct Mma<32> {
+  static constexpr int NR = 16, NSLOT = 2;
+  typedef floatx16 Acc;
+  static __device__ inline Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+  static __device__ inline int row(int r, int lane) { return 8 * (r / 4) + 4 * (lane >> 5) + (r % 4); }
+};
+
+// 16x16x4: lane l supplies A[row l%16][k l/16] and B[k l/16][col l%16]; accumulator
+// element r of lane l is row 4*(l/16) + r, column l%16.
+template <>
+struct Mma<16> {
+  static constexpr int NR = 4, NSLOT = 4;
+  typedef floatx4 Acc;
+  static __device__ inline Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+  static __device__ inline int row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
+__device__ inline float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ inline float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
+__device__ inline float elem(const float4 &v, int c) { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
+__device__ inline float sigm_r(float x) { return 1.f / (1.f + expf(-x)); }
+
+constexpr int kRoundThreads = 512;
+constexpr int kRoundWaves = kRoundThreads / 64;
+
+// Sums the per-wavefront partial tiles of NP products into `red` in k-split order and
+// leaves them laid out as [row tile][product][accumulator element][lane].
+template <int TILE, int NP, int KS>
+__device__ inline void reduce_partials(float *red, const typename Mma<TILE>::Acc (&acc)[NP], int rt, int ks, int lane) {
+  constexpr int NR = Mma<TILE>::NR;
+  for (int w = 0; w < KS; w++) {
+    if (ks == w) {
+#pragma unroll
+      for (int p = 0; p < NP; p++)
+#pragma unroll
+        for (int r = 0; r < NR; r++) {
+          float *q = red + ((rt * NP + p) * NR + r) * 64 + lane;
+          *q = (w == 0) ? acc[p][r] : *q + acc[p][r];
+        }
+    }
+    __syncthreads();
+  }
+}
+
+// ------------------------------------------------------------------ forward
+struct RoundFwdArgs {
+  const float *pool;   // [*, 2H] message pool, rows [h|c]
+  const int *child;    // [2n] pool rows of the children of slab row b at 2b, 2b+1 (-1: none)
+  const int *pair;     // [n] pool row the message of slab row b goes to (-1: nowhere)
+  const float *xW;     // [n, 4H] (ld_xw) blocks [i|o|u|f]
+  long ld_xw;
+  const float *U;      // [H, 3H] blocks [i|o|u], then [H, H] (forget gate)
+  const float *bias;   // [4H] blocks [i|f|u|o]
+  float *G;            // [2n, 2H] gathered children (saved for backward)
+  float *hlr;          // [n, H] h_l + h_r (saved for the weight gradient)
+  float *gates;        // [n, 6H]
+  float *msg;          // [n, 2H]
+  float *pool_out;     // same buffer as pool: rows of this round are written, rows of earlier rounds read
+  int n, H;
+};
+
+template <int TILE, int RT>
+__global__ __launch_bounds__(kRoundThreads) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
+  using M = Mma<TILE>;
+  using Acc = typename M::Acc;
+  constexpr int KS = kRoundWaves / RT, GK = 4 * M::NSLOT, NP = 5, NR = M::NR;
+  constexpr int UG = 2;  // k-groups per pipeline stage
+  __shared__ float red[RT * NP * NR * 64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rt = wave / KS, ks = wave % KS;
+  const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int H = a.H;
+  const long H2 = 2L * H, H3 = 3L * H;
+  const int j0 = blockIdx.x * TILE;
+  const int row = (blockIdx.y * RT + rt) * TILE + x;
+  int cl = -1, cr = -1;
+  if (row < a.n) {
+    cl = a.child[2 * row];
+    cr = a.child[2 * row + 1];
+  }
+  const float *pl = a.pool + (cl >= 0 ? cl : 0) * H2, *pr = a.pool + (cr >= 0 ? cr : 0) * H2;
+  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
+  const int kb = ks * kper, ke = min(H, kb + kper);
+  const float *Uio = a.U + j0 + x, *Uf = a.U + H3 * H + j0 + x;
+
+  Acc acc[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
+
+  struct Frag {
+    float4 hl[UG], hr[UG];
+    float b[UG][4][4];
+  };
+  auto fetch = [&](int k0, Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+      const int kk = k0 + GK * u + 4 * slot;
+      const bool kin = kk < ke;  // H is a multiple of 4: a float4 is wholly in or out
+      f.hl[u] = (kin && cl >= 0) ? ld4(pl + kk) : zero4();
+      f.hr[u] = (kin && cr >= 0) ? ld4(pr + kk) : zero4();
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float *ui = Uio + (long)(kin ? kk + c : 0) * H3;
+        f.b[u][0][c] = kin ? ui[0] : 0.f;
+        f.b[u][1][c] = kin ? ui[H] : 0.f;
+        f.b[u][2][c] = kin ? ui[2 * H] : 0.f;
+        f.b[u][3][c] = kin ? Uf[(long)(kk + c) * H] : 0.f;
+      }
+    }
+  };
+  auto multiply = [&](const Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float hl = elem(f.hl[u], c), hr = elem(f.hr[u], c), hs = hl + hr;
+        acc[0] = M::mma(hs, f.b[u][0][c], acc[0]);
+        acc[1] = M::mma(hs, f.b[u][1][c], acc[1]);
+        acc[2] = M::mma(hs, f.b[u][2][c], acc[2]);
+        acc[3] = M::mma(hl, f.b[u][3][c], acc[3]);
+        acc[4] = M::mma(hr, f.b[u][3][c], acc[4]);
+      }
+  };
+  Frag f0, f1;
+  constexpr int S = GK * UG;
+  if (kb < ke) fetch(kb, f0);
+  for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+    if (k0 + S < ke) fetch(k0 + S, f1);
+    multiply(f0);
+    if (k0 + S < ke) {
+      if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+      multiply(f1);
+    }
+  }
+
+  reduce_partials<TILE, NP, KS>(red, acc, rt, ks, lane);
+
+  // epilogue: element (t, r, l2) of the workgroup's tiles is slab row b, column j
+  const float *bias = a.bias;
+  for (int e = tid; e < RT * NR * 64; e += kRoundThreads) {
+    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
+    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2), j = j0 + (l2 & (TILE - 1));
+    if (b >= a.n) continue;
+    const float *pre = red + (t * NP * NR + r) * 64 + l2;
+    const float hi = pre[0], ho = pre[NR * 64], hu = pre[2 * NR * 64], fl = pre[3 * NR * 64], fr = pre[4 * NR * 64];
+    const int c_l = a.child[2 * b], c_r = a.child[2 * b + 1];
+    float hl = 0.f, cl_ = 0.f, hr = 0.f, cr_ = 0.f;
+    if (c_l >= 0) { hl = a.pool[c_l * H2 + j]; cl_ = a.pool[c_l * H2 + H + j]; }
+    if (c_r >= 0) { hr = a.pool[c_r * H2 + j]; cr_ = a.pool[c_r * H2 + H + j]; }
+    const float *xw = a.xW + b * a.ld_xw + j;
+    // same association as the separate gate kernel: (x*W + h*U) + bias
+    const float i = sigm_r((xw[0] + hi) + bias[j]);
+    const float o = sigm_r((xw[H] + ho) + bias[3 * H + j]);
+    const float u = tanhf((xw[2 * H] + hu) + bias[2 * H + j]);
+    const float f_l = sigm_r((xw[3 * H] + fl) + bias[H + j]);
+    const float f_r = sigm_r((xw[3 * H] + fr) + bias[H + j]);
+    const float c = (i * u + f_l * cl_) + f_r * cr_;
+    const float tc = tanhf(c);
+    const float h = o * tc;
+    float *g = a.gates + (long)b * 6 * H + j;
+    g[0] = i; g[H] = o; g[2 * H] = u; g[3 * H] = f_l; g[4 * H] = f_r; g[5 * H] = tc;
+    float *m = a.msg + b * H2 + j;
+    m[0] = h; m[H] = c;
+    const int dst = a.pair[b];
+    if (dst >= 0) {
+      a.pool_out[dst * H2 + j] = h;
+      a.pool_out[dst * H2 + H + j] = c;
+    }
+    float *gl = a.G + (2L * b) * H2 + j, *gr = gl + H2;
+    gl[0] = hl; gl[H] = cl_; gr[0] = hr; gr[H] = cr_;
+    a.hlr[(long)b * H + j] = hl + hr;
+  }
+}
+
+// ------------------------------------------------------------------ backward, gate part
+// Elementwise: reads the message gradient through the scatter list (grad of Scatter is
+// Gather), writes the pre-activation gradients and the c half of the children's message
+// gradients straight into the children's pool rows (grad of Gather is Scatter).
+struct RoundBwdGatesArgs {
+  const float *dpool;   // [*, 2H] gradient of the message pool
+  const int *pair;      // [n]
+  const int *child;     // [2n] or nullptr for a round of leaves
+  const float *dret;    // [n, H] gradient of the pushed return value
+  const float *gates;   // [n, 6H]
+  const float *G;       // [2n, 2H] or nullptr for leaves
+  float *dxW;           // [n, 4H] (ld_dxw) blocks [i|o|u|f_l+f_r]
+  long ld_dxw;
+  float *dF;            // [2n, H] rows (2b: f_l, 2b+1: f_r) or nullptr
+  float *dpool_out;     // same buffer as dpool
+  int n, H;
+};
+
+template <int W>
+__global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
+  const int H = a.H, hw = H / W;
+  const long H2 = 2L * H;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int src = a.pair[r];
+  const float *g = a.gates + (long)r * 6 * H + j;
+  const bool internal = a.child != nullptr;
+  int c_l = -1, c_r = -1;
+  if (internal) { c_l = a.child[2 * r]; c_r = a.child[2 * r + 1]; }
+  float dmh[W], dmc[W], dr[W], gi[W], go[W], gu[W], gfl[W], gfr[W], gtc[W], cl[W], cr[W];
+  if constexpr (W == 4) {
+    auto ld = [](const float *p, float (&o)[W]) { float4 v = ld4(p); o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; };
+    ld(g, gi); ld(g + H, go); ld(g + 2 * H, gu); ld(g + 3 * H, gfl); ld(g + 4 * H, gfr); ld(g + 5 * H, gtc);
+    ld(a.dret + (long)r * H + j, dr);
+    if (src >= 0) { ld(a.dpool + src * H2 + j, dmh); ld(a.dpool + src * H2 + H + j, dmc); }
+    if (internal) { ld(a.G + (2L * r) * H2 + H + j, cl); ld(a.G + (2L * r + 1) * H2 + H + j, cr); }
+  } else {
+#pragma unroll
+    for (int k = 0; k < W; k++) {
+      gi[k] = g[k]; go[k] = g[H + k]; gu[k] = g[2 * H + k]; gfl[k] = g[3 * H + k]; gfr[k] = g[4 * H + k]; gtc[k] = g[5 * H + k];
+      dr[k] = a.dret[(long)r * H + j + k];
+      if (src >= 0) { dmh[k] = a.dpool[src * H2 + j + k]; dmc[k] = a.dpool[src * H2 + H + j + k]; }
+      if (internal) { cl[k] = a.G[(2L * r) * H2 + H + j + k]; cr[k] = a.G[(2L * r + 1) * H2 + H + j + k]; }
+    }
+  }
+  float di[W], dvo[W], du[W], dfs[W], dfl[W], dfr[W], dcl[W], dcr[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const float mh = src >= 0 ? dmh[k] : 0.f, mc = src >= 0 ? dmc[k] : 0.f;
+    const float c_left = internal ? cl[k] : 0.f, c_right = internal ? cr[k] : 0.f;
+    const float i = gi[k], o = go[k], u = gu[k], f_l = gfl[k], f_r = gfr[k], tc = gtc[k];
+    const float dh = mh + dr[k];
+    const float d_o = dh * tc;
+    const float dc = mc + (dh * o) * (1.f - tc * tc);
+    const float del_fl = (dc * c_left) * (f_l * (1.f - f_l));
+    const float del_fr = (dc * c_right) * (f_r * (1.f - f_r));
+    di[k] = (dc * u) * (i * (1.f - i));
+    dvo[k] = d_o * (o * (1.f - o));
+    du[k] = (dc * i) * (1.f - u * u);
+    dfs[k] = del_fl + del_fr;
+    dfl[k] = del_fl; dfr[k] = del_fr;
+    dcl[k] = dc * f_l; dcr[k] = dc * f_r;
+  }
+  auto st = [](float *p, const float (&v)[W]) {
+    if constexpr (W == 4) {
+      *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < W; k++) p[k] = v[k];
+    }
+  };
+  float *dx = a.dxW + r * a.ld_dxw + j;
+  st(dx, di); st(dx + H, dvo); st(dx + 2 * H, du); st(dx + 3 * H, dfs);
+  if (internal) {
+    st(a.dF + (2L * r) * H + j, dfl);
+    st(a.dF + (2L * r + 1) * H + j, dfr);
+    if (c_l >= 0) st(a.dpool_out + c_l * H2 + H + j, dcl);
+    if (c_r >= 0) st(a.dpool_out + c_r * H2 + H + j, dcr);
+  }
+}
+
+// ------------------------------------------------------------------ backward, children part
+// dh_l = [d_i|d_o|d_u] * U_iou^T + d_fl * U_f^T, dh_r likewise with d_fr, written into the h
+// half of the children's pool-gradient rows.  UT holds the transposed weights ([3H,H] then
+// [H,H]) so that the B operand is TILE consecutive floats per k, as in the forward kernel.
+struct RoundBwdChildArgs {
+  const float *dxW;   // [n, 4H] (ld_dxw); columns [0, 3H) are read
+  long ld_dxw;
+  const float *dF;    // [2n, H]
+  const float *UT;    // [3H, H] = U_iou^T, then [H, H] = U_f^T
+  const int *child;   // [2n]
+  float *dpool;       // [*, 2H]
+  int n, H;
+};
+
+template <int TILE, int RT>
+__global__ __launch_bounds__(kRoundThreads) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
+  using M = Mma<TILE>;
+  using Acc = typename M::Acc;
+  constexpr int KS = kRoundWaves / RT, GK = 4 * M::NSLOT, NP = 3, NR = M::NR;
+  constexpr int UG = 2;
+  __shared__ float red[RT * NP * NR * 64];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rt = wave / KS, ks = wave % KS;
+  const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int H = a.H;
+  const long H2 = 2L * H;
+  const int j0 = blockIdx.x * TILE;
+  const int row = (blockIdx.y * RT + rt) * TILE + x;
+  const bool rin = row < a.n;
+  const float *px = a.dxW + (rin ? row : 0) * a.ld_dxw;
+  const float *pfl = a.dF + (rin ? 2L * row : 0) * H, *pfr = pfl + (rin ? H : 0);
+  const float *UTio = a.UT + j0 + x, *UTf = a.UT + 3L * H * H + j0 + x;
+
+  Acc acc[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
+
+  constexpr int S = GK * UG;
+  {  // P0: K = 3H
+    const int K = 3 * H;
+    const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
+    const int kb = ks * kper, ke = min(K, kb + kper);
+    struct Frag {
+      float4 a[UG];
+      float b[UG][4];
+    };
+    auto fetch = [&](int k0, Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++) {
+        const int kk = k0 + GK * u + 4 * slot;
+        const bool kin = kk < ke;
+        f.a[u] = (kin && rin) ? ld4(px + kk) : zero4();
+#pragma unroll
+        for (int c = 0; c < 4; c++) f.b[u][c] = kin ? UTio[(long)(kk + c) * H] : 0.f;
+      }
+    };
+    auto multiply = [&](const Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[0] = M::mma(elem(f.a[u], c), f.b[u][c], acc[0]);
+    };
+    Frag f0, f1;
+    if (kb < ke) fetch(kb, f0);
+    for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+      if (k0 + S < ke) fetch(k0 + S, f1);
+      multiply(f0);
+      if (k0 + S < ke) {
+        if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+        multiply(f1);
+      }
+    }
+  }
+  {  // P1, P2: K = H, one B operand for both
+    const int K = H;
+    const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
+    const int kb = ks * kper, ke = min(K, kb + kper);
+    struct Frag {
+      float4 l[UG], r[UG];
+      float b[UG][4];
+    };
+    auto fetch = [&](int k0, Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++) {
+        const int kk = k0 + GK * u + 4 * slot;
+        const bool kin = kk < ke;
+        f.l[u] = (kin && rin) ? ld4(pfl + kk) : zero4();
+        f.r[u] = (kin && rin) ? ld4(pfr + kk) : zero4();
+#pragma unroll
+        for (int c = 0; c < 4; c++) f.b[u][c] = kin ? UTf[(long)(kk + c) * H] : 0.f;
+      }
+    };
+    auto multiply = [&](const Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          acc[1] = M::mma(elem(f.l[u], c), f.b[u][c], acc[1]);
+          acc[2] = M::mma(elem(f.r[u], c), f.b[u][c], acc[2]);
+        }
+    };
+    Frag f0, f1;
+    if (kb < ke) fetch(kb, f0);
+    for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+      if (k0 + S < ke) fetch(k0 + S, f1);
+      multiply(f0);
+      if (k0 + S < ke) {
+        if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+        multiply(f1);
+      }
+    }
+  }
+
+  reduce_partials<TILE, NP, KS>(red, acc, rt, ks, lane);
+
+  for (int e = tid; e < RT * NR * 64; e += kRoundThreads) {
+    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
+    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2), j = j0 + (l2 & (TILE - 1));
+    if (b >= a.n) continue;
+    const float *pre = red + (t * NP * NR + r) * 64 + l2;
+    const float p0 = pre[0], p1 = pre[NR * 64], p2 = pre[2 * NR * 64];
+    const int c_l = a.child[2 * b], c_r = a.child[2 * b + 1];
+    if (c_l >= 0) a.dpool[c_l * H2 + j] = p0 + p1;
+    if (c_r >= 0) a.dpool[c_r * H2 + j] = p0 + p2;
+  }
+}
+
+// out[c][r] = in[r][c]
+__global__ void transpose_kernel(float *__restrict__ out, const float *__restrict__ in, int rows, int cols) {
+  __shared__ float tile[32][33];
+  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  for (int i = ty; i < 32; i += 8)
+    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = in[(long)(r0 + i) * cols + c0 + tx];
+  __syncthreads();
+  for (int i = ty; i < 32; i += 8)
+    if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+static bool round_shape_ok(int H) { return H > 0 && H % 32 == 0; }
+
+// tile shape and row tiles per workgroup for a round of n rows
+struct RoundPlan {
+  int tile, rt;
+};
+static RoundPlan plan_round(int n) {
+  if (n <= 16) return {16, 1};
+  if (n <= 32) return {16, 2};
+  if (n <= 64) return {16, 4};
+  return {32, n > 512 ? 2 : 1};
+}
+
+}  // namespace cavs
+
+using namespace cavs;
+
+extern "C" {
+
+int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                            const float *U, const float *bias, float *G, float *hlr, float *gates,
+                            float *msg, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && ld_xw >= 4 * H && ld_xw % 4 == 0,
+               "cavs_treelstm_round_fwd: bad shape n=%d H=%d ld_xw=%d (H must be a multiple of 32)", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && child && pair && xW && U && bias && G && hlr && gates && msg, "cavs_treelstm_round_fwd: null pointer");
+  CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
+  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, n, H};
+  const RoundPlan p = plan_round(n);
+  dim3 grid(H / p.tile, (n + p.tile * p.rt - 1) / (p.tile * p.rt));
+  hipStream_t st = as_stream(stream);
+  if (p.tile == 16 && p.rt == 1) treelstm_round_fwd_kernel<16, 1><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.tile == 16 && p.rt == 2) treelstm_round_fwd_kernel<16, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.tile == 16) treelstm_round_fwd_kernel<16, 4><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.rt == 1) treelstm_round_fwd_kernel<32, 1><<<grid, kRoundThreads, 0, st>>>(a);
+  else treelstm_round_fwd_kernel<32, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret,
+                                  const float *gates, const float *G, float *dxW, int ld_dxw, float *dF,
+                                  int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && ld_dxw >= 4 * H, "cavs_treelstm_round_bwd_gates: bad shape n=%d H=%d ld=%d", n, H, ld_dxw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dpool && pair && dret && gates && dxW, "cavs_treelstm_round_bwd_gates: null pointer");
+  CAVS_REQUIRE((child && G && dF) || (!child && !G && !dF),
+               "cavs_treelstm_round_bwd_gates: child, G and dF must be all set (internal round) or all null (leaves)");
+  RoundBwdGatesArgs a{dpool, pair, child, dret, gates, G, dxW, ld_dxw, dF, dpool, n, H};
+  hipStream_t st = as_stream(stream);
+  const bool vec = H % 4 == 0 && ld_dxw % 4 == 0 && aligned16(dpool) && aligned16(dret) && aligned16(gates) &&
+                   aligned16(dxW) && (!G || aligned16(G)) && (!dF || aligned16(dF));
+  if (vec) {
+    long total = (long)n * (H / 4);
+    treelstm_round_bwd_gates_kernel<4><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a);
+  } else {
+    long total = (long)n * H;
+    treelstm_round_bwd_gates_kernel<1><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a);
+  }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *dF, const float *UT,
+                                     const int *child, float *dpool, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && ld_dxw >= 4 * H && ld_dxw % 4 == 0,
+               "cavs_treelstm_round_bwd_children: bad shape n=%d H=%d ld=%d (H must be a multiple of 32)", n, H, ld_dxw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dxW && dF && UT && child && dpool, "cavs_treelstm_round_bwd_children: null pointer");
+  CAVS_REQUIRE(aligned16(dxW) && aligned16(dF), "cavs_treelstm_round_bwd_children: dxW and dF must be 16-byte aligned");
+  RoundBwdChildArgs a{dxW, ld_dxw, dF, UT, child, dpool, n, H};
+  const RoundPlan p = plan_round(n);
+  dim3 grid(H / p.tile, (n + p.tile * p.rt - 1) / (p.tile * p.rt));
+  hipStream_t st = as_stream(stream);
+  if (p.tile == 16 && p.rt == 1) treelstm_round_bwd_children_kernel<16, 1><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.tile == 16 && p.rt == 2) treelstm_round_bwd_children_kernel<16, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.tile == 16) treelstm_round_bwd_children_kernel<16, 4><<<grid, kRoundThreads, 0, st>>>(a);
+  else if (p.rt == 1) treelstm_round_bwd_children_kernel<32, 1><<<grid, kRoundThreads, 0, st>>>(a);
+  else treelstm_round_bwd_children_kernel<32, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream) {
+  CAVS_REQUIRE(rows >= 0 && cols >= 0, "cavs_transpose: bad shape %d x %d", rows, cols);
+  if (rows == 0 || cols == 0) return CAVS_OK;
+  CAVS_REQUIRE(out && in && out != in, "cavs_transpose: null or aliased pointer");
+  dim3 grid((cols + 31) / 32, (rows + 31) / 32);
+  transpose_kernel<<<grid, 256, 0, as_stream(stream)>>>(out, in, rows, cols);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // extern "C"

@@ -67,6 +67,10 @@ _SIGS = {
     "cavs_lstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treefc_fwd": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treefc_bwd": [_P, _P, _P, _P, _I, _I, _I, _P],
+    "cavs_treelstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
+    "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_fused_compile": [C.c_char_p, C.c_char_p, C.POINTER(_P)],
     "cavs_fused_launch": [_P, C.POINTER(_P), _I, C.POINTER(_P), _I, C.POINTER(_I), C.POINTER(_I), _I, _P],
     "cavs_fused_release": [_P],

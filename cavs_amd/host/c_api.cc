@@ -127,9 +127,9 @@ int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double 
   if (int rc = need(s, "session")) return rc;
   if (int rc = need(total_ms, "output")) return rc;
   if (int rc = need(launches, "output")) return rc;
-  static const char *names[] = {"gemm", "gather", "scatter", "gates", "other"};
+  static const char *names[] = {"gemm", "gather", "scatter", "gates", "other", "round"};
   int cls = -1;
-  for (int i = 0; i < 5; i++)
+  for (int i = 0; i < 6; i++)
     if (kernel_class && !std::strcmp(kernel_class, names[i])) cls = i;
   if (cls < 0) {
     g_error = "unknown kernel class";

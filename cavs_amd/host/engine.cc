@@ -241,6 +241,7 @@ void Engine::reserve_edges() {
     R(r_z_, rc * H);
   }
   if (cfg_.model == CAVS_MODEL_TREELSTM) {
+    if (fused_rows() > 0) R(UT_, (size_t)4 * H * H);
     R(hlr_, cap * H);
     R(dF_, cap * 2 * H);
     R(r_hU_, rc * 3 * H);
@@ -327,6 +328,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
                             "(graph_scheduler.cc:180) and leaves its rows undefined");
   N_ = sched_.N;
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
+  c_round_flops_ = 0;
   reserve_edges();
   upload_index_arena();
   parse_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -426,6 +428,14 @@ void Engine::pop_ret(float *graph_out) { scatter(graph_out, cfg_.H, d_t2j_, msg_
 // (Pull, EmbeddingLookup, x*W) is hoisted out of the round loop and done once for all N
 // vertices in tensor-id order; rounds of leaves skip the child GEMMs because their
 // gathered rows are zero.
+// The fused round kernels need the batch scheduler's rounds (every vertex of an internal
+// round has both children) and H in whole MFMA tiles.
+int Engine::fused_rows() const {
+  if (cfg_.model != CAVS_MODEL_TREELSTM || !(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.H % 32 != 0) return 0;
+  if (cfg_.fused_round_rows < 0) return 0;
+  return cfg_.fused_round_rows > 0 ? cfg_.fused_round_rows : 4096;
+}
+
 void Engine::treelstm_forward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w, *Bv = param("Bv").w;
@@ -437,12 +447,23 @@ void Engine::treelstm_forward() {
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
   }
+  const int fused = fused_rows();
   for (const Round &r : sched_.rounds) {
     const size_t off = r.offset;
     float *msg = msg_.at(off * 2 * H);
     if (leaf_round(r)) {
       CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, nullptr, nullptr, nullptr, Bv,
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
+    } else if (r.n <= fused) {
+      // Gather, both recurrent products, the gates and Scatter in one launch
+      CAVS_TIMED(K_ROUND, cavs_treelstm_round_fwd(pool_.get(), d_child_ + 2 * off, d_pair_ + off, xW_.at(off * 4 * H), 4 * H, U, Bv,
+                                                  G_.at(2 * off * 2 * H), hlr_.at(off * H), gates_.at(off * 6 * H), msg, r.n, H,
+                                                  stream_));
+      c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
+      c_gather_rows_ += 2.0 * r.n;
+      c_scatter_rows_ += r.n;
+      c_launches_ += 1;
+      continue;
     } else {
       float *G = G_.at(2 * off * 2 * H), *hlr = hlr_.at(off * H);
       {
@@ -467,9 +488,33 @@ void Engine::treelstm_backward() {
   const float *W = param("W").w, *U = param("U").w;
   gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);  // grad of Push is Pull
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
+  const int fused = fused_rows();
+  if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
+    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), U, H, 3 * H, stream_));
+    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.at((size_t)3 * H * H), U + (size_t)3 * H * H, H, H, stream_));
+    c_launches_ += 2;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
+    if (r.n <= fused) {
+      // Gather of the message gradient, gate gradients and the Scatter of d c_child in one
+      // launch; the children's d h (both products and their Scatter) in a second
+      const bool leaf = leaf_round(r);
+      const int *child = leaf ? nullptr : d_child_ + 2 * off;
+      float *dxW = dxW_.at(off * 4 * H), *dF = leaf ? nullptr : dF_.at(2 * off * H);
+      CAVS_TIMED(K_GATES, cavs_treelstm_round_bwd_gates(dpool_.get(), d_pair_ + off, child, dret_.at(off * H), gates_.at(off * 6 * H),
+                                                        leaf ? nullptr : G_.at(2 * off * 2 * H), dxW, 4 * H, dF, r.n, H, stream_));
+      c_gather_rows_ += r.n;
+      c_launches_ += 1;
+      if (!leaf) {
+        CAVS_TIMED(K_ROUND, cavs_treelstm_round_bwd_children(dxW, 4 * H, dF, UT_.get(), child, dpool_.get(), r.n, H, stream_));
+        c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
+        c_scatter_rows_ += 2.0 * r.n;
+        c_launches_ += 1;
+      }
+      continue;
+    }
     // grad of Scatter is Gather on the recorded scatter list; rows without an entry read zero
     gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
     if (leaf_round(r)) {
@@ -724,6 +769,7 @@ double Engine::counter(const std::string &key) const {
   if (key == "gather_bytes") return c_gather_bytes_;
   if (key == "scatter_bytes") return c_scatter_bytes_;
   if (key == "gemm_flops") return c_gemm_flops_;
+  if (key == "round_flops") return c_round_flops_;
   if (key == "launches") return c_launches_;
   if (key == "rounds") return (double)sched_.rounds.size();
   fail(CAVS_EINVAL, "unknown counter '" + key + "'");

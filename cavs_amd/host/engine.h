@@ -51,7 +51,7 @@ class Engine {
   double counter(const std::string &key) const;
   // Per-kernel-class device time: when enabled every launch is bracketed by a pair of
   // events on the session's stream; read() waits for the stream and sums them.
-  enum KernelClass { K_GEMM = 0, K_GATHER, K_SCATTER, K_GATES, K_OTHER, K_CLASSES };
+  enum KernelClass { K_GEMM = 0, K_GATHER, K_SCATTER, K_GATES, K_OTHER, K_ROUND, K_CLASSES };
   void profile_enable(bool on);
   void profile_read(int cls, double *total_ms, double *launches);
   const Schedule &schedule() const { return sched_; }
@@ -131,8 +131,12 @@ class Engine {
   DeviceArray<float> xs_, e_, xW_, G_, hlr_, gates_, msg_, pool_, GO_, dGO_, dret_, dpool_, dxW_,
       dF_, de_, logits_, dlogits_, loss_, ws_;
   DeviceArray<float> r_hU_, r_hUf_, r_dmsg_, r_dG_, r_dhlr_, r_z_;  // round-local
+  DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
+  // rounds of at most this many rows run as fused launches (0: none)
+  int fused_rows() const;
 
   // counters of the last step
+  double c_round_flops_ = 0;
   double c_gather_rows_ = 0, c_scatter_rows_ = 0, c_gemm_flops_ = 0, c_launches_ = 0,
          c_gather_bytes_ = 0, c_scatter_bytes_ = 0;
 };

@@ -205,6 +205,34 @@ int cavs_treefc_fwd(const float *z, const float *bias, const float *x, float *h,
 int cavs_treefc_bwd(const float *dh_m, const float *dret, const float *h, float *dz, int n,
                     int H, int act, void *stream);
 
+/* ------------------------------------------------------------------ fused rounds
+ * One round of the Tree-LSTM vertex function (apps/paper/tree-lstm-cavs.cc:129-172)
+ * with its graph operators folded in: Gather (op_impl_graphop.cu:50-110) becomes the
+ * operand fetch of the recurrent products, Scatter (op_impl_graphop.cu:128-190) the
+ * store of the epilogue.  Same operand layouts as the gate kernels above; H must be a
+ * multiple of 32.
+ *   pool [*,2H] message pool rows [h|c]; child [2n] pool rows of the children of slab
+ *   row b at 2b, 2b+1 (-1 = none, reads as zero); pair [n] pool row the message of slab
+ *   row b is written to (-1 = nowhere); U = U_iou [H,3H] then U_f [H,H].
+ * Writes msg [n,2H], pool rows pair[b], and what backward reads again: gates [n,6H],
+ * G [2n,2H] (gathered children), hlr [n,H] (h_l + h_r). */
+int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW,
+                            int ld_xw, const float *U, const float *bias, float *G, float *hlr,
+                            float *gates, float *msg, int n, int H, void *stream);
+/* Backward of the gates of a round.  The message gradient of slab row b is read from
+ * dpool row pair[b] (grad of Scatter is Gather on the same list, zero for -1); the c
+ * half of the children's message gradients is written to dpool rows child[2b], child[2b+1]
+ * (grad of Gather is Scatter).  child, G and dF are all NULL for a round of leaves. */
+int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret,
+                                  const float *gates, const float *G, float *dxW, int ld_dxw,
+                                  float *dF, int n, int H, void *stream);
+/* The h half: dh_child = [d_i|d_o|d_u] * U_iou^T + d_f(child) * U_f^T written to dpool rows
+ * child[2b], child[2b+1].  UT = U_iou^T [3H,H] then U_f^T [H,H] (cavs_transpose). */
+int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *dF, const float *UT,
+                                     const int *child, float *dpool, int n, int H, void *stream);
+/* out [cols,rows] = in [rows,cols]^T */
+int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream);
+
 /* ------------------------------------------------------------------ generic fused op
  * FusedKernelOpImpl (cavs/backend/op_impl_fused_kernel.cu:17-71): compiles the
  * source the fusion pass generated (runtime_compiler/code_generator.cc:20-100;

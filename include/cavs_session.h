@@ -44,6 +44,10 @@ typedef struct {
   int use_bias;       /* Tree-FC */
   int use_x;          /* Tree-FC: add the Pull'ed [H] input row */
   int device;
+  /* Tree-LSTM: rounds of at most this many vertices run as one fused launch forward and
+   * two backward (cavs_treelstm_round_*); larger rounds run gather / GEMM / gates / scatter
+   * as separate launches.  0 = default limit, negative = never fuse. */
+  int fused_round_rows;
 } cavs_session_config;
 
 const char *cavs_session_error(void);
@@ -87,14 +91,15 @@ int cavs_session_timing(cavs_session *s, const char *name, float *ms);
 /* Device time per kernel class.  While enabled, every launch of the session is
  * bracketed by a pair of events on the session's stream; profile_read waits for the
  * stream and returns the summed elapsed time and launch count since profiling was
- * enabled.  Classes: "gemm" "gather" "scatter" "gates". */
+ * enabled.  Classes: "gemm" "gather" "scatter" "gates" "round" (fused rounds) "other". */
 int cavs_session_profile(cavs_session *s, int enable);
 int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double *total_ms,
                               double *launches);
 /* Raw stream the session enqueues on (for callers that want to bracket it with events). */
 void *cavs_session_stream(cavs_session *s);
 /* Per-step counts for roofline accounting: rows moved by indexed copies and GEMM flops
- * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" "rounds" "launches". */
+ * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" (separate GEMM launches)
+ * "round_flops" (products inside fused round launches) "rounds" "launches". */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);
 
 #ifdef __cplusplus

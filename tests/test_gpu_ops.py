@@ -479,3 +479,88 @@ def test_reference_elementwise_smoke_values(g):
     out = g.zeros(6)
     g.call("cavs_ew_binary", hip.EW_BINARY["add"], g.P(out), g.P(g.devf(a)), 6, g.P(g.devf(b)), 6, 6, 0, g.stream())
     np.testing.assert_array_equal(g.host(out), np.array(kat["expect"], np.float32))
+
+
+@pytest.mark.parametrize("n,H", [(1, 32), (16, 64), (17, 32), (33, 96), (64, 64), (65, 32), (130, 64), (600, 64), (300, 512)])
+def test_fused_tree_lstm_rounds(g, oracle, n, H):
+    """A whole round in one launch (forward) / two (backward) against the same round
+    composed from the oracle's gather, GEMM and gate functions."""
+    r = rng(7 * n + H)
+    P_rows = 2 * n + 5                      # pool: children rows, then this round's rows
+    pool = (r.bulk_normal((P_rows + n) * 2 * H).reshape(P_rows + n, 2 * H) * 0.5).astype(np.float32)
+    perm = np.argsort(r.bulk_normal(P_rows))[: 2 * n].astype(np.int32)
+    child = perm.copy()
+    pair = (P_rows + np.arange(n)).astype(np.int32)
+    if n > 2:
+        child[3] = -1                       # a missing child reads as zero
+        pair[n - 1] = -1                    # a root: its message goes nowhere
+    xW = r.bulk_normal(n * 4 * H).reshape(n, 4 * H)
+    U = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)
+    Uiou, Uf = U[: 3 * H * H].reshape(H, 3 * H), U[3 * H * H:].reshape(H, H)
+    bias = r.bulk_normal(4 * H)
+    # expected, from the oracle's pieces
+    def gather0(src, ids):  # the oracle's gather with "-1 reads as zero" of the C ABI on top
+        out = oracle.gather_rows(src, np.maximum(ids, 0))
+        out[ids < 0] = 0
+        return out
+
+    G_w = gather0(pool, child)                                              # [2n, 2H]
+    hlr_w = (G_w[0::2, :H] + G_w[1::2, :H]).astype(np.float32)
+    hU_w = oracle.sgemm(0, 0, hlr_w, Uiou)
+    hUf_w = oracle.sgemm(0, 0, np.ascontiguousarray(G_w[:, :H]), Uf)
+    gates_w, msg_w = oracle.treelstm_gates_fwd(xW, hU_w, hUf_w, G_w, bias)
+    pool_w = pool.copy()
+    pool_w[pair[pair >= 0]] = msg_w[pair >= 0]
+
+    d_pool, d_child, d_pair = g.devf(pool), g.devi(child), g.devi(pair)
+    G, hlr, gates, msg = g.zeros(2 * n, 2 * H), g.zeros(n, H), g.zeros(n, 6 * H), g.zeros(n, 2 * H)
+    g.call("cavs_treelstm_round_fwd", g.P(d_pool), g.P(d_child), g.P(d_pair), g.P(g.devf(xW)), 4 * H, g.P(g.devf(U)),
+           g.P(g.devf(bias)), g.P(G), g.P(hlr), g.P(gates), g.P(msg), n, H, g.stream())
+    np.testing.assert_array_equal(g.host(G), G_w)
+    np.testing.assert_array_equal(g.host(hlr), hlr_w)
+    close(g.host(gates), gates_w, "gates")
+    close(g.host(msg), msg_w, "msg")
+    close(g.host(d_pool), pool_w, "pool")
+
+    # backward: message gradients of this round sit in dpool rows pair[b]
+    dpool = r.bulk_normal((P_rows + n) * 2 * H).reshape(P_rows + n, 2 * H)
+    dret = r.bulk_normal(n * H).reshape(n, H)
+    dmsg_w = gather0(dpool, pair)
+    dxW_w, dF_w, dG_w = oracle.treelstm_gates_bwd(dmsg_w, dret, gates_w, G_w)
+    dhlr_w = oracle.sgemm(0, 1, np.ascontiguousarray(dxW_w[:, : 3 * H]), np.ascontiguousarray(Uiou))
+    dGh_w = oracle.sgemm(0, 1, dF_w, np.ascontiguousarray(Uf)) + np.repeat(dhlr_w, 2, axis=0)
+    dG_w[:, :H] = dGh_w
+    dpool_w = dpool.copy()
+    dpool_w[child[child >= 0]] = dG_w[child >= 0]
+
+    UT = g.zeros(4 * H * H)
+    d_U = g.devf(U)
+    g.call("cavs_transpose", g.P(UT), g.P(d_U), H, 3 * H, g.stream())
+    g.call("cavs_transpose", g.P(UT) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, H, H, g.stream())
+    np.testing.assert_array_equal(g.host(UT)[: 3 * H * H].reshape(3 * H, H), Uiou.T)
+    np.testing.assert_array_equal(g.host(UT)[3 * H * H:].reshape(H, H), Uf.T)
+    d_dpool, dxW, dF = g.devf(dpool), g.zeros(n, 4 * H), g.zeros(2 * n, H)
+    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool), g.P(d_pair), g.P(d_child), g.P(g.devf(dret)), g.P(g.devf(gates_w)),
+           g.P(g.devf(G_w)), g.P(dxW), 4 * H, g.P(dF), n, H, g.stream())
+    g.call("cavs_treelstm_round_bwd_children", g.P(dxW), 4 * H, g.P(dF), g.P(UT), g.P(d_child), g.P(d_dpool), n, H, g.stream())
+    close(g.host(dxW), dxW_w, "dxW")
+    close(g.host(dF), dF_w, "dF")
+    close(g.host(d_dpool), dpool_w, "dpool", rtol=2e-4, atol=2e-5)
+
+    # a round of leaves: no children, nothing scattered downwards
+    gates_l, _ = oracle.treelstm_gates_fwd(xW, 0 * hU_w, 0 * hUf_w, 0 * G_w, bias)
+    dxW_l, _, _ = oracle.treelstm_gates_bwd(dmsg_w, dret, gates_l, 0 * G_w)
+    d_dpool2 = g.devf(dpool)
+    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool2), g.P(d_pair), None, g.P(g.devf(dret)), g.P(g.devf(gates_l)),
+           None, g.P(dxW), 4 * H, None, n, H, g.stream())
+    close(g.host(dxW), dxW_l, "leaf dxW")
+    np.testing.assert_array_equal(g.host(d_dpool2), dpool)
+
+
+def test_fused_round_entry_points_reject_bad_shapes():
+    with pytest.raises(hip.CavsError, match="multiple of 32"):
+        hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 5, 24, 0)
+    with pytest.raises(hip.CavsError, match="multiple of 32"):
+        hip.call("cavs_treelstm_round_bwd_children", 0, 4 * 24, 0, 0, 0, 0, 5, 24, 0)
+    with pytest.raises(hip.CavsError, match="all set"):
+        hip.call("cavs_treelstm_round_bwd_gates", 16, 16, 16, 16, 16, 0, 16, 4 * 32, 0, 5, 32, 0)
