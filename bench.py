@@ -121,19 +121,32 @@ def main():
     # session bracketed by HIP events on the session's own stream (the bracketing costs a
     # little launch throughput, so it is kept out of the throughput figure above).
     s.profile(True)
-    flops = rows = gbytes = sbytes = 0.0
+    flops = rflops = gbytes = sbytes = 0.0
     for i in range(a.warmup, a.warmup + a.steps):
         g, x, lab = feeds[i % len(feeds)]
         s.step(g, x, lab, backward=True, lr=a.lr)
         flops += s.counter("gemm_flops")
+        rflops += s.counter("round_flops")
         gbytes += s.counter("gather_bytes")
         sbytes += s.counter("scatter_bytes")
     gemm_ms, gemm_n = s.profile_read("gemm")
     gat_ms, gat_n = s.profile_read("gather")
     sca_ms, sca_n = s.profile_read("scatter")
     gates_ms, gates_n = s.profile_read("gates")
+    round_ms, round_n = s.profile_read("round")
+    other_ms, other_n = s.profile_read("other")
     s.profile(False)
-    achieved_tf = flops / (gemm_ms * 1e-3) / 1e12 if gemm_ms else 0.0
+    # the two MFMA-bound kernel classes; the roofline entry describes whichever takes more device time
+    mfma = {
+        "gemm": dict(ms=gemm_ms, n=gemm_n, flops=flops,
+                     kernel="sgemm_mfma_kernel / sgemm_skinny_kernel (x*W, weight-gradient and head GEMMs of a step)"),
+        "round": dict(ms=round_ms, n=round_n, flops=rflops,
+                      kernel="treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel (one launch per round: "
+                             "gather + recurrent products + gates + scatter)"),
+    }
+    for v in mfma.values():
+        v["tf"] = v["flops"] / (v["ms"] * 1e-3) / 1e12 if v["ms"] else 0.0
+    dom = max(mfma.values(), key=lambda v: v["ms"])
     rounds = s.counter("rounds")
     launches = s.counter("launches")
 
@@ -146,19 +159,23 @@ def main():
                                f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing, "rounds_last_batch": rounds,
                    "launches_last_batch": launches},
-        "roofline": {"bound": "mfma", "achieved": round(achieved_tf, 3), "peak": FP32_MFMA_PEAK_TF,
-                     "unit": "TFLOP/s", "frac": round(achieved_tf / FP32_MFMA_PEAK_TF, 5), "traffic": None,
-                     "kernel": "sgemm_mfma_kernel (all gate / weight-gradient / head GEMMs of a step)",
-                     "avg_launch_us": round(1e3 * gemm_ms / gemm_n, 3) if gemm_n else None,
-                     "flops_per_launch": round(flops / gemm_n, 1) if gemm_n else None},
+        "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
+                     "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": None,
+                     "kernel": dom["kernel"],
+                     "avg_launch_us": round(1e3 * dom["ms"] / dom["n"], 3) if dom["n"] else None,
+                     "flops_per_launch": round(dom["flops"] / dom["n"], 1) if dom["n"] else None},
         "kernels": {
+            **{k: {"bound": "mfma", "achieved": round(v["tf"], 3), "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
+                   "avg_launch_us": round(1e3 * v["ms"] / max(v["n"], 1), 3), "launches_per_step": round(v["n"] / a.steps, 1)}
+               for k, v in mfma.items()},
             "gather": {"bound": "hbm", "achieved": round(gbytes / (gat_ms * 1e-3) / 1e9, 2) if gat_ms else None,
                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * gat_ms / max(gat_n, 1), 3)},
             "scatter": {"bound": "hbm", "achieved": round(sbytes / (sca_ms * 1e-3) / 1e9, 2) if sca_ms else None,
                         "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * sca_ms / max(sca_n, 1), 3)},
             "gates": {"avg_launch_us": round(1e3 * gates_ms / max(gates_n, 1), 3)},
-            "device_ms_per_step": {"gemm": round(gemm_ms / a.steps, 4), "gather": round(gat_ms / a.steps, 4),
-                                   "scatter": round(sca_ms / a.steps, 4), "gates": round(gates_ms / a.steps, 4)},
+            "device_ms_per_step": {"gemm": round(gemm_ms / a.steps, 4), "round": round(round_ms / a.steps, 4),
+                                   "gather": round(gat_ms / a.steps, 4), "scatter": round(sca_ms / a.steps, 4),
+                                   "gates": round(gates_ms / a.steps, 4), "other": round(other_ms / a.steps, 4)},
         },
         "timers_ms": {"GraphParsing": round(s.timing("GraphParsing"), 4), "RNNForward": round(s.timing("RNNForward"), 4),
                       "RNNBackward": round(s.timing("RNNBackward"), 4)},

@@ -53,27 +53,37 @@ __device__ inline float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 __device__ inline float elem(const float4 &v, int c) { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
 __device__ inline float sigm_r(float x) { return 1.f / (1.f + expf(-x)); }
 
-constexpr int kRoundThreads = 512;
-constexpr int kRoundWaves = kRoundThreads / 64;
 
-// Sums the per-wavefront partial tiles of NP products into `red` in k-split order and
-// leaves them laid out as [row tile][product][accumulator element][lane].
-template <int TILE, int NP, int KS>
-__device__ inline void reduce_partials(float *red, const typename Mma<TILE>::Acc (&acc)[NP], int rt, int ks, int lane) {
+// Parks the per-wavefront partial tiles of NP products in LDS as
+// [region][row tile][product][accumulator element][lane].  There are NREG regions: the
+// wavefronts with k-split index below NREG write theirs, the others add onto region
+// ks % NREG in a second, third ... step, so that the reader only has to sum NREG values
+// per element, always in the same order (deterministic).
+template <int TILE, int NP, int KS, int NREG, int RT>
+__device__ inline void park_partials(float *red, const typename Mma<TILE>::Acc (&acc)[NP], int rt, int ks, int lane) {
   constexpr int NR = Mma<TILE>::NR;
-  for (int w = 0; w < KS; w++) {
-    if (ks == w) {
+  static_assert(KS % NREG == 0, "k-splits must fill whole steps");
+  for (int step = 0; step < KS / NREG; step++) {
+    if (ks / NREG == step) {
+      float *base = red + (ks % NREG) * (RT * NP * NR * 64);
 #pragma unroll
       for (int p = 0; p < NP; p++)
 #pragma unroll
         for (int r = 0; r < NR; r++) {
-          float *q = red + ((rt * NP + p) * NR + r) * 64 + lane;
-          *q = (w == 0) ? acc[p][r] : *q + acc[p][r];
+          float *q = base + ((rt * NP + p) * NR + r) * 64 + lane;
+          *q = (step == 0) ? acc[p][r] : *q + acc[p][r];
         }
     }
     __syncthreads();
   }
 }
+
+// regions for a tile shape: all eight for the small tile (40 KB for five products), four for
+// the large one (80 KB)
+template <int TILE, int KS>
+struct Regions {
+  static constexpr int N = TILE == 16 ? KS : (KS >= 4 ? 4 : KS);
+};
 
 // ------------------------------------------------------------------ forward
 struct RoundFwdArgs {
@@ -92,13 +102,15 @@ struct RoundFwdArgs {
   int n, H;
 };
 
-template <int TILE, int RT>
-__global__ __launch_bounds__(kRoundThreads) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
+template <int TILE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
-  constexpr int KS = kRoundWaves / RT, GK = 4 * M::NSLOT, NP = 5, NR = M::NR;
+  constexpr int RT = 1, kRoundThreads = WAVES * 64;
+  constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 5, NR = M::NR;
   constexpr int UG = 2;  // k-groups per pipeline stage
-  __shared__ float red[RT * NP * NR * 64];
+  constexpr int NREG = Regions<TILE, KS>::N, RSZ = RT * NP * NR * 64;
+  __shared__ float red[NREG * RSZ];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rt = wave / KS, ks = wave % KS;
@@ -116,6 +128,35 @@ __global__ __launch_bounds__(kRoundThreads) void treelstm_round_fwd_kernel(Round
   const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
   const int kb = ks * kper, ke = min(H, kb + kper);
   const float *Uio = a.U + j0 + x, *Uf = a.U + H3 * H + j0 + x;
+
+  // operands of the epilogue, fetched now so that their latency hides behind the products
+  constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
+  struct Epi {
+    bool on;
+    int b, j, dst, lds;
+    float xw[4], bias[4], hl, cl, hr, cr;
+  } epi[EPT];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    Epi &ep = epi[q];
+    const int e = tid + q * kRoundThreads;
+    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
+    ep.b = (blockIdx.y * RT + t) * TILE + M::row(r, l2);
+    ep.j = j0 + (l2 & (TILE - 1));
+    ep.lds = (t * NP * NR + r) * 64 + l2;
+    ep.on = e < RT * NR * 64 && ep.b < a.n;
+    ep.hl = ep.cl = ep.hr = ep.cr = 0.f;
+    ep.dst = -1;
+    if (ep.on) {
+      const int c_l = a.child[2 * ep.b], c_r = a.child[2 * ep.b + 1];
+      ep.dst = a.pair[ep.b];
+      if (c_l >= 0) { ep.hl = a.pool[c_l * H2 + ep.j]; ep.cl = a.pool[c_l * H2 + H + ep.j]; }
+      if (c_r >= 0) { ep.hr = a.pool[c_r * H2 + ep.j]; ep.cr = a.pool[c_r * H2 + H + ep.j]; }
+      const float *xw = a.xW + ep.b * a.ld_xw + ep.j;
+#pragma unroll
+      for (int k = 0; k < 4; k++) { ep.xw[k] = xw[k * H]; ep.bias[k] = a.bias[k * H + ep.j]; }
+    }
+  }
 
   Acc acc[NP];
 #pragma unroll
@@ -169,42 +210,44 @@ __global__ __launch_bounds__(kRoundThreads) void treelstm_round_fwd_kernel(Round
     }
   }
 
-  reduce_partials<TILE, NP, KS>(red, acc, rt, ks, lane);
+  park_partials<TILE, NP, KS, NREG, RT>(red, acc, rt, ks, lane);
 
-  // epilogue: element (t, r, l2) of the workgroup's tiles is slab row b, column j
-  const float *bias = a.bias;
-  for (int e = tid; e < RT * NR * 64; e += kRoundThreads) {
-    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
-    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2), j = j0 + (l2 & (TILE - 1));
-    if (b >= a.n) continue;
-    const float *pre = red + (t * NP * NR + r) * 64 + l2;
-    const float hi = pre[0], ho = pre[NR * 64], hu = pre[2 * NR * 64], fl = pre[3 * NR * 64], fr = pre[4 * NR * 64];
-    const int c_l = a.child[2 * b], c_r = a.child[2 * b + 1];
-    float hl = 0.f, cl_ = 0.f, hr = 0.f, cr_ = 0.f;
-    if (c_l >= 0) { hl = a.pool[c_l * H2 + j]; cl_ = a.pool[c_l * H2 + H + j]; }
-    if (c_r >= 0) { hr = a.pool[c_r * H2 + j]; cr_ = a.pool[c_r * H2 + H + j]; }
-    const float *xw = a.xW + b * a.ld_xw + j;
+  // epilogue: element (t, r, l2) of the workgroup's tiles is slab row b, column j; its
+  // operands were fetched before the products started
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    const Epi &ep = epi[q];
+    if (!ep.on) continue;
+    const float *pre = red + ep.lds;
+    float v[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      float s = pre[p * NR * 64];
+#pragma unroll
+      for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+      v[p] = s;
+    }
+    const int b = ep.b, j = ep.j;
     // same association as the separate gate kernel: (x*W + h*U) + bias
-    const float i = sigm_r((xw[0] + hi) + bias[j]);
-    const float o = sigm_r((xw[H] + ho) + bias[3 * H + j]);
-    const float u = tanhf((xw[2 * H] + hu) + bias[2 * H + j]);
-    const float f_l = sigm_r((xw[3 * H] + fl) + bias[H + j]);
-    const float f_r = sigm_r((xw[3 * H] + fr) + bias[H + j]);
-    const float c = (i * u + f_l * cl_) + f_r * cr_;
+    const float i = sigm_r((ep.xw[0] + v[0]) + ep.bias[0]);
+    const float o = sigm_r((ep.xw[1] + v[1]) + ep.bias[3]);
+    const float u = tanhf((ep.xw[2] + v[2]) + ep.bias[2]);
+    const float f_l = sigm_r((ep.xw[3] + v[3]) + ep.bias[1]);
+    const float f_r = sigm_r((ep.xw[3] + v[4]) + ep.bias[1]);
+    const float c = (i * u + f_l * ep.cl) + f_r * ep.cr;
     const float tc = tanhf(c);
     const float h = o * tc;
     float *g = a.gates + (long)b * 6 * H + j;
     g[0] = i; g[H] = o; g[2 * H] = u; g[3 * H] = f_l; g[4 * H] = f_r; g[5 * H] = tc;
     float *m = a.msg + b * H2 + j;
     m[0] = h; m[H] = c;
-    const int dst = a.pair[b];
-    if (dst >= 0) {
-      a.pool_out[dst * H2 + j] = h;
-      a.pool_out[dst * H2 + H + j] = c;
+    if (ep.dst >= 0) {
+      a.pool_out[ep.dst * H2 + j] = h;
+      a.pool_out[ep.dst * H2 + H + j] = c;
     }
     float *gl = a.G + (2L * b) * H2 + j, *gr = gl + H2;
-    gl[0] = hl; gl[H] = cl_; gr[0] = hr; gr[H] = cr_;
-    a.hlr[(long)b * H + j] = hl + hr;
+    gl[0] = ep.hl; gl[H] = ep.cl; gr[0] = ep.hr; gr[H] = ep.cr;
+    a.hlr[(long)b * H + j] = ep.hl + ep.hr;
   }
 }
 
@@ -304,13 +347,15 @@ struct RoundBwdChildArgs {
   int n, H;
 };
 
-template <int TILE, int RT>
-__global__ __launch_bounds__(kRoundThreads) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
+template <int TILE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
-  constexpr int KS = kRoundWaves / RT, GK = 4 * M::NSLOT, NP = 3, NR = M::NR;
+  constexpr int RT = 1, kRoundThreads = WAVES * 64;
+  constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 3, NR = M::NR;
   constexpr int UG = 2;
-  __shared__ float red[RT * NP * NR * 64];
+  constexpr int NREG = Regions<TILE, KS>::N, RSZ = RT * NP * NR * 64;
+  __shared__ float red[NREG * RSZ];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rt = wave / KS, ks = wave % KS;
@@ -406,17 +451,24 @@ __global__ __launch_bounds__(kRoundThreads) void treelstm_round_bwd_children_ker
     }
   }
 
-  reduce_partials<TILE, NP, KS>(red, acc, rt, ks, lane);
+  park_partials<TILE, NP, KS, NREG, RT>(red, acc, rt, ks, lane);
 
   for (int e = tid; e < RT * NR * 64; e += kRoundThreads) {
     const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
     const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2), j = j0 + (l2 & (TILE - 1));
     if (b >= a.n) continue;
     const float *pre = red + (t * NP * NR + r) * 64 + l2;
-    const float p0 = pre[0], p1 = pre[NR * 64], p2 = pre[2 * NR * 64];
+    float v[NP];
+#pragma unroll
+    for (int p = 0; p < NP; p++) {
+      float s = pre[p * NR * 64];
+#pragma unroll
+      for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+      v[p] = s;
+    }
     const int c_l = a.child[2 * b], c_r = a.child[2 * b + 1];
-    if (c_l >= 0) a.dpool[c_l * H2 + j] = p0 + p1;
-    if (c_r >= 0) a.dpool[c_r * H2 + j] = p0 + p2;
+    if (c_l >= 0) a.dpool[c_l * H2 + j] = v[0] + v[1];
+    if (c_r >= 0) a.dpool[c_r * H2 + j] = v[0] + v[2];
   }
 }
 
@@ -434,15 +486,17 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
 
 static bool round_shape_ok(int H) { return H > 0 && H % 32 == 0; }
 
-// tile shape and row tiles per workgroup for a round of n rows
+// tile shape and wavefronts per workgroup for a round of n rows
 struct RoundPlan {
-  int tile, rt;
+  int tile, waves;
 };
+// Measured on MI355X at H=512: the 16x16 tile wins while a round is too small to give every
+// CU a 32x32 tile (its workgroups finish in 8 us against 20), eight wavefronts per workgroup
+// up to 64 rows, four beyond (several workgroups then share a CU and overlap their latencies).
 static RoundPlan plan_round(int n) {
-  if (n <= 16) return {16, 1};
-  if (n <= 32) return {16, 2};
-  if (n <= 64) return {16, 4};
-  return {32, n > 512 ? 2 : 1};
+  if (n <= 64) return {16, 8};
+  if (n <= 200) return {16, 4};
+  return {32, 8};
 }
 
 }  // namespace cavs
@@ -461,13 +515,12 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
   RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, n, H};
   const RoundPlan p = plan_round(n);
-  dim3 grid(H / p.tile, (n + p.tile * p.rt - 1) / (p.tile * p.rt));
+  dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.rt == 1) treelstm_round_fwd_kernel<16, 1><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.tile == 16 && p.rt == 2) treelstm_round_fwd_kernel<16, 2><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.tile == 16) treelstm_round_fwd_kernel<16, 4><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.rt == 1) treelstm_round_fwd_kernel<32, 1><<<grid, kRoundThreads, 0, st>>>(a);
-  else treelstm_round_fwd_kernel<32, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  if (p.tile == 16 && p.waves == 4) treelstm_round_fwd_kernel<16, 4><<<grid, 256, 0, st>>>(a);
+  else if (p.tile == 16) treelstm_round_fwd_kernel<16, 8><<<grid, 512, 0, st>>>(a);
+  else if (p.waves == 4) treelstm_round_fwd_kernel<32, 4><<<grid, 256, 0, st>>>(a);
+  else treelstm_round_fwd_kernel<32, 8><<<grid, 512, 0, st>>>(a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -504,13 +557,12 @@ int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *
   CAVS_REQUIRE(aligned16(dxW) && aligned16(dF), "cavs_treelstm_round_bwd_children: dxW and dF must be 16-byte aligned");
   RoundBwdChildArgs a{dxW, ld_dxw, dF, UT, child, dpool, n, H};
   const RoundPlan p = plan_round(n);
-  dim3 grid(H / p.tile, (n + p.tile * p.rt - 1) / (p.tile * p.rt));
+  dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.rt == 1) treelstm_round_bwd_children_kernel<16, 1><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.tile == 16 && p.rt == 2) treelstm_round_bwd_children_kernel<16, 2><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.tile == 16) treelstm_round_bwd_children_kernel<16, 4><<<grid, kRoundThreads, 0, st>>>(a);
-  else if (p.rt == 1) treelstm_round_bwd_children_kernel<32, 1><<<grid, kRoundThreads, 0, st>>>(a);
-  else treelstm_round_bwd_children_kernel<32, 2><<<grid, kRoundThreads, 0, st>>>(a);
+  if (p.tile == 16 && p.waves == 4) treelstm_round_bwd_children_kernel<16, 4><<<grid, 256, 0, st>>>(a);
+  else if (p.tile == 16) treelstm_round_bwd_children_kernel<16, 8><<<grid, 512, 0, st>>>(a);
+  else if (p.waves == 4) treelstm_round_bwd_children_kernel<32, 4><<<grid, 256, 0, st>>>(a);
+  else treelstm_round_bwd_children_kernel<32, 8><<<grid, 512, 0, st>>>(a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel roofline measurements through the C ABI (no model around the kernels).
 
-    python -m cavs_amd.kernel_bench [--set copies|gemm|gates|all] [--iters 50]
+    python -m cavs_amd.kernel_bench [--set copies|gemm|gates|rounds|all] [--iters 50]
 
 For each case: launches the entry point `iters` times back to back on one stream between two
 HIP events and reports the average duration per launch, the algorithmic bytes / flops
@@ -128,9 +128,58 @@ def gates(iters, st):
         _emit("treelstm_gates_bwd", f"{tag}: n={n} H={H}", us, nbytes=4 * n * H * 19)
 
 
+def rounds(iters, st):
+    """One Tree-LSTM round as fused launches, beside the same round as separate launches."""
+    f32 = dict(dtype=torch.float32, device="cuda")
+    for n, H, tag in [(4, 512, "C3 tail"), (16, 512, "C3 tail"), (32, 512, "C3 tail"), (64, 512, "C3 tail"),
+                      (150, 512, "C3 mid"), (300, 512, "C3 mid"), (600, 512, "C3 mid"), (1200, 512, "2x C3"),
+                      (2400, 512, "4x C3"), (2048, 1024, "C5 small round")]:
+        rows = 3 * n
+        pool = torch.randn(rows, 2 * H, **f32) * 0.5
+        g = torch.Generator(device="cpu").manual_seed(n)
+        child = torch.randperm(2 * n, generator=g).to(torch.int32).cuda()
+        pair = (2 * n + torch.arange(n)).to(torch.int32).cuda()
+        xW, bias = torch.randn(n, 4 * H, **f32), torch.randn(4 * H, **f32)
+        U = torch.randn(4 * H * H, **f32) / H ** 0.5
+        G, hlr = torch.empty(2 * n, 2 * H, **f32), torch.empty(n, H, **f32)
+        gt, msg = torch.empty(n, 6 * H, **f32), torch.empty(n, 2 * H, **f32)
+        flops = 2.0 * n * H * 5 * H
+        us = _time(lambda: hip.call("cavs_treelstm_round_fwd", pool.data_ptr(), child.data_ptr(), pair.data_ptr(),
+                                    xW.data_ptr(), 4 * H, U.data_ptr(), bias.data_ptr(), G.data_ptr(), hlr.data_ptr(),
+                                    gt.data_ptr(), msg.data_ptr(), n, H, st), iters, st)
+        _emit("treelstm_round_fwd", f"{tag}: n={n} H={H}", us, flops=flops)
+        hU, hUf = torch.empty(n, 3 * H, **f32), torch.empty(2 * n, H, **f32)
+
+        def separate_fwd():
+            hip.call("cavs_gather_children", G.data_ptr(), hlr.data_ptr(), pool.data_ptr(), child.data_ptr(), n, 2 * H, H, st)
+            hip.call("cavs_sgemm", 0, 0, n, 3 * H, H, 1.0, hlr.data_ptr(), H, U.data_ptr(), 3 * H, 0.0, hU.data_ptr(), 3 * H, st)
+            hip.call("cavs_sgemm", 0, 0, 2 * n, H, H, 1.0, G.data_ptr(), 2 * H, U.data_ptr() + 4 * 3 * H * H, H, 0.0,
+                     hUf.data_ptr(), H, st)
+            hip.call("cavs_treelstm_gates_fwd", xW.data_ptr(), 4 * H, hU.data_ptr(), hUf.data_ptr(), G.data_ptr(),
+                     bias.data_ptr(), gt.data_ptr(), msg.data_ptr(), n, H, st)
+            hip.call("cavs_scatter_rows", pool.data_ptr(), 2 * H, pair.data_ptr(), msg.data_ptr(), 2 * H, n, 2 * H, st)
+
+        us = _time(separate_fwd, iters, st)
+        _emit("round fwd as 5 launches", f"{tag}: n={n} H={H}", us, flops=flops)
+        UT = torch.empty(4 * H * H, **f32)
+        hip.call("cavs_transpose", UT.data_ptr(), U.data_ptr(), H, 3 * H, st)
+        hip.call("cavs_transpose", UT.data_ptr() + 4 * 3 * H * H, U.data_ptr() + 4 * 3 * H * H, H, H, st)
+        dpool, dret = torch.randn(rows, 2 * H, **f32), torch.randn(n, H, **f32)
+        dxW, dF = torch.empty(n, 4 * H, **f32), torch.empty(2 * n, H, **f32)
+        us = _time(lambda: hip.call("cavs_treelstm_round_bwd_gates", dpool.data_ptr(), pair.data_ptr(), child.data_ptr(),
+                                    dret.data_ptr(), gt.data_ptr(), G.data_ptr(), dxW.data_ptr(), 4 * H, dF.data_ptr(),
+                                    n, H, st), iters, st)
+        # reads dmsg 2H, dret H, gates 6H, c_l c_r 2H; writes dxW 4H, dF 2H, dc_l dc_r 2H
+        _emit("treelstm_round_bwd_gates", f"{tag}: n={n} H={H}", us, nbytes=4 * n * H * 19)
+        us = _time(lambda: hip.call("cavs_treelstm_round_bwd_children", dxW.data_ptr(), 4 * H, dF.data_ptr(), UT.data_ptr(),
+                                    child.data_ptr(), dpool.data_ptr(), n, H, st), iters, st)
+        _emit("treelstm_round_bwd_children", f"{tag}: n={n} H={H}", us, flops=flops)
+        del pool, xW, U, G, hlr, gt, msg, hU, hUf, UT, dpool, dret, dxW, dF
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", default="all", choices=["copies", "gemm", "gates", "all"])
+    ap.add_argument("--set", default="all", choices=["copies", "gemm", "gates", "rounds", "all"])
     ap.add_argument("--iters", type=int, default=50)
     a = ap.parse_args()
     assert torch.cuda.is_available(), "kernel_bench needs the MI355X"
@@ -142,6 +191,8 @@ def main():
         gemm(a.iters, st)
     if a.set in ("gates", "all"):
         gates(a.iters, st)
+    if a.set in ("rounds", "all"):
+        rounds(a.iters, st)
 
 
 if __name__ == "__main__":
