@@ -329,7 +329,8 @@ static GemmPlan plan_gemm(int tA, int tB, int M, int N, int K, bool skinny_allow
   const long t64 = (long)((M + 63) / 64) * ((N + 63) / 64);
   p.splits = 1;
   p.kchunk = K > 0 ? K : 1;
-  if (t128 >= cus) {
+  // the large tile needs at least two rounds of workgroups to hide its ragged last round
+  if (t128 >= 2 * cus) {
     p.kind = GemmPlan::TILE128;
     p.tiles = t128;
     return p;
@@ -337,7 +338,9 @@ static GemmPlan plan_gemm(int tA, int tB, int M, int N, int K, bool skinny_allow
   p.kind = GemmPlan::TILE64;
   p.tiles = t64;
   if (t64 >= 2 * cus || K < 64) return p;
-  if (skinny_allowed) {
+  // the skinny kernel reads a k-contiguous B (NT) sixteen bytes per lane and row, which only
+  // pays for a handful of rows; with B row-major (NN) it holds up to about a thousand
+  if (skinny_allowed && M <= (tB ? 128 : 1024)) {
     p.kind = GemmPlan::SKINNY;
     return p;
   }

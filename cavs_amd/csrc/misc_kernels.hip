@@ -71,12 +71,34 @@ __global__ void embed_fwd_kernel(float *__restrict__ out, long ld_out, const flo
   }
 }
 
+// Scatter-add of dy rows into the table.  A workgroup takes kEmbedChunk consecutive rows and
+// first adds up the ones that share an id (parse trees look up one and the same row for every
+// internal vertex), so a hot row receives one atomic add per chunk instead of one per vertex.
+constexpr int kEmbedChunk = 16;
 __global__ void embed_bwd_kernel(float *__restrict__ dtable, const float *__restrict__ ids,
                                  const float *__restrict__ dy, long ld_dy, int n, int E) {
-  const int row = blockIdx.x;
-  const long off = (long)(int)(ids[row] * (float)E);
-  for (int c = threadIdx.x; c < E; c += blockDim.x)
-    unsafeAtomicAdd(dtable + off + c, dy[(long)row * ld_dy + c]);
+  __shared__ long off[kEmbedChunk];
+  __shared__ int lead[kEmbedChunk];
+  const int row0 = blockIdx.x * kEmbedChunk, tid = threadIdx.x;
+  if (tid < kEmbedChunk) off[tid] = row0 + tid < n ? (long)(int)(ids[row0 + tid] * (float)E) : -1 - tid;
+  __syncthreads();
+  if (tid < kEmbedChunk) {
+    int l = tid;
+    for (int r = tid - 1; r >= 0; r--)
+      if (off[r] == off[tid]) l = r;
+    lead[tid] = l;  // first row of the chunk with this id
+  }
+  __syncthreads();
+  for (int c = tid; c < E; c += blockDim.x) {
+#pragma unroll
+    for (int r = 0; r < kEmbedChunk; r++) {
+      if (lead[r] != r || off[r] < 0) continue;
+      float s = dy[(long)(row0 + r) * ld_dy + c];
+      for (int q = r + 1; q < kEmbedChunk; q++)
+        if (lead[q] == r) s += dy[(long)(row0 + q) * ld_dy + c];
+      unsafeAtomicAdd(dtable + off[r] + c, s);
+    }
+  }
 }
 
 // ------------------------------------------------------------------ bias add
@@ -231,7 +253,7 @@ int cavs_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, 
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dtable && ids && dy, "cavs_embed_bwd: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
-  embed_bwd_kernel<<<n, block, 0, as_stream(stream)>>>(dtable, ids, dy, ld_dy, n, E);
+  embed_bwd_kernel<<<(n + kEmbedChunk - 1) / kEmbedChunk, block, 0, as_stream(stream)>>>(dtable, ids, dy, ld_dy, n, E);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -1,0 +1,371 @@
+// Per-step work around the rounds, folded into few launches: the classifier head
+// (FullyConnected + SoftmaxEntropyLoss and their gradients) for a handful of classes, the
+// SGD update of all dense parameters in one launch, a row-sparse update of the embedding
+// table, and the bias gradient (column sums of the four gate blocks) in one launch.
+// Every one of these is a few microseconds of HBM traffic; as separate library-style
+// launches their fixed costs add up to more than a round of the vertex function.
+#include "common.h"
+
+namespace cavs {
+
+__device__ inline float wsum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+// ------------------------------------------------------------------ classifier head
+// One wavefront per row, lane l owning columns l, l+64, ... (Q of them) of x and of every row
+// of W, all in registers: logits = x * W^T + b by C dot products reduced across the wave,
+// softmax / loss / d logits, d x = d logits * W.  The weight and bias gradients accumulate in
+// registers over the rows a wavefront owns, are combined per workgroup through LDS and parked
+// in `part[workgroup]`; a second kernel sums the workgroups in index order.
+template <int C, int Q>
+__global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ X, const float *__restrict__ W,
+                                                      const float *__restrict__ b, const float *__restrict__ labels,
+                                                      float *__restrict__ loss, float *__restrict__ logits,
+                                                      float *__restrict__ dX, float *__restrict__ part, int n, int H,
+                                                      float inv_n) {
+  extern __shared__ float sm[];  // [4][C*H] weight-gradient partials, then [4][C] bias
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int CH = C * H;
+  const bool grad = part != nullptr;
+  float w[C][Q], acc[C][Q], dbacc[C], bias[C];
+#pragma unroll
+  for (int c = 0; c < C; c++) {
+    bias[c] = b[c];
+    dbacc[c] = 0.f;
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      const int col = q * 64 + lane;
+      w[c][q] = col < H ? W[c * H + col] : 0.f;
+      acc[c][q] = 0.f;
+    }
+  }
+  for (int row = blockIdx.x * 4 + wave; row < n; row += gridDim.x * 4) {
+    const float *x = X + (long)row * H;
+    float xv[Q], z[C];
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      const int col = q * 64 + lane;
+      xv[q] = col < H ? x[col] : 0.f;
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      float s = 0.f;
+#pragma unroll
+      for (int q = 0; q < Q; q++) s += xv[q] * w[c][q];
+      z[c] = wsum(s) + bias[c];
+      mx = fmaxf(mx, z[c]);
+    }
+    // cavs/backend/op_impl_softmax_entropy_logits_loss.cu:94-140, :212-250
+    const int lab = (int)labels[row];
+    float sum = 0.f, zl = 0.f;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      sum += expf(z[c] - mx);
+      if (c == lab) zl = z[c];
+    }
+    if (lane == 0) loss[row] = -logf(expf(zl - mx) / sum);
+    if (logits) {
+#pragma unroll
+      for (int c = 0; c < C; c++)
+        if (lane == c) logits[(long)row * C + c] = z[c];
+    }
+    if (!grad) continue;
+    float d[C];
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+      const float p = expf(z[c] - mx) / sum;
+      d[c] = (c == lab ? p - 1.f : p) * inv_n;
+      dbacc[c] += d[c];
+    }
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      float dx = 0.f;
+#pragma unroll
+      for (int c = 0; c < C; c++) {
+        dx += d[c] * w[c][q];
+        acc[c][q] += d[c] * xv[q];
+      }
+      const int col = q * 64 + lane;
+      if (col < H) dX[(long)row * H + col] = dx;
+    }
+  }
+  if (!grad) return;
+  float *mine = sm + wave * CH, *sdb = sm + 4 * CH;
+#pragma unroll
+  for (int c = 0; c < C; c++) {
+#pragma unroll
+    for (int q = 0; q < Q; q++) {
+      const int col = q * 64 + lane;
+      if (col < H) mine[c * H + col] = acc[c][q];
+    }
+    if (lane == 0) sdb[wave * C + c] = dbacc[c];
+  }
+  __syncthreads();
+  float *out = part + (long)blockIdx.x * (CH + C);
+  for (int i = tid; i < CH; i += 256) out[i] = (sm[i] + sm[CH + i]) + (sm[2 * CH + i] + sm[3 * CH + i]);
+  if (tid < C) out[CH + tid] = (sdb[tid] + sdb[C + tid]) + (sdb[2 * C + tid] + sdb[3 * C + tid]);
+}
+
+// out[i] = sum over the workgroups' partials: four interleaved slices per output, each added
+// in index order, combined in a fixed order
+__global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__restrict__ part, int nparts, int total,
+                                                             int CH, float *__restrict__ dW, float *__restrict__ db) {
+  __shared__ float s[4][64];
+  const int o = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int i = blockIdx.x * 64 + o;
+  float a0 = 0.f, a1 = 0.f;
+  if (i < total) {
+    int p = q;
+    for (; p + 4 < nparts; p += 8) {
+      a0 += part[(long)p * total + i];
+      a1 += part[(long)(p + 4) * total + i];
+    }
+    for (; p < nparts; p += 4) a0 += part[(long)p * total + i];
+  }
+  s[q][o] = a0 + a1;
+  __syncthreads();
+  if (q == 0 && i < total) {
+    const float v = (s[0][o] + s[1][o]) + (s[2][o] + s[3][o]);
+    if (i < CH) dW[i] = v; else db[i - CH] = v;
+  }
+}
+
+static int head_blocks(int n) {
+  int want = (n + 7) / 8;  // two rows per wavefront
+  int cap = num_cus() / 2;
+  return want < cap ? (want < 1 ? 1 : want) : cap;
+}
+
+// columns per lane (Q) for a width; the weights and their gradient live in 2*C*Q registers
+static int head_q(int H) { return H <= 256 ? 4 : (H <= 512 ? 8 : 16); }
+static bool head_supported(int H, int C) {
+  return C >= 1 && C <= 8 && H >= 1 && H <= 1024 && C * head_q(H) <= 64 && (size_t)(4 * C * H + 4 * C) * 4 <= 64 * 1024;
+}
+
+// ------------------------------------------------------------------ SGD over several tensors
+constexpr int kMaxTensors = 8;
+struct SgdBatch {
+  float *w[kMaxTensors];
+  const float *g[kMaxTensors];
+  size_t end[kMaxTensors];  // running element count
+  int count;
+};
+
+__global__ void sgd_multi_kernel(SgdBatch t, float lr) {
+  const size_t total = t.end[t.count - 1];
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += stride) {
+    int k = 0;
+    while (i >= t.end[k]) k++;
+    const size_t j = i - (k ? t.end[k - 1] : 0);
+    t.w[k][j] -= lr * t.g[k][j];
+  }
+}
+
+// ------------------------------------------------------------------ row-sparse embedding update
+// A row that was looked up several times in the step is updated once: the first workgroup
+// to raise the row's stamp to this step's epoch owns it.  A workgroup takes kSgdChunk lookups
+// and asks for a row once however often it occurs among them (parse trees look up one and
+// the same row for every internal vertex; one atomic per vertex would serialise on it).
+constexpr int kSgdChunk = 16;
+__global__ void embed_sgd_kernel(float *__restrict__ table, const float *__restrict__ dtable,
+                                 const float *__restrict__ ids, int n, int E, float lr, int *__restrict__ stamp,
+                                 int epoch) {
+  __shared__ int row[kSgdChunk];
+  __shared__ int owner[kSgdChunk];
+  const int v0 = blockIdx.x * kSgdChunk, tid = threadIdx.x;
+  if (tid < kSgdChunk) row[tid] = v0 + tid < n ? (int)ids[v0 + tid] : -1 - tid;
+  __syncthreads();
+  if (tid < kSgdChunk) {
+    bool first = row[tid] >= 0;
+    for (int r = 0; r < tid; r++) first = first && row[r] != row[tid];
+    owner[tid] = first && atomicMax(stamp + row[tid], epoch) < epoch;
+  }
+  __syncthreads();
+  for (int r = 0; r < kSgdChunk; r++) {
+    if (!owner[r]) continue;
+    const long off = (long)(int)(ids[v0 + r] * (float)E);
+    for (int c = tid; c < E; c += blockDim.x) table[off + c] -= lr * dtable[off + c];
+  }
+}
+
+__global__ void embed_zero_rows_kernel(float *__restrict__ dtable, const float *__restrict__ ids, int E) {
+  const long off = (long)(int)(ids[blockIdx.x] * (float)E);
+  for (int c = threadIdx.x; c < E; c += blockDim.x) dtable[off + c] = 0.f;
+}
+
+// ------------------------------------------------------------------ column sums of column blocks
+// out[dst[k]*bw + c] = sum over rows of inp[r][k*bw + c], for nb blocks of bw columns.
+// Workgroup = 4 wavefronts over a strip of 64 columns and a chunk of rows; chunk sums go to
+// part[chunk][nb*bw]; the second kernel adds the chunks in index order and permutes.
+struct BlockMap {
+  int dst[8];
+};
+
+__global__ __launch_bounds__(256) void colsum_part_kernel(float *__restrict__ part, const float *__restrict__ inp,
+                                                          long ld, int n, int w, int rows_per_chunk) {
+  __shared__ float s[4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + lane;
+  const int r0 = blockIdx.y * rows_per_chunk, r1 = min(n, r0 + rows_per_chunk);
+  float a0 = 0.f, a1 = 0.f;
+  if (col < w) {
+    int r = r0 + wave;
+    for (; r + 4 < r1; r += 8) {
+      a0 += inp[(long)r * ld + col];
+      a1 += inp[(long)(r + 4) * ld + col];
+    }
+    for (; r < r1; r += 4) a0 += inp[(long)r * ld + col];
+  }
+  s[wave][lane] = a0 + a1;
+  __syncthreads();
+  if (wave == 0 && col < w) part[(long)blockIdx.y * w + col] = (s[0][lane] + s[1][lane]) + (s[2][lane] + s[3][lane]);
+}
+
+__global__ __launch_bounds__(256) void colsum_blocks_reduce_kernel(float *__restrict__ out, const float *__restrict__ part,
+                                                                   int chunks, int w, int bw, BlockMap map) {
+  __shared__ float s[4][64];
+  const int o = threadIdx.x & 63, q = threadIdx.x >> 6;
+  const int col = blockIdx.x * 64 + o;
+  float a = 0.f;
+  if (col < w)
+    for (int c = q; c < chunks; c += 4) a += part[(long)c * w + col];
+  s[q][o] = a;
+  __syncthreads();
+  if (q == 0 && col < w) out[map.dst[col / bw] * bw + col % bw] = (s[0][o] + s[1][o]) + (s[2][o] + s[3][o]);
+}
+
+static int colsum_chunks(int n) {
+  int c = (n + 127) / 128;
+  return c < 1 ? 1 : (c > 32 ? 32 : c);
+}
+
+}  // namespace cavs
+
+using namespace cavs;
+
+extern "C" {
+
+size_t cavs_fc_softmax_xent_workspace(int n, int H, int C) {
+  if (n <= 0 || !head_supported(H, C)) return 0;
+  return (size_t)head_blocks(n) * ((size_t)C * H + C) * sizeof(float);
+}
+
+int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const float *labels, float *loss,
+                         float *logits, float *dX, float *dW, float *db, void *workspace,
+                         size_t workspace_bytes, int n, int H, int C, void *stream) {
+  CAVS_REQUIRE(n >= 0 && head_supported(H, C), "cavs_fc_softmax_xent: unsupported shape n=%d H=%d C=%d (C <= 8, H <= 1024, C * columns-per-lane <= 64)", n, H, C);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(X && W && b && labels && loss, "cavs_fc_softmax_xent: null pointer");
+  const bool grad = dX || dW || db;
+  CAVS_REQUIRE(!grad || (dX && dW && db), "cavs_fc_softmax_xent: dX, dW and db must be all set or all null");
+  const int blocks = head_blocks(n);
+  const size_t need = (size_t)blocks * ((size_t)C * H + C) * sizeof(float);
+  CAVS_REQUIRE(!grad || (workspace && workspace_bytes >= need), "cavs_fc_softmax_xent: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  float *part = grad ? static_cast<float *>(workspace) : nullptr;
+  const size_t lds = (size_t)(4 * C * H + 4 * C) * sizeof(float);
+  hipStream_t st = as_stream(stream);
+  const float inv_n = 1.f / (float)n;
+  const int q = head_q(H);
+#define CAVS_HEAD(CC)                                                                                              \
+  case CC:                                                                                                         \
+    if (q == 4) fc_xent_kernel<CC, 4><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n);       \
+    else if (q == 8) fc_xent_kernel<CC, 8><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n);  \
+    else fc_xent_kernel<(CC <= 4 ? CC : 1), 16><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n); \
+    break
+  switch (C) {
+    CAVS_HEAD(1); CAVS_HEAD(2); CAVS_HEAD(3); CAVS_HEAD(4); CAVS_HEAD(5); CAVS_HEAD(6); CAVS_HEAD(7); CAVS_HEAD(8);
+  }
+#undef CAVS_HEAD
+  CAVS_LAUNCH_CHECK();
+  if (grad) {
+    const int total = C * H + C;
+    fc_xent_reduce_kernel<<<(total + 63) / 64, 256, 0, st>>>(part, blocks, total, C * H, dW, db);
+    CAVS_LAUNCH_CHECK();
+  }
+  return CAVS_OK;
+}
+
+int cavs_sgd_multi(int count, float *const *w, const float *const *g, const size_t *n, float lr, void *stream) {
+  CAVS_REQUIRE(count >= 0 && (count == 0 || (w && g && n)), "cavs_sgd_multi: bad arguments");
+  hipStream_t st = as_stream(stream);
+  for (int i = 0; i < count;) {
+    SgdBatch t{};
+    size_t run = 0;
+    int k = 0;
+    for (; i < count && k < kMaxTensors; i++) {
+      if (n[i] == 0) continue;
+      CAVS_REQUIRE(w[i] && g[i], "cavs_sgd_multi: null tensor %d", i);
+      run += n[i];
+      t.w[k] = w[i];
+      t.g[k] = g[i];
+      t.end[k] = run;
+      k++;
+    }
+    if (k == 0) continue;
+    t.count = k;
+    size_t blocks = (run + 255) / 256, cap = (size_t)num_cus() * 16;
+    sgd_multi_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, st>>>(t, lr);
+    CAVS_LAUNCH_CHECK();
+  }
+  return CAVS_OK;
+}
+
+int cavs_embed_sgd(float *table, const float *dtable, const float *ids, int n, int E, float lr, int *stamp,
+                   int epoch, void *stream) {
+  CAVS_REQUIRE(n >= 0 && E > 0, "cavs_embed_sgd: bad shape n=%d E=%d", n, E);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(table && dtable && ids && stamp, "cavs_embed_sgd: null pointer");
+  int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
+  embed_sgd_kernel<<<(n + kSgdChunk - 1) / kSgdChunk, block, 0, as_stream(stream)>>>(table, dtable, ids, n, E, lr, stamp, epoch);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_embed_zero_rows(float *dtable, const float *ids, int n, int E, void *stream) {
+  CAVS_REQUIRE(n >= 0 && E > 0, "cavs_embed_zero_rows: bad shape n=%d E=%d", n, E);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dtable && ids, "cavs_embed_zero_rows: null pointer");
+  int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
+  embed_zero_rows_kernel<<<n, block, 0, as_stream(stream)>>>(dtable, ids, E);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+size_t cavs_colsum_blocks_workspace(int n, int bw, int nb) {
+  if (n <= 0 || bw <= 0 || nb <= 0) return 0;
+  return (size_t)colsum_chunks(n) * bw * nb * sizeof(float);
+}
+
+int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int nb, const int *dst_block,
+                       void *workspace, size_t workspace_bytes, void *stream) {
+  CAVS_REQUIRE(n >= 0 && bw > 0 && nb > 0 && nb <= 8 && ld >= bw * nb, "cavs_colsum_blocks: bad shape n=%d bw=%d nb=%d ld=%d", n, bw, nb, ld);
+  CAVS_REQUIRE(out && dst_block, "cavs_colsum_blocks: null pointer");
+  BlockMap map{};
+  unsigned seen = 0;
+  for (int k = 0; k < nb; k++) {
+    CAVS_REQUIRE(dst_block[k] >= 0 && dst_block[k] < nb && !(seen >> dst_block[k] & 1u), "cavs_colsum_blocks: dst_block is not a permutation");
+    seen |= 1u << dst_block[k];
+    map.dst[k] = dst_block[k];
+  }
+  const int w = bw * nb;
+  if (n == 0) return cavs_zero(out, (size_t)w * 4, stream);
+  CAVS_REQUIRE(inp, "cavs_colsum_blocks: null input");
+  const int chunks = colsum_chunks(n);
+  const size_t need = (size_t)chunks * w * sizeof(float);
+  CAVS_REQUIRE(workspace && workspace_bytes >= need, "cavs_colsum_blocks: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+  const int rpc = ((n + chunks - 1) / chunks + 3) / 4 * 4;
+  hipStream_t st = as_stream(stream);
+  float *part = static_cast<float *>(workspace);
+  colsum_part_kernel<<<dim3((w + 63) / 64, chunks), 256, 0, st>>>(part, inp, ld, n, w, rpc);
+  CAVS_LAUNCH_CHECK();
+  colsum_blocks_reduce_kernel<<<(w + 63) / 64, 256, 0, st>>>(out, part, chunks, w, bw, map);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // extern "C"

@@ -7,6 +7,7 @@
 #include <cstddef>
 #include <stdexcept>
 #include <string>
+#include <utility>
 
 #include "cavs_hip.h"
 
@@ -47,6 +48,10 @@ class DeviceArray {
   T *get() const { return p_; }
   size_t capacity() const { return cap_; }
   T *at(size_t i) const { return p_ + i; }
+  void swap(DeviceArray &o) {
+    std::swap(p_, o.p_);
+    std::swap(cap_, o.cap_);
+  }
 
  private:
   T *p_ = nullptr;

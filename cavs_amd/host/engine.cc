@@ -230,6 +230,10 @@ void Engine::reserve_edges() {
   R(r_dG_, rc * nch_ * mw);
   if (cfg_.model != CAVS_MODEL_TREEFC) {
     R(xs_, cap);
+    if (xs_prev_.capacity() < cap) {  // the list of dirty rows does not survive a reallocation
+      R(xs_prev_, cap);
+      emb_sparse_valid_ = false;
+    }
     R(e_, cap * E_);
     R(de_, cap * E_);
     R(xW_, cap * 4 * H);
@@ -276,7 +280,13 @@ void Engine::upload_index_arena() {
   // upload that last read it has finished
   const int slot = idx_slot_;
   idx_slot_ ^= 1;
-  if (idx_pending_[slot]) check(cavs_event_sync(idx_copied_[slot]));
+  if (idx_pending_[slot]) {
+    auto w0 = std::chrono::steady_clock::now();
+    check(cavs_event_sync(idx_copied_[slot]));
+    wait_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
+  } else {
+    wait_ms_ = 0.f;
+  }
   idx_pending_[slot] = false;
   idx_host_[slot].reserve(total);
   if (idx_dev_.capacity() < total) {
@@ -322,6 +332,7 @@ void Engine::upload_index_arena() {
 void Engine::begin_step(const int *graph, int B, int maxlen) {
   auto t0 = std::chrono::steady_clock::now();
   std::string err = build_schedule(graph, B, maxlen, (cfg_.opt & CAVS_OPT_BATCHING) != 0, &sched_);
+  sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
   if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
   if (sched_.executed != sched_.N)
     fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample; the reference never executes such a vertex "
@@ -365,6 +376,12 @@ void Engine::backward_only(const float *dgraph_out) {
 
 void Engine::step(const int *graph, int B, int maxlen, const void *x, const void *labels,
                   bool on_device, bool backward, float lr) {
+  auto step_t0 = std::chrono::steady_clock::now();
+  struct StepTimer {
+    Engine *e;
+    std::chrono::steady_clock::time_point t0;
+    ~StepTimer() { e->host_step_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count(); }
+  } step_timer{this, step_t0};
   begin_step(graph, B, maxlen);
   const int N = N_, H = cfg_.H;
   const bool needs_x = cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x;
@@ -411,11 +428,31 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     }
     check(cavs_event_record(ev_[3], stream_));
     ev_bwd_valid_ = true;
-    if (lr != 0.f)
+    if (lr != 0.f) {
+      // w -= lr * g (cavs/backend/op_impl_sgd.cu); the embedding table by its looked-up rows
+      // only: every other row of its gradient is zero, so the dense update would not move it
+      std::vector<float *> ws;
+      std::vector<const float *> gs;
+      std::vector<size_t> ns;
       for (auto &kv : params_) {
-        check(cavs_sgd(kv.second->w, kv.second->g, lr, kv.second->n, stream_));
-        c_launches_ += 1;
+        Param &p = *kv.second;
+        if (kv.first == "Emb" && emb_dirty_n_ == N) {
+          const int E = (int)(p.n / cfg_.V);
+          if (emb_stamp_.capacity() < (size_t)cfg_.V) {
+            emb_stamp_.reserve(cfg_.V);
+            check(cavs_zero(emb_stamp_.get(), (size_t)cfg_.V * 4, stream_));
+          }
+          check(cavs_embed_sgd(p.w, p.g, xs_prev_.get(), N, E, lr, emb_stamp_.get(), ++emb_epoch_, stream_));
+          c_launches_ += 1;
+          continue;
+        }
+        ws.push_back(p.w);
+        gs.push_back(p.g);
+        ns.push_back(p.n);
       }
+      check(cavs_sgd_multi((int)ws.size(), ws.data(), gs.data(), ns.data(), lr, stream_));
+      c_launches_ += 1;
+    }
   }
 }
 
@@ -544,21 +581,36 @@ void Engine::treelstm_backward() {
   // accumulates the same sums round by round)
   const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
   gemm(0, 1, N, E, 4 * H, dxW_.get(), 4 * H, W, 4 * H, 0.f, de_.get(), E);
-  Param &emb = param("Emb");
-  check(cavs_zero(emb.g, emb.n * 4, stream_));
-  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), E, N, E, stream_));
-  c_launches_ += 2;
+  embedding_backward(E);
   gemm_splitk(1, 0, E, 4 * H, N, e_.get(), E, dxW_.get(), 4 * H, param("W").g, 4 * H);
   float *dU = param("U").g;
   gemm_splitk(1, 0, H, 3 * H, N - lp, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H);
   gemm_splitk(1, 0, H, H, 2 * (N - lp), G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
               dU + (size_t)3 * H * H, H);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
-  float *dB = param("Bv").g;
-  const int src_block[4] = {0, 3, 2, 1};
-  for (int k = 0; k < 4; k++)
-    check(cavs_colsum(dB + (size_t)k * H, dxW_.get() + (size_t)src_block[k] * H, 4 * H, N, H, 0, stream_));
-  c_launches_ += 4;
+  const int dst_block[4] = {0, 3, 2, 1};  // dxW block k ([i|o|u|f]) lands in bias block dst_block[k]
+  const size_t cs_bytes = cavs_colsum_blocks_workspace(N, H, 4);
+  float *cs_ws = workspace(cs_bytes);
+  check(cavs_colsum_blocks(param("Bv").g, dxW_.get(), 4 * H, N, H, 4, dst_block, cs_ws, cs_bytes, stream_));
+  c_launches_ += 2;
+}
+
+// EmbeddingLookup_grad (cavs/backend/op_impl_embedding.cu:58-92): scatter-add of the rows of
+// de into a zeroed table.  The table is kept zero outside the rows of the previous step, so
+// clearing it costs those rows, not the vocabulary.
+void Engine::embedding_backward(int E) {
+  Param &emb = param("Emb");
+  const bool owned = emb.g == emb.own_g.get();
+  if (owned && emb_sparse_valid_) {
+    if (emb_dirty_n_ > 0) check(cavs_embed_zero_rows(emb.g, xs_prev_.get(), emb_dirty_n_, E, stream_));
+  } else {
+    check(cavs_zero(emb.g, emb.n * 4, stream_));
+  }
+  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), E, N_, E, stream_));
+  c_launches_ += 2;
+  xs_.swap(xs_prev_);  // this step's ids: the rows that are dirty now
+  emb_dirty_n_ = N_;
+  emb_sparse_valid_ = owned;
 }
 
 // ------------------------------------------------------------------ chain LSTM
@@ -608,10 +660,7 @@ void Engine::lstm_backward() {
   }
   const int lp = sched_.leaf_prefix;
   gemm(0, 1, N, H, 4 * H, dxW_.get(), 4 * H, Wx, 4 * H, 0.f, de_.get(), H);
-  Param &emb = param("Emb");
-  check(cavs_zero(emb.g, emb.n * 4, stream_));
-  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), H, N, H, stream_));
-  c_launches_ += 2;
+  embedding_backward(H);
   float *dW = param("W").g;
   gemm_splitk(1, 0, H, 4 * H, N, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H);
   gemm_splitk(1, 0, H, 4 * H, N - lp, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
@@ -682,6 +731,14 @@ void Engine::head_forward_backward(bool backward) {
     // FullyConnected + SoftmaxEntropyLoss (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79,
     // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
     Param &Wfc = param("Wfc"), &bfc = param("bfc");
+    const size_t head_bytes = cavs_fc_softmax_xent_workspace(N, H, C);
+    if (head_bytes > 0) {  // few classes: the whole head and its gradients in two launches
+      float *hw = workspace(head_bytes);
+      check(cavs_fc_softmax_xent(GO_.get(), Wfc.w, bfc.w, d_labels_, loss_.get(), logits_.get(), backward ? dGO_.get() : nullptr,
+                                 backward ? Wfc.g : nullptr, backward ? bfc.g : nullptr, hw, head_bytes, N, H, C, stream_));
+      c_launches_ += backward ? 2 : 1;
+      return;
+    }
     gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w, H, 0.f, logits_.get(), C);
     check(cavs_bias_add_rows(logits_.get(), logits_.get(), bfc.w, N, C, stream_));
     check(cavs_softmax_xent(loss_.get(), backward ? dlogits_.get() : nullptr, logits_.get(), d_labels_, N, C, stream_));
@@ -752,6 +809,11 @@ void Engine::fetch(const std::string &what, float *host, size_t n) {
 float Engine::timing(const std::string &name) {
   float ms = 0.f;
   if (name == "GraphParsing") return parse_ms_;
+  // host-side split of a step: building the schedule, waiting for the index staging buffer
+  // of two steps ago (i.e. for the device), and the whole enqueueing call
+  if (name == "HostSchedule") return sched_ms_;
+  if (name == "HostWait") return wait_ms_;
+  if (name == "HostStep") return host_step_ms_;
   if (name == "RNNForward" && ev_valid_) {
     check(cavs_event_elapsed_ms(&ms, ev_[0], ev_[1]));
     return ms;

@@ -108,7 +108,7 @@ class Engine {
   bool own_stream_ = true;
   void *ev_[4] = {nullptr, nullptr, nullptr, nullptr};  // fwd begin/end, bwd begin/end
   bool ev_valid_ = false, ev_bwd_valid_ = false;
-  float parse_ms_ = 0.f;
+  float parse_ms_ = 0.f, sched_ms_ = 0.f, wait_ms_ = 0.f, host_step_ms_ = 0.f;
   std::map<std::string, std::unique_ptr<Param>> params_;
 
   Schedule sched_;
@@ -131,6 +131,13 @@ class Engine {
   DeviceArray<float> xs_, e_, xW_, G_, hlr_, gates_, msg_, pool_, GO_, dGO_, dret_, dpool_, dxW_,
       dF_, de_, logits_, dlogits_, loss_, ws_;
   DeviceArray<float> r_hU_, r_hUf_, r_dmsg_, r_dG_, r_dhlr_, r_z_;  // round-local
+  // Embedding gradient: only the rows looked up in a step are non-zero, so the table is
+  // cleared and updated by those rows.  xs_prev_ lists the rows the last backward pass wrote.
+  DeviceArray<float> xs_prev_;
+  DeviceArray<int> emb_stamp_;
+  int emb_dirty_n_ = 0, emb_epoch_ = 0;
+  bool emb_sparse_valid_ = true;  // the table is zero outside xs_prev_[0, emb_dirty_n_)
+  void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
   // rounds of at most this many rows run as fused launches (0: none)
   int fused_rows() const;

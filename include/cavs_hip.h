@@ -205,6 +205,37 @@ int cavs_treefc_fwd(const float *z, const float *bias, const float *x, float *h,
 int cavs_treefc_bwd(const float *dh_m, const float *dret, const float *h, float *dz, int n,
                     int H, int act, void *stream);
 
+/* ------------------------------------------------------------------ per-step folds
+ * The work of a training step around the rounds, each group in one or two launches.
+ *
+ * cavs_fc_softmax_xent: FullyConnected (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79)
+ * + SoftmaxEntropyLoss (op_impl_softmax_entropy_logits_loss.cu:94-140) and, when dX, dW and db
+ * are given, their gradients (:150-163, :212-250) for a head of at most 8 classes:
+ * X [n,H], W [C,H], b [C], labels [n] (class ids as floats); loss [n], logits [n,C] (may be
+ * NULL), dX [n,H], dW [C,H], db [C]; d logits = (softmax - onehot) / n.  The workspace query
+ * returns 0 for a shape this entry point does not take (C > 8, H > 1024, or C * ceil-pow2(H/64) > 64). */
+size_t cavs_fc_softmax_xent_workspace(int n, int H, int C);
+int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const float *labels,
+                         float *loss, float *logits, float *dX, float *dW, float *db,
+                         void *workspace, size_t workspace_bytes, int n, int H, int C, void *stream);
+/* SGD (cavs/backend/op_impl_sgd.cu) over `count` tensors in one launch; the arrays are host arrays. */
+int cavs_sgd_multi(int count, float *const *w, const float *const *g, const size_t *n, float lr,
+                   void *stream);
+/* SGD of an embedding table restricted to the rows ids[0..n) (ids as floats, like
+ * EmbeddingLookup).  Equal to the dense update when every other row of dtable is zero.  A row
+ * listed several times is updated once: stamp [rows of the table] must start at zero and epoch
+ * must grow by one per call. */
+int cavs_embed_sgd(float *table, const float *dtable, const float *ids, int n, int E, float lr,
+                   int *stamp, int epoch, void *stream);
+/* dtable rows ids[0..n) = 0 */
+int cavs_embed_zero_rows(float *dtable, const float *ids, int n, int E, void *stream);
+/* Column sums of nb (<= 8) adjacent column blocks of bw columns of inp [n, ld], block k written
+ * to out block dst_block[k] (a permutation; host array).  Deterministic: row chunks are summed
+ * in index order.  The bias gradient of the gates (cavs/backend/op_impl_elementwise.cuh:24-34). */
+size_t cavs_colsum_blocks_workspace(int n, int bw, int nb);
+int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int nb,
+                       const int *dst_block, void *workspace, size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------ fused rounds
  * One round of the Tree-LSTM vertex function (apps/paper/tree-lstm-cavs.cc:129-172)
  * with its graph operators folded in: Gather (op_impl_graphop.cu:50-110) becomes the

@@ -86,7 +86,9 @@ int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int w
                         int *out, int cap);
 
 /* Timers of the last step in ms, by the reference's names (cavs/midend/statement.cc:
- * 53,65,68,84,102,122): "GraphParsing" (host), "RNNForward", "RNNBackward" (device). */
+ * 53,65,68,84,102,122): "GraphParsing" (host), "RNNForward", "RNNBackward" (device); and the
+ * host-side split "HostSchedule" (scheduler), "HostWait" (waiting for the device to release
+ * an index staging buffer), "HostStep" (the whole enqueueing call). */
 int cavs_session_timing(cavs_session *s, const char *name, float *ms);
 /* Device time per kernel class.  While enabled, every launch of the session is
  * bracketed by a pair of events on the session's stream; profile_read waits for the

@@ -212,3 +212,31 @@ def test_fused_rounds_match_oracle(oracle, H, limit, pairing):
     s.close()
     compare(got, want)
     assert (fused_flops > 0) == (limit >= 0), (fused_flops, sizes)
+
+
+@pytest.mark.parametrize("model", ["treelstm", "lstm"])
+def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
+    """Four SGD steps over three different batches (token ids overlap between steps, one
+    step runs without an update in between): every parameter, the embedding table in
+    particular, follows the oracle's dense w -= lr * g, and the gradients of the last step
+    stay readable."""
+    kw = dict(B=6, H=32, E=12, V=17, C=4)            # a tiny vocabulary: many repeated rows
+    batches = [small_workload(model, 101 + k, **kw) for k in range(3)]
+    H, E, V, C_ = 32, (32 if model == "lstm" else 12), 17, 4
+    s = session.Session(model, H=H, E=E, V=V, C_=C_)
+    s.set_params(batches[0]["params"])
+    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc") if model == "treelstm" else ("Emb", "W", "Bv", "Wfc", "bfc")
+    p = {k: np.array(batches[0]["params"][k], np.float32) for k in names}
+    plan = [(0, 0.5), (1, 0.0), (2, 0.25), (0, 0.5)]  # (batch, lr); lr 0 leaves the gradient in place
+    for step, (bi, lr) in enumerate(plan):
+        w = batches[bi]
+        print(f"[case] {model} sgd step {step} batch {bi} lr {lr}", flush=True)
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
+        s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
+        got = s.grads()
+        for k in names:
+            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", rtol=3e-4, atol=3e-5)
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    for k in names:
+        close(s.param(k, p[k].shape), p[k], f"{k} after the steps", rtol=3e-4, atol=3e-5)
+    s.close()

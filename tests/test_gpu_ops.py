@@ -564,3 +564,101 @@ def test_fused_round_entry_points_reject_bad_shapes():
         hip.call("cavs_treelstm_round_bwd_children", 0, 4 * 24, 0, 0, 0, 0, 5, 24, 0)
     with pytest.raises(hip.CavsError, match="all set"):
         hip.call("cavs_treelstm_round_bwd_gates", 16, 16, 16, 16, 16, 0, 16, 4 * 32, 0, 5, 32, 0)
+
+
+@pytest.mark.parametrize("n,H,C_", [(1, 64, 2), (19, 96, 5), (2482, 512, 5), (300, 100, 8), (77, 1024, 3)])
+def test_fused_classifier_head(g, oracle, n, H, C_):
+    """FullyConnected + softmax cross-entropy and their gradients in two launches, against
+    the oracle's GEMM, softmax and column-sum pieces."""
+    import ctypes as C
+
+    r = rng(n + H + C_)
+    X = r.bulk_normal(n * H).reshape(n, H)
+    W = (r.bulk_normal(C_ * H).reshape(C_, H) / np.sqrt(H)).astype(np.float32)
+    b = r.bulk_normal(C_)
+    labels = np.floor(r.bulk_uniform(n) * C_).astype(np.float32)
+    logits_w = oracle.sgemm(0, 1, X, W) + b[None, :]
+    loss_w, d_w = oracle.softmax_xent(logits_w, labels)
+    dX_w = oracle.sgemm(0, 0, d_w, W)
+    dW_w = oracle.sgemm(1, 0, d_w, X)
+    db_w = d_w.astype(np.float64).sum(0)
+    nb = hip.lib().cavs_fc_softmax_xent_workspace(n, H, C_)
+    assert nb > 0
+    ws = g.zeros(nb // 4)
+    loss, logits, dX, dW, db = g.zeros(n), g.zeros(n, C_), g.zeros(n, H), g.zeros(C_, H), g.zeros(C_)
+    args = (g.P(g.devf(X)), g.P(g.devf(W)), g.P(g.devf(b)), g.P(g.devf(labels)), g.P(loss), g.P(logits))
+    g.call("cavs_fc_softmax_xent", *args, g.P(dX), g.P(dW), g.P(db), g.P(ws), nb, n, H, C_, g.stream())
+    close(g.host(logits), logits_w, "logits")
+    close(g.host(loss), loss_w, "loss")
+    close(g.host(dX), dX_w, "dX", atol=1e-7)
+    close(g.host(dW), dW_w, "dW", atol=1e-6)
+    close(g.host(db), db_w, "db", atol=1e-6)
+    # forward only: no gradient buffers, no workspace
+    loss2 = g.zeros(n)
+    g.call("cavs_fc_softmax_xent", *args[:4], g.P(loss2), None, None, None, None, None, 0, n, H, C_, g.stream())
+    np.testing.assert_array_equal(g.host(loss2), g.host(loss))
+    assert hip.lib().cavs_fc_softmax_xent_workspace(10, 512, 9) == 0      # too many classes
+    assert hip.lib().cavs_fc_softmax_xent_workspace(10, 4096, 5) == 0     # accumulators exceed LDS
+    with pytest.raises(hip.CavsError, match="unsupported shape"):
+        hip.call("cavs_fc_softmax_xent", 16, 16, 16, 16, 16, 0, 0, 0, 0, 0, 0, 4, 512, 9, 0)
+
+
+def test_sgd_over_several_tensors_and_sparse_embedding_update(g):
+    import ctypes as C
+
+    r = rng(11)
+    sizes = [5, 1000, 0, 77777, 3, 64, 512, 129, 1, 4096]      # more than one batch of eight, one empty
+    ws = [r.bulk_normal(max(k, 1))[:k] for k in sizes]
+    gs = [r.bulk_normal(max(k, 1))[:k] for k in sizes]
+    dw, dg = [g.devf(a) if len(a) else None for a in ws], [g.devf(a) if len(a) else None for a in gs]
+    pw = (C.c_void_p * len(sizes))(*[g.P(t) for t in dw])
+    pg = (C.c_void_p * len(sizes))(*[g.P(t) for t in dg])
+    pn = (C.c_size_t * len(sizes))(*sizes)
+    g.call("cavs_sgd_multi", len(sizes), pw, pg, pn, 0.25, g.stream())
+    for a, b, t in zip(ws, gs, dw):
+        if len(a):
+            np.testing.assert_array_equal(g.host(t), a - np.float32(0.25) * b)
+
+    # the row-sparse update equals the dense one when the gradient is zero off the listed rows
+    V, E, n = 500, 37, 120
+    table = r.bulk_normal(V * E).reshape(V, E)
+    ids = np.floor(r.bulk_uniform(n) * V).astype(np.float32)
+    ids[:40] = ids[0]                                           # one row looked up many times
+    grad = np.zeros((V, E), np.float32)
+    rows = np.unique(ids.astype(np.int64))
+    grad[rows] = r.bulk_normal(len(rows) * E).reshape(len(rows), E)
+    stamp = g.devi(np.zeros(V, np.int32))
+    t, dgrad, dids = g.devf(table), g.devf(grad), g.devf(ids)
+    want = table.copy()
+    for epoch in (1, 2):                                        # a second step must update again
+        g.call("cavs_embed_sgd", g.P(t), g.P(dgrad), g.P(dids), n, E, 0.5, g.P(stamp), epoch, g.stream())
+        want = want - np.float32(0.5) * grad
+        np.testing.assert_array_equal(g.host(t), want)
+    g.call("cavs_embed_zero_rows", g.P(dgrad), g.P(dids), n, E, g.stream())
+    assert not g.host(dgrad).any()
+
+
+@pytest.mark.parametrize("n,bw,perm", [(1, 4, [0]), (2482, 512, [0, 3, 2, 1]), (63, 6, [2, 0, 1]), (5000, 64, [1, 0])])
+def test_column_sums_of_permuted_blocks(g, n, bw, perm):
+    import ctypes as C
+
+    r = rng(n + bw)
+    nb = len(perm)
+    ld = bw * nb + 8
+    X = r.bulk_normal(n * ld).reshape(n, ld)
+    exact = X[:, : bw * nb].astype(np.float64).sum(0).reshape(nb, bw)
+    want = np.zeros((nb, bw))
+    for k, d in enumerate(perm):
+        want[d] = exact[k]
+    nbytes = hip.lib().cavs_colsum_blocks_workspace(n, bw, nb)
+    ws, out = g.zeros(nbytes // 4), g.zeros(nb * bw, fill=float("nan"))
+    dst = (C.c_int * nb)(*perm)
+    dX = g.devf(X)
+    g.call("cavs_colsum_blocks", g.P(out), g.P(dX), ld, n, bw, nb, dst, g.P(ws), nbytes, g.stream())
+    first = g.host(out).copy()
+    close(first, want.ravel(), rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    g.call("cavs_colsum_blocks", g.P(out), g.P(dX), ld, n, bw, nb, dst, g.P(ws), nbytes, g.stream())
+    np.testing.assert_array_equal(g.host(out), first)           # fixed summation order
+    with pytest.raises(hip.CavsError, match="permutation"):
+        hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * nb)(*([0] * nb)), 16, nbytes, 0) if nb > 1 else \
+            hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * 1)(3), 16, nbytes, 0)
