@@ -27,6 +27,8 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
+# (workload, kernel class) -> HBM bytes per dispatch, profiles/bench_C3_hbm_traffic_pmc.txt
+PMC_TRAFFIC_BYTES = {("C3", "round"): 16.05e6}
 
 
 def model_kwargs(w):
@@ -148,7 +150,11 @@ def main():
     }
     for v in mfma.values():
         v["tf"] = v["flops"] / (v["ms"] * 1e-3) / 1e12 if v["ms"] else 0.0
-    dom = max(mfma.values(), key=lambda v: v["ms"])
+    dom_name, dom = max(mfma.items(), key=lambda kv: kv[1]["ms"])
+    # HBM bytes per dispatch of that class from the two rocprofv3 --pmc runs (FETCH_SIZE scaled by the
+    # factor a plain copy of known size gives, plus WRITE_SIZE) summarised under profiles/; measured
+    # for the default workload only
+    traffic = PMC_TRAFFIC_BYTES.get((a.workload, dom_name)) if a.pairing == "reference" else None
     rounds = s.counter("rounds")
     launches = s.counter("launches")
 
@@ -162,7 +168,7 @@ def main():
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing, "rounds_last_batch": rounds,
                    "launches_last_batch": launches},
         "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
-                     "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": None,
+                     "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": traffic,
                      "kernel": dom["kernel"],
                      "avg_launch_us": round(1e3 * dom["ms"] / dom["n"], 3) if dom["n"] else None,
                      "flops_per_launch": round(dom["flops"] / dom["n"], 1) if dom["n"] else None},

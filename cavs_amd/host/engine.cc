@@ -470,7 +470,8 @@ void Engine::pop_ret(float *graph_out) { scatter(graph_out, cfg_.H, d_t2j_, msg_
 int Engine::fused_rows() const {
   if (cfg_.model != CAVS_MODEL_TREELSTM || !(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.H % 32 != 0) return 0;
   if (cfg_.fused_round_rows < 0) return 0;
-  return cfg_.fused_round_rows > 0 ? cfg_.fused_round_rows : 4096;
+  // measured crossover with the separate launches: about 2400 rows at H=512, 1500 at H=1024
+  return cfg_.fused_round_rows > 0 ? cfg_.fused_round_rows : (cfg_.H <= 512 ? 2048 : 1024);
 }
 
 void Engine::treelstm_forward() {
