@@ -3,6 +3,7 @@
 #define CAVS_CSRC_COMMON_H_
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <cstdarg>
 #include <cstdint>
@@ -20,6 +21,28 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int kWave = 64;
 int num_cus();  // compute units of the current device (256 on MI355X)
+
+// Timing probe of the calling thread (cavs_profile_arm): while armed, the first kernel an
+// entry point launches records `start` when it begins and every kernel records `stop` when
+// it ends, so the pair brackets exactly the device time of the entry point's kernels.
+struct LaunchProbe {
+  hipEvent_t start = nullptr, stop = nullptr;
+  bool armed = false, started = false;
+};
+LaunchProbe &launch_probe();
+
+// Every kernel of this library is launched through here.
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t st, Args &&...args) {
+  LaunchProbe &p = launch_probe();
+  if (p.armed) {
+    hipEvent_t s = p.started ? nullptr : p.start;
+    p.started = true;
+    hipExtLaunchKernelGGL(kernel, grid, block, (unsigned)lds, st, s, p.stop, 0, static_cast<KArgs>(args)...);
+  } else {
+    hipLaunchKernelGGL(kernel, grid, block, (unsigned)lds, st, static_cast<KArgs>(args)...);
+  }
+}
 
 }  // namespace cavs
 

@@ -134,11 +134,11 @@ static int launch_gather(float *out, int ld_out, const float *src, int ld_src, c
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(out, ld_out, src, ld_src, w)) {
     int wv = w / 4;
-    gather_rows_kernel<float4><<<grid, block_for(wv), 0, st>>>(
+    launch(gather_rows_kernel<float4>, grid, block_for(wv), 0, st, 
         reinterpret_cast<float4 *>(out), ld_out / 4, reinterpret_cast<const float4 *>(src),
         ld_src / 4, ids, n, wv);
   } else {
-    gather_rows_kernel<float><<<grid, block_for(w), 0, st>>>(out, ld_out, src, ld_src, ids, n, w);
+    launch(gather_rows_kernel<float>, grid, block_for(w), 0, st, out, ld_out, src, ld_src, ids, n, w);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
@@ -173,10 +173,10 @@ int cavs_add_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, i
   hipStream_t st = as_stream(stream);
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(out, ld_out, inp, ld_inp, w))
-    add_rows_kernel<float4><<<grid, block_for(w / 4), 0, st>>>(reinterpret_cast<float4 *>(out), ld_out / 4,
+    launch(add_rows_kernel<float4>, grid, block_for(w / 4), 0, st, reinterpret_cast<float4 *>(out), ld_out / 4,
                                                                reinterpret_cast<const float4 *>(inp), ld_inp / 4, n, w / 4);
   else
-    add_rows_kernel<float><<<grid, block_for(w), 0, st>>>(out, ld_out, inp, ld_inp, n, w);
+    launch(add_rows_kernel<float>, grid, block_for(w), 0, st, out, ld_out, inp, ld_inp, n, w);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -197,11 +197,11 @@ int cavs_scatter_rows(float *dst, int ld_dst, const int *ids, const float *inp, 
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(dst, ld_dst, inp, ld_inp, w)) {
     int wv = w / 4;
-    scatter_rows_kernel<float4><<<grid, block_for(wv), 0, st>>>(
+    launch(scatter_rows_kernel<float4>, grid, block_for(wv), 0, st, 
         reinterpret_cast<float4 *>(dst), ld_dst / 4, ids, reinterpret_cast<const float4 *>(inp),
         ld_inp / 4, n, wv);
   } else {
-    scatter_rows_kernel<float><<<grid, block_for(w), 0, st>>>(dst, ld_dst, ids, inp, ld_inp, n, w);
+    launch(scatter_rows_kernel<float>, grid, block_for(w), 0, st, dst, ld_dst, ids, inp, ld_inp, n, w);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
@@ -215,11 +215,11 @@ int cavs_gather_children(float *G, float *hsum, const float *pool, const int *id
   hipStream_t st = as_stream(stream);
   int grid = (n + 1) / 2;
   if (w % 4 == 0 && hw % 4 == 0 && aligned16(G) && aligned16(pool) && (!hsum || aligned16(hsum))) {
-    gather_children_kernel<float4><<<grid, block_for(w / 4), 0, st>>>(
+    launch(gather_children_kernel<float4>, grid, block_for(w / 4), 0, st, 
         reinterpret_cast<float4 *>(G), reinterpret_cast<float4 *>(hsum),
         reinterpret_cast<const float4 *>(pool), ids, n, w / 4, hw / 4);
   } else {
-    gather_children_kernel<float><<<grid, block_for(w), 0, st>>>(G, hsum, pool, ids, n, w, hw);
+    launch(gather_children_kernel<float>, grid, block_for(w), 0, st, G, hsum, pool, ids, n, w, hw);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;

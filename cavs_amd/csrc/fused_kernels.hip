@@ -87,8 +87,16 @@ int cavs_fused_launch(void *handle, float *const *outs, int nouts, const float *
   for (auto &c : counts) args.push_back(&c);
   args.push_back(&n_elements);
   unsigned grid = (unsigned)((n_elements + kFusedBlock - 1) / kFusedBlock);
-  CAVS_HIP_TRY(hipModuleLaunchKernel(k->fn, grid, 1, 1, kFusedBlock, 1, 1, 0, as_stream(stream),
-                                     args.data(), nullptr));
+  LaunchProbe &p = launch_probe();
+  if (p.armed) {
+    hipEvent_t s = p.started ? nullptr : p.start;
+    p.started = true;
+    CAVS_HIP_TRY(hipExtModuleLaunchKernel(k->fn, grid * kFusedBlock, 1, 1, kFusedBlock, 1, 1, 0, as_stream(stream),
+                                          args.data(), nullptr, s, p.stop, 0));
+  } else {
+    CAVS_HIP_TRY(hipModuleLaunchKernel(k->fn, grid, 1, 1, kFusedBlock, 1, 1, 0, as_stream(stream),
+                                       args.data(), nullptr));
+  }
   return CAVS_OK;
 }
 

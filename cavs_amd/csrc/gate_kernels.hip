@@ -271,9 +271,9 @@ int cavs_treelstm_gates_fwd(const float *xW, int ld_xw, const float *hU, const f
   CAVS_REQUIRE((hU && hUf && G) || (!hU && !hUf && !G), "cavs_treelstm_gates_fwd: hU, hUf and G must be all set or all null");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && ld_xw % 4 == 0 && all_aligned({xW, hU, hUf, G, bias, gates, msg}))
-    treelstm_fwd_kernel<4><<<GATE_GRID(n, H, 4), 0, st>>>(xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
+    launch(treelstm_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
   else
-    treelstm_fwd_kernel<1><<<GATE_GRID(n, H, 1), 0, st>>>(xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
+    launch(treelstm_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -287,9 +287,9 @@ int cavs_treelstm_gates_bwd(const float *dmsg, const float *dret, const float *g
   CAVS_REQUIRE((G && dF && dG) || (!G && !dF && !dG), "cavs_treelstm_gates_bwd: G, dF and dG must be all set or all null");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && ld_dxw % 4 == 0 && all_aligned({dmsg, dret, gates, G, dxW, dF, dG}))
-    treelstm_bwd_kernel<4><<<GATE_GRID(n, H, 4), 0, st>>>(dmsg, dret, gates, G, dxW, ld_dxw, dF, dG, n, H);
+    launch(treelstm_bwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, dmsg, dret, gates, G, dxW, ld_dxw, dF, dG, n, H);
   else
-    treelstm_bwd_kernel<1><<<GATE_GRID(n, H, 1), 0, st>>>(dmsg, dret, gates, G, dxW, ld_dxw, dF, dG, n, H);
+    launch(treelstm_bwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, dmsg, dret, gates, G, dxW, ld_dxw, dF, dG, n, H);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -301,9 +301,9 @@ int cavs_lstm_gates_fwd(const float *a, int ld_a, const float *a2, const float *
   CAVS_REQUIRE(a && bias && gates && msg, "cavs_lstm_gates_fwd: null pointer");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && ld_a % 4 == 0 && all_aligned({a, a2, G, bias, gates, msg}))
-    lstm_fwd_kernel<4><<<GATE_GRID(n, H, 4), 0, st>>>(a, ld_a, a2, G, bias, gates, msg, n, H);
+    launch(lstm_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, a, ld_a, a2, G, bias, gates, msg, n, H);
   else
-    lstm_fwd_kernel<1><<<GATE_GRID(n, H, 1), 0, st>>>(a, ld_a, a2, G, bias, gates, msg, n, H);
+    launch(lstm_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, a, ld_a, a2, G, bias, gates, msg, n, H);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -316,9 +316,9 @@ int cavs_lstm_gates_bwd(const float *dmsg, const float *dret, const float *gates
   CAVS_REQUIRE((G && dG) || (!G && !dG), "cavs_lstm_gates_bwd: G and dG must be both set or both null");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && ld_da % 4 == 0 && all_aligned({dmsg, dret, gates, G, da, dG}))
-    lstm_bwd_kernel<4><<<GATE_GRID(n, H, 4), 0, st>>>(dmsg, dret, gates, G, da, ld_da, dG, n, H);
+    launch(lstm_bwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, dmsg, dret, gates, G, da, ld_da, dG, n, H);
   else
-    lstm_bwd_kernel<1><<<GATE_GRID(n, H, 1), 0, st>>>(dmsg, dret, gates, G, da, ld_da, dG, n, H);
+    launch(lstm_bwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, dmsg, dret, gates, G, da, ld_da, dG, n, H);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -330,9 +330,9 @@ int cavs_treefc_fwd(const float *z, const float *bias, const float *x, float *h,
   CAVS_REQUIRE(h, "cavs_treefc_fwd: null output");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && all_aligned({z, bias, x, h}))
-    treefc_fwd_kernel<4><<<GATE_GRID(n, H, 4), 0, st>>>(z, bias, x, h, n, H, act);
+    launch(treefc_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, z, bias, x, h, n, H, act);
   else
-    treefc_fwd_kernel<1><<<GATE_GRID(n, H, 1), 0, st>>>(z, bias, x, h, n, H, act);
+    launch(treefc_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, z, bias, x, h, n, H, act);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -345,9 +345,9 @@ int cavs_treefc_bwd(const float *dh_m, const float *dret, const float *h, float 
   hipStream_t st = as_stream(stream);
   long total = (long)n * H;
   if (total % 4 == 0 && all_aligned({dh_m, dret, h, dz}))
-    treefc_bwd_kernel<4><<<dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st>>>(dh_m, dret, h, dz, total, act);
+    launch(treefc_bwd_kernel<4>, dim3((unsigned)((total / 4 + 255) / 256)), dim3(256), 0, st, dh_m, dret, h, dz, total, act);
   else
-    treefc_bwd_kernel<1><<<dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st>>>(dh_m, dret, h, dz, total, act);
+    launch(treefc_bwd_kernel<1>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st, dh_m, dret, h, dz, total, act);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -378,9 +378,9 @@ static void launch_tile(const GemmArgs &g, int tA, int tB, bool vec, const GemmP
   dim3 grid((unsigned)p.tiles, p.splits), block(kThreads);
 #define CAVS_GEMM_CASE(TA, TB)                                                  \
   if (vec)                                                                      \
-    sgemm_mfma_kernel<BM, BN, BK, TA, TB, true><<<grid, block, 0, st>>>(g);      \
+    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, true>, grid, block, 0, st, g);      \
   else                                                                          \
-    sgemm_mfma_kernel<BM, BN, BK, TA, TB, false><<<grid, block, 0, st>>>(g)
+    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, false>, grid, block, 0, st, g)
   if (!tA && !tB) { CAVS_GEMM_CASE(false, false); }
   else if (!tA && tB) { CAVS_GEMM_CASE(false, true); }
   else if (tA && !tB) { CAVS_GEMM_CASE(true, false); }
@@ -406,10 +406,10 @@ static void launch_skinny(const GemmArgs &g, hipStream_t st) {
   constexpr int W = 8;
   if (g.M <= 32) {
     dim3 grid((g.N + 31) / 32, 1);
-    sgemm_skinny_kernel<1, TB, W><<<grid, W * 64, 0, st>>>(g);
+    launch(sgemm_skinny_kernel<1, TB, W>, grid, W * 64, 0, st, g);
   } else {
     dim3 grid((g.N + 31) / 32, (g.M + 63) / 64);
-    sgemm_skinny_kernel<2, TB, W><<<grid, W * 64, 0, st>>>(g);
+    launch(sgemm_skinny_kernel<2, TB, W>, grid, W * 64, 0, st, g);
   }
 }
 
@@ -439,7 +439,7 @@ static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float 
   CAVS_LAUNCH_CHECK();
   if (p.splits > 1) {
     long total = (long)M * N;
-    splitk_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, st>>>(g, p.splits);
+    launch(splitk_reduce_kernel, (unsigned)((total + 255) / 256), 256, 0, st, g, p.splits);
     CAVS_LAUNCH_CHECK();
   }
   return CAVS_OK;

@@ -231,7 +231,7 @@ int cavs_colsum(float *out, const float *inp, int ld, int n, int w, int accumula
     int rc = cavs_zero(out, (size_t)w * 4, stream);
     if (rc) return rc;
   }
-  colsum_kernel<<<dim3(strips, chunks), 256, 0, st>>>(out, inp, ld, n, w, rpc, chunks > 1, accumulate);
+  launch(colsum_kernel, dim3(strips, chunks), 256, 0, st, out, inp, ld, n, w, rpc, chunks > 1, accumulate);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -242,7 +242,7 @@ int cavs_embed_fwd(float *out, int ld_out, const float *ids, const float *table,
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(out && ids && table, "cavs_embed_fwd: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
-  embed_fwd_kernel<<<(n + 3) / 4, block, 0, as_stream(stream)>>>(out, ld_out, ids, table, n, E);
+  launch(embed_fwd_kernel, (n + 3) / 4, block, 0, as_stream(stream), out, ld_out, ids, table, n, E);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -253,7 +253,7 @@ int cavs_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, 
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dtable && ids && dy, "cavs_embed_bwd: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
-  embed_bwd_kernel<<<(n + kEmbedChunk - 1) / kEmbedChunk, block, 0, as_stream(stream)>>>(dtable, ids, dy, ld_dy, n, E);
+  launch(embed_bwd_kernel, (n + kEmbedChunk - 1) / kEmbedChunk, block, 0, as_stream(stream), dtable, ids, dy, ld_dy, n, E);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -263,7 +263,7 @@ int cavs_bias_add_rows(float *out, const float *inp, const float *bias, int n, i
   long total = (long)n * w;
   if (total == 0) return CAVS_OK;
   CAVS_REQUIRE(out && inp && bias, "cavs_bias_add_rows: null pointer");
-  bias_add_rows_kernel<<<(unsigned)((total + 255) / 256), 256, 0, as_stream(stream)>>>(out, inp, bias, total, w);
+  launch(bias_add_rows_kernel, (unsigned)((total + 255) / 256), 256, 0, as_stream(stream), out, inp, bias, total, w);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -273,7 +273,7 @@ int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const fl
   CAVS_REQUIRE(n >= 0 && C > 0, "cavs_softmax_xent: bad shape n=%d C=%d", n, C);
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(logits && labels, "cavs_softmax_xent: null pointer");
-  softmax_xent_kernel<<<(n + 3) / 4, 256, 0, as_stream(stream)>>>(loss, dlogits, logits, labels, n, C, 1.f / (float)n);
+  launch(softmax_xent_kernel, (n + 3) / 4, 256, 0, as_stream(stream), loss, dlogits, logits, labels, n, C, 1.f / (float)n);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -281,7 +281,7 @@ int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const fl
 int cavs_sgd(float *w, const float *g, float lr, size_t n, void *stream) {
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(w && g, "cavs_sgd: null pointer");
-  sgd_kernel<<<stream_grid(n), 256, 0, as_stream(stream)>>>(w, g, lr, n);
+  launch(sgd_kernel, stream_grid(n), 256, 0, as_stream(stream), w, g, lr, n);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -289,7 +289,7 @@ int cavs_sgd(float *w, const float *g, float lr, size_t n, void *stream) {
 int cavs_scale(float *out, const float *a, float s, size_t n, void *stream) {
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(out && a, "cavs_scale: null pointer");
-  scale_kernel<<<stream_grid(n), 256, 0, as_stream(stream)>>>(out, a, s, n);
+  launch(scale_kernel, stream_grid(n), 256, 0, as_stream(stream), out, a, s, n);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -300,7 +300,7 @@ int cavs_ew_binary(int op, float *out, const float *a, size_t na, const float *b
   CAVS_REQUIRE(out && a && b && na > 0 && nb > 0 && na <= n && nb <= n, "cavs_ew_binary: bad operands (na=%zu nb=%zu n=%zu)", na, nb, n);
   hipStream_t st = as_stream(stream);
   unsigned grid = stream_grid(n);
-#define CAVS_EWB(OP) case OP: ew_binary_kernel<OP><<<grid, 256, 0, st>>>(out, a, na, b, nb, n, accumulate); break
+#define CAVS_EWB(OP) case OP: launch(ew_binary_kernel<OP>, grid, 256, 0, st, out, a, na, b, nb, n, accumulate); break
   switch (op) {
     CAVS_EWB(CAVS_EW_ADD); CAVS_EWB(CAVS_EW_SUB); CAVS_EWB(CAVS_EW_MUL); CAVS_EWB(CAVS_EW_DIV);
     CAVS_EWB(CAVS_EW_SIGMOID_GRAD); CAVS_EWB(CAVS_EW_TANH_GRAD); CAVS_EWB(CAVS_EW_RELU_GRAD);
@@ -317,7 +317,7 @@ int cavs_ew_unary(int op, float *out, const float *a, size_t n, int accumulate, 
   CAVS_REQUIRE(out && a, "cavs_ew_unary: null pointer");
   hipStream_t st = as_stream(stream);
   unsigned grid = stream_grid(n);
-#define CAVS_EWU(OP) case OP: ew_unary_kernel<OP><<<grid, 256, 0, st>>>(out, a, n, accumulate); break
+#define CAVS_EWU(OP) case OP: launch(ew_unary_kernel<OP>, grid, 256, 0, st, out, a, n, accumulate); break
   switch (op) {
     CAVS_EWU(CAVS_EW_ASSIGN); CAVS_EWU(CAVS_EW_NEG); CAVS_EWU(CAVS_EW_ABS); CAVS_EWU(CAVS_EW_SQUARE);
     CAVS_EWU(CAVS_EW_SIGMOID); CAVS_EWU(CAVS_EW_TANH); CAVS_EWU(CAVS_EW_RELU);

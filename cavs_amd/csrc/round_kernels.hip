@@ -517,10 +517,10 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   const RoundPlan p = plan_round(n);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.waves == 4) treelstm_round_fwd_kernel<16, 4><<<grid, 256, 0, st>>>(a);
-  else if (p.tile == 16) treelstm_round_fwd_kernel<16, 8><<<grid, 512, 0, st>>>(a);
-  else if (p.waves == 4) treelstm_round_fwd_kernel<32, 4><<<grid, 256, 0, st>>>(a);
-  else treelstm_round_fwd_kernel<32, 8><<<grid, 512, 0, st>>>(a);
+  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_fwd_kernel<16, 4>, grid, 256, 0, st, a);
+  else if (p.tile == 16) launch(treelstm_round_fwd_kernel<16, 8>, grid, 512, 0, st, a);
+  else if (p.waves == 4) launch(treelstm_round_fwd_kernel<32, 4>, grid, 256, 0, st, a);
+  else launch(treelstm_round_fwd_kernel<32, 8>, grid, 512, 0, st, a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -539,10 +539,10 @@ int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *chil
                    aligned16(dxW) && (!G || aligned16(G)) && (!dF || aligned16(dF));
   if (vec) {
     long total = (long)n * (H / 4);
-    treelstm_round_bwd_gates_kernel<4><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a);
+    launch(treelstm_round_bwd_gates_kernel<4>, (unsigned)((total + 255) / 256), 256, 0, st, a);
   } else {
     long total = (long)n * H;
-    treelstm_round_bwd_gates_kernel<1><<<(unsigned)((total + 255) / 256), 256, 0, st>>>(a);
+    launch(treelstm_round_bwd_gates_kernel<1>, (unsigned)((total + 255) / 256), 256, 0, st, a);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
@@ -559,10 +559,10 @@ int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *
   const RoundPlan p = plan_round(n);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.waves == 4) treelstm_round_bwd_children_kernel<16, 4><<<grid, 256, 0, st>>>(a);
-  else if (p.tile == 16) treelstm_round_bwd_children_kernel<16, 8><<<grid, 512, 0, st>>>(a);
-  else if (p.waves == 4) treelstm_round_bwd_children_kernel<32, 4><<<grid, 256, 0, st>>>(a);
-  else treelstm_round_bwd_children_kernel<32, 8><<<grid, 512, 0, st>>>(a);
+  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4>, grid, 256, 0, st, a);
+  else if (p.tile == 16) launch(treelstm_round_bwd_children_kernel<16, 8>, grid, 512, 0, st, a);
+  else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<32, 4>, grid, 256, 0, st, a);
+  else launch(treelstm_round_bwd_children_kernel<32, 8>, grid, 512, 0, st, a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -572,7 +572,7 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
   if (rows == 0 || cols == 0) return CAVS_OK;
   CAVS_REQUIRE(out && in && out != in, "cavs_transpose: null or aliased pointer");
   dim3 grid((cols + 31) / 32, (rows + 31) / 32);
-  transpose_kernel<<<grid, 256, 0, as_stream(stream)>>>(out, in, rows, cols);
+  launch(transpose_kernel, grid, 256, 0, as_stream(stream), out, in, rows, cols);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

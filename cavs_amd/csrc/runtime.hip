@@ -16,6 +16,11 @@ int set_error(int code, const char *fmt, ...) {
   return code;
 }
 
+LaunchProbe &launch_probe() {
+  static thread_local LaunchProbe probe;
+  return probe;
+}
+
 int num_cus() {
   if (g_cus == 0) {
     int dev = 0;
@@ -46,17 +51,17 @@ static int fill_impl(float *ptr, float value, size_t n, hipStream_t st) {
   // align to 16 bytes, then vector stores, then the tail
   while (head < n && !aligned16(ptr + head)) head++;
   if (head) {
-    fill_kernel<<<1, 64, 0, st>>>(ptr, value, head);
+    launch(fill_kernel, 1, 64, 0, st, ptr, value, head);
   }
   size_t n4 = (n - head) / 4;
   if (n4) {
     size_t blocks = (n4 + 255) / 256;
     size_t cap = (size_t)num_cus() * 8;
-    fill4_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, st>>>(
+    launch(fill4_kernel, (unsigned)(blocks < cap ? blocks : cap), 256, 0, st, 
         reinterpret_cast<float4 *>(ptr + head), value, n4);
   }
   size_t done = head + n4 * 4;
-  if (done < n) fill_kernel<<<1, 64, 0, st>>>(ptr + done, value, n - done);
+  if (done < n) launch(fill_kernel, 1, 64, 0, st, ptr + done, value, n - done);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -196,6 +201,23 @@ int cavs_event_elapsed_ms(float *ms, void *start, void *stop) {
   CAVS_REQUIRE(ms && start && stop, "cavs_event_elapsed_ms: null argument");
   CAVS_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
   CAVS_HIP_TRY(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return CAVS_OK;
+}
+
+int cavs_profile_arm(void *start_event, void *stop_event) {
+  CAVS_REQUIRE(start_event && stop_event, "cavs_profile_arm: null event");
+  LaunchProbe &p = launch_probe();
+  p.start = static_cast<hipEvent_t>(start_event);
+  p.stop = static_cast<hipEvent_t>(stop_event);
+  p.armed = true;
+  p.started = false;
+  return CAVS_OK;
+}
+
+int cavs_profile_disarm(int *launched) {
+  LaunchProbe &p = launch_probe();
+  if (launched) *launched = p.armed && p.started;
+  p = LaunchProbe{};
   return CAVS_OK;
 }
 

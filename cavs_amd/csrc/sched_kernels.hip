@@ -153,12 +153,12 @@ int cavs_schedule_frontier(const int *parent, int N, int *tids_to_jobids, int *j
   int *nchild = scratch, *cmin = scratch + N, *cmax = scratch + 2 * (size_t)N,
       *level = scratch + 3 * (size_t)N;
   if (N > 0) {
-    sched_init_kernel<<<(N + 255) / 256, 256, 0, st>>>(N, nchild, cmin, cmax, level);
+    launch(sched_init_kernel, (N + 255) / 256, 256, 0, st, N, nchild, cmin, cmax, level);
     CAVS_LAUNCH_CHECK();
-    sched_children_kernel<<<(N + 255) / 256, 256, 0, st>>>(parent, N, nchild, cmin, cmax);
+    launch(sched_children_kernel, (N + 255) / 256, 256, 0, st, parent, N, nchild, cmin, cmax);
     CAVS_LAUNCH_CHECK();
   }
-  sched_frontier_kernel<<<1, kSchedThreads, 0, st>>>(parent, N, nchild, cmin, cmax, tids_to_jobids,
+  launch(sched_frontier_kernel, 1, kSchedThreads, 0, st, parent, N, nchild, cmin, cmax, tids_to_jobids,
                                                     jobids_to_tids, level, round_of_tid,
                                                     round2offset, n_rounds);
   CAVS_LAUNCH_CHECK();

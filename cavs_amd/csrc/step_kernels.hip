@@ -273,9 +273,9 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
   const int q = head_q(H);
 #define CAVS_HEAD(CC)                                                                                              \
   case CC:                                                                                                         \
-    if (q == 4) fc_xent_kernel<CC, 4><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n);       \
-    else if (q == 8) fc_xent_kernel<CC, 8><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n);  \
-    else fc_xent_kernel<(CC <= 4 ? CC : 1), 16><<<blocks, 256, lds, st>>>(X, W, b, labels, loss, logits, dX, part, n, H, inv_n); \
+    if (q == 4) launch(fc_xent_kernel<CC, 4>, blocks, 256, lds, st, X, W, b, labels, loss, logits, dX, part, n, H, inv_n);       \
+    else if (q == 8) launch(fc_xent_kernel<CC, 8>, blocks, 256, lds, st, X, W, b, labels, loss, logits, dX, part, n, H, inv_n);  \
+    else launch(fc_xent_kernel<(CC > 4 ? 1 : CC), 16>, blocks, 256, lds, st, X, W, b, labels, loss, logits, dX, part, n, H, inv_n); \
     break
   switch (C) {
     CAVS_HEAD(1); CAVS_HEAD(2); CAVS_HEAD(3); CAVS_HEAD(4); CAVS_HEAD(5); CAVS_HEAD(6); CAVS_HEAD(7); CAVS_HEAD(8);
@@ -284,7 +284,7 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
   CAVS_LAUNCH_CHECK();
   if (grad) {
     const int total = C * H + C;
-    fc_xent_reduce_kernel<<<(total + 63) / 64, 256, 0, st>>>(part, blocks, total, C * H, dW, db);
+    launch(fc_xent_reduce_kernel, (total + 63) / 64, 256, 0, st, part, blocks, total, C * H, dW, db);
     CAVS_LAUNCH_CHECK();
   }
   return CAVS_OK;
@@ -309,7 +309,7 @@ int cavs_sgd_multi(int count, float *const *w, const float *const *g, const size
     if (k == 0) continue;
     t.count = k;
     size_t blocks = (run + 255) / 256, cap = (size_t)num_cus() * 16;
-    sgd_multi_kernel<<<(unsigned)(blocks < cap ? blocks : cap), 256, 0, st>>>(t, lr);
+    launch(sgd_multi_kernel, (unsigned)(blocks < cap ? blocks : cap), 256, 0, st, t, lr);
     CAVS_LAUNCH_CHECK();
   }
   return CAVS_OK;
@@ -321,7 +321,7 @@ int cavs_embed_sgd(float *table, const float *dtable, const float *ids, int n, i
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(table && dtable && ids && stamp, "cavs_embed_sgd: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
-  embed_sgd_kernel<<<(n + kSgdChunk - 1) / kSgdChunk, block, 0, as_stream(stream)>>>(table, dtable, ids, n, E, lr, stamp, epoch);
+  launch(embed_sgd_kernel, (n + kSgdChunk - 1) / kSgdChunk, block, 0, as_stream(stream), table, dtable, ids, n, E, lr, stamp, epoch);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -331,7 +331,7 @@ int cavs_embed_zero_rows(float *dtable, const float *ids, int n, int E, void *st
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dtable && ids, "cavs_embed_zero_rows: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
-  embed_zero_rows_kernel<<<n, block, 0, as_stream(stream)>>>(dtable, ids, E);
+  launch(embed_zero_rows_kernel, n, block, 0, as_stream(stream), dtable, ids, E);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -361,9 +361,9 @@ int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int 
   const int rpc = ((n + chunks - 1) / chunks + 3) / 4 * 4;
   hipStream_t st = as_stream(stream);
   float *part = static_cast<float *>(workspace);
-  colsum_part_kernel<<<dim3((w + 63) / 64, chunks), 256, 0, st>>>(part, inp, ld, n, w, rpc);
+  launch(colsum_part_kernel, dim3((w + 63) / 64, chunks), 256, 0, st, part, inp, ld, n, w, rpc);
   CAVS_LAUNCH_CHECK();
-  colsum_blocks_reduce_kernel<<<(w + 63) / 64, 256, 0, st>>>(out, part, chunks, w, bw, map);
+  launch(colsum_blocks_reduce_kernel, (w + 63) / 64, 256, 0, st, out, part, chunks, w, bw, map);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

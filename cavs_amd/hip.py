@@ -71,6 +71,8 @@ _SIGS = {
     "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
+    "cavs_profile_arm": [_P, _P],
+    "cavs_profile_disarm": [_P],
     "cavs_fc_softmax_xent": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _P],
     "cavs_sgd_multi": [_I, _P, _P, _P, _F, _P],
     "cavs_embed_sgd": [_P, _P, _P, _I, _I, _F, _P, _I, _P],

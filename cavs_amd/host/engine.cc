@@ -127,12 +127,13 @@ Engine::ProfScope::ProfScope(Engine *eng, int cls) : e(eng), s{cls, nullptr, nul
   if (!on) return;
   s.a = e->prof_event();
   s.b = e->prof_event();
-  check(cavs_event_record(s.a, e->stream_));
+  check(cavs_profile_arm(s.a, s.b));
 }
 
 Engine::ProfScope::~ProfScope() {
   if (!on) return;
-  if (cavs_event_record(s.b, e->stream_) == CAVS_OK) e->spans_.push_back(s);
+  int launched = 0;
+  if (cavs_profile_disarm(&launched) == CAVS_OK && launched) e->spans_.push_back(s);
 }
 
 void Engine::profile_enable(bool on) {

@@ -90,7 +90,7 @@ class Engine {
     int cls;
     void *a, *b;
   };
-  struct ProfScope {  // brackets the launches made during its lifetime
+  struct ProfScope {  // times the kernels launched during its lifetime (cavs_profile_arm)
     Engine *e;
     Span s;
     bool on;

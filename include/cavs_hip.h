@@ -63,7 +63,15 @@ int cavs_event_create(void **event);
 int cavs_event_destroy(void *event);
 int cavs_event_record(void *event, void *stream);
 int cavs_event_sync(void *event); /* host waits until the event has happened */
-int cavs_event_elapsed_ms(float *ms, void *start, void *stop); /* waits for `stop` */
+int cavs_event_elapsed_ms(float *ms, void *start, void *stop);
+/* Kernel timing without brackets of its own on the stream: while the calling thread is armed,
+ * the first kernel an entry point launches stamps `start` when it begins executing and every
+ * kernel stamps `stop` when it ends, so cavs_event_elapsed_ms(start, stop) is the device time
+ * of that entry point's kernels (the interval a kernel trace reports), not launch gaps.
+ * cavs_profile_disarm tells whether anything was launched in between.  No counterpart in the
+ * reference (it times whole statements on the host, cavs/midend/statement.cc:53-84). */
+int cavs_profile_arm(void *start_event, void *stop_event);
+int cavs_profile_disarm(int *launched); /* waits for `stop` */
 
 /* ------------------------------------------------------------------ graph ops
  * Replace GraphGatherOp / GraphScatterOp / GraphPushOp / GraphPullOp /

@@ -90,9 +90,9 @@ int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int w
  * host-side split "HostSchedule" (scheduler), "HostWait" (waiting for the device to release
  * an index staging buffer), "HostStep" (the whole enqueueing call). */
 int cavs_session_timing(cavs_session *s, const char *name, float *ms);
-/* Device time per kernel class.  While enabled, every launch of the session is
- * bracketed by a pair of events on the session's stream; profile_read waits for the
- * stream and returns the summed elapsed time and launch count since profiling was
+/* Device time per kernel class.  While enabled, every entry point the session calls has its
+ * kernels stamp a pair of events at their own begin and end (cavs_profile_arm); profile_read
+ * waits for the stream and returns the summed kernel time and call count since profiling was
  * enabled.  Classes: "gemm" "gather" "scatter" "gates" "round" (fused rounds) "other". */
 int cavs_session_profile(cavs_session *s, int enable);
 int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double *total_ms,
