@@ -99,6 +99,8 @@ struct RoundFwdArgs {
   float *gates;        // [n, 6H]
   float *msg;          // [n, 2H]
   float *pool_out;     // same buffer as pool: rows of this round are written, rows of earlier rounds read
+  float *go;           // [*, H] or nullptr: the pushed return value h of slab row b goes to row out_rows[b]
+  const int *out_rows; // [n] (FunctionPopRet folded in)
   int n, H;
 };
 
@@ -119,21 +121,22 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
   const long H2 = 2L * H, H3 = 3L * H;
   const int j0 = blockIdx.x * TILE;
   const int row = (blockIdx.y * RT + rt) * TILE + x;
+  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
+  const int kb = ks * kper, ke = min(H, kb + kper);
+  const float *Uio = a.U + j0 + x, *Uf = a.U + H3 * H + j0 + x;
+
+  // Issue order of the prologue: (1) every row id this thread needs, (2) what does not depend
+  // on them -- the first B fragments and the x*W / bias operands of the epilogue -- so that it
+  // travels while the ids do, (3) the rows the ids name.
   int cl = -1, cr = -1;
   if (row < a.n) {
     cl = a.child[2 * row];
     cr = a.child[2 * row + 1];
   }
-  const float *pl = a.pool + (cl >= 0 ? cl : 0) * H2, *pr = a.pool + (cr >= 0 ? cr : 0) * H2;
-  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
-  const int kb = ks * kper, ke = min(H, kb + kper);
-  const float *Uio = a.U + j0 + x, *Uf = a.U + H3 * H + j0 + x;
-
-  // operands of the epilogue, fetched now so that their latency hides behind the products
   constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
   struct Epi {
     bool on;
-    int b, j, dst, lds;
+    int b, j, dst, lds, c_l, c_r, out;
     float xw[4], bias[4], hl, cl, hr, cr;
   } epi[EPT];
 #pragma unroll
@@ -145,16 +148,12 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
     ep.j = j0 + (l2 & (TILE - 1));
     ep.lds = (t * NP * NR + r) * 64 + l2;
     ep.on = e < RT * NR * 64 && ep.b < a.n;
-    ep.hl = ep.cl = ep.hr = ep.cr = 0.f;
-    ep.dst = -1;
+    ep.c_l = ep.c_r = ep.dst = ep.out = -1;
     if (ep.on) {
-      const int c_l = a.child[2 * ep.b], c_r = a.child[2 * ep.b + 1];
+      ep.c_l = a.child[2 * ep.b];
+      ep.c_r = a.child[2 * ep.b + 1];
       ep.dst = a.pair[ep.b];
-      if (c_l >= 0) { ep.hl = a.pool[c_l * H2 + ep.j]; ep.cl = a.pool[c_l * H2 + H + ep.j]; }
-      if (c_r >= 0) { ep.hr = a.pool[c_r * H2 + ep.j]; ep.cr = a.pool[c_r * H2 + H + ep.j]; }
-      const float *xw = a.xW + ep.b * a.ld_xw + ep.j;
-#pragma unroll
-      for (int k = 0; k < 4; k++) { ep.xw[k] = xw[k * H]; ep.bias[k] = a.bias[k * H + ep.j]; }
+      if (a.go) ep.out = a.out_rows[ep.b];
     }
   }
 
@@ -168,13 +167,11 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
     float4 hl[UG], hr[UG];
     float b[UG][4][4];
   };
-  auto fetch = [&](int k0, Frag &f) {
+  auto fetch_b = [&](int k0, Frag &f) {
 #pragma unroll
     for (int u = 0; u < UG; u++) {
       const int kk = k0 + GK * u + 4 * slot;
-      const bool kin = kk < ke;  // H is a multiple of 4: a float4 is wholly in or out
-      f.hl[u] = (kin && cl >= 0) ? ld4(pl + kk) : zero4();
-      f.hr[u] = (kin && cr >= 0) ? ld4(pr + kk) : zero4();
+      const bool kin = kk < ke;  // H is a multiple of 4: a group of 4 k is wholly in or out
 #pragma unroll
       for (int c = 0; c < 4; c++) {
         const float *ui = Uio + (long)(kin ? kk + c : 0) * H3;
@@ -184,6 +181,20 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
         f.b[u][3][c] = kin ? Uf[(long)(kk + c) * H] : 0.f;
       }
     }
+  };
+  const float *pl = nullptr, *pr = nullptr;
+  auto fetch_a = [&](int k0, Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+      const int kk = k0 + GK * u + 4 * slot;
+      const bool kin = kk < ke;
+      f.hl[u] = (kin && cl >= 0) ? ld4(pl + kk) : zero4();
+      f.hr[u] = (kin && cr >= 0) ? ld4(pr + kk) : zero4();
+    }
+  };
+  auto fetch = [&](int k0, Frag &f) {
+    fetch_b(k0, f);
+    fetch_a(k0, f);
   };
   auto multiply = [&](const Frag &f) {
 #pragma unroll
@@ -200,7 +211,26 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
   };
   Frag f0, f1;
   constexpr int S = GK * UG;
-  if (kb < ke) fetch(kb, f0);
+  if (kb < ke) fetch_b(kb, f0);
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    Epi &ep = epi[q];
+    if (!ep.on) continue;
+    const float *xw = a.xW + ep.b * a.ld_xw + ep.j;
+#pragma unroll
+    for (int k = 0; k < 4; k++) { ep.xw[k] = xw[k * H]; ep.bias[k] = a.bias[k * H + ep.j]; }
+  }
+  pl = a.pool + (cl >= 0 ? cl : 0) * H2;
+  pr = a.pool + (cr >= 0 ? cr : 0) * H2;
+  if (kb < ke) fetch_a(kb, f0);
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    Epi &ep = epi[q];
+    ep.hl = ep.cl = ep.hr = ep.cr = 0.f;
+    if (ep.c_l >= 0) { ep.hl = a.pool[ep.c_l * H2 + ep.j]; ep.cl = a.pool[ep.c_l * H2 + H + ep.j]; }
+    if (ep.c_r >= 0) { ep.hr = a.pool[ep.c_r * H2 + ep.j]; ep.cr = a.pool[ep.c_r * H2 + H + ep.j]; }
+  }
+
   for (int k0 = kb; k0 < ke; k0 += 2 * S) {
     if (k0 + S < ke) fetch(k0 + S, f1);
     multiply(f0);
@@ -245,10 +275,61 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwd
       a.pool_out[ep.dst * H2 + j] = h;
       a.pool_out[ep.dst * H2 + H + j] = c;
     }
+    if (ep.out >= 0) a.go[(long)ep.out * H + j] = h;
     float *gl = a.G + (2L * b) * H2 + j, *gr = gl + H2;
     gl[0] = ep.hl; gl[H] = ep.cl; gr[0] = ep.hr; gr[H] = ep.cr;
     a.hlr[(long)b * H + j] = ep.hl + ep.hr;
   }
+}
+
+// ------------------------------------------------------------------ forward, a round of leaves
+// No children: the gates of x*W + bias only, the message written to the pool row the scatter
+// list names and the return value to its output row.
+struct RoundLeavesArgs {
+  const float *xW;
+  long ld_xw;
+  const float *bias;
+  const int *pair;
+  float *gates, *msg, *pool, *go;
+  const int *out_rows;
+  int n, H;
+};
+
+template <int W>
+__global__ void treelstm_round_leaves_fwd_kernel(RoundLeavesArgs a) {
+  const int H = a.H, hw = H / W;
+  const long H2 = 2L * H;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int dst = a.pair[r], out = a.go ? a.out_rows[r] : -1;
+  const float *xw = a.xW + r * a.ld_xw + j;
+  float gi[W], go[W], gu[W], gf[W], gtc[W], mh[W], mc[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    // same association as with children: (x*W + 0) + bias
+    const float i = sigm_r((xw[k] + 0.f) + a.bias[j + k]);
+    const float o = sigm_r((xw[H + k] + 0.f) + a.bias[3 * H + j + k]);
+    const float u = tanhf((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
+    const float f = sigm_r((xw[3 * H + k] + 0.f) + a.bias[H + j + k]);
+    const float c = (i * u + f * 0.f) + f * 0.f;
+    const float tc = tanhf(c);
+    gi[k] = i; go[k] = o; gu[k] = u; gf[k] = f; gtc[k] = tc; mh[k] = o * tc; mc[k] = c;
+  }
+  auto st = [](float *p, const float (&v)[W]) {
+    if constexpr (W == 4) {
+      *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+#pragma unroll
+      for (int k = 0; k < W; k++) p[k] = v[k];
+    }
+  };
+  float *g = a.gates + (long)r * 6 * H + j;
+  st(g, gi); st(g + H, go); st(g + 2 * H, gu); st(g + 3 * H, gf); st(g + 4 * H, gf); st(g + 5 * H, gtc);
+  float *m = a.msg + r * H2 + j;
+  st(m, mh); st(m + H, mc);
+  if (dst >= 0) { st(a.pool + dst * H2 + j, mh); st(a.pool + dst * H2 + H + j, mc); }
+  if (out >= 0) st(a.go + (long)out * H + j, mh);
 }
 
 // ------------------------------------------------------------------ backward, gate part
@@ -259,7 +340,8 @@ struct RoundBwdGatesArgs {
   const float *dpool;   // [*, 2H] gradient of the message pool
   const int *pair;      // [n]
   const int *child;     // [2n] or nullptr for a round of leaves
-  const float *dret;    // [n, H] gradient of the pushed return value
+  const float *dret;    // gradient of the pushed return value: row b, or row dret_rows[b] if given
+  const int *dret_rows; // [n] or nullptr (grad of FunctionPopRet folded in)
   const float *gates;   // [n, 6H]
   const float *G;       // [2n, 2H] or nullptr for leaves
   float *dxW;           // [n, 4H] (ld_dxw) blocks [i|o|u|f_l+f_r]
@@ -277,6 +359,7 @@ __global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
   if (idx >= (long)a.n * hw) return;
   const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
   const int src = a.pair[r];
+  const int dr_row = a.dret_rows ? a.dret_rows[r] : r;
   const float *g = a.gates + (long)r * 6 * H + j;
   const bool internal = a.child != nullptr;
   int c_l = -1, c_r = -1;
@@ -285,14 +368,14 @@ __global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
   if constexpr (W == 4) {
     auto ld = [](const float *p, float (&o)[W]) { float4 v = ld4(p); o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; };
     ld(g, gi); ld(g + H, go); ld(g + 2 * H, gu); ld(g + 3 * H, gfl); ld(g + 4 * H, gfr); ld(g + 5 * H, gtc);
-    ld(a.dret + (long)r * H + j, dr);
+    ld(a.dret + (long)dr_row * H + j, dr);
     if (src >= 0) { ld(a.dpool + src * H2 + j, dmh); ld(a.dpool + src * H2 + H + j, dmc); }
     if (internal) { ld(a.G + (2L * r) * H2 + H + j, cl); ld(a.G + (2L * r + 1) * H2 + H + j, cr); }
   } else {
 #pragma unroll
     for (int k = 0; k < W; k++) {
       gi[k] = g[k]; go[k] = g[H + k]; gu[k] = g[2 * H + k]; gfl[k] = g[3 * H + k]; gfr[k] = g[4 * H + k]; gtc[k] = g[5 * H + k];
-      dr[k] = a.dret[(long)r * H + j + k];
+      dr[k] = a.dret[(long)dr_row * H + j + k];
       if (src >= 0) { dmh[k] = a.dpool[src * H2 + j + k]; dmc[k] = a.dpool[src * H2 + H + j + k]; }
       if (internal) { cl[k] = a.G[(2L * r) * H2 + H + j + k]; cr[k] = a.G[(2L * r + 1) * H2 + H + j + k]; }
     }
@@ -368,6 +451,25 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel
   const float *px = a.dxW + (rin ? row : 0) * a.ld_dxw;
   const float *pfl = a.dF + (rin ? 2L * row : 0) * H, *pfr = pfl + (rin ? H : 0);
   const float *UTio = a.UT + j0 + x, *UTf = a.UT + 3L * H * H + j0 + x;
+
+  // the epilogue's targets, fetched now: child rows of the elements this thread will write
+  constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
+  bool eon[EPT];
+  int ecl[EPT], ecr[EPT], ej[EPT], elds[EPT];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    const int e = tid + q * kRoundThreads;
+    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
+    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2);
+    ej[q] = j0 + (l2 & (TILE - 1));
+    elds[q] = (t * NP * NR + r) * 64 + l2;
+    eon[q] = e < RT * NR * 64 && b < a.n;
+    ecl[q] = ecr[q] = -1;
+    if (eon[q]) {
+      ecl[q] = a.child[2 * b];
+      ecr[q] = a.child[2 * b + 1];
+    }
+  }
 
   Acc acc[NP];
 #pragma unroll
@@ -453,11 +555,10 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel
 
   park_partials<TILE, NP, KS, NREG, RT>(red, acc, rt, ks, lane);
 
-  for (int e = tid; e < RT * NR * 64; e += kRoundThreads) {
-    const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
-    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2), j = j0 + (l2 & (TILE - 1));
-    if (b >= a.n) continue;
-    const float *pre = red + (t * NP * NR + r) * 64 + l2;
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    if (!eon[q]) continue;
+    const float *pre = red + elds[q];
     float v[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
@@ -466,9 +567,8 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel
       for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
       v[p] = s;
     }
-    const int c_l = a.child[2 * b], c_r = a.child[2 * b + 1];
-    if (c_l >= 0) a.dpool[c_l * H2 + j] = v[0] + v[1];
-    if (c_r >= 0) a.dpool[c_r * H2 + j] = v[0] + v[2];
+    if (ecl[q] >= 0) a.dpool[ecl[q] * H2 + ej[q]] = v[0] + v[1];
+    if (ecr[q] >= 0) a.dpool[ecr[q] * H2 + ej[q]] = v[0] + v[2];
   }
 }
 
@@ -507,13 +607,14 @@ extern "C" {
 
 int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
                             const float *U, const float *bias, float *G, float *hlr, float *gates,
-                            float *msg, int n, int H, void *stream) {
+                            float *msg, float *graph_out, const int *out_rows, int n, int H, void *stream) {
   CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && ld_xw >= 4 * H && ld_xw % 4 == 0,
                "cavs_treelstm_round_fwd: bad shape n=%d H=%d ld_xw=%d (H must be a multiple of 32)", n, H, ld_xw);
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(pool && child && pair && xW && U && bias && G && hlr && gates && msg, "cavs_treelstm_round_fwd: null pointer");
   CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
-  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, n, H};
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd: graph_out needs out_rows");
+  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
   const RoundPlan p = plan_round(n);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
@@ -525,15 +626,37 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   return CAVS_OK;
 }
 
+int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw, const float *bias,
+                                   float *gates, float *msg, float *graph_out, const int *out_rows, int n, int H,
+                                   void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && ld_xw >= 4 * H, "cavs_treelstm_round_leaves_fwd: bad shape n=%d H=%d ld=%d", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && pair && xW && bias && gates && msg, "cavs_treelstm_round_leaves_fwd: null pointer");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_leaves_fwd: graph_out needs out_rows");
+  RoundLeavesArgs a{xW, ld_xw, bias, pair, gates, msg, pool, graph_out, out_rows, n, H};
+  hipStream_t st = as_stream(stream);
+  const bool vec = H % 4 == 0 && ld_xw % 4 == 0 && aligned16(pool) && aligned16(xW) && aligned16(bias) && aligned16(gates) &&
+                   aligned16(msg) && (!graph_out || aligned16(graph_out));
+  if (vec) {
+    long total = (long)n * (H / 4);
+    launch(treelstm_round_leaves_fwd_kernel<4>, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  } else {
+    long total = (long)n * H;
+    launch(treelstm_round_leaves_fwd_kernel<1>, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
 int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret,
-                                  const float *gates, const float *G, float *dxW, int ld_dxw, float *dF,
-                                  int n, int H, void *stream) {
+                                  const int *dret_rows, const float *gates, const float *G, float *dxW,
+                                  int ld_dxw, float *dF, int n, int H, void *stream) {
   CAVS_REQUIRE(n >= 0 && H > 0 && ld_dxw >= 4 * H, "cavs_treelstm_round_bwd_gates: bad shape n=%d H=%d ld=%d", n, H, ld_dxw);
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dpool && pair && dret && gates && dxW, "cavs_treelstm_round_bwd_gates: null pointer");
   CAVS_REQUIRE((child && G && dF) || (!child && !G && !dF),
                "cavs_treelstm_round_bwd_gates: child, G and dF must be all set (internal round) or all null (leaves)");
-  RoundBwdGatesArgs a{dpool, pair, child, dret, gates, G, dxW, ld_dxw, dF, dpool, n, H};
+  RoundBwdGatesArgs a{dpool, pair, child, dret, dret_rows, gates, G, dxW, ld_dxw, dF, dpool, n, H};
   hipStream_t st = as_stream(stream);
   const bool vec = H % 4 == 0 && ld_dxw % 4 == 0 && aligned16(dpool) && aligned16(dret) && aligned16(gates) &&
                    aligned16(dxW) && (!G || aligned16(G)) && (!dF || aligned16(dF));

@@ -67,8 +67,9 @@ _SIGS = {
     "cavs_lstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treefc_fwd": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treefc_bwd": [_P, _P, _P, _P, _I, _I, _I, _P],
-    "cavs_treelstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P],
-    "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
+    "cavs_treelstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_profile_arm": [_P, _P],

@@ -351,12 +351,14 @@ void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_de
   if ((cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x) && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
   d_x_ = x_dev;
   check(cavs_event_record(ev_[0], stream_));
+  fwd_out_ = graph_out ? graph_out : GO_.get();
+  out_folded_ = false;
   switch (cfg_.model) {
     case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
     case CAVS_MODEL_LSTM: lstm_forward(); break;
     default: treefc_forward();
   }
-  pop_ret(graph_out ? graph_out : GO_.get());
+  pop_ret(fwd_out_);
   check(cavs_event_record(ev_[1], stream_));
   ev_valid_ = true;
   ev_bwd_valid_ = false;
@@ -408,6 +410,8 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
   }
 
   check(cavs_event_record(ev_[0], stream_));
+  fwd_out_ = GO_.get();
+  out_folded_ = false;
   switch (cfg_.model) {
     case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
     case CAVS_MODEL_LSTM: lstm_forward(); break;
@@ -459,7 +463,10 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
 
 // FunctionPopRet (cavs/backend/op_impl_graphop.cu:304-318): GraphOutput[tids_to_jobids[t]] =
 // ret[t].  Push's slab copy is folded in: the h half of the message slab is the return value.
-void Engine::pop_ret(float *graph_out) { scatter(graph_out, cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H); }
+void Engine::pop_ret(float *graph_out) {
+  if (out_folded_) return;  // already written by the rounds
+  scatter(graph_out, cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H);
+}
 
 // ------------------------------------------------------------------ Tree-LSTM
 // apps/paper/tree-lstm-cavs.cc:129-172.  Everything that does not depend on the children
@@ -487,17 +494,26 @@ void Engine::treelstm_forward() {
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
   }
   const int fused = fused_rows();
+  // when every round runs fused, Push + FunctionPopRet ride along in the rounds' epilogues
+  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  float *go = out_folded_ ? fwd_out_ : nullptr;
   for (const Round &r : sched_.rounds) {
     const size_t off = r.offset;
     float *msg = msg_.at(off * 2 * H);
-    if (leaf_round(r)) {
+    if (leaf_round(r) && r.n <= fused) {
+      CAVS_TIMED(K_GATES, cavs_treelstm_round_leaves_fwd(pool_.get(), d_pair_ + off, xW_.at(off * 4 * H), 4 * H, Bv, gates_.at(off * 6 * H),
+                                                         msg, go, d_t2j_ + off, r.n, H, stream_));
+      c_scatter_rows_ += r.n;
+      c_launches_ += 1;
+      continue;
+    } else if (leaf_round(r)) {
       CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, nullptr, nullptr, nullptr, Bv,
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
     } else if (r.n <= fused) {
       // Gather, both recurrent products, the gates and Scatter in one launch
       CAVS_TIMED(K_ROUND, cavs_treelstm_round_fwd(pool_.get(), d_child_ + 2 * off, d_pair_ + off, xW_.at(off * 4 * H), 4 * H, U, Bv,
-                                                  G_.at(2 * off * 2 * H), hlr_.at(off * H), gates_.at(off * 6 * H), msg, r.n, H,
-                                                  stream_));
+                                                  G_.at(2 * off * 2 * H), hlr_.at(off * H), gates_.at(off * 6 * H), msg, go,
+                                                  d_t2j_ + off, r.n, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
       c_gather_rows_ += 2.0 * r.n;
       c_scatter_rows_ += r.n;
@@ -525,9 +541,11 @@ void Engine::treelstm_forward() {
 void Engine::treelstm_backward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w;
-  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);  // grad of Push is Pull
-  if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   const int fused = fused_rows();
+  // grad of Push is Pull: read through the list by the fused gate kernels, or gathered up front
+  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
     CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), U, H, 3 * H, stream_));
     CAVS_TIMED(K_OTHER, cavs_transpose(UT_.at((size_t)3 * H * H), U + (size_t)3 * H * H, H, H, stream_));
@@ -542,7 +560,8 @@ void Engine::treelstm_backward() {
       const bool leaf = leaf_round(r);
       const int *child = leaf ? nullptr : d_child_ + 2 * off;
       float *dxW = dxW_.at(off * 4 * H), *dF = leaf ? nullptr : dF_.at(2 * off * H);
-      CAVS_TIMED(K_GATES, cavs_treelstm_round_bwd_gates(dpool_.get(), d_pair_ + off, child, dret_.at(off * H), gates_.at(off * 6 * H),
+      CAVS_TIMED(K_GATES, cavs_treelstm_round_bwd_gates(dpool_.get(), d_pair_ + off, child, dret_folded ? d_dgo_ : dret_.at(off * H),
+                                                        dret_folded ? d_t2j_ + off : nullptr, gates_.at(off * 6 * H),
                                                         leaf ? nullptr : G_.at(2 * off * 2 * H), dxW, 4 * H, dF, r.n, H, stream_));
       c_gather_rows_ += r.n;
       c_launches_ += 1;

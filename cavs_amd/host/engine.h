@@ -113,6 +113,8 @@ class Engine {
 
   Schedule sched_;
   bool did_backward_ = false;
+  float *fwd_out_ = nullptr;   // where the forward pass returns h by vertex id
+  bool out_folded_ = false;    // the rounds wrote it themselves
   int N_ = 0, cap_ = 0, rcap_ = 0, E_ = 0, mw_ = 0, nch_ = 1;
 
   // per-step device index arena: [t2j | pair | child | roots]

@@ -146,7 +146,7 @@ def rounds(iters, st):
         flops = 2.0 * n * H * 5 * H
         us = _time(lambda: hip.call("cavs_treelstm_round_fwd", pool.data_ptr(), child.data_ptr(), pair.data_ptr(),
                                     xW.data_ptr(), 4 * H, U.data_ptr(), bias.data_ptr(), G.data_ptr(), hlr.data_ptr(),
-                                    gt.data_ptr(), msg.data_ptr(), n, H, st), iters, st)
+                                    gt.data_ptr(), msg.data_ptr(), None, None, n, H, st), iters, st)
         _emit("treelstm_round_fwd", f"{tag}: n={n} H={H}", us, flops=flops)
         hU, hUf = torch.empty(n, 3 * H, **f32), torch.empty(2 * n, H, **f32)
 
@@ -167,7 +167,7 @@ def rounds(iters, st):
         dpool, dret = torch.randn(rows, 2 * H, **f32), torch.randn(n, H, **f32)
         dxW, dF = torch.empty(n, 4 * H, **f32), torch.empty(2 * n, H, **f32)
         us = _time(lambda: hip.call("cavs_treelstm_round_bwd_gates", dpool.data_ptr(), pair.data_ptr(), child.data_ptr(),
-                                    dret.data_ptr(), gt.data_ptr(), G.data_ptr(), dxW.data_ptr(), 4 * H, dF.data_ptr(),
+                                    dret.data_ptr(), None, gt.data_ptr(), G.data_ptr(), dxW.data_ptr(), 4 * H, dF.data_ptr(),
                                     n, H, st), iters, st)
         # reads dmsg 2H, dret H, gates 6H, c_l c_r 2H; writes dxW 4H, dF 2H, dc_l dc_r 2H
         _emit("treelstm_round_bwd_gates", f"{tag}: n={n} H={H}", us, nbytes=4 * n * H * 19)

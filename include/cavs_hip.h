@@ -254,17 +254,26 @@ int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int 
  *   row b at 2b, 2b+1 (-1 = none, reads as zero); pair [n] pool row the message of slab
  *   row b is written to (-1 = nowhere); U = U_iou [H,3H] then U_f [H,H].
  * Writes msg [n,2H], pool rows pair[b], and what backward reads again: gates [n,6H],
- * G [2n,2H] (gathered children), hlr [n,H] (h_l + h_r). */
+ * G [2n,2H] (gathered children), hlr [n,H] (h_l + h_r).  With graph_out [*,H] given, the pushed
+ * return value h of slab row b is also written to row out_rows[b] (Push + FunctionPopRet,
+ * op_impl_graphop.cu:168-206,274-327, folded in). */
 int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW,
                             int ld_xw, const float *U, const float *bias, float *G, float *hlr,
-                            float *gates, float *msg, int n, int H, void *stream);
+                            float *gates, float *msg, float *graph_out, const int *out_rows, int n,
+                            int H, void *stream);
+/* The same for a round of leaves (no children: gates of x*W + bias only). */
+int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw,
+                                   const float *bias, float *gates, float *msg, float *graph_out,
+                                   const int *out_rows, int n, int H, void *stream);
 /* Backward of the gates of a round.  The message gradient of slab row b is read from
  * dpool row pair[b] (grad of Scatter is Gather on the same list, zero for -1); the c
  * half of the children's message gradients is written to dpool rows child[2b], child[2b+1]
- * (grad of Gather is Scatter).  child, G and dF are all NULL for a round of leaves. */
+ * (grad of Gather is Scatter).  child, G and dF are all NULL for a round of leaves.  The
+ * gradient of the pushed return value of slab row b is dret row b, or row dret_rows[b] when
+ * that list is given (grad of FunctionPopRet folded in). */
 int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret,
-                                  const float *gates, const float *G, float *dxW, int ld_dxw,
-                                  float *dF, int n, int H, void *stream);
+                                  const int *dret_rows, const float *gates, const float *G,
+                                  float *dxW, int ld_dxw, float *dF, int n, int H, void *stream);
 /* The h half: dh_child = [d_i|d_o|d_u] * U_iou^T + d_f(child) * U_f^T written to dpool rows
  * child[2b], child[2b+1].  UT = U_iou^T [3H,H] then U_f^T [H,H] (cavs_transpose). */
 int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *dF, const float *UT,

@@ -514,8 +514,13 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
 
     d_pool, d_child, d_pair = g.devf(pool), g.devi(child), g.devi(pair)
     G, hlr, gates, msg = g.zeros(2 * n, 2 * H), g.zeros(n, H), g.zeros(n, 6 * H), g.zeros(n, 2 * H)
+    out_rows = np.argsort(r.bulk_normal(n + 3))[:n].astype(np.int32)     # Push + PopRet folded in
+    go = g.zeros(n + 3, H, fill=-7.0)
     g.call("cavs_treelstm_round_fwd", g.P(d_pool), g.P(d_child), g.P(d_pair), g.P(g.devf(xW)), 4 * H, g.P(g.devf(U)),
-           g.P(g.devf(bias)), g.P(G), g.P(hlr), g.P(gates), g.P(msg), n, H, g.stream())
+           g.P(g.devf(bias)), g.P(G), g.P(hlr), g.P(gates), g.P(msg), g.P(go), g.P(g.devi(out_rows)), n, H, g.stream())
+    go_w = np.full((n + 3, H), -7.0, np.float32)
+    go_w[out_rows] = msg_w[:, :H]
+    close(g.host(go), go_w, "graph_out")
     np.testing.assert_array_equal(g.host(G), G_w)
     np.testing.assert_array_equal(g.host(hlr), hlr_w)
     close(g.host(gates), gates_w, "gates")
@@ -540,7 +545,7 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     np.testing.assert_array_equal(g.host(UT)[: 3 * H * H].reshape(3 * H, H), Uiou.T)
     np.testing.assert_array_equal(g.host(UT)[3 * H * H:].reshape(H, H), Uf.T)
     d_dpool, dxW, dF = g.devf(dpool), g.zeros(n, 4 * H), g.zeros(2 * n, H)
-    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool), g.P(d_pair), g.P(d_child), g.P(g.devf(dret)), g.P(g.devf(gates_w)),
+    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool), g.P(d_pair), g.P(d_child), g.P(g.devf(dret)), None, g.P(g.devf(gates_w)),
            g.P(g.devf(G_w)), g.P(dxW), 4 * H, g.P(dF), n, H, g.stream())
     g.call("cavs_treelstm_round_bwd_children", g.P(dxW), 4 * H, g.P(dF), g.P(UT), g.P(d_child), g.P(d_dpool), n, H, g.stream())
     close(g.host(dxW), dxW_w, "dxW")
@@ -551,19 +556,39 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     gates_l, _ = oracle.treelstm_gates_fwd(xW, 0 * hU_w, 0 * hUf_w, 0 * G_w, bias)
     dxW_l, _, _ = oracle.treelstm_gates_bwd(dmsg_w, dret, gates_l, 0 * G_w)
     d_dpool2 = g.devf(dpool)
-    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool2), g.P(d_pair), None, g.P(g.devf(dret)), g.P(g.devf(gates_l)),
+    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool2), g.P(d_pair), None, g.P(g.devf(dret)), None, g.P(g.devf(gates_l)),
            None, g.P(dxW), 4 * H, None, n, H, g.stream())
     close(g.host(dxW), dxW_l, "leaf dxW")
     np.testing.assert_array_equal(g.host(d_dpool2), dpool)
+    # the same with the return-value gradient read through a row list (grad of PopRet folded in)
+    dgo = np.zeros((n + 3, H), np.float32)
+    dgo[out_rows] = dret
+    dxW2 = g.zeros(n, 4 * H)
+    g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool2), g.P(d_pair), None, g.P(g.devf(dgo)), g.P(g.devi(out_rows)),
+           g.P(g.devf(gates_l)), None, g.P(dxW2), 4 * H, None, n, H, g.stream())
+    np.testing.assert_array_equal(g.host(dxW2), g.host(dxW))
+    # a round of leaves forward: gates, message, Scatter and PopRet in one launch
+    _, msg_l = oracle.treelstm_gates_fwd(xW, 0 * hU_w, 0 * hUf_w, 0 * G_w, bias)
+    pool2, gates2, msg2, go2 = g.devf(pool), g.zeros(n, 6 * H), g.zeros(n, 2 * H), g.zeros(n + 3, H, fill=-7.0)
+    g.call("cavs_treelstm_round_leaves_fwd", g.P(pool2), g.P(d_pair), g.P(g.devf(xW)), 4 * H, g.P(g.devf(bias)), g.P(gates2),
+           g.P(msg2), g.P(go2), g.P(g.devi(out_rows)), n, H, g.stream())
+    close(g.host(gates2), gates_l, "leaf gates")
+    close(g.host(msg2), msg_l, "leaf msg")
+    pool_l = pool.copy()
+    pool_l[pair[pair >= 0]] = msg_l[pair >= 0]
+    close(g.host(pool2), pool_l, "leaf pool")
+    go_l = np.full((n + 3, H), -7.0, np.float32)
+    go_l[out_rows] = msg_l[:, :H]
+    close(g.host(go2), go_l, "leaf graph_out")
 
 
 def test_fused_round_entry_points_reject_bad_shapes():
     with pytest.raises(hip.CavsError, match="multiple of 32"):
-        hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 5, 24, 0)
+        hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 0, 0, 5, 24, 0)
     with pytest.raises(hip.CavsError, match="multiple of 32"):
         hip.call("cavs_treelstm_round_bwd_children", 0, 4 * 24, 0, 0, 0, 0, 5, 24, 0)
     with pytest.raises(hip.CavsError, match="all set"):
-        hip.call("cavs_treelstm_round_bwd_gates", 16, 16, 16, 16, 16, 0, 16, 4 * 32, 0, 5, 32, 0)
+        hip.call("cavs_treelstm_round_bwd_gates", 16, 16, 16, 16, 0, 16, 0, 16, 4 * 32, 0, 5, 32, 0)
 
 
 @pytest.mark.parametrize("n,H,C_", [(1, 64, 2), (19, 96, 5), (2482, 512, 5), (300, 100, 8), (77, 1024, 3)])
