@@ -71,29 +71,13 @@ def cpu_baseline(w, budget_s=12.0):
                        "semantics (the reference has no CPU kernels)")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C3")
-    ap.add_argument("--pool", type=int, default=16)
-    ap.add_argument("--lr", type=float, default=1e-3)
-    ap.add_argument("--pairing", default="reference", choices=["reference", "rowid"])
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--host-feeds", action="store_true",
-                    help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        sys.exit("bench.py: this build runs the F-over-G path on one GPU; instance graphs shard by sample "
-                 "across GPUs (see DESIGN.md) but no multi-GPU path is built -- run with --gpus 1")
-
+def measure(a, workload, steps, warmup, n_pool):
+    """Times `steps` training steps of one workload and returns the fields of the JSON line."""
     import torch
 
     from cavs_amd import session
 
-    assert torch.cuda.is_available(), "bench.py needs the MI355X"
-    pool = make_pool(a.workload, a.pool)
+    pool = make_pool(workload, n_pool)
     w0 = pool[0]
     kw = model_kwargs(w0)
     s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
@@ -113,25 +97,25 @@ def main():
             g, x, lab = feeds[i % len(feeds)]
             s.step(g, x, lab, backward=True, lr=a.lr)
 
-    run(0, a.warmup)
+    run(0, warmup)
     s.sync()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    run(a.warmup, a.steps)
+    run(warmup, steps)
     s.sync()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    ms_per_step = 1e3 * elapsed / a.steps
+    ms_per_step = 1e3 * elapsed / steps
     # host side of the last timed step (the profiled pass below slows the host down)
     host_ms = {k: round(s.timing(k), 4) for k in ("GraphParsing", "HostSchedule", "HostWait", "HostStep")}
-    value = w0["B"] * a.steps / elapsed
+    value = w0["B"] * steps / elapsed
 
-    # Roofline of the dominant kernel: the same K steps again with every launch of the
-    # session bracketed by HIP events on the session's own stream (the bracketing costs a
-    # little launch throughput, so it is kept out of the throughput figure above).
+    # Roofline of the dominant kernel: the same steps again with the kernels of every entry point
+    # stamping a start and a stop event themselves (the interval a kernel trace reports) on the
+    # session's own stream; kept out of the throughput figure above.
     s.profile(True)
     flops = rflops = gbytes = sbytes = 0.0
-    for i in range(a.warmup, a.warmup + a.steps):
+    for i in range(warmup, warmup + steps):
         g, x, lab = feeds[i % len(feeds)]
         s.step(g, x, lab, backward=True, lr=a.lr)
         flops += s.counter("gemm_flops")
@@ -148,7 +132,8 @@ def main():
     # the two MFMA-bound kernel classes; the roofline entry describes whichever takes more device time
     mfma = {
         "gemm": dict(ms=gemm_ms, n=gemm_n, flops=flops,
-                     kernel="sgemm_mfma_kernel / sgemm_skinny_kernel (x*W, weight-gradient and head GEMMs of a step)"),
+                     kernel="sgemm_mfma_kernel / sgemm_skinny_kernel (x*W, weight-gradient and head GEMMs of a step"
+                            "; also the recurrent products of rounds too large for the fused kernels)"),
         "round": dict(ms=round_ms, n=round_n, flops=rflops,
                       kernel="treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel (one launch per round: "
                              "gather + recurrent products + gates + scatter)"),
@@ -159,20 +144,22 @@ def main():
     # HBM bytes per dispatch of that class from the two rocprofv3 --pmc runs (FETCH_SIZE scaled by the
     # factor a plain copy of known size gives, plus WRITE_SIZE) summarised under profiles/; measured
     # for the default workload only
-    traffic = PMC_TRAFFIC_BYTES.get((a.workload, dom_name)) if a.pairing == "reference" else None
+    traffic = PMC_TRAFFIC_BYTES.get((workload, dom_name)) if a.pairing == "reference" else None
     rounds = s.counter("rounds")
     launches = s.counter("launches")
 
+    def hbm(nbytes, ms, n):
+        return {"bound": "hbm", "achieved": round(nbytes / (ms * 1e-3) / 1e9, 2) if ms else None, "peak": HBM_PEAK_GBS,
+                "unit": "GB/s", "avg_launch_us": round(1e3 * ms / max(n, 1), 3), "launches_per_step": round(n / steps, 1)}
+
     out = {
-        "metric": "train samples/sec (fwd+bwd) Tree-LSTM h=512 bs=64; % HBM/MFMA peak",
-        "value": round(value, 2), "unit": "samples/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{a.workload}: {w0['model']} V={w0['V']} E={w0['E']} H={w0['H']} B={w0['B']} "
+        "value": round(value, 2), "unit": "samples/s", "steps": steps, "warmup": warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "config": {"workload": f"{workload}: {w0['model']} V={w0['V']} E={w0['E']} H={w0['H']} B={w0['B']} "
                                f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing,
-                   "feeds": "pageable host memory, copied every step" if a.host_feeds else "resident in HBM", "rounds_last_batch": rounds,
-                   "launches_last_batch": launches},
+                   "feeds": "pageable host memory, copied every step" if a.host_feeds else "resident in HBM",
+                   "rounds_last_batch": rounds, "launches_last_batch": launches},
         "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
                      "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": traffic,
                      "kernel": dom["kernel"],
@@ -180,23 +167,61 @@ def main():
                      "flops_per_launch": round(dom["flops"] / dom["n"], 1) if dom["n"] else None},
         "kernels": {
             **{k: {"bound": "mfma", "achieved": round(v["tf"], 3), "peak": FP32_MFMA_PEAK_TF, "unit": "TFLOP/s",
-                   "avg_launch_us": round(1e3 * v["ms"] / max(v["n"], 1), 3), "launches_per_step": round(v["n"] / a.steps, 1)}
+                   "frac": round(v["tf"] / FP32_MFMA_PEAK_TF, 4),
+                   "avg_launch_us": round(1e3 * v["ms"] / max(v["n"], 1), 3), "launches_per_step": round(v["n"] / steps, 1)}
                for k, v in mfma.items()},
-            "gather": {"bound": "hbm", "achieved": round(gbytes / (gat_ms * 1e-3) / 1e9, 2) if gat_ms else None,
-                       "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * gat_ms / max(gat_n, 1), 3)},
-            "scatter": {"bound": "hbm", "achieved": round(sbytes / (sca_ms * 1e-3) / 1e9, 2) if sca_ms else None,
-                        "peak": HBM_PEAK_GBS, "unit": "GB/s", "avg_launch_us": round(1e3 * sca_ms / max(sca_n, 1), 3)},
+            # separate gather / scatter launches only (rounds that run fused move their rows inside the round kernel)
+            "gather": hbm(gbytes, gat_ms, gat_n), "scatter": hbm(sbytes, sca_ms, sca_n),
             "gates": {"avg_launch_us": round(1e3 * gates_ms / max(gates_n, 1), 3)},
-            "device_ms_per_step": {"gemm": round(gemm_ms / a.steps, 4), "round": round(round_ms / a.steps, 4),
-                                   "gather": round(gat_ms / a.steps, 4), "scatter": round(sca_ms / a.steps, 4),
-                                   "gates": round(gates_ms / a.steps, 4), "other": round(other_ms / a.steps, 4)},
+            "device_ms_per_step": {"gemm": round(gemm_ms / steps, 4), "round": round(round_ms / steps, 4),
+                                   "gather": round(gat_ms / steps, 4), "scatter": round(sca_ms / steps, 4),
+                                   "gates": round(gates_ms / steps, 4), "other": round(other_ms / steps, 4)},
         },
         "timers_ms": {**host_ms, "RNNForward": round(s.timing("RNNForward"), 4),
                       "RNNBackward": round(s.timing("RNNBackward"), 4)},
     }
+    s.close()
+    del feeds
+    torch.cuda.empty_cache()
+    return out, w0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C3")
+    ap.add_argument("--pool", type=int, default=16)
+    ap.add_argument("--lr", type=float, default=1e-3)
+    ap.add_argument("--pairing", default="reference", choices=["reference", "rowid"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--host-feeds", action="store_true",
+                    help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
+    ap.add_argument("--also", default="C5",
+                    help="a second workload measured with few steps and reported under 'also' (the large Tree-LSTM "
+                         "configuration, where rounds are GEMM-sized); 'none' to skip")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs the F-over-G path on one GPU; instance graphs shard by sample "
+                 "across GPUs (see DESIGN.md) but no multi-GPU path is built -- run with --gpus 1")
+
+    import torch
+
+    assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    res, w0 = measure(a, a.workload, a.steps, a.warmup, a.pool)
+    out = {
+        "metric": "train samples/sec (fwd+bwd) Tree-LSTM h=512 bs=64; % HBM/MFMA peak",
+        "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": res["config"], "roofline": res["roofline"], "kernels": res["kernels"], "timers_ms": res["timers_ms"],
+    }
+    if a.also.lower() != "none" and a.also != a.workload:
+        also, _ = measure(a, a.also, 10, 3, 2)
+        out["also"] = {a.also: {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
-    s.close()
     print(json.dumps(out))
 
 
