@@ -1,0 +1,624 @@
+// Fused rounds of the chain LSTM (apps/paper/seq-lstm-cavs.cc:62-86) and of Tree-FC
+// (apps/paper/tree-fc-cavs.cc:28-36): the same construction as the Tree-LSTM round kernels --
+// a workgroup owns TILE rows x TILE hidden columns, its wavefronts split K and feed the MFMA
+// straight from global memory with the gather as the operand fetch, partial tiles are
+// parked per wavefront in LDS, and the epilogue applies the pointwise part of the vertex
+// function and scatters the message.  A chain round is one sequence step for all live
+// sequences (n <= batch size): without fusion it is four dependent launches of latency.
+#include "round_common.h"
+
+namespace cavs {
+
+// One product chain: acc[p] += A[row, kb:ke) * B_p[kb:ke, col] for NB B operands that share A.
+// a_row: the lane's A row (k-contiguous, 16-byte aligned) or nullptr for a zero row;
+// b[p]: the lane's column of B operand p at k = 0, row stride ldb.
+template <int TILE, int NB>
+__device__ inline void product_chain(typename Mma<TILE>::Acc (&acc)[NB], const float *a_row, const float *const (&b)[NB],
+                                     long ldb, int kb, int ke, int slot) {
+  using M = Mma<TILE>;
+  constexpr int GK = 4 * M::NSLOT, UG = 2, S = GK * UG;
+  struct Frag {
+    float4 a[UG];
+    float b[UG][NB][4];
+  };
+  auto fetch = [&](int k0, Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+      const int kk = k0 + GK * u + 4 * slot;
+      const bool kin = kk < ke;
+#pragma unroll
+      for (int p = 0; p < NB; p++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) f.b[u][p][c] = kin ? b[p][(long)(kk + c) * ldb] : 0.f;
+      f.a[u] = (kin && a_row) ? ld4(a_row + kk) : zero4();
+    }
+  };
+  auto multiply = [&](const Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++)
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int p = 0; p < NB; p++) acc[p] = M::mma(elem(f.a[u], c), f.b[u][p][c], acc[p]);
+  };
+  Frag f0, f1;
+  if (kb < ke) fetch(kb, f0);
+  for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+    if (k0 + S < ke) fetch(k0 + S, f1);
+    multiply(f0);
+    if (k0 + S < ke) {
+      if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+      multiply(f1);
+    }
+  }
+}
+
+// element (q-th of this thread) of the workgroup's tile: slab row, column, LDS offset
+template <int TILE, int NP, int THREADS>
+struct TileElems {
+  using M = Mma<TILE>;
+  static constexpr int NR = M::NR, EPT = (NR * 64 + THREADS - 1) / THREADS;
+  bool on[EPT];
+  int b[EPT], j[EPT], lds[EPT];
+  __device__ inline void init(int tid, int row0, int j0, int n) {
+#pragma unroll
+    for (int q = 0; q < EPT; q++) {
+      const int e = tid + q * THREADS;
+      const int l2 = e & 63, r = (e >> 6) % NR;
+      b[q] = row0 + M::row(r, l2);
+      j[q] = j0 + (l2 & (TILE - 1));
+      lds[q] = r * 64 + l2;
+      on[q] = e < NR * 64 && b[q] < n;
+    }
+  }
+};
+
+template <int NP, int NR, int NREG>
+__device__ inline void sum_regions(float (&v)[NP], const float *red, int lds, int rsz) {
+#pragma unroll
+  for (int p = 0; p < NP; p++) {
+    float s = red[lds + p * NR * 64];
+#pragma unroll
+    for (int g = 1; g < NREG; g++) s += red[g * rsz + lds + p * NR * 64];
+    v[p] = s;
+  }
+}
+
+template <int W>
+__device__ inline void stw(float *p, const float (&v)[W]) {
+  if constexpr (W == 4) {
+    *reinterpret_cast<float4 *>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  } else {
+#pragma unroll
+    for (int k = 0; k < W; k++) p[k] = v[k];
+  }
+}
+template <int W>
+__device__ inline void ldw(const float *p, float (&v)[W]) {
+  if constexpr (W == 4) {
+    const float4 t = ld4(p);
+    v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+  } else {
+#pragma unroll
+    for (int k = 0; k < W; k++) v[k] = p[k];
+  }
+}
+
+// ================================================================== chain LSTM
+struct LstmFwdArgs {
+  const float *pool;    // [*, 2H] rows [h|c]
+  const int *child;     // [n] pool row of the predecessor (-1: none) or nullptr (first step of every sequence)
+  const int *pair;      // [n]
+  const float *xW;      // [n, 4H] (ld) blocks [i|f|u|o]
+  long ld_xw;
+  const float *Wh;      // [H, 4H]
+  const float *bias;    // [4H]
+  float *G;             // [n, 2H] gathered predecessor
+  float *gates;         // [n, 5H] = [i|f|u|o|tanh c]
+  float *msg;           // [n, 2H]
+  float *pool_out;
+  float *go;
+  const int *out_rows;
+  int n, H;
+};
+
+template <int TILE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs a) {
+  using M = Mma<TILE>;
+  using Acc = typename M::Acc;
+  constexpr int THREADS = WAVES * 64, KS = WAVES, GK = 4 * M::NSLOT, NP = 4, NR = M::NR;
+  constexpr int NREG = Regions<TILE, KS>::N, RSZ = NP * NR * 64;
+  __shared__ float red[NREG * RSZ];
+  const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
+  const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int H = a.H;
+  const long H2 = 2L * H, H4 = 4L * H;
+  const int j0 = blockIdx.x * TILE, row0 = blockIdx.y * TILE;
+  const int row = row0 + x;
+  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
+  const int kb = ks * kper, ke = min(H, kb + kper);
+
+  int cp = -1;
+  if (row < a.n) cp = a.child[row];
+  TileElems<TILE, NP, THREADS> el;
+  el.init(tid, row0, j0, a.n);
+  constexpr int EPT = TileElems<TILE, NP, THREADS>::EPT;
+  int ecp[EPT], edst[EPT], eout[EPT];
+  float exw[EPT][4], ebias[EPT][4];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    ecp[q] = edst[q] = eout[q] = -1;
+    if (el.on[q]) {
+      ecp[q] = a.child[el.b[q]];
+      edst[q] = a.pair[el.b[q]];
+      if (a.go) eout[q] = a.out_rows[el.b[q]];
+      const float *xw = a.xW + el.b[q] * a.ld_xw + el.j[q];
+#pragma unroll
+      for (int k = 0; k < 4; k++) { exw[q][k] = xw[k * H]; ebias[q][k] = a.bias[k * H + el.j[q]]; }
+    }
+  }
+
+  Acc acc[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++)
+#pragma unroll
+    for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
+  const float *bcol[NP];
+#pragma unroll
+  for (int p = 0; p < NP; p++) bcol[p] = a.Wh + p * H + j0 + x;
+  product_chain<TILE, NP>(acc, cp >= 0 ? a.pool + cp * H2 : nullptr, bcol, H4, kb, ke, slot);
+
+  float ehp[EPT], ecprev[EPT];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    ehp[q] = ecprev[q] = 0.f;
+    if (ecp[q] >= 0) { ehp[q] = a.pool[ecp[q] * H2 + el.j[q]]; ecprev[q] = a.pool[ecp[q] * H2 + H + el.j[q]]; }
+  }
+  park_partials<TILE, NP, KS, NREG, 1>(red, acc, 0, ks, lane);
+
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    if (!el.on[q]) continue;
+    float v[NP];
+    sum_regions<NP, NR, NREG>(v, red, el.lds[q], RSZ);
+    const int b = el.b[q], j = el.j[q];
+    // same association as the separate path: (x*W + h*W') + bias
+    const float i = sigm_r((exw[q][0] + v[0]) + ebias[q][0]);
+    const float f = sigm_r((exw[q][1] + v[1]) + ebias[q][1]);
+    const float u = tanhf((exw[q][2] + v[2]) + ebias[q][2]);
+    const float o = sigm_r((exw[q][3] + v[3]) + ebias[q][3]);
+    const float c = i * u + f * ecprev[q];
+    const float tc = tanhf(c);
+    const float h = o * tc;
+    float *g = a.gates + (long)b * 5 * H + j;
+    g[0] = i; g[H] = f; g[2 * H] = u; g[3 * H] = o; g[4 * H] = tc;
+    float *m = a.msg + b * H2 + j;
+    m[0] = h; m[H] = c;
+    if (edst[q] >= 0) { a.pool_out[edst[q] * H2 + j] = h; a.pool_out[edst[q] * H2 + H + j] = c; }
+    if (eout[q] >= 0) a.go[(long)eout[q] * H + j] = h;
+    float *gp = a.G + b * H2 + j;
+    gp[0] = ehp[q]; gp[H] = ecprev[q];
+  }
+}
+
+// first step of every sequence (no predecessor), and the gate gradients of any round:
+// elementwise, with the row movement folded in
+struct LstmLeavesArgs {
+  const float *xW;
+  long ld_xw;
+  const float *bias;
+  const int *pair;
+  float *gates, *msg, *pool, *go;
+  const int *out_rows;
+  int n, H;
+};
+
+template <int W>
+__global__ void lstm_round_leaves_fwd_kernel(LstmLeavesArgs a) {
+  const int H = a.H, hw = H / W;
+  const long H2 = 2L * H;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int dst = a.pair[r], out = a.go ? a.out_rows[r] : -1;
+  const float *xw = a.xW + r * a.ld_xw + j;
+  float gi[W], gf[W], gu[W], go[W], gtc[W], mh[W], mc[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const float i = sigm_r((xw[k] + 0.f) + a.bias[j + k]);
+    const float f = sigm_r((xw[H + k] + 0.f) + a.bias[H + j + k]);
+    const float u = tanhf((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
+    const float o = sigm_r((xw[3 * H + k] + 0.f) + a.bias[3 * H + j + k]);
+    const float c = i * u + f * 0.f;
+    const float tc = tanhf(c);
+    gi[k] = i; gf[k] = f; gu[k] = u; go[k] = o; gtc[k] = tc; mh[k] = o * tc; mc[k] = c;
+  }
+  float *g = a.gates + (long)r * 5 * H + j;
+  stw<W>(g, gi); stw<W>(g + H, gf); stw<W>(g + 2 * H, gu); stw<W>(g + 3 * H, go); stw<W>(g + 4 * H, gtc);
+  float *m = a.msg + r * H2 + j;
+  stw<W>(m, mh); stw<W>(m + H, mc);
+  if (dst >= 0) { stw<W>(a.pool + dst * H2 + j, mh); stw<W>(a.pool + dst * H2 + H + j, mc); }
+  if (out >= 0) stw<W>(a.go + (long)out * H + j, mh);
+}
+
+struct LstmBwdGatesArgs {
+  const float *dpool;
+  const int *pair;
+  const int *child;      // [n] or nullptr (first step)
+  const float *dret;
+  const int *dret_rows;  // or nullptr
+  const float *gates;    // [n, 5H]
+  const float *G;        // [n, 2H] or nullptr
+  float *da;             // [n, 4H] (ld) blocks [i|f|u|o]
+  long ld_da;
+  float *dpool_out;
+  int n, H;
+};
+
+template <int W>
+__global__ void lstm_round_bwd_gates_kernel(LstmBwdGatesArgs a) {
+  const int H = a.H, hw = H / W;
+  const long H2 = 2L * H;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int src = a.pair[r];
+  const int dr_row = a.dret_rows ? a.dret_rows[r] : r;
+  const int cp = a.child ? a.child[r] : -1;
+  const float *g = a.gates + (long)r * 5 * H + j;
+  float gi[W], gf[W], gu[W], go[W], gtc[W], dmh[W], dmc[W], dr[W], cprev[W];
+  ldw<W>(g, gi); ldw<W>(g + H, gf); ldw<W>(g + 2 * H, gu); ldw<W>(g + 3 * H, go); ldw<W>(g + 4 * H, gtc);
+  ldw<W>(a.dret + (long)dr_row * H + j, dr);
+  if (src >= 0) { ldw<W>(a.dpool + src * H2 + j, dmh); ldw<W>(a.dpool + src * H2 + H + j, dmc); }
+  if (a.G) ldw<W>(a.G + r * H2 + H + j, cprev);
+  float di[W], df[W], du[W], dvo[W], dcp[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const float mh = src >= 0 ? dmh[k] : 0.f, mc = src >= 0 ? dmc[k] : 0.f, cpv = a.G ? cprev[k] : 0.f;
+    const float i = gi[k], f = gf[k], u = gu[k], o = go[k], tc = gtc[k];
+    const float dh = mh + dr[k];
+    const float d_o = dh * tc;
+    const float dc = mc + (dh * o) * (1.f - tc * tc);
+    di[k] = (dc * u) * (i * (1.f - i));
+    df[k] = (dc * cpv) * (f * (1.f - f));
+    du[k] = (dc * i) * (1.f - u * u);
+    dvo[k] = d_o * (o * (1.f - o));
+    dcp[k] = dc * f;
+  }
+  float *d = a.da + r * a.ld_da + j;
+  stw<W>(d, di); stw<W>(d + H, df); stw<W>(d + 2 * H, du); stw<W>(d + 3 * H, dvo);
+  if (cp >= 0) stw<W>(a.dpool_out + cp * H2 + H + j, dcp);
+}
+
+// Gradient of the gathered children's h: for child p of slab row b,
+//   dpool[child[b*NB + p]][0:H) = dA[b, 0:K) * BT[0:K, p*H : (p+1)*H)
+// (grad of Gather is Scatter, folded into the product's epilogue).  Chain LSTM: NB = 1,
+// dA = da [n,4H], BT = W'^T [4H,H].  Tree-FC: NB = 2, dA = dz [n,H], BT = W^T [H,2H].
+struct ChildBwdArgs {
+  const float *dA;    // [n, K] (ld)
+  long ld;
+  const float *BT;    // [K, ldb]
+  long ldb;
+  const int *child;   // [n * NB]
+  float *dpool;       // [*, mw]
+  long mw;            // row width of the pool
+  int n, H, K;
+};
+
+template <int TILE, int WAVES, int NB>
+__global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwdArgs a) {
+  using M = Mma<TILE>;
+  using Acc = typename M::Acc;
+  constexpr int THREADS = WAVES * 64, KS = WAVES, GK = 4 * M::NSLOT, NR = M::NR;
+  constexpr int NREG = Regions<TILE, KS>::N, RSZ = NB * NR * 64;
+  __shared__ float red[NREG * RSZ];
+  const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
+  const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int H = a.H, K = a.K;
+  const int j0 = blockIdx.x * TILE, row0 = blockIdx.y * TILE;
+  const int row = row0 + x;
+  const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
+  const int kb = ks * kper, ke = min(K, kb + kper);
+  TileElems<TILE, NB, THREADS> el;
+  el.init(tid, row0, j0, a.n);
+  constexpr int EPT = TileElems<TILE, NB, THREADS>::EPT;
+  int ecp[EPT][NB];
+#pragma unroll
+  for (int q = 0; q < EPT; q++)
+#pragma unroll
+    for (int p = 0; p < NB; p++) ecp[q][p] = el.on[q] ? a.child[el.b[q] * NB + p] : -1;
+  Acc acc[NB];
+  const float *bcol[NB];
+#pragma unroll
+  for (int p = 0; p < NB; p++) {
+    bcol[p] = a.BT + (long)p * H + j0 + x;
+#pragma unroll
+    for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
+  }
+  product_chain<TILE, NB>(acc, row < a.n ? a.dA + row * a.ld : nullptr, bcol, a.ldb, kb, ke, slot);
+  park_partials<TILE, NB, KS, NREG, 1>(red, acc, 0, ks, lane);
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    if (!el.on[q]) continue;
+    float v[NB];
+    sum_regions<NB, NR, NREG>(v, red, el.lds[q], RSZ);
+#pragma unroll
+    for (int p = 0; p < NB; p++)
+      if (ecp[q][p] >= 0) a.dpool[ecp[q][p] * a.mw + el.j[q]] = v[p];
+  }
+}
+
+// ================================================================== Tree-FC
+// h = act(W^T [h_l ; h_r] + b + x): one product whose A row is the concatenation of the two
+// children's rows (k < H from the left child, k >= H from the right one).
+struct TreeFcFwdArgs {
+  const float *pool;    // [*, H]
+  const int *child;     // [2n]
+  const int *pair;      // [n]
+  const float *W;       // [2H, H]
+  const float *bias;    // [H] or nullptr
+  const float *x;       // [n, H] or nullptr
+  float *G;             // [n, 2H] gathered children [h_l | h_r]
+  float *msg;           // [n, H]
+  float *pool_out;
+  float *go;
+  const int *out_rows;
+  int n, H, act;
+};
+
+template <int TILE, int WAVES>
+__global__ __launch_bounds__(WAVES * 64) void treefc_round_fwd_kernel(TreeFcFwdArgs a) {
+  using M = Mma<TILE>;
+  using Acc = typename M::Acc;
+  constexpr int THREADS = WAVES * 64, KS = WAVES, GK = 4 * M::NSLOT, NP = 1, NR = M::NR;
+  constexpr int NREG = Regions<TILE, KS>::N, RSZ = NP * NR * 64;
+  __shared__ float red[NREG * RSZ];
+  const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
+  const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int H = a.H;
+  const int j0 = blockIdx.x * TILE, row0 = blockIdx.y * TILE;
+  const int row = row0 + x;
+  // the wavefronts split each half of K (one half per child) between them
+  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
+  const int kb = ks * kper, ke = min(H, kb + kper);
+  int cl = -1, cr = -1;
+  if (row < a.n) { cl = a.child[2 * row]; cr = a.child[2 * row + 1]; }
+  TileElems<TILE, NP, THREADS> el;
+  el.init(tid, row0, j0, a.n);
+  constexpr int EPT = TileElems<TILE, NP, THREADS>::EPT;
+  int ecl[EPT], ecr[EPT], edst[EPT], eout[EPT];
+  float eb[EPT], ex[EPT];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    ecl[q] = ecr[q] = edst[q] = eout[q] = -1;
+    eb[q] = ex[q] = 0.f;
+    if (el.on[q]) {
+      ecl[q] = a.child[2 * el.b[q]];
+      ecr[q] = a.child[2 * el.b[q] + 1];
+      edst[q] = a.pair[el.b[q]];
+      if (a.go) eout[q] = a.out_rows[el.b[q]];
+      if (a.bias) eb[q] = a.bias[el.j[q]];
+      if (a.x) ex[q] = a.x[(long)el.b[q] * H + el.j[q]];
+    }
+  }
+  Acc acc[NP];
+#pragma unroll
+  for (int r = 0; r < NR; r++) acc[0][r] = 0.f;
+  const float *bl[NP] = {a.W + j0 + x};
+  const float *br[NP] = {a.W + (long)H * H + j0 + x};
+  product_chain<TILE, NP>(acc, cl >= 0 ? a.pool + (long)cl * H : nullptr, bl, H, kb, ke, slot);
+  product_chain<TILE, NP>(acc, cr >= 0 ? a.pool + (long)cr * H : nullptr, br, H, kb, ke, slot);
+  float ehl[EPT], ehr[EPT];
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    ehl[q] = ecl[q] >= 0 ? a.pool[(long)ecl[q] * H + el.j[q]] : 0.f;
+    ehr[q] = ecr[q] >= 0 ? a.pool[(long)ecr[q] * H + el.j[q]] : 0.f;
+  }
+  park_partials<TILE, NP, KS, NREG, 1>(red, acc, 0, ks, lane);
+#pragma unroll
+  for (int q = 0; q < EPT; q++) {
+    if (!el.on[q]) continue;
+    float v[NP];
+    sum_regions<NP, NR, NREG>(v, red, el.lds[q], RSZ);
+    const int b = el.b[q], j = el.j[q];
+    float t = v[0];
+    if (a.bias) t += eb[q];
+    if (a.x) t += ex[q];
+    const float h = a.act ? tanhf(t) : (t > 0.f ? t : 0.f);
+    a.msg[(long)b * H + j] = h;
+    if (edst[q] >= 0) a.pool_out[(long)edst[q] * H + j] = h;
+    if (eout[q] >= 0) a.go[(long)eout[q] * H + j] = h;
+    float *gp = a.G + (long)b * 2 * H + j;
+    gp[0] = ehl[q]; gp[H] = ehr[q];
+  }
+}
+
+// leaves forward and the pointwise gradient of any round, with the row movement folded in
+struct TreeFcLeavesArgs {
+  const float *bias, *x;
+  const int *pair;
+  float *msg, *pool, *go;
+  const int *out_rows;
+  int n, H, act;
+};
+
+template <int W>
+__global__ void treefc_round_leaves_fwd_kernel(TreeFcLeavesArgs a) {
+  const int H = a.H, hw = H / W;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int dst = a.pair[r], out = a.go ? a.out_rows[r] : -1;
+  float h[W];
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    float t = 0.f;
+    if (a.bias) t += a.bias[j + k];
+    if (a.x) t += a.x[(long)r * H + j + k];
+    h[k] = a.act ? tanhf(t) : (t > 0.f ? t : 0.f);
+  }
+  stw<W>(a.msg + (long)r * H + j, h);
+  if (dst >= 0) stw<W>(a.pool + (long)dst * H + j, h);
+  if (out >= 0) stw<W>(a.go + (long)out * H + j, h);
+}
+
+struct TreeFcBwdArgs {
+  const float *dpool;
+  const int *pair;
+  const float *dret;
+  const int *dret_rows;
+  const float *h;   // [n, H] forward output of the round
+  float *dz;        // [n, H]
+  int n, H, act;
+};
+
+template <int W>
+__global__ void treefc_round_bwd_kernel(TreeFcBwdArgs a) {
+  const int H = a.H, hw = H / W;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int r = (int)(idx / hw), j = (int)(idx % hw) * W;
+  const int src = a.pair[r];
+  const int dr_row = a.dret_rows ? a.dret_rows[r] : r;
+  float y[W], dm[W], dr[W], o[W];
+  ldw<W>(a.h + (long)r * H + j, y);
+  ldw<W>(a.dret + (long)dr_row * H + j, dr);
+  if (src >= 0) ldw<W>(a.dpool + (long)src * H + j, dm);
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const float dh = (src >= 0 ? dm[k] : 0.f) + dr[k];
+    o[k] = a.act ? dh * (1.f - y[k] * y[k]) : (y[k] > 0.f ? dh : 0.f);
+  }
+  stw<W>(a.dz + (long)r * H + j, o);
+}
+
+template <typename KernelArgs, typename K16x8, typename K16x4, typename K32x8>
+static void launch_round(const KernelArgs &a, int n, int H, hipStream_t st, K16x8 k168, K16x4 k164, K32x8 k328) {
+  const RoundPlan p = plan_round(n);
+  dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
+  if (p.tile == 16 && p.waves == 8) launch(k168, grid, 512, 0, st, a);
+  else if (p.tile == 16) launch(k164, grid, 256, 0, st, a);
+  else launch(k328, grid, 512, 0, st, a);
+}
+
+template <typename A, typename K4, typename K1>
+static void launch_pointwise(const A &a, int n, int H, bool vec, hipStream_t st, K4 k4, K1 k1) {
+  if (vec) {
+    long total = (long)n * (H / 4);
+    launch(k4, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  } else {
+    long total = (long)n * H;
+    launch(k1, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  }
+}
+
+static bool all16(std::initializer_list<const void *> ps) {
+  for (const void *p : ps)
+    if (p && !aligned16(p)) return false;
+  return true;
+}
+
+}  // namespace cavs
+
+using namespace cavs;
+
+extern "C" {
+
+int cavs_lstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw, const float *Wh,
+                        const float *bias, float *G, float *gates, float *msg, float *graph_out, const int *out_rows,
+                        int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && ld_xw >= 4 * H, "cavs_lstm_round_fwd: bad shape n=%d H=%d ld=%d (H must be a multiple of 32)", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && child && pair && xW && Wh && bias && G && gates && msg, "cavs_lstm_round_fwd: null pointer");
+  CAVS_REQUIRE(aligned16(pool), "cavs_lstm_round_fwd: pool must be 16-byte aligned");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_lstm_round_fwd: graph_out needs out_rows");
+  LstmFwdArgs a{pool, child, pair, xW, ld_xw, Wh, bias, G, gates, msg, pool, graph_out, out_rows, n, H};
+  launch_round(a, n, H, as_stream(stream), lstm_round_fwd_kernel<16, 8>, lstm_round_fwd_kernel<16, 4>, lstm_round_fwd_kernel<32, 8>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_lstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw, const float *bias, float *gates,
+                               float *msg, float *graph_out, const int *out_rows, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && ld_xw >= 4 * H, "cavs_lstm_round_leaves_fwd: bad shape n=%d H=%d ld=%d", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && pair && xW && bias && gates && msg, "cavs_lstm_round_leaves_fwd: null pointer");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_lstm_round_leaves_fwd: graph_out needs out_rows");
+  LstmLeavesArgs a{xW, ld_xw, bias, pair, gates, msg, pool, graph_out, out_rows, n, H};
+  const bool vec = H % 4 == 0 && ld_xw % 4 == 0 && all16({pool, xW, bias, gates, msg, graph_out});
+  launch_pointwise(a, n, H, vec, as_stream(stream), lstm_round_leaves_fwd_kernel<4>, lstm_round_leaves_fwd_kernel<1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_lstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret, const int *dret_rows,
+                              const float *gates, const float *G, float *da, int ld_da, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && ld_da >= 4 * H, "cavs_lstm_round_bwd_gates: bad shape n=%d H=%d ld=%d", n, H, ld_da);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dpool && pair && dret && gates && da, "cavs_lstm_round_bwd_gates: null pointer");
+  CAVS_REQUIRE((child && G) || (!child && !G), "cavs_lstm_round_bwd_gates: child and G must be both set or both null");
+  LstmBwdGatesArgs a{dpool, pair, child, dret, dret_rows, gates, G, da, ld_da, dpool, n, H};
+  const bool vec = H % 4 == 0 && ld_da % 4 == 0 && all16({dpool, dret, gates, G, da});
+  launch_pointwise(a, n, H, vec, as_stream(stream), lstm_round_bwd_gates_kernel<4>, lstm_round_bwd_gates_kernel<1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int ldb, int nchild, const int *child,
+                            float *dpool, int pool_width, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && K > 0 && K % 4 == 0 && ld >= K && ld % 4 == 0 && pool_width >= H &&
+                   (nchild == 1 || nchild == 2) && ldb >= nchild * H,
+               "cavs_round_bwd_children: bad shape n=%d H=%d K=%d ld=%d ldb=%d nchild=%d pool_width=%d", n, H, K, ld, ldb, nchild, pool_width);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dA && BT && child && dpool, "cavs_round_bwd_children: null pointer");
+  CAVS_REQUIRE(aligned16(dA), "cavs_round_bwd_children: dA must be 16-byte aligned");
+  ChildBwdArgs a{dA, ld, BT, ldb, child, dpool, pool_width, n, H, K};
+  hipStream_t st = as_stream(stream);
+  if (nchild == 1)
+    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 1>, round_bwd_children_kernel<16, 4, 1>, round_bwd_children_kernel<32, 8, 1>);
+  else
+    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 2>, round_bwd_children_kernel<16, 4, 2>, round_bwd_children_kernel<32, 8, 2>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treefc_round_fwd(float *pool, const int *child, const int *pair, const float *W, const float *bias,
+                          const float *x, float *G, float *msg, float *graph_out, const int *out_rows, int n, int H,
+                          int act, void *stream) {
+  CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && (act == 0 || act == 1), "cavs_treefc_round_fwd: bad argument n=%d H=%d act=%d (H must be a multiple of 32)", n, H, act);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && child && pair && W && G && msg, "cavs_treefc_round_fwd: null pointer");
+  CAVS_REQUIRE(aligned16(pool), "cavs_treefc_round_fwd: pool must be 16-byte aligned");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treefc_round_fwd: graph_out needs out_rows");
+  TreeFcFwdArgs a{pool, child, pair, W, bias, x, G, msg, pool, graph_out, out_rows, n, H, act};
+  launch_round(a, n, H, as_stream(stream), treefc_round_fwd_kernel<16, 8>, treefc_round_fwd_kernel<16, 4>, treefc_round_fwd_kernel<32, 8>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treefc_round_leaves_fwd(float *pool, const int *pair, const float *bias, const float *x, float *msg,
+                                 float *graph_out, const int *out_rows, int n, int H, int act, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && (act == 0 || act == 1), "cavs_treefc_round_leaves_fwd: bad argument n=%d H=%d act=%d", n, H, act);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && pair && msg, "cavs_treefc_round_leaves_fwd: null pointer");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treefc_round_leaves_fwd: graph_out needs out_rows");
+  TreeFcLeavesArgs a{bias, x, pair, msg, pool, graph_out, out_rows, n, H, act};
+  const bool vec = H % 4 == 0 && all16({pool, bias, x, msg, graph_out});
+  launch_pointwise(a, n, H, vec, as_stream(stream), treefc_round_leaves_fwd_kernel<4>, treefc_round_leaves_fwd_kernel<1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treefc_round_bwd(const float *dpool, const int *pair, const float *dret, const int *dret_rows, const float *h,
+                          float *dz, int n, int H, int act, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && (act == 0 || act == 1), "cavs_treefc_round_bwd: bad argument n=%d H=%d act=%d", n, H, act);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dpool && pair && dret && h && dz, "cavs_treefc_round_bwd: null pointer");
+  TreeFcBwdArgs a{dpool, pair, dret, dret_rows, h, dz, n, H, act};
+  const bool vec = H % 4 == 0 && all16({dpool, dret, h, dz});
+  launch_pointwise(a, n, H, vec, as_stream(stream), treefc_round_bwd_kernel<4>, treefc_round_bwd_kernel<1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // extern "C"

@@ -245,8 +245,8 @@ void Engine::reserve_edges() {
     R(dxW_, cap * H);
     R(r_z_, rc * H);
   }
+  if (fused_rows() > 0) R(UT_, (size_t)(cfg_.model == CAVS_MODEL_TREEFC ? 2 : 4) * H * H);
   if (cfg_.model == CAVS_MODEL_TREELSTM) {
-    if (fused_rows() > 0) R(UT_, (size_t)4 * H * H);
     R(hlr_, cap * H);
     R(dF_, cap * 2 * H);
     R(r_hU_, rc * 3 * H);
@@ -476,7 +476,7 @@ void Engine::pop_ret(float *graph_out) {
 // The fused round kernels need the batch scheduler's rounds (every vertex of an internal
 // round has both children) and H in whole MFMA tiles.
 int Engine::fused_rows() const {
-  if (cfg_.model != CAVS_MODEL_TREELSTM || !(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.H % 32 != 0) return 0;
+  if (!(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.H % 32 != 0) return 0;
   if (cfg_.fused_round_rows < 0) return 0;
   // measured crossover with the separate launches: about 2400 rows at H=512, 1500 at H=1024
   return cfg_.fused_round_rows > 0 ? cfg_.fused_round_rows : (cfg_.H <= 512 ? 2048 : 1024);
@@ -644,9 +644,26 @@ void Engine::lstm_forward() {
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  const int fused = fused_rows();
+  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  float *go = out_folded_ ? fwd_out_ : nullptr;
   for (const Round &r : sched_.rounds) {
     const size_t off = r.offset;
     float *a = xW_.at(off * 4 * H), *msg = msg_.at(off * 2 * H), *G = nullptr;
+    if (r.n <= fused) {  // one launch: Gather, h*W', gates, Scatter, Push/PopRet
+      if (leaf_round(r)) {
+        CAVS_TIMED(K_GATES, cavs_lstm_round_leaves_fwd(pool_.get(), d_pair_ + off, a, 4 * H, Bv, gates_.at(off * 5 * H), msg, go,
+                                                       d_t2j_ + off, r.n, H, stream_));
+      } else {
+        CAVS_TIMED(K_ROUND, cavs_lstm_round_fwd(pool_.get(), d_child_ + off, d_pair_ + off, a, 4 * H, Wh, Bv, G_.at(off * 2 * H),
+                                                gates_.at(off * 5 * H), msg, go, d_t2j_ + off, r.n, H, stream_));
+        c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
+        c_gather_rows_ += r.n;
+      }
+      c_scatter_rows_ += r.n;
+      c_launches_ += 1;
+      continue;
+    }
     if (!leaf_round(r)) {
       G = G_.at(off * 2 * H);
       gather(G, 2 * H, pool_.get(), 2 * H, d_child_ + off, r.n, 2 * H);
@@ -661,12 +678,34 @@ void Engine::lstm_forward() {
 void Engine::lstm_backward() {
   const int N = N_, H = cfg_.H;
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H;
-  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  const int fused = fused_rows();
+  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
+    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), Wh, H, 4 * H, stream_));
+    c_launches_ += 1;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
-    gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
     float *da = dxW_.at(off * 4 * H);
+    if (r.n <= fused) {
+      const bool leaf = leaf_round(r);
+      const int *child = leaf ? nullptr : d_child_ + off;
+      CAVS_TIMED(K_GATES, cavs_lstm_round_bwd_gates(dpool_.get(), d_pair_ + off, child, dret_folded ? d_dgo_ : dret_.at(off * H),
+                                                    dret_folded ? d_t2j_ + off : nullptr, gates_.at(off * 5 * H),
+                                                    leaf ? nullptr : G_.at(off * 2 * H), da, 4 * H, r.n, H, stream_));
+      c_gather_rows_ += r.n;
+      c_launches_ += 1;
+      if (!leaf) {
+        CAVS_TIMED(K_ROUND, cavs_round_bwd_children(da, 4 * H, 4 * H, UT_.get(), H, 1, child, dpool_.get(), 2 * H, r.n, H, stream_));
+        c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
+        c_scatter_rows_ += r.n;
+        c_launches_ += 1;
+      }
+      continue;
+    }
+    gather(r_dmsg_.get(), 2 * H, dpool_.get(), 2 * H, d_pair_ + off, r.n, 2 * H);
     if (leaf_round(r)) {
       CAVS_TIMED(K_GATES, cavs_lstm_gates_bwd(r_dmsg_.get(), dret_.at(off * H), gates_.at(off * 5 * H), nullptr, da, 4 * H,
                                 nullptr, r.n, H, stream_));
@@ -698,10 +737,27 @@ void Engine::treefc_forward() {
   const float *Bv = cfg_.use_bias ? param("Bv").w : nullptr;
   if (cfg_.use_x) gather(xs_.get(), H, d_x_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  const int fused = fused_rows();
+  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  float *go = out_folded_ ? fwd_out_ : nullptr;
   for (const Round &r : sched_.rounds) {
     const size_t off = r.offset;
     const float *xin = cfg_.use_x ? xs_.at(off * H) : nullptr;
     float *msg = msg_.at(off * H);
+    if (r.n <= fused) {  // one launch: Gather, [h_l;h_r]*W, activation, Scatter, Push/PopRet
+      if (leaf_round(r)) {
+        CAVS_TIMED(K_GATES, cavs_treefc_round_leaves_fwd(pool_.get(), d_pair_ + off, Bv, xin, msg, go, d_t2j_ + off, r.n, H, cfg_.act,
+                                                         stream_));
+      } else {
+        CAVS_TIMED(K_ROUND, cavs_treefc_round_fwd(pool_.get(), d_child_ + 2 * off, d_pair_ + off, W, Bv, xin, G_.at(2 * off * H), msg, go,
+                                                  d_t2j_ + off, r.n, H, cfg_.act, stream_));
+        c_round_flops_ += 2.0 * r.n * H * 2.0 * H;
+        c_gather_rows_ += 2.0 * r.n;
+      }
+      c_scatter_rows_ += r.n;
+      c_launches_ += 1;
+      continue;
+    }
     if (leaf_round(r)) {
       CAVS_TIMED(K_GATES, cavs_treefc_fwd(nullptr, Bv, xin, msg, r.n, H, cfg_.act, stream_));
     } else {
@@ -724,12 +780,31 @@ void Engine::treefc_forward() {
 void Engine::treefc_backward() {
   const int N = N_, H = cfg_.H;
   const float *W = param("W").w;
-  gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  const int fused = fused_rows();
+  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (fused > 0) {  // W^T [H, 2H]: the B operand of d[h_l;h_r] = dz * W^T, k-major
+    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), W, 2 * H, H, stream_));
+    c_launches_ += 1;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
-    gather(r_dmsg_.get(), H, dpool_.get(), H, d_pair_ + off, r.n, H);
     float *dz = dxW_.at(off * H);
+    if (r.n <= fused) {
+      CAVS_TIMED(K_GATES, cavs_treefc_round_bwd(dpool_.get(), d_pair_ + off, dret_folded ? d_dgo_ : dret_.at(off * H),
+                                                dret_folded ? d_t2j_ + off : nullptr, msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));
+      c_gather_rows_ += r.n;
+      c_launches_ += 1;
+      if (!leaf_round(r)) {
+        CAVS_TIMED(K_ROUND, cavs_round_bwd_children(dz, H, H, UT_.get(), 2 * H, 2, d_child_ + 2 * off, dpool_.get(), H, r.n, H, stream_));
+        c_round_flops_ += 2.0 * r.n * H * 2.0 * H;
+        c_scatter_rows_ += 2.0 * r.n;
+        c_launches_ += 1;
+      }
+      continue;
+    }
+    gather(r_dmsg_.get(), H, dpool_.get(), H, d_pair_ + off, r.n, H);
     CAVS_TIMED(K_GATES, cavs_treefc_bwd(r_dmsg_.get(), dret_.at(off * H), msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));
     c_launches_ += 1;
     if (leaf_round(r)) continue;

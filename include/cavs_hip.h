@@ -278,6 +278,33 @@ int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *chil
  * child[2b], child[2b+1].  UT = U_iou^T [3H,H] then U_f^T [H,H] (cavs_transpose). */
 int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *dF, const float *UT,
                                      const int *child, float *dpool, int n, int H, void *stream);
+/* The same construction for the chain LSTM (apps/paper/seq-lstm-cavs.cc:62-86; one child per
+ * vertex: child [n]; Wh [H,4H] blocks [i|f|u|o]; gates [n,5H] = [i|f|u|o|tanh c]; G [n,2H] the
+ * gathered predecessor) and for Tree-FC (apps/paper/tree-fc-cavs.cc:28-36; messages are h only:
+ * pool [*,H]; W [2H,H]; bias / x may be NULL; G [n,2H] = [h_l|h_r]; act 0 relu, 1 tanh). */
+int cavs_lstm_round_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                        const float *Wh, const float *bias, float *G, float *gates, float *msg,
+                        float *graph_out, const int *out_rows, int n, int H, void *stream);
+int cavs_lstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw,
+                               const float *bias, float *gates, float *msg, float *graph_out,
+                               const int *out_rows, int n, int H, void *stream);
+int cavs_lstm_round_bwd_gates(float *dpool, const int *pair, const int *child, const float *dret,
+                              const int *dret_rows, const float *gates, const float *G, float *da,
+                              int ld_da, int n, int H, void *stream);
+int cavs_treefc_round_fwd(float *pool, const int *child, const int *pair, const float *W,
+                          const float *bias, const float *x, float *G, float *msg, float *graph_out,
+                          const int *out_rows, int n, int H, int act, void *stream);
+int cavs_treefc_round_leaves_fwd(float *pool, const int *pair, const float *bias, const float *x,
+                                 float *msg, float *graph_out, const int *out_rows, int n, int H,
+                                 int act, void *stream);
+/* dz = act'(h) * (d msg read from dpool row pair[b] + d return value) */
+int cavs_treefc_round_bwd(const float *dpool, const int *pair, const float *dret, const int *dret_rows,
+                          const float *h, float *dz, int n, int H, int act, void *stream);
+/* Gradient of the gathered children's h, product and Scatter in one launch: for child p < nchild
+ * of slab row b, dpool[child[b*nchild+p]][0:H) = dA[b,0:K) * BT[0:K, p*H:(p+1)*H).  Chain LSTM:
+ * nchild 1, dA = da [n,4H], BT = Wh^T [4H,H].  Tree-FC: nchild 2, dA = dz [n,H], BT = W^T [H,2H]. */
+int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int ldb, int nchild,
+                            const int *child, float *dpool, int pool_width, int n, int H, void *stream);
 /* out [cols,rows] = in [rows,cols]^T */
 int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream);
 

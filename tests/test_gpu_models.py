@@ -194,24 +194,30 @@ def test_full_size_tree_lstm_properties():
 
 @pytest.mark.parametrize("H,limit", [(32, 0), (64, 0), (96, 0), (64, 20), (64, -1)])
 @pytest.mark.parametrize("pairing", ["reference", "rowid"])
-def test_fused_rounds_match_oracle(oracle, H, limit, pairing):
-    """Tree-LSTM with whole rounds as single launches: 70 trees give rounds above 64 rows
-    (32x32 tiles), between 17 and 64 (16x16 tiles, several row tiles per workgroup) and
-    down to one row.  limit=20 mixes fused and separate rounds in one step, -1 never fuses."""
-    w = small_workload("treelstm", 91, B=70, H=H, E=12, V=31, C=5)
-    print(f"[case] fused rounds H={H} limit={limit} pairing={pairing} N={w['N']}", flush=True)
-    want = oracle.model_step("treelstm", w["graph"], w["x"], w["labels"], w["params"], H=H, E=12, V=31, Cc=5,
-                             pairing=pairing)
-    s = session.Session("treelstm", H=H, E=12, V=31, C_=5, pairing=pairing, fused_round_rows=limit)
-    s.set_params(w["params"])
+@pytest.mark.parametrize("model,kw", CASES)
+def test_fused_rounds_match_oracle(oracle, model, kw, H, limit, pairing):
+    """Whole rounds as single launches for all three vertex functions: 70 samples give rounds
+    above 64 rows (32x32 tiles, or 16x16 with four wavefronts), between 17 and 64 (16x16 tiles)
+    and down to one row.  limit=20 mixes fused and separate rounds in one step, -1 never fuses."""
+    w = small_workload(model, 91, B=70, H=H, E=12, V=31, C=5)
+    E = H if model == "lstm" else 12
+    loss = "softmax" if model != "treefc" else "root_sq"
+    print(f"[case] fused rounds {model} {kw} H={H} limit={limit} pairing={pairing} N={w['N']}", flush=True)
+    want = oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=H, E=E, V=31, Cc=5, pairing=pairing,
+                             loss=loss, **kw)
+    s = session.Session(model, H=H, E=E, V=31, C_=5, pairing=pairing, fused_round_rows=limit, loss=loss, **kw)
+    names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
+             "treefc": ("W", "Bv") if kw.get("use_bias") else ("W",)}[model]
+    if loss == "softmax":
+        names += ("Wfc", "bfc")
+    s.set_params({k: w["params"][k] for k in names})
     s.step(w["graph"], w["x"], w["labels"], backward=True)
     got = dict(loss=s.fetch("loss"), graph_out=s.fetch("graph_out"), dgraph_out=s.fetch("dgraph_out"),
                msg_pool=s.fetch("msg_pool"), grads=s.grads(), trace=s.schedule_trace())
-    sizes = sorted({len(rd["jobs"]) if "jobs" in rd else 0 for rd in got["trace"]["fwd"]})
     fused_flops = s.counter("round_flops")
     s.close()
     compare(got, want)
-    assert (fused_flops > 0) == (limit >= 0), (fused_flops, sizes)
+    assert (fused_flops > 0) == (limit >= 0), fused_flops
 
 
 @pytest.mark.parametrize("model", ["treelstm", "lstm"])

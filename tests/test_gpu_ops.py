@@ -687,3 +687,28 @@ def test_column_sums_of_permuted_blocks(g, n, bw, perm):
     with pytest.raises(hip.CavsError, match="permutation"):
         hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * nb)(*([0] * nb)), 16, nbytes, 0) if nb > 1 else \
             hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * 1)(3), 16, nbytes, 0)
+
+
+@pytest.mark.parametrize("n,H,K,nchild", [(1, 32, 128, 1), (40, 64, 256, 1), (130, 32, 32, 2), (300, 64, 64, 2), (17, 96, 96, 2)])
+def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
+    """dpool[child[b*nchild+p]][0:H) = dA[b] * BT[:, p*H:(p+1)*H): product and Scatter in one launch."""
+    r = rng(n + H + K)
+    dA = r.bulk_normal(n * (K + 4)).reshape(n, K + 4)           # leading dimension wider than K
+    BT = (r.bulk_normal(K * nchild * H).reshape(K, nchild * H) / np.sqrt(K)).astype(np.float32)
+    rows = nchild * n + 7
+    mw = 2 * H if nchild == 1 else H
+    child = np.argsort(r.bulk_normal(rows))[: nchild * n].astype(np.int32)
+    if n > 2:
+        child[1] = -1
+    dpool = r.bulk_normal(rows * mw).reshape(rows, mw)
+    want = dpool.astype(np.float64).copy()
+    full = dA[:, :K].astype(np.float64) @ BT.astype(np.float64)  # [n, nchild*H]
+    for b in range(n):
+        for p in range(nchild):
+            c = child[b * nchild + p]
+            if c >= 0:
+                want[c, :H] = full[b, p * H:(p + 1) * H]
+    d = g.devf(dpool)
+    g.call("cavs_round_bwd_children", g.P(g.devf(dA)), K + 4, K, g.P(g.devf(BT)), nchild * H, nchild, g.P(g.devi(child)),
+           g.P(d), mw, n, H, g.stream())
+    close(g.host(d), want, "dpool", rtol=2e-4, atol=2e-5)
