@@ -81,7 +81,7 @@ def measure(a, workload, steps, warmup, n_pool):
     w0 = pool[0]
     kw = model_kwargs(w0)
     s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
-                        opt=session.OPT_BATCHING, **kw)
+                        opt=session.OPT_BATCHING, fused_round_rows=a.fused_round_rows, **kw)
     s.set_params(w0["params"])
     feeds = []
     for w in pool:  # inputs resident in HBM before the timed region
@@ -198,6 +198,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--host-feeds", action="store_true",
                     help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
+    ap.add_argument("--fused-round-rows", type=int, default=0,
+                    help="rounds of at most this many vertices run as fused launches (0: default limit, -1: never)")
     ap.add_argument("--also", default="C5",
                     help="a second workload measured with few steps and reported under 'also' (the large Tree-LSTM "
                          "configuration, where rounds are GEMM-sized); 'none' to skip")
