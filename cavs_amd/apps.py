@@ -44,10 +44,11 @@ class App:
     """model: treelstm | lstm | treefc | treefc_x.  opt: OPT_* bitmask, or -1 to only
     declare the program (no device)."""
 
-    def __init__(self, model, *, B, maxlen, H, E=0, V=0, C_=0, opt=session.OPT_BATCHING, lr=0.0,
+    def __init__(self, model, *, B, maxlen, H, E=0, V=0, C_=0, opt=session.OPT_BATCHING, lr=0.0, clip=0.0,
                  pairing="reference", allow_fused=True):
         a, _ = libs()
         self.model, self.B, self.maxlen, self.H, self.E, self.V, self.C = model, B, maxlen, H, E, V, C_
+        a.cavs_app_set_clip(C.c_float(clip))
         rc = a.cavs_app_create(model.encode(), B, maxlen, V, E, H, C_, opt, lr)
         if rc != 0:
             raise hip.CavsError(f"cavs_app_create({model}) -> {rc}")

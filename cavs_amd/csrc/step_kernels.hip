@@ -4,6 +4,8 @@
 // table, and the bias gradient (column sums of the four gate blocks) in one launch.
 // Every one of these is a few microseconds of HBM traffic; as separate library-style
 // launches their fixed costs add up to more than a round of the vertex function.
+#include <vector>
+
 #include "common.h"
 
 namespace cavs {
@@ -364,6 +366,103 @@ int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int 
   launch(colsum_part_kernel, dim3((w + 63) / 64, chunks), 256, 0, st, part, inp, ld, n, w, rpc);
   CAVS_LAUNCH_CHECK();
   launch(colsum_blocks_reduce_kernel, (w + 63) / 64, 256, 0, st, out, part, chunks, w, bw, map);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------ gradient clipping
+// ClipOpImpl (cavs/backend/op_impl_clip.cu:26-50): every gradient is scaled by
+// clip / max(sum_i ||g_i||_2, clip) -- the SUM of the tensors' norms, as the reference adds
+// them.  Three launches, all deterministic: partial sums of squares per tensor in fixed
+// chunks, one workgroup that adds them in index order and forms the factor, and the scaling.
+namespace cavs {
+
+constexpr int kClipParts = 64;
+
+struct ClipBatch {
+  float *g[kMaxTensors];
+  size_t n[kMaxTensors];
+  int count;
+};
+
+__global__ __launch_bounds__(256) void clip_sumsq_kernel(ClipBatch t, float *__restrict__ part) {
+  __shared__ float s[256];
+  const int k = blockIdx.y, p = blockIdx.x;
+  const size_t n = t.n[k], per = (n + kClipParts - 1) / kClipParts;
+  const size_t b = (size_t)p * per, e = b + per < n ? b + per : n;
+  float a = 0.f;
+  for (size_t i = b + threadIdx.x; i < e; i += 256) {
+    const float v = t.g[k][i];
+    a += v * v;
+  }
+  s[threadIdx.x] = a;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) s[threadIdx.x] += s[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) part[k * kClipParts + p] = s[0];
+}
+
+// factor[0] = clip / max(sum of norms, clip); factor[1] = the sum of norms (for inspection)
+__global__ void clip_factor_kernel(const float *__restrict__ part, int count, float clip, float base,
+                                   float *__restrict__ factor, int last) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float total = base;
+  for (int k = 0; k < count; k++) {
+    float ss = 0.f;
+    for (int p = 0; p < kClipParts; p++) ss += part[k * kClipParts + p];
+    total += sqrtf(ss);
+  }
+  factor[1] = total;
+  if (last) factor[0] = clip / fmaxf(total, clip);
+}
+
+__global__ void clip_scale_kernel(ClipBatch t, const float *__restrict__ factor) {
+  const float f = factor[0];
+  if (f == 1.f) return;
+  const int k = blockIdx.y;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < t.n[k]; i += stride) t.g[k][i] *= f;
+}
+
+}  // namespace cavs
+
+extern "C" {
+
+size_t cavs_clip_grads_workspace(int count) {
+  return count <= 0 ? 0 : ((size_t)cavs::kMaxTensors * cavs::kClipParts + 2) * sizeof(float);
+}
+
+int cavs_clip_grads(int count, float *const *g, const size_t *n, float clip, void *workspace, size_t workspace_bytes,
+                    void *stream) {
+  CAVS_REQUIRE(count >= 0 && clip > 0.f && (count == 0 || (g && n)), "cavs_clip_grads: bad arguments (count=%d clip=%g)", count, (double)clip);
+  if (count == 0) return CAVS_OK;
+  CAVS_REQUIRE(workspace && workspace_bytes >= cavs_clip_grads_workspace(count), "cavs_clip_grads: workspace of %zu bytes needed, %zu given",
+               cavs_clip_grads_workspace(count), workspace_bytes);
+  hipStream_t st = as_stream(stream);
+  float *part = static_cast<float *>(workspace), *factor = part + kMaxTensors * kClipParts;
+  // norms, eight tensors per pass; the running sum of norms is carried in factor[1]
+  std::vector<ClipBatch> batches;
+  for (int i = 0; i < count;) {
+    ClipBatch t{};
+    for (; i < count && t.count < kMaxTensors; i++) {
+      if (n[i] == 0) continue;
+      CAVS_REQUIRE(g[i], "cavs_clip_grads: null tensor %d", i);
+      t.g[t.count] = g[i];
+      t.n[t.count] = n[i];
+      t.count++;
+    }
+    if (t.count) batches.push_back(t);
+  }
+  if (batches.empty()) return CAVS_OK;
+  CAVS_REQUIRE(batches.size() == 1, "cavs_clip_grads: at most %d non-empty tensors", kMaxTensors);
+  const ClipBatch &t = batches[0];
+  launch(clip_sumsq_kernel, dim3(kClipParts, t.count), 256, 0, st, t, part);
+  launch(clip_factor_kernel, 1, 64, 0, st, (const float *)part, t.count, clip, 0.f, factor, 1);
+  launch(clip_scale_kernel, dim3((unsigned)num_cus() * 4, t.count), 256, 0, st, t, (const float *)factor);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

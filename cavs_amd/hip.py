@@ -83,6 +83,7 @@ _SIGS = {
     "cavs_profile_disarm": [_P],
     "cavs_fc_softmax_xent": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _P],
     "cavs_sgd_multi": [_I, _P, _P, _P, _F, _P],
+    "cavs_clip_grads": [_I, _P, _P, _F, _P, _Z, _P],
     "cavs_embed_sgd": [_P, _P, _P, _I, _I, _F, _P, _I, _P],
     "cavs_embed_zero_rows": [_P, _P, _I, _I, _P],
     "cavs_colsum_blocks": [_P, _P, _I, _I, _I, _I, _P, _P, _Z, _P],
@@ -92,9 +93,11 @@ _SIGS = {
     "cavs_schedule_frontier": [_P, _I, _P, _P, _P, _P, _P, _P, _P],
 }
 _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z,
-            "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z}
+            "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
+            "cavs_clip_grads_workspace": _Z}
 _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I],
-            "cavs_fc_softmax_xent_workspace": [_I, _I, _I], "cavs_colsum_blocks_workspace": [_I, _I, _I]}
+            "cavs_fc_softmax_xent_workspace": [_I, _I, _I], "cavs_colsum_blocks_workspace": [_I, _I, _I],
+            "cavs_clip_grads_workspace": [_I]}
 
 EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)
 EW_UNARY = dict(assign=0, neg=1, abs=2, square=3, sigmoid=4, tanh=5, relu=6)

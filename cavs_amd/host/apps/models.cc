@@ -158,6 +158,10 @@ extern "C" {
 
 // model: "treelstm" | "lstm" | "treefc" (reference app) | "treefc_x" (tanh + bias + input, sum of
 // squares at the roots).  Declares the program and opens a session.  One app per process at a time.
+// gradient clipping threshold of the optimizer the next cavs_app_create declares (0: none)
+static float g_clip = 0.f;
+void cavs_app_set_clip(float clip) { g_clip = clip; }
+
 int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, int C, int opt, float lr) {
   try {
     delete g_app;
@@ -209,7 +213,7 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       app->loss = app->graph_output.Reduce_sum();  // tree-fc-cavs.cc:96
       app->total = app->loss;
     }
-    app->train = app->loss.Optimizer({}, lr);
+    app->train = app->loss.Optimizer({}, lr, g_clip);
     if (opt >= 0) app->sess = std::make_unique<Session>(opt);  // opt < 0: declare only (no device needed)
     g_app = app.release();
     return 0;

@@ -722,7 +722,17 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       if (d.name() == "GraphOutput_grad") run_graph_output_grad(d); else exec(d, mainctx);
     }
     // SGD: w -= lr * g (cavs/backend/op_impl_sgd.cu); clipping is not on the measured path
-    if (g.opt.clip != 0.f) fail(CAVS_EUNSUPPORTED, "gradient clipping is not implemented");
+    if (g.opt.clip > 0.f) {  // Clip precedes SGD (cavs/midend/graph_util.cc, op_impl_clip.cu)
+      std::vector<float *> gp;
+      std::vector<size_t> gn;
+      for (auto &v : g.opt.vars) {
+        Tensor &gr = tensor(GetGradientName(v));
+        gp.push_back(gr.base);
+        gn.push_back(gr.count());
+      }
+      const size_t bytes = cavs_clip_grads_workspace((int)gp.size());
+      check(cavs_clip_grads((int)gp.size(), gp.data(), gn.data(), g.opt.clip, workspace(bytes), bytes, stream_));
+    }
     for (auto &v : g.opt.vars) {
       Tensor &w = tensor(v), &gr = tensor(GetGradientName(v));
       check(cavs_sgd(w.base, gr.base, g.opt.lr, w.count(), stream_));

@@ -229,6 +229,13 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
 /* SGD (cavs/backend/op_impl_sgd.cu) over `count` tensors in one launch; the arrays are host arrays. */
 int cavs_sgd_multi(int count, float *const *w, const float *const *g, const size_t *n, float lr,
                    void *stream);
+/* Clip (cavs/backend/op_impl_clip.cu:26-50): scales every gradient in place by
+ * clip / max(sum_i ||g_i||_2, clip) -- the sum of the tensors' 2-norms, as the reference adds
+ * them; at most 8 non-empty tensors per call; the arrays are host arrays.  After the call
+ * workspace[512] holds the factor and workspace[513] the sum of norms (floats). */
+size_t cavs_clip_grads_workspace(int count);
+int cavs_clip_grads(int count, float *const *g, const size_t *n, float clip, void *workspace,
+                    size_t workspace_bytes, void *stream);
 /* SGD of an embedding table restricted to the rows ids[0..n) (ids as floats, like
  * EmbeddingLookup).  Equal to the dense update when every other row of dtable is zero.  A row
  * listed several times is updated once: stamp [rows of the table] must start at zero and epoch

@@ -185,3 +185,23 @@ def test_reference_smoke_programs_print_their_known_values():
         np.testing.assert_allclose(np.array(e[:]), np.array(kat["fusion_E"]["expect"], np.float32), rtol=1e-6)
         np.testing.assert_allclose(np.array(yy[:]), np.array(kat["fusion_YY"]["expect"], np.float32), rtol=1e-6)
         assert n.value == expect_kernels
+
+
+def test_optimizer_with_gradient_clipping(oracle):
+    """Optimizer(vars, lr, clip): gradients are scaled by clip / max(sum of norms, clip) before
+    w -= lr * g (cavs/backend/op_impl_clip.cu); the threshold is chosen below the sum of norms."""
+    w = small_workload("treelstm", 87, B=4, H=8, E=6, V=19, C=3)
+    B, maxlen = w["graph"].shape
+    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc")
+    want = oracle_step(oracle, w, "treelstm")
+    norms = sum(float(np.sqrt((want["grads"]["d" + k].astype(np.float64) ** 2).sum())) for k in names)
+    clip, lr = 0.25 * norms, 0.5
+    a = apps.App("treelstm", B=B, maxlen=maxlen, H=8, E=6, V=19, C_=3, opt=session.OPT_BATCHING, lr=lr, clip=clip)
+    a.set_params(w["params"])
+    a.step(w["graph"], w["x"], w["labels"], train=True)
+    shapes = {"Emb": (19, 6), "W": (6, 32), "U": (4 * 64,), "Bv": (32,), "Wfc": (3, 8), "bfc": (3,)}
+    for k in names:
+        p0 = np.asarray(w["params"][k], np.float32).reshape(shapes[k])
+        step = np.float32(lr) * np.float32(0.25) * want["grads"]["d" + k].reshape(shapes[k])
+        close(a.grad(k, shapes[k], grad=False), p0 - step, f"{k} after a clipped step", rtol=3e-4, atol=3e-5)
+    a.close()

@@ -712,3 +712,29 @@ def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
     g.call("cavs_round_bwd_children", g.P(g.devf(dA)), K + 4, K, g.P(g.devf(BT)), nchild * H, nchild, g.P(g.devi(child)),
            g.P(d), mw, n, H, g.stream())
     close(g.host(d), want, "dpool", rtol=2e-4, atol=2e-5)
+
+
+def test_gradient_clipping_by_the_sum_of_norms(g):
+    """Clip of the reference: every tensor times clip / max(sum of the tensors' 2-norms, clip)."""
+    import ctypes as C
+
+    r = rng(17)
+    sizes = [5, 70000, 0, 333, 1]
+    gs = [r.bulk_normal(max(k, 1))[:k] for k in sizes]
+    total = sum(float(np.sqrt((a.astype(np.float64) ** 2).sum())) for a in gs)
+    nb = hip.lib().cavs_clip_grads_workspace(len(sizes))
+    for clip in (0.5 * total, 10 * total):            # active, then inactive (factor exactly 1)
+        ws = g.zeros(nb // 4)
+        dg = [g.devf(a) if len(a) else None for a in gs]
+        pg = (C.c_void_p * len(sizes))(*[g.P(t) for t in dg])
+        pn = (C.c_size_t * len(sizes))(*sizes)
+        g.call("cavs_clip_grads", len(sizes), pg, pn, clip, g.P(ws), nb, g.stream())
+        factor, norm_sum = g.host(ws)[512], g.host(ws)[513]
+        assert abs(norm_sum - total) <= 1e-5 * total
+        want = clip / max(total, clip)
+        assert abs(factor - want) <= 1e-6
+        for a, t in zip(gs, dg):
+            if len(a):
+                close(g.host(t), a * np.float32(factor), "scaled gradient", rtol=1e-6, atol=1e-7)
+    with pytest.raises(hip.CavsError, match="bad arguments"):
+        hip.call("cavs_clip_grads", 1, 16, 16, 0.0, 16, nb, 0)
