@@ -65,10 +65,17 @@ def cpu_baseline(w, budget_s=12.0):
         el = time.perf_counter() - t0
         if el > budget_s or steps >= 400 or el + el / steps > 1.5 * budget_s:
             break
+    # the same on one thread (a bounded sample: two steps)
+    t1 = time.perf_counter()
+    for _ in range(2):
+        pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **dict(args, threads=1))
+    el1 = time.perf_counter() - t1
     return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port",
                 sample=f"{steps} full fwd+bwd step(s) of the {w['name']} batch (B={w['B']}, N={w['N']}) "
                        f"in {el:.1f} s with {threads} OpenMP threads; CPU restatement of the reference's "
-                       "semantics (the reference has no CPU kernels)")
+                       "semantics (the reference has no CPU kernels)",
+                single_thread=dict(value=round(w["B"] * 2 / el1, 3), unit="samples/s", cores=1,
+                                   sample=f"2 steps of the same batch in {el1:.1f} s"))
 
 
 def measure(a, workload, steps, warmup, n_pool):
@@ -135,8 +142,10 @@ def measure(a, workload, steps, warmup, n_pool):
                      kernel="sgemm_mfma_kernel / sgemm_skinny_kernel (x*W, weight-gradient and head GEMMs of a step"
                             "; also the recurrent products of rounds too large for the fused kernels)"),
         "round": dict(ms=round_ms, n=round_n, flops=rflops,
-                      kernel="treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel (one launch per round: "
-                             "gather + recurrent products + gates + scatter)"),
+                      kernel={"treelstm": "treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel",
+                              "lstm": "lstm_round_fwd_kernel / round_bwd_children_kernel",
+                              "treefc": "treefc_round_fwd_kernel / round_bwd_children_kernel"}[w0["model"]] +
+                             " (one launch per round: gather + recurrent products + gates + scatter)"),
     }
     for v in mfma.values():
         v["tf"] = v["flops"] / (v["ms"] * 1e-3) / 1e12 if v["ms"] else 0.0
@@ -200,9 +209,9 @@ def main():
                     help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
     ap.add_argument("--fused-round-rows", type=int, default=0,
                     help="rounds of at most this many vertices run as fused launches (0: default limit, -1: never)")
-    ap.add_argument("--also", default="C5",
-                    help="a second workload measured with few steps and reported under 'also' (the large Tree-LSTM "
-                         "configuration, where rounds are GEMM-sized); 'none' to skip")
+    ap.add_argument("--also", default="C1,C2,C4,C5",
+                    help="further workloads measured with few steps and reported under 'also' (C5 is the large "
+                         "Tree-LSTM configuration, where rounds are GEMM-sized); 'none' to skip")
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs the F-over-G path on one GPU; instance graphs shard by sample "
@@ -219,9 +228,14 @@ def main():
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": res["config"], "roofline": res["roofline"], "kernels": res["kernels"], "timers_ms": res["timers_ms"],
     }
-    if a.also.lower() != "none" and a.also != a.workload:
-        also, _ = measure(a, a.also, 10, 3, 2)
-        out["also"] = {a.also: {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}}
+    if a.also.lower() != "none":
+        out["also"] = {}
+        for name in a.also.split(","):
+            if name == a.workload:
+                continue
+            big = name == "C5"
+            also, _ = measure(a, name, 10 if big else 30, 3 if big else 5, 2 if big else 4)
+            out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
     print(json.dumps(out))
