@@ -116,6 +116,12 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise CavsError(f"{LIB_PATH} is missing: build it with `python -m cavs_amd.build` "
                             "(there is no CPU fallback)")
+        # PyTorch ships its own HIP runtime; a process that uses both must load PyTorch's first,
+        # or the two runtimes each try to own the device and the second one finds none
+        try:
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         l = C.CDLL(LIB_PATH)
         for name, args in _SIGS.items():
             fn = getattr(l, name)
