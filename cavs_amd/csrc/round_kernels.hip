@@ -414,57 +414,79 @@ __global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel
 #pragma unroll
     for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
 
-  // One loop over the hidden index k: the three column blocks of [d_i|d_o|d_u] against the
-  // three row blocks of U_iou^T, and d_fl, d_fr against U_f^T -- five MFMAs per k step into
-  // three accumulators, the same shape as the forward kernel's loop.
   constexpr int S = GK * UG;
-  const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
-  const int kb = ks * kper, ke = min(H, kb + kper);
-  struct Frag {
-    float4 a[UG][5];   // d_i, d_o, d_u, d_fl, d_fr at k
-    float b[UG][4][4]; // U_iou^T rows k, H+k, 2H+k and U_f^T row k
-  };
-  auto fetch = [&](int k0, Frag &f) {
+  {  // P0: K = 3H
+    const int K = 3 * H;
+    const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
+    const int kb = ks * kper, ke = min(K, kb + kper);
+    struct Frag {
+      float4 a[UG];
+      float b[UG][4];
+    };
+    auto fetch = [&](int k0, Frag &f) {
 #pragma unroll
-    for (int u = 0; u < UG; u++) {
-      const int kk = k0 + GK * u + 4 * slot;
-      const bool kin = kk < ke;
+      for (int u = 0; u < UG; u++) {
+        const int kk = k0 + GK * u + 4 * slot;
+        const bool kin = kk < ke;
+        f.a[u] = (kin && rin) ? ld4(px + kk) : zero4();
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        const long k = kin ? kk + c : 0;
-        f.b[u][0][c] = kin ? UTio[k * H] : 0.f;
-        f.b[u][1][c] = kin ? UTio[(k + H) * H] : 0.f;
-        f.b[u][2][c] = kin ? UTio[(k + 2 * H) * H] : 0.f;
-        f.b[u][3][c] = kin ? UTf[k * H] : 0.f;
+        for (int c = 0; c < 4; c++) f.b[u][c] = kin ? UTio[(long)(kk + c) * H] : 0.f;
       }
-      const bool in = kin && rin;
-      f.a[u][0] = in ? ld4(px + kk) : zero4();
-      f.a[u][1] = in ? ld4(px + H + kk) : zero4();
-      f.a[u][2] = in ? ld4(px + 2 * H + kk) : zero4();
-      f.a[u][3] = in ? ld4(pfl + kk) : zero4();
-      f.a[u][4] = in ? ld4(pfr + kk) : zero4();
+    };
+    auto multiply = [&](const Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc[0] = M::mma(elem(f.a[u], c), f.b[u][c], acc[0]);
+    };
+    Frag f0, f1;
+    if (kb < ke) fetch(kb, f0);
+    for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+      if (k0 + S < ke) fetch(k0 + S, f1);
+      multiply(f0);
+      if (k0 + S < ke) {
+        if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+        multiply(f1);
+      }
     }
-  };
-  auto multiply = [&](const Frag &f) {
+  }
+  {  // P1, P2: K = H, one B operand for both
+    const int K = H;
+    const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
+    const int kb = ks * kper, ke = min(K, kb + kper);
+    struct Frag {
+      float4 l[UG], r[UG];
+      float b[UG][4];
+    };
+    auto fetch = [&](int k0, Frag &f) {
 #pragma unroll
-    for (int u = 0; u < UG; u++)
+      for (int u = 0; u < UG; u++) {
+        const int kk = k0 + GK * u + 4 * slot;
+        const bool kin = kk < ke;
+        f.l[u] = (kin && rin) ? ld4(pfl + kk) : zero4();
+        f.r[u] = (kin && rin) ? ld4(pfr + kk) : zero4();
 #pragma unroll
-      for (int c = 0; c < 4; c++) {
-        acc[0] = M::mma(elem(f.a[u][0], c), f.b[u][0][c], acc[0]);
-        acc[1] = M::mma(elem(f.a[u][3], c), f.b[u][3][c], acc[1]);
-        acc[2] = M::mma(elem(f.a[u][4], c), f.b[u][3][c], acc[2]);
-        acc[0] = M::mma(elem(f.a[u][1], c), f.b[u][1][c], acc[0]);
-        acc[0] = M::mma(elem(f.a[u][2], c), f.b[u][2][c], acc[0]);
+        for (int c = 0; c < 4; c++) f.b[u][c] = kin ? UTf[(long)(kk + c) * H] : 0.f;
       }
-  };
-  Frag f0, f1;
-  if (kb < ke) fetch(kb, f0);
-  for (int k0 = kb; k0 < ke; k0 += 2 * S) {
-    if (k0 + S < ke) fetch(k0 + S, f1);
-    multiply(f0);
-    if (k0 + S < ke) {
-      if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
-      multiply(f1);
+    };
+    auto multiply = [&](const Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          acc[1] = M::mma(elem(f.l[u], c), f.b[u][c], acc[1]);
+          acc[2] = M::mma(elem(f.r[u], c), f.b[u][c], acc[2]);
+        }
+    };
+    Frag f0, f1;
+    if (kb < ke) fetch(kb, f0);
+    for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+      if (k0 + S < ke) fetch(k0 + S, f1);
+      multiply(f0);
+      if (k0 + S < ke) {
+        if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+        multiply(f1);
+      }
     }
   }
 
