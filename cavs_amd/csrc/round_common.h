@@ -77,14 +77,14 @@ struct RoundPlan {
   int tile, waves;
 };
 // Measured on MI355X at H=512: the 16x16 tile wins while a round is too small to give every
-// CU a 32x32 tile (its workgroups finish in 8 us against 20), eight wavefronts per workgroup
-// up to 64 rows, four beyond (several workgroups then share a CU and overlap their latencies).
+// CU several 32x32 tiles (600 rows: 32 us against 40).  Eight wavefronts per workgroup up to
+// 64 rows (shortest latency chain); four beyond, compiled for four workgroups per CU so that
+// their latency chains overlap; 32x32 tiles above a thousand rows, where operand reuse counts.
 inline RoundPlan plan_round(int n) {
   if (n <= 64) return {16, 8};
-  if (n <= 200) return {16, 4};
+  if (n <= 1024) return {16, 4};
   return {32, 8};
 }
-
 
 }  // namespace cavs
 #endif

@@ -42,12 +42,14 @@ struct RoundFwdArgs {
 };
 
 template <int TILE, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
   constexpr int RT = 1, kRoundThreads = WAVES * 64;
   constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 5, NR = M::NR;
-  constexpr int UG = 2;  // k-groups per pipeline stage
+  // k-groups per pipeline stage; the four-wavefront 16x16 variant keeps one, to stay within the
+  // registers of four workgroups per CU
+  constexpr int UG = (TILE == 16 && WAVES == 4) ? 1 : 2;
   constexpr int NREG = Regions<TILE, KS>::N, RSZ = RT * NP * NR * 64;
   __shared__ float red[NREG * RSZ];
 
@@ -368,12 +370,12 @@ struct RoundBwdChildArgs {
 };
 
 template <int TILE, int WAVES>
-__global__ __launch_bounds__(WAVES * 64) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
+__global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
   constexpr int RT = 1, kRoundThreads = WAVES * 64;
   constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 3, NR = M::NR;
-  constexpr int UG = 2;
+  constexpr int UG = (TILE == 16 && WAVES == 4) ? 1 : 2;
   constexpr int NREG = Regions<TILE, KS>::N, RSZ = RT * NP * NR * 64;
   __shared__ float red[NREG * RSZ];
 
