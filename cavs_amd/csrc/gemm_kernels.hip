@@ -335,6 +335,24 @@ static GemmPlan plan_gemm(int tA, int tB, int M, int N, int K, bool skinny_allow
     p.tiles = t128;
     return p;
   }
+  // Tall-K products whose large tiles give each CU one workgroup or less (the deferred weight
+  // gradients of big batches: 8x32 tiles, K = all rows): one workgroup per CU cannot hide the
+  // latency of its own global loads, so K is split until about three share a CU.
+  if (allow_split && 4 * t128 >= cus && K >= 4096) {
+    long s = (3 * cus + t128 - 1) / t128;
+    if (s > K / 1024) s = K / 1024;
+    if (s > 1) {
+      int kchunk = (int)(((K + s - 1) / s + 31) / 32 * 32);
+      int splits = (K + kchunk - 1) / kchunk;
+      if (splits > 1) {
+        p.kind = GemmPlan::TILE128;
+        p.tiles = t128;
+        p.splits = splits;
+        p.kchunk = kchunk;
+        return p;
+      }
+    }
+  }
   p.kind = GemmPlan::TILE64;
   p.tiles = t64;
   if (t64 >= 2 * cus || K < 64) return p;
