@@ -738,3 +738,35 @@ def test_gradient_clipping_by_the_sum_of_norms(g):
                 close(g.host(t), a * np.float32(factor), "scaled gradient", rtol=1e-6, atol=1e-7)
     with pytest.raises(hip.CavsError, match="bad arguments"):
         hip.call("cavs_clip_grads", 1, 16, 16, 0.0, 16, nb, 0)
+
+
+def test_kernel_stamped_timing_probe(g):
+    """cavs_profile_arm: the kernels of the next entry points stamp start / stop themselves;
+    disarm reports whether anything was launched."""
+    import ctypes as C
+
+    e0, e1 = C.c_void_p(), C.c_void_p()
+    hip.call("cavs_event_create", C.byref(e0))
+    hip.call("cavs_event_create", C.byref(e1))
+    n = 1 << 22
+    a, out = g.zeros(n, fill=1.0), g.zeros(n)
+    launched = C.c_int(-1)
+    hip.call("cavs_profile_arm", e0, e1)
+    hip.call("cavs_profile_disarm", C.byref(launched))
+    assert launched.value == 0                       # armed, nothing launched
+    hip.call("cavs_profile_arm", e0, e1)
+    g.call("cavs_scale", g.P(out), g.P(a), 2.0, n, g.stream())
+    g.call("cavs_scale", g.P(out), g.P(out), 2.0, n, g.stream())   # stop moves to the last kernel
+    hip.call("cavs_profile_disarm", C.byref(launched))
+    assert launched.value == 1
+    ms = C.c_float(-1)
+    hip.call("cavs_event_elapsed_ms", C.byref(ms), e0, e1)
+    # two passes over 16 MiB in and out: at least 8 us at 8 TB/s, and far below a millisecond
+    assert 0.008 <= ms.value < 1.0, ms.value
+    np.testing.assert_array_equal(g.host(out)[:4], np.full(4, 4.0, np.float32))
+    g.call("cavs_scale", g.P(out), g.P(a), 3.0, n, g.stream())     # disarmed: plain launch
+    assert g.host(out)[0] == 3.0
+    hip.call("cavs_event_destroy", e0)
+    hip.call("cavs_event_destroy", e1)
+    with pytest.raises(hip.CavsError, match="null event"):
+        hip.call("cavs_profile_arm", None, None)
