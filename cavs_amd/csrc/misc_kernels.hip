@@ -89,15 +89,24 @@ __global__ void embed_bwd_kernel(float *__restrict__ dtable, const float *__rest
     lead[tid] = l;  // first row of the chunk with this id
   }
   __syncthreads();
+  // all rows of a column are in flight before the sums; rows that share an id are added in
+  // row order into the first of them
   for (int c = tid; c < E; c += blockDim.x) {
+    float v[kEmbedChunk];
 #pragma unroll
-    for (int r = 0; r < kEmbedChunk; r++) {
-      if (lead[r] != r || off[r] < 0) continue;
-      float s = dy[(long)(row0 + r) * ld_dy + c];
-      for (int q = r + 1; q < kEmbedChunk; q++)
-        if (lead[q] == r) s += dy[(long)(row0 + q) * ld_dy + c];
-      unsafeAtomicAdd(dtable + off[r] + c, s);
+    for (int r = 0; r < kEmbedChunk; r++) v[r] = off[r] >= 0 ? dy[(long)(row0 + r) * ld_dy + c] : 0.f;
+#pragma unroll
+    for (int r = 1; r < kEmbedChunk; r++) {
+      const int l = lead[r];
+      if (l != r) {
+#pragma unroll
+        for (int q = 0; q < r; q++)
+          if (q == l) v[q] += v[r];
+      }
     }
+#pragma unroll
+    for (int r = 0; r < kEmbedChunk; r++)
+      if (lead[r] == r && off[r] >= 0) unsafeAtomicAdd(dtable + off[r] + c, v[r]);
   }
 }
 

@@ -178,20 +178,32 @@ __global__ void embed_sgd_kernel(float *__restrict__ table, const float *__restr
                                  const float *__restrict__ ids, int n, int E, float lr, int *__restrict__ stamp,
                                  int epoch) {
   __shared__ int row[kSgdChunk];
-  __shared__ int owner[kSgdChunk];
+  __shared__ long owned[kSgdChunk];
+  __shared__ int n_owned;
   const int v0 = blockIdx.x * kSgdChunk, tid = threadIdx.x;
   if (tid < kSgdChunk) row[tid] = v0 + tid < n ? (int)ids[v0 + tid] : -1 - tid;
+  if (tid == 0) n_owned = 0;
   __syncthreads();
   if (tid < kSgdChunk) {
     bool first = row[tid] >= 0;
     for (int r = 0; r < tid; r++) first = first && row[r] != row[tid];
-    owner[tid] = first && atomicMax(stamp + row[tid], epoch) < epoch;
+    if (first && atomicMax(stamp + row[tid], epoch) < epoch)
+      owned[atomicAdd(&n_owned, 1)] = (long)(int)(ids[v0 + tid] * (float)E);
   }
   __syncthreads();
-  for (int r = 0; r < kSgdChunk; r++) {
-    if (!owner[r]) continue;
-    const long off = (long)(int)(ids[v0 + r] * (float)E);
-    for (int c = tid; c < E; c += blockDim.x) table[off + c] -= lr * dtable[off + c];
+  // every owned row of a column is in flight before the first store
+  const int cnt = n_owned;
+  for (int c = tid; c < E; c += blockDim.x) {
+    float t[kSgdChunk], d[kSgdChunk];
+#pragma unroll
+    for (int r = 0; r < kSgdChunk; r++)
+      if (r < cnt) {
+        t[r] = table[owned[r] + c];
+        d[r] = dtable[owned[r] + c];
+      }
+#pragma unroll
+    for (int r = 0; r < kSgdChunk; r++)
+      if (r < cnt) table[owned[r] + c] = t[r] - lr * d[r];
   }
 }
 

@@ -246,3 +246,31 @@ def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     for k in names:
         close(s.param(k, p[k].shape), p[k], f"{k} after the steps", rtol=3e-4, atol=3e-5)
     s.close()
+
+
+@pytest.mark.parametrize("kind", ["trees", "tokens"])
+def test_training_step_on_reader_batches(oracle, kind):
+    """The text readers (cavs_amd/data.py) feed the session directly: the fixture corpora
+    through one training step, against the oracle on the same arrays."""
+    import os
+
+    from cavs_amd import data
+
+    golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    if kind == "trees":
+        r = data.TreeReader(*[os.path.join(golden, "sst_tiny", f) for f in ("sents_idx.txt", "labels.txt", "parents.txt")],
+                            batch=3, max_vertices=9, max_words=5)
+        graph, x, labels = r.next_batch(pack_inputs=True)
+        model, V, C = "treelstm", 21, 5
+    else:
+        r = data.PtbReader(os.path.join(golden, "ptb_tiny.txt"), batch=2, max_length=5)
+        graph, x, labels = r.batch_at(2)
+        model, V, C = "lstm", 23, 23
+    N = sum(int(np.argmax(row == -1)) + 1 for row in graph)  # a sample ends at its first -1, the root
+    x, labels = x[:N].copy(), labels[:N].copy()
+    labels[labels < 0] = 0  # the last token of a sentence has no successor: class 0
+    w = small_workload(model, 77, H=16, E=16, V=V, C=C)
+    w.update(graph=graph, x=x, labels=labels, N=N)
+    print(f"[case] reader kind={kind} N={N}", flush=True)
+    got, want = run_both(oracle, w)
+    compare(got, want)
