@@ -310,7 +310,7 @@ __global__ __launch_bounds__(W * 64) void sgemm_skinny_kernel(GemmArgs g) {
 }
 
 struct GemmPlan {
-  enum Kind { TILE128, TILE64, SKINNY, T64K16, T128x64, T64x128 } kind;
+  enum Kind { TILE128, TILE64, SKINNY } kind;
   int splits;   // > 1: partial tiles to the workspace + reduce kernel (TILE64 only)
   int kchunk;
   long tiles;
@@ -329,19 +329,6 @@ static GemmPlan plan_gemm(int tA, int tB, int M, int N, int K, bool skinny_allow
   const long t64 = (long)((M + 63) / 64) * ((N + 63) / 64);
   p.splits = 1;
   p.kchunk = K > 0 ? K : 1;
-  if (const char *e = getenv("CAVS_GEMM_PLAN")) {  // EXPERIMENT
-    int kind = 0, s = 1;
-    sscanf(e, "%d:%d", &kind, &s);
-    p.kind = (GemmPlan::Kind)kind;
-    int bm = (kind == 0 || kind == 4) ? 128 : 64, bn = (kind == 0 || kind == 5) ? 128 : 64;
-    p.tiles = (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
-    if (s > 1 && allow_split) {
-      int kchunk = (int)(((K + s - 1) / s + 31) / 32 * 32);
-      int splits = (K + kchunk - 1) / kchunk;
-      if (splits > 1) { p.splits = splits; p.kchunk = kchunk; }
-    }
-    return p;
-  }
   // the large tile needs at least two rounds of workgroups to hide its ragged last round
   if (t128 >= 2 * cus) {
     p.kind = GemmPlan::TILE128;
@@ -465,12 +452,6 @@ static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float 
   bool vec = vec_path_ok(g, tA, tB);
   if (p.kind == GemmPlan::TILE128)
     launch_tile<128, 128, 16>(g, tA, tB, vec, p, st);
-  else if (p.kind == GemmPlan::T64K16)
-    launch_tile<64, 64, 16>(g, tA, tB, vec, p, st);
-  else if (p.kind == GemmPlan::T128x64)
-    launch_tile<128, 64, 16>(g, tA, tB, vec, p, st);
-  else if (p.kind == GemmPlan::T64x128)
-    launch_tile<64, 128, 16>(g, tA, tB, vec, p, st);
   else
     launch_tile<64, 64, 32>(g, tA, tB, vec, p, st);
   CAVS_LAUNCH_CHECK();
