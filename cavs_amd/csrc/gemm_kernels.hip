@@ -13,6 +13,8 @@
 // kernel whose wavefronts split K inside the workgroup, tall-K ones (the deferred
 // weight gradients) split K over workgroups with the partials reduced in a fixed
 // order by a second kernel.
+#include <algorithm>
+
 #include "common.h"
 
 namespace cavs {
@@ -108,19 +110,19 @@ __device__ inline int xcd_remap(int l, int total) {
   return xcd * per + (xcd < rem ? xcd : rem) + local;
 }
 
+// One BM x BN tile of C (or of split `z` of its K range) by the calling workgroup.  `t` is the
+// tile's index, row-major over the tiles of C; As / Bs are the workgroup's two LDS panels of
+// 2 * BK * (BM + PAD) and 2 * BK * (BN + PAD) floats.
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
-__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
+__device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float *__restrict__ As_, float *__restrict__ Bs_) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int LDA = BM + PAD, LDB = BN + PAD;
-  __shared__ __attribute__((aligned(16))) float As[2][BK * LDA];
-  __shared__ __attribute__((aligned(16))) float Bs[2][BK * LDB];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tilesN = (g.N + BN - 1) / BN, tilesM = (g.M + BM - 1) / BM;
-  const int t = xcd_remap(blockIdx.x, tilesM * tilesN);
+  const int tilesN = (g.N + BN - 1) / BN;
   const int m0 = (t / tilesN) * BM, n0 = (t % tilesN) * BN;
-  const int kbeg = blockIdx.y * g.kchunk;
+  const int kbeg = z * g.kchunk;
   const int kend = min(g.K, kbeg + g.kchunk);
 
   TileLoader<BM, BK, !TA, VEC> la;
@@ -138,8 +140,8 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
   if (nk > 0) {
     la.load(g.A, g.lda, m0, kbeg, g.M, kend, tid);
     lb.load(g.B, g.ldb, n0, kbeg, g.N, kend, tid);
-    la.store(As[0], tid);
-    lb.store(Bs[0], tid);
+    la.store(As_, tid);
+    lb.store(Bs_, tid);
   }
   __syncthreads();
   const int arow = wm * WM + (lane & 31), brow = wn * WN + (lane & 31), khalf = lane >> 5;
@@ -149,7 +151,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
       la.load(g.A, g.lda, m0, kbeg + (kt + 1) * BK, g.M, kend, tid);
       lb.load(g.B, g.ldb, n0, kbeg + (kt + 1) * BK, g.N, kend, tid);
     }
-    const float *as = As[cur], *bs = Bs[cur];
+    const float *as = As_ + cur * (BK * LDA), *bs = Bs_ + cur * (BK * LDB);
 #pragma unroll
     for (int kk = 0; kk < BK; kk += 2) {
       float a[TM], b[TN];
@@ -164,8 +166,8 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < nk) {
-      la.store(As[cur ^ 1], tid);
-      lb.store(Bs[cur ^ 1], tid);
+      la.store(As_ + (cur ^ 1) * (BK * LDA), tid);
+      lb.store(Bs_ + (cur ^ 1) * (BK * LDB), tid);
     }
     __syncthreads();
   }
@@ -183,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
         const int row = m0 + wm * WM + 32 * i + 8 * (r / 4) + 4 * khalf + (r % 4);
         if (row >= g.M) continue;
         if (g.ws) {  // split K: park the partial sum, the reduce kernel finishes the job
-          g.ws[((long)blockIdx.y * g.M + row) * g.N + col] = acc[i][j][r];
+          g.ws[((long)z * g.M + row) * g.N + col] = acc[i][j][r];
           continue;
         }
         float v = g.alpha * acc[i][j][r];
@@ -194,6 +196,70 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
     }
 }
 
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+__global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
+  __shared__ __attribute__((aligned(16))) float As[2 * BK * (BM + PAD)];
+  __shared__ __attribute__((aligned(16))) float Bs[2 * BK * (BN + PAD)];
+  const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+  gemm_tile<BM, BN, BK, TA, TB, VEC>(g, xcd_remap(blockIdx.x, tiles), blockIdx.y, As, Bs);
+}
+
+// Several independent products in one launch (the deferred weight gradients of a step and the
+// embedding gradient's product): alone, each of them is a single round of workgroups that all
+// load, multiply and store at the same time; together their phases overlap and the chip sees
+// one long launch.  Workgroup b belongs to product p with first[p] <= b < first[p+1] (each
+// product's share is padded to a multiple of 8, so that b % 8 is the XCD within the share as
+// well); within the share, tile = local % tiles[p] and K split = local / tiles[p].
+constexpr int kGroupMax = 4;
+struct GemmGroup {
+  GemmArgs g[kGroupMax];
+  int first[kGroupMax + 1];
+  int tiles[kGroupMax];
+  int splits[kGroupMax];
+  int form[kGroupMax];  // transA * 2 + transB
+  int count;
+};
+
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void sgemm_group_kernel(GemmGroup G) {
+  constexpr int BM = 64, BN = 64, BK = 32;
+  __shared__ __attribute__((aligned(16))) float As[2 * BK * (BM + PAD)];
+  __shared__ __attribute__((aligned(16))) float Bs[2 * BK * (BN + PAD)];
+  int p = 0;
+  while (p + 1 < G.count && (int)blockIdx.x >= G.first[p + 1]) p++;
+  const int local = blockIdx.x - G.first[p];
+  const int share = G.tiles[p] * G.splits[p];
+  const int padded = G.first[p + 1] - G.first[p];
+  const int w = xcd_remap(local, padded);
+  if (w >= share) return;
+  const int t = w % G.tiles[p], z = w / G.tiles[p];
+  const GemmArgs &g = G.g[p];
+  switch (G.form[p]) {
+    case 0: gemm_tile<BM, BN, BK, false, false, VEC>(g, t, z, As, Bs); break;
+    case 1: gemm_tile<BM, BN, BK, false, true, VEC>(g, t, z, As, Bs); break;
+    case 2: gemm_tile<BM, BN, BK, true, false, VEC>(g, t, z, As, Bs); break;
+    default: gemm_tile<BM, BN, BK, true, true, VEC>(g, t, z, As, Bs); break;
+  }
+}
+
+// the split products of a group, reduced in one launch (same fixed order as splitk_reduce_kernel)
+__global__ void splitk_reduce_group_kernel(GemmGroup R) {
+  // first[] counts 256-thread workgroups per product here
+  int p = 0;
+  while (p + 1 < R.count && (int)blockIdx.x >= R.first[p + 1]) p++;
+  const GemmArgs &g = R.g[p];
+  const int splits = R.splits[p];
+  long idx = (long)(blockIdx.x - R.first[p]) * blockDim.x + threadIdx.x;
+  long total = (long)g.M * g.N;
+  if (idx >= total) return;
+  float acc = 0.f;
+  for (int z = 0; z < splits; z++) acc += g.ws[(long)z * total + idx];
+  int r = (int)(idx / g.N), c = (int)(idx % g.N);
+  float v = g.alpha * acc;
+  if (g.beta != 0.f) v += g.beta * g.C[r * g.ldc + c];
+  if (g.D) v += g.D[(long)(r >> g.dshift) * g.ldd + c];
+  g.C[r * g.ldc + c] = v;
+}
 
 // C = alpha * sum_z ws[z] + beta * C (+ D rows), z ascending: a fixed order, so the
 // result does not depend on how the workgroups were scheduled.
@@ -463,11 +529,116 @@ static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float 
   return CAVS_OK;
 }
 
+// Plans a group: every product on the 64x64 tile, K split so that all workgroups of the group
+// together are about four per CU (what a CU holds at once), each with at least 256 of K.
+static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_bytes, size_t *need_out, void *stream) {
+  CAVS_REQUIRE(count >= 0 && count <= kGroupMax, "cavs_sgemm_group: %d products, at most %d", count, kGroupMax);
+  CAVS_REQUIRE(count == 0 || d, "cavs_sgemm_group: null descriptors");
+  GemmGroup G{}, R{};
+  double work = 0;
+  long tiles[kGroupMax];
+  bool alone[kGroupMax];
+  int grouped = 0;
+  size_t most = 0;
+  for (int p = 0; p < count; p++) {
+    const cavs_gemm_desc &q = d[p];
+    if (!need_out) {
+      int rc = check_gemm("cavs_sgemm_group", q.transA, q.transB, q.M, q.N, q.K, q.A, q.lda, q.B, q.ldb, q.C, q.ldc);
+      if (rc) return rc;
+    }
+    CAVS_REQUIRE(q.M >= 0 && q.N >= 0 && q.K >= 0, "cavs_sgemm_group: negative dimension in product %d", p);
+    tiles[p] = (long)((q.M + 63) / 64) * ((q.N + 63) / 64);
+    // a product that fills the chip with large tiles by itself is better off on them, alone
+    alone[p] = q.M > 0 && q.N > 0 && plan_gemm(q.transA, q.transB, q.M, q.N, q.K, false, true).kind == GemmPlan::TILE128;
+    if (!alone[p] && q.M > 0 && q.N > 0) grouped++;
+  }
+  for (int p = 0; p < count; p++) {
+    const cavs_gemm_desc &q = d[p];
+    if (q.M == 0 || q.N == 0) continue;
+    if (!alone[p] && grouped >= 2) {
+      work += (double)tiles[p] * q.K;
+      continue;
+    }
+    alone[p] = true;
+    most = std::max(most, plan_workspace(plan_gemm(q.transA, q.transB, q.M, q.N, q.K, false, true), q.M, q.N));
+  }
+  const long slots = 4 * num_cus();
+  long kc = (long)(work / (double)slots);
+  kc = (kc + 31) / 32 * 32;
+  if (kc < 256) kc = 256;
+  size_t need = 0;
+  bool vec = true;
+  int n = 0, nr = 0;
+  for (int p = 0; p < count; p++) {
+    const cavs_gemm_desc &q = d[p];
+    if (q.M == 0 || q.N == 0 || alone[p]) continue;
+    long s = q.K > 0 ? (q.K + kc / 2) / kc : 1;
+    if (s < 1) s = 1;
+    int kchunk = q.K > 0 ? (int)(((q.K + s - 1) / s + 31) / 32 * 32) : 1;
+    int splits = q.K > 0 ? (q.K + kchunk - 1) / kchunk : 1;
+    GemmArgs g{q.M, q.N, q.K, q.A, q.lda, q.B, q.ldb, q.C, q.ldc, q.alpha, q.beta, nullptr, 0, 0, kchunk, nullptr};
+    if (splits > 1) {
+      if (ws) g.ws = reinterpret_cast<float *>(static_cast<char *>(ws) + need);
+      need += ((size_t)splits * q.M * q.N * sizeof(float) + 255) / 256 * 256;
+    }
+    if (!need_out && !vec_path_ok(g, q.transA, q.transB)) vec = false;
+    G.g[n] = g;
+    G.tiles[n] = (int)tiles[p];
+    G.splits[n] = splits;
+    G.form[n] = (q.transA ? 2 : 0) + (q.transB ? 1 : 0);
+    G.first[n + 1] = G.first[n] + (int)((tiles[p] * splits + 7) / 8 * 8);
+    n++;
+    if (splits > 1) {
+      R.g[nr] = g;
+      R.splits[nr] = splits;
+      R.first[nr + 1] = R.first[nr] + (int)(((long)q.M * q.N + 255) / 256);
+      nr++;
+    }
+  }
+  G.count = n;
+  R.count = nr;
+  need = std::max(need, most);
+  if (need_out) {
+    *need_out = need;
+    return CAVS_OK;
+  }
+  CAVS_REQUIRE(need == 0 || (ws && ws_bytes >= need && aligned16(ws)), "cavs_sgemm_group: workspace of %zu bytes needed, %zu given", need, ws_bytes);
+  // the products that run alone share the workspace with the group: the stream orders them
+  for (int p = 0; p < count; p++) {
+    const cavs_gemm_desc &q = d[p];
+    if (q.M == 0 || q.N == 0 || !alone[p]) continue;
+    int rc = run_gemm("cavs_sgemm_group", q.transA, q.transB, q.M, q.N, q.K, q.alpha, q.A, q.lda, q.B, q.ldb, q.beta,
+                      q.C, q.ldc, nullptr, 0, 0, ws, ws_bytes, stream);
+    if (rc) return rc;
+  }
+  if (n == 0) return CAVS_OK;
+  hipStream_t st = as_stream(stream);
+  if (vec) launch(sgemm_group_kernel<true>, (unsigned)G.first[n], kThreads, 0, st, G);
+  else launch(sgemm_group_kernel<false>, (unsigned)G.first[n], kThreads, 0, st, G);
+  CAVS_LAUNCH_CHECK();
+  if (nr > 0) {
+    launch(splitk_reduce_group_kernel, (unsigned)R.first[nr], 256, 0, st, R);
+    CAVS_LAUNCH_CHECK();
+  }
+  return CAVS_OK;
+}
+
 }  // namespace cavs
 
 using namespace cavs;
 
 extern "C" {
+
+size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products) {
+  size_t need = 0;
+  if (run_group(count, products, nullptr, 0, &need, nullptr) != CAVS_OK) return 0;
+  return need;
+}
+
+int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace, size_t workspace_bytes,
+                     void *stream) {
+  return run_group(count, products, workspace, workspace_bytes, nullptr, stream);
+}
 
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,
                const float *B, int ldb, float beta, float *C, int ldc, void *stream) {

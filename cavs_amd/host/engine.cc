@@ -177,6 +177,15 @@ void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, 
   c_launches_ += 1;
 }
 
+void Engine::gemm_group(const std::vector<cavs_gemm_desc> &products) {
+  const int count = (int)products.size();
+  float *ws = workspace(cavs_sgemm_group_workspace(count, products.data()));
+  ProfScope ps(this, K_GEMM);
+  check(cavs_sgemm_group(count, products.data(), ws, ws_.capacity() * 4, stream_));
+  for (const cavs_gemm_desc &q : products) c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
+  c_launches_ += 1;
+}
+
 void Engine::gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda,
                          const float *B, int ldb, float *C, int ldc) {
   gemm(tA, tB, M, N, K, A, lda, B, ldb, 0.f, C, ldc);
@@ -601,13 +610,15 @@ void Engine::treelstm_backward() {
   // weight gradients once over all rows (OPT_BATCHING semantics; without it the reference
   // accumulates the same sums round by round)
   const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
-  gemm(0, 1, N, E, 4 * H, dxW_.get(), 4 * H, W, 4 * H, 0.f, de_.get(), E);
-  embedding_backward(E);
-  gemm_splitk(1, 0, E, 4 * H, N, e_.get(), E, dxW_.get(), 4 * H, param("W").g, 4 * H);
   float *dU = param("U").g;
-  gemm_splitk(1, 0, H, 3 * H, N - lp, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H);
-  gemm_splitk(1, 0, H, H, 2 * (N - lp), G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
-              dU + (size_t)3 * H * H, H);
+  gemm_group({
+      {0, 1, N, E, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, W, 4 * H, de_.get(), E},
+      {1, 0, E, 4 * H, N, 1.f, 0.f, e_.get(), E, dxW_.get(), 4 * H, param("W").g, 4 * H},
+      {1, 0, H, 3 * H, N - lp, 1.f, 0.f, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H},
+      {1, 0, H, H, 2 * (N - lp), 1.f, 0.f, G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
+       dU + (size_t)3 * H * H, H},
+  });
+  embedding_backward(E);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
   const int dst_block[4] = {0, 3, 2, 1};  // dxW block k ([i|o|u|f]) lands in bias block dst_block[k]
   const size_t cs_bytes = cavs_colsum_blocks_workspace(N, H, 4);
@@ -719,12 +730,14 @@ void Engine::lstm_backward() {
     scatter(dpool_.get(), 2 * H, d_child_ + off, r_dG_.get(), 2 * H, r.n, 2 * H);
   }
   const int lp = sched_.leaf_prefix;
-  gemm(0, 1, N, H, 4 * H, dxW_.get(), 4 * H, Wx, 4 * H, 0.f, de_.get(), H);
-  embedding_backward(H);
   float *dW = param("W").g;
-  gemm_splitk(1, 0, H, 4 * H, N, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H);
-  gemm_splitk(1, 0, H, 4 * H, N - lp, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
-              dW + (size_t)4 * H * H, 4 * H);
+  gemm_group({
+      {0, 1, N, H, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, Wx, 4 * H, de_.get(), H},
+      {1, 0, H, 4 * H, N, 1.f, 0.f, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H},
+      {1, 0, H, 4 * H, N - lp, 1.f, 0.f, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
+       dW + (size_t)4 * H * H, 4 * H},
+  });
+  embedding_backward(H);
   check(cavs_colsum(param("Bv").g, dxW_.get(), 4 * H, N, 4 * H, 0, stream_));
   c_launches_ += 1;
 }

@@ -78,6 +78,8 @@ class Engine {
   float *workspace(size_t bytes);
   void gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B, int ldb,
             float beta, float *C, int ldc);
+  // independent products in one launch (cavs_sgemm_group)
+  void gemm_group(const std::vector<cavs_gemm_desc> &products);
   void gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
                    int ldb, float *C, int ldc);
   void gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n, int w);

@@ -120,6 +120,26 @@ size_t cavs_sgemm_splitk_workspace(int M, int N, int K);
 int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                       int lda, const float *B, int ldb, float beta, float *C, int ldc,
                       void *workspace, size_t workspace_bytes, void *stream);
+/* Up to four independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
+ * (plus one for the K splits): the once-per-step block of
+ * cavs/midend/batch_weight_updater.h:12-84 -- the weight-gradient GEMMs -- and the embedding
+ * gradient's product next to it.  Each of them alone gives every CU one round of workgroups
+ * that load, multiply and store in step; launched together their phases overlap.  Results are
+ * those of cavs_sgemm_splitk (fixed summation order).  The outputs must not overlap each other
+ * or any input.  cavs_sgemm_group_workspace returns the workspace bytes for the same list. */
+typedef struct cavs_gemm_desc {
+  int transA, transB, M, N, K;
+  float alpha, beta;
+  const float *A;
+  int lda;
+  const float *B;
+  int ldb;
+  float *C;
+  int ldc;
+} cavs_gemm_desc;
+size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products);
+int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace,
+                     size_t workspace_bytes, void *stream);
 /* C[r,:] = op(A)*op(B) + D[r >> d_shift, :]: the GEMM and the Accumulate that
  * follows it in the backward of a Mirror'ed operand
  * (cavs/backend/op_decl_slice_join.cc:173-182) in one pass.  Workspace as above. */

@@ -187,6 +187,68 @@ def test_sgemm_splitk_is_deterministic_and_correct(g, oracle, M, N, K):
     close(outs[0], oracle.sgemm(1, 0, A, B, beta=1.0, Cin=C0))
 
 
+GROUPS = {
+    # the once-per-step block of the Tree-LSTM backward at the headline shape: de, dW, dU_iou, dU_f
+    "treelstm_step": [(0, 1, 2482, 300, 2048), (1, 0, 300, 2048, 2482), (1, 0, 512, 1536, 1241), (1, 0, 512, 512, 2482)],
+    # all four forms, ragged edges, one empty product, K below one tile, K not a multiple of 4
+    "ragged": [(0, 0, 70, 33, 300), (1, 1, 40, 72, 641), (0, 1, 0, 16, 64), (1, 0, 5, 130, 31)],
+    "single": [(1, 0, 64, 96, 3000)],
+    # one product large enough for the big tile (it runs by itself) next to two that share a launch
+    "mixed": [(1, 0, 1024, 1024, 4096), (0, 1, 700, 512, 2048), (1, 0, 512, 512, 700)],
+}
+
+
+@pytest.mark.parametrize("name", sorted(GROUPS))
+def test_sgemm_group_matches_separate_products(g, oracle, name):
+    """Several products in one launch: each equals its own fp64 product and the oracle's
+    sgemm (alpha, beta honoured), bit-identical when repeated, neighbours untouched."""
+    import ctypes as C
+
+    import torch
+
+    shapes = GROUPS[name]
+    r = rng(len(name) + 11)
+    descs = (hip.GemmDesc * len(shapes))()
+    keep, host = [], []
+    for p, (tA, tB, M, N, K) in enumerate(shapes):
+        A = r.bulk_uniform(max(M * K, 1), -1, 1)[:M * K].reshape((K, M) if tA else (M, K))
+        B = r.bulk_uniform(max(N * K, 1), -1, 1)[:N * K].reshape((N, K) if tB else (K, N))
+        beta = 0.0 if p % 2 == 0 else 0.5
+        C0 = r.bulk_uniform(max(M * (N + 3), 1), -1, 1)[:M * (N + 3)].reshape(M, N + 3)  # ldc = N + 3: a column block of a wider slab
+        Ad, Bd = g.devf(A.reshape(-1) if A.size else np.zeros(1)), g.devf(B.reshape(-1) if B.size else np.zeros(1))
+        keep += [Ad, Bd]
+        host.append((A, B, C0, beta))
+        descs[p] = hip.GemmDesc(tA, tB, M, N, K, 1.5, beta, g.P(Ad), max(A.shape[1], 1), g.P(Bd), max(B.shape[1], 1), None, N + 3)
+    nbytes = hip.lib().cavs_sgemm_group_workspace(len(shapes), descs)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    runs = []
+    for _ in range(2):
+        outs = []
+        for p, (A, B, C0, beta) in enumerate(host):
+            Cd = g.devf(C0 if C0.size else np.zeros(1))
+            if beta == 0.0 and C0.size:  # beta = 0 must not read C
+                Cd[:, :C0.shape[1] - 3] = float("nan")
+            outs.append(Cd)
+            descs[p].C = g.P(Cd)
+        g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes, g.stream())
+        runs.append([g.host(o) for o in outs])
+    for p, ((tA, tB, M, N, K), (A, B, C0, beta)) in enumerate(zip(shapes, host)):
+        if M == 0:
+            continue
+        got = runs[0][p]
+        np.testing.assert_array_equal(got, runs[1][p])
+        np.testing.assert_array_equal(got[:, N:], C0[:, N:])  # columns beyond N untouched
+        exact = 1.5 * (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64) + beta * C0[:, :N]
+        close(got[:, :N], exact, f"product {p} vs fp64")
+        if 2.0 * M * N * K < 2e9:  # the oracle's plain loops take seconds beyond this
+            close(got[:, :N], oracle.sgemm(tA, tB, A, B, alpha=1.5, beta=beta, Cin=np.ascontiguousarray(C0[:, :N])), f"product {p} vs oracle")
+    with pytest.raises(hip.CavsError, match="at most 4"):
+        g.call("cavs_sgemm_group", 5, descs, g.P(ws), nbytes, g.stream())
+    if nbytes:
+        with pytest.raises(hip.CavsError, match="workspace"):
+            g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes - 256, g.stream())
+
+
 @pytest.mark.parametrize("tA,tB,M,N,K", [(0, 0, 30, 1536, 512), (0, 1, 8, 512, 1536), (0, 1, 130, 512, 512),
                                           (0, 0, 1, 64, 4096), (1, 1, 40, 72, 640), (0, 0, 33, 40, 300),
                                           (0, 1, 65, 33, 68), (0, 0, 600, 1536, 512), (0, 1, 1200, 512, 1536),
