@@ -71,6 +71,33 @@ __global__ void embed_fwd_kernel(float *__restrict__ out, long ld_out, const flo
   }
 }
 
+// Pull + lookup in one pass: vertex b of the slab is vertex rows[b] of the feed; its id is
+// kept in ids_out[b] for the backward pass.
+__global__ void embed_pull_fwd_kernel(float *__restrict__ out, long ld_out, float *__restrict__ ids_out,
+                                      const float *__restrict__ x, const int *__restrict__ rows,
+                                      const float *__restrict__ table, int n, int E) {
+  constexpr int R = 4;
+  const int row0 = blockIdx.x * R;
+  long off[R];
+#pragma unroll
+  for (int r = 0; r < R; r++) {
+    off[r] = -1;
+    if (row0 + r < n) {
+      const float id = x[rows[row0 + r]];
+      off[r] = (long)(int)(id * (float)E);
+      if (threadIdx.x == 0) ids_out[row0 + r] = id;
+    }
+  }
+  for (int c = threadIdx.x; c < E; c += blockDim.x) {
+    float v[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) v[r] = off[r] >= 0 ? table[off[r] + c] : 0.f;
+#pragma unroll
+    for (int r = 0; r < R; r++)
+      if (row0 + r < n) out[(long)(row0 + r) * ld_out + c] = v[r];
+  }
+}
+
 // Scatter-add of dy rows into the table.  A workgroup takes kEmbedChunk consecutive rows and
 // first adds up the ones that share an id (parse trees look up one and the same row for every
 // internal vertex), so a hot row receives one atomic add per chunk instead of one per vertex.
@@ -252,6 +279,17 @@ int cavs_embed_fwd(float *out, int ld_out, const float *ids, const float *table,
   CAVS_REQUIRE(out && ids && table, "cavs_embed_fwd: null pointer");
   int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
   launch(embed_fwd_kernel, (n + 3) / 4, block, 0, as_stream(stream), out, ld_out, ids, table, n, E);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_embed_pull_fwd(float *out, int ld_out, float *ids_out, const float *x, const int *rows,
+                        const float *table, int n, int E, void *stream) {
+  CAVS_REQUIRE(n >= 0 && E > 0 && ld_out >= E, "cavs_embed_pull_fwd: bad shape n=%d E=%d ld=%d", n, E, ld_out);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(out && ids_out && x && rows && table, "cavs_embed_pull_fwd: null pointer");
+  int block = E >= 256 ? 256 : (E > 64 ? 128 : 64);
+  launch(embed_pull_fwd_kernel, (n + 3) / 4, block, 0, as_stream(stream), out, ld_out, ids_out, x, rows, table, n, E);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

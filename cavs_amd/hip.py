@@ -23,7 +23,6 @@ _lib = None
 _P, _I, _F, _Z = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 
 
-
 class GemmDesc(C.Structure):
     """cavs_gemm_desc: one product of cavs_sgemm_group"""
     _fields_ = [("transA", _I), ("transB", _I), ("M", _I), ("N", _I), ("K", _I), ("alpha", _F), ("beta", _F),
@@ -63,6 +62,7 @@ _SIGS = {
     "cavs_sgemm_splitk": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _Z, _P],
     "cavs_colsum": [_P, _P, _I, _I, _I, _I, _P],
     "cavs_embed_fwd": [_P, _I, _P, _P, _I, _I, _P],
+    "cavs_embed_pull_fwd": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
     "cavs_embed_bwd": [_P, _P, _P, _I, _I, _I, _P],
     "cavs_bias_add_rows": [_P, _P, _P, _I, _I, _P],
     "cavs_softmax_xent": [_P, _P, _P, _P, _I, _I, _P],
@@ -80,6 +80,7 @@ _SIGS = {
     "cavs_treelstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_transpose_batch": [_I, C.POINTER(_P), C.POINTER(_P), C.POINTER(_I), C.POINTER(_I), _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],

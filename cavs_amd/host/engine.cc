@@ -494,8 +494,7 @@ int Engine::fused_rows() const {
 void Engine::treelstm_forward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w, *Bv = param("Bv").w;
-  gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
-  check(cavs_embed_fwd(e_.get(), E, xs_.get(), param("Emb").w, N, E, stream_));
+  check(cavs_embed_pull_fwd(e_.get(), E, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, E, e_.get(), E, W, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
@@ -556,9 +555,11 @@ void Engine::treelstm_backward() {
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
-    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), U, H, 3 * H, stream_));
-    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.at((size_t)3 * H * H), U + (size_t)3 * H * H, H, H, stream_));
-    c_launches_ += 2;
+    float *const outs[2] = {UT_.get(), UT_.at((size_t)3 * H * H)};
+    const float *const ins[2] = {U, U + (size_t)3 * H * H};
+    const int rows[2] = {H, H}, cols[2] = {3 * H, H};
+    CAVS_TIMED(K_OTHER, cavs_transpose_batch(2, outs, ins, rows, cols, stream_));
+    c_launches_ += 1;
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -650,8 +651,7 @@ void Engine::embedding_backward(int E) {
 void Engine::lstm_forward() {
   const int N = N_, H = cfg_.H;
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w;
-  gather(xs_.get(), 1, d_x_, 1, d_t2j_, N, 1);
-  check(cavs_embed_fwd(e_.get(), H, xs_.get(), param("Emb").w, N, H, stream_));
+  check(cavs_embed_pull_fwd(e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));

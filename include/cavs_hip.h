@@ -156,6 +156,11 @@ int cavs_embed_fwd(float *out, int ld_out, const float *ids, const float *table,
                    void *stream);
 int cavs_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, int n, int E,
                    void *stream);
+/* GraphPullOp (cavs/backend/op_impl_graphop.cu:208-258) of the word id and the lookup that
+ * follows it (apps/paper/tree-lstm-cavs.cc:139-141) in one pass: ids_out[b] = x[rows[b]],
+ * out[b, 0:E] = table[int(ids_out[b] * E) ...]. */
+int cavs_embed_pull_fwd(float *out, int ld_out, float *ids_out, const float *x, const int *rows,
+                        const float *table, int n, int E, void *stream);
 /* out[r, :] = inp[r, :] + bias[:]  (BinaryBroadcastingKernel,
  * cavs/backend/op_impl_elementwise.cuh:128-139; also the ones-vector bias GEMM of
  * cavs/backend/op_impl_fullyconnected_cublas.cc:74-76) */
@@ -334,6 +339,9 @@ int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int
                             const int *child, float *dpool, int pool_width, int n, int H, void *stream);
 /* out [cols,rows] = in [rows,cols]^T */
 int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream);
+/* Up to four of them in one launch. */
+int cavs_transpose_batch(int count, float *const *outs, const float *const *ins, const int *rows,
+                         const int *cols, void *stream);
 
 /* ------------------------------------------------------------------ generic fused op
  * FusedKernelOpImpl (cavs/backend/op_impl_fused_kernel.cu:17-71): compiles the

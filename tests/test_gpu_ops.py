@@ -382,6 +382,14 @@ def test_embedding(g, oracle, V, E, n):
     out = g.zeros(n, E)
     g.call("cavs_embed_fwd", g.P(out), E, g.P(g.devf(ids)), g.P(g.devf(table)), n, E, g.stream())
     np.testing.assert_array_equal(g.host(out), oracle.embed_fwd(ids, table))
+    # Pull of the id and the lookup in one pass: vertex b of the slab is vertex rows[b] of the feed
+    rows = np.argsort(r.bulk_uniform(n)).astype(np.int32)
+    out2, ids2 = g.zeros(n, E + 4, fill=7.0), g.zeros(n)
+    g.call("cavs_embed_pull_fwd", g.P(out2), E + 4, g.P(ids2), g.P(g.devf(ids)), g.P(g.devi(rows)), g.P(g.devf(table)),
+           n, E, g.stream())
+    np.testing.assert_array_equal(g.host(ids2), ids[rows])
+    np.testing.assert_array_equal(g.host(out2)[:, :E], oracle.embed_fwd(ids[rows], table))
+    np.testing.assert_array_equal(g.host(out2)[:, E:], np.full((n, 4), 7.0, np.float32))  # beyond E untouched
     dy = r.bulk_normal(n * E).reshape(n, E)
     d0 = r.bulk_normal(V * E).reshape(V, E)
     want = oracle.embed_bwd(d0.copy(), ids, dy)
@@ -606,6 +614,14 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     g.call("cavs_transpose", g.P(UT) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, H, H, g.stream())
     np.testing.assert_array_equal(g.host(UT)[: 3 * H * H].reshape(3 * H, H), Uiou.T)
     np.testing.assert_array_equal(g.host(UT)[3 * H * H:].reshape(H, H), Uf.T)
+    # both in one launch
+    import ctypes as C
+
+    UT2 = g.zeros(4 * H * H)
+    outs = (C.c_void_p * 2)(g.P(UT2), g.P(UT2) + 4 * 3 * H * H)
+    ins = (C.c_void_p * 2)(g.P(d_U), g.P(d_U) + 4 * 3 * H * H)
+    g.call("cavs_transpose_batch", 2, outs, ins, (C.c_int * 2)(H, H), (C.c_int * 2)(3 * H, H), g.stream())
+    np.testing.assert_array_equal(g.host(UT2), g.host(UT))
     d_dpool, dxW, dF = g.devf(dpool), g.zeros(n, 4 * H), g.zeros(2 * n, H)
     g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool), g.P(d_pair), g.P(d_child), g.P(g.devf(dret)), None, g.P(g.devf(gates_w)),
            g.P(g.devf(G_w)), g.P(dxW), 4 * H, g.P(dF), n, H, g.stream())
