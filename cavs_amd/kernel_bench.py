@@ -108,6 +108,23 @@ def gemm(iters, st):
         _emit("sgemm", f"{tag}: {'T' if tA else 'N'}{'T' if tB else 'N'} M={M} N={Nn} K={K}", us,
               flops=2.0 * M * Nn * K)
         del A, B, Cm, ws
+    # the once-per-step products of a C3 batch as one grouped launch
+    H, E, N = 512, 300, 2482
+    shapes = [(0, 1, N, E, 4 * H), (1, 0, E, 4 * H, N), (1, 0, H, 3 * H, N // 2), (1, 0, H, H, N)]
+    descs = (hip.GemmDesc * len(shapes))()
+    keep = []
+    for p, (tA, tB, M, Nn, K) in enumerate(shapes):
+        A = torch.randn((K, M) if tA else (M, K), **f32)
+        B = torch.randn((Nn, K) if tB else (K, Nn), **f32)
+        Cm = torch.empty(M, Nn, **f32)
+        keep += [A, B, Cm]
+        descs[p] = hip.GemmDesc(tA, tB, M, Nn, K, 1.0, 0.0, A.data_ptr(), A.shape[1], B.data_ptr(), B.shape[1],
+                                Cm.data_ptr(), Nn)
+    nb = hip.lib().cavs_sgemm_group_workspace(len(shapes), descs)
+    ws = torch.empty(max(nb // 4, 4), **f32)
+    us = _time(lambda: hip.call("cavs_sgemm_group", len(shapes), descs, ws.data_ptr(), nb, st), iters, st)
+    _emit("sgemm_group", "C3 step: de + dW + dU_iou + dU_f in one launch (+ one reduce)", us,
+          flops=sum(2.0 * M * Nn * K for _, _, M, Nn, K in shapes))
 
 
 def gates(iters, st):

@@ -192,6 +192,29 @@ def test_full_size_tree_lstm_properties():
     s.close()
 
 
+@pytest.mark.parametrize("name", ["C3", "C4", "C5"])
+def test_full_size_fused_rounds_equal_separate_launches(name):
+    """At the benchmark's own sizes the two ways a round runs -- one fused launch, or gather,
+    GEMMs, gates and scatter as separate launches -- must give the same step (they share no
+    MFMA kernel: the fused rounds feed the matrix cores from global memory, the separate path
+    goes through the LDS-tiled GEMM; the deferred products are grouped in both)."""
+    w = synth.make_workload(name)
+    kw = dict(H=w["H"], E=w["E"], V=w["V"], C_=w["C"])
+    outs = []
+    for limit in (0, -1):
+        print(f"[case] {name} full N={w['N']} fused_round_rows={limit}", flush=True)
+        s = session.Session(w["model"], fused_round_rows=limit, **kw)
+        s.set_params(w["params"])
+        s.step(w["graph"], w["x"], w["labels"], backward=True)
+        outs.append(dict(loss=s.fetch("loss"), go=s.fetch("graph_out"), grads=s.grads(), rf=s.counter("round_flops")))
+        s.close()
+    assert outs[0]["rf"] > 0 and outs[1]["rf"] == 0  # the first really ran fused rounds, the second none
+    close(outs[0]["loss"], outs[1]["loss"], "loss")
+    close(outs[0]["go"], outs[1]["go"], "graph_out")
+    for k, v in outs[1]["grads"].items():
+        close(outs[0]["grads"][k], v, k, rtol=2e-4, atol=2e-5)
+
+
 @pytest.mark.parametrize("H,limit", [(32, 0), (64, 0), (96, 0), (64, 20), (64, -1)])
 @pytest.mark.parametrize("pairing", ["reference", "rowid"])
 @pytest.mark.parametrize("model,kw", CASES)
