@@ -71,6 +71,7 @@ def cpu_baseline(w, budget_s=12.0):
         pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **dict(args, threads=1))
     el1 = time.perf_counter() - t1
     return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port",
+                host=dict(nproc=os.cpu_count(), affinity=len(os.sched_getaffinity(0)), omp_threads=threads),
                 sample=f"{steps} full fwd+bwd step(s) of the {w['name']} batch (B={w['B']}, N={w['N']}) "
                        f"in {el:.1f} s with {threads} OpenMP threads; CPU restatement of the reference's "
                        "semantics (the reference has no CPU kernels)",
