@@ -373,7 +373,7 @@ def test_colsum(g, oracle, n, w):
     close(g.host(out), exact + acc0, rtol=1e-4, atol=1e-5 * np.sqrt(n))
 
 
-@pytest.mark.parametrize("V,E,n", [(23, 6, 31), (21701, 300, 500), (1000, 128, 64)])
+@pytest.mark.parametrize("V,E,n", [(23, 6, 31), (21701, 300, 500), (1000, 128, 64), (21701, 300, 2482), (50, 512, 1100)])
 def test_embedding(g, oracle, V, E, n):
     r = rng(V + E)
     table = r.bulk_normal(V * E).reshape(V, E)
