@@ -44,14 +44,28 @@ __global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ 
       acc[c][q] = 0.f;
     }
   }
-  for (int row = blockIdx.x * 4 + wave; row < n; row += gridDim.x * 4) {
+  // the next row of this wavefront is fetched while the current one goes through its chain of
+  // wave reductions and exponentials
+  const int step = gridDim.x * 4;
+  float xn[Q];
+  int lab_n = 0;
+  auto fetch = [&](int row) {
+    if (row >= n) return;
     const float *x = X + (long)row * H;
-    float xv[Q], z[C];
 #pragma unroll
     for (int q = 0; q < Q; q++) {
       const int col = q * 64 + lane;
-      xv[q] = col < H ? x[col] : 0.f;
+      xn[q] = col < H ? x[col] : 0.f;
     }
+    lab_n = (int)labels[row];
+  };
+  fetch(blockIdx.x * 4 + wave);
+  for (int row = blockIdx.x * 4 + wave; row < n; row += step) {
+    float xv[Q], z[C];
+#pragma unroll
+    for (int q = 0; q < Q; q++) xv[q] = xn[q];
+    const int lab = lab_n;
+    fetch(row + step);
     float mx = -INFINITY;
 #pragma unroll
     for (int c = 0; c < C; c++) {
@@ -62,7 +76,6 @@ __global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ 
       mx = fmaxf(mx, z[c]);
     }
     // cavs/backend/op_impl_softmax_entropy_logits_loss.cu:94-140, :212-250
-    const int lab = (int)labels[row];
     float sum = 0.f, zl = 0.f;
 #pragma unroll
     for (int c = 0; c < C; c++) {
