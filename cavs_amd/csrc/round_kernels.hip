@@ -18,8 +18,6 @@
 //     children, h_l+h_r).
 // TILE is 32 (v_mfma_f32_32x32x2_f32) or, for rounds of a few rows near the roots, 16
 // (v_mfma_f32_16x16x4_f32), which spreads a tiny round over four times as many CUs.
-#include <algorithm>
-
 #include "round_common.h"
 
 namespace cavs {
@@ -525,28 +523,6 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
     if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
 }
 
-// several transposes in one launch: blockIdx.z picks the matrix
-struct TransposeBatch {
-  float *out[4];
-  const float *in[4];
-  int rows[4], cols[4];
-};
-
-__global__ void transpose_batch_kernel(TransposeBatch b) {
-  __shared__ float tile[32][33];
-  const int m = blockIdx.z, rows = b.rows[m], cols = b.cols[m];
-  const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
-  if (c0 >= cols || r0 >= rows) return;
-  const float *__restrict__ in = b.in[m];
-  float *__restrict__ out = b.out[m];
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  for (int i = ty; i < 32; i += 8)
-    if (r0 + i < rows && c0 + tx < cols) tile[i][tx] = in[(long)(r0 + i) * cols + c0 + tx];
-  __syncthreads();
-  for (int i = ty; i < 32; i += 8)
-    if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
-}
-
 }  // namespace cavs
 
 using namespace cavs;
@@ -644,31 +620,6 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
   CAVS_REQUIRE(out && in && out != in, "cavs_transpose: null or aliased pointer");
   dim3 grid((cols + 31) / 32, (rows + 31) / 32);
   launch(transpose_kernel, grid, 256, 0, as_stream(stream), out, in, rows, cols);
-  CAVS_LAUNCH_CHECK();
-  return CAVS_OK;
-}
-
-int cavs_transpose_batch(int count, float *const *outs, const float *const *ins, const int *rows, const int *cols,
-                         void *stream) {
-  CAVS_REQUIRE(count >= 0 && count <= 4, "cavs_transpose_batch: %d matrices, at most 4", count);
-  if (count == 0) return CAVS_OK;
-  CAVS_REQUIRE(outs && ins && rows && cols, "cavs_transpose_batch: null argument");
-  TransposeBatch b{};
-  int gx = 0, gy = 0, m = 0;
-  for (int i = 0; i < count; i++) {
-    CAVS_REQUIRE(rows[i] >= 0 && cols[i] >= 0, "cavs_transpose_batch: bad shape %d x %d", rows[i], cols[i]);
-    if (rows[i] == 0 || cols[i] == 0) continue;
-    CAVS_REQUIRE(outs[i] && ins[i] && outs[i] != ins[i], "cavs_transpose_batch: null or aliased pointer");
-    b.out[m] = outs[i];
-    b.in[m] = ins[i];
-    b.rows[m] = rows[i];
-    b.cols[m] = cols[i];
-    gx = std::max(gx, (cols[i] + 31) / 32);
-    gy = std::max(gy, (rows[i] + 31) / 32);
-    m++;
-  }
-  if (m == 0) return CAVS_OK;
-  launch(transpose_batch_kernel, dim3(gx, gy, m), 256, 0, as_stream(stream), b);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -187,13 +187,19 @@ __global__ void sgd_multi_kernel(SgdBatch t, float lr) {
 // and asks for a row once however often it occurs among them (parse trees look up one and
 // the same row for every internal vertex; one atomic per vertex would serialise on it).
 constexpr int kSgdChunk = 16;
-__global__ void embed_sgd_kernel(float *__restrict__ table, const float *__restrict__ dtable,
-                                 const float *__restrict__ ids, int n, int E, float lr, int *__restrict__ stamp,
-                                 int epoch) {
-  __shared__ int row[kSgdChunk];
-  __shared__ long owned[kSgdChunk];
-  __shared__ int n_owned;
-  const int v0 = blockIdx.x * kSgdChunk, tid = threadIdx.x;
+struct EmbedSgdLds {
+  int row[kSgdChunk];
+  long owned[kSgdChunk];
+  int n_owned;
+};
+
+__device__ inline void embed_sgd_block(float *__restrict__ table, const float *__restrict__ dtable,
+                                       const float *__restrict__ ids, int n, int E, float lr, int *__restrict__ stamp,
+                                       int epoch, int block, EmbedSgdLds &lds) {
+  int (&row)[kSgdChunk] = lds.row;
+  long (&owned)[kSgdChunk] = lds.owned;
+  int &n_owned = lds.n_owned;
+  const int v0 = block * kSgdChunk, tid = threadIdx.x;
   if (tid < kSgdChunk) row[tid] = v0 + tid < n ? (int)ids[v0 + tid] : -1 - tid;
   if (tid == 0) n_owned = 0;
   __syncthreads();
@@ -220,9 +226,73 @@ __global__ void embed_sgd_kernel(float *__restrict__ table, const float *__restr
   }
 }
 
+__global__ void embed_sgd_kernel(float *__restrict__ table, const float *__restrict__ dtable,
+                                 const float *__restrict__ ids, int n, int E, float lr, int *__restrict__ stamp,
+                                 int epoch) {
+  __shared__ EmbedSgdLds lds;
+  embed_sgd_block(table, dtable, ids, n, E, lr, stamp, epoch, blockIdx.x, lds);
+}
+
 __global__ void embed_zero_rows_kernel(float *__restrict__ dtable, const float *__restrict__ ids, int E) {
   const long off = (long)(int)(ids[blockIdx.x] * (float)E);
   for (int c = threadIdx.x; c < E; c += blockDim.x) dtable[off + c] = 0.f;
+}
+
+// ------------------------------------------------------------------ several small jobs, one launch
+// The jobs around the rounds that do not depend on each other (the weight transposes and the
+// clearing of the embedding gradient before backward; the updates of the dense parameters and of
+// the embedding table after it) are a few microseconds each, most of it launch and drain.  One
+// launch runs a list of them: workgroup b belongs to job k with first[k] <= b < first[k+1].
+constexpr int kMaxTasks = 12;
+struct TaskList {
+  cavs_task t[kMaxTasks];
+  int first[kMaxTasks + 1];
+  int count;
+};
+
+__global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
+  __shared__ union {
+    float tile[32][33];
+    EmbedSgdLds sgd;
+  } lds;
+  int k = 0;
+  while (k + 1 < L.count && (int)blockIdx.x >= L.first[k + 1]) k++;
+  const cavs_task &t = L.t[k];
+  const int b = blockIdx.x - L.first[k], nb = L.first[k + 1] - L.first[k], tid = threadIdx.x;
+  switch (t.kind) {
+    case CAVS_TASK_TRANSPOSE: {  // p0[c][r] = p1[r][c], n0 rows, n1 columns
+      const float *__restrict__ in = static_cast<const float *>(t.p1);
+      float *__restrict__ out = static_cast<float *>(t.p0);
+      const int rows = (int)t.n0, cols = (int)t.n1, gx = (cols + 31) / 32;
+      const int c0 = (b % gx) * 32, r0 = (b / gx) * 32, tx = tid & 31, ty = tid >> 5;
+      for (int i = ty; i < 32; i += 8)
+        if (r0 + i < rows && c0 + tx < cols) lds.tile[i][tx] = in[(long)(r0 + i) * cols + c0 + tx];
+      __syncthreads();
+      for (int i = ty; i < 32; i += 8)
+        if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = lds.tile[tx][i];
+      break;
+    }
+    case CAVS_TASK_ZERO_ROWS: {  // p0[int(p1[r] * n1) ...] = 0 for n1 columns, r < n0: one row per workgroup
+      float *__restrict__ dtable = static_cast<float *>(t.p0);
+      const float *__restrict__ ids = static_cast<const float *>(t.p1);
+      const int E = (int)t.n1;
+      const long off = (long)(int)(ids[b] * (float)E);
+      for (int c = tid; c < E; c += 256) dtable[off + c] = 0.f;
+      break;
+    }
+    case CAVS_TASK_SGD: {  // p0[i] -= f0 * p1[i], i < n0
+      float *__restrict__ w = static_cast<float *>(t.p0);
+      const float *__restrict__ g = static_cast<const float *>(t.p1);
+      const size_t n = (size_t)t.n0, stride = (size_t)nb * 256;
+      for (size_t i = (size_t)b * 256 + tid; i < n; i += stride) w[i] -= t.f0 * g[i];
+      break;
+    }
+    case CAVS_TASK_EMBED_SGD:  // cavs_embed_sgd(p0 = table, p1 = dtable, p2 = ids, n0 = n, n1 = E, f0 = lr, p3 = stamp, n2 = epoch)
+      embed_sgd_block(static_cast<float *>(t.p0), static_cast<const float *>(t.p1), static_cast<const float *>(t.p2),
+                      (int)t.n0, (int)t.n1, t.f0, static_cast<int *>(t.p3), (int)t.n2, b, lds.sgd);
+      break;
+    default: break;
+  }
 }
 
 // ------------------------------------------------------------------ column sums of column blocks
@@ -314,6 +384,56 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
     launch(fc_xent_reduce_kernel, (total + 63) / 64, 256, 0, st, part, blocks, total, C * H, dW, db);
     CAVS_LAUNCH_CHECK();
   }
+  return CAVS_OK;
+}
+
+int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
+  CAVS_REQUIRE(count >= 0 && count <= kMaxTasks, "cavs_run_tasks: %d jobs, at most %d", count, kMaxTasks);
+  CAVS_REQUIRE(count == 0 || tasks, "cavs_run_tasks: null list");
+  TaskList L{};
+  int k = 0;
+  for (int i = 0; i < count; i++) {
+    const cavs_task &t = tasks[i];
+    long blocks = 0;
+    switch (t.kind) {
+      case CAVS_TASK_TRANSPOSE:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 30) && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad transpose shape", i);
+        if (t.n0 == 0 || t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1, "cavs_run_tasks: job %d: null or aliased pointer", i);
+        blocks = ((t.n0 + 31) / 32) * ((t.n1 + 31) / 32);
+        break;
+      case CAVS_TASK_ZERO_ROWS:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 > 0 && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad shape", i);
+        if (t.n0 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1, "cavs_run_tasks: job %d: null pointer", i);
+        blocks = t.n0;
+        break;
+      case CAVS_TASK_SGD: {
+        CAVS_REQUIRE(t.n0 >= 0, "cavs_run_tasks: job %d: negative size", i);
+        if (t.n0 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1, "cavs_run_tasks: job %d: null pointer", i);
+        const long want = (t.n0 + 1023) / 1024, cap = (long)num_cus() * 4;
+        blocks = want < cap ? want : cap;
+        break;
+      }
+      case CAVS_TASK_EMBED_SGD:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 > 0 && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad shape", i);
+        if (t.n0 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p2 && t.p3, "cavs_run_tasks: job %d: null pointer", i);
+        blocks = (t.n0 + kSgdChunk - 1) / kSgdChunk;
+        break;
+      default:
+        CAVS_REQUIRE(false, "cavs_run_tasks: job %d: unknown kind %d", i, t.kind);
+    }
+    CAVS_REQUIRE(blocks > 0 && L.first[k] + blocks < (1L << 30), "cavs_run_tasks: job %d: too many workgroups", i);
+    L.t[k] = t;
+    L.first[k + 1] = L.first[k] + (int)blocks;
+    k++;
+  }
+  if (k == 0) return CAVS_OK;
+  L.count = k;
+  launch(tasks_kernel, (unsigned)L.first[k], 256, 0, as_stream(stream), L);
+  CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
 

@@ -23,6 +23,15 @@ _lib = None
 _P, _I, _F, _Z = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 
 
+class Task(C.Structure):
+    """cavs_task: one job of cavs_run_tasks"""
+    _fields_ = [("kind", _I), ("f0", _F), ("n0", C.c_longlong), ("n1", C.c_longlong), ("n2", C.c_longlong),
+                ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P)]
+
+
+TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD = 0, 1, 2, 3
+
+
 class GemmDesc(C.Structure):
     """cavs_gemm_desc: one product of cavs_sgemm_group"""
     _fields_ = [("transA", _I), ("transB", _I), ("M", _I), ("N", _I), ("K", _I), ("alpha", _F), ("beta", _F),
@@ -80,7 +89,6 @@ _SIGS = {
     "cavs_treelstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
-    "cavs_transpose_batch": [_I, C.POINTER(_P), C.POINTER(_P), C.POINTER(_I), C.POINTER(_I), _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
@@ -92,6 +100,7 @@ _SIGS = {
     "cavs_profile_arm": [_P, _P],
     "cavs_profile_disarm": [_P],
     "cavs_fc_softmax_xent": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _P],
+    "cavs_run_tasks": [_I, C.POINTER(Task), _P],
     "cavs_sgd_multi": [_I, _P, _P, _P, _F, _P],
     "cavs_clip_grads": [_I, _P, _P, _F, _P, _Z, _P],
     "cavs_embed_sgd": [_P, _P, _P, _I, _I, _F, _P, _I, _P],

@@ -445,9 +445,8 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     if (lr != 0.f) {
       // w -= lr * g (cavs/backend/op_impl_sgd.cu); the embedding table by its looked-up rows
       // only: every other row of its gradient is zero, so the dense update would not move it
-      std::vector<float *> ws;
-      std::vector<const float *> gs;
-      std::vector<size_t> ns;
+      // all of it in one launch: the updates touch disjoint tensors
+      std::vector<cavs_task> tasks;
       for (auto &kv : params_) {
         Param &p = *kv.second;
         if (kv.first == "Emb" && emb_dirty_n_ == N) {
@@ -456,15 +455,12 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
             emb_stamp_.reserve(cfg_.V);
             check(cavs_zero(emb_stamp_.get(), (size_t)cfg_.V * 4, stream_));
           }
-          check(cavs_embed_sgd(p.w, p.g, xs_prev_.get(), N, E, lr, emb_stamp_.get(), ++emb_epoch_, stream_));
-          c_launches_ += 1;
+          tasks.push_back({CAVS_TASK_EMBED_SGD, lr, N, E, ++emb_epoch_, p.w, p.g, xs_prev_.get(), emb_stamp_.get()});
           continue;
         }
-        ws.push_back(p.w);
-        gs.push_back(p.g);
-        ns.push_back(p.n);
+        tasks.push_back({CAVS_TASK_SGD, lr, (long long)p.n, 0, 0, p.w, p.g, nullptr, nullptr});
       }
-      check(cavs_sgd_multi((int)ws.size(), ws.data(), gs.data(), ns.data(), lr, stream_));
+      check(cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
       c_launches_ += 1;
     }
   }
@@ -555,11 +551,10 @@ void Engine::treelstm_backward() {
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
-    float *const outs[2] = {UT_.get(), UT_.at((size_t)3 * H * H)};
-    const float *const ins[2] = {U, U + (size_t)3 * H * H};
-    const int rows[2] = {H, H}, cols[2] = {3 * H, H};
-    CAVS_TIMED(K_OTHER, cavs_transpose_batch(2, outs, ins, rows, cols, stream_));
-    c_launches_ += 1;
+    backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr},
+                       {CAVS_TASK_TRANSPOSE, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H,
+                        nullptr, nullptr}},
+                      true);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -631,10 +626,28 @@ void Engine::treelstm_backward() {
 // EmbeddingLookup_grad (cavs/backend/op_impl_embedding.cu:58-92): scatter-add of the rows of
 // de into a zeroed table.  The table is kept zero outside the rows of the previous step, so
 // clearing it costs those rows, not the vocabulary.
+// The transposed weights of the fused backward rounds and -- `with_embedding` -- the clearing of
+// the embedding gradient (the rows the previous step looked up) do not depend on each other:
+// one launch.
+void Engine::backward_prologue(std::vector<cavs_task> tasks, bool with_embedding) {
+  if (with_embedding) {
+    Param &emb = param("Emb");
+    if (emb.g == emb.own_g.get() && emb_sparse_valid_) {
+      if (emb_dirty_n_ > 0)
+        tasks.push_back({CAVS_TASK_ZERO_ROWS, 0.f, emb_dirty_n_, (long long)(emb.n / cfg_.V), 0, emb.g, xs_prev_.get(), nullptr, nullptr});
+      emb_cleared_ = true;
+    }
+  }
+  CAVS_TIMED(K_OTHER, cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
+  c_launches_ += 1;
+}
+
 void Engine::embedding_backward(int E) {
   Param &emb = param("Emb");
   const bool owned = emb.g == emb.own_g.get();
-  if (owned && emb_sparse_valid_) {
+  if (emb_cleared_) {
+    emb_cleared_ = false;  // the prologue of this backward pass did it
+  } else if (owned && emb_sparse_valid_) {
     if (emb_dirty_n_ > 0) check(cavs_embed_zero_rows(emb.g, xs_prev_.get(), emb_dirty_n_, E, stream_));
   } else {
     check(cavs_zero(emb.g, emb.n * 4, stream_));
@@ -693,8 +706,7 @@ void Engine::lstm_backward() {
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
-    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), Wh, H, 4 * H, stream_));
-    c_launches_ += 1;
+    backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr, nullptr}}, true);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -797,8 +809,7 @@ void Engine::treefc_backward() {
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W^T [H, 2H]: the B operand of d[h_l;h_r] = dz * W^T, k-major
-    CAVS_TIMED(K_OTHER, cavs_transpose(UT_.get(), W, 2 * H, H, stream_));
-    c_launches_ += 1;
+    backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, 2 * H, H, 0, UT_.get(), const_cast<float *>(W), nullptr, nullptr}}, false);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];

@@ -80,6 +80,7 @@ class Engine {
             float beta, float *C, int ldc);
   // independent products in one launch (cavs_sgemm_group)
   void gemm_group(const std::vector<cavs_gemm_desc> &products);
+  void backward_prologue(std::vector<cavs_task> tasks, bool with_embedding);
   void gemm_splitk(int tA, int tB, int M, int N, int K, const float *A, int lda, const float *B,
                    int ldb, float *C, int ldc);
   void gather(float *out, int ld_out, const float *src, int ld_src, const int *ids, int n, int w);
@@ -141,6 +142,7 @@ class Engine {
   DeviceArray<int> emb_stamp_;
   int emb_dirty_n_ = 0, emb_epoch_ = 0;
   bool emb_sparse_valid_ = true;  // the table is zero outside xs_prev_[0, emb_dirty_n_)
+  bool emb_cleared_ = false;      // the backward prologue of this step already cleared those rows
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
   // rounds of at most this many rows run as fused launches (0: none)

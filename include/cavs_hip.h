@@ -339,9 +339,23 @@ int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int
                             const int *child, float *dpool, int pool_width, int n, int H, void *stream);
 /* out [cols,rows] = in [rows,cols]^T */
 int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream);
-/* Up to four of them in one launch. */
-int cavs_transpose_batch(int count, float *const *outs, const float *const *ins, const int *rows,
-                         const int *cols, void *stream);
+/* Several small jobs that do not depend on each other, in one launch (no counterpart in the
+ * reference, where each is an op of its own: cavs/backend/op_impl_sgd.cu,
+ * op_impl_embedding_lookup.cu, the transposes cuBLAS does inside its calls).  Results are those
+ * of the separate entry points.  At most 12 jobs; a job must not write what another reads.
+ *   CAVS_TASK_TRANSPOSE  p0[c][r] = p1[r][c]               n0 rows, n1 columns
+ *   CAVS_TASK_ZERO_ROWS  cavs_embed_zero_rows(p0 = dtable, p1 = ids, n0 = n, n1 = E)
+ *   CAVS_TASK_SGD        p0[i] -= f0 * p1[i]               i < n0
+ *   CAVS_TASK_EMBED_SGD  cavs_embed_sgd(p0 = table, p1 = dtable, p2 = ids, n0 = n, n1 = E,
+ *                                       f0 = lr, p3 = stamp, n2 = epoch) */
+enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3 };
+typedef struct cavs_task {
+  int kind;
+  float f0;
+  long long n0, n1, n2;
+  void *p0, *p1, *p2, *p3;
+} cavs_task;
+int cavs_run_tasks(int count, const cavs_task *tasks, void *stream);
 
 /* ------------------------------------------------------------------ generic fused op
  * FusedKernelOpImpl (cavs/backend/op_impl_fused_kernel.cu:17-71): compiles the

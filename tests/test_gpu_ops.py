@@ -615,12 +615,10 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     np.testing.assert_array_equal(g.host(UT)[: 3 * H * H].reshape(3 * H, H), Uiou.T)
     np.testing.assert_array_equal(g.host(UT)[3 * H * H:].reshape(H, H), Uf.T)
     # both in one launch
-    import ctypes as C
-
     UT2 = g.zeros(4 * H * H)
-    outs = (C.c_void_p * 2)(g.P(UT2), g.P(UT2) + 4 * 3 * H * H)
-    ins = (C.c_void_p * 2)(g.P(d_U), g.P(d_U) + 4 * 3 * H * H)
-    g.call("cavs_transpose_batch", 2, outs, ins, (C.c_int * 2)(H, H), (C.c_int * 2)(3 * H, H), g.stream())
+    tasks = (hip.Task * 2)(hip.Task(hip.TASK_TRANSPOSE, 0.0, H, 3 * H, 0, g.P(UT2), g.P(d_U), None, None),
+                           hip.Task(hip.TASK_TRANSPOSE, 0.0, H, H, 0, g.P(UT2) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, None, None))
+    g.call("cavs_run_tasks", 2, tasks, g.stream())
     np.testing.assert_array_equal(g.host(UT2), g.host(UT))
     d_dpool, dxW, dF = g.devf(dpool), g.zeros(n, 4 * H), g.zeros(2 * n, H)
     g.call("cavs_treelstm_round_bwd_gates", g.P(d_dpool), g.P(d_pair), g.P(d_child), g.P(g.devf(dret)), None, g.P(g.devf(gates_w)),
@@ -739,6 +737,48 @@ def test_sgd_over_several_tensors_and_sparse_embedding_update(g):
         np.testing.assert_array_equal(g.host(t), want)
     g.call("cavs_embed_zero_rows", g.P(dgrad), g.P(dids), n, E, g.stream())
     assert not g.host(dgrad).any()
+
+
+def test_several_small_jobs_in_one_launch(g):
+    """cavs_run_tasks: transposes, clearing of looked-up rows, dense SGD updates and the row-sparse
+    embedding update as one launch give what the separate entry points give (bit-exact)."""
+    r = rng(23)
+    A, B = r.bulk_normal(70 * 33).reshape(70, 33), r.bulk_normal(64 * 192).reshape(64, 192)
+    V, E, n = 300, 41, 90
+    ids = np.floor(r.bulk_uniform(n) * V).astype(np.float32)
+    ids[:30] = ids[0]
+    rows = np.unique(ids.astype(np.int64))
+    dirty = r.bulk_normal(V * E).reshape(V, E)                  # to be cleared in the listed rows only
+    table = r.bulk_normal(V * E).reshape(V, E)
+    grad = np.zeros((V, E), np.float32)
+    grad[rows] = r.bulk_normal(len(rows) * E).reshape(len(rows), E)
+    w1, g1 = r.bulk_normal(100003), r.bulk_normal(100003)
+    w2, g2 = r.bulk_normal(7), r.bulk_normal(7)
+    dA, dB, dAT, dBT = g.devf(A), g.devf(B), g.zeros(33, 70), g.zeros(192, 64)
+    d_dirty, d_ids, d_table, d_grad = g.devf(dirty), g.devf(ids), g.devf(table), g.devf(grad)
+    d_w1, d_g1, d_w2, d_g2 = g.devf(w1), g.devf(g1), g.devf(w2), g.devf(g2)
+    stamp = g.devi(np.zeros(V, np.int32))
+    T = hip.Task
+    jobs = [T(hip.TASK_TRANSPOSE, 0.0, 70, 33, 0, g.P(dAT), g.P(dA), None, None),
+            T(hip.TASK_SGD, 0.25, 100003, 0, 0, g.P(d_w1), g.P(d_g1), None, None),
+            T(hip.TASK_ZERO_ROWS, 0.0, n, E, 0, g.P(d_dirty), g.P(d_ids), None, None),
+            T(hip.TASK_TRANSPOSE, 0.0, 64, 192, 0, g.P(dBT), g.P(dB), None, None),
+            T(hip.TASK_SGD, 0.5, 0, 0, 0, None, None, None, None),                     # an empty job is skipped
+            T(hip.TASK_EMBED_SGD, 0.5, n, E, 1, g.P(d_table), g.P(d_grad), g.P(d_ids), g.P(stamp)),
+            T(hip.TASK_SGD, 2.0, 7, 0, 0, g.P(d_w2), g.P(d_g2), None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    np.testing.assert_array_equal(g.host(dAT), A.T)
+    np.testing.assert_array_equal(g.host(dBT), B.T)
+    np.testing.assert_array_equal(g.host(d_w1), w1 - np.float32(0.25) * g1)
+    np.testing.assert_array_equal(g.host(d_w2), w2 - np.float32(2.0) * g2)
+    want = dirty.copy()
+    want[rows] = 0
+    np.testing.assert_array_equal(g.host(d_dirty), want)
+    np.testing.assert_array_equal(g.host(d_table), table - np.float32(0.5) * grad)
+    with pytest.raises(hip.CavsError, match="unknown kind"):
+        g.call("cavs_run_tasks", 1, (T * 1)(T(9, 0.0, 1, 1, 0, g.P(dA), g.P(dB), None, None)), g.stream())
+    with pytest.raises(hip.CavsError, match="at most 12"):
+        g.call("cavs_run_tasks", 13, (T * 13)(), g.stream())
 
 
 @pytest.mark.parametrize("n,bw,perm", [(1, 4, [0]), (2482, 512, [0, 3, 2, 1]), (63, 6, [2, 0, 1]), (5000, 64, [1, 0])])
