@@ -127,11 +127,10 @@ __global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ 
 
 // out[i] = sum over the workgroups' partials: four interleaved slices per output, each added
 // in index order, combined in a fixed order
-__global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__restrict__ part, int nparts, int total,
-                                                             int CH, float *__restrict__ dW, float *__restrict__ db) {
-  __shared__ float s[4][64];
+__device__ inline void sum_parts_block(const float *__restrict__ part, int nparts, int total, int CH,
+                                       float *__restrict__ dW, float *__restrict__ db, int block, float (&s)[4][64]) {
   const int o = threadIdx.x & 63, q = threadIdx.x >> 6;
-  const int i = blockIdx.x * 64 + o;
+  const int i = block * 64 + o;
   float a0 = 0.f, a1 = 0.f;
   if (i < total) {
     int p = q;
@@ -147,6 +146,12 @@ __global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__rest
     const float v = (s[0][o] + s[1][o]) + (s[2][o] + s[3][o]);
     if (i < CH) dW[i] = v; else db[i - CH] = v;
   }
+}
+
+__global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__restrict__ part, int nparts, int total,
+                                                             int CH, float *__restrict__ dW, float *__restrict__ db) {
+  __shared__ float s[4][64];
+  sum_parts_block(part, nparts, total, CH, dW, db, blockIdx.x, s);
 }
 
 static int head_blocks(int n) {
@@ -254,6 +259,7 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
   __shared__ union {
     float tile[32][33];
     EmbedSgdLds sgd;
+    float sums[4][64];
   } lds;
   int k = 0;
   while (k + 1 < L.count && (int)blockIdx.x >= L.first[k + 1]) k++;
@@ -290,6 +296,10 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
     case CAVS_TASK_EMBED_SGD:  // cavs_embed_sgd(p0 = table, p1 = dtable, p2 = ids, n0 = n, n1 = E, f0 = lr, p3 = stamp, n2 = epoch)
       embed_sgd_block(static_cast<float *>(t.p0), static_cast<const float *>(t.p1), static_cast<const float *>(t.p2),
                       (int)t.n0, (int)t.n1, t.f0, static_cast<int *>(t.p3), (int)t.n2, b, lds.sgd);
+      break;
+    case CAVS_TASK_SUM_PARTS:  // p1[i] (i < n2) or p2[i - n2] = sum over p < n0 of p0[p * n1 + i], i < n1
+      sum_parts_block(static_cast<const float *>(t.p0), (int)t.n0, (int)t.n1, (int)t.n2, static_cast<float *>(t.p1),
+                      static_cast<float *>(t.p2), b, lds.sums);
       break;
     default: break;
   }
@@ -352,6 +362,8 @@ size_t cavs_fc_softmax_xent_workspace(int n, int H, int C) {
   return (size_t)head_blocks(n) * ((size_t)C * H + C) * sizeof(float);
 }
 
+int cavs_fc_softmax_xent_parts(int n) { return n > 0 ? head_blocks(n) : 0; }
+
 int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const float *labels, float *loss,
                          float *logits, float *dX, float *dW, float *db, void *workspace,
                          size_t workspace_bytes, int n, int H, int C, void *stream) {
@@ -359,7 +371,8 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(X && W && b && labels && loss, "cavs_fc_softmax_xent: null pointer");
   const bool grad = dX || dW || db;
-  CAVS_REQUIRE(!grad || (dX && dW && db), "cavs_fc_softmax_xent: dX, dW and db must be all set or all null");
+  const bool deferred = dX && !dW && !db;  // the caller sums the partials (CAVS_TASK_SUM_PARTS)
+  CAVS_REQUIRE(!grad || deferred || (dX && dW && db), "cavs_fc_softmax_xent: dX alone, or dX, dW and db, or none of them");
   const int blocks = head_blocks(n);
   const size_t need = (size_t)blocks * ((size_t)C * H + C) * sizeof(float);
   CAVS_REQUIRE(!grad || (workspace && workspace_bytes >= need), "cavs_fc_softmax_xent: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
@@ -379,7 +392,7 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
   }
 #undef CAVS_HEAD
   CAVS_LAUNCH_CHECK();
-  if (grad) {
+  if (grad && !deferred) {
     const int total = C * H + C;
     launch(fc_xent_reduce_kernel, (total + 63) / 64, 256, 0, st, part, blocks, total, C * H, dW, db);
     CAVS_LAUNCH_CHECK();
@@ -421,6 +434,13 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         if (t.n0 == 0) continue;
         CAVS_REQUIRE(t.p0 && t.p1 && t.p2 && t.p3, "cavs_run_tasks: job %d: null pointer", i);
         blocks = (t.n0 + kSgdChunk - 1) / kSgdChunk;
+        break;
+      case CAVS_TASK_SUM_PARTS:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n1 < (1 << 30) && t.n0 < (1 << 30) && t.n2 >= 0 && t.n2 <= t.n1,
+                     "cavs_run_tasks: job %d: bad shape", i);
+        if (t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p0 && (t.n2 == 0 || t.p1) && (t.n2 == t.n1 || t.p2), "cavs_run_tasks: job %d: null pointer", i);
+        blocks = (t.n1 + 63) / 64;
         break;
       default:
         CAVS_REQUIRE(false, "cavs_run_tasks: job %d: unknown kind %d", i, t.kind);

@@ -555,6 +555,8 @@ void Engine::treelstm_backward() {
                        {CAVS_TASK_TRANSPOSE, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H,
                         nullptr, nullptr}},
                       true);
+  } else {
+    backward_prologue({}, true);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -630,6 +632,8 @@ void Engine::treelstm_backward() {
 // the embedding gradient (the rows the previous step looked up) do not depend on each other:
 // one launch.
 void Engine::backward_prologue(std::vector<cavs_task> tasks, bool with_embedding) {
+  tasks.insert(tasks.end(), pending_tasks_.begin(), pending_tasks_.end());
+  pending_tasks_.clear();
   if (with_embedding) {
     Param &emb = param("Emb");
     if (emb.g == emb.own_g.get() && emb_sparse_valid_) {
@@ -638,6 +642,7 @@ void Engine::backward_prologue(std::vector<cavs_task> tasks, bool with_embedding
       emb_cleared_ = true;
     }
   }
+  if (tasks.empty()) return;
   CAVS_TIMED(K_OTHER, cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
   c_launches_ += 1;
 }
@@ -707,6 +712,8 @@ void Engine::lstm_backward() {
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr, nullptr}}, true);
+  } else {
+    backward_prologue({}, true);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -810,6 +817,8 @@ void Engine::treefc_backward() {
   if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W^T [H, 2H]: the B operand of d[h_l;h_r] = dz * W^T, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, 2 * H, H, 0, UT_.get(), const_cast<float *>(W), nullptr, nullptr}}, false);
+  } else {
+    backward_prologue({}, false);
   }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
@@ -852,11 +861,15 @@ void Engine::head_forward_backward(bool backward) {
     // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
     Param &Wfc = param("Wfc"), &bfc = param("bfc");
     const size_t head_bytes = cavs_fc_softmax_xent_workspace(N, H, C);
-    if (head_bytes > 0) {  // few classes: the whole head and its gradients in two launches
-      float *hw = workspace(head_bytes);
+    if (head_bytes > 0) {  // few classes: the whole head and its gradients in one launch; the sum of
+                           // its weight-gradient partials rides in the launch that opens backward
+      if (head_parts_.capacity() * 4 < head_bytes) head_parts_.reserve(head_bytes / 4 + 1);
       check(cavs_fc_softmax_xent(GO_.get(), Wfc.w, bfc.w, d_labels_, loss_.get(), logits_.get(), backward ? dGO_.get() : nullptr,
-                                 backward ? Wfc.g : nullptr, backward ? bfc.g : nullptr, hw, head_bytes, N, H, C, stream_));
-      c_launches_ += backward ? 2 : 1;
+                                 nullptr, nullptr, head_parts_.get(), head_bytes, N, H, C, stream_));
+      if (backward)
+        pending_tasks_.push_back({CAVS_TASK_SUM_PARTS, 0.f, cavs_fc_softmax_xent_parts(N), (long long)C * H + C, (long long)C * H,
+                                  head_parts_.get(), Wfc.g, bfc.g, nullptr});
+      c_launches_ += 1;
       return;
     }
     gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w, H, 0.f, logits_.get(), C);

@@ -143,6 +143,8 @@ class Engine {
   int emb_dirty_n_ = 0, emb_epoch_ = 0;
   bool emb_sparse_valid_ = true;  // the table is zero outside xs_prev_[0, emb_dirty_n_)
   bool emb_cleared_ = false;      // the backward prologue of this step already cleared those rows
+  std::vector<cavs_task> pending_tasks_;  // jobs queued for the launch that opens backward
+  DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
   // rounds of at most this many rows run as fused launches (0: none)

@@ -246,8 +246,12 @@ int cavs_treefc_bwd(const float *dh_m, const float *dret, const float *h, float 
  * are given, their gradients (:150-163, :212-250) for a head of at most 8 classes:
  * X [n,H], W [C,H], b [C], labels [n] (class ids as floats); loss [n], logits [n,C] (may be
  * NULL), dX [n,H], dW [C,H], db [C]; d logits = (softmax - onehot) / n.  The workspace query
- * returns 0 for a shape this entry point does not take (C > 8, H > 1024, or C * ceil-pow2(H/64) > 64). */
+ * returns 0 for a shape this entry point does not take (C > 8, H > 1024, or C * ceil-pow2(H/64) > 64).
+ * With dX given and dW, db NULL the weight and bias gradients stay in the workspace as
+ * cavs_fc_softmax_xent_parts(n) partial sums of C*H + C floats each, to be added up by a
+ * CAVS_TASK_SUM_PARTS job of cavs_run_tasks (n0 = parts, n1 = C*H + C, n2 = C*H). */
 size_t cavs_fc_softmax_xent_workspace(int n, int H, int C);
+int cavs_fc_softmax_xent_parts(int n);
 int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const float *labels,
                          float *loss, float *logits, float *dX, float *dW, float *db,
                          void *workspace, size_t workspace_bytes, int n, int H, int C, void *stream);
@@ -347,8 +351,11 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *   CAVS_TASK_ZERO_ROWS  cavs_embed_zero_rows(p0 = dtable, p1 = ids, n0 = n, n1 = E)
  *   CAVS_TASK_SGD        p0[i] -= f0 * p1[i]               i < n0
  *   CAVS_TASK_EMBED_SGD  cavs_embed_sgd(p0 = table, p1 = dtable, p2 = ids, n0 = n, n1 = E,
- *                                       f0 = lr, p3 = stamp, n2 = epoch) */
-enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3 };
+ *                                       f0 = lr, p3 = stamp, n2 = epoch)
+ *   CAVS_TASK_SUM_PARTS  out[i] = sum over p < n0 of p0[p * n1 + i] in a fixed order, i < n1, where
+ *                        out[i] is p1[i] for i < n2 and p2[i - n2] above */
+enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
+       CAVS_TASK_SUM_PARTS = 4 };
 typedef struct cavs_task {
   int kind;
   float f0;

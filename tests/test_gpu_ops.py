@@ -694,6 +694,17 @@ def test_fused_classifier_head(g, oracle, n, H, C_):
     close(g.host(dX), dX_w, "dX", atol=1e-7)
     close(g.host(dW), dW_w, "dW", atol=1e-6)
     close(g.host(db), db_w, "db", atol=1e-6)
+    # dX alone: the weight-gradient partials stay in the workspace and a job of the multi-job
+    # launch adds them up -- the same sums, bit for bit
+    dX2, dW2, db2 = g.zeros(n, H), g.zeros(C_, H), g.zeros(C_)
+    ws2 = g.zeros(nb // 4)
+    g.call("cavs_fc_softmax_xent", *args, g.P(dX2), None, None, g.P(ws2), nb, n, H, C_, g.stream())
+    parts = hip.lib().cavs_fc_softmax_xent_parts(n)
+    assert parts * (C_ * H + C_) * 4 == nb
+    job = hip.Task(hip.TASK_SUM_PARTS, 0.0, parts, C_ * H + C_, C_ * H, g.P(ws2), g.P(dW2), g.P(db2), None)
+    g.call("cavs_run_tasks", 1, (hip.Task * 1)(job), g.stream())
+    for a, b2, what in ((dX2, dX, "dX"), (dW2, dW, "dW"), (db2, db, "db")):
+        np.testing.assert_array_equal(g.host(a), g.host(b2), what)
     # forward only: no gradient buffers, no workspace
     loss2 = g.zeros(n)
     g.call("cavs_fc_softmax_xent", *args[:4], g.P(loss2), None, None, None, None, None, 0, n, H, C_, g.stream())
