@@ -152,18 +152,29 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
       lb.load(g.B, g.ldb, n0, kbeg + (kt + 1) * BK, g.N, kend, tid);
     }
     const float *as = As_ + cur * (BK * LDA), *bs = Bs_ + cur * (BK * LDB);
+    // operand fragments of the k-tile: the reads of AHEAD steps are in flight while a step's
+    // MFMAs issue, so a wavefront does not stall on LDS latency between them
+    constexpr int STEPS = BK / 2, AHEAD = (TM * TN == 1) ? 4 : 2;
+    float a[STEPS][TM], b[STEPS][TN];
+    auto read = [&](int st) {
 #pragma unroll
-    for (int kk = 0; kk < BK; kk += 2) {
-      float a[TM], b[TN];
+      for (int i = 0; i < TM; i++) a[st][i] = as[(2 * st + khalf) * LDA + arow + 32 * i];
 #pragma unroll
-      for (int i = 0; i < TM; i++) a[i] = as[(kk + khalf) * LDA + arow + 32 * i];
+      for (int j = 0; j < TN; j++) b[st][j] = bs[(2 * st + khalf) * LDB + brow + 32 * j];
+    };
 #pragma unroll
-      for (int j = 0; j < TN; j++) b[j] = bs[(kk + khalf) * LDB + brow + 32 * j];
+    for (int st = 0; st < AHEAD && st < STEPS; st++) read(st);
+    __builtin_amdgcn_sched_barrier(0);  // the compiler's scheduler would sink each read to its use
+#pragma unroll
+    for (int st = 0; st < STEPS; st++) {
+      if (st + AHEAD < STEPS) read(st + AHEAD);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int i = 0; i < TM; i++)
 #pragma unroll
         for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[i], b[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[st][i], b[st][j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (kt + 1 < nk) {
       la.store(As_ + (cur ^ 1) * (BK * LDA), tid);
@@ -180,18 +191,32 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
     for (int j = 0; j < TN; j++) {
       const int col = n0 + wn * WN + 32 * j + (lane & 31);
       if (col >= g.N) continue;
+      const int rbase = m0 + wm * WM + 32 * i + 4 * khalf;
+      // the three forms of the store are chosen once per tile (the conditions are the same
+      // for every lane), not once per element
+      if (g.ws) {  // split K: park the partial sum, the reduce kernel finishes the job
+        float *w = g.ws + (long)z * g.M * g.N + col;
 #pragma unroll
-      for (int r = 0; r < 16; r++) {
-        const int row = m0 + wm * WM + 32 * i + 8 * (r / 4) + 4 * khalf + (r % 4);
-        if (row >= g.M) continue;
-        if (g.ws) {  // split K: park the partial sum, the reduce kernel finishes the job
-          g.ws[((long)z * g.M + row) * g.N + col] = acc[i][j][r];
-          continue;
+        for (int r = 0; r < 16; r++) {
+          const int row = rbase + 8 * (r / 4) + (r % 4);
+          if (row < g.M) w[(long)row * g.N] = acc[i][j][r];
         }
-        float v = g.alpha * acc[i][j][r];
-        if (g.beta != 0.f) v += g.beta * g.C[row * g.ldc + col];
-        if (g.D) v += g.D[(long)(row >> g.dshift) * g.ldd + col];
-        g.C[row * g.ldc + col] = v;
+      } else if (g.beta == 0.f && !g.D) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int row = rbase + 8 * (r / 4) + (r % 4);
+          if (row < g.M) g.C[row * g.ldc + col] = g.alpha * acc[i][j][r];
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          const int row = rbase + 8 * (r / 4) + (r % 4);
+          if (row >= g.M) continue;
+          float v = g.alpha * acc[i][j][r];
+          if (g.beta != 0.f) v += g.beta * g.C[row * g.ldc + col];
+          if (g.D) v += g.D[(long)(row >> g.dshift) * g.ldd + col];
+          g.C[row * g.ldc + col] = v;
+        }
       }
     }
 }
