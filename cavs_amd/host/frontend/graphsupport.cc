@@ -6,6 +6,11 @@
 
 #include "cavs/util/op_def_builder.h"
 
+GraphSupport::GraphSupport(const Sym &graph_placeholder, const Sym &vertex_placeholder)
+    : graph_placeholder_(graph_placeholder), vertex_placeholder_(vertex_placeholder) {}
+
+GraphSupport::~GraphSupport() = default;
+
 Sym GraphSupport::Output() {
   FuncConf::FuncDefineBegin("Node");
   this->Node();
@@ -20,20 +25,20 @@ Sym GraphSupport::Output() {
   for (size_t i = 0; i < n; i++) width *= dim[i];
   std::free(dim);
   int max_nodes = 1;
-  for (int d : raw_graph_.shape(0)) max_nodes *= d;
-  return Sym(OpDefBuilder("GraphOutput").Input(raw_graph_.output(0)).Input(raw_vertex_.output(0))
-                 .Dtype(raw_vertex_.type()).Device(raw_vertex_.device()).Shape({-1, width})
+  for (int d : graph_placeholder_.shape(0)) max_nodes *= d;
+  return Sym(OpDefBuilder("GraphOutput").Input(graph_placeholder_.output(0)).Input(vertex_placeholder_.output(0))
+                 .Dtype(vertex_placeholder_.type()).Device(vertex_placeholder_.device()).Shape({-1, width})
                  .AttrSingle("Wavefront", true).AttrSingle("MaxGraphNodeCount", max_nodes).Finalize());
 }
 
 Sym GraphSupport::Gather(int child, const std::vector<int> &shape) {
   CHECK(!shape.empty());
-  return Sym(OpDefBuilder("Gather").Dtype(raw_vertex_.type()).Device(raw_vertex_.device()).Shape(shape)
+  return Sym(OpDefBuilder("Gather").Dtype(vertex_placeholder_.type()).Device(vertex_placeholder_.device()).Shape(shape)
                  .AttrSingle("Child", child).Finalize());
 }
 
 Sym GraphSupport::Pull(int offset, const std::vector<int> &shape) {
-  return Sym(OpDefBuilder("Pull").Dtype(raw_vertex_.type()).Device(raw_vertex_.device()).Shape(shape)
+  return Sym(OpDefBuilder("Pull").Dtype(vertex_placeholder_.type()).Device(vertex_placeholder_.device()).Shape(shape)
                  .AttrSingle("Offset", offset).Finalize());
 }
 
