@@ -199,8 +199,10 @@ def measure(a, workload, steps, warmup, n_pool):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=20)
+    # the device needs about a hundred steps (60 ms) of this workload to reach its steady clocks:
+    # 20 warm-up steps read 0.62 ms per step, 100 and more 0.575
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=150)
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--pool", type=int, default=16)
     ap.add_argument("--lr", type=float, default=1e-3)
@@ -235,7 +237,7 @@ def main():
             if name == a.workload:
                 continue
             big = name == "C5"
-            also, _ = measure(a, name, 10 if big else 30, 3 if big else 5, 2 if big else 4)
+            also, _ = measure(a, name, 20 if big else 100, 5 if big else 50, 2 if big else 4)
             out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
