@@ -105,6 +105,17 @@ def measure(a, workload, steps, warmup, n_pool):
             g, x, lab = feeds[i % len(feeds)]
             s.step(g, x, lab, backward=True, lr=a.lr)
 
+    # untimed, before the W warm-up steps: the device takes ~60 ms of this kind of work to reach its
+    # steady clocks, whatever W the caller picked
+    # (continuous work: a synchronisation every few steps lets it idle and the ramp never happens)
+    settle = 0
+    if a.settle_ms > 0:
+        t_probe = time.perf_counter()
+        run(0, 10)
+        s.sync()
+        per_step = max((time.perf_counter() - t_probe) / 10, 1e-5)
+        settle = 10 + min(5000, int(a.settle_ms * 1e-3 / per_step))
+        run(10, settle - 10)
     run(0, warmup)
     s.sync()
     torch.cuda.synchronize()
@@ -169,7 +180,8 @@ def measure(a, workload, steps, warmup, n_pool):
                                f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing,
                    "feeds": "pageable host memory, copied every step" if a.host_feeds else "resident in HBM",
-                   "rounds_last_batch": rounds, "launches_last_batch": launches},
+                   "rounds_last_batch": rounds, "launches_last_batch": launches,
+                   "untimed_settle_steps": settle},
         "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
                      "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": traffic,
                      "kernel": dom["kernel"],
@@ -203,6 +215,8 @@ def main():
     # 20 warm-up steps read 0.62 ms per step, 100 and more 0.575
     ap.add_argument("--steps", type=int, default=300)
     ap.add_argument("--warmup", type=int, default=150)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="untimed steps run for this long before the warm-up steps (clock ramp); 0 to skip")
     ap.add_argument("--workload", default="C3")
     ap.add_argument("--pool", type=int, default=16)
     ap.add_argument("--lr", type=float, default=1e-3)
