@@ -208,8 +208,10 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     const float h = o * tc;
     float *g = a.gates + (long)b * 6 * H + j;
     g[0] = i; g[H] = o; g[2 * H] = u; g[3 * H] = f_l; g[4 * H] = f_r; g[5 * H] = tc;
-    float *m = a.msg + b * H2 + j;
-    m[0] = h; m[H] = c;
+    if (a.msg) {
+      float *m = a.msg + b * H2 + j;
+      m[0] = h; m[H] = c;
+    }
     if (ep.dst >= 0) {
       a.pool_out[ep.dst * H2 + j] = h;
       a.pool_out[ep.dst * H2 + H + j] = c;
@@ -265,8 +267,10 @@ __global__ void treelstm_round_leaves_fwd_kernel(RoundLeavesArgs a) {
   };
   float *g = a.gates + (long)r * 6 * H + j;
   st(g, gi); st(g + H, go); st(g + 2 * H, gu); st(g + 3 * H, gf); st(g + 4 * H, gf); st(g + 5 * H, gtc);
-  float *m = a.msg + r * H2 + j;
-  st(m, mh); st(m + H, mc);
+  if (a.msg) {
+    float *m = a.msg + r * H2 + j;
+    st(m, mh); st(m + H, mc);
+  }
   if (dst >= 0) { st(a.pool + dst * H2 + j, mh); st(a.pool + dst * H2 + H + j, mc); }
   if (out >= 0) st(a.go + (long)out * H + j, mh);
 }
@@ -535,7 +539,7 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   CAVS_REQUIRE(n >= 0 && round_shape_ok(H) && ld_xw >= 4 * H && ld_xw % 4 == 0,
                "cavs_treelstm_round_fwd: bad shape n=%d H=%d ld_xw=%d (H must be a multiple of 32)", n, H, ld_xw);
   if (n == 0) return CAVS_OK;
-  CAVS_REQUIRE(pool && child && pair && xW && U && bias && G && hlr && gates && msg, "cavs_treelstm_round_fwd: null pointer");
+  CAVS_REQUIRE(pool && child && pair && xW && U && bias && G && hlr && gates, "cavs_treelstm_round_fwd: null pointer");
   CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd: graph_out needs out_rows");
   RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
@@ -555,12 +559,12 @@ int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW
                                    void *stream) {
   CAVS_REQUIRE(n >= 0 && H > 0 && ld_xw >= 4 * H, "cavs_treelstm_round_leaves_fwd: bad shape n=%d H=%d ld=%d", n, H, ld_xw);
   if (n == 0) return CAVS_OK;
-  CAVS_REQUIRE(pool && pair && xW && bias && gates && msg, "cavs_treelstm_round_leaves_fwd: null pointer");
+  CAVS_REQUIRE(pool && pair && xW && bias && gates, "cavs_treelstm_round_leaves_fwd: null pointer");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_leaves_fwd: graph_out needs out_rows");
   RoundLeavesArgs a{xW, ld_xw, bias, pair, gates, msg, pool, graph_out, out_rows, n, H};
   hipStream_t st = as_stream(stream);
   const bool vec = H % 4 == 0 && ld_xw % 4 == 0 && aligned16(pool) && aligned16(xW) && aligned16(bias) && aligned16(gates) &&
-                   aligned16(msg) && (!graph_out || aligned16(graph_out));
+                   (!msg || aligned16(msg)) && (!graph_out || aligned16(graph_out));
   if (vec) {
     long total = (long)n * (H / 4);
     launch(treelstm_round_leaves_fwd_kernel<4>, (unsigned)((total + 255) / 256), 256, 0, st, a);

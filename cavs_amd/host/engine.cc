@@ -503,7 +503,9 @@ void Engine::treelstm_forward() {
   float *go = out_folded_ ? fwd_out_ : nullptr;
   for (const Round &r : sched_.rounds) {
     const size_t off = r.offset;
-    float *msg = msg_.at(off * 2 * H);
+    // the message slab is only read back by FunctionPopRet; when the rounds write the output
+    // rows themselves nobody reads it and the fused launches skip it
+    float *msg = out_folded_ ? nullptr : msg_.at(off * 2 * H);
     if (leaf_round(r) && r.n <= fused) {
       CAVS_TIMED(K_GATES, cavs_treelstm_round_leaves_fwd(pool_.get(), d_pair_ + off, xW_.at(off * 4 * H), 4 * H, Bv, gates_.at(off * 6 * H),
                                                          msg, go, d_t2j_ + off, r.n, H, stream_));

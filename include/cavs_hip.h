@@ -289,7 +289,7 @@ int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int 
  *   pool [*,2H] message pool rows [h|c]; child [2n] pool rows of the children of slab
  *   row b at 2b, 2b+1 (-1 = none, reads as zero); pair [n] pool row the message of slab
  *   row b is written to (-1 = nowhere); U = U_iou [H,3H] then U_f [H,H].
- * Writes msg [n,2H], pool rows pair[b], and what backward reads again: gates [n,6H],
+ * Writes msg [n,2H] (may be NULL: skipped), pool rows pair[b], and what backward reads again: gates [n,6H],
  * G [2n,2H] (gathered children), hlr [n,H] (h_l + h_r).  With graph_out [*,H] given, the pushed
  * return value h of slab row b is also written to row out_rows[b] (Push + FunctionPopRet,
  * op_impl_graphop.cu:168-206,274-327, folded in). */
