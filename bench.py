@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, profiles/bench_C3_hbm_traffic_pmc.txt
-PMC_TRAFFIC_BYTES = {("C3", "round"): 17.19e6}
+PMC_TRAFFIC_BYTES = {("C3", "round"): 16.98e6}
 
 
 def model_kwargs(w):
@@ -77,6 +77,37 @@ def cpu_baseline(w, budget_s=12.0):
                        "semantics (the reference has no CPU kernels)",
                 single_thread=dict(value=round(w["B"] * 2 / el1, 3), unit="samples/s", cores=1,
                                    sample=f"2 steps of the same batch in {el1:.1f} s"))
+
+
+def front_end_modes(w, steps=60, warmup=30):
+    """The same training step through the reference's own API (Sym / GraphSupport / Session::Run with
+    host feeds, one device synchronisation per Run, loss head and optimizer as ordinary ops), in the
+    three ways the session can execute F: lowered onto the fused round kernels, op by op with the
+    fusion pass's generated kernels, and plain op by op -- the reference's execution model on this GPU."""
+    import torch
+
+    from cavs_amd import apps, session
+
+    B, maxlen = w["graph"].shape
+    out = {}
+    for name, opt, lowered in (("lowered", session.OPT_BATCHING, True),
+                               ("op_by_op_fusion", session.OPT_BATCHING | session.OPT_FUSION, False),
+                               ("op_by_op", session.OPT_BATCHING, False)):
+        app = apps.App(w["model"], B=B, maxlen=maxlen, H=w["H"], E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=1e-3,
+                       allow_fused=lowered)
+        app.set_params(w["params"])
+        for _ in range(warmup):
+            app.step(w["graph"], w["x"], w["labels"], fetch=False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            app.step(w["graph"], w["x"], w["labels"], fetch=False)
+        torch.cuda.synchronize()
+        ms = 1e3 * (time.perf_counter() - t0) / steps
+        out[name] = {"ms_per_step": round(ms, 4), "value": round(B / ms * 1e3, 1), "unit": "samples/s", "steps": steps,
+                     "generated_kernels": app.generated_kernels}
+        app.close()
+    return out
 
 
 def measure(a, workload, steps, warmup, n_pool):
@@ -222,6 +253,8 @@ def main():
     ap.add_argument("--lr", type=float, default=1e-3)
     ap.add_argument("--pairing", default="reference", choices=["reference", "rowid"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-front-end", action="store_true",
+                    help="skip the 'front_end' field (the step through Session::Run in its three execution modes)")
     ap.add_argument("--host-feeds", action="store_true",
                     help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
     ap.add_argument("--fused-round-rows", type=int, default=0,
@@ -253,6 +286,8 @@ def main():
             big = name == "C5"
             also, _ = measure(a, name, 20 if big else 100, 5 if big else 50, 2 if big else 4)
             out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}
+    if not a.no_front_end and w0["model"] in ("treelstm", "lstm"):
+        out["front_end"] = front_end_modes(w0)
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
     print(json.dumps(out))

@@ -85,7 +85,9 @@ class App:
             buf[: p.size] = p
         return buf
 
-    def step(self, graph, x=None, labels=None, train=True, root_mask=None):
+    def step(self, graph, x=None, labels=None, train=True, root_mask=None, fetch=True):
+        """One Session::Run.  fetch=False (training only) requests just the optimizer symbol, as the
+        reference apps' loops do, and reads nothing back."""
         a, _ = libs()
         g = np.ascontiguousarray(graph, np.int32)
         xw = self.H if self.model == "treefc_x" else 1
@@ -95,6 +97,11 @@ class App:
             labels = None
         xb, lb = self._placeholder(x, xw), self._placeholder(labels)
         mb = self._placeholder(root_mask, self.H) if self.model == "treefc_x" else np.zeros(1, np.float32)
+        if train and not fetch:
+            n = a.cavs_app_step(g.ctypes.data, xb.ctypes.data, lb.ctypes.data, mb.ctypes.data, 1, None, 0, None, 0)
+            if n < 0:
+                raise hip.CavsError(f"cavs_app_step -> {n}")
+            return None
         cap = self.B * self.maxlen
         loss = np.zeros(cap, np.float32)
         go = np.zeros(cap * self.H, np.float32)

@@ -259,6 +259,10 @@ long cavs_app_step(const int *graph, const float *x, const float *labels, const 
     if (a.model == "treefc_x") feeds.push_back({a.mask, (void *)mask});
     vector<Sym> outs;
     if (train) outs.push_back(a.train);
+    if (train && !loss_out && !go_out) {  // as the reference apps loop: sess.Run({train}, feeds), nothing read back
+      a.sess->Run(outs, feeds);
+      return 0;
+    }
     outs.push_back(a.loss);
     outs.push_back(a.graph_output);
     a.sess->Run(outs, feeds);
