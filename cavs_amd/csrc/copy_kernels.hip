@@ -40,7 +40,7 @@ __global__ void gather_rows_kernel(V *__restrict__ out, long ld_out, const V *__
     if (row < n && src) id = ids ? ids[row] : row;
     srow[r] = id;
   }
-  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < wv; c += gridDim.y * blockDim.x) {
     V v[kRowsPerBlock];
 #pragma unroll
     for (int r = 0; r < kRowsPerBlock; r++)
@@ -56,7 +56,7 @@ template <typename V>
 __global__ void add_rows_kernel(V *__restrict__ out, long ld_out, const V *__restrict__ inp, long ld_inp,
                                 int n, int wv) {
   const int row0 = blockIdx.x * kRowsPerBlock;
-  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < wv; c += gridDim.y * blockDim.x) {
 #pragma unroll
     for (int r = 0; r < kRowsPerBlock; r++)
       if (row0 + r < n) {
@@ -79,7 +79,7 @@ __global__ void scatter_rows_kernel(V *__restrict__ dst, long ld_dst, const int 
   }
   // loads are unconditional (rows past the end re-read the last row) so that all four are
   // in flight before the first store; only the stores are predicated
-  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < wv; c += gridDim.y * blockDim.x) {
     V v[kRowsPerBlock];
 #pragma unroll
     for (int r = 0; r < kRowsPerBlock; r++) v[r] = inp[(long)min(row0 + r, n - 1) * ld_inp + c];
@@ -105,7 +105,7 @@ __global__ void gather_children_kernel(V *__restrict__ G, V *__restrict__ hsum,
     int row = 2 * b0 + r;
     srow[r] = row < 2 * n ? (long)ids[row] : -1;
   }
-  for (int c = threadIdx.x; c < wv; c += blockDim.x) {
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < wv; c += gridDim.y * blockDim.x) {
     V v[2 * kNodes];
 #pragma unroll
     for (int r = 0; r < 2 * kNodes; r++)
@@ -123,6 +123,20 @@ __global__ void gather_children_kernel(V *__restrict__ G, V *__restrict__ hsum,
 
 inline int block_for(int wv) { return wv >= 256 ? 256 : (wv > 128 ? 256 : (wv > 64 ? 128 : 64)); }
 
+// grid for `row_blocks` workgroups' worth of rows, wv vector columns each: few but wide rows (a
+// flat parameter viewed as one row) are split along the columns as well, so that the launch still
+// covers the chip
+inline dim3 grid_for(int row_blocks, int wv, int block) {
+  int gy = 1;
+  if (row_blocks < 1024) {
+    const int by_width = (wv + 4 * block - 1) / (4 * block);  // at least four columns per lane
+    const int wanted = (1024 + row_blocks - 1) / row_blocks;
+    gy = by_width < wanted ? by_width : wanted;
+    if (gy < 1) gy = 1;
+  }
+  return dim3(row_blocks, gy);
+}
+
 inline bool vec_ok(const void *a, long lda, const void *b, long ldb, int w) {
   return (w % 4 == 0) && (lda % 4 == 0) && (ldb % 4 == 0) && (!a || aligned16(a)) &&
          (!b || aligned16(b));
@@ -134,11 +148,11 @@ static int launch_gather(float *out, int ld_out, const float *src, int ld_src, c
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(out, ld_out, src, ld_src, w)) {
     int wv = w / 4;
-    launch(gather_rows_kernel<float4>, grid, block_for(wv), 0, st, 
+    launch(gather_rows_kernel<float4>, grid_for(grid, wv, block_for(wv)), block_for(wv), 0, st,
         reinterpret_cast<float4 *>(out), ld_out / 4, reinterpret_cast<const float4 *>(src),
         ld_src / 4, ids, n, wv);
   } else {
-    launch(gather_rows_kernel<float>, grid, block_for(w), 0, st, out, ld_out, src, ld_src, ids, n, w);
+    launch(gather_rows_kernel<float>, grid_for(grid, w, block_for(w)), block_for(w), 0, st, out, ld_out, src, ld_src, ids, n, w);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
@@ -173,10 +187,10 @@ int cavs_add_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, i
   hipStream_t st = as_stream(stream);
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(out, ld_out, inp, ld_inp, w))
-    launch(add_rows_kernel<float4>, grid, block_for(w / 4), 0, st, reinterpret_cast<float4 *>(out), ld_out / 4,
-                                                               reinterpret_cast<const float4 *>(inp), ld_inp / 4, n, w / 4);
+    launch(add_rows_kernel<float4>, grid_for(grid, w / 4, block_for(w / 4)), block_for(w / 4), 0, st,
+           reinterpret_cast<float4 *>(out), ld_out / 4, reinterpret_cast<const float4 *>(inp), ld_inp / 4, n, w / 4);
   else
-    launch(add_rows_kernel<float>, grid, block_for(w), 0, st, out, ld_out, inp, ld_inp, n, w);
+    launch(add_rows_kernel<float>, grid_for(grid, w, block_for(w)), block_for(w), 0, st, out, ld_out, inp, ld_inp, n, w);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -197,11 +211,11 @@ int cavs_scatter_rows(float *dst, int ld_dst, const int *ids, const float *inp, 
   int grid = (n + kRowsPerBlock - 1) / kRowsPerBlock;
   if (vec_ok(dst, ld_dst, inp, ld_inp, w)) {
     int wv = w / 4;
-    launch(scatter_rows_kernel<float4>, grid, block_for(wv), 0, st, 
+    launch(scatter_rows_kernel<float4>, grid_for(grid, wv, block_for(wv)), block_for(wv), 0, st,
         reinterpret_cast<float4 *>(dst), ld_dst / 4, ids, reinterpret_cast<const float4 *>(inp),
         ld_inp / 4, n, wv);
   } else {
-    launch(scatter_rows_kernel<float>, grid, block_for(w), 0, st, dst, ld_dst, ids, inp, ld_inp, n, w);
+    launch(scatter_rows_kernel<float>, grid_for(grid, w, block_for(w)), block_for(w), 0, st, dst, ld_dst, ids, inp, ld_inp, n, w);
   }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;

@@ -42,7 +42,9 @@ def close(got, want, what="", rtol=RTOL, atol=ATOL):
 
 # ---------------------------------------------------------------- row movement
 @pytest.mark.parametrize("n,w,ld_extra", [(1, 4, 0), (7, 1024, 0), (33, 256, 0), (130, 36, 4),
-                                           (50, 37, 3), (5, 2048, 0), (1000, 512, 0)])
+                                           (50, 37, 3), (5, 2048, 0), (1000, 512, 0),
+                                           # few, very wide rows (a flat parameter viewed as one row): split along the columns
+                                           (1, 786432, 0), (3, 100003, 1), (2, 65536, 4)])
 def test_gather_scatter_zero_copy_rows_bit_exact(g, oracle, n, w, ld_extra):
     r = rng(n * 131 + w)
     rows = 2 * n + 3
