@@ -41,6 +41,9 @@ Executor::Executor(int opt, const std::string &name) : opt_(opt), name_(name) {
 Executor::~Executor() {
   cavs_stream_sync(stream_);
   engine_.reset();
+  for (auto &kv : feed_stages_)
+    for (void *e : kv.second.uploaded)
+      if (e) cavs_event_destroy(e);
   for (auto &kv : fused_handles_)
     if (kv.second) cavs_fused_release(kv.second);
   tensors_.clear();
@@ -682,7 +685,22 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
         t.own.reserve(t.width);
       }
       t.base = t.own.get();
-      check(cavs_memcpy_h2d(t.base, f.second->data.data(), (size_t)t.width * 4, stream_));
+      // through pinned memory, so that the upload is truly asynchronous and the caller's buffer
+      // is free as soon as Run returns
+      FeedStage &st = feed_stages_[f.first];
+      const int k = st.next;
+      st.next ^= 1;
+      const size_t bytes = (size_t)t.width * 4;
+      if (st.pending[k]) {
+        check(cavs_event_sync(st.uploaded[k]));
+        st.pending[k] = false;
+      }
+      if (!st.uploaded[k]) check(cavs_event_create(&st.uploaded[k]));
+      st.slot[k].reserve(bytes);
+      std::memcpy(st.slot[k].get(), f.second->data.data(), bytes);
+      check(cavs_memcpy_h2d(t.base, st.slot[k].get(), bytes, stream_));
+      check(cavs_event_record(st.uploaded[k], stream_));
+      st.pending[k] = true;
     }
   }
   bool train = false;
@@ -738,8 +756,19 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       check(cavs_sgd(w.base, gr.base, g.opt.lr, w.count(), stream_));
     }
   }
-  check(cavs_stream_sync(stream_));
   results->assign(outputs.size(), nullptr);
+  // A Run that asks for the optimizer only (the training loop of the reference's apps) has
+  // nothing to hand back: it returns with the step still in flight, and the host prepares the
+  // next batch meanwhile.  Whatever reads a value afterwards waits for the stream first.
+  bool reads = false;
+  for (auto &o : outputs)
+    if (!(g.opt.present && o == g.opt.output)) reads = true;
+  if (!reads) {
+    dirty_ = true;
+    return;
+  }
+  check(cavs_stream_sync(stream_));
+  dirty_ = false;
   for (size_t i = 0; i < outputs.size(); i++) {
     if (g.opt.present && outputs[i] == g.opt.output) continue;
     Tensor &t = tensor(outputs[i]);

@@ -29,6 +29,16 @@ struct Tensor {
   size_t count() const { return (size_t)(per_vertex ? rows * width : width); }
 };
 
+// Pinned staging of one device placeholder's feed: two slots alternate, each guarded by an
+// event recorded after its upload, so that Run can return while the copy is still in flight and
+// the caller may overwrite its own buffer at once.
+struct FeedStage {
+  PinnedArray<char> slot[2];
+  void *uploaded[2] = {nullptr, nullptr};
+  bool pending[2] = {false, false};
+  int next = 0;
+};
+
 struct HostTensor {  // C_Tensor of the C API
   std::string name;
   std::vector<int> shape;
@@ -80,6 +90,8 @@ class Executor {
   bool allow_fused_ = true, lowered_ = false;
   int pairing_ = 0;
   std::map<std::string, std::unique_ptr<Tensor>> tensors_;
+  std::map<std::string, FeedStage> feed_stages_;
+  bool dirty_ = false;  // device work queued by a Run that returned without waiting for it
   std::map<std::string, std::vector<float>> pending_vars_;  // SetVariable before compile
   bool vars_initialised_ = false;
 
