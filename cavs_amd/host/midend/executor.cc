@@ -751,10 +751,17 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       const size_t bytes = cavs_clip_grads_workspace((int)gp.size());
       check(cavs_clip_grads((int)gp.size(), gp.data(), gn.data(), g.opt.clip, workspace(bytes), bytes, stream_));
     }
+    // every variable's update in one launch (they touch disjoint tensors)
+    std::vector<cavs_task> updates;
     for (auto &v : g.opt.vars) {
       Tensor &w = tensor(v), &gr = tensor(GetGradientName(v));
-      check(cavs_sgd(w.base, gr.base, g.opt.lr, w.count(), stream_));
+      updates.push_back({CAVS_TASK_SGD, g.opt.lr, (long long)w.count(), 0, 0, w.base, gr.base, nullptr, nullptr});
+      if (updates.size() == 12) {
+        check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
+        updates.clear();
+      }
     }
+    check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
   }
   results->assign(outputs.size(), nullptr);
   // A Run that asks for the optimizer only (the training loop of the reference's apps) has

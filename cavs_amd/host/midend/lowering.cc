@@ -401,13 +401,20 @@ void Executor::lowered_backward(const OpDef &d) {
     Tensor &t = *slot;
     t.width = e->width();
     t.per_vertex = false;
+    bool acc = accs && i < (int)accs->value_.list_i.size() && accs->value_.list_i[i] != 0;
+    float *src = const_cast<float *>(engine_->grad_ptr(s.param)) + s.offset;
+    if (!acc) {
+      // a view of the engine's gradient array: it stays valid until the next backward pass, and
+      // whoever consumes it in the main scope reads it in this Run
+      t.base = src;
+      continue;
+    }
     if (t.own.capacity() < (size_t)t.width) {
       check(cavs_stream_sync(stream_));
       t.own.reserve(t.width);
     }
-    t.base = t.own.get();
-    bool acc = accs && i < (int)accs->value_.list_i.size() && accs->value_.list_i[i] != 0;
-    check(cavs_ew_unary(CAVS_EW_ASSIGN, t.base, engine_->grad_ptr(s.param) + s.offset, (size_t)s.count, acc ? 1 : 0, stream_));
+    t.base = t.own.get();  // zeroed at the start of the pass like every accumulating output
+    check(cavs_ew_unary(CAVS_EW_ASSIGN, t.base, src, (size_t)s.count, 1, stream_));
   }
 }
 
