@@ -265,7 +265,7 @@ def main():
     a = ap.parse_args()
     if a.gpus != 1:
         sys.exit("bench.py: this build runs the F-over-G path on one GPU; instance graphs shard by sample "
-                 "across GPUs (see DESIGN.md) but no multi-GPU path is built -- run with --gpus 1")
+                 "across GPUs, one all-reduce of the weight gradients per step, but no multi-GPU path is built -- run with --gpus 1")
 
     import torch
 
