@@ -297,6 +297,19 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
       embed_sgd_block(static_cast<float *>(t.p0), static_cast<const float *>(t.p1), static_cast<const float *>(t.p2),
                       (int)t.n0, (int)t.n1, t.f0, static_cast<int *>(t.p3), (int)t.n2, b, lds.sgd);
       break;
+    case CAVS_TASK_BLOCKS_SGD: {  // block k of p1 ([n1 blocks of n0]) -> block perm(k) of p2 (and p0 -= f0 * it)
+      float *__restrict__ w = static_cast<float *>(t.p0);
+      const float *__restrict__ src = static_cast<const float *>(t.p1);
+      float *__restrict__ gout = static_cast<float *>(t.p2);
+      const int bw = (int)t.n0, total = bw * (int)t.n1;
+      for (int i = b * 256 + tid; i < total; i += nb * 256) {
+        const int k = i / bw, d = (int)((t.n2 >> (4 * k)) & 15) * bw + i % bw;
+        const float g = src[i];
+        if (gout) gout[d] = g;
+        if (w) w[d] -= t.f0 * g;
+      }
+      break;
+    }
     case CAVS_TASK_SUM_PARTS:  // p1[i] (i < n2) or p2[i - n2] = sum over p < n0 of p0[p * n1 + i], i < n1
       sum_parts_block(static_cast<const float *>(t.p0), (int)t.n0, (int)t.n1, (int)t.n2, static_cast<float *>(t.p1),
                       static_cast<float *>(t.p2), b, lds.sums);
@@ -435,6 +448,19 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         CAVS_REQUIRE(t.p0 && t.p1 && t.p2 && t.p3, "cavs_run_tasks: job %d: null pointer", i);
         blocks = (t.n0 + kSgdChunk - 1) / kSgdChunk;
         break;
+      case CAVS_TASK_BLOCKS_SGD: {
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n1 <= 8 && t.n0 < (1 << 26), "cavs_run_tasks: job %d: bad shape", i);
+        if (t.n0 == 0 || t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p1 && (t.p0 || t.p2), "cavs_run_tasks: job %d: null pointer", i);
+        unsigned seen = 0;
+        for (int k = 0; k < (int)t.n1; k++) {
+          const int d = (int)((t.n2 >> (4 * k)) & 15);
+          CAVS_REQUIRE(d < (int)t.n1 && !(seen >> d & 1u), "cavs_run_tasks: job %d: the block map is not a permutation", i);
+          seen |= 1u << d;
+        }
+        blocks = (t.n0 * t.n1 + 1023) / 1024;
+        break;
+      }
       case CAVS_TASK_SUM_PARTS:
         CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n1 < (1 << 30) && t.n0 < (1 << 30) && t.n2 >= 0 && t.n2 <= t.n1,
                      "cavs_run_tasks: job %d: bad shape", i);

@@ -29,7 +29,7 @@ class Task(C.Structure):
                 ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P)]
 
 
-TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS = 0, 1, 2, 3, 4
+TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD = 0, 1, 2, 3, 4, 5
 
 
 class GemmDesc(C.Structure):

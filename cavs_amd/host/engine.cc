@@ -28,6 +28,7 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
   if (cfg.H <= 0) fail(CAVS_EINVAL, "hidden size must be positive");
   const size_t H = cfg.H;
   E_ = cfg.model == CAVS_MODEL_LSTM ? cfg.H : cfg.E;  // the chain LSTM requires E == H
+  ld_e_ = cfg.model == CAVS_MODEL_TREELSTM ? E_ + 4 : E_;
   mw_ = cfg.model == CAVS_MODEL_TREEFC ? cfg.H : 2 * cfg.H;
   nch_ = cfg.model == CAVS_MODEL_LSTM ? 1 : 2;
   if (cfg.model != CAVS_MODEL_TREEFC && (cfg.V <= 0 || E_ <= 0))
@@ -45,7 +46,7 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
   switch (cfg.model) {
     case CAVS_MODEL_TREELSTM:
       add_param("Emb", (size_t)cfg.V * E_);
-      add_param("W", (size_t)E_ * 4 * H);
+      add_param("W", (size_t)E_ * 4 * H, 4 * 4 * H);  // four more rows (one used): the bias gradient comes out of the same product
       add_param("U", 4 * H * H);
       add_param("Bv", 4 * H);
       break;
@@ -72,11 +73,11 @@ Engine::~Engine() {
   if (own_stream_) cavs_stream_destroy(stream_);
 }
 
-void Engine::add_param(const std::string &name, size_t n) {
+void Engine::add_param(const std::string &name, size_t n, size_t extra_grad) {
   auto p = std::make_unique<Param>();
   p->n = n;
   p->own_w.reserve(n);
-  p->own_g.reserve(n);
+  p->own_g.reserve(n + extra_grad);
   p->w = p->own_w.get();
   p->g = p->own_g.get();
   check(cavs_zero(p->w, n * 4, stream_));
@@ -244,7 +245,17 @@ void Engine::reserve_edges() {
       R(xs_prev_, cap);
       emb_sparse_valid_ = false;
     }
-    R(e_, cap * E_);
+    R(e_, cap * ld_e_);
+    if (ld_e_ != E_ && e_ones_rows_ < cap) {  // (re)allocated: zero padding and the column of ones
+      std::vector<float> col(ld_e_, 0.f);
+      col[E_] = 1.f;
+      ones_col_.reserve(ld_e_);
+      check(cavs_memcpy_h2d(ones_col_.get(), col.data(), col.size() * 4, stream_));
+      check(cavs_stream_sync(stream_));
+      check(cavs_zero(e_.get(), cap * ld_e_ * 4, stream_));
+      check(cavs_bias_add_rows(e_.get(), e_.get(), ones_col_.get(), (int)cap, ld_e_, stream_));
+      e_ones_rows_ = cap;
+    }
     R(de_, cap * E_);
     R(xW_, cap * 4 * H);
     R(dxW_, cap * 4 * H);
@@ -382,6 +393,7 @@ void Engine::backward_only(const float *dgraph_out) {
     case CAVS_MODEL_LSTM: lstm_backward(); break;
     default: treefc_backward();
   }
+  settle_bias_row(0.f, nullptr);  // no update follows in here: the bias gradient is delivered now
   check(cavs_event_record(ev_[3], stream_));
   ev_bwd_valid_ = true;
 }
@@ -447,8 +459,11 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       // only: every other row of its gradient is zero, so the dense update would not move it
       // all of it in one launch: the updates touch disjoint tensors
       std::vector<cavs_task> tasks;
+      const bool bias_job = bias_row_pending_;
+      settle_bias_row(lr, &tasks);
       for (auto &kv : params_) {
         Param &p = *kv.second;
+        if (kv.first == "Bv" && bias_job) continue;  // updated by the job that delivers its gradient
         if (kv.first == "Emb" && emb_dirty_n_ == N) {
           const int E = (int)(p.n / cfg_.V);
           if (emb_stamp_.capacity() < (size_t)cfg_.V) {
@@ -462,6 +477,8 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       }
       check(cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
       c_launches_ += 1;
+    } else {
+      settle_bias_row(0.f, nullptr);
     }
   }
 }
@@ -490,9 +507,9 @@ int Engine::fused_rows() const {
 void Engine::treelstm_forward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w, *Bv = param("Bv").w;
-  check(cavs_embed_pull_fwd(e_.get(), E, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
+  check(cavs_embed_pull_fwd(e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
   c_launches_ += 1;
-  gemm(0, 0, N, 4 * H, E, e_.get(), E, W, 4 * H, 0.f, xW_.get(), 4 * H);
+  gemm(0, 0, N, 4 * H, E, e_.get(), ld_e_, W, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
@@ -611,20 +628,49 @@ void Engine::treelstm_backward() {
   // accumulates the same sums round by round)
   const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
   float *dU = param("U").g;
+  const bool bias_row = bias_row_ok();  // the ones column of e_ turns row E of dW into the column sums of dxW
   gemm_group({
       {0, 1, N, E, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, W, 4 * H, de_.get(), E},
-      {1, 0, E, 4 * H, N, 1.f, 0.f, e_.get(), E, dxW_.get(), 4 * H, param("W").g, 4 * H},
+      // (all four padding columns of e_ take part, so that the product keeps 16-byte operand loads)
+      {1, 0, bias_row ? ld_e_ : E, 4 * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), 4 * H, param("W").g, 4 * H},
       {1, 0, H, 3 * H, N - lp, 1.f, 0.f, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H},
       {1, 0, H, H, 2 * (N - lp), 1.f, 0.f, G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
        dU + (size_t)3 * H * H, H},
   });
   embedding_backward(E);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
+  if (bias_row) {
+    bias_row_pending_ = true;  // settled by the launch that ends the step (or right after this pass)
+    return;
+  }
   const int dst_block[4] = {0, 3, 2, 1};  // dxW block k ([i|o|u|f]) lands in bias block dst_block[k]
   const size_t cs_bytes = cavs_colsum_blocks_workspace(N, H, 4);
   float *cs_ws = workspace(cs_bytes);
   check(cavs_colsum_blocks(param("Bv").g, dxW_.get(), 4 * H, N, H, 4, dst_block, cs_ws, cs_bytes, stream_));
   c_launches_ += 2;
+}
+
+// The gradient of W lives in the engine's own array, which has the spare row.
+bool Engine::bias_row_ok() const {
+  if (cfg_.model != CAVS_MODEL_TREELSTM) return false;
+  const Param &w = *params_.at("W");
+  return w.g == w.own_g.get();
+}
+
+// Row E of dW ([i|o|u|f] blocks) -> Bv.g ([i|f|u|o]), and the update of Bv with it when lr != 0:
+// as a job of `tasks` if given, else as a launch of its own.
+void Engine::settle_bias_row(float lr, std::vector<cavs_task> *tasks) {
+  if (!bias_row_pending_) return;
+  bias_row_pending_ = false;
+  Param &w = param("W"), &b = param("Bv");
+  const long long map = 0 | (3 << 4) | (2 << 8) | (1 << 12);  // block k of the row lands in bias block map[k]
+  cavs_task t{CAVS_TASK_BLOCKS_SGD, lr, cfg_.H, 4, map, lr != 0.f ? b.w : nullptr, w.g + w.n, b.g, nullptr};
+  if (tasks) {
+    tasks->push_back(t);
+  } else {
+    check(cavs_run_tasks(1, &t, stream_));
+    c_launches_ += 1;
+  }
 }
 
 // EmbeddingLookup_grad (cavs/backend/op_impl_embedding.cu:58-92): scatter-add of the rows of

@@ -60,7 +60,7 @@ class Engine {
 
  private:
   Param &param(const std::string &name);
-  void add_param(const std::string &name, size_t n);
+  void add_param(const std::string &name, size_t n, size_t extra_grad = 0);
   void reserve_edges();
   void ensure(DeviceArray<float> &a, size_t n);  // grow after draining the stream
   void upload_index_arena();
@@ -144,6 +144,14 @@ class Engine {
   bool emb_sparse_valid_ = true;  // the table is zero outside xs_prev_[0, emb_dirty_n_)
   bool emb_cleared_ = false;      // the backward prologue of this step already cleared those rows
   std::vector<cavs_task> pending_tasks_;  // jobs queued for the launch that opens backward
+  // Tree-LSTM: e_ carries a column of ones after its E columns, so that the deferred product
+  // e^T * dxW yields the bias gradient (column sums of dxW) as row E of dW for free
+  int ld_e_ = 0;
+  size_t e_ones_rows_ = 0;       // rows of e_ whose ones column is initialised
+  DeviceArray<float> ones_col_;  // [ld_e_]: 1 at column E
+  bool bias_row_pending_ = false;  // row E of dW holds this step's bias gradient, not yet in Bv.g
+  bool bias_row_ok() const;
+  void settle_bias_row(float lr, std::vector<cavs_task> *tasks);
   DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds

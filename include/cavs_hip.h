@@ -353,9 +353,13 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *   CAVS_TASK_EMBED_SGD  cavs_embed_sgd(p0 = table, p1 = dtable, p2 = ids, n0 = n, n1 = E,
  *                                       f0 = lr, p3 = stamp, n2 = epoch)
  *   CAVS_TASK_SUM_PARTS  out[i] = sum over p < n0 of p0[p * n1 + i] in a fixed order, i < n1, where
- *                        out[i] is p1[i] for i < n2 and p2[i - n2] above */
+ *                        out[i] is p1[i] for i < n2 and p2[i - n2] above
+ *   CAVS_TASK_BLOCKS_SGD p1 holds n1 (<= 8) blocks of n0 floats; block k goes to block d_k of p2 (if
+ *                        given) and p0[d_k block] -= f0 * it (if p0 given); d_k = (n2 >> 4k) & 15, a
+ *                        permutation.  A gradient that arrives in another block order than its
+ *                        parameter's (the gate bias, apps/paper/tree-lstm-cavs.cc:120-123 vs :143-148). */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
-       CAVS_TASK_SUM_PARTS = 4 };
+       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5 };
 typedef struct cavs_task {
   int kind;
   float f0;

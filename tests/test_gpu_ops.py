@@ -788,6 +788,19 @@ def test_several_small_jobs_in_one_launch(g):
     want[rows] = 0
     np.testing.assert_array_equal(g.host(d_dirty), want)
     np.testing.assert_array_equal(g.host(d_table), table - np.float32(0.5) * grad)
+    # a gradient that arrives in another block order than its parameter's
+    bw, perm = 37, [0, 3, 2, 1]
+    src, wb = r.bulk_normal(4 * bw), r.bulk_normal(4 * bw)
+    d_src, d_wb, d_gb = g.devf(src), g.devf(wb), g.zeros(4 * bw)
+    code = sum(d << (4 * k) for k, d in enumerate(perm))
+    g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_BLOCKS_SGD, 0.5, bw, 4, code, g.P(d_wb), g.P(d_src), g.P(d_gb), None)), g.stream())
+    want_g = np.empty(4 * bw, np.float32)
+    for k, d in enumerate(perm):
+        want_g[d * bw:(d + 1) * bw] = src[k * bw:(k + 1) * bw]
+    np.testing.assert_array_equal(g.host(d_gb), want_g)
+    np.testing.assert_array_equal(g.host(d_wb), wb - np.float32(0.5) * want_g)
+    with pytest.raises(hip.CavsError, match="not a permutation"):
+        g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_BLOCKS_SGD, 0.5, bw, 4, 0, g.P(d_wb), g.P(d_src), g.P(d_gb), None)), g.stream())
     with pytest.raises(hip.CavsError, match="unknown kind"):
         g.call("cavs_run_tasks", 1, (T * 1)(T(9, 0.0, 1, 1, 0, g.P(dA), g.P(dB), None, None)), g.stream())
     with pytest.raises(hip.CavsError, match="at most 12"):
