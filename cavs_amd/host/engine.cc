@@ -653,6 +653,9 @@ void Engine::treelstm_backward() {
 // The gradient of W lives in the engine's own array, which has the spare row.
 bool Engine::bias_row_ok() const {
   if (cfg_.model != CAVS_MODEL_TREELSTM) return false;
+  // free only while the extra rows stay inside the last row tile of the product (E = 300: yes;
+  // E = 1024 would grow the 128-row tiling from 8 to 9 tiles)
+  if ((E_ + 4 + 127) / 128 != (E_ + 127) / 128) return false;
   const Param &w = *params_.at("W");
   return w.g == w.own_g.get();
 }
