@@ -923,15 +923,21 @@ void Engine::head_forward_backward(bool backward) {
       c_launches_ += 1;
       return;
     }
-    gemm(0, 1, N, C, H, GO_.get(), H, Wfc.w, H, 0.f, logits_.get(), C);
-    check(cavs_bias_add_rows(logits_.get(), logits_.get(), bfc.w, N, C, stream_));
+    {  // logits = GO * Wfc^T + bfc: the bias rides in the product's epilogue (row r adds D[r >> 30] = D[0])
+      float *ws = workspace(cavs_sgemm_splitk_workspace(N, C, H));
+      ProfScope ps(this, K_GEMM);
+      check(cavs_sgemm_addrows(0, 1, N, C, H, GO_.get(), H, Wfc.w, H, bfc.w, C, 30, logits_.get(), C, ws, ws_.capacity() * 4, stream_));
+      c_gemm_flops_ += 2.0 * N * C * H;
+      c_launches_ += 1;
+    }
     check(cavs_softmax_xent(loss_.get(), backward ? dlogits_.get() : nullptr, logits_.get(), d_labels_, N, C, stream_));
-    c_launches_ += 2;
+    c_launches_ += 1;
     if (backward) {
-      gemm_splitk(1, 0, C, H, N, dlogits_.get(), C, GO_.get(), H, Wfc.g, H);
+      // both read d logits and write different outputs: one launch when they are small
+      gemm_group({{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, GO_.get(), H, Wfc.g, H},
+                  {0, 0, N, H, C, 1.f, 0.f, dlogits_.get(), C, Wfc.w, H, dGO_.get(), H}});
       check(cavs_colsum(bfc.g, dlogits_.get(), C, N, C, 0, stream_));
       c_launches_ += 1;
-      gemm(0, 0, N, H, C, dlogits_.get(), C, Wfc.w, H, 0.f, dGO_.get(), H);
     }
     return;
   }
