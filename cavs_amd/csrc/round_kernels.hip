@@ -276,6 +276,27 @@ __global__ void treelstm_round_leaves_fwd_kernel(RoundLeavesArgs a) {
 }
 
 // ------------------------------------------------------------------ backward, gate part
+// Gate gradients of one hidden unit of one vertex.  mh, mc: gradient of the vertex's message
+// ([h|c] halves); dr: gradient of its pushed return value; c_left, c_right: the children's c
+// (zero for a leaf).
+struct GateGrad {
+  float di, d_o, du, dfl, dfr, dc;
+};
+__device__ inline GateGrad gate_grad(float i, float o, float u, float f_l, float f_r, float tc, float mh, float mc, float dr,
+                                     float c_left, float c_right) {
+  GateGrad g;
+  const float dh = mh + dr;
+  const float d_o = dh * tc;
+  const float dc = mc + (dh * o) * (1.f - tc * tc);
+  g.dfl = (dc * c_left) * (f_l * (1.f - f_l));
+  g.dfr = (dc * c_right) * (f_r * (1.f - f_r));
+  g.di = (dc * u) * (i * (1.f - i));
+  g.d_o = d_o * (o * (1.f - o));
+  g.du = (dc * i) * (1.f - u * u);
+  g.dc = dc;
+  return g;
+}
+
 // Elementwise: reads the message gradient through the scatter list (grad of Scatter is
 // Gather), writes the pre-activation gradients and the c half of the children's message
 // gradients straight into the children's pool rows (grad of Gather is Scatter).
@@ -328,18 +349,11 @@ __global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
   for (int k = 0; k < W; k++) {
     const float mh = src >= 0 ? dmh[k] : 0.f, mc = src >= 0 ? dmc[k] : 0.f;
     const float c_left = internal ? cl[k] : 0.f, c_right = internal ? cr[k] : 0.f;
-    const float i = gi[k], o = go[k], u = gu[k], f_l = gfl[k], f_r = gfr[k], tc = gtc[k];
-    const float dh = mh + dr[k];
-    const float d_o = dh * tc;
-    const float dc = mc + (dh * o) * (1.f - tc * tc);
-    const float del_fl = (dc * c_left) * (f_l * (1.f - f_l));
-    const float del_fr = (dc * c_right) * (f_r * (1.f - f_r));
-    di[k] = (dc * u) * (i * (1.f - i));
-    dvo[k] = d_o * (o * (1.f - o));
-    du[k] = (dc * i) * (1.f - u * u);
-    dfs[k] = del_fl + del_fr;
-    dfl[k] = del_fl; dfr[k] = del_fr;
-    dcl[k] = dc * f_l; dcr[k] = dc * f_r;
+    const GateGrad q = gate_grad(gi[k], go[k], gu[k], gfl[k], gfr[k], gtc[k], mh, mc, dr[k], c_left, c_right);
+    di[k] = q.di; dvo[k] = q.d_o; du[k] = q.du;
+    dfs[k] = q.dfl + q.dfr;
+    dfl[k] = q.dfl; dfr[k] = q.dfr;
+    dcl[k] = q.dc * gfl[k]; dcr[k] = q.dc * gfr[k];
   }
   auto st = [](float *p, const float (&v)[W]) {
     if constexpr (W == 4) {
@@ -359,10 +373,59 @@ __global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
   }
 }
 
+// The same for the vertices nobody sends a message gradient to (the roots), named by a list of
+// slab rows over whole-batch slabs: d c of a vertex goes to row v of `dc`, from where the launch
+// of the vertex's own round hands it on to the children.
+struct BwdGatesRowsArgs {
+  const int *rows;       // [n] slab rows
+  const float *dret;     // gradient of the pushed return value: row dret_rows[v]
+  const int *dret_rows;  // [*] by slab row
+  const float *gates;    // [*, 6H]
+  const float *G;        // [2*, 2H]
+  float *dxW;            // [*, 4H] (ld_dxw)
+  long ld_dxw;
+  float *dF;             // [2*, H]
+  float *dc;             // [*, H]
+  int n, H, leaf_rows;   // slab rows below leaf_rows are leaves
+};
+
+template <int W>
+__global__ void treelstm_bwd_gates_rows_kernel(BwdGatesRowsArgs a) {
+  const int H = a.H, hw = H / W;
+  const long H2 = 2L * H;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int j = (int)(idx % hw) * W;
+  const long v = a.rows[idx / hw];
+  const bool internal = v >= a.leaf_rows;
+  const float *g = a.gates + v * 6 * H + j;
+  const float *dr = a.dret + (long)a.dret_rows[v] * H + j;
+  const float *cl = a.G + (2 * v) * H2 + H + j, *cr = cl + H2;
+  float *dx = a.dxW + v * a.ld_dxw + j;
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const GateGrad q = gate_grad(g[k], g[H + k], g[2 * H + k], g[3 * H + k], g[4 * H + k], g[5 * H + k], 0.f, 0.f, dr[k],
+                                 internal ? cl[k] : 0.f, internal ? cr[k] : 0.f);
+    dx[k] = q.di; dx[H + k] = q.d_o; dx[2 * H + k] = q.du; dx[3 * H + k] = q.dfl + q.dfr;
+    if (internal) {
+      a.dF[(2 * v) * H + j + k] = q.dfl;
+      a.dF[(2 * v + 1) * H + j + k] = q.dfr;
+      a.dc[v * H + j + k] = q.dc;
+    }
+  }
+}
+
 // ------------------------------------------------------------------ backward, children part
 // dh_l = [d_i|d_o|d_u] * U_iou^T + d_fl * U_f^T, dh_r likewise with d_fr, written into the h
 // half of the children's pool-gradient rows.  UT holds the transposed weights ([3H,H] then
 // [H,H]) so that the B operand is TILE consecutive floats per k, as in the forward kernel.
+//
+// FOLD: the launch also does the gate part of the children.  `child` then names the children
+// by slab row over whole-batch slabs; the thread that holds d h of hidden unit j of a child has
+// everything the child's gate gradients of that unit need (its saved gates, its d return value,
+// d c = d c(parent) * f(parent)), so it writes the child's rows of dxW / dF / dc directly and
+// the message gradient never makes the trip through the pool.  What it needs besides the
+// products is fetched while they run.
 struct RoundBwdChildArgs {
   const float *dxW;   // [n, 4H] (ld_dxw); columns [0, 3H) are read
   long ld_dxw;
@@ -371,9 +434,14 @@ struct RoundBwdChildArgs {
   const int *child;   // [2n]
   float *dpool;       // [*, 2H]
   int n, H;
+  // FOLD only; whole-batch slabs, the round starts at slab row row0
+  float *dxW_all, *dF_all, *dc_all;
+  const float *gates_all, *G_all, *dret;
+  const int *dret_rows;
+  int row0, leaf_rows;
 };
 
-template <int TILE, int WAVES>
+template <int TILE, int WAVES, bool FOLD>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -398,7 +466,7 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   // the epilogue's targets, fetched now: child rows of the elements this thread will write
   constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
   bool eon[EPT];
-  int ecl[EPT], ecr[EPT], ej[EPT], elds[EPT];
+  int ecl[EPT], ecr[EPT], ej[EPT], elds[EPT], eb[EPT];
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
     const int e = tid + q * kRoundThreads;
@@ -412,7 +480,55 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       ecl[q] = a.child[2 * b];
       ecr[q] = a.child[2 * b + 1];
     }
+    if constexpr (FOLD) eb[q] = b;
   }
+  // FOLD: operands of the children's gate gradients ([q][side])
+  struct Kid {
+    float g[6], dr, cl, cr;
+  };
+  Kid kid[FOLD ? EPT : 1][2];
+  float pdc[FOLD ? EPT : 1], pf[FOLD ? EPT : 1][2];
+  int kdr[FOLD ? EPT : 1][2];
+  if constexpr (FOLD) {
+#pragma unroll
+    for (int q = 0; q < EPT; q++) {
+      kdr[q][0] = ecl[q] >= 0 ? a.dret_rows[ecl[q]] : 0;
+      kdr[q][1] = ecr[q] >= 0 ? a.dret_rows[ecr[q]] : 0;
+    }
+  }
+  auto fetch_kids = [&]() {
+    if constexpr (FOLD) {
+#pragma unroll
+      for (int q = 0; q < EPT; q++) {
+        const int j = ej[q];
+        const long b = a.row0 + eb[q];
+        pdc[q] = pf[q][0] = pf[q][1] = 0.f;
+        if (eon[q]) {
+          pdc[q] = a.dc_all[b * H + j];
+          pf[q][0] = a.gates_all[b * 6 * H + 3 * H + j];
+          pf[q][1] = a.gates_all[b * 6 * H + 4 * H + j];
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const long v = s ? ecr[q] : ecl[q];
+          Kid &kd = kid[q][s];
+#pragma unroll
+          for (int t = 0; t < 6; t++) kd.g[t] = 0.f;
+          kd.dr = kd.cl = kd.cr = 0.f;
+          if (v >= 0) {
+            const float *g = a.gates_all + v * 6 * H + j;
+#pragma unroll
+            for (int t = 0; t < 6; t++) kd.g[t] = g[(long)t * H];
+            kd.dr = a.dret[(long)kdr[q][s] * H + j];
+            if (v >= a.leaf_rows) {
+              kd.cl = a.G_all[(2 * v) * H2 + H + j];
+              kd.cr = a.G_all[(2 * v + 1) * H2 + H + j];
+            }
+          }
+        }
+      }
+    }
+  };
 
   Acc acc[NP];
 #pragma unroll
@@ -456,6 +572,7 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       }
     }
   }
+  fetch_kids();
   {  // P1, P2: K = H, one B operand for both
     const int K = H;
     const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
@@ -510,8 +627,27 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
       v[p] = s;
     }
-    if (ecl[q] >= 0) a.dpool[ecl[q] * H2 + ej[q]] = v[0] + v[1];
-    if (ecr[q] >= 0) a.dpool[ecr[q] * H2 + ej[q]] = v[0] + v[2];
+    if constexpr (FOLD) {
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        const long c = s ? ecr[q] : ecl[q];
+        if (c < 0) continue;
+        const Kid &kd = kid[q][s];
+        const int j = ej[q];
+        const GateGrad gg = gate_grad(kd.g[0], kd.g[1], kd.g[2], kd.g[3], kd.g[4], kd.g[5], v[0] + v[1 + s], pdc[q] * pf[q][s],
+                                      kd.dr, kd.cl, kd.cr);
+        float *dx = a.dxW_all + c * a.ld_dxw + j;
+        dx[0] = gg.di; dx[H] = gg.d_o; dx[2 * H] = gg.du; dx[3 * H] = gg.dfl + gg.dfr;
+        if (c >= a.leaf_rows) {
+          a.dF_all[(2 * c) * H + j] = gg.dfl;
+          a.dF_all[(2 * c + 1) * H + j] = gg.dfr;
+          a.dc_all[c * H + j] = gg.dc;
+        }
+      }
+    } else {
+      if (ecl[q] >= 0) a.dpool[ecl[q] * H2 + ej[q]] = v[0] + v[1];
+      if (ecr[q] >= 0) a.dpool[ecr[q] * H2 + ej[q]] = v[0] + v[2];
+    }
   }
 }
 
@@ -525,6 +661,16 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
   __syncthreads();
   for (int i = ty; i < 32; i += 8)
     if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
+}
+
+template <bool FOLD>
+static void launch_bwd_children(const RoundBwdChildArgs &a, hipStream_t st) {
+  const RoundPlan p = plan_round(a.n);
+  dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
+  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, FOLD>, grid, 256, 0, st, a);
+  else if (p.tile == 16) launch(treelstm_round_bwd_children_kernel<16, 8, FOLD>, grid, 512, 0, st, a);
+  else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<32, 4, FOLD>, grid, 256, 0, st, a);
+  else launch(treelstm_round_bwd_children_kernel<32, 8, FOLD>, grid, 512, 0, st, a);
 }
 
 }  // namespace cavs
@@ -606,14 +752,45 @@ int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dxW && dF && UT && child && dpool, "cavs_treelstm_round_bwd_children: null pointer");
   CAVS_REQUIRE(aligned16(dxW) && aligned16(dF), "cavs_treelstm_round_bwd_children: dxW and dF must be 16-byte aligned");
-  RoundBwdChildArgs a{dxW, ld_dxw, dF, UT, child, dpool, n, H};
-  const RoundPlan p = plan_round(n);
-  dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
+  RoundBwdChildArgs a{dxW, ld_dxw, dF, UT, child, dpool, n, H, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+  launch_bwd_children<false>(a, as_stream(stream));
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_round_bwd_children_gates(float *dxW, int ld_dxw, float *dF, float *dc, const float *UT,
+                                           const int *child_rows, const float *gates, const float *G, const float *dret,
+                                           const int *dret_rows, int row0, int n, int leaf_rows, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && row0 >= 0 && leaf_rows >= 0 && round_shape_ok(H) && ld_dxw >= 4 * H && ld_dxw % 4 == 0,
+               "cavs_treelstm_round_bwd_children_gates: bad shape row0=%d n=%d leaf_rows=%d H=%d ld=%d (H must be a multiple of 32)",
+               row0, n, leaf_rows, H, ld_dxw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dxW && dF && dc && UT && child_rows && gates && G && dret && dret_rows,
+               "cavs_treelstm_round_bwd_children_gates: null pointer");
+  CAVS_REQUIRE(aligned16(dxW) && aligned16(dF), "cavs_treelstm_round_bwd_children_gates: dxW and dF must be 16-byte aligned");
+  RoundBwdChildArgs a{dxW + (long)row0 * ld_dxw, ld_dxw, dF + 2L * row0 * H, UT, child_rows, nullptr, n, H,
+                      dxW, dF, dc, gates, G, dret, dret_rows, row0, leaf_rows};
+  launch_bwd_children<true>(a, as_stream(stream));
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_bwd_gates_rows(const int *rows, int n, const float *dret, const int *dret_rows, const float *gates,
+                                 const float *G, float *dxW, int ld_dxw, float *dF, float *dc, int leaf_rows, int H,
+                                 void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && leaf_rows >= 0 && ld_dxw >= 4 * H, "cavs_treelstm_bwd_gates_rows: bad shape n=%d H=%d ld=%d", n, H,
+               ld_dxw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(rows && dret && dret_rows && gates && G && dxW && dF && dc, "cavs_treelstm_bwd_gates_rows: null pointer");
+  BwdGatesRowsArgs a{rows, dret, dret_rows, gates, G, dxW, ld_dxw, dF, dc, n, H, leaf_rows};
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4>, grid, 256, 0, st, a);
-  else if (p.tile == 16) launch(treelstm_round_bwd_children_kernel<16, 8>, grid, 512, 0, st, a);
-  else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<32, 4>, grid, 256, 0, st, a);
-  else launch(treelstm_round_bwd_children_kernel<32, 8>, grid, 512, 0, st, a);
+  if (H % 4 == 0) {
+    long total = (long)n * (H / 4);
+    launch(treelstm_bwd_gates_rows_kernel<4>, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  } else {
+    long total = (long)n * H;
+    launch(treelstm_bwd_gates_rows_kernel<1>, (unsigned)((total + 255) / 256), 256, 0, st, a);
+  }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

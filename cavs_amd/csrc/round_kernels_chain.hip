@@ -241,6 +241,27 @@ __global__ void lstm_round_leaves_fwd_kernel(LstmLeavesArgs a) {
   if (out >= 0) stw<W>(a.go + (long)out * H + j, mh);
 }
 
+// Gate gradients of one hidden unit of one chain vertex.  mh, mc: gradient of its message
+// ([h|c] halves); dr: gradient of its pushed return value; cprev: the predecessor's c (zero at
+// the first step).
+struct LstmGateGrad {
+  float di, df, du, d_o, dc;
+};
+__device__ inline LstmGateGrad lstm_gate_grad(float i, float f, float u, float o, float tc, float mh, float mc, float dr,
+                                              float cprev) {
+  LstmGateGrad g;
+  const float dh = mh + dr;
+  const float d_o = dh * tc;
+  const float dc = mc + (dh * o) * (1.f - tc * tc);
+  g.di = (dc * u) * (i * (1.f - i));
+  g.df = (dc * cprev) * (f * (1.f - f));
+  g.du = (dc * i) * (1.f - u * u);
+  g.d_o = d_o * (o * (1.f - o));
+  g.dc = dc;
+  return g;
+}
+__device__ inline float treefc_dz(float dh, float y, int act) { return act ? dh * (1.f - y * y) : (y > 0.f ? dh : 0.f); }
+
 struct LstmBwdGatesArgs {
   const float *dpool;
   const int *pair;
@@ -275,25 +296,77 @@ __global__ void lstm_round_bwd_gates_kernel(LstmBwdGatesArgs a) {
 #pragma unroll
   for (int k = 0; k < W; k++) {
     const float mh = src >= 0 ? dmh[k] : 0.f, mc = src >= 0 ? dmc[k] : 0.f, cpv = a.G ? cprev[k] : 0.f;
-    const float i = gi[k], f = gf[k], u = gu[k], o = go[k], tc = gtc[k];
-    const float dh = mh + dr[k];
-    const float d_o = dh * tc;
-    const float dc = mc + (dh * o) * (1.f - tc * tc);
-    di[k] = (dc * u) * (i * (1.f - i));
-    df[k] = (dc * cpv) * (f * (1.f - f));
-    du[k] = (dc * i) * (1.f - u * u);
-    dvo[k] = d_o * (o * (1.f - o));
-    dcp[k] = dc * f;
+    const LstmGateGrad q = lstm_gate_grad(gi[k], gf[k], gu[k], go[k], gtc[k], mh, mc, dr[k], cpv);
+    di[k] = q.di; df[k] = q.df; du[k] = q.du; dvo[k] = q.d_o;
+    dcp[k] = q.dc * gf[k];
   }
   float *d = a.da + r * a.ld_da + j;
   stw<W>(d, di); stw<W>(d + H, df); stw<W>(d + 2 * H, du); stw<W>(d + 3 * H, dvo);
   if (cp >= 0) stw<W>(a.dpool_out + cp * H2 + H + j, dcp);
 }
 
+// The pointwise backward part for the vertices nobody sends a message gradient to (the last step
+// of every sequence, the roots of the trees), named by a list of slab rows over whole-batch slabs.
+struct LstmBwdRowsArgs {
+  const int *rows;
+  const float *dret;
+  const int *dret_rows;  // [*] by slab row
+  const float *gates;    // [*, 5H]
+  const float *G;        // [*, 2H]
+  float *da;             // [*, 4H] (ld)
+  long ld_da;
+  float *dc;             // [*, H]
+  int n, H, leaf_rows;
+};
+
+template <int W>
+__global__ void lstm_bwd_gates_rows_kernel(LstmBwdRowsArgs a) {
+  const int H = a.H, hw = H / W;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int j = (int)(idx % hw) * W;
+  const long v = a.rows[idx / hw];
+  const bool later = v >= a.leaf_rows;
+  const float *g = a.gates + v * 5 * H + j, *dr = a.dret + (long)a.dret_rows[v] * H + j, *cp = a.G + v * 2 * H + H + j;
+  float *d = a.da + v * a.ld_da + j;
+#pragma unroll
+  for (int k = 0; k < W; k++) {
+    const LstmGateGrad q = lstm_gate_grad(g[k], g[H + k], g[2 * H + k], g[3 * H + k], g[4 * H + k], 0.f, 0.f, dr[k], later ? cp[k] : 0.f);
+    d[k] = q.di; d[H + k] = q.df; d[2 * H + k] = q.du; d[3 * H + k] = q.d_o;
+    if (later) a.dc[v * H + j + k] = q.dc;
+  }
+}
+
+struct TreeFcBwdRowsArgs {
+  const int *rows;
+  const float *dret;
+  const int *dret_rows;
+  const float *h;  // [*, H]
+  float *dz;       // [*, H]
+  int n, H, act;
+};
+
+template <int W>
+__global__ void treefc_bwd_rows_kernel(TreeFcBwdRowsArgs a) {
+  const int H = a.H, hw = H / W;
+  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)a.n * hw) return;
+  const int j = (int)(idx % hw) * W;
+  const long v = a.rows[idx / hw];
+  const float *dr = a.dret + (long)a.dret_rows[v] * H + j, *y = a.h + v * H + j;
+#pragma unroll
+  for (int k = 0; k < W; k++) a.dz[v * H + j + k] = treefc_dz(0.f + dr[k], y[k], a.act);
+}
+
 // Gradient of the gathered children's h: for child p of slab row b,
 //   dpool[child[b*NB + p]][0:H) = dA[b, 0:K) * BT[0:K, p*H : (p+1)*H)
 // (grad of Gather is Scatter, folded into the product's epilogue).  Chain LSTM: NB = 1,
 // dA = da [n,4H], BT = W'^T [4H,H].  Tree-FC: NB = 2, dA = dz [n,H], BT = W^T [H,2H].
+//
+// FOLD 1 (chain LSTM) and 2 (Tree-FC): the launch goes on to the pointwise backward part of the
+// children.  `child` then names them by slab row over whole-batch slabs, and the thread that
+// holds d h of hidden unit j of a child writes the child's row of dA (and d c) directly; the
+// message gradient never passes through the pool.
 struct ChildBwdArgs {
   const float *dA;    // [n, K] (ld)
   long ld;
@@ -303,9 +376,14 @@ struct ChildBwdArgs {
   float *dpool;       // [*, mw]
   long mw;            // row width of the pool
   int n, H, K;
+  // FOLD only; whole-batch slabs, the round starts at slab row row0
+  float *dA_all, *dc_all;
+  const float *gates_all, *G_all, *h_all, *dret;
+  const int *dret_rows;
+  int row0, leaf_rows, act;
 };
 
-template <int TILE, int WAVES, int NB>
+template <int TILE, int WAVES, int NB, int FOLD>
 __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -327,6 +405,40 @@ __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwd
   for (int q = 0; q < EPT; q++)
 #pragma unroll
     for (int p = 0; p < NB; p++) ecp[q][p] = el.on[q] ? a.child[el.b[q] * NB + p] : -1;
+  // FOLD: what the children's pointwise part needs besides d h, fetched while the product runs
+  struct Kid {
+    float g[FOLD == 1 ? 5 : 1], dr, cp;
+  };
+  Kid kid[FOLD ? EPT : 1][NB];
+  float pdc[FOLD ? EPT : 1];
+  if constexpr (FOLD != 0) {
+#pragma unroll
+    for (int q = 0; q < EPT; q++) {
+      const int j = el.j[q];
+      pdc[q] = 0.f;
+      if constexpr (FOLD == 1) {
+        const long gb = a.row0 + el.b[q];
+        if (el.on[q]) pdc[q] = a.dc_all[gb * H + j] * a.gates_all[gb * 5 * H + H + j];  // d c handed on: d c * f
+      }
+#pragma unroll
+      for (int p = 0; p < NB; p++) {
+        const long v = ecp[q][p];
+        Kid &kd = kid[q][p];
+        kd.dr = kd.cp = 0.f;
+#pragma unroll
+        for (int t = 0; t < (FOLD == 1 ? 5 : 1); t++) kd.g[t] = 0.f;
+        if (v < 0) continue;
+        kd.dr = a.dret[(long)a.dret_rows[v] * H + j];
+        if constexpr (FOLD == 1) {
+#pragma unroll
+          for (int t = 0; t < 5; t++) kd.g[t] = a.gates_all[v * 5 * H + (long)t * H + j];
+          if (v >= a.leaf_rows) kd.cp = a.G_all[v * 2 * H + H + j];
+        } else {
+          kd.g[0] = a.h_all[v * H + j];
+        }
+      }
+    }
+  }
   Acc acc[NB];
   const float *bcol[NB];
 #pragma unroll
@@ -343,8 +455,22 @@ __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwd
     float v[NB];
     sum_regions<NB, NR, NREG>(v, red, el.lds[q], RSZ);
 #pragma unroll
-    for (int p = 0; p < NB; p++)
-      if (ecp[q][p] >= 0) a.dpool[ecp[q][p] * a.mw + el.j[q]] = v[p];
+    for (int p = 0; p < NB; p++) {
+      const long c = ecp[q][p];
+      if (c < 0) continue;
+      const int j = el.j[q];
+      if constexpr (FOLD == 1) {
+        const Kid &kd = kid[q][p];
+        const LstmGateGrad gg = lstm_gate_grad(kd.g[0], kd.g[1], kd.g[2], kd.g[3], kd.g[4], v[p], pdc[q], kd.dr, kd.cp);
+        float *d = a.dA_all + c * a.ld + j;
+        d[0] = gg.di; d[H] = gg.df; d[2 * H] = gg.du; d[3 * H] = gg.d_o;
+        if (c >= a.leaf_rows) a.dc_all[c * H + j] = gg.dc;
+      } else if constexpr (FOLD == 2) {
+        a.dA_all[c * a.ld + j] = treefc_dz(v[p] + kid[q][p].dr, kid[q][p].g[0], a.act);
+      } else {
+        a.dpool[c * a.mw + j] = v[p];
+      }
+    }
   }
 }
 
@@ -486,8 +612,7 @@ __global__ void treefc_round_bwd_kernel(TreeFcBwdArgs a) {
   if (src >= 0) ldw<W>(a.dpool + (long)src * H + j, dm);
 #pragma unroll
   for (int k = 0; k < W; k++) {
-    const float dh = (src >= 0 ? dm[k] : 0.f) + dr[k];
-    o[k] = a.act ? dh * (1.f - y[k] * y[k]) : (y[k] > 0.f ? dh : 0.f);
+    o[k] = treefc_dz((src >= 0 ? dm[k] : 0.f) + dr[k], y[k], a.act);
   }
   stw<W>(a.dz + (long)r * H + j, o);
 }
@@ -572,12 +697,64 @@ int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(dA && BT && child && dpool, "cavs_round_bwd_children: null pointer");
   CAVS_REQUIRE(aligned16(dA), "cavs_round_bwd_children: dA must be 16-byte aligned");
-  ChildBwdArgs a{dA, ld, BT, ldb, child, dpool, pool_width, n, H, K};
+  ChildBwdArgs a{dA, ld, BT, ldb, child, dpool, pool_width, n, H, K, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
   hipStream_t st = as_stream(stream);
   if (nchild == 1)
-    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 1>, round_bwd_children_kernel<16, 4, 1>, round_bwd_children_kernel<32, 8, 1>);
+    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 1, 0>, round_bwd_children_kernel<16, 4, 1, 0>, round_bwd_children_kernel<32, 8, 1, 0>);
   else
-    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 2>, round_bwd_children_kernel<16, 4, 2>, round_bwd_children_kernel<32, 8, 2>);
+    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 2, 0>, round_bwd_children_kernel<16, 4, 2, 0>, round_bwd_children_kernel<32, 8, 2, 0>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_lstm_round_bwd_children_gates(float *da, int ld_da, float *dc, const float *WhT, const int *child_rows,
+                                       const float *gates, const float *G, const float *dret, const int *dret_rows, int row0,
+                                       int n, int leaf_rows, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && row0 >= 0 && leaf_rows >= 0 && round_shape_ok(H) && ld_da >= 4 * H && ld_da % 4 == 0,
+               "cavs_lstm_round_bwd_children_gates: bad shape row0=%d n=%d leaf_rows=%d H=%d ld=%d (H must be a multiple of 32)", row0, n,
+               leaf_rows, H, ld_da);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(da && dc && WhT && child_rows && gates && G && dret && dret_rows, "cavs_lstm_round_bwd_children_gates: null pointer");
+  CAVS_REQUIRE(aligned16(da), "cavs_lstm_round_bwd_children_gates: da must be 16-byte aligned");
+  ChildBwdArgs a{da + (long)row0 * ld_da, ld_da, WhT, H, child_rows, nullptr, 0, n, H, 4 * H, da, dc, gates, G, nullptr, dret, dret_rows, row0, leaf_rows, 0};
+  launch_round(a, n, H, as_stream(stream), round_bwd_children_kernel<16, 8, 1, 1>, round_bwd_children_kernel<16, 4, 1, 1>,
+               round_bwd_children_kernel<32, 8, 1, 1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_lstm_bwd_gates_rows(const int *rows, int n, const float *dret, const int *dret_rows, const float *gates, const float *G,
+                             float *da, int ld_da, float *dc, int leaf_rows, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && leaf_rows >= 0 && ld_da >= 4 * H, "cavs_lstm_bwd_gates_rows: bad shape n=%d H=%d ld=%d", n, H, ld_da);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(rows && dret && dret_rows && gates && G && da && dc, "cavs_lstm_bwd_gates_rows: null pointer");
+  LstmBwdRowsArgs a{rows, dret, dret_rows, gates, G, da, ld_da, dc, n, H, leaf_rows};
+  launch_pointwise(a, n, H, H % 4 == 0, as_stream(stream), lstm_bwd_gates_rows_kernel<4>, lstm_bwd_gates_rows_kernel<1>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treefc_round_bwd_children_act(float *dz, const float *WT, const int *child_rows, const float *h, const float *dret,
+                                       const int *dret_rows, int row0, int n, int H, int act, void *stream) {
+  CAVS_REQUIRE(n >= 0 && row0 >= 0 && round_shape_ok(H) && (act == 0 || act == 1),
+               "cavs_treefc_round_bwd_children_act: bad argument row0=%d n=%d H=%d act=%d (H must be a multiple of 32)", row0, n, H, act);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dz && WT && child_rows && h && dret && dret_rows, "cavs_treefc_round_bwd_children_act: null pointer");
+  CAVS_REQUIRE(aligned16(dz), "cavs_treefc_round_bwd_children_act: dz must be 16-byte aligned");
+  ChildBwdArgs a{dz + (long)row0 * H, H, WT, 2L * H, child_rows, nullptr, 0, n, H, H, dz, nullptr, nullptr, nullptr, h, dret, dret_rows, row0, 0, act};
+  launch_round(a, n, H, as_stream(stream), round_bwd_children_kernel<16, 8, 2, 2>, round_bwd_children_kernel<16, 4, 2, 2>,
+               round_bwd_children_kernel<32, 8, 2, 2>);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treefc_bwd_rows(const int *rows, int n, const float *dret, const int *dret_rows, const float *h, float *dz, int H,
+                         int act, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && (act == 0 || act == 1), "cavs_treefc_bwd_rows: bad argument n=%d H=%d act=%d", n, H, act);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(rows && dret && dret_rows && h && dz, "cavs_treefc_bwd_rows: null pointer");
+  TreeFcBwdRowsArgs a{rows, dret, dret_rows, h, dz, n, H, act};
+  launch_pointwise(a, n, H, H % 4 == 0, as_stream(stream), treefc_bwd_rows_kernel<4>, treefc_bwd_rows_kernel<1>);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -89,6 +89,8 @@ _SIGS = {
     "cavs_treelstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_bwd_children_gates": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "cavs_treelstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
@@ -97,6 +99,10 @@ _SIGS = {
     "cavs_treefc_round_leaves_fwd": [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treefc_round_bwd": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_round_bwd_children": [_P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _P],
+    "cavs_lstm_round_bwd_children_gates": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "cavs_lstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
+    "cavs_treefc_round_bwd_children_act": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "cavs_treefc_bwd_rows": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
     "cavs_profile_arm": [_P, _P],
     "cavs_profile_disarm": [_P],
     "cavs_fc_softmax_xent": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _Z, _I, _I, _I, _P],

@@ -260,6 +260,7 @@ void Engine::reserve_edges() {
     R(xW_, cap * 4 * H);
     R(dxW_, cap * 4 * H);
     R(gates_, cap * 6 * H);
+    R(dc_, cap * H);
   } else {
     if (cfg_.use_x) R(xs_, cap * H);
     R(dxW_, cap * H);
@@ -295,7 +296,8 @@ void Engine::reserve_edges() {
 void Engine::upload_index_arena() {
   const Schedule &s = sched_;
   const int N = N_;
-  const size_t total = (size_t)N * (2 + nch_) + s.B;
+  const bool want_forest = !cfg_.split_backward_rounds && fused_rows() > 0;
+  const size_t total = (size_t)N * (2 + nch_) + s.B + (want_forest ? (size_t)N * (nch_ + 1) : 0);
   // two pinned staging buffers alternate, so the host can build the lists of the next
   // step while the device still runs this one; a buffer is rewritten only after the
   // upload that last read it has finished
@@ -340,6 +342,7 @@ void Engine::upload_index_arena() {
   int nr = 0;
   for (int v = 0; v < N; v++)
     if (s.parent[v] < 0) roots[nr++] = v;
+  forest_ = want_forest && build_forest_lists(roots + s.B, roots + s.B + (size_t)nch_ * N);
   check(cavs_memcpy_h2d(idx_dev_.get(), idx_host_[slot].get(), total * sizeof(int), stream_));
   check(cavs_event_record(idx_copied_[slot], stream_));
   idx_pending_[slot] = true;
@@ -347,6 +350,52 @@ void Engine::upload_index_arena() {
   d_pair_ = d_t2j_ + N;
   d_child_ = d_pair_ + N;
   d_roots_ = d_child_ + (size_t)nch_ * N;
+  d_kid_rows_ = d_roots_ + s.B;
+  d_orphans_ = d_kid_rows_ + (size_t)nch_ * N;
+}
+
+// The backward launch that folds the children's gate gradients in addresses a child by its slab
+// row, not by the pool row its message went through.  That is the same thing only while the
+// message flow is a forest: every pool row a Gather reads was written by exactly one slab row of
+// an earlier round and is read by exactly one (vertex, child slot).  Reads the host copies of
+// `pair` and `child` in the staging buffer that is about to be uploaded.
+bool Engine::build_forest_lists(int *kid_rows, int *orphans) {
+  const Schedule &s = sched_;
+  const int N = N_;
+  const int *pair = kid_rows - s.B - (size_t)nch_ * N - N, *child = pair + N;
+  n_orphans_ = 0;
+  if (!s.batching || s.rounds.empty() || !leaf_round(s.rounds[0]) || s.rounds[0].n != s.leaf_prefix) return false;
+  inv_pair_.assign(N, -1);
+  round_of_row_.resize(N);
+  const int fused = fused_rows();
+  for (size_t k = 0; k < s.rounds.size(); k++) {
+    const Round &r = s.rounds[k];
+    if (k > 0 && (leaf_round(r) || r.n > fused)) return false;  // every round with children runs as a fused launch
+    for (int b = 0; b < r.n; b++) round_of_row_[r.offset + b] = (int)k;
+  }
+  for (int v = 0; v < N; v++) {
+    const int p = pair[v];
+    if (p < 0) continue;
+    if (p >= N || inv_pair_[p] >= 0) return false;  // two writers of one pool row
+    inv_pair_[p] = v;
+  }
+  std::vector<char> read(N, 0);
+  for (size_t i = 0; i < (size_t)nch_ * N; i++) {
+    kid_rows[i] = -1;
+    const int p = child[i];
+    if (p < 0) continue;
+    const int b = (int)(i / nch_);
+    if (p >= N || inv_pair_[p] < 0 || read[p]) return false;  // reads a row nobody wrote, or a second reader
+    const int v = inv_pair_[p];
+    if (round_of_row_[v] >= round_of_row_[b]) return false;
+    read[p] = 1;
+    kid_rows[i] = v;
+  }
+  for (int v = 0; v < N; v++) {
+    if (pair[v] >= 0 && !read[pair[v]]) return false;  // a message nobody reads: its gradient is whatever the pool holds
+    if (pair[v] < 0) orphans[n_orphans_++] = v;
+  }
+  return true;
 }
 
 // ------------------------------------------------------------------ step
@@ -567,7 +616,7 @@ void Engine::treelstm_backward() {
   const int fused = fused_rows();
   // grad of Push is Pull: read through the list by the fused gate kernels, or gathered up front
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
-  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr},
@@ -577,9 +626,28 @@ void Engine::treelstm_backward() {
   } else {
     backward_prologue({}, true);
   }
+  // one launch per round when the message flow is a forest: the roots' gate gradients first, then
+  // every round hands d h, d c on to its children and does their gate gradients in its epilogue
+  const bool folded = forest_;
+  if (folded) {
+    CAVS_TIMED(K_GATES, cavs_treelstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
+                                                     dF_.get(), dc_.get(), sched_.leaf_prefix, H, stream_));
+    c_launches_ += 1;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
+    if (folded) {
+      c_gather_rows_ += r.n;
+      if (leaf_round(r)) continue;
+      CAVS_TIMED(K_ROUND, cavs_treelstm_round_bwd_children_gates(dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_ + 2 * off,
+                                                                 gates_.get(), G_.get(), d_dgo_, d_t2j_, (int)off, r.n,
+                                                                 sched_.leaf_prefix, H, stream_));
+      c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
+      c_scatter_rows_ += 2.0 * r.n;
+      c_launches_ += 1;
+      continue;
+    }
     if (r.n <= fused) {
       // Gather of the message gradient, gate gradients and the Scatter of d c_child in one
       // launch; the children's d h (both products and their Scatter) in a second
@@ -760,16 +828,32 @@ void Engine::lstm_backward() {
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H;
   const int fused = fused_rows();
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
-  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr, nullptr}}, true);
   } else {
     backward_prologue({}, true);
   }
+  const bool folded = forest_;  // one launch per round, as in treelstm_backward
+  if (folded) {
+    CAVS_TIMED(K_GATES, cavs_lstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
+                                                 dc_.get(), sched_.leaf_prefix, H, stream_));
+    c_launches_ += 1;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
     float *da = dxW_.at(off * 4 * H);
+    if (folded) {
+      c_gather_rows_ += r.n;
+      if (leaf_round(r)) continue;
+      CAVS_TIMED(K_ROUND, cavs_lstm_round_bwd_children_gates(dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(),
+                                                             G_.get(), d_dgo_, d_t2j_, (int)off, r.n, sched_.leaf_prefix, H, stream_));
+      c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
+      c_scatter_rows_ += r.n;
+      c_launches_ += 1;
+      continue;
+    }
     if (r.n <= fused) {
       const bool leaf = leaf_round(r);
       const int *child = leaf ? nullptr : d_child_ + off;
@@ -865,16 +949,31 @@ void Engine::treefc_backward() {
   const float *W = param("W").w;
   const int fused = fused_rows();
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
-  if (!dret_folded) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W^T [H, 2H]: the B operand of d[h_l;h_r] = dz * W^T, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, 2 * H, H, 0, UT_.get(), const_cast<float *>(W), nullptr, nullptr}}, false);
   } else {
     backward_prologue({}, false);
   }
+  const bool folded = forest_;  // one launch per round, as in treelstm_backward
+  if (folded) {
+    CAVS_TIMED(K_GATES, cavs_treefc_bwd_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, msg_.get(), dxW_.get(), H, cfg_.act, stream_));
+    c_launches_ += 1;
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
     const size_t off = r.offset;
     float *dz = dxW_.at(off * H);
+    if (folded) {
+      c_gather_rows_ += r.n;
+      if (leaf_round(r)) continue;
+      CAVS_TIMED(K_ROUND, cavs_treefc_round_bwd_children_act(dxW_.get(), UT_.get(), d_kid_rows_ + 2 * off, msg_.get(), d_dgo_, d_t2j_,
+                                                             (int)off, r.n, H, cfg_.act, stream_));
+      c_round_flops_ += 2.0 * r.n * H * 2.0 * H;
+      c_scatter_rows_ += 2.0 * r.n;
+      c_launches_ += 1;
+      continue;
+    }
     if (r.n <= fused) {
       CAVS_TIMED(K_GATES, cavs_treefc_round_bwd(dpool_.get(), d_pair_ + off, dret_folded ? d_dgo_ : dret_.at(off * H),
                                                 dret_folded ? d_t2j_ + off : nullptr, msg_.at(off * H), dz, r.n, H, cfg_.act, stream_));

@@ -120,13 +120,20 @@ class Engine {
   bool out_folded_ = false;    // the rounds wrote it themselves
   int N_ = 0, cap_ = 0, rcap_ = 0, E_ = 0, mw_ = 0, nch_ = 1;
 
-  // per-step device index arena: [t2j | pair | child | roots]
+  // per-step device index arena: [t2j | pair | child | roots | kid_rows | orphans]
   PinnedArray<int> idx_host_[2];
   void *idx_copied_[2] = {nullptr, nullptr};  // events: upload out of idx_host_[k] finished
   bool idx_pending_[2] = {false, false};
   int idx_slot_ = 0;
   DeviceArray<int> idx_dev_;
   const int *d_t2j_ = nullptr, *d_pair_ = nullptr, *d_child_ = nullptr, *d_roots_ = nullptr;
+  // Tree-LSTM, message flow of the batch is a forest: children by slab row, and the slab rows
+  // nobody sends a message to
+  const int *d_kid_rows_ = nullptr, *d_orphans_ = nullptr;
+  int n_orphans_ = 0;
+  bool forest_ = false;
+  std::vector<int> inv_pair_, round_of_row_;
+  bool build_forest_lists(int *kid_rows, int *orphans);
 
   // feeds
   DeviceArray<float> x_in_, labels_in_;
@@ -136,6 +143,7 @@ class Engine {
   DeviceArray<float> xs_, e_, xW_, G_, hlr_, gates_, msg_, pool_, GO_, dGO_, dret_, dpool_, dxW_,
       dF_, de_, logits_, dlogits_, loss_, ws_;
   DeviceArray<float> r_hU_, r_hUf_, r_dmsg_, r_dG_, r_dhlr_, r_z_;  // round-local
+  DeviceArray<float> dc_;  // [N, H] d c of every vertex (folded backward rounds)
   // Embedding gradient: only the rows looked up in a step are non-zero, so the table is
   // cleared and updated by those rows.  xs_prev_ lists the rows the last backward pass wrote.
   DeviceArray<float> xs_prev_;

@@ -314,6 +314,23 @@ int cavs_treelstm_round_bwd_gates(float *dpool, const int *pair, const int *chil
  * child[2b], child[2b+1].  UT = U_iou^T [3H,H] then U_f^T [H,H] (cavs_transpose). */
 int cavs_treelstm_round_bwd_children(const float *dxW, int ld_dxw, const float *dF, const float *UT,
                                      const int *child, float *dpool, int n, int H, void *stream);
+/* Both parts of the backward round in one launch, for a batch whose message flow is a forest
+ * (every message has exactly one reader): the launch that computes d h of the children of a
+ * round (rows [row0, row0 + n) of the whole-batch slabs) goes on to the children's gate
+ * gradients and writes the children's rows of dxW / dF and d c of each child to row v of
+ * dc [N,H]; the message gradient does not pass through the pool (Scatter_grad followed by the
+ * next round's Gather_grad, cavs/backend/op_impl_graphop.cu:137-166 and 45-100, composed).
+ * child_rows [2n]: the children of round row b by SLAB row (-1: none); rows below leaf_rows are
+ * leaves; dret_rows [N]: the gradient of the return value of slab row v is dret row
+ * dret_rows[v].  The rows nobody sends a message to (the roots) get their gate gradients from
+ * cavs_treelstm_bwd_gates_rows (message gradient zero) before the first such launch. */
+int cavs_treelstm_round_bwd_children_gates(float *dxW, int ld_dxw, float *dF, float *dc, const float *UT,
+                                           const int *child_rows, const float *gates, const float *G,
+                                           const float *dret, const int *dret_rows, int row0, int n,
+                                           int leaf_rows, int H, void *stream);
+int cavs_treelstm_bwd_gates_rows(const int *rows, int n, const float *dret, const int *dret_rows,
+                                 const float *gates, const float *G, float *dxW, int ld_dxw, float *dF,
+                                 float *dc, int leaf_rows, int H, void *stream);
 /* The same construction for the chain LSTM (apps/paper/seq-lstm-cavs.cc:62-86; one child per
  * vertex: child [n]; Wh [H,4H] blocks [i|f|u|o]; gates [n,5H] = [i|f|u|o|tanh c]; G [n,2H] the
  * gathered predecessor) and for Tree-FC (apps/paper/tree-fc-cavs.cc:28-36; messages are h only:
@@ -341,6 +358,23 @@ int cavs_treefc_round_bwd(const float *dpool, const int *pair, const float *dret
  * nchild 1, dA = da [n,4H], BT = Wh^T [4H,H].  Tree-FC: nchild 2, dA = dz [n,H], BT = W^T [H,2H]. */
 int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int ldb, int nchild,
                             const int *child, float *dpool, int pool_width, int n, int H, void *stream);
+/* The chain LSTM's and Tree-FC's backward round as one launch, as
+ * cavs_treelstm_round_bwd_children_gates does it for the Tree-LSTM: whole-batch slabs, the
+ * round is rows [row0, row0 + n), child_rows names the children by slab row, and the launch
+ * writes the children's rows of da (and d c of each to dc [N,H]) resp. dz.  The rows nobody sends
+ * a message to (the last step of every sequence / the roots) come from the *_rows launches. */
+int cavs_lstm_round_bwd_children_gates(float *da, int ld_da, float *dc, const float *WhT,
+                                       const int *child_rows, const float *gates, const float *G,
+                                       const float *dret, const int *dret_rows, int row0, int n,
+                                       int leaf_rows, int H, void *stream);
+int cavs_lstm_bwd_gates_rows(const int *rows, int n, const float *dret, const int *dret_rows,
+                             const float *gates, const float *G, float *da, int ld_da, float *dc,
+                             int leaf_rows, int H, void *stream);
+int cavs_treefc_round_bwd_children_act(float *dz, const float *WT, const int *child_rows, const float *h,
+                                       const float *dret, const int *dret_rows, int row0, int n, int H,
+                                       int act, void *stream);
+int cavs_treefc_bwd_rows(const int *rows, int n, const float *dret, const int *dret_rows, const float *h,
+                         float *dz, int H, int act, void *stream);
 /* out [cols,rows] = in [rows,cols]^T */
 int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream);
 /* Several small jobs that do not depend on each other, in one launch (no counterpart in the

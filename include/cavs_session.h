@@ -48,6 +48,10 @@ typedef struct {
    * two backward (cavs_treelstm_round_*); larger rounds run gather / GEMM / gates / scatter
    * as separate launches.  0 = default limit, negative = never fuse. */
   int fused_round_rows;
+  /* All rounds fused: 0 = when the batch's message flow is a forest, the launch that computes
+   * d h of a round's children also does their gate gradients (one launch per backward round,
+   * cavs_*_round_bwd_children_gates / _act); 1 = always two launches per round. */
+  int split_backward_rounds;
 } cavs_session_config;
 
 const char *cavs_session_error(void);

@@ -243,6 +243,35 @@ def test_fused_rounds_match_oracle(oracle, model, kw, H, limit, pairing):
     assert (fused_flops > 0) == (limit >= 0), fused_flops
 
 
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+@pytest.mark.parametrize("model,kw", CASES)
+def test_backward_rounds_as_one_launch_or_two(oracle, model, kw, pairing):
+    """A backward round either as two launches (gate gradients, then the children's d h through
+    the pool) or as one that goes on to the children's gate gradients: both against the oracle,
+    and the launch count shows that each really ran."""
+    H = 64
+    E = H if model == "lstm" else 12
+    loss = "softmax" if model != "treefc" else "root_sq"
+    w = small_workload(model, 57, B=40, H=H, E=12, V=31, C=5)
+    want = oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=H, E=E, V=31, Cc=5, pairing=pairing, loss=loss, **kw)
+    names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
+             "treefc": ("W", "Bv") if kw.get("use_bias") else ("W",)}[model]
+    if loss == "softmax":
+        names += ("Wfc", "bfc")
+    launches = []
+    for split in (False, True):
+        print(f"[case] {model} {kw} backward rounds split={split} pairing={pairing} N={w['N']}", flush=True)
+        s = session.Session(model, H=H, E=E, V=31, C_=5, pairing=pairing, split_backward_rounds=split, loss=loss, **kw)
+        s.set_params({k: w["params"][k] for k in names})
+        s.step(w["graph"], w["x"], w["labels"], backward=True)
+        got = dict(loss=s.fetch("loss"), graph_out=s.fetch("graph_out"), dgraph_out=s.fetch("dgraph_out"),
+                   msg_pool=s.fetch("msg_pool"), grads=s.grads(), trace=s.schedule_trace())
+        launches.append(s.counter("launches"))
+        s.close()
+        compare(got, want)
+    assert launches[0] < launches[1], launches
+
+
 @pytest.mark.parametrize("model", ["treelstm", "lstm"])
 def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     """Four SGD steps over three different batches (token ids overlap between steps, one

@@ -660,6 +660,77 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     close(g.host(go2), go_l, "leaf graph_out")
 
 
+@pytest.mark.parametrize("L,m,n,H", [(20, 5, 3, 32), (300, 70, 40, 64), (900, 200, 130, 64), (2600, 100, 1100, 32), (1300, 500, 300, 512)])
+def test_backward_rounds_with_the_childrens_gate_gradients_folded_in(g, oracle, L, m, n, H):
+    """Three levels over whole-batch slabs (leaves, a middle round, a top round of roots): the
+    roots' gate gradients from the row-list launch, then one launch per round that hands d h,
+    d c on to the children and does their gate gradients, against the same chain composed
+    round by round from the oracle's gate-gradient and GEMM functions."""
+    r = rng(11 * L + 3 * n + H)
+    N = L + m + n
+    mid0, top0 = L, L + m
+    order = np.argsort(r.bulk_normal(L)).astype(np.int32)
+    kids = np.full(2 * N, -1, np.int32)
+    kids[2 * mid0: 2 * top0] = order[: 2 * m]                      # the middle round's children are leaves
+    assert m <= 2 * n - 1 and 2 * m + 2 * n - m <= L
+    top_kids = np.concatenate([np.arange(mid0, top0, dtype=np.int32), order[2 * m: 2 * m + 2 * n - m]])
+    top_kids = top_kids[np.argsort(r.bulk_normal(2 * n))]          # the top round's: every middle row, and leaves
+    top_kids[np.flatnonzero(top_kids < L)[0]] = -1                 # a missing child
+    kids[2 * top0:] = top_kids
+    sig = lambda a: (1.0 / (1.0 + np.exp(-a))).astype(np.float32)
+    gates = r.bulk_normal(N * 6 * H).reshape(N, 6 * H)
+    gates[:, : 2 * H] = sig(gates[:, : 2 * H])
+    gates[:, 2 * H: 3 * H] = np.tanh(gates[:, 2 * H: 3 * H])
+    gates[:, 3 * H: 5 * H] = sig(gates[:, 3 * H: 5 * H])
+    gates[:, 5 * H:] = np.tanh(gates[:, 5 * H:])
+    G = (r.bulk_normal(2 * N * 2 * H).reshape(2 * N, 2 * H) * 0.5).astype(np.float32)
+    G[: 2 * L] = 0                                                 # leaves gathered nothing
+    U = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)
+    Uiou, Uf = U[: 3 * H * H].reshape(H, 3 * H), U[3 * H * H:].reshape(H, H)
+    dret_rows = np.argsort(r.bulk_normal(N + 3))[:N].astype(np.int32)
+    dgo = r.bulk_normal((N + 3) * H).reshape(N + 3, H)
+
+    # expected, top-down
+    dmsg = np.zeros((N, 2 * H), np.float32)
+    reached = np.zeros(N, bool)
+    reached[top0:] = True
+    dxW_w, dF_w = np.zeros((N, 4 * H), np.float32), np.zeros((2 * N, H), np.float32)
+    for lo, hi in ((top0, N), (mid0, top0), (0, L)):
+        a, b, c = oracle.treelstm_gates_bwd(dmsg[lo:hi], dgo[dret_rows[lo:hi]], gates[lo:hi], G[2 * lo: 2 * hi])
+        dxW_w[lo:hi], dF_w[2 * lo: 2 * hi] = a, b
+        if lo == 0:
+            break
+        dhlr = oracle.sgemm(0, 1, np.ascontiguousarray(a[:, : 3 * H]), np.ascontiguousarray(Uiou))
+        c[:, :H] = oracle.sgemm(0, 1, b, np.ascontiguousarray(Uf)) + np.repeat(dhlr, 2, axis=0)
+        k = kids[2 * lo: 2 * hi]
+        dmsg[k[k >= 0]] = c[k >= 0]
+        reached[k[k >= 0]] = True
+
+    UT = g.zeros(4 * H * H)
+    d_U = g.devf(U)
+    g.call("cavs_transpose", g.P(UT), g.P(d_U), H, 3 * H, g.stream())
+    g.call("cavs_transpose", g.P(UT) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, H, H, g.stream())
+    dxW, dF, dc = g.zeros(N, 4 * H, fill=-3.0), g.zeros(2 * N, H, fill=-3.0), g.zeros(N, H, fill=-3.0)
+    d_gates, d_G, d_dgo, d_rows, d_kids = g.devf(gates), g.devf(G), g.devf(dgo), g.devi(dret_rows), g.devi(kids)
+    roots = np.arange(top0, N, dtype=np.int32)
+    g.call("cavs_treelstm_bwd_gates_rows", g.P(g.devi(roots)), n, g.P(d_dgo), g.P(d_rows), g.P(d_gates), g.P(d_G), g.P(dxW), 4 * H,
+           g.P(dF), g.P(dc), L, H, g.stream())
+    close(g.host(dxW)[top0:], dxW_w[top0:], "roots dxW")
+    close(g.host(dF)[2 * top0:], dF_w[2 * top0:], "roots dF")
+    assert (g.host(dxW)[:top0] == -3.0).all() and (g.host(dc)[:top0] == -3.0).all()
+    for lo, cnt in ((top0, n), (mid0, m)):
+        g.call("cavs_treelstm_round_bwd_children_gates", g.P(dxW), 4 * H, g.P(dF), g.P(dc), g.P(UT), g.P(d_kids) + 4 * 2 * lo,
+               g.P(d_gates), g.P(d_G), g.P(d_dgo), g.P(d_rows), lo, cnt, L, H, g.stream())
+    got_x, got_F = g.host(dxW), g.host(dF)
+    close(got_x[reached], dxW_w[reached], "dxW", rtol=2e-4, atol=2e-5)
+    internal = reached.copy()
+    internal[:L] = False
+    close(got_F[np.repeat(internal, 2)], dF_w[np.repeat(internal, 2)], "dF", rtol=2e-4, atol=2e-5)
+    # rows no message reaches are left alone, and so are the leaves' rows of dF and dc
+    assert (got_x[~reached] == -3.0).all()
+    assert (got_F[: 2 * L] == -3.0).all() and (g.host(dc)[:L] == -3.0).all()
+
+
 def test_fused_round_entry_points_reject_bad_shapes():
     with pytest.raises(hip.CavsError, match="multiple of 32"):
         hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 0, 0, 5, 24, 0)
@@ -667,6 +738,10 @@ def test_fused_round_entry_points_reject_bad_shapes():
         hip.call("cavs_treelstm_round_bwd_children", 0, 4 * 24, 0, 0, 0, 0, 5, 24, 0)
     with pytest.raises(hip.CavsError, match="all set"):
         hip.call("cavs_treelstm_round_bwd_gates", 16, 16, 16, 16, 0, 16, 0, 16, 4 * 32, 0, 5, 32, 0)
+    with pytest.raises(hip.CavsError, match="multiple of 32"):
+        hip.call("cavs_treelstm_round_bwd_children_gates", 16, 4 * 24, 16, 16, 16, 16, 16, 16, 16, 16, 0, 5, 0, 24, 0)
+    with pytest.raises(hip.CavsError, match="null pointer"):
+        hip.call("cavs_treelstm_bwd_gates_rows", 0, 5, 16, 16, 16, 16, 16, 4 * 32, 16, 16, 0, 32, 0)
 
 
 @pytest.mark.parametrize("n,H,C_", [(1, 64, 2), (19, 96, 5), (2482, 512, 5), (300, 100, 8), (77, 1024, 3)])
@@ -856,6 +931,91 @@ def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
     g.call("cavs_round_bwd_children", g.P(g.devf(dA)), K + 4, K, g.P(g.devf(BT)), nchild * H, nchild, g.P(g.devi(child)),
            g.P(d), mw, n, H, g.stream())
     close(g.host(d), want, "dpool", rtol=2e-4, atol=2e-5)
+
+
+@pytest.mark.parametrize("model,L,m,n,H", [("lstm", 20, 2, 3, 32), ("lstm", 300, 60, 70, 64), ("lstm", 2600, 600, 1100, 32),
+                                           ("treefc", 20, 5, 3, 32), ("treefc", 400, 100, 70, 64), ("treefc", 2600, 100, 1100, 32),
+                                           ("treefc", 900, 200, 130, 96)])
+def test_chain_and_tree_fc_backward_rounds_with_the_childrens_pointwise_part_folded_in(g, oracle, model, L, m, n, H):
+    """The construction of the Tree-LSTM test above for the other two vertex functions: three
+    levels over whole-batch slabs, the top rows from the row-list launch, then one launch per
+    round, against the chain composed round by round from the oracle's functions."""
+    r = rng(13 * L + 5 * n + H + len(model))
+    nch = 1 if model == "lstm" else 2
+    N = L + m + n
+    mid0, top0 = L, L + m
+    order = np.argsort(r.bulk_normal(L)).astype(np.int32)
+    kids = np.full(nch * N, -1, np.int32)
+    kids[nch * mid0: nch * top0] = order[: nch * m]
+    assert m <= nch * n - 1 and nch * m + nch * n - m <= L
+    top_kids = np.concatenate([np.arange(mid0, top0, dtype=np.int32), order[nch * m: nch * m + nch * n - m]])
+    top_kids = top_kids[np.argsort(r.bulk_normal(nch * n))]
+    top_kids[np.flatnonzero(top_kids < L)[0]] = -1
+    kids[nch * top0:] = top_kids
+    dret_rows = np.argsort(r.bulk_normal(N + 3))[:N].astype(np.int32)
+    dgo = r.bulk_normal((N + 3) * H).reshape(N + 3, H)
+    act = 1 if L in (400, 900) else 0
+    if model == "lstm":
+        sig = lambda a: (1.0 / (1.0 + np.exp(-a))).astype(np.float32)
+        gates = r.bulk_normal(N * 5 * H).reshape(N, 5 * H)
+        gates[:, : 2 * H] = sig(gates[:, : 2 * H])
+        gates[:, 2 * H: 3 * H] = np.tanh(gates[:, 2 * H: 3 * H])
+        gates[:, 3 * H: 4 * H] = sig(gates[:, 3 * H: 4 * H])
+        gates[:, 4 * H:] = np.tanh(gates[:, 4 * H:])
+        G = (r.bulk_normal(N * 2 * H).reshape(N, 2 * H) * 0.5).astype(np.float32)
+        G[:L] = 0
+        W = (r.bulk_normal(H * 4 * H).reshape(H, 4 * H) / np.sqrt(H)).astype(np.float32)   # W' [H,4H]
+        K, wd = 4 * H, 2 * H
+    else:
+        h = np.tanh(r.bulk_normal(N * H).reshape(N, H)).astype(np.float32)                 # relu: sign of h decides
+        W = (r.bulk_normal(2 * H * H).reshape(2 * H, H) / np.sqrt(H)).astype(np.float32)   # W [2H,H]
+        K, wd = H, H
+    WT = np.ascontiguousarray(W.T)                                                         # [K, nch*H]
+
+    dmsg = np.zeros((N, wd), np.float32)
+    reached = np.zeros(N, bool)
+    reached[top0:] = True
+    dA_w = np.zeros((N, K), np.float32)
+    for lo, hi in ((top0, N), (mid0, top0), (0, L)):
+        if model == "lstm":
+            a, c = oracle.lstm_gates_bwd(dmsg[lo:hi], dgo[dret_rows[lo:hi]], gates[lo:hi], G[lo:hi])
+        else:
+            a = oracle.treefc_bwd(dmsg[lo:hi], dgo[dret_rows[lo:hi]], h[lo:hi], act)
+        dA_w[lo:hi] = a
+        if lo == 0:
+            break
+        dh = oracle.sgemm(0, 0, a, WT)                       # [rows, nch*H]
+        k = kids[nch * lo: nch * hi]
+        if model == "lstm":
+            c[:, :H] = dh
+            dmsg[k[k >= 0]] = c[k >= 0]
+        else:
+            dmsg[k[k >= 0]] = dh.reshape(-1, H)[k >= 0]
+        reached[k[k >= 0]] = True
+
+    dA, dc = g.zeros(N, K, fill=-3.0), g.zeros(N, H, fill=-3.0)
+    d_dgo, d_rows, d_kids, d_WT = g.devf(dgo), g.devi(dret_rows), g.devi(kids), g.devf(WT)
+    roots = g.devi(np.arange(top0, N, dtype=np.int32))
+    if model == "lstm":
+        d_gates, d_G = g.devf(gates), g.devf(G)
+        g.call("cavs_lstm_bwd_gates_rows", g.P(roots), n, g.P(d_dgo), g.P(d_rows), g.P(d_gates), g.P(d_G), g.P(dA), K, g.P(dc), L, H,
+               g.stream())
+    else:
+        d_h = g.devf(h)
+        g.call("cavs_treefc_bwd_rows", g.P(roots), n, g.P(d_dgo), g.P(d_rows), g.P(d_h), g.P(dA), H, act, g.stream())
+    close(g.host(dA)[top0:], dA_w[top0:], "top rows")
+    assert (g.host(dA)[:top0] == -3.0).all()
+    for lo, cnt in ((top0, n), (mid0, m)):
+        if model == "lstm":
+            g.call("cavs_lstm_round_bwd_children_gates", g.P(dA), K, g.P(dc), g.P(d_WT), g.P(d_kids) + 4 * lo, g.P(d_gates), g.P(d_G),
+                   g.P(d_dgo), g.P(d_rows), lo, cnt, L, H, g.stream())
+        else:
+            g.call("cavs_treefc_round_bwd_children_act", g.P(dA), g.P(d_WT), g.P(d_kids) + 4 * 2 * lo, g.P(d_h), g.P(d_dgo), g.P(d_rows),
+                   lo, cnt, H, act, g.stream())
+    got = g.host(dA)
+    close(got[reached], dA_w[reached], "dA", rtol=2e-4, atol=2e-5)
+    assert (got[~reached] == -3.0).all()
+    assert (g.host(dc)[:L] == -3.0).all()
 
 
 def test_gradient_clipping_by_the_sum_of_norms(g):
