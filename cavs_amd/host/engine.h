@@ -34,6 +34,11 @@ class Engine {
   // end's Variable tensors) instead of the engine's own copies.  g may be null: then the
   // engine keeps the gradient in its own buffer (read it with grad_ptr()).
   void bind_param(const std::string &name, float *w, float *g);
+  // where the next backward pass leaves the gradient of `name` (null: the engine's own buffer)
+  void bind_param_grad(const std::string &name, float *g) {
+    Param &p = param(name);
+    p.g = g ? g : p.own_g.get();
+  }
   const float *grad_ptr(const std::string &name) { return param(name).g; }
   float *graph_out_ptr() const { return GO_.get(); }
   // The two halves of step() for a caller that runs the loss head itself: forward F into

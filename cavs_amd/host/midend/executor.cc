@@ -730,13 +730,27 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       mp.fwd.swap(fwd);
       mp.bwd.swap(bwd);
     }
+    if (train && lowered_) {
+      plan_gradient_binds(&mp);
+      plan_fused_head(&mp);
+    }
     it = main_cache_.emplace(key, std::move(mp)).first;
   }
-  for (const OpDef &d : it->second.fwd) {
+  binds_ = &it->second.binds;
+  const HeadFuse &head = it->second.head;
+  bool head_fused = false;
+  for (size_t i = 0; i < it->second.fwd.size(); i++) {
+    const OpDef &d = it->second.fwd[i];
+    if ((int)i == head.fc) head_fused = run_fused_head(it->second);
+    if (head_fused && ((int)i == head.fc || (int)i == head.loss)) continue;
     if (d.name() == "GraphOutput") run_graph_output(d); else exec(d, mainctx);
   }
   if (train) {
-    for (const OpDef &d : it->second.bwd) {
+    const std::vector<char> &skip = it->second.skip_bwd;
+    for (size_t i = 0; i < it->second.bwd.size(); i++) {
+      const OpDef &d = it->second.bwd[i];
+      if (i < skip.size() && skip[i]) continue;
+      if (head_fused && ((int)i == head.loss_grad || (int)i == head.fc_grad || (int)i == head.seed)) continue;
       if (d.name() == "GraphOutput_grad") run_graph_output_grad(d); else exec(d, mainctx);
     }
     // SGD: w -= lr * g (cavs/backend/op_impl_sgd.cu); clipping is not on the measured path

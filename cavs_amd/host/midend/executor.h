@@ -109,7 +109,33 @@ class Executor {
   // programs of the vertex function as executed (after the fusion pass when OPT_FUSION is set)
   std::vector<OpDef> func_fwd_, func_bwd_, func_def_;
   std::vector<OpDef> main_all_;
-  struct MainProgram { std::vector<OpDef> fwd, bwd; };
+  // The lowered F writes a parameter's gradient where the main scope wants it: when the gradients
+  // of all the slices of a Variable come out of the lowered F and only get added into the
+  // Variable's zero-filled gradient, the engine's gradient array is bound to that place and the
+  // Fill and PartialAccumulate operators are skipped.
+  struct GradBind {
+    std::string param, dst;  // engine parameter; main-scope gradient tensor
+    long offset;             // the parameter's gradient starts at tensor(dst).base + offset
+  };
+  // A classifier head FullyConnected -> SoftmaxEntropyLoss whose gradients the program also
+  // wants runs as one call (cavs_fc_softmax_xent) at the FullyConnected operator, on the lowered
+  // path, whenever the batch's shape fits that entry point; the three other operators are skipped.
+  struct HeadFuse {
+    int fc = -1, loss = -1;           // indices into fwd
+    int loss_grad = -1, fc_grad = -1; // indices into bwd
+    int seed = -1;                    // the ConstOp that seeds d loss, if nobody else reads it
+  };
+  struct MainProgram {
+    std::vector<OpDef> fwd, bwd;
+    std::vector<char> skip_bwd;
+    std::vector<GradBind> binds;
+    HeadFuse head;
+  };
+  void plan_fused_head(MainProgram *mp) const;
+  bool run_fused_head(const MainProgram &mp);
+  float *output_storage(const std::string &name, long *count);
+  void plan_gradient_binds(MainProgram *mp) const;
+  const std::vector<GradBind> *binds_ = nullptr;  // of the program being run
   std::map<std::string, MainProgram> main_cache_;  // keyed by the requested targets
   std::map<std::string, void *> fused_handles_;    // kernel name -> compiled module
   int fused_groups_ = 0;

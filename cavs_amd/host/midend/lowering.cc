@@ -1,5 +1,7 @@
 #include "lowering.h"
 
+#include <algorithm>
+
 #include <functional>
 #include <sstream>
 
@@ -382,8 +384,242 @@ void Executor::lowered_forward(const int32_t *graph, int B, int maxlen, float *)
   go.rows = N_;
 }
 
+// See GradBind.  A PartialAccumulate qualifies when what it adds is an output of the lowered F
+// that is written, not accumulated (possibly through ReshapeLike views); a Variable qualifies
+// when its gradient is written by one zero Fill and qualifying PartialAccumulates only, whose
+// blocks tile it and line up with the engine's layout of whole parameters.
+void Executor::plan_gradient_binds(MainProgram *mp) const {
+  const Lowering &lw = *lowering_;
+  const std::vector<OpDef> &ops = mp->bwd;
+  mp->skip_bwd.assign(ops.size(), 0);
+  mp->binds.clear();
+  int gi = -1;
+  for (size_t i = 0; i < ops.size(); i++)
+    if (ops[i].name() == "GraphOutput_grad") gi = (int)i;
+  if (gi < 0) return;
+  const OpDef &go = ops[gi];
+  auto slots = role_slots(lw);
+  std::map<std::string, std::string> role_of_edge;
+  for (auto &kv : lw.roles) role_of_edge[kv.second] = kv.first;
+  std::map<std::string, std::string> role_of_grad;  // written (not accumulated) outputs of the lowered F
+  auto *accs = go.find_attr("Acc");
+  for (int i = 0; i < go.output_size(); i++) {
+    const bool acc = accs && i < (int)accs->value_.list_i.size() && accs->value_.list_i[i] != 0;
+    auto rit = role_of_edge.find(GetOriginName(go.output(i)));
+    if (!acc && rit != role_of_edge.end()) role_of_grad[go.output(i)] = rit->second;
+  }
+  std::map<std::string, int> producer;
+  std::map<std::string, std::vector<int>> writers;
+  for (size_t i = 0; i < ops.size(); i++)
+    for (int k = 0; k < ops[i].output_size(); k++) {
+      producer[ops[i].output(k)] = (int)i;
+      writers[ops[i].output(k)].push_back((int)i);
+    }
+  struct Block {
+    int op;
+    std::string role;
+    long offset, stride;
+    std::vector<int> views;  // the ReshapeLike operators between the lowered F's output and the block
+  };
+  std::map<std::string, std::vector<Block>> blocks;  // by destination
+  std::map<std::string, bool> bad;
+  for (size_t i = gi + 1; i < ops.size(); i++) {
+    const OpDef &d = ops[i];
+    if (d.name() != "PartialAccumulate") continue;
+    const std::string &dst = d.output(0);
+    const Edge *we = edge(dst);
+    if (!we || we->per_vertex()) { bad[dst] = true; continue; }
+    long stride, offset;
+    if (d.find_attr("Split")) {
+      stride = we->width() / GetSingleArg<int>(d, "Split");
+      offset = stride * GetSingleArg<int>(d, "Index");
+    } else {
+      offset = GetSingleArg<int>(d, "Offset");
+      stride = GetSingleArg<int>(d, "Stride");
+    }
+    std::string src = d.input(0);
+    std::vector<int> views;
+    for (int hops = 0; hops < 8 && !role_of_grad.count(src); hops++) {
+      auto pit = producer.find(src);
+      if (pit == producer.end() || pit->second <= gi || ops[pit->second].name() != "ReshapeLike") break;
+      views.push_back(pit->second);
+      src = ops[pit->second].input(0);
+    }
+    auto rit = role_of_grad.find(src);
+    if (rit == role_of_grad.end()) { bad[dst] = true; continue; }
+    blocks[dst].push_back({(int)i, rit->second, offset, stride, views});
+  }
+  for (auto &kv : blocks) {
+    const std::string &dst = kv.first;
+    std::vector<Block> &bl = kv.second;
+    if (bad[dst]) continue;
+    const Edge *we = edge(dst);
+    // writers: one Fill with zero, then the blocks
+    int fill = -1;
+    bool ok = true;
+    for (int w : writers[dst]) {
+      const OpDef &d = ops[w];
+      if (d.name() == "Fill" && d.input_size() == 1 && GetSingleArg<float>(d, "Value", 0.f) == 0.f && fill < 0) fill = w;
+      else if (d.name() != "PartialAccumulate") ok = false;
+    }
+    if (!ok || fill < 0 || fill > bl.front().op) continue;
+    // the blocks tile the Variable
+    std::sort(bl.begin(), bl.end(), [](const Block &a, const Block &b) { return a.offset < b.offset; });
+    long at = 0;
+    for (const Block &b : bl) {
+      if (b.offset != at) ok = false;
+      at += b.stride;
+    }
+    if (!ok || at != we->width()) continue;
+    // and are whole engine parameters in the engine's layout
+    std::map<std::string, long> base;    // param -> offset of its gradient inside dst
+    std::map<std::string, long> covered; // param -> elements covered
+    for (const Block &b : bl) {
+      const Slot &s = slots.at(b.role);
+      if (b.stride != s.count) ok = false;
+      const long off = b.offset - s.offset;
+      if (base.count(s.param) && base[s.param] != off) ok = false;
+      base[s.param] = off;
+      covered[s.param] += s.count;
+    }
+    for (auto &pv : covered) {
+      long total = 0;
+      for (auto &sv : slots)
+        if (pv.first == sv.second.param) total += sv.second.count;
+      if (total != pv.second) ok = false;  // a slice of the parameter goes somewhere else
+    }
+    if (!ok) continue;
+    mp->skip_bwd[fill] = 1;
+    for (const Block &b : bl) {
+      mp->skip_bwd[b.op] = 1;
+      // a copy whose only readers are skipped is dead too (nearest to the block first)
+      for (int v : b.views) {
+        bool read = false;
+        for (size_t i = 0; i < ops.size(); i++) {
+          if (mp->skip_bwd[i]) continue;
+          for (int k = 0; k < ops[i].input_size(); k++) read |= ops[i].input(k) == ops[v].output(0);
+        }
+        if (read) break;
+        mp->skip_bwd[v] = 1;
+      }
+    }
+    for (auto &pv : base) mp->binds.push_back({pv.first, dst, pv.second});
+  }
+}
+
+// See HeadFuse.
+void Executor::plan_fused_head(MainProgram *mp) const {
+  HeadFuse h;
+  const std::vector<OpDef> &fwd = mp->fwd, &bwd = mp->bwd;
+  auto no_acc = [](const OpDef &d) {
+    auto *a = d.find_attr("Acc");
+    if (a)
+      for (int v : a->value_.list_i)
+        if (v) return false;
+    return true;
+  };
+  for (size_t i = 0; i < fwd.size() && h.loss < 0; i++) {
+    if (fwd[i].name() != "SoftmaxEntropyLoss") continue;
+    for (size_t k = 0; k < i; k++)
+      if (fwd[k].name() == "FullyConnected" && fwd[k].output(0) == fwd[i].input(0)) {
+        h.fc = (int)k;
+        h.loss = (int)i;
+      }
+  }
+  if (h.loss < 0) return;
+  const OpDef &fc = fwd[h.fc], &loss = fwd[h.loss];
+  // the labels must exist when the FullyConnected operator runs
+  for (size_t k = h.fc; k < fwd.size(); k++)
+    for (int o = 0; o < fwd[k].output_size(); o++)
+      if (fwd[k].output(o) == loss.input(1)) return;
+  for (size_t i = 0; i < bwd.size(); i++) {
+    const OpDef &d = bwd[i];
+    if (d.name() == "SoftmaxEntropyLoss_grad" && d.input(0) == fc.output(0) && d.input(1) == loss.input(1)) h.loss_grad = (int)i;
+  }
+  if (h.loss_grad < 0) return;
+  const std::string &dy = bwd[h.loss_grad].output(0);
+  for (size_t i = 0; i < bwd.size(); i++) {
+    const OpDef &d = bwd[i];
+    bool reads = false;
+    for (int k = 0; k < d.input_size(); k++) reads |= d.input(k) == dy;
+    if (!reads) continue;
+    if (d.name() != "FullyConnected_grad" || h.fc_grad >= 0 || d.input(0) != dy || d.input(1) != fc.input(0) ||
+        d.input(2) != fc.input(1))
+      return;  // someone else wants d logits
+    h.fc_grad = (int)i;
+  }
+  if (h.fc_grad < 0 || !no_acc(bwd[h.fc_grad]) || !no_acc(bwd[h.loss_grad])) return;
+  for (size_t i = 0; i < bwd.size(); i++) {  // the seed of d loss: SoftmaxEntropyLoss_grad does not read it
+    if (bwd[i].name() != "ConstOp" || bwd[i].output(0) != GetGradientName(loss.output(0))) continue;
+    bool read = false;
+    for (auto &d : bwd)
+      for (int k = 0; k < d.input_size(); k++) read |= d.input(k) == bwd[i].output(0);
+    if (!read) h.seed = (int)i;
+  }
+  mp->head = h;
+}
+
+float *Executor::output_storage(const std::string &name, long *count) {
+  const Edge *e = edge(name);
+  if (!e) fail(CAVS_EINVAL, "no edge for '" + name + "'");
+  auto &slot = tensors_[name];
+  if (!slot) slot = std::make_unique<Tensor>();
+  Tensor &t = *slot;
+  t.width = e->width();
+  t.per_vertex = e->per_vertex();
+  if (t.per_vertex) t.rows = N_;
+  const size_t need = t.count();
+  if (t.own.capacity() < need) {
+    check(cavs_stream_sync(stream_));
+    t.own.reserve(need + need / 4);
+  }
+  t.base = t.own.get();
+  if (count) *count = (long)need;
+  return t.base;
+}
+
+// Returns false (and does nothing) when the shape of this batch is not one the fused entry point takes.
+bool Executor::run_fused_head(const MainProgram &mp) {
+  const HeadFuse &h = mp.head;
+  if (h.fc < 0) return false;
+  const OpDef &fc = mp.fwd[h.fc], &loss = mp.fwd[h.loss], &fg = mp.bwd[h.fc_grad];
+  RoundCtx c{0, 0, false};
+  long n0, w0, n1, w1, nb, wb, nl, wl;
+  const float *x = view(fc.input(0), c, &n0, &w0), *w = view(fc.input(1), c, &n1, &w1);
+  const float *b = view(fc.input(2), c, &nb, &wb), *lab = view(loss.input(1), c, &nl, &wl);
+  const int K = (int)w0, Nrow = (int)(n0 / w0), C = (int)(n1 / K);
+  const size_t bytes = cavs_fc_softmax_xent_workspace(Nrow, K, C);
+  if (bytes == 0 || nb != C || nl != Nrow) return false;
+  long cnt;
+  float *logits = output_storage(fc.output(0), &cnt);
+  float *lo = output_storage(loss.output(0), &cnt);
+  if (cnt != Nrow) return false;
+  float *dW = output_storage(fg.output(0), &cnt);
+  float *dB = output_storage(fg.output(1), &cnt);
+  float *dX = output_storage(fg.output(2), &cnt);
+  float *ws = workspace(bytes);
+  check(cavs_fc_softmax_xent(x, w, b, lab, lo, logits, dX, dW, dB, ws, ws_.capacity() * 4, Nrow, K, C, stream_));
+  return true;
+}
+
 void Executor::lowered_backward(const OpDef &d) {
   const Lowering &lw = *lowering_;
+  if (binds_) {
+    for (const GradBind &b : *binds_) {
+      const Edge *e = edge(b.dst);
+      auto &slot = tensors_[b.dst];
+      if (!slot) slot = std::make_unique<Tensor>();
+      Tensor &t = *slot;
+      t.width = e->width();
+      t.per_vertex = false;
+      if (t.own.capacity() < (size_t)t.width) {
+        check(cavs_stream_sync(stream_));
+        t.own.reserve(t.width);
+      }
+      t.base = t.own.get();
+      engine_->bind_param_grad(b.param, t.base + b.offset);
+    }
+  }
   engine_->backward_only(dgo_);
   // hand the gradients of the external edges to the main-scope backward program
   auto slots = role_slots(lw);
