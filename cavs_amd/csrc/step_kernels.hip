@@ -302,9 +302,11 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
       const float *__restrict__ src = static_cast<const float *>(t.p1);
       float *__restrict__ gout = static_cast<float *>(t.p2);
       const int bw = (int)t.n0, total = bw * (int)t.n1;
+      const int parts = (int)(t.n2 >> 32);  // 0 or 1: p1 is the row itself; more: rows to add up, in index order
       for (int i = b * 256 + tid; i < total; i += nb * 256) {
         const int k = i / bw, d = (int)((t.n2 >> (4 * k)) & 15) * bw + i % bw;
-        const float g = src[i];
+        float g = src[i];
+        for (int q = 1; q < parts; q++) g += src[(long)q * total + i];
         if (gout) gout[d] = g;
         if (w) w[d] -= t.f0 * g;
       }
@@ -449,7 +451,8 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         blocks = (t.n0 + kSgdChunk - 1) / kSgdChunk;
         break;
       case CAVS_TASK_BLOCKS_SGD: {
-        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n1 <= 8 && t.n0 < (1 << 26), "cavs_run_tasks: job %d: bad shape", i);
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n1 <= 8 && t.n0 < (1 << 26) && t.n2 >= 0 && (t.n2 >> 32) <= 4096,
+                     "cavs_run_tasks: job %d: bad shape", i);
         if (t.n0 == 0 || t.n1 == 0) continue;
         CAVS_REQUIRE(t.p1 && (t.p0 || t.p2), "cavs_run_tasks: job %d: null pointer", i);
         unsigned seen = 0;
@@ -534,28 +537,31 @@ size_t cavs_colsum_blocks_workspace(int n, int bw, int nb) {
   return (size_t)colsum_chunks(n) * bw * nb * sizeof(float);
 }
 
+int cavs_colsum_parts(int n) { return colsum_chunks(n); }
+
 int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int nb, const int *dst_block,
                        void *workspace, size_t workspace_bytes, void *stream) {
   CAVS_REQUIRE(n >= 0 && bw > 0 && nb > 0 && nb <= 8 && ld >= bw * nb, "cavs_colsum_blocks: bad shape n=%d bw=%d nb=%d ld=%d", n, bw, nb, ld);
-  CAVS_REQUIRE(out && dst_block, "cavs_colsum_blocks: null pointer");
+  CAVS_REQUIRE(!out || dst_block, "cavs_colsum_blocks: null block map");
   BlockMap map{};
   unsigned seen = 0;
-  for (int k = 0; k < nb; k++) {
+  for (int k = 0; out && k < nb; k++) {
     CAVS_REQUIRE(dst_block[k] >= 0 && dst_block[k] < nb && !(seen >> dst_block[k] & 1u), "cavs_colsum_blocks: dst_block is not a permutation");
     seen |= 1u << dst_block[k];
     map.dst[k] = dst_block[k];
   }
   const int w = bw * nb;
-  if (n == 0) return cavs_zero(out, (size_t)w * 4, stream);
-  CAVS_REQUIRE(inp, "cavs_colsum_blocks: null input");
   const int chunks = colsum_chunks(n);
   const size_t need = (size_t)chunks * w * sizeof(float);
+  if (n == 0) return out ? cavs_zero(out, (size_t)w * 4, stream) : (workspace ? cavs_zero(workspace, need, stream) : CAVS_OK);
+  CAVS_REQUIRE(inp, "cavs_colsum_blocks: null input");
   CAVS_REQUIRE(workspace && workspace_bytes >= need, "cavs_colsum_blocks: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
   const int rpc = ((n + chunks - 1) / chunks + 3) / 4 * 4;
   hipStream_t st = as_stream(stream);
   float *part = static_cast<float *>(workspace);
   launch(colsum_part_kernel, dim3((w + 63) / 64, chunks), 256, 0, st, part, inp, ld, n, w, rpc);
   CAVS_LAUNCH_CHECK();
+  if (!out) return CAVS_OK;  // the chunk sums stay in the workspace
   launch(colsum_blocks_reduce_kernel, (w + 63) / 64, 256, 0, st, out, part, chunks, w, bw, map);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;

@@ -410,6 +410,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
   N_ = sched_.N;
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   c_round_flops_ = 0;
+  bias_jobs_.clear();
   reserve_edges();
   upload_index_arena();
   parse_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
@@ -442,7 +443,7 @@ void Engine::backward_only(const float *dgraph_out) {
     case CAVS_MODEL_LSTM: lstm_backward(); break;
     default: treefc_backward();
   }
-  settle_bias_row(0.f, nullptr);  // no update follows in here: the bias gradient is delivered now
+  settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
   check(cavs_event_record(ev_[3], stream_));
   ev_bwd_valid_ = true;
 }
@@ -508,11 +509,12 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       // only: every other row of its gradient is zero, so the dense update would not move it
       // all of it in one launch: the updates touch disjoint tensors
       std::vector<cavs_task> tasks;
-      const bool bias_job = bias_row_pending_;
-      settle_bias_row(lr, &tasks);
+      std::vector<std::string> by_job;
+      for (const BiasJob &j : bias_jobs_) by_job.push_back(j.param);
+      settle_bias_jobs(lr, &tasks);
       for (auto &kv : params_) {
         Param &p = *kv.second;
-        if (kv.first == "Bv" && bias_job) continue;  // updated by the job that delivers its gradient
+        if (std::find(by_job.begin(), by_job.end(), kv.first) != by_job.end()) continue;  // updated by the job that delivers its gradient
         if (kv.first == "Emb" && emb_dirty_n_ == N) {
           const int E = (int)(p.n / cfg_.V);
           if (emb_stamp_.capacity() < (size_t)cfg_.V) {
@@ -527,7 +529,7 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       check(cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
       c_launches_ += 1;
     } else {
-      settle_bias_row(0.f, nullptr);
+      settle_bias_jobs(0.f, nullptr);
     }
   }
 }
@@ -708,7 +710,9 @@ void Engine::treelstm_backward() {
   embedding_backward(E);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
   if (bias_row) {
-    bias_row_pending_ = true;  // settled by the launch that ends the step (or right after this pass)
+    // settled by the launch that ends the step (or right after this pass); block k of the row
+    // ([i|o|u|f]) lands in bias block map[k] ([i|f|u|o])
+    bias_jobs_.push_back({"Bv", param("W").g + param("W").n, 1, H, 4, 0 | (3 << 4) | (2 << 8) | (1 << 12)});
     return;
   }
   const int dst_block[4] = {0, 3, 2, 1};  // dxW block k ([i|o|u|f]) lands in bias block dst_block[k]
@@ -728,18 +732,58 @@ bool Engine::bias_row_ok() const {
   return w.g == w.own_g.get();
 }
 
-// Row E of dW ([i|o|u|f] blocks) -> Bv.g ([i|f|u|o]), and the update of Bv with it when lr != 0:
-// as a job of `tasks` if given, else as a launch of its own.
-void Engine::settle_bias_row(float lr, std::vector<cavs_task> *tasks) {
-  if (!bias_row_pending_) return;
-  bias_row_pending_ = false;
-  Param &w = param("W"), &b = param("Bv");
-  const long long map = 0 | (3 << 4) | (2 << 8) | (1 << 12);  // block k of the row lands in bias block map[k]
-  cavs_task t{CAVS_TASK_BLOCKS_SGD, lr, cfg_.H, 4, map, lr != 0.f ? b.w : nullptr, w.g + w.n, b.g, nullptr};
-  if (tasks) {
-    tasks->push_back(t);
-  } else {
+// One launch leaves the chunk sums; the job that ends the step adds them up in index order.
+void Engine::bias_gradient(const std::string &name, const float *inp, int n, int w, DeviceArray<float> &parts) {
+  const size_t bytes = cavs_colsum_blocks_workspace(n, w, 1);
+  if (parts.capacity() * 4 < bytes) {
+    check(cavs_stream_sync(stream_));
+    parts.reserve(bytes / 4 + 1);
+  }
+  check(cavs_colsum_blocks(nullptr, inp, w, n, w, 1, nullptr, parts.get(), parts.capacity() * 4, stream_));
+  c_launches_ += 1;
+  bias_jobs_.push_back({name, parts.get(), cavs_colsum_parts(n), w, 1, 0});
+}
+
+// out [w] = column sums of inp [n, w], chunks of rows added in index order
+void Engine::colsum_fixed(float *out, const float *inp, int n, int w) {
+  if (w == 1) {  // a short vector to a scalar: one workgroup
+    cavs_task t{CAVS_TASK_SUM_PARTS, 0.f, n, 1, 1, const_cast<float *>(inp), out, nullptr, nullptr};
     check(cavs_run_tasks(1, &t, stream_));
+    c_launches_ += 1;
+    return;
+  }
+  if (n <= 64) {  // a single chunk of rows: cavs_colsum adds nothing atomically
+    check(cavs_colsum(out, inp, w, n, w, 0, stream_));
+    c_launches_ += 1;
+    return;
+  }
+  const int identity[1] = {0};
+  const size_t bytes = cavs_colsum_blocks_workspace(n, w, 1);
+  float *ws = workspace(bytes);
+  check(cavs_colsum_blocks(out, inp, w, n, w, 1, identity, ws, bytes, stream_));
+  c_launches_ += 2;
+}
+
+bool Engine::has_bias_job(const std::string &name) const {
+  for (const BiasJob &j : bias_jobs_)
+    if (j.param == name) return true;
+  return false;
+}
+
+// Each pending row set -> the parameter's gradient, and the update of the parameter with it when
+// lr != 0: as jobs of `tasks` if given, else as a launch of their own.
+void Engine::settle_bias_jobs(float lr, std::vector<cavs_task> *tasks) {
+  if (bias_jobs_.empty()) return;
+  std::vector<cavs_task> own;
+  for (const BiasJob &j : bias_jobs_) {
+    Param &b = param(j.param);
+    cavs_task t{CAVS_TASK_BLOCKS_SGD, lr, j.bw, j.nb, j.map | ((long long)j.parts << 32), lr != 0.f ? b.w : nullptr,
+                const_cast<float *>(j.src), b.g, nullptr};
+    (tasks ? *tasks : own).push_back(t);
+  }
+  bias_jobs_.clear();
+  if (!own.empty()) {
+    check(cavs_run_tasks((int)own.size(), own.data(), stream_));
     c_launches_ += 1;
   }
 }
@@ -892,8 +936,7 @@ void Engine::lstm_backward() {
        dW + (size_t)4 * H * H, 4 * H},
   });
   embedding_backward(H);
-  check(cavs_colsum(param("Bv").g, dxW_.get(), 4 * H, N, 4 * H, 0, stream_));
-  c_launches_ += 1;
+  bias_gradient("Bv", dxW_.get(), N, 4 * H, bias_parts_);
 }
 
 // ------------------------------------------------------------------ Tree-FC
@@ -998,8 +1041,7 @@ void Engine::treefc_backward() {
   gemm_splitk(1, 0, 2 * H, H, N - lp, G_.at((size_t)2 * lp * H), 2 * H, dxW_.at((size_t)lp * H), H,
               param("W").g, H);
   if (cfg_.use_bias) {
-    check(cavs_colsum(param("Bv").g, dxW_.get(), H, N, H, 0, stream_));
-    c_launches_ += 1;
+    bias_gradient("Bv", dxW_.get(), N, H, bias_parts_);
   }
 }
 
@@ -1035,8 +1077,7 @@ void Engine::head_forward_backward(bool backward) {
       // both read d logits and write different outputs: one launch when they are small
       gemm_group({{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, GO_.get(), H, Wfc.g, H},
                   {0, 0, N, H, C, 1.f, 0.f, dlogits_.get(), C, Wfc.w, H, dGO_.get(), H}});
-      check(cavs_colsum(bfc.g, dlogits_.get(), C, N, C, 0, stream_));
-      c_launches_ += 1;
+      bias_gradient("bfc", dlogits_.get(), N, C, head_bias_parts_);
     }
     return;
   }
@@ -1045,9 +1086,9 @@ void Engine::head_forward_backward(bool backward) {
     // sum over roots of h^2; gradient 2h on root rows, zero elsewhere
     gather(tmp, H, GO_.get(), H, d_roots_, B, H);
     check(cavs_ew_unary(CAVS_EW_SQUARE, dlogits_.get(), tmp, (size_t)B * H, 0, stream_));
-    check(cavs_colsum(colacc, dlogits_.get(), H, B, H, 0, stream_));
-    check(cavs_colsum(loss_.get(), colacc, 1, H, 1, 0, stream_));
-    c_launches_ += 3;
+    colsum_fixed(colacc, dlogits_.get(), B, H);
+    colsum_fixed(loss_.get(), colacc, H, 1);
+    c_launches_ += 1;  // the squares
     if (backward) {
       check(cavs_zero(dGO_.get(), (size_t)N * H * 4, stream_));
       check(cavs_scale(dlogits_.get(), tmp, 2.f, (size_t)B * H, stream_));
@@ -1058,9 +1099,9 @@ void Engine::head_forward_backward(bool backward) {
     // Reduce_sum is a sum of absolute values whose gradient op is a constant fill
     // (cavs/backend/op_impl_blas1_cublas.cc:62-77, cavs/backend/op_decl_reduction.cc:19-28)
     check(cavs_ew_unary(CAVS_EW_ABS, dlogits_.get(), GO_.get(), (size_t)N * H, 0, stream_));
-    check(cavs_colsum(colacc, dlogits_.get(), H, N, H, 0, stream_));
-    check(cavs_colsum(loss_.get(), colacc, 1, H, 1, 0, stream_));
-    c_launches_ += 3;
+    colsum_fixed(colacc, dlogits_.get(), N, H);
+    colsum_fixed(loss_.get(), colacc, H, 1);
+    c_launches_ += 1;
     if (backward) {
       check(cavs_fill(dGO_.get(), 1.f, (size_t)N * H, stream_));
       c_launches_ += 1;

@@ -162,9 +162,23 @@ class Engine {
   int ld_e_ = 0;
   size_t e_ones_rows_ = 0;       // rows of e_ whose ones column is initialised
   DeviceArray<float> ones_col_;  // [ld_e_]: 1 at column E
-  bool bias_row_pending_ = false;  // row E of dW holds this step's bias gradient, not yet in Bv.g
   bool bias_row_ok() const;
-  void settle_bias_row(float lr, std::vector<cavs_task> *tasks);
+  // Bias gradients that exist as rows still to be added up and / or permuted (row E of dW; the
+  // chunk sums of a column sum): delivered, and the parameter updated, by one job each of the
+  // launch that ends the step.
+  struct BiasJob {
+    std::string param;
+    const float *src;
+    int parts;
+    long long bw, nb, map;
+  };
+  std::vector<BiasJob> bias_jobs_;
+  DeviceArray<float> bias_parts_, head_bias_parts_;
+  // column sums of inp [n, w] as the gradient of `name`, in a fixed order
+  void bias_gradient(const std::string &name, const float *inp, int n, int w, DeviceArray<float> &parts);
+  void colsum_fixed(float *out, const float *inp, int n, int w);
+  bool has_bias_job(const std::string &name) const;
+  void settle_bias_jobs(float lr, std::vector<cavs_task> *tasks);
   DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds

@@ -275,8 +275,11 @@ int cavs_embed_sgd(float *table, const float *dtable, const float *ids, int n, i
 int cavs_embed_zero_rows(float *dtable, const float *ids, int n, int E, void *stream);
 /* Column sums of nb (<= 8) adjacent column blocks of bw columns of inp [n, ld], block k written
  * to out block dst_block[k] (a permutation; host array).  Deterministic: row chunks are summed
- * in index order.  The bias gradient of the gates (cavs/backend/op_impl_elementwise.cuh:24-34). */
+ * in index order.  The bias gradient of the gates (cavs/backend/op_impl_elementwise.cuh:24-34).
+ * With out NULL (dst_block may be NULL too) the chunk sums stay in the workspace as
+ * cavs_colsum_parts(n) rows of bw*nb floats, for a CAVS_TASK_BLOCKS_SGD job to add up. */
 size_t cavs_colsum_blocks_workspace(int n, int bw, int nb);
+int cavs_colsum_parts(int n);
 int cavs_colsum_blocks(float *out, const float *inp, int ld, int n, int bw, int nb,
                        const int *dst_block, void *workspace, size_t workspace_bytes, void *stream);
 
@@ -391,7 +394,9 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *   CAVS_TASK_BLOCKS_SGD p1 holds n1 (<= 8) blocks of n0 floats; block k goes to block d_k of p2 (if
  *                        given) and p0[d_k block] -= f0 * it (if p0 given); d_k = (n2 >> 4k) & 15, a
  *                        permutation.  A gradient that arrives in another block order than its
- *                        parameter's (the gate bias, apps/paper/tree-lstm-cavs.cc:120-123 vs :143-148). */
+ *                        parameter's (the gate bias, apps/paper/tree-lstm-cavs.cc:120-123 vs :143-148).
+ *                        With P = n2 >> 32 above 1, p1 holds P such rows and the job adds them up first,
+ *                        in index order (the chunk sums cavs_colsum_blocks leaves behind). */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
        CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5 };
 typedef struct cavs_task {

@@ -272,6 +272,32 @@ def test_backward_rounds_as_one_launch_or_two(oracle, model, kw, pairing):
     assert launches[0] < launches[1], launches
 
 
+@pytest.mark.parametrize("name", ["C1", "C2", "C3"])
+def test_a_step_is_reproducible_bit_for_bit(name):
+    """Every sum on the path runs in a fixed order (partial tiles through LDS in wavefront order,
+    split-K partials and column sums by index), so two runs of the same step agree bit for bit --
+    all but the embedding gradient, whose repeated rows are added with atomics."""
+    w = synth.make_workload(name)
+    kw = dict(H=w["H"], E=w["E"], V=w["V"], C_=w["C"])
+    if w["model"] == "treefc":
+        kw.update(loss="root_sq", act=1, use_bias=True, use_x=True)
+    runs = []
+    for k in range(2):
+        print(f"[case] {name} reproducibility run {k}", flush=True)
+        s = session.Session(w["model"], **kw)
+        s.set_params(w["params"])
+        s.step(w["graph"], w["x"], w["labels"], backward=True)
+        runs.append(dict(loss=s.fetch("loss"), go=s.fetch("graph_out"), dgo=s.fetch("dgraph_out"), grads=s.grads()))
+        s.close()
+    for k in ("loss", "go", "dgo"):
+        np.testing.assert_array_equal(runs[0][k], runs[1][k], err_msg=k)
+    for k, v in runs[0]["grads"].items():
+        if k == "dEmb":
+            close(v, runs[1]["grads"][k], k)
+        else:
+            np.testing.assert_array_equal(v, runs[1]["grads"][k], err_msg=k)
+
+
 @pytest.mark.parametrize("model", ["treelstm", "lstm"])
 def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     """Four SGD steps over three different batches (token ids overlap between steps, one

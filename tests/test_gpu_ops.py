@@ -903,6 +903,22 @@ def test_column_sums_of_permuted_blocks(g, n, bw, perm):
     close(first, want.ravel(), rtol=1e-4, atol=1e-5 * np.sqrt(n))
     g.call("cavs_colsum_blocks", g.P(out), g.P(dX), ld, n, bw, nb, dst, g.P(ws), nbytes, g.stream())
     np.testing.assert_array_equal(g.host(out), first)           # fixed summation order
+    # the same in two halves: the chunk sums left in the workspace, added up (permuted, and
+    # applied to a parameter) by a job of the launch that ends a step
+    parts = hip.lib().cavs_colsum_parts(n)
+    assert 1 <= parts and parts * bw * nb * 4 == nbytes
+    g.call("cavs_colsum_blocks", None, g.P(dX), ld, n, bw, nb, None, g.P(ws), nbytes, g.stream())
+    w0 = r.bulk_normal(nb * bw)
+    d_w, out2 = g.devf(w0), g.zeros(nb * bw, fill=float("nan"))
+    bmap = sum(d << (4 * k) for k, d in enumerate(perm)) | (parts << 32)
+    job = (hip.Task * 1)(hip.Task(hip.TASK_BLOCKS_SGD, 0.5, bw, nb, bmap, g.P(d_w), g.P(ws), g.P(out2), None))
+    g.call("cavs_run_tasks", 1, job, g.stream())
+    second = g.host(out2).copy()
+    close(second, want.ravel(), rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    np.testing.assert_array_equal(g.host(d_w), w0 - np.float32(0.5) * second)
+    job[0].p0 = None                                            # gradient only, again: same bits
+    g.call("cavs_run_tasks", 1, job, g.stream())
+    np.testing.assert_array_equal(g.host(out2), second)
     with pytest.raises(hip.CavsError, match="permutation"):
         hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * nb)(*([0] * nb)), 16, nbytes, 0) if nb > 1 else \
             hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * 1)(3), 16, nbytes, 0)
