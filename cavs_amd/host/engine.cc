@@ -342,7 +342,7 @@ void Engine::upload_index_arena() {
   int nr = 0;
   for (int v = 0; v < N; v++)
     if (s.parent[v] < 0) roots[nr++] = v;
-  forest_ = want_forest && build_forest_lists(roots + s.B, roots + s.B + (size_t)nch_ * N);
+  forest_ = want_forest && build_forest_lists(pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N);
   check(cavs_memcpy_h2d(idx_dev_.get(), idx_host_[slot].get(), total * sizeof(int), stream_));
   check(cavs_event_record(idx_copied_[slot], stream_));
   idx_pending_[slot] = true;
@@ -357,12 +357,11 @@ void Engine::upload_index_arena() {
 // The backward launch that folds the children's gate gradients in addresses a child by its slab
 // row, not by the pool row its message went through.  That is the same thing only while the
 // message flow is a forest: every pool row a Gather reads was written by exactly one slab row of
-// an earlier round and is read by exactly one (vertex, child slot).  Reads the host copies of
-// `pair` and `child` in the staging buffer that is about to be uploaded.
-bool Engine::build_forest_lists(int *kid_rows, int *orphans) {
+// an earlier round and is read by exactly one (vertex, child slot).  `pair` and `child` are the
+// host copies of the lists in the staging buffer that is about to be uploaded.
+bool Engine::build_forest_lists(const int *pair, const int *child, int *kid_rows, int *orphans) {
   const Schedule &s = sched_;
   const int N = N_;
-  const int *pair = kid_rows - s.B - (size_t)nch_ * N - N, *child = pair + N;
   n_orphans_ = 0;
   if (!s.batching || s.rounds.empty() || !leaf_round(s.rounds[0]) || s.rounds[0].n != s.leaf_prefix) return false;
   inv_pair_.assign(N, -1);

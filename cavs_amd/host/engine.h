@@ -138,7 +138,7 @@ class Engine {
   int n_orphans_ = 0;
   bool forest_ = false;
   std::vector<int> inv_pair_, round_of_row_;
-  bool build_forest_lists(int *kid_rows, int *orphans);
+  bool build_forest_lists(const int *pair, const int *child, int *kid_rows, int *orphans);
 
   // feeds
   DeviceArray<float> x_in_, labels_in_;
