@@ -86,5 +86,71 @@ inline RoundPlan plan_round(int n) {
   return {32, 8};
 }
 
+// The product loop of the fused round kernels when the wavefront's k range is an even number of
+// whole pipeline stages (exact_stages below): acc[i] += A_i[row, k) * B[k, col] for NA operands
+// A_i that share one B.  B comes through buffer loads -- a descriptor in scalar registers, a
+// scalar byte offset that advances with k, and this lane's byte offsets vb[c] of column col in
+// row 4 * slot + c of a k-group, fixed before the loop -- so no address arithmetic runs on the
+// vector ALU (spelled out per load, its 64-bit row * stride products cost as much time as the
+// MFMAs).  A rows are per-lane pointers (already at this wavefront's first k plus 4 * slot),
+// bumped once per k-group.  Nothing in the loop is conditional, so the wait counts of the two
+// stage buffers come out exact and one stage's loads are in flight under the other's MFMAs; the
+// scheduler barriers keep that order (left alone, the compiler sinks every load to its use).
+template <int TILE, int UG, int NA>
+__device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float *(&arow)[NA], __amdgpu_buffer_rsrc_t bbuf,
+                                      const int (&vb)[4], int sb, int b_row_bytes, int nst) {
+  using M = Mma<TILE>;
+  constexpr int GK = 4 * M::NSLOT;
+  struct Frag {
+    float4 a[UG][NA];
+    float b[UG][4];
+  };
+  auto fetch = [&](Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+#pragma unroll
+      for (int c = 0; c < 4; c++) f.b[u][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb, 0));
+#pragma unroll
+      for (int i = 0; i < NA; i++) {
+        f.a[u][i] = ld4(arow[i]);
+        arow[i] += GK;
+      }
+      sb += GK * b_row_bytes;
+    }
+  };
+  auto multiply = [&](const Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++)
+#pragma unroll
+      for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int i = 0; i < NA; i++) acc[i] = M::mma(elem(f.a[u][i], c), f.b[u][c], acc[i]);
+  };
+  Frag f0, f1;
+  fetch(f0);
+  for (int st = 0; st + 2 < nst; st += 2) {
+    fetch(f1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(f0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(f0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(f1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  fetch(f1);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(f0);
+  multiply(f1);
+}
+
+// K = H splits into an even number of whole pipeline stages for every wavefront of the plan's
+// kernels (K-splits = wavefronts; a k-group is 16 k for either MFMA shape; one group per stage for
+// the four-wavefront 16x16 kernels, two otherwise), and the weights' byte offsets fit 31 bits
+inline bool exact_stages(int H, const RoundPlan &p) {
+  const int ug = (p.tile == 16 && p.waves == 4) ? 1 : 2;
+  return H % (p.waves * 16 * ug * 2) == 0 && H <= 8192;
+}
+
 }  // namespace cavs
 #endif

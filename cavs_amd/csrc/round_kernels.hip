@@ -41,7 +41,14 @@ struct RoundFwdArgs {
   int n, H;
 };
 
-template <int TILE, int WAVES>
+// EXACT: H splits into an even number of whole pipeline stages for every wavefront.  The product
+// loop then has no ragged end and no conditions: the weights come through buffer loads whose
+// address is a descriptor of U in scalar registers, a scalar offset that advances with k and a
+// per-lane offset fixed before the loop (no address arithmetic on the vector ALU, whose 64-bit
+// row * stride products otherwise cost as much time as the MFMAs), the rows of A through
+// per-lane pointers that are bumped once per k-group, and the wait counts of the two stage
+// buffers come out exact, so the loads of one stage are in flight under the MFMAs of the other.
+template <int TILE, int WAVES, bool EXACT>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -150,6 +157,21 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   };
   Frag f0, f1;
   constexpr int S = GK * UG;
+  // EXACT: a missing child (no message to gather) is masked where the operand is used
+  const bool has_l = cl >= 0, has_r = cr >= 0;
+  auto xmultiply = [&](const Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float hl = has_l ? elem(f.hl[u], c) : 0.f, hr = has_r ? elem(f.hr[u], c) : 0.f, hs = hl + hr;
+        acc[0] = M::mma(hs, f.b[u][0][c], acc[0]);
+        acc[1] = M::mma(hs, f.b[u][1][c], acc[1]);
+        acc[2] = M::mma(hs, f.b[u][2][c], acc[2]);
+        acc[3] = M::mma(hl, f.b[u][3][c], acc[3]);
+        acc[4] = M::mma(hr, f.b[u][3][c], acc[4]);
+      }
+  };
   if (kb < ke) fetch_b(kb, f0);
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
@@ -170,12 +192,60 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     if (ep.c_r >= 0) { ep.hr = a.pool[ep.c_r * H2 + ep.j]; ep.cr = a.pool[ep.c_r * H2 + H + ep.j]; }
   }
 
-  for (int k0 = kb; k0 < ke; k0 += 2 * S) {
-    if (k0 + S < ke) fetch(k0 + S, f1);
-    multiply(f0);
-    if (k0 + S < ke) {
-      if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
-      multiply(f1);
+  if constexpr (EXACT) {
+    const __amdgpu_buffer_rsrc_t ubuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.U), 0, 4 * H * H * 4, 0x00020000);
+    int vio[4], vf[4];  // byte offsets of this lane's column in row 4 * slot + c of a k-group
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+      vio[c] = ((4 * slot + c) * 3 * H + j0 + x) * 4;
+      vf[c] = ((4 * slot + c) * H + j0 + x) * 4;
+    }
+    const int kbu = __builtin_amdgcn_readfirstlane(kb), nst = __builtin_amdgcn_readfirstlane((ke - kb) / S);
+    int sio = (kbu + S) * 3 * H * 4, sf = (3 * H * H + (kbu + S) * H) * 4;  // scalar byte offsets of the next k-group
+    const float *al = pl + kb + S + 4 * slot, *ar = pr + kb + S + 4 * slot;
+    auto xfetch = [&](Frag &f) {
+#pragma unroll
+      for (int u = 0; u < UG; u++) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          f.b[u][0][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio, 0));
+          f.b[u][1][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 4, 0));
+          f.b[u][2][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 8, 0));
+          f.b[u][3][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vf[c], sf, 0));
+        }
+        f.hl[u] = ld4(al);
+        f.hr[u] = ld4(ar);
+        sio += GK * 3 * H * 4;
+        sf += GK * H * 4;
+        al += GK;
+        ar += GK;
+      }
+    };
+    // (the first stage was fetched above through the general path; nst is even)
+    // (the scheduler barriers keep a stage's loads ahead of the other stage's MFMAs; left alone,
+    // the compiler sinks every load to just before its use)
+    for (int st = 0; st + 2 < nst; st += 2) {
+      xfetch(f1);
+      __builtin_amdgcn_sched_barrier(0);
+      xmultiply(f0);
+      __builtin_amdgcn_sched_barrier(0);
+      xfetch(f0);
+      __builtin_amdgcn_sched_barrier(0);
+      xmultiply(f1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    xfetch(f1);
+    __builtin_amdgcn_sched_barrier(0);
+    xmultiply(f0);
+    xmultiply(f1);
+  } else {
+    for (int k0 = kb; k0 < ke; k0 += 2 * S) {
+      if (k0 + S < ke) fetch(k0 + S, f1);
+      multiply(f0);
+      if (k0 + S < ke) {
+        if (k0 + 2 * S < ke) fetch(k0 + 2 * S, f0);
+        multiply(f1);
+      }
     }
   }
 
@@ -441,7 +511,7 @@ struct RoundBwdChildArgs {
   int row0, leaf_rows;
 };
 
-template <int TILE, int WAVES, bool FOLD>
+template <int TILE, int WAVES, bool FOLD, bool EXACT>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -537,6 +607,24 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
 
   constexpr int S = GK * UG;
+  if constexpr (EXACT) {
+    const __amdgpu_buffer_rsrc_t tbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(a.UT), 0, 4 * H * H * 4, 0x00020000);
+    int vb[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) vb[c] = ((4 * slot + c) * H + j0 + x) * 4;
+    const int ksu = __builtin_amdgcn_readfirstlane(ks);
+    {  // P0: K = 3H
+      const int kb = ksu * (3 * H / KS);
+      const float *arow[1] = {px + kb + 4 * slot};
+      exact_products<TILE, UG, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, 3 * H / KS / S);
+    }
+    fetch_kids();
+    {  // P1, P2: K = H, one B operand for both
+      const int kb = ksu * (H / KS);
+      const float *arow[2] = {pfl + kb + 4 * slot, pfr + kb + 4 * slot};
+      exact_products<TILE, UG, 2>(&acc[1], arow, tbuf, vb, (3 * H * H + kb * H) * 4, H * 4, H / KS / S);
+    }
+  } else {
   {  // P0: K = 3H
     const int K = 3 * H;
     const int kper = ((K + KS - 1) / KS + GK - 1) / GK * GK;
@@ -612,6 +700,7 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       }
     }
   }
+  }
 
   park_partials<TILE, NP, KS, NREG, RT>(red, acc, rt, ks, lane);
 
@@ -667,10 +756,18 @@ template <bool FOLD>
 static void launch_bwd_children(const RoundBwdChildArgs &a, hipStream_t st) {
   const RoundPlan p = plan_round(a.n);
   dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
-  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, FOLD>, grid, 256, 0, st, a);
-  else if (p.tile == 16) launch(treelstm_round_bwd_children_kernel<16, 8, FOLD>, grid, 512, 0, st, a);
-  else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<32, 4, FOLD>, grid, 256, 0, st, a);
-  else launch(treelstm_round_bwd_children_kernel<32, 8, FOLD>, grid, 512, 0, st, a);
+  const bool exact = exact_stages(a.H, p);
+  if (p.tile == 16 && p.waves == 4) {
+    if (exact) launch(treelstm_round_bwd_children_kernel<16, 4, FOLD, true>, grid, 256, 0, st, a);
+    else launch(treelstm_round_bwd_children_kernel<16, 4, FOLD, false>, grid, 256, 0, st, a);
+  } else if (p.tile == 16) {
+    if (exact) launch(treelstm_round_bwd_children_kernel<16, 8, FOLD, true>, grid, 512, 0, st, a);
+    else launch(treelstm_round_bwd_children_kernel<16, 8, FOLD, false>, grid, 512, 0, st, a);
+  } else if (p.waves == 4) {
+    launch(treelstm_round_bwd_children_kernel<32, 4, FOLD, false>, grid, 256, 0, st, a);
+  } else {
+    launch(treelstm_round_bwd_children_kernel<32, 8, FOLD, false>, grid, 512, 0, st, a);
+  }
 }
 
 }  // namespace cavs
@@ -692,10 +789,18 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   const RoundPlan p = plan_round(n);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
-  if (p.tile == 16 && p.waves == 4) launch(treelstm_round_fwd_kernel<16, 4>, grid, 256, 0, st, a);
-  else if (p.tile == 16) launch(treelstm_round_fwd_kernel<16, 8>, grid, 512, 0, st, a);
-  else if (p.waves == 4) launch(treelstm_round_fwd_kernel<32, 4>, grid, 256, 0, st, a);
-  else launch(treelstm_round_fwd_kernel<32, 8>, grid, 512, 0, st, a);
+  const bool exact = exact_stages(H, p);
+  if (p.tile == 16 && p.waves == 4) {
+    if (exact) launch(treelstm_round_fwd_kernel<16, 4, true>, grid, 256, 0, st, a);
+    else launch(treelstm_round_fwd_kernel<16, 4, false>, grid, 256, 0, st, a);
+  } else if (p.tile == 16) {
+    if (exact) launch(treelstm_round_fwd_kernel<16, 8, true>, grid, 512, 0, st, a);
+    else launch(treelstm_round_fwd_kernel<16, 8, false>, grid, 512, 0, st, a);
+  } else if (p.waves == 4) {
+    launch(treelstm_round_fwd_kernel<32, 4, false>, grid, 256, 0, st, a);
+  } else {
+    launch(treelstm_round_fwd_kernel<32, 8, false>, grid, 512, 0, st, a);
+  }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
