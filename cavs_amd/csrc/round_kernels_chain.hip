@@ -53,6 +53,74 @@ __device__ inline void product_chain(typename Mma<TILE>::Acc (&acc)[NB], const f
   }
 }
 
+// The same chain when the wavefront's k range is an even number of whole stages of 32 k
+// (chain_exact): the B operands come through buffer loads -- descriptor and k offset in scalar
+// registers, this lane's byte offsets fixed before the loop -- so that no address arithmetic
+// runs on the vector ALU, nothing in the loop is conditional and the wait counts come out exact
+// (see exact_products).  B operand p is the block of columns [p * blk, p * blk + H) of the
+// row-major matrix `bmat` (`bfloats` floats, row stride ldb); the chain covers its rows
+// [krow, krow + 32 * nst).  a_row is already at this wavefront's first k; a lane without a row
+// passes any readable address and has = false.
+template <int TILE, int NB>
+__device__ inline void product_chain_exact(typename Mma<TILE>::Acc (&acc)[NB], const float *a_row, bool has, const float *bmat,
+                                           int bfloats, int col, int blk, int ldb, int krow, int nst, int slot) {
+  using M = Mma<TILE>;
+  constexpr int GK = 4 * M::NSLOT, UG = 2;
+  const __amdgpu_buffer_rsrc_t bbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(bmat), 0, bfloats * 4, 0x00020000);
+  int vb[4];
+#pragma unroll
+  for (int c = 0; c < 4; c++) vb[c] = ((4 * slot + c) * ldb + col) * 4;
+  int sb = krow * ldb * 4;
+  a_row += 4 * slot;
+  struct Frag {
+    float4 a[UG];
+    float b[UG][NB][4];
+  };
+  auto fetch = [&](Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+#pragma unroll
+      for (int p = 0; p < NB; p++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+          f.b[u][p][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb + p * blk * 4, 0));
+      f.a[u] = ld4(a_row);
+      a_row += GK;
+      sb += GK * ldb * 4;
+    }
+  };
+  auto multiply = [&](const Frag &f) {
+#pragma unroll
+    for (int u = 0; u < UG; u++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        const float av = has ? elem(f.a[u], c) : 0.f;
+#pragma unroll
+        for (int p = 0; p < NB; p++) acc[p] = M::mma(av, f.b[u][p][c], acc[p]);
+      }
+  };
+  Frag f0, f1;
+  fetch(f0);
+  for (int st = 0; st + 2 < nst; st += 2) {
+    fetch(f1);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(f0);
+    __builtin_amdgcn_sched_barrier(0);
+    fetch(f0);
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(f1);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  fetch(f1);
+  __builtin_amdgcn_sched_barrier(0);
+  multiply(f0);
+  multiply(f1);
+}
+
+// K rows of B split over `waves` wavefronts into an even number of whole stages each, and the
+// byte offsets into B fit 31 bits
+inline bool chain_exact(long K, int waves, long bfloats) { return K > 0 && K % (waves * 64) == 0 && bfloats < (1L << 28); }
+
 // element (q-th of this thread) of the workgroup's tile: slab row, column, LDS offset
 template <int TILE, int NP, int THREADS>
 struct TileElems {
@@ -122,7 +190,7 @@ struct LstmFwdArgs {
   int n, H;
 };
 
-template <int TILE, int WAVES>
+template <int TILE, int WAVES, bool EXACT>
 __global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -166,7 +234,13 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs 
   const float *bcol[NP];
 #pragma unroll
   for (int p = 0; p < NP; p++) bcol[p] = a.Wh + p * H + j0 + x;
-  product_chain<TILE, NP>(acc, cp >= 0 ? a.pool + cp * H2 : nullptr, bcol, H4, kb, ke, slot);
+  if constexpr (EXACT) {
+    const int kbu = __builtin_amdgcn_readfirstlane(ks) * (H / KS);
+    product_chain_exact<TILE, NP>(acc, a.pool + (cp >= 0 ? cp : 0) * H2 + kbu, cp >= 0, a.Wh, 4 * H * H, j0 + x, H, 4 * H, kbu,
+                                  H / KS / 32, slot);
+  } else {
+    product_chain<TILE, NP>(acc, cp >= 0 ? a.pool + cp * H2 : nullptr, bcol, H4, kb, ke, slot);
+  }
 
   float ehp[EPT], ecprev[EPT];
 #pragma unroll
@@ -383,7 +457,7 @@ struct ChildBwdArgs {
   int row0, leaf_rows, act;
 };
 
-template <int TILE, int WAVES, int NB, int FOLD>
+template <int TILE, int WAVES, bool EXACT, int NB, int FOLD>
 __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -447,7 +521,13 @@ __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwd
 #pragma unroll
     for (int r = 0; r < NR; r++) acc[p][r] = 0.f;
   }
-  product_chain<TILE, NB>(acc, row < a.n ? a.dA + row * a.ld : nullptr, bcol, a.ldb, kb, ke, slot);
+  if constexpr (EXACT) {
+    const int kbu = __builtin_amdgcn_readfirstlane(ks) * (K / KS);
+    product_chain_exact<TILE, NB>(acc, a.dA + (row < a.n ? row : 0) * a.ld + kbu, row < a.n, a.BT, K * (int)a.ldb, j0 + x, H, (int)a.ldb,
+                                  kbu, K / KS / 32, slot);
+  } else {
+    product_chain<TILE, NB>(acc, row < a.n ? a.dA + row * a.ld : nullptr, bcol, a.ldb, kb, ke, slot);
+  }
   park_partials<TILE, NB, KS, NREG, 1>(red, acc, 0, ks, lane);
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
@@ -492,7 +572,7 @@ struct TreeFcFwdArgs {
   int n, H, act;
 };
 
-template <int TILE, int WAVES>
+template <int TILE, int WAVES, bool EXACT>
 __global__ __launch_bounds__(WAVES * 64) void treefc_round_fwd_kernel(TreeFcFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -532,8 +612,16 @@ __global__ __launch_bounds__(WAVES * 64) void treefc_round_fwd_kernel(TreeFcFwdA
   for (int r = 0; r < NR; r++) acc[0][r] = 0.f;
   const float *bl[NP] = {a.W + j0 + x};
   const float *br[NP] = {a.W + (long)H * H + j0 + x};
-  product_chain<TILE, NP>(acc, cl >= 0 ? a.pool + (long)cl * H : nullptr, bl, H, kb, ke, slot);
-  product_chain<TILE, NP>(acc, cr >= 0 ? a.pool + (long)cr * H : nullptr, br, H, kb, ke, slot);
+  if constexpr (EXACT) {
+    const int kbu = __builtin_amdgcn_readfirstlane(ks) * (H / KS);
+    product_chain_exact<TILE, NP>(acc, a.pool + (long)(cl >= 0 ? cl : 0) * H + kbu, cl >= 0, a.W, 2 * H * H, j0 + x, 0, H, kbu,
+                                  H / KS / 32, slot);
+    product_chain_exact<TILE, NP>(acc, a.pool + (long)(cr >= 0 ? cr : 0) * H + kbu, cr >= 0, a.W, 2 * H * H, j0 + x, 0, H, H + kbu,
+                                  H / KS / 32, slot);
+  } else {
+    product_chain<TILE, NP>(acc, cl >= 0 ? a.pool + (long)cl * H : nullptr, bl, H, kb, ke, slot);
+    product_chain<TILE, NP>(acc, cr >= 0 ? a.pool + (long)cr * H : nullptr, br, H, kb, ke, slot);
+  }
   float ehl[EPT], ehr[EPT];
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
@@ -617,14 +705,23 @@ __global__ void treefc_round_bwd_kernel(TreeFcBwdArgs a) {
   stw<W>(a.dz + (long)r * H + j, o);
 }
 
-template <typename KernelArgs, typename K16x8, typename K16x4, typename K32x8>
-static void launch_round(const KernelArgs &a, int n, int H, hipStream_t st, K16x8 k168, K16x4 k164, K32x8 k328) {
-  const RoundPlan p = plan_round(n);
-  dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
-  if (p.tile == 16 && p.waves == 8) launch(k168, grid, 512, 0, st, a);
-  else if (p.tile == 16) launch(k164, grid, 256, 0, st, a);
-  else launch(k328, grid, 512, 0, st, a);
-}
+// KERNEL<tile, wavefronts, exact, ...> for a round of n rows whose products run over K rows of a
+// B matrix of BFLOATS floats
+#define CAVS_LAUNCH_ROUND(KERNEL, a, n, H, K, BFLOATS, st, ...)                                                  \
+  do {                                                                                                           \
+    const RoundPlan p_ = plan_round(n);                                                                          \
+    const dim3 grid_((H) / p_.tile, ((n) + p_.tile - 1) / p_.tile);                                              \
+    const bool ex_ = chain_exact(K, p_.waves, BFLOATS);                                                          \
+    if (p_.tile == 16 && p_.waves == 8) {                                                                        \
+      if (ex_) launch(KERNEL<16, 8, true, ##__VA_ARGS__>, grid_, 512, 0, st, a);                                 \
+      else launch(KERNEL<16, 8, false, ##__VA_ARGS__>, grid_, 512, 0, st, a);                                    \
+    } else if (p_.tile == 16) {                                                                                  \
+      if (ex_) launch(KERNEL<16, 4, true, ##__VA_ARGS__>, grid_, 256, 0, st, a);                                 \
+      else launch(KERNEL<16, 4, false, ##__VA_ARGS__>, grid_, 256, 0, st, a);                                    \
+    } else {                                                                                                     \
+      launch(KERNEL<32, 8, false, ##__VA_ARGS__>, grid_, 512, 0, st, a);                                         \
+    }                                                                                                            \
+  } while (0)
 
 template <typename A, typename K4, typename K1>
 static void launch_pointwise(const A &a, int n, int H, bool vec, hipStream_t st, K4 k4, K1 k1) {
@@ -658,7 +755,7 @@ int cavs_lstm_round_fwd(float *pool, const int *child, const int *pair, const fl
   CAVS_REQUIRE(aligned16(pool), "cavs_lstm_round_fwd: pool must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_lstm_round_fwd: graph_out needs out_rows");
   LstmFwdArgs a{pool, child, pair, xW, ld_xw, Wh, bias, G, gates, msg, pool, graph_out, out_rows, n, H};
-  launch_round(a, n, H, as_stream(stream), lstm_round_fwd_kernel<16, 8>, lstm_round_fwd_kernel<16, 4>, lstm_round_fwd_kernel<32, 8>);
+  CAVS_LAUNCH_ROUND(lstm_round_fwd_kernel, a, n, H, H, 4L * H * H, as_stream(stream));
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -700,9 +797,9 @@ int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int
   ChildBwdArgs a{dA, ld, BT, ldb, child, dpool, pool_width, n, H, K, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0};
   hipStream_t st = as_stream(stream);
   if (nchild == 1)
-    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 1, 0>, round_bwd_children_kernel<16, 4, 1, 0>, round_bwd_children_kernel<32, 8, 1, 0>);
+    CAVS_LAUNCH_ROUND(round_bwd_children_kernel, a, n, H, K, (long)K * ldb, st, 1, 0);
   else
-    launch_round(a, n, H, st, round_bwd_children_kernel<16, 8, 2, 0>, round_bwd_children_kernel<16, 4, 2, 0>, round_bwd_children_kernel<32, 8, 2, 0>);
+    CAVS_LAUNCH_ROUND(round_bwd_children_kernel, a, n, H, K, (long)K * ldb, st, 2, 0);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -717,8 +814,7 @@ int cavs_lstm_round_bwd_children_gates(float *da, int ld_da, float *dc, const fl
   CAVS_REQUIRE(da && dc && WhT && child_rows && gates && G && dret && dret_rows, "cavs_lstm_round_bwd_children_gates: null pointer");
   CAVS_REQUIRE(aligned16(da), "cavs_lstm_round_bwd_children_gates: da must be 16-byte aligned");
   ChildBwdArgs a{da + (long)row0 * ld_da, ld_da, WhT, H, child_rows, nullptr, 0, n, H, 4 * H, da, dc, gates, G, nullptr, dret, dret_rows, row0, leaf_rows, 0};
-  launch_round(a, n, H, as_stream(stream), round_bwd_children_kernel<16, 8, 1, 1>, round_bwd_children_kernel<16, 4, 1, 1>,
-               round_bwd_children_kernel<32, 8, 1, 1>);
+  CAVS_LAUNCH_ROUND(round_bwd_children_kernel, a, n, H, 4 * H, 4L * H * H, as_stream(stream), 1, 1);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -742,8 +838,7 @@ int cavs_treefc_round_bwd_children_act(float *dz, const float *WT, const int *ch
   CAVS_REQUIRE(dz && WT && child_rows && h && dret && dret_rows, "cavs_treefc_round_bwd_children_act: null pointer");
   CAVS_REQUIRE(aligned16(dz), "cavs_treefc_round_bwd_children_act: dz must be 16-byte aligned");
   ChildBwdArgs a{dz + (long)row0 * H, H, WT, 2L * H, child_rows, nullptr, 0, n, H, H, dz, nullptr, nullptr, nullptr, h, dret, dret_rows, row0, 0, act};
-  launch_round(a, n, H, as_stream(stream), round_bwd_children_kernel<16, 8, 2, 2>, round_bwd_children_kernel<16, 4, 2, 2>,
-               round_bwd_children_kernel<32, 8, 2, 2>);
+  CAVS_LAUNCH_ROUND(round_bwd_children_kernel, a, n, H, H, 2L * H * H, as_stream(stream), 2, 2);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }
@@ -768,7 +863,7 @@ int cavs_treefc_round_fwd(float *pool, const int *child, const int *pair, const 
   CAVS_REQUIRE(aligned16(pool), "cavs_treefc_round_fwd: pool must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treefc_round_fwd: graph_out needs out_rows");
   TreeFcFwdArgs a{pool, child, pair, W, bias, x, G, msg, pool, graph_out, out_rows, n, H, act};
-  launch_round(a, n, H, as_stream(stream), treefc_round_fwd_kernel<16, 8>, treefc_round_fwd_kernel<16, 4>, treefc_round_fwd_kernel<32, 8>);
+  CAVS_LAUNCH_ROUND(treefc_round_fwd_kernel, a, n, H, H, 2L * H * H, as_stream(stream));
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

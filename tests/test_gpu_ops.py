@@ -553,7 +553,8 @@ def test_reference_elementwise_smoke_values(g):
     np.testing.assert_array_equal(g.host(out), np.array(kat["expect"], np.float32))
 
 
-@pytest.mark.parametrize("n,H", [(1, 32), (16, 64), (17, 32), (33, 96), (64, 64), (65, 32), (130, 64), (600, 64), (300, 512)])
+@pytest.mark.parametrize("n,H", [(1, 32), (16, 64), (17, 32), (33, 96), (64, 64), (65, 32), (130, 64), (600, 64), (300, 512),
+                                 (40, 512), (3, 1024), (100, 128), (90, 256)])
 def test_fused_tree_lstm_rounds(g, oracle, n, H):
     """A whole round in one launch (forward) / two (backward) against the same round
     composed from the oracle's gather, GEMM and gate functions."""
@@ -660,7 +661,8 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     close(g.host(go2), go_l, "leaf graph_out")
 
 
-@pytest.mark.parametrize("L,m,n,H", [(20, 5, 3, 32), (300, 70, 40, 64), (900, 200, 130, 64), (2600, 100, 1100, 32), (1300, 500, 300, 512)])
+@pytest.mark.parametrize("L,m,n,H", [(20, 5, 3, 32), (300, 70, 40, 64), (900, 200, 130, 64), (2600, 100, 1100, 32), (1300, 500, 300, 512),
+                                     (300, 70, 40, 512), (300, 100, 90, 128)])
 def test_backward_rounds_with_the_childrens_gate_gradients_folded_in(g, oracle, L, m, n, H):
     """Three levels over whole-batch slabs (leaves, a middle round, a top round of roots): the
     roots' gate gradients from the row-list launch, then one launch per round that hands d h,
@@ -924,7 +926,9 @@ def test_column_sums_of_permuted_blocks(g, n, bw, perm):
             hip.call("cavs_colsum_blocks", 16, 16, ld, n, bw, nb, (C.c_int * 1)(3), 16, nbytes, 0)
 
 
-@pytest.mark.parametrize("n,H,K,nchild", [(1, 32, 128, 1), (40, 64, 256, 1), (130, 32, 32, 2), (300, 64, 64, 2), (17, 96, 96, 2)])
+@pytest.mark.parametrize("n,H,K,nchild", [(1, 32, 128, 1), (40, 64, 256, 1), (130, 32, 32, 2), (300, 64, 64, 2), (17, 96, 96, 2),
+                                          # k ranges of whole pipeline stages: the loops that fetch B through buffer loads
+                                          (130, 64, 256, 1), (40, 64, 512, 2), (64, 32, 1024, 1), (700, 32, 512, 2)])
 def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
     """dpool[child[b*nchild+p]][0:H) = dA[b] * BT[:, p*H:(p+1)*H): product and Scatter in one launch."""
     r = rng(n + H + K)
@@ -951,7 +955,9 @@ def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
 
 @pytest.mark.parametrize("model,L,m,n,H", [("lstm", 20, 2, 3, 32), ("lstm", 300, 60, 70, 64), ("lstm", 2600, 600, 1100, 32),
                                            ("treefc", 20, 5, 3, 32), ("treefc", 400, 100, 70, 64), ("treefc", 2600, 100, 1100, 32),
-                                           ("treefc", 900, 200, 130, 96)])
+                                           ("treefc", 900, 200, 130, 96),
+                                           # hidden sizes whose k ranges are whole pipeline stages (buffer-load loops)
+                                           ("lstm", 300, 60, 70, 256), ("treefc", 400, 100, 70, 256), ("treefc", 300, 60, 40, 512)])
 def test_chain_and_tree_fc_backward_rounds_with_the_childrens_pointwise_part_folded_in(g, oracle, model, L, m, n, H):
     """The construction of the Tree-LSTM test above for the other two vertex functions: three
     levels over whole-batch slabs, the top rows from the row-list launch, then one launch per
