@@ -36,7 +36,14 @@ struct Mma<16> {
 __device__ inline float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
 __device__ inline float4 zero4() { return make_float4(0.f, 0.f, 0.f, 0.f); }
 __device__ inline float elem(const float4 &v, int c) { return c == 0 ? v.x : c == 1 ? v.y : c == 2 ? v.z : v.w; }
-__device__ inline float sigm_r(float x) { return 1.f / (1.f + expf(-x)); }
+// The gates of the fused round kernels: exp through v_exp_f32 and the reciprocal through
+// v_rcp_f32 (1 ulp each; 4 and 6 instructions against the 26 and 28 of 1.f / (1.f + expf(-x)) and
+// tanhf, of which a thread's epilogue has six).  Saturation comes out right without special
+// cases: exp overflows to inf, whose reciprocal is 0, and underflows to 0.  tanh_r is accurate to
+// 1e-7 absolute; near zero that is a large relative error of a tiny number.
+__device__ inline float exp_r(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ inline float sigm_r(float x) { return __builtin_amdgcn_rcpf(1.f + exp_r(-x)); }
+__device__ inline float tanh_r(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + exp_r(2.f * x)); }
 
 
 // Parks the per-wavefront partial tiles of NP products in LDS as

@@ -270,11 +270,11 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     // same association as the separate gate kernel: (x*W + h*U) + bias
     const float i = sigm_r((ep.xw[0] + v[0]) + ep.bias[0]);
     const float o = sigm_r((ep.xw[1] + v[1]) + ep.bias[3]);
-    const float u = tanhf((ep.xw[2] + v[2]) + ep.bias[2]);
+    const float u = tanh_r((ep.xw[2] + v[2]) + ep.bias[2]);
     const float f_l = sigm_r((ep.xw[3] + v[3]) + ep.bias[1]);
     const float f_r = sigm_r((ep.xw[3] + v[4]) + ep.bias[1]);
     const float c = (i * u + f_l * ep.cl) + f_r * ep.cr;
-    const float tc = tanhf(c);
+    const float tc = tanh_r(c);
     const float h = o * tc;
     float *g = a.gates + (long)b * 6 * H + j;
     g[0] = i; g[H] = o; g[2 * H] = u; g[3 * H] = f_l; g[4 * H] = f_r; g[5 * H] = tc;
@@ -321,10 +321,10 @@ __global__ void treelstm_round_leaves_fwd_kernel(RoundLeavesArgs a) {
     // same association as with children: (x*W + 0) + bias
     const float i = sigm_r((xw[k] + 0.f) + a.bias[j + k]);
     const float o = sigm_r((xw[H + k] + 0.f) + a.bias[3 * H + j + k]);
-    const float u = tanhf((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
+    const float u = tanh_r((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
     const float f = sigm_r((xw[3 * H + k] + 0.f) + a.bias[H + j + k]);
     const float c = (i * u + f * 0.f) + f * 0.f;
-    const float tc = tanhf(c);
+    const float tc = tanh_r(c);
     gi[k] = i; go[k] = o; gu[k] = u; gf[k] = f; gtc[k] = tc; mh[k] = o * tc; mc[k] = c;
   }
   auto st = [](float *p, const float (&v)[W]) {

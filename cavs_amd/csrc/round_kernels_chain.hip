@@ -259,10 +259,10 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs 
     // same association as the separate path: (x*W + h*W') + bias
     const float i = sigm_r((exw[q][0] + v[0]) + ebias[q][0]);
     const float f = sigm_r((exw[q][1] + v[1]) + ebias[q][1]);
-    const float u = tanhf((exw[q][2] + v[2]) + ebias[q][2]);
+    const float u = tanh_r((exw[q][2] + v[2]) + ebias[q][2]);
     const float o = sigm_r((exw[q][3] + v[3]) + ebias[q][3]);
     const float c = i * u + f * ecprev[q];
-    const float tc = tanhf(c);
+    const float tc = tanh_r(c);
     const float h = o * tc;
     float *g = a.gates + (long)b * 5 * H + j;
     g[0] = i; g[H] = f; g[2 * H] = u; g[3 * H] = o; g[4 * H] = tc;
@@ -301,10 +301,10 @@ __global__ void lstm_round_leaves_fwd_kernel(LstmLeavesArgs a) {
   for (int k = 0; k < W; k++) {
     const float i = sigm_r((xw[k] + 0.f) + a.bias[j + k]);
     const float f = sigm_r((xw[H + k] + 0.f) + a.bias[H + j + k]);
-    const float u = tanhf((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
+    const float u = tanh_r((xw[2 * H + k] + 0.f) + a.bias[2 * H + j + k]);
     const float o = sigm_r((xw[3 * H + k] + 0.f) + a.bias[3 * H + j + k]);
     const float c = i * u + f * 0.f;
-    const float tc = tanhf(c);
+    const float tc = tanh_r(c);
     gi[k] = i; gf[k] = f; gu[k] = u; go[k] = o; gtc[k] = tc; mh[k] = o * tc; mc[k] = c;
   }
   float *g = a.gates + (long)r * 5 * H + j;
@@ -638,7 +638,7 @@ __global__ __launch_bounds__(WAVES * 64) void treefc_round_fwd_kernel(TreeFcFwdA
     float t = v[0];
     if (a.bias) t += eb[q];
     if (a.x) t += ex[q];
-    const float h = a.act ? tanhf(t) : (t > 0.f ? t : 0.f);
+    const float h = a.act ? tanh_r(t) : (t > 0.f ? t : 0.f);
     a.msg[(long)b * H + j] = h;
     if (edst[q] >= 0) a.pool_out[(long)edst[q] * H + j] = h;
     if (eout[q] >= 0) a.go[(long)eout[q] * H + j] = h;
@@ -669,7 +669,7 @@ __global__ void treefc_round_leaves_fwd_kernel(TreeFcLeavesArgs a) {
     float t = 0.f;
     if (a.bias) t += a.bias[j + k];
     if (a.x) t += a.x[(long)r * H + j + k];
-    h[k] = a.act ? tanhf(t) : (t > 0.f ? t : 0.f);
+    h[k] = a.act ? tanh_r(t) : (t > 0.f ? t : 0.f);
   }
   stw<W>(a.msg + (long)r * H + j, h);
   if (dst >= 0) stw<W>(a.pool + (long)dst * H + j, h);
