@@ -76,13 +76,16 @@ __global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ 
       mx = fmaxf(mx, z[c]);
     }
     // cavs/backend/op_impl_softmax_entropy_logits_loss.cu:94-140, :212-250
-    float sum = 0.f, zl = 0.f;
+    // every lane repeats this per row: exp through v_exp_f32, one reciprocal for all classes, and
+    // -log(e_label / sum) taken as log(sum) - (z_label - max)
+    float sum = 0.f, zl = 0.f, e[C];
 #pragma unroll
     for (int c = 0; c < C; c++) {
-      sum += expf(z[c] - mx);
+      e[c] = __builtin_amdgcn_exp2f((z[c] - mx) * 1.4426950408889634f);
+      sum += e[c];
       if (c == lab) zl = z[c];
     }
-    if (lane == 0) loss[row] = -logf(expf(zl - mx) / sum);
+    if (lane == 0) loss[row] = __builtin_amdgcn_logf(sum) * 0.6931471805599453f - (zl - mx);
     if (logits) {
 #pragma unroll
       for (int c = 0; c < C; c++)
@@ -90,9 +93,10 @@ __global__ __launch_bounds__(256) void fc_xent_kernel(const float *__restrict__ 
     }
     if (!grad) continue;
     float d[C];
+    const float inv_sum = __builtin_amdgcn_rcpf(sum);
 #pragma unroll
     for (int c = 0; c < C; c++) {
-      const float p = expf(z[c] - mx) / sum;
+      const float p = e[c] * inv_sum;
       d[c] = (c == lab ? p - 1.f : p) * inv_n;
       dbacc[c] += d[c];
     }
