@@ -48,36 +48,51 @@ struct TileLoader {
   static constexpr int KQ = BK / 4;                  // float4 per row of a k-contiguous tile
   static constexpr int PER = BX / 4;                 // float4 per k row otherwise
   float4 reg[NV];
+  // Fixed per thread before the k loop (prepare): where float4 i of this thread sits in the
+  // operand at k = 0, which of its x are inside, and its k relative to the tile's first.  In
+  // the loop only the tile's k advances -- a pointer bump, or a wave-uniform k * ld -- instead
+  // of a 64-bit row * stride product on the vector ALU per load and k-tile.
+  long base[NV];
+  int krel[NV];
+  bool xin[NV][4];
 
-  __device__ inline void load(const float *__restrict__ P, long ld, int x0, int k0, int X,
-                              int Kend, int tid) {
+  __device__ inline void prepare(long ld, int x0, int X, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
-      int gx, gk;
-      long off;
-      bool xin[4], kin[4];
       if constexpr (KC) {
-        gx = x0 + tid / KQ + (kThreads / KQ) * i;
-        gk = k0 + 4 * (tid % KQ);
-        off = (long)gx * ld + gk;
+        const int gx = x0 + tid / KQ + (kThreads / KQ) * i;
+        krel[i] = 4 * (tid % KQ);
+        base[i] = (long)gx * ld + krel[i];
 #pragma unroll
-        for (int c = 0; c < 4; c++) { xin[c] = gx < X; kin[c] = gk + c < Kend; }
+        for (int c = 0; c < 4; c++) xin[i][c] = gx < X;
       } else {
-        gk = k0 + tid / PER + (kThreads / PER) * i;
-        gx = x0 + 4 * (tid % PER);
-        off = (long)gk * ld + gx;
+        const int gx = x0 + 4 * (tid % PER);
+        krel[i] = tid / PER + (kThreads / PER) * i;
+        base[i] = (long)krel[i] * ld + gx;
 #pragma unroll
-        for (int c = 0; c < 4; c++) { xin[c] = gx + c < X; kin[c] = gk < Kend; }
+        for (int c = 0; c < 4; c++) xin[i][c] = gx + c < X;
       }
+    }
+  }
+
+  // the tile whose first k is k0 (wave-uniform)
+  __device__ inline void load(const float *__restrict__ P, long ld, int k0, int Kend) {
+    const float *Pk = KC ? P + k0 : P + (long)k0 * ld;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      bool kin[4];
+#pragma unroll
+      for (int c = 0; c < 4; c++) kin[c] = KC ? (k0 + krel[i] + c < Kend) : (k0 + krel[i] < Kend);
+      const float *q = Pk + base[i];
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
       if constexpr (VEC) {
         // whole float4 in or out (X, K multiples of 4 along the contiguous index)
-        if (xin[0] && kin[0]) v = *reinterpret_cast<const float4 *>(P + off);
+        if (xin[i][0] && kin[0]) v = *reinterpret_cast<const float4 *>(q);
       } else {
-        if (xin[0] && kin[0]) v.x = P[off];
-        if (xin[1] && kin[1]) v.y = P[off + 1];
-        if (xin[2] && kin[2]) v.z = P[off + 2];
-        if (xin[3] && kin[3]) v.w = P[off + 3];
+        if (xin[i][0] && kin[0]) v.x = q[0];
+        if (xin[i][1] && kin[1]) v.y = q[1];
+        if (xin[i][2] && kin[2]) v.z = q[2];
+        if (xin[i][3] && kin[3]) v.w = q[3];
       }
       reg[i] = v;
     }
@@ -127,6 +142,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
 
   TileLoader<BM, BK, !TA, VEC> la;
   TileLoader<BN, BK, TB, VEC> lb;
+  la.prepare(g.lda, m0, g.M, tid);
+  lb.prepare(g.ldb, n0, g.N, tid);
 
   floatx16 acc[TM][TN];
 #pragma unroll
@@ -138,8 +155,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
 
   const int nk = (kend - kbeg + BK - 1) / BK;
   if (nk > 0) {
-    la.load(g.A, g.lda, m0, kbeg, g.M, kend, tid);
-    lb.load(g.B, g.ldb, n0, kbeg, g.N, kend, tid);
+    la.load(g.A, g.lda, kbeg, kend);
+    lb.load(g.B, g.ldb, kbeg, kend);
     la.store(As_, tid);
     lb.store(Bs_, tid);
   }
@@ -148,8 +165,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
   for (int kt = 0; kt < nk; kt++) {
     const int cur = kt & 1;
     if (kt + 1 < nk) {
-      la.load(g.A, g.lda, m0, kbeg + (kt + 1) * BK, g.M, kend, tid);
-      lb.load(g.B, g.ldb, n0, kbeg + (kt + 1) * BK, g.N, kend, tid);
+      la.load(g.A, g.lda, kbeg + (kt + 1) * BK, kend);
+      lb.load(g.B, g.ldb, kbeg + (kt + 1) * BK, kend);
     }
     const float *as = As_ + cur * (BK * LDA), *bs = Bs_ + cur * (BK * LDB);
     // operand fragments of the k-tile: the reads of AHEAD steps are in flight while a step's
