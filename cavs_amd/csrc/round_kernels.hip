@@ -613,12 +613,15 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
 #pragma unroll
     for (int c = 0; c < 4; c++) vb[c] = ((4 * slot + c) * H + j0 + x) * 4;
     const int ksu = __builtin_amdgcn_readfirstlane(ks);
+    // the operands of the children's gate gradients travel under the longer of the two product
+    // groups: with eight wavefronts (a round of a few rows) the second is only two stages
+    if constexpr (WAVES == 8) fetch_kids();
     {  // P0: K = 3H
       const int kb = ksu * (3 * H / KS);
       const float *arow[1] = {px + kb + 4 * slot};
       exact_products<TILE, UG, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, 3 * H / KS / S);
     }
-    fetch_kids();
+    if constexpr (WAVES != 8) fetch_kids();
     {  // P1, P2: K = H, one B operand for both
       const int kb = ksu * (H / KS);
       const float *arow[2] = {pfl + kb + 4 * slot, pfr + kb + 4 * slot};
