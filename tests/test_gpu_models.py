@@ -106,6 +106,19 @@ def test_benchmark_configs_scaled(oracle, name, scale):
     compare(got, want)
 
 
+@pytest.mark.parametrize("name", ["C1", "C2", "C3"])
+def test_benchmark_configs_at_full_size(oracle, name):
+    """The benchmark's own batches at their own widths against the oracle (it needs under a second
+    for these three; C4's 10000-way head and C5 are covered scaled above and through properties
+    below), at the same 1e-4 relative / 1e-5 absolute bar as the small cases."""
+    w = synth.make_workload(name)
+    kw, loss = {}, "softmax"
+    if w["model"] == "treefc":
+        kw, loss = dict(act=1, use_bias=True, use_x=True), "root_sq"
+    got, want = run_both(oracle, w, loss=loss, **kw)
+    compare(got, want)
+
+
 def test_steps_are_repeatable_and_sessions_reusable(oracle):
     """Two different batches through one session (buffers grow, lists are re-uploaded),
     then the first again: identical results, no state leaks between steps."""
