@@ -103,11 +103,18 @@ inline RoundPlan plan_round(int n) {
 // bumped once per k-group.  Nothing in the loop is conditional, so the wait counts of the two
 // stage buffers come out exact and one stage's loads are in flight under the other's MFMAs; the
 // scheduler barriers keep that order (left alone, the compiler sinks every load to its use).
-template <int TILE, int UG, int NA>
+// PACKED (16x16 tiles): B is in the tile-major layout CAVS_TASK_PACK_T writes -- the lane's four k
+// of a k-group are one float4, number slot * 16 + x of the 1 KB block of the k-group and column
+// tile; bpk points at this lane's float4 of the wavefront's first block and b_row_bytes is the
+// distance to the next k-group's block -- so a wavefront's B fragment is one load of a
+// contiguous kilobyte instead of four loads of four 64-byte pieces each (the texture-address
+// unit charges per piece).
+template <int TILE, int UG, int NA, bool PACKED = false>
 __device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float *(&arow)[NA], __amdgpu_buffer_rsrc_t bbuf,
-                                      const int (&vb)[4], int sb, int b_row_bytes, int nst) {
+                                      const int (&vb)[4], int sb, int b_row_bytes, int nst, const float4 *bpk = nullptr) {
   using M = Mma<TILE>;
   constexpr int GK = 4 * M::NSLOT;
+  static_assert(!PACKED || TILE == 16, "the packed layout is for 16x16 tiles");
   struct Frag {
     float4 a[UG][NA];
     float b[UG][4];
@@ -115,14 +122,21 @@ __device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float 
   auto fetch = [&](Frag &f) {
 #pragma unroll
     for (int u = 0; u < UG; u++) {
+      if constexpr (PACKED) {
+        const float4 v = *bpk;
+        bpk = reinterpret_cast<const float4 *>(reinterpret_cast<const char *>(bpk) + b_row_bytes);
 #pragma unroll
-      for (int c = 0; c < 4; c++) f.b[u][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb, 0));
+        for (int c = 0; c < 4; c++) f.b[u][c] = elem(v, c);
+      } else {
+#pragma unroll
+        for (int c = 0; c < 4; c++) f.b[u][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb, 0));
+      }
 #pragma unroll
       for (int i = 0; i < NA; i++) {
         f.a[u][i] = ld4(arow[i]);
         arow[i] += GK;
       }
-      sb += GK * b_row_bytes;
+      if constexpr (!PACKED) sb += GK * b_row_bytes;
     }
   };
   auto multiply = [&](const Frag &f) {

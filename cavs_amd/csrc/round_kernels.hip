@@ -511,7 +511,8 @@ struct RoundBwdChildArgs {
   int row0, leaf_rows;
 };
 
-template <int TILE, int WAVES, bool FOLD, bool EXACT>
+// PACKED (with EXACT, 16x16 tiles): UT is in the tile-major layout of CAVS_TASK_PACK_T.
+template <int TILE, int WAVES, bool FOLD, bool EXACT, bool PACKED = false>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -613,19 +614,29 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
 #pragma unroll
     for (int c = 0; c < 4; c++) vb[c] = ((4 * slot + c) * H + j0 + x) * 4;
     const int ksu = __builtin_amdgcn_readfirstlane(ks);
+    // packed: this lane's float4 in the 1 KB block of k-group 0 and this workgroup's column tile,
+    // and the distance in bytes between the blocks of consecutive k-groups
+    const float4 *lane_pk = reinterpret_cast<const float4 *>(a.UT) + blockIdx.x * 64 + slot * 16 + x;
+    const int gstep = (H / 16) * 1024;
     // the operands of the children's gate gradients travel under the longer of the two product
     // groups: with eight wavefronts (a round of a few rows) the second is only two stages
     if constexpr (WAVES == 8) fetch_kids();
     {  // P0: K = 3H
       const int kb = ksu * (3 * H / KS);
       const float *arow[1] = {px + kb + 4 * slot};
-      exact_products<TILE, UG, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, 3 * H / KS / S);
+      if constexpr (PACKED)
+        exact_products<TILE, UG, 1, true>(&acc[0], arow, tbuf, vb, 0, gstep, 3 * H / KS / S, lane_pk + (kb / 16) * (gstep / 16));
+      else
+        exact_products<TILE, UG, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, 3 * H / KS / S);
     }
     if constexpr (WAVES != 8) fetch_kids();
     {  // P1, P2: K = H, one B operand for both
       const int kb = ksu * (H / KS);
       const float *arow[2] = {pfl + kb + 4 * slot, pfr + kb + 4 * slot};
-      exact_products<TILE, UG, 2>(&acc[1], arow, tbuf, vb, (3 * H * H + kb * H) * 4, H * 4, H / KS / S);
+      if constexpr (PACKED)
+        exact_products<TILE, UG, 2, true>(&acc[1], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + 3 * H * H / 4 + (kb / 16) * (gstep / 16));
+      else
+        exact_products<TILE, UG, 2>(&acc[1], arow, tbuf, vb, (3 * H * H + kb * H) * 4, H * 4, H / KS / S);
     }
   } else {
   {  // P0: K = 3H
@@ -755,6 +766,14 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
     if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = tile[tx][i];
 }
 
+// the packed variants exist for the shapes cavs_round_packed_ok admits: 16x16 tiles, exact stages
+static void launch_bwd_children_packed(const RoundBwdChildArgs &a, hipStream_t st) {
+  const RoundPlan p = plan_round(a.n);
+  dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
+  if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, true, true, true>, grid, 256, 0, st, a);
+  else launch(treelstm_round_bwd_children_kernel<16, 8, true, true, true>, grid, 512, 0, st, a);
+}
+
 template <bool FOLD>
 static void launch_bwd_children(const RoundBwdChildArgs &a, hipStream_t st) {
   const RoundPlan p = plan_round(a.n);
@@ -879,6 +898,31 @@ int cavs_treelstm_round_bwd_children_gates(float *dxW, int ld_dxw, float *dF, fl
   RoundBwdChildArgs a{dxW + (long)row0 * ld_dxw, ld_dxw, dF + 2L * row0 * H, UT, child_rows, nullptr, n, H,
                       dxW, dF, dc, gates, G, dret, dret_rows, row0, leaf_rows};
   launch_bwd_children<true>(a, as_stream(stream));
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_round_packed_ok(int n, int H) {
+  if (n < 0 || !round_shape_ok(H)) return 0;
+  const RoundPlan p = plan_round(n > 0 ? n : 1);
+  return p.tile == 16 && exact_stages(H, p) ? 1 : 0;
+}
+
+int cavs_treelstm_round_bwd_children_gates_packed(float *dxW, int ld_dxw, float *dF, float *dc, const float *UTp,
+                                                  const int *child_rows, const float *gates, const float *G,
+                                                  const float *dret, const int *dret_rows, int row0, int n, int leaf_rows,
+                                                  int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && row0 >= 0 && leaf_rows >= 0 && ld_dxw >= 4 * H && ld_dxw % 4 == 0 && cavs_round_packed_ok(n, H),
+               "cavs_treelstm_round_bwd_children_gates_packed: bad shape row0=%d n=%d leaf_rows=%d H=%d ld=%d (see cavs_round_packed_ok)",
+               row0, n, leaf_rows, H, ld_dxw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(dxW && dF && dc && UTp && child_rows && gates && G && dret && dret_rows,
+               "cavs_treelstm_round_bwd_children_gates_packed: null pointer");
+  CAVS_REQUIRE(aligned16(dxW) && aligned16(dF) && aligned16(UTp),
+               "cavs_treelstm_round_bwd_children_gates_packed: dxW, dF and UTp must be 16-byte aligned");
+  RoundBwdChildArgs a{dxW + (long)row0 * ld_dxw, ld_dxw, dF + 2L * row0 * H, UTp, child_rows, nullptr, n, H,
+                      dxW, dF, dc, gates, G, dret, dret_rows, row0, leaf_rows};
+  launch_bwd_children_packed(a, as_stream(stream));
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

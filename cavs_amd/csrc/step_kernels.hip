@@ -282,6 +282,21 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
         if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = lds.tile[tx][i];
       break;
     }
+    case CAVS_TASK_PACK_T: {
+      // B = p1^T ([K = n1, N = n0]; p1 is [n0, n1] row-major) in the tile-major layout the round
+      // kernels' packed product loops read: for k-group g (16 k) and column tile t (16 columns)
+      // 256 consecutive floats [slot][x][c] hold B[16g + 4 slot + c][16t + x], so that lane
+      // (x, slot) of a wavefront fetches its four k of a k-group as one float4 and the wavefront's
+      // sixty-four float4 are one contiguous kilobyte.  A workgroup moves 16 columns x 64 k.
+      const float *__restrict__ in = static_cast<const float *>(t.p1);
+      float4 *__restrict__ out = static_cast<float4 *>(t.p0);
+      const int N = (int)t.n0, K = (int)t.n1, kc = K / 64;
+      const int tcol = b / kc, k0 = (b % kc) * 64, r = tid >> 4, q = tid & 15;
+      const float4 v = *reinterpret_cast<const float4 *>(in + (long)(16 * tcol + r) * K + k0 + 4 * q);
+      const long g = k0 / 16 + q / 4;
+      out[((g * (N / 16) + tcol) * 4 + (q & 3)) * 16 + r] = v;
+      break;
+    }
     case CAVS_TASK_ZERO_ROWS: {  // p0[int(p1[r] * n1) ...] = 0 for n1 columns, r < n0: one row per workgroup
       float *__restrict__ dtable = static_cast<float *>(t.p0);
       const float *__restrict__ ids = static_cast<const float *>(t.p1);
@@ -433,6 +448,14 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         if (t.n0 == 0 || t.n1 == 0) continue;
         CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1, "cavs_run_tasks: job %d: null or aliased pointer", i);
         blocks = ((t.n0 + 31) / 32) * ((t.n1 + 31) / 32);
+        break;
+      case CAVS_TASK_PACK_T:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 24) && t.n1 < (1 << 24) && t.n0 % 16 == 0 && t.n1 % 64 == 0,
+                     "cavs_run_tasks: job %d: bad shape to pack (rows a multiple of 16, columns of 64)", i);
+        if (t.n0 == 0 || t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1, "cavs_run_tasks: job %d: null or aliased pointer", i);
+        CAVS_REQUIRE(aligned16(t.p0) && aligned16(t.p1), "cavs_run_tasks: job %d: pack needs 16-byte aligned pointers", i);
+        blocks = (t.n0 / 16) * (t.n1 / 64);
         break;
       case CAVS_TASK_ZERO_ROWS:
         CAVS_REQUIRE(t.n0 >= 0 && t.n1 > 0 && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad shape", i);

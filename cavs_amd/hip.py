@@ -29,7 +29,7 @@ class Task(C.Structure):
                 ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P)]
 
 
-TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD = 0, 1, 2, 3, 4, 5
+TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T = 0, 1, 2, 3, 4, 5, 6
 
 
 class GemmDesc(C.Structure):
@@ -91,6 +91,7 @@ _SIGS = {
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children_gates": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_treelstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_bwd_children_gates_packed": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
@@ -120,11 +121,11 @@ _SIGS = {
 _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z,
             "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
             "cavs_clip_grads_workspace": _Z, "cavs_sgemm_group_workspace": _Z, "cavs_fc_softmax_xent_parts": _I,
-            "cavs_colsum_parts": _I}
+            "cavs_colsum_parts": _I, "cavs_round_packed_ok": _I}
 _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I],
             "cavs_fc_softmax_xent_workspace": [_I, _I, _I], "cavs_colsum_blocks_workspace": [_I, _I, _I],
             "cavs_clip_grads_workspace": [_I], "cavs_sgemm_group_workspace": [_I, C.POINTER(GemmDesc)],
-            "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I]}
+            "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I], "cavs_round_packed_ok": [_I, _I]}
 
 EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)
 EW_UNARY = dict(assign=0, neg=1, abs=2, square=3, sigmoid=4, tanh=5, relu=6)

@@ -331,6 +331,17 @@ int cavs_treelstm_round_bwd_children_gates(float *dxW, int ld_dxw, float *dF, fl
                                            const int *child_rows, const float *gates, const float *G,
                                            const float *dret, const int *dret_rows, int row0, int n,
                                            int leaf_rows, int H, void *stream);
+/* The same launch with the transposed weights in the tile-major layout a CAVS_TASK_PACK_T job
+ * writes (UTp = pack(U_iou) [K = 3H, N = H], then pack(U_f) [K = H, N = H] at float 3H*H): a
+ * wavefront's weight fragment of a k-group is then one contiguous kilobyte.  For the shapes
+ * cavs_round_packed_ok(n, H) admits: rounds of at most 1024 vertices whose kernels split H into
+ * whole pipeline stages (H a multiple of 512, or of 128 for rounds above 64 vertices). */
+int cavs_round_packed_ok(int n, int H);
+int cavs_treelstm_round_bwd_children_gates_packed(float *dxW, int ld_dxw, float *dF, float *dc,
+                                                  const float *UTp, const int *child_rows,
+                                                  const float *gates, const float *G, const float *dret,
+                                                  const int *dret_rows, int row0, int n, int leaf_rows,
+                                                  int H, void *stream);
 int cavs_treelstm_bwd_gates_rows(const int *rows, int n, const float *dret, const int *dret_rows,
                                  const float *gates, const float *G, float *dxW, int ld_dxw, float *dF,
                                  float *dc, int leaf_rows, int H, void *stream);
@@ -396,9 +407,13 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *                        permutation.  A gradient that arrives in another block order than its
  *                        parameter's (the gate bias, apps/paper/tree-lstm-cavs.cc:120-123 vs :143-148).
  *                        With P = n2 >> 32 above 1, p1 holds P such rows and the job adds them up first,
- *                        in index order (the chunk sums cavs_colsum_blocks leaves behind). */
+ *                        in index order (the chunk sums cavs_colsum_blocks leaves behind).
+ *   CAVS_TASK_PACK_T     p0 = B = p1^T (p1 [n0, n1] row-major, so B is [K = n1, N = n0]; n0 a multiple of 16,
+ *                        n1 of 64) in the tile-major layout of the packed round entry points: for k-group
+ *                        g (16 k) and column tile t (16 columns), floats [((g * N/16 + t) * 256, +256) hold
+ *                        B[16g + 4s + c][16t + x] at [s][x][c], s < 4, x < 16, c < 4. */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
-       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5 };
+       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6 };
 typedef struct cavs_task {
   int kind;
   float f0;

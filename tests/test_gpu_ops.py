@@ -733,6 +733,65 @@ def test_backward_rounds_with_the_childrens_gate_gradients_folded_in(g, oracle, 
     assert (got_F[: 2 * L] == -3.0).all() and (g.host(dc)[:L] == -3.0).all()
 
 
+def pack_tiles(B):
+    """The tile-major layout of CAVS_TASK_PACK_T, spelled out: B [K, N] -> [K/16][N/16][slot][x][c]."""
+    K, N = B.shape
+    out = np.zeros(K * N, np.float32)
+    g, t, sl, x, c = np.meshgrid(np.arange(K // 16), np.arange(N // 16), np.arange(4), np.arange(16), np.arange(4), indexing="ij")
+    out[((((g * (N // 16) + t) * 4 + sl) * 16 + x) * 4 + c).ravel()] = B[(16 * g + 4 * sl + c).ravel(), (16 * t + x).ravel()]
+    return out
+
+
+@pytest.mark.parametrize("L,m,n,H", [(300, 70, 40, 512), (1300, 500, 300, 512), (300, 100, 90, 128), (40, 9, 5, 1024)])
+def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L, m, n, H):
+    """The pack job against the layout written out in numpy, then the backward launch reading
+    the packed weights against the one reading the plain transposes: same products in the same
+    order, so every output agrees bit for bit."""
+    r = rng(17 * L + n + H)
+    N = L + m + n
+    U = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)
+    Uiou, Uf = U[: 3 * H * H].reshape(H, 3 * H), U[3 * H * H:].reshape(H, H)
+    d_U, UT, UTp = g.devf(U), g.zeros(4 * H * H), g.zeros(4 * H * H, fill=-9.0)
+    T = hip.Task
+    jobs = [T(hip.TASK_TRANSPOSE, 0.0, H, 3 * H, 0, g.P(UT), g.P(d_U), None, None),
+            T(hip.TASK_TRANSPOSE, 0.0, H, H, 0, g.P(UT) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, None, None),
+            T(hip.TASK_PACK_T, 0.0, H, 3 * H, 0, g.P(UTp), g.P(d_U), None, None),
+            T(hip.TASK_PACK_T, 0.0, H, H, 0, g.P(UTp) + 4 * 3 * H * H, g.P(d_U) + 4 * 3 * H * H, None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    got = g.host(UTp)
+    np.testing.assert_array_equal(got[: 3 * H * H], pack_tiles(np.ascontiguousarray(Uiou.T)))
+    np.testing.assert_array_equal(got[3 * H * H:], pack_tiles(np.ascontiguousarray(Uf.T)))
+
+    mid0, top0 = L, L + m
+    order = np.argsort(r.bulk_normal(L)).astype(np.int32)
+    kids = np.full(2 * N, -1, np.int32)
+    kids[2 * mid0: 2 * top0] = order[: 2 * m]
+    top_kids = np.concatenate([np.arange(mid0, top0, dtype=np.int32), order[2 * m: 2 * m + 2 * n - m]])
+    kids[2 * top0:] = top_kids[np.argsort(r.bulk_normal(2 * n))]
+    gates = np.tanh(r.bulk_normal(N * 6 * H).reshape(N, 6 * H)).astype(np.float32)
+    G = (r.bulk_normal(2 * N * 2 * H).reshape(2 * N, 2 * H) * 0.5).astype(np.float32)
+    dret_rows = np.argsort(r.bulk_normal(N))[:N].astype(np.int32)
+    dgo = r.bulk_normal(N * H).reshape(N, H)
+    d_gates, d_G, d_dgo, d_rows, d_kids = g.devf(gates), g.devf(G), g.devf(dgo), g.devi(dret_rows), g.devi(kids)
+    roots = g.devi(np.arange(top0, N, dtype=np.int32))
+    outs = []
+    for entry, W in (("cavs_treelstm_round_bwd_children_gates", UT), ("cavs_treelstm_round_bwd_children_gates_packed", UTp)):
+        dxW, dF, dc = g.zeros(N, 4 * H, fill=-3.0), g.zeros(2 * N, H, fill=-3.0), g.zeros(N, H, fill=-3.0)
+        g.call("cavs_treelstm_bwd_gates_rows", g.P(roots), n, g.P(d_dgo), g.P(d_rows), g.P(d_gates), g.P(d_G), g.P(dxW), 4 * H,
+               g.P(dF), g.P(dc), L, H, g.stream())
+        for lo, cnt in ((top0, n), (mid0, m)):
+            assert hip.lib().cavs_round_packed_ok(cnt, H) == 1
+            g.call(entry, g.P(dxW), 4 * H, g.P(dF), g.P(dc), g.P(W), g.P(d_kids) + 4 * 2 * lo, g.P(d_gates), g.P(d_G), g.P(d_dgo),
+                   g.P(d_rows), lo, cnt, L, H, g.stream())
+        outs.append((g.host(dxW), g.host(dF), g.host(dc)))
+    for a, b, what in zip(outs[0], outs[1], ("dxW", "dF", "dc")):
+        np.testing.assert_array_equal(a, b, err_msg=what)
+    assert (outs[0][0][:L] != -3.0).any()
+    assert hip.lib().cavs_round_packed_ok(40, 96) == 0 and hip.lib().cavs_round_packed_ok(2000, 512) == 0
+    with pytest.raises(hip.CavsError, match="cavs_round_packed_ok"):
+        hip.call("cavs_treelstm_round_bwd_children_gates_packed", 16, 4 * 96, 16, 16, 16, 16, 16, 16, 16, 16, 0, 5, 0, 96, 0)
+
+
 def test_fused_round_entry_points_reject_bad_shapes():
     with pytest.raises(hip.CavsError, match="multiple of 32"):
         hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 0, 0, 5, 24, 0)
