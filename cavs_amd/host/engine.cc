@@ -619,10 +619,15 @@ void Engine::treelstm_backward() {
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
+  // one launch per round when the message flow is a forest (below); then, if every such launch has
+  // a packed variant, the transposed weights are written tile-major instead of plain
+  bool packed = forest_;
+  for (const Round &r : sched_.rounds)
+    if (!leaf_round(r) && !cavs_round_packed_ok(r.n, H)) packed = false;
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
-    backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr},
-                       {CAVS_TASK_TRANSPOSE, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H,
-                        nullptr, nullptr}},
+    const int kind = packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE;
+    backward_prologue({{kind, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr},
+                       {kind, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H, nullptr, nullptr}},
                       true);
   } else {
     backward_prologue({}, true);
@@ -641,9 +646,9 @@ void Engine::treelstm_backward() {
     if (folded) {
       c_gather_rows_ += r.n;
       if (leaf_round(r)) continue;
-      CAVS_TIMED(K_ROUND, cavs_treelstm_round_bwd_children_gates(dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_ + 2 * off,
-                                                                 gates_.get(), G_.get(), d_dgo_, d_t2j_, (int)off, r.n,
-                                                                 sched_.leaf_prefix, H, stream_));
+      CAVS_TIMED(K_ROUND, (packed ? cavs_treelstm_round_bwd_children_gates_packed : cavs_treelstm_round_bwd_children_gates)(
+                              dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_ + 2 * off, gates_.get(), G_.get(), d_dgo_,
+                              d_t2j_, (int)off, r.n, sched_.leaf_prefix, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
       c_scatter_rows_ += 2.0 * r.n;
       c_launches_ += 1;
