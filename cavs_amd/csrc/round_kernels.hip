@@ -30,6 +30,7 @@ struct RoundFwdArgs {
   const float *xW;     // [n, 4H] (ld_xw) blocks [i|o|u|f]
   long ld_xw;
   const float *U;      // [H, 3H] blocks [i|o|u], then [H, H] (forget gate)
+  const float *Upk;    // PACKED: the same two matrices tile-major (a CAVS_TASK_SGD_PACK job writes them)
   const float *bias;   // [4H] blocks [i|f|u|o]
   float *G;            // [2n, 2H] gathered children (saved for backward)
   float *hlr;          // [n, H] h_l + h_r (saved for the weight gradient)
@@ -48,8 +49,12 @@ struct RoundFwdArgs {
 // row * stride products otherwise cost as much time as the MFMAs), the rows of A through
 // per-lane pointers that are bumped once per k-group, and the wait counts of the two stage
 // buffers come out exact, so the loads of one stage are in flight under the MFMAs of the other.
-template <int TILE, int WAVES, bool EXACT>
+// PACKED: the loop reads the weights from the tile-major copy, one float4 per lane, gate and
+// k-group -- a wavefront's fragment is one contiguous kilobyte instead of four 64-byte pieces per
+// dword load (the texture-address unit charges per piece).
+template <int TILE, int WAVES, bool EXACT, bool PACKED = false>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
+  static_assert(!PACKED || (EXACT && TILE == 16), "the packed layout is for the exact loops over 16x16 tiles");
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
   constexpr int RT = 1, kRoundThreads = WAVES * 64;
@@ -203,20 +208,39 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     const int kbu = __builtin_amdgcn_readfirstlane(kb), nst = __builtin_amdgcn_readfirstlane((ke - kb) / S);
     int sio = (kbu + S) * 3 * H * 4, sf = (3 * H * H + (kbu + S) * H) * 4;  // scalar byte offsets of the next k-group
     const float *al = pl + kb + S + 4 * slot, *ar = pr + kb + S + 4 * slot;
+    // PACKED: float4 (slot, x) of tile (k-group, column tile); gates i, o, u are column tiles
+    // H/16 apart in the [H, 3H] matrix's packing, the forget gate's matrix follows it
+    const int kg1 = (kb + S) / GK;
+    const float4 *pio = reinterpret_cast<const float4 *>(a.Upk) + ((long)kg1 * (3 * H / 16) + blockIdx.x) * 64 + slot * 16 + x;
+    const float4 *pf = reinterpret_cast<const float4 *>(a.Upk) + 3L * H * H / 4 + ((long)kg1 * (H / 16) + blockIdx.x) * 64 + slot * 16 + x;
+    const int gate4 = H * 4;  // float4 between the gates' column tiles
     auto xfetch = [&](Frag &f) {
 #pragma unroll
       for (int u = 0; u < UG; u++) {
+        if constexpr (PACKED) {
+          const float4 bi = pio[0], bo = pio[gate4], bu = pio[2 * gate4], bf = *pf;
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-          f.b[u][0][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio, 0));
-          f.b[u][1][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 4, 0));
-          f.b[u][2][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 8, 0));
-          f.b[u][3][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vf[c], sf, 0));
+          for (int c = 0; c < 4; c++) {
+            f.b[u][0][c] = elem(bi, c);
+            f.b[u][1][c] = elem(bo, c);
+            f.b[u][2][c] = elem(bu, c);
+            f.b[u][3][c] = elem(bf, c);
+          }
+          pio += 3 * gate4;
+          pf += gate4;
+        } else {
+#pragma unroll
+          for (int c = 0; c < 4; c++) {
+            f.b[u][0][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio, 0));
+            f.b[u][1][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 4, 0));
+            f.b[u][2][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio + H * 8, 0));
+            f.b[u][3][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vf[c], sf, 0));
+          }
+          sio += GK * 3 * H * 4;
+          sf += GK * H * 4;
         }
         f.hl[u] = ld4(al);
         f.hr[u] = ld4(ar);
-        sio += GK * 3 * H * 4;
-        sf += GK * H * 4;
         al += GK;
         ar += GK;
       }
@@ -807,7 +831,7 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   CAVS_REQUIRE(pool && child && pair && xW && U && bias && G && hlr && gates, "cavs_treelstm_round_fwd: null pointer");
   CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd: graph_out needs out_rows");
-  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
+  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, nullptr, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
   const RoundPlan p = plan_round(n);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
@@ -823,6 +847,25 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   } else {
     launch(treelstm_round_fwd_kernel<32, 8, false>, grid, 512, 0, st, a);
   }
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                                   const float *U, const float *Upk, const float *bias, float *G, float *hlr, float *gates,
+                                   float *msg, float *graph_out, const int *out_rows, int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && ld_xw >= 4 * H && ld_xw % 4 == 0 && cavs_round_packed_ok(n, H),
+               "cavs_treelstm_round_fwd_packed: bad shape n=%d H=%d ld_xw=%d (see cavs_round_packed_ok)", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && child && pair && xW && U && Upk && bias && G && hlr && gates, "cavs_treelstm_round_fwd_packed: null pointer");
+  CAVS_REQUIRE(aligned16(pool) && aligned16(U) && aligned16(Upk), "cavs_treelstm_round_fwd_packed: pool, U and Upk must be 16-byte aligned");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd_packed: graph_out needs out_rows");
+  RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, Upk, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
+  const RoundPlan p = plan_round(n);
+  dim3 grid(H / 16, (n + 15) / 16);
+  hipStream_t st = as_stream(stream);
+  if (p.waves == 4) launch(treelstm_round_fwd_kernel<16, 4, true, true>, grid, 256, 0, st, a);
+  else launch(treelstm_round_fwd_kernel<16, 8, true, true>, grid, 512, 0, st, a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -262,6 +262,7 @@ struct TaskList {
 __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
   __shared__ union {
     float tile[32][33];
+    float pk[16][65];
     EmbedSgdLds sgd;
     float sums[4][64];
   } lds;
@@ -295,6 +296,28 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
       const float4 v = *reinterpret_cast<const float4 *>(in + (long)(16 * tcol + r) * K + k0 + 4 * q);
       const long g = k0 / 16 + q / 4;
       out[((g * (N / 16) + tcol) * 4 + (q & 3)) * 16 + r] = v;
+      break;
+    }
+    case CAVS_TASK_SGD_PACK: {
+      // B = p1 ([K = n0, N = n1] row-major) after p1 -= f0 * p2 (if p2 is given), packed tile-major
+      // into p0 as above.  A workgroup moves one k-group x 64 columns through LDS.
+      float *__restrict__ w = static_cast<float *>(t.p1);
+      const float *__restrict__ g = static_cast<const float *>(t.p2);
+      float4 *__restrict__ out = static_cast<float4 *>(t.p0);
+      const int N = (int)t.n1, nc = N / 64;
+      const int kg = b / nc, cb = b % nc, kk = tid >> 4, q = tid & 15;
+      const long at = (long)(16 * kg + kk) * N + 64 * cb + 4 * q;
+      float4 v = *reinterpret_cast<const float4 *>(w + at);
+      if (g) {
+        const float4 d = *reinterpret_cast<const float4 *>(g + at);
+        v.x -= t.f0 * d.x; v.y -= t.f0 * d.y; v.z -= t.f0 * d.z; v.w -= t.f0 * d.w;
+        *reinterpret_cast<float4 *>(w + at) = v;
+      }
+      lds.pk[kk][4 * q] = v.x; lds.pk[kk][4 * q + 1] = v.y; lds.pk[kk][4 * q + 2] = v.z; lds.pk[kk][4 * q + 3] = v.w;
+      __syncthreads();
+      const int tt = tid >> 6, slot = (tid >> 4) & 3, x = tid & 15, col = 16 * tt + x;
+      out[(((long)kg * (N / 16) + 4 * cb + tt) * 4 + slot) * 16 + x] =
+          make_float4(lds.pk[4 * slot][col], lds.pk[4 * slot + 1][col], lds.pk[4 * slot + 2][col], lds.pk[4 * slot + 3][col]);
       break;
     }
     case CAVS_TASK_ZERO_ROWS: {  // p0[int(p1[r] * n1) ...] = 0 for n1 columns, r < n0: one row per workgroup
@@ -455,6 +478,14 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         if (t.n0 == 0 || t.n1 == 0) continue;
         CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1, "cavs_run_tasks: job %d: null or aliased pointer", i);
         CAVS_REQUIRE(aligned16(t.p0) && aligned16(t.p1), "cavs_run_tasks: job %d: pack needs 16-byte aligned pointers", i);
+        blocks = (t.n0 / 16) * (t.n1 / 64);
+        break;
+      case CAVS_TASK_SGD_PACK:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 24) && t.n1 < (1 << 24) && t.n0 % 16 == 0 && t.n1 % 64 == 0,
+                     "cavs_run_tasks: job %d: bad shape to pack (rows a multiple of 16, columns of 64)", i);
+        if (t.n0 == 0 || t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1 && t.p0 != t.p2, "cavs_run_tasks: job %d: null or aliased pointer", i);
+        CAVS_REQUIRE(aligned16(t.p0) && aligned16(t.p1) && aligned16(t.p2), "cavs_run_tasks: job %d: pack needs 16-byte aligned pointers", i);
         blocks = (t.n0 / 16) * (t.n1 / 64);
         break;
       case CAVS_TASK_ZERO_ROWS:

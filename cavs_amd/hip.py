@@ -29,7 +29,7 @@ class Task(C.Structure):
                 ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P)]
 
 
-TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T = 0, 1, 2, 3, 4, 5, 6
+TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T, TASK_SGD_PACK = 0, 1, 2, 3, 4, 5, 6, 7
 
 
 class GemmDesc(C.Structure):
@@ -86,6 +86,7 @@ _SIGS = {
     "cavs_treefc_fwd": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treefc_bwd": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treelstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_round_fwd_packed": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children": [_P, _I, _P, _P, _P, _P, _I, _I, _P],

@@ -96,6 +96,7 @@ void Engine::bind_param(const std::string &name, float *w, float *g) {
   if (!w) fail(CAVS_EINVAL, "bind_param('" + name + "'): null weight pointer");
   p.w = w;
   p.g = g ? g : p.own_g.get();
+  upk_valid_ = false;
 }
 
 void Engine::set_param(const std::string &name, const float *host, size_t n) {
@@ -104,6 +105,7 @@ void Engine::set_param(const std::string &name, const float *host, size_t n) {
     fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
   check(cavs_memcpy_h2d(p.w, host, n * 4, stream_));
   check(cavs_stream_sync(stream_));
+  upk_valid_ = false;
 }
 
 void Engine::get_param(const std::string &name, float *host, size_t n, bool grad) {
@@ -267,6 +269,8 @@ void Engine::reserve_edges() {
     R(r_z_, rc * H);
   }
   if (fused_rows() > 0) R(UT_, (size_t)(cfg_.model == CAVS_MODEL_TREEFC ? 2 : 4) * H * H);
+  if (fused_rows() > 0 && cfg_.model == CAVS_MODEL_TREELSTM && (cavs_round_packed_ok(1, H) || cavs_round_packed_ok(65, H)))
+    R(Upk_, (size_t)4 * H * H);
   if (cfg_.model == CAVS_MODEL_TREELSTM) {
     R(hlr_, cap * H);
     R(dF_, cap * 2 * H);
@@ -523,6 +527,13 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
           tasks.push_back({CAVS_TASK_EMBED_SGD, lr, N, E, ++emb_epoch_, p.w, p.g, xs_prev_.get(), emb_stamp_.get()});
           continue;
         }
+        if (kv.first == "U" && Upk_.capacity() > 0) {  // the update and the packed copy of the next forward pass
+          const long long H = cfg_.H;
+          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, 3 * H, 0, Upk_.get(), p.w, p.g, nullptr});
+          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, H, 0, Upk_.at((size_t)3 * H * H), p.w + 3 * H * H, p.g + 3 * H * H, nullptr});
+          upk_valid_ = p.w == p.own_w.get();
+          continue;
+        }
         tasks.push_back({CAVS_TASK_SGD, lr, (long long)p.n, 0, 0, p.w, p.g, nullptr, nullptr});
       }
       check(cavs_run_tasks((int)tasks.size(), tasks.data(), stream_));
@@ -557,6 +568,18 @@ int Engine::fused_rows() const {
 void Engine::treelstm_forward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w, *Bv = param("Bv").w;
+  const int fused = fused_rows();
+  bool any_packed = false;
+  if (Upk_.capacity() > 0)
+    for (const Round &r : sched_.rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_round_packed_ok(r.n, H);
+  if (any_packed && !upk_valid_) {  // U was written by somebody else since the last update here
+    cavs_task pack[2] = {{CAVS_TASK_SGD_PACK, 0.f, H, 3 * H, 0, Upk_.get(), const_cast<float *>(U), nullptr, nullptr},
+                         {CAVS_TASK_SGD_PACK, 0.f, H, H, 0, Upk_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H, nullptr,
+                          nullptr}};
+    check(cavs_run_tasks(2, pack, stream_));
+    c_launches_ += 1;
+    upk_valid_ = U == param("U").own_w.get();
+  }
   check(cavs_embed_pull_fwd(e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, E, e_.get(), ld_e_, W, 4 * H, 0.f, xW_.get(), 4 * H);
@@ -564,7 +587,6 @@ void Engine::treelstm_forward() {
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
   }
-  const int fused = fused_rows();
   // when every round runs fused, Push + FunctionPopRet ride along in the rounds' epilogues
   out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
@@ -584,9 +606,14 @@ void Engine::treelstm_forward() {
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
     } else if (r.n <= fused) {
       // Gather, both recurrent products, the gates and Scatter in one launch
-      CAVS_TIMED(K_ROUND, cavs_treelstm_round_fwd(pool_.get(), d_child_ + 2 * off, d_pair_ + off, xW_.at(off * 4 * H), 4 * H, U, Bv,
-                                                  G_.at(2 * off * 2 * H), hlr_.at(off * H), gates_.at(off * 6 * H), msg, go,
-                                                  d_t2j_ + off, r.n, H, stream_));
+      if (any_packed && cavs_round_packed_ok(r.n, H))
+        CAVS_TIMED(K_ROUND, cavs_treelstm_round_fwd_packed(pool_.get(), d_child_ + 2 * off, d_pair_ + off, xW_.at(off * 4 * H), 4 * H, U,
+                                                           Upk_.get(), Bv, G_.at(2 * off * 2 * H), hlr_.at(off * H),
+                                                           gates_.at(off * 6 * H), msg, go, d_t2j_ + off, r.n, H, stream_));
+      else
+        CAVS_TIMED(K_ROUND, cavs_treelstm_round_fwd(pool_.get(), d_child_ + 2 * off, d_pair_ + off, xW_.at(off * 4 * H), 4 * H, U, Bv,
+                                                    G_.at(2 * off * 2 * H), hlr_.at(off * H), gates_.at(off * 6 * H), msg, go,
+                                                    d_t2j_ + off, r.n, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
       c_gather_rows_ += 2.0 * r.n;
       c_scatter_rows_ += r.n;

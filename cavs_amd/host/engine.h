@@ -182,6 +182,10 @@ class Engine {
   DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
+  // Tree-LSTM: U tile-major for the packed forward rounds.  Written by the job that applies U's
+  // SGD update; current while nobody else has written U since (set_param, a caller's own tensor).
+  DeviceArray<float> Upk_;
+  bool upk_valid_ = false;
   // rounds of at most this many rows run as fused launches (0: none)
   int fused_rows() const;
 

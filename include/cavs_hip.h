@@ -300,6 +300,14 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
                             int ld_xw, const float *U, const float *bias, float *G, float *hlr,
                             float *gates, float *msg, float *graph_out, const int *out_rows, int n,
                             int H, void *stream);
+/* cavs_treelstm_round_fwd with the loop's weights read from Upk, the tile-major copy a
+ * CAVS_TASK_SGD_PACK job writes (pack(U_iou) [K = H, N = 3H], then pack(U_f) [K = H, N = H] at float
+ * 3H*H); U is still read for the first k-groups.  Same results bit for bit; for the shapes
+ * cavs_round_packed_ok(n, H) admits. */
+int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                                   const float *U, const float *Upk, const float *bias, float *G, float *hlr,
+                                   float *gates, float *msg, float *graph_out, const int *out_rows, int n, int H,
+                                   void *stream);
 /* The same for a round of leaves (no children: gates of x*W + bias only). */
 int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw,
                                    const float *bias, float *gates, float *msg, float *graph_out,
@@ -411,9 +419,13 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *   CAVS_TASK_PACK_T     p0 = B = p1^T (p1 [n0, n1] row-major, so B is [K = n1, N = n0]; n0 a multiple of 16,
  *                        n1 of 64) in the tile-major layout of the packed round entry points: for k-group
  *                        g (16 k) and column tile t (16 columns), floats [((g * N/16 + t) * 256, +256) hold
- *                        B[16g + 4s + c][16t + x] at [s][x][c], s < 4, x < 16, c < 4. */
+ *                        B[16g + 4s + c][16t + x] at [s][x][c], s < 4, x < 16, c < 4.
+ *   CAVS_TASK_SGD_PACK   p1[i] -= f0 * p2[i] (skipped when p2 is null), then p0 = B = p1 ([K = n0, N = n1]
+ *                        row-major; n0 a multiple of 16, n1 of 64) in the same tile-major layout: the
+ *                        parameter update (cavs/backend/op_impl_sgd.cu) and the packed copy the next
+ *                        forward pass reads, in one pass over the weights. */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
-       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6 };
+       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6, CAVS_TASK_SGD_PACK = 7 };
 typedef struct cavs_task {
   int kind;
   float f0;

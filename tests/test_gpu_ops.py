@@ -792,6 +792,63 @@ def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L
         hip.call("cavs_treelstm_round_bwd_children_gates_packed", 16, 4 * 96, 16, 16, 16, 16, 16, 16, 16, 16, 0, 5, 0, 96, 0)
 
 
+@pytest.mark.parametrize("n,H", [(40, 512), (300, 512), (1000, 512), (90, 128), (5, 1024)])
+def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
+    """The update-and-pack job against w - lr * g and the layout written out in numpy, then the
+    forward launch reading the packed weights against the one reading the plain ones."""
+    r = rng(29 * n + H)
+    U = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)
+    dU = r.bulk_normal(4 * H * H)
+    lr = np.float32(0.125)
+    d_U, d_plain, d_dU, Upk = g.devf(U), g.devf(U), g.devf(dU), g.zeros(4 * H * H, fill=-9.0)
+    T = hip.Task
+    at = 4 * 3 * H * H
+    jobs = [T(hip.TASK_SGD_PACK, lr, H, 3 * H, 0, g.P(Upk), g.P(d_U), g.P(d_dU), None),
+            T(hip.TASK_SGD_PACK, lr, H, H, 0, g.P(Upk) + at, g.P(d_U) + at, g.P(d_dU) + at, None),
+            T(hip.TASK_SGD, lr, 4 * H * H, 0, 0, g.P(d_plain), g.P(d_dU), None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    U1 = g.host(d_U)
+    np.testing.assert_array_equal(U1, g.host(d_plain))           # the same update as the plain job's
+    close(U1, U - lr * dU, "updated weights")
+    got = g.host(Upk)
+    np.testing.assert_array_equal(got[: 3 * H * H], pack_tiles(U1[: 3 * H * H].reshape(H, 3 * H)))
+    np.testing.assert_array_equal(got[3 * H * H:], pack_tiles(U1[3 * H * H:].reshape(H, H)))
+    # without a gradient: the pack alone, the weights untouched
+    again = g.zeros(4 * H * H, fill=-9.0)
+    jobs = [T(hip.TASK_SGD_PACK, lr, H, 3 * H, 0, g.P(again), g.P(d_U), None, None),
+            T(hip.TASK_SGD_PACK, lr, H, H, 0, g.P(again) + at, g.P(d_U) + at, None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    np.testing.assert_array_equal(g.host(again), got)
+    np.testing.assert_array_equal(g.host(d_U), U1)
+
+    P_rows = 2 * n + 5
+    pool = (r.bulk_normal((P_rows + n) * 2 * H).reshape(P_rows + n, 2 * H) * 0.5).astype(np.float32)
+    child = np.argsort(r.bulk_normal(P_rows))[: 2 * n].astype(np.int32)
+    pair = (P_rows + np.arange(n)).astype(np.int32)
+    child[3] = -1
+    pair[n - 1] = -1
+    d_child, d_pair = g.devi(child), g.devi(pair)
+    d_xW, d_bias = g.devf(r.bulk_normal(n * 4 * H)), g.devf(r.bulk_normal(4 * H))
+    d_rows = g.devi(np.argsort(r.bulk_normal(n + 3))[:n].astype(np.int32))
+    assert hip.lib().cavs_round_packed_ok(n, H) == 1
+    outs = []
+    for packed in (False, True):
+        d_pool = g.devf(pool)
+        G, hlr, gates, msg, go = g.zeros(2 * n, 2 * H), g.zeros(n, H), g.zeros(n, 6 * H), g.zeros(n, 2 * H), g.zeros(n + 3, H, fill=-7.0)
+        weights = (g.P(d_U), g.P(Upk)) if packed else (g.P(d_U),)
+        g.call("cavs_treelstm_round_fwd_packed" if packed else "cavs_treelstm_round_fwd", g.P(d_pool), g.P(d_child), g.P(d_pair),
+               g.P(d_xW), 4 * H, *weights, g.P(d_bias), g.P(G), g.P(hlr), g.P(gates), g.P(msg), g.P(go), g.P(d_rows), n, H, g.stream())
+        outs.append([g.host(t) for t in (d_pool, G, hlr, gates, msg, go)])
+    for a, b, what in zip(outs[0], outs[1], ("pool", "G", "hlr", "gates", "msg", "graph_out")):
+        np.testing.assert_array_equal(a, b, err_msg=what)
+    assert (outs[0][3] != 0).all()
+    with pytest.raises(hip.CavsError, match="cavs_round_packed_ok"):
+        hip.call("cavs_treelstm_round_fwd_packed", 16, 16, 16, 16, 4 * 96, 16, 16, 16, 16, 16, 16, 0, 0, 0, 5, 96, 0)
+    with pytest.raises(hip.CavsError, match="bad shape to pack"):
+        bad = T(hip.TASK_SGD_PACK, lr, 24, 64, 0, g.P(Upk), g.P(d_U), None, None)
+        g.call("cavs_run_tasks", 1, (T * 1)(bad), g.stream())
+
+
 def test_fused_round_entry_points_reject_bad_shapes():
     with pytest.raises(hip.CavsError, match="multiple of 32"):
         hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 0, 0, 5, 24, 0)
