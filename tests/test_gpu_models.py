@@ -343,6 +343,36 @@ def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     s.close()
 
 
+def test_the_packed_copy_of_the_recurrent_weights_follows_every_writer(oracle):
+    """Tree-LSTM rounds of more than 64 vertices at H=128 read U from its tile-major copy.  The copy
+    is written by the update job; set_param writes U behind its back.  Three steps -- the first packs
+    on demand, the second reads what the first step's update left, the third follows a set_params
+    -- each against the oracle on the parameters the session should hold."""
+    H, E, V, C_ = 128, 16, 37, 5
+    w = small_workload("treelstm", 333, B=70, H=H, E=E, V=V, C=C_, skew=False)
+    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc")
+    p = {k: np.array(w["params"][k], np.float32) for k in names}
+    p["U"] = (p["U"] * np.float32(0.2)).astype(np.float32)
+    s = session.Session("treelstm", H=H, E=E, V=V, C_=C_)
+    assert hip.lib().cavs_round_packed_ok(70, H) == 1
+    s.set_params(p)
+    lr = 0.25
+    for step in range(3):
+        print(f"[case] packed copy step {step}", flush=True)
+        if step == 2:
+            p["U"] = (p["U"][::-1] * np.float32(0.5)).astype(np.float32)
+            s.set_params(dict(U=p["U"]))
+        want = oracle.model_step("treelstm", w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
+        s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
+        close(s.fetch("graph_out"), want["graph_out"], f"graph_out at step {step}", rtol=3e-4, atol=3e-5)
+        got = s.grads()
+        for k in names:
+            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", rtol=3e-4, atol=3e-5)
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    close(s.param("U", p["U"].shape), p["U"], "U after the steps", rtol=3e-4, atol=3e-5)
+    s.close()
+
+
 @pytest.mark.parametrize("kind", ["trees", "tokens"])
 def test_training_step_on_reader_batches(oracle, kind):
     """The text readers (cavs_amd/data.py) feed the session directly: the fixture corpora
