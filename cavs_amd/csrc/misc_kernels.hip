@@ -194,6 +194,55 @@ __global__ __launch_bounds__(256) void softmax_xent_kernel(float *__restrict__ l
   }
 }
 
+// One workgroup per row, the row held in registers between the passes (NV float4 per thread,
+// C <= 1024 NV): the logits are read once and the gradient written once, both as float4 -- an
+// HBM-bound kernel of 8 bytes per element.  Sums run in a fixed order (lane, wavefront).
+template <int NV>
+__global__ __launch_bounds__(256) void softmax_xent_rows_kernel(float *__restrict__ loss, float *__restrict__ dlogits,
+                                                                const float *__restrict__ logits,
+                                                                const float *__restrict__ labels, int C, float inv_n) {
+  __shared__ float part[2][4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, row = blockIdx.x, C4 = C / 4;
+  const float4 *x = reinterpret_cast<const float4 *>(logits + (long)row * C);
+  float4 v[NV];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int k = 0; k < NV; k++) {
+    const int j = tid + 256 * k;
+    v[k] = j < C4 ? x[j] : make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+    mx = fmaxf(fmaxf(mx, fmaxf(v[k].x, v[k].y)), fmaxf(v[k].z, v[k].w));
+  }
+  mx = wave_max(mx);
+  if (lane == 0) part[0][wave] = mx;
+  __syncthreads();
+  mx = fmaxf(fmaxf(part[0][0], part[0][1]), fmaxf(part[0][2], part[0][3]));
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < NV; k++) {  // exp(-inf) = 0 past the end of the row
+    v[k].x = expf(v[k].x - mx); v[k].y = expf(v[k].y - mx); v[k].z = expf(v[k].z - mx); v[k].w = expf(v[k].w - mx);
+    sum += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+  }
+  sum = wave_sum(sum);
+  if (lane == 0) part[1][wave] = sum;
+  __syncthreads();
+  sum = (part[1][0] + part[1][1]) + (part[1][2] + part[1][3]);
+  const int lab = (int)labels[row];
+  if (loss && tid == 0) loss[row] = -logf(expf(logits[(long)row * C + lab] - mx) / sum);
+  if (!dlogits) return;
+  float4 *d = reinterpret_cast<float4 *>(dlogits + (long)row * C);
+#pragma unroll
+  for (int k = 0; k < NV; k++) {
+    const int j = tid + 256 * k;
+    if (j >= C4) continue;
+    float4 p = make_float4(v[k].x / sum, v[k].y / sum, v[k].z / sum, v[k].w / sum);
+    if (lab >> 2 == j) {
+      const int c = lab & 3;
+      (c == 0 ? p.x : c == 1 ? p.y : c == 2 ? p.z : p.w) -= 1.f;
+    }
+    d[j] = make_float4(p.x * inv_n, p.y * inv_n, p.z * inv_n, p.w * inv_n);
+  }
+}
+
 // ------------------------------------------------------------------ elementwise
 __global__ void sgd_kernel(float *__restrict__ w, const float *__restrict__ g, float lr, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -341,7 +390,17 @@ int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const fl
   CAVS_REQUIRE(n >= 0 && C > 0, "cavs_softmax_xent: bad shape n=%d C=%d", n, C);
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(logits && labels, "cavs_softmax_xent: null pointer");
-  launch(softmax_xent_kernel, (n + 3) / 4, 256, 0, as_stream(stream), loss, dlogits, logits, labels, n, C, 1.f / (float)n);
+  const float inv_n = 1.f / (float)n;
+  hipStream_t st = as_stream(stream);
+  // wide rows: a workgroup per row with the row in registers; narrow ones: a wavefront per row
+  if (C >= 512 && C % 4 == 0 && C <= 16384 && aligned16(logits) && (!dlogits || aligned16(dlogits))) {
+    if (C <= 2048) launch(softmax_xent_rows_kernel<2>, n, 256, 0, st, loss, dlogits, logits, labels, C, inv_n);
+    else if (C <= 4096) launch(softmax_xent_rows_kernel<4>, n, 256, 0, st, loss, dlogits, logits, labels, C, inv_n);
+    else if (C <= 10240) launch(softmax_xent_rows_kernel<10>, n, 256, 0, st, loss, dlogits, logits, labels, C, inv_n);
+    else launch(softmax_xent_rows_kernel<16>, n, 256, 0, st, loss, dlogits, logits, labels, C, inv_n);
+  } else {
+    launch(softmax_xent_kernel, (n + 3) / 4, 256, 0, st, loss, dlogits, logits, labels, n, C, inv_n);
+  }
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

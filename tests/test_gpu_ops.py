@@ -400,7 +400,10 @@ def test_embedding(g, oracle, V, E, n):
     close(g.host(dt), want, atol=1e-5 * np.sqrt(n))
 
 
-@pytest.mark.parametrize("n,C_", [(19, 5), (300, 1000), (1, 2), (64, 10000)])
+# (rows of 512 to 16384 classes in whole float4s go a workgroup per row, in four register sizes;
+# the others a wavefront per row)
+@pytest.mark.parametrize("n,C_", [(19, 5), (300, 1000), (1, 2), (64, 10000), (7, 512), (5, 2052), (3, 4100), (4, 12000),
+                                  (3, 16384), (6, 1001), (2, 16388)])
 def test_softmax_xent_bias_sgd(g, oracle, n, C_):
     r = rng(n + C_)
     logits = 3 * r.bulk_normal(n * C_).reshape(n, C_)
