@@ -61,11 +61,17 @@ __device__ inline void product_chain(typename Mma<TILE>::Acc (&acc)[NB], const f
 // row-major matrix `bmat` (`bfloats` floats, row stride ldb); the chain covers its rows
 // [krow, krow + 32 * nst).  a_row is already at this wavefront's first k; a lane without a row
 // passes any readable address and has = false.
-template <int TILE, int NB>
+// PACKED: `bmat` is the same matrix tile-major (a CAVS_TASK_PACK_T / CAVS_TASK_SGD_PACK job
+// writes it): float4 (slot, x) of the 16 x 16 tile (k-group, column tile) holds this lane's four
+// k, so a wavefront's fragment is one contiguous kilobyte.  `ldb` is the matrix's column count.
+template <int TILE, int NB, bool PACKED = false>
 __device__ inline void product_chain_exact(typename Mma<TILE>::Acc (&acc)[NB], const float *a_row, bool has, const float *bmat,
                                            int bfloats, int col, int blk, int ldb, int krow, int nst, int slot) {
   using M = Mma<TILE>;
   constexpr int GK = 4 * M::NSLOT, UG = 2;
+  static_assert(!PACKED || TILE == 16, "the packed layout is for 16x16 tiles");
+  const float4 *bpk = reinterpret_cast<const float4 *>(bmat) + ((long)(krow / 16) * (ldb / 16) + col / 16) * 64 + slot * 16 + (col & 15);
+  const int pstep = blk * 4, gstep = ldb * 4;  // float4 between column blocks, between k-groups
   const __amdgpu_buffer_rsrc_t bbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(bmat), 0, bfloats * 4, 0x00020000);
   int vb[4];
 #pragma unroll
@@ -79,14 +85,24 @@ __device__ inline void product_chain_exact(typename Mma<TILE>::Acc (&acc)[NB], c
   auto fetch = [&](Frag &f) {
 #pragma unroll
     for (int u = 0; u < UG; u++) {
+      if constexpr (PACKED) {
 #pragma unroll
-      for (int p = 0; p < NB; p++)
+        for (int p = 0; p < NB; p++) {
+          const float4 v = bpk[p * pstep];
 #pragma unroll
-        for (int c = 0; c < 4; c++)
-          f.b[u][p][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb + p * blk * 4, 0));
+          for (int c = 0; c < 4; c++) f.b[u][p][c] = elem(v, c);
+        }
+        bpk += gstep;
+      } else {
+#pragma unroll
+        for (int p = 0; p < NB; p++)
+#pragma unroll
+          for (int c = 0; c < 4; c++)
+            f.b[u][p][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(bbuf, vb[c], sb + p * blk * 4, 0));
+        sb += GK * ldb * 4;
+      }
       f.a[u] = ld4(a_row);
       a_row += GK;
-      sb += GK * ldb * 4;
     }
   };
   auto multiply = [&](const Frag &f) {
@@ -190,7 +206,7 @@ struct LstmFwdArgs {
   int n, H;
 };
 
-template <int TILE, int WAVES, bool EXACT>
+template <int TILE, int WAVES, bool EXACT, bool PACKED = false>
 __global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -236,8 +252,8 @@ __global__ __launch_bounds__(WAVES * 64) void lstm_round_fwd_kernel(LstmFwdArgs 
   for (int p = 0; p < NP; p++) bcol[p] = a.Wh + p * H + j0 + x;
   if constexpr (EXACT) {
     const int kbu = __builtin_amdgcn_readfirstlane(ks) * (H / KS);
-    product_chain_exact<TILE, NP>(acc, a.pool + (cp >= 0 ? cp : 0) * H2 + kbu, cp >= 0, a.Wh, 4 * H * H, j0 + x, H, 4 * H, kbu,
-                                  H / KS / 32, slot);
+    product_chain_exact<TILE, NP, PACKED>(acc, a.pool + (cp >= 0 ? cp : 0) * H2 + kbu, cp >= 0, a.Wh, 4 * H * H, j0 + x, H, 4 * H, kbu,
+                                          H / KS / 32, slot);
   } else {
     product_chain<TILE, NP>(acc, cp >= 0 ? a.pool + cp * H2 : nullptr, bcol, H4, kb, ke, slot);
   }
@@ -457,7 +473,7 @@ struct ChildBwdArgs {
   int row0, leaf_rows, act;
 };
 
-template <int TILE, int WAVES, bool EXACT, int NB, int FOLD>
+template <int TILE, int WAVES, bool EXACT, int NB, int FOLD, bool PACKED = false>
 __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwdArgs a) {
   using M = Mma<TILE>;
   using Acc = typename M::Acc;
@@ -523,8 +539,8 @@ __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwd
   }
   if constexpr (EXACT) {
     const int kbu = __builtin_amdgcn_readfirstlane(ks) * (K / KS);
-    product_chain_exact<TILE, NB>(acc, a.dA + (row < a.n ? row : 0) * a.ld + kbu, row < a.n, a.BT, K * (int)a.ldb, j0 + x, H, (int)a.ldb,
-                                  kbu, K / KS / 32, slot);
+    product_chain_exact<TILE, NB, PACKED>(acc, a.dA + (row < a.n ? row : 0) * a.ld + kbu, row < a.n, a.BT, K * (int)a.ldb, j0 + x, H,
+                                          (int)a.ldb, kbu, K / KS / 32, slot);
   } else {
     product_chain<TILE, NB>(acc, row < a.n ? a.dA + row * a.ld : nullptr, bcol, a.ldb, kb, ke, slot);
   }
@@ -760,6 +776,29 @@ int cavs_lstm_round_fwd(float *pool, const int *child, const int *pair, const fl
   return CAVS_OK;
 }
 
+int cavs_lstm_round_packed_ok(int n, int H) {
+  if (n < 0 || !round_shape_ok(H)) return 0;
+  const RoundPlan p = plan_round(n > 0 ? n : 1);
+  return p.tile == 16 && chain_exact(H, p.waves, 4L * H * H) ? 1 : 0;  // K = H forward; K = 4H backward follows
+}
+
+int cavs_lstm_round_fwd_packed(float *pool, const int *child, const int *pair, const float *xW, int ld_xw, const float *Whp,
+                               const float *bias, float *G, float *gates, float *msg, float *graph_out, const int *out_rows,
+                               int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && ld_xw >= 4 * H && cavs_lstm_round_packed_ok(n, H),
+               "cavs_lstm_round_fwd_packed: bad shape n=%d H=%d ld=%d (see cavs_lstm_round_packed_ok)", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(pool && child && pair && xW && Whp && bias && G && gates && msg, "cavs_lstm_round_fwd_packed: null pointer");
+  CAVS_REQUIRE(aligned16(pool) && aligned16(Whp), "cavs_lstm_round_fwd_packed: pool and Whp must be 16-byte aligned");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_lstm_round_fwd_packed: graph_out needs out_rows");
+  LstmFwdArgs a{pool, child, pair, xW, ld_xw, Whp, bias, G, gates, msg, pool, graph_out, out_rows, n, H};
+  const dim3 grid(H / 16, (n + 15) / 16);
+  if (plan_round(n).waves == 8) launch(lstm_round_fwd_kernel<16, 8, true, true>, grid, 512, 0, as_stream(stream), a);
+  else launch(lstm_round_fwd_kernel<16, 4, true, true>, grid, 256, 0, as_stream(stream), a);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
 int cavs_lstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw, const float *bias, float *gates,
                                float *msg, float *graph_out, const int *out_rows, int n, int H, void *stream) {
   CAVS_REQUIRE(n >= 0 && H > 0 && ld_xw >= 4 * H, "cavs_lstm_round_leaves_fwd: bad shape n=%d H=%d ld=%d", n, H, ld_xw);
@@ -815,6 +854,23 @@ int cavs_lstm_round_bwd_children_gates(float *da, int ld_da, float *dc, const fl
   CAVS_REQUIRE(aligned16(da), "cavs_lstm_round_bwd_children_gates: da must be 16-byte aligned");
   ChildBwdArgs a{da + (long)row0 * ld_da, ld_da, WhT, H, child_rows, nullptr, 0, n, H, 4 * H, da, dc, gates, G, nullptr, dret, dret_rows, row0, leaf_rows, 0};
   CAVS_LAUNCH_ROUND(round_bwd_children_kernel, a, n, H, 4 * H, 4L * H * H, as_stream(stream), 1, 1);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_lstm_round_bwd_children_gates_packed(float *da, int ld_da, float *dc, const float *WhTp, const int *child_rows,
+                                              const float *gates, const float *G, const float *dret, const int *dret_rows,
+                                              int row0, int n, int leaf_rows, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && row0 >= 0 && leaf_rows >= 0 && ld_da >= 4 * H && ld_da % 4 == 0 && cavs_lstm_round_packed_ok(n, H),
+               "cavs_lstm_round_bwd_children_gates_packed: bad shape row0=%d n=%d leaf_rows=%d H=%d ld=%d (see cavs_lstm_round_packed_ok)",
+               row0, n, leaf_rows, H, ld_da);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(da && dc && WhTp && child_rows && gates && G && dret && dret_rows, "cavs_lstm_round_bwd_children_gates_packed: null pointer");
+  CAVS_REQUIRE(aligned16(da) && aligned16(WhTp), "cavs_lstm_round_bwd_children_gates_packed: da and WhTp must be 16-byte aligned");
+  ChildBwdArgs a{da + (long)row0 * ld_da, ld_da, WhTp, H, child_rows, nullptr, 0, n, H, 4 * H, da, dc, gates, G, nullptr, dret, dret_rows, row0, leaf_rows, 0};
+  const dim3 grid(H / 16, (n + 15) / 16);
+  if (plan_round(n).waves == 8) launch(round_bwd_children_kernel<16, 8, true, 1, 1, true>, grid, 512, 0, as_stream(stream), a);
+  else launch(round_bwd_children_kernel<16, 4, true, 1, 1, true>, grid, 256, 0, as_stream(stream), a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

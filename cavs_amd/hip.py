@@ -95,6 +95,7 @@ _SIGS = {
     "cavs_treelstm_round_bwd_children_gates_packed": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_lstm_round_fwd_packed": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_leaves_fwd": [_P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_bwd_gates": [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_treefc_round_fwd": [_P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
@@ -102,6 +103,7 @@ _SIGS = {
     "cavs_treefc_round_bwd": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_round_bwd_children": [_P, _I, _I, _P, _I, _I, _P, _P, _I, _I, _I, _P],
     "cavs_lstm_round_bwd_children_gates": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "cavs_lstm_round_bwd_children_gates_packed": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_lstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _I, _I, _P],
     "cavs_treefc_round_bwd_children_act": [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_treefc_bwd_rows": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
@@ -122,11 +124,12 @@ _SIGS = {
 _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z,
             "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
             "cavs_clip_grads_workspace": _Z, "cavs_sgemm_group_workspace": _Z, "cavs_fc_softmax_xent_parts": _I,
-            "cavs_colsum_parts": _I, "cavs_round_packed_ok": _I}
+            "cavs_colsum_parts": _I, "cavs_round_packed_ok": _I, "cavs_lstm_round_packed_ok": _I}
 _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I],
             "cavs_fc_softmax_xent_workspace": [_I, _I, _I], "cavs_colsum_blocks_workspace": [_I, _I, _I],
             "cavs_clip_grads_workspace": [_I], "cavs_sgemm_group_workspace": [_I, C.POINTER(GemmDesc)],
-            "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I], "cavs_round_packed_ok": [_I, _I]}
+            "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I], "cavs_round_packed_ok": [_I, _I],
+            "cavs_lstm_round_packed_ok": [_I, _I]}
 
 EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)
 EW_UNARY = dict(assign=0, neg=1, abs=2, square=3, sigmoid=4, tanh=5, relu=6)

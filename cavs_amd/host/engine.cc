@@ -269,7 +269,8 @@ void Engine::reserve_edges() {
     R(r_z_, rc * H);
   }
   if (fused_rows() > 0) R(UT_, (size_t)(cfg_.model == CAVS_MODEL_TREEFC ? 2 : 4) * H * H);
-  if (fused_rows() > 0 && cfg_.model == CAVS_MODEL_TREELSTM && (cavs_round_packed_ok(1, H) || cavs_round_packed_ok(65, H)))
+  if (fused_rows() > 0 && ((cfg_.model == CAVS_MODEL_TREELSTM && (cavs_round_packed_ok(1, H) || cavs_round_packed_ok(65, H))) ||
+                           (cfg_.model == CAVS_MODEL_LSTM && (cavs_lstm_round_packed_ok(1, H) || cavs_lstm_round_packed_ok(65, H)))))
     R(Upk_, (size_t)4 * H * H);
   if (cfg_.model == CAVS_MODEL_TREELSTM) {
     R(hlr_, cap * H);
@@ -525,6 +526,13 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
             check(cavs_zero(emb_stamp_.get(), (size_t)cfg_.V * 4, stream_));
           }
           tasks.push_back({CAVS_TASK_EMBED_SGD, lr, N, E, ++emb_epoch_, p.w, p.g, xs_prev_.get(), emb_stamp_.get()});
+          continue;
+        }
+        if (kv.first == "W" && cfg_.model == CAVS_MODEL_LSTM && Upk_.capacity() > 0) {  // [U' | W'], W' with its packed copy
+          const long long H = cfg_.H, half = 4 * H * H;
+          tasks.push_back({CAVS_TASK_SGD, lr, half, 0, 0, p.w, p.g, nullptr, nullptr});
+          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, 4 * H, 0, Upk_.get(), p.w + half, p.g + half, nullptr});
+          upk_valid_ = p.w == p.own_w.get();
           continue;
         }
         if (kv.first == "U" && Upk_.capacity() > 0) {  // the update and the packed copy of the next forward pass
@@ -868,6 +876,15 @@ void Engine::lstm_forward() {
   gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
   const int fused = fused_rows();
+  bool any_packed = false;
+  if (Upk_.capacity() > 0)
+    for (const Round &r : sched_.rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_lstm_round_packed_ok(r.n, H);
+  if (any_packed && !upk_valid_) {  // W' was written by somebody else since the last update here
+    cavs_task pack{CAVS_TASK_SGD_PACK, 0.f, H, 4 * H, 0, Upk_.get(), const_cast<float *>(Wh), nullptr, nullptr};
+    check(cavs_run_tasks(1, &pack, stream_));
+    c_launches_ += 1;
+    upk_valid_ = Wx == param("W").own_w.get();
+  }
   out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
   for (const Round &r : sched_.rounds) {
@@ -878,8 +895,10 @@ void Engine::lstm_forward() {
         CAVS_TIMED(K_GATES, cavs_lstm_round_leaves_fwd(pool_.get(), d_pair_ + off, a, 4 * H, Bv, gates_.at(off * 5 * H), msg, go,
                                                        d_t2j_ + off, r.n, H, stream_));
       } else {
-        CAVS_TIMED(K_ROUND, cavs_lstm_round_fwd(pool_.get(), d_child_ + off, d_pair_ + off, a, 4 * H, Wh, Bv, G_.at(off * 2 * H),
-                                                gates_.at(off * 5 * H), msg, go, d_t2j_ + off, r.n, H, stream_));
+        const bool pk = any_packed && cavs_lstm_round_packed_ok(r.n, H);
+        CAVS_TIMED(K_ROUND, (pk ? cavs_lstm_round_fwd_packed : cavs_lstm_round_fwd)(
+                                pool_.get(), d_child_ + off, d_pair_ + off, a, 4 * H, pk ? Upk_.get() : Wh, Bv, G_.at(off * 2 * H),
+                                gates_.at(off * 5 * H), msg, go, d_t2j_ + off, r.n, H, stream_));
         c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
         c_gather_rows_ += r.n;
       }
@@ -904,8 +923,13 @@ void Engine::lstm_backward() {
   const int fused = fused_rows();
   const bool dret_folded = fused > 0 && sched_.max_round <= fused;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
+  bool packed = forest_;  // as in treelstm_backward
+  for (const Round &r : sched_.rounds)
+    if (!leaf_round(r) && !cavs_lstm_round_packed_ok(r.n, H)) packed = false;
   if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
-    backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr, nullptr}}, true);
+    backward_prologue({{packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr,
+                        nullptr}},
+                      true);
   } else {
     backward_prologue({}, true);
   }
@@ -922,8 +946,9 @@ void Engine::lstm_backward() {
     if (folded) {
       c_gather_rows_ += r.n;
       if (leaf_round(r)) continue;
-      CAVS_TIMED(K_ROUND, cavs_lstm_round_bwd_children_gates(dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(),
-                                                             G_.get(), d_dgo_, d_t2j_, (int)off, r.n, sched_.leaf_prefix, H, stream_));
+      CAVS_TIMED(K_ROUND, (packed ? cavs_lstm_round_bwd_children_gates_packed : cavs_lstm_round_bwd_children_gates)(
+                              dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(), G_.get(), d_dgo_, d_t2j_, (int)off,
+                              r.n, sched_.leaf_prefix, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
       c_scatter_rows_ += r.n;
       c_launches_ += 1;

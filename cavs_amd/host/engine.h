@@ -182,8 +182,9 @@ class Engine {
   DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
   void embedding_backward(int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
-  // Tree-LSTM: U tile-major for the packed forward rounds.  Written by the job that applies U's
-  // SGD update; current while nobody else has written U since (set_param, a caller's own tensor).
+  // The recurrent weights (Tree-LSTM: U; chain LSTM: W') tile-major for the packed forward rounds.
+  // Written by the job that applies their SGD update; current while nobody else has written them
+  // since (set_param, a caller's own tensor).
   DeviceArray<float> Upk_;
   bool upk_valid_ = false;
   // rounds of at most this many rows run as fused launches (0: none)

@@ -380,6 +380,18 @@ int cavs_treefc_round_bwd(const float *dpool, const int *pair, const float *dret
  * nchild 1, dA = da [n,4H], BT = Wh^T [4H,H].  Tree-FC: nchild 2, dA = dz [n,H], BT = W^T [H,2H]. */
 int cavs_round_bwd_children(const float *dA, int ld, int K, const float *BT, int ldb, int nchild,
                             const int *child, float *dpool, int pool_width, int n, int H, void *stream);
+/* cavs_lstm_round_fwd / cavs_lstm_round_bwd_children_gates with the recurrent weights tile-major:
+ * Whp = W' [K = H, N = 4H] as a CAVS_TASK_SGD_PACK job writes it, WhTp = W'^T [K = 4H, N = H] as a
+ * CAVS_TASK_PACK_T job does.  Same results bit for bit; for the shapes cavs_lstm_round_packed_ok(n, H)
+ * admits (rounds of at most 1024 vertices, H a multiple of 512, or of 256 above 64 vertices). */
+int cavs_lstm_round_packed_ok(int n, int H);
+int cavs_lstm_round_fwd_packed(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                               const float *Whp, const float *bias, float *G, float *gates, float *msg,
+                               float *graph_out, const int *out_rows, int n, int H, void *stream);
+int cavs_lstm_round_bwd_children_gates_packed(float *da, int ld_da, float *dc, const float *WhTp,
+                                              const int *child_rows, const float *gates, const float *G,
+                                              const float *dret, const int *dret_rows, int row0, int n,
+                                              int leaf_rows, int H, void *stream);
 /* The chain LSTM's and Tree-FC's backward round as one launch, as
  * cavs_treelstm_round_bwd_children_gates does it for the Tree-LSTM: whole-batch slabs, the
  * round is rows [row0, row0 + n), child_rows names the children by slab row, and the launch

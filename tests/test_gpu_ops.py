@@ -852,6 +852,73 @@ def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
         g.call("cavs_run_tasks", 1, (T * 1)(bad), g.stream())
 
 
+@pytest.mark.parametrize("L,m,n,H", [(300, 90, 100, 256), (200, 30, 40, 512), (500, 128, 128, 512), (1500, 500, 600, 256)])
+def test_packed_weights_give_the_same_chain_lstm_rounds_bit_for_bit(g, L, m, n, H):
+    """Chain LSTM: the forward launch and the folded backward launch reading W' / W'^T tile-major
+    against the ones reading them row-major (themselves checked against the oracle above)."""
+    r = rng(31 * L + n + H)
+    N = L + m + n
+    Wh = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)          # W' [H, 4H]
+    d_Wh, WhT, Whp, WhTp = g.devf(Wh), g.zeros(4 * H * H), g.zeros(4 * H * H), g.zeros(4 * H * H)
+    T = hip.Task
+    jobs = [T(hip.TASK_TRANSPOSE, 0.0, H, 4 * H, 0, g.P(WhT), g.P(d_Wh), None, None),
+            T(hip.TASK_PACK_T, 0.0, H, 4 * H, 0, g.P(WhTp), g.P(d_Wh), None, None),
+            T(hip.TASK_SGD_PACK, 0.0, H, 4 * H, 0, g.P(Whp), g.P(d_Wh), None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    np.testing.assert_array_equal(g.host(Whp), pack_tiles(Wh.reshape(H, 4 * H)))
+    np.testing.assert_array_equal(g.host(WhTp), pack_tiles(np.ascontiguousarray(Wh.reshape(H, 4 * H).T)))
+    assert hip.lib().cavs_lstm_round_packed_ok(n, H) == 1 and hip.lib().cavs_lstm_round_packed_ok(m, H) == 1
+
+    # forward: one round of n vertices over a pool of L + m earlier rows
+    pool = (r.bulk_normal((N + 2) * 2 * H).reshape(N + 2, 2 * H) * 0.5).astype(np.float32)
+    child = np.argsort(r.bulk_normal(L + m))[:n].astype(np.int32)
+    child[1] = -1
+    pair = (L + m + np.arange(n)).astype(np.int32)
+    pair[n - 1] = -1
+    d_child, d_pair = g.devi(child), g.devi(pair)
+    d_xW, d_bias = g.devf(r.bulk_normal(n * 4 * H)), g.devf(r.bulk_normal(4 * H))
+    d_out = g.devi(np.argsort(r.bulk_normal(n + 3))[:n].astype(np.int32))
+    outs = []
+    for entry, W in (("cavs_lstm_round_fwd", d_Wh), ("cavs_lstm_round_fwd_packed", Whp)):
+        d_pool = g.devf(pool)
+        G, gates, msg, go = g.zeros(n, 2 * H), g.zeros(n, 5 * H), g.zeros(n, 2 * H), g.zeros(n + 3, H, fill=-7.0)
+        g.call(entry, g.P(d_pool), g.P(d_child), g.P(d_pair), g.P(d_xW), 4 * H, g.P(W), g.P(d_bias), g.P(G), g.P(gates), g.P(msg),
+               g.P(go), g.P(d_out), n, H, g.stream())
+        outs.append([g.host(t) for t in (d_pool, G, gates, msg, go)])
+    for a, b, what in zip(outs[0], outs[1], ("pool", "G", "gates", "msg", "graph_out")):
+        np.testing.assert_array_equal(a, b, err_msg=what)
+    assert (outs[0][2] != 0).all()
+
+    # backward: the top n rows from the row-list launch, then two folded launches (top, middle)
+    order = np.argsort(r.bulk_normal(L)).astype(np.int32)
+    kids = np.full(N, -1, np.int32)
+    kids[L: L + m] = order[:m]
+    top_kids = np.concatenate([np.arange(L, L + m, dtype=np.int32), order[m: n]]) if n > m else np.arange(L, L + n, dtype=np.int32)
+    kids[L + m:] = top_kids[np.argsort(r.bulk_normal(n))]
+    gates = np.tanh(r.bulk_normal(N * 5 * H).reshape(N, 5 * H)).astype(np.float32)
+    G = (r.bulk_normal(N * 2 * H).reshape(N, 2 * H) * 0.5).astype(np.float32)
+    d_gates, d_G, d_kids = g.devf(gates), g.devf(G), g.devi(kids)
+    d_dgo, d_rows = g.devf(r.bulk_normal(N * H)), g.devi(np.argsort(r.bulk_normal(N)).astype(np.int32))
+    roots = g.devi(np.arange(L + m, N, dtype=np.int32))
+    outs = []
+    for entry, W in (("cavs_lstm_round_bwd_children_gates", WhT), ("cavs_lstm_round_bwd_children_gates_packed", WhTp)):
+        dA, dc = g.zeros(N, 4 * H, fill=-3.0), g.zeros(N, H, fill=-3.0)
+        g.call("cavs_lstm_bwd_gates_rows", g.P(roots), n, g.P(d_dgo), g.P(d_rows), g.P(d_gates), g.P(d_G), g.P(dA), 4 * H, g.P(dc), L, H,
+               g.stream())
+        for lo, cnt in ((L + m, n), (L, m)):
+            g.call(entry, g.P(dA), 4 * H, g.P(dc), g.P(W), g.P(d_kids) + 4 * lo, g.P(d_gates), g.P(d_G), g.P(d_dgo), g.P(d_rows), lo, cnt,
+                   L, H, g.stream())
+        outs.append((g.host(dA), g.host(dc)))
+    np.testing.assert_array_equal(outs[0][0], outs[1][0], err_msg="dA")
+    np.testing.assert_array_equal(outs[0][1], outs[1][1], err_msg="dc")
+    assert (outs[0][0][order[:m]] != -3.0).all()
+    assert hip.lib().cavs_lstm_round_packed_ok(16, 128) == 0 and hip.lib().cavs_lstm_round_packed_ok(100, 128) == 0
+    with pytest.raises(hip.CavsError, match="cavs_lstm_round_packed_ok"):
+        hip.call("cavs_lstm_round_fwd_packed", 16, 16, 16, 16, 4 * 128, 16, 16, 16, 16, 16, 0, 0, 16, 128, 0)
+    with pytest.raises(hip.CavsError, match="cavs_lstm_round_packed_ok"):
+        hip.call("cavs_lstm_round_bwd_children_gates_packed", 16, 4 * 128, 16, 16, 16, 16, 16, 16, 16, 0, 16, 0, 128, 0)
+
+
 def test_fused_round_entry_points_reject_bad_shapes():
     with pytest.raises(hip.CavsError, match="multiple of 32"):
         hip.call("cavs_treelstm_round_fwd", 0, 0, 0, 0, 4 * 24, 0, 0, 0, 0, 0, 0, 0, 0, 5, 24, 0)
