@@ -343,33 +343,37 @@ def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     s.close()
 
 
-def test_the_packed_copy_of_the_recurrent_weights_follows_every_writer(oracle):
-    """Tree-LSTM rounds of more than 64 vertices at H=128 read U from its tile-major copy.  The copy
-    is written by the update job; set_param writes U behind its back.  Three steps -- the first packs
-    on demand, the second reads what the first step's update left, the third follows a set_params
-    -- each against the oracle on the parameters the session should hold."""
-    H, E, V, C_ = 128, 16, 37, 5
-    w = small_workload("treelstm", 333, B=70, H=H, E=E, V=V, C=C_, skew=False)
-    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc")
+@pytest.mark.parametrize("model,H", [("treelstm", 128), ("lstm", 256)])
+def test_the_packed_copy_of_the_recurrent_weights_follows_every_writer(oracle, model, H):
+    """Rounds of more than 64 vertices at these hidden sizes read the recurrent weights (U; W' of
+    the chain LSTM) from their tile-major copy.  The copy is written by the update job; set_param
+    writes the weights behind its back.  Three steps -- the first packs on demand, the second reads
+    what the first step's update left, the third follows a set_params -- each against the oracle
+    on the parameters the session should hold."""
+    E, V, C_ = (16 if model == "treelstm" else H), 37, 5
+    w = small_workload(model, 333, B=70, H=H, E=E, V=V, C=C_, skew=False)
+    rec = "U" if model == "treelstm" else "W"
+    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc") if model == "treelstm" else ("Emb", "W", "Bv", "Wfc", "bfc")
     p = {k: np.array(w["params"][k], np.float32) for k in names}
-    p["U"] = (p["U"] * np.float32(0.2)).astype(np.float32)
-    s = session.Session("treelstm", H=H, E=E, V=V, C_=C_)
-    assert hip.lib().cavs_round_packed_ok(70, H) == 1
+    p[rec] = (p[rec] * np.float32(0.2)).astype(np.float32)
+    s = session.Session(model, H=H, E=E, V=V, C_=C_)
+    ok = hip.lib().cavs_round_packed_ok if model == "treelstm" else hip.lib().cavs_lstm_round_packed_ok
+    assert ok(70, H) == 1
     s.set_params(p)
     lr = 0.25
     for step in range(3):
-        print(f"[case] packed copy step {step}", flush=True)
+        print(f"[case] packed copy {model} step {step}", flush=True)
         if step == 2:
-            p["U"] = (p["U"][::-1] * np.float32(0.5)).astype(np.float32)
-            s.set_params(dict(U=p["U"]))
-        want = oracle.model_step("treelstm", w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
+            p[rec] = (p[rec][::-1] * np.float32(0.5)).astype(np.float32)
+            s.set_params({rec: p[rec]})
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
         s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
         close(s.fetch("graph_out"), want["graph_out"], f"graph_out at step {step}", rtol=3e-4, atol=3e-5)
         got = s.grads()
         for k in names:
             close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", rtol=3e-4, atol=3e-5)
             p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
-    close(s.param("U", p["U"].shape), p["U"], "U after the steps", rtol=3e-4, atol=3e-5)
+    close(s.param(rec, p[rec].shape), p[rec], f"{rec} after the steps", rtol=3e-4, atol=3e-5)
     s.close()
 
 
