@@ -94,9 +94,26 @@ Param &Engine::param(const std::string &name) {
 void Engine::bind_param(const std::string &name, float *w, float *g) {
   Param &p = param(name);
   if (!w) fail(CAVS_EINVAL, "bind_param('" + name + "'): null weight pointer");
+  if (p.w != w) upk_valid_ = false;
   p.w = w;
   p.g = g ? g : p.own_g.get();
-  upk_valid_ = false;
+}
+
+bool Engine::update_jobs(float *w, float *g, float lr, std::vector<cavs_task> *out) {
+  if (Upk_.capacity() == 0 || !w || !g) return false;
+  const long long H = cfg_.H;
+  if (cfg_.model == CAVS_MODEL_TREELSTM && w == param("U").w) {
+    out->push_back({CAVS_TASK_SGD_PACK, lr, H, 3 * H, 0, Upk_.get(), w, g, nullptr});
+    out->push_back({CAVS_TASK_SGD_PACK, lr, H, H, 0, Upk_.at((size_t)3 * H * H), w + 3 * H * H, g + 3 * H * H, nullptr});
+  } else if (cfg_.model == CAVS_MODEL_LSTM && w == param("W").w) {  // [U' | W'], W' with its packed copy
+    const long long half = 4 * H * H;
+    out->push_back({CAVS_TASK_SGD, lr, half, 0, 0, w, g, nullptr, nullptr});
+    out->push_back({CAVS_TASK_SGD_PACK, lr, H, 4 * H, 0, Upk_.get(), w + half, g + half, nullptr});
+  } else {
+    return false;
+  }
+  upk_valid_ = true;
+  return true;
 }
 
 void Engine::set_param(const std::string &name, const float *host, size_t n) {
@@ -528,18 +545,8 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
           tasks.push_back({CAVS_TASK_EMBED_SGD, lr, N, E, ++emb_epoch_, p.w, p.g, xs_prev_.get(), emb_stamp_.get()});
           continue;
         }
-        if (kv.first == "W" && cfg_.model == CAVS_MODEL_LSTM && Upk_.capacity() > 0) {  // [U' | W'], W' with its packed copy
-          const long long H = cfg_.H, half = 4 * H * H;
-          tasks.push_back({CAVS_TASK_SGD, lr, half, 0, 0, p.w, p.g, nullptr, nullptr});
-          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, 4 * H, 0, Upk_.get(), p.w + half, p.g + half, nullptr});
-          upk_valid_ = p.w == p.own_w.get();
-          continue;
-        }
-        if (kv.first == "U" && Upk_.capacity() > 0) {  // the update and the packed copy of the next forward pass
-          const long long H = cfg_.H;
-          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, 3 * H, 0, Upk_.get(), p.w, p.g, nullptr});
-          tasks.push_back({CAVS_TASK_SGD_PACK, lr, H, H, 0, Upk_.at((size_t)3 * H * H), p.w + 3 * H * H, p.g + 3 * H * H, nullptr});
-          upk_valid_ = p.w == p.own_w.get();
+        if (update_jobs(p.w, p.g, lr, &tasks)) {  // the recurrent weights: the update and the packed copy in one job
+          upk_valid_ = p.w == p.own_w.get();  // a caller's own tensor may be written behind the engine's back
           continue;
         }
         tasks.push_back({CAVS_TASK_SGD, lr, (long long)p.n, 0, 0, p.w, p.g, nullptr, nullptr});

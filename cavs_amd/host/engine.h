@@ -40,6 +40,12 @@ class Engine {
     p.g = g ? g : p.own_g.get();
   }
   const float *grad_ptr(const std::string &name) { return param(name).g; }
+  // For a caller that applies w -= lr * g to bound parameters itself (the front end's optimizer):
+  // when w is the recurrent weights whose tile-major copy the forward rounds read, appends the
+  // jobs of a cavs_run_tasks launch that update them and the copy together and returns true --
+  // the copy then counts as current until the parameter is bound elsewhere; otherwise false, and
+  // the caller's plain update will do.  Such a caller must route every write of w through here.
+  bool update_jobs(float *w, float *g, float lr, std::vector<cavs_task> *out);
   float *graph_out_ptr() const { return GO_.get(); }
   // The two halves of step() for a caller that runs the loss head itself: forward F into
   // graph_out [N,H] (vertex order), then backward F from d graph_out.

@@ -769,11 +769,13 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     std::vector<cavs_task> updates;
     for (auto &v : g.opt.vars) {
       Tensor &w = tensor(v), &gr = tensor(GetGradientName(v));
-      updates.push_back({CAVS_TASK_SGD, g.opt.lr, (long long)w.count(), 0, 0, w.base, gr.base, nullptr, nullptr});
-      if (updates.size() == 12) {
+      if (updates.size() + 2 > 12) {
         check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
         updates.clear();
       }
+      // the lowered F reads its recurrent weights from a packed copy that the update keeps current
+      if (engine_ && engine_->update_jobs(w.base, gr.base, g.opt.lr, &updates)) continue;
+      updates.push_back({CAVS_TASK_SGD, g.opt.lr, (long long)w.count(), 0, 0, w.base, gr.base, nullptr, nullptr});
     }
     check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
   }

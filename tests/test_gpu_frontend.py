@@ -134,6 +134,34 @@ def test_training_steps_update_variables_like_the_oracle(oracle):
     a.close()
 
 
+@pytest.mark.parametrize("model,H", [("treelstm", 128), ("lstm", 256)])
+def test_training_steps_at_sizes_whose_rounds_read_packed_weights(oracle, model, H):
+    """Rounds of 70 vertices at these hidden sizes read the recurrent weights from a tile-major
+    copy.  The parameters live in the Variables' own tensors and the optimizer is an ordinary op
+    of the main scope: the first forward pass packs on demand, later ones read the copy that the
+    optimizer's update of that Variable keeps current.  Losses and the final weights against the
+    oracle over three steps."""
+    E, V, C_ = (16 if model == "treelstm" else H), 37, 5
+    w = small_workload(model, 334, B=70, H=H, E=E, V=V, C=C_, skew=False)
+    rec = "U" if model == "treelstm" else "W"
+    names = ("Emb", "W", "U", "Bv", "Wfc", "bfc") if model == "treelstm" else ("Emb", "W", "Bv", "Wfc", "bfc")
+    p = {k: np.array(w["params"][k], np.float32) for k in names}
+    p[rec] = (p[rec] * np.float32(0.2)).astype(np.float32)
+    B, maxlen = w["graph"].shape
+    lr = 0.25
+    a = apps.App(model, B=B, maxlen=maxlen, H=H, E=E, V=V, C_=C_, opt=session.OPT_BATCHING, lr=lr)
+    a.set_params(p)
+    for step in range(3):
+        print(f"[case] front end, packed weights, {model} step {step}", flush=True)
+        want = oracle_step(oracle, dict(w, params=p), model)
+        loss, _ = a.step(w["graph"], w["x"], w["labels"], train=True)
+        close(loss, want["loss"], f"loss at step {step}", rtol=2e-4, atol=2e-5)
+        for k in names:
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    close(a.grad(rec, p[rec].shape, grad=False), p[rec], f"{rec} after 3 steps", rtol=3e-4, atol=3e-5)
+    a.close()
+
+
 def _root_mask(w):
     mask = np.zeros((w["N"], w["H"]), np.float32)
     off = 0
