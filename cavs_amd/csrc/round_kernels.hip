@@ -177,7 +177,31 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
         acc[4] = M::mma(hr, f.b[u][3][c], acc[4]);
       }
   };
-  if (kb < ke) fetch_b(kb, f0);
+  // PACKED: float4 (slot, x) of tile (k-group, column tile); gates i, o, u are column tiles
+  // H/16 apart in the [H, 3H] matrix's packing, the forget gate's matrix follows it
+  const float4 *pio = reinterpret_cast<const float4 *>(a.Upk) + ((long)(kb / GK) * (3 * H / 16) + blockIdx.x) * 64 + slot * 16 + x;
+  const float4 *pf = reinterpret_cast<const float4 *>(a.Upk) + 3L * H * H / 4 + ((long)(kb / GK) * (H / 16) + blockIdx.x) * 64 + slot * 16 + x;
+  const int gate4 = H * 4;  // float4 between the gates' column tiles
+  auto pfetch_b = [&](Frag &f) {  // a stage's weights from the packed copy; moves on to the next stage
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+      const float4 bi = pio[0], bo = pio[gate4], bu = pio[2 * gate4], bf = *pf;
+#pragma unroll
+      for (int c = 0; c < 4; c++) {
+        f.b[u][0][c] = elem(bi, c);
+        f.b[u][1][c] = elem(bo, c);
+        f.b[u][2][c] = elem(bu, c);
+        f.b[u][3][c] = elem(bf, c);
+      }
+      pio += 3 * gate4;
+      pf += gate4;
+    }
+  };
+  if constexpr (PACKED) {
+    pfetch_b(f0);
+  } else {
+    if (kb < ke) fetch_b(kb, f0);
+  }
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
     Epi &ep = epi[q];
@@ -208,27 +232,11 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     const int kbu = __builtin_amdgcn_readfirstlane(kb), nst = __builtin_amdgcn_readfirstlane((ke - kb) / S);
     int sio = (kbu + S) * 3 * H * 4, sf = (3 * H * H + (kbu + S) * H) * 4;  // scalar byte offsets of the next k-group
     const float *al = pl + kb + S + 4 * slot, *ar = pr + kb + S + 4 * slot;
-    // PACKED: float4 (slot, x) of tile (k-group, column tile); gates i, o, u are column tiles
-    // H/16 apart in the [H, 3H] matrix's packing, the forget gate's matrix follows it
-    const int kg1 = (kb + S) / GK;
-    const float4 *pio = reinterpret_cast<const float4 *>(a.Upk) + ((long)kg1 * (3 * H / 16) + blockIdx.x) * 64 + slot * 16 + x;
-    const float4 *pf = reinterpret_cast<const float4 *>(a.Upk) + 3L * H * H / 4 + ((long)kg1 * (H / 16) + blockIdx.x) * 64 + slot * 16 + x;
-    const int gate4 = H * 4;  // float4 between the gates' column tiles
     auto xfetch = [&](Frag &f) {
+      if constexpr (PACKED) pfetch_b(f);
 #pragma unroll
       for (int u = 0; u < UG; u++) {
-        if constexpr (PACKED) {
-          const float4 bi = pio[0], bo = pio[gate4], bu = pio[2 * gate4], bf = *pf;
-#pragma unroll
-          for (int c = 0; c < 4; c++) {
-            f.b[u][0][c] = elem(bi, c);
-            f.b[u][1][c] = elem(bo, c);
-            f.b[u][2][c] = elem(bu, c);
-            f.b[u][3][c] = elem(bf, c);
-          }
-          pio += 3 * gate4;
-          pf += gate4;
-        } else {
+        if constexpr (!PACKED) {
 #pragma unroll
           for (int c = 0; c < 4; c++) {
             f.b[u][0][c] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ubuf, vio[c], sio, 0));

@@ -165,6 +165,17 @@ def rounds(iters, st):
                                     xW.data_ptr(), 4 * H, U.data_ptr(), bias.data_ptr(), G.data_ptr(), hlr.data_ptr(),
                                     gt.data_ptr(), msg.data_ptr(), None, None, n, H, st), iters, st)
         _emit("treelstm_round_fwd", f"{tag}: n={n} H={H}", us, flops=flops)
+        if hip.lib().cavs_round_packed_ok(n, H):  # the same launch reading U from its tile-major copy
+            Upk = torch.empty(4 * H * H, **f32)
+            T = hip.Task
+            jobs = [T(hip.TASK_SGD_PACK, 0.0, H, 3 * H, 0, Upk.data_ptr(), U.data_ptr(), None, None),
+                    T(hip.TASK_SGD_PACK, 0.0, H, H, 0, Upk.data_ptr() + 4 * 3 * H * H, U.data_ptr() + 4 * 3 * H * H, None, None)]
+            hip.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), st)
+            us = _time(lambda: hip.call("cavs_treelstm_round_fwd_packed", pool.data_ptr(), child.data_ptr(), pair.data_ptr(),
+                                        xW.data_ptr(), 4 * H, U.data_ptr(), Upk.data_ptr(), bias.data_ptr(), G.data_ptr(),
+                                        hlr.data_ptr(), gt.data_ptr(), msg.data_ptr(), None, None, n, H, st), iters, st)
+            _emit("treelstm_round_fwd_packed", f"{tag}: n={n} H={H}", us, flops=flops)
+            del Upk
         hU, hUf = torch.empty(n, 3 * H, **f32), torch.empty(2 * n, H, **f32)
 
         def separate_fwd():

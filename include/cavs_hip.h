@@ -302,7 +302,7 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
                             int H, void *stream);
 /* cavs_treelstm_round_fwd with the loop's weights read from Upk, the tile-major copy a
  * CAVS_TASK_SGD_PACK job writes (pack(U_iou) [K = H, N = 3H], then pack(U_f) [K = H, N = H] at float
- * 3H*H); U is still read for the first k-groups.  Same results bit for bit; for the shapes
+ * 3H*H), which must hold the same values as U.  Same results bit for bit; for the shapes
  * cavs_round_packed_ok(n, H) admits. */
 int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
                                    const float *U, const float *Upk, const float *bias, float *G, float *hlr,
