@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, profiles/bench_C3_hbm_traffic_pmc.txt
-PMC_TRAFFIC_BYTES = {("C3", "round"): 18.25e6}
+PMC_TRAFFIC_BYTES = {("C3", "round"): 17.56e6}
 
 
 def model_kwargs(w):
