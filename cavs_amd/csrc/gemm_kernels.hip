@@ -609,6 +609,25 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
   long kc = (long)(work / (double)slots);
   kc = (kc + 31) / 32 * 32;
   if (kc < 256) kc = 256;
+  // The chip holds `slots` of these workgroups at once.  A launch of a few more runs them as a
+  // second round behind the first -- a whole workgroup's time for a handful of tiles (measured:
+  // 1024 workgroups 95 us, 1032 workgroups 122 us) -- so the k chunk grows until the launch fits,
+  // unless the tiles alone overflow it.
+  auto launch_size = [&](long chunk) {
+    long total = 0;
+    for (int p = 0; p < count; p++) {
+      const cavs_gemm_desc &q = d[p];
+      if (q.M == 0 || q.N == 0 || alone[p]) continue;
+      long s = q.K > 0 ? (q.K + chunk / 2) / chunk : 1;
+      if (s < 1) s = 1;
+      const long kchunk = q.K > 0 ? ((q.K + s - 1) / s + 31) / 32 * 32 : 1;
+      const long splits = q.K > 0 ? (q.K + kchunk - 1) / kchunk : 1;
+      total += (tiles[p] * splits + 7) / 8 * 8;
+    }
+    return total;
+  };
+  if (launch_size(1L << 30) <= slots)
+    while (launch_size(kc) > slots) kc += 32;
   size_t need = 0;
   bool vec = true;
   int n = 0, nr = 0;
