@@ -558,8 +558,16 @@ static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float 
     g.ws = static_cast<float *>(ws);
   }
   bool vec = vec_path_ok(g, tA, tB);
+  // The chip holds four 64x64 workgroups per CU with K panels of 32 (their LDS) and eight with
+  // panels of 16.  A launch of a few more than four per CU runs them as a second round behind
+  // the first (2048 x 2048 x 300: 29.0 us; 2112 rows: 36.7), so launches between one and two
+  // rounds take the narrow panels and stay resident at once (2482 rows: 40.2 -> 33.1 us);
+  // everywhere else the wide panels are faster.
+  const long wgs = p.tiles * p.splits, slots = 4L * num_cus();
   if (p.kind == GemmPlan::TILE128)
     launch_tile<128, 128, 16>(g, tA, tB, vec, p, st);
+  else if (wgs > slots && wgs <= 2 * slots)
+    launch_tile<64, 64, 16>(g, tA, tB, vec, p, st);
   else
     launch_tile<64, 64, 32>(g, tA, tB, vec, p, st);
   CAVS_LAUNCH_CHECK();

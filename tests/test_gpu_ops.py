@@ -119,7 +119,9 @@ def test_gather_children(g, oracle, n, w, hw):
 
 # ---------------------------------------------------------------- GEMM
 SHAPES = [(13, 17, 29), (1, 64, 64), (200, 256, 64), (128, 128, 16), (129, 131, 300), (77, 2048, 300),
-          (300, 1536, 512), (5, 512, 40), (640, 5, 512), (512, 384, 2052)]
+          (300, 1536, 512), (5, 512, 40), (640, 5, 512), (512, 384, 2052),
+          # between one and two rounds of resident 64x64 workgroups: the narrow-K-panel variant
+          (2482, 2048, 300), (2100, 2050, 70)]
 
 
 @pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
