@@ -21,6 +21,9 @@ inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 
 
 constexpr int kWave = 64;
 int num_cus();  // compute units of the current device (256 on MI355X)
+// Device address of the built-in split-K scratch on the current device (looked up once per
+// device; defined next to the array in gemm_kernels.hip).  `out` may be null.
+int static_scratch_setup(float **out);
 
 // Timing probe of the calling thread (cavs_profile_arm): while armed, the first kernel an
 // entry point launches records `start` when it begins and every kernel records `stop` when

@@ -693,11 +693,59 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
   return CAVS_OK;
 }
 
+// Split-K partials of cavs_sgemm_splitk_static: device memory that exists from the moment the
+// code object is loaded, so that entry point never has to ask the allocator for any.  Every GPU
+// the library runs on holds its own copy until the process ends.
+constexpr size_t kStaticScratchBytes = size_t(32) << 20;
+constexpr int kStaticScratchDevices = 64;
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+// Device address of `scratch` on each GPU (the array's name is only a host-side stand-in for the
+// symbol; kernels, fills and copies take the address looked up here).
+static float *g_scratch_ptr[kStaticScratchDevices] = {};
+
+// Looks the address up for the current device, once.
+int static_scratch_setup(float **out) {
+  int dev = 0;
+  CAVS_HIP_TRY(hipGetDevice(&dev));
+  CAVS_REQUIRE(dev >= 0 && dev < kStaticScratchDevices, "static scratch: device %d out of range", dev);
+  if (!g_scratch_ptr[dev]) {
+    float *ptr = nullptr;
+    CAVS_HIP_TRY(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    CAVS_REQUIRE(ptr && aligned16(ptr), "static scratch: no usable address on device %d", dev);
+    g_scratch_ptr[dev] = ptr;
+  }
+  if (out) *out = g_scratch_ptr[dev];
+  return CAVS_OK;
+}
+
 }  // namespace cavs
 
 using namespace cavs;
 
 extern "C" {
+
+size_t cavs_sgemm_splitk_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                             int lda, const float *B, int ldb, float beta, float *C, int ldc, void *stream) {
+  float *ptr = nullptr;
+  int rc = static_scratch_setup(&ptr);
+  if (rc) return rc;
+  if (M > 0 && N > 0 && K > 0) {
+    // the same plan run_gemm makes when it is handed a workspace
+    GemmPlan p = plan_gemm(transA, transB, M, N, K, skinny_ok(transA, transB, K, A, lda, B, ldb), true);
+    size_t need = p.kind == GemmPlan::SKINNY ? 0 : plan_workspace(p, M, N);
+    if (need > kStaticScratchBytes)
+      return set_error(CAVS_EINVAL,
+                       "cavs_sgemm_splitk_static: M=%d N=%d K=%d needs %zu bytes of split-K partials, the built-in "
+                       "scratch holds %zu; use cavs_sgemm_splitk with a workspace of the caller's",
+                       M, N, K, need, kStaticScratchBytes);
+  }
+  // partials are written before they are read, every element of them: nothing of the previous
+  // call's contents has to be cleared
+  return run_gemm("cavs_sgemm_splitk_static", transA, transB, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc,
+                  nullptr, 0, 0, ptr, kStaticScratchBytes, stream);
+}
 
 size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products) {
   size_t need = 0;

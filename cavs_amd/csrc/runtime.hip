@@ -79,7 +79,8 @@ int cavs_init(int device) {
   CAVS_HIP_TRY(hipSetDevice(device));
   g_cus = 0;
   num_cus();
-  return CAVS_OK;
+  // the entry point that allocates nothing finds its scratch here, with this device current
+  return static_scratch_setup(nullptr);
 }
 
 int cavs_device_name(char *buf, size_t len) {

@@ -120,6 +120,19 @@ size_t cavs_sgemm_splitk_workspace(int M, int N, int K);
 int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                       int lda, const float *B, int ldb, float beta, float *C, int ldc,
                       void *workspace, size_t workspace_bytes, void *stream);
+/* cavs_sgemm_splitk without a workspace argument and without any allocation: the K-split
+ * partials go to a buffer built into the library's code object (32 MiB per GPU, held until the
+ * process ends; cavs_sgemm_splitk_static_max_bytes() returns that size).  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory -- code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels, same plan and
+ * bit-for-bit the results of cavs_sgemm_splitk; a shape whose partials would not fit
+ * (cavs_sgemm_splitk_workspace(M, N, K) above the maximum) is refused with CAVS_EINVAL.  All
+ * calls on a GPU share that GPU's buffer: calls that overlap in time on one GPU (two streams,
+ * two threads) race; calls on one stream are ordered by it. */
+size_t cavs_sgemm_splitk_static_max_bytes(void);
+int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                             int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                             void *stream);
 /* Up to four independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
  * (plus one for the K splits): the once-per-step block of
  * cavs/midend/batch_weight_updater.h:12-84 -- the weight-gradient GEMMs -- and the embedding
