@@ -13,7 +13,7 @@
  *   scheduler (or_sched_*)      hand-derived known-answer vectors, invariants,
  *                               brute-force topological checks
  *   row copies (or_*_rows)      closed form out = in[perm], round trips
- *   or_sgemm                    numpy matmul
+ *   or_sgemm                    numpy matmul (fp32), exact rational sums (ord_sgemm)
  *   gate math / model steps     textbook Tree-LSTM / LSTM / Tree-FC in fp64
  *                               autograd (row-preserving mode and same-shape
  *                               batches), finite differences (both modes)
@@ -29,6 +29,31 @@
 
 #ifdef __cplusplus
 extern "C" {
+#endif
+
+/* The op and model restatements are compiled twice from the same source
+ * (ops.c, model.c):
+ *   or_*   real = float  : fp32 throughout, as the reference computes;
+ *   ord_*  real = double : the same dataflow, operation for operation, with every
+ *          value and every sum held in double (build with -DOR_F64).  Inputs are the
+ *          same fp32 numbers widened.  This is what an fp32 implementation is held to
+ *          the path's tolerance against: the checker's own fp32 rounding then takes no
+ *          share of the budget.
+ * The scheduler (or_sched_*) is integer work and exists once. */
+#ifdef OR_F64
+typedef double real;
+#define ORF(name) ord_##name
+#define R_EXP exp
+#define R_TANH tanh
+#define R_LOG log
+#define R_FABS fabs
+#else
+typedef float real;
+#define ORF(name) or_##name
+#define R_EXP expf
+#define R_TANH tanhf
+#define R_LOG logf
+#define R_FABS fabsf
 #endif
 
 /* ------------------------------------------------------------------ scheduler */
@@ -76,33 +101,33 @@ int or_sched_trace(const int *parent_ids, int B, int maxlen, int batching,
 
 /* ------------------------------------------------------------------ row copies */
 /* cavs/backend/functor_batched_memcpy.cuh:33-46 : out[b,:] = inp[ids[b],:] */
-void or_gather_rows(float *out, int ld_out, const float *inp, int ld_inp,
+void ORF(gather_rows)(real *out, int ld_out, const real *inp, int ld_inp,
                     const int *ids, int n, int w);
 /* cavs/backend/functor_batched_memcpy.cuh:48-61 : out[ids[b],:] = inp[b,:] */
-void or_scatter_rows(float *out, int ld_out, const int *ids, const float *inp,
+void ORF(scatter_rows)(real *out, int ld_out, const int *ids, const real *inp,
                      int ld_inp, int n, int w);
 /* cavs/backend/functor_batched_memcpy.cuh:63-75 : out[b,:] = 0, b < n */
-void or_zero_rows(float *out, int ld_out, int n, int w);
+void ORF(zero_rows)(real *out, int ld_out, int n, int w);
 /* cavs/backend/functor_batched_memcpy.cuh:18-31 : column-block copy */
-void or_copy_rows(float *out, int ld_out, const float *inp, int ld_inp, int n, int w);
+void ORF(copy_rows)(real *out, int ld_out, const real *inp, int ld_inp, int n, int w);
 
 /* ------------------------------------------------------------------ dense math */
 /* Row-major C = alpha*op(A)*op(B) + beta*C, cavs/backend/cublas_wrapper.cc:12-28 */
-void or_sgemm(int transA, int transB, int M, int N, int K, float alpha,
-              const float *A, int lda, const float *B, int ldb, float beta,
-              float *C, int ldc);
+void ORF(sgemm)(int transA, int transB, int M, int N, int K, real alpha,
+              const real *A, int lda, const real *B, int ldb, real beta,
+              real *C, int ldc);
 /* out[j] (+)= sum_r inp[r,j]; cavs/backend/op_impl_elementwise.cuh:24-34 */
-void or_colsum(float *out, const float *inp, int ld, int n, int w, int accumulate);
-/* cavs/backend/op_impl_embedding_lookup.cu:22-35 ; ids are floats */
-void or_embed_fwd(float *out, int ld_out, const float *ids, const float *table, int n, int E);
+void ORF(colsum)(real *out, const real *inp, int ld, int n, int w, int accumulate);
+/* cavs/backend/op_impl_embedding_lookup.cu:22-35 ; ids are floating-point values */
+void ORF(embed_fwd)(real *out, int ld_out, const real *ids, const real *table, int n, int E);
 /* cavs/backend/op_impl_embedding_lookup.cu:90-103 */
-void or_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, int n, int E);
+void ORF(embed_bwd)(real *dtable, const real *ids, const real *dy, int ld_dy, int n, int E);
 /* cavs/backend/op_impl_softmax_entropy_logits_loss.cu:94-140 (loss) and
  * :150-164,212-250 (grad = (softmax - onehot)/n).  Either output may be NULL. */
-void or_softmax_xent(float *loss, float *dlogits, const float *logits,
-                     const float *labels, int n, int C);
+void ORF(softmax_xent)(real *loss, real *dlogits, const real *logits,
+                     const real *labels, int n, int C);
 /* cavs/backend/op_impl_sgd.cu : w -= lr*g */
-void or_sgd(float *w, const float *g, float lr, long n);
+void ORF(sgd)(real *w, const real *g, real lr, long n);
 
 /* ------------------------------------------------------------------ gate math
  * Slab-level fused restatements of the elementwise chains of the three vertex
@@ -116,30 +141,30 @@ void or_sgd(float *w, const float *g, float lr, long n);
  *  hUf [2n,H] rows 2r=f_l, 2r+1=f_r pre-activations from U_f
  *  G   [2n,2H]  bias [4H] blocks [i|f|u|o]
  *  gates [n,6H] = [i|o|u|f_l|f_r|tanh(c)] (saved for backward), msg [n,2H]=[h|c] */
-void or_treelstm_gates_fwd(const float *xW, int ld_xw, const float *hU, const float *hUf,
-                           const float *G, const float *bias, float *gates,
-                           float *msg, int n, int H);
+void ORF(treelstm_gates_fwd)(const real *xW, int ld_xw, const real *hU, const real *hUf,
+                           const real *G, const real *bias, real *gates,
+                           real *msg, int n, int H);
 /* Backward of the above.
  *  dmsg [n,2H] gathered-back [dh_m|dc_m]; dret [n,H] pulled d GraphOutput
  *  outputs: dxW [n,4H] = [d_i|d_o|d_u|d_fl+d_fr]; dF [2n,H] rows (d_fl,d_fr);
  *           dG [2n,2H]: only the c half (cols H..2H) is written here
  *           (dc_l, dc_r); the h half comes from the U GEMMs. */
-void or_treelstm_gates_bwd(const float *dmsg, const float *dret, const float *gates,
-                           const float *G, float *dxW, int ld_dxw, float *dF, float *dG,
+void ORF(treelstm_gates_bwd)(const real *dmsg, const real *dret, const real *gates,
+                           const real *G, real *dxW, int ld_dxw, real *dF, real *dG,
                            int n, int H);
 /* Chain LSTM, apps/paper/seq-lstm-cavs.cc:62-86.
  *  a [n,4H] = e*U' + h_p*W' cols [i|f|u|o]; G [n,2H]=[h_p|c_p]; bias [4H] same order
  *  gates [n,5H] = [i|f|u|o|tanh(c)] */
-void or_lstm_gates_fwd(const float *a, int ld_a, const float *G, const float *bias,
-                       float *gates, float *msg, int n, int H);
-void or_lstm_gates_bwd(const float *dmsg, const float *dret, const float *gates,
-                       const float *G, float *da, int ld_da, float *dG, int n, int H);
+void ORF(lstm_gates_fwd)(const real *a, int ld_a, const real *G, const real *bias,
+                       real *gates, real *msg, int n, int H);
+void ORF(lstm_gates_bwd)(const real *dmsg, const real *dret, const real *gates,
+                       const real *G, real *da, int ld_da, real *dG, int n, int H);
 /* Tree-FC, apps/paper/tree-fc-cavs.cc:28-36 : h = act(z [+ bias] [+ x]).
  *  act 0 = relu (reference app), 1 = tanh.  bias, x may be NULL. */
-void or_treefc_fwd(const float *z, const float *bias, const float *x, float *h,
+void ORF(treefc_fwd)(const real *z, const real *bias, const real *x, real *h,
                    int n, int H, int act);
 /* dz = dh * act'(h) */
-void or_treefc_bwd(const float *dh_m, const float *dret, const float *h, float *dz,
+void ORF(treefc_bwd)(const real *dh_m, const real *dret, const real *h, real *dz,
                    int n, int H, int act);
 
 /* ------------------------------------------------------------------ model steps
@@ -173,17 +198,17 @@ typedef struct {
   int threads;    /* OpenMP threads for the GEMMs (0/1 = serial) */
 } or_config;
 
-/* All parameter pointers are row-major fp32; unused ones may be NULL.
+/* All parameter pointers are row-major arrays of `real`; unused ones may be NULL.
  *   Tree-LSTM: Emb[V,E] W[E,4H] U[4*H*H] Bv[4H]      (apps/paper/tree-lstm-cavs.cc:110-126)
  *   LSTM     : Emb[V,H] W[8*H*H] (U' then W') Bv[4H]  (apps/paper/seq-lstm-cavs.cc:49-59)
  *   Tree-FC  : W[2H,H] Bv[H]
  *   head     : Wfc[C,H] bfc[C] */
 typedef struct {
-  const float *Emb, *W, *U, *Bv, *Wfc, *bfc;
-} or_params;
+  const real *Emb, *W, *U, *Bv, *Wfc, *bfc;
+} ORF(params);
 typedef struct {
-  float *dEmb, *dW, *dU, *dBv, *dWfc, *dbfc;
-} or_grads;
+  real *dEmb, *dW, *dU, *dBv, *dWfc, *dbfc;
+} ORF(grads);
 
 /* graph [B,maxlen] int32 parent ids; x: vertex inputs packed by global vertex id
  * (word ids as floats, or [N,H] rows for Tree-FC with use_x); labels [N] floats
@@ -191,9 +216,9 @@ typedef struct {
  * Outputs (any may be NULL): loss_rows [N] (softmax) or [1]; graph_out [N,H] in
  * vertex-id order; dgraph_out [N,H]; msg_pool [N,2H or H] by tensor id;
  * grads are overwritten.  Returns N (>0) or a negative error. */
-int or_model_step(const or_config *cfg, const or_params *p, const int *graph, int B,
-                  int maxlen, const float *x, const float *labels, float *loss_rows,
-                  float *graph_out, float *dgraph_out, float *msg_pool, or_grads *g);
+int ORF(model_step)(const or_config *cfg, const ORF(params) *p, const int *graph, int B,
+                  int maxlen, const real *x, const real *labels, real *loss_rows,
+                  real *graph_out, real *dgraph_out, real *msg_pool, ORF(grads) *g);
 
 #ifdef __cplusplus
 }

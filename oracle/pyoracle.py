@@ -55,6 +55,29 @@ def _f32(a):
     return None if a is None else np.ascontiguousarray(a, dtype=np.float32)
 
 
+def _fx(a, precise):
+    """The array as the checker's `real`: fp32, or (precise) the same fp32 values widened to
+    double for the ord_* build, which evaluates the same dataflow in double."""
+    if a is None:
+        return None
+    if precise and np.asarray(a).dtype == np.float64:
+        return np.ascontiguousarray(a)  # a double result of an earlier stage: chained as it is
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    return a.astype(np.float64) if precise else a
+
+
+def _fn(name, precise):
+    return getattr(lib(), ("ord_" if precise else "or_") + name)
+
+
+def _dt(precise):
+    return np.float64 if precise else np.float32
+
+
+def _real(v, precise):
+    return C.c_double(v) if precise else C.c_float(v)
+
+
 def sched_trace(graph, batching=True, with_backward=True):
     """Returns dict(N, fwd=[round...], bwd=[round...], tids_to_jobids, round2offset);
     each round is dict(offset, exec, gather=[l0,l1], scatter=[l0,l1], gather_init)."""
@@ -109,21 +132,21 @@ def scatter_rows(out, ids, inp):
     return out
 
 
-def sgemm(tA, tB, A, B, alpha=1.0, beta=0.0, Cin=None):
-    A, B = _f32(A), _f32(B)
+def sgemm(tA, tB, A, B, alpha=1.0, beta=0.0, Cin=None, precise=False):
+    A, B = _fx(A, precise), _fx(B, precise)
     M, K = (A.shape[1], A.shape[0]) if tA else A.shape
     N = B.shape[0] if tB else B.shape[1]
-    Cm = np.zeros((M, N), np.float32) if Cin is None else _f32(Cin).copy()
-    lib().or_sgemm(int(tA), int(tB), M, N, K, C.c_float(alpha), _p(A), A.shape[1], _p(B),
-                   B.shape[1], C.c_float(beta), _p(Cm), N)
+    Cm = np.zeros((M, N), _dt(precise)) if Cin is None else _fx(Cin, precise).copy()
+    _fn("sgemm", precise)(int(tA), int(tB), M, N, K, _real(alpha, precise), _p(A), A.shape[1], _p(B),
+                          B.shape[1], _real(beta, precise), _p(Cm), N)
     return Cm
 
 
-def colsum(inp, accumulate_into=None):
-    inp = _f32(inp)
+def colsum(inp, accumulate_into=None, precise=False):
+    inp = _fx(inp, precise)
     n, w = inp.shape
-    out = np.zeros(w, np.float32) if accumulate_into is None else _f32(accumulate_into).copy()
-    lib().or_colsum(_p(out), _p(inp), w, n, w, int(accumulate_into is not None))
+    out = np.zeros(w, _dt(precise)) if accumulate_into is None else _fx(accumulate_into, precise).copy()
+    _fn("colsum", precise)(_p(out), _p(inp), w, n, w, int(accumulate_into is not None))
     return out
 
 
@@ -141,105 +164,108 @@ def embed_bwd(dtable, ids, dy):
     return dtable
 
 
-def softmax_xent(logits, labels):
-    logits, labels = _f32(logits), _f32(labels)
+def softmax_xent(logits, labels, precise=False):
+    logits, labels = _fx(logits, precise), _fx(labels, precise)
     n, Cc = logits.shape
-    loss = np.zeros(n, np.float32)
-    d = np.zeros((n, Cc), np.float32)
-    lib().or_softmax_xent(_p(loss), _p(d), _p(logits), _p(labels), n, Cc)
+    loss = np.zeros(n, _dt(precise))
+    d = np.zeros((n, Cc), _dt(precise))
+    _fn("softmax_xent", precise)(_p(loss), _p(d), _p(logits), _p(labels), n, Cc)
     return loss, d
 
 
-def treelstm_gates_fwd(xW, hU, hUf, G, bias):
-    xW, hU, hUf, G, bias = map(_f32, (xW, hU, hUf, G, bias))
+def treelstm_gates_fwd(xW, hU, hUf, G, bias, precise=False):
+    xW, hU, hUf, G, bias = (_fx(a, precise) for a in (xW, hU, hUf, G, bias))
     n, H = xW.shape[0], xW.shape[1] // 4
-    gates = np.zeros((n, 6 * H), np.float32)
-    msg = np.zeros((n, 2 * H), np.float32)
-    lib().or_treelstm_gates_fwd(_p(xW), 4 * H, _p(hU), _p(hUf), _p(G), _p(bias), _p(gates),
-                                _p(msg), n, H)
+    gates = np.zeros((n, 6 * H), _dt(precise))
+    msg = np.zeros((n, 2 * H), _dt(precise))
+    _fn("treelstm_gates_fwd", precise)(_p(xW), 4 * H, _p(hU), _p(hUf), _p(G), _p(bias), _p(gates),
+                                       _p(msg), n, H)
     return gates, msg
 
 
-def treelstm_gates_bwd(dmsg, dret, gates, G):
-    dmsg, dret, gates, G = map(_f32, (dmsg, dret, gates, G))
+def treelstm_gates_bwd(dmsg, dret, gates, G, precise=False):
+    dmsg, dret, gates, G = (_fx(a, precise) for a in (dmsg, dret, gates, G))
     n, H = dret.shape
-    dxW = np.zeros((n, 4 * H), np.float32)
-    dF = np.zeros((2 * n, H), np.float32)
-    dG = np.zeros((2 * n, 2 * H), np.float32)
-    lib().or_treelstm_gates_bwd(_p(dmsg), _p(dret), _p(gates), _p(G), _p(dxW), 4 * H, _p(dF),
-                                _p(dG), n, H)
+    dxW = np.zeros((n, 4 * H), _dt(precise))
+    dF = np.zeros((2 * n, H), _dt(precise))
+    dG = np.zeros((2 * n, 2 * H), _dt(precise))
+    _fn("treelstm_gates_bwd", precise)(_p(dmsg), _p(dret), _p(gates), _p(G), _p(dxW), 4 * H, _p(dF),
+                                       _p(dG), n, H)
     return dxW, dF, dG
 
 
-def lstm_gates_fwd(a, G, bias):
-    a, G, bias = map(_f32, (a, G, bias))
+def lstm_gates_fwd(a, G, bias, precise=False):
+    a, G, bias = (_fx(t, precise) for t in (a, G, bias))
     n, H = a.shape[0], a.shape[1] // 4
-    gates = np.zeros((n, 5 * H), np.float32)
-    msg = np.zeros((n, 2 * H), np.float32)
-    lib().or_lstm_gates_fwd(_p(a), 4 * H, _p(G), _p(bias), _p(gates), _p(msg), n, H)
+    gates = np.zeros((n, 5 * H), _dt(precise))
+    msg = np.zeros((n, 2 * H), _dt(precise))
+    _fn("lstm_gates_fwd", precise)(_p(a), 4 * H, _p(G), _p(bias), _p(gates), _p(msg), n, H)
     return gates, msg
 
 
-def lstm_gates_bwd(dmsg, dret, gates, G):
-    dmsg, dret, gates, G = map(_f32, (dmsg, dret, gates, G))
+def lstm_gates_bwd(dmsg, dret, gates, G, precise=False):
+    dmsg, dret, gates, G = (_fx(a, precise) for a in (dmsg, dret, gates, G))
     n, H = dret.shape
-    da = np.zeros((n, 4 * H), np.float32)
-    dG = np.zeros((n, 2 * H), np.float32)
-    lib().or_lstm_gates_bwd(_p(dmsg), _p(dret), _p(gates), _p(G), _p(da), 4 * H, _p(dG), n, H)
+    da = np.zeros((n, 4 * H), _dt(precise))
+    dG = np.zeros((n, 2 * H), _dt(precise))
+    _fn("lstm_gates_bwd", precise)(_p(dmsg), _p(dret), _p(gates), _p(G), _p(da), 4 * H, _p(dG), n, H)
     return da, dG
 
 
-def treefc_fwd(z, bias, x, act):
-    z = _f32(z)
+def treefc_fwd(z, bias, x, act, precise=False):
+    z = _fx(z, precise)
     n, H = z.shape
-    h = np.zeros((n, H), np.float32)
-    bias, x = _f32(bias), _f32(x)
-    lib().or_treefc_fwd(_p(z), _p(bias), _p(x), _p(h), n, H, int(act))
+    h = np.zeros((n, H), _dt(precise))
+    bias, x = _fx(bias, precise), _fx(x, precise)
+    _fn("treefc_fwd", precise)(_p(z), _p(bias), _p(x), _p(h), n, H, int(act))
     return h
 
 
-def treefc_bwd(dh_m, dret, h, act):
-    dh_m, dret, h = map(_f32, (dh_m, dret, h))
+def treefc_bwd(dh_m, dret, h, act, precise=False):
+    dh_m, dret, h = (_fx(a, precise) for a in (dh_m, dret, h))
     n, H = h.shape
-    dz = np.zeros((n, H), np.float32)
-    lib().or_treefc_bwd(_p(dh_m), _p(dret), _p(h), _p(dz), n, H, int(act))
+    dz = np.zeros((n, H), _dt(precise))
+    _fn("treefc_bwd", precise)(_p(dh_m), _p(dret), _p(h), _p(dz), n, H, int(act))
     return dz
 
 
 def model_step(model, graph, x, labels, params, *, H, E=0, V=0, Cc=0, loss="softmax",
                pairing="reference", batching=True, act=0, use_bias=False, use_x=False,
-               threads=1, want_grads=True):
-    """One fwd+bwd pass.  Returns dict(N, loss, graph_out, dgraph_out, msg_pool, grads)."""
+               threads=1, want_grads=True, precise=False):
+    """One fwd+bwd pass.  Returns dict(N, loss, graph_out, dgraph_out, msg_pool, grads).
+    precise: the same dataflow with every value and sum in double (ord_model_step); the
+    results come back as float64."""
     g = np.ascontiguousarray(graph, np.int32)
     B, maxlen = g.shape
-    x, labels = _f32(x), _f32(labels)
+    x, labels = _fx(x, precise), _fx(labels, precise)
+    dt = _dt(precise)
     cfg = _Config(MODEL[model], LOSS[loss], PAIR[pairing], int(batching), V, E, H, Cc, int(act),
                   int(use_bias), int(use_x), threads)
-    keep = {k: _f32(v) for k, v in params.items()}
+    keep = {k: _fx(v, precise) for k, v in params.items()}
     prm = _Params(*[_p(keep.get(k)) for k in ("Emb", "W", "U", "Bv", "Wfc", "bfc")])
     N = int(sum(int(np.argmax(r == -1)) + 1 for r in g))
     mw = H if model == "treefc" else 2 * H
     Ee = H if model == "lstm" else E
-    loss_rows = np.zeros(N if loss == "softmax" else 1, np.float32)
-    GO = np.zeros((N, H), np.float32)
-    dGO = np.zeros((N, H), np.float32)
-    pool = np.zeros((N, mw), np.float32)
+    loss_rows = np.zeros(N if loss == "softmax" else 1, dt)
+    GO = np.zeros((N, H), dt)
+    dGO = np.zeros((N, H), dt)
+    pool = np.zeros((N, mw), dt)
     grads = {}
     if want_grads:
         if model == "treelstm":
-            grads = dict(dEmb=np.zeros((V, Ee), np.float32), dW=np.zeros((Ee, 4 * H), np.float32),
-                         dU=np.zeros(4 * H * H, np.float32), dBv=np.zeros(4 * H, np.float32))
+            grads = dict(dEmb=np.zeros((V, Ee), dt), dW=np.zeros((Ee, 4 * H), dt),
+                         dU=np.zeros(4 * H * H, dt), dBv=np.zeros(4 * H, dt))
         elif model == "lstm":
-            grads = dict(dEmb=np.zeros((V, Ee), np.float32), dW=np.zeros(8 * H * H, np.float32),
-                         dBv=np.zeros(4 * H, np.float32))
+            grads = dict(dEmb=np.zeros((V, Ee), dt), dW=np.zeros(8 * H * H, dt),
+                         dBv=np.zeros(4 * H, dt))
         else:
-            grads = dict(dW=np.zeros((2 * H, H), np.float32), dBv=np.zeros(H, np.float32))
+            grads = dict(dW=np.zeros((2 * H, H), dt), dBv=np.zeros(H, dt))
         if loss == "softmax":
-            grads["dWfc"] = np.zeros((Cc, H), np.float32)
-            grads["dbfc"] = np.zeros(Cc, np.float32)
+            grads["dWfc"] = np.zeros((Cc, H), dt)
+            grads["dbfc"] = np.zeros(Cc, dt)
     gs = _Grads(*[_p(grads.get(k)) for k in ("dEmb", "dW", "dU", "dBv", "dWfc", "dbfc")])
-    rc = lib().or_model_step(C.byref(cfg), C.byref(prm), _p(g), B, maxlen, _p(x), _p(labels),
-                             _p(loss_rows), _p(GO), _p(dGO), _p(pool),
-                             C.byref(gs) if want_grads else None)
-    assert rc == N, f"or_model_step failed: {rc}"
+    rc = _fn("model_step", precise)(C.byref(cfg), C.byref(prm), _p(g), B, maxlen, _p(x), _p(labels),
+                                    _p(loss_rows), _p(GO), _p(dGO), _p(pool),
+                                    C.byref(gs) if want_grads else None)
+    assert rc == N, f"model_step failed: {rc}"
     return dict(N=N, loss=loss_rows, graph_out=GO, dgraph_out=dGO, msg_pool=pool, grads=grads)

@@ -1,15 +1,15 @@
 """End-to-end GPU parity: one forward+backward pass through the host runtime and the
 HIP backend against the oracle on the same seeded inputs.  Schedule and index lists
-bit-exact; fp32 losses, activations and gradients within 1e-4 relative / 1e-5 absolute."""
+bit-exact; fp32 losses, activations and gradients within 1e-4 relative / 1e-5 absolute of the
+oracle's dataflow evaluated in double precision (tolerance.py), at every site."""
 import numpy as np
 import pytest
 
 from cavs_amd import hip, session, synth
 from test_oracle_models import small_workload
+from tolerance import close
 
 pytestmark = pytest.mark.gpu
-
-RTOL, ATOL = 1e-4, 1e-5
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -19,19 +19,11 @@ def _gpu():
     assert torch.cuda.is_available(), "these tests need the MI355X"
 
 
-def close(got, want, what, rtol=RTOL, atol=ATOL):
-    got, want = np.asarray(got, np.float64).ravel(), np.asarray(want, np.float64).ravel()
-    assert got.shape == want.shape, what
-    scale = max(1.0, float(np.abs(want).max())) if want.size else 1.0
-    err = np.abs(got - want)
-    tol = atol * scale + rtol * np.abs(want)
-    assert (err <= tol).all(), f"{what}: max err {err.max():.3e} at {int(err.argmax())} (want {want[err.argmax()]:.4e})"
-
-
 def run_both(oracle, w, *, loss="softmax", pairing="reference", batching=True, **kw):
     print(f"[case] model={w['model']} N={w['N']} H={w['H']} loss={loss} pairing={pairing} batching={batching}", flush=True)
     want = oracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], H=w["H"], E=w["E"],
-                             V=w["V"], Cc=w["C"], loss=loss, pairing=pairing, batching=batching, **kw)
+                             V=w["V"], Cc=w["C"], loss=loss, pairing=pairing, batching=batching, precise=True,
+                             threads=16, **kw)
     s = session.Session(w["model"], H=w["H"], E=w["E"], V=w["V"], C_=w["C"], loss=loss, pairing=pairing,
                         opt=session.OPT_BATCHING if batching else 0, **kw)
     names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
@@ -87,35 +79,39 @@ def test_odd_sizes_take_the_unaligned_paths(oracle, model, kw):
     compare(got, want)
 
 
-@pytest.mark.parametrize("name,scale", [("C1", 0.25), ("C2", 0.25), ("C3", 0.125), ("C4", 0.0625)])
+@pytest.mark.parametrize("name,scale", [("C1", 0.25), ("C2", 0.25), ("C3", 0.125), ("C4", 0.0625), ("C5", 0.0625)])
 def test_benchmark_configs_scaled(oracle, name, scale):
-    """The benchmark batches (real graph shapes and batch sizes) at reduced widths so
-    the oracle finishes in seconds."""
-    w = synth.make_workload(name, scale=scale, B=None if name != "C4" else 32)
+    """The benchmark batches -- their own graphs, batch sizes (C4: 128 sequences, C5: 256 trees of up
+    to 511 vertices, N ~ 72 k), vocabularies and class counts (C4: the 10000-way head) -- at reduced
+    widths so that the oracle finishes in seconds."""
+    w = synth.make_workload(name, scale=scale)
     kw, loss = {}, "softmax"
     if w["model"] == "treefc":
         kw, loss = dict(act=1, use_bias=True, use_x=True), "root_sq"
-    if name == "C4":  # a 10000-way head at N~2k is slow on the scalar oracle; keep the vocabulary small
-        w["V"] = w["C"] = 50
-        w["x"] = np.floor(w["x"] % 50).astype(np.float32)
-        w["labels"] = np.floor(w["labels"] % 50).astype(np.float32)
-        w["params"]["Emb"] = w["params"]["Emb"][:50].copy()
-        w["params"]["Wfc"] = w["params"]["Wfc"][:50].copy()
-        w["params"]["bfc"] = w["params"]["bfc"][:50].copy()
     got, want = run_both(oracle, w, loss=loss, **kw)
     compare(got, want)
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3"])
 def test_benchmark_configs_at_full_size(oracle, name):
-    """The benchmark's own batches at their own widths against the oracle (it needs under a second
-    for these three; C4's 10000-way head and C5 are covered scaled above and through properties
-    below), at the same 1e-4 relative / 1e-5 absolute bar as the small cases."""
+    """The benchmark's own batches at their own widths against the oracle (it needs a second or
+    two for these three; C4 and C5 meet it at their own batch sizes and reduced widths above, and
+    at full size below), at the same 1e-4 relative / 1e-5 absolute bar as the small cases."""
     w = synth.make_workload(name)
     kw, loss = {}, "softmax"
     if w["model"] == "treefc":
         kw, loss = dict(act=1, use_bias=True, use_x=True), "root_sq"
     got, want = run_both(oracle, w, loss=loss, **kw)
+    compare(got, want)
+
+
+@pytest.mark.parametrize("name,B", [("C4", 8), ("C5", 6)])
+def test_benchmark_configs_at_full_width(oracle, name, B):
+    """C4 and C5 at their own widths (H = 512 with the 10000-way head; E = H = 1024 with trees of up
+    to 511 vertices) on a few samples of their batches, which is what the oracle can evaluate in
+    double within seconds: the values the wide kernels produce, end to end, against the oracle."""
+    w = synth.make_workload(name, B=B)
+    got, want = run_both(oracle, w)
     compare(got, want)
 
 
@@ -134,7 +130,8 @@ def test_steps_are_repeatable_and_sessions_reusable(oracle):
     np.testing.assert_array_equal(outs[0][0], outs[2][0])
     for k in ("dW", "dU", "dBv", "dWfc"):
         np.testing.assert_array_equal(outs[0][1][k], outs[2][1][k])
-    want = oracle.model_step("treelstm", b["graph"], b["x"], b["labels"], a["params"], H=16, E=12, V=a["V"], Cc=a["C"])
+    want = oracle.model_step("treelstm", b["graph"], b["x"], b["labels"], a["params"], H=16, E=12, V=a["V"], Cc=a["C"],
+                             precise=True)
     close(outs[1][0], want["loss"], "loss of second batch")
     s.close()
 
@@ -150,7 +147,7 @@ def test_device_resident_feeds_and_sgd(oracle):
     torch.cuda.synchronize()
     s.step(w["graph"], x, lab, backward=True, lr=0.5)
     g = s.grads()
-    want = oracle.model_step("lstm", w["graph"], w["x"], w["labels"], w["params"], H=16, V=w["V"], Cc=w["C"])
+    want = oracle.model_step("lstm", w["graph"], w["x"], w["labels"], w["params"], H=16, V=w["V"], Cc=w["C"], precise=True)
     close(g["dW"], want["grads"]["dW"], "dW")
     close(s.param("W", (8 * 16 * 16,)), w["params"]["W"] - np.float32(0.5) * g["dW"], "W after SGD", rtol=1e-6, atol=1e-7)
     assert s.timing("RNNForward") > 0 and s.timing("RNNBackward") > 0 and s.timing("GraphParsing") >= 0
@@ -201,7 +198,7 @@ def test_full_size_tree_lstm_properties():
     close(s.fetch("graph_out"), GO[idx], "graph_out under sample permutation", rtol=1e-5, atol=1e-6)
     gp = s.grads()
     for k in ("dW", "dU", "dBv", "dWfc", "dbfc"):
-        close(gp[k], g[k], k + " under sample permutation", rtol=2e-4, atol=2e-5)
+        close(gp[k], g[k], k + " under sample permutation")
     s.close()
 
 
@@ -225,7 +222,7 @@ def test_full_size_fused_rounds_equal_separate_launches(name):
     close(outs[0]["loss"], outs[1]["loss"], "loss")
     close(outs[0]["go"], outs[1]["go"], "graph_out")
     for k, v in outs[1]["grads"].items():
-        close(outs[0]["grads"][k], v, k, rtol=2e-4, atol=2e-5)
+        close(outs[0]["grads"][k], v, k)
 
 
 @pytest.mark.parametrize("H,limit", [(32, 0), (64, 0), (96, 0), (64, 20), (64, -1), (256, 0), (512, 0)])
@@ -236,11 +233,17 @@ def test_fused_rounds_match_oracle(oracle, model, kw, H, limit, pairing):
     above 64 rows (32x32 tiles, or 16x16 with four wavefronts), between 17 and 64 (16x16 tiles)
     and down to one row.  limit=20 mixes fused and separate rounds in one step, -1 never fuses."""
     w = small_workload(model, 91, B=70, H=H, E=12, V=31, C=5)
+    if model == "treefc" and H >= 256:
+        # small_workload draws W from U(-0.4, 0.4) whatever H is.  A sum of 2H = 1024 such terms has a
+        # standard deviation of 7: each level of the tree multiplies a rounding error of its inputs by
+        # about that, and after ten levels no fp32 summation order is within 1e-5 of the exact value.
+        # Scaled to the spread the benchmark's own U(-0.1, 0.1) has at H = 256.
+        w["params"]["W"] = (w["params"]["W"] * np.float32(0.25 * np.sqrt(256.0 / H))).astype(np.float32)
     E = H if model == "lstm" else 12
     loss = "softmax" if model != "treefc" else "root_sq"
     print(f"[case] fused rounds {model} {kw} H={H} limit={limit} pairing={pairing} N={w['N']}", flush=True)
     want = oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=H, E=E, V=31, Cc=5, pairing=pairing,
-                             loss=loss, **kw)
+                             loss=loss, precise=True, threads=16, **kw)
     s = session.Session(model, H=H, E=E, V=31, C_=5, pairing=pairing, fused_round_rows=limit, loss=loss, **kw)
     names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
              "treefc": ("W", "Bv") if kw.get("use_bias") else ("W",)}[model]
@@ -252,11 +255,7 @@ def test_fused_rounds_match_oracle(oracle, model, kw, H, limit, pairing):
                msg_pool=s.fetch("msg_pool"), grads=s.grads(), trace=s.schedule_trace())
     fused_flops = s.counter("round_flops")
     s.close()
-    # Tree-FC at H >= 256: each output is a sum of 2H terms taken in another order than the oracle's,
-    # pushed through a saturating activation level after level; the separate-launch path (LDS-tiled
-    # GEMM) deviates from the oracle by the same 2e-5 there
-    tol = dict(rtol=2e-4, atol=5e-5) if model == "treefc" and H >= 256 else {}
-    compare(got, want, **tol)
+    compare(got, want)
     assert (fused_flops > 0) == (limit >= 0), fused_flops
 
 
@@ -270,7 +269,8 @@ def test_backward_rounds_as_one_launch_or_two(oracle, model, kw, pairing):
     E = H if model == "lstm" else 12
     loss = "softmax" if model != "treefc" else "root_sq"
     w = small_workload(model, 57, B=40, H=H, E=12, V=31, C=5)
-    want = oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=H, E=E, V=31, Cc=5, pairing=pairing, loss=loss, **kw)
+    want = oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=H, E=E, V=31, Cc=5, pairing=pairing, loss=loss,
+                             precise=True, threads=16, **kw)
     names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
              "treefc": ("W", "Bv") if kw.get("use_bias") else ("W",)}[model]
     if loss == "softmax":
@@ -332,14 +332,14 @@ def test_training_steps_with_the_row_sparse_embedding_update(oracle, model):
     for step, (bi, lr) in enumerate(plan):
         w = batches[bi]
         print(f"[case] {model} sgd step {step} batch {bi} lr {lr}", flush=True)
-        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_, precise=True, threads=16)
         s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
         got = s.grads()
         for k in names:
-            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", rtol=3e-4, atol=3e-5)
+            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}")
             p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
     for k in names:
-        close(s.param(k, p[k].shape), p[k], f"{k} after the steps", rtol=3e-4, atol=3e-5)
+        close(s.param(k, p[k].shape), p[k], f"{k} after the steps")
     s.close()
 
 
@@ -366,14 +366,14 @@ def test_the_packed_copy_of_the_recurrent_weights_follows_every_writer(oracle, m
         if step == 2:
             p[rec] = (p[rec][::-1] * np.float32(0.5)).astype(np.float32)
             s.set_params({rec: p[rec]})
-        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_)
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=E, V=V, Cc=C_, precise=True, threads=16)
         s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
-        close(s.fetch("graph_out"), want["graph_out"], f"graph_out at step {step}", rtol=3e-4, atol=3e-5)
+        close(s.fetch("graph_out"), want["graph_out"], f"graph_out at step {step}")
         got = s.grads()
         for k in names:
-            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", rtol=3e-4, atol=3e-5)
+            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}")
             p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
-    close(s.param(rec, p[rec].shape), p[rec], f"{rec} after the steps", rtol=3e-4, atol=3e-5)
+    close(s.param(rec, p[rec].shape), p[rec], f"{rec} after the steps")
     s.close()
 
 

@@ -8,9 +8,32 @@ import pytest
 
 from cavs_amd import hip, synth
 
+from tolerance import close
+
 pytestmark = pytest.mark.gpu
 
-RTOL, ATOL = 1e-4, 1e-5
+_ARITHMETIC = ("sgemm", "colsum", "softmax_xent", "treelstm_gates_fwd", "treelstm_gates_bwd", "lstm_gates_fwd",
+               "lstm_gates_bwd", "treefc_fwd", "treefc_bwd", "model_step")
+
+
+class _InDouble:
+    """The oracle with its arithmetic evaluated in double (the ord_* build of the same sources):
+    what the fp32 kernels are held to 1e-4 relative / 1e-5 absolute against.  Row movement and
+    index work pass through unchanged (they are compared bit for bit)."""
+
+    def __init__(self, oracle):
+        self._o = oracle
+
+    def __getattr__(self, name):
+        fn = getattr(self._o, name)
+        if name in _ARITHMETIC:
+            return lambda *a, **k: fn(*a, **{"precise": True, **k})
+        return fn
+
+
+@pytest.fixture
+def oracle(oracle):
+    return _InDouble(oracle)
 
 
 @pytest.fixture(scope="module")
@@ -32,12 +55,6 @@ def _release_device_temporaries(g):
 
 def rng(seed):
     return synth.SplitMix64(seed)
-
-
-def close(got, want, what="", rtol=RTOL, atol=ATOL):
-    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
-    scale = max(1.0, float(np.abs(want).max())) if want.size else 1.0
-    np.testing.assert_allclose(got, want, rtol=rtol, atol=atol * scale, err_msg=what)
 
 
 # ---------------------------------------------------------------- row movement
@@ -370,11 +387,11 @@ def test_colsum(g, oracle, n, w):
     exact = X.astype(np.float64).sum(0)
     out = g.zeros(w, fill=float("nan"))
     g.call("cavs_colsum", g.P(out), g.P(g.devf(X)), w, n, w, 0, g.stream())
-    close(g.host(out), exact, rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    close(g.host(out), exact)
     acc0 = r.bulk_normal(w)
     out = g.devf(acc0)
     g.call("cavs_colsum", g.P(out), g.P(g.devf(X)), w, n, w, 1, g.stream())
-    close(g.host(out), exact + acc0, rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    close(g.host(out), exact + acc0)
 
 
 @pytest.mark.parametrize("V,E,n", [(23, 6, 31), (21701, 300, 500), (1000, 128, 64), (21701, 300, 2482), (50, 512, 1100)])
@@ -399,7 +416,7 @@ def test_embedding(g, oracle, V, E, n):
     want = oracle.embed_bwd(d0.copy(), ids, dy)
     dt = g.devf(d0)
     g.call("cavs_embed_bwd", g.P(dt), g.P(g.devf(ids)), g.P(g.devf(dy)), E, n, E, g.stream())
-    close(g.host(dt), want, atol=1e-5 * np.sqrt(n))
+    close(g.host(dt), want)
 
 
 # (rows of 512 to 16384 classes in whole float4s go a workgroup per row, in four register sizes;
@@ -419,9 +436,9 @@ def test_softmax_xent_bias_sgd(g, oracle, n, C_):
     out = g.zeros(n, C_)
     g.call("cavs_bias_add_rows", g.P(out), g.P(g.devf(logits)), g.P(g.devf(bias)), n, C_, g.stream())
     np.testing.assert_array_equal(g.host(out), logits + bias[None, :])
-    w = g.devf(logits)
-    g.call("cavs_sgd", g.P(w), g.P(g.devf(d_w)), 0.5, n * C_, g.stream())
-    np.testing.assert_array_equal(g.host(w), logits - np.float32(0.5) * d_w)
+    w, grad = g.devf(logits), d_w.astype(np.float32)
+    g.call("cavs_sgd", g.P(w), g.P(g.devf(grad)), 0.5, n * C_, g.stream())
+    np.testing.assert_array_equal(g.host(w), logits - np.float32(0.5) * grad)
 
 
 def test_elementwise_family(g):
@@ -634,7 +651,7 @@ def test_fused_tree_lstm_rounds(g, oracle, n, H):
     g.call("cavs_treelstm_round_bwd_children", g.P(dxW), 4 * H, g.P(dF), g.P(UT), g.P(d_child), g.P(d_dpool), n, H, g.stream())
     close(g.host(dxW), dxW_w, "dxW")
     close(g.host(dF), dF_w, "dF")
-    close(g.host(d_dpool), dpool_w, "dpool", rtol=2e-4, atol=2e-5)
+    close(g.host(d_dpool), dpool_w, "dpool")
 
     # a round of leaves: no children, nothing scattered downwards
     gates_l, _ = oracle.treelstm_gates_fwd(xW, 0 * hU_w, 0 * hUf_w, 0 * G_w, bias)
@@ -729,10 +746,10 @@ def test_backward_rounds_with_the_childrens_gate_gradients_folded_in(g, oracle, 
         g.call("cavs_treelstm_round_bwd_children_gates", g.P(dxW), 4 * H, g.P(dF), g.P(dc), g.P(UT), g.P(d_kids) + 4 * 2 * lo,
                g.P(d_gates), g.P(d_G), g.P(d_dgo), g.P(d_rows), lo, cnt, L, H, g.stream())
     got_x, got_F = g.host(dxW), g.host(dF)
-    close(got_x[reached], dxW_w[reached], "dxW", rtol=2e-4, atol=2e-5)
+    close(got_x[reached], dxW_w[reached], "dxW")
     internal = reached.copy()
     internal[:L] = False
-    close(got_F[np.repeat(internal, 2)], dF_w[np.repeat(internal, 2)], "dF", rtol=2e-4, atol=2e-5)
+    close(got_F[np.repeat(internal, 2)], dF_w[np.repeat(internal, 2)], "dF")
     # rows no message reaches are left alone, and so are the leaves' rows of dF and dc
     assert (got_x[~reached] == -3.0).all()
     assert (got_F[: 2 * L] == -3.0).all() and (g.host(dc)[:L] == -3.0).all()
@@ -1090,7 +1107,7 @@ def test_column_sums_of_permuted_blocks(g, n, bw, perm):
     dX = g.devf(X)
     g.call("cavs_colsum_blocks", g.P(out), g.P(dX), ld, n, bw, nb, dst, g.P(ws), nbytes, g.stream())
     first = g.host(out).copy()
-    close(first, want.ravel(), rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    close(first, want.ravel())
     g.call("cavs_colsum_blocks", g.P(out), g.P(dX), ld, n, bw, nb, dst, g.P(ws), nbytes, g.stream())
     np.testing.assert_array_equal(g.host(out), first)           # fixed summation order
     # the same in two halves: the chunk sums left in the workspace, added up (permuted, and
@@ -1104,7 +1121,7 @@ def test_column_sums_of_permuted_blocks(g, n, bw, perm):
     job = (hip.Task * 1)(hip.Task(hip.TASK_BLOCKS_SGD, 0.5, bw, nb, bmap, g.P(d_w), g.P(ws), g.P(out2), None))
     g.call("cavs_run_tasks", 1, job, g.stream())
     second = g.host(out2).copy()
-    close(second, want.ravel(), rtol=1e-4, atol=1e-5 * np.sqrt(n))
+    close(second, want.ravel())
     np.testing.assert_array_equal(g.host(d_w), w0 - np.float32(0.5) * second)
     job[0].p0 = None                                            # gradient only, again: same bits
     g.call("cavs_run_tasks", 1, job, g.stream())
@@ -1138,7 +1155,7 @@ def test_children_gradient_product_with_scatter(g, n, H, K, nchild):
     d = g.devf(dpool)
     g.call("cavs_round_bwd_children", g.P(g.devf(dA)), K + 4, K, g.P(g.devf(BT)), nchild * H, nchild, g.P(g.devi(child)),
            g.P(d), mw, n, H, g.stream())
-    close(g.host(d), want, "dpool", rtol=2e-4, atol=2e-5)
+    close(g.host(d), want, "dpool")
 
 
 @pytest.mark.parametrize("model,L,m,n,H", [("lstm", 20, 2, 3, 32), ("lstm", 300, 60, 70, 64), ("lstm", 2600, 600, 1100, 32),
@@ -1223,7 +1240,7 @@ def test_chain_and_tree_fc_backward_rounds_with_the_childrens_pointwise_part_fol
             g.call("cavs_treefc_round_bwd_children_act", g.P(dA), g.P(d_WT), g.P(d_kids) + 4 * 2 * lo, g.P(d_h), g.P(d_dgo), g.P(d_rows),
                    lo, cnt, H, act, g.stream())
     got = g.host(dA)
-    close(got[reached], dA_w[reached], "dA", rtol=2e-4, atol=2e-5)
+    close(got[reached], dA_w[reached], "dA")
     assert (got[~reached] == -3.0).all()
     assert (g.host(dc)[:L] == -3.0).all()
 

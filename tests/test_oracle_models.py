@@ -150,3 +150,72 @@ def test_sum_abs_loss_has_the_gradient_of_a_plain_sum(oracle):
     assert (res["graph_out"] < 0).any()
     _close(res["loss"], [np.abs(res["graph_out"].astype(np.float64)).sum()], "sum|h|")
     np.testing.assert_array_equal(res["dgraph_out"], np.ones_like(res["dgraph_out"]))
+
+
+# ---- the double-precision build of the same sources (ord_*): what the fp32 GPU results are
+# held to the path's tolerance against.  It must (a) be the same dataflow as the fp32 build and
+# (b) really hold every value and sum in double -- a single float intermediate would leave an
+# error of ~1e-7 relative, far above the 1e-11 asked for here.
+TIGHT = dict(rtol=1e-10, atol=1e-12)
+
+
+def _compare_tight(res, ref):
+    assert res["loss"].dtype == np.float64
+    _close(res["loss"], ref["loss"], "loss", **TIGHT)
+    _close(res["graph_out"], ref["graph_out"], "graph_out", **TIGHT)
+    _close(res["dgraph_out"], ref["dgraph_out"], "dgraph_out", **TIGHT)
+    for k, v in res["grads"].items():
+        if k in ref["grads"]:
+            _close(v, ref["grads"][k], k, **TIGHT)
+
+
+@pytest.mark.parametrize("model,kw", CASES)
+@pytest.mark.parametrize("loss", ["softmax", "root_sq"])
+def test_double_build_equals_fp64_textbook_to_1e10(oracle, model, kw, loss):
+    w = small_workload(model, 61)
+    ref = textbook.per_sample(model, w["graph"], w["x"], w["labels"], w["params"], w["H"], loss=loss, **kw)
+    res = _run_oracle(oracle, w, loss=loss, pairing="rowid", precise=True, **kw)
+    _compare_tight(res, ref)
+    # the reference pairing on a skewed batch: autograd over the round-based dataflow
+    tr = oracle.sched_trace(w["graph"])
+    ref = textbook.round_based(model, w["graph"], tr, w["x"], w["labels"], w["params"], w["H"],
+                               loss=loss, pairing="reference", **kw)
+    res = _run_oracle(oracle, w, loss=loss, pairing="reference", precise=True, **kw)
+    _compare_tight(res, ref)
+    # serial scheduling, weight gradients accumulated per round
+    ref = textbook.per_sample(model, w["graph"], w["x"], w["labels"], w["params"], w["H"], loss=loss, **kw)
+    res = _run_oracle(oracle, w, loss=loss, batching=False, precise=True, **kw)
+    _compare_tight(res, ref)
+
+
+@pytest.mark.parametrize("model,kw", CASES)
+def test_double_build_and_fp32_build_are_the_same_dataflow(oracle, model, kw):
+    w = small_workload(model, 62)
+    for pairing in ("reference", "rowid"):
+        f32 = _run_oracle(oracle, w, pairing=pairing, **kw)
+        f64 = _run_oracle(oracle, w, pairing=pairing, precise=True, **kw)
+        _compare(f32, f64)
+
+
+def test_double_build_of_the_ops(oracle):
+    r = synth.SplitMix64(63)
+    A = r.bulk_uniform(7 * 33, -1, 1).reshape(7, 33)
+    B = r.bulk_uniform(33 * 5, -1, 1).reshape(33, 5)
+    C0 = r.bulk_uniform(35, -1, 1).reshape(7, 5)
+    exact = 0.75 * (A.astype(np.float64) @ B.astype(np.float64)) + 0.5 * C0
+    got = oracle.sgemm(0, 0, A, B, alpha=0.75, beta=0.5, Cin=C0, precise=True)
+    assert got.dtype == np.float64
+    np.testing.assert_allclose(got, exact, rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(oracle.sgemm(1, 1, A.T.copy(), B.T.copy(), precise=True),
+                               A.astype(np.float64) @ B.astype(np.float64), rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(oracle.colsum(A, precise=True), A.astype(np.float64).sum(0), rtol=1e-14)
+    import torch
+
+    logits = r.bulk_uniform(6 * 9, -3, 3).reshape(6, 9)
+    labels = np.array([0, 8, 3, 3, 1, 5], np.float32)
+    t = torch.tensor(logits, dtype=torch.float64, requires_grad=True)
+    rows = torch.nn.functional.cross_entropy(t, torch.tensor(labels, dtype=torch.long), reduction="none")
+    rows.mean().backward()
+    loss, d = oracle.softmax_xent(logits, labels, precise=True)
+    np.testing.assert_allclose(loss, rows.detach().numpy(), rtol=1e-12)
+    np.testing.assert_allclose(d, t.grad.numpy(), rtol=1e-11, atol=1e-14)
