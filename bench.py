@@ -29,6 +29,10 @@ HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, profiles/bench_C3_hbm_traffic_pmc.txt
 PMC_TRAFFIC_BYTES = {("C3", "round"): 17.56e6}
+# a constant taken from the profile named, not a counter read during this run
+PMC_TRAFFIC_SOURCE = {k: f"profiles/bench_{k[0]}_hbm_traffic_pmc.txt (two rocprofv3 --pmc runs of this command, FETCH_SIZE and "
+                         "WRITE_SIZE per dispatch of the class; a constant copied from there, not read in this run)"
+                      for k in PMC_TRAFFIC_BYTES}
 
 
 def model_kwargs(w):
@@ -70,7 +74,24 @@ def cpu_baseline(w, budget_s=12.0):
     for _ in range(2):
         pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **dict(args, threads=1))
     el1 = time.perf_counter() - t1
-    return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port",
+    # configuration C1 as the survey defines it: the chain LSTM (V=1000, E=H=128, T=20, B=16) on the
+    # reference's CPU path -- its serial scheduler (cavs/midend/graph_scheduler.cc:83-167), one
+    # forward+backward step, single thread
+    from cavs_amd import synth
+
+    c1 = synth.make_workload("C1")
+    c1_args = dict(H=c1["H"], E=c1["E"], V=c1["V"], Cc=c1["C"], threads=1, batching=False)
+    pyoracle.model_step(c1["model"], c1["graph"], c1["x"], c1["labels"], c1["params"], **c1_args)  # warm
+    t2 = time.perf_counter()
+    n1 = 0
+    while n1 < 3 or (time.perf_counter() - t2 < 2.0 and n1 < 50):
+        pyoracle.model_step(c1["model"], c1["graph"], c1["x"], c1["labels"], c1["params"], **c1_args)
+        n1 += 1
+    el2 = time.perf_counter() - t2
+    c1_entry = dict(value=round(c1["B"] * n1 / el2, 3), unit="samples/s", cores=1, kind="port", ms_per_step=round(1e3 * el2 / n1, 3),
+                    sample=f"{n1} forward+backward steps of the C1 batch (B={c1['B']}, N={c1['N']}) on the serial scheduler "
+                           f"(one vertex per round, no batching) in {el2:.1f} s on one thread")
+    return dict(value=round(w["B"] * steps / el, 3), unit="samples/s", cores=threads, kind="port", C1=c1_entry,
                 host=dict(nproc=os.cpu_count(), affinity=len(os.sched_getaffinity(0)), omp_threads=threads),
                 sample=f"{steps} full fwd+bwd step(s) of the {w['name']} batch (B={w['B']}, N={w['N']}) "
                        f"in {el:.1f} s with {threads} OpenMP threads; CPU restatement of the reference's "
@@ -114,8 +135,44 @@ def front_end_modes(w, steps=60, warmup=30):
     return out
 
 
-def measure(a, workload, steps, warmup, n_pool):
-    """Times `steps` training steps of one workload and returns the fields of the JSON line."""
+class StepClock:
+    """One event on the session's stream after every timed step: the intervals between
+    consecutive events are the device's time per step in the steady state of the pipeline
+    (the host runs ahead), whose median is reported next to the mean of the timed region."""
+
+    def __init__(self, stream, n):
+        import ctypes as C
+
+        from cavs_amd import hip
+
+        self.hip, self.stream, self.C = hip, stream, C
+        self.events = []
+        for _ in range(n + 1):
+            e = C.c_void_p()
+            hip.call("cavs_event_create", C.byref(e))
+            self.events.append(e)
+        self.k = 0
+
+    def tick(self):
+        self.hip.call("cavs_event_record", self.events[self.k], self.stream)
+        self.k += 1
+
+    def intervals_ms(self):
+        out, ms = [], self.C.c_float()
+        for a, b in zip(self.events[: self.k - 1], self.events[1: self.k]):
+            self.hip.call("cavs_event_elapsed_ms", self.C.byref(ms), a, b)
+            out.append(ms.value)
+        return out
+
+    def close(self):
+        for e in self.events:
+            self.hip.call("cavs_event_destroy", e)
+
+
+def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, profile=True):
+    """Times `steps` training steps of one workload and returns the fields of the JSON line.
+    schedule / plan_cache: who builds the round schedule and whether plans are cached
+    (cavs_session_config); profile=False skips the per-kernel-class pass."""
     import torch
 
     from cavs_amd import session
@@ -124,7 +181,8 @@ def measure(a, workload, steps, warmup, n_pool):
     w0 = pool[0]
     kw = model_kwargs(w0)
     s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
-                        opt=session.OPT_BATCHING, fused_round_rows=a.fused_round_rows, **kw)
+                        opt=session.OPT_BATCHING, fused_round_rows=a.fused_round_rows, schedule=schedule,
+                        plan_cache=plan_cache, **kw)
     s.set_params(w0["params"])
     feeds = []
     for w in pool:  # inputs resident in HBM before the timed region
@@ -152,17 +210,36 @@ def measure(a, workload, steps, warmup, n_pool):
         settle = 10 + min(5000, int(a.settle_ms * 1e-3 / per_step))
         run(10, settle - 10)
     run(0, warmup)
+    clock = StepClock(s.stream, steps)
+    parse_ms = []
     s.sync()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    run(warmup, steps)
+    clock.tick()
+    for i in range(warmup, warmup + steps):
+        g, x, lab = feeds[i % len(feeds)]
+        s.step(g, x, lab, backward=True, lr=a.lr)
+        clock.tick()
+        parse_ms.append(s.timing("GraphParsing"))
     s.sync()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
     ms_per_step = 1e3 * elapsed / steps
+    median_ms = float(np.median(clock.intervals_ms()))
+    clock.close()
     # host side of the last timed step (the profiled pass below slows the host down)
     host_ms = {k: round(s.timing(k), 4) for k in ("GraphParsing", "HostSchedule", "HostWait", "HostStep")}
+    host_ms["GraphParsing_median"] = round(float(np.median(parse_ms)), 4)
     value = w0["B"] * steps / elapsed
+    if not profile:
+        out = {"value": round(value, 2), "unit": "samples/s", "steps": steps, "ms_per_step": round(ms_per_step, 4),
+               "median_ms_per_step": round(median_ms, 4), "GraphParsing_ms": host_ms["GraphParsing_median"],
+               "HostSchedule_ms": host_ms["HostSchedule"], "plan_hits": s.counter("plan_hits"),
+               "plan_misses": s.counter("plan_misses")}
+        s.close()
+        del feeds
+        torch.cuda.empty_cache()
+        return out, w0
 
     # Roofline of the dominant kernel: the same steps again with the kernels of every entry point
     # stamping a start and a stop event themselves (the interval a kernel trace reports) on the
@@ -210,7 +287,7 @@ def measure(a, workload, steps, warmup, n_pool):
 
     out = {
         "value": round(value, 2), "unit": "samples/s", "steps": steps, "warmup": warmup,
-        "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step": round(ms_per_step, 4), "median_ms_per_step": round(median_ms, 4),
         "config": {"workload": f"{workload}: {w0['model']} V={w0['V']} E={w0['E']} H={w0['H']} B={w0['B']} "
                                f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing,
@@ -219,6 +296,7 @@ def measure(a, workload, steps, warmup, n_pool):
                    "untimed_settle_steps": settle},
         "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
                      "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": traffic,
+                     "traffic_source": PMC_TRAFFIC_SOURCE.get((workload, dom_name)) if traffic else None,
                      "kernel": dom["kernel"],
                      "avg_launch_us": round(1e3 * dom["ms"] / dom["n"], 3) if dom["n"] else None,
                      "flops_per_launch": round(dom["flops"] / dom["n"], 1) if dom["n"] else None},
@@ -259,6 +337,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-front-end", action="store_true",
                     help="skip the 'front_end' field (the step through Session::Run in its three execution modes)")
+    ap.add_argument("--no-schedule-modes", action="store_true",
+                    help="skip 'schedule_modes' (the step with the schedule built on the host / on the GPU / from the plan cache)")
     ap.add_argument("--host-feeds", action="store_true",
                     help="feed x and labels from pageable host memory every step (PCIe-inclusive rate; not the headline value)")
     ap.add_argument("--fused-round-rows", type=int, default=0,
@@ -278,7 +358,8 @@ def main():
     out = {
         "metric": "train samples/sec (fwd+bwd) Tree-LSTM h=512 bs=64; % HBM/MFMA peak",
         "value": res["value"], "unit": res["unit"], "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": res["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": res["ms_per_step"], "median_ms_per_step": res["median_ms_per_step"],
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": res["config"], "roofline": res["roofline"], "kernels": res["kernels"], "timers_ms": res["timers_ms"],
     }
@@ -286,6 +367,17 @@ def main():
     # workload about 15 % slower)
     if not a.no_front_end and w0["model"] in ("treelstm", "lstm"):
         out["front_end"] = front_end_modes(w0)
+        # the same step as a user of the reference's API gets it: Session::Run with host feeds
+        out["session_run"] = dict(out["front_end"]["lowered"], path="Sym / GraphSupport / Session::Run, vertex function "
+                                  "lowered onto the fused round kernels, host feeds, optimizer as an op of the main scope")
+    if not a.no_schedule_modes:
+        # who builds the round schedule and the index lists: the host scheduler (the headline above),
+        # the GPU (cavs_schedule_arena), or the plan cache replaying a structure seen before
+        modes = {}
+        for name, sched, cache in (("host", "host", 0), ("device", "device", 0), ("cached", "host", a.pool)):
+            modes[name], _ = measure(a, a.workload, a.steps, a.warmup, a.pool, schedule=sched, plan_cache=cache, profile=False)
+        out["schedule_modes"] = modes
+        out["timers_ms"]["GraphParsing_by_mode"] = {k: v["GraphParsing_ms"] for k, v in modes.items()}
     if a.also.lower() != "none":
         out["also"] = {}
         for name in a.also.split(","):
@@ -293,7 +385,8 @@ def main():
                 continue
             big = name == "C5"
             also, _ = measure(a, name, 20 if big else 100, 5 if big else 50, 2 if big else 4)
-            out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "config", "roofline", "kernels")}
+            out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "median_ms_per_step",
+                                                      "config", "roofline", "kernels")}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
     print(json.dumps(out))

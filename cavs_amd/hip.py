@@ -121,17 +121,20 @@ _SIGS = {
     "cavs_fused_launch": [_P, C.POINTER(_P), _I, C.POINTER(_P), _I, C.POINTER(_I), C.POINTER(_I), _I, _P],
     "cavs_fused_release": [_P],
     "cavs_schedule_frontier": [_P, _I, _P, _P, _P, _P, _P, _P, _P],
+    "cavs_schedule_arena": [_P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, C.c_long, _P, _P, _Z, _P],
 }
 _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z,
             "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
             "cavs_clip_grads_workspace": _Z, "cavs_sgemm_group_workspace": _Z, "cavs_fc_softmax_xent_parts": _I,
             "cavs_colsum_parts": _I, "cavs_round_packed_ok": _I, "cavs_lstm_round_packed_ok": _I,
-            "cavs_sgemm_splitk_static_max_bytes": _Z}
+            "cavs_sgemm_splitk_static_max_bytes": _Z,
+            "cavs_schedule_arena_scratch": _Z}
 _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I],
             "cavs_fc_softmax_xent_workspace": [_I, _I, _I], "cavs_colsum_blocks_workspace": [_I, _I, _I],
             "cavs_clip_grads_workspace": [_I], "cavs_sgemm_group_workspace": [_I, C.POINTER(GemmDesc)],
             "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I], "cavs_round_packed_ok": [_I, _I],
-            "cavs_lstm_round_packed_ok": [_I, _I], "cavs_sgemm_splitk_static_max_bytes": []}
+            "cavs_lstm_round_packed_ok": [_I, _I], "cavs_sgemm_splitk_static_max_bytes": [],
+            "cavs_schedule_arena_scratch": [_I, _I]}
 
 EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)
 EW_UNARY = dict(assign=0, neg=1, abs=2, square=3, sigmoid=4, tanh=5, relu=6)

@@ -98,7 +98,9 @@ int cavs_session_total_length(cavs_session *s) { return s ? s->engine.total_leng
 
 int cavs_session_schedule_trace(cavs_session *s, int *out, int cap) {
   if (!s) return 0;
-  return emit(s->engine.schedule().trace(true), out, cap);
+  std::vector<int> t;
+  if (guarded([&] { t = s->engine.schedule().trace(true); }) != CAVS_OK) return 0;
+  return emit(t, out, cap);
 }
 
 int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int with_backward, int *out,
@@ -109,6 +111,37 @@ int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int w
     g_error = err;
     return 0;
   }
+  return emit(sch.trace(with_backward != 0), out, cap);
+}
+
+int cavs_schedule_index_lists(const int *graph, int B, int maxlen, int nchild, int pairing, int fused_limit, int *t2j,
+                              int *pair, int *child, int *roots, int *kid_rows, int *orphans, int *n_orphans) {
+  cavs::Schedule sch;
+  std::string err = cavs::build_schedule(graph, B, maxlen, true, &sch);
+  if (err.empty() && sch.executed != sch.N) err = "the batch holds a single-vertex sample";
+  if (err.empty() && (nchild < 1 || nchild > 2 || pairing < 0 || pairing > 1)) err = "bad nchild or pairing";
+  if (err.empty() && !(t2j && pair && child && roots)) err = "null output";
+  if (err.empty()) err = cavs::build_index_lists(sch, nchild, pairing, t2j, pair, child, roots);
+  if (!err.empty()) {
+    g_error = err;
+    return 0;
+  }
+  if (n_orphans) {
+    int n = 0;
+    const bool ok = kid_rows && orphans && cavs::build_forest_lists(sch, nchild, fused_limit, pair, child, kid_rows, orphans, &n);
+    *n_orphans = ok ? n : -1;
+  }
+  return sch.N;
+}
+
+int cavs_schedule_trace_from_lists(int B, int maxlen, int N, int nchild, const int *round2offset, int R, const int *t2j,
+                                   const int *pair, const int *child, const int *roots, int with_backward, int *out, int cap) {
+  if (B <= 0 || N <= 0 || R < 0 || !round2offset || !t2j || !pair || !child || !roots) {
+    g_error = "bad arguments";
+    return 0;
+  }
+  cavs::Schedule sch;
+  cavs::schedule_from_lists(B, maxlen, N, nchild, round2offset, R, t2j, pair, child, roots, &sch);
   return emit(sch.trace(with_backward != 0), out, cap);
 }
 

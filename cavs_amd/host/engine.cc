@@ -70,6 +70,12 @@ Engine::~Engine() {
   for (auto &e : ev_) cavs_event_destroy(e);
   for (auto &e : idx_copied_) cavs_event_destroy(e);
   for (auto &e : prof_events_) cavs_event_destroy(e);
+  if (sched_stream_) {
+    cavs_stream_sync(sched_stream_);
+    cavs_stream_destroy(sched_stream_);
+  }
+  for (auto &d : dsched_)
+    if (d.free_ev) cavs_event_destroy(d.free_ev);
   if (own_stream_) cavs_stream_destroy(stream_);
 }
 
@@ -246,7 +252,7 @@ void Engine::ensure(DeviceArray<float> &a, size_t n) {
 void Engine::reserve_edges() {
   const size_t H = cfg_.H, N = N_;
   if ((size_t)cap_ < N) cap_ = (int)grow(N, cap_);
-  if (rcap_ < sched_.max_round) rcap_ = (int)grow(sched_.max_round, rcap_);
+  if (rcap_ < sched_->max_round) rcap_ = (int)grow(sched_->max_round, rcap_);
   const size_t cap = cap_, rc = rcap_, mw = mw_;
   auto R = [&](DeviceArray<float> &a, size_t n) { ensure(a, n); };
   R(msg_, cap * mw);
@@ -302,8 +308,8 @@ void Engine::reserve_edges() {
     R(loss_, cap);
   } else {
     R(loss_, std::max<size_t>(cap, 2 * H + 2));
-    R(logits_, (size_t)sched_.B * H + 1);   // root rows / |h| scratch
-    R(dlogits_, std::max<size_t>((size_t)sched_.B * H, cap * H));
+    R(logits_, (size_t)sched_->B * H + 1);   // root rows / |h| scratch
+    R(dlogits_, std::max<size_t>((size_t)sched_->B * H, cap * H));
   }
 }
 
@@ -316,7 +322,7 @@ void Engine::reserve_edges() {
 //                  backward Scatter writes
 //   roots [B]      vertex ids of the roots (sum-of-squares loss)
 void Engine::upload_index_arena() {
-  const Schedule &s = sched_;
+  const Schedule &s = *sched_;
   const int N = N_;
   const bool want_forest = !cfg_.split_backward_rounds && fused_rows() > 0;
   const size_t total = (size_t)N * (2 + nch_) + s.B + (want_forest ? (size_t)N * (nch_ + 1) : 0);
@@ -329,8 +335,6 @@ void Engine::upload_index_arena() {
     auto w0 = std::chrono::steady_clock::now();
     check(cavs_event_sync(idx_copied_[slot]));
     wait_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
-  } else {
-    wait_ms_ = 0.f;
   }
   idx_pending_[slot] = false;
   idx_host_[slot].reserve(total);
@@ -339,32 +343,9 @@ void Engine::upload_index_arena() {
     idx_dev_.reserve(grow(total, idx_dev_.capacity()));
   }
   int *t2j = idx_host_[slot].get(), *pair = t2j + N, *child = pair + N, *roots = child + (size_t)nch_ * N;
-  std::memcpy(t2j, s.tids_to_jobids.data(), sizeof(int) * N);
-  std::fill(pair, pair + N, -1);
-  std::fill(child, child + (size_t)nch_ * N, -1);
-  for (const Round &r : s.rounds) {
-    const int m = r.scatter_end - r.scatter_begin;
-    if (cfg_.pairing == CAVS_PAIR_REFERENCE) {
-      // b-th list entry <-> b-th slab row (op_impl_graphop.cu:148-157)
-      for (int b = 0; b < m; b++) pair[r.offset + b] = s.scatter_ids[r.scatter_begin + b];
-    } else {
-      for (int b = 0; b < m; b++) pair[s.scatter_ids[r.scatter_begin + b]] = s.scatter_ids[r.scatter_begin + b];
-    }
-    if (leaf_round(r)) continue;
-    for (int c = 0; c < nch_; c++) {
-      const int len = r.gather_end[c] - r.gather_begin[c];
-      if (len != r.n)
-        fail(CAVS_EUNSUPPORTED, "round at tensor id " + std::to_string(r.offset) + " mixes vertices with and without child " +
-                                    std::to_string(c) + " (the reference's gather lists misalign there too)");
-      for (int b = 0; b < len; b++) child[(size_t)nch_ * (r.offset + b) + c] = s.gather_ids[c][r.gather_begin[c] + b];
-    }
-    if (nch_ == 1 && r.gather_end[1] != r.gather_begin[1])
-      fail(CAVS_EUNSUPPORTED, "a chain vertex function got a vertex with two children");
-  }
-  int nr = 0;
-  for (int v = 0; v < N; v++)
-    if (s.parent[v] < 0) roots[nr++] = v;
-  forest_ = want_forest && build_forest_lists(pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N);
+  std::string err = build_index_lists(s, nch_, cfg_.pairing, t2j, pair, child, roots);
+  if (!err.empty()) fail(CAVS_EUNSUPPORTED, err);
+  forest_ = want_forest && build_forest_lists(s, nch_, fused_rows(), pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N, &n_orphans_);
   check(cavs_memcpy_h2d(idx_dev_.get(), idx_host_[slot].get(), total * sizeof(int), stream_));
   check(cavs_event_record(idx_copied_[slot], stream_));
   idx_pending_[slot] = true;
@@ -372,68 +353,251 @@ void Engine::upload_index_arena() {
   d_pair_ = d_t2j_ + N;
   d_child_ = d_pair_ + N;
   d_roots_ = d_child_ + (size_t)nch_ * N;
-  d_kid_rows_ = d_roots_ + s.B;
-  d_orphans_ = d_kid_rows_ + (size_t)nch_ * N;
+  d_kid_rows_ = want_forest ? d_roots_ + s.B : nullptr;
+  d_orphans_ = want_forest ? d_kid_rows_ + (size_t)nch_ * N : nullptr;
 }
 
-// The backward launch that folds the children's gate gradients in addresses a child by its slab
-// row, not by the pool row its message went through.  That is the same thing only while the
-// message flow is a forest: every pool row a Gather reads was written by exactly one slab row of
-// an earlier round and is read by exactly one (vertex, child slot).  `pair` and `child` are the
-// host copies of the lists in the staging buffer that is about to be uploaded.
-bool Engine::build_forest_lists(const int *pair, const int *child, int *kid_rows, int *orphans) {
-  const Schedule &s = sched_;
-  const int N = N_;
-  n_orphans_ = 0;
-  if (!s.batching || s.rounds.empty() || !leaf_round(s.rounds[0]) || s.rounds[0].n != s.leaf_prefix) return false;
-  inv_pair_.assign(N, -1);
-  round_of_row_.resize(N);
-  const int fused = fused_rows();
-  for (size_t k = 0; k < s.rounds.size(); k++) {
-    const Round &r = s.rounds[k];
-    if (k > 0 && (leaf_round(r) || r.n > fused)) return false;  // every round with children runs as a fused launch
-    for (int b = 0; b < r.n; b++) round_of_row_[r.offset + b] = (int)k;
+// ------------------------------------------------------------------ step
+namespace {
+// 64-bit mix over the feed's words (not cryptographic: a hit is confirmed by comparing the bytes)
+uint64_t hash_feed(const int32_t *g, size_t n, int B, int maxlen, int pairing) {
+  uint64_t h = 0x9e3779b97f4a7c15ull ^ ((uint64_t)B << 32) ^ (uint64_t)maxlen ^ ((uint64_t)pairing << 60);
+  size_t i = 0;
+  for (; i + 2 <= n; i += 2) {
+    uint64_t w;
+    std::memcpy(&w, g + i, 8);
+    h = (h ^ w) * 0xff51afd7ed558ccdull;
+    h ^= h >> 32;
   }
-  for (int v = 0; v < N; v++) {
-    const int p = pair[v];
-    if (p < 0) continue;
-    if (p >= N || inv_pair_[p] >= 0) return false;  // two writers of one pool row
-    inv_pair_[p] = v;
+  if (i < n) h = (h ^ (uint32_t)g[i]) * 0xc4ceb9fe1a85ec53ull;
+  return h ^ (h >> 29);
+}
+}  // namespace
+
+Engine::Plan *Engine::find_plan(const int *graph, int B, int maxlen, uint64_t hash) {
+  for (auto &p : plans_)
+    if (p->hash == hash && p->B == B && p->maxlen == maxlen && p->pairing == cfg_.pairing &&
+        std::memcmp(p->graph.data(), graph, sizeof(int32_t) * (size_t)B * maxlen) == 0)
+      return p.get();
+  return nullptr;
+}
+
+// Keeps what this step's scheduling produced: the schedule and a compact device copy of its lists.
+void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
+  std::unique_ptr<Plan> p;
+  if ((int)plans_.size() >= cfg_.plan_cache) {
+    // the least recently used plan goes; kernels still in flight may be reading its lists
+    size_t lru = 0;
+    for (size_t i = 1; i < plans_.size(); i++)
+      if (plans_[i]->last_used < plans_[lru]->last_used) lru = i;
+    check(cavs_stream_sync(stream_));
+    p = std::move(plans_[lru]);
+    plans_.erase(plans_.begin() + lru);
+  } else {
+    p = std::make_unique<Plan>();
   }
-  std::vector<char> read(N, 0);
-  for (size_t i = 0; i < (size_t)nch_ * N; i++) {
-    kid_rows[i] = -1;
-    const int p = child[i];
-    if (p < 0) continue;
-    const int b = (int)(i / nch_);
-    if (p >= N || inv_pair_[p] < 0 || read[p]) return false;  // reads a row nobody wrote, or a second reader
-    const int v = inv_pair_[p];
-    if (round_of_row_[v] >= round_of_row_[b]) return false;
-    read[p] = 1;
-    kid_rows[i] = v;
+  const size_t N = N_, nk = (size_t)nch_ * N;
+  p->hash = hash;
+  p->B = B;
+  p->maxlen = maxlen;
+  p->pairing = cfg_.pairing;
+  p->graph.assign(graph, graph + (size_t)B * maxlen);
+  p->sched = sched_;
+  p->lists_on_host = sched_lists_on_host_;
+  p->n_orphans = n_orphans_;
+  p->forest = forest_;
+  p->last_used = ++plan_clock_;
+  p->lists.reserve(2 * N + 2 * nk + B + N);
+  int *base = p->lists.get();
+  const bool kids = d_kid_rows_ != nullptr;
+  check(cavs_memcpy_d2d(base, d_t2j_, N * 4, stream_));
+  check(cavs_memcpy_d2d(base + N, d_pair_, N * 4, stream_));
+  check(cavs_memcpy_d2d(base + 2 * N, d_child_, nk * 4, stream_));
+  check(cavs_memcpy_d2d(base + 2 * N + nk, d_roots_, (size_t)B * 4, stream_));
+  if (kids) {
+    check(cavs_memcpy_d2d(base + 2 * N + nk + B, d_kid_rows_, nk * 4, stream_));
+    check(cavs_memcpy_d2d(base + 2 * N + 2 * nk + B, d_orphans_, (size_t)n_orphans_ * 4, stream_));
   }
-  for (int v = 0; v < N; v++) {
-    if (pair[v] >= 0 && !read[pair[v]]) return false;  // a message nobody reads: its gradient is whatever the pool holds
-    if (pair[v] < 0) orphans[n_orphans_++] = v;
+  // this step reads the copy as well, so that the buffers the lists were built in are free again
+  d_t2j_ = base;
+  d_pair_ = base + N;
+  d_child_ = base + 2 * N;
+  d_roots_ = base + 2 * N + nk;
+  d_kid_rows_ = kids ? base + 2 * N + nk + B : nullptr;
+  d_orphans_ = kids ? base + 2 * N + 2 * nk + B : nullptr;
+  plans_.push_back(std::move(p));
+}
+
+void Engine::schedule_on_host(const int *graph, int B, int maxlen) {
+  auto t0 = std::chrono::steady_clock::now();
+  auto fresh = std::make_shared<Schedule>();
+  std::string err = build_schedule(graph, B, maxlen, (cfg_.opt & CAVS_OPT_BATCHING) != 0, fresh.get());
+  sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
+  if (fresh->executed != fresh->N)
+    fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample; the reference never executes such a vertex "
+                            "(graph_scheduler.cc:180) and leaves its rows undefined");
+  sched_ = fresh;
+  sched_lists_on_host_ = true;
+  N_ = sched_->N;
+  upload_index_arena();
+}
+
+// The graph feed goes to the device, cavs_schedule_arena builds every list there, the host gets
+// the round offsets back and drives the rounds with them.  The scheduler's kernels run on a
+// stream of their own, so that waiting for the offsets does not wait for the previous step.
+void Engine::schedule_on_device(const int *graph, int B, int maxlen) {
+  auto t0 = std::chrono::steady_clock::now();
+  DeviceSched &d = dsched_[dsched_slot_];
+  dsched_slot_ ^= 1;
+  if (!sched_stream_) check(cavs_stream_create(&sched_stream_));
+  if (!d.free_ev) check(cavs_event_create(&d.free_ev));
+  if (d.busy) {  // the step before last read these lists
+    auto w0 = std::chrono::steady_clock::now();
+    check(cavs_event_sync(d.free_ev));
+    wait_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
+    d.busy = false;
   }
-  return true;
+  const size_t BM = (size_t)B * maxlen, nmeta = (size_t)maxlen + 9;
+  const size_t need = BM * (2 + 2 * (size_t)nch_) + 2 * (size_t)B;
+  d.graph_host.reserve(BM);
+  d.meta_host.reserve(nmeta);
+  d.graph_dev.reserve(BM);
+  d.meta_dev.reserve(nmeta);
+  d.lists.reserve(need);
+  d.cap = (long)BM;
+  const size_t sbytes = cavs_schedule_arena_scratch(B, maxlen);
+  dsched_scratch_.reserve(sbytes / 4 + 1);
+  std::memcpy(d.graph_host.get(), graph, BM * sizeof(int));
+  check(cavs_memcpy_h2d(d.graph_dev.get(), d.graph_host.get(), BM * sizeof(int), sched_stream_));
+  int *t2j = d.lists.get(), *pair = t2j + BM, *child = pair + BM, *kid = child + (size_t)nch_ * BM,
+      *roots = kid + (size_t)nch_ * BM, *orph = roots + B;
+  check(cavs_schedule_arena(d.graph_dev.get(), B, maxlen, nch_, cfg_.pairing, t2j, pair, child, kid, roots, orph, d.cap,
+                            d.meta_dev.get(), dsched_scratch_.get(), sbytes, sched_stream_));
+  check(cavs_memcpy_d2h(d.meta_host.get(), d.meta_dev.get(), nmeta * sizeof(int), sched_stream_));
+  check(cavs_stream_sync(sched_stream_));
+  c_launches_ += 5;
+  const int *meta = d.meta_host.get();
+  const int N = meta[0], R = meta[1], bad = meta[2];
+  if (bad) {
+    std::string why;
+    if (bad & 1) why += " a sample has no -1 terminator within maxlen;";
+    if (bad & 2) why += " a parent id is out of range;";
+    if (bad & 8) why += " the batch holds a single-vertex sample, which the reference never executes (graph_scheduler.cc:180);";
+    if (bad & 4) why += std::string(" a vertex has children, but not ") + (nch_ == 2 ? "two children" : "one child") +
+                        " (the round mixes vertices with and without a child);";
+    if (bad & 16) why += " vertices never become ready: the parent array holds a cycle;";
+    fail((bad & 8) ? CAVS_EUNSUPPORTED : CAVS_EINVAL, "graph feed rejected:" + why);
+  }
+  // the rounds, as far as the loops over them need: offsets, sizes, which one holds the leaves
+  auto fresh = std::make_shared<Schedule>();
+  Schedule &s = *fresh;
+  s.B = B;
+  s.maxlen = maxlen;
+  s.N = s.executed = N;
+  s.batching = true;
+  s.round2offset.assign(meta + 8, meta + 8 + R + 1);
+  for (int r = 0; r < R; r++) {
+    Round rd{};
+    rd.offset = meta[8 + r];
+    rd.n = meta[8 + r + 1] - meta[8 + r];
+    // only whether the gather ranges are empty is read from a schedule without lists
+    rd.gather_end[0] = rd.gather_end[1] = r > 0 ? rd.n : 0;
+    if (nch_ == 1) rd.gather_end[1] = 0;
+    s.rounds.push_back(rd);
+    s.max_round = std::max(s.max_round, rd.n);
+  }
+  for (int k = R - 1; k >= 0; k--) s.bwd_rounds.push_back(k);
+  s.leaf_prefix = R > 0 ? meta[9] : 0;
+  sched_ = fresh;
+  sched_lists_on_host_ = false;
+  N_ = N;
+  d_t2j_ = t2j;
+  d_pair_ = pair;
+  d_child_ = child;
+  d_kid_rows_ = kid;
+  d_roots_ = roots;
+  d_orphans_ = orph;
+  // every sample has one root, so B slab rows send no message; the message flow of a well-formed
+  // batch is a forest by construction, what remains to ask is whether every round with children
+  // runs as a fused launch
+  n_orphans_ = B;
+  forest_ = !cfg_.split_backward_rounds && fused_rows() > 0;
+  for (int r = 1; r < R && forest_; r++) forest_ = s.rounds[r].n <= fused_rows();
+  last_dsched_ = &d;
+  sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+}
+
+const Schedule &Engine::schedule() {
+  if (!sched_lists_on_host_ && N_ > 0) {
+    const size_t N = N_, nk = (size_t)nch_ * N;
+    std::vector<int> t2j(N), pair(N), child(nk), roots(sched_->B);
+    check(cavs_memcpy_d2h(t2j.data(), d_t2j_, N * 4, stream_));
+    check(cavs_memcpy_d2h(pair.data(), d_pair_, N * 4, stream_));
+    check(cavs_memcpy_d2h(child.data(), d_child_, nk * 4, stream_));
+    check(cavs_memcpy_d2h(roots.data(), d_roots_, (size_t)sched_->B * 4, stream_));
+    check(cavs_stream_sync(stream_));
+    auto full = std::make_shared<Schedule>();
+    schedule_from_lists(sched_->B, sched_->maxlen, N_, nch_, sched_->round2offset.data(), (int)sched_->rounds.size(), t2j.data(),
+                        pair.data(), child.data(), roots.data(), full.get());
+    for (auto &p : plans_)
+      if (p->sched == sched_) {  // the cached plan gets the complete schedule too
+        p->sched = full;
+        p->lists_on_host = true;
+      }
+    sched_ = full;
+    sched_lists_on_host_ = true;
+  }
+  return *sched_;
 }
 
 // ------------------------------------------------------------------ step
 void Engine::begin_step(const int *graph, int B, int maxlen) {
   auto t0 = std::chrono::steady_clock::now();
-  std::string err = build_schedule(graph, B, maxlen, (cfg_.opt & CAVS_OPT_BATCHING) != 0, &sched_);
-  sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
-  if (!err.empty()) fail(CAVS_EINVAL, "graph feed rejected: " + err);
-  if (sched_.executed != sched_.N)
-    fail(CAVS_EUNSUPPORTED, "the batch holds a single-vertex sample; the reference never executes such a vertex "
-                            "(graph_scheduler.cc:180) and leaves its rows undefined");
-  N_ = sched_.N;
+  if (!graph || B <= 0 || maxlen <= 0) fail(CAVS_EINVAL, "graph feed rejected: empty graph feed");
+  if (last_dsched_) {  // everything that reads the previous step's device-built lists is enqueued by now
+    check(cavs_event_record(last_dsched_->free_ev, stream_));
+    last_dsched_->busy = true;
+    last_dsched_ = nullptr;
+  }
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   c_round_flops_ = 0;
   bias_jobs_.clear();
+  wait_ms_ = 0.f;
+  uint64_t hash = 0;
+  Plan *hit = nullptr;
+  if (cfg_.plan_cache > 0) {
+    hash = hash_feed(graph, (size_t)B * maxlen, B, maxlen, cfg_.pairing);
+    hit = find_plan(graph, B, maxlen, hash);
+  }
+  if (hit) {
+    // a batch structure seen before: its schedule and its lists are where the last such step left them
+    hit->last_used = ++plan_clock_;
+    c_plan_hits_ += 1;
+    sched_ = hit->sched;
+    sched_lists_on_host_ = hit->lists_on_host;
+    N_ = sched_->N;
+    n_orphans_ = hit->n_orphans;
+    const bool want_forest = !cfg_.split_backward_rounds && fused_rows() > 0;
+    forest_ = hit->forest && want_forest;
+    const size_t N = N_, nk = (size_t)nch_ * N;
+    const int *base = hit->lists.get();
+    d_t2j_ = base;
+    d_pair_ = base + N;
+    d_child_ = base + 2 * N;
+    d_roots_ = base + 2 * N + nk;
+    d_kid_rows_ = base + 2 * N + nk + B;
+    d_orphans_ = base + 2 * N + 2 * nk + B;
+    sched_ms_ = 0.f;
+  } else {
+    const bool on_device = cfg_.schedule_mode == 1 && (cfg_.opt & CAVS_OPT_BATCHING) && maxlen <= 2048;
+    if (on_device) schedule_on_device(graph, B, maxlen); else schedule_on_host(graph, B, maxlen);
+    if (cfg_.plan_cache > 0) {
+      c_plan_misses_ += 1;
+      remember_plan(graph, B, maxlen, hash);
+    }
+  }
   reserve_edges();
-  upload_index_arena();
   parse_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
 }
 
@@ -586,7 +750,7 @@ void Engine::treelstm_forward() {
   const int fused = fused_rows();
   bool any_packed = false;
   if (Upk_.capacity() > 0)
-    for (const Round &r : sched_.rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_round_packed_ok(r.n, H);
+    for (const Round &r : sched_->rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_round_packed_ok(r.n, H);
   if (any_packed && !upk_valid_) {  // U was written by somebody else since the last update here
     cavs_task pack[2] = {{CAVS_TASK_SGD_PACK, 0.f, H, 3 * H, 0, Upk_.get(), const_cast<float *>(U), nullptr, nullptr},
                          {CAVS_TASK_SGD_PACK, 0.f, H, H, 0, Upk_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H, nullptr,
@@ -598,14 +762,14 @@ void Engine::treelstm_forward() {
   check(cavs_embed_pull_fwd(e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, E, e_.get(), ld_e_, W, 4 * H, 0.f, xW_.get(), 4 * H);
-  if (!sched_.batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
+  if (!sched_->batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
   }
   // when every round runs fused, Push + FunctionPopRet ride along in the rounds' epilogues
-  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  out_folded_ = fused > 0 && sched_->max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
-  for (const Round &r : sched_.rounds) {
+  for (const Round &r : sched_->rounds) {
     const size_t off = r.offset;
     // the message slab is only read back by FunctionPopRet; when the rounds write the output
     // rows themselves nobody reads it and the fused launches skip it
@@ -658,13 +822,13 @@ void Engine::treelstm_backward() {
   const float *W = param("W").w, *U = param("U").w;
   const int fused = fused_rows();
   // grad of Push is Pull: read through the list by the fused gate kernels, or gathered up front
-  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  const bool dret_folded = fused > 0 && sched_->max_round <= fused;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
-  if (!sched_.batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
+  if (!sched_->batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   // one launch per round when the message flow is a forest (below); then, if every such launch has
   // a packed variant, the transposed weights are written tile-major instead of plain
   bool packed = forest_;
-  for (const Round &r : sched_.rounds)
+  for (const Round &r : sched_->rounds)
     if (!leaf_round(r) && !cavs_round_packed_ok(r.n, H)) packed = false;
   if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
     const int kind = packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE;
@@ -679,18 +843,18 @@ void Engine::treelstm_backward() {
   const bool folded = forest_;
   if (folded) {
     CAVS_TIMED(K_GATES, cavs_treelstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
-                                                     dF_.get(), dc_.get(), sched_.leaf_prefix, H, stream_));
+                                                     dF_.get(), dc_.get(), sched_->leaf_prefix, H, stream_));
     c_launches_ += 1;
   }
-  for (int k : sched_.bwd_rounds) {
-    const Round &r = sched_.rounds[k];
+  for (int k : sched_->bwd_rounds) {
+    const Round &r = sched_->rounds[k];
     const size_t off = r.offset;
     if (folded) {
       c_gather_rows_ += r.n;
       if (leaf_round(r)) continue;
       CAVS_TIMED(K_ROUND, (packed ? cavs_treelstm_round_bwd_children_gates_packed : cavs_treelstm_round_bwd_children_gates)(
                               dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_ + 2 * off, gates_.get(), G_.get(), d_dgo_,
-                              d_t2j_, (int)off, r.n, sched_.leaf_prefix, H, stream_));
+                              d_t2j_, (int)off, r.n, sched_->leaf_prefix, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 5.0 * H;
       c_scatter_rows_ += 2.0 * r.n;
       c_launches_ += 1;
@@ -742,7 +906,7 @@ void Engine::treelstm_backward() {
   }
   // weight gradients once over all rows (OPT_BATCHING semantics; without it the reference
   // accumulates the same sums round by round)
-  const int lp = sched_.leaf_prefix;  // leaves contribute exact zeros to dU
+  const int lp = sched_->leaf_prefix;  // leaves contribute exact zeros to dU
   float *dU = param("U").g;
   const bool bias_row = bias_row_ok();  // the ones column of e_ turns row E of dW into the column sums of dxW
   gemm_group({
@@ -881,20 +1045,20 @@ void Engine::lstm_forward() {
   check(cavs_embed_pull_fwd(e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, stream_));
   c_launches_ += 1;
   gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
-  if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  if (!sched_->batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
   const int fused = fused_rows();
   bool any_packed = false;
   if (Upk_.capacity() > 0)
-    for (const Round &r : sched_.rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_lstm_round_packed_ok(r.n, H);
+    for (const Round &r : sched_->rounds) any_packed |= !leaf_round(r) && r.n <= fused && cavs_lstm_round_packed_ok(r.n, H);
   if (any_packed && !upk_valid_) {  // W' was written by somebody else since the last update here
     cavs_task pack{CAVS_TASK_SGD_PACK, 0.f, H, 4 * H, 0, Upk_.get(), const_cast<float *>(Wh), nullptr, nullptr};
     check(cavs_run_tasks(1, &pack, stream_));
     c_launches_ += 1;
     upk_valid_ = Wx == param("W").own_w.get();
   }
-  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  out_folded_ = fused > 0 && sched_->max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
-  for (const Round &r : sched_.rounds) {
+  for (const Round &r : sched_->rounds) {
     const size_t off = r.offset;
     float *a = xW_.at(off * 4 * H), *msg = msg_.at(off * 2 * H), *G = nullptr;
     if (r.n <= fused) {  // one launch: Gather, h*W', gates, Scatter, Push/PopRet
@@ -928,10 +1092,10 @@ void Engine::lstm_backward() {
   const int N = N_, H = cfg_.H;
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H;
   const int fused = fused_rows();
-  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  const bool dret_folded = fused > 0 && sched_->max_round <= fused;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   bool packed = forest_;  // as in treelstm_backward
-  for (const Round &r : sched_.rounds)
+  for (const Round &r : sched_->rounds)
     if (!leaf_round(r) && !cavs_lstm_round_packed_ok(r.n, H)) packed = false;
   if (fused > 0) {  // W'^T: the B operand of d h_prev = da * W'^T, k-major
     backward_prologue({{packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE, 0.f, H, 4 * H, 0, UT_.get(), const_cast<float *>(Wh), nullptr,
@@ -943,11 +1107,11 @@ void Engine::lstm_backward() {
   const bool folded = forest_;  // one launch per round, as in treelstm_backward
   if (folded) {
     CAVS_TIMED(K_GATES, cavs_lstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
-                                                 dc_.get(), sched_.leaf_prefix, H, stream_));
+                                                 dc_.get(), sched_->leaf_prefix, H, stream_));
     c_launches_ += 1;
   }
-  for (int k : sched_.bwd_rounds) {
-    const Round &r = sched_.rounds[k];
+  for (int k : sched_->bwd_rounds) {
+    const Round &r = sched_->rounds[k];
     const size_t off = r.offset;
     float *da = dxW_.at(off * 4 * H);
     if (folded) {
@@ -955,7 +1119,7 @@ void Engine::lstm_backward() {
       if (leaf_round(r)) continue;
       CAVS_TIMED(K_ROUND, (packed ? cavs_lstm_round_bwd_children_gates_packed : cavs_lstm_round_bwd_children_gates)(
                               dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(), G_.get(), d_dgo_, d_t2j_, (int)off,
-                              r.n, sched_.leaf_prefix, H, stream_));
+                              r.n, sched_->leaf_prefix, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
       c_scatter_rows_ += r.n;
       c_launches_ += 1;
@@ -990,7 +1154,7 @@ void Engine::lstm_backward() {
     gemm(0, 1, r.n, H, 4 * H, da, 4 * H, Wh, 4 * H, 0.f, r_dG_.get(), 2 * H);  // dh_p = da * W'^T
     scatter(dpool_.get(), 2 * H, d_child_ + off, r_dG_.get(), 2 * H, r.n, 2 * H);
   }
-  const int lp = sched_.leaf_prefix;
+  const int lp = sched_->leaf_prefix;
   float *dW = param("W").g;
   gemm_group({
       {0, 1, N, H, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, Wx, 4 * H, de_.get(), H},
@@ -1009,11 +1173,11 @@ void Engine::treefc_forward() {
   const float *W = param("W").w;
   const float *Bv = cfg_.use_bias ? param("Bv").w : nullptr;
   if (cfg_.use_x) gather(xs_.get(), H, d_x_, H, d_t2j_, N, H);
-  if (!sched_.batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
+  if (!sched_->batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
   const int fused = fused_rows();
-  out_folded_ = fused > 0 && sched_.max_round <= fused && fwd_out_ != nullptr;
+  out_folded_ = fused > 0 && sched_->max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
-  for (const Round &r : sched_.rounds) {
+  for (const Round &r : sched_->rounds) {
     const size_t off = r.offset;
     const float *xin = cfg_.use_x ? xs_.at(off * H) : nullptr;
     float *msg = msg_.at(off * H);
@@ -1054,7 +1218,7 @@ void Engine::treefc_backward() {
   const int N = N_, H = cfg_.H;
   const float *W = param("W").w;
   const int fused = fused_rows();
-  const bool dret_folded = fused > 0 && sched_.max_round <= fused;
+  const bool dret_folded = fused > 0 && sched_->max_round <= fused;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (fused > 0) {  // W^T [H, 2H]: the B operand of d[h_l;h_r] = dz * W^T, k-major
     backward_prologue({{CAVS_TASK_TRANSPOSE, 0.f, 2 * H, H, 0, UT_.get(), const_cast<float *>(W), nullptr, nullptr}}, false);
@@ -1066,8 +1230,8 @@ void Engine::treefc_backward() {
     CAVS_TIMED(K_GATES, cavs_treefc_bwd_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, msg_.get(), dxW_.get(), H, cfg_.act, stream_));
     c_launches_ += 1;
   }
-  for (int k : sched_.bwd_rounds) {
-    const Round &r = sched_.rounds[k];
+  for (int k : sched_->bwd_rounds) {
+    const Round &r = sched_->rounds[k];
     const size_t off = r.offset;
     float *dz = dxW_.at(off * H);
     if (folded) {
@@ -1100,7 +1264,7 @@ void Engine::treefc_backward() {
     gemm(0, 1, r.n, 2 * H, H, dz, H, W, H, 0.f, r_dG_.get(), 2 * H);
     scatter(dpool_.get(), H, d_child_ + 2 * off, r_dG_.get(), H, 2 * r.n, H);
   }
-  const int lp = sched_.leaf_prefix;
+  const int lp = sched_->leaf_prefix;
   gemm_splitk(1, 0, 2 * H, H, N - lp, G_.at((size_t)2 * lp * H), 2 * H, dxW_.at((size_t)lp * H), H,
               param("W").g, H);
   if (cfg_.use_bias) {
@@ -1110,7 +1274,7 @@ void Engine::treefc_backward() {
 
 // ------------------------------------------------------------------ loss head
 void Engine::head_forward_backward(bool backward) {
-  const int N = N_, H = cfg_.H, C = cfg_.C, B = sched_.B;
+  const int N = N_, H = cfg_.H, C = cfg_.C, B = sched_->B;
   if (cfg_.loss == CAVS_LOSS_SOFTMAX) {
     // FullyConnected + SoftmaxEntropyLoss (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79,
     // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
@@ -1226,7 +1390,9 @@ double Engine::counter(const std::string &key) const {
   if (key == "gemm_flops") return c_gemm_flops_;
   if (key == "round_flops") return c_round_flops_;
   if (key == "launches") return c_launches_;
-  if (key == "rounds") return (double)sched_.rounds.size();
+  if (key == "rounds") return (double)sched_->rounds.size();
+  if (key == "plan_hits") return c_plan_hits_;
+  if (key == "plan_misses") return c_plan_misses_;
   fail(CAVS_EINVAL, "unknown counter '" + key + "'");
 }
 

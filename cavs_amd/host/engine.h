@@ -7,6 +7,7 @@
 #ifndef CAVS_HOST_ENGINE_H_
 #define CAVS_HOST_ENGINE_H_
 
+#include <cstdint>
 #include <map>
 #include <memory>
 #include <string>
@@ -65,9 +66,11 @@ class Engine {
   enum KernelClass { K_GEMM = 0, K_GATHER, K_SCATTER, K_GATES, K_OTHER, K_ROUND, K_CLASSES };
   void profile_enable(bool on);
   void profile_read(int cls, double *total_ms, double *launches);
-  const Schedule &schedule() const { return sched_; }
+  // The last step's schedule with all its lists.  When the device scheduler built it, the host
+  // holds the rounds only; the lists are then read back and the schedule completed (synchronises).
+  const Schedule &schedule();
   void *stream() const { return stream_; }
-  int total_length() const { return sched_.N; }
+  int total_length() const { return sched_->N; }
 
  private:
   Param &param(const std::string &name);
@@ -125,7 +128,8 @@ class Engine {
   float parse_ms_ = 0.f, sched_ms_ = 0.f, wait_ms_ = 0.f, host_step_ms_ = 0.f;
   std::map<std::string, std::unique_ptr<Param>> params_;
 
-  Schedule sched_;
+  std::shared_ptr<Schedule> sched_ = std::make_shared<Schedule>();
+  bool sched_lists_on_host_ = true;  // false: the device scheduler built the lists, sched_ holds the rounds only
   bool did_backward_ = false;
   float *fwd_out_ = nullptr;   // where the forward pass returns h by vertex id
   bool out_folded_ = false;    // the rounds wrote it themselves
@@ -143,8 +147,44 @@ class Engine {
   const int *d_kid_rows_ = nullptr, *d_orphans_ = nullptr;
   int n_orphans_ = 0;
   bool forest_ = false;
-  std::vector<int> inv_pair_, round_of_row_;
-  bool build_forest_lists(const int *pair, const int *child, int *kid_rows, int *orphans);
+
+  // ---- schedule on the device (cfg.schedule_mode 1): the graph feed goes up, cavs_schedule_arena
+  // builds every list there, and only the round offsets come back.  Two sets of buffers alternate,
+  // so that the lists of step k + 1 are built while the kernels of step k still read theirs.
+  struct DeviceSched {
+    PinnedArray<int> graph_host, meta_host;
+    DeviceArray<int> graph_dev, lists, meta_dev;
+    long cap = 0;          // rows per list
+    void *free_ev = nullptr;  // recorded once everything that read `lists` has been enqueued
+    bool busy = false;
+  } dsched_[2];
+  DeviceArray<int> dsched_scratch_;
+  void *sched_stream_ = nullptr;
+  int dsched_slot_ = 0;
+  DeviceSched *last_dsched_ = nullptr;  // the buffers the current step's lists live in, if device-built
+  void schedule_on_device(const int *graph, int B, int maxlen);
+  void schedule_on_host(const int *graph, int B, int maxlen);
+  void point_lists(const int *base, long cap);
+
+  // ---- plan cache (cfg.plan_cache entries): the schedule and the device lists of a graph feed,
+  // keyed by the feed's bytes, so that a batch structure seen before costs neither the scheduler
+  // nor an upload
+  struct Plan {
+    uint64_t hash = 0;
+    int B = 0, maxlen = 0, pairing = 0;
+    std::vector<int32_t> graph;
+    std::shared_ptr<Schedule> sched;
+    bool lists_on_host = true;
+    DeviceArray<int> lists;  // [t2j | pair | child | roots | kid_rows | orphans], N rows each
+    int n_orphans = 0;
+    bool forest = false;
+    uint64_t last_used = 0;
+  };
+  std::vector<std::unique_ptr<Plan>> plans_;
+  uint64_t plan_clock_ = 0;
+  double c_plan_hits_ = 0, c_plan_misses_ = 0;
+  Plan *find_plan(const int *graph, int B, int maxlen, uint64_t hash);
+  void remember_plan(const int *graph, int B, int maxlen, uint64_t hash);
 
   // feeds
   DeviceArray<float> x_in_, labels_in_;

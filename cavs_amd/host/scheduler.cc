@@ -161,8 +161,145 @@ std::string build_schedule(const int32_t *graph, int B, int maxlen, bool batchin
   if (!graph || B <= 0 || maxlen <= 0) return "empty graph feed";
   std::string err = load_graph(graph, B, maxlen, out);
   if (!err.empty()) return err;
+  for (int v = 0; v < out->N; v++)
+    if (nchild(*out, v) > 2)
+      return "vertex " + std::to_string(v) + " has " + std::to_string(nchild(*out, v)) +
+             " children; the scheduler's gather lists hold two (graph_scheduler.h:16-18)";
   if (batching) batch_rounds(out); else serial_rounds(out);
+  if (out->executed != out->N) {
+    // A sample of a single vertex is never executed (graph_scheduler.cc:180); the schedule of the
+    // rest stands, and it is the caller's business whether it accepts such a batch.  Any other
+    // vertex that did not run sits on a parent cycle.
+    int singles = 0;
+    for (int i = 0; i < B; i++) {
+      const int hi = i + 1 < B ? out->sample_offset[i + 1] : out->N;
+      if (hi - out->sample_offset[i] == 1) singles++;
+    }
+    if (out->executed + singles != out->N)
+      return std::to_string(out->N - out->executed - singles) + " vertices never become ready: the parent array holds a cycle "
+             "(a vertex that is its own ancestor)";
+  }
   return "";
+}
+
+std::string build_index_lists(const Schedule &s, int nch, int pairing, int *t2j, int *pair, int *child, int *roots) {
+  const int N = s.N;
+  std::copy(s.tids_to_jobids.begin(), s.tids_to_jobids.end(), t2j);
+  std::fill(pair, pair + N, -1);
+  std::fill(child, child + (size_t)nch * N, -1);
+  for (const Round &r : s.rounds) {
+    const int m = r.scatter_end - r.scatter_begin;
+    if (pairing == 0) {
+      for (int b = 0; b < m; b++) pair[r.offset + b] = s.scatter_ids[r.scatter_begin + b];
+    } else {
+      for (int b = 0; b < m; b++) pair[s.scatter_ids[r.scatter_begin + b]] = s.scatter_ids[r.scatter_begin + b];
+    }
+    if (r.gather_begin[0] == r.gather_end[0] && r.gather_begin[1] == r.gather_end[1]) continue;  // a round of leaves
+    for (int c = 0; c < nch; c++) {
+      const int len = r.gather_end[c] - r.gather_begin[c];
+      if (len != r.n)
+        return "round at tensor id " + std::to_string(r.offset) + " mixes vertices with and without child " + std::to_string(c) +
+               " (the reference's gather lists misalign there too)";
+      for (int b = 0; b < len; b++) child[(size_t)nch * (r.offset + b) + c] = s.gather_ids[c][r.gather_begin[c] + b];
+    }
+    if (nch == 1 && r.gather_end[1] != r.gather_begin[1]) return "a chain vertex function got a vertex with two children";
+  }
+  int nr = 0;
+  for (int v = 0; v < N; v++)
+    if (s.parent[v] < 0) roots[nr++] = v;
+  return "";
+}
+
+bool build_forest_lists(const Schedule &s, int nch, int fused_limit, const int *pair, const int *child, int *kid_rows,
+                        int *orphans, int *n_orphans) {
+  const int N = s.N;
+  *n_orphans = 0;
+  auto leaf_round = [](const Round &r) { return r.gather_begin[0] == r.gather_end[0] && r.gather_begin[1] == r.gather_end[1]; };
+  if (!s.batching || s.rounds.empty() || !leaf_round(s.rounds[0]) || s.rounds[0].n != s.leaf_prefix) return false;
+  std::vector<int> inv_pair(N, -1), round_of_row(N);
+  for (size_t k = 0; k < s.rounds.size(); k++) {
+    const Round &r = s.rounds[k];
+    if (k > 0 && (leaf_round(r) || r.n > fused_limit)) return false;  // every round with children runs as a fused launch
+    for (int b = 0; b < r.n; b++) round_of_row[r.offset + b] = (int)k;
+  }
+  for (int v = 0; v < N; v++) {
+    const int p = pair[v];
+    if (p < 0) continue;
+    if (p >= N || inv_pair[p] >= 0) return false;  // two writers of one pool row
+    inv_pair[p] = v;
+  }
+  std::vector<char> read(N, 0);
+  for (size_t i = 0; i < (size_t)nch * N; i++) {
+    kid_rows[i] = -1;
+    const int p = child[i];
+    if (p < 0) continue;
+    const int b = (int)(i / nch);
+    if (p >= N || inv_pair[p] < 0 || read[p]) return false;  // reads a row nobody wrote, or a second reader
+    const int v = inv_pair[p];
+    if (round_of_row[v] >= round_of_row[b]) return false;
+    read[p] = 1;
+    kid_rows[i] = v;
+  }
+  for (int v = 0; v < N; v++) {
+    if (pair[v] >= 0 && !read[pair[v]]) return false;  // a message nobody reads: its gradient is whatever the pool holds
+    if (pair[v] < 0) orphans[(*n_orphans)++] = v;
+  }
+  return true;
+}
+
+void schedule_from_lists(int B, int maxlen, int N, int nch, const int *round2offset, int R, const int *t2j,
+                         const int *pair, const int *child, const int *roots, Schedule *out) {
+  *out = Schedule();
+  Schedule &s = *out;
+  s.B = B;
+  s.maxlen = maxlen;
+  s.N = N;
+  s.batching = true;
+  s.tids_to_jobids.assign(t2j, t2j + N);
+  s.jobids_to_tids.assign(N, 0);
+  for (int t = 0; t < N; t++) s.jobids_to_tids[t2j[t]] = t;
+  s.round2offset.assign(round2offset, round2offset + R + 1);
+  std::vector<char> is_root(N, 0);
+  for (int i = 0; i < B; i++) is_root[roots[i]] = 1;
+  // sample offsets and parents follow from the roots (each sample ends at its root) and the child lists
+  s.sample_offset.assign(B, 0);
+  for (int i = 1; i < B; i++) s.sample_offset[i] = roots[i - 1] + 1;
+  s.parent.assign(N, -1);
+  for (int r = 0; r < R; r++) {
+    Round rd;
+    rd.offset = round2offset[r];
+    rd.n = round2offset[r + 1] - round2offset[r];
+    for (int c = 0; c < 2; c++) rd.gather_begin[c] = (int)s.gather_ids[c].size();
+    rd.scatter_begin = (int)s.scatter_ids.size();
+    for (int b = 0; b < rd.n; b++) {
+      const int t = rd.offset + b;
+      for (int c = 0; c < nch; c++) {
+        const int p = child[(size_t)nch * t + c];
+        if (p < 0) continue;
+        s.gather_ids[c].push_back(p);
+        s.parent[t2j[p]] = t2j[t];
+      }
+      // the scatter list is the round's non-root jobs in job order under either pairing
+      if (!is_root[t2j[t]]) s.scatter_ids.push_back(t); else s.root_tids.push_back(t);
+    }
+    for (int c = 0; c < 2; c++) rd.gather_end[c] = (int)s.gather_ids[c].size();
+    rd.scatter_end = (int)s.scatter_ids.size();
+    s.rounds.push_back(rd);
+    s.max_round = std::max(s.max_round, rd.n);
+  }
+  (void)pair;
+  s.executed = N;
+  s.leaf_prefix = R > 0 ? round2offset[1] : 0;
+  for (int k = R - 1; k >= 0; k--) s.bwd_rounds.push_back(k);
+  // children in ascending vertex id, as LoadGraph builds them
+  s.child_begin.assign(N + 1, 0);
+  for (int v = 0; v < N; v++)
+    if (s.parent[v] >= 0) s.child_begin[s.parent[v] + 1]++;
+  for (int v = 0; v < N; v++) s.child_begin[v + 1] += s.child_begin[v];
+  s.child.assign(s.child_begin[N], 0);
+  std::vector<int> fill(s.child_begin.begin(), s.child_begin.end() - 1);
+  for (int v = 0; v < N; v++)
+    if (s.parent[v] >= 0) s.child[fill[s.parent[v]]++] = v;
 }
 
 // trace_format: [N, R_fwd, R_bwd, then per round: offset, n_exec, exec..., n_g0, g0...,

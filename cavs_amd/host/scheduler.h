@@ -49,8 +49,37 @@ struct Schedule {
 
 // Returns an empty string on success, else the reason the graph was rejected.
 // graph: [B, maxlen] int32, entry j = local parent of vertex j, first -1 = root and
-// end of sample (cavs/midend/graph_scheduler.cc:35-43).
+// end of sample (cavs/midend/graph_scheduler.cc:35-43).  Rejected besides malformed rows: a
+// vertex with more than two children (the reference CHECK-aborts when it fills its two gather
+// lists, graph_scheduler.cc:223) and parent cycles (their vertices never become ready).  A sample
+// of a single vertex is scheduled around, as the reference does (graph_scheduler.cc:180):
+// executed < N then tells the caller, who decides whether to accept such a batch.
 std::string build_schedule(const int32_t *graph, int B, int maxlen, bool batching, Schedule *out);
+
+// The index lists the kernels consume, one entry per slab row, from a schedule:
+//   t2j   [N]      tensor id -> global vertex id (Pull, FunctionPopRet)
+//   pair  [N]      per slab row: pool row the forward Scatter writes and the backward Gather
+//                  reads, or -1.  pairing 0: b-th entry of the round's compacted scatter list with
+//                  the b-th slab row (cavs/backend/op_impl_graphop.cu:148-157); 1: the row itself
+//   child [nch*N]  per slab row and child slot: pool row the forward Gather reads (-1: none)
+//   roots [B]      vertex ids of the roots
+// nch: children of an internal vertex (1 chains, 2 binary trees); a round in which some but not
+// all vertices have child c is an error (the reference's gather lists misalign there too).
+std::string build_index_lists(const Schedule &s, int nch, int pairing, int *t2j, int *pair, int *child, int *roots);
+
+// For the backward launches that address a child by the slab row that wrote its pool row:
+// kid_rows [nch*N] (-1: none) and the slab rows nobody reads a message from (orphans, ascending;
+// *n_orphans of them).  False when the message flow of the batch is not a forest (a pool row with
+// two writers or two readers, a message nobody reads, a reader in a round not after its writer's)
+// or a round with children is larger than `fused_limit`.
+bool build_forest_lists(const Schedule &s, int nch, int fused_limit, const int *pair, const int *child, int *kid_rows,
+                        int *orphans, int *n_orphans);
+
+// The inverse of build_index_lists for a batch schedule: rounds and lists of a Schedule from the
+// arrays (as a device scheduler leaves them) and the round offsets; `out` compares equal, trace
+// for trace, to the schedule the lists came from.
+void schedule_from_lists(int B, int maxlen, int N, int nch, const int *round2offset, int R, const int *t2j,
+                         const int *pair, const int *child, const int *roots, Schedule *out);
 
 }  // namespace cavs
 #endif

@@ -22,7 +22,8 @@ PAIR = {"reference": 0, "rowid": 1}
 
 class _Config(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("model", "loss", "pairing", "opt", "V", "E", "H", "C", "act",
-                                      "use_bias", "use_x", "device", "fused_round_rows", "split_backward_rounds")]
+                                      "use_bias", "use_x", "device", "fused_round_rows", "split_backward_rounds",
+                                      "schedule_mode", "plan_cache")]
 
 
 _lib = None
@@ -51,6 +52,8 @@ def lib():
             "cavs_session_total_length": [P],
             "cavs_session_schedule_trace": [P, P, I],
             "cavs_schedule_trace": [P, I, I, I, I, P, I],
+            "cavs_schedule_index_lists": [P, I, I, I, I, I, P, P, P, P, P, P, P],
+            "cavs_schedule_trace_from_lists": [I, I, I, I, P, I, P, P, P, P, I, P, I],
             "cavs_session_timing": [P, C.c_char_p, C.POINTER(F)],
             "cavs_session_counter": [P, C.c_char_p, C.POINTER(C.c_double)],
             "cavs_session_profile": [P, I],
@@ -109,17 +112,51 @@ def schedule_trace(graph, batching=True, with_backward=True):
     return _parse_trace(out)
 
 
+def index_lists(graph, nchild, pairing="reference", fused_limit=1 << 30):
+    """Host-only: the index lists a step's kernels consume, as the host scheduler builds them.
+    Returns dict(N, t2j, pair, child, roots, kid, orphans); kid / orphans are None when the
+    batch's message flow is not a forest."""
+    g = np.ascontiguousarray(graph, np.int32)
+    B, maxlen = g.shape
+    cap = B * maxlen
+    t2j, pair, orph = (np.zeros(cap, np.int32) for _ in range(3))
+    child, kid = np.zeros(nchild * cap, np.int32), np.zeros(nchild * cap, np.int32)
+    roots, n_orph = np.zeros(B, np.int32), C.c_int(0)
+    N = lib().cavs_schedule_index_lists(g.ctypes.data, B, maxlen, nchild, PAIR[pairing], fused_limit, t2j.ctypes.data,
+                                        pair.ctypes.data, child.ctypes.data, roots.ctypes.data, kid.ctypes.data,
+                                        orph.ctypes.data, C.addressof(n_orph))
+    if N <= 0:
+        raise hip.CavsError("graph feed rejected: " + lib().cavs_session_error().decode())
+    forest = n_orph.value >= 0
+    return dict(N=N, t2j=t2j[:N], pair=pair[:N], child=child[: nchild * N], roots=roots,
+                kid=kid[: nchild * N] if forest else None, orphans=orph[: n_orph.value] if forest else None)
+
+
+def trace_from_lists(B, maxlen, nchild, round2offset, t2j, pair, child, roots, with_backward=True):
+    """Host-only: the inverse of index_lists -- the complete schedule the lists describe."""
+    I32 = lambda a: np.ascontiguousarray(a, np.int32)
+    r2o, t2j, pair, child, roots = I32(round2offset), I32(t2j), I32(pair), I32(child), I32(roots)
+    N, R = len(t2j), len(r2o) - 1
+    cap = 64 + 40 * B * maxlen
+    out = np.zeros(cap, np.int32)
+    n = lib().cavs_schedule_trace_from_lists(B, maxlen, N, nchild, r2o.ctypes.data, R, t2j.ctypes.data, pair.ctypes.data,
+                                             child.ctypes.data, roots.ctypes.data, int(with_backward), out.ctypes.data, cap)
+    assert n > 0, n
+    return _parse_trace(out)
+
+
 class Session:
     """One model bound to the device.  `opt` is the reference's bitmask
     (OPT_BATCHING selects the level-wise batch scheduler)."""
 
     def __init__(self, model, *, H, E=0, V=0, C_=0, loss="softmax", pairing="reference",
                  opt=OPT_BATCHING, act=0, use_bias=False, use_x=False, device=0, fused_round_rows=0,
-                 split_backward_rounds=False):
+                 split_backward_rounds=False, schedule="host", plan_cache=0):
         self.model, self.H, self.E, self.V, self.C, self.loss = model, H, (H if model == "lstm" else E), V, C_, loss
         self.mw = H if model == "treefc" else 2 * H
         cfg = _Config(MODEL[model], LOSS[loss], PAIR[pairing], opt, V, E, H, C_, int(act), int(use_bias),
-                      int(use_x), device, int(fused_round_rows), int(split_backward_rounds))
+                      int(use_x), device, int(fused_round_rows), int(split_backward_rounds),
+                      {"host": 0, "device": 1}[schedule], int(plan_cache))
         self._h = C.c_void_p()
         _check(lib().cavs_session_create(C.byref(cfg), C.byref(self._h)), "cavs_session_create")
         self._keep = None

@@ -484,6 +484,28 @@ int cavs_fused_release(void *handle);
 int cavs_schedule_frontier(const int *parent, int N, int *tids_to_jobids, int *jobids_to_tids,
                            int *round_of_tid, int *round2offset, int *n_rounds, int *scratch,
                            void *stream);
+/* The whole per-step index arena on the GPU, from the graph feed as the application hands it over
+ * (cavs/midend/graph_scheduler.cc:12-71 LoadGraph, :169-245 Initialize / ActivateNext, and the
+ * index lists Gather / Scatter / Pull / FunctionPopRet read, cavs/backend/op_impl_graphop.cu:67-76,
+ * 148-157,241-249,304-318).  graph: device int32 [B, maxlen], entry j = local parent of vertex j,
+ * the first -1 ends the sample; nchild: children of an internal vertex (1 chains, 2 binary trees);
+ * pairing: 0 = the reference's (b-th entry of a round's compacted scatter list with slab row b),
+ * 1 = row-id preserving.  Outputs, device, `cap` >= B * maxlen rows each:
+ *   t2j [cap]            tensor id -> global vertex id (tids_to_jobids)
+ *   pair [cap]           slab row -> pool row its message is scattered to / gathered back from, -1 none
+ *   child [nchild * cap] slab row, child slot -> pool row of that child (the gather lists), -1 for leaves
+ *   kid_rows [nchild * cap]  the same by the slab row that wrote that pool row
+ *   roots [B]            vertex ids of the roots;  orphans [B]: slab rows with pair < 0, ascending
+ *   meta [maxlen + 9]    [0] N, [1] rounds R, [2] error bits (1 no terminator, 2 parent out of range,
+ *                        4 a vertex with children but not `nchild` of them, 8 single-vertex sample,
+ *                        16 parent cycle), [3] largest round, [8 + r] round2offset[r] for r <= R.
+ * Three dependent launches of one wavefront per sample / one workgroup per round (no grid-wide
+ * barrier): the schedule of a batch is the schedules of its samples merged round by round.  With
+ * error bits set the lists are undefined.  maxlen <= 2048. */
+size_t cavs_schedule_arena_scratch(int B, int maxlen);
+int cavs_schedule_arena(const int *graph, int B, int maxlen, int nchild, int pairing, int *t2j, int *pair,
+                        int *child, int *kid_rows, int *roots, int *orphans, long cap, int *meta,
+                        void *scratch, size_t scratch_bytes, void *stream);
 
 #ifdef __cplusplus
 }

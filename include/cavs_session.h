@@ -52,6 +52,15 @@ typedef struct {
    * d h of a round's children also does their gate gradients (one launch per backward round,
    * cavs_*_round_bwd_children_gates / _act); 1 = always two launches per round. */
   int split_backward_rounds;
+  /* Who builds the round schedule and the index lists of a step (cavs/midend/graph_scheduler.cc:
+   * 169-245): 0 = the host scheduler, lists uploaded once per step; 1 = the GPU
+   * (cavs_schedule_arena: the graph feed goes up, only the round offsets come back).  Mode 1 needs
+   * OPT_BATCHING and samples of at most 2048 vertices and falls back to 0 otherwise. */
+  int schedule_mode;
+  /* Plan cache: keep the schedule and the device-resident lists of the last `plan_cache` distinct
+   * graph feeds, keyed by the feed's bytes; a step on a feed seen before skips the scheduler and
+   * the upload.  0 = off. */
+  int plan_cache;
 } cavs_session_config;
 
 const char *cavs_session_error(void);
@@ -89,6 +98,21 @@ int cavs_session_schedule_trace(cavs_session *s, int *out, int cap);
 int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int with_backward,
                         int *out, int cap);
 
+/* Pure host calls (no device) around the index lists a step's kernels consume -- what the host
+ * scheduler uploads and what cavs_schedule_arena (cavs_hip.h) builds on the GPU; layouts as
+ * documented there.  cavs_schedule_index_lists: graph feed -> lists; arrays of N (t2j, pair),
+ * nchild * N (child, kid_rows), B (roots) and N (orphans) ints; *n_orphans = -1 and kid_rows /
+ * orphans undefined when the batch's message flow is not a forest or a round with children
+ * exceeds fused_limit.  Returns N, or 0 with the reason in cavs_session_error().
+ * cavs_schedule_trace_from_lists: the inverse -- lists and round offsets back to a complete
+ * schedule, serialised like cavs_schedule_trace. */
+int cavs_schedule_index_lists(const int *graph, int B, int maxlen, int nchild, int pairing, int fused_limit,
+                              int *t2j, int *pair, int *child, int *roots, int *kid_rows, int *orphans,
+                              int *n_orphans);
+int cavs_schedule_trace_from_lists(int B, int maxlen, int N, int nchild, const int *round2offset, int R,
+                                   const int *t2j, const int *pair, const int *child, const int *roots,
+                                   int with_backward, int *out, int cap);
+
 /* Timers of the last step in ms, by the reference's names (cavs/midend/statement.cc:
  * 53,65,68,84,102,122): "GraphParsing" (host), "RNNForward", "RNNBackward" (device); and the
  * host-side split "HostSchedule" (scheduler), "HostWait" (waiting for the device to release
@@ -105,7 +129,8 @@ int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double 
 void *cavs_session_stream(cavs_session *s);
 /* Per-step counts for roofline accounting: rows moved by indexed copies and GEMM flops
  * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" (separate GEMM launches)
- * "round_flops" (products inside fused round launches) "rounds" "launches". */
+ * "round_flops" (products inside fused round launches) "rounds" "launches"; "plan_hits" /
+ * "plan_misses" of the plan cache since the session was created. */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);
 
 #ifdef __cplusplus

@@ -115,6 +115,92 @@ def test_benchmark_configs_at_full_width(oracle, name, B):
     compare(got, want)
 
 
+@pytest.mark.parametrize("model,kw", CASES)
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_schedule_built_on_the_device(oracle, model, kw, pairing):
+    """schedule="device": the graph feed goes to the GPU, cavs_schedule_arena builds every index
+    list there and the host only learns the round offsets.  Same results as with the host
+    scheduler, against the oracle; the schedule read back from the device lists equals the
+    oracle's trace; and several steps in a row alternate the two sets of list buffers."""
+    loss = "softmax" if model != "treefc" else "root_sq"
+    batches = [small_workload(model, 171 + k, B=5 + 4 * k, H=32, E=12, V=31, C=5) for k in range(3)]
+    E = 32 if model == "lstm" else 12
+    names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv"),
+             "treefc": ("W", "Bv") if kw.get("use_bias") else ("W",)}[model]
+    if loss == "softmax":
+        names += ("Wfc", "bfc")
+    s = session.Session(model, H=32, E=E, V=31, C_=5, pairing=pairing, loss=loss, schedule="device", **kw)
+    s.set_params({k: batches[0]["params"][k] for k in names})
+    for step, w in enumerate(batches + batches[:1]):
+        print(f"[case] device schedule {model} {kw} pairing={pairing} step {step} N={w['N']}", flush=True)
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], batches[0]["params"], H=32, E=E, V=31, Cc=5,
+                                 pairing=pairing, loss=loss, precise=True, **kw)
+        s.step(w["graph"], w["x"], w["labels"], backward=True)
+        got = dict(loss=s.fetch("loss"), graph_out=s.fetch("graph_out"), dgraph_out=s.fetch("dgraph_out"),
+                   msg_pool=s.fetch("msg_pool"), grads=s.grads())
+        got["trace"] = s.schedule_trace()
+        assert got["trace"] == oracle.sched_trace(w["graph"])
+        compare(got, want)
+    s.close()
+
+
+def test_device_schedule_rejects_what_the_host_scheduler_rejects():
+    s = session.Session("treelstm", H=8, E=8, V=10, C_=3, schedule="device")
+    with pytest.raises(hip.CavsError, match="terminator"):
+        s.step(np.array([[1, 2, 0]], np.int32), np.zeros(3), np.zeros(3))
+    with pytest.raises(hip.CavsError, match="single-vertex"):
+        s.step(np.array([[-1, -1], [1, -1]], np.int32), np.zeros(3), np.zeros(3))
+    with pytest.raises(hip.CavsError, match="out of range"):
+        s.step(np.array([[7, 2, -1]], np.int32), np.zeros(3), np.zeros(3))
+    with pytest.raises(hip.CavsError, match="cycle"):
+        s.step(np.array([[1, 0, 3, -1]], np.int32), np.zeros(4), np.zeros(4))
+    with pytest.raises(hip.CavsError, match="two children|mixes"):
+        c = session.Session("lstm", H=8, V=10, C_=3, schedule="device")
+        c.step(np.array([[2, 2, -1]], np.int32), np.zeros(3), np.zeros(3))
+    s.close()
+
+
+@pytest.mark.parametrize("schedule", ["host", "device"])
+def test_plan_cache_replays_a_batch_structure_seen_before(oracle, schedule):
+    """plan_cache=2: three structures cycled.  A structure met again within the last two skips the
+    scheduler and the upload (plan_hits counts it) and gives the same step bit for bit as the
+    first time; the third structure evicts the least recently used one.  New vertex inputs on a
+    cached structure are a new computation on the old plan."""
+    ws = [small_workload("treelstm", 181 + k, B=6 + k, H=32, E=12, V=31, C=5) for k in range(3)]
+    s = session.Session("treelstm", H=32, E=12, V=31, C_=5, schedule=schedule, plan_cache=2)
+    s.set_params(ws[0]["params"])
+    seen = {}
+    order = [0, 1, 0, 0, 2, 0, 1]        # hits at steps 2, 3, 5; step 4 evicts plan 1; step 6 misses again
+    want_hits = [0, 0, 1, 2, 2, 3, 3]
+    for step, k in enumerate(order):
+        w = ws[k]
+        print(f"[case] plan cache schedule={schedule} step {step} structure {k}", flush=True)
+        s.step(w["graph"], w["x"], w["labels"], backward=True)
+        got = (s.fetch("loss"), s.fetch("graph_out"), s.grads())
+        assert s.counter("plan_hits") == want_hits[step], (step, s.counter("plan_hits"))
+        assert s.schedule_trace() == oracle.sched_trace(w["graph"])
+        if k in seen:
+            np.testing.assert_array_equal(got[0], seen[k][0])
+            np.testing.assert_array_equal(got[1], seen[k][1])
+            for name in ("dW", "dU", "dBv", "dWfc"):
+                np.testing.assert_array_equal(got[2][name], seen[k][2][name])
+        else:
+            want = oracle.model_step("treelstm", w["graph"], w["x"], w["labels"], ws[0]["params"], H=32, E=12, V=31, Cc=5,
+                                     precise=True)
+            close(got[0], want["loss"], "loss")
+            close(got[2]["dU"], want["grads"]["dU"], "dU")
+            seen[k] = got
+    # the same structure with other words: a hit, and the oracle's result for the new inputs
+    w = ws[0]
+    x2 = ((w["x"] + 3) % 31).astype(np.float32)
+    s.step(w["graph"], x2, w["labels"], backward=True)
+    assert s.counter("plan_hits") == 4
+    want = oracle.model_step("treelstm", w["graph"], x2, w["labels"], ws[0]["params"], H=32, E=12, V=31, Cc=5, precise=True)
+    close(s.fetch("loss"), want["loss"], "loss with new inputs")
+    close(s.grads()["dW"], want["grads"]["dW"], "dW with new inputs")
+    s.close()
+
+
 def test_steps_are_repeatable_and_sessions_reusable(oracle):
     """Two different batches through one session (buffers grow, lists are re-uploaded),
     then the first again: identical results, no state leaks between steps."""

@@ -563,6 +563,89 @@ def test_device_frontier_matches_host_schedule_bit_exact(g, oracle, kind, seed, 
     assert g.host(rot).tolist() == want_round.tolist()
 
 
+def _device_arena(g, graph, nch, pairing):
+    """Runs cavs_schedule_arena on a graph feed; returns (meta, lists) as numpy arrays."""
+    import torch
+
+    graph = np.ascontiguousarray(graph, np.int32)
+    B, maxlen = graph.shape
+    cap = B * maxlen + 7  # any capacity of at least B * maxlen rows
+    I = lambda k: torch.full((k,), -77, dtype=torch.int32, device="cuda")
+    t2j, pair, child, kid, roots, orph, meta = I(cap), I(cap), I(nch * cap), I(nch * cap), I(B), I(B), I(maxlen + 9)
+    nbytes = hip.lib().cavs_schedule_arena_scratch(B, maxlen)
+    scratch = I(nbytes // 4)
+    g.call("cavs_schedule_arena", g.P(g.devi(graph)), B, maxlen, nch, 0 if pairing == "reference" else 1, g.P(t2j), g.P(pair),
+           g.P(child), g.P(kid), g.P(roots), g.P(orph), cap, g.P(meta), g.P(scratch), nbytes, g.stream())
+    return g.host(meta), dict(t2j=g.host(t2j), pair=g.host(pair), child=g.host(child), kid=g.host(kid), roots=g.host(roots),
+                              orphans=g.host(orph))
+
+
+def _check_device_arena(g, oracle, graph, nch, pairing):
+    import arena
+
+    want = arena.expected_arena(oracle.sched_trace(graph), graph, nch, pairing)
+    meta, got = _device_arena(g, graph, nch, pairing)
+    N, R = want["N"], want["R"]
+    assert meta[2] == 0, f"error bits {meta[2]}"
+    assert (meta[0], meta[1]) == (N, R)
+    assert meta[8: 8 + R + 1].tolist() == want["round2offset"].tolist()
+    assert meta[3] == int(np.diff(want["round2offset"]).max())
+    assert got["t2j"][:N].tolist() == want["t2j"].tolist()
+    assert got["pair"][:N].tolist() == want["pair"].tolist()
+    assert got["child"][: nch * N].tolist() == want["child"].tolist()
+    assert got["kid"][: nch * N].tolist() == want["kid"].tolist()
+    assert got["roots"].tolist() == want["roots"].tolist()
+    assert got["orphans"].tolist() == want["orphans"].tolist()
+
+
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_device_scheduler_writes_the_whole_index_arena_bit_exact(g, oracle, pairing):
+    """cavs_schedule_arena against the lists of the oracle's scheduler: the hand-derived known
+    answers, skewed and same-shape batches of trees and chains, and the graphs of the benchmark
+    configurations C1-C5 at their own batch sizes."""
+    import json
+    import os
+
+    kats = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "sched_kat.json")))["cases"]
+    for case in kats:
+        graph = np.array(case["graph"], np.int32)
+        tr = oracle.sched_trace(graph)
+        # the arena is defined for what the kernels run: every internal vertex with all its children
+        arity = {len([1 for c in range(2) if rd["gather"][c]]) for rd in tr["fwd"][1:]}
+        if len(arity) != 1 or any(len(rd["gather"][c]) not in (0, len(rd["exec"])) for rd in tr["fwd"] for c in range(2)):
+            continue
+        print(f"[case] arena KAT {case['name']} pairing={pairing}", flush=True)
+        _check_device_arena(g, oracle, graph, arity.pop(), pairing)
+    for kind, seed, B, lo, hi in [("tree", 1, 1, 2, 2), ("tree", 2, 7, 2, 30), ("chain", 4, 9, 2, 40), ("tree", 5, 40, 32, 256),
+                                  ("chain", 6, 300, 1 + 1, 70)]:
+        print(f"[case] arena {kind} seed={seed} B={B} pairing={pairing}", flush=True)
+        graph = (synth.tree_batch if kind == "tree" else synth.chain_batch)(seed, B, lo, hi)[0]
+        _check_device_arena(g, oracle, graph, 2 if kind == "tree" else 1, pairing)
+    for name in ("C1", "C2", "C3", "C4", "C5"):
+        w = synth.make_workload(name, scale=0.03125)  # the graphs do not depend on the widths
+        print(f"[case] arena {name} B={w['graph'].shape[0]} N={w['N']} pairing={pairing}", flush=True)
+        _check_device_arena(g, oracle, w["graph"], 1 if w["model"] == "lstm" else 2, pairing)
+
+
+def test_device_scheduler_flags_what_the_host_scheduler_rejects(g):
+    bad = {
+        1: [[1, 2, 0, 0]],                      # no -1 within maxlen
+        2: [[5, 2, -1, -1]],                    # parent out of range
+        4: [[3, 3, 3, -1]],                     # three children
+        8: [[-1, -1, -1, -1], [1, -1, -1, -1]],  # single-vertex sample
+        16: [[1, 0, 3, -1]],                    # vertices 0 and 1 are each other's parent
+    }
+    for bit, graph in bad.items():
+        print(f"[case] arena error bit {bit}", flush=True)
+        meta, _ = _device_arena(g, np.array(graph, np.int32), 2, "reference")
+        assert meta[2] & bit, (bit, meta[:4])
+    # a chain fed to a binary vertex function: internal vertices with one child
+    meta, _ = _device_arena(g, np.array([[1, 2, -1]], np.int32), 2, "reference")
+    assert meta[2] & 4
+    meta, _ = _device_arena(g, np.array([[1, 2, -1]], np.int32), 1, "reference")
+    assert meta[2] == 0 and meta[0] == 3 and meta[1] == 3
+
+
 def test_reference_elementwise_smoke_values(g):
     """The Add the reference's op_impl_elementwise_test.cc prints: {1..6} + {0..5}."""
     import json

@@ -1,6 +1,7 @@
 """The production scheduler (cavs_amd/host/scheduler.cc) must expose bit-exactly the
 rounds and index lists of the reference's schedulers.  Checked against the hand-derived
 known answers and, over random batches, against the oracle.  Host only: no GPU."""
+import functools
 import json
 import os
 
@@ -20,6 +21,7 @@ def test_known_answers(case):
         assert tr[k] == case[k], k
 
 
+@functools.lru_cache(maxsize=None)
 def _graphs():
     out = []
     for seed in range(10):
@@ -50,3 +52,41 @@ def test_rejects_malformed_feeds():
         session.schedule_trace(np.array([[1, 2, 0]], np.int32))
     with pytest.raises(hip.CavsError, match="out of range"):
         session.schedule_trace(np.array([[5, -1, -1]], np.int32))
+    with pytest.raises(hip.CavsError, match="3 children"):
+        session.schedule_trace(np.array([[3, 3, 3, -1]], np.int32))
+    with pytest.raises(hip.CavsError, match="single-vertex"):
+        session.index_lists(np.array([[-1, -1], [1, -1]], np.int32), 1)
+    with pytest.raises(hip.CavsError, match="cycle"):   # vertices 0 and 1 are each other's parent
+        session.schedule_trace(np.array([[1, 0, 3, -1]], np.int32))
+    with pytest.raises(hip.CavsError, match="cycle"):   # a vertex that is its own parent
+        session.schedule_trace(np.array([[0, 2, -1]], np.int32))
+
+
+@pytest.mark.parametrize("idx", range(18))
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_index_lists_match_the_oracles_schedule_and_invert(oracle, idx, pairing):
+    """The lists the kernels consume (one entry per slab row) against the oracle's per-round
+    lists, and back: the lists alone determine the complete schedule."""
+    import arena
+
+    graph = _graphs()[idx]
+    tr = oracle.sched_trace(graph)
+    nch = 2 if any(rd["gather"][1] for rd in tr["fwd"]) else 1
+    want = arena.expected_arena(tr, graph, nch, pairing)
+    got = session.index_lists(graph, nch, pairing)
+    assert got["N"] == want["N"]
+    for k in ("t2j", "pair", "child", "roots", "kid", "orphans"):
+        assert got[k].tolist() == want[k].tolist(), k
+    B, maxlen = graph.shape
+    back = session.trace_from_lists(B, maxlen, nch, tr["round2offset"], got["t2j"], got["pair"], got["child"], got["roots"])
+    assert back == session.schedule_trace(graph) == tr
+
+
+def test_index_lists_refuse_mixed_arity_and_report_non_forests():
+    with pytest.raises(hip.CavsError, match="mixes"):    # a chain inside a binary vertex function
+        session.index_lists(np.array([[1, 2, -1]], np.int32), 2)
+    with pytest.raises(hip.CavsError, match="two children"):
+        session.index_lists(np.array([[2, 2, -1]], np.int32), 1)
+    g = synth.tree_batch(7, 9, 2, 20)[0]
+    assert session.index_lists(g, 2)["kid"] is not None
+    assert session.index_lists(g, 2, fused_limit=3)["kid"] is None   # a round with children above the limit

@@ -182,3 +182,41 @@ def test_rejects_sample_without_terminator(oracle):
     n = oracle.lib().or_sched_trace(g.ctypes.data_as(C.c_void_p), 1, 3, 1, 0,
                                     out.ctypes.data_as(C.c_void_p), 64)
     assert n == 0  # LoadGraph's length CHECK (graph_scheduler.cc:41)
+
+
+@pytest.mark.parametrize("kind,seed,B,lo,hi", [("tree", 11, 5, 2, 9), ("tree", 12, 33, 2, 40), ("chain", 13, 9, 2, 30),
+                                               ("tree", 14, 1, 7, 7)])
+def test_batch_schedule_is_the_samples_schedules_merged_round_by_round(oracle, kind, seed, B, lo, hi):
+    """What the device scheduler builds on: every round of a batch lists its vertices sample by
+    sample, each sample's in the order that sample alone would produce them, so
+    tensor id = round2offset[r] + (vertices of earlier samples in round r) + position in the
+    sample's own round; and under the reference pairing slab row (tensor id - roots of earlier
+    samples in the round) holds the message of a non-root vertex."""
+    import arena
+
+    graph = (synth.tree_batch if kind == "tree" else synth.chain_batch)(seed, B, lo, hi)[0]
+    tr = oracle.sched_trace(graph)
+    nch = 2 if kind == "tree" else 1
+    want = arena.expected_arena(tr, graph, nch, "reference")
+    singles = [oracle.sched_trace(graph[i:i + 1]) for i in range(B)]
+    R = len(tr["fwd"])
+    cnt = np.zeros((B, R + 1), np.int64)
+    for s, st in enumerate(singles):
+        for r, rd in enumerate(st["fwd"]):
+            cnt[s, r] = len(rd["exec"])
+    depth = [len(st["fwd"]) for st in singles]
+    r2o = np.concatenate([[0], np.cumsum(cnt.sum(0))])
+    assert r2o[: R + 1].tolist() == tr["round2offset"]
+    soff = np.concatenate([[0], np.cumsum([st["N"] for st in singles])])
+    t2j, pair = np.full(tr["N"], -1), np.full(tr["N"], -1)
+    for s, st in enumerate(singles):
+        for r, rd in enumerate(st["fwd"]):
+            before = cnt[:s, r].sum()
+            roots_before = sum(1 for q in range(s) if depth[q] - 1 == r)
+            for i, v in enumerate(rd["exec"]):
+                t = r2o[r] + before + i
+                t2j[t] = soff[s] + v
+                if r < depth[s] - 1:
+                    pair[t - roots_before] = t
+    assert t2j.tolist() == want["t2j"].tolist()
+    assert pair.tolist() == want["pair"].tolist()
