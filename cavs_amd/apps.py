@@ -45,10 +45,11 @@ class App:
     declare the program (no device)."""
 
     def __init__(self, model, *, B, maxlen, H, E=0, V=0, C_=0, opt=session.OPT_BATCHING, lr=0.0, clip=0.0,
-                 pairing="reference", allow_fused=True):
+                 pairing="reference", allow_fused=True, iters=1):
         a, _ = libs()
         self.model, self.B, self.maxlen, self.H, self.E, self.V, self.C = model, B, maxlen, H, E, V, C_
         a.cavs_app_set_clip(C.c_float(clip))
+        a.cavs_app_set_iters(int(iters))
         rc = a.cavs_app_create(model.encode(), B, maxlen, V, E, H, C_, opt, lr)
         if rc != 0:
             raise hip.CavsError(f"cavs_app_create({model}) -> {rc}")

@@ -161,6 +161,9 @@ extern "C" {
 // gradient clipping threshold of the optimizer the next cavs_app_create declares (0: none)
 static float g_clip = 0.f;
 void cavs_app_set_clip(float clip) { g_clip = clip; }
+// passes of the optimizer's scope per Session::Run of the next app (Optimizer(vars, lr, clip, iters))
+static int g_iters = 1;
+void cavs_app_set_iters(int iters) { g_iters = iters > 0 ? iters : 1; }
 
 int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, int C, int opt, float lr) {
   try {
@@ -213,7 +216,7 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       app->loss = app->graph_output.Reduce_sum();  // tree-fc-cavs.cc:96
       app->total = app->loss;
     }
-    app->train = app->loss.Optimizer({}, lr, g_clip);
+    app->train = app->loss.Optimizer({}, lr, g_clip, g_iters);
     if (opt >= 0) app->sess = std::make_unique<Session>(opt);  // opt < 0: declare only (no device needed)
     g_app = app.release();
     return 0;

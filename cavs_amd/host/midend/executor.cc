@@ -175,11 +175,22 @@ void Executor::compile() {
   for (auto &n : g.main.nodes) main_all_.push_back(n->def);
   if (g.func)
     for (auto &n : g.func->nodes) func_fwd_.push_back(n->def);
+  round_zero_.clear();
   if ((opt_ & OPT_FUSION) && g.func && !lowered_) {
     std::vector<OpDef> fwd = fused(func_fwd_, {&func_bwd_, &func_def_, &main_all_, &g.opt.backward}, {});
-    std::vector<OpDef> bwd = fused(func_bwd_, {&func_fwd_, &func_def_, &main_all_, &g.opt.backward}, {});
+    // the per-round backward program, with the deferred ops that fit riding along as reducing outputs
+    FusionEnv env = graph_env(g);
+    for (auto *o : {&func_fwd_, &main_all_, &g.opt.backward})
+      for (auto &d : *o)
+        for (int k = 0; k < operands_read(d); k++) env.live.insert(d.input(k));
+    for (auto &v : g.opt.vars) env.live.insert(GetGradientName(v));
+    BackwardFusion bf = fuse_function_backward(func_bwd_, func_def_, env);
+    fused_groups_ += bf.groups;
+    round_zero_ = bf.zero_before_loop;
+    std::vector<OpDef> &kept_bwd = bf.per_round, &new_def = bf.deferred;
     func_fwd_.swap(fwd);
-    func_bwd_.swap(bwd);
+    func_bwd_.swap(kept_bwd);
+    func_def_.swap(new_def);
   }
 }
 
@@ -207,11 +218,15 @@ void Executor::exec_fused(const OpDef &d, const RoundCtx &c) {
   std::vector<float *> outs;
   std::vector<const float *> ins;
   std::vector<int> oc, ic;
+  // the element range is that of the widest argument (cavs/backend/op_impl_fused_kernel.cu:44-58);
+  // outputs narrower than it are added to with atomicAdd
   long cnt, w, n_elements = 0;
   for (auto &x : d.input()) {
     ins.push_back(view(x, c, &cnt, &w));
     ic.push_back((int)cnt);
+    n_elements = std::max(n_elements, cnt);
   }
+  const std::vector<std::string> zero_first = GetListArgS(d, "ZeroEnforced");
   for (int i = 0; i < d.output_size(); i++) {
     const std::string &name = d.output(i);
     const Edge *e = edge(name);
@@ -230,6 +245,10 @@ void Executor::exec_fused(const OpDef &d, const RoundCtx &c) {
     outs.push_back(view(name, c, &cnt, &w));
     oc.push_back((int)cnt);
     n_elements = std::max(n_elements, cnt);
+    // a reduced output this kernel is the first writer of starts from zero: here, or -- inside the
+    // backward round loop, where every round adds to it -- once before the loop
+    if (!c.in_round_loop && std::find(zero_first.begin(), zero_first.end(), name) != zero_first.end())
+      check(cavs_zero(outs.back(), (size_t)cnt * 4, stream_));
   }
   if (n_elements == 0) return;
   check(cavs_fused_launch(h, outs.data(), (int)outs.size(), ins.data(), (int)ins.size(), oc.data(), ic.data(),
@@ -653,9 +672,25 @@ void Executor::run_graph_output_grad(const OpDef &d) {
     lowered_backward(d);
     return;
   }
+  // outputs the per-round generated kernels add every round's rows onto
+  for (auto &name : round_zero_) {
+    const Edge *e = edge(name);
+    if (!e) fail(CAVS_EINVAL, "no edge for reduced output '" + name + "'");
+    auto &slot = tensors_[name];
+    if (!slot) slot = std::make_unique<Tensor>();
+    Tensor &t = *slot;
+    t.width = e->width();
+    t.per_vertex = false;
+    if (t.own.capacity() < t.count()) {
+      check(cavs_stream_sync(stream_));
+      t.own.reserve(t.count());
+    }
+    if (!t.base) t.base = t.own.get();
+    check(cavs_zero(t.base, t.count() * 4, stream_));
+  }
   for (int k : sched_.bwd_rounds) {
     const Round &r = sched_.rounds[k];
-    RoundCtx c{r.offset, r.n, true};
+    RoundCtx c{r.offset, r.n, true, true};
     for (const OpDef &gd : func_bwd_) exec(gd, c);
   }
   RoundCtx all{0, N_, true};
@@ -738,6 +773,11 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
   }
   binds_ = &it->second.binds;
   const HeadFuse &head = it->second.head;
+  // The optimizer's scope -- the replayed forward ops, the gradients and the update -- runs
+  // `iters` times per Run (ScopedNode(s_, name, iters), cavs/midend/graph_util.cc:266-283;
+  // BasicBlock::Run, cavs/midend/statement.h:66-75).
+  const int passes = train ? std::max(1, g.opt.iters) : 1;
+  for (int pass = 0; pass < passes; pass++) {
   bool head_fused = false;
   for (size_t i = 0; i < it->second.fwd.size(); i++) {
     const OpDef &d = it->second.fwd[i];
@@ -779,6 +819,7 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     }
     check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
   }
+  }  // passes
   results->assign(outputs.size(), nullptr);
   // A Run that asks for the optimizer only (the training loop of the reference's apps) has
   // nothing to hand back: it returns with the step still in flight, and the host prepares the

@@ -64,6 +64,7 @@ class Executor {
   struct RoundCtx {
     long off = 0, n = 0;
     bool in_function = false;
+    bool in_round_loop = false;  // one of the backward rounds: reduced outputs were zeroed before the loop
   };
   void compile();
   void init_variables();
@@ -108,6 +109,7 @@ class Executor {
   const float *dgo_ = nullptr;        // d GraphOutput during the backward function
   // programs of the vertex function as executed (after the fusion pass when OPT_FUSION is set)
   std::vector<OpDef> func_fwd_, func_bwd_, func_def_;
+  std::vector<std::string> round_zero_;  // reduced outputs of the per-round generated kernels: zeroed before the backward loop
   std::vector<OpDef> main_all_;
   // The lowered F writes a parameter's gradient where the main scope wants it: when the gradients
   // of all the slices of a Variable come out of the lowered F and only get added into the

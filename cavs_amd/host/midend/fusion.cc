@@ -77,15 +77,32 @@ struct UnionFind {
 std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv &env, int *groups_made) {
   const int n = (int)prog.size();
   static int kernel_id = 0;
-  // An op can join a group only if every output covers the full element range of the op
-  // (no reducing outputs) -- the generator's atomicAdd path for narrower outputs is not used.
-  // The class of an op is (per-row?, width) of its single output, encoded as +-width; -1... 0
-  // means "cannot be fused".  Operands have the same class or are static rows that divide it.
-  auto full_count = [&](const OpDef &d) -> long {
+  // The class of an op is the geometry of the element range it runs over, (per-row?, width)
+  // encoded as +-width; 0 means "cannot be fused".  Operands have the same class or are static
+  // rows that divide it.  The output normally covers the whole range.  A *reducing* op is one
+  // whose operands are per-row slabs while its output is a static row whose width divides
+  // theirs (the gradient of an operand that was broadcast over the rows: a bias): it runs over
+  // its operands' range and every element is added onto out[idx % out_count] -- the
+  // generator's atomicAdd form for outputs narrower than n_elements
+  // (cavs/midend/runtime_compiler/code_generator.cc:84-100).
+  std::vector<char> reducing(n, 0);
+  auto full_count = [&](const OpDef &d, char *reduces) -> long {
+    *reduces = 0;
     if (d.output_size() != 1 || d.input_size() < arity(d.name())) return 0;
-    const bool rows = env.per_row(d.output(0));
-    const long w = env.width(d.output(0));
+    bool rows = env.per_row(d.output(0));
+    long w = env.width(d.output(0));
     if (w <= 0) return 0;
+    if (!rows) {
+      long win = 0;
+      for (int k = 0; k < arity(d.name()); k++)
+        if (env.per_row(d.input(k))) win = std::max(win, env.width(d.input(k)));
+      if (win > 0) {  // per-row operands, static output
+        if (win % w != 0) return 0;
+        *reduces = 1;
+        rows = true;
+        w = win;
+      }
+    }
     for (int k = 0; k < arity(d.name()); k++) {
       const std::string &i = d.input(k);
       long wi = env.width(i);
@@ -102,7 +119,7 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
   std::map<std::string, int> producer;  // last writer of an edge within the program
   std::vector<std::vector<int>> readers_of(n);
   for (int i = 0; i < n; i++) {
-    if (fusable(prog[i].name())) width[i] = full_count(prog[i]);
+    if (fusable(prog[i].name())) width[i] = full_count(prog[i], &reducing[i]);
     for (auto &o : prog[i].output()) producer[o] = i;
   }
   UnionFind uf(n);
@@ -114,7 +131,9 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
         auto it = last.find(in);
         if (it == last.end()) continue;
         int p = it->second;
-        if (width[i] != 0 && width[i] == width[p]) uf.unite(i, p);
+        // (what a reducing op produces is complete only when its kernel has finished: nobody
+        // joins a group through it)
+        if (width[i] != 0 && width[i] == width[p] && !reducing[p]) uf.unite(i, p);
       }
       for (auto &o : prog[i].output()) last[o] = i;
     }
@@ -160,15 +179,32 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
       work.push_back(below);
       continue;
     }
+    {
+      // a member must not read what a reducing member of the same group adds up
+      std::set<std::string> reduced;
+      int offender = -1;
+      for (int i : members) {
+        for (int k = 0; k < arity(prog[i].name()) && offender < 0; k++)
+          if (reduced.count(prog[i].input(k))) offender = i;
+        if (reducing[i]) reduced.insert(prog[i].output(0));
+      }
+      if (offender >= 0) {
+        std::vector<int> above, below;
+        for (int i : members) (i < offender ? above : below).push_back(i);
+        work.push_back(above);
+        work.push_back(below);
+        continue;
+      }
+    }
     int benefit = 0;
-    for (int i : members) benefit += deserved(prog[i].name());
+    for (int i : members) benefit += deserved(prog[i].name()) || reducing[i];
     if (members.size() < 2 || benefit <= 1) continue;  // parser.cc:118-131: kept iff benefit > 1
 
     std::set<int> in(members.begin(), members.end());
     const long cls = width[members[0]];
     std::set<std::string> written;
-    std::vector<std::string> inputs, outputs, stateful;
-    std::set<std::string> seen_in;
+    std::vector<std::string> inputs, outputs, stateful, zero_first;
+    std::set<std::string> seen_in, reduced_out;
     std::ostringstream body;
     bool clash = false;
     for (int i : members) {
@@ -181,6 +217,20 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
       }
       const std::string &o = d.output(0);
       bool acc = accumulates(d, 0);
+      if (reducing[i]) {
+        // tmp_o holds this element's contribution only; the store adds it onto out[idx % count].
+        // An output the group is the first writer of must be zero when the kernel first runs.
+        if (written.count(o) && !reduced_out.count(o)) { clash = true; break; }
+        if (seen_in.count(o)) { clash = true; break; }
+        std::string e = expression(d, args);
+        if (reduced_out.count(o)) body << "    tmp_" << o << " = tmp_" << o << " + (" << e << ");\n";
+        else body << "    float tmp_" << o << " = " << e << ";\n";
+        if (!acc && !reduced_out.count(o)) zero_first.push_back(o);
+        reduced_out.insert(o);
+        written.insert(o);
+        continue;
+      }
+      if (reduced_out.count(o)) { clash = true; break; }
       if (acc && !written.count(o)) {  // accumulates onto a value produced outside the group
         if (seen_in.count(o)) { clash = true; break; }  // read as an operand and updated in place
         stateful.push_back(o);
@@ -224,11 +274,20 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
     };
     for (auto &x : inputs) src << "    float tmp_" << x << " = " << x << index(x) << ";\n";
     src << body.str();
-    for (auto &o : outputs) src << "    " << o << "[idx] = tmp_" << o << ";\n";
+    for (auto &o : outputs) {
+      if (reduced_out.count(o)) src << "    atomicAdd(&" << o << "[idx % " << o << "_count], tmp_" << o << ");\n";
+      else src << "    " << o << "[idx] = tmp_" << o << ";\n";
+    }
     src << "  }\n}\n";
+    // Stateful: outputs the kernel accumulates onto a value written before it; Reduced: outputs
+    // narrower than the element range, added to with atomicAdd; ZeroEnforced: those of them the
+    // kernel is the first writer of, which must hold zero before its first launch of an iteration
+    // (code_generator.cc:155-164; the reference zeroes such buffers once per iteration,
+    // cavs/midend/tensor.cc:283-300)
     OpDefBuilder b("FusedKernel");
     b.Input(inputs).Output(outputs).AttrSingle("KernelName", name).AttrSingle("KernelSource", src.str())
-        .AttrList("ZeroEnforced", stateful);
+        .AttrList("Stateful", stateful).AttrList("Reduced", std::vector<std::string>(reduced_out.begin(), reduced_out.end()))
+        .AttrList("ZeroEnforced", zero_first);
     fused_at[members.back()] = b.Finalize();
     for (int i : members) group_of[i] = members.back();
     made++;
@@ -239,6 +298,50 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
     else if (group_of[i] == i) out.push_back(fused_at[i]);
   }
   if (groups_made) *groups_made = made;
+  return out;
+}
+
+BackwardFusion fuse_function_backward(const std::vector<OpDef> &per_round, const std::vector<OpDef> &deferred, FusionEnv env) {
+  BackwardFusion out;
+  std::vector<OpDef> offered = per_round;
+  std::map<std::string, int> writers;
+  for (auto &d : deferred)
+    for (auto &o : d.output()) writers[o]++;
+  std::vector<char> moved(deferred.size(), 0);
+  for (size_t i = 0; i < deferred.size(); i++) {
+    const OpDef &d = deferred[i];
+    if (d.name() != "Assign" && d.name() != "Accumulate" && d.name() != "Neg") continue;
+    if (d.output_size() != 1 || d.input_size() < 1 || accumulates(d, 0) || writers[d.output(0)] != 1) continue;
+    if (env.per_row(d.output(0)) || !env.per_row(d.input(0))) continue;
+    // right behind the op that produces its operand, so that nothing between them reads what the
+    // group they may form produces
+    int at = -1;
+    for (size_t j = 0; j < offered.size(); j++)
+      for (auto &o : offered[j].output())
+        if (o == d.input(0)) at = (int)j;
+    if (at < 0) continue;  // the operand does not come out of the per-round program
+    moved[i] = 1;
+    offered.insert(offered.begin() + at + 1, d);
+  }
+  for (size_t i = 0; i < deferred.size(); i++)
+    if (!moved[i])
+      for (int k = 0; k < operands_read(deferred[i]); k++) env.live.insert(deferred[i].input(k));
+  std::vector<OpDef> fused = fuse_program(offered, env, &out.groups);
+  std::set<std::string> came_back;  // offered ops the pass left as they were
+  for (auto &d : fused) {
+    bool was_deferred = false;
+    for (size_t i = 0; i < deferred.size(); i++)
+      if (moved[i] && d.name() == deferred[i].name() && d.output_size() == 1 && d.output(0) == deferred[i].output(0)) was_deferred = true;
+    if (was_deferred) {
+      came_back.insert(d.output(0));
+    } else {
+      out.per_round.push_back(d);
+      if (d.name() == "FusedKernel")
+        for (auto &z : GetListArgS(d, "ZeroEnforced")) out.zero_before_loop.push_back(z);
+    }
+  }
+  for (size_t i = 0; i < deferred.size(); i++)
+    if (!moved[i] || came_back.count(deferred[i].output(0))) out.deferred.push_back(deferred[i]);
   return out;
 }
 
@@ -291,7 +394,9 @@ std::string dump_fused(const Graph &g) {
   emit("main", fuse_program(main_all, live_of({&fwd, &g.func_backward, &g.func_deferred, &g.opt.backward})));
   if (g.func) {
     emit("function", fuse_program(fwd, live_of({&g.func_backward, &g.func_deferred, &main_all, &g.opt.backward})));
-    emit("function_grad", fuse_program(g.func_backward, live_of({&fwd, &g.func_deferred, &main_all, &g.opt.backward})));
+    BackwardFusion bf = fuse_function_backward(g.func_backward, g.func_deferred, live_of({&fwd, &main_all, &g.opt.backward}));
+    emit("function_grad", bf.per_round);
+    emit("function_grad_deferred", bf.deferred);
   }
   if (g.opt.present) emit("backward", fuse_program(g.opt.backward, live_of({&fwd, &g.func_backward, &g.func_deferred})));
   return o.str();

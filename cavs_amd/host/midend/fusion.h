@@ -33,6 +33,22 @@ std::vector<OpDef> fuse_program(const std::vector<OpDef> &prog, const FusionEnv 
 // operands of `d` that its implementation reads (the *_grad operators carry an unused one)
 int operands_read(const OpDef &d);
 
+// The backward vertex function after the pass.  Its deferred part (the gradient ops that run
+// once over all rows after the round loop, cavs/midend/batch_weight_updater.h:12-84) holds ops
+// that only add a per-row value up over the rows -- the gradient of an operand that was broadcast
+// over the rows, e.g. a bias.  Such an op can ride in a per-round generated kernel as a reducing
+// output: the kernel adds each round's rows onto the output, which is zeroed once before the
+// loop (`zero_before_loop`).  They are offered to the pass behind the per-round program; those
+// it does not take into a kernel stay deferred.  Only the sole writer of its output qualifies
+// (another deferred writer would run after it and overwrite the sum).  `env.live` must hold what
+// everything outside the backward function reads.
+struct BackwardFusion {
+  std::vector<OpDef> per_round, deferred;
+  std::vector<std::string> zero_before_loop;
+  int groups = 0;
+};
+BackwardFusion fuse_function_backward(const std::vector<OpDef> &per_round, const std::vector<OpDef> &deferred, FusionEnv env);
+
 struct Graph;
 // geometry callbacks over the declared program (the live set is left empty)
 FusionEnv graph_env(const Graph &g);

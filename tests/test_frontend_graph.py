@@ -107,3 +107,28 @@ def test_fusion_pass_keeps_small_groups_unfused():
         a.close()
     fn = d[d.index("function:"):d.index("function_grad:")]
     assert "FusedKernel(" not in fn  # forward F has a single Relu
+
+
+def test_fusion_pass_takes_bias_gradients_in_as_reducing_outputs():
+    """The gradient of a bias is a sum over the rows of a per-row value.  The pass takes those
+    deferred ops into the per-round backward kernel as outputs narrower than the element range,
+    stored with atomicAdd onto out[idx % out_count] (cavs/midend/runtime_compiler/
+    code_generator.cc:84-100) and listed in ZeroEnforced; what reads the sums stays deferred."""
+    import re
+    from cavs_amd import apps
+
+    for model, reduced in (("treefc_x", 1), ("treelstm", 5), ("lstm", 4)):
+        a = apps.App(model, B=2, maxlen=7, H=8, E=8, V=10, C_=3, opt=-1, lr=0.1)
+        try:
+            d = a.dump_fused()
+        finally:
+            a.close()
+        bw = d[d.index("function_grad:"):d.index("function_grad_deferred:")]
+        deferred = d[d.index("function_grad_deferred:"):d.index("backward:")]
+        stores = re.findall(r"atomicAdd\(&(\w+)\[idx % \1_count\], tmp_\1\);", bw)
+        assert len(stores) == reduced, (model, stores)
+        for name in stores:
+            assert f"{name}[idx] =" not in bw                       # never stored as a full-range output
+            assert not re.search(rf"= {name}\[idx", bw)             # nor read back
+            assert re.search(rf"^  \w+\({name}[,)]", deferred, re.M)  # its reader runs after the loop
+            assert not re.search(rf"-> \({name}\)", deferred)       # the op that produced it is gone from there

@@ -234,3 +234,26 @@ def test_optimizer_with_gradient_clipping(oracle):
         step = np.float32(lr) * np.float32(0.25) * want["grads"]["d" + k].reshape(shapes[k])
         close(a.grad(k, shapes[k], grad=False), p0 - step, f"{k} after a clipped step")
     a.close()
+
+
+@pytest.mark.parametrize("allow_fused", [True, False])
+def test_optimizer_iters_runs_the_training_scope_that_many_times_per_run(allow_fused):
+    """Optimizer(vars, lr, clip, iters): one Session::Run makes `iters` passes of forward, backward
+    and update (ScopedNode(s_, name, iters), cavs/midend/graph_util.cc:266-283).  One Run with
+    iters=3 leaves the variables where three Runs with iters=1 leave them (up to the summation order
+    of the embedding gradient's atomics)."""
+    w = small_workload("lstm", 88, B=4, H=16, V=19, C=4)
+    B, maxlen = w["graph"].shape
+    finals = []
+    for iters, runs in ((1, 3), (3, 1)):
+        a = apps.App("lstm", B=B, maxlen=maxlen, H=16, E=16, V=19, C_=4, opt=session.OPT_BATCHING, lr=0.25, iters=iters,
+                     allow_fused=allow_fused)
+        a.set_params(w["params"])
+        for _ in range(runs):
+            print(f"[case] iters={iters} fused={allow_fused}", flush=True)
+            a.step(w["graph"], w["x"], w["labels"], train=True)
+        finals.append({k: a.grad(k, shp, grad=False) for k, shp in (("W", (8 * 16 * 16,)), ("Bv", (64,)), ("Wfc", (4, 16)))})
+        a.close()
+    assert not np.array_equal(finals[0]["W"], np.asarray(w["params"]["W"], np.float32).ravel())
+    for k in finals[0]:
+        close(finals[0][k], finals[1][k], k, rtol=1e-5, atol=1e-6)

@@ -529,6 +529,43 @@ extern "C" __global__ void FusedKernel_0(float *E, const float *A, const float *
     ic = (C.c_int * 3)(6, 6, 6)
     hip.call("cavs_fused_launch", h, outs, 1, ins, 3, oc, ic, 6, g.stream())
     np.testing.assert_allclose(g.host(out), [7.1, 7.2, 7.3, 7.4, 7.5, 7.6], rtol=1e-6)
+    # an output narrower than the element range: the generator's atomicAdd branch.  Six elements onto
+    # a row of three (elements k and k + 3 land on E[k]); E starts at zero, as ZeroEnforced makes it
+    row = g.zeros(3)
+    outs = (C.c_void_p * 1)(g.P(row))
+    oc = (C.c_int * 1)(3)
+    hip.call("cavs_fused_launch", h, outs, 1, ins, 3, oc, ic, 6, g.stream())
+    np.testing.assert_allclose(g.host(row), [7.1 + 7.4, 7.2 + 7.5, 7.3 + 7.6], rtol=1e-6)
+    hip.call("cavs_fused_release", h)
+    # the form this build's fusion pass emits for a reducing output: the element's contribution is
+    # added, nothing is read back; a broadcast operand wraps
+    src2 = r'''
+extern "C" __global__ void FusedKernel_1(float *S, float *Y, const float *X, const float *b,
+    const int S_count, const int Y_count, const int X_count, const int b_count, const int n_elements)
+{
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < n_elements) {
+    float tmp_X = X[idx];
+    float tmp_b = b[idx % b_count];
+    float tmp_Y = tmp_X * tmp_b;
+    float tmp_S = tmp_Y;
+    atomicAdd(&S[idx % S_count], tmp_S);
+    Y[idx] = tmp_Y;
+  }
+}'''
+    hip.call("cavs_fused_compile", b"FusedKernel_1", src2.encode(), C.byref(h))
+    n, w = 700, 40
+    r = rng(5)
+    X, bvec = r.bulk_normal(n * w).reshape(n, w), r.bulk_normal(w)
+    S, Y = g.zeros(w), g.zeros(n, w)
+    outs = (C.c_void_p * 2)(g.P(S), g.P(Y))
+    ins = (C.c_void_p * 2)(g.P(g.devf(X)), g.P(g.devf(bvec)))
+    oc = (C.c_int * 2)(w, n * w)
+    ic = (C.c_int * 2)(n * w, w)
+    hip.call("cavs_fused_launch", h, outs, 2, ins, 2, oc, ic, n * w, g.stream())
+    want = X.astype(np.float64) * bvec.astype(np.float64)
+    close(g.host(Y), want, "Y")
+    close(g.host(S), want.sum(0), "column sums through atomicAdd")
     hip.call("cavs_fused_release", h)
     bad = C.c_void_p()
     with pytest.raises(hip.CavsError, match="compile"):
