@@ -42,7 +42,6 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
     check(cavs_stream_create(&stream_));
   }
   for (auto &e : ev_) check(cavs_event_create(&e));
-  for (auto &e : idx_copied_) check(cavs_event_create(&e));
   switch (cfg.model) {
     case CAVS_MODEL_TREELSTM:
       add_param("Emb", (size_t)cfg.V * E_);
@@ -68,7 +67,10 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
 Engine::~Engine() {
   cavs_stream_sync(stream_);
   for (auto &e : ev_) cavs_event_destroy(e);
-  for (auto &e : idx_copied_) cavs_event_destroy(e);
+  for (auto &h : hlists_) {
+    if (h.free_ev) cavs_event_destroy(h.free_ev);
+    if (h.up_ev) cavs_event_destroy(h.up_ev);
+  }
   for (auto &e : prof_events_) cavs_event_destroy(e);
   if (sched_stream_) {
     cavs_stream_sync(sched_stream_);
@@ -326,30 +328,33 @@ void Engine::upload_index_arena() {
   const int N = N_;
   const bool want_forest = !cfg_.split_backward_rounds && fused_rows() > 0;
   const size_t total = (size_t)N * (2 + nch_) + s.B + (want_forest ? (size_t)N * (nch_ + 1) : 0);
-  // two pinned staging buffers alternate, so the host can build the lists of the next
-  // step while the device still runs this one; a buffer is rewritten only after the
-  // upload that last read it has finished
-  const int slot = idx_slot_;
-  idx_slot_ ^= 1;
-  if (idx_pending_[slot]) {
+  // Two sets of buffers (pinned staging + device lists) alternate, and the copy runs on a stream
+  // of its own: the lists of step k + 1 are built and uploaded while the kernels of step k run,
+  // instead of the copy sitting in the compute stream between two steps.  A set is rewritten only
+  // after everything that read its device lists has finished (the step before last).
+  HostLists &h = hlists_[hlists_slot_];
+  hlists_slot_ ^= 1;
+  if (!sched_stream_) check(cavs_stream_create(&sched_stream_));
+  if (!h.free_ev) check(cavs_event_create(&h.free_ev));
+  if (!h.up_ev) check(cavs_event_create(&h.up_ev));
+  if (h.busy) {
     auto w0 = std::chrono::steady_clock::now();
-    check(cavs_event_sync(idx_copied_[slot]));
+    check(cavs_event_sync(h.free_ev));
     wait_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - w0).count();
+    h.busy = false;
   }
-  idx_pending_[slot] = false;
-  idx_host_[slot].reserve(total);
-  if (idx_dev_.capacity() < total) {
-    check(cavs_stream_sync(stream_));
-    idx_dev_.reserve(grow(total, idx_dev_.capacity()));
-  }
-  int *t2j = idx_host_[slot].get(), *pair = t2j + N, *child = pair + N, *roots = child + (size_t)nch_ * N;
+  h.host.reserve(total);
+  h.dev.reserve(grow(total, h.dev.capacity()));
+  int *t2j = h.host.get(), *pair = t2j + N, *child = pair + N, *roots = child + (size_t)nch_ * N;
   std::string err = build_index_lists(s, nch_, cfg_.pairing, t2j, pair, child, roots);
   if (!err.empty()) fail(CAVS_EUNSUPPORTED, err);
   forest_ = want_forest && build_forest_lists(s, nch_, fused_rows(), pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N, &n_orphans_);
-  check(cavs_memcpy_h2d(idx_dev_.get(), idx_host_[slot].get(), total * sizeof(int), stream_));
-  check(cavs_event_record(idx_copied_[slot], stream_));
-  idx_pending_[slot] = true;
-  d_t2j_ = idx_dev_.get();
+  check(cavs_memcpy_h2d(h.dev.get(), h.host.get(), total * sizeof(int), sched_stream_));
+  check(cavs_event_record(h.up_ev, sched_stream_));
+  check(cavs_event_sync(h.up_ev));  // a few microseconds; the compute stream is still busy with the previous step
+  last_free_ev_ = h.free_ev;
+  last_busy_ = &h.busy;
+  d_t2j_ = h.dev.get();
   d_pair_ = d_t2j_ + N;
   d_child_ = d_pair_ + N;
   d_roots_ = d_child_ + (size_t)nch_ * N;
@@ -524,7 +529,8 @@ void Engine::schedule_on_device(const int *graph, int B, int maxlen) {
   n_orphans_ = B;
   forest_ = !cfg_.split_backward_rounds && fused_rows() > 0;
   for (int r = 1; r < R && forest_; r++) forest_ = s.rounds[r].n <= fused_rows();
-  last_dsched_ = &d;
+  last_free_ev_ = d.free_ev;
+  last_busy_ = &d.busy;
   sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
 }
 
@@ -555,10 +561,10 @@ const Schedule &Engine::schedule() {
 void Engine::begin_step(const int *graph, int B, int maxlen) {
   auto t0 = std::chrono::steady_clock::now();
   if (!graph || B <= 0 || maxlen <= 0) fail(CAVS_EINVAL, "graph feed rejected: empty graph feed");
-  if (last_dsched_) {  // everything that reads the previous step's device-built lists is enqueued by now
-    check(cavs_event_record(last_dsched_->free_ev, stream_));
-    last_dsched_->busy = true;
-    last_dsched_ = nullptr;
+  if (last_free_ev_) {  // everything that reads the previous step's lists is enqueued by now
+    check(cavs_event_record(last_free_ev_, stream_));
+    *last_busy_ = true;
+    last_free_ev_ = nullptr;
   }
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   c_round_flops_ = 0;

@@ -136,11 +136,16 @@ class Engine {
   int N_ = 0, cap_ = 0, rcap_ = 0, E_ = 0, mw_ = 0, nch_ = 1;
 
   // per-step device index arena: [t2j | pair | child | roots | kid_rows | orphans]
-  PinnedArray<int> idx_host_[2];
-  void *idx_copied_[2] = {nullptr, nullptr};  // events: upload out of idx_host_[k] finished
-  bool idx_pending_[2] = {false, false};
-  int idx_slot_ = 0;
-  DeviceArray<int> idx_dev_;
+  struct HostLists {  // host-built lists: pinned staging, their device copy, and who still reads it
+    PinnedArray<int> host;
+    DeviceArray<int> dev;
+    void *free_ev = nullptr, *up_ev = nullptr;
+    bool busy = false;
+  } hlists_[2];
+  int hlists_slot_ = 0;
+  // the event to record, and the flag to raise, once the current step's kernels are all enqueued
+  void *last_free_ev_ = nullptr;
+  bool *last_busy_ = nullptr;
   const int *d_t2j_ = nullptr, *d_pair_ = nullptr, *d_child_ = nullptr, *d_roots_ = nullptr;
   // Tree-LSTM, message flow of the batch is a forest: children by slab row, and the slab rows
   // nobody sends a message to
@@ -161,7 +166,6 @@ class Engine {
   DeviceArray<int> dsched_scratch_;
   void *sched_stream_ = nullptr;
   int dsched_slot_ = 0;
-  DeviceSched *last_dsched_ = nullptr;  // the buffers the current step's lists live in, if device-built
   void schedule_on_device(const int *graph, int B, int maxlen);
   void schedule_on_host(const int *graph, int B, int maxlen);
   void point_lists(const int *base, long cap);
