@@ -100,7 +100,7 @@ def cpu_baseline(w, budget_s=12.0):
                                    sample=f"2 steps of the same batch in {el1:.1f} s"))
 
 
-def front_end_modes(w, steps=60, warmup=30):
+def front_end_modes(pool, steps=60, warmup=30):
     """The same training step through the reference's own API (Sym / GraphSupport / Session::Run with
     host feeds, one device synchronisation per Run, loss head and optimizer as ordinary ops), in the
     three ways the session can execute F: lowered onto the fused round kernels, op by op with the
@@ -109,6 +109,7 @@ def front_end_modes(w, steps=60, warmup=30):
 
     from cavs_amd import apps, session
 
+    w = pool[0]
     B, maxlen = w["graph"].shape
     out = {}
     for name, opt, lowered in (("lowered", session.OPT_BATCHING, True),
@@ -118,15 +119,18 @@ def front_end_modes(w, steps=60, warmup=30):
                        allow_fused=lowered)
         app.set_params(w["params"])
         # untimed: at least `warmup` steps and 150 ms of continuous work (steady clocks, as in measure())
+        # the same pool of batch structures as the headline measurement, cycled the same way
         done, t0 = 0, time.perf_counter()
         while done < warmup or time.perf_counter() - t0 < 0.15:
-            app.step(w["graph"], w["x"], w["labels"], fetch=False)
+            q = pool[done % len(pool)]
+            app.step(q["graph"], q["x"], q["labels"], fetch=False)
             done += 1
-        n = steps if not lowered else 4 * steps
+        n = steps if not lowered else 5 * steps
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(n):
-            app.step(w["graph"], w["x"], w["labels"], fetch=False)
+        for i in range(n):
+            q = pool[i % len(pool)]
+            app.step(q["graph"], q["x"], q["labels"], fetch=False)
         torch.cuda.synchronize()
         ms = 1e3 * (time.perf_counter() - t0) / n
         out[name] = {"ms_per_step": round(ms, 4), "value": round(B / ms * 1e3, 1), "unit": "samples/s", "steps": n,
@@ -366,7 +370,7 @@ def main():
     # (before the other configurations: for a while after C5's 30 ms steps the device runs this small
     # workload about 15 % slower)
     if not a.no_front_end and w0["model"] in ("treelstm", "lstm"):
-        out["front_end"] = front_end_modes(w0)
+        out["front_end"] = front_end_modes(make_pool(a.workload, a.pool))
         # the same step as a user of the reference's API gets it: Session::Run with host feeds
         out["session_run"] = dict(out["front_end"]["lowered"], path="Sym / GraphSupport / Session::Run, vertex function "
                                   "lowered onto the fused round kernels, host feeds, optimizer as an op of the main scope")

@@ -625,7 +625,12 @@ void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_de
   ev_bwd_valid_ = false;
 }
 
-void Engine::backward_only(const float *dgraph_out) {
+void Engine::update_bias_jobs(float lr, std::vector<cavs_task> *out, std::vector<const float *> *updated) {
+  for (const BiasJob &j : bias_jobs_) updated->push_back(param(j.param).w);
+  settle_bias_jobs(lr, out);
+}
+
+void Engine::backward_only(const float *dgraph_out, bool settle_biases) {
   if (!dgraph_out || N_ == 0) fail(CAVS_EINVAL, "backward_only needs d graph_out of a forward pass");
   d_dgo_ = dgraph_out;
   check(cavs_event_record(ev_[2], stream_));
@@ -634,7 +639,7 @@ void Engine::backward_only(const float *dgraph_out) {
     case CAVS_MODEL_LSTM: lstm_backward(); break;
     default: treefc_backward();
   }
-  settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
+  if (settle_biases) settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
   check(cavs_event_record(ev_[3], stream_));
   ev_bwd_valid_ = true;
 }

@@ -51,7 +51,15 @@ class Engine {
   // The two halves of step() for a caller that runs the loss head itself: forward F into
   // graph_out [N,H] (vertex order), then backward F from d graph_out.
   void forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out);
-  void backward_only(const float *dgraph_out);
+  // settle_biases = false leaves the bias gradients that exist as rows still to be added up
+  // (row E of dW, chunk sums) pending: the caller then takes them with update_bias_jobs() into the
+  // launch that applies its parameter updates, instead of a launch of their own here.
+  void backward_only(const float *dgraph_out, bool settle_biases = true);
+  // The pending bias jobs as jobs of the caller's update launch: each delivers the gradient and
+  // applies w -= lr * g to the bias parameter.  `updated` receives the weight pointers they cover.
+  void update_bias_jobs(float lr, std::vector<cavs_task> *out, std::vector<const float *> *updated);
+  // A job for the launch that opens the next backward pass (it runs before anything of that pass).
+  void queue_prologue_task(const cavs_task &t) { pending_tasks_.push_back(t); }
   void set_pairing(int pairing) { cfg_.pairing = pairing; }
   void set_param(const std::string &name, const float *host, size_t n);
   void get_param(const std::string &name, float *host, size_t n, bool grad);

@@ -41,9 +41,12 @@ Executor::Executor(int opt, const std::string &name) : opt_(opt), name_(name) {
 Executor::~Executor() {
   cavs_stream_sync(stream_);
   engine_.reset();
-  for (auto &kv : feed_stages_)
-    for (void *e : kv.second.uploaded)
-      if (e) cavs_event_destroy(e);
+  if (copy_stream_) {
+    cavs_stream_sync(copy_stream_);
+    cavs_stream_destroy(copy_stream_);
+  }
+  for (void *e : {feeds_up_ev_, run_done_ev_[0], run_done_ev_[1]})
+    if (e) cavs_event_destroy(e);
   for (auto &kv : fused_handles_)
     if (kv.second) cavs_fused_release(kv.second);
   tensors_.clear();
@@ -704,6 +707,13 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
   compile();
   init_variables();
   // feeds: the graph placeholder stays on the host, everything else goes to the device
+  const int parity = run_parity_;
+  run_parity_ ^= 1;
+  if (run_busy_[parity]) {  // the Run before last read this set of feed buffers
+    check(cavs_event_sync(run_done_ev_[parity]));
+    run_busy_[parity] = false;
+  }
+  bool uploads = false;
   for (auto &f : feeds) {
     const Edge *e = g.main.find(f.first);
     if (!e || !e->src || e->src->def.name() != "Placeholder") fail(CAVS_EINVAL, "'" + f.first + "' is not a Placeholder");
@@ -715,29 +725,35 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     if (e->src->def.device() == CPU) {
       t.base = reinterpret_cast<float *>(const_cast<char *>(f.second->data.data()));
     } else {
-      if (t.own.capacity() < (size_t)t.width) {
-        check(cavs_stream_sync(stream_));
-        t.own.reserve(t.width);
+      if (!copy_stream_) {
+        check(cavs_stream_create(&copy_stream_));
+        check(cavs_event_create(&feeds_up_ev_));
+        check(cavs_event_create(&run_done_ev_[0]));
+        check(cavs_event_create(&run_done_ev_[1]));
       }
-      t.base = t.own.get();
-      // through pinned memory, so that the upload is truly asynchronous and the caller's buffer
-      // is free as soon as Run returns
       FeedStage &st = feed_stages_[f.first];
-      const int k = st.next;
-      st.next ^= 1;
       const size_t bytes = (size_t)t.width * 4;
-      if (st.pending[k]) {
-        check(cavs_event_sync(st.uploaded[k]));
-        st.pending[k] = false;
-      }
-      if (!st.uploaded[k]) check(cavs_event_create(&st.uploaded[k]));
-      st.slot[k].reserve(bytes);
-      std::memcpy(st.slot[k].get(), f.second->data.data(), bytes);
-      check(cavs_memcpy_h2d(t.base, st.slot[k].get(), bytes, stream_));
-      check(cavs_event_record(st.uploaded[k], stream_));
-      st.pending[k] = true;
+      st.slot[parity].reserve(bytes);
+      st.dev[parity].reserve(t.width);
+      t.base = st.dev[parity].get();
+      std::memcpy(st.slot[parity].get(), f.second->data.data(), bytes);
+      check(cavs_memcpy_h2d(t.base, st.slot[parity].get(), bytes, copy_stream_));
+      uploads = true;
     }
   }
+  if (uploads) {
+    // a few microseconds of waiting, while the compute stream is still busy with the previous Run
+    check(cavs_event_record(feeds_up_ev_, copy_stream_));
+    check(cavs_event_sync(feeds_up_ev_));
+  }
+  struct MarkRunDone {  // once everything this Run enqueues is in the stream, whichever way it leaves
+    Executor *e;
+    int parity;
+    bool on;
+    ~MarkRunDone() {
+      if (on && cavs_event_record(e->run_done_ev_[parity], e->stream_) == CAVS_OK) e->run_busy_[parity] = true;
+    }
+  } mark_done{this, parity, uploads};
   bool train = false;
   std::vector<std::string> targets;
   for (auto &o : outputs) {
@@ -777,6 +793,23 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
   // `iters` times per Run (ScopedNode(s_, name, iters), cavs/midend/graph_util.cc:266-283;
   // BasicBlock::Run, cavs/midend/statement.h:66-75).
   const int passes = train ? std::max(1, g.opt.iters) : 1;
+  // Launches that can ride in others when the lowered vertex function's backward pass follows in
+  // this Run: the sum of the head's gradient partials (into the launch that opens that pass) and,
+  // when nothing between that pass and the update reads them (no clipping, every later gradient op
+  // planned away), the engine's pending bias gradients (into the launch that applies the updates).
+  head_defer_ = defer_bias_ = false;
+  if (train && lowered_) {
+    int at = -1;
+    const std::vector<char> &skip = it->second.skip_bwd;
+    for (size_t i = 0; i < it->second.bwd.size(); i++)
+      if (it->second.bwd[i].name() == "GraphOutput_grad") at = (int)i;
+    if (at >= 0 && head.fc >= 0 && head.fc_grad >= 0 && head.fc_grad < at) head_defer_ = true;
+    if (at >= 0 && g.opt.clip <= 0.f) {
+      defer_bias_ = true;
+      for (size_t i = at + 1; i < it->second.bwd.size(); i++)
+        if (!(i < skip.size() && skip[i])) defer_bias_ = false;
+    }
+  }
   for (int pass = 0; pass < passes; pass++) {
   bool head_fused = false;
   for (size_t i = 0; i < it->second.fwd.size(); i++) {
@@ -807,8 +840,11 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     }
     // every variable's update in one launch (they touch disjoint tensors)
     std::vector<cavs_task> updates;
+    std::vector<const float *> by_bias_job;
+    if (engine_ && defer_bias_) engine_->update_bias_jobs(g.opt.lr, &updates, &by_bias_job);
     for (auto &v : g.opt.vars) {
       Tensor &w = tensor(v), &gr = tensor(GetGradientName(v));
+      if (std::find(by_bias_job.begin(), by_bias_job.end(), w.base) != by_bias_job.end()) continue;  // gradient and update by that job
       if (updates.size() + 2 > 12) {
         check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
         updates.clear();

@@ -29,14 +29,13 @@ struct Tensor {
   size_t count() const { return (size_t)(per_vertex ? rows * width : width); }
 };
 
-// Pinned staging of one device placeholder's feed: two slots alternate, each guarded by an
-// event recorded after its upload, so that Run can return while the copy is still in flight and
-// the caller may overwrite its own buffer at once.
+// A device-resident feed goes through two sets of buffers (pinned staging + device copy) that
+// alternate from Run to Run; the copies run on a stream of their own, so that the feeds of Run
+// k + 1 go up while the kernels of Run k are still running, instead of sitting in the compute
+// stream between two steps.  A set is rewritten only after the Run that read it has finished.
 struct FeedStage {
   PinnedArray<char> slot[2];
-  void *uploaded[2] = {nullptr, nullptr};
-  bool pending[2] = {false, false};
-  int next = 0;
+  DeviceArray<float> dev[2];
 };
 
 struct HostTensor {  // C_Tensor of the C API
@@ -92,6 +91,15 @@ class Executor {
   int pairing_ = 0;
   std::map<std::string, std::unique_ptr<Tensor>> tensors_;
   std::map<std::string, FeedStage> feed_stages_;
+  // this Run: the head's gradient partials are summed by the engine's backward prologue; the
+  // engine's pending bias gradients are settled by the launch that applies the updates
+  bool head_defer_ = false, defer_bias_ = false;
+  DeviceArray<float> head_parts_;
+  void *copy_stream_ = nullptr;
+  void *feeds_up_ev_ = nullptr;                 // the current Run's feeds have arrived
+  void *run_done_ev_[2] = {nullptr, nullptr};   // everything a Run enqueued has finished, by Run parity
+  bool run_busy_[2] = {false, false};
+  int run_parity_ = 0;
   bool dirty_ = false;  // device work queued by a Run that returned without waiting for it
   std::map<std::string, std::vector<float>> pending_vars_;  // SetVariable before compile
   bool vars_initialised_ = false;

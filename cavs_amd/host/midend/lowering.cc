@@ -597,6 +597,20 @@ bool Executor::run_fused_head(const MainProgram &mp) {
   float *dW = output_storage(fg.output(0), &cnt);
   float *dB = output_storage(fg.output(1), &cnt);
   float *dX = output_storage(fg.output(2), &cnt);
+  // The weight and bias gradients come out as partial sums.  With the engine's backward pass
+  // following in this Run, adding them up is a job of the launch that opens that pass (one launch
+  // less); the partials then live in a buffer of their own until it has run.
+  if (engine_ && head_defer_) {
+    if (head_parts_.capacity() * 4 < bytes) {
+      check(cavs_stream_sync(stream_));
+      head_parts_.reserve(bytes / 4 + 1);
+    }
+    check(cavs_fc_softmax_xent(x, w, b, lab, lo, logits, dX, nullptr, nullptr, head_parts_.get(), head_parts_.capacity() * 4, Nrow, K,
+                               C, stream_));
+    engine_->queue_prologue_task({CAVS_TASK_SUM_PARTS, 0.f, cavs_fc_softmax_xent_parts(Nrow), (long long)C * K + C, (long long)C * K,
+                                  head_parts_.get(), dW, dB, nullptr});
+    return true;
+  }
   float *ws = workspace(bytes);
   check(cavs_fc_softmax_xent(x, w, b, lab, lo, logits, dX, dW, dB, ws, ws_.capacity() * 4, Nrow, K, C, stream_));
   return true;
@@ -620,7 +634,7 @@ void Executor::lowered_backward(const OpDef &d) {
       engine_->bind_param_grad(b.param, t.base + b.offset);
     }
   }
-  engine_->backward_only(dgo_);
+  engine_->backward_only(dgo_, !defer_bias_);
   // hand the gradients of the external edges to the main-scope backward program
   auto slots = role_slots(lw);
   std::map<std::string, std::string> role_of_edge;
