@@ -109,12 +109,19 @@ inline RoundPlan plan_round(int n) {
 // distance to the next k-group's block -- so a wavefront's B fragment is one load of a
 // contiguous kilobyte instead of four loads of four 64-byte pieces each (the texture-address
 // unit charges per piece).
-template <int TILE, int UG, int NA, bool PACKED = false>
+// QUAD (16x16 tiles): arow[i] is the pointer of lane l into tile row l / 4 at k = 4 * (l % 4), so
+// that the four lanes of a quad read 64 consecutive bytes of one row -- the texture-address unit
+// works through a 16-byte-per-lane load a quad at a time, and a quad that spans four rows costs
+// it four cache lines where this costs one.  The MFMA wants row x = l % 16, k-slot l / 16; the
+// fragment crosses lanes (from lane 4 * x + slot) through the LDS crossbar just before it is used.
+template <int TILE, int UG, int NA, bool PACKED = false, bool QUAD = false>
 __device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float *(&arow)[NA], __amdgpu_buffer_rsrc_t bbuf,
                                       const int (&vb)[4], int sb, int b_row_bytes, int nst, const float4 *bpk = nullptr) {
   using M = Mma<TILE>;
   constexpr int GK = 4 * M::NSLOT;
   static_assert(!PACKED || TILE == 16, "the packed layout is for 16x16 tiles");
+  static_assert(!QUAD || TILE == 16, "the quad-contiguous A loads are for 16x16 tiles");
+  const int lane_ = threadIdx.x & 63, from4 = 4 * (4 * (lane_ & 15) + (lane_ >> 4));
   struct Frag {
     float4 a[UG][NA];
     float b[UG][4];
@@ -140,12 +147,29 @@ __device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float 
     }
   };
   auto multiply = [&](const Frag &f) {
+    if constexpr (QUAD) {
+      float av[UG][NA][4];
 #pragma unroll
-    for (int u = 0; u < UG; u++)
+      for (int u = 0; u < UG; u++)
 #pragma unroll
-      for (int c = 0; c < 4; c++)
+        for (int i = 0; i < NA; i++)
 #pragma unroll
-        for (int i = 0; i < NA; i++) acc[i] = M::mma(elem(f.a[u][i], c), f.b[u][c], acc[i]);
+          for (int c = 0; c < 4; c++)
+            av[u][i][c] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from4, __builtin_bit_cast(int, elem(f.a[u][i], c))));
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+          for (int i = 0; i < NA; i++) acc[i] = M::mma(av[u][i][c], f.b[u][c], acc[i]);
+    } else {
+#pragma unroll
+      for (int u = 0; u < UG; u++)
+#pragma unroll
+        for (int c = 0; c < 4; c++)
+#pragma unroll
+          for (int i = 0; i < NA; i++) acc[i] = M::mma(elem(f.a[u][i], c), f.b[u][c], acc[i]);
+    }
   };
   Frag f0, f1;
   fetch(f0);

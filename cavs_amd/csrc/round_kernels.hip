@@ -84,6 +84,15 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     cl = a.child[2 * row];
     cr = a.child[2 * row + 1];
   }
+  // PACKED: A is read a quad of lanes per row piece (lane l: tile row l / 4, k = 4 * (l % 4); see
+  // exact_products) and crosses to the MFMA's lanes just before use
+  constexpr bool QUAD = PACKED;
+  const int qrow = (blockIdx.y * RT + rt) * TILE + (lane >> 2), from4 = 4 * (4 * x + slot);
+  int qcl = -1, qcr = -1;
+  if (QUAD && qrow < a.n) {
+    qcl = a.child[2 * qrow];
+    qcr = a.child[2 * qrow + 1];
+  }
   constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
   struct Epi {
     bool on;
@@ -169,7 +178,14 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     for (int u = 0; u < UG; u++)
 #pragma unroll
       for (int c = 0; c < 4; c++) {
-        const float hl = has_l ? elem(f.hl[u], c) : 0.f, hr = has_r ? elem(f.hr[u], c) : 0.f, hs = hl + hr;
+        float hl = elem(f.hl[u], c), hr = elem(f.hr[u], c);
+        if constexpr (QUAD) {
+          hl = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from4, __builtin_bit_cast(int, hl)));
+          hr = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(from4, __builtin_bit_cast(int, hr)));
+        }
+        hl = has_l ? hl : 0.f;
+        hr = has_r ? hr : 0.f;
+        const float hs = hl + hr;
         acc[0] = M::mma(hs, f.b[u][0][c], acc[0]);
         acc[1] = M::mma(hs, f.b[u][1][c], acc[1]);
         acc[2] = M::mma(hs, f.b[u][2][c], acc[2]);
@@ -210,9 +226,19 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
 #pragma unroll
     for (int k = 0; k < 4; k++) { ep.xw[k] = xw[k * H]; ep.bias[k] = a.bias[k * H + ep.j]; }
   }
-  pl = a.pool + (cl >= 0 ? cl : 0) * H2;
-  pr = a.pool + (cr >= 0 ? cr : 0) * H2;
-  if (kb < ke) fetch_a(kb, f0);
+  if constexpr (QUAD) {  // a missing child reads row 0 and is masked where the operand is used
+    pl = a.pool + (qcl >= 0 ? qcl : 0) * H2 + 4 * (lane & 3) - 4 * slot;
+    pr = a.pool + (qcr >= 0 ? qcr : 0) * H2 + 4 * (lane & 3) - 4 * slot;
+#pragma unroll
+    for (int u = 0; u < UG; u++) {
+      f0.hl[u] = ld4(pl + kb + GK * u + 4 * slot);
+      f0.hr[u] = ld4(pr + kb + GK * u + 4 * slot);
+    }
+  } else {
+    pl = a.pool + (cl >= 0 ? cl : 0) * H2;
+    pr = a.pool + (cr >= 0 ? cr : 0) * H2;
+    if (kb < ke) fetch_a(kb, f0);
+  }
 #pragma unroll
   for (int q = 0; q < EPT; q++) {
     Epi &ep = epi[q];
@@ -562,8 +588,12 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   const int j0 = blockIdx.x * TILE;
   const int row = (blockIdx.y * RT + rt) * TILE + x;
   const bool rin = row < a.n;
-  const float *px = a.dxW + (rin ? row : 0) * a.ld_dxw;
-  const float *pfl = a.dF + (rin ? 2L * row : 0) * H, *pfr = pfl + (rin ? H : 0);
+  // QUAD: the exact packed loops read A a quad of lanes per row piece (see exact_products)
+  constexpr bool QUAD = EXACT && PACKED;
+  const int arow_ = QUAD ? (blockIdx.y * RT + rt) * TILE + (lane >> 2) : row, aslot = QUAD ? (lane & 3) : slot;
+  const bool ain = arow_ < a.n;
+  const float *px = a.dxW + (ain ? arow_ : 0) * a.ld_dxw;
+  const float *pfl = a.dF + (ain ? 2L * arow_ : 0) * H, *pfr = pfl + (ain ? H : 0);
   const float *UTio = a.UT + j0 + x, *UTf = a.UT + 3L * H * H + j0 + x;
 
   // the epilogue's targets, fetched now: child rows of the elements this thread will write
@@ -655,18 +685,21 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     if constexpr (WAVES == 8) fetch_kids();
     {  // P0: K = 3H
       const int kb = ksu * (3 * H / KS);
-      const float *arow[1] = {px + kb + 4 * slot};
+      const float *arow[1] = {px + kb + 4 * aslot};
+      // one accumulator: a stage of UG k-groups is only 4 * UG MFMAs, too short to cover its own
+      // loads, so this product runs with stages three times as long (as many stages as K = H has)
+      constexpr int UG0 = 3 * UG;
       if constexpr (PACKED)
-        exact_products<TILE, UG, 1, true>(&acc[0], arow, tbuf, vb, 0, gstep, 3 * H / KS / S, lane_pk + (kb / 16) * (gstep / 16));
+        exact_products<TILE, UG0, 1, true, true>(&acc[0], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + (kb / 16) * (gstep / 16));
       else
-        exact_products<TILE, UG, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, 3 * H / KS / S);
+        exact_products<TILE, UG0, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, H / KS / S);
     }
     if constexpr (WAVES != 8) fetch_kids();
     {  // P1, P2: K = H, one B operand for both
       const int kb = ksu * (H / KS);
-      const float *arow[2] = {pfl + kb + 4 * slot, pfr + kb + 4 * slot};
+      const float *arow[2] = {pfl + kb + 4 * aslot, pfr + kb + 4 * aslot};
       if constexpr (PACKED)
-        exact_products<TILE, UG, 2, true>(&acc[1], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + 3 * H * H / 4 + (kb / 16) * (gstep / 16));
+        exact_products<TILE, UG, 2, true, true>(&acc[1], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + 3 * H * H / 4 + (kb / 16) * (gstep / 16));
       else
         exact_products<TILE, UG, 2>(&acc[1], arow, tbuf, vb, (3 * H * H + kb * H) * 4, H * 4, H / KS / S);
     }

@@ -202,6 +202,26 @@ def rounds(iters, st):
         us = _time(lambda: hip.call("cavs_treelstm_round_bwd_children", dxW.data_ptr(), 4 * H, dF.data_ptr(), UT.data_ptr(),
                                     child.data_ptr(), dpool.data_ptr(), n, H, st), iters, st)
         _emit("treelstm_round_bwd_children", f"{tag}: n={n} H={H}", us, flops=flops)
+        # the backward round as the engine launches it when the batch's message flow is a forest: the
+        # children's d h and their gate gradients in one launch, transposed weights tile-major.
+        # Whole-batch slabs of 3n rows: the round is rows [2n, 3n), its children rows [0, 2n)
+        if hip.lib().cavs_round_packed_ok(n, H):
+            R3 = 3 * n
+            UTp = torch.empty(4 * H * H, **f32)
+            tasks = (hip.Task * 2)(hip.Task(hip.TASK_PACK_T, 0.0, H, 3 * H, 0, UTp.data_ptr(), U.data_ptr(), None, None),
+                                   hip.Task(hip.TASK_PACK_T, 0.0, H, H, 0, UTp.data_ptr() + 4 * 3 * H * H,
+                                            U.data_ptr() + 4 * 3 * H * H, None, None))
+            hip.call("cavs_run_tasks", 2, tasks, st)
+            dxW_all, dF_all, dc_all = torch.randn(R3, 4 * H, **f32), torch.randn(2 * R3, H, **f32), torch.randn(R3, H, **f32)
+            gates_all, G_all = torch.rand(R3, 6 * H, **f32), torch.randn(2 * R3, 2 * H, **f32)
+            dgo = torch.randn(R3, H, **f32)
+            rows_all = torch.arange(R3, dtype=torch.int32, device="cuda")
+            kids = torch.randperm(2 * n, generator=torch.Generator(device="cpu").manual_seed(n)).to(torch.int32).cuda()
+            us = _time(lambda: hip.call("cavs_treelstm_round_bwd_children_gates_packed", dxW_all.data_ptr(), 4 * H, dF_all.data_ptr(),
+                                        dc_all.data_ptr(), UTp.data_ptr(), kids.data_ptr(), gates_all.data_ptr(), G_all.data_ptr(),
+                                        dgo.data_ptr(), rows_all.data_ptr(), 2 * n, n, n, H, st), iters, st)
+            _emit("treelstm_round_bwd_children_gates_packed", f"{tag}: n={n} H={H}", us, flops=flops)
+            del UTp, dxW_all, dF_all, dc_all, gates_all, G_all, dgo
         del pool, xW, U, G, hlr, gt, msg, hU, hUf, UT, dpool, dret, dxW, dF
 
 
