@@ -87,11 +87,12 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   // PACKED: A is read a quad of lanes per row piece (lane l: tile row l / 4, k = 4 * (l % 4); see
   // exact_products) and crosses to the MFMA's lanes just before use
   constexpr bool QUAD = PACKED;
-  const int qrow = (blockIdx.y * RT + rt) * TILE + (lane >> 2), from4 = 4 * (4 * x + slot);
+  const int from4 = 4 * (4 * x + slot);
+  // (the child ids of tile row l / 4 are with lane l / 4, whose x is that row: no second fetch)
   int qcl = -1, qcr = -1;
-  if (QUAD && qrow < a.n) {
-    qcl = a.child[2 * qrow];
-    qcr = a.child[2 * qrow + 1];
+  if constexpr (QUAD) {
+    qcl = __builtin_amdgcn_ds_bpermute(4 * (lane >> 2), cl);
+    qcr = __builtin_amdgcn_ds_bpermute(4 * (lane >> 2), cr);
   }
   constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
   struct Epi {
