@@ -405,27 +405,6 @@ __global__ void treelstm_round_leaves_fwd_kernel(RoundLeavesArgs a) {
 }
 
 // ------------------------------------------------------------------ backward, gate part
-// Gate gradients of one hidden unit of one vertex.  mh, mc: gradient of the vertex's message
-// ([h|c] halves); dr: gradient of its pushed return value; c_left, c_right: the children's c
-// (zero for a leaf).
-struct GateGrad {
-  float di, d_o, du, dfl, dfr, dc;
-};
-__device__ inline GateGrad gate_grad(float i, float o, float u, float f_l, float f_r, float tc, float mh, float mc, float dr,
-                                     float c_left, float c_right) {
-  GateGrad g;
-  const float dh = mh + dr;
-  const float d_o = dh * tc;
-  const float dc = mc + (dh * o) * (1.f - tc * tc);
-  g.dfl = (dc * c_left) * (f_l * (1.f - f_l));
-  g.dfr = (dc * c_right) * (f_r * (1.f - f_r));
-  g.di = (dc * u) * (i * (1.f - i));
-  g.d_o = d_o * (o * (1.f - o));
-  g.du = (dc * i) * (1.f - u * u);
-  g.dc = dc;
-  return g;
-}
-
 // Elementwise: reads the message gradient through the scatter list (grad of Scatter is
 // Gather), writes the pre-activation gradients and the c half of the children's message
 // gradients straight into the children's pool rows (grad of Gather is Scatter).
@@ -502,46 +481,11 @@ __global__ void treelstm_round_bwd_gates_kernel(RoundBwdGatesArgs a) {
   }
 }
 
-// The same for the vertices nobody sends a message gradient to (the roots), named by a list of
-// slab rows over whole-batch slabs: d c of a vertex goes to row v of `dc`, from where the launch
-// of the vertex's own round hands it on to the children.
-struct BwdGatesRowsArgs {
-  const int *rows;       // [n] slab rows
-  const float *dret;     // gradient of the pushed return value: row dret_rows[v]
-  const int *dret_rows;  // [*] by slab row
-  const float *gates;    // [*, 6H]
-  const float *G;        // [2*, 2H]
-  float *dxW;            // [*, 4H] (ld_dxw)
-  long ld_dxw;
-  float *dF;             // [2*, H]
-  float *dc;             // [*, H]
-  int n, H, leaf_rows;   // slab rows below leaf_rows are leaves
-};
-
+// The same for the vertices nobody sends a message gradient to (the roots): BwdGatesRowsArgs and
+// treelstm_gates_rows_at (shared with the job form of cavs_run_tasks) are in round_common.h.
 template <int W>
 __global__ void treelstm_bwd_gates_rows_kernel(BwdGatesRowsArgs a) {
-  const int H = a.H, hw = H / W;
-  const long H2 = 2L * H;
-  long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (long)a.n * hw) return;
-  const int j = (int)(idx % hw) * W;
-  const long v = a.rows[idx / hw];
-  const bool internal = v >= a.leaf_rows;
-  const float *g = a.gates + v * 6 * H + j;
-  const float *dr = a.dret + (long)a.dret_rows[v] * H + j;
-  const float *cl = a.G + (2 * v) * H2 + H + j, *cr = cl + H2;
-  float *dx = a.dxW + v * a.ld_dxw + j;
-#pragma unroll
-  for (int k = 0; k < W; k++) {
-    const GateGrad q = gate_grad(g[k], g[H + k], g[2 * H + k], g[3 * H + k], g[4 * H + k], g[5 * H + k], 0.f, 0.f, dr[k],
-                                 internal ? cl[k] : 0.f, internal ? cr[k] : 0.f);
-    dx[k] = q.di; dx[H + k] = q.d_o; dx[2 * H + k] = q.du; dx[3 * H + k] = q.dfl + q.dfr;
-    if (internal) {
-      a.dF[(2 * v) * H + j + k] = q.dfl;
-      a.dF[(2 * v + 1) * H + j + k] = q.dfr;
-      a.dc[v * H + j + k] = q.dc;
-    }
-  }
+  treelstm_gates_rows_at<W>(a, (long)blockIdx.x * blockDim.x + threadIdx.x);
 }
 
 // ------------------------------------------------------------------ backward, children part

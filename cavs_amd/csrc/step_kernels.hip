@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "common.h"
+#include "round_common.h"
 
 namespace cavs {
 
@@ -358,6 +359,14 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
       sum_parts_block(static_cast<const float *>(t.p0), (int)t.n0, (int)t.n1, (int)t.n2, static_cast<float *>(t.p1),
                       static_cast<float *>(t.p2), b, lds.sums);
       break;
+    case CAVS_TASK_TREELSTM_GATES_ROWS: {  // cavs_treelstm_bwd_gates_rows as a job
+      const BwdGatesRowsArgs a{static_cast<const int *>(t.p0), static_cast<const float *>(t.p1), static_cast<const int *>(t.p2),
+                               static_cast<const float *>(t.p3), static_cast<const float *>(t.p4), static_cast<float *>(t.p5),
+                               (long)(t.n2 >> 32), static_cast<float *>(t.p6), static_cast<float *>(t.p7), (int)t.n0, (int)t.n1,
+                               (int)(t.n2 & 0xffffffffll)};
+      treelstm_gates_rows_at<4>(a, (long)b * 256 + tid);
+      break;
+    }
     default: break;
   }
 }
@@ -520,6 +529,15 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
           seen |= 1u << d;
         }
         blocks = (t.n0 * t.n1 + 1023) / 1024;
+        break;
+      }
+      case CAVS_TASK_TREELSTM_GATES_ROWS: {
+        const long long ld = t.n2 >> 32;
+        CAVS_REQUIRE(t.n0 >= 0 && t.n0 < (1 << 24) && t.n1 > 0 && t.n1 < (1 << 20) && t.n1 % 4 == 0 && t.n2 >= 0 && ld >= 4 * t.n1,
+                     "cavs_run_tasks: job %d: bad shape of the gate gradients of listed rows", i);
+        if (t.n0 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p2 && t.p3 && t.p4 && t.p5 && t.p6 && t.p7, "cavs_run_tasks: job %d: null pointer", i);
+        blocks = (t.n0 * (t.n1 / 4) + 255) / 256;
         break;
       }
       case CAVS_TASK_SUM_PARTS:

@@ -26,10 +26,11 @@ _P, _I, _F, _Z = C.c_void_p, C.c_int, C.c_float, C.c_size_t
 class Task(C.Structure):
     """cavs_task: one job of cavs_run_tasks"""
     _fields_ = [("kind", _I), ("f0", _F), ("n0", C.c_longlong), ("n1", C.c_longlong), ("n2", C.c_longlong),
-                ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P)]
+                ("p0", _P), ("p1", _P), ("p2", _P), ("p3", _P), ("p4", _P), ("p5", _P), ("p6", _P), ("p7", _P)]
 
 
 TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T, TASK_SGD_PACK = 0, 1, 2, 3, 4, 5, 6, 7
+TASK_TREELSTM_GATES_ROWS = 8
 
 
 class GemmDesc(C.Structure):

@@ -841,18 +841,23 @@ void Engine::treelstm_backward() {
   bool packed = forest_;
   for (const Round &r : sched_->rounds)
     if (!leaf_round(r) && !cavs_round_packed_ok(r.n, H)) packed = false;
-  if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
-    const int kind = packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE;
-    backward_prologue({{kind, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr},
-                       {kind, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H, nullptr, nullptr}},
-                      true);
-  } else {
-    backward_prologue({}, true);
-  }
   // one launch per round when the message flow is a forest: the roots' gate gradients first, then
   // every round hands d h, d c on to its children and does their gate gradients in its epilogue
   const bool folded = forest_;
-  if (folded) {
+  // (those of the roots depend on nothing the opening launch writes and ride in it)
+  const bool roots_ride = folded && fused > 0 && H % 4 == 0 && n_orphans_ > 0;
+  std::vector<cavs_task> opening;
+  if (fused > 0) {  // U_iou^T and U_f^T: the B operand of the children products, k-major
+    const int kind = packed ? CAVS_TASK_PACK_T : CAVS_TASK_TRANSPOSE;
+    opening.push_back({kind, 0.f, H, 3 * H, 0, UT_.get(), const_cast<float *>(U), nullptr, nullptr});
+    opening.push_back({kind, 0.f, H, H, 0, UT_.at((size_t)3 * H * H), const_cast<float *>(U) + (size_t)3 * H * H, nullptr, nullptr});
+  }
+  if (roots_ride)
+    opening.push_back({CAVS_TASK_TREELSTM_GATES_ROWS, 0.f, n_orphans_, H, (long long)sched_->leaf_prefix | ((long long)(4 * H) << 32),
+                       const_cast<int *>(d_orphans_), const_cast<float *>(d_dgo_), const_cast<int *>(d_t2j_), gates_.get(), G_.get(),
+                       dxW_.get(), dF_.get(), dc_.get()});
+  backward_prologue(opening, true);
+  if (folded && !roots_ride) {
     CAVS_TIMED(K_GATES, cavs_treelstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
                                                      dF_.get(), dc_.get(), sched_->leaf_prefix, H, stream_));
     c_launches_ += 1;

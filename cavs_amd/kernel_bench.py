@@ -96,6 +96,9 @@ def gemm(iters, st):
             (1, 0, H, 3 * H, N // 2, f"{tag} dU_iou = h_lr^T*d(hU)"),
         ]
     cases += [(0, 0, 32, 1536, 512, "C3 tail round (32 rows)"), (0, 0, 8192, 8192, 8192, "square 8192")]
+    # the 10000-way head of the variable-length LSTM configuration (7331 tokens per batch)
+    cases += [(0, 0, 7331, 10000, 512, "C4 head logits = h*Wc"), (1, 0, 512, 10000, 7331, "C4 head dWc = h^T*dlogits"),
+              (0, 1, 7331, 512, 10000, "C4 head dh = dlogits*Wc^T"), (0, 0, 7331, 2048, 512, "C4 x*W all rows")]
     for tA, tB, M, Nn, K, tag in cases:
         A = torch.randn((K, M) if tA else (M, K), **f32)
         B = torch.randn((Nn, K) if tB else (K, Nn), **f32)

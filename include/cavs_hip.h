@@ -448,14 +448,21 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *   CAVS_TASK_SGD_PACK   p1[i] -= f0 * p2[i] (skipped when p2 is null), then p0 = B = p1 ([K = n0, N = n1]
  *                        row-major; n0 a multiple of 16, n1 of 64) in the same tile-major layout: the
  *                        parameter update (cavs/backend/op_impl_sgd.cu) and the packed copy the next
- *                        forward pass reads, in one pass over the weights. */
+ *                        forward pass reads, in one pass over the weights.
+ *   CAVS_TASK_TREELSTM_GATES_ROWS  cavs_treelstm_bwd_gates_rows(rows = p0, n = n0, dret = p1,
+ *                        dret_rows = p2, gates = p3, G = p4, dxW = p5, ld_dxw = n2 >> 32, dF = p6,
+ *                        dc = p7, leaf_rows = n2 & 0xffffffff, H = n1; H a multiple of 4): the gate
+ *                        gradients of the roots ride in the launch that opens the backward pass.
+ * p4 .. p7 are read by that last kind only and may stay null otherwise. */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
-       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6, CAVS_TASK_SGD_PACK = 7 };
+       CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6, CAVS_TASK_SGD_PACK = 7,
+       CAVS_TASK_TREELSTM_GATES_ROWS = 8 };
 typedef struct cavs_task {
   int kind;
   float f0;
   long long n0, n1, n2;
   void *p0, *p1, *p2, *p3;
+  void *p4, *p5, *p6, *p7;
 } cavs_task;
 int cavs_run_tasks(int count, const cavs_task *tasks, void *stream);
 

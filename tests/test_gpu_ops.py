@@ -1201,6 +1201,31 @@ def test_several_small_jobs_in_one_launch(g):
         want_g[d * bw:(d + 1) * bw] = src[k * bw:(k + 1) * bw]
     np.testing.assert_array_equal(g.host(d_gb), want_g)
     np.testing.assert_array_equal(g.host(d_wb), wb - np.float32(0.5) * want_g)
+    # the gate gradients of listed slab rows (the roots) as a job, beside a transpose: what the
+    # entry point of their own gives, bit for bit
+    R, H, leaf_rows = 20, 32, 5
+    rows_l = np.array([19, 2, 7, 11, 0, 5, 16], np.int32)
+    dret_rows = np.argsort(r.bulk_uniform(R)).astype(np.int32)
+    gates, Gm, dgo = r.bulk_uniform(R * 6 * H), r.bulk_normal(2 * R * 2 * H), r.bulk_normal(R * H)
+    d_rows_l, d_dret_rows, d_gates, d_Gm, d_dgo = g.devi(rows_l), g.devi(dret_rows), g.devf(gates), g.devf(Gm), g.devf(dgo)
+    outs = []
+    for as_job in (False, True):
+        dxW, dF, dc = g.devf(np.full(R * 4 * H, 7, np.float32)), g.devf(np.full(2 * R * H, 7, np.float32)), g.devf(np.full(R * H, 7, np.float32))
+        if as_job:
+            jobs = [T(hip.TASK_TRANSPOSE, 0.0, 70, 33, 0, g.P(dAT), g.P(dA), None, None),
+                    T(hip.TASK_TREELSTM_GATES_ROWS, 0.0, len(rows_l), H, leaf_rows | ((4 * H) << 32), g.P(d_rows_l), g.P(d_dgo),
+                      g.P(d_dret_rows), g.P(d_gates), g.P(d_Gm), g.P(dxW), g.P(dF), g.P(dc))]
+            g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+        else:
+            g.call("cavs_treelstm_bwd_gates_rows", g.P(d_rows_l), len(rows_l), g.P(d_dgo), g.P(d_dret_rows), g.P(d_gates), g.P(d_Gm),
+                   g.P(dxW), 4 * H, g.P(dF), g.P(dc), leaf_rows, H, g.stream())
+        outs.append((g.host(dxW), g.host(dF), g.host(dc)))
+    for a_, b_ in zip(*outs):
+        assert (a_ != 7).any()
+        np.testing.assert_array_equal(a_, b_)
+    with pytest.raises(hip.CavsError, match="null pointer"):
+        g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_TREELSTM_GATES_ROWS, 0.0, 3, H, leaf_rows | ((4 * H) << 32), g.P(d_rows_l), g.P(d_dgo),
+                                              g.P(d_dret_rows), g.P(d_gates))), g.stream())
     with pytest.raises(hip.CavsError, match="not a permutation"):
         g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_BLOCKS_SGD, 0.5, bw, 4, 0, g.P(d_wb), g.P(d_src), g.P(d_gb), None)), g.stream())
     with pytest.raises(hip.CavsError, match="unknown kind"):
