@@ -16,6 +16,7 @@
 #include <algorithm>
 
 #include "common.h"
+#include "embed_common.h"
 
 namespace cavs {
 
@@ -303,6 +304,42 @@ __global__ void splitk_reduce_group_kernel(GemmGroup R) {
   g.C[r * g.ldc + c] = v;
 }
 
+// The embedding gradient behind one product of a group (cavs_sgemm_group_embed_bwd): the rows of
+// that product's result are scatter-added into the table by extra workgroups of the launch that
+// reduces the other products' K splits, reading the product's own partials directly.
+struct EmbedTail {
+  float *dtable;
+  const float *ids;
+  const float *dy;   // the result, or the first of `parts` partial results `part_stride` floats apart
+  long ld_dy, part_stride;
+  int parts;
+  float *copy;       // where the summed result goes as well (the product's C) when parts > 1
+  long ld_copy;
+  int n, E, gx;      // gx row chunks of 64
+};
+
+__global__ __launch_bounds__(256) void splitk_reduce_group_embed_kernel(GemmGroup R, EmbedTail e) {
+  const int nred = R.first[R.count];
+  if ((int)blockIdx.x >= nred) {
+    const int vb = blockIdx.x - nred;
+    embed_bwd_block(e.dtable, e.ids, e.dy, e.ld_dy, e.parts, e.part_stride, e.copy, e.ld_copy, e.n, e.E, vb % e.gx, vb / e.gx);
+    return;
+  }
+  int p = 0;
+  while (p + 1 < R.count && (int)blockIdx.x >= R.first[p + 1]) p++;
+  const GemmArgs &g = R.g[p];
+  const int splits = R.splits[p];
+  long idx = (long)(blockIdx.x - R.first[p]) * blockDim.x + threadIdx.x;
+  long total = (long)g.M * g.N;
+  if (idx >= total) return;
+  float acc = 0.f;
+  for (int z = 0; z < splits; z++) acc += g.ws[(long)z * total + idx];
+  int r = (int)(idx / g.N), c = (int)(idx % g.N);
+  float v = g.alpha * acc;
+  if (g.beta != 0.f) v += g.beta * g.C[r * g.ldc + c];
+  g.C[r * g.ldc + c] = v;
+}
+
 // C = alpha * sum_z ws[z] + beta * C (+ D rows), z ascending: a fixed order, so the
 // result does not depend on how the workgroups were scheduled.
 __global__ void splitk_reduce_kernel(GemmArgs g, int splits) {
@@ -582,9 +619,20 @@ static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float 
 // Plans a group: every product on the 64x64 tile, K split so that all workgroups of the group
 // together are about four per CU (what a CU holds at once; inside a training step eight per CU
 // measured no better, though it is in a back-to-back loop), each with at least 256 of K.
-static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_bytes, size_t *need_out, void *stream) {
+// `tail_product` >= 0: that product's result is handed on to the embedding scatter-add (dtable, ids)
+static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_bytes, size_t *need_out, void *stream,
+                     int tail_product = -1, float *dtable = nullptr, const float *ids = nullptr) {
   CAVS_REQUIRE(count >= 0 && count <= kGroupMax, "cavs_sgemm_group: %d products, at most %d", count, kGroupMax);
   CAVS_REQUIRE(count == 0 || d, "cavs_sgemm_group: null descriptors");
+  EmbedTail tail{};
+  if (tail_product >= 0 && !need_out) {
+    CAVS_REQUIRE(tail_product < count, "cavs_sgemm_group_embed_bwd: product %d of %d", tail_product, count);
+    const cavs_gemm_desc &q = d[tail_product];
+    CAVS_REQUIRE(q.alpha == 1.f && q.beta == 0.f, "cavs_sgemm_group_embed_bwd: the product that feeds the table takes alpha = 1, beta = 0");
+    CAVS_REQUIRE((q.M == 0 || q.N == 0) || (dtable && ids), "cavs_sgemm_group_embed_bwd: null pointer");
+    // unsplit (or run alone): the scatter-add reads C
+    tail = EmbedTail{dtable, ids, q.C, q.ldc, 0, 1, nullptr, 0, q.M, q.N, (q.M + kEmbedRows - 1) / kEmbedRows};
+  }
   GemmGroup G{}, R{};
   double work = 0;
   long tiles[kGroupMax];
@@ -658,7 +706,15 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
     G.form[n] = (q.transA ? 2 : 0) + (q.transB ? 1 : 0);
     G.first[n + 1] = G.first[n] + (int)((tiles[p] * splits + 7) / 8 * 8);
     n++;
-    if (splits > 1) {
+    if (splits > 1 && p == tail_product && !need_out) {
+      // the scatter-add sums this product's partials itself (and leaves the sum in C as well)
+      tail.dy = g.ws;
+      tail.ld_dy = q.N;
+      tail.part_stride = (long)q.M * q.N;
+      tail.parts = splits;
+      tail.copy = q.C;
+      tail.ld_copy = q.ldc;
+    } else if (splits > 1) {
       R.g[nr] = g;
       R.splits[nr] = splits;
       R.first[nr + 1] = R.first[nr] + (int)(((long)q.M * q.N + 255) / 256);
@@ -681,12 +737,18 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
                       q.C, q.ldc, nullptr, 0, 0, ws, ws_bytes, stream);
     if (rc) return rc;
   }
-  if (n == 0) return CAVS_OK;
   hipStream_t st = as_stream(stream);
-  if (vec) launch(sgemm_group_kernel<true>, (unsigned)G.first[n], kThreads, 0, st, G);
-  else launch(sgemm_group_kernel<false>, (unsigned)G.first[n], kThreads, 0, st, G);
-  CAVS_LAUNCH_CHECK();
-  if (nr > 0) {
+  if (n > 0) {
+    if (vec) launch(sgemm_group_kernel<true>, (unsigned)G.first[n], kThreads, 0, st, G);
+    else launch(sgemm_group_kernel<false>, (unsigned)G.first[n], kThreads, 0, st, G);
+    CAVS_LAUNCH_CHECK();
+  }
+  const bool with_tail = tail_product >= 0 && tail.n > 0 && tail.E > 0;
+  if (with_tail) {
+    const int gy = (tail.E + kEmbedCols - 1) / kEmbedCols;
+    launch(splitk_reduce_group_embed_kernel, (unsigned)(R.first[nr] + tail.gx * gy), 256, 0, st, R, tail);
+    CAVS_LAUNCH_CHECK();
+  } else if (nr > 0) {
     launch(splitk_reduce_group_kernel, (unsigned)R.first[nr], 256, 0, st, R);
     CAVS_LAUNCH_CHECK();
   }
@@ -756,6 +818,12 @@ size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products) {
 int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace, size_t workspace_bytes,
                      void *stream) {
   return run_group(count, products, workspace, workspace_bytes, nullptr, stream);
+}
+
+int cavs_sgemm_group_embed_bwd(int count, const cavs_gemm_desc *products, int embed_product, float *dtable, const float *ids,
+                               void *workspace, size_t workspace_bytes, void *stream) {
+  CAVS_REQUIRE(embed_product >= 0, "cavs_sgemm_group_embed_bwd: product %d", embed_product);
+  return run_group(count, products, workspace, workspace_bytes, nullptr, stream, embed_product, dtable, ids);
 }
 
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,

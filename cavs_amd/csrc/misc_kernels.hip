@@ -2,6 +2,7 @@
 // scatter-add, row-broadcast bias add, softmax cross-entropy, SGD and the generic
 // elementwise family.  All HBM-bound streaming kernels.
 #include "common.h"
+#include "embed_common.h"
 
 namespace cavs {
 
@@ -98,64 +99,11 @@ __global__ void embed_pull_fwd_kernel(float *__restrict__ out, long ld_out, floa
   }
 }
 
-// Scatter-add of dy rows into the table.  A workgroup takes 64 consecutive rows and 64 columns.
-// Parse trees look up one and the same table row for every internal vertex, and atomic adds to
-// one address serialise, so the workgroup first finds the id that occurs most often among its
-// rows (its "hot" id), adds those rows up (each wavefront its 16 rows in registers, then the
-// four partial sums in wavefront order) and issues one atomic add per column for them; every
-// other row goes to the table with an atomic add of its own.
-constexpr int kEmbedRows = 64, kEmbedCols = 64;
+// Scatter-add of dy rows into the table: embed_bwd_block in embed_common.h, a workgroup per 64
+// consecutive rows and 64 columns.
 __global__ __launch_bounds__(256) void embed_bwd_kernel(float *__restrict__ dtable, const float *__restrict__ ids,
                                                         const float *__restrict__ dy, long ld_dy, int n, int E) {
-  __shared__ long off[kEmbedRows];
-  __shared__ int count[kEmbedRows];
-  __shared__ int hot_row;
-  __shared__ float part[4][kEmbedCols];
-  const int row0 = blockIdx.x * kEmbedRows, tid = threadIdx.x;
-  const int rows = min(kEmbedRows, n - row0);
-  if (tid < kEmbedRows) off[tid] = tid < rows ? (long)(int)(ids[row0 + tid] * (float)E) : -1 - tid;
-  __syncthreads();
-  if (tid < kEmbedRows) {  // occurrences of this row's id, counted at its first occurrence only
-    int c = 0;
-    bool first = tid < rows;
-    for (int r = 0; r < rows; r++) {
-      if (off[r] == off[tid]) {
-        c++;
-        if (r < tid) first = false;
-      }
-    }
-    count[tid] = first ? c : 0;
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int best = 0;
-    for (int r = 1; r < rows; r++)
-      if (count[r] > count[best]) best = r;  // ties: the earliest row
-    hot_row = best;
-  }
-  __syncthreads();
-  const long hot = off[hot_row];
-  const bool combine = count[hot_row] > 1;
-  const int q = tid >> 6, lane = tid & 63, c = blockIdx.y * kEmbedCols + lane;
-  constexpr int U = kEmbedRows / 4;  // rows per wavefront, all in flight
-  const int r0 = q * U;
-  float sum = 0.f;
-  if (c < E) {
-    float v[U];
-#pragma unroll
-    for (int u = 0; u < U; u++) v[u] = r0 + u < rows ? dy[(long)(row0 + r0 + u) * ld_dy + c] : 0.f;
-#pragma unroll
-    for (int u = 0; u < U; u++) {
-      if (r0 + u >= rows) continue;
-      const long o = off[r0 + u];
-      if (combine && o == hot) sum += v[u];  // in row order
-      else unsafeAtomicAdd(dtable + o + c, v[u]);
-    }
-  }
-  if (!combine) return;  // the same for the whole workgroup
-  part[q][lane] = sum;
-  __syncthreads();
-  if (q == 0 && c < E) unsafeAtomicAdd(dtable + hot + c, ((part[0][lane] + part[1][lane]) + part[2][lane]) + part[3][lane]);
+  embed_bwd_block(dtable, ids, dy, ld_dy, 1, 0, nullptr, 0, n, E, blockIdx.x, blockIdx.y);
 }
 
 // ------------------------------------------------------------------ bias add

@@ -925,15 +925,14 @@ void Engine::treelstm_backward() {
   const int lp = sched_->leaf_prefix;  // leaves contribute exact zeros to dU
   float *dU = param("U").g;
   const bool bias_row = bias_row_ok();  // the ones column of e_ turns row E of dW into the column sums of dxW
-  gemm_group({
+  gemm_group_embedding_backward({
       {0, 1, N, E, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, W, 4 * H, de_.get(), E},
       // (all four padding columns of e_ take part, so that the product keeps 16-byte operand loads)
       {1, 0, bias_row ? ld_e_ : E, 4 * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), 4 * H, param("W").g, 4 * H},
       {1, 0, H, 3 * H, N - lp, 1.f, 0.f, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H},
       {1, 0, H, H, 2 * (N - lp), 1.f, 0.f, G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
        dU + (size_t)3 * H * H, H},
-  });
-  embedding_backward(E);
+  }, E);
   // bias blocks [i|f|u|o] from dxW columns [i|o|u|f]
   if (bias_row) {
     // settled by the launch that ends the step (or right after this pass); block k of the row
@@ -1036,17 +1035,27 @@ void Engine::backward_prologue(std::vector<cavs_task> tasks, bool with_embedding
   c_launches_ += 1;
 }
 
-void Engine::embedding_backward(int E) {
+// `products[0]` is de = dxW * W^T; its rows go on into the embedding gradient in the launch that
+// reduces the group's K splits (cavs_sgemm_group_embed_bwd).
+void Engine::gemm_group_embedding_backward(const std::vector<cavs_gemm_desc> &products, int E) {
   Param &emb = param("Emb");
   const bool owned = emb.g == emb.own_g.get();
   if (emb_cleared_) {
     emb_cleared_ = false;  // the prologue of this backward pass did it
   } else if (owned && emb_sparse_valid_) {
     if (emb_dirty_n_ > 0) check(cavs_embed_zero_rows(emb.g, xs_prev_.get(), emb_dirty_n_, E, stream_));
+    c_launches_ += 1;
   } else {
     check(cavs_zero(emb.g, emb.n * 4, stream_));
+    c_launches_ += 1;
   }
-  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), E, N_, E, stream_));
+  const int count = (int)products.size();
+  float *ws = workspace(cavs_sgemm_group_workspace(count, products.data()));
+  {
+    ProfScope ps(this, K_GEMM);
+    check(cavs_sgemm_group_embed_bwd(count, products.data(), 0, emb.g, xs_.get(), ws, ws_.capacity() * 4, stream_));
+  }
+  for (const cavs_gemm_desc &q : products) c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
   c_launches_ += 2;
   xs_.swap(xs_prev_);  // this step's ids: the rows that are dirty now
   emb_dirty_n_ = N_;
@@ -1172,13 +1181,12 @@ void Engine::lstm_backward() {
   }
   const int lp = sched_->leaf_prefix;
   float *dW = param("W").g;
-  gemm_group({
+  gemm_group_embedding_backward({
       {0, 1, N, H, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, Wx, 4 * H, de_.get(), H},
       {1, 0, H, 4 * H, N, 1.f, 0.f, e_.get(), H, dxW_.get(), 4 * H, dW, 4 * H},
       {1, 0, H, 4 * H, N - lp, 1.f, 0.f, G_.at((size_t)lp * 2 * H), 2 * H, dxW_.at((size_t)lp * 4 * H), 4 * H,
        dW + (size_t)4 * H * H, 4 * H},
-  });
-  embedding_backward(H);
+  }, H);
   bias_gradient("Bv", dxW_.get(), N, 4 * H, bias_parts_);
 }
 

@@ -238,7 +238,7 @@ class Engine {
   bool has_bias_job(const std::string &name) const;
   void settle_bias_jobs(float lr, std::vector<cavs_task> *tasks);
   DeviceArray<float> head_parts_;         // weight-gradient partials of the classifier head
-  void embedding_backward(int E);
+  void gemm_group_embedding_backward(const std::vector<cavs_gemm_desc> &products, int E);
   DeviceArray<float> UT_;  // transposed recurrent weights for the fused backward rounds
   // The recurrent weights (Tree-LSTM: U; chain LSTM: W') tile-major for the packed forward rounds.
   // Written by the job that applies their SGD update; current while nobody else has written them

@@ -153,6 +153,16 @@ typedef struct cavs_gemm_desc {
 size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products);
 int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace,
                      size_t workspace_bytes, void *stream);
+/* cavs_sgemm_group followed by cavs_embed_bwd(dtable, ids, C_k, ldc_k, M_k, N_k) on the result of
+ * product k = embed_product (alpha 1, beta 0; its rows are the gradients of looked-up embedding
+ * rows): MatMul's input gradient and EmbeddingLookup_grad
+ * (cavs/backend/op_impl_blas3_cublas.cc:34-70, op_impl_embedding_lookup.cu:92-148) back to back.
+ * The scatter-add runs as extra workgroups of the launch that reduces the other products' K
+ * splits and sums product k's own partials itself, so the step has one launch less; C_k still
+ * receives the product.  Same workspace as cavs_sgemm_group for the same list. */
+int cavs_sgemm_group_embed_bwd(int count, const cavs_gemm_desc *products, int embed_product,
+                               float *dtable, const float *ids, void *workspace,
+                               size_t workspace_bytes, void *stream);
 /* C[r,:] = op(A)*op(B) + D[r >> d_shift, :]: the GEMM and the Accumulate that
  * follows it in the backward of a Mirror'ed operand
  * (cavs/backend/op_decl_slice_join.cc:173-182) in one pass.  Workspace as above. */

@@ -270,6 +270,56 @@ def test_sgemm_group_matches_separate_products(g, oracle, name):
             g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes - 256, g.stream())
 
 
+@pytest.mark.parametrize("name,k", [("treelstm_step", 0), ("ragged", 0), ("single", 0), ("mixed", 1), ("mixed", 0)])
+def test_sgemm_group_with_the_embedding_gradient_behind_one_product(g, name, k):
+    """cavs_sgemm_group_embed_bwd: the products come out bit for bit as from cavs_sgemm_group (the one
+    that feeds the table too, whether its K was split, not split, or it ran alone on the large tile) and
+    the table as from cavs_embed_bwd on that product (atomic adds: to the tolerance, in fp64 terms)."""
+    import torch
+
+    shapes = GROUPS[name]
+    n, E = shapes[k][2], shapes[k][3]
+    V = 97
+    r = rng(len(name) * 7 + k)
+    descs = (hip.GemmDesc * len(shapes))()
+    keep = []
+    for p, (tA, tB, M, N, K) in enumerate(shapes):
+        A = r.bulk_uniform(max(M * K, 1), -1, 1)[:M * K].reshape((K, M) if tA else (M, K))
+        B = r.bulk_uniform(max(N * K, 1), -1, 1)[:N * K].reshape((N, K) if tB else (K, N))
+        Ad, Bd = g.devf(A.reshape(-1) if A.size else np.zeros(1)), g.devf(B.reshape(-1) if B.size else np.zeros(1))
+        keep += [Ad, Bd]
+        descs[p] = hip.GemmDesc(tA, tB, M, N, K, 1.0, 0.0, g.P(Ad), max(A.shape[1], 1), g.P(Bd), max(B.shape[1], 1), None, N + 4)
+    ids = np.floor(r.bulk_uniform(max(n, 1)) * V).astype(np.float32)[:n]
+    ids[:n // 2] = 3.0  # one row looked up by half of the vertices, as in a batch of parse trees
+    d_ids = g.devf(ids if n else np.zeros(1))
+    table0 = r.bulk_normal(V * E).reshape(V, E)
+    nbytes = hip.lib().cavs_sgemm_group_workspace(len(shapes), descs)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    res = []
+    for combined in (False, True):
+        outs = [torch.full((max(M, 1), N + 4), float("nan"), dtype=torch.float32, device="cuda") for (_, _, M, N, _) in shapes]
+        for p, o in enumerate(outs):
+            descs[p].C = g.P(o)
+        table = g.devf(table0)
+        if combined:
+            g.call("cavs_sgemm_group_embed_bwd", len(shapes), descs, k, g.P(table), g.P(d_ids), g.P(ws), nbytes, g.stream())
+        else:
+            g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes, g.stream())
+            g.call("cavs_embed_bwd", g.P(table), g.P(d_ids), g.P(outs[k]), E + 4, n, E, g.stream())
+        res.append(([g.host(o) for o in outs], g.host(table)))
+    for p, (_, _, M, N, _) in enumerate(shapes):
+        if M:
+            np.testing.assert_array_equal(res[0][0][p][:, :N], res[1][0][p][:, :N])
+    if n:
+        want = table0.astype(np.float64)
+        np.add.at(want, ids.astype(np.int64), res[0][0][k][:n, :E].astype(np.float64))
+        close(res[0][1], want, "table, separate calls")
+        close(res[1][1], want, "table, combined call")
+    with pytest.raises(hip.CavsError, match="alpha = 1"):
+        descs[k].beta = 0.5
+        g.call("cavs_sgemm_group_embed_bwd", len(shapes), descs, k, g.P(table), g.P(d_ids), g.P(ws), nbytes, g.stream())
+
+
 @pytest.mark.parametrize("tA,tB,M,N,K", [(0, 0, 30, 1536, 512), (0, 1, 8, 512, 1536), (0, 1, 130, 512, 512),
                                           (0, 0, 1, 64, 4096), (1, 1, 40, 72, 640), (0, 0, 33, 40, 300),
                                           (0, 1, 65, 33, 68), (0, 0, 600, 1536, 512), (0, 1, 1200, 512, 1536),
