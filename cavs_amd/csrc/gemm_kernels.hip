@@ -39,6 +39,15 @@ struct GemmArgs {
   int dshift;
   int kchunk;      // K range per blockIdx.y (multiple of BK); == K when not split
   float *ws;       // split-K workspace (counters + partial tiles) or nullptr
+  // cavs_embed_pull_sgemm (NN form only): row r of A is row int(pull_x[pull_rows[r]] * K) / K of the
+  // table A points at (a negative id: a zero row); the workgroups of a row tile also leave the
+  // rows they read in pull_copy (row stride ld_copy; each takes every tilesN-th k-tile) and those
+  // of the first column tile the ids in pull_ids
+  const int *pull_rows = nullptr;
+  const float *pull_x = nullptr;
+  float *pull_copy = nullptr;
+  long ld_copy = 0;
+  float *pull_ids = nullptr;
 };
 
 // Loader of one BX x BK operand tile.  KC: the operand's k index is the contiguous
@@ -56,10 +65,16 @@ struct TileLoader {
   long base[NV];
   int krel[NV];
   bool xin[NV][4];
+  // gathered rows (prepare_pull): where the float4 goes as well, or nullptr; the workgroup copies
+  // the k-tiles whose number is copy_rem modulo copy_mod (the column tiles of a row tile share the
+  // copying of the panel they all read)
+  float *copy[NV];
+  int copy_mod = 1, copy_rem = 0;
 
   __device__ inline void prepare(long ld, int x0, int X, int tid) {
 #pragma unroll
     for (int i = 0; i < NV; i++) {
+      copy[i] = nullptr;
       if constexpr (KC) {
         const int gx = x0 + tid / KQ + (kThreads / KQ) * i;
         krel[i] = 4 * (tid % KQ);
@@ -73,6 +88,30 @@ struct TileLoader {
 #pragma unroll
         for (int c = 0; c < 4; c++) xin[i][c] = gx + c < X;
       }
+    }
+  }
+
+  // k-contiguous operand whose rows are looked up: row x0 + r of the operand is the table row that
+  // starts at float int(ids(x0 + r) * K) of P (EmbeddingLookup's offset), ids(b) = px[rows[b]]
+  __device__ inline void prepare_pull(const int *__restrict__ rows, const float *__restrict__ px, int K, int x0, int X, int tid,
+                                      float *__restrict__ copy_to, long ld_copy, float *__restrict__ ids_out, int mod, int rem) {
+    static_assert(KC, "looked-up rows are k-contiguous");
+    copy_mod = mod;
+    copy_rem = rem;
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+      const int gx = x0 + tid / KQ + (kThreads / KQ) * i;
+      krel[i] = 4 * (tid % KQ);
+      long off = -1;
+      if (gx < X) {
+        const float id = px[rows[gx]];
+        off = (long)(int)(id * (float)K);
+        if (ids_out && krel[i] == 0) ids_out[gx] = id;
+      }
+      base[i] = (off >= 0 ? off : 0) + krel[i];
+#pragma unroll
+      for (int c = 0; c < 4; c++) xin[i][c] = off >= 0;
+      copy[i] = (copy_to && gx < X) ? copy_to + (long)gx * ld_copy + krel[i] : nullptr;
     }
   }
 
@@ -96,6 +135,18 @@ struct TileLoader {
         if (xin[i][3] && kin[3]) v.w = q[3];
       }
       reg[i] = v;
+      if constexpr (KC) {
+        if (copy[i] && (k0 / BK) % copy_mod == copy_rem) {  // (a row without an id leaves zeros)
+          if constexpr (VEC) {
+            if (kin[0]) *reinterpret_cast<float4 *>(copy[i] + k0) = v;
+          } else {
+            if (kin[0]) copy[i][k0] = v.x;
+            if (kin[1]) copy[i][k0 + 1] = v.y;
+            if (kin[2]) copy[i][k0 + 2] = v.z;
+            if (kin[3]) copy[i][k0 + 3] = v.w;
+          }
+        }
+      }
     }
   }
 
@@ -143,7 +194,13 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
 
   TileLoader<BM, BK, !TA, VEC> la;
   TileLoader<BN, BK, TB, VEC> lb;
-  la.prepare(g.lda, m0, g.M, tid);
+  if constexpr (!TA) {
+    if (g.pull_rows) la.prepare_pull(g.pull_rows, g.pull_x, g.K, m0, g.M, tid, g.pull_copy, g.ld_copy, n0 == 0 ? g.pull_ids : nullptr,
+                                     tilesN, t % tilesN);
+    else la.prepare(g.lda, m0, g.M, tid);
+  } else {
+    la.prepare(g.lda, m0, g.M, tid);
+  }
   lb.prepare(g.ldb, n0, g.N, tid);
 
   floatx16 acc[TM][TN];
@@ -576,14 +633,30 @@ static void launch_skinny(const GemmArgs &g, hipStream_t st) {
   }
 }
 
+// the looked-up rows of cavs_embed_pull_sgemm (GemmArgs::pull_*)
+struct PullRows {
+  const int *rows;
+  const float *x;
+  float *copy;
+  long ld_copy;
+  float *ids;
+};
+
 static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float alpha, const float *A,
                     int lda, const float *B, int ldb, float beta, float *C, int ldc, const float *D,
-                    int ldd, int dshift, void *ws, size_t ws_bytes, void *stream) {
+                    int ldd, int dshift, void *ws, size_t ws_bytes, void *stream, const PullRows *pull = nullptr) {
   int rc = check_gemm(who, tA, tB, M, N, K, A, lda, B, ldb, C, ldc);
   if (rc || M == 0 || N == 0) return rc;
-  GemmPlan p = plan_gemm(tA, tB, M, N, K, skinny_ok(tA, tB, K, A, lda, B, ldb), ws != nullptr);
+  GemmPlan p = plan_gemm(tA, tB, M, N, K, !pull && skinny_ok(tA, tB, K, A, lda, B, ldb), ws != nullptr);
   hipStream_t st = as_stream(stream);
   GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, D, ldd, dshift, p.kchunk, nullptr};
+  if (pull) {
+    g.pull_rows = pull->rows;
+    g.pull_x = pull->x;
+    g.pull_copy = pull->copy;
+    g.ld_copy = pull->ld_copy;
+    g.pull_ids = pull->ids;
+  }
   if (p.kind == GemmPlan::SKINNY) {
     if (tB) launch_skinny<true>(g, st); else launch_skinny<false>(g, st);
     CAVS_LAUNCH_CHECK();
@@ -824,6 +897,24 @@ int cavs_sgemm_group_embed_bwd(int count, const cavs_gemm_desc *products, int em
                                void *workspace, size_t workspace_bytes, void *stream) {
   CAVS_REQUIRE(embed_product >= 0, "cavs_sgemm_group_embed_bwd: product %d", embed_product);
   return run_group(count, products, workspace, workspace_bytes, nullptr, stream, embed_product, dtable, ids);
+}
+
+int cavs_embed_pull_sgemm(float *C, int ldc, float *e_out, int ld_e, float *ids_out, const float *x, const int *rows,
+                          const float *table, int n, int E, const float *B, int ldb, int N, void *stream) {
+  CAVS_REQUIRE(n >= 0 && E > 0 && N >= 0 && ld_e >= E, "cavs_embed_pull_sgemm: bad shape n=%d E=%d N=%d ld_e=%d", n, E, N, ld_e);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(e_out && ids_out && x && rows && table, "cavs_embed_pull_sgemm: null pointer");
+  // the copy goes out in whole float4s on the vector path
+  CAVS_REQUIRE(E % 4 != 0 || (aligned16(e_out) && ld_e % 4 == 0), "cavs_embed_pull_sgemm: e_out must be 16-byte aligned with ld_e a multiple of 4");
+  // A product large enough for the 128 x 128 tiles gains nothing from the saved launch and its
+  // workgroups are slowed by the lookups (7331 x 2048 x 512: 157 -> 180 us): the two calls then.
+  if (N == 0 || plan_gemm(0, 0, n, N, E, false, false).kind == GemmPlan::TILE128) {
+    int rc = cavs_embed_pull_fwd(e_out, ld_e, ids_out, x, rows, table, n, E, stream);
+    if (rc || N == 0) return rc;
+    return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, e_out, ld_e, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream);
+  }
+  const PullRows pull{rows, x, e_out, ld_e, ids_out};
+  return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, table, E, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream, &pull);
 }
 
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,

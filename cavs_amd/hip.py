@@ -75,6 +75,7 @@ _SIGS = {
     "cavs_colsum": [_P, _P, _I, _I, _I, _I, _P],
     "cavs_embed_fwd": [_P, _I, _P, _P, _I, _I, _P],
     "cavs_embed_pull_fwd": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_embed_pull_sgemm": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _P],
     "cavs_embed_bwd": [_P, _P, _P, _I, _I, _I, _P],
     "cavs_bias_add_rows": [_P, _P, _P, _I, _I, _P],
     "cavs_softmax_xent": [_P, _P, _P, _P, _I, _I, _P],

@@ -770,9 +770,13 @@ void Engine::treelstm_forward() {
     c_launches_ += 1;
     upk_valid_ = U == param("U").own_w.get();
   }
-  check(cavs_embed_pull_fwd(e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, stream_));
+  // Pull of the word id, the lookup and x * W: one launch
+  {
+    ProfScope ps(this, K_GEMM);
+    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, W, 4 * H, 4 * H, stream_));
+  }
+  c_gemm_flops_ += 2.0 * N * 4 * H * E;
   c_launches_ += 1;
-  gemm(0, 0, N, 4 * H, E, e_.get(), ld_e_, W, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_->batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
@@ -1067,9 +1071,12 @@ void Engine::gemm_group_embedding_backward(const std::vector<cavs_gemm_desc> &pr
 void Engine::lstm_forward() {
   const int N = N_, H = cfg_.H;
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w;
-  check(cavs_embed_pull_fwd(e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, stream_));
+  {  // Pull of the token id, the lookup and x * W_x: one launch
+    ProfScope ps(this, K_GEMM);
+    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, Wx, 4 * H, 4 * H, stream_));
+  }
+  c_gemm_flops_ += 2.0 * N * 4 * H * H;
   c_launches_ += 1;
-  gemm(0, 0, N, 4 * H, H, e_.get(), H, Wx, 4 * H, 0.f, xW_.get(), 4 * H);
   if (!sched_->batching) check(cavs_zero(G_.get(), (size_t)N * 2 * H * 4, stream_));
   const int fused = fused_rows();
   bool any_packed = false;

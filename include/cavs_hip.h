@@ -184,6 +184,15 @@ int cavs_embed_bwd(float *dtable, const float *ids, const float *dy, int ld_dy, 
  * out[b, 0:E] = table[int(ids_out[b] * E) ...]. */
 int cavs_embed_pull_fwd(float *out, int ld_out, float *ids_out, const float *x, const int *rows,
                         const float *table, int n, int E, void *stream);
+/* cavs_embed_pull_fwd followed by MatMul against B [E, N] (apps/paper/tree-lstm-cavs.cc:139-143:
+ * Pull, EmbeddingLookup, MatMul with W) in one launch: C[b, 0:N] = table row of x[rows[b]] times B.
+ * The product's A loader reads the table rows through the two lists; the workgroups also leave
+ * them in e_out (what the backward pass multiplies by; the column tiles of a row tile share that
+ * copying) and the ids in ids_out, exactly as cavs_embed_pull_fwd would.  Results are those of the
+ * two calls, bit for bit. */
+int cavs_embed_pull_sgemm(float *C, int ldc, float *e_out, int ld_e, float *ids_out, const float *x,
+                          const int *rows, const float *table, int n, int E, const float *B, int ldb,
+                          int N, void *stream);
 /* out[r, :] = inp[r, :] + bias[:]  (BinaryBroadcastingKernel,
  * cavs/backend/op_impl_elementwise.cuh:128-139; also the ones-vector bias GEMM of
  * cavs/backend/op_impl_fullyconnected_cublas.cc:74-76) */

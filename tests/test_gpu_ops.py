@@ -270,6 +270,41 @@ def test_sgemm_group_matches_separate_products(g, oracle, name):
             g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes - 256, g.stream())
 
 
+@pytest.mark.parametrize("n,E,N,ld_e", [(2482, 300, 2048, 304), (7331, 512, 2048, 512), (320, 128, 512, 128), (70, 33, 50, 40), (5, 8, 64, 8)])
+def test_pull_lookup_and_product_in_one_launch(g, n, E, N, ld_e):
+    """cavs_embed_pull_sgemm against cavs_embed_pull_fwd + cavs_sgemm: the product, the looked-up rows
+    it leaves behind (padding columns untouched) and the ids, bit for bit; an id below zero reads as a
+    zero row."""
+    V, nx = 211, n + 9
+    r = rng(n + E)
+    x = np.floor(r.bulk_uniform(nx) * V).astype(np.float32)
+    x[::7] = -1.0
+    rows = np.argsort(r.bulk_uniform(nx)).astype(np.int32)[:n]
+    table, B = r.bulk_normal(V * E).reshape(V, E), r.bulk_uniform(E * N, -0.1, 0.1).reshape(E, N)
+    d_x, d_rows, d_table, d_B = g.devf(x), g.devi(rows), g.devf(table), g.devf(B)
+    res = []
+    for fused in (False, True):
+        e_out, ids_out, Cd = g.devf(np.full((n, ld_e), 9, np.float32)), g.devf(np.full(n, 9, np.float32)), g.devf(np.full((n, N + 4), 9, np.float32))
+        if fused:
+            g.call("cavs_embed_pull_sgemm", g.P(Cd), N + 4, g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E,
+                   g.P(d_B), N, N, g.stream())
+        else:
+            g.call("cavs_embed_pull_fwd", g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E, g.stream())
+            g.call("cavs_sgemm", 0, 0, n, N, E, 1.0, g.P(e_out), ld_e, g.P(d_B), N, 0.0, g.P(Cd), N + 4, g.stream())
+        res.append((g.host(Cd), g.host(e_out), g.host(ids_out)))
+    ids = x[rows]
+    want_e = np.where(ids[:, None] >= 0, table[np.maximum(ids, 0).astype(np.int64)], 0).astype(np.float32)
+    np.testing.assert_array_equal(res[1][1][:, :E], want_e)
+    np.testing.assert_array_equal(res[1][1][:, E:], 9)
+    np.testing.assert_array_equal(res[1][2], ids)
+    np.testing.assert_array_equal(res[1][0][:, N:], 9)
+    close(res[1][0][:, :N], want_e.astype(np.float64) @ B.astype(np.float64), "product vs fp64")
+    if E >= 64 and n > 1024:  # same tile kernel on both sides (smaller shapes take the skinny kernel when called alone)
+        np.testing.assert_array_equal(res[1][0], res[0][0])
+    else:
+        close(res[1][0][:, :N], res[0][0][:, :N], "fused vs separate")
+
+
 @pytest.mark.parametrize("name,k", [("treelstm_step", 0), ("ragged", 0), ("single", 0), ("mixed", 1), ("mixed", 0)])
 def test_sgemm_group_with_the_embedding_gradient_behind_one_product(g, name, k):
     """cavs_sgemm_group_embed_bwd: the products come out bit for bit as from cavs_sgemm_group (the one
