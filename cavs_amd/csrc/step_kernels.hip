@@ -139,6 +139,17 @@ __device__ inline void sum_parts_block(const float *__restrict__ part, int npart
   float a0 = 0.f, a1 = 0.f;
   if (i < total) {
     int p = q;
+    // (eight loads in flight; the same additions in the same order as the loops below)
+    for (; p + 28 < nparts; p += 32) {
+      float v[8];
+#pragma unroll
+      for (int k = 0; k < 8; k++) v[k] = part[(long)(p + 4 * k) * total + i];
+#pragma unroll
+      for (int k = 0; k < 8; k += 2) {
+        a0 += v[k];
+        a1 += v[k + 1];
+      }
+    }
     for (; p + 4 < nparts; p += 8) {
       a0 += part[(long)p * total + i];
       a1 += part[(long)(p + 4) * total + i];
@@ -161,7 +172,7 @@ __global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__rest
 
 static int head_blocks(int n) {
   int want = (n + 7) / 8;  // two rows per wavefront
-  int cap = num_cus() / 2;
+  int cap = num_cus();
   return want < cap ? (want < 1 ? 1 : want) : cap;
 }
 
