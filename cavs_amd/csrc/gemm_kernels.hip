@@ -361,6 +361,27 @@ __global__ void splitk_reduce_group_kernel(GemmGroup R) {
   g.C[r * g.ldc + c] = v;
 }
 
+// What the matrix pipes sustain with nothing else in the way (cavs_mfma_probe): every wavefront
+// issues `iters` rounds of eight independent 32x32x2 MFMAs on operands it keeps in registers.
+__global__ __launch_bounds__(256) void mfma_probe_kernel(float *__restrict__ out, int iters) {
+  floatx16 acc[8];
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[i][r] = 0.f;
+  const float a = 1.f + (threadIdx.x & 7) * 0.125f, b = 0.5f - (threadIdx.x & 3) * 0.0625f;
+  for (int it = 0; it < iters; it++) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, acc[i], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) s += acc[i][r];
+  out[(long)blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // The embedding gradient behind one product of a group (cavs_sgemm_group_embed_bwd): the rows of
 // that product's result are scatter-added into the table by extra workgroups of the launch that
 // reduces the other products' K splits, reading the product's own partials directly.
@@ -858,6 +879,15 @@ int static_scratch_setup(float **out) {
 using namespace cavs;
 
 extern "C" {
+
+int cavs_mfma_probe(float *out, size_t out_floats, int iters, double *flops, void *stream) {
+  const int blocks = 4 * num_cus();
+  CAVS_REQUIRE(out && iters > 0 && out_floats >= (size_t)blocks * 256, "cavs_mfma_probe: output of %d floats needed", blocks * 256);
+  launch(mfma_probe_kernel, blocks, 256, 0, as_stream(stream), out, iters);
+  CAVS_LAUNCH_CHECK();
+  if (flops) *flops = (double)blocks * 4 * iters * 8 * 2.0 * 32 * 32 * 2;
+  return CAVS_OK;
+}
 
 size_t cavs_sgemm_splitk_static_max_bytes(void) { return kStaticScratchBytes; }
 

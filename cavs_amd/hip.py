@@ -69,6 +69,7 @@ _SIGS = {
     "cavs_sgemm": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "cavs_sgemm_addrows": [_I, _I, _I, _I, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _Z, _P],
     "cavs_sgemm_group": [_I, C.POINTER(GemmDesc), _P, _Z, _P],
+    "cavs_mfma_probe": [_P, _Z, _I, C.POINTER(C.c_double), _P],
     "cavs_sgemm_group_embed_bwd": [_I, C.POINTER(GemmDesc), _I, _P, _P, _P, _Z, _P],
     "cavs_sgemm_splitk": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _Z, _P],
     "cavs_sgemm_splitk_static": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],

@@ -115,6 +115,12 @@ def gemm(iters, st):
     # the 10000-way head of the variable-length LSTM configuration (7331 tokens per batch)
     cases += [(0, 0, 7331, 10000, 512, "C4 head logits = h*Wc"), (1, 0, 512, 10000, 7331, "C4 head dWc = h^T*dlogits"),
               (0, 1, 7331, 512, 10000, "C4 head dh = dlogits*Wc^T"), (0, 0, 7331, 2048, 512, "C4 x*W all rows")]
+    # what the matrix pipes sustain with register operands only, in launches of ~1 ms and ~10 ms
+    buf = torch.empty(1 << 20, **f32)
+    for mf_iters in (4000, 40000):
+        fl = C.c_double()
+        us = _time(lambda: hip.call("cavs_mfma_probe", buf.data_ptr(), buf.numel(), mf_iters, C.byref(fl), st), max(iters // 10, 3), st)
+        _emit("mfma_probe", f"register operands only, {mf_iters} x 8 MFMA 32x32x2 per wavefront, 4 workgroups per CU", us, flops=fl.value)
     for tA, tB, M, Nn, K, tag in cases:
         A = torch.randn((K, M) if tA else (M, K), **f32)
         B = torch.randn((Nn, K) if tB else (K, Nn), **f32)

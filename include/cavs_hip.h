@@ -129,6 +129,12 @@ int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, 
  * (cavs_sgemm_splitk_workspace(M, N, K) above the maximum) is refused with CAVS_EINVAL.  All
  * calls on a GPU share that GPU's buffer: calls that overlap in time on one GPU (two streams,
  * two threads) race; calls on one stream are ordered by it. */
+/* Measurement aid (no counterpart in the reference): one launch in which every wavefront of
+ * four workgroups per CU issues iters * 8 independent v_mfma_f32_32x32x2_f32 on register operands
+ * and nothing else -- what the matrix pipes sustain at the clocks the device holds under that
+ * load, to set beside the nominal peak.  `out` takes 4 * CUs * 256 floats (1024 * 256 on MI355X);
+ * *flops receives the launch's FLOP count. */
+int cavs_mfma_probe(float *out, size_t out_floats, int iters, double *flops, void *stream);
 size_t cavs_sgemm_splitk_static_max_bytes(void);
 int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                              int lda, const float *B, int ldb, float beta, float *C, int ldc,
