@@ -22,7 +22,12 @@ HBM_GBS = 8000.0
 MFMA_TF = 157.3
 
 
+_last_timing = "back to back"
+
+
 def _time(fn, iters, stream):
+    global _last_timing
+    _last_timing = "back to back"
     e0, e1 = C.c_void_p(), C.c_void_p()
     hip.call("cavs_event_create", C.byref(e0))
     hip.call("cavs_event_create", C.byref(e1))
@@ -50,13 +55,14 @@ def _time(fn, iters, stream):
             hip.call("cavs_event_elapsed_ms", C.byref(ms), e0, e1)
             total += ms.value
         us = total * 1e3 / iters
+        _last_timing = "kernel-stamped"
     hip.call("cavs_event_destroy", e0)
     hip.call("cavs_event_destroy", e1)
     return us
 
 
 def _emit(kernel, shape, us, nbytes=None, flops=None):
-    rec = dict(kernel=kernel, shape=shape, us_per_launch=round(us, 3))
+    rec = dict(kernel=kernel, shape=shape, us_per_launch=round(us, 3), timing=_last_timing)
     if nbytes is not None:
         gbs = nbytes / us / 1e3
         rec.update(bound="hbm", bytes_per_launch=int(nbytes), achieved_GBs=round(gbs, 1),
