@@ -3,6 +3,8 @@
 #ifndef CAVS_CSRC_ROUND_COMMON_H_
 #define CAVS_CSRC_ROUND_COMMON_H_
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace cavs {
@@ -31,6 +33,18 @@ struct Mma<16> {
   typedef floatx4 Acc;
   static __device__ inline Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
   static __device__ inline int row(int r, int lane) { return 4 * (lane >> 4) + r; }
+};
+
+// 4x4x1, sixteen blocks per instruction: lane l supplies A[row l%4] and B[col l%4] of block l/4;
+// accumulator element r of lane l is row r, column l%4 of block l/4.  The round kernels use it for
+// tiles of four rows by sixteen columns: block l/4 = (column group (l/4)%4, k slot l/16), so the
+// operand fragments are those of the 16x16x4 shape with the A row taken modulo four, and the four
+// k slots of an element (lanes x, x+16, x+32, x+48) are added up after the loop.
+struct Mma4 {
+  static constexpr int NR = 4, NSLOT = 4;
+  typedef floatx4 Acc;
+  static __device__ inline Acc mma(float a, float b, Acc c) { return __builtin_amdgcn_mfma_f32_4x4x1f32(a, b, c, 0, 0, 0); }
+  static __device__ inline int row(int r, int lane) { return r; }
 };
 
 __device__ inline float4 ld4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
@@ -151,6 +165,12 @@ struct RoundPlan {
 // CU several 32x32 tiles (600 rows: 32 us against 40).  Eight wavefronts per workgroup up to
 // 64 rows (shortest latency chain); four beyond, compiled for four workgroups per CU so that
 // their latency chains overlap; 32x32 tiles above a thousand rows, where operand reuse counts.
+// Packed Tree-LSTM launches of at most this many rows use tiles of four rows (Mma4): measured in
+// the C3 step, 0.4206 ms with sixteen-row tiles throughout, 0.4160 with four-row tiles up to 16
+// rows, 0.4137 up to 32; a forward launch of 64 rows takes 11.4 us that way against 8.4 (every
+// row tile streams the whole weight panel).
+constexpr int kRows4Max = 32;
+
 inline RoundPlan plan_round(int n) {
   if (n <= 64) return {16, 8};
   if (n <= 1024) return {16, 4};
@@ -178,14 +198,17 @@ inline RoundPlan plan_round(int n) {
 // works through a 16-byte-per-lane load a quad at a time, and a quad that spans four rows costs
 // it four cache lines where this costs one.  The MFMA wants row x = l % 16, k-slot l / 16; the
 // fragment crosses lanes (from lane 4 * x + slot) through the LDS crossbar just before it is used.
-template <int TILE, int UG, int NA, bool PACKED = false, bool QUAD = false>
+// ROWS4 (with QUAD): tiles of four rows on the 4x4x1 shape (Mma4); arow[i] then belongs to tile row
+// (l / 4) % 4.
+template <int TILE, int UG, int NA, bool PACKED = false, bool QUAD = false, bool ROWS4 = false>
 __device__ inline void exact_products(typename Mma<TILE>::Acc *acc, const float *(&arow)[NA], __amdgpu_buffer_rsrc_t bbuf,
                                       const int (&vb)[4], int sb, int b_row_bytes, int nst, const float4 *bpk = nullptr) {
-  using M = Mma<TILE>;
+  using M = std::conditional_t<ROWS4, Mma4, Mma<TILE>>;
+  static_assert(!ROWS4 || (QUAD && TILE == 16), "the four-row tiles go with the quad-contiguous loads of the 16-column tile");
   constexpr int GK = 4 * M::NSLOT;
   static_assert(!PACKED || TILE == 16, "the packed layout is for 16x16 tiles");
   static_assert(!QUAD || TILE == 16, "the quad-contiguous A loads are for 16x16 tiles");
-  const int lane_ = threadIdx.x & 63, from4 = 4 * (4 * (lane_ & 15) + (lane_ >> 4));
+  const int lane_ = threadIdx.x & 63, from4 = 4 * (4 * (lane_ & (ROWS4 ? 3 : 15)) + (lane_ >> 4));
   struct Frag {
     float4 a[UG][NA];
     float b[UG][4];

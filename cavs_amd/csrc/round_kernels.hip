@@ -18,6 +18,8 @@
 //     children, h_l+h_r).
 // TILE is 32 (v_mfma_f32_32x32x2_f32) or, for rounds of a few rows near the roots, 16
 // (v_mfma_f32_16x16x4_f32), which spreads a tiny round over four times as many CUs.
+#include <type_traits>
+
 #include "round_common.h"
 
 namespace cavs {
@@ -52,10 +54,15 @@ struct RoundFwdArgs {
 // PACKED: the loop reads the weights from the tile-major copy, one float4 per lane, gate and
 // k-group -- a wavefront's fragment is one contiguous kilobyte instead of four 64-byte pieces per
 // dword load (the texture-address unit charges per piece).
-template <int TILE, int WAVES, bool EXACT, bool PACKED = false>
+// ROWS4 (with PACKED): tiles of four rows by sixteen columns on the 4x4x1 MFMA shape -- a round of
+// a few rows spends a quarter of the matrix-pipe time per tile and spreads over four times as
+// many CUs.
+template <int TILE, int WAVES, bool EXACT, bool PACKED = false, bool ROWS4 = false>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_fwd_kernel(RoundFwdArgs a) {
   static_assert(!PACKED || (EXACT && TILE == 16), "the packed layout is for the exact loops over 16x16 tiles");
-  using M = Mma<TILE>;
+  static_assert(!ROWS4 || PACKED, "the four-row tiles read packed weights");
+  using M = std::conditional_t<ROWS4, Mma4, Mma<TILE>>;
+  constexpr int TR = ROWS4 ? 4 : TILE;  // rows of a tile
   using Acc = typename M::Acc;
   constexpr int RT = 1, kRoundThreads = WAVES * 64;
   constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 5, NR = M::NR;
@@ -68,10 +75,11 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int rt = wave / KS, ks = wave % KS;
   const int x = lane & (TILE - 1), slot = lane / TILE;
+  const int xr = x & (TR - 1);  // tile row of this lane's A operand
   const int H = a.H;
   const long H2 = 2L * H, H3 = 3L * H;
   const int j0 = blockIdx.x * TILE;
-  const int row = (blockIdx.y * RT + rt) * TILE + x;
+  const int row = (blockIdx.y * RT + rt) * TR + xr;
   const int kper = ((H + KS - 1) / KS + GK - 1) / GK * GK;
   const int kb = ks * kper, ke = min(H, kb + kper);
   const float *Uio = a.U + j0 + x, *Uf = a.U + H3 * H + j0 + x;
@@ -87,12 +95,12 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   // PACKED: A is read a quad of lanes per row piece (lane l: tile row l / 4, k = 4 * (l % 4); see
   // exact_products) and crosses to the MFMA's lanes just before use
   constexpr bool QUAD = PACKED;
-  const int from4 = 4 * (4 * x + slot);
+  const int from4 = 4 * (4 * xr + slot);
   // (the child ids of tile row l / 4 are with lane l / 4, whose x is that row: no second fetch)
   int qcl = -1, qcr = -1;
   if constexpr (QUAD) {
-    qcl = __builtin_amdgcn_ds_bpermute(4 * (lane >> 2), cl);
-    qcr = __builtin_amdgcn_ds_bpermute(4 * (lane >> 2), cr);
+    qcl = __builtin_amdgcn_ds_bpermute(4 * ((lane >> 2) & (TR - 1)), cl);
+    qcr = __builtin_amdgcn_ds_bpermute(4 * ((lane >> 2) & (TR - 1)), cr);
   }
   constexpr int EPT = (RT * NR * 64 + kRoundThreads - 1) / kRoundThreads;
   struct Epi {
@@ -109,6 +117,12 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     ep.j = j0 + (l2 & (TILE - 1));
     ep.lds = (t * NP * NR + r) * 64 + l2;
     ep.on = e < RT * NR * 64 && ep.b < a.n;
+    if constexpr (ROWS4) {  // sixty-four elements: row e / 16, column e % 16, four k slots each
+      ep.b = blockIdx.y * TR + (e >> 4);
+      ep.j = j0 + (e & 15);
+      ep.lds = (e >> 4) * 64 + (e & 15);
+      ep.on = e < TR * 16 && ep.b < a.n;
+    }
     ep.c_l = ep.c_r = ep.dst = ep.out = -1;
     if (ep.on) {
       ep.c_l = a.child[2 * ep.b];
@@ -320,9 +334,18 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     float v[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
-      float s = pre[p * NR * 64];
+      float s;
+      if constexpr (ROWS4) {
+        s = 0.f;
 #pragma unroll
-      for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+        for (int g = 0; g < NREG; g++)
+          s += (pre[g * RSZ + p * NR * 64] + pre[g * RSZ + p * NR * 64 + 16]) +
+               (pre[g * RSZ + p * NR * 64 + 32] + pre[g * RSZ + p * NR * 64 + 48]);
+      } else {
+        s = pre[p * NR * 64];
+#pragma unroll
+        for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+      }
       v[p] = s;
     }
     const int b = ep.b, j = ep.j;
@@ -515,9 +538,12 @@ struct RoundBwdChildArgs {
 };
 
 // PACKED (with EXACT, 16x16 tiles): UT is in the tile-major layout of CAVS_TASK_PACK_T.
-template <int TILE, int WAVES, bool FOLD, bool EXACT, bool PACKED = false>
+// ROWS4 (with FOLD, EXACT, PACKED): tiles of four rows on the 4x4x1 shape, as in the forward kernel.
+template <int TILE, int WAVES, bool FOLD, bool EXACT, bool PACKED = false, bool ROWS4 = false>
 __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) void treelstm_round_bwd_children_kernel(RoundBwdChildArgs a) {
-  using M = Mma<TILE>;
+  static_assert(!ROWS4 || (FOLD && EXACT && PACKED), "the four-row tiles are for the folded packed launches");
+  using M = std::conditional_t<ROWS4, Mma4, Mma<TILE>>;
+  constexpr int TR = ROWS4 ? 4 : TILE;  // rows of a tile
   using Acc = typename M::Acc;
   constexpr int RT = 1, kRoundThreads = WAVES * 64;
   constexpr int KS = WAVES / RT, GK = 4 * M::NSLOT, NP = 3, NR = M::NR;
@@ -531,11 +557,11 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   const int H = a.H;
   const long H2 = 2L * H;
   const int j0 = blockIdx.x * TILE;
-  const int row = (blockIdx.y * RT + rt) * TILE + x;
+  const int row = (blockIdx.y * RT + rt) * TR + (x & (TR - 1));
   const bool rin = row < a.n;
   // QUAD: the exact packed loops read A a quad of lanes per row piece (see exact_products)
   constexpr bool QUAD = EXACT && PACKED;
-  const int arow_ = QUAD ? (blockIdx.y * RT + rt) * TILE + (lane >> 2) : row, aslot = QUAD ? (lane & 3) : slot;
+  const int arow_ = QUAD ? (blockIdx.y * RT + rt) * TR + ((lane >> 2) & (TR - 1)) : row, aslot = QUAD ? (lane & 3) : slot;
   const bool ain = arow_ < a.n;
   const float *px = a.dxW + (ain ? arow_ : 0) * a.ld_dxw;
   const float *pfl = a.dF + (ain ? 2L * arow_ : 0) * H, *pfr = pfl + (ain ? H : 0);
@@ -549,10 +575,16 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
   for (int q = 0; q < EPT; q++) {
     const int e = tid + q * kRoundThreads;
     const int l2 = e & 63, r = (e >> 6) % NR, t = e / (64 * NR);
-    const int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2);
+    int b = (blockIdx.y * RT + t) * TILE + M::row(r, l2);
     ej[q] = j0 + (l2 & (TILE - 1));
     elds[q] = (t * NP * NR + r) * 64 + l2;
     eon[q] = e < RT * NR * 64 && b < a.n;
+    if constexpr (ROWS4) {  // sixty-four elements: row e / 16, column e % 16, four k slots each
+      b = blockIdx.y * TR + (e >> 4);
+      ej[q] = j0 + (e & 15);
+      elds[q] = (e >> 4) * 64 + (e & 15);
+      eon[q] = e < TR * 16 && b < a.n;
+    }
     ecl[q] = ecr[q] = -1;
     if (eon[q]) {
       ecl[q] = a.child[2 * b];
@@ -635,7 +667,7 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       // loads, so this product runs with stages three times as long (as many stages as K = H has)
       constexpr int UG0 = 3 * UG;
       if constexpr (PACKED)
-        exact_products<TILE, UG0, 1, true, true>(&acc[0], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + (kb / 16) * (gstep / 16));
+        exact_products<TILE, UG0, 1, true, true, ROWS4>(&acc[0], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + (kb / 16) * (gstep / 16));
       else
         exact_products<TILE, UG0, 1>(&acc[0], arow, tbuf, vb, kb * H * 4, H * 4, H / KS / S);
     }
@@ -644,7 +676,7 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       const int kb = ksu * (H / KS);
       const float *arow[2] = {pfl + kb + 4 * aslot, pfr + kb + 4 * aslot};
       if constexpr (PACKED)
-        exact_products<TILE, UG, 2, true, true>(&acc[1], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + 3 * H * H / 4 + (kb / 16) * (gstep / 16));
+        exact_products<TILE, UG, 2, true, true, ROWS4>(&acc[1], arow, tbuf, vb, 0, gstep, H / KS / S, lane_pk + 3 * H * H / 4 + (kb / 16) * (gstep / 16));
       else
         exact_products<TILE, UG, 2>(&acc[1], arow, tbuf, vb, (3 * H * H + kb * H) * 4, H * 4, H / KS / S);
     }
@@ -735,9 +767,18 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
     float v[NP];
 #pragma unroll
     for (int p = 0; p < NP; p++) {
-      float s = pre[p * NR * 64];
+      float s;
+      if constexpr (ROWS4) {
+        s = 0.f;
 #pragma unroll
-      for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+        for (int g = 0; g < NREG; g++)
+          s += (pre[g * RSZ + p * NR * 64] + pre[g * RSZ + p * NR * 64 + 16]) +
+               (pre[g * RSZ + p * NR * 64 + 32] + pre[g * RSZ + p * NR * 64 + 48]);
+      } else {
+        s = pre[p * NR * 64];
+#pragma unroll
+        for (int g = 1; g < NREG; g++) s += pre[g * RSZ + p * NR * 64];
+      }
       v[p] = s;
     }
     if constexpr (FOLD) {
@@ -780,7 +821,8 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
 static void launch_bwd_children_packed(const RoundBwdChildArgs &a, hipStream_t st) {
   const RoundPlan p = plan_round(a.n);
   dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
-  if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, true, true, true>, grid, 256, 0, st, a);
+  if (a.n <= kRows4Max) launch(treelstm_round_bwd_children_kernel<16, 8, true, true, true, true>, dim3(a.H / 16, (a.n + 3) / 4), 512, 0, st, a);
+  else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, true, true, true>, grid, 256, 0, st, a);
   else launch(treelstm_round_bwd_children_kernel<16, 8, true, true, true>, grid, 512, 0, st, a);
 }
 
@@ -850,7 +892,8 @@ int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pai
   const RoundPlan p = plan_round(n);
   dim3 grid(H / 16, (n + 15) / 16);
   hipStream_t st = as_stream(stream);
-  if (p.waves == 4) launch(treelstm_round_fwd_kernel<16, 4, true, true>, grid, 256, 0, st, a);
+  if (n <= kRows4Max) launch(treelstm_round_fwd_kernel<16, 8, true, true, true>, dim3(H / 16, (n + 3) / 4), 512, 0, st, a);
+  else if (p.waves == 4) launch(treelstm_round_fwd_kernel<16, 4, true, true>, grid, 256, 0, st, a);
   else launch(treelstm_round_fwd_kernel<16, 8, true, true>, grid, 512, 0, st, a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;

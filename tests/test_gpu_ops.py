@@ -969,7 +969,8 @@ def pack_tiles(B):
     return out
 
 
-@pytest.mark.parametrize("L,m,n,H", [(300, 70, 40, 512), (1300, 500, 300, 512), (300, 100, 90, 128), (40, 9, 5, 1024)])
+@pytest.mark.parametrize("L,m,n,H", [(300, 70, 40, 512), (1300, 500, 300, 512), (300, 100, 90, 128), (40, 9, 5, 1024), (60, 16, 13, 512),
+                                     (12, 4, 1, 512)])
 def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L, m, n, H):
     """The pack job against the layout written out in numpy, then the backward launch reading
     the packed weights against the one reading the plain transposes: same products in the same
@@ -1012,14 +1013,19 @@ def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L
                    g.P(d_rows), lo, cnt, L, H, g.stream())
         outs.append((g.host(dxW), g.host(dF), g.host(dc)))
     for a, b, what in zip(outs[0], outs[1], ("dxW", "dF", "dc")):
-        np.testing.assert_array_equal(a, b, err_msg=what)
+        if min(n, m) <= 32:
+            # rounds of at most 32 rows run on tiles of four rows, whose k slots are added up
+            # after the loop instead of inside the MFMA: the same terms in another order
+            close(b, a.astype(np.float64), what)
+        else:
+            np.testing.assert_array_equal(a, b, err_msg=what)
     assert (outs[0][0][:L] != -3.0).any()
     assert hip.lib().cavs_round_packed_ok(40, 96) == 0 and hip.lib().cavs_round_packed_ok(2000, 512) == 0
     with pytest.raises(hip.CavsError, match="cavs_round_packed_ok"):
         hip.call("cavs_treelstm_round_bwd_children_gates_packed", 16, 4 * 96, 16, 16, 16, 16, 16, 16, 16, 16, 0, 5, 0, 96, 0)
 
 
-@pytest.mark.parametrize("n,H", [(40, 512), (300, 512), (1000, 512), (90, 128), (5, 1024)])
+@pytest.mark.parametrize("n,H", [(40, 512), (300, 512), (1000, 512), (90, 128), (5, 1024), (1, 512), (4, 512), (13, 512), (16, 1024), (31, 512)])
 def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
     """The update-and-pack job against w - lr * g and the layout written out in numpy, then the
     forward launch reading the packed weights against the one reading the plain ones."""
@@ -1052,7 +1058,7 @@ def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
     pool = (r.bulk_normal((P_rows + n) * 2 * H).reshape(P_rows + n, 2 * H) * 0.5).astype(np.float32)
     child = np.argsort(r.bulk_normal(P_rows))[: 2 * n].astype(np.int32)
     pair = (P_rows + np.arange(n)).astype(np.int32)
-    child[3] = -1
+    child[min(3, 2 * n - 1)] = -1
     pair[n - 1] = -1
     d_child, d_pair = g.devi(child), g.devi(pair)
     d_xW, d_bias = g.devf(r.bulk_normal(n * 4 * H)), g.devf(r.bulk_normal(4 * H))
@@ -1067,7 +1073,12 @@ def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
                g.P(d_xW), 4 * H, *weights, g.P(d_bias), g.P(G), g.P(hlr), g.P(gates), g.P(msg), g.P(go), g.P(d_rows), n, H, g.stream())
         outs.append([g.host(t) for t in (d_pool, G, hlr, gates, msg, go)])
     for a, b, what in zip(outs[0], outs[1], ("pool", "G", "hlr", "gates", "msg", "graph_out")):
-        np.testing.assert_array_equal(a, b, err_msg=what)
+        if n <= 32 and what not in ("G", "hlr"):
+            # rounds of at most 32 rows run on tiles of four rows, whose k slots are added up
+            # after the loop instead of inside the MFMA: the same terms in another order
+            close(b, a.astype(np.float64), what)
+        else:
+            np.testing.assert_array_equal(a, b, err_msg=what)
     assert (outs[0][3] != 0).all()
     with pytest.raises(hip.CavsError, match="cavs_round_packed_ok"):
         hip.call("cavs_treelstm_round_fwd_packed", 16, 16, 16, 16, 4 * 96, 16, 16, 16, 16, 16, 16, 0, 0, 0, 5, 96, 0)
