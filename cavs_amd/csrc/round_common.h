@@ -162,8 +162,8 @@ struct RoundPlan {
   int tile, waves;
 };
 // Measured on MI355X at H=512: the 16x16 tile wins while a round is too small to give every
-// CU several 32x32 tiles (600 rows: 32 us against 40).  Eight wavefronts per workgroup up to
-// 64 rows (shortest latency chain); four beyond, compiled for four workgroups per CU so that
+// CU several 32x32 tiles (600 rows: 32 us against 40).  Eight wavefronts per workgroup for the
+// smallest rounds (shortest latency chain); four beyond, compiled for four workgroups per CU so that
 // their latency chains overlap; 32x32 tiles above a thousand rows, where operand reuse counts.
 // Packed Tree-LSTM launches of at most this many rows use tiles of four rows (Mma4): measured in
 // the C3 step, 0.4206 ms with sixteen-row tiles throughout, 0.4160 with four-row tiles up to 16
@@ -171,8 +171,10 @@ struct RoundPlan {
 // row tile streams the whole weight panel).
 constexpr int kRows4Max = 32;
 
-inline RoundPlan plan_round(int n) {
-  if (n <= 64) return {16, 8};
+// Eight wavefronts reach up to 128 rows where H lets them keep their exact loops (a multiple of
+// 512): C3 step 0.4135 ms with the limit at 64, 0.4114 at 96, 0.4101 at 128, 0.4143 at 192.
+inline RoundPlan plan_round(int n, int H) {
+  if (n <= (H % 512 == 0 ? 128 : 64)) return {16, 8};
   if (n <= 1024) return {16, 4};
   return {32, 8};
 }

@@ -819,7 +819,7 @@ __global__ void transpose_kernel(float *__restrict__ out, const float *__restric
 
 // the packed variants exist for the shapes cavs_round_packed_ok admits: 16x16 tiles, exact stages
 static void launch_bwd_children_packed(const RoundBwdChildArgs &a, hipStream_t st) {
-  const RoundPlan p = plan_round(a.n);
+  const RoundPlan p = plan_round(a.n, a.H);
   dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
   if (a.n <= kRows4Max) launch(treelstm_round_bwd_children_kernel<16, 8, true, true, true, true>, dim3(a.H / 16, (a.n + 3) / 4), 512, 0, st, a);
   else if (p.waves == 4) launch(treelstm_round_bwd_children_kernel<16, 4, true, true, true>, grid, 256, 0, st, a);
@@ -828,7 +828,7 @@ static void launch_bwd_children_packed(const RoundBwdChildArgs &a, hipStream_t s
 
 template <bool FOLD>
 static void launch_bwd_children(const RoundBwdChildArgs &a, hipStream_t st) {
-  const RoundPlan p = plan_round(a.n);
+  const RoundPlan p = plan_round(a.n, a.H);
   dim3 grid(a.H / p.tile, (a.n + p.tile - 1) / p.tile);
   const bool exact = exact_stages(a.H, p);
   if (p.tile == 16 && p.waves == 4) {
@@ -860,7 +860,7 @@ int cavs_treelstm_round_fwd(float *pool, const int *child, const int *pair, cons
   CAVS_REQUIRE(aligned16(pool) && aligned16(U), "cavs_treelstm_round_fwd: pool and U must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd: graph_out needs out_rows");
   RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, nullptr, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
-  const RoundPlan p = plan_round(n);
+  const RoundPlan p = plan_round(n, H);
   dim3 grid(H / p.tile, (n + p.tile - 1) / p.tile);
   hipStream_t st = as_stream(stream);
   const bool exact = exact_stages(H, p);
@@ -889,7 +889,7 @@ int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pai
   CAVS_REQUIRE(aligned16(pool) && aligned16(U) && aligned16(Upk), "cavs_treelstm_round_fwd_packed: pool, U and Upk must be 16-byte aligned");
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_round_fwd_packed: graph_out needs out_rows");
   RoundFwdArgs a{pool, child, pair, xW, ld_xw, U, Upk, bias, G, hlr, gates, msg, pool, graph_out, out_rows, n, H};
-  const RoundPlan p = plan_round(n);
+  const RoundPlan p = plan_round(n, H);
   dim3 grid(H / 16, (n + 15) / 16);
   hipStream_t st = as_stream(stream);
   if (n <= kRows4Max) launch(treelstm_round_fwd_kernel<16, 8, true, true, true>, dim3(H / 16, (n + 3) / 4), 512, 0, st, a);
@@ -976,7 +976,7 @@ int cavs_treelstm_round_bwd_children_gates(float *dxW, int ld_dxw, float *dF, fl
 
 int cavs_round_packed_ok(int n, int H) {
   if (n < 0 || !round_shape_ok(H)) return 0;
-  const RoundPlan p = plan_round(n > 0 ? n : 1);
+  const RoundPlan p = plan_round(n > 0 ? n : 1, H);
   return p.tile == 16 && exact_stages(H, p) ? 1 : 0;
 }
 

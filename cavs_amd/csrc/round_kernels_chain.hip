@@ -725,7 +725,7 @@ __global__ void treefc_round_bwd_kernel(TreeFcBwdArgs a) {
 // B matrix of BFLOATS floats
 #define CAVS_LAUNCH_ROUND(KERNEL, a, n, H, K, BFLOATS, st, ...)                                                  \
   do {                                                                                                           \
-    const RoundPlan p_ = plan_round(n);                                                                          \
+    const RoundPlan p_ = plan_round(n, H);                                                                          \
     const dim3 grid_((H) / p_.tile, ((n) + p_.tile - 1) / p_.tile);                                              \
     const bool ex_ = chain_exact(K, p_.waves, BFLOATS);                                                          \
     if (p_.tile == 16 && p_.waves == 8) {                                                                        \
@@ -778,7 +778,7 @@ int cavs_lstm_round_fwd(float *pool, const int *child, const int *pair, const fl
 
 int cavs_lstm_round_packed_ok(int n, int H) {
   if (n < 0 || !round_shape_ok(H)) return 0;
-  const RoundPlan p = plan_round(n > 0 ? n : 1);
+  const RoundPlan p = plan_round(n > 0 ? n : 1, H);
   return p.tile == 16 && chain_exact(H, p.waves, 4L * H * H) ? 1 : 0;  // K = H forward; K = 4H backward follows
 }
 
@@ -793,7 +793,7 @@ int cavs_lstm_round_fwd_packed(float *pool, const int *child, const int *pair, c
   CAVS_REQUIRE(!graph_out || out_rows, "cavs_lstm_round_fwd_packed: graph_out needs out_rows");
   LstmFwdArgs a{pool, child, pair, xW, ld_xw, Whp, bias, G, gates, msg, pool, graph_out, out_rows, n, H};
   const dim3 grid(H / 16, (n + 15) / 16);
-  if (plan_round(n).waves == 8) launch(lstm_round_fwd_kernel<16, 8, true, true>, grid, 512, 0, as_stream(stream), a);
+  if (plan_round(n, H).waves == 8) launch(lstm_round_fwd_kernel<16, 8, true, true>, grid, 512, 0, as_stream(stream), a);
   else launch(lstm_round_fwd_kernel<16, 4, true, true>, grid, 256, 0, as_stream(stream), a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
@@ -869,7 +869,7 @@ int cavs_lstm_round_bwd_children_gates_packed(float *da, int ld_da, float *dc, c
   CAVS_REQUIRE(aligned16(da) && aligned16(WhTp), "cavs_lstm_round_bwd_children_gates_packed: da and WhTp must be 16-byte aligned");
   ChildBwdArgs a{da + (long)row0 * ld_da, ld_da, WhTp, H, child_rows, nullptr, 0, n, H, 4 * H, da, dc, gates, G, nullptr, dret, dret_rows, row0, leaf_rows, 0};
   const dim3 grid(H / 16, (n + 15) / 16);
-  if (plan_round(n).waves == 8) launch(round_bwd_children_kernel<16, 8, true, 1, 1, true>, grid, 512, 0, as_stream(stream), a);
+  if (plan_round(n, H).waves == 8) launch(round_bwd_children_kernel<16, 8, true, 1, 1, true>, grid, 512, 0, as_stream(stream), a);
   else launch(round_bwd_children_kernel<16, 4, true, 1, 1, true>, grid, 256, 0, as_stream(stream), a);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
