@@ -14,6 +14,7 @@
 // weight gradients) split K over workgroups with the partials reduced in a fixed
 // order by a second kernel.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 #include "embed_common.h"
@@ -52,7 +53,7 @@ struct GemmArgs {
 
 // Loader of one BX x BK operand tile.  KC: the operand's k index is the contiguous
 // one in memory (element (x,k) at P[x*ld + k]); otherwise element at P[k*ld + x].
-template <int BX, int BK, bool KC, bool VEC>
+template <int BX, int BK, bool KC, bool VEC, bool FASTK = false>
 struct TileLoader {
   static constexpr int NV = BX * BK / 4 / kThreads;  // float4 per thread
   static constexpr int KQ = BK / 4;                  // float4 per row of a k-contiguous tile
@@ -65,6 +66,13 @@ struct TileLoader {
   long base[NV];
   int krel[NV];
   bool xin[NV][4];
+  // Fast path (VEC): when every x of the tile is inside the operand and the offsets fit 32 bits,
+  // a k-tile that lies wholly inside the k range is fetched with unconditional loads at a
+  // wave-uniform pointer plus this byte offset -- no predicate, no 64-bit address arithmetic on
+  // the vector ALU (8192^3: 126.6 -> 133.9 TFLOP/s).  The k loop runs in two parts, the k-tiles
+  // that take it and the rest, so that neither carries the other's code.
+  unsigned boff[NV];
+  bool fast = false;
   // gathered rows (prepare_pull): where the float4 goes as well, or nullptr; the workgroup copies
   // the k-tiles whose number is copy_rem modulo copy_mod (the column tiles of a row tile share the
   // copying of the panel they all read)
@@ -88,7 +96,9 @@ struct TileLoader {
 #pragma unroll
         for (int c = 0; c < 4; c++) xin[i][c] = gx + c < X;
       }
+      if constexpr (FASTK) boff[i] = (unsigned)(base[i] * 4);
     }
+    if constexpr (FASTK) fast = VEC && x0 + BX <= X && (KC ? (long)X * ld : (long)BK * ld) < (1L << 30);
   }
 
   // k-contiguous operand whose rows are looked up: row x0 + r of the operand is the table row that
@@ -98,6 +108,7 @@ struct TileLoader {
     static_assert(KC, "looked-up rows are k-contiguous");
     copy_mod = mod;
     copy_rem = rem;
+    fast = false;
 #pragma unroll
     for (int i = 0; i < NV; i++) {
       const int gx = x0 + tid / KQ + (kThreads / KQ) * i;
@@ -113,6 +124,13 @@ struct TileLoader {
       for (int c = 0; c < 4; c++) xin[i][c] = off >= 0;
       copy[i] = (copy_to && gx < X) ? copy_to + (long)gx * ld_copy + krel[i] : nullptr;
     }
+  }
+
+  // the tile whose first k is k0, wholly inside the k range, of an operand with `fast` set
+  __device__ inline void load_fast(const float *__restrict__ P, long ld, int k0) {
+    const char *Pk = reinterpret_cast<const char *>(KC ? P + k0 : P + (long)k0 * ld);
+#pragma unroll
+    for (int i = 0; i < NV; i++) reg[i] = *reinterpret_cast<const float4 *>(Pk + boff[i]);
   }
 
   // the tile whose first k is k0 (wave-uniform)
@@ -180,7 +198,9 @@ __device__ inline int xcd_remap(int l, int total) {
 // One BM x BN tile of C (or of split `z` of its K range) by the calling workgroup.  `t` is the
 // tile's index, row-major over the tiles of C; As / Bs are the workgroup's two LDS panels of
 // 2 * BK * (BM + PAD) and 2 * BK * (BN + PAD) floats.
-template <int BM, int BN, int BK, bool TA, bool TB, bool VEC>
+// FASTK: the k loop has a first part for k-tiles that take the loaders' fast path (left out of the
+// grouped launch, whose four bodies in one kernel it slowed down: 134.6 -> 147.3 us).
+template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, bool FASTK = true>
 __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float *__restrict__ As_, float *__restrict__ Bs_) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
   constexpr int LDA = BM + PAD, LDB = BN + PAD;
@@ -192,8 +212,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
   const int kbeg = z * g.kchunk;
   const int kend = min(g.K, kbeg + g.kchunk);
 
-  TileLoader<BM, BK, !TA, VEC> la;
-  TileLoader<BN, BK, TB, VEC> lb;
+  TileLoader<BM, BK, !TA, VEC, FASTK> la;
+  TileLoader<BN, BK, TB, VEC, FASTK> lb;
   if constexpr (!TA) {
     if (g.pull_rows) la.prepare_pull(g.pull_rows, g.pull_x, g.K, m0, g.M, tid, g.pull_copy, g.ld_copy, n0 == 0 ? g.pull_ids : nullptr,
                                      tilesN, t % tilesN);
@@ -212,52 +232,89 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
   const int nk = (kend - kbeg + BK - 1) / BK;
+  // k-tiles 0 .. nfast - 1 lie wholly inside the k range of operands that take the fast loads
+  const int nfast = (FASTK && la.fast && lb.fast) ? (kend - kbeg) / BK : 0;
   if (nk > 0) {
-    la.load(g.A, g.lda, kbeg, kend);
-    lb.load(g.B, g.ldb, kbeg, kend);
+    if (FASTK && nfast > 0) {
+      la.load_fast(g.A, g.lda, kbeg);
+      lb.load_fast(g.B, g.ldb, kbeg);
+    } else {
+      la.load(g.A, g.lda, kbeg, kend);
+      lb.load(g.B, g.ldb, kbeg, kend);
+    }
     la.store(As_, tid);
     lb.store(Bs_, tid);
   }
   __syncthreads();
   const int arow = wm * WM + (lane & 31), brow = wn * WN + (lane & 31), khalf = lane >> 5;
-  for (int kt = 0; kt < nk; kt++) {
-    const int cur = kt & 1;
-    if (kt + 1 < nk) {
-      la.load(g.A, g.lda, kbeg + (kt + 1) * BK, kend);
-      lb.load(g.B, g.ldb, kbeg + (kt + 1) * BK, kend);
-    }
-    const float *as = As_ + cur * (BK * LDA), *bs = Bs_ + cur * (BK * LDB);
-    // operand fragments of the k-tile: the reads of AHEAD steps are in flight while a step's
-    // MFMAs issue, so a wavefront does not stall on LDS latency between them
-    constexpr int STEPS = BK / 2, AHEAD = (TM * TN == 1) ? 4 : 2;
-    float a[STEPS][TM], b[STEPS][TN];
-    auto read = [&](int st) {
-#pragma unroll
-      for (int i = 0; i < TM; i++) a[st][i] = as[(2 * st + khalf) * LDA + arow + 32 * i];
-#pragma unroll
-      for (int j = 0; j < TN; j++) b[st][j] = bs[(2 * st + khalf) * LDB + brow + 32 * j];
-    };
-#pragma unroll
-    for (int st = 0; st < AHEAD && st < STEPS; st++) read(st);
-    __builtin_amdgcn_sched_barrier(0);  // the compiler's scheduler would sink each read to its use
-#pragma unroll
-    for (int st = 0; st < STEPS; st++) {
-      if (st + AHEAD < STEPS) read(st + AHEAD);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < TM; i++)
-#pragma unroll
-        for (int j = 0; j < TN; j++)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[st][i], b[st][j], acc[i][j], 0, 0, 0);
-      __builtin_amdgcn_sched_barrier(0);
-    }
-    if (kt + 1 < nk) {
+  // The MFMAs of the k-tile in LDS buffer `cur` (spelled out in each loop through a macro: as a
+  // lambda the compiler scheduled the 64 x 64 kernels 2 % slower).  Operand fragments: the reads of
+  // AHEAD steps are in flight while a step's MFMAs issue, so a wavefront does not stall on LDS
+  // latency between them; the scheduler barriers keep that order (the compiler's scheduler would
+  // sink each read to its use).
+  constexpr int STEPS = BK / 2, AHEAD = (TM * TN == 1) ? 4 : 2;
+#define CAVS_TILE_PRODUCTS(cur)                                                                            \
+  do {                                                                                                     \
+    const float *as = As_ + (cur) * (BK * LDA), *bs = Bs_ + (cur) * (BK * LDB);                            \
+    float a[STEPS][TM], b[STEPS][TN];                                                                      \
+    auto read = [&](int st) {                                                                              \
+      _Pragma("unroll") for (int i = 0; i < TM; i++) a[st][i] = as[(2 * st + khalf) * LDA + arow + 32 * i]; \
+      _Pragma("unroll") for (int j = 0; j < TN; j++) b[st][j] = bs[(2 * st + khalf) * LDB + brow + 32 * j]; \
+    };                                                                                                     \
+    _Pragma("unroll") for (int st = 0; st < AHEAD && st < STEPS; st++) read(st);                           \
+    __builtin_amdgcn_sched_barrier(0);                                                                     \
+    _Pragma("unroll") for (int st = 0; st < STEPS; st++) {                                                 \
+      if (st + AHEAD < STEPS) read(st + AHEAD);                                                            \
+      __builtin_amdgcn_sched_barrier(0);                                                                   \
+      _Pragma("unroll") for (int i = 0; i < TM; i++)                                                       \
+        _Pragma("unroll") for (int j = 0; j < TN; j++)                                                     \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[st][i], b[st][j], acc[i][j], 0, 0, 0);        \
+      __builtin_amdgcn_sched_barrier(0);                                                                   \
+    }                                                                                                      \
+  } while (0)
+  // iteration kt fetches tile kt + 1 while it multiplies tile kt
+  if constexpr (FASTK) {
+    // first the iterations whose next tile takes the fast loads, then the rest
+    const int split = nfast > 1 ? nfast - 1 : 0;
+    for (int kt = 0; kt < split; kt++) {
+      const int cur = kt & 1;
+      la.load_fast(g.A, g.lda, kbeg + (kt + 1) * BK);
+      lb.load_fast(g.B, g.ldb, kbeg + (kt + 1) * BK);
+      CAVS_TILE_PRODUCTS(cur);
       la.store(As_ + (cur ^ 1) * (BK * LDA), tid);
       lb.store(Bs_ + (cur ^ 1) * (BK * LDB), tid);
+      __syncthreads();
     }
-    __syncthreads();
+    for (int kt = split; kt < nk; kt++) {
+      const int cur = kt & 1;
+      if (kt + 1 < nk) {
+        la.load(g.A, g.lda, kbeg + (kt + 1) * BK, kend);
+        lb.load(g.B, g.ldb, kbeg + (kt + 1) * BK, kend);
+      }
+      CAVS_TILE_PRODUCTS(cur);
+      if (kt + 1 < nk) {
+        la.store(As_ + (cur ^ 1) * (BK * LDA), tid);
+        lb.store(Bs_ + (cur ^ 1) * (BK * LDB), tid);
+      }
+      __syncthreads();
+    }
+  } else {
+    for (int kt = 0; kt < nk; kt++) {
+      const int cur = kt & 1;
+      if (kt + 1 < nk) {
+        la.load(g.A, g.lda, kbeg + (kt + 1) * BK, kend);
+        lb.load(g.B, g.ldb, kbeg + (kt + 1) * BK, kend);
+      }
+      CAVS_TILE_PRODUCTS(cur);
+      if (kt + 1 < nk) {
+        la.store(As_ + (cur ^ 1) * (BK * LDA), tid);
+        lb.store(Bs_ + (cur ^ 1) * (BK * LDB), tid);
+      }
+      __syncthreads();
+    }
   }
 
+#undef CAVS_TILE_PRODUCTS
   // C layout of the 32x32 accumulator: element r of lane l is row 8*(r/4) + 4*(l/32) + r%4,
   // column l%32.
 #pragma unroll
@@ -301,7 +358,9 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) float As[2 * BK * (BM + PAD)];
   __shared__ __attribute__((aligned(16))) float Bs[2 * BK * (BN + PAD)];
   const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
-  gemm_tile<BM, BN, BK, TA, TB, VEC>(g, xcd_remap(blockIdx.x, tiles), blockIdx.y, As, Bs);
+  // (the fast part of the k loop pays on the large tile; the 64 x 64 launches are products with
+  // short K or ragged edges, which it only made larger)
+  gemm_tile<BM, BN, BK, TA, TB, VEC, BM == 128>(g, xcd_remap(blockIdx.x, tiles), blockIdx.y, As, Bs);
 }
 
 // Several independent products in one launch (the deferred weight gradients of a step and the
@@ -335,10 +394,10 @@ __global__ __launch_bounds__(kThreads) void sgemm_group_kernel(GemmGroup G) {
   const int t = w % G.tiles[p], z = w / G.tiles[p];
   const GemmArgs &g = G.g[p];
   switch (G.form[p]) {
-    case 0: gemm_tile<BM, BN, BK, false, false, VEC>(g, t, z, As, Bs); break;
-    case 1: gemm_tile<BM, BN, BK, false, true, VEC>(g, t, z, As, Bs); break;
-    case 2: gemm_tile<BM, BN, BK, true, false, VEC>(g, t, z, As, Bs); break;
-    default: gemm_tile<BM, BN, BK, true, true, VEC>(g, t, z, As, Bs); break;
+    case 0: gemm_tile<BM, BN, BK, false, false, VEC, false>(g, t, z, As, Bs); break;
+    case 1: gemm_tile<BM, BN, BK, false, true, VEC, false>(g, t, z, As, Bs); break;
+    case 2: gemm_tile<BM, BN, BK, true, false, VEC, false>(g, t, z, As, Bs); break;
+    default: gemm_tile<BM, BN, BK, true, true, VEC, false>(g, t, z, As, Bs); break;
   }
 }
 
