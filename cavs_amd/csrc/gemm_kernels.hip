@@ -198,8 +198,7 @@ __device__ inline int xcd_remap(int l, int total) {
 // One BM x BN tile of C (or of split `z` of its K range) by the calling workgroup.  `t` is the
 // tile's index, row-major over the tiles of C; As / Bs are the workgroup's two LDS panels of
 // 2 * BK * (BM + PAD) and 2 * BK * (BN + PAD) floats.
-// FASTK: the k loop has a first part for k-tiles that take the loaders' fast path (left out of the
-// grouped launch, whose four bodies in one kernel it slowed down: 134.6 -> 147.3 us).
+// FASTK: the k loop has a first part for k-tiles that take the loaders' fast path.
 template <int BM, int BN, int BK, bool TA, bool TB, bool VEC, bool FASTK = true>
 __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float *__restrict__ As_, float *__restrict__ Bs_) {
   constexpr int WM = BM / 2, WN = BN / 2, TM = WM / 32, TN = WN / 32;
@@ -394,10 +393,10 @@ __global__ __launch_bounds__(kThreads) void sgemm_group_kernel(GemmGroup G) {
   const int t = w % G.tiles[p], z = w / G.tiles[p];
   const GemmArgs &g = G.g[p];
   switch (G.form[p]) {
-    case 0: gemm_tile<BM, BN, BK, false, false, VEC, false>(g, t, z, As, Bs); break;
-    case 1: gemm_tile<BM, BN, BK, false, true, VEC, false>(g, t, z, As, Bs); break;
-    case 2: gemm_tile<BM, BN, BK, true, false, VEC, false>(g, t, z, As, Bs); break;
-    default: gemm_tile<BM, BN, BK, true, true, VEC, false>(g, t, z, As, Bs); break;
+    case 0: gemm_tile<BM, BN, BK, false, false, VEC, true>(g, t, z, As, Bs); break;
+    case 1: gemm_tile<BM, BN, BK, false, true, VEC, true>(g, t, z, As, Bs); break;
+    case 2: gemm_tile<BM, BN, BK, true, false, VEC, true>(g, t, z, As, Bs); break;
+    default: gemm_tile<BM, BN, BK, true, true, VEC, true>(g, t, z, As, Bs); break;
   }
 }
 
