@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, from profiles/bench_<workload>_hbm_traffic_pmc.txt
-PMC_TRAFFIC_BYTES = {("C3", "round"): 17.52e6, ("C4", "gemm"): 319.3e6, ("C5", "gemm"): 939.6e6}
+PMC_TRAFFIC_BYTES = {("C3", "round"): 17.52e6, ("C4", "gemm"): 328.2e6, ("C5", "gemm"): 970.4e6}
 # a constant taken from the profile named, not a counter read during this run
 PMC_TRAFFIC_SOURCE = {k: f"profiles/bench_{k[0]}_hbm_traffic_pmc.txt (two rocprofv3 --pmc runs of this command, FETCH_SIZE and "
                          "WRITE_SIZE per dispatch of the class; a constant copied from there, not read in this run)"
