@@ -172,7 +172,7 @@ __global__ __launch_bounds__(256) void fc_xent_reduce_kernel(const float *__rest
 
 static int head_blocks(int n) {
   int want = (n + 7) / 8;  // two rows per wavefront
-  int cap = num_cus();
+  int cap = num_cus() * 3 / 2;  // (C3: 0.4086 ms with one workgroup per CU, 0.4076 with one and a half, 0.4081 with two)
   return want < cap ? (want < 1 ? 1 : want) : cap;
 }
 
