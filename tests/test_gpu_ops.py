@@ -161,6 +161,29 @@ def test_sgemm_matches_oracle(g, oracle, tA, tB, M, N, K):
     close(g.host(Cd), exact, "sgemm vs fp64")
 
 
+@pytest.mark.parametrize("tA,tB", [(0, 0), (0, 1), (1, 0), (1, 1)])
+@pytest.mark.parametrize("M,N,K", [(2900, 2950, 116), (1000, 1100, 4100), (2944, 2944, 128)])
+def test_sgemm_on_the_large_tile_with_ragged_edges(g, tA, tB, M, N, K):
+    """Shapes that take the 128 x 128 tile (alone, and with K split over workgroups): tiles at the
+    ragged edges and the k tail go through the general loads, everything else through the fast part of
+    the k loop; each form against the fp64 product."""
+    import torch
+
+    r = rng(M + 3 * N + 5 * K + 2 * tA + tB)
+    A = r.bulk_uniform(M * K, -1, 1).reshape((K, M) if tA else (M, K))
+    B = r.bulk_uniform(N * K, -1, 1).reshape((N, K) if tB else (K, N))
+    nbytes = hip.lib().cavs_sgemm_splitk_workspace(M, N, K)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    Cd = g.zeros(M, N + 4, fill=float("nan"))
+    Cd[:, N:] = 5.0
+    g.call("cavs_sgemm_splitk", tA, tB, M, N, K, 1.0, g.P(g.devf(A)), A.shape[1], g.P(g.devf(B)), B.shape[1], 0.0, g.P(Cd), N + 4,
+           g.P(ws), nbytes, g.stream())
+    got = g.host(Cd)
+    np.testing.assert_array_equal(got[:, N:], 5.0)
+    exact = (A.T if tA else A).astype(np.float64) @ (B.T if tB else B).astype(np.float64)
+    close(got[:, :N], exact, "large-tile product vs fp64")
+
+
 def test_sgemm_strided_operands_and_addrows(g, oracle):
     """The shapes the Tree-LSTM backward uses: A is a column block of a wider slab,
     C a column block of the child-gradient slab, plus the per-vertex addend."""
