@@ -993,7 +993,7 @@ def pack_tiles(B):
 
 
 @pytest.mark.parametrize("L,m,n,H", [(300, 70, 40, 512), (1300, 500, 300, 512), (300, 100, 90, 128), (40, 9, 5, 1024), (60, 16, 13, 512),
-                                     (12, 4, 1, 512)])
+                                     (12, 4, 1, 512), (400, 120, 70, 512)])
 def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L, m, n, H):
     """The pack job against the layout written out in numpy, then the backward launch reading
     the packed weights against the one reading the plain transposes: same products in the same
@@ -1048,7 +1048,7 @@ def test_packed_transposed_weights_give_the_same_backward_round_bit_for_bit(g, L
         hip.call("cavs_treelstm_round_bwd_children_gates_packed", 16, 4 * 96, 16, 16, 16, 16, 16, 16, 16, 16, 0, 5, 0, 96, 0)
 
 
-@pytest.mark.parametrize("n,H", [(40, 512), (300, 512), (1000, 512), (90, 128), (5, 1024), (1, 512), (4, 512), (13, 512), (16, 1024), (31, 512)])
+@pytest.mark.parametrize("n,H", [(40, 512), (300, 512), (1000, 512), (90, 128), (5, 1024), (1, 512), (4, 512), (13, 512), (16, 1024), (31, 512), (100, 512), (128, 1024)])
 def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
     """The update-and-pack job against w - lr * g and the layout written out in numpy, then the
     forward launch reading the packed weights against the one reading the plain ones."""
