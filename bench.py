@@ -74,7 +74,7 @@ def cpu_baseline(w, budget_s=12.0):
     for _ in range(2):
         pyoracle.model_step(w["model"], w["graph"], w["x"], w["labels"], w["params"], **dict(args, threads=1))
     el1 = time.perf_counter() - t1
-    # configuration C1 as the survey defines it: the chain LSTM (V=1000, E=H=128, T=20, B=16) on the
+    # configuration C1, the reference's own CPU-runnable case: the chain LSTM (V=1000, E=H=128, T=20, B=16) on the
     # reference's CPU path -- its serial scheduler (cavs/midend/graph_scheduler.cc:83-167), one
     # forward+backward step, single thread
     from cavs_amd import synth
