@@ -28,7 +28,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, from profiles/bench_<workload>_hbm_traffic_pmc.txt
-PMC_TRAFFIC_BYTES = {("C3", "round"): 17.52e6, ("C4", "gemm"): 328.2e6, ("C5", "gemm"): 970.4e6}
+PMC_TRAFFIC_BYTES = {("C3", "round"): 17.54e6, ("C4", "gemm"): 328.6e6, ("C5", "gemm"): 921.8e6}
 # a constant taken from the profile named, not a counter read during this run
 PMC_TRAFFIC_SOURCE = {k: f"profiles/bench_{k[0]}_hbm_traffic_pmc.txt (two rocprofv3 --pmc runs of this command, FETCH_SIZE and "
                          "WRITE_SIZE per dispatch of the class; a constant copied from there, not read in this run)"
@@ -249,11 +249,12 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
     # stamping a start and a stop event themselves (the interval a kernel trace reports) on the
     # session's own stream; kept out of the throughput figure above.
     s.profile(True)
-    flops = rflops = gbytes = sbytes = 0.0
+    flops = hinted = rflops = gbytes = sbytes = 0.0
     for i in range(warmup, warmup + steps):
         g, x, lab = feeds[i % len(feeds)]
         s.step(g, x, lab, backward=True, lr=a.lr)
         flops += s.counter("gemm_flops")
+        hinted += s.counter("gemm_flops_hinted")
         rflops += s.counter("round_flops")
         gbytes += s.counter("gather_bytes")
         sbytes += s.counter("scatter_bytes")
@@ -309,6 +310,9 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
                    "frac": round(v["tf"] / FP32_MFMA_PEAK_TF, 4),
                    "avg_launch_us": round(1e3 * v["ms"] / max(v["n"], 1), 3), "launches_per_step": round(v["n"] / steps, 1)}
                for k, v in mfma.items()},
+            # of the GEMM class's flops (2*M*N*K of the reference's products): the share that multiplies blocks
+            # known to be zero or unused (forget-gate columns of the leaves) and is skipped tile by tile
+            "gemm_flops_hinted_frac": round(hinted / flops, 4) if flops else 0.0,
             # separate gather / scatter launches only (rounds that run fused move their rows inside the round kernel)
             "gather": hbm(gbytes, gat_ms, gat_n), "scatter": hbm(sbytes, sca_ms, sca_n),
             "gates": {"avg_launch_us": round(1e3 * gates_ms / max(gates_n, 1), 3)},

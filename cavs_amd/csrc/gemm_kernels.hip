@@ -49,6 +49,14 @@ struct GemmArgs {
   float *pull_copy = nullptr;
   long ld_copy = 0;
   float *pull_ids = nullptr;
+  // A block the caller knows about (cavs_gemm_desc::zero_kind and friends): the tiles it covers
+  // run a shorter k range, or none
+  int zkind = 0, zrows = 0, zcol = 0;
+  // > 0: the launch is two launches back to back, the first zseg tiles (the row tiles inside the
+  // block, whose workgroups do less) and the rest, each padded to a multiple of 8 workgroups and
+  // dealt to the XCDs by itself: with one deal over all tiles the XCDs that hold the first
+  // tiles would finish early and the others set the time as before
+  int zseg = 0;
 };
 
 // Loader of one BX x BK operand tile.  KC: the operand's k index is the contiguous
@@ -208,14 +216,25 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs &g, int t, int z, float
   const int wm = wave >> 1, wn = wave & 1;
   const int tilesN = (g.N + BN - 1) / BN;
   const int m0 = (t / tilesN) * BM, n0 = (t % tilesN) * BN;
-  const int kbeg = z * g.kchunk;
-  const int kend = min(g.K, kbeg + g.kchunk);
+  int kbeg = z * g.kchunk;
+  int kend = min(g.K, kbeg + g.kchunk);
+  if (g.zkind == CAVS_GEMM_C_UNUSED) {  // rows below zrows of C are not wanted from column zcol on: left zero
+    if (m0 + BM <= g.zrows && n0 >= g.zcol) kend = kbeg;
+  } else if (g.zkind == CAVS_GEMM_A_ZERO) {  // rows below zrows of A (row-major M x K) are zero from k = zcol on
+    if (!TA && m0 + BM <= g.zrows) kend = max(kbeg, min(kend, g.zcol));
+  } else if (g.zkind == CAVS_GEMM_B_ZERO) {  // rows k < zrows of B (row-major K x N) are zero from column zcol on
+    if (!TB && n0 >= g.zcol) kbeg = min(kend, max(kbeg, g.zrows / 32 * 32));
+  }
 
   TileLoader<BM, BK, !TA, VEC, FASTK> la;
   TileLoader<BN, BK, TB, VEC, FASTK> lb;
   if constexpr (!TA) {
-    if (g.pull_rows) la.prepare_pull(g.pull_rows, g.pull_x, g.K, m0, g.M, tid, g.pull_copy, g.ld_copy, n0 == 0 ? g.pull_ids : nullptr,
-                                     tilesN, t % tilesN);
+    if (g.pull_rows) {
+      // the column tiles of this row tile that do run share the copying
+      const int active = (g.zkind == CAVS_GEMM_C_UNUSED && m0 + BM <= g.zrows) ? min(tilesN, (g.zcol + BN - 1) / BN) : tilesN;
+      la.prepare_pull(g.pull_rows, g.pull_x, g.K, m0, g.M, tid, g.pull_copy, g.ld_copy, n0 == 0 ? g.pull_ids : nullptr, active,
+                      t % tilesN);
+    }
     else la.prepare(g.lda, m0, g.M, tid);
   } else {
     la.prepare(g.lda, m0, g.M, tid);
@@ -357,9 +376,24 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
   __shared__ __attribute__((aligned(16))) float As[2 * BK * (BM + PAD)];
   __shared__ __attribute__((aligned(16))) float Bs[2 * BK * (BN + PAD)];
   const int tiles = ((g.M + BM - 1) / BM) * ((g.N + BN - 1) / BN);
+  int t;
+  if (g.zseg > 0) {
+    const int first = (g.zseg + 7) & ~7, b = blockIdx.x;
+    if (b < first) {
+      t = xcd_remap(b, first);
+      if (t >= g.zseg) return;
+    } else {
+      const int rest = tiles - g.zseg;
+      t = xcd_remap(b - first, (rest + 7) & ~7);
+      if (t >= rest) return;
+      t += g.zseg;
+    }
+  } else {
+    t = xcd_remap(blockIdx.x, tiles);
+  }
   // (the fast part of the k loop pays on the large tile; the 64 x 64 launches are products with
   // short K or ragged edges, which it only made larger)
-  gemm_tile<BM, BN, BK, TA, TB, VEC, BM == 128>(g, xcd_remap(blockIdx.x, tiles), blockIdx.y, As, Bs);
+  gemm_tile<BM, BN, BK, TA, TB, VEC, BM == 128>(g, t, blockIdx.y, As, Bs);
 }
 
 // Several independent products in one launch (the deferred weight gradients of a step and the
@@ -682,8 +716,16 @@ static bool vec_path_ok(const GemmArgs &g, int tA, int tB) {
 }
 
 template <int BM, int BN, int BK>
-static void launch_tile(const GemmArgs &g, int tA, int tB, bool vec, const GemmPlan &p, hipStream_t st) {
+static void launch_tile(const GemmArgs &args, int tA, int tB, bool vec, const GemmPlan &p, hipStream_t st) {
+  GemmArgs g = args;
   dim3 grid((unsigned)p.tiles, p.splits), block(kThreads);
+  if (g.zkind == CAVS_GEMM_A_ZERO || g.zkind == CAVS_GEMM_C_UNUSED) {
+    const long inside = (long)(std::min(g.zrows, g.M) / BM) * ((g.N + BN - 1) / BN);
+    if (inside > 0 && inside < p.tiles) {
+      g.zseg = (int)inside;
+      grid.x = (unsigned)((inside + 7) / 8 * 8 + (p.tiles - inside + 7) / 8 * 8);
+    }
+  }
 #define CAVS_GEMM_CASE(TA, TB)                                                  \
   if (vec)                                                                      \
     launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, true>, grid, block, 0, st, g);      \
@@ -730,14 +772,32 @@ struct PullRows {
   float *ids;
 };
 
+// What the caller knows about a block of an operand or of the result (cavs_gemm_desc::zero_kind,
+// zero_rows, zero_col).  It is a licence, not an order: set() keeps it only in the forms the tile
+// routine acts on and the kernels that never look at it give the plain product.
+struct BlockHint {
+  int kind = 0, rows = 0, col = 0;
+  void set(GemmArgs *g, int tA, int tB, bool plain_store) const {
+    if (rows <= 0 || col < 0) return;
+    const bool ok = (kind == CAVS_GEMM_C_UNUSED && plain_store && col > 0) || (kind == CAVS_GEMM_A_ZERO && !tA && col % 4 == 0) ||
+                    (kind == CAVS_GEMM_B_ZERO && !tB);
+    if (!ok) return;
+    g->zkind = kind;
+    g->zrows = rows;
+    g->zcol = col;
+  }
+};
+
 static int run_gemm(const char *who, int tA, int tB, int M, int N, int K, float alpha, const float *A,
                     int lda, const float *B, int ldb, float beta, float *C, int ldc, const float *D,
-                    int ldd, int dshift, void *ws, size_t ws_bytes, void *stream, const PullRows *pull = nullptr) {
+                    int ldd, int dshift, void *ws, size_t ws_bytes, void *stream, const PullRows *pull = nullptr,
+                    const BlockHint *hint = nullptr) {
   int rc = check_gemm(who, tA, tB, M, N, K, A, lda, B, ldb, C, ldc);
   if (rc || M == 0 || N == 0) return rc;
   GemmPlan p = plan_gemm(tA, tB, M, N, K, !pull && skinny_ok(tA, tB, K, A, lda, B, ldb), ws != nullptr);
   hipStream_t st = as_stream(stream);
   GemmArgs g{M, N, K, A, lda, B, ldb, C, ldc, alpha, beta, D, ldd, dshift, p.kchunk, nullptr};
+  if (hint) hint->set(&g, tA, tB, beta == 0.f && !D);
   if (pull) {
     g.pull_rows = pull->rows;
     g.pull_x = pull->x;
@@ -807,6 +867,8 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
       if (rc) return rc;
     }
     CAVS_REQUIRE(q.M >= 0 && q.N >= 0 && q.K >= 0, "cavs_sgemm_group: negative dimension in product %d", p);
+    CAVS_REQUIRE(q.zero_kind >= 0 && q.zero_kind <= CAVS_GEMM_B_ZERO && q.zero_rows >= 0 && q.zero_col >= 0,
+                 "cavs_sgemm_group: bad block hint in product %d (kind %d, rows %d, col %d)", p, q.zero_kind, q.zero_rows, q.zero_col);
     tiles[p] = (long)((q.M + 63) / 64) * ((q.N + 63) / 64);
     // a product that fills the chip with large tiles by itself is better off on them, alone
     alone[p] = q.M > 0 && q.N > 0 && plan_gemm(q.transA, q.transB, q.M, q.N, q.K, false, true).kind == GemmPlan::TILE128;
@@ -856,6 +918,7 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
     int kchunk = q.K > 0 ? (int)(((q.K + s - 1) / s + 31) / 32 * 32) : 1;
     int splits = q.K > 0 ? (q.K + kchunk - 1) / kchunk : 1;
     GemmArgs g{q.M, q.N, q.K, q.A, q.lda, q.B, q.ldb, q.C, q.ldc, q.alpha, q.beta, nullptr, 0, 0, kchunk, nullptr};
+    BlockHint{q.zero_kind, q.zero_rows, q.zero_col}.set(&g, q.transA, q.transB, q.beta == 0.f);
     if (splits > 1) {
       if (ws) g.ws = reinterpret_cast<float *>(static_cast<char *>(ws) + need);
       need += ((size_t)splits * q.M * q.N * sizeof(float) + 255) / 256 * 256;
@@ -894,8 +957,9 @@ static int run_group(int count, const cavs_gemm_desc *d, void *ws, size_t ws_byt
   for (int p = 0; p < count; p++) {
     const cavs_gemm_desc &q = d[p];
     if (q.M == 0 || q.N == 0 || !alone[p]) continue;
+    const BlockHint hint{q.zero_kind, q.zero_rows, q.zero_col};
     int rc = run_gemm("cavs_sgemm_group", q.transA, q.transB, q.M, q.N, q.K, q.alpha, q.A, q.lda, q.B, q.ldb, q.beta,
-                      q.C, q.ldc, nullptr, 0, 0, ws, ws_bytes, stream);
+                      q.C, q.ldc, nullptr, 0, 0, ws, ws_bytes, stream, nullptr, &hint);
     if (rc) return rc;
   }
   hipStream_t st = as_stream(stream);
@@ -997,8 +1061,11 @@ int cavs_sgemm_group_embed_bwd(int count, const cavs_gemm_desc *products, int em
 }
 
 int cavs_embed_pull_sgemm(float *C, int ldc, float *e_out, int ld_e, float *ids_out, const float *x, const int *rows,
-                          const float *table, int n, int E, const float *B, int ldb, int N, void *stream) {
+                          const float *table, int n, int E, const float *B, int ldb, int N, int unused_rows, int unused_col,
+                          void *stream) {
   CAVS_REQUIRE(n >= 0 && E > 0 && N >= 0 && ld_e >= E, "cavs_embed_pull_sgemm: bad shape n=%d E=%d N=%d ld_e=%d", n, E, N, ld_e);
+  CAVS_REQUIRE(unused_rows >= 0 && unused_col >= 0, "cavs_embed_pull_sgemm: bad unused block (rows %d, col %d)", unused_rows, unused_col);
+  const BlockHint hint{CAVS_GEMM_C_UNUSED, unused_rows, unused_col};
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(e_out && ids_out && x && rows && table, "cavs_embed_pull_sgemm: null pointer");
   // the copy goes out in whole float4s on the vector path
@@ -1008,10 +1075,12 @@ int cavs_embed_pull_sgemm(float *C, int ldc, float *e_out, int ld_e, float *ids_
   if (N == 0 || plan_gemm(0, 0, n, N, E, false, false).kind == GemmPlan::TILE128) {
     int rc = cavs_embed_pull_fwd(e_out, ld_e, ids_out, x, rows, table, n, E, stream);
     if (rc || N == 0) return rc;
-    return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, e_out, ld_e, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream);
+    return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, e_out, ld_e, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream,
+                    nullptr, &hint);
   }
   const PullRows pull{rows, x, e_out, ld_e, ids_out};
-  return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, table, E, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream, &pull);
+  return run_gemm("cavs_embed_pull_sgemm", 0, 0, n, N, E, 1.f, table, E, B, ldb, 0.f, C, ldc, nullptr, 0, 0, nullptr, 0, stream, &pull,
+                  &hint);
 }
 
 int cavs_sgemm(int transA, int transB, int M, int N, int K, float alpha, const float *A, int lda,

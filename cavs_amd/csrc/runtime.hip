@@ -73,7 +73,7 @@ using namespace cavs;
 extern "C" {
 
 const char *cavs_last_error(void) { return g_err; }
-int cavs_abi_version(void) { return 1; }
+int cavs_abi_version(void) { return 2; }
 
 int cavs_init(int device) {
   CAVS_HIP_TRY(hipSetDevice(device));

@@ -36,7 +36,11 @@ TASK_TREELSTM_GATES_ROWS = 8
 class GemmDesc(C.Structure):
     """cavs_gemm_desc: one product of cavs_sgemm_group"""
     _fields_ = [("transA", _I), ("transB", _I), ("M", _I), ("N", _I), ("K", _I), ("alpha", _F), ("beta", _F),
-                ("A", _P), ("lda", _I), ("B", _P), ("ldb", _I), ("C", _P), ("ldc", _I)]
+                ("A", _P), ("lda", _I), ("B", _P), ("ldb", _I), ("C", _P), ("ldc", _I),
+                ("zero_kind", _I), ("zero_rows", _I), ("zero_col", _I)]
+
+
+GEMM_C_UNUSED, GEMM_A_ZERO, GEMM_B_ZERO = 1, 2, 3
 
 
 # name -> argtypes (every function returns int unless listed in _RESTYPE)
@@ -76,7 +80,7 @@ _SIGS = {
     "cavs_colsum": [_P, _P, _I, _I, _I, _I, _P],
     "cavs_embed_fwd": [_P, _I, _P, _P, _I, _I, _P],
     "cavs_embed_pull_fwd": [_P, _I, _P, _P, _P, _P, _I, _I, _P],
-    "cavs_embed_pull_sgemm": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _P],
+    "cavs_embed_pull_sgemm": [_P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _P],
     "cavs_embed_bwd": [_P, _P, _P, _I, _I, _I, _P],
     "cavs_bias_add_rows": [_P, _P, _P, _I, _I, _P],
     "cavs_softmax_xent": [_P, _P, _P, _P, _I, _I, _P],

@@ -205,12 +205,26 @@ void Engine::gemm(int tA, int tB, int M, int N, int K, const float *A, int lda, 
   c_launches_ += 1;
 }
 
+// flops of a product that its block hint declares to be zero or unwanted (the kernels skip them
+// tile by tile)
+static double hinted_flops(const cavs_gemm_desc &q) {
+  double mnk = 0;
+  if (q.zero_kind == CAVS_GEMM_A_ZERO && !q.transA)
+    mnk = (double)std::min(q.zero_rows, q.M) * std::max(0, q.K - q.zero_col) * q.N;
+  else if (q.zero_kind == CAVS_GEMM_B_ZERO && !q.transB)
+    mnk = (double)std::min(q.zero_rows, q.K) * std::max(0, q.N - q.zero_col) * q.M;
+  return 2.0 * mnk;
+}
+
 void Engine::gemm_group(const std::vector<cavs_gemm_desc> &products) {
   const int count = (int)products.size();
   float *ws = workspace(cavs_sgemm_group_workspace(count, products.data()));
   ProfScope ps(this, K_GEMM);
   check(cavs_sgemm_group(count, products.data(), ws, ws_.capacity() * 4, stream_));
-  for (const cavs_gemm_desc &q : products) c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
+  for (const cavs_gemm_desc &q : products) {
+    c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
+    c_gemm_flops_hinted_ += hinted_flops(q);
+  }
   c_launches_ += 1;
 }
 
@@ -566,7 +580,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     *last_busy_ = true;
     last_free_ev_ = nullptr;
   }
-  c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
+  c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_gemm_flops_hinted_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   c_round_flops_ = 0;
   bias_jobs_.clear();
   wait_ms_ = 0.f;
@@ -773,9 +787,12 @@ void Engine::treelstm_forward() {
   // Pull of the word id, the lookup and x * W: one launch
   {
     ProfScope ps(this, K_GEMM);
-    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, W, 4 * H, 4 * H, stream_));
+    // (a leaf gathers zero rows, so its forget gates multiply zero: their columns of x * W are not wanted)
+    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E, W, 4 * H, 4 * H,
+                                sched_->leaf_prefix, 3 * H, stream_));
   }
   c_gemm_flops_ += 2.0 * N * 4 * H * E;
+  c_gemm_flops_hinted_ += 2.0 * sched_->leaf_prefix * H * E;
   c_launches_ += 1;
   if (!sched_->batching) {  // leaves are interleaved with internal vertices: their child rows must read as zero
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
@@ -926,13 +943,15 @@ void Engine::treelstm_backward() {
   }
   // weight gradients once over all rows (OPT_BATCHING semantics; without it the reference
   // accumulates the same sums round by round)
-  const int lp = sched_->leaf_prefix;  // leaves contribute exact zeros to dU
+  // leaves contribute exact zeros to dU, and the f columns of their rows of dxW are exact zeros
+  const int lp = sched_->leaf_prefix;
   float *dU = param("U").g;
   const bool bias_row = bias_row_ok();  // the ones column of e_ turns row E of dW into the column sums of dxW
   gemm_group_embedding_backward({
-      {0, 1, N, E, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, W, 4 * H, de_.get(), E},
+      {0, 1, N, E, 4 * H, 1.f, 0.f, dxW_.get(), 4 * H, W, 4 * H, de_.get(), E, CAVS_GEMM_A_ZERO, lp, 3 * H},
       // (all four padding columns of e_ take part, so that the product keeps 16-byte operand loads)
-      {1, 0, bias_row ? ld_e_ : E, 4 * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), 4 * H, param("W").g, 4 * H},
+      {1, 0, bias_row ? ld_e_ : E, 4 * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), 4 * H, param("W").g, 4 * H, CAVS_GEMM_B_ZERO, lp,
+       3 * H},
       {1, 0, H, 3 * H, N - lp, 1.f, 0.f, hlr_.at((size_t)lp * H), H, dxW_.at((size_t)lp * 4 * H), 4 * H, dU, 3 * H},
       {1, 0, H, H, 2 * (N - lp), 1.f, 0.f, G_.at((size_t)2 * lp * 2 * H), 2 * H, dF_.at((size_t)2 * lp * H), H,
        dU + (size_t)3 * H * H, H},
@@ -1059,7 +1078,10 @@ void Engine::gemm_group_embedding_backward(const std::vector<cavs_gemm_desc> &pr
     ProfScope ps(this, K_GEMM);
     check(cavs_sgemm_group_embed_bwd(count, products.data(), 0, emb.g, xs_.get(), ws, ws_.capacity() * 4, stream_));
   }
-  for (const cavs_gemm_desc &q : products) c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
+  for (const cavs_gemm_desc &q : products) {
+    c_gemm_flops_ += 2.0 * q.M * q.N * q.K;
+    c_gemm_flops_hinted_ += hinted_flops(q);
+  }
   c_launches_ += 2;
   xs_.swap(xs_prev_);  // this step's ids: the rows that are dirty now
   emb_dirty_n_ = N_;
@@ -1073,7 +1095,8 @@ void Engine::lstm_forward() {
   const float *Wx = param("W").w, *Wh = Wx + (size_t)4 * H * H, *Bv = param("Bv").w;
   {  // Pull of the token id, the lookup and x * W_x: one launch
     ProfScope ps(this, K_GEMM);
-    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, Wx, 4 * H, 4 * H, stream_));
+    check(cavs_embed_pull_sgemm(xW_.get(), 4 * H, e_.get(), H, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, H, Wx, 4 * H, 4 * H, 0, 0,
+                                stream_));
   }
   c_gemm_flops_ += 2.0 * N * 4 * H * H;
   c_launches_ += 1;
@@ -1419,6 +1442,7 @@ double Engine::counter(const std::string &key) const {
   if (key == "gather_bytes") return c_gather_bytes_;
   if (key == "scatter_bytes") return c_scatter_bytes_;
   if (key == "gemm_flops") return c_gemm_flops_;
+  if (key == "gemm_flops_hinted") return c_gemm_flops_hinted_;
   if (key == "round_flops") return c_round_flops_;
   if (key == "launches") return c_launches_;
   if (key == "rounds") return (double)sched_->rounds.size();

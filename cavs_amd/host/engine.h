@@ -250,7 +250,7 @@ class Engine {
 
   // counters of the last step
   double c_round_flops_ = 0;
-  double c_gather_rows_ = 0, c_scatter_rows_ = 0, c_gemm_flops_ = 0, c_launches_ = 0,
+  double c_gather_rows_ = 0, c_scatter_rows_ = 0, c_gemm_flops_ = 0, c_gemm_flops_hinted_ = 0, c_launches_ = 0,
          c_gather_bytes_ = 0, c_scatter_bytes_ = 0;
 };
 

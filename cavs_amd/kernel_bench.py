@@ -156,6 +156,17 @@ def gemm(iters, st):
     us = _time(lambda: hip.call("cavs_sgemm_group", len(shapes), descs, ws.data_ptr(), nb, st), iters, st)
     _emit("sgemm_group", "C3 step: de + dW + dU_iou + dU_f in one launch (+ one reduce)", us,
           flops=sum(2.0 * M * Nn * K for _, _, M, Nn, K in shapes))
+    del keep, ws
+    # C5's de with the block hint of a step: the first half of the slab rows are leaves, whose forget-gate
+    # columns of dxW are zero; the flops are those left to do
+    H, E, N = 1024, 1024, 73000
+    A, B, Cm = torch.randn(N, 4 * H, **f32), torch.randn(E, 4 * H, **f32), torch.empty(N, E, **f32)
+    A[:N // 2, 3 * H:] = 0
+    one = (hip.GemmDesc * 1)()
+    one[0] = hip.GemmDesc(0, 1, N, E, 4 * H, 1.0, 0.0, A.data_ptr(), 4 * H, B.data_ptr(), 4 * H, Cm.data_ptr(), E, hip.GEMM_A_ZERO, N // 2, 3 * H)
+    us = _time(lambda: hip.call("cavs_sgemm_group", 1, one, None, 0, st), max(5, iters // 5), st)
+    _emit("sgemm_group", f"C5 de = dxW*W^T, f columns of {N // 2} leaf rows known zero: NT M={N} N={E} K={4 * H}", us,
+          flops=2.0 * N * E * 4 * H - 2.0 * (N // 2) * E * H)
 
 
 def gates(iters, st):

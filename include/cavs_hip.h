@@ -129,16 +129,16 @@ int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, 
  * (cavs_sgemm_splitk_workspace(M, N, K) above the maximum) is refused with CAVS_EINVAL.  All
  * calls on a GPU share that GPU's buffer: calls that overlap in time on one GPU (two streams,
  * two threads) race; calls on one stream are ordered by it. */
+size_t cavs_sgemm_splitk_static_max_bytes(void);
+int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
+                             int lda, const float *B, int ldb, float beta, float *C, int ldc,
+                             void *stream);
 /* Measurement aid (no counterpart in the reference): one launch in which every wavefront of
  * four workgroups per CU issues iters * 8 independent v_mfma_f32_32x32x2_f32 on register operands
  * and nothing else -- what the matrix pipes sustain at the clocks the device holds under that
  * load, to set beside the nominal peak.  `out` takes 4 * CUs * 256 floats (1024 * 256 on MI355X);
  * *flops receives the launch's FLOP count. */
 int cavs_mfma_probe(float *out, size_t out_floats, int iters, double *flops, void *stream);
-size_t cavs_sgemm_splitk_static_max_bytes(void);
-int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
-                             int lda, const float *B, int ldb, float beta, float *C, int ldc,
-                             void *stream);
 /* Up to four independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
  * (plus one for the K splits): the once-per-step block of
  * cavs/midend/batch_weight_updater.h:12-84 -- the weight-gradient GEMMs -- and the embedding
@@ -155,7 +155,20 @@ typedef struct cavs_gemm_desc {
   int ldb;
   float *C;
   int ldc;
+  /* Optional: a block the caller knows about, so that the tiles it covers can stop early.  The
+   * rows of a batch that belong to leaves come first in every slab, a leaf gathers zero rows
+   * (cavs/backend/op_impl_graphop.cu:77-86) and so its forget gates multiply zero and receive
+   * a zero gradient (apps/paper/tree-lstm-cavs.cc:160-171): the f columns of x*W are unused in
+   * those rows and the f columns of its gradient are exact zeros there.
+   *   CAVS_GEMM_A_ZERO (transA = 0): A[r, k] == 0 for r < zero_rows, k >= zero_col;
+   *   CAVS_GEMM_B_ZERO (transB = 0): B[k, c] == 0 for k < zero_rows, c >= zero_col;
+   *   CAVS_GEMM_C_UNUSED (beta = 0): C[r, c] is not wanted for r < zero_rows, c >= zero_col and
+   *     comes out as the product or as zero.
+   * With the zeros where the caller says, results are those without the hint bit for bit (the
+   * skipped terms are +-0); a hint is a licence, never an obligation.  0: none. */
+  int zero_kind, zero_rows, zero_col;
 } cavs_gemm_desc;
+enum { CAVS_GEMM_C_UNUSED = 1, CAVS_GEMM_A_ZERO = 2, CAVS_GEMM_B_ZERO = 3 };
 size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products);
 int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace,
                      size_t workspace_bytes, void *stream);
@@ -195,10 +208,12 @@ int cavs_embed_pull_fwd(float *out, int ld_out, float *ids_out, const float *x, 
  * The product's A loader reads the table rows through the two lists; the workgroups also leave
  * them in e_out (what the backward pass multiplies by; the column tiles of a row tile share that
  * copying) and the ids in ids_out, exactly as cavs_embed_pull_fwd would.  Results are those of the
- * two calls, bit for bit. */
+ * two calls, bit for bit.  unused_rows, unused_col: C[b, c] with b < unused_rows and
+ * c >= unused_col is not wanted (CAVS_GEMM_C_UNUSED above: the f columns of the leaves) and comes
+ * out as the product or as zero; 0, 0: everything is wanted. */
 int cavs_embed_pull_sgemm(float *C, int ldc, float *e_out, int ld_e, float *ids_out, const float *x,
                           const int *rows, const float *table, int n, int E, const float *B, int ldb,
-                          int N, void *stream);
+                          int N, int unused_rows, int unused_col, void *stream);
 /* out[r, :] = inp[r, :] + bias[:]  (BinaryBroadcastingKernel,
  * cavs/backend/op_impl_elementwise.cuh:128-139; also the ones-vector bias GEMM of
  * cavs/backend/op_impl_fullyconnected_cublas.cc:74-76) */

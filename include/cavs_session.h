@@ -128,7 +128,9 @@ int cavs_session_profile_read(cavs_session *s, const char *kernel_class, double 
 /* Raw stream the session enqueues on (for callers that want to bracket it with events). */
 void *cavs_session_stream(cavs_session *s);
 /* Per-step counts for roofline accounting: rows moved by indexed copies and GEMM flops
- * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" (separate GEMM launches)
+ * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" (separate GEMM launches: 2*M*N*K
+ * of the reference's products) "gemm_flops_hinted" (the part of those that multiplies blocks known
+ * to be zero or unused -- the forget-gate columns of the leaves -- and is skipped tile by tile)
  * "round_flops" (products inside fused round launches) "rounds" "launches"; "plan_hits" /
  * "plan_misses" of the plan cache since the session was created. */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);

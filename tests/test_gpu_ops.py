@@ -293,6 +293,109 @@ def test_sgemm_group_matches_separate_products(g, oracle, name):
             g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes - 256, g.stream())
 
 
+# (the 7331-row case runs as lookup + product on the 128 x 128 tile, the others in one launch)
+@pytest.mark.parametrize("n,E,N,ld_e,urows,ucol", [(2482, 300, 2048, 304, 1260, 1536), (7331, 512, 2048, 512, 3700, 1536),
+                                                   (320, 128, 512, 128, 130, 384), (70, 33, 50, 40, 64, 3), (200, 64, 256, 64, 200, 1)])
+def test_pull_lookup_and_product_with_an_unused_block(g, n, E, N, ld_e, urows, ucol):
+    """cavs_embed_pull_sgemm with rows below `urows` not wanted from column `ucol` on (the forget-gate
+    columns of the leaves): everything else, the looked-up rows and the ids are those of the call
+    without the block, bit for bit; inside the block an element is the product or zero, and the
+    tiles that lie wholly inside it are zero."""
+    V, nx = 211, n + 9
+    r = rng(n + E + 1)
+    x = np.floor(r.bulk_uniform(nx) * V).astype(np.float32)
+    x[::7] = -1.0
+    rows = np.argsort(r.bulk_uniform(nx))[:n].astype(np.int32)
+    table, B = r.bulk_uniform(V * E, -1, 1).reshape(V, E), r.bulk_uniform(E * N, -1, 1).reshape(E, N)
+    d_x, d_rows, d_table, d_B = g.devf(x), g.devi(rows), g.devf(table), g.devf(B)
+    res = []
+    for ur, uc in ((0, 0), (urows, ucol)):
+        e_out, ids_out, Cd = g.devf(np.full((n, ld_e), 9, np.float32)), g.devf(np.full(n, 9, np.float32)), g.devf(np.full((n, N + 4), 9, np.float32))
+        g.call("cavs_embed_pull_sgemm", g.P(Cd), N + 4, g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E,
+               g.P(d_B), N, N, ur, uc, g.stream())
+        res.append((g.host(Cd), g.host(e_out), g.host(ids_out)))
+    (want, e_want, ids_want), (got, e_got, ids_got) = res
+    np.testing.assert_array_equal(e_got, e_want)
+    np.testing.assert_array_equal(ids_got, ids_want)
+    inside = np.zeros_like(want, dtype=bool)
+    inside[:urows, ucol:N] = True
+    np.testing.assert_array_equal(got[~inside], want[~inside])
+    assert np.all((got[inside] == want[inside]) | (got[inside] == 0))
+    # tiles of 128 rows and columns that lie wholly inside the block (whatever tile the plan took)
+    r1, c0 = urows // 128 * 128, -(-ucol // 128) * 128
+    if r1 > 0 and c0 < N:
+        assert not got[:r1, c0:N].any()
+    with pytest.raises(hip.CavsError, match="unused block"):
+        g.call("cavs_embed_pull_sgemm", g.P(Cd), N + 4, g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E,
+               g.P(d_B), N, N, -1, 0, g.stream())
+
+
+HINTED = {
+    # the deferred products of a batch of trees whose first 1260 slab rows are leaves: de = dxW * W^T
+    # and dW = e^T * dxW, the forget-gate columns of dxW zero in the leaves' rows
+    "c3": [(0, 1, 2482, 300, 2048, hip.GEMM_A_ZERO, 1260, 1536), (1, 0, 304, 2048, 2482, hip.GEMM_B_ZERO, 1260, 1536),
+           (1, 0, 512, 1536, 1222, 0, 0, 0)],
+    # large enough for the 128 x 128 tile, each by itself
+    "alone": [(0, 1, 9000, 1024, 2048, hip.GEMM_A_ZERO, 4500, 1536), (1, 0, 1024, 2048, 9000, hip.GEMM_B_ZERO, 4500, 1536)],
+    # hints that do not apply (transposed operand, a first zero k that is no multiple of 4) are ignored
+    "ignored": [(1, 1, 300, 200, 512, hip.GEMM_A_ZERO, 100, 256), (0, 1, 300, 200, 512, hip.GEMM_A_ZERO, 100, 255),
+                (0, 1, 300, 200, 512, hip.GEMM_B_ZERO, 100, 64)],
+}
+
+
+@pytest.mark.parametrize("name", sorted(HINTED))
+def test_sgemm_group_with_known_zero_blocks(g, name):
+    """Products whose descriptor names a zero block of an operand: bit for bit the results of the
+    same products without the hint.  Where the hint applies and the tiles are wholly inside it the
+    block is not read at all -- shown by a second run with NaN there (rows below a multiple of 128,
+    columns from a multiple of 128 on: inside for every tile shape)."""
+    import torch
+
+    shapes = HINTED[name]
+    r = rng(len(name) + 23)
+    n = len(shapes)
+    plain, hinted = (hip.GemmDesc * n)(), (hip.GemmDesc * n)()
+    keep, outs, poison = [], [], []
+    for p, (tA, tB, M, N, K, kind, zr, zc) in enumerate(shapes):
+        A = r.bulk_uniform(M * K, -1, 1).reshape((K, M) if tA else (M, K))
+        B = r.bulk_uniform(N * K, -1, 1).reshape((N, K) if tB else (K, N))
+        applies = (kind == hip.GEMM_A_ZERO and not tA and zc % 4 == 0) or (kind == hip.GEMM_B_ZERO and not tB)
+        Z = A if kind == hip.GEMM_A_ZERO else B
+        if applies:
+            Z[:zr, zc:] = 0.0
+        Ad, Bd = g.devf(A), g.devf(B)
+        keep += [Ad, Bd]
+        plain[p] = hip.GemmDesc(tA, tB, M, N, K, 1.0, 0.0, g.P(Ad), A.shape[1], g.P(Bd), B.shape[1], None, N)
+        hinted[p] = hip.GemmDesc(tA, tB, M, N, K, 1.0, 0.0, g.P(Ad), A.shape[1], g.P(Bd), B.shape[1], None, N, kind, zr, zc)
+        # rows of the block every tile shape skips: A rows in whole 128-row tiles; B rows k below a multiple of 32
+        skip_rows = zr // 128 * 128 if kind == hip.GEMM_A_ZERO else zr // 32 * 32
+        poison.append((Ad if kind == hip.GEMM_A_ZERO else Bd, skip_rows, zc) if applies and zc % 128 == 0 else None)
+    nbytes = hip.lib().cavs_sgemm_group_workspace(n, hinted)
+    assert nbytes == hip.lib().cavs_sgemm_group_workspace(n, plain)
+    ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device="cuda")
+    results = []
+    for descs, nan in ((plain, False), (hinted, False), (hinted, True)):
+        if nan:
+            for q in poison:
+                if q:
+                    q[0][:q[1], q[2]:] = float("nan")
+        outs = []
+        for p, (tA, tB, M, N, K, *_h) in enumerate(shapes):
+            Cd = g.devf(np.full((M, N), 7, np.float32))
+            outs.append(Cd)
+            descs[p].C = g.P(Cd)
+        g.call("cavs_sgemm_group", n, descs, g.P(ws), nbytes, g.stream())
+        results.append([g.host(o) for o in outs])
+    for p in range(n):
+        np.testing.assert_array_equal(results[1][p], results[0][p], err_msg=f"product {p}: hinted vs plain")
+        np.testing.assert_array_equal(results[2][p], results[0][p], err_msg=f"product {p}: the block was read")
+    bad = (hip.GemmDesc * 1)()
+    bad[0] = hinted[0]
+    bad[0].zero_kind = 4
+    with pytest.raises(hip.CavsError, match="block hint"):
+        g.call("cavs_sgemm_group", 1, bad, g.P(ws), nbytes, g.stream())
+
+
 @pytest.mark.parametrize("n,E,N,ld_e", [(2482, 300, 2048, 304), (7331, 512, 2048, 512), (320, 128, 512, 128), (70, 33, 50, 40), (5, 8, 64, 8)])
 def test_pull_lookup_and_product_in_one_launch(g, n, E, N, ld_e):
     """cavs_embed_pull_sgemm against cavs_embed_pull_fwd + cavs_sgemm: the product, the looked-up rows
@@ -310,7 +413,7 @@ def test_pull_lookup_and_product_in_one_launch(g, n, E, N, ld_e):
         e_out, ids_out, Cd = g.devf(np.full((n, ld_e), 9, np.float32)), g.devf(np.full(n, 9, np.float32)), g.devf(np.full((n, N + 4), 9, np.float32))
         if fused:
             g.call("cavs_embed_pull_sgemm", g.P(Cd), N + 4, g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E,
-                   g.P(d_B), N, N, g.stream())
+                   g.P(d_B), N, N, 0, 0, g.stream())
         else:
             g.call("cavs_embed_pull_fwd", g.P(e_out), ld_e, g.P(ids_out), g.P(d_x), g.P(d_rows), g.P(d_table), n, E, g.stream())
             g.call("cavs_sgemm", 0, 0, n, N, E, 1.0, g.P(e_out), ld_e, g.P(d_B), N, 0.0, g.P(Cd), N + 4, g.stream())
