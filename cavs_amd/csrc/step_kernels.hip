@@ -295,6 +295,27 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
         if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = lds.tile[tx][i];
       break;
     }
+    case CAVS_TASK_SGD_TRANSPOSE: {  // p1 -= f0 * p2 (if p2 is given), then p0[c][r] = p1[r][c]
+      float *__restrict__ w = static_cast<float *>(t.p1);
+      const float *__restrict__ g = static_cast<const float *>(t.p2);
+      float *__restrict__ out = static_cast<float *>(t.p0);
+      const int rows = (int)t.n0, cols = (int)t.n1, gx = (cols + 31) / 32;
+      const int c0 = (b % gx) * 32, r0 = (b / gx) * 32, tx = tid & 31, ty = tid >> 5;
+      for (int i = ty; i < 32; i += 8)
+        if (r0 + i < rows && c0 + tx < cols) {
+          const long at = (long)(r0 + i) * cols + c0 + tx;
+          float v = w[at];
+          if (g) {
+            v -= t.f0 * g[at];
+            w[at] = v;
+          }
+          lds.tile[i][tx] = v;
+        }
+      __syncthreads();
+      for (int i = ty; i < 32; i += 8)
+        if (c0 + i < cols && r0 + tx < rows) out[(long)(c0 + i) * rows + r0 + tx] = lds.tile[tx][i];
+      break;
+    }
     case CAVS_TASK_PACK_T: {
       // B = p1^T ([K = n1, N = n0]; p1 is [n0, n1] row-major) in the tile-major layout the round
       // kernels' packed product loops read: for k-group g (16 k) and column tile t (16 columns)
@@ -490,6 +511,12 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
         CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 30) && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad transpose shape", i);
         if (t.n0 == 0 || t.n1 == 0) continue;
         CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1, "cavs_run_tasks: job %d: null or aliased pointer", i);
+        blocks = ((t.n0 + 31) / 32) * ((t.n1 + 31) / 32);
+        break;
+      case CAVS_TASK_SGD_TRANSPOSE:
+        CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 30) && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad transpose shape", i);
+        if (t.n0 == 0 || t.n1 == 0) continue;
+        CAVS_REQUIRE(t.p0 && t.p1 && t.p0 != t.p1 && t.p0 != t.p2, "cavs_run_tasks: job %d: null or aliased pointer", i);
         blocks = ((t.n0 + 31) / 32) * ((t.n1 + 31) / 32);
         break;
       case CAVS_TASK_PACK_T:

@@ -31,6 +31,7 @@ class Task(C.Structure):
 
 TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T, TASK_SGD_PACK = 0, 1, 2, 3, 4, 5, 6, 7
 TASK_TREELSTM_GATES_ROWS = 8
+TASK_SGD_TRANSPOSE = 9
 
 
 class GemmDesc(C.Structure):

@@ -245,6 +245,9 @@ class Engine {
   // since (set_param, a caller's own tensor).
   DeviceArray<float> Upk_;
   bool upk_valid_ = false;
+  DeviceArray<float> WfcT_;  // [H, C] copy of a wide head's weights (head_forward_backward)
+  bool wfct_valid_ = false;
+  bool wide_head() const;
   // rounds of at most this many rows run as fused launches (0: none)
   int fused_rows() const;
 

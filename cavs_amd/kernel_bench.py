@@ -118,9 +118,12 @@ def gemm(iters, st):
             (1, 0, H, 3 * H, N // 2, f"{tag} dU_iou = h_lr^T*d(hU)"),
         ]
     cases += [(0, 0, 32, 1536, 512, "C3 tail round (32 rows)"), (0, 0, 8192, 8192, 8192, "square 8192")]
-    # the 10000-way head of the variable-length LSTM configuration (7331 tokens per batch)
-    cases += [(0, 0, 7331, 10000, 512, "C4 head logits = h*Wc"), (1, 0, 512, 10000, 7331, "C4 head dWc = h^T*dlogits"),
-              (0, 1, 7331, 512, 10000, "C4 head dh = dlogits*Wc^T"), (0, 0, 7331, 2048, 512, "C4 x*W all rows")]
+    # the 10000-way head of the variable-length LSTM configuration (7331 tokens per batch) in the forms the
+    # engine runs: the weights Wc [C, H] are read through their [H, C] copy
+    cases += [(0, 0, 7331, 10000, 512, "C4 head logits = h*WcT"), (1, 0, 10000, 512, 7331, "C4 head dWc = dlogits^T*h"),
+              (0, 1, 7331, 512, 10000, "C4 head dh = dlogits*WcT^T"), (0, 0, 7331, 2048, 512, "C4 x*W all rows"),
+              # (the same two products on Wc itself, as they ran before the copy)
+              (0, 1, 7331, 10000, 512, "C4 head logits = h*Wc^T, on Wc"), (0, 0, 7331, 512, 10000, "C4 head dh = dlogits*Wc, on Wc")]
     # what the matrix pipes sustain with register operands only, in launches of ~1 ms and ~10 ms
     buf = torch.empty(1 << 20, **f32)
     for mf_iters in (4000, 40000):

@@ -489,6 +489,10 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *                        row-major; n0 a multiple of 16, n1 of 64) in the same tile-major layout: the
  *                        parameter update (cavs/backend/op_impl_sgd.cu) and the packed copy the next
  *                        forward pass reads, in one pass over the weights.
+ *   CAVS_TASK_SGD_TRANSPOSE  p1[i] -= f0 * p2[i] (skipped when p2 is null), then p0[c][r] = p1[r][c], n0 rows,
+ *                        n1 columns: the update of a wide classifier's weights [C, H]
+ *                        (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79) and the [H, C] copy the
+ *                        next step's products read, in one pass.
  *   CAVS_TASK_TREELSTM_GATES_ROWS  cavs_treelstm_bwd_gates_rows(rows = p0, n = n0, dret = p1,
  *                        dret_rows = p2, gates = p3, G = p4, dxW = p5, ld_dxw = n2 >> 32, dF = p6,
  *                        dc = p7, leaf_rows = n2 & 0xffffffff, H = n1; H a multiple of 4): the gate
@@ -496,7 +500,7 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  * p4 .. p7 are read by that last kind only and may stay null otherwise. */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
        CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6, CAVS_TASK_SGD_PACK = 7,
-       CAVS_TASK_TREELSTM_GATES_ROWS = 8 };
+       CAVS_TASK_TREELSTM_GATES_ROWS = 8, CAVS_TASK_SGD_TRANSPOSE = 9 };
 typedef struct cavs_task {
   int kind;
   float f0;

@@ -463,6 +463,35 @@ def test_the_packed_copy_of_the_recurrent_weights_follows_every_writer(oracle, m
     s.close()
 
 
+def test_the_transposed_copy_of_a_wide_heads_weights_follows_every_writer(oracle):
+    """A classifier of C * H >= 2^18 weights is multiplied through an [H, C] copy of them.  The copy is
+    written by the update job; set_param writes the weights behind its back.  Three steps -- the
+    first copies on demand, the second reads what the first step's update left, the third follows
+    a set_params -- each against the oracle on the parameters the session should hold."""
+    model, H, V, C_ = "lstm", 64, 37, 4100
+    w = small_workload(model, 77, B=6, H=H, E=H, V=V, C=C_, skew=False)
+    names = ("Emb", "W", "Bv", "Wfc", "bfc")
+    p = {k: np.array(w["params"][k], np.float32) for k in names}
+    s = session.Session(model, H=H, E=H, V=V, C_=C_)
+    s.set_params(p)
+    lr = 0.25
+    for step in range(3):
+        print(f"[case] wide head step {step}", flush=True)
+        if step == 2:
+            p["Wfc"] = (p["Wfc"][::-1] * np.float32(0.5)).astype(np.float32)
+            s.set_params({"Wfc": p["Wfc"]})
+        want = oracle.model_step(model, w["graph"], w["x"], w["labels"], p, H=H, E=H, V=V, Cc=C_, precise=True, threads=16)
+        s.step(w["graph"], w["x"], w["labels"], backward=True, lr=lr)
+        close(s.fetch("loss"), want["loss"], f"loss at step {step}")
+        close(s.fetch("dgraph_out"), want["dgraph_out"], f"dgraph_out at step {step}")
+        got = s.grads()
+        for k in names:
+            close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}")
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    close(s.param("Wfc", p["Wfc"].shape), p["Wfc"], "Wfc after the steps")
+    s.close()
+
+
 @pytest.mark.parametrize("kind", ["trees", "tokens"])
 def test_training_step_on_reader_batches(oracle, kind):
     """The text readers (cavs_amd/data.py) feed the session directly: the fixture corpora

@@ -1213,6 +1213,30 @@ def test_packed_weights_give_the_same_forward_round_bit_for_bit(g, n, H):
         g.call("cavs_run_tasks", 1, (T * 1)(bad), g.stream())
 
 
+@pytest.mark.parametrize("rows,cols", [(10000, 512), (1000, 32), (37, 70), (1, 5), (64, 64)])
+def test_update_and_transposed_copy_in_one_job(g, rows, cols):
+    """CAVS_TASK_SGD_TRANSPOSE: the weights after the job are those of the plain update job bit for
+    bit and the copy is their transpose; without a gradient the job only copies."""
+    r = rng(rows + 3 * cols)
+    W, dW = r.bulk_normal(rows * cols).reshape(rows, cols), r.bulk_normal(rows * cols).reshape(rows, cols)
+    lr = np.float32(0.375)
+    d_W, d_plain, d_dW, WT = g.devf(W), g.devf(W), g.devf(dW), g.zeros(cols, rows, fill=-9.0)
+    T = hip.Task
+    jobs = [T(hip.TASK_SGD_TRANSPOSE, lr, rows, cols, 0, g.P(WT), g.P(d_W), g.P(d_dW), None),
+            T(hip.TASK_SGD, lr, rows * cols, 0, 0, g.P(d_plain), g.P(d_dW), None, None)]
+    g.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), g.stream())
+    W1 = g.host(d_W)
+    np.testing.assert_array_equal(W1, g.host(d_plain))
+    close(W1, W.astype(np.float64) - float(lr) * dW.astype(np.float64), "updated weights")
+    np.testing.assert_array_equal(g.host(WT), W1.T)
+    again = g.zeros(cols, rows, fill=-9.0)
+    g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_SGD_TRANSPOSE, lr, rows, cols, 0, g.P(again), g.P(d_W), None, None)), g.stream())
+    np.testing.assert_array_equal(g.host(again), W1.T)
+    np.testing.assert_array_equal(g.host(d_W), W1)
+    with pytest.raises(hip.CavsError, match="aliased"):
+        g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_SGD_TRANSPOSE, lr, rows, cols, 0, g.P(d_W), g.P(d_W), None, None)), g.stream())
+
+
 @pytest.mark.parametrize("L,m,n,H", [(300, 90, 100, 256), (200, 30, 40, 512), (500, 128, 128, 512), (1500, 500, 600, 256)])
 def test_packed_weights_give_the_same_chain_lstm_rounds_bit_for_bit(g, L, m, n, H):
     """Chain LSTM: the forward launch and the folded backward launch reading W' / W'^T tile-major
@@ -1451,7 +1475,7 @@ def test_several_small_jobs_in_one_launch(g):
     with pytest.raises(hip.CavsError, match="not a permutation"):
         g.call("cavs_run_tasks", 1, (T * 1)(T(hip.TASK_BLOCKS_SGD, 0.5, bw, 4, 0, g.P(d_wb), g.P(d_src), g.P(d_gb), None)), g.stream())
     with pytest.raises(hip.CavsError, match="unknown kind"):
-        g.call("cavs_run_tasks", 1, (T * 1)(T(9, 0.0, 1, 1, 0, g.P(dA), g.P(dB), None, None)), g.stream())
+        g.call("cavs_run_tasks", 1, (T * 1)(T(99, 0.0, 1, 1, 0, g.P(dA), g.P(dB), None, None)), g.stream())
     with pytest.raises(hip.CavsError, match="at most 12"):
         g.call("cavs_run_tasks", 13, (T * 13)(), g.stream())
 
