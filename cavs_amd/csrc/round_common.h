@@ -60,6 +60,28 @@ __device__ inline float sigm_r(float x) { return __builtin_amdgcn_rcpf(1.f + exp
 __device__ inline float tanh_r(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + exp_r(2.f * x)); }
 
 
+// The gates of one hidden unit of one vertex (apps/paper/tree-lstm-cavs.cc:132-171): xw = the unit's
+// four columns of x * W ([i|o|u|f]), v = its five recurrent pre-activations (i, o, u, f_l, f_r),
+// bias = its four bias entries in the bias's own block order ([i|f|u|o]), c_left / c_right = the
+// children's c.  One function for every kernel that finishes a forward round, so that they all
+// evaluate the same expressions in the same association: (x * W + h * U) + bias.
+struct TreeLstmCell {
+  float i, o, u, f_l, f_r, tc, h, c;
+};
+__device__ inline TreeLstmCell treelstm_cell(const float (&xw)[4], const float (&v)[5], const float (&bias)[4], float c_left,
+                                             float c_right) {
+  TreeLstmCell q;
+  q.i = sigm_r((xw[0] + v[0]) + bias[0]);
+  q.o = sigm_r((xw[1] + v[1]) + bias[3]);
+  q.u = tanh_r((xw[2] + v[2]) + bias[2]);
+  q.f_l = sigm_r((xw[3] + v[3]) + bias[1]);
+  q.f_r = sigm_r((xw[3] + v[4]) + bias[1]);
+  q.c = (q.i * q.u + q.f_l * c_left) + q.f_r * c_right;
+  q.tc = tanh_r(q.c);
+  q.h = q.o * q.tc;
+  return q;
+}
+
 // Gate gradients of one hidden unit of one vertex.  mh, mc: gradient of the vertex's message
 // ([h|c] halves); dr: gradient of its pushed return value; c_left, c_right: the children's c
 // (zero for a leaf).

@@ -349,15 +349,8 @@ __global__ __launch_bounds__(WAVES * 64, (TILE == 16 && WAVES == 4) ? 4 : 1) voi
       v[p] = s;
     }
     const int b = ep.b, j = ep.j;
-    // same association as the separate gate kernel: (x*W + h*U) + bias
-    const float i = sigm_r((ep.xw[0] + v[0]) + ep.bias[0]);
-    const float o = sigm_r((ep.xw[1] + v[1]) + ep.bias[3]);
-    const float u = tanh_r((ep.xw[2] + v[2]) + ep.bias[2]);
-    const float f_l = sigm_r((ep.xw[3] + v[3]) + ep.bias[1]);
-    const float f_r = sigm_r((ep.xw[3] + v[4]) + ep.bias[1]);
-    const float c = (i * u + f_l * ep.cl) + f_r * ep.cr;
-    const float tc = tanh_r(c);
-    const float h = o * tc;
+    const TreeLstmCell q_ = treelstm_cell(ep.xw, v, ep.bias, ep.cl, ep.cr);
+    const float i = q_.i, o = q_.o, u = q_.u, f_l = q_.f_l, f_r = q_.f_r, c = q_.c, tc = q_.tc, h = q_.h;
     float *g = a.gates + (long)b * 6 * H + j;
     g[0] = i; g[H] = o; g[2 * H] = u; g[3 * H] = f_l; g[4 * H] = f_r; g[5 * H] = tc;
     if (a.msg) {

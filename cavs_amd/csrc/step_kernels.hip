@@ -269,6 +269,7 @@ struct TaskList {
   cavs_task t[kMaxTasks];
   int first[kMaxTasks + 1];
   int count;
+  const int *guard;  // CAVS_TASK_GUARD: when the word it points at is not zero, no job of the launch runs
 };
 
 __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
@@ -278,6 +279,7 @@ __global__ __launch_bounds__(256) void tasks_kernel(TaskList L) {
     EmbedSgdLds sgd;
     float sums[4][64];
   } lds;
+  if (L.guard && __hip_atomic_load(L.guard, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
   int k = 0;
   while (k + 1 < L.count && (int)blockIdx.x >= L.first[k + 1]) k++;
   const cavs_task &t = L.t[k];
@@ -499,13 +501,18 @@ int cavs_fc_softmax_xent(const float *X, const float *W, const float *b, const f
 }
 
 int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
-  CAVS_REQUIRE(count >= 0 && count <= kMaxTasks, "cavs_run_tasks: %d jobs, at most %d", count, kMaxTasks);
+  CAVS_REQUIRE(count >= 0 && count <= kMaxTasks + 1, "cavs_run_tasks: %d jobs, at most %d and a guard", count, kMaxTasks);
   CAVS_REQUIRE(count == 0 || tasks, "cavs_run_tasks: null list");
   TaskList L{};
   int k = 0;
   for (int i = 0; i < count; i++) {
     const cavs_task &t = tasks[i];
     long blocks = 0;
+    if (t.kind == CAVS_TASK_GUARD) {
+      CAVS_REQUIRE(t.p0 && !L.guard, "cavs_run_tasks: job %d: a guard needs a word to watch, and a launch takes one guard", i);
+      L.guard = static_cast<const int *>(t.p0);
+      continue;
+    }
     switch (t.kind) {
       case CAVS_TASK_TRANSPOSE:
         CAVS_REQUIRE(t.n0 >= 0 && t.n1 >= 0 && t.n0 < (1 << 30) && t.n1 < (1 << 30), "cavs_run_tasks: job %d: bad transpose shape", i);
@@ -588,6 +595,7 @@ int cavs_run_tasks(int count, const cavs_task *tasks, void *stream) {
       default:
         CAVS_REQUIRE(false, "cavs_run_tasks: job %d: unknown kind %d", i, t.kind);
     }
+    CAVS_REQUIRE(k < kMaxTasks, "cavs_run_tasks: more than %d jobs", kMaxTasks);
     CAVS_REQUIRE(blocks > 0 && L.first[k] + blocks < (1L << 30), "cavs_run_tasks: job %d: too many workgroups", i);
     L.t[k] = t;
     L.first[k + 1] = L.first[k] + (int)blocks;

@@ -32,6 +32,7 @@ class Task(C.Structure):
 TASK_TRANSPOSE, TASK_ZERO_ROWS, TASK_SGD, TASK_EMBED_SGD, TASK_SUM_PARTS, TASK_BLOCKS_SGD, TASK_PACK_T, TASK_SGD_PACK = 0, 1, 2, 3, 4, 5, 6, 7
 TASK_TREELSTM_GATES_ROWS = 8
 TASK_SGD_TRANSPOSE = 9
+TASK_GUARD = 10
 
 
 class GemmDesc(C.Structure):
@@ -103,6 +104,9 @@ _SIGS = {
     "cavs_treelstm_round_bwd_children_gates": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_treelstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children_gates_packed": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "cavs_tail_probe": [_P, _I, _I, _P],
+    "cavs_treelstm_tail_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _I, _P],
+    "cavs_treelstm_tail_bwd": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _P, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd_packed": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
@@ -136,6 +140,7 @@ _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_s
             "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
             "cavs_clip_grads_workspace": _Z, "cavs_sgemm_group_workspace": _Z, "cavs_fc_softmax_xent_parts": _I,
             "cavs_colsum_parts": _I, "cavs_round_packed_ok": _I, "cavs_lstm_round_packed_ok": _I,
+            "cavs_tail_rounds_ok": _I, "cavs_tail_max_rounds": _I, "cavs_tail_max_groups": _I, "cavs_tail_sync_bytes": _Z,
             "cavs_sgemm_splitk_static_max_bytes": _Z,
             "cavs_schedule_arena_scratch": _Z}
 _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_workspace": [_I, _I, _I],
@@ -143,6 +148,7 @@ _NOCHECK = {"cavs_last_error": [], "cavs_abi_version": [], "cavs_sgemm_splitk_wo
             "cavs_clip_grads_workspace": [_I], "cavs_sgemm_group_workspace": [_I, C.POINTER(GemmDesc)],
             "cavs_fc_softmax_xent_parts": [_I], "cavs_colsum_parts": [_I], "cavs_round_packed_ok": [_I, _I],
             "cavs_lstm_round_packed_ok": [_I, _I], "cavs_sgemm_splitk_static_max_bytes": [],
+            "cavs_tail_rounds_ok": [_I, _I], "cavs_tail_max_rounds": [], "cavs_tail_max_groups": [], "cavs_tail_sync_bytes": [],
             "cavs_schedule_arena_scratch": [_I, _I]}
 
 EW_BINARY = dict(add=0, sub=1, mul=2, div=3, sigmoid_grad=4, tanh_grad=5, relu_grad=6, equal=7)

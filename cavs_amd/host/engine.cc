@@ -15,6 +15,8 @@
 namespace cavs {
 
 namespace {
+// polls of a tail launch's bounded wait (a poll is a round trip to the L2 and a short sleep: ~1 us)
+constexpr int kTailSpins = 1 << 19;
 inline size_t grow(size_t need, size_t have) {
   if (need <= have) return have;
   size_t g = have + have / 4;
@@ -63,6 +65,146 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
     add_param("Wfc", (size_t)cfg.C * H);
     add_param("bfc", cfg.C);
   }
+  tail_setup();
+}
+
+// ------------------------------------------------------------------ the rounds near the roots in one launch
+// Whether this device runs the workgroups of such a launch all at once on one XCD is asked once,
+// with the barrier alone (cavs_tail_probe); a device that does not keeps to one launch per round.
+void Engine::tail_setup() {
+  tail_ready_ = false;
+  if (cfg_.model != CAVS_MODEL_TREELSTM || !(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.tail_rows < 0) return;
+  if (!cavs_tail_rounds_ok(1, cfg_.H)) return;
+  const size_t words = cavs_tail_sync_bytes() / sizeof(int);
+  tail_sync_.reserve(words);
+  check(cavs_zero(tail_sync_.get(), words * sizeof(int), stream_));
+  check(cavs_tail_probe(reinterpret_cast<unsigned *>(tail_sync_.get()), cfg_.H, kTailSpins, stream_));
+  int head[4] = {0, 0, 0, 0};
+  check(cavs_memcpy_d2h(head, tail_sync_.get(), sizeof(head), stream_));
+  check(cavs_stream_sync(stream_));
+  tail_ready_ = head[1] == 0;
+  if (!tail_ready_) check(cavs_zero(tail_sync_.get(), words * sizeof(int), stream_));
+}
+
+int Engine::tail_limit() const {
+  if (!tail_ready_ || fused_rows() <= 0) return 0;
+  const int most = 32;
+  return cfg_.tail_rows > 0 ? std::min(cfg_.tail_rows, most) : most;
+}
+
+// Which rounds run inside the tail launches, and who runs which row.  The rounds are a suffix of the
+// forward order (a prefix of the backward order).  Inside it the message flow is a forest over slab
+// rows (kid_rows: the rows whose messages a row consumes); a tree of that forest goes to one group
+// as a whole, so nothing a group reads is written by another during the launch.  Trees are dealt
+// heaviest first to the group with the fewest rows so far; the suffix starts at the earliest round
+// from which no group gets more rows of a round than a launch takes.
+void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
+  tail_ = TailPlan();
+  const int lim = tail_limit();
+  const Schedule &s = *sched_;
+  const int R = (int)s.rounds.size(), N = s.N, G = cavs_tail_max_groups(), cap = cavs_tail_max_rounds();
+  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || Upk_.capacity() == 0) return;
+  int k0 = 1;
+  while (k0 < R && (s.rounds[k0].n > G * lim || leaf_round(s.rounds[k0]))) k0++;
+  std::vector<int> comp, weight, group, order, per;
+  for (; R - k0 >= 2; k0++) {
+    bool ok = true;
+    for (int k = k0; k < R && ok; k++) ok = !leaf_round(s.rounds[k]) && cavs_tail_rounds_ok(std::min(s.rounds[k].n, lim), cfg_.H);
+    if (!ok) continue;
+    const int lo = s.rounds[k0].offset;
+    comp.assign(N - lo, -1);
+    weight.clear();
+    for (int v = N - 1; v >= lo; v--) {  // a row's consumer sits in a later round: parents come first
+      if (comp[v - lo] < 0) {
+        comp[v - lo] = (int)weight.size();
+        weight.push_back(0);
+      }
+      weight[comp[v - lo]]++;
+      for (int i = 0; i < 2; i++) {
+        const int c = kid_rows[2 * (size_t)v + i];
+        if (c >= lo) comp[c - lo] = comp[v - lo];
+      }
+    }
+    order.resize(weight.size());
+    for (size_t i = 0; i < order.size(); i++) order[i] = (int)i;
+    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return weight[a] > weight[b]; });
+    group.assign(weight.size(), 0);
+    int load[16] = {0};
+    for (int c : order) {
+      int best = 0;
+      for (int g = 1; g < G; g++)
+        if (load[g] < load[best]) best = g;
+      group[c] = best;
+      load[best] += weight[c];
+    }
+    // rows of round k that group g runs
+    const int nr = R - k0;
+    per.assign((size_t)G * nr, 0);
+    for (int k = k0; k < R; k++)
+      for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) per[(size_t)group[comp[b - lo]] * nr + (k - k0)]++;
+    int lists = 0;
+    for (int g = 0; g < G && ok; g++) {
+      int mine = 0;
+      for (int k = 0; k < nr; k++) {
+        if (per[(size_t)g * nr + k] > lim) ok = false;
+        mine += per[(size_t)g * nr + k] > 0;
+      }
+      if (mine > cap) ok = false;
+      lists = std::max(lists, mine);
+    }
+    if (!ok) continue;
+    // the lists: per group, round by round
+    TailPlan &t = tail_;
+    t.first = k0;
+    t.max_rounds = std::max(lists, 1);
+    t.nrounds.assign(G, 0);
+    t.start.assign((size_t)G * t.max_rounds, 0);
+    t.count.assign((size_t)G * t.max_rounds, 0);
+    std::vector<int> at((size_t)G * nr, -1);
+    size_t fill = 0;
+    for (int g = 0; g < G; g++)
+      for (int k = 0; k < nr; k++) {
+        const int c = per[(size_t)g * nr + k];
+        if (c == 0) continue;
+        const int i = t.nrounds[g]++;
+        t.start[(size_t)g * t.max_rounds + i] = (int)fill;
+        t.count[(size_t)g * t.max_rounds + i] = c;
+        at[(size_t)g * nr + k] = (int)fill;
+        fill += c;
+      }
+    for (int k = k0; k < R; k++)
+      for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) rows_out[at[(size_t)group[comp[b - lo]] * nr + (k - k0)]++] = b;
+    t.rows = fill;
+    t.bstart = t.start;
+    t.bcount = t.count;
+    for (int g = 0; g < G; g++) {
+      std::reverse(t.bstart.begin() + (size_t)g * t.max_rounds, t.bstart.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
+      std::reverse(t.bcount.begin() + (size_t)g * t.max_rounds, t.bcount.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
+    }
+    t.vertices = (double)fill;
+    t.flops = 2.0 * fill * cfg_.H * 5.0 * cfg_.H;
+    return;
+  }
+}
+
+void Engine::tail_check() {
+  if (!tail_pending_) return;
+  tail_pending_ = false;
+  int words[4] = {0, 0, 0, 0};
+  check(cavs_memcpy_d2h(words, tail_sync_.get(), sizeof(words), stream_));
+  check(cavs_stream_sync(stream_));
+  if (words[1] == 0) return;
+  // every launch since the one that gave up left at once, and every parameter update watched the
+  // word: the parameters are those of the last good step.  From here on: one launch per round.
+  tail_ready_ = false;
+  upk_valid_ = wfct_valid_ = false;
+  emb_sparse_valid_ = false;
+  check(cavs_zero(tail_sync_.get(), cavs_tail_sync_bytes(), stream_));
+  fail(CAVS_EHIP, std::string("a launch over the rounds near the roots gave up (") +
+                      (words[1] == CAVS_TAIL_TIMEOUT ? "its workgroups were not all resident within the wait's bound"
+                                                     : "its workgroups did not share one XCD") +
+                      "): the results of the steps since the last synchronisation are undefined and their parameter updates were "
+                      "skipped; the session continues with one launch per round");
 }
 
 Engine::~Engine() {
@@ -354,7 +496,8 @@ void Engine::upload_index_arena() {
   const Schedule &s = *sched_;
   const int N = N_;
   const bool want_forest = !cfg_.split_backward_rounds && fused_rows() > 0;
-  const size_t total = (size_t)N * (2 + nch_) + s.B + (want_forest ? (size_t)N * (nch_ + 1) : 0);
+  const bool want_tail = want_forest && tail_limit() > 0;
+  const size_t total = (size_t)N * (2 + nch_) + s.B + (want_forest ? (size_t)N * (nch_ + 1) : 0) + (want_tail ? (size_t)N : 0);
   // Two sets of buffers (pinned staging + device lists) alternate, and the copy runs on a stream
   // of its own: the lists of step k + 1 are built and uploaded while the kernels of step k run,
   // instead of the copy sitting in the compute stream between two steps.  A set is rewritten only
@@ -376,6 +519,9 @@ void Engine::upload_index_arena() {
   std::string err = build_index_lists(s, nch_, cfg_.pairing, t2j, pair, child, roots);
   if (!err.empty()) fail(CAVS_EUNSUPPORTED, err);
   forest_ = want_forest && build_forest_lists(s, nch_, fused_rows(), pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N, &n_orphans_);
+  tail_ = TailPlan();
+  int *tail_rows = roots + s.B + (size_t)N * (nch_ + 1);
+  if (want_tail && forest_) build_tail_plan(roots + s.B, tail_rows);
   check(cavs_memcpy_h2d(h.dev.get(), h.host.get(), total * sizeof(int), sched_stream_));
   check(cavs_event_record(h.up_ev, sched_stream_));
   check(cavs_event_sync(h.up_ev));  // a few microseconds; the compute stream is still busy with the previous step
@@ -387,6 +533,7 @@ void Engine::upload_index_arena() {
   d_roots_ = d_child_ + (size_t)nch_ * N;
   d_kid_rows_ = want_forest ? d_roots_ + s.B : nullptr;
   d_orphans_ = want_forest ? d_kid_rows_ + (size_t)nch_ * N : nullptr;
+  d_tail_rows_ = want_tail ? d_orphans_ + N : nullptr;
 }
 
 // ------------------------------------------------------------------ step
@@ -439,7 +586,8 @@ void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
   p->n_orphans = n_orphans_;
   p->forest = forest_;
   p->last_used = ++plan_clock_;
-  p->lists.reserve(2 * N + 2 * nk + B + N);
+  p->tail = tail_;
+  p->lists.reserve(2 * N + 2 * nk + B + N + N);
   int *base = p->lists.get();
   const bool kids = d_kid_rows_ != nullptr;
   check(cavs_memcpy_d2d(base, d_t2j_, N * 4, stream_));
@@ -450,6 +598,7 @@ void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
     check(cavs_memcpy_d2d(base + 2 * N + nk + B, d_kid_rows_, nk * 4, stream_));
     check(cavs_memcpy_d2d(base + 2 * N + 2 * nk + B, d_orphans_, (size_t)n_orphans_ * 4, stream_));
   }
+  if (tail_.first >= 0) check(cavs_memcpy_d2d(base + 3 * N + 2 * nk + B, d_tail_rows_, tail_.rows * 4, stream_));
   // this step reads the copy as well, so that the buffers the lists were built in are free again
   d_t2j_ = base;
   d_pair_ = base + N;
@@ -457,6 +606,7 @@ void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
   d_roots_ = base + 2 * N + nk;
   d_kid_rows_ = kids ? base + 2 * N + nk + B : nullptr;
   d_orphans_ = kids ? base + 2 * N + 2 * nk + B : nullptr;
+  d_tail_rows_ = base + 3 * N + 2 * nk + B;
   plans_.push_back(std::move(p));
 }
 
@@ -595,6 +745,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
   }
   c_gather_rows_ = c_scatter_rows_ = c_gemm_flops_ = c_gemm_flops_hinted_ = c_launches_ = c_gather_bytes_ = c_scatter_bytes_ = 0;
   c_round_flops_ = 0;
+  c_tail_rounds_ = c_tail_launches_ = 0;
   bias_jobs_.clear();
   wait_ms_ = 0.f;
   uint64_t hash = 0;
@@ -621,8 +772,11 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     d_roots_ = base + 2 * N + nk;
     d_kid_rows_ = base + 2 * N + nk + B;
     d_orphans_ = base + 2 * N + 2 * nk + B;
+    d_tail_rows_ = base + 3 * N + 2 * nk + B;
+    tail_ = (forest_ && tail_limit() > 0) ? hit->tail : TailPlan();
     sched_ms_ = 0.f;
   } else {
+    tail_ = TailPlan();  // (the host-built lists bring a new one)
     const bool on_device = cfg_.schedule_mode == 1 && (cfg_.opt & CAVS_OPT_BATCHING) && maxlen <= 2048;
     if (on_device) schedule_on_device(graph, B, maxlen); else schedule_on_host(graph, B, maxlen);
     if (cfg_.plan_cache > 0) {
@@ -732,6 +886,7 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       // only: every other row of its gradient is zero, so the dense update would not move it
       // all of it in one launch: the updates touch disjoint tensors
       std::vector<cavs_task> tasks;
+      if (update_guard()) tasks.push_back({CAVS_TASK_GUARD, 0.f, 0, 0, 0, const_cast<int *>(update_guard()), nullptr, nullptr, nullptr});
       std::vector<std::string> by_job;
       for (const BiasJob &j : bias_jobs_) by_job.push_back(j.param);
       settle_bias_jobs(lr, &tasks);
@@ -816,7 +971,25 @@ void Engine::treelstm_forward() {
   // when every round runs fused, Push + FunctionPopRet ride along in the rounds' epilogues
   out_folded_ = fused > 0 && sched_->max_round <= fused && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
-  for (const Round &r : sched_->rounds) {
+  // the last rounds, a few vertices each: one launch for all of them
+  const size_t tail_from = (tail_.first >= 0 && any_packed) ? (size_t)tail_.first : sched_->rounds.size();
+  for (size_t rk = 0; rk < sched_->rounds.size(); rk++) {
+    const Round &r = sched_->rounds[rk];
+    if (rk == tail_from) {
+      CAVS_TIMED(K_ROUND, cavs_treelstm_tail_fwd(pool_.get(), d_child_, d_pair_, xW_.get(), 4 * H, Upk_.get(), Bv, G_.get(), hlr_.get(),
+                                                 gates_.get(), out_folded_ ? nullptr : msg_.get(), go, d_t2j_, d_tail_rows_,
+                                                 (int)tail_.nrounds.size(), tail_.nrounds.data(), tail_.start.data(), tail_.count.data(),
+                                                 tail_.max_rounds, H, reinterpret_cast<unsigned *>(tail_sync_.get()), kTailSpins, 0,
+                                                 stream_));
+      c_round_flops_ += tail_.flops;
+      c_gather_rows_ += 2.0 * tail_.vertices;
+      c_scatter_rows_ += tail_.vertices;
+      c_launches_ += 1;
+      c_tail_launches_ += 1;
+      c_tail_rounds_ += (double)(sched_->rounds.size() - tail_from);
+      tail_pending_ = true;
+      break;
+    }
     const size_t off = r.offset;
     // the message slab is only read back by FunctionPopRet; when the rounds write the output
     // rows themselves nobody reads it and the fused launches skip it
@@ -898,7 +1071,28 @@ void Engine::treelstm_backward() {
                                                      dF_.get(), dc_.get(), sched_->leaf_prefix, H, stream_));
     c_launches_ += 1;
   }
-  for (int k : sched_->bwd_rounds) {
+  // the first rounds of the backward pass, a few vertices each: one launch for all of them
+  size_t tail_n = 0;
+  if (folded && packed && tail_.first >= 0) {
+    tail_n = sched_->rounds.size() - (size_t)tail_.first;
+    // (the backward order is the forward order reversed: the launches' rounds are its first tail_n)
+    if (sched_->bwd_rounds.size() < tail_n || sched_->bwd_rounds[tail_n - 1] != tail_.first) tail_n = 0;
+  }
+  if (tail_n > 0) {
+    CAVS_TIMED(K_ROUND, cavs_treelstm_tail_bwd(dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_, gates_.get(), G_.get(), d_dgo_,
+                                               d_t2j_, sched_->leaf_prefix, d_tail_rows_, (int)tail_.nrounds.size(), tail_.nrounds.data(),
+                                               tail_.bstart.data(), tail_.bcount.data(), tail_.max_rounds, H,
+                                               reinterpret_cast<unsigned *>(tail_sync_.get()), kTailSpins, 0, stream_));
+    c_gather_rows_ += tail_.vertices;
+    c_round_flops_ += tail_.flops;
+    c_scatter_rows_ += 2.0 * tail_.vertices;
+    c_launches_ += 1;
+    c_tail_launches_ += 1;
+    c_tail_rounds_ += (double)tail_n;
+    tail_pending_ = true;
+  }
+  for (size_t bi = tail_n; bi < sched_->bwd_rounds.size(); bi++) {
+    const int k = sched_->bwd_rounds[bi];
     const Round &r = sched_->rounds[k];
     const size_t off = r.offset;
     if (folded) {
@@ -1424,7 +1618,10 @@ void Engine::head_forward_backward(bool backward) {
   }
 }
 
-void Engine::sync() { check(cavs_stream_sync(stream_)); }
+void Engine::sync() {
+  check(cavs_stream_sync(stream_));
+  tail_check();
+}
 
 void Engine::fetch(const std::string &what, float *host, size_t n) {
   const size_t N = N_, H = cfg_.H;
@@ -1449,6 +1646,7 @@ void Engine::fetch(const std::string &what, float *host, size_t n) {
   if (n != want || !host) fail(CAVS_EINVAL, "'" + what + "' holds " + std::to_string(want) + " floats, got " + std::to_string(n));
   check(cavs_memcpy_d2h(host, src, want * 4, stream_));
   check(cavs_stream_sync(stream_));
+  tail_check();
 }
 
 float Engine::timing(const std::string &name) {
@@ -1480,6 +1678,9 @@ double Engine::counter(const std::string &key) const {
   if (key == "round_flops") return c_round_flops_;
   if (key == "launches") return c_launches_;
   if (key == "rounds") return (double)sched_->rounds.size();
+  if (key == "tail_rounds") return c_tail_rounds_;
+  if (key == "tail_launches") return c_tail_launches_;
+  if (key == "tail_ready") return tail_ready_ ? 1.0 : 0.0;
   if (key == "plan_hits") return c_plan_hits_;
   if (key == "plan_misses") return c_plan_misses_;
   fail(CAVS_EINVAL, "unknown counter '" + key + "'");

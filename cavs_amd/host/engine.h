@@ -178,6 +178,18 @@ class Engine {
   void schedule_on_host(const int *graph, int B, int maxlen);
   void point_lists(const int *base, long cap);
 
+  // ---- the rounds near the roots as one launch per direction (cavs_treelstm_tail_fwd / _bwd)
+  // What those launches run, for one batch structure: the rounds from `first` on, their rows dealt
+  // to the groups by whole trees of the message flow (no message crosses groups).
+  struct TailPlan {
+    int first = -1;  // first round (forward order) inside the launches; -1: none
+    int max_rounds = 0;
+    std::vector<int> nrounds, start, count;      // per group; lists in forward order
+    std::vector<int> bstart, bcount;             // the same lists in backward order
+    size_t rows = 0;                             // length of the device list of slab rows
+    double flops = 0, vertices = 0;
+  };
+
   // ---- plan cache (cfg.plan_cache entries): the schedule and the device lists of a graph feed,
   // keyed by the feed's bytes, so that a batch structure seen before costs neither the scheduler
   // nor an upload
@@ -190,6 +202,7 @@ class Engine {
     DeviceArray<int> lists;  // [t2j | pair | child | roots | kid_rows | orphans], N rows each
     int n_orphans = 0;
     bool forest = false;
+    TailPlan tail;
     uint64_t last_used = 0;
   };
   std::vector<std::unique_ptr<Plan>> plans_;
@@ -250,6 +263,27 @@ class Engine {
   bool wide_head() const;
   // rounds of at most this many rows run as fused launches (0: none)
   int fused_rows() const;
+
+  // (the tail launches, continued)
+  TailPlan tail_;
+  const int *d_tail_rows_ = nullptr;
+  DeviceArray<int> tail_sync_;  // the launches' sync block
+  bool tail_ready_ = false;     // the device ran the probe's workgroups all at once, each group on one XCD
+  bool tail_pending_ = false;   // a tail launch was enqueued since the status word was last read
+  double c_tail_rounds_ = 0, c_tail_launches_ = 0;
+  int tail_limit() const;       // rows per group and round a tail launch may take (0: no tail launches)
+  void tail_setup();
+  // fills tail_ and writes the groups' row lists to `rows_out` (room for N ints) from the host copy of
+  // the children-by-slab-row lists of a batch whose message flow is a forest
+  void build_tail_plan(const int *kid_rows, int *rows_out);
+ public:
+  // After the stream has drained: reads the status word of the tail launches.  A launch that gave
+  // up leaves the results of the steps since undefined (their parameter updates were skipped: they
+  // watch the word); the session goes on with one launch per round and this call fails.
+  void tail_check();
+  // the word a parameter-update launch must watch (CAVS_TASK_GUARD), or null
+  const int *update_guard() const { return tail_ready_ ? tail_sync_.get() + 1 : nullptr; }
+ private:
 
   // counters of the last step
   double c_round_flops_ = 0;

@@ -841,6 +841,10 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     // every variable's update in one launch (they touch disjoint tensors)
     std::vector<cavs_task> updates;
     std::vector<const float *> by_bias_job;
+    // (the lowered F's launches over the rounds near the roots can give up: no update runs then)
+    const int *guard = engine_ ? engine_->update_guard() : nullptr;
+    const cavs_task guard_task{CAVS_TASK_GUARD, 0.f, 0, 0, 0, const_cast<int *>(guard), nullptr, nullptr, nullptr};
+    if (guard) updates.push_back(guard_task);
     if (engine_ && defer_bias_) engine_->update_bias_jobs(g.opt.lr, &updates, &by_bias_job);
     for (auto &v : g.opt.vars) {
       Tensor &w = tensor(v), &gr = tensor(GetGradientName(v));
@@ -848,6 +852,7 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       if (updates.size() + 2 > 12) {
         check(cavs_run_tasks((int)updates.size(), updates.data(), stream_));
         updates.clear();
+        if (guard) updates.push_back(guard_task);
       }
       // the lowered F reads its recurrent weights from a packed copy that the update keeps current
       if (engine_ && engine_->update_jobs(w.base, gr.base, g.opt.lr, &updates)) continue;
@@ -879,6 +884,7 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     (*results)[i] = h;
   }
   check(cavs_stream_sync(stream_));
+  if (engine_) engine_->tail_check();
 }
 
 long Executor::read_tensor(const std::string &name, float *out, size_t cap) {
@@ -890,6 +896,7 @@ long Executor::read_tensor(const std::string &name, float *out, size_t cap) {
   if (!out || cap < n) return -(long)n;
   check(cavs_memcpy_d2h(out, t->base, n * 4, stream_));
   check(cavs_stream_sync(stream_));
+  if (engine_) engine_->tail_check();
   return (long)n;
 }
 

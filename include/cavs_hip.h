@@ -365,6 +365,53 @@ int cavs_treelstm_round_fwd_packed(float *pool, const int *child, const int *pai
 int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW, int ld_xw,
                                    const float *bias, float *gates, float *msg, float *graph_out,
                                    const int *out_rows, int n, int H, void *stream);
+/* ------------------------------------------------------------------ the rounds near the roots in one launch
+ * The per-round loop of GraphStatement::Run / GraphGradStatement::Run (cavs/midend/statement.cc:
+ * 69-76,106-111) for rounds of a few vertices each, as ONE launch per direction.  The caller deals
+ * the rows of those rounds to up to 8 groups such that no message passes between groups (whole
+ * trees of the batch's message flow per group); a group is run by the H / 16 workgroups of one XCD,
+ * which stay resident, keep their share of the recurrent weights in registers and walk the group's
+ * rounds behind a barrier of their own (arrival counter and results in that XCD's L2; no L2
+ * write-back or invalidate; groups never wait for each other).  Same arithmetic in the same order
+ * as cavs_treelstm_round_fwd_packed / cavs_treelstm_round_bwd_children_gates_packed called once
+ * per round: results equal bit for bit.
+ *   rows (device): the groups' lists of slab rows.  Group g runs nrounds[g] lists one after the
+ *   other, list i = rows[start[g * max_rounds + i] .. + count[g * max_rounds + i]), 1..32 rows each
+ *   (nrounds, start, count: host arrays).  What a list's rows read must have been written before
+ *   the launch or by earlier lists of the same group.
+ *   Every other array is the whole-batch array the per-round entry points take slices of (child
+ *   [2N], pair [N], out_rows [N], xW [N,4H], G [2N,2H], hlr [N,H], gates [N,6H], msg [N,2H] or NULL;
+ *   backward: dxW [N,4H], dF [2N,H], dc [N,H], child_rows [2N]).
+ *   sync: cavs_tail_sync_bytes() of device memory, zero before the first launch; a launch that
+ *   completes leaves it zero.  Word 1 is the status: 0, CAVS_TAIL_TIMEOUT (a wait gave up after
+ *   spin_max polls: a group's workgroups were not all resident at once) or CAVS_TAIL_SPREAD (they
+ *   did not share one XCD).  With a non-zero status every wave has left the kernel, the results of
+ *   the launch are undefined, and the caller must clear the block before the next launch.
+ *   Launches on one block must not overlap.  extra_arrivals > 0 makes every wait expect that many
+ *   more arrivals than there are workgroups: the way to see the give-up path from a test.
+ * For H = 512 (cavs_tail_rounds_ok); at most cavs_tail_max_rounds() lists per group. */
+enum { CAVS_TAIL_OK = 0, CAVS_TAIL_TIMEOUT = 1, CAVS_TAIL_SPREAD = 2 };
+int cavs_tail_rounds_ok(int n, int H);
+int cavs_tail_max_rounds(void);
+int cavs_tail_max_groups(void);
+size_t cavs_tail_sync_bytes(void);
+/* Three barriers of the same workgroups with the same footprint and nothing else: tells (through
+ * the status word, after the stream has drained) whether this device runs every group's
+ * workgroups all at once on one XCD. */
+int cavs_tail_probe(unsigned *sync, int H, int spin_max, void *stream);
+int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw,
+                           const float *Upk, const float *bias, float *G, float *hlr, float *gates,
+                           float *msg, float *graph_out, const int *out_rows, const int *rows,
+                           int ngroups, const int *nrounds, const int *start, const int *count,
+                           int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
+                           void *stream);
+int cavs_treelstm_tail_bwd(float *dxW, int ld_dxw, float *dF, float *dc, const float *UTp,
+                           const int *child_rows, const float *gates, const float *G,
+                           const float *dret, const int *dret_rows, int leaf_rows, const int *rows,
+                           int ngroups, const int *nrounds, const int *start, const int *count,
+                           int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
+                           void *stream);
+
 /* Backward of the gates of a round.  The message gradient of slab row b is read from
  * dpool row pair[b] (grad of Scatter is Gather on the same list, zero for -1); the c
  * half of the children's message gradients is written to dpool rows child[2b], child[2b+1]
@@ -497,10 +544,14 @@ int cavs_transpose(float *out, const float *in, int rows, int cols, void *stream
  *                        dret_rows = p2, gates = p3, G = p4, dxW = p5, ld_dxw = n2 >> 32, dF = p6,
  *                        dc = p7, leaf_rows = n2 & 0xffffffff, H = n1; H a multiple of 4): the gate
  *                        gradients of the roots ride in the launch that opens the backward pass.
- * p4 .. p7 are read by that last kind only and may stay null otherwise. */
+ *   CAVS_TASK_GUARD      not a job: when the int p0 points at is not zero as the launch runs, none of
+ *                        its jobs does anything (the parameter updates of a step whose
+ *                        cavs_treelstm_tail_* launch gave up: p0 = the status word of its sync block).
+ *                        At most one per launch; it does not count towards the 12.
+ * p4 .. p7 are read by CAVS_TASK_TREELSTM_GATES_ROWS only and may stay null otherwise. */
 enum { CAVS_TASK_TRANSPOSE = 0, CAVS_TASK_ZERO_ROWS = 1, CAVS_TASK_SGD = 2, CAVS_TASK_EMBED_SGD = 3,
        CAVS_TASK_SUM_PARTS = 4, CAVS_TASK_BLOCKS_SGD = 5, CAVS_TASK_PACK_T = 6, CAVS_TASK_SGD_PACK = 7,
-       CAVS_TASK_TREELSTM_GATES_ROWS = 8, CAVS_TASK_SGD_TRANSPOSE = 9 };
+       CAVS_TASK_TREELSTM_GATES_ROWS = 8, CAVS_TASK_SGD_TRANSPOSE = 9, CAVS_TASK_GUARD = 10 };
 typedef struct cavs_task {
   int kind;
   float f0;

@@ -61,6 +61,13 @@ typedef struct {
    * graph feeds, keyed by the feed's bytes; a step on a feed seen before skips the scheduler and
    * the upload.  0 = off. */
   int plan_cache;
+  /* Tree-LSTM, H = 512, batches whose message flow is a forest: the consecutive rounds of at most
+   * this many vertices nearest the roots (the last forward rounds, the first backward rounds) run
+   * as one launch per direction (cavs_treelstm_tail_fwd / _bwd) instead of one launch per round
+   * (cavs/midend/statement.cc:69-76,106-111).  0 = default (32, the most those launches take),
+   * negative = never.  The session checks once, when it is created, that the device runs such a
+   * launch's workgroups all at once on one XCD, and keeps to one launch per round if not. */
+  int tail_rows;
 } cavs_session_config;
 
 const char *cavs_session_error(void);
@@ -131,8 +138,10 @@ void *cavs_session_stream(cavs_session *s);
  * of the last step. keys: "gather_rows" "scatter_rows" "gemm_flops" (separate GEMM launches: 2*M*N*K
  * of the reference's products) "gemm_flops_hinted" (the part of those that multiplies blocks known
  * to be zero or unused -- the forget-gate columns of the leaves -- and is skipped tile by tile)
- * "round_flops" (products inside fused round launches) "rounds" "launches"; "plan_hits" /
- * "plan_misses" of the plan cache since the session was created. */
+ * "round_flops" (products inside fused round launches) "rounds" "launches"; "tail_rounds" (rounds,
+ * forward and backward, that ran inside cavs_treelstm_tail_* launches) "tail_launches"; "plan_hits" /
+ * "plan_misses" of the plan cache since the session was created; "tail_ready" (1 when the session may
+ * use the tail launches). */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);
 
 #ifdef __cplusplus

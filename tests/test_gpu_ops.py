@@ -1477,7 +1477,9 @@ def test_several_small_jobs_in_one_launch(g):
     with pytest.raises(hip.CavsError, match="unknown kind"):
         g.call("cavs_run_tasks", 1, (T * 1)(T(99, 0.0, 1, 1, 0, g.P(dA), g.P(dB), None, None)), g.stream())
     with pytest.raises(hip.CavsError, match="at most 12"):
-        g.call("cavs_run_tasks", 13, (T * 13)(), g.stream())
+        g.call("cavs_run_tasks", 14, (T * 14)(), g.stream())
+    with pytest.raises(hip.CavsError, match="more than 12 jobs"):
+        g.call("cavs_run_tasks", 13, (T * 13)(*[T(hip.TASK_SGD, 0.5, 4, 0, 0, g.P(dA), g.P(dB), None, None)] * 13), g.stream())
 
 
 @pytest.mark.parametrize("n,bw,perm", [(1, 4, [0]), (2482, 512, [0, 3, 2, 1]), (63, 6, [2, 0, 1]), (5000, 64, [1, 0])])
