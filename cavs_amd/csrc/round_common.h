@@ -55,9 +55,15 @@ __device__ inline float elem(const float4 &v, int c) { return c == 0 ? v.x : c =
 // tanhf, of which a thread's epilogue has six).  Saturation comes out right without special
 // cases: exp overflows to inf, whose reciprocal is 0, and underflows to 0.  tanh_r is accurate to
 // 1e-7 absolute; near zero that is a large relative error of a tiny number.
+// (No multiply-add contraction in these and in the gate functions below: whether the compiler
+// fuses a product into a following sum depends on the code around it, and kernels that inline the
+// same function must produce the same bits.)
 __device__ inline float exp_r(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
 __device__ inline float sigm_r(float x) { return __builtin_amdgcn_rcpf(1.f + exp_r(-x)); }
-__device__ inline float tanh_r(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + exp_r(2.f * x)); }
+__device__ inline float tanh_r(float x) {
+#pragma clang fp contract(off)
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + exp_r(2.f * x));
+}
 
 
 // The gates of one hidden unit of one vertex (apps/paper/tree-lstm-cavs.cc:132-171): xw = the unit's
@@ -70,6 +76,7 @@ struct TreeLstmCell {
 };
 __device__ inline TreeLstmCell treelstm_cell(const float (&xw)[4], const float (&v)[5], const float (&bias)[4], float c_left,
                                              float c_right) {
+#pragma clang fp contract(off)
   TreeLstmCell q;
   q.i = sigm_r((xw[0] + v[0]) + bias[0]);
   q.o = sigm_r((xw[1] + v[1]) + bias[3]);
@@ -90,6 +97,7 @@ struct GateGrad {
 };
 __device__ inline GateGrad gate_grad(float i, float o, float u, float f_l, float f_r, float tc, float mh, float mc, float dr,
                                      float c_left, float c_right) {
+#pragma clang fp contract(off)
   GateGrad g;
   const float dh = mh + dr;
   const float d_o = dh * tc;

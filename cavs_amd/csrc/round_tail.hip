@@ -76,7 +76,6 @@ __device__ inline bool tail_wait(unsigned *status, unsigned *gsync, unsigned tar
         bail = 1;
         break;
       }
-      __builtin_amdgcn_s_sleep(1);
     }
     if (!bail && check_xcc) {
       const unsigned seen = __hip_atomic_load(gsync + TAIL_XCC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -228,6 +227,9 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       pf += gate4;
     }
   }
+  // Wavefronts w and w + 4 share a SIMD and would run their MFMA and vector-ALU phases in step,
+  // each at half speed with the matrix pipe idle in between: one of them goes first.
+  if (ks < 4) __builtin_amdgcn_s_setprio(2);
   // the element of a tile this thread finishes: wavefront ks does tile ks, row lane / 16, column x
   const int ej = j0 + x;
   float bias[4];
@@ -264,19 +266,6 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       __syncthreads();
     }
 
-    // operand rows: one float4 per child and tile (see CAVS_MMA4)
-    float4 al[8], ar[8];
-    const int ka = kb + 16 * ((lane >> 2) & 3) + 4 * slot;
-#pragma unroll
-    for (int t = 0; t < 8; t++) {
-      al[t] = ar[t] = zero4();
-      if (t < T) {
-        const int ra = 4 * t + (lane & 3);
-        const int cl = s_child[par][2 * ra], cr = s_child[par][2 * ra + 1];
-        if (cl >= 0) al[t] = ld4(a.pool + (long)cl * H2 + ka);
-        if (cr >= 0) ar[t] = ld4(a.pool + (long)cr * H2 + ka);
-      }
-    }
     // the epilogue's children
     int e_cl = -1, e_cr = -1, e_dst = -1, e_out = -1;
     float e_hl = 0.f, e_cl_c = 0.f, e_hr = 0.f, e_cr_c = 0.f;
@@ -289,13 +278,24 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       if (e_cr >= 0) { e_hr = ld_row(a.pool + (long)e_cr * H2 + ej); e_cr_c = ld_row(a.pool + (long)e_cr * H2 + H + ej); }
     }
 
-#pragma unroll
-    for (int t = 0; t < 8; t++) {
-      if (t >= T) break;
+    // Operand rows: one float4 per child and tile (see CAVS_MMA4).  The loads of a tile are issued
+    // while the tile before it multiplies, unconditionally (a missing child reads row 0 and is masked
+    // where the operand is used; past the last tile the last one is fetched again), so that the wait
+    // before a tile's MFMAs counts exactly the two loads behind it.
+    const int ka = kb + 16 * ((lane >> 2) & 3) + 4 * slot;
+    auto fetch = [&](int t, float4 &l, float4 &rr, int &cl, int &cr) {
+      const int ra = 4 * (t < T ? t : T - 1) + (lane & 3);
+      cl = s_child[par][2 * ra];
+      cr = s_child[par][2 * ra + 1];
+      l = ld4(a.pool + (long)(cl >= 0 ? cl : 0) * H2 + ka);
+      rr = ld4(a.pool + (long)(cr >= 0 ? cr : 0) * H2 + ka);
+    };
+    auto tile = [&](int t, float4 hl4, float4 hr4, int cl, int cr) {
+      if (cl < 0) hl4 = zero4();
+      if (cr < 0) hr4 = zero4();
       floatx4 acc[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const float4 hl4 = al[t], hr4 = ar[t];
       const float4 hs4 = make_float4(hl4.x + hr4.x, hl4.y + hr4.y, hl4.z + hr4.z, hl4.w + hr4.w);
       // (k-group g, step c: k = 16 g + 4 slot + c; the five products take turns as in the per-round kernels)
 #define CAVS_FWD_STEP(g, comp)                    \
@@ -313,9 +313,25 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       sum_slots_rows<NP>(acc);
 #pragma unroll
       for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = acc[p][0];
+    };
+    {
+      float4 la, ra4, lb, rb4;
+      int cla, cra, clb, crb;
+      fetch(0, la, ra4, cla, cra);
+      for (int t = 0; t < T; t += 2) {
+        fetch(t + 1, lb, rb4, clb, crb);
+        __builtin_amdgcn_sched_barrier(0);
+        tile(t, la, ra4, cla, cra);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(t + 2, la, ra4, cla, cra);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < T) tile(t + 1, lb, rb4, clb, crb);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     __syncthreads();
 
+    TreeLstmCell q{};
     if (eon) {
       const float *pre = red + (ks * 8 * (NP * 4) + (lane >> 4)) * 16 + x;  // tile ks, wavefront 0, row lane / 16
       float v[NP];
@@ -326,7 +342,15 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
         for (int g = 0; g < 8; g++) s += pre[(g * NP * 4 + p * 4) * 16];
         v[p] = s;
       }
-      const TreeLstmCell q = treelstm_cell(xw, v, bias, e_cl_c, e_cr_c);
+      q = treelstm_cell(xw, v, bias, e_cl_c, e_cr_c);
+      // the message first: it is all a later round of this launch reads
+      if (e_dst >= 0) {
+        a.pool[(long)e_dst * H2 + ej] = q.h;
+        a.pool[(long)e_dst * H2 + H + ej] = q.c;
+      }
+    }
+    tail_arrive(gsync, total);
+    if (eon) {  // what the backward pass and the caller read: on its way while the next round starts
       const long b = erow;
       float *g = a.gates + b * 6 * H + ej;
       g[0] = q.i; g[H] = q.o; g[2 * H] = q.u; g[3 * H] = q.f_l; g[4 * H] = q.f_r; g[5 * H] = q.tc;
@@ -334,16 +358,11 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
         float *m = a.msg + b * H2 + ej;
         m[0] = q.h; m[H] = q.c;
       }
-      if (e_dst >= 0) {
-        a.pool[(long)e_dst * H2 + ej] = q.h;
-        a.pool[(long)e_dst * H2 + H + ej] = q.c;
-      }
       if (e_out >= 0) a.go[(long)e_out * H + ej] = q.h;
       float *gl = a.G + (2 * b) * H2 + ej, *gr = gl + H2;
       gl[0] = e_hl; gl[H] = e_cl_c; gr[0] = e_hr; gr[H] = e_cr_c;
       a.hlr[b * H + ej] = e_hl + e_hr;
     }
-    tail_arrive(gsync, total);
   }
 }
 
@@ -389,6 +408,7 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
     for (int g = 0; g < 4; g++) w1[g] = p1[(long)g * gstep4];
   }
   const int ej = j0 + x;
+  if (ks < 4) __builtin_amdgcn_s_setprio(2);  // (see the forward kernel)
   if (tid == 0 && nrounds > 1) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   const unsigned total = (unsigned)nrounds * a.expect;
 
@@ -438,57 +458,61 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
     }
     const float pdc = eon ? ld_row(a.dc + erow * H + ej) : 0.f;
 
-    // four tiles at a time; per tile five float4 per lane (see CAVS_MMA4): three of [d_i|d_o|d_u]
-    // (K = 3H: twelve k-groups per wavefront), one each of d_fl, d_fr (K = H)
+    // Per tile five float4 per lane (see CAVS_MMA4): three of [d_i|d_o|d_u] (K = 3H: twelve k-groups
+    // per wavefront), one each of d_fl, d_fr (K = H); a tile's are issued while the tile before it
+    // multiplies (past the last tile the last one is fetched again), so the wait before a tile's
+    // MFMAs counts exactly the five loads behind it.
     const int kq = 16 * ((lane >> 2) & 3) + 4 * slot;
+    struct Opnd {
+      float4 x[3], fl, fr;
+    };
+    auto fetch = [&](int t, Opnd &o) {
+      const long row = s_row[par][4 * (t < T ? t : T - 1) + (lane & 3)];
+      const float *px = a.dxW + row * a.ld_dxw + ks * (3 * H / 8) + kq;
 #pragma unroll
-    for (int t0 = 0; t0 < 8; t0 += 4) {
-      if (t0 >= T) break;
-      float4 ax[4][3], afl[4], afr[4];
+      for (int q = 0; q < 3; q++) o.x[q] = ld4(px + 64 * q);
+      const float *pl = a.dF + 2 * row * H + ks * (H / 8) + kq;
+      o.fl = ld4(pl);
+      o.fr = ld4(pl + H);
+    };
+    auto tile = [&](int t, const Opnd &o) {
+      floatx4 acc[NP];
 #pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const int t = t0 + u;
-#pragma unroll
-        for (int q = 0; q < 3; q++) ax[u][q] = zero4();
-        afl[u] = afr[u] = zero4();
-        if (t < T) {
-          const long row = s_row[par][4 * t + (lane & 3)];
-          const float *px = a.dxW + row * a.ld_dxw + ks * (3 * H / 8) + kq;
-#pragma unroll
-          for (int q = 0; q < 3; q++) ax[u][q] = ld4(px + 64 * q);
-          const float *pl = a.dF + 2 * row * H + ks * (H / 8) + kq;
-          afl[u] = ld4(pl);
-          afr[u] = ld4(pl + H);
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < 4; u++) {
-        const int t = t0 + u;
-        if (t >= T) break;
-        floatx4 acc[NP];
-#pragma unroll
-        for (int p = 0; p < NP; p++) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
-        // (k-group 4 q + g of the K = 3H product: component by component of ax[u][q], broadcast from block g)
-#define CAVS_P0_GROUP(q, g)                                \
-        CAVS_MMA4(acc[0], ax[u][q].x, w0[4 * q + g].x, g); \
-        CAVS_MMA4(acc[0], ax[u][q].y, w0[4 * q + g].y, g); \
-        CAVS_MMA4(acc[0], ax[u][q].z, w0[4 * q + g].z, g); \
-        CAVS_MMA4(acc[0], ax[u][q].w, w0[4 * q + g].w, g);
+      for (int p = 0; p < NP; p++) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
+      // (k-group 4 q + g of the K = 3H product: component by component of o.x[q], broadcast from block g)
+#define CAVS_P0_GROUP(q, g)                           \
+      CAVS_MMA4(acc[0], o.x[q].x, w0[4 * q + g].x, g); \
+      CAVS_MMA4(acc[0], o.x[q].y, w0[4 * q + g].y, g); \
+      CAVS_MMA4(acc[0], o.x[q].z, w0[4 * q + g].z, g); \
+      CAVS_MMA4(acc[0], o.x[q].w, w0[4 * q + g].w, g);
 #define CAVS_P0_LOAD(q) CAVS_P0_GROUP(q, 0) CAVS_P0_GROUP(q, 1) CAVS_P0_GROUP(q, 2) CAVS_P0_GROUP(q, 3)
-        CAVS_P0_LOAD(0) CAVS_P0_LOAD(1) CAVS_P0_LOAD(2)
+      CAVS_P0_LOAD(0) CAVS_P0_LOAD(1) CAVS_P0_LOAD(2)
 #undef CAVS_P0_LOAD
 #undef CAVS_P0_GROUP
-#define CAVS_P12_STEP(g, comp)                         \
-        CAVS_MMA4(acc[1], afl[u].comp, w1[g].comp, g); \
-        CAVS_MMA4(acc[2], afr[u].comp, w1[g].comp, g);
+#define CAVS_P12_STEP(g, comp)                    \
+      CAVS_MMA4(acc[1], o.fl.comp, w1[g].comp, g); \
+      CAVS_MMA4(acc[2], o.fr.comp, w1[g].comp, g);
 #define CAVS_P12_GROUP(g) CAVS_P12_STEP(g, x) CAVS_P12_STEP(g, y) CAVS_P12_STEP(g, z) CAVS_P12_STEP(g, w)
-        CAVS_P12_GROUP(0) CAVS_P12_GROUP(1) CAVS_P12_GROUP(2) CAVS_P12_GROUP(3)
+      CAVS_P12_GROUP(0) CAVS_P12_GROUP(1) CAVS_P12_GROUP(2) CAVS_P12_GROUP(3)
 #undef CAVS_P12_GROUP
 #undef CAVS_P12_STEP
-        float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
-        sum_slots_rows<NP>(acc);
+      float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
+      sum_slots_rows<NP>(acc);
 #pragma unroll
-        for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = acc[p][0];
+      for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = acc[p][0];
+    };
+    {
+      Opnd oa, ob;
+      fetch(0, oa);
+      for (int t = 0; t < T; t += 2) {
+        fetch(t + 1, ob);
+        __builtin_amdgcn_sched_barrier(0);
+        tile(t, oa);
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(t + 2, oa);
+        __builtin_amdgcn_sched_barrier(0);
+        if (t + 1 < T) tile(t + 1, ob);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
     __syncthreads();

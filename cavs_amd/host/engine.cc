@@ -181,6 +181,12 @@ void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
       std::reverse(t.bstart.begin() + (size_t)g * t.max_rounds, t.bstart.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
       std::reverse(t.bcount.begin() + (size_t)g * t.max_rounds, t.bcount.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
     }
+    for (int g = 0; g < G; g++) {
+      int tiles = 0;
+      for (int i = 0; i < t.nrounds[g]; i++) tiles += (t.count[(size_t)g * t.max_rounds + i] + 3) / 4;
+      t.tiles_max = std::max(t.tiles_max, tiles);
+      t.lists_max = std::max(t.lists_max, t.nrounds[g]);
+    }
     t.vertices = (double)fill;
     t.flops = 2.0 * fill * cfg_.H * 5.0 * cfg_.H;
     return;
@@ -1681,6 +1687,10 @@ double Engine::counter(const std::string &key) const {
   if (key == "tail_rounds") return c_tail_rounds_;
   if (key == "tail_launches") return c_tail_launches_;
   if (key == "tail_ready") return tail_ready_ ? 1.0 : 0.0;
+  if (key == "tail_first_round") return (double)tail_.first;
+  if (key == "tail_lists_max") return (double)tail_.lists_max;
+  if (key == "tail_tiles_max") return (double)tail_.tiles_max;
+  if (key == "tail_vertices") return tail_.vertices;
   if (key == "plan_hits") return c_plan_hits_;
   if (key == "plan_misses") return c_plan_misses_;
   fail(CAVS_EINVAL, "unknown counter '" + key + "'");

@@ -188,6 +188,7 @@ class Engine {
     std::vector<int> bstart, bcount;             // the same lists in backward order
     size_t rows = 0;                             // length of the device list of slab rows
     double flops = 0, vertices = 0;
+    int lists_max = 0, tiles_max = 0;            // the longest group: its lists, its tiles of four rows
   };
 
   // ---- plan cache (cfg.plan_cache entries): the schedule and the device lists of a graph feed,

@@ -141,7 +141,8 @@ void *cavs_session_stream(cavs_session *s);
  * "round_flops" (products inside fused round launches) "rounds" "launches"; "tail_rounds" (rounds,
  * forward and backward, that ran inside cavs_treelstm_tail_* launches) "tail_launches"; "plan_hits" /
  * "plan_misses" of the plan cache since the session was created; "tail_ready" (1 when the session may
- * use the tail launches). */
+ * use the tail launches); the last step's tail plan: "tail_first_round" (-1: none), "tail_vertices",
+ * and of its longest group "tail_lists_max" (rounds) and "tail_tiles_max" (tiles of four rows). */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);
 
 #ifdef __cplusplus
