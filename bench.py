@@ -271,7 +271,8 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
                      kernel="sgemm_mfma_kernel / sgemm_skinny_kernel (x*W, weight-gradient and head GEMMs of a step"
                             "; also the recurrent products of rounds too large for the fused kernels)"),
         "round": dict(ms=round_ms, n=round_n, flops=rflops,
-                      kernel={"treelstm": "treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel",
+                      kernel={"treelstm": "treelstm_round_fwd_kernel / treelstm_round_bwd_children_kernel / treelstm_tail_fwd_kernel / "
+                                          "treelstm_tail_bwd_kernel (the rounds near the roots: one launch per direction)",
                               "lstm": "lstm_round_fwd_kernel / round_bwd_children_kernel",
                               "treefc": "treefc_round_fwd_kernel / round_bwd_children_kernel"}[w0["model"]] +
                              " (one launch per round: gather + recurrent products + gates + scatter)"),
@@ -392,9 +393,15 @@ def main():
             if name == a.workload:
                 continue
             big = name == "C5"
-            also, _ = measure(a, name, 20 if big else 100, 5 if big else 50, 2 if big else 4)
+            steps, warm, npool = (20, 5, 2) if big else (100, 50, 4)
+            also, _ = measure(a, name, steps, warm, npool)
             out["also"][name] = {k: also[k] for k in ("value", "unit", "steps", "warmup", "ms_per_step", "median_ms_per_step",
                                                       "config", "roofline", "kernels")}
+            if not a.no_schedule_modes:  # the same steps with the lists built on the GPU
+                dev, _ = measure(a, name, steps, warm, npool, schedule="device", profile=False)
+                out["also"][name]["schedule_modes"] = {
+                    "host": {k: also[k] for k in ("value", "ms_per_step", "median_ms_per_step")},
+                    "device": {k: dev[k] for k in ("value", "ms_per_step", "median_ms_per_step", "GraphParsing_ms")}}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
     print(json.dumps(out))

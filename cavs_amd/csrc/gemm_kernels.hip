@@ -16,6 +16,9 @@
 #include <algorithm>
 #include <type_traits>
 
+#include <atomic>
+
+#include "bench_probes.h"
 #include "common.h"
 #include "embed_common.h"
 
@@ -988,20 +991,21 @@ constexpr int kStaticScratchDevices = 64;
 static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
 // Device address of `scratch` on each GPU (the array's name is only a host-side stand-in for the
 // symbol; kernels, fills and copies take the address looked up here).
-static float *g_scratch_ptr[kStaticScratchDevices] = {};
+static std::atomic<float *> g_scratch_ptr[kStaticScratchDevices];
 
-// Looks the address up for the current device, once.
+// Looks the address up for the current device, once (two threads that both find it missing look
+// it up twice and store the same value).
 int static_scratch_setup(float **out) {
   int dev = 0;
   CAVS_HIP_TRY(hipGetDevice(&dev));
   CAVS_REQUIRE(dev >= 0 && dev < kStaticScratchDevices, "static scratch: device %d out of range", dev);
-  if (!g_scratch_ptr[dev]) {
-    float *ptr = nullptr;
+  float *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
     CAVS_HIP_TRY(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
     CAVS_REQUIRE(ptr && aligned16(ptr), "static scratch: no usable address on device %d", dev);
-    g_scratch_ptr[dev] = ptr;
+    g_scratch_ptr[dev].store(ptr, std::memory_order_release);
   }
-  if (out) *out = g_scratch_ptr[dev];
+  if (out) *out = ptr;
   return CAVS_OK;
 }
 

@@ -79,8 +79,10 @@ int cavs_init(int device) {
   CAVS_HIP_TRY(hipSetDevice(device));
   g_cus = 0;
   num_cus();
-  // the entry point that allocates nothing finds its scratch here, with this device current
-  return static_scratch_setup(nullptr);
+  // The entry point that allocates nothing finds its scratch here, with this device current.  A
+  // device on which the lookup fails keeps everything else: that entry point reports it.
+  (void)static_scratch_setup(nullptr);
+  return CAVS_OK;
 }
 
 int cavs_device_name(char *buf, size_t len) {

@@ -75,7 +75,6 @@ _SIGS = {
     "cavs_sgemm": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "cavs_sgemm_addrows": [_I, _I, _I, _I, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _Z, _P],
     "cavs_sgemm_group": [_I, C.POINTER(GemmDesc), _P, _Z, _P],
-    "cavs_mfma_probe": [_P, _Z, _I, C.POINTER(C.c_double), _P],
     "cavs_sgemm_group_embed_bwd": [_I, C.POINTER(GemmDesc), _I, _P, _P, _P, _Z, _P],
     "cavs_sgemm_splitk": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _Z, _P],
     "cavs_sgemm_splitk_static": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
@@ -136,6 +135,8 @@ _SIGS = {
     "cavs_schedule_frontier": [_P, _I, _P, _P, _P, _P, _P, _P, _P],
     "cavs_schedule_arena": [_P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, C.c_long, _P, _P, _Z, _P],
 }
+# measurement aids of cavs_amd.kernel_bench (cavs_amd/csrc/bench_probes.h): exported, not part of include/cavs_hip.h
+_BENCH_SIGS = {"cavs_mfma_probe": [_P, _Z, _I, C.POINTER(C.c_double), _P]}
 _RESTYPE = {"cavs_last_error": C.c_char_p, "cavs_abi_version": _I, "cavs_sgemm_splitk_workspace": _Z,
             "cavs_fc_softmax_xent_workspace": _Z, "cavs_colsum_blocks_workspace": _Z,
             "cavs_clip_grads_workspace": _Z, "cavs_sgemm_group_workspace": _Z, "cavs_fc_softmax_xent_parts": _I,
@@ -175,7 +176,7 @@ def lib():
         except ImportError:
             pass
         l = C.CDLL(LIB_PATH)
-        for name, args in _SIGS.items():
+        for name, args in list(_SIGS.items()) + list(_BENCH_SIGS.items()):
             fn = getattr(l, name)
             fn.argtypes, fn.restype = args, _I
         for name, args in _NOCHECK.items():

@@ -1,4 +1,5 @@
 // extern "C" surface of the host runtime (cavs_session.h): exceptions end here.
+#include <vector>
 #include <cstdio>
 #include <cstring>
 #include <string>
@@ -140,6 +141,45 @@ int cavs_schedule_trace_from_lists(int B, int maxlen, int N, int nchild, const i
     g_error = "bad arguments";
     return 0;
   }
+  // the lists index each other: nothing out of range may reach the rebuilding code
+  if (nchild < 1 || nchild > 2 || maxlen <= 0) {
+    g_error = "bad arguments: 1 or 2 children per vertex, positive maxlen";
+    return 0;
+  }
+  if (round2offset[0] != 0 || round2offset[R] != N) {
+    g_error = "round offsets must start at 0 and end at N";
+    return 0;
+  }
+  for (int r = 0; r < R; r++)
+    if (round2offset[r + 1] < round2offset[r]) {
+      g_error = "round offsets must not decrease";
+      return 0;
+    }
+  {
+    std::vector<char> seen((size_t)N, 0);
+    for (int t = 0; t < N; t++) {
+      if (t2j[t] < 0 || t2j[t] >= N || seen[t2j[t]]) {
+        g_error = "t2j is not a permutation of the vertex ids";
+        return 0;
+      }
+      seen[t2j[t]] = 1;
+    }
+  }
+  for (int i = 0; i < B; i++)
+    if (roots[i] < 0 || roots[i] >= N || (i > 0 && roots[i] <= roots[i - 1])) {
+      g_error = "roots must be increasing vertex ids below N";
+      return 0;
+    }
+  for (size_t i = 0; i < (size_t)nchild * N; i++)
+    if (child[i] >= N) {
+      g_error = "a child list names a row beyond N";
+      return 0;
+    }
+  for (int t = 0; t < N; t++)
+    if (pair[t] >= N) {
+      g_error = "the scatter list names a row beyond N";
+      return 0;
+    }
   cavs::Schedule sch;
   cavs::schedule_from_lists(B, maxlen, N, nchild, round2offset, R, t2j, pair, child, roots, &sch);
   return emit(sch.trace(with_backward != 0), out, cap);

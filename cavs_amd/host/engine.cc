@@ -753,6 +753,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
   c_round_flops_ = 0;
   c_tail_rounds_ = c_tail_launches_ = 0;
   bias_jobs_.clear();
+  pending_tasks_.clear();  // (a step that failed half way may have left a job for a backward pass that never ran)
   wait_ms_ = 0.f;
   uint64_t hash = 0;
   Plan *hit = nullptr;
@@ -764,6 +765,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     // a batch structure seen before: its schedule and its lists are where the last such step left them
     hit->last_used = ++plan_clock_;
     c_plan_hits_ += 1;
+    scheduler_used_ = 2;
     sched_ = hit->sched;
     sched_lists_on_host_ = hit->lists_on_host;
     N_ = sched_->N;
@@ -783,8 +785,13 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     sched_ms_ = 0.f;
   } else {
     tail_ = TailPlan();  // (the host-built lists bring a new one)
-    const bool on_device = cfg_.schedule_mode == 1 && (cfg_.opt & CAVS_OPT_BATCHING) && maxlen <= 2048;
+    const bool on_device = cfg_.schedule_mode == 1 && (cfg_.opt & CAVS_OPT_BATCHING);
+    // (one wavefront per sample with its parent row in LDS: a limit of the kernels, and the caller's to know)
+    if (on_device && maxlen > 2048)
+      fail(CAVS_EUNSUPPORTED, "the device scheduler takes samples of at most 2048 vertices (maxlen = " + std::to_string(maxlen) +
+                                  "); use schedule_mode 0, the host scheduler");
     if (on_device) schedule_on_device(graph, B, maxlen); else schedule_on_host(graph, B, maxlen);
+    scheduler_used_ = on_device ? 1 : 0;
     if (cfg_.plan_cache > 0) {
       c_plan_misses_ += 1;
       remember_plan(graph, B, maxlen, hash);
@@ -1551,7 +1558,10 @@ void Engine::head_forward_backward(bool backward) {
     const size_t head_bytes = cavs_fc_softmax_xent_workspace(N, H, C);
     if (head_bytes > 0) {  // few classes: the whole head and its gradients in one launch; the sum of
                            // its weight-gradient partials rides in the launch that opens backward
-      if (head_parts_.capacity() * 4 < head_bytes) head_parts_.reserve(head_bytes / 4 + 1);
+      if (head_parts_.capacity() * 4 < head_bytes) {
+        check(cavs_stream_sync(stream_));  // the last step's jobs may still read the old buffer
+        head_parts_.reserve(head_bytes / 4 + 1);
+      }
       check(cavs_fc_softmax_xent(GO_.get(), Wfc.w, bfc.w, d_labels_, loss_.get(), logits_.get(), backward ? dGO_.get() : nullptr,
                                  nullptr, nullptr, head_parts_.get(), head_bytes, N, H, C, stream_));
       if (backward)
@@ -1686,6 +1696,7 @@ double Engine::counter(const std::string &key) const {
   if (key == "rounds") return (double)sched_->rounds.size();
   if (key == "tail_rounds") return c_tail_rounds_;
   if (key == "tail_launches") return c_tail_launches_;
+  if (key == "scheduler") return (double)scheduler_used_;
   if (key == "tail_ready") return tail_ready_ ? 1.0 : 0.0;
   if (key == "tail_first_round") return (double)tail_.first;
   if (key == "tail_lists_max") return (double)tail_.lists_max;

@@ -209,6 +209,7 @@ class Engine {
   std::vector<std::unique_ptr<Plan>> plans_;
   uint64_t plan_clock_ = 0;
   double c_plan_hits_ = 0, c_plan_misses_ = 0;
+  int scheduler_used_ = 0;  // who produced the last step's lists: 0 host scheduler, 1 device scheduler, 2 plan cache
   Plan *find_plan(const int *graph, int B, int maxlen, uint64_t hash);
   void remember_plan(const int *graph, int B, int maxlen, uint64_t hash);
 

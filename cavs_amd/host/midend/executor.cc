@@ -733,6 +733,13 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
       }
       FeedStage &st = feed_stages_[f.first];
       const size_t bytes = (size_t)t.width * 4;
+      // A placeholder the Run before this one did not feed still points at this set's buffer, and
+      // that Run's kernels may be reading it: wait for them too (the usual case, a placeholder fed
+      // by every Run, alternates between the sets and needs no such wait).
+      if (t.base && t.base == st.dev[parity].get() && run_busy_[parity ^ 1]) {
+        check(cavs_event_sync(run_done_ev_[parity ^ 1]));
+        run_busy_[parity ^ 1] = false;
+      }
       st.slot[parity].reserve(bytes);
       st.dev[parity].reserve(t.width);
       t.base = st.dev[parity].get();
@@ -753,7 +760,7 @@ void Executor::run(const std::vector<std::string> &outputs, std::vector<HostTens
     ~MarkRunDone() {
       if (on && cavs_event_record(e->run_done_ev_[parity], e->stream_) == CAVS_OK) e->run_busy_[parity] = true;
     }
-  } mark_done{this, parity, uploads};
+  } mark_done{this, parity, copy_stream_ != nullptr};  // every Run, so that a later one can tell when this one's reads are over
   bool train = false;
   std::vector<std::string> targets;
   for (auto &o : outputs) {

@@ -126,19 +126,16 @@ int cavs_sgemm_splitk(int transA, int transB, int M, int N, int K, float alpha, 
  * reference: it is for callers that cannot allocate device memory -- code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels, same plan and
  * bit-for-bit the results of cavs_sgemm_splitk; a shape whose partials would not fit
- * (cavs_sgemm_splitk_workspace(M, N, K) above the maximum) is refused with CAVS_EINVAL.  All
+ * (cavs_sgemm_splitk_workspace(M, N, K) above the maximum) is refused with CAVS_EINVAL -- the
+ * number of K splits, and with it the size of the partials, follows the device's CU count, so
+ * ask cavs_sgemm_splitk_workspace on the device in question.  A device whose copy of the buffer
+ * cannot be found (hipGetSymbolAddress) fails this call only; cavs_init succeeds regardless.  All
  * calls on a GPU share that GPU's buffer: calls that overlap in time on one GPU (two streams,
  * two threads) race; calls on one stream are ordered by it. */
 size_t cavs_sgemm_splitk_static_max_bytes(void);
 int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                              int lda, const float *B, int ldb, float beta, float *C, int ldc,
                              void *stream);
-/* Measurement aid (no counterpart in the reference): one launch in which every wavefront of
- * four workgroups per CU issues iters * 8 independent v_mfma_f32_32x32x2_f32 on register operands
- * and nothing else -- what the matrix pipes sustain at the clocks the device holds under that
- * load, to set beside the nominal peak.  `out` takes 4 * CUs * 256 floats (1024 * 256 on MI355X);
- * *flops receives the launch's FLOP count. */
-int cavs_mfma_probe(float *out, size_t out_floats, int iters, double *flops, void *stream);
 /* Up to four independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
  * (plus one for the K splits): the once-per-step block of
  * cavs/midend/batch_weight_updater.h:12-84 -- the weight-gradient GEMMs -- and the embedding

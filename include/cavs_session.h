@@ -54,8 +54,10 @@ typedef struct {
   int split_backward_rounds;
   /* Who builds the round schedule and the index lists of a step (cavs/midend/graph_scheduler.cc:
    * 169-245): 0 = the host scheduler, lists uploaded once per step; 1 = the GPU
-   * (cavs_schedule_arena: the graph feed goes up, only the round offsets come back).  Mode 1 needs
-   * OPT_BATCHING and samples of at most 2048 vertices and falls back to 0 otherwise. */
+   * (cavs_schedule_arena: the graph feed goes up, only the round offsets come back).  Mode 1 runs
+   * the serial scheduler's sessions (no OPT_BATCHING) on the host all the same, and refuses a feed
+   * whose samples exceed 2048 vertices (CAVS_EUNSUPPORTED).  The counter "scheduler" says who built
+   * the last step's lists. */
   int schedule_mode;
   /* Plan cache: keep the schedule and the device-resident lists of the last `plan_cache` distinct
    * graph feeds, keyed by the feed's bytes; a step on a feed seen before skips the scheduler and
@@ -140,7 +142,8 @@ void *cavs_session_stream(cavs_session *s);
  * to be zero or unused -- the forget-gate columns of the leaves -- and is skipped tile by tile)
  * "round_flops" (products inside fused round launches) "rounds" "launches"; "tail_rounds" (rounds,
  * forward and backward, that ran inside cavs_treelstm_tail_* launches) "tail_launches"; "plan_hits" /
- * "plan_misses" of the plan cache since the session was created; "tail_ready" (1 when the session may
+ * "plan_misses" of the plan cache since the session was created; "scheduler" (who produced the last
+ * step's lists: 0 host scheduler, 1 device scheduler, 2 plan cache); "tail_ready" (1 when the session may
  * use the tail launches); the last step's tail plan: "tail_first_round" (-1: none), "tail_vertices",
  * and of its longest group "tail_lists_max" (rounds) and "tail_tiles_max" (tiles of four rows). */
 int cavs_session_counter(cavs_session *s, const char *key, double *value);

@@ -38,7 +38,13 @@ def run_both(oracle, w, *, loss="softmax", pairing="reference", batching=True, *
     return got, want
 
 
-def compare(got, want, **tol):
+def compare(got, want, loss="softmax", **tol):
+    """The softmax configurations (the headline among them) are held to the literal bar, 1e-4
+    relative / 1e-5 absolute with no tensor-scale factor; the sum-of-squares and sum-of-magnitudes
+    losses, whose weight gradients reach the tens, measure "absolute" in units of the tensor's
+    largest entry (tolerance.py)."""
+    if loss == "softmax":
+        tol.setdefault("scaled", False)
     for k in ("loss", "graph_out", "dgraph_out"):
         close(got[k], want[k], k, **tol)
     # pool rows of roots are never written by any Scatter: their content is unspecified
@@ -59,7 +65,7 @@ CASES = [("treelstm", dict()), ("lstm", dict()), ("treefc", dict(act=1, use_bias
 def test_small_skewed_batches(oracle, model, kw, pairing, loss):
     w = small_workload(model, 61, B=6, H=16, E=12)
     got, want = run_both(oracle, w, loss=loss, pairing=pairing, **kw)
-    compare(got, want)
+    compare(got, want, loss=loss)
     assert got["trace"] == oracle.sched_trace(w["graph"])  # bit-exact lists on the running session
 
 
@@ -89,7 +95,7 @@ def test_benchmark_configs_scaled(oracle, name, scale):
     if w["model"] == "treefc":
         kw, loss = dict(act=1, use_bias=True, use_x=True), "root_sq"
     got, want = run_both(oracle, w, loss=loss, **kw)
-    compare(got, want)
+    compare(got, want, loss=loss)
 
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3"])
@@ -102,7 +108,38 @@ def test_benchmark_configs_at_full_size(oracle, name):
     if w["model"] == "treefc":
         kw, loss = dict(act=1, use_bias=True, use_x=True), "root_sq"
     got, want = run_both(oracle, w, loss=loss, **kw)
-    compare(got, want)
+    compare(got, want, loss=loss)
+
+
+@pytest.mark.parametrize("name", ["C4", "C5"])
+def test_benchmark_configs_at_full_size_against_recorded_values(name):
+    """C4 and C5 at their full sizes.  The checker needs minutes for these in double precision, so
+    its results were recorded once (tests/golden/make_fullsize_fixtures.py: per tensor the norm and
+    512 entries at fixed positions); the GPU step is held to them at the literal bar, 1e-4 relative /
+    1e-5 absolute."""
+    import os
+
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", f"fullsize_{name}.npz"))
+    w = synth.make_workload(name)
+    assert int(fx["N"]) == w["N"]
+    print(f"[case] full size {name} N={w['N']} H={w['H']}", flush=True)
+    s = session.Session(w["model"], H=w["H"], E=w["E"], V=w["V"], C_=w["C"], loss="softmax", pairing="reference")
+    names = {"treelstm": ("Emb", "W", "U", "Bv"), "lstm": ("Emb", "W", "Bv")}[w["model"]] + ("Wfc", "bfc")
+    s.set_params({k: w["params"][k] for k in names})
+    s.step(w["graph"], w["x"], w["labels"], backward=True)
+    got = dict(loss=s.fetch("loss"), graph_out=s.fetch("graph_out"), dgraph_out=s.fetch("dgraph_out"), **s.grads())
+    s.close()
+    checked = 0
+    for k, v in got.items():
+        if k + ".idx" not in fx:
+            continue
+        flat = np.asarray(v, np.float64).ravel()
+        assert tuple(fx[k + ".shape"]) == tuple(np.shape(v)) or flat.size == int(np.prod(fx[k + ".shape"])), k
+        close(flat[fx[k + ".idx"]], fx[k + ".val"], f"{name} {k} (recorded entries)", scaled=False)
+        norm = float(np.sqrt((flat * flat).sum()))
+        assert abs(norm - float(fx[k + ".norm"])) <= 1e-4 * float(fx[k + ".norm"]) + 1e-7, (k, norm, float(fx[k + ".norm"]))
+        checked += 1
+    assert checked >= 8, checked
 
 
 @pytest.mark.parametrize("name,B", [("C4", 8), ("C5", 6)])
@@ -140,7 +177,25 @@ def test_schedule_built_on_the_device(oracle, model, kw, pairing):
                    msg_pool=s.fetch("msg_pool"), grads=s.grads())
         got["trace"] = s.schedule_trace()
         assert got["trace"] == oracle.sched_trace(w["graph"])
-        compare(got, want)
+        assert s.counter("scheduler") == 1, "the lists of this step were not built on the device"
+        compare(got, want, loss=loss)
+    s.close()
+
+
+def test_device_scheduler_refuses_samples_it_cannot_hold():
+    """Samples of more than 2048 vertices are the host scheduler's: the device scheduler says so
+    instead of quietly handing the feed over."""
+    T = 2100
+    graph = np.full((1, T), -1, np.int32)
+    graph[0, : T - 1] = np.arange(1, T)
+    x, labels = np.zeros(T, np.float32), np.zeros(T, np.float32)
+    s = session.Session("lstm", H=16, V=7, C_=3, schedule="device")
+    with pytest.raises(hip.CavsError, match="at most 2048 vertices"):
+        s.step(graph, x, labels, backward=False)
+    s.close()
+    s = session.Session("lstm", H=16, V=7, C_=3, schedule="host")
+    s.step(graph, x, labels, backward=False)
+    assert s.N == T and s.counter("scheduler") == 0
     s.close()
 
 
@@ -341,7 +396,7 @@ def test_fused_rounds_match_oracle(oracle, model, kw, H, limit, pairing):
                msg_pool=s.fetch("msg_pool"), grads=s.grads(), trace=s.schedule_trace())
     fused_flops = s.counter("round_flops")
     s.close()
-    compare(got, want)
+    compare(got, want, loss=loss)
     assert (fused_flops > 0) == (limit >= 0), fused_flops
 
 
@@ -371,7 +426,7 @@ def test_backward_rounds_as_one_launch_or_two(oracle, model, kw, pairing):
                    msg_pool=s.fetch("msg_pool"), grads=s.grads(), trace=s.schedule_trace())
         launches.append(s.counter("launches"))
         s.close()
-        compare(got, want)
+        compare(got, want, loss=loss)
     assert launches[0] < launches[1], launches
 
 

@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (cavs_sgemm_splitk_static) against the entry
 point it is a variant of (cavs_sgemm_splitk): bit for bit, on two calls in a row, the
 second with a smaller input, so that what the first call left in the built-in scratch
-is there when the second runs.  Runs last in the suite and alone in a fresh process."""
+is there when the second runs; and the device's free memory is the same before and after
+the calls.  Collected last, so that a failure here hides no other test."""
 import numpy as np
 import pytest
 
@@ -36,8 +37,15 @@ def _product(g, oracle, tA, tB, M, N, K, seed):
     print(f"[case] splitk tA={tA} tB={tB} M={M} N={N} K={K} seed={seed}", flush=True)
     g.call("cavs_sgemm_splitk", tA, tB, M, N, K, 1.0, g.P(Ad), A.shape[1], g.P(Bd), B.shape[1], 0.5,
            g.P(want_d), N, g.P(ws), nbytes, g.stream())
+    # nothing is allocated by the call: the device reports the same free memory before and after
+    # (torch's caching allocator is not involved: the call sees raw pointers only)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
     g.call("cavs_sgemm_splitk_static", tA, tB, M, N, K, 1.0, g.P(Ad), A.shape[1], g.P(Bd), B.shape[1], 0.5,
            g.P(got_d), N, g.stream())
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, f"device memory changed across the call: {free_before} -> {free_after} bytes free"
     want, got = g.host(want_d), g.host(got_d)
     np.testing.assert_array_equal(got, want)
     # and the product itself is right (not two equal wrong answers)
