@@ -31,13 +31,16 @@ namespace cavs {
 constexpr int kTailH = 512;        // K / 8 per wavefront = 64 k = one float4 per lane and operand row
 constexpr int kTailRows = 32;      // at most eight tiles of four rows per group and round
 constexpr int kTailGroups = 8;     // one per XCD
-constexpr int kTailMaxRounds = 24; // per group
+constexpr int kTailMaxRounds = 32; // lists per group
 
-// what each group does: nrounds[g] lists of slab rows, list i = rows[start[g][i] .. + count[g][i])
+// What each group does: nrounds[g] lists of slab rows, list i = rows[start[g][i] .. + count[g][i]).
+// flags[g][i]: bit 0 -- the group's workgroups tell each other when the list is done (an arrival);
+// the rest -- how many of the group's arrivals must be in before the list starts (0: none, e.g. the
+// second slice of a round that does not fit one list).
 struct TailPlan {
-  int nrounds[kTailGroups];
+  int nrounds[kTailGroups], arrivals[kTailGroups];
   int start[kTailGroups][kTailMaxRounds];
-  int count[kTailGroups][kTailMaxRounds];
+  short count[kTailGroups][kTailMaxRounds], flags[kTailGroups][kTailMaxRounds];
 };
 
 // The sync block: word 1 = status (all groups); group g owns the 32 words from 32 (g + 1): arrivals,
@@ -100,7 +103,7 @@ __device__ inline bool tail_wait(unsigned *status, unsigned *gsync, unsigned tar
 __device__ inline float ld_row(const float *p) { return *p; }
 
 // The four k slots of an element added up across the wavefront, for the four rows of NP products
-// at once: on return the lanes of k slot s hold, in acc[p][0], the sum of row s of product p --
+// at once: afterwards the lanes of k slot s hold, in r[p][0], the sum of row s of product p --
 // (v[x] + v[x+16]) + (v[x+32] + v[x+48]) with v = that row's accumulator, the order in which the
 // per-round kernels add the slots up.  v_permlane16_swap exchanges the odd 16-lane rows of its first
 // operand with the even rows of its second, v_permlane32_swap the upper half of the first with the
@@ -108,16 +111,61 @@ __device__ inline float ld_row(const float *p) { return *p; }
 // one register, a butterfly of three swaps and three adds per product on the vector ALU (a shuffle
 // through the LDS crossbar costs eight cycles of a unit all eight wavefronts share).  Spelled out
 // as instructions because the compiler's builtins for the two swaps return the first result twice.
-// The accumulators come straight from MFMAs, whose results a vector-ALU instruction may read only
-// some cycles later, and the compiler does not look inside the statement: the wait is in it
-// (twelve cycles cover the six a two-pass MFMA asks for).  Between the stages the other products'
-// instructions stand between a result and its use, plus a short wait.
+// The compiler does not look inside such a statement, so the waits an instruction needs after the
+// one that produced its operand are the caller's: all() carries its own (twelve cycles cover the
+// six a two-pass MFMA asks for before a vector-ALU read, two between an add and the swap that reads
+// it); the stages are for callers that put at least that many instructions between them.
 template <int NP>
-__device__ inline void sum_slots_rows(floatx4 (&acc)[NP]);
+struct SlotSums;
 template <>
-__device__ inline void sum_slots_rows<5>(floatx4 (&acc)[5]) {
-  float r00 = acc[0][0], r01 = acc[0][1], r02 = acc[0][2], r03 = acc[0][3], r10 = acc[1][0], r11 = acc[1][1], r12 = acc[1][2], r13 = acc[1][3], r20 = acc[2][0], r21 = acc[2][1], r22 = acc[2][2], r23 = acc[2][3], r30 = acc[3][0], r31 = acc[3][1], r32 = acc[3][2], r33 = acc[3][3], r40 = acc[4][0], r41 = acc[4][1], r42 = acc[4][2], r43 = acc[4][3];
-  asm volatile(
+struct SlotSums<5> {
+  float r[5][4];
+  __device__ inline void take(const floatx4 (&acc)[5]) {
+#pragma unroll
+    for (int p = 0; p < 5; p++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) r[p][k] = acc[p][k];
+  }
+  // the stages one at a time, for a caller that puts other work (MFMAs of the next tile) between them
+  __device__ inline void stage_a() {
+    asm volatile(
+        "v_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
+        "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\t"
+        "v_permlane16_swap_b32 %8, %9\n\tv_permlane16_swap_b32 %10, %11\n\t"
+        "v_permlane16_swap_b32 %12, %13\n\tv_permlane16_swap_b32 %14, %15\n\t"
+        "v_permlane16_swap_b32 %16, %17\n\tv_permlane16_swap_b32 %18, %19"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]), "+v"(r[3][0]), "+v"(r[3][1]), "+v"(r[3][2]), "+v"(r[3][3]), "+v"(r[4][0]), "+v"(r[4][1]), "+v"(r[4][2]), "+v"(r[4][3]));
+  }
+  __device__ inline void stage_b() {
+    asm volatile(
+        "v_add_f32 %0, %0, %1\n\tv_add_f32 %2, %2, %3\n\t"
+        "v_add_f32 %4, %4, %5\n\tv_add_f32 %6, %6, %7\n\t"
+        "v_add_f32 %8, %8, %9\n\tv_add_f32 %10, %10, %11\n\t"
+        "v_add_f32 %12, %12, %13\n\tv_add_f32 %14, %14, %15\n\t"
+        "v_add_f32 %16, %16, %17\n\tv_add_f32 %18, %18, %19"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]), "+v"(r[3][0]), "+v"(r[3][1]), "+v"(r[3][2]), "+v"(r[3][3]), "+v"(r[4][0]), "+v"(r[4][1]), "+v"(r[4][2]), "+v"(r[4][3]));
+  }
+  __device__ inline void stage_c() {
+    asm volatile(
+        "v_permlane32_swap_b32 %0, %2\n\t"
+        "v_permlane32_swap_b32 %4, %6\n\t"
+        "v_permlane32_swap_b32 %8, %10\n\t"
+        "v_permlane32_swap_b32 %12, %14\n\t"
+        "v_permlane32_swap_b32 %16, %18"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]), "+v"(r[3][0]), "+v"(r[3][1]), "+v"(r[3][2]), "+v"(r[3][3]), "+v"(r[4][0]), "+v"(r[4][1]), "+v"(r[4][2]), "+v"(r[4][3]));
+  }
+  __device__ inline void stage_d() {
+    asm volatile(
+        "v_add_f32 %0, %0, %2\n\t"
+        "v_add_f32 %4, %4, %6\n\t"
+        "v_add_f32 %8, %8, %10\n\t"
+        "v_add_f32 %12, %12, %14\n\t"
+        "v_add_f32 %16, %16, %18"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]), "+v"(r[3][0]), "+v"(r[3][1]), "+v"(r[3][2]), "+v"(r[3][3]), "+v"(r[4][0]), "+v"(r[4][1]), "+v"(r[4][2]), "+v"(r[4][3]));
+  }
+  // all of it at once, right after the MFMAs that produced the accumulators
+  __device__ inline void all() {
+    asm volatile(
       "s_nop 7\n\ts_nop 3\n\t"
       "v_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
       "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\t"
@@ -142,13 +190,50 @@ __device__ inline void sum_slots_rows<5>(floatx4 (&acc)[5]) {
       "v_add_f32 %8, %8, %10\n\t"
       "v_add_f32 %12, %12, %14\n\t"
       "v_add_f32 %16, %16, %18"
-      : "+v"(r00), "+v"(r01), "+v"(r02), "+v"(r03), "+v"(r10), "+v"(r11), "+v"(r12), "+v"(r13), "+v"(r20), "+v"(r21), "+v"(r22), "+v"(r23), "+v"(r30), "+v"(r31), "+v"(r32), "+v"(r33), "+v"(r40), "+v"(r41), "+v"(r42), "+v"(r43));
-  acc[0][0] = r00; acc[1][0] = r10; acc[2][0] = r20; acc[3][0] = r30; acc[4][0] = r40;
-}
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]), "+v"(r[3][0]), "+v"(r[3][1]), "+v"(r[3][2]), "+v"(r[3][3]), "+v"(r[4][0]), "+v"(r[4][1]), "+v"(r[4][2]), "+v"(r[4][3]));
+  }
+};
 template <>
-__device__ inline void sum_slots_rows<3>(floatx4 (&acc)[3]) {
-  float r00 = acc[0][0], r01 = acc[0][1], r02 = acc[0][2], r03 = acc[0][3], r10 = acc[1][0], r11 = acc[1][1], r12 = acc[1][2], r13 = acc[1][3], r20 = acc[2][0], r21 = acc[2][1], r22 = acc[2][2], r23 = acc[2][3];
-  asm volatile(
+struct SlotSums<3> {
+  float r[3][4];
+  __device__ inline void take(const floatx4 (&acc)[3]) {
+#pragma unroll
+    for (int p = 0; p < 3; p++)
+#pragma unroll
+      for (int k = 0; k < 4; k++) r[p][k] = acc[p][k];
+  }
+  // the stages one at a time, for a caller that puts other work (MFMAs of the next tile) between them
+  __device__ inline void stage_a() {
+    asm volatile(
+        "v_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
+        "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\t"
+        "v_permlane16_swap_b32 %8, %9\n\tv_permlane16_swap_b32 %10, %11"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]));
+  }
+  __device__ inline void stage_b() {
+    asm volatile(
+        "v_add_f32 %0, %0, %1\n\tv_add_f32 %2, %2, %3\n\t"
+        "v_add_f32 %4, %4, %5\n\tv_add_f32 %6, %6, %7\n\t"
+        "v_add_f32 %8, %8, %9\n\tv_add_f32 %10, %10, %11"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]));
+  }
+  __device__ inline void stage_c() {
+    asm volatile(
+        "v_permlane32_swap_b32 %0, %2\n\t"
+        "v_permlane32_swap_b32 %4, %6\n\t"
+        "v_permlane32_swap_b32 %8, %10"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]));
+  }
+  __device__ inline void stage_d() {
+    asm volatile(
+        "v_add_f32 %0, %0, %2\n\t"
+        "v_add_f32 %4, %4, %6\n\t"
+        "v_add_f32 %8, %8, %10"
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]));
+  }
+  // all of it at once, right after the MFMAs that produced the accumulators
+  __device__ inline void all() {
+    asm volatile(
       "s_nop 7\n\ts_nop 3\n\t"
       "v_permlane16_swap_b32 %0, %1\n\tv_permlane16_swap_b32 %2, %3\n\t"
       "v_permlane16_swap_b32 %4, %5\n\tv_permlane16_swap_b32 %6, %7\n\t"
@@ -165,9 +250,9 @@ __device__ inline void sum_slots_rows<3>(floatx4 (&acc)[3]) {
       "v_add_f32 %0, %0, %2\n\t"
       "v_add_f32 %4, %4, %6\n\t"
       "v_add_f32 %8, %8, %10"
-      : "+v"(r00), "+v"(r01), "+v"(r02), "+v"(r03), "+v"(r10), "+v"(r11), "+v"(r12), "+v"(r13), "+v"(r20), "+v"(r21), "+v"(r22), "+v"(r23));
-  acc[0][0] = r00; acc[1][0] = r10; acc[2][0] = r20;
-}
+        : "+v"(r[0][0]), "+v"(r[0][1]), "+v"(r[0][2]), "+v"(r[0][3]), "+v"(r[1][0]), "+v"(r[1][1]), "+v"(r[1][2]), "+v"(r[1][3]), "+v"(r[2][0]), "+v"(r[2][1]), "+v"(r[2][2]), "+v"(r[2][3]));
+  }
+};
 
 // One k-group of four-row tiles is four MFMAs of sixteen 4 x 4 x 1 blocks each; block l / 4 of
 // lane l is (column group (l / 4) % 4, k slot l / 16).  An MFMA can take its A operand, for the four
@@ -235,12 +320,15 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
   float bias[4];
 #pragma unroll
   for (int k = 0; k < 4; k++) bias[k] = a.bias[k * H + ej];
-  if (tid == 0 && nrounds > 1) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const unsigned total = (unsigned)nrounds * a.expect;
+  const unsigned total = (unsigned)a.plan.arrivals[grp] * a.expect;
+  if (tid == 0 && total > 0) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  bool first_wait = true;
 
   for (int r = 0; r < nrounds; r++) {
     const int *rows = a.rows + a.plan.start[grp][r];
     const int n = a.plan.count[grp][r], T = (n + 3) >> 2, par = r & 1;
+    const int need = a.plan.flags[grp][r] >> 1;
+    const bool arrives = a.plan.flags[grp][r] & 1;
     // what does not depend on the rounds before: the round's lists, the epilogue's x * W
     if (tid < 64) {
       s_child[par][tid] = tid < 2 * n ? a.child[2L * rows[tid >> 1] + (tid & 1)] : -1;
@@ -260,8 +348,9 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
 #pragma unroll
       for (int k = 0; k < 4; k++) xw[k] = p[k * H];
     }
-    if (r > 0) {
-      if (!tail_wait(status, gsync, (unsigned)r * a.expect, a.spin_max, r == 1, &s_bail)) return;
+    if (need > 0) {
+      if (!tail_wait(status, gsync, (unsigned)need * a.expect, a.spin_max, first_wait, &s_bail)) return;
+      first_wait = false;
     } else {
       __syncthreads();
     }
@@ -278,21 +367,28 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       if (e_cr >= 0) { e_hr = ld_row(a.pool + (long)e_cr * H2 + ej); e_cr_c = ld_row(a.pool + (long)e_cr * H2 + H + ej); }
     }
 
-    // Operand rows: one float4 per child and tile (see CAVS_MMA4).  The loads of a tile are issued
-    // while the tile before it multiplies, unconditionally (a missing child reads row 0 and is masked
-    // where the operand is used; past the last tile the last one is fetched again), so that the wait
-    // before a tile's MFMAs counts exactly the two loads behind it.
+    // Operand rows: one float4 per child and tile (see CAVS_MMA4), unconditionally (a missing child
+    // reads row 0 and is masked where the operand is used; past the last tile the last one is fetched
+    // again).  A tile's instruction stream carries, between the four k-groups of its MFMAs, the two
+    // loads of the next tile and the slot sums of the tile before it: a wavefront stalled in a load's
+    // issue or busy on the vector ALU issues no MFMAs, and with every wavefront of the CU in the
+    // same phase the matrix pipes idled through both (measured: the three costs simply added up).
     const int ka = kb + 16 * ((lane >> 2) & 3) + 4 * slot;
-    auto fetch = [&](int t, float4 &l, float4 &rr, int &cl, int &cr) {
-      const int ra = 4 * (t < T ? t : T - 1) + (lane & 3);
-      cl = s_child[par][2 * ra];
-      cr = s_child[par][2 * ra + 1];
-      l = ld4(a.pool + (long)(cl >= 0 ? cl : 0) * H2 + ka);
-      rr = ld4(a.pool + (long)(cr >= 0 ? cr : 0) * H2 + ka);
+    struct Opnd {
+      float4 l, r;
+      int cl, cr;
     };
-    auto tile = [&](int t, float4 hl4, float4 hr4, int cl, int cr) {
-      if (cl < 0) hl4 = zero4();
-      if (cr < 0) hr4 = zero4();
+    auto child_of = [&](int t, int side) { return s_child[par][2 * (4 * (t < T ? t : T - 1) + (lane & 3)) + side]; };
+    SlotSums<NP> sums;
+    auto park = [&](int t) {
+      float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
+#pragma unroll
+      for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = sums.r[p][0];
+    };
+    // tile t from `o`, fetching tile t + 1 into `nx`; PREV: tile t - 1 waits in `sums`
+    auto tile = [&](auto prev, int t, const Opnd &o, Opnd &nx) {
+      constexpr bool PREV = decltype(prev)::value;
+      const float4 hl4 = o.cl >= 0 ? o.l : zero4(), hr4 = o.cr >= 0 ? o.r : zero4();
       floatx4 acc[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -305,29 +401,46 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       CAVS_MMA4(acc[3], hl4.comp, wf[g].comp, g); \
       CAVS_MMA4(acc[4], hr4.comp, wf[g].comp, g);
 #define CAVS_FWD_GROUP(g) CAVS_FWD_STEP(g, x) CAVS_FWD_STEP(g, y) CAVS_FWD_STEP(g, z) CAVS_FWD_STEP(g, w)
-      CAVS_FWD_GROUP(0) CAVS_FWD_GROUP(1) CAVS_FWD_GROUP(2) CAVS_FWD_GROUP(3)
+      nx.cl = child_of(t + 1, 0);
+      nx.cr = child_of(t + 1, 1);
+      CAVS_FWD_GROUP(0)
+      __builtin_amdgcn_sched_barrier(0);
+      nx.l = ld4(a.pool + (long)(nx.cl >= 0 ? nx.cl : 0) * H2 + ka);
+      if constexpr (PREV) sums.stage_a();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_FWD_GROUP(1)
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (PREV) sums.stage_b();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_FWD_GROUP(2)
+      __builtin_amdgcn_sched_barrier(0);
+      nx.r = ld4(a.pool + (long)(nx.cr >= 0 ? nx.cr : 0) * H2 + ka);
+      if constexpr (PREV) sums.stage_c();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_FWD_GROUP(3)
+      __builtin_amdgcn_sched_barrier(0);
 #undef CAVS_FWD_GROUP
 #undef CAVS_FWD_STEP
-      // the four k slots of an element added up inside the wavefront; lanes of slot s park row s
-      float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
-      sum_slots_rows<NP>(acc);
-#pragma unroll
-      for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = acc[p][0];
+      if constexpr (PREV) {
+        sums.stage_d();
+        park(t - 1);  // lanes of slot s park row s
+      }
+      sums.take(acc);
+      __builtin_amdgcn_sched_barrier(0);
     };
     {
-      float4 la, ra4, lb, rb4;
-      int cla, cra, clb, crb;
-      fetch(0, la, ra4, cla, cra);
-      for (int t = 0; t < T; t += 2) {
-        fetch(t + 1, lb, rb4, clb, crb);
-        __builtin_amdgcn_sched_barrier(0);
-        tile(t, la, ra4, cla, cra);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(t + 2, la, ra4, cla, cra);
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < T) tile(t + 1, lb, rb4, clb, crb);
-        __builtin_amdgcn_sched_barrier(0);
+      Opnd oa, ob;
+      oa.cl = child_of(0, 0);
+      oa.cr = child_of(0, 1);
+      oa.l = ld4(a.pool + (long)(oa.cl >= 0 ? oa.cl : 0) * H2 + ka);
+      oa.r = ld4(a.pool + (long)(oa.cr >= 0 ? oa.cr : 0) * H2 + ka);
+      tile(std::false_type{}, 0, oa, ob);
+      for (int t = 1; t < T; t += 2) {
+        tile(std::true_type{}, t, ob, oa);
+        if (t + 1 < T) tile(std::true_type{}, t + 1, oa, ob);
       }
+      sums.all();
+      park(T - 1);
     }
     __syncthreads();
 
@@ -349,7 +462,8 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
         a.pool[(long)e_dst * H2 + H + ej] = q.c;
       }
     }
-    tail_arrive(gsync, total);
+    if (arrives) tail_arrive(gsync, total);
+    else __syncthreads();
     if (eon) {  // what the backward pass and the caller read: on its way while the next round starts
       const long b = erow;
       float *g = a.gates + b * 6 * H + ej;
@@ -409,12 +523,15 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
   }
   const int ej = j0 + x;
   if (ks < 4) __builtin_amdgcn_s_setprio(2);  // (see the forward kernel)
-  if (tid == 0 && nrounds > 1) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const unsigned total = (unsigned)nrounds * a.expect;
+  const unsigned total = (unsigned)a.plan.arrivals[grp] * a.expect;
+  if (tid == 0 && total > 0) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  bool first_wait = true;
 
   for (int r = 0; r < nrounds; r++) {
     const int *rows = a.rows + a.plan.start[grp][r];
     const int n = a.plan.count[grp][r], T = (n + 3) >> 2, par = r & 1;
+    const int need = a.plan.flags[grp][r] >> 1;
+    const bool arrives = a.plan.flags[grp][r] & 1;
     // (rows past the list's end stand for its first row; their results are not written)
     if (tid < kTailRows) s_row[par][tid] = rows[tid < n ? tid : 0];
     // the operands of the children's gate gradients: everything except d c of the parent was
@@ -451,69 +568,100 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
         }
       }
     }
-    if (r > 0) {
-      if (!tail_wait(status, gsync, (unsigned)r * a.expect, a.spin_max, r == 1, &s_bail)) return;
+    if (need > 0) {
+      if (!tail_wait(status, gsync, (unsigned)need * a.expect, a.spin_max, first_wait, &s_bail)) return;
+      first_wait = false;
     } else {
       __syncthreads();
     }
     const float pdc = eon ? ld_row(a.dc + erow * H + ej) : 0.f;
 
     // Per tile five float4 per lane (see CAVS_MMA4): three of [d_i|d_o|d_u] (K = 3H: twelve k-groups
-    // per wavefront), one each of d_fl, d_fr (K = H); a tile's are issued while the tile before it
-    // multiplies (past the last tile the last one is fetched again), so the wait before a tile's
-    // MFMAs counts exactly the five loads behind it.
+    // per wavefront), one each of d_fl, d_fr (K = H).  As in the forward kernel a tile's instruction
+    // stream carries the five loads of the next tile (past the last tile the last one is fetched
+    // again) and the slot sums of the tile before it between its MFMAs; the K = H products' MFMAs
+    // stand between those of the K = 3H product, whose single accumulator makes every one of them
+    // wait for the one before.
     const int kq = 16 * ((lane >> 2) & 3) + 4 * slot;
     struct Opnd {
       float4 x[3], fl, fr;
     };
-    auto fetch = [&](int t, Opnd &o) {
-      const long row = s_row[par][4 * (t < T ? t : T - 1) + (lane & 3)];
-      const float *px = a.dxW + row * a.ld_dxw + ks * (3 * H / 8) + kq;
+    auto row_of = [&](int t) { return (long)s_row[par][4 * (t < T ? t : T - 1) + (lane & 3)]; };
+    SlotSums<NP> sums;
+    auto park = [&](int t) {
+      float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
 #pragma unroll
-      for (int q = 0; q < 3; q++) o.x[q] = ld4(px + 64 * q);
-      const float *pl = a.dF + 2 * row * H + ks * (H / 8) + kq;
-      o.fl = ld4(pl);
-      o.fr = ld4(pl + H);
+      for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = sums.r[p][0];
     };
-    auto tile = [&](int t, const Opnd &o) {
+    auto tile = [&](auto prev, int t, const Opnd &o, Opnd &nx) {
+      constexpr bool PREV = decltype(prev)::value;
       floatx4 acc[NP];
 #pragma unroll
       for (int p = 0; p < NP; p++) acc[p] = floatx4{0.f, 0.f, 0.f, 0.f};
+      const long nrow = row_of(t + 1);
+      const float *px = a.dxW + nrow * a.ld_dxw + ks * (3 * H / 8) + kq;
+      const float *pl = a.dF + 2 * nrow * H + ks * (H / 8) + kq;
       // (k-group 4 q + g of the K = 3H product: component by component of o.x[q], broadcast from block g)
-#define CAVS_P0_GROUP(q, g)                           \
-      CAVS_MMA4(acc[0], o.x[q].x, w0[4 * q + g].x, g); \
-      CAVS_MMA4(acc[0], o.x[q].y, w0[4 * q + g].y, g); \
-      CAVS_MMA4(acc[0], o.x[q].z, w0[4 * q + g].z, g); \
-      CAVS_MMA4(acc[0], o.x[q].w, w0[4 * q + g].w, g);
-#define CAVS_P0_LOAD(q) CAVS_P0_GROUP(q, 0) CAVS_P0_GROUP(q, 1) CAVS_P0_GROUP(q, 2) CAVS_P0_GROUP(q, 3)
-      CAVS_P0_LOAD(0) CAVS_P0_LOAD(1) CAVS_P0_LOAD(2)
-#undef CAVS_P0_LOAD
-#undef CAVS_P0_GROUP
-#define CAVS_P12_STEP(g, comp)                    \
+#define CAVS_P0_GROUP(q, g)                            \
+      CAVS_MMA4(acc[0], o.x[q].x, w0[4 * (q) + (g)].x, g); \
+      CAVS_MMA4(acc[0], o.x[q].y, w0[4 * (q) + (g)].y, g); \
+      CAVS_MMA4(acc[0], o.x[q].z, w0[4 * (q) + (g)].z, g); \
+      CAVS_MMA4(acc[0], o.x[q].w, w0[4 * (q) + (g)].w, g);
+#define CAVS_P12_STEP(g, comp)                     \
       CAVS_MMA4(acc[1], o.fl.comp, w1[g].comp, g); \
       CAVS_MMA4(acc[2], o.fr.comp, w1[g].comp, g);
-#define CAVS_P12_GROUP(g) CAVS_P12_STEP(g, x) CAVS_P12_STEP(g, y) CAVS_P12_STEP(g, z) CAVS_P12_STEP(g, w)
-      CAVS_P12_GROUP(0) CAVS_P12_GROUP(1) CAVS_P12_GROUP(2) CAVS_P12_GROUP(3)
-#undef CAVS_P12_GROUP
+      // one quarter of the tile: three k-groups of the long product around one of the short ones
+#define CAVS_BWD_QUARTER(g)                                                             \
+      CAVS_P0_GROUP((3 * g) / 4, (3 * g) % 4) CAVS_P12_STEP(g, x)                        \
+      CAVS_P0_GROUP((3 * g + 1) / 4, (3 * g + 1) % 4) CAVS_P12_STEP(g, y) CAVS_P12_STEP(g, z) \
+      CAVS_P0_GROUP((3 * g + 2) / 4, (3 * g + 2) % 4) CAVS_P12_STEP(g, w)
+      CAVS_BWD_QUARTER(0)
+      __builtin_amdgcn_sched_barrier(0);
+      nx.x[0] = ld4(px);
+      nx.x[1] = ld4(px + 64);
+      if constexpr (PREV) sums.stage_a();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_BWD_QUARTER(1)
+      __builtin_amdgcn_sched_barrier(0);
+      nx.x[2] = ld4(px + 128);
+      if constexpr (PREV) sums.stage_b();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_BWD_QUARTER(2)
+      __builtin_amdgcn_sched_barrier(0);
+      nx.fl = ld4(pl);
+      nx.fr = ld4(pl + H);
+      if constexpr (PREV) sums.stage_c();
+      __builtin_amdgcn_sched_barrier(0);
+      CAVS_BWD_QUARTER(3)
+      __builtin_amdgcn_sched_barrier(0);
+#undef CAVS_BWD_QUARTER
 #undef CAVS_P12_STEP
-      float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
-      sum_slots_rows<NP>(acc);
-#pragma unroll
-      for (int p = 0; p < NP; p++) dst[(p * 4 + slot) * 16] = acc[p][0];
+#undef CAVS_P0_GROUP
+      if constexpr (PREV) {
+        sums.stage_d();
+        park(t - 1);
+      }
+      sums.take(acc);
+      __builtin_amdgcn_sched_barrier(0);
     };
     {
       Opnd oa, ob;
-      fetch(0, oa);
-      for (int t = 0; t < T; t += 2) {
-        fetch(t + 1, ob);
-        __builtin_amdgcn_sched_barrier(0);
-        tile(t, oa);
-        __builtin_amdgcn_sched_barrier(0);
-        fetch(t + 2, oa);
-        __builtin_amdgcn_sched_barrier(0);
-        if (t + 1 < T) tile(t + 1, ob);
-        __builtin_amdgcn_sched_barrier(0);
+      {
+        const long row = row_of(0);
+        const float *px = a.dxW + row * a.ld_dxw + ks * (3 * H / 8) + kq;
+        const float *pl = a.dF + 2 * row * H + ks * (H / 8) + kq;
+#pragma unroll
+        for (int q = 0; q < 3; q++) oa.x[q] = ld4(px + 64 * q);
+        oa.fl = ld4(pl);
+        oa.fr = ld4(pl + H);
       }
+      tile(std::false_type{}, 0, oa, ob);
+      for (int t = 1; t < T; t += 2) {
+        tile(std::true_type{}, t, ob, oa);
+        if (t + 1 < T) tile(std::true_type{}, t + 1, oa, ob);
+      }
+      sums.all();
+      park(T - 1);
     }
     __syncthreads();
 
@@ -542,7 +690,8 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
         }
       }
     }
-    tail_arrive(gsync, total);
+    if (arrives) tail_arrive(gsync, total);
+    else __syncthreads();
   }
 }
 
@@ -561,23 +710,35 @@ __global__ __launch_bounds__(512, 1) void tail_probe_kernel(unsigned *sync, int 
 }
 
 // Copies the caller's description of the groups and checks it (host arrays: group g runs
-// nrounds[g] lists, list i of group g is rows[start[g * max_rounds + i] .. + count[g * max_rounds + i])).
-static int tail_plan(const char *who, int ngroups, const int *nrounds, const int *start, const int *count, int max_rounds, TailPlan *out) {
+// nrounds[g] lists, list i of group g is rows[start[g * max_rounds + i] .. + count[g * max_rounds + i]);
+// flags as in TailPlan, or null: every list waits for all the lists before it and arrives).
+static int tail_plan(const char *who, int ngroups, const int *nrounds, const int *start, const int *count, const int *flags,
+                     int max_rounds, TailPlan *out) {
   CAVS_REQUIRE(ngroups >= 1 && ngroups <= kTailGroups && nrounds && start && count && max_rounds >= 1,
                "%s: bad plan (1..%d groups)", who, kTailGroups);
   *out = TailPlan{};
   int any = 0;
   for (int g = 0; g < ngroups; g++) {
-    CAVS_REQUIRE(nrounds[g] >= 0 && nrounds[g] <= kTailMaxRounds && nrounds[g] <= max_rounds, "%s: group %d has %d rounds, at most %d", who, g,
+    CAVS_REQUIRE(nrounds[g] >= 0 && nrounds[g] <= kTailMaxRounds && nrounds[g] <= max_rounds, "%s: group %d has %d lists, at most %d", who, g,
                  nrounds[g], kTailMaxRounds < max_rounds ? kTailMaxRounds : max_rounds);
     out->nrounds[g] = nrounds[g];
     any += nrounds[g];
+    int arrived = 0;
     for (int i = 0; i < nrounds[g]; i++) {
       const int s = start[g * max_rounds + i], c = count[g * max_rounds + i];
-      CAVS_REQUIRE(s >= 0 && c >= 1 && c <= kTailRows, "%s: group %d round %d: %d rows from %d (1..%d rows)", who, g, i, c, s, kTailRows);
+      CAVS_REQUIRE(s >= 0 && c >= 1 && c <= kTailRows, "%s: group %d list %d: %d rows from %d (1..%d rows)", who, g, i, c, s, kTailRows);
+      const int f = flags ? flags[g * max_rounds + i] : ((i << 1) | 1);
+      CAVS_REQUIRE(f >= 0 && (f >> 1) <= arrived, "%s: group %d list %d waits for %d arrivals, %d lists before it arrive", who, g, i, f >> 1,
+                   arrived);
       out->start[g][i] = s;
-      out->count[g][i] = c;
+      out->count[g][i] = (short)c;
+      out->flags[g][i] = (short)f;
+      arrived += f & 1;
     }
+    // (the last arrival of a launch clears the counter: nobody may still be waiting on it then)
+    for (int i = nrounds[g] - 1; i >= 0 && !(out->flags[g][i] & 1); i--)
+      CAVS_REQUIRE((out->flags[g][i] >> 1) == 0, "%s: group %d list %d waits, but no list from it on arrives", who, g, i);
+    out->arrivals[g] = arrived;
   }
   return any > 0 ? 1 : 0;  // 0: nothing to do
 }
@@ -611,8 +772,8 @@ int cavs_tail_probe(unsigned *sync, int H, int spin_max, void *stream) {
 int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const float *xW, int ld_xw, const float *Upk,
                            const float *bias, float *G, float *hlr, float *gates, float *msg, float *graph_out,
                            const int *out_rows, const int *rows, int ngroups, const int *nrounds, const int *start,
-                           const int *count, int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
-                           void *stream) {
+                           const int *count, const int *flags, int max_rounds, int H, unsigned *sync, int spin_max,
+                           int extra_arrivals, void *stream) {
   CAVS_REQUIRE(H == kTailH && ld_xw >= 4 * H && ld_xw % 4 == 0, "cavs_treelstm_tail_fwd: bad shape H=%d ld_xw=%d (H = %d only)", H, ld_xw,
                kTailH);
   CAVS_REQUIRE(pool && child && pair && xW && Upk && bias && G && hlr && gates && rows && sync, "cavs_treelstm_tail_fwd: null pointer");
@@ -621,7 +782,7 @@ int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const
   CAVS_REQUIRE(spin_max >= 0 && extra_arrivals >= 0, "cavs_treelstm_tail_fwd: bad wait bound");
   TailFwdArgs a{pool, child, pair, xW, ld_xw, Upk, bias, G, hlr, gates, msg, graph_out, out_rows, rows, sync, spin_max,
                 H / 16 + extra_arrivals, {}};
-  const int todo = tail_plan("cavs_treelstm_tail_fwd", ngroups, nrounds, start, count, max_rounds, &a.plan);
+  const int todo = tail_plan("cavs_treelstm_tail_fwd", ngroups, nrounds, start, count, flags, max_rounds, &a.plan);
   if (todo <= 0) return todo;
   constexpr size_t lds = 8 * 8 * 20 * 16 * sizeof(float);
   static int attr = tail_lds_attr(reinterpret_cast<const void *>(treelstm_tail_fwd_kernel), lds);
@@ -634,7 +795,8 @@ int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const
 int cavs_treelstm_tail_bwd(float *dxW, int ld_dxw, float *dF, float *dc, const float *UTp, const int *child_rows,
                            const float *gates, const float *G, const float *dret, const int *dret_rows, int leaf_rows,
                            const int *rows, int ngroups, const int *nrounds, const int *start, const int *count,
-                           int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals, void *stream) {
+                           const int *flags, int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
+                           void *stream) {
   CAVS_REQUIRE(H == kTailH && ld_dxw >= 4 * H && ld_dxw % 4 == 0 && leaf_rows >= 0,
                "cavs_treelstm_tail_bwd: bad shape H=%d ld=%d leaf_rows=%d (H = %d only)", H, ld_dxw, leaf_rows, kTailH);
   CAVS_REQUIRE(dxW && dF && dc && UTp && child_rows && gates && G && dret && dret_rows && rows && sync,
@@ -643,7 +805,7 @@ int cavs_treelstm_tail_bwd(float *dxW, int ld_dxw, float *dF, float *dc, const f
   CAVS_REQUIRE(spin_max >= 0 && extra_arrivals >= 0, "cavs_treelstm_tail_bwd: bad wait bound");
   TailBwdArgs a{dxW, ld_dxw, dF, dc, UTp, child_rows, gates, G, dret, dret_rows, rows, sync, leaf_rows, spin_max,
                 H / 16 + extra_arrivals, {}};
-  const int todo = tail_plan("cavs_treelstm_tail_bwd", ngroups, nrounds, start, count, max_rounds, &a.plan);
+  const int todo = tail_plan("cavs_treelstm_tail_bwd", ngroups, nrounds, start, count, flags, max_rounds, &a.plan);
   if (todo <= 0) return todo;
   constexpr size_t lds = 8 * 8 * 12 * 16 * sizeof(float);
   static int attr = tail_lds_attr(reinterpret_cast<const void *>(treelstm_tail_bwd_kernel), lds);

@@ -104,8 +104,8 @@ _SIGS = {
     "cavs_treelstm_bwd_gates_rows": [_P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "cavs_treelstm_round_bwd_children_gates_packed": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "cavs_tail_probe": [_P, _I, _I, _P],
-    "cavs_treelstm_tail_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _P, _I, _I, _P],
-    "cavs_treelstm_tail_bwd": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _I, _I, _P, _I, _I, _P],
+    "cavs_treelstm_tail_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _P],
+    "cavs_treelstm_tail_bwd": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P, _I, _I, _P],
     "cavs_transpose": [_P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_round_fwd_packed": [_P, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],

@@ -88,8 +88,9 @@ void Engine::tail_setup() {
 
 int Engine::tail_limit() const {
   if (!tail_ready_ || fused_rows() <= 0) return 0;
-  const int most = 32;
-  return cfg_.tail_rows > 0 ? std::min(cfg_.tail_rows, most) : most;
+  // a round whose rows are dealt so that some group gets more than this stays a launch of its own
+  // (the launches take a group's share of a round in slices of at most 32 rows)
+  return cfg_.tail_rows > 0 ? cfg_.tail_rows : 32;
 }
 
 // Which rounds run inside the tail launches, and who runs which row.  The rounds are a suffix of the
@@ -97,19 +98,19 @@ int Engine::tail_limit() const {
 // rows (kid_rows: the rows whose messages a row consumes); a tree of that forest goes to one group
 // as a whole, so nothing a group reads is written by another during the launch.  Trees are dealt
 // heaviest first to the group with the fewest rows so far; the suffix starts at the earliest round
-// from which no group gets more rows of a round than a launch takes.
+// from which no group gets more rows of a round than the limit, nor more lists than a launch takes.
 void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
   tail_ = TailPlan();
   const int lim = tail_limit();
   const Schedule &s = *sched_;
-  const int R = (int)s.rounds.size(), N = s.N, G = cavs_tail_max_groups(), cap = cavs_tail_max_rounds();
-  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || Upk_.capacity() == 0) return;
+  const int R = (int)s.rounds.size(), N = s.N, G = cavs_tail_max_groups(), cap = cavs_tail_max_rounds(), slice = 32;
+  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || Upk_.capacity() == 0 || !cavs_tail_rounds_ok(1, cfg_.H)) return;
   int k0 = 1;
   while (k0 < R && (s.rounds[k0].n > G * lim || leaf_round(s.rounds[k0]))) k0++;
   std::vector<int> comp, weight, group, order, per;
   for (; R - k0 >= 2; k0++) {
     bool ok = true;
-    for (int k = k0; k < R && ok; k++) ok = !leaf_round(s.rounds[k]) && cavs_tail_rounds_ok(std::min(s.rounds[k].n, lim), cfg_.H);
+    for (int k = k0; k < R && ok; k++) ok = !leaf_round(s.rounds[k]);
     if (!ok) continue;
     const int lo = s.rounds[k0].offset;
     comp.assign(N - lo, -1);
@@ -137,7 +138,7 @@ void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
       group[c] = best;
       load[best] += weight[c];
     }
-    // rows of round k that group g runs
+    // rows of round k that group g runs, and the lists that makes
     const int nr = R - k0;
     per.assign((size_t)G * nr, 0);
     for (int k = k0; k < R; k++)
@@ -147,46 +148,54 @@ void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
       int mine = 0;
       for (int k = 0; k < nr; k++) {
         if (per[(size_t)g * nr + k] > lim) ok = false;
-        mine += per[(size_t)g * nr + k] > 0;
+        mine += (per[(size_t)g * nr + k] + slice - 1) / slice;
       }
       if (mine > cap) ok = false;
       lists = std::max(lists, mine);
     }
     if (!ok) continue;
-    // the lists: per group, round by round
     TailPlan &t = tail_;
     t.first = k0;
     t.max_rounds = std::max(lists, 1);
+    const size_t M = t.max_rounds;
     t.nrounds.assign(G, 0);
-    t.start.assign((size_t)G * t.max_rounds, 0);
-    t.count.assign((size_t)G * t.max_rounds, 0);
+    for (auto *v : {&t.start, &t.count, &t.flags, &t.bstart, &t.bcount, &t.bflags}) v->assign((size_t)G * M, 0);
+    // the device list: group by group, round by round
     std::vector<int> at((size_t)G * nr, -1);
     size_t fill = 0;
     for (int g = 0; g < G; g++)
       for (int k = 0; k < nr; k++) {
-        const int c = per[(size_t)g * nr + k];
-        if (c == 0) continue;
-        const int i = t.nrounds[g]++;
-        t.start[(size_t)g * t.max_rounds + i] = (int)fill;
-        t.count[(size_t)g * t.max_rounds + i] = c;
         at[(size_t)g * nr + k] = (int)fill;
-        fill += c;
+        fill += per[(size_t)g * nr + k];
       }
-    for (int k = k0; k < R; k++)
-      for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) rows_out[at[(size_t)group[comp[b - lo]] * nr + (k - k0)]++] = b;
-    t.rows = fill;
-    t.bstart = t.start;
-    t.bcount = t.count;
-    for (int g = 0; g < G; g++) {
-      std::reverse(t.bstart.begin() + (size_t)g * t.max_rounds, t.bstart.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
-      std::reverse(t.bcount.begin() + (size_t)g * t.max_rounds, t.bcount.begin() + (size_t)g * t.max_rounds + t.nrounds[g]);
+    {
+      std::vector<int> cur(at);
+      for (int k = k0; k < R; k++)
+        for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) rows_out[cur[(size_t)group[comp[b - lo]] * nr + (k - k0)]++] = b;
     }
+    // A group's share of a round as lists of at most `slice` rows: the first waits for the rounds the
+    // group has done so far, the last is an arrival.  Forward: rounds in order; backward: reversed.
     for (int g = 0; g < G; g++) {
       int tiles = 0;
-      for (int i = 0; i < t.nrounds[g]; i++) tiles += (t.count[(size_t)g * t.max_rounds + i] + 3) / 4;
+      for (int dir = 0; dir < 2; dir++) {
+        std::vector<int> &st = dir ? t.bstart : t.start, &ct = dir ? t.bcount : t.count, &fl = dir ? t.bflags : t.flags;
+        int i = 0, done = 0;
+        for (int kk = 0; kk < nr; kk++) {
+          const int k = dir ? nr - 1 - kk : kk, c = per[(size_t)g * nr + k];
+          for (int c0 = 0; c0 < c; c0 += slice, i++) {
+            st[g * M + i] = at[(size_t)g * nr + k] + c0;
+            ct[g * M + i] = std::min(slice, c - c0);
+            fl[g * M + i] = ((c0 == 0 ? done : 0) << 1) | (c0 + slice >= c ? 1 : 0);
+            if (!dir) tiles += (ct[g * M + i] + 3) / 4;
+          }
+          done += c > 0;
+        }
+        t.nrounds[g] = i;
+      }
       t.tiles_max = std::max(t.tiles_max, tiles);
       t.lists_max = std::max(t.lists_max, t.nrounds[g]);
     }
+    t.rows = fill;
     t.vertices = (double)fill;
     t.flops = 2.0 * fill * cfg_.H * 5.0 * cfg_.H;
     return;
@@ -992,7 +1001,7 @@ void Engine::treelstm_forward() {
       CAVS_TIMED(K_ROUND, cavs_treelstm_tail_fwd(pool_.get(), d_child_, d_pair_, xW_.get(), 4 * H, Upk_.get(), Bv, G_.get(), hlr_.get(),
                                                  gates_.get(), out_folded_ ? nullptr : msg_.get(), go, d_t2j_, d_tail_rows_,
                                                  (int)tail_.nrounds.size(), tail_.nrounds.data(), tail_.start.data(), tail_.count.data(),
-                                                 tail_.max_rounds, H, reinterpret_cast<unsigned *>(tail_sync_.get()), kTailSpins, 0,
+                                                 tail_.flags.data(), tail_.max_rounds, H, reinterpret_cast<unsigned *>(tail_sync_.get()), kTailSpins, 0,
                                                  stream_));
       c_round_flops_ += tail_.flops;
       c_gather_rows_ += 2.0 * tail_.vertices;
@@ -1094,7 +1103,7 @@ void Engine::treelstm_backward() {
   if (tail_n > 0) {
     CAVS_TIMED(K_ROUND, cavs_treelstm_tail_bwd(dxW_.get(), 4 * H, dF_.get(), dc_.get(), UT_.get(), d_kid_rows_, gates_.get(), G_.get(), d_dgo_,
                                                d_t2j_, sched_->leaf_prefix, d_tail_rows_, (int)tail_.nrounds.size(), tail_.nrounds.data(),
-                                               tail_.bstart.data(), tail_.bcount.data(), tail_.max_rounds, H,
+                                               tail_.bstart.data(), tail_.bcount.data(), tail_.bflags.data(), tail_.max_rounds, H,
                                                reinterpret_cast<unsigned *>(tail_sync_.get()), kTailSpins, 0, stream_));
     c_gather_rows_ += tail_.vertices;
     c_round_flops_ += tail_.flops;

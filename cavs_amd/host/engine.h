@@ -184,8 +184,8 @@ class Engine {
   struct TailPlan {
     int first = -1;  // first round (forward order) inside the launches; -1: none
     int max_rounds = 0;
-    std::vector<int> nrounds, start, count;      // per group; lists in forward order
-    std::vector<int> bstart, bcount;             // the same lists in backward order
+    std::vector<int> nrounds, start, count, flags;  // per group; lists in forward order
+    std::vector<int> bstart, bcount, bflags;        // the same lists in backward order
     size_t rows = 0;                             // length of the device list of slab rows
     double flops = 0, vertices = 0;
     int lists_max = 0, tiles_max = 0;            // the longest group: its lists, its tiles of four rows

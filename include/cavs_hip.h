@@ -374,8 +374,11 @@ int cavs_treelstm_round_leaves_fwd(float *pool, const int *pair, const float *xW
  * per round: results equal bit for bit.
  *   rows (device): the groups' lists of slab rows.  Group g runs nrounds[g] lists one after the
  *   other, list i = rows[start[g * max_rounds + i] .. + count[g * max_rounds + i]), 1..32 rows each
- *   (nrounds, start, count: host arrays).  What a list's rows read must have been written before
- *   the launch or by earlier lists of the same group.
+ *   (nrounds, start, count, flags: host arrays).  What a list's rows read must have been written
+ *   before the launch or by earlier lists of the same group that it waits for: flags[.] = 2 * w + a,
+ *   where the list starts once w of the group's arrivals are in (0: at once -- a further slice of a
+ *   round of more than 32 rows) and a = 1 makes the end of the list an arrival (the last slice of a
+ *   round).  flags == NULL: every list waits for all the lists before it and arrives.
  *   Every other array is the whole-batch array the per-round entry points take slices of (child
  *   [2N], pair [N], out_rows [N], xW [N,4H], G [2N,2H], hlr [N,H], gates [N,6H], msg [N,2H] or NULL;
  *   backward: dxW [N,4H], dF [2N,H], dc [N,H], child_rows [2N]).
@@ -400,14 +403,14 @@ int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const
                            const float *Upk, const float *bias, float *G, float *hlr, float *gates,
                            float *msg, float *graph_out, const int *out_rows, const int *rows,
                            int ngroups, const int *nrounds, const int *start, const int *count,
-                           int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
-                           void *stream);
+                           const int *flags, int max_rounds, int H, unsigned *sync, int spin_max,
+                           int extra_arrivals, void *stream);
 int cavs_treelstm_tail_bwd(float *dxW, int ld_dxw, float *dF, float *dc, const float *UTp,
                            const int *child_rows, const float *gates, const float *G,
                            const float *dret, const int *dret_rows, int leaf_rows, const int *rows,
                            int ngroups, const int *nrounds, const int *start, const int *count,
-                           int max_rounds, int H, unsigned *sync, int spin_max, int extra_arrivals,
-                           void *stream);
+                           const int *flags, int max_rounds, int H, unsigned *sync, int spin_max,
+                           int extra_arrivals, void *stream);
 
 /* Backward of the gates of a round.  The message gradient of slab row b is read from
  * dpool row pair[b] (grad of Scatter is Gather on the same list, zero for -1); the c

@@ -63,12 +63,14 @@ typedef struct {
    * graph feeds, keyed by the feed's bytes; a step on a feed seen before skips the scheduler and
    * the upload.  0 = off. */
   int plan_cache;
-  /* Tree-LSTM, H = 512, batches whose message flow is a forest: the consecutive rounds of at most
-   * this many vertices nearest the roots (the last forward rounds, the first backward rounds) run
-   * as one launch per direction (cavs_treelstm_tail_fwd / _bwd) instead of one launch per round
-   * (cavs/midend/statement.cc:69-76,106-111).  0 = default (32, the most those launches take),
-   * negative = never.  The session checks once, when it is created, that the device runs such a
-   * launch's workgroups all at once on one XCD, and keeps to one launch per round if not. */
+  /* Tree-LSTM, H = 512, batches whose message flow is a forest: the rounds from the first one on
+   * whose rows can be dealt to eight groups, whole trees of the message flow per group, with at
+   * most this many rows per group (the last forward rounds, the first backward rounds) run as one launch per
+   * direction (cavs_treelstm_tail_fwd / _bwd) instead of one launch per round
+   * (cavs/midend/statement.cc:69-76,106-111).  0 = default (32: larger shares were measured no faster
+   * than launches of their own), negative = never.  The session
+   * checks once, when it is created, that the device runs such a launch's workgroups all at once,
+   * each group on one XCD, and keeps to one launch per round if not. */
   int tail_rows;
 } cavs_session_config;
 

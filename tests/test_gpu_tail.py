@@ -78,7 +78,9 @@ def sync_block(g):
 def plan_groups(offs, sizes, child, ngroups, backward=False):
     """Deals the rows of the rounds (first slab rows `offs`, `sizes` rows each, in the order they
     run) to `ngroups` groups, whole trees of the message flow among those rows per group, and
-    returns (rows, nrounds [8], start [8 * R], count [8 * R]) as the tail entry points take them."""
+    returns (rows, nrounds [8], start, count, flags, max lists per group) as the tail entry points
+    take them.  A group's share of a round goes into lists of at most 32 rows: the first waits for
+    the group's earlier rounds, the last is an arrival."""
     R = len(sizes)
     lo = min(offs)
     comp = {}
@@ -94,22 +96,29 @@ def plan_groups(offs, sizes, child, ngroups, backward=False):
                 if c >= lo:
                     comp[c] = comp[b]
     group_of = [c % ngroups for c in range(ncomp)]
-    rows, nrounds = [], np.zeros(8, np.int32)
-    start, count = np.zeros(8 * R, np.int32), np.zeros(8 * R, np.int32)
+    lists = [[] for _ in range(8)]  # per group: (rows, flags)
     for gi in range(ngroups):
+        arrived = 0
         for k in range(R):
             mine = [b for b in range(offs[k], offs[k] + sizes[k]) if group_of[comp[b]] == gi]
-            if not mine:
-                continue
-            start[gi * R + nrounds[gi]], count[gi * R + nrounds[gi]] = len(rows), len(mine)
-            nrounds[gi] += 1
+            for c0 in range(0, len(mine), 32):
+                last = c0 + 32 >= len(mine)
+                lists[gi].append((mine[c0: c0 + 32], ((arrived if c0 == 0 else 0) << 1) | int(last)))
+            arrived += 1 if mine else 0
+    maxr = max(1, max(len(l) for l in lists))
+    rows, nrounds = [], np.zeros(8, np.int32)
+    start, count, flags = np.zeros(8 * maxr, np.int32), np.zeros(8 * maxr, np.int32), np.zeros(8 * maxr, np.int32)
+    for gi in range(8):
+        nrounds[gi] = len(lists[gi])
+        for i, (mine, fl) in enumerate(lists[gi]):
+            start[gi * maxr + i], count[gi * maxr + i], flags[gi * maxr + i] = len(rows), len(mine), fl
             rows.extend(mine)
-    return np.asarray(rows, np.int32), nrounds, start, count
+    return np.asarray(rows, np.int32), nrounds, start, count, flags, maxr
 
 
 @pytest.mark.parametrize("sizes,base,ngroups", [((30, 22, 13, 6, 3, 1, 1), 300, 1), ((32, 32, 17), 200, 1), ((5,), 40, 1), ((1, 1, 1, 1), 9, 8),
                                                 ((16, 8, 4, 4, 2, 2, 1), 64, 3), ((166, 111, 76, 60, 43, 30, 22, 13, 6, 3, 1, 1), 700, 8),
-                                                ((30, 22, 13, 6, 3, 1, 1), 300, 8)])
+                                                ((30, 22, 13, 6, 3, 1, 1), 300, 8), ((100, 70, 33, 5), 400, 1), ((425, 252, 166, 111, 76, 40, 9, 2), 1300, 8)])
 def test_forward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base, ngroups):
     r = rng(1000 * len(sizes) + sum(sizes))
     U = (r.bulk_normal(4 * H * H) / np.sqrt(H)).astype(np.float32)
@@ -121,9 +130,9 @@ def test_forward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base, 
     pool0 = (r.bulk_normal(N * 2 * H).reshape(N, 2 * H) * 0.5).astype(np.float32)
     d_child, d_pair, d_out = g.devi(child), g.devi(pair), g.devi(out_rows)
     d_xW, d_bias = g.devf(r.bulk_normal(N * 4 * H)), g.devf(r.bulk_normal(4 * H) * 0.1)
-    rows, nrounds, start, count = plan_groups(offs, sizes, child, ngroups)
+    rows, nrounds, start, count, flags, maxr = plan_groups(offs, sizes, child, ngroups)
     assert count.max() <= 32
-    d_tail_rows = g.devi(rows)
+    d_tail_rows, flags_ptr = g.devi(rows), flags.ctypes.data
     outs = []
     for tail in (False, True):
         pool = g.devf(pool0)
@@ -133,7 +142,7 @@ def test_forward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base, 
             sync = sync_block(g)
             g.call("cavs_treelstm_tail_fwd", g.P(pool), g.P(d_child), g.P(d_pair), g.P(d_xW), 4 * H, g.P(Upk), g.P(d_bias), g.P(G),
                    g.P(hlr), g.P(gates), g.P(msg), g.P(go), g.P(d_out), g.P(d_tail_rows), ngroups, nrounds.ctypes.data, start.ctypes.data,
-                   count.ctypes.data, len(sizes), H, g.P(sync), 1 << 20, 0, g.stream())
+                   count.ctypes.data, flags_ptr, maxr, H, g.P(sync), 1 << 20, 0, g.stream())
             assert not g.host(sync).any(), "sync words after a completed launch"
         else:
             # (a round of more than 32 rows as slices of at most 32: the per-round launch then runs on
@@ -157,7 +166,8 @@ def test_forward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base, 
 @pytest.mark.parametrize("sizes,base,leaves,ngroups", [((1, 1, 3, 6, 13, 22, 30), 300, 200, 1), ((17, 32, 32), 200, 120, 1), ((5,), 40, 40, 1),
                                                       ((1, 1, 1, 1), 9, 5, 8), ((1, 2, 2, 4, 4, 8, 16), 64, 30, 3),
                                                       ((1, 1, 3, 6, 13, 22, 30, 43, 60, 76, 111, 166), 700, 400, 8),
-                                                      ((1, 1, 3, 6, 13, 22, 30), 300, 200, 8)])
+                                                      ((1, 1, 3, 6, 13, 22, 30), 300, 200, 8), ((5, 33, 70, 100), 400, 200, 1),
+                                                      ((2, 9, 40, 76, 111, 166, 252, 425), 1300, 800, 8)])
 def test_backward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base, leaves, ngroups):
     """`sizes` lists the rounds in the order the backward pass runs them (roots first); in slab
     order they are the last rounds of the batch, smallest last."""
@@ -174,9 +184,9 @@ def test_backward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base,
     taken = set(int(k) for k in kids if k >= 0)
     orphans = np.array([v for v in range(N) if v not in taken], np.int32)  # nobody's child: their gradients come first
     d_orph = g.devi(orphans)
-    rows, nrounds, start, count = plan_groups(offs, sizes, kids, ngroups, backward=True)
+    rows, nrounds, start, count, flags, maxr = plan_groups(offs, sizes, kids, ngroups, backward=True)
     assert count.max() <= 32
-    d_tail_rows = g.devi(rows)
+    d_tail_rows, flags_ptr = g.devi(rows), flags.ctypes.data
     outs = []
     for tail in (False, True):
         dxW, dF, dc = g.zeros(N, 4 * H, fill=-3.0), g.zeros(2 * N, H, fill=-3.0), g.zeros(N, H, fill=-3.0)
@@ -185,7 +195,7 @@ def test_backward_tail_equals_the_per_round_launches_bit_for_bit(g, sizes, base,
         if tail:
             sync = sync_block(g)
             g.call("cavs_treelstm_tail_bwd", g.P(dxW), 4 * H, g.P(dF), g.P(dc), g.P(UTp), g.P(d_kids), g.P(d_gates), g.P(d_G), g.P(d_dgo),
-                   g.P(d_rows), leaves, g.P(d_tail_rows), ngroups, nrounds.ctypes.data, start.ctypes.data, count.ctypes.data, len(sizes), H,
+                   g.P(d_rows), leaves, g.P(d_tail_rows), ngroups, nrounds.ctypes.data, start.ctypes.data, count.ctypes.data, flags_ptr, maxr, H,
                    g.P(sync), 1 << 20, 0, g.stream())
             assert not g.host(sync).any(), "sync words after a completed launch"
         else:
@@ -212,14 +222,14 @@ def test_a_wait_that_cannot_complete_gives_up_and_every_wave_leaves(g):
     d_child, d_pair, d_out = g.devi(child), g.devi(pair), g.devi(np.arange(N, dtype=np.int32))
     d_xW, d_bias = g.devf(r.bulk_normal(N * 4 * H)), g.devf(np.zeros(4 * H))
     pool0 = (r.bulk_normal(N * 2 * H).reshape(N, 2 * H) * 0.5).astype(np.float32)
-    rows, nrounds, start, count = plan_groups(offs, sizes, child, 2)
+    rows, nrounds, start, count, _, maxr = plan_groups(offs, sizes, child, 2)
     d_tail_rows = g.devi(rows)
 
     def run(sync, extra, spins):
         pool = g.devf(pool0)
         G, hlr, gates = g.zeros(2 * N, 2 * H), g.zeros(N, H), g.zeros(N, 6 * H)
         g.call("cavs_treelstm_tail_fwd", g.P(pool), g.P(d_child), g.P(d_pair), g.P(d_xW), 4 * H, g.P(Upk), g.P(d_bias), g.P(G), g.P(hlr),
-               g.P(gates), None, None, None, g.P(d_tail_rows), 2, nrounds.ctypes.data, start.ctypes.data, count.ctypes.data, len(sizes), H,
+               g.P(gates), None, None, None, g.P(d_tail_rows), 2, nrounds.ctypes.data, start.ctypes.data, count.ctypes.data, None, maxr, H,
                g.P(sync), spins, extra, g.stream())
         return g.host(pool), g.host(gates)
 
@@ -247,13 +257,17 @@ def test_tail_entry_points_reject_what_they_cannot_run():
     one, zero, big = np.asarray([1], np.int32), np.asarray([0], np.int32), np.asarray([40], np.int32)
     with pytest.raises(hip.CavsError, match="1..32 rows"):
         hip.call("cavs_treelstm_tail_fwd", 16, 16, 16, 16, 4 * H, 16, 16, 16, 16, 16, None, None, None, 16, 1, one.ctypes.data, zero.ctypes.data,
-                 big.ctypes.data, 1, H, 16, 10, 0, None)
+                 big.ctypes.data, None, 1, H, 16, 10, 0, None)
+    waits = np.asarray([2], np.int32)  # the only list waits for an arrival nobody makes
+    with pytest.raises(hip.CavsError, match="waits for 1 arrivals"):
+        hip.call("cavs_treelstm_tail_fwd", 16, 16, 16, 16, 4 * H, 16, 16, 16, 16, 16, None, None, None, 16, 1, one.ctypes.data, zero.ctypes.data,
+                 one.ctypes.data, waits.ctypes.data, 1, H, 16, 10, 0, None)
     with pytest.raises(hip.CavsError, match="H = 512"):
         hip.call("cavs_treelstm_tail_bwd", 16, 4 * 256, 16, 16, 16, 16, 16, 16, 16, 16, 0, 16, 1, one.ctypes.data, zero.ctypes.data,
-                 one.ctypes.data, 1, 256, 16, 10, 0, None)
+                 one.ctypes.data, None, 1, 256, 16, 10, 0, None)
     with pytest.raises(hip.CavsError, match="1..8 groups"):
         hip.call("cavs_treelstm_tail_bwd", 16, 4 * H, 16, 16, 16, 16, 16, 16, 16, 16, 0, 16, 9, one.ctypes.data, zero.ctypes.data,
-                 one.ctypes.data, 1, H, 16, 10, 0, None)
+                 one.ctypes.data, None, 1, H, 16, 10, 0, None)
 
 
 @pytest.mark.parametrize("pairing", ["rowid", "reference"])
