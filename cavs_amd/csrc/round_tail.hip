@@ -37,6 +37,10 @@ constexpr int kTailMaxRounds = 32; // lists per group
 // flags[g][i]: bit 0 -- the group's workgroups tell each other when the list is done (an arrival);
 // the rest -- how many of the group's arrivals must be in before the list starts (0: none, e.g. the
 // second slice of a round that does not fit one list).
+// LDS of the two kernels: the parked partial sums (floats), then five index tables of one int per list position
+constexpr int kTailFwdRed = 8 * 8 * 20 * 16, kTailBwdRed = 8 * 8 * 12 * 16;
+constexpr size_t kTailTabBytes = 5 * sizeof(int) * kTailMaxRounds * kTailRows;
+
 struct TailPlan {
   int nrounds[kTailGroups], arrivals[kTailGroups];
   int start[kTailGroups][kTailMaxRounds];
@@ -290,11 +294,34 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
   if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
   constexpr int H = kTailH, H2 = 2 * H, NP = 5;
   const int ct = blockIdx.x >> 3;  // column tile
-  extern __shared__ float red[];   // [tile][wavefront][product * 4 + row][column]: 8 * 8 * 20 * 16 floats
-  __shared__ int s_child[2][2 * kTailRows], s_row[2][kTailRows], s_pair[2][kTailRows], s_out[2][kTailRows], s_bail;
+  extern __shared__ float red[];   // [tile][wavefront][product * 4 + row][column]: 8 * 8 * 20 * 16 floats, then the index table
+  __shared__ int s_bail;
   const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
   const int x = lane & 15, slot = lane >> 4;
   const int j0 = ct * 16, kb = ks * (H / 8);
+
+  // The group's index table, [what][list][position]: slab row, left and right child, the row of the
+  // pool the message goes to, the row of the graph output (-1 = none, also past a list's end).  Read
+  // from global memory where a round needs them these are chains of two and three dependent loads
+  // on every workgroup's way to the round's barrier; here they are fetched once, under the weights.
+  constexpr int TAB = kTailMaxRounds * kTailRows;
+  int *tab = reinterpret_cast<int *>(red + kTailFwdRed);
+  for (int e = tid; e < nrounds * kTailRows; e += 512) {
+    const int r = e / kTailRows, i = e % kTailRows;
+    int row = -1, cl = -1, cr = -1, dst = -1, out = -1;
+    if (i < a.plan.count[grp][r]) {
+      row = a.rows[a.plan.start[grp][r] + i];
+      cl = a.child[2L * row];
+      cr = a.child[2L * row + 1];
+      dst = a.pair[row];
+      if (a.go) out = a.out_rows[row];
+    }
+    tab[e] = row;
+    tab[TAB + e] = cl;
+    tab[2 * TAB + e] = cr;
+    tab[3 * TAB + e] = dst;
+    tab[4 * TAB + e] = out;
+  }
 
   // this wavefront's weights: k-groups kb/16 .. kb/16 + 3 of column tile ct, four gates
   float4 wi[4], wo[4], wu[4], wf[4];
@@ -323,25 +350,17 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
   const unsigned total = (unsigned)a.plan.arrivals[grp] * a.expect;
   if (tid == 0 && total > 0) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   bool first_wait = true;
+  __syncthreads();
 
   for (int r = 0; r < nrounds; r++) {
-    const int *rows = a.rows + a.plan.start[grp][r];
-    const int n = a.plan.count[grp][r], T = (n + 3) >> 2, par = r & 1;
+    const int n = a.plan.count[grp][r], T = (n + 3) >> 2;
     const int need = a.plan.flags[grp][r] >> 1;
     const bool arrives = a.plan.flags[grp][r] & 1;
-    // what does not depend on the rounds before: the round's lists, the epilogue's x * W
-    if (tid < 64) {
-      s_child[par][tid] = tid < 2 * n ? a.child[2L * rows[tid >> 1] + (tid & 1)] : -1;
-    } else if (tid < 96) {
-      const int row = tid - 64 < n ? rows[tid - 64] : -1;
-      s_row[par][tid - 64] = row;
-      s_pair[par][tid - 64] = row >= 0 ? a.pair[row] : -1;
-    } else if (tid < 128) {
-      s_out[par][tid - 96] = (a.go && tid - 96 < n) ? a.out_rows[rows[tid - 96]] : -1;
-    }
+    const int *rtab = tab + r * kTailRows;
+    // what does not depend on the rounds before: the epilogue's x * W
     const int eb = 4 * ks + (lane >> 4);
     const bool eon = eb < n;
-    const long erow = eon ? rows[eb] : 0;
+    const long erow = eon ? rtab[eb] : 0;
     float xw[4] = {0.f, 0.f, 0.f, 0.f};
     if (eon) {
       const float *p = a.xW + erow * a.ld_xw + ej;
@@ -359,10 +378,10 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
     int e_cl = -1, e_cr = -1, e_dst = -1, e_out = -1;
     float e_hl = 0.f, e_cl_c = 0.f, e_hr = 0.f, e_cr_c = 0.f;
     if (eon) {
-      e_cl = s_child[par][2 * eb];
-      e_cr = s_child[par][2 * eb + 1];
-      e_dst = s_pair[par][eb];
-      e_out = s_out[par][eb];
+      e_cl = rtab[TAB + eb];
+      e_cr = rtab[2 * TAB + eb];
+      e_dst = rtab[3 * TAB + eb];
+      e_out = rtab[4 * TAB + eb];
       if (e_cl >= 0) { e_hl = ld_row(a.pool + (long)e_cl * H2 + ej); e_cl_c = ld_row(a.pool + (long)e_cl * H2 + H + ej); }
       if (e_cr >= 0) { e_hr = ld_row(a.pool + (long)e_cr * H2 + ej); e_cr_c = ld_row(a.pool + (long)e_cr * H2 + H + ej); }
     }
@@ -378,7 +397,7 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_fwd_kernel(TailFwdArgs a
       float4 l, r;
       int cl, cr;
     };
-    auto child_of = [&](int t, int side) { return s_child[par][2 * (4 * (t < T ? t : T - 1) + (lane & 3)) + side]; };
+    auto child_of = [&](int t, int side) { return rtab[(1 + side) * TAB + 4 * (t < T ? t : T - 1) + (lane & 3)]; };
     SlotSums<NP> sums;
     auto park = [&](int t) {
       float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
@@ -503,11 +522,32 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
   if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) return;
   constexpr int H = kTailH, H2 = 2 * H, NP = 3;
   const int ct = blockIdx.x >> 3;
-  extern __shared__ float red[];  // [tile][wavefront][product * 4 + row][column]: 8 * 8 * 12 * 16 floats
-  __shared__ int s_row[2][kTailRows], s_bail;
+  extern __shared__ float red[];  // [tile][wavefront][product * 4 + row][column]: 8 * 8 * 12 * 16 floats, then the index table
+  __shared__ int s_bail;
   const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
   const int x = lane & 15, slot = lane >> 4;
   const int j0 = ct * 16;
+
+  // the group's index table (see the forward kernel): slab row, its two children, the rows of
+  // `dret` that hold the children's gradients from outside (-1 = none, also past a list's end)
+  constexpr int TAB = kTailMaxRounds * kTailRows;
+  int *tab = reinterpret_cast<int *>(red + kTailBwdRed);
+  for (int e = tid; e < nrounds * kTailRows; e += 512) {
+    const int r = e / kTailRows, i = e % kTailRows;
+    int row = -1, k0 = -1, k1 = -1, d0 = -1, d1 = -1;
+    if (i < a.plan.count[grp][r]) {
+      row = a.rows[a.plan.start[grp][r] + i];
+      k0 = a.kids[2L * row];
+      k1 = a.kids[2L * row + 1];
+      if (k0 >= 0) d0 = a.dret_rows[k0];
+      if (k1 >= 0) d1 = a.dret_rows[k1];
+    }
+    tab[e] = row;
+    tab[TAB + e] = k0;
+    tab[2 * TAB + e] = k1;
+    tab[3 * TAB + e] = d0;
+    tab[4 * TAB + e] = d1;
+  }
 
   // weights: twelve k-groups of U_iou^T (K = 3H) and four of U_f^T (K = H) per wavefront
   float4 w0[12], w1[4];
@@ -526,27 +566,28 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
   const unsigned total = (unsigned)a.plan.arrivals[grp] * a.expect;
   if (tid == 0 && total > 0) __hip_atomic_fetch_or(gsync + TAIL_XCC, 1u << xcc_id(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   bool first_wait = true;
+  __syncthreads();
 
   for (int r = 0; r < nrounds; r++) {
-    const int *rows = a.rows + a.plan.start[grp][r];
-    const int n = a.plan.count[grp][r], T = (n + 3) >> 2, par = r & 1;
+    const int n = a.plan.count[grp][r], T = (n + 3) >> 2;
     const int need = a.plan.flags[grp][r] >> 1;
     const bool arrives = a.plan.flags[grp][r] & 1;
-    // (rows past the list's end stand for its first row; their results are not written)
-    if (tid < kTailRows) s_row[par][tid] = rows[tid < n ? tid : 0];
+    const int *rtab = tab + r * kTailRows;
     // the operands of the children's gate gradients: everything except d c of the parent was
     // written before this launch
     const int eb = 4 * ks + (lane >> 4);
     const bool eon = eb < n;
-    const long erow = eon ? rows[eb] : 0;
-    int kc[2] = {-1, -1};
+    const long erow = eon ? rtab[eb] : 0;
+    int kc[2] = {-1, -1}, kdr[2] = {-1, -1};
     float pf[2] = {0.f, 0.f};
     struct Kid {
       float g[6], dr, cl, cr;
     } kid[2];
     if (eon) {
-      kc[0] = a.kids[2 * erow];
-      kc[1] = a.kids[2 * erow + 1];
+      kc[0] = rtab[TAB + eb];
+      kc[1] = rtab[2 * TAB + eb];
+      kdr[0] = rtab[3 * TAB + eb];
+      kdr[1] = rtab[4 * TAB + eb];
       pf[0] = a.gates[erow * 6 * H + 3 * H + ej];
       pf[1] = a.gates[erow * 6 * H + 4 * H + ej];
     }
@@ -561,7 +602,7 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
         const float *g = a.gates + v * 6 * H + ej;
 #pragma unroll
         for (int t = 0; t < 6; t++) kd.g[t] = g[(long)t * H];
-        kd.dr = a.dret[(long)a.dret_rows[v] * H + ej];
+        kd.dr = a.dret[(long)kdr[s] * H + ej];
         if (v >= a.leaf_rows) {
           kd.cl = a.G[(2 * v) * H2 + H + ej];
           kd.cr = a.G[(2 * v + 1) * H2 + H + ej];
@@ -586,7 +627,11 @@ __global__ __launch_bounds__(512, 1) void treelstm_tail_bwd_kernel(TailBwdArgs a
     struct Opnd {
       float4 x[3], fl, fr;
     };
-    auto row_of = [&](int t) { return (long)s_row[par][4 * (t < T ? t : T - 1) + (lane & 3)]; };
+    // (rows past the list's end stand for its first row; their results are not written)
+    auto row_of = [&](int t) {
+      const int i = 4 * (t < T ? t : T - 1) + (lane & 3);
+      return (long)rtab[i < n ? i : 0];
+    };
     SlotSums<NP> sums;
     auto park = [&](int t) {
       float *dst = red + ((t * 8 + ks) * (NP * 4)) * 16 + x;
@@ -761,7 +806,7 @@ size_t cavs_tail_sync_bytes(void) { return (size_t)TAIL_GROUP_WORDS * (kTailGrou
 
 int cavs_tail_probe(unsigned *sync, int H, int spin_max, void *stream) {
   CAVS_REQUIRE(sync && H == kTailH && spin_max >= 0, "cavs_tail_probe: bad arguments (H = %d only)", kTailH);
-  constexpr size_t lds = 8 * 8 * 20 * 16 * sizeof(float);
+  constexpr size_t lds = kTailFwdRed * sizeof(float) + kTailTabBytes;
   static int attr = tail_lds_attr(reinterpret_cast<const void *>(tail_probe_kernel), lds);
   if (attr != CAVS_OK) return attr;
   launch(tail_probe_kernel, dim3(8 * (H / 16)), 512, lds, as_stream(stream), sync, spin_max, H / 16);
@@ -784,7 +829,7 @@ int cavs_treelstm_tail_fwd(float *pool, const int *child, const int *pair, const
                 H / 16 + extra_arrivals, {}};
   const int todo = tail_plan("cavs_treelstm_tail_fwd", ngroups, nrounds, start, count, flags, max_rounds, &a.plan);
   if (todo <= 0) return todo;
-  constexpr size_t lds = 8 * 8 * 20 * 16 * sizeof(float);
+  constexpr size_t lds = kTailFwdRed * sizeof(float) + kTailTabBytes;
   static int attr = tail_lds_attr(reinterpret_cast<const void *>(treelstm_tail_fwd_kernel), lds);
   if (attr != CAVS_OK) return attr;
   launch(treelstm_tail_fwd_kernel, dim3(8 * (H / 16)), 512, lds, as_stream(stream), a);
@@ -807,7 +852,7 @@ int cavs_treelstm_tail_bwd(float *dxW, int ld_dxw, float *dF, float *dc, const f
                 H / 16 + extra_arrivals, {}};
   const int todo = tail_plan("cavs_treelstm_tail_bwd", ngroups, nrounds, start, count, flags, max_rounds, &a.plan);
   if (todo <= 0) return todo;
-  constexpr size_t lds = 8 * 8 * 12 * 16 * sizeof(float);
+  constexpr size_t lds = kTailBwdRed * sizeof(float) + kTailTabBytes;
   static int attr = tail_lds_attr(reinterpret_cast<const void *>(treelstm_tail_bwd_kernel), lds);
   if (attr != CAVS_OK) return attr;
   launch(treelstm_tail_bwd_kernel, dim3(8 * (H / 16)), 512, lds, as_stream(stream), a);
