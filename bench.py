@@ -173,9 +173,10 @@ class StepClock:
             self.hip.call("cavs_event_destroy", e)
 
 
-def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, profile=True):
+def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, profile=True, graph_replay=False):
     """Times `steps` training steps of one workload and returns the fields of the JSON line.
-    schedule / plan_cache: who builds the round schedule and whether plans are cached
+    schedule / plan_cache / graph_replay: who builds the round schedule, whether plans are cached, and whether
+    a cached plan's launches are replayed from a recorded graph
     (cavs_session_config); profile=False skips the per-kernel-class pass."""
     import torch
 
@@ -186,7 +187,7 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
     kw = model_kwargs(w0)
     s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
                         opt=session.OPT_BATCHING, fused_round_rows=a.fused_round_rows, schedule=schedule,
-                        plan_cache=plan_cache, tail_rows=a.tail_rows, **kw)
+                        plan_cache=plan_cache, tail_rows=a.tail_rows, graph_replay=graph_replay, **kw)
     s.set_params(w0["params"])
     feeds = []
     for w in pool:  # inputs resident in HBM before the timed region
@@ -240,6 +241,8 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
                "median_ms_per_step": round(median_ms, 4), "GraphParsing_ms": host_ms["GraphParsing_median"],
                "HostSchedule_ms": host_ms["HostSchedule"], "plan_hits": s.counter("plan_hits"),
                "plan_misses": s.counter("plan_misses")}
+        if graph_replay:
+            out["graph_replays"] = s.counter("graph_replays")
         s.close()
         del feeds
         torch.cuda.empty_cache()
@@ -386,8 +389,10 @@ def main():
         # who builds the round schedule and the index lists: the host scheduler (the headline above),
         # the GPU (cavs_schedule_arena), or the plan cache replaying a structure seen before
         modes = {}
-        for name, sched, cache in (("host", "host", 0), ("device", "device", 0), ("cached", "host", a.pool)):
-            modes[name], _ = measure(a, a.workload, a.steps, a.warmup, a.pool, schedule=sched, plan_cache=cache, profile=False)
+        for name, sched, cache, replay in (("host", "host", 0, False), ("device", "device", 0, False), ("cached", "host", a.pool, False),
+                                           ("cached_replay", "host", a.pool, True)):
+            modes[name], _ = measure(a, a.workload, a.steps, a.warmup, a.pool, schedule=sched, plan_cache=cache, profile=False,
+                                     graph_replay=replay)
         out["schedule_modes"] = modes
         out["timers_ms"]["GraphParsing_by_mode"] = {k: v["GraphParsing_ms"] for k, v in modes.items()}
     if a.also.lower() != "none":
@@ -402,9 +407,13 @@ def main():
                                                       "config", "roofline", "kernels")}
             if not a.no_schedule_modes:  # the same steps with the lists built on the GPU
                 dev, _ = measure(a, name, steps, warm, npool, schedule="device", profile=False)
+                hit, _ = measure(a, name, steps, warm, npool, plan_cache=npool, profile=False)
+                rep, _ = measure(a, name, steps, warm, npool, plan_cache=npool, profile=False, graph_replay=True)
+                keys = ("value", "ms_per_step", "median_ms_per_step", "GraphParsing_ms")
                 out["also"][name]["schedule_modes"] = {
                     "host": {k: also[k] for k in ("value", "ms_per_step", "median_ms_per_step")},
-                    "device": {k: dev[k] for k in ("value", "ms_per_step", "median_ms_per_step", "GraphParsing_ms")}}
+                    "device": {k: dev[k] for k in keys}, "cached": {k: hit[k] for k in keys},
+                    "cached_replay": {k: rep[k] for k in keys}}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(w0)
     print(json.dumps(out))

@@ -207,6 +207,50 @@ int cavs_event_elapsed_ms(float *ms, void *start, void *stop) {
   return CAVS_OK;
 }
 
+int cavs_graph_capture_begin(void *stream) {
+  CAVS_REQUIRE(stream, "cavs_graph_capture_begin: the default stream cannot be captured");
+  // relaxed: other threads of the process (an allocator, another session) may go on calling the runtime
+  CAVS_HIP_TRY(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+  return CAVS_OK;
+}
+
+int cavs_graph_capture_end(void *stream, void **graph_exec) {
+  CAVS_REQUIRE(stream, "cavs_graph_capture_end: null stream");
+  hipGraph_t graph = nullptr;
+  const hipError_t rc = hipStreamEndCapture(as_stream(stream), &graph);
+  if (!graph_exec) {  // the caller gives the capture up
+    if (graph) (void)hipGraphDestroy(graph);
+    (void)hipGetLastError();
+    return CAVS_OK;
+  }
+  *graph_exec = nullptr;
+  if (rc != hipSuccess || !graph) {
+    (void)hipGetLastError();
+    if (graph) (void)hipGraphDestroy(graph);
+    return cavs::set_error(CAVS_EHIP, "cavs_graph_capture_end: the capture was invalidated (%s)", hipGetErrorString(rc));
+  }
+  hipGraphExec_t exec = nullptr;
+  const hipError_t ri = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  if (ri != hipSuccess) {
+    (void)hipGetLastError();
+    return cavs::set_error(CAVS_EHIP, "cavs_graph_capture_end: hipGraphInstantiate: %s", hipGetErrorString(ri));
+  }
+  *graph_exec = exec;
+  return CAVS_OK;
+}
+
+int cavs_graph_launch(void *graph_exec, void *stream) {
+  CAVS_REQUIRE(graph_exec, "cavs_graph_launch: null graph");
+  CAVS_HIP_TRY(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+  return CAVS_OK;
+}
+
+int cavs_graph_destroy(void *graph_exec) {
+  if (graph_exec) CAVS_HIP_TRY(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+  return CAVS_OK;
+}
+
 int cavs_profile_arm(void *start_event, void *stop_event) {
   CAVS_REQUIRE(start_event && stop_event, "cavs_profile_arm: null event");
   LaunchProbe &p = launch_probe();

@@ -64,6 +64,10 @@ _SIGS = {
     "cavs_event_create": [C.POINTER(_P)],
     "cavs_event_destroy": [_P],
     "cavs_event_record": [_P, _P],
+    "cavs_graph_capture_begin": [_P],
+    "cavs_graph_capture_end": [_P, C.POINTER(_P)],
+    "cavs_graph_launch": [_P, _P],
+    "cavs_graph_destroy": [_P],
     "cavs_event_sync": [_P],
     "cavs_event_elapsed_ms": [C.POINTER(_F), _P, _P],
     "cavs_gather_rows": [_P, _I, _P, _I, _P, _I, _I, _P],

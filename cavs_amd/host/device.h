@@ -4,7 +4,9 @@
 #ifndef CAVS_HOST_DEVICE_H_
 #define CAVS_HOST_DEVICE_H_
 
+#include <atomic>
 #include <cstddef>
+#include <cstdint>
 #include <stdexcept>
 #include <string>
 #include <utility>
@@ -24,6 +26,13 @@ inline void check(int rc) {
 
 [[noreturn]] inline void fail(int code, const std::string &msg) { throw Error(code, msg); }
 
+// Counts the times any DeviceArray let go of its storage: whoever keeps device addresses beyond a
+// call (a recorded graph of launches) compares the count it saw with the current one.
+inline std::atomic<uint64_t> &device_array_epoch() {
+  static std::atomic<uint64_t> epoch{0};
+  return epoch;
+}
+
 // Device array that only ever grows; contents are not preserved across growth
 // (the reference's TensorBuffer::Resize behaves the same, cavs/midend/tensor.cc:44-50).
 template <typename T>
@@ -32,10 +41,14 @@ class DeviceArray {
   DeviceArray() = default;
   DeviceArray(const DeviceArray &) = delete;
   DeviceArray &operator=(const DeviceArray &) = delete;
-  ~DeviceArray() { cavs_free(p_); }
+  ~DeviceArray() {
+    if (p_) device_array_epoch()++;
+    cavs_free(p_);
+  }
   // returns true when the storage was reallocated
   bool reserve(size_t n) {
     if (n <= cap_) return false;
+    if (p_) device_array_epoch()++;
     check(cavs_free(p_));
     p_ = nullptr;
     cap_ = 0;
@@ -48,7 +61,7 @@ class DeviceArray {
   T *get() const { return p_; }
   size_t capacity() const { return cap_; }
   T *at(size_t i) const { return p_ + i; }
-  void swap(DeviceArray &o) {
+  void swap(DeviceArray &o) {  // (no storage is let go of)
     std::swap(p_, o.p_);
     std::swap(cap_, o.cap_);
   }

@@ -104,7 +104,7 @@ void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
   const int lim = tail_limit();
   const Schedule &s = *sched_;
   const int R = (int)s.rounds.size(), N = s.N, G = cavs_tail_max_groups(), cap = cavs_tail_max_rounds(), slice = 32;
-  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || Upk_.capacity() == 0 || !cavs_tail_rounds_ok(1, cfg_.H)) return;
+  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || !cavs_round_packed_ok(1, cfg_.H) || !cavs_tail_rounds_ok(1, cfg_.H)) return;
   int k0 = 1;
   while (k0 < R && (s.rounds[k0].n > G * lim || leaf_round(s.rounds[k0]))) k0++;
   std::vector<int> comp, weight, group, order, per;
@@ -212,6 +212,7 @@ void Engine::tail_check() {
   // every launch since the one that gave up left at once, and every parameter update watched the
   // word: the parameters are those of the last good step.  From here on: one launch per round.
   tail_ready_ = false;
+  state_epoch_++;
   upk_valid_ = wfct_valid_ = false;
   emb_sparse_valid_ = false;
   check(cavs_zero(tail_sync_.get(), cavs_tail_sync_bytes(), stream_));
@@ -261,6 +262,7 @@ void Engine::bind_param(const std::string &name, float *w, float *g) {
   Param &p = param(name);
   if (!w) fail(CAVS_EINVAL, "bind_param('" + name + "'): null weight pointer");
   if (p.w != w) upk_valid_ = wfct_valid_ = false;
+  state_epoch_++;
   p.w = w;
   p.g = g ? g : p.own_g.get();
 }
@@ -301,6 +303,7 @@ void Engine::set_param(const std::string &name, const float *host, size_t n) {
   check(cavs_memcpy_h2d(p.w, host, n * 4, stream_));
   check(cavs_stream_sync(stream_));
   upk_valid_ = wfct_valid_ = false;
+  state_epoch_++;
 }
 
 void Engine::get_param(const std::string &name, float *host, size_t n, bool grad) {
@@ -586,6 +589,7 @@ void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
       if (plans_[i]->last_used < plans_[lru]->last_used) lru = i;
     check(cavs_stream_sync(stream_));
     p = std::move(plans_[lru]);
+    p->drop_graphs();
     plans_.erase(plans_.begin() + lru);
   } else {
     p = std::make_unique<Plan>();
@@ -770,6 +774,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     hash = hash_feed(graph, (size_t)B * maxlen, B, maxlen, cfg_.pairing);
     hit = find_plan(graph, B, maxlen, hash);
   }
+  hit_plan_ = hit;
   if (hit) {
     // a batch structure seen before: its schedule and its lists are where the last such step left them
     hit->last_used = ++plan_clock_;
@@ -811,6 +816,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
 }
 
 void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out) {
+  state_epoch_++;
   begin_step(graph, B, maxlen);
   if ((cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x) && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
   d_x_ = x_dev;
@@ -835,6 +841,7 @@ void Engine::update_bias_jobs(float lr, std::vector<cavs_task> *out, std::vector
 
 void Engine::backward_only(const float *dgraph_out, bool settle_biases) {
   if (!dgraph_out || N_ == 0) fail(CAVS_EINVAL, "backward_only needs d graph_out of a forward pass");
+  state_epoch_++;
   d_dgo_ = dgraph_out;
   check(cavs_event_record(ev_[2], stream_));
   switch (cfg_.model) {
@@ -845,6 +852,103 @@ void Engine::backward_only(const float *dgraph_out, bool settle_biases) {
   if (settle_biases) settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
   check(cavs_event_record(ev_[3], stream_));
   ev_bwd_valid_ = true;
+}
+
+// The forward rounds, the loss head and the backward rounds of a step (everything between the
+// feeds and the parameter update).  While a graph is being recorded the timing events stay out of it.
+void Engine::run_passes(bool backward) {
+  if (!capturing_) check(cavs_event_record(ev_[0], stream_));
+  fwd_out_ = GO_.get();
+  out_folded_ = false;
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
+    case CAVS_MODEL_LSTM: lstm_forward(); break;
+    default: treefc_forward();
+  }
+  pop_ret(GO_.get());
+  if (!capturing_) check(cavs_event_record(ev_[1], stream_));
+  ev_valid_ = !capturing_;
+  head_forward_backward(backward);
+  d_dgo_ = dGO_.get();
+  did_backward_ = backward;
+  ev_bwd_valid_ = false;
+  if (backward) {
+    if (!capturing_) check(cavs_event_record(ev_[2], stream_));
+    switch (cfg_.model) {
+      case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
+      case CAVS_MODEL_LSTM: lstm_backward(); break;
+      default: treefc_backward();
+    }
+    if (!capturing_) check(cavs_event_record(ev_[3], stream_));
+    ev_bwd_valid_ = !capturing_;
+  }
+}
+
+Engine::StepSig Engine::step_signature(const void *x, const void *labels, bool backward) const {
+  StepSig g;
+  g.x = x;
+  g.labels = labels;
+  g.xs = xs_.get();
+  g.xs_prev = xs_prev_.get();
+  g.backward = backward;
+  g.emb_sparse_valid = emb_sparse_valid_;
+  g.emb_cleared = emb_cleared_;
+  g.upk_valid = upk_valid_;
+  g.wfct_valid = wfct_valid_;
+  g.emb_dirty_n = emb_dirty_n_;
+  g.pairing = cfg_.pairing;
+  g.e_ones_rows = e_ones_rows_;
+  g.alloc_epoch = device_array_epoch().load();
+  g.state_epoch = state_epoch_;
+  return g;
+}
+
+Engine::StepState Engine::step_state() const {
+  StepState st;
+  st.did_backward = did_backward_;
+  st.out_folded = out_folded_;
+  st.emb_sparse_valid = emb_sparse_valid_;
+  st.emb_cleared = emb_cleared_;
+  st.upk_valid = upk_valid_;
+  st.wfct_valid = wfct_valid_;
+  st.tail_pending = tail_pending_;
+  st.fwd_out = fwd_out_;
+  st.d_dgo = d_dgo_;
+  st.xs = xs_.get();
+  st.emb_dirty_n = emb_dirty_n_;
+  st.bias_jobs = bias_jobs_;
+  st.pending_tasks = pending_tasks_;
+  const double c[10] = {c_round_flops_, c_gather_rows_, c_scatter_rows_, c_gemm_flops_, c_gemm_flops_hinted_,
+                        c_launches_,    c_gather_bytes_, c_scatter_bytes_, c_tail_rounds_, c_tail_launches_};
+  std::copy(c, c + 10, st.counters);
+  return st;
+}
+
+void Engine::restore_step_state(const StepState &st) {
+  did_backward_ = st.did_backward;
+  out_folded_ = st.out_folded;
+  emb_sparse_valid_ = st.emb_sparse_valid;
+  emb_cleared_ = st.emb_cleared;
+  upk_valid_ = st.upk_valid;
+  wfct_valid_ = st.wfct_valid;
+  tail_pending_ = tail_pending_ || st.tail_pending;
+  fwd_out_ = st.fwd_out;
+  d_dgo_ = st.d_dgo;
+  if (xs_.get() != st.xs) xs_.swap(xs_prev_);
+  emb_dirty_n_ = st.emb_dirty_n;
+  bias_jobs_ = st.bias_jobs;
+  pending_tasks_ = st.pending_tasks;
+  c_round_flops_ = st.counters[0];
+  c_gather_rows_ = st.counters[1];
+  c_scatter_rows_ = st.counters[2];
+  c_gemm_flops_ = st.counters[3];
+  c_gemm_flops_hinted_ = st.counters[4];
+  c_launches_ = st.counters[5];
+  c_gather_bytes_ = st.counters[6];
+  c_scatter_bytes_ = st.counters[7];
+  c_tail_rounds_ = st.counters[8];
+  c_tail_launches_ = st.counters[9];
+  ev_valid_ = ev_bwd_valid_ = false;
 }
 
 void Engine::step(const int *graph, int B, int maxlen, const void *x, const void *labels,
@@ -879,30 +983,56 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     check(cavs_stream_sync(stream_));
   }
 
-  check(cavs_event_record(ev_[0], stream_));
-  fwd_out_ = GO_.get();
-  out_folded_ = false;
-  switch (cfg_.model) {
-    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
-    case CAVS_MODEL_LSTM: lstm_forward(); break;
-    default: treefc_forward();
+  // A batch structure seen before, on the same feed buffers, with the session in the state it was
+  // in the last time: the passes below as one recorded graph of launches.
+  Plan *plan = hit_plan_;
+  const bool may_replay = cfg_.graph_replay && plan && on_device && !profile_ && pending_tasks_.empty() && !plan->graph_off;
+  StepGraph *recorded = nullptr;
+  bool record = false;
+  StepSig sig;
+  if (may_replay) {
+    sig = step_signature(x, labels, backward);
+    for (StepGraph &g : plan->graphs)
+      if (g.sig == sig) recorded = &g;
+    // (a plan whose signatures keep changing -- new feed buffers every step -- stops recording)
+    if (!recorded) record = plan->recordings++ < 6;
   }
-  pop_ret(GO_.get());
-  check(cavs_event_record(ev_[1], stream_));
-  ev_valid_ = true;
-  head_forward_backward(backward);
-  d_dgo_ = dGO_.get();
-  did_backward_ = backward;
-  ev_bwd_valid_ = false;
-  if (backward) {
-    check(cavs_event_record(ev_[2], stream_));
-    switch (cfg_.model) {
-      case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
-      case CAVS_MODEL_LSTM: lstm_backward(); break;
-      default: treefc_backward();
+  if (recorded) {
+    check(cavs_graph_launch(recorded->exec, stream_));
+    restore_step_state(recorded->after);
+    c_graph_replays_ += 1;
+  } else if (record) {
+    const StepState before = step_state();
+    void *exec = nullptr;
+    bool ok = false;
+    check(cavs_graph_capture_begin(stream_));
+    capturing_ = true;
+    try {
+      run_passes(backward);
+      capturing_ = false;
+      check(cavs_graph_capture_end(stream_, &exec));
+      ok = true;
+    } catch (const Error &) {  // something in there had to wait for the stream (a buffer that grew): not this time
+      if (capturing_) cavs_graph_capture_end(stream_, nullptr);
+      capturing_ = false;
     }
-    check(cavs_event_record(ev_[3], stream_));
-    ev_bwd_valid_ = true;
+    if (ok) {
+      if (plan->graphs.size() >= 4) {
+        cavs_graph_destroy(plan->graphs.front().exec);
+        plan->graphs.erase(plan->graphs.begin());
+      }
+      plan->graphs.push_back({exec, sig, step_state()});
+      check(cavs_graph_launch(exec, stream_));  // (recording enqueued nothing)
+      c_graph_replays_ += 1;
+    } else {
+      restore_step_state(before);
+      plan->graph_off = true;
+      run_passes(backward);
+    }
+  } else {
+    run_passes(backward);
+  }
+  if (backward) {
     if (lr != 0.f) {
       // w -= lr * g (cavs/backend/op_impl_sgd.cu); the embedding table by its looked-up rows
       // only: every other row of its gradient is zero, so the dense update would not move it
@@ -1711,6 +1841,7 @@ double Engine::counter(const std::string &key) const {
   if (key == "tail_lists_max") return (double)tail_.lists_max;
   if (key == "tail_tiles_max") return (double)tail_.tiles_max;
   if (key == "tail_vertices") return tail_.vertices;
+  if (key == "graph_replays") return c_graph_replays_;
   if (key == "plan_hits") return c_plan_hits_;
   if (key == "plan_misses") return c_plan_misses_;
   fail(CAVS_EINVAL, "unknown counter '" + key + "'");

@@ -37,6 +37,7 @@ class Engine {
   void bind_param(const std::string &name, float *w, float *g);
   // where the next backward pass leaves the gradient of `name` (null: the engine's own buffer)
   void bind_param_grad(const std::string &name, float *g) {
+    state_epoch_++;
     Param &p = param(name);
     p.g = g ? g : p.own_g.get();
   }
@@ -60,7 +61,10 @@ class Engine {
   void update_bias_jobs(float lr, std::vector<cavs_task> *out, std::vector<const float *> *updated);
   // A job for the launch that opens the next backward pass (it runs before anything of that pass).
   void queue_prologue_task(const cavs_task &t) { pending_tasks_.push_back(t); }
-  void set_pairing(int pairing) { cfg_.pairing = pairing; }
+  void set_pairing(int pairing) {
+    if (pairing != cfg_.pairing) state_epoch_++;
+    cfg_.pairing = pairing;
+  }
   void set_param(const std::string &name, const float *host, size_t n);
   void get_param(const std::string &name, float *host, size_t n, bool grad);
   void step(const int *graph, int B, int maxlen, const void *x, const void *labels,
@@ -194,7 +198,67 @@ class Engine {
   // ---- plan cache (cfg.plan_cache entries): the schedule and the device lists of a graph feed,
   // keyed by the feed's bytes, so that a batch structure seen before costs neither the scheduler
   // nor an upload
+  // ---- replay of a cached plan's launches (cfg.graph_replay): the forward pass, the loss head and
+  // the backward pass of a step as one recorded graph.  What such a graph does depends on more than
+  // the batch structure: on the feed buffers and on the state the session was in when the step began
+  // (which rows of the embedding gradient are dirty, whether the repacked weights are current, which
+  // of the two id buffers is this step's ...).  StepSig is all of that, StepState is what the
+  // recorded step left behind on the host; a graph is replayed only under an equal signature and the
+  // state it left is then put in place as if the launches had been issued one by one.
+  struct StepSig {
+    const void *x = nullptr, *labels = nullptr, *xs = nullptr, *xs_prev = nullptr;
+    bool backward = false, emb_sparse_valid = false, emb_cleared = false, upk_valid = false, wfct_valid = false;
+    int emb_dirty_n = 0, pairing = 0;
+    size_t e_ones_rows = 0;
+    uint64_t alloc_epoch = 0, state_epoch = 0;
+    bool operator==(const StepSig &o) const {
+      return x == o.x && labels == o.labels && xs == o.xs && xs_prev == o.xs_prev && backward == o.backward &&
+             emb_sparse_valid == o.emb_sparse_valid && emb_cleared == o.emb_cleared && upk_valid == o.upk_valid &&
+             wfct_valid == o.wfct_valid && emb_dirty_n == o.emb_dirty_n && pairing == o.pairing && e_ones_rows == o.e_ones_rows &&
+             alloc_epoch == o.alloc_epoch && state_epoch == o.state_epoch;
+    }
+  };
+  struct BiasJob {
+    std::string param;
+    const float *src;
+    int parts;
+    long long bw, nb, map;
+  };
+  struct StepState {
+    bool did_backward = false, out_folded = false, emb_sparse_valid = false, emb_cleared = false, upk_valid = false,
+         wfct_valid = false, tail_pending = false;
+    float *fwd_out = nullptr;
+    const float *d_dgo = nullptr;
+    const void *xs = nullptr;
+    int emb_dirty_n = 0;
+    std::vector<BiasJob> bias_jobs;
+    std::vector<cavs_task> pending_tasks;
+    double counters[10] = {0};
+  };
+  struct StepGraph {
+    void *exec = nullptr;
+    StepSig sig;
+    StepState after;
+  };
+  StepSig step_signature(const void *x, const void *labels, bool backward) const;
+  StepState step_state() const;
+  void restore_step_state(const StepState &st);
+  void run_passes(bool backward);  // forward rounds, loss head, backward rounds of a step
+  bool capturing_ = false;
+  uint64_t state_epoch_ = 0;  // bumped by every call other than step() that changes what a step enqueues
+  double c_graph_replays_ = 0;
+
   struct Plan {
+    ~Plan() { drop_graphs(); }
+    void drop_graphs() {
+      for (StepGraph &g : graphs) cavs_graph_destroy(g.exec);
+      graphs.clear();
+      graph_off = false;
+      recordings = 0;
+    }
+    std::vector<StepGraph> graphs;
+    bool graph_off = false;  // recording failed once: ordinary steps from then on
+    int recordings = 0;
     uint64_t hash = 0;
     int B = 0, maxlen = 0, pairing = 0;
     std::vector<int32_t> graph;
@@ -210,6 +274,7 @@ class Engine {
   uint64_t plan_clock_ = 0;
   double c_plan_hits_ = 0, c_plan_misses_ = 0;
   int scheduler_used_ = 0;  // who produced the last step's lists: 0 host scheduler, 1 device scheduler, 2 plan cache
+  Plan *hit_plan_ = nullptr;  // the cached plan this step runs on (null: it was scheduled afresh)
   Plan *find_plan(const int *graph, int B, int maxlen, uint64_t hash);
   void remember_plan(const int *graph, int B, int maxlen, uint64_t hash);
 
@@ -239,12 +304,6 @@ class Engine {
   // Bias gradients that exist as rows still to be added up and / or permuted (row E of dW; the
   // chunk sums of a column sum): delivered, and the parameter updated, by one job each of the
   // launch that ends the step.
-  struct BiasJob {
-    std::string param;
-    const float *src;
-    int parts;
-    long long bw, nb, map;
-  };
   std::vector<BiasJob> bias_jobs_;
   DeviceArray<float> bias_parts_, head_bias_parts_;
   // column sums of inp [n, w] as the gradient of `name`, in a fixed order

@@ -73,6 +73,18 @@ int cavs_event_elapsed_ms(float *ms, void *start, void *stop);
 int cavs_profile_arm(void *start_event, void *stop_event);
 int cavs_profile_disarm(int *launched); /* waits for `stop` */
 
+/* A stretch of a stream's work recorded once and enqueued again as one call: everything enqueued on
+ * `stream` between cavs_graph_capture_begin and cavs_graph_capture_end is recorded instead of run
+ * (kernel launches and copies of this library are fine; nothing in between may wait for the
+ * stream or for an event).  cavs_graph_capture_end hands back the replayable graph, or, called with
+ * graph_exec = NULL, ends a capture the caller gives up.  cavs_graph_launch enqueues the recorded
+ * work -- same kernels, same arguments, same order.  For the host loop that re-issues the launches
+ * of a batch structure seen before (GraphStatement::Run's round loop, cavs/midend/statement.cc:69-76). */
+int cavs_graph_capture_begin(void *stream);
+int cavs_graph_capture_end(void *stream, void **graph_exec);
+int cavs_graph_launch(void *graph_exec, void *stream);
+int cavs_graph_destroy(void *graph_exec);
+
 /* ------------------------------------------------------------------ graph ops
  * Replace GraphGatherOp / GraphScatterOp / GraphPushOp / GraphPullOp /
  * FunctionPopRetOp (cavs/backend/op_impl_graphop.cu:17-327) and their kernels

@@ -72,6 +72,15 @@ typedef struct {
    * checks once, when it is created, that the device runs such a launch's workgroups all at once,
    * each group on one XCD, and keeps to one launch per round if not. */
   int tail_rows;
+  /* With a plan cache: 1 = a step on a batch structure seen before, with the same input buffers
+   * (inputs_on_device) and the session in the same state as the last time, enqueues its forward
+   * pass, loss head and backward pass as one recorded graph of launches (cavs_graph_launch) instead
+   * of re-issuing every launch from the host loop (cavs/midend/statement.cc:69-76); the launch that
+   * applies the parameter updates stays a launch of its own.  The first such step records, the
+   * later ones replay.  Any other call on the session, or a buffer that had to grow, makes
+   * the next step an ordinary one.  Replayed steps have no "RNNForward" / "RNNBackward" timings.
+   * The counter "graph_replays" counts them.  0 = off. */
+  int graph_replay;
 } cavs_session_config;
 
 const char *cavs_session_error(void);

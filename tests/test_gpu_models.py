@@ -573,3 +573,60 @@ def test_training_step_on_reader_batches(oracle, kind):
     print(f"[case] reader kind={kind} N={N}", flush=True)
     got, want = run_both(oracle, w)
     compare(got, want)
+
+
+@pytest.mark.parametrize("model,H,pool", [("treefc", 32, 3), ("treelstm", 32, 3), ("lstm", 32, 2), ("treelstm", 512, 2)])
+def test_recorded_graph_of_a_cached_plan_gives_the_steps_of_the_host_loop(model, H, pool):
+    """graph_replay: on a batch structure seen before, with the same device-resident feeds, the
+    forward pass, loss head and backward pass are enqueued as one recorded graph.  Training steps
+    (with the parameter update) through such a session and through one that issues every launch
+    from the host loop give the same losses and parameters -- bit for bit where no gradient is
+    accumulated with atomics (Tree-FC), to the tolerance of the accumulation order elsewhere.
+    H = 512 puts the launches over the rounds near the roots inside the graph."""
+    import torch
+    V, Cc = 31, 5
+    E = H if model == "lstm" else 12
+    loss = "softmax" if model != "treefc" else "root_sq"
+    ws = [small_workload(model, 401 + k, B=5 + k, H=H, E=E, V=V, C=Cc) for k in range(pool)]
+    names = {"treelstm": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",)}[model]
+    params = {k: np.asarray(ws[0]["params"][k], np.float32) for k in names}
+    sessions = [session.Session(model, H=H, E=E, V=V, C_=Cc, loss=loss, plan_cache=4, graph_replay=bool(r)) for r in (0, 1)]
+    for s in sessions:
+        s.set_params(params)
+    feeds = [(w["graph"], torch.from_numpy(np.ascontiguousarray(w["x"], np.float32)).cuda(),
+              torch.from_numpy(np.ascontiguousarray(w["labels"], np.float32)).cuda()) for w in ws]
+    torch.cuda.synchronize()
+    steps = 5 * pool
+    for i in range(steps):
+        g, x, lab = feeds[i % pool]
+        print(f"[case] graph replay {model} H={H} step {i}", flush=True)
+        losses = []
+        for s in sessions:
+            s.step(g, x, lab, backward=True, lr=0.05)
+            losses.append(s.fetch("loss"))
+        if model == "treefc":
+            np.testing.assert_array_equal(losses[1], losses[0])
+        else:
+            np.testing.assert_allclose(losses[1], losses[0], rtol=2e-5, atol=1e-6)
+    assert sessions[0].counter("graph_replays") == 0
+    # every structure: a miss, then a recording, then replays (an odd cycle of structures meets each
+    # of the two id buffers in turn and records once per buffer)
+    assert sessions[1].counter("graph_replays") >= steps - 2 * pool, sessions[1].counter("graph_replays")
+    assert sessions[1].counter("plan_hits") == steps - pool
+    for n in names:
+        a, b = (s.param(n, params[n].shape) for s in sessions)
+        if model == "treefc":
+            np.testing.assert_array_equal(b, a)
+        else:
+            np.testing.assert_allclose(b, a, rtol=2e-5, atol=2e-6)
+    # a call in between (new parameters) makes the next step an ordinary one, with the host loop's result
+    for s in sessions:
+        s.set_params(params)
+    g, x, lab = feeds[0]
+    out = []
+    for s in sessions:
+        s.step(g, x, lab, backward=True, lr=0.0)
+        out.append(s.fetch("loss"))
+    np.testing.assert_allclose(out[1], out[0], rtol=2e-6, atol=1e-7)
+    for s in sessions:
+        s.close()
