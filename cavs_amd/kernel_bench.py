@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Per-kernel roofline measurements through the C ABI (no model around the kernels).
 
-    python -m cavs_amd.kernel_bench [--set copies|gemm|gates|rounds|all] [--iters 50]
+    python -m cavs_amd.kernel_bench [--set copies|gemm|gates|rounds|tails|all] [--iters 50]
 
 For each case: launches the entry point `iters` times back to back on one stream between two
 HIP events (launches shorter than 12 us: timed one at a time by the events their own kernels
@@ -270,9 +270,98 @@ def rounds(iters, st):
         del pool, xW, U, G, hlr, gt, msg, hU, hUf, UT, dpool, dret, dxW, dF
 
 
+def tails(iters, st):
+    """The rounds near the roots of a Tree-LSTM batch (H = 512) as one launch per direction, beside the
+    same rounds as one packed launch each.  The batch: 8 x `width` complete binary trees side by
+    side, rounds of 8 * width, 4 * width ... 8 rows above 16 * width leaf rows; a group runs `width` trees."""
+    import numpy as np
+    f32 = dict(dtype=torch.float32, device="cuda")
+    H = 512
+    for width in (8, 32):
+        sizes = []
+        n = 8 * width
+        while n >= 8:
+            sizes.append(n)
+            n //= 2
+        leaves = 2 * sizes[0]
+        offs = np.concatenate([[leaves], leaves + np.cumsum(sizes)[:-1]]).astype(np.int64)
+        N = int(leaves + sum(sizes))
+        child = np.full(2 * N, -1, np.int32)
+        for r, (off, nr) in enumerate(zip(offs, sizes)):
+            below = 0 if r == 0 else offs[r - 1]
+            i = np.arange(nr)
+            child[2 * (off + i)] = below + 2 * i
+            child[2 * (off + i) + 1] = below + 2 * i + 1
+        # group g: the rows i with i * 8 // nr == g of every round, round by round
+        rows, start, count = [], np.zeros((8, len(sizes)), np.int32), np.zeros((8, len(sizes)), np.int32)
+        for g in range(8):
+            for r, (off, nr) in enumerate(zip(offs, sizes)):
+                mine = off + np.arange(g * nr // 8, (g + 1) * nr // 8)
+                start[g, r], count[g, r] = len(rows), len(mine)
+                rows.extend(mine.tolist())
+        nrounds = np.full(8, len(sizes), np.int32)
+        flags = np.tile(np.arange(len(sizes), dtype=np.int32) * 2 + 1, (8, 1)).astype(np.int32)  # wait for the lists before, arrive
+        bstart, bcount = np.ascontiguousarray(start[:, ::-1]), np.ascontiguousarray(count[:, ::-1])
+        d_rows = torch.tensor(rows, dtype=torch.int32, device="cuda")
+        d_child = torch.from_numpy(child).cuda()
+        d_pair = torch.arange(N, dtype=torch.int32, device="cuda")
+        pool = torch.randn(N, 2 * H, **f32) * 0.5
+        xW, bias = torch.randn(N, 4 * H, **f32), torch.zeros(4 * H, **f32)
+        U = torch.randn(4 * H * H, **f32) / H ** 0.5
+        Upk, UTp = torch.empty(4 * H * H, **f32), torch.empty(4 * H * H, **f32)
+        T = hip.Task
+        jobs = [T(hip.TASK_SGD_PACK, 0.0, H, 3 * H, 0, Upk.data_ptr(), U.data_ptr(), None, None),
+                T(hip.TASK_SGD_PACK, 0.0, H, H, 0, Upk.data_ptr() + 4 * 3 * H * H, U.data_ptr() + 4 * 3 * H * H, None, None),
+                T(hip.TASK_PACK_T, 0.0, H, 3 * H, 0, UTp.data_ptr(), U.data_ptr(), None, None),
+                T(hip.TASK_PACK_T, 0.0, H, H, 0, UTp.data_ptr() + 4 * 3 * H * H, U.data_ptr() + 4 * 3 * H * H, None, None)]
+        hip.call("cavs_run_tasks", len(jobs), (T * len(jobs))(*jobs), st)
+        G, hlr = torch.zeros(2 * N, 2 * H, **f32), torch.zeros(N, H, **f32)
+        gt, go = torch.rand(N, 6 * H, **f32), torch.zeros(N, H, **f32)
+        d_out = torch.arange(N, dtype=torch.int32, device="cuda")
+        sync = torch.zeros(hip.lib().cavs_tail_sync_bytes() // 4, dtype=torch.int32, device="cuda")
+        M = len(sizes)
+        flops = 2.0 * sum(sizes) * H * 5 * H
+        tag = f"rounds of {sizes[0]} .. {sizes[-1]} rows ({sum(sizes)} vertices), 8 groups, H={H}"
+
+        def fwd_tail():
+            hip.call("cavs_treelstm_tail_fwd", pool.data_ptr(), d_child.data_ptr(), d_pair.data_ptr(), xW.data_ptr(), 4 * H, Upk.data_ptr(),
+                     bias.data_ptr(), G.data_ptr(), hlr.data_ptr(), gt.data_ptr(), None, go.data_ptr(), d_out.data_ptr(), d_rows.data_ptr(),
+                     8, nrounds.ctypes.data, start.ctypes.data, count.ctypes.data, flags.ctypes.data, M, H, sync.data_ptr(), 1 << 20, 0, st)
+
+        def fwd_rounds():
+            for off, nr in zip(offs.tolist(), sizes):
+                hip.call("cavs_treelstm_round_fwd_packed", pool.data_ptr(), d_child.data_ptr() + 8 * off, d_pair.data_ptr() + 4 * off,
+                         xW.data_ptr() + 16 * off * H, 4 * H, U.data_ptr(), Upk.data_ptr(), bias.data_ptr(), G.data_ptr() + 16 * off * H,
+                         hlr.data_ptr() + 4 * off * H, gt.data_ptr() + 24 * off * H, None, go.data_ptr(), d_out.data_ptr() + 4 * off, nr, H, st)
+
+        us = _time(fwd_tail, iters, st)
+        _emit("treelstm_tail_fwd", tag, us, flops=flops)
+        us = _time(fwd_rounds, iters, st)
+        _emit(f"the same as {M} cavs_treelstm_round_fwd_packed", tag, us, flops=flops)
+        Gv = torch.randn(2 * N, 2 * H, **f32) * 0.5
+        dgo = torch.randn(N, H, **f32)
+        dxW, dF, dc = torch.zeros(N, 4 * H, **f32), torch.zeros(2 * N, H, **f32), torch.zeros(N, H, **f32)
+
+        def bwd_tail():
+            hip.call("cavs_treelstm_tail_bwd", dxW.data_ptr(), 4 * H, dF.data_ptr(), dc.data_ptr(), UTp.data_ptr(), d_child.data_ptr(),
+                     gt.data_ptr(), Gv.data_ptr(), dgo.data_ptr(), d_out.data_ptr(), leaves, d_rows.data_ptr(), 8, nrounds.ctypes.data,
+                     bstart.ctypes.data, bcount.ctypes.data, flags.ctypes.data, M, H, sync.data_ptr(), 1 << 20, 0, st)
+
+        def bwd_rounds():
+            for off, nr in zip(offs.tolist()[::-1], sizes[::-1]):
+                hip.call("cavs_treelstm_round_bwd_children_gates_packed", dxW.data_ptr(), 4 * H, dF.data_ptr(), dc.data_ptr(), UTp.data_ptr(),
+                         d_child.data_ptr() + 8 * off, gt.data_ptr(), Gv.data_ptr(), dgo.data_ptr(), d_out.data_ptr(), off, nr, leaves, H, st)
+
+        us = _time(bwd_tail, iters, st)
+        _emit("treelstm_tail_bwd", tag, us, flops=flops)
+        us = _time(bwd_rounds, iters, st)
+        _emit(f"the same as {M} cavs_treelstm_round_bwd_children_gates_packed", tag, us, flops=flops)
+        assert int(sync[1].item()) == 0, "a tail launch gave up"
+
+
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--set", default="all", choices=["copies", "gemm", "gates", "rounds", "all"])
+    ap.add_argument("--set", default="all", choices=["copies", "gemm", "gates", "rounds", "tails", "all"])
     ap.add_argument("--iters", type=int, default=50)
     a = ap.parse_args()
     assert torch.cuda.is_available(), "kernel_bench needs the MI355X"
@@ -286,6 +375,8 @@ def main():
         gates(a.iters, st)
     if a.set in ("rounds", "all"):
         rounds(a.iters, st)
+    if a.set in ("tails", "all"):
+        tails(a.iters, st)
 
 
 if __name__ == "__main__":
