@@ -725,6 +725,22 @@ void Engine::schedule_on_device(const int *graph, int B, int maxlen) {
   n_orphans_ = B;
   forest_ = !cfg_.split_backward_rounds && fused_rows() > 0;
   for (int r = 1; r < R && forest_; r++) forest_ = s.rounds[r].n <= fused_rows();
+  // The tail launches want whole trees of the message flow dealt to their groups, which is host
+  // work on the children-by-slab-row list: it comes back (2N ints), the groups' row lists go up.
+  tail_ = TailPlan();
+  if (forest_ && nch_ == 2 && tail_limit() > 0 && N > 0) {
+    d.kid_host.reserve(2 * (size_t)N);
+    d.tail_host.reserve(N);
+    check(cavs_memcpy_d2h(d.kid_host.get(), kid, 2 * (size_t)N * sizeof(int), sched_stream_));
+    check(cavs_stream_sync(sched_stream_));
+    build_tail_plan(d.kid_host.get(), d.tail_host.get());
+    if (tail_.first >= 0) {
+      d.tail_dev.reserve(grow(N, d.tail_dev.capacity()));
+      check(cavs_memcpy_h2d(d.tail_dev.get(), d.tail_host.get(), tail_.rows * sizeof(int), sched_stream_));
+      check(cavs_stream_sync(sched_stream_));
+      d_tail_rows_ = d.tail_dev.get();
+    }
+  }
   last_free_ev_ = d.free_ev;
   last_busy_ = &d.busy;
   sched_ms_ = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();

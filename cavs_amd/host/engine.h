@@ -169,8 +169,8 @@ class Engine {
   // builds every list there, and only the round offsets come back.  Two sets of buffers alternate,
   // so that the lists of step k + 1 are built while the kernels of step k still read theirs.
   struct DeviceSched {
-    PinnedArray<int> graph_host, meta_host;
-    DeviceArray<int> graph_dev, lists, meta_dev;
+    PinnedArray<int> graph_host, meta_host, kid_host, tail_host;
+    DeviceArray<int> graph_dev, lists, meta_dev, tail_dev;
     long cap = 0;          // rows per list
     void *free_ev = nullptr;  // recorded once everything that read `lists` has been enqueued
     bool busy = false;

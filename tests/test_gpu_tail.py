@@ -317,6 +317,34 @@ def test_a_training_step_is_the_same_with_and_without_the_tail_launches(g, pairi
             close(grb[k], gra[k].astype(np.float64), k + ", " + what)
 
 
+def test_the_device_built_schedule_runs_the_tail_launches_too(g):
+    """schedule="device": the children-by-slab-row list comes back from the device scheduler, the host
+    deals its trees to the groups and the row lists go up; the step is the one of the host scheduler
+    (same plan, same launches) bit for bit, apart from the embedding gradient's atomics."""
+    from cavs_amd import session
+    from tolerance import close
+
+    w = synth.make_workload("C3", B=24)
+    res = {}
+    for schedule in ("host", "device"):
+        s = session.Session("treelstm", H=w["H"], E=w["E"], V=w["V"], C_=w["C"], schedule=schedule)
+        s.set_params(w["params"])
+        s.step(w["graph"], w["x"], w["labels"], backward=True, lr=0.0)
+        res[schedule] = (s.fetch("loss"), s.fetch("graph_out"), s.grads(), s.counter("tail_rounds"), s.counter("launches"),
+                         s.counter("tail_first_round"), s.counter("scheduler"))
+        s.close()
+    h, d = res["host"], res["device"]
+    assert d[6] == 1 and h[6] == 0
+    assert d[3] == h[3] > 0 and d[5] == h[5], "the device-scheduled step did not run the same tail launches"
+    np.testing.assert_array_equal(d[0], h[0])
+    np.testing.assert_array_equal(d[1], h[1])
+    for k in h[2]:
+        if k == "dEmb":
+            close(d[2][k], h[2][k].astype(np.float64), k)
+        else:
+            np.testing.assert_array_equal(d[2][k], h[2][k], err_msg=k)
+
+
 def test_a_guarded_launch_of_jobs_runs_only_while_the_watched_word_is_zero(g):
     """CAVS_TASK_GUARD: the parameter updates of a step watch the status word of the tail launches."""
     T = hip.Task
