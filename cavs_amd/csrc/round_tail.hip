@@ -19,7 +19,9 @@
 //     polls it with a bound and gives up into a status word the host reads (every wave then leaves);
 //   * the weights never move again: a wavefront owns one eighth of K (64 k at H = 512) of its
 //     workgroup's sixteen columns, i.e. sixteen float4 of the tile-major weights, and keeps them in
-//     registers for the whole launch.  A round then fetches only its operand rows.
+//     registers for the whole launch.  A round then fetches only its operand rows;
+//   * the index lists of a group (slab rows, children, destination rows) are fetched once, into a
+//     table in LDS, while the weights arrive.
 // The arithmetic is that of the four-row tiles of the per-round kernels (treelstm_round_fwd_kernel
 // / treelstm_round_bwd_children_kernel with ROWS4): the same MFMAs on the same operands in the
 // same order, the same order of sums, the same gate function -- and a row's result does not
@@ -33,14 +35,14 @@ constexpr int kTailRows = 32;      // at most eight tiles of four rows per group
 constexpr int kTailGroups = 8;     // one per XCD
 constexpr int kTailMaxRounds = 32; // lists per group
 
-// What each group does: nrounds[g] lists of slab rows, list i = rows[start[g][i] .. + count[g][i]).
-// flags[g][i]: bit 0 -- the group's workgroups tell each other when the list is done (an arrival);
-// the rest -- how many of the group's arrivals must be in before the list starts (0: none, e.g. the
-// second slice of a round that does not fit one list).
 // LDS of the two kernels: the parked partial sums (floats), then five index tables of one int per list position
 constexpr int kTailFwdRed = 8 * 8 * 20 * 16, kTailBwdRed = 8 * 8 * 12 * 16;
 constexpr size_t kTailTabBytes = 5 * sizeof(int) * kTailMaxRounds * kTailRows;
 
+// What each group does: nrounds[g] lists of slab rows, list i = rows[start[g][i] .. + count[g][i]).
+// flags[g][i]: bit 0 -- the group's workgroups tell each other when the list is done (an arrival);
+// the rest -- how many of the group's arrivals must be in before the list starts (0: none, e.g. the
+// second slice of a round that does not fit one list).
 struct TailPlan {
   int nrounds[kTailGroups], arrivals[kTailGroups];
   int start[kTailGroups][kTailMaxRounds];

@@ -1,4 +1,5 @@
 // extern "C" surface of the host runtime (cavs_session.h): exceptions end here.
+#include <algorithm>
 #include <vector>
 #include <cstdio>
 #include <cstring>
@@ -133,6 +134,46 @@ int cavs_schedule_index_lists(const int *graph, int B, int maxlen, int nchild, i
     *n_orphans = ok ? n : -1;
   }
   return sch.N;
+}
+
+int cavs_schedule_tail_lists(const int *graph, int B, int maxlen, int pairing, int fused_limit, int rows_limit, int groups,
+                             int max_lists, int *meta, int *nrounds, int *start, int *count, int *flags, int *bstart, int *bcount,
+                             int *bflags, int *rows_out) {
+  if (!graph || B <= 0 || maxlen <= 0 || pairing < 0 || pairing > 1 || groups < 1 || groups > 8 || max_lists < 1 || rows_limit < 1 ||
+      !meta || !nrounds || !start || !count || !flags || !bstart || !bcount || !bflags || !rows_out) {
+    g_error = "bad arguments";
+    return -1;
+  }
+  cavs::Schedule sch;
+  std::string err = cavs::build_schedule(graph, B, maxlen, true, &sch);
+  if (err.empty() && sch.executed != sch.N) err = "the batch holds a single-vertex sample";
+  const size_t N = err.empty() ? (size_t)sch.N : 0;
+  std::vector<int> t2j(N), pair(N), child(2 * N), roots((size_t)B), kid(2 * N), orphans(N);
+  if (err.empty()) err = cavs::build_index_lists(sch, 2, pairing, t2j.data(), pair.data(), child.data(), roots.data());
+  if (!err.empty()) {
+    g_error = err;
+    return -1;
+  }
+  meta[0] = -1;
+  meta[1] = meta[2] = meta[3] = 0;
+  int n_orphans = 0;
+  if (!cavs::build_forest_lists(sch, 2, fused_limit, pair.data(), child.data(), kid.data(), orphans.data(), &n_orphans)) return 0;
+  cavs::TailLists t;
+  cavs::build_tail_lists(sch, kid.data(), rows_limit, groups, max_lists, 32, &t, rows_out);
+  if (t.first < 0) return 0;
+  meta[0] = t.first;
+  meta[1] = t.max_rounds;
+  meta[2] = t.lists_max;
+  meta[3] = t.tiles_max;
+  std::copy(t.nrounds.begin(), t.nrounds.end(), nrounds);
+  const size_t n = (size_t)groups * t.max_rounds;
+  std::copy(t.start.begin(), t.start.begin() + n, start);
+  std::copy(t.count.begin(), t.count.begin() + n, count);
+  std::copy(t.flags.begin(), t.flags.begin() + n, flags);
+  std::copy(t.bstart.begin(), t.bstart.begin() + n, bstart);
+  std::copy(t.bcount.begin(), t.bcount.begin() + n, bcount);
+  std::copy(t.bflags.begin(), t.bflags.begin() + n, bflags);
+  return (int)t.rows;
 }
 
 int cavs_schedule_trace_from_lists(int B, int maxlen, int N, int nchild, const int *round2offset, int R, const int *t2j,

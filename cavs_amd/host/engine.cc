@@ -93,113 +93,15 @@ int Engine::tail_limit() const {
   return cfg_.tail_rows > 0 ? cfg_.tail_rows : 32;
 }
 
-// Which rounds run inside the tail launches, and who runs which row.  The rounds are a suffix of the
-// forward order (a prefix of the backward order).  Inside it the message flow is a forest over slab
-// rows (kid_rows: the rows whose messages a row consumes); a tree of that forest goes to one group
-// as a whole, so nothing a group reads is written by another during the launch.  Trees are dealt
-// heaviest first to the group with the fewest rows so far; the suffix starts at the earliest round
-// from which no group gets more rows of a round than the limit, nor more lists than a launch takes.
+// The rounds inside the tail launches and who runs which row (build_tail_lists): the groups' row
+// lists go to `rows_out` (room for N ints), the plan to tail_.
 void Engine::build_tail_plan(const int *kid_rows, int *rows_out) {
   tail_ = TailPlan();
   const int lim = tail_limit();
-  const Schedule &s = *sched_;
-  const int R = (int)s.rounds.size(), N = s.N, G = cavs_tail_max_groups(), cap = cavs_tail_max_rounds(), slice = 32;
-  if (lim <= 0 || !s.batching || R < 3 || nch_ != 2 || !cavs_round_packed_ok(1, cfg_.H) || !cavs_tail_rounds_ok(1, cfg_.H)) return;
-  int k0 = 1;
-  while (k0 < R && (s.rounds[k0].n > G * lim || leaf_round(s.rounds[k0]))) k0++;
-  std::vector<int> comp, weight, group, order, per;
-  for (; R - k0 >= 2; k0++) {
-    bool ok = true;
-    for (int k = k0; k < R && ok; k++) ok = !leaf_round(s.rounds[k]);
-    if (!ok) continue;
-    const int lo = s.rounds[k0].offset;
-    comp.assign(N - lo, -1);
-    weight.clear();
-    for (int v = N - 1; v >= lo; v--) {  // a row's consumer sits in a later round: parents come first
-      if (comp[v - lo] < 0) {
-        comp[v - lo] = (int)weight.size();
-        weight.push_back(0);
-      }
-      weight[comp[v - lo]]++;
-      for (int i = 0; i < 2; i++) {
-        const int c = kid_rows[2 * (size_t)v + i];
-        if (c >= lo) comp[c - lo] = comp[v - lo];
-      }
-    }
-    order.resize(weight.size());
-    for (size_t i = 0; i < order.size(); i++) order[i] = (int)i;
-    std::stable_sort(order.begin(), order.end(), [&](int a, int b) { return weight[a] > weight[b]; });
-    group.assign(weight.size(), 0);
-    int load[16] = {0};
-    for (int c : order) {
-      int best = 0;
-      for (int g = 1; g < G; g++)
-        if (load[g] < load[best]) best = g;
-      group[c] = best;
-      load[best] += weight[c];
-    }
-    // rows of round k that group g runs, and the lists that makes
-    const int nr = R - k0;
-    per.assign((size_t)G * nr, 0);
-    for (int k = k0; k < R; k++)
-      for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) per[(size_t)group[comp[b - lo]] * nr + (k - k0)]++;
-    int lists = 0;
-    for (int g = 0; g < G && ok; g++) {
-      int mine = 0;
-      for (int k = 0; k < nr; k++) {
-        if (per[(size_t)g * nr + k] > lim) ok = false;
-        mine += (per[(size_t)g * nr + k] + slice - 1) / slice;
-      }
-      if (mine > cap) ok = false;
-      lists = std::max(lists, mine);
-    }
-    if (!ok) continue;
-    TailPlan &t = tail_;
-    t.first = k0;
-    t.max_rounds = std::max(lists, 1);
-    const size_t M = t.max_rounds;
-    t.nrounds.assign(G, 0);
-    for (auto *v : {&t.start, &t.count, &t.flags, &t.bstart, &t.bcount, &t.bflags}) v->assign((size_t)G * M, 0);
-    // the device list: group by group, round by round
-    std::vector<int> at((size_t)G * nr, -1);
-    size_t fill = 0;
-    for (int g = 0; g < G; g++)
-      for (int k = 0; k < nr; k++) {
-        at[(size_t)g * nr + k] = (int)fill;
-        fill += per[(size_t)g * nr + k];
-      }
-    {
-      std::vector<int> cur(at);
-      for (int k = k0; k < R; k++)
-        for (int b = s.rounds[k].offset; b < s.rounds[k].offset + s.rounds[k].n; b++) rows_out[cur[(size_t)group[comp[b - lo]] * nr + (k - k0)]++] = b;
-    }
-    // A group's share of a round as lists of at most `slice` rows: the first waits for the rounds the
-    // group has done so far, the last is an arrival.  Forward: rounds in order; backward: reversed.
-    for (int g = 0; g < G; g++) {
-      int tiles = 0;
-      for (int dir = 0; dir < 2; dir++) {
-        std::vector<int> &st = dir ? t.bstart : t.start, &ct = dir ? t.bcount : t.count, &fl = dir ? t.bflags : t.flags;
-        int i = 0, done = 0;
-        for (int kk = 0; kk < nr; kk++) {
-          const int k = dir ? nr - 1 - kk : kk, c = per[(size_t)g * nr + k];
-          for (int c0 = 0; c0 < c; c0 += slice, i++) {
-            st[g * M + i] = at[(size_t)g * nr + k] + c0;
-            ct[g * M + i] = std::min(slice, c - c0);
-            fl[g * M + i] = ((c0 == 0 ? done : 0) << 1) | (c0 + slice >= c ? 1 : 0);
-            if (!dir) tiles += (ct[g * M + i] + 3) / 4;
-          }
-          done += c > 0;
-        }
-        t.nrounds[g] = i;
-      }
-      t.tiles_max = std::max(t.tiles_max, tiles);
-      t.lists_max = std::max(t.lists_max, t.nrounds[g]);
-    }
-    t.rows = fill;
-    t.vertices = (double)fill;
-    t.flops = 2.0 * fill * cfg_.H * 5.0 * cfg_.H;
-    return;
-  }
+  if (lim <= 0 || nch_ != 2 || !cavs_round_packed_ok(1, cfg_.H) || !cavs_tail_rounds_ok(1, cfg_.H)) return;
+  build_tail_lists(*sched_, kid_rows, lim, cavs_tail_max_groups(), cavs_tail_max_rounds(), 32, &tail_, rows_out);
+  tail_.vertices = (double)tail_.rows;
+  tail_.flops = 2.0 * tail_.rows * cfg_.H * 5.0 * cfg_.H;
 }
 
 void Engine::tail_check() {

@@ -185,14 +185,8 @@ class Engine {
   // ---- the rounds near the roots as one launch per direction (cavs_treelstm_tail_fwd / _bwd)
   // What those launches run, for one batch structure: the rounds from `first` on, their rows dealt
   // to the groups by whole trees of the message flow (no message crosses groups).
-  struct TailPlan {
-    int first = -1;  // first round (forward order) inside the launches; -1: none
-    int max_rounds = 0;
-    std::vector<int> nrounds, start, count, flags;  // per group; lists in forward order
-    std::vector<int> bstart, bcount, bflags;        // the same lists in backward order
-    size_t rows = 0;                             // length of the device list of slab rows
+  struct TailPlan : TailLists {
     double flops = 0, vertices = 0;
-    int lists_max = 0, tiles_max = 0;            // the longest group: its lists, its tiles of four rows
   };
 
   // ---- plan cache (cfg.plan_cache entries): the schedule and the device lists of a graph feed,

@@ -75,6 +75,22 @@ std::string build_index_lists(const Schedule &s, int nch, int pairing, int *t2j,
 bool build_forest_lists(const Schedule &s, int nch, int fused_limit, const int *pair, const int *child, int *kid_rows,
                         int *orphans, int *n_orphans);
 
+// What the launches over the rounds near the roots run (cavs_treelstm_tail_fwd / _bwd), for one
+// batch structure: the rounds from `first` on, their rows dealt to the groups by whole trees of
+// the message flow (no message crosses groups), each group's share of a round as lists of at
+// most `slice` rows with the flag word the launches take (2 * arrivals to wait for + arrives).
+struct TailLists {
+  int first = -1;  // first round (forward order) inside the launches; -1: none
+  int max_rounds = 0;                             // lists per group the arrays below are laid out for
+  std::vector<int> nrounds, start, count, flags;  // per group; lists in forward order
+  std::vector<int> bstart, bcount, bflags;        // the same lists in backward order
+  size_t rows = 0;                                // length of the list of slab rows
+  int lists_max = 0, tiles_max = 0;               // the longest group: its lists, its tiles of four rows
+};
+// kid_rows as build_forest_lists leaves them (binary trees); rows_out: room for N ints.
+void build_tail_lists(const Schedule &s, const int *kid_rows, int lim, int groups, int max_lists, int slice, TailLists *out,
+                      int *rows_out);
+
 // The inverse of build_index_lists for a batch schedule: rounds and lists of a Schedule from the
 // arrays (as a device scheduler leaves them) and the round offsets; `out` compares equal, trace
 // for trace, to the schedule the lists came from.

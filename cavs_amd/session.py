@@ -53,6 +53,7 @@ def lib():
             "cavs_session_schedule_trace": [P, P, I],
             "cavs_schedule_trace": [P, I, I, I, I, P, I],
             "cavs_schedule_index_lists": [P, I, I, I, I, I, P, P, P, P, P, P, P],
+            "cavs_schedule_tail_lists": [P, I, I, I, I, I, I, I, P, P, P, P, P, P, P, P, P],
             "cavs_schedule_trace_from_lists": [I, I, I, I, P, I, P, P, P, P, I, P, I],
             "cavs_session_timing": [P, C.c_char_p, C.POINTER(F)],
             "cavs_session_counter": [P, C.c_char_p, C.POINTER(C.c_double)],
@@ -130,6 +131,29 @@ def index_lists(graph, nchild, pairing="reference", fused_limit=1 << 30):
     forest = n_orph.value >= 0
     return dict(N=N, t2j=t2j[:N], pair=pair[:N], child=child[: nchild * N], roots=roots,
                 kid=kid[: nchild * N] if forest else None, orphans=orph[: n_orph.value] if forest else None)
+
+
+def tail_lists(graph, pairing="reference", fused_limit=1 << 30, rows_limit=32, groups=8, max_lists=32):
+    """Host-only: how the rounds near the roots of a batch of binary trees are dealt to the groups of the
+    tail launches.  None when no suffix of the rounds can be dealt within the limits; else
+    dict(first, M, lists_max, tiles_max, nrounds [groups], start / count / flags and bstart / bcount /
+    bflags [groups, M], rows)."""
+    g = np.ascontiguousarray(graph, np.int32)
+    B, maxlen = g.shape
+    meta, nrounds = np.zeros(4, np.int32), np.zeros(groups, np.int32)
+    arr = [np.zeros(groups * max_lists, np.int32) for _ in range(6)]
+    rows = np.zeros(B * maxlen, np.int32)
+    n = lib().cavs_schedule_tail_lists(g.ctypes.data, B, maxlen, PAIR[pairing], fused_limit, rows_limit, groups, max_lists,
+                                       meta.ctypes.data, nrounds.ctypes.data, *[a.ctypes.data for a in arr], rows.ctypes.data)
+    if n < 0:
+        raise hip.CavsError("graph feed rejected: " + lib().cavs_session_error().decode())
+    if n == 0:
+        return None
+    M = int(meta[1])
+    names = ("start", "count", "flags", "bstart", "bcount", "bflags")
+    out = dict(first=int(meta[0]), M=M, lists_max=int(meta[2]), tiles_max=int(meta[3]), nrounds=nrounds, rows=rows[:n])
+    out.update({k: a[: groups * M].reshape(groups, M) for k, a in zip(names, arr)})
+    return out
 
 
 def trace_from_lists(B, maxlen, nchild, round2offset, t2j, pair, child, roots, with_backward=True):

@@ -129,6 +129,18 @@ int cavs_schedule_trace(const int *graph, int B, int maxlen, int batching, int w
 int cavs_schedule_index_lists(const int *graph, int B, int maxlen, int nchild, int pairing, int fused_limit,
                               int *t2j, int *pair, int *child, int *roots, int *kid_rows, int *orphans,
                               int *n_orphans);
+/* Pure host call: for a batch of binary trees, what the launches over the rounds near the roots
+ * (cavs_treelstm_tail_fwd / _bwd, cavs_hip.h) would be given -- the deal the session makes when its
+ * tail_rows allows.  rows_limit: most rows of a round a group may get; groups (1..8), max_lists: what
+ * the launches take (cavs_tail_max_groups, cavs_tail_max_rounds).  Out: meta[0] = first round inside
+ * the launches, meta[1] = M, the lists per group the arrays are laid out for, meta[2] / meta[3] = lists
+ * and four-row tiles of the longest group; nrounds [groups]; start, count, flags (forward order) and
+ * bstart, bcount, bflags (backward order), each [groups * max_lists] with list i of group g at
+ * g * M + i; rows_out [B * maxlen]: the groups' slab rows.  Returns the number of slab rows (0: no
+ * suffix of the rounds can be dealt that way), or -1 with the reason in cavs_session_error(). */
+int cavs_schedule_tail_lists(const int *graph, int B, int maxlen, int pairing, int fused_limit, int rows_limit, int groups,
+                             int max_lists, int *meta, int *nrounds, int *start, int *count, int *flags, int *bstart,
+                             int *bcount, int *bflags, int *rows_out);
 int cavs_schedule_trace_from_lists(int B, int maxlen, int N, int nchild, const int *round2offset, int R,
                                    const int *t2j, const int *pair, const int *child, const int *roots,
                                    int with_backward, int *out, int cap);
