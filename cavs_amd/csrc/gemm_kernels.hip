@@ -718,6 +718,10 @@ static bool vec_path_ok(const GemmArgs &g, int tA, int tB) {
   return true;
 }
 
+// LDS a tile launch of the calling thread asks for on top of its panels (cavs_sgemm_group_beside): the
+// workgroups then take more of a CU than they use, and fewer of them share one
+static thread_local unsigned t_lds_pad = 0;
+
 template <int BM, int BN, int BK>
 static void launch_tile(const GemmArgs &args, int tA, int tB, bool vec, const GemmPlan &p, hipStream_t st) {
   GemmArgs g = args;
@@ -731,9 +735,9 @@ static void launch_tile(const GemmArgs &args, int tA, int tB, bool vec, const Ge
   }
 #define CAVS_GEMM_CASE(TA, TB)                                                  \
   if (vec)                                                                      \
-    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, true>, grid, block, 0, st, g);      \
+    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, true>, grid, block, t_lds_pad, st, g);      \
   else                                                                          \
-    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, false>, grid, block, 0, st, g)
+    launch(sgemm_mfma_kernel<BM, BN, BK, TA, TB, false>, grid, block, t_lds_pad, st, g)
   if (!tA && !tB) { CAVS_GEMM_CASE(false, false); }
   else if (!tA && tB) { CAVS_GEMM_CASE(false, true); }
   else if (tA && !tB) { CAVS_GEMM_CASE(true, false); }
@@ -1056,6 +1060,14 @@ size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products) {
 int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace, size_t workspace_bytes,
                      void *stream) {
   return run_group(count, products, workspace, workspace_bytes, nullptr, stream);
+}
+
+int cavs_sgemm_group_beside(int count, const cavs_gemm_desc *products, void *workspace, size_t workspace_bytes,
+                            void *stream) {
+  t_lds_pad = 22u << 10;  // with the 33 KB of a tile's panels: two workgroups per CU
+  const int rc = run_group(count, products, workspace, workspace_bytes, nullptr, stream);
+  t_lds_pad = 0;
+  return rc;
 }
 
 int cavs_sgemm_group_embed_bwd(int count, const cavs_gemm_desc *products, int embed_product, float *dtable, const float *ids,

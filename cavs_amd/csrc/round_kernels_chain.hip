@@ -480,6 +480,9 @@ __global__ __launch_bounds__(WAVES * 64) void round_bwd_children_kernel(ChildBwd
   constexpr int THREADS = WAVES * 64, KS = WAVES, GK = 4 * M::NSLOT, NR = M::NR;
   constexpr int NREG = Regions<TILE, KS>::N, RSZ = NB * NR * 64;
   __shared__ float red[NREG * RSZ];
+  // A round of the backward chain is latency, not work: where it shares CUs with a long product on
+  // another stream, its wavefronts go first.
+  __builtin_amdgcn_s_setprio(3);
   const int tid = threadIdx.x, lane = tid & 63, ks = tid >> 6;
   const int x = lane & (TILE - 1), slot = lane / TILE;
   const int H = a.H, K = a.K;

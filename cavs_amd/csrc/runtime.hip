@@ -194,6 +194,12 @@ int cavs_event_record(void *event, void *stream) {
   return CAVS_OK;
 }
 
+int cavs_stream_wait_event(void *stream, void *event) {
+  CAVS_REQUIRE(event, "cavs_stream_wait_event: null event");
+  CAVS_HIP_TRY(hipStreamWaitEvent(as_stream(stream), static_cast<hipEvent_t>(event), 0));
+  return CAVS_OK;
+}
+
 int cavs_event_sync(void *event) {
   CAVS_REQUIRE(event, "cavs_event_sync: null event");
   CAVS_HIP_TRY(hipEventSynchronize(static_cast<hipEvent_t>(event)));

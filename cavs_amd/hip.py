@@ -64,6 +64,7 @@ _SIGS = {
     "cavs_event_create": [C.POINTER(_P)],
     "cavs_event_destroy": [_P],
     "cavs_event_record": [_P, _P],
+    "cavs_stream_wait_event": [_P, _P],
     "cavs_graph_capture_begin": [_P],
     "cavs_graph_capture_end": [_P, C.POINTER(_P)],
     "cavs_graph_launch": [_P, _P],
@@ -79,6 +80,7 @@ _SIGS = {
     "cavs_sgemm": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],
     "cavs_sgemm_addrows": [_I, _I, _I, _I, _I, _P, _I, _P, _I, _P, _I, _I, _P, _I, _P, _Z, _P],
     "cavs_sgemm_group": [_I, C.POINTER(GemmDesc), _P, _Z, _P],
+    "cavs_sgemm_group_beside": [_I, C.POINTER(GemmDesc), _P, _Z, _P],
     "cavs_sgemm_group_embed_bwd": [_I, C.POINTER(GemmDesc), _I, _P, _P, _P, _Z, _P],
     "cavs_sgemm_splitk": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P, _Z, _P],
     "cavs_sgemm_splitk_static": [_I, _I, _I, _I, _I, _F, _P, _I, _P, _I, _F, _P, _I, _P],

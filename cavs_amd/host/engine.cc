@@ -137,6 +137,12 @@ Engine::~Engine() {
     cavs_stream_sync(sched_stream_);
     cavs_stream_destroy(sched_stream_);
   }
+  if (aux_stream_) {
+    cavs_stream_sync(aux_stream_);
+    cavs_stream_destroy(aux_stream_);
+    cavs_event_destroy(aux_fork_ev_);
+    cavs_event_destroy(aux_join_ev_);
+  }
   for (auto &d : dsched_)
     if (d.free_ev) cavs_event_destroy(d.free_ev);
   if (own_stream_) cavs_stream_destroy(stream_);
@@ -212,6 +218,7 @@ void Engine::get_param(const std::string &name, float *host, size_t n, bool grad
   Param &p = param(name);
   if (n != p.n || !host)
     fail(CAVS_EINVAL, "parameter '" + name + "' has " + std::to_string(p.n) + " elements, got " + std::to_string(n));
+  aux_join();
   check(cavs_memcpy_d2h(host, grad ? p.g : p.w, n * 4, stream_));
   check(cavs_stream_sync(stream_));
 }
@@ -951,6 +958,7 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
     run_passes(backward);
   }
   if (backward) {
+    aux_join();  // (the head's weight gradients)
     if (lr != 0.f) {
       // w -= lr * g (cavs/backend/op_impl_sgd.cu); the embedding table by its looked-up rows
       // only: every other row of its gradient is zero, so the dense update would not move it
@@ -1260,13 +1268,13 @@ bool Engine::bias_row_ok() const {
 }
 
 // One launch leaves the chunk sums; the job that ends the step adds them up in index order.
-void Engine::bias_gradient(const std::string &name, const float *inp, int n, int w, DeviceArray<float> &parts) {
+void Engine::bias_gradient(const std::string &name, const float *inp, int n, int w, DeviceArray<float> &parts, void *stream) {
   const size_t bytes = cavs_colsum_blocks_workspace(n, w, 1);
   if (parts.capacity() * 4 < bytes) {
     check(cavs_stream_sync(stream_));
     parts.reserve(bytes / 4 + 1);
   }
-  check(cavs_colsum_blocks(nullptr, inp, w, n, w, 1, nullptr, parts.get(), parts.capacity() * 4, stream_));
+  check(cavs_colsum_blocks(nullptr, inp, w, n, w, 1, nullptr, parts.get(), parts.capacity() * 4, stream ? stream : stream_));
   c_launches_ += 1;
   bias_jobs_.push_back({name, parts.get(), cavs_colsum_parts(n), w, 1, 0});
 }
@@ -1655,11 +1663,37 @@ void Engine::head_forward_backward(bool backward) {
     check(cavs_softmax_xent(loss_.get(), backward ? dlogits_.get() : nullptr, logits_.get(), d_labels_, N, C, stream_));
     c_launches_ += 1;
     if (backward) {
-      // both read d logits and write different outputs: one launch when they are small
-      gemm_group({{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, GO_.get(), H, Wfc.g, H},
-                  wide ? cavs_gemm_desc{0, 1, N, H, C, 1.f, 0.f, dlogits_.get(), C, WfcT_.get(), C, dGO_.get(), H}
-                       : cavs_gemm_desc{0, 0, N, H, C, 1.f, 0.f, dlogits_.get(), C, Wfc.w, H, dGO_.get(), H}});
-      bias_gradient("bfc", dlogits_.get(), N, C, head_bias_parts_);
+      const cavs_gemm_desc dWd{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, GO_.get(), H, Wfc.g, H};
+      const cavs_gemm_desc dGd = wide ? cavs_gemm_desc{0, 1, N, H, C, 1.f, 0.f, dlogits_.get(), C, WfcT_.get(), C, dGO_.get(), H}
+                                      : cavs_gemm_desc{0, 0, N, H, C, 1.f, 0.f, dlogits_.get(), C, Wfc.w, H, dGO_.get(), H};
+      if (wide && !profile_ && !capturing_) {
+        // Only d GraphOutput is on the way of the backward rounds.  The weight and bias gradients are
+        // wanted at the update: they run on the side stream, under the rounds.
+        if (!aux_stream_) {
+          check(cavs_stream_create(&aux_stream_));
+          check(cavs_event_create(&aux_fork_ev_));
+          check(cavs_event_create(&aux_join_ev_));
+        }
+        const size_t need = cavs_sgemm_group_workspace(1, &dWd);
+        if (ws_aux_.capacity() * 4 < need) {
+          check(cavs_stream_sync(aux_stream_));
+          ws_aux_.reserve(need / 4 + 1);
+        }
+        // (forked behind the d GraphOutput product: side by side the two would only share the chip)
+        gemm_group({dGd});
+        check(cavs_event_record(aux_fork_ev_, stream_));
+        check(cavs_stream_wait_event(aux_stream_, aux_fork_ev_));
+        check(cavs_sgemm_group_beside(1, &dWd, ws_aux_.get(), ws_aux_.capacity() * 4, aux_stream_));
+        c_gemm_flops_ += 2.0 * dWd.M * dWd.N * dWd.K;
+        c_launches_ += 1;
+        bias_gradient("bfc", dlogits_.get(), N, C, head_bias_parts_, aux_stream_);
+        check(cavs_event_record(aux_join_ev_, aux_stream_));
+        aux_pending_ = true;
+      } else {
+        // both read d logits and write different outputs: one launch when they are small
+        gemm_group({dWd, dGd});
+        bias_gradient("bfc", dlogits_.get(), N, C, head_bias_parts_);
+      }
     }
     return;
   }
@@ -1691,7 +1725,15 @@ void Engine::head_forward_backward(bool backward) {
   }
 }
 
+// The session's stream takes up what the side stream has been doing.
+void Engine::aux_join() {
+  if (!aux_pending_) return;
+  check(cavs_stream_wait_event(stream_, aux_join_ev_));
+  aux_pending_ = false;
+}
+
 void Engine::sync() {
+  aux_join();
   check(cavs_stream_sync(stream_));
   tail_check();
 }

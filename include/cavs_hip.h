@@ -63,6 +63,8 @@ int cavs_event_create(void **event);
 int cavs_event_destroy(void *event);
 int cavs_event_record(void *event, void *stream);
 int cavs_event_sync(void *event); /* host waits until the event has happened */
+/* work enqueued on `stream` after this call starts once `event` (recorded on another stream) has happened */
+int cavs_stream_wait_event(void *stream, void *event);
 int cavs_event_elapsed_ms(float *ms, void *start, void *stop);
 /* Kernel timing without brackets of its own on the stream: while the calling thread is armed,
  * the first kernel an entry point launches stamps `start` when it begins executing and every
@@ -181,6 +183,13 @@ enum { CAVS_GEMM_C_UNUSED = 1, CAVS_GEMM_A_ZERO = 2, CAVS_GEMM_B_ZERO = 3 };
 size_t cavs_sgemm_group_workspace(int count, const cavs_gemm_desc *products);
 int cavs_sgemm_group(int count, const cavs_gemm_desc *products, void *workspace,
                      size_t workspace_bytes, void *stream);
+/* cavs_sgemm_group for a caller that enqueues the products on a second stream beside a chain of short
+ * dependent launches (the weight gradient of a wide classifier head under the backward rounds,
+ * cavs/midend/statement.cc:106-111): the tile launches of products that run alone ask for LDS they do
+ * not use, so that at most two of their workgroups share a CU and the chain's workgroups find room
+ * on every CU.  Same results. */
+int cavs_sgemm_group_beside(int count, const cavs_gemm_desc *products, void *workspace, size_t workspace_bytes,
+                            void *stream);
 /* cavs_sgemm_group followed by cavs_embed_bwd(dtable, ids, C_k, ldc_k, M_k, N_k) on the result of
  * product k = embed_product (alpha 1, beta 0; its rows are the gradients of looked-up embedding
  * rows): MatMul's input gradient and EmbeddingLookup_grad
