@@ -227,6 +227,13 @@ int cavs_graph_capture_end(void *stream, void **graph_exec) {
   if (!graph_exec) {  // the caller gives the capture up
     if (graph) (void)hipGraphDestroy(graph);
     (void)hipGetLastError();
+    // (an invalidated capture is supposed to end here; if the stream is still in it, say so)
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(as_stream(stream), &status) != hipSuccess || status != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return cavs::set_error(CAVS_EHIP, "cavs_graph_capture_end: the stream is still in a capture (%s, status %d)", hipGetErrorString(rc),
+                             (int)status);
+    }
     return CAVS_OK;
   }
   *graph_exec = nullptr;

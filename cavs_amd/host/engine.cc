@@ -1,7 +1,6 @@
 #include "engine.h"
 
 #include <algorithm>
-#include <cstdlib>
 #include <chrono>
 #include <cstring>
 
@@ -937,9 +936,16 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
       capturing_ = false;
       check(cavs_graph_capture_end(stream_, &exec));
       ok = true;
-    } catch (const Error &) {  // something in there had to wait for the stream (a buffer that grew): not this time
-      if (capturing_) cavs_graph_capture_end(stream_, nullptr);
+    } catch (const Error &e) {  // something in there had to wait for the stream (a buffer that grew): not this time
+      const std::string why = e.what();
+      const int left = capturing_ ? cavs_graph_capture_end(stream_, nullptr) : CAVS_OK;
       capturing_ = false;
+      plan->graph_off = true;
+      // (seen on ROCm 7.2: a capture that was invalidated cannot be ended, and the stream refuses
+      // everything from then on -- better said once than met at every later call)
+      if (left != CAVS_OK)
+        fail(CAVS_EHIP, "recording the launches of a step failed (" + why + ") and the stream did not leave the failed capture (" +
+                            cavs_last_error() + "): this session cannot go on; create it without graph_replay");
     }
     if (ok) {
       if (plan->graphs.size() >= 4) {
@@ -1666,7 +1672,9 @@ void Engine::head_forward_backward(bool backward) {
       const cavs_gemm_desc dWd{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, GO_.get(), H, Wfc.g, H};
       const cavs_gemm_desc dGd = wide ? cavs_gemm_desc{0, 1, N, H, C, 1.f, 0.f, dlogits_.get(), C, WfcT_.get(), C, dGO_.get(), H}
                                       : cavs_gemm_desc{0, 0, N, H, C, 1.f, 0.f, dlogits_.get(), C, Wfc.w, H, dGO_.get(), H};
-      if (wide && !profile_ && !capturing_) {
+      // (not in a session that records graphs: on this runtime a capture on the session's stream comes
+      // out invalidated once that stream has waited for an event of another stream)
+      if (wide && !profile_ && !cfg_.graph_replay) {
         // Only d GraphOutput is on the way of the backward rounds.  The weight and bias gradients are
         // wanted at the update: they run on the side stream, under the rounds.
         if (!aux_stream_) {

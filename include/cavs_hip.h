@@ -79,7 +79,8 @@ int cavs_profile_disarm(int *launched); /* waits for `stop` */
  * `stream` between cavs_graph_capture_begin and cavs_graph_capture_end is recorded instead of run
  * (kernel launches and copies of this library are fine; nothing in between may wait for the
  * stream or for an event).  cavs_graph_capture_end hands back the replayable graph, or, called with
- * graph_exec = NULL, ends a capture the caller gives up.  cavs_graph_launch enqueues the recorded
+ * graph_exec = NULL, ends a capture the caller gives up (an error then means the stream did not
+ * leave the capture: a capture invalidated by a forbidden call cannot be ended on every runtime).  cavs_graph_launch enqueues the recorded
  * work -- same kernels, same arguments, same order.  For the host loop that re-issues the launches
  * of a batch structure seen before (GraphStatement::Run's round loop, cavs/midend/statement.cc:69-76). */
 int cavs_graph_capture_begin(void *stream);

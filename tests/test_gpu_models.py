@@ -575,16 +575,18 @@ def test_training_step_on_reader_batches(oracle, kind):
     compare(got, want)
 
 
-@pytest.mark.parametrize("model,H,pool", [("treefc", 32, 3), ("treelstm", 32, 3), ("lstm", 32, 2), ("treelstm", 512, 2)])
-def test_recorded_graph_of_a_cached_plan_gives_the_steps_of_the_host_loop(model, H, pool):
+@pytest.mark.parametrize("model,H,pool,Cc", [("treefc", 32, 3, 5), ("treelstm", 32, 3, 5), ("lstm", 32, 2, 5), ("treelstm", 512, 2, 5),
+                                             ("lstm", 32, 2, 9000)])
+def test_recorded_graph_of_a_cached_plan_gives_the_steps_of_the_host_loop(model, H, pool, Cc):
     """graph_replay: on a batch structure seen before, with the same device-resident feeds, the
     forward pass, loss head and backward pass are enqueued as one recorded graph.  Training steps
     (with the parameter update) through such a session and through one that issues every launch
     from the host loop give the same losses and parameters -- bit for bit where no gradient is
     accumulated with atomics (Tree-FC), to the tolerance of the accumulation order elsewhere.
-    H = 512 puts the launches over the rounds near the roots inside the graph."""
+    H = 512 puts the launches over the rounds near the roots inside the graph; 9000 classes make the
+    head a wide one (its weight gradient goes to a side stream in the session that does not record)."""
     import torch
-    V, Cc = 31, 5
+    V = 31
     E = H if model == "lstm" else 12
     loss = "softmax" if model != "treefc" else "root_sq"
     ws = [small_workload(model, 401 + k, B=5 + k, H=H, E=E, V=V, C=Cc) for k in range(pool)]
