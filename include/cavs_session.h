@@ -67,8 +67,9 @@ typedef struct {
    * whose rows can be dealt to eight groups, whole trees of the message flow per group, with at
    * most this many rows per group (the last forward rounds, the first backward rounds) run as one launch per
    * direction (cavs_treelstm_tail_fwd / _bwd) instead of one launch per round
-   * (cavs/midend/statement.cc:69-76,106-111).  0 = default (32: larger shares were measured no faster
-   * than launches of their own), negative = never.  The session
+   * (cavs/midend/statement.cc:69-76,106-111).  0 = default (64, which at 64 trees per batch takes in
+   * every round above the leaves; a group's share of a round runs in slices of at most 32 rows),
+   * negative = never.  The session
    * checks once, when it is created, that the device runs such a launch's workgroups all at once,
    * each group on one XCD, and keeps to one launch per round if not. */
   int tail_rows;
