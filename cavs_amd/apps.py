@@ -135,6 +135,12 @@ class App:
         return bool(a.cavs_app_uses_fused_path())
 
     @property
+    def fused_kind(self):
+        """0: F runs op by op; 1: on the hand-written round kernels; 2: on kernels generated for it."""
+        a, _ = libs()
+        return int(a.cavs_app_uses_fused_path())
+
+    @property
     def generated_kernels(self):
         """Kernels the OPT_FUSION pass generated for the programs compiled so far."""
         a, _ = libs()

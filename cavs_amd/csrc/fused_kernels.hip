@@ -19,6 +19,39 @@ struct FusedKernel {
 
 constexpr int kFusedBlock = 256;
 
+// A vertex function's generated round kernels: one module, its kernels by a fixed order of names.
+constexpr int kCellKernels = 6;
+const char *const kCellKernelNames[kCellKernels] = {"cell_fwd", "cell_leaves", "cell_bwd", "cell_bwd_rows", "cell_transpose", "cell_bias"};
+struct CellModule {
+  hipModule_t module = nullptr;
+  hipFunction_t fn[kCellKernels] = {};
+};
+
+// compiles `source` for gfx950 into `code`; the log of a failed compile goes into the error text
+int rtc_compile(const char *what, const char *source, std::vector<char> *code) {
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source, (std::string(what) + ".hip").c_str(), 0, nullptr, nullptr);
+  if (r != HIPRTC_SUCCESS) return set_error(CAVS_EHIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
+  // FMA contraction off: the reference builds fused kernels with --fmad=false; packed fp32 math is
+  // disabled on this target by policy
+  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  r = hiprtcCompileProgram(prog, 7, opts);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, &log[0]);
+    hiprtcDestroyProgram(&prog);
+    return set_error(CAVS_EINVAL, "hiprtc compile of %s failed: %.380s", what, log.c_str());
+  }
+  size_t code_size = 0;
+  hiprtcGetCodeSize(prog, &code_size);
+  code->resize(code_size);
+  hiprtcGetCode(prog, code->data());
+  hiprtcDestroyProgram(&prog);
+  return CAVS_OK;
+}
+
 }  // namespace cavs
 
 using namespace cavs;
@@ -28,27 +61,8 @@ extern "C" {
 int cavs_fused_compile(const char *kernel_name, const char *source, void **handle) {
   CAVS_REQUIRE(kernel_name && source && handle, "cavs_fused_compile: null argument");
   *handle = nullptr;
-  hiprtcProgram prog;
-  hiprtcResult r = hiprtcCreateProgram(&prog, source, (std::string(kernel_name) + ".hip").c_str(), 0,
-                                       nullptr, nullptr);
-  if (r != HIPRTC_SUCCESS)
-    return set_error(CAVS_EHIP, "hiprtcCreateProgram: %s", hiprtcGetErrorString(r));
-  // FMA contraction off: the reference builds fused kernels with --fmad=false
-  const char *opts[] = {"--offload-arch=gfx950", "-O3", "-ffp-contract=off"};
-  r = hiprtcCompileProgram(prog, 3, opts);
-  if (r != HIPRTC_SUCCESS) {
-    size_t n = 0;
-    hiprtcGetProgramLogSize(prog, &n);
-    std::string log(n, '\0');
-    if (n) hiprtcGetProgramLog(prog, &log[0]);
-    hiprtcDestroyProgram(&prog);
-    return set_error(CAVS_EINVAL, "hiprtc compile of %s failed: %.380s", kernel_name, log.c_str());
-  }
-  size_t code_size = 0;
-  hiprtcGetCodeSize(prog, &code_size);
-  std::vector<char> code(code_size);
-  hiprtcGetCode(prog, code.data());
-  hiprtcDestroyProgram(&prog);
+  std::vector<char> code;
+  if (int rc = rtc_compile(kernel_name, source, &code)) return rc;
   FusedKernel *k = new FusedKernel;
   k->name = kernel_name;
   hipError_t e = hipModuleLoadData(&k->module, code.data());
@@ -105,6 +119,55 @@ int cavs_fused_release(void *handle) {
   FusedKernel *k = static_cast<FusedKernel *>(handle);
   hipError_t e = hipModuleUnload(k->module);
   delete k;
+  CAVS_HIP_TRY(e);
+  return CAVS_OK;
+}
+
+int cavs_cell_compile(const char *source, void **handle) {
+  CAVS_REQUIRE(source && handle, "cavs_cell_compile: null argument");
+  *handle = nullptr;
+  std::vector<char> code;
+  if (int rc = rtc_compile("cell", source, &code)) return rc;
+  CellModule *m = new CellModule;
+  hipError_t e = hipModuleLoadData(&m->module, code.data());
+  for (int i = 0; i < kCellKernels && e == hipSuccess; i++) e = hipModuleGetFunction(&m->fn[i], m->module, kCellKernelNames[i]);
+  if (e != hipSuccess) {
+    if (m->module) (void)hipModuleUnload(m->module);
+    delete m;
+    return set_error(CAVS_EHIP, "loading the generated round kernels: %s", hipGetErrorString(e));
+  }
+  *handle = m;
+  return CAVS_OK;
+}
+
+int cavs_cell_launch(void *handle, int kernel, unsigned grid_x, unsigned grid_y, unsigned grid_z, unsigned block, const void *args,
+                     size_t args_bytes, void *stream) {
+  CAVS_REQUIRE(handle && args, "cavs_cell_launch: null argument");
+  CAVS_REQUIRE(kernel >= 0 && kernel < kCellKernels, "cavs_cell_launch: no kernel %d", kernel);
+  CAVS_REQUIRE(block >= 64 && block <= 256 && block % 64 == 0 && args_bytes > 0 && args_bytes <= 4096,
+               "cavs_cell_launch: bad launch shape (block=%u, %zu argument bytes)", block, args_bytes);
+  if (grid_x == 0 || grid_y == 0 || grid_z == 0) return CAVS_OK;
+  CellModule *m = static_cast<CellModule *>(handle);
+  // the kernels take one struct by value: its bytes are the argument buffer
+  size_t bytes = args_bytes;
+  void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, const_cast<void *>(args), HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+  LaunchProbe &p = launch_probe();
+  if (p.armed) {
+    hipEvent_t s = p.started ? nullptr : p.start;
+    p.started = true;
+    CAVS_HIP_TRY(hipExtModuleLaunchKernel(m->fn[kernel], grid_x * block, grid_y, grid_z, block, 1, 1, 0, as_stream(stream), nullptr, config,
+                                          s, p.stop, 0));
+  } else {
+    CAVS_HIP_TRY(hipModuleLaunchKernel(m->fn[kernel], grid_x, grid_y, grid_z, block, 1, 1, 0, as_stream(stream), nullptr, config));
+  }
+  return CAVS_OK;
+}
+
+int cavs_cell_release(void *handle) {
+  if (!handle) return CAVS_OK;
+  CellModule *m = static_cast<CellModule *>(handle);
+  hipError_t e = hipModuleUnload(m->module);
+  delete m;
   CAVS_HIP_TRY(e);
   return CAVS_OK;
 }

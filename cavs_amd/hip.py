@@ -138,6 +138,9 @@ _SIGS = {
     "cavs_fused_compile": [C.c_char_p, C.c_char_p, C.POINTER(_P)],
     "cavs_fused_launch": [_P, C.POINTER(_P), _I, C.POINTER(_P), _I, C.POINTER(_I), C.POINTER(_I), _I, _P],
     "cavs_fused_release": [_P],
+    "cavs_cell_compile": [C.c_char_p, C.POINTER(_P)],
+    "cavs_cell_launch": [_P, _I, C.c_uint, C.c_uint, C.c_uint, C.c_uint, _P, C.c_size_t, _P],
+    "cavs_cell_release": [_P],
     "cavs_schedule_frontier": [_P, _I, _P, _P, _P, _P, _P, _P, _P],
     "cavs_schedule_arena": [_P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, C.c_long, _P, _P, _Z, _P],
 }

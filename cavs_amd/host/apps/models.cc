@@ -74,6 +74,93 @@ class TreeLSTM : public GraphSupport {
   Sym b_i, b_f, b_u, b_o, U_iou, U_f;
 };
 
+// A binary Tree-LSTM whose forget gates have a recurrent matrix per child (f_l = sigmoid(x W_f +
+// h_l U_fl + b_f), f_r likewise with U_fr), with the gates' biases in the order of their columns:
+// not one of the reference's applications -- a vertex function a user might write, which the
+// hand-written round kernels do not cover.  U holds [U_iou (H x 3H) | U_fl (H x H) | U_fr (H x H)].
+class TreeLSTM2 : public GraphSupport {
+ public:
+  TreeLSTM2(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {4 * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    U = Sym::Variable(DT_FLOAT, {5 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {4 * H}, Sym::Zeros());
+    b_iou = B.Slice(0, 3 * H);
+    b_f = B.Slice(3 * H, H);
+    U_iou = U.Slice(0, 3 * H * H).Reshape({H, 3 * H});
+    U_fl = U.Slice(3 * H * H, H * H).Reshape({H, H});
+    U_fr = U.Slice(4 * H * H, H * H).Reshape({H, H});
+  }
+  void Node() override {
+    Sym left = Gather(0, {2 * H});
+    Sym right = Gather(1, {2 * H});
+    Sym h_l, c_l, h_r, c_r;
+    tie(h_l, c_l) = left.Split2();
+    tie(h_r, c_r) = right.Split2();
+    Sym h_lr = h_l.Mirror() + h_r.Mirror();
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, 4 * H}).Mirror()).Reshape({H * 4});
+    Sym xW_iou = xW.Slice(0, 3 * H);
+    Sym xW_f = xW.Slice(3 * H, H);
+    Sym iou = xW_iou + Sym::MatMul(h_lr.Reshape({1, H}), U_iou.Mirror()).Reshape({H * 3}) + b_iou.Mirror();
+    Sym gi, go, gu;
+    tie(gi, go, gu) = iou.Split3();
+    Sym i = gi.Sigmoid(), o = go.Sigmoid(), u = gu.Tanh();
+    Sym f_l = (xW_f.Mirror() + Sym::MatMul(h_l.Mirror().Reshape({1, H}), U_fl.Mirror()).Reshape({H}) + b_f.Mirror()).Sigmoid();
+    Sym f_r = (xW_f.Mirror() + Sym::MatMul(h_r.Mirror().Reshape({1, H}), U_fr.Mirror()).Reshape({H}) + b_f.Mirror()).Sigmoid();
+    Sym c = i * u + f_l * c_l + f_r * c_r;
+    Sym h = o * Sym::Tanh(c.Mirror());
+    Scatter(Sym::Concat({h.Mirror(), c.Mirror()}));
+    Push(h.Mirror());
+  }
+  Sym embedding, W, U, B;
+
+ private:
+  int E, H;
+  Sym b_iou, b_f, U_iou, U_fl, U_fr;
+};
+
+// A gated tree cell with one state block: z = sigmoid(x W_z + (h_l + h_r) U_z + b_z),
+// u = tanh(x W_u + h_l U_l + h_r U_r + b_u), h = u * z + (h_l + h_r) - z * (h_l + h_r) scaled by a half.
+// The children's states enter both through products and elementwise, and the product of u takes the
+// concatenation of the children as its left operand.
+class TreeGate : public GraphSupport {
+ public:
+  TreeGate(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {2 * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    U = Sym::Variable(DT_FLOAT, {3 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {2 * H}, Sym::Zeros());
+    U_z = U.Slice(0, H * H).Reshape({H, H});
+    U_lr = U.Slice(H * H, 2 * H * H).Reshape({2 * H, H});
+  }
+  void Node() override {
+    Sym h_l = Gather(0, {H});
+    Sym h_r = Gather(1, {H});
+    Sym hs = h_l.Mirror() + h_r.Mirror();
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, 2 * H}).Mirror()).Reshape({H * 2});
+    Sym xW_z, xW_u;
+    tie(xW_z, xW_u) = xW.Split2();
+    Sym b_z, b_u;
+    tie(b_z, b_u) = B.Mirror().Split2();
+    Sym z = (xW_z + Sym::MatMul(hs.Mirror().Reshape({1, H}), U_z.Mirror()).Reshape({H}) + b_z).Sigmoid();
+    Sym lr = Sym::Concat({h_l.Mirror(), h_r.Mirror()});
+    Sym u = (xW_u + Sym::MatMul(lr.Reshape({1, 2 * H}), U_lr.Mirror()).Reshape({H}) + b_u).Tanh();
+    Sym half = hs.Mirror() * hs.Mirror().Sigmoid();  // a smooth stand-in for a constant factor
+    Sym h = u * z.Mirror() + half.Mirror() - z.Mirror() * half.Mirror();
+    Scatter(h.Mirror());
+    Push(h.Mirror());
+  }
+  Sym embedding, W, U, B;
+
+ private:
+  int E, H;
+  Sym U_z, U_lr;
+};
+
 class SeqLSTM : public GraphSupport {
  public:
   SeqLSTM(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), H(d.H) {
@@ -186,6 +273,14 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       auto *m = new TreeLSTM(app->graph, app->vertex, d);
       app->gs.reset(m);
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model == "treelstm2") {
+      auto *m = new TreeLSTM2(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model == "treegate") {
+      auto *m = new TreeGate(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model == "lstm") {
       auto *m = new SeqLSTM(app->graph, app->vertex, d);
       app->gs.reset(m);
@@ -244,7 +339,7 @@ int cavs_app_set_param(const char *name, const float *data, size_t n) {
 void cavs_app_configure(int pairing, int allow_fused) {
   if (!g_app) return;
   g_app->sess->SetPairing(pairing);
-  g_app->sess->AllowFusedPath(allow_fused != 0);
+  g_app->sess->SetLoweringMode(allow_fused);
 }
 
 // One Session::Run of {train, loss, graph_output} (or without train).  graph is the
@@ -304,7 +399,7 @@ long cavs_app_read(const char *edge, float *out, size_t cap) {
   return C_ReadTensor(g_app->sess->handle(), edge, out, cap);
 }
 
-int cavs_app_uses_fused_path(void) { return g_app && g_app->sess->UsesFusedPath(); }
+int cavs_app_uses_fused_path(void) { return g_app ? g_app->sess->FusedPathKind() : 0; }
 int cavs_app_generated_kernels(void) { return g_app ? g_app->sess->GeneratedKernels() : 0; }
 
 void cavs_app_destroy(void) {

@@ -1,0 +1,100 @@
+// Description of a vertex function of the general one-stage shape
+//
+//   state' , ret = f( x*W , sum_t A_t * B_t , bias , states of the children )      (f elementwise)
+//
+// as the engine runs it on generated round kernels: which views of which parameters feed the
+// products, which sums of children's state blocks are their left operands, how many values a vertex
+// keeps for the backward pass, and the source of the kernels (the product loops written out for this
+// function, the elementwise part f and its derivative generated from the operator graph).  Takes the
+// place of the reference's kernel fusion for a whole vertex function
+// (cavs/midend/runtime_compiler/parser.cc:73-139, code_generator.cc:104-185) with the products inside.
+#ifndef CAVS_HOST_CELL_H_
+#define CAVS_HOST_CELL_H_
+
+#include <string>
+#include <vector>
+
+namespace cavs {
+
+struct CellParamRef {
+  int param = -1;    // index into CellSpec::params
+  long offset = 0;   // first element of the view inside that parameter
+};
+
+// Left operand of a product: the sum over the children in `mask` (bit k = child k) of block `block`
+// of their state rows; a missing child contributes zero.
+struct CellASrc {
+  int mask = 0, block = 0;
+};
+
+// One accumulator of the round kernels: sum over its terms of  A[asrc] (1 x H)  *  B[brow .. brow + H) x [col .. col + H).
+struct CellTerm {
+  int asrc = 0;
+  long brow = 0;
+};
+struct CellProduct {
+  std::vector<CellTerm> terms;
+  CellParamRef B;   // the view the rows and columns count from, row-major with leading dimension ldb
+  int ldb = 0;
+  long col = 0;
+  int dcol = -1;    // block of the per-vertex gradient rows that holds d(this accumulator)
+};
+
+struct CellBias {
+  CellParamRef ref;  // H values
+  int dcol = -1;     // block of the gradient rows whose column sums are its gradient
+};
+
+struct CellParam {
+  std::string name;  // engine parameter ("Emb" for the embedding table, else "P<i>")
+  long size = 0;
+};
+
+struct CellSpec {
+  int H = 0, K = 0, S = 0;      // block width, children per vertex, state blocks per message
+  int E = 0, V = 0, NX = 0;     // embedding width, vocabulary, blocks of x * W (0: F reads no vertex input)
+  CellParamRef W;               // [E, NX * H]
+  std::vector<CellParam> params;
+  std::vector<CellASrc> asrc;
+  std::vector<CellProduct> products;
+  std::vector<CellBias> biases;
+  int ND = 0;                   // blocks of a vertex's gradient row: d(x*W) blocks first, in order
+  int NSV = 0;                  // blocks a vertex saves for the backward pass
+  int waves = 0;                // wavefronts per workgroup of the round kernels (they split the k range)
+  std::string source;           // the kernels
+  std::string key;              // canonical text of the function (equal keys: equal kernels)
+  int terms() const {
+    int n = 0;
+    for (const CellProduct &p : products) n += (int)p.terms.size();
+    return n;
+  }
+};
+
+// Order of the 8-byte argument slots of the generated kernels (struct CellArgs in their source).
+enum CellArg {
+  CA_POOL = 0,   // float*  message pool [*, S*H]
+  CA_CHILD,      // int*    pool rows of the children by slab row [K * N]
+  CA_PAIR,       // int*    pool row a slab row's message goes to [N]
+  CA_KIDS,       // int*    slab rows of the children by slab row [K * N]
+  CA_T2J,        // int*    vertex id by slab row [N]
+  CA_ROWS,       // int*    slab rows for the rows kernel (the vertices nobody sends a gradient to)
+  CA_XW,         // float*  [N, NX*H]
+  CA_SV,         // float*  [N, NSV*H]
+  CA_ASRC,       // float*  [N, NA*H]
+  CA_GO,         // float*  [N, H] by vertex id: the pushed value / its gradient
+  CA_D,          // float*  [N, ND*H]
+  CA_DS,         // float*  [N, S*H] elementwise part of a vertex's message gradient
+  CA_BT,         // float*  transposed H x H blocks of the products' terms
+  CA_COLSUM,     // float*  [ND*H] column sums of D
+  CA_OFF,        // long    first slab row of the round
+  CA_N,          // long    rows
+  CA_PARAM0,     // float*  parameters, then their gradients, in CellSpec::params order
+  CA_MAX_PARAMS = 8,
+  CA_SLOTS = CA_PARAM0 + 2 * CA_MAX_PARAMS
+};
+
+// kernels of a compiled cell, in the order cavs_cell_compile looks them up
+enum CellKernel { CK_FWD = 0, CK_LEAVES, CK_BWD, CK_BWD_ROWS, CK_TRANSPOSE, CK_BIAS, CK_COUNT };
+
+}  // namespace cavs
+#endif

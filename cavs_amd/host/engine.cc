@@ -23,8 +23,10 @@ inline size_t grow(size_t need, size_t have) {
 }
 }  // namespace
 
-Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg) {
-  if (cfg.model < 0 || cfg.model > 2) fail(CAVS_EINVAL, "unknown model " + std::to_string(cfg.model));
+Engine::Engine(const cavs_session_config &cfg, void *external_stream, std::shared_ptr<const CellSpec> cell) : cfg_(cfg), cell_(std::move(cell)) {
+  if (cfg.model < 0 || cfg.model > CAVS_MODEL_CELL) fail(CAVS_EINVAL, "unknown model " + std::to_string(cfg.model));
+  if ((cfg.model == CAVS_MODEL_CELL) != (cell_ != nullptr))
+    fail(CAVS_EINVAL, "model CAVS_MODEL_CELL is a vertex function lowered by the front end and comes with its description");
   if (cfg.loss < 0 || cfg.loss > 2) fail(CAVS_EINVAL, "unknown loss " + std::to_string(cfg.loss));
   if (cfg.pairing < 0 || cfg.pairing > 1) fail(CAVS_EINVAL, "unknown pairing");
   if (cfg.H <= 0) fail(CAVS_EINVAL, "hidden size must be positive");
@@ -33,7 +35,15 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
   ld_e_ = cfg.model == CAVS_MODEL_TREELSTM ? E_ + 4 : E_;
   mw_ = cfg.model == CAVS_MODEL_TREEFC ? cfg.H : 2 * cfg.H;
   nch_ = cfg.model == CAVS_MODEL_LSTM ? 1 : 2;
-  if (cfg.model != CAVS_MODEL_TREEFC && (cfg.V <= 0 || E_ <= 0))
+  if (cell_) {
+    if (cell_->H != cfg.H || cell_->K < 1 || cell_->K > 2 || (int)cell_->params.size() > CA_MAX_PARAMS)
+      fail(CAVS_EINVAL, "the description of the lowered vertex function does not fit the session");
+    E_ = ld_e_ = cell_->E;
+    mw_ = cell_->S * cfg.H;
+    nch_ = cell_->K;
+  }
+  const bool reads_x = cell_ ? cell_->NX > 0 : cfg.model != CAVS_MODEL_TREEFC;
+  if (reads_x && (cfg.V <= 0 || E_ <= 0))
     fail(CAVS_EINVAL, "vocabulary and embedding sizes must be positive");
   if (cfg.loss == CAVS_LOSS_SOFTMAX && cfg.C <= 0) fail(CAVS_EINVAL, "class count must be positive");
   check(cavs_init(cfg.device));
@@ -55,6 +65,10 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream) : cfg_(cfg
       add_param("Emb", (size_t)cfg.V * H);
       add_param("W", 8 * H * H);
       add_param("Bv", 4 * H);
+      break;
+    case CAVS_MODEL_CELL:
+      for (const CellParam &p : cell_->params) add_param(p.name, (size_t)p.size);
+      check(cavs_cell_compile(cell_->source.c_str(), &cell_module_));
       break;
     default:
       add_param("W", 2 * H * H);
@@ -128,6 +142,7 @@ void Engine::tail_check() {
 
 Engine::~Engine() {
   cavs_stream_sync(stream_);
+  cavs_cell_release(cell_module_);
   for (auto &e : ev_) cavs_event_destroy(e);
   for (auto &h : hlists_) {
     if (h.free_ev) cavs_event_destroy(h.free_ev);
@@ -363,7 +378,25 @@ void Engine::reserve_edges() {
   R(G_, cap * nch_ * mw);
   R(r_dmsg_, rc * mw);
   R(r_dG_, rc * nch_ * mw);
-  if (cfg_.model != CAVS_MODEL_TREEFC) {
+  if (cell_) {
+    const CellSpec &c = *cell_;
+    if (c.NX > 0) {
+      R(xs_, cap);
+      if (xs_prev_.capacity() < cap) {
+        R(xs_prev_, cap);
+        emb_sparse_valid_ = false;
+      }
+      R(e_, cap * E_);
+      R(de_, cap * E_);
+      R(xW_, cap * c.NX * H);
+    }
+    R(gates_, cap * std::max(1, c.NSV) * H);          // what a vertex keeps for the backward pass
+    R(hlr_, cap * c.asrc.size() * H);                 // the products' left operands by slab row
+    R(dxW_, cap * c.ND * H);                          // the gradient rows
+    R(dc_, cap * mw);                                 // elementwise part of the message gradients
+    R(UT_, (size_t)c.terms() * H * H);
+    R(cell_colsum_, (size_t)c.ND * H);
+  } else if (cfg_.model != CAVS_MODEL_TREEFC) {
     R(xs_, cap);
     if (xs_prev_.capacity() < cap) {  // the list of dirty rows does not survive a reallocation
       R(xs_prev_, cap);
@@ -390,7 +423,7 @@ void Engine::reserve_edges() {
     R(dxW_, cap * H);
     R(r_z_, rc * H);
   }
-  if (fused_rows() > 0) R(UT_, (size_t)(cfg_.model == CAVS_MODEL_TREEFC ? 2 : 4) * H * H);
+  if (fused_rows() > 0 && !cell_) R(UT_, (size_t)(cfg_.model == CAVS_MODEL_TREEFC ? 2 : 4) * H * H);
   if (fused_rows() > 0 && ((cfg_.model == CAVS_MODEL_TREELSTM && (cavs_round_packed_ok(1, H) || cavs_round_packed_ok(65, H))) ||
                            (cfg_.model == CAVS_MODEL_LSTM && (cavs_lstm_round_packed_ok(1, H) || cavs_lstm_round_packed_ok(65, H)))))
     R(Upk_, (size_t)4 * H * H);
@@ -744,16 +777,13 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
 void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out) {
   state_epoch_++;
   begin_step(graph, B, maxlen);
-  if ((cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x) && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
+  const bool reads_x = cell_ ? cell_->NX > 0 : (cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x);
+  if (reads_x && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
   d_x_ = x_dev;
   check(cavs_event_record(ev_[0], stream_));
   fwd_out_ = graph_out ? graph_out : GO_.get();
   out_folded_ = false;
-  switch (cfg_.model) {
-    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
-    case CAVS_MODEL_LSTM: lstm_forward(); break;
-    default: treefc_forward();
-  }
+  model_forward();
   pop_ret(fwd_out_);
   check(cavs_event_record(ev_[1], stream_));
   ev_valid_ = true;
@@ -770,11 +800,7 @@ void Engine::backward_only(const float *dgraph_out, bool settle_biases) {
   state_epoch_++;
   d_dgo_ = dgraph_out;
   check(cavs_event_record(ev_[2], stream_));
-  switch (cfg_.model) {
-    case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
-    case CAVS_MODEL_LSTM: lstm_backward(); break;
-    default: treefc_backward();
-  }
+  model_backward();
   if (settle_biases) settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
   check(cavs_event_record(ev_[3], stream_));
   ev_bwd_valid_ = true;
@@ -786,11 +812,7 @@ void Engine::run_passes(bool backward) {
   if (!capturing_) check(cavs_event_record(ev_[0], stream_));
   fwd_out_ = GO_.get();
   out_folded_ = false;
-  switch (cfg_.model) {
-    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
-    case CAVS_MODEL_LSTM: lstm_forward(); break;
-    default: treefc_forward();
-  }
+  model_forward();
   pop_ret(GO_.get());
   if (!capturing_) check(cavs_event_record(ev_[1], stream_));
   ev_valid_ = !capturing_;
@@ -800,11 +822,7 @@ void Engine::run_passes(bool backward) {
   ev_bwd_valid_ = false;
   if (backward) {
     if (!capturing_) check(cavs_event_record(ev_[2], stream_));
-    switch (cfg_.model) {
-      case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
-      case CAVS_MODEL_LSTM: lstm_backward(); break;
-      default: treefc_backward();
-    }
+    model_backward();
     if (!capturing_) check(cavs_event_record(ev_[3], stream_));
     ev_bwd_valid_ = !capturing_;
   }
@@ -1006,6 +1024,24 @@ void Engine::step(const int *graph, int B, int maxlen, const void *x, const void
 
 // FunctionPopRet (cavs/backend/op_impl_graphop.cu:304-318): GraphOutput[tids_to_jobids[t]] =
 // ret[t].  Push's slab copy is folded in: the h half of the message slab is the return value.
+void Engine::model_forward() {
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_forward(); break;
+    case CAVS_MODEL_LSTM: lstm_forward(); break;
+    case CAVS_MODEL_CELL: cell_forward(); break;
+    default: treefc_forward();
+  }
+}
+
+void Engine::model_backward() {
+  switch (cfg_.model) {
+    case CAVS_MODEL_TREELSTM: treelstm_backward(); break;
+    case CAVS_MODEL_LSTM: lstm_backward(); break;
+    case CAVS_MODEL_CELL: cell_backward(); break;
+    default: treefc_backward();
+  }
+}
+
 void Engine::pop_ret(float *graph_out) {
   if (out_folded_) return;  // already written by the rounds
   scatter(graph_out, cfg_.H, d_t2j_, msg_.get(), mw_, N_, cfg_.H);
@@ -1020,6 +1056,7 @@ void Engine::pop_ret(float *graph_out) {
 // round has both children) and H in whole MFMA tiles.
 int Engine::fused_rows() const {
   if (!(cfg_.opt & CAVS_OPT_BATCHING) || cfg_.H % 32 != 0) return 0;
+  if (cell_) return 1 << 30;  // the generated kernels take rounds of any size
   if (cfg_.fused_round_rows < 0) return 0;
   // measured crossover with the separate launches: about 2400 rows at H=512, 1500 at H=1024
   return cfg_.fused_round_rows > 0 ? cfg_.fused_round_rows : (cfg_.H <= 512 ? 2048 : 1024);
@@ -1618,6 +1655,176 @@ void Engine::treefc_backward() {
               param("W").g, H);
   if (cfg_.use_bias) {
     bias_gradient("Bv", dxW_.get(), N, H, bias_parts_);
+  }
+}
+
+// ------------------------------------------------------------------ a vertex function on generated kernels
+// The general one-stage shape (cell.h): x * W for all vertices up front, one launch per round that
+// gathers, multiplies, runs the elementwise part and scatters; backward one launch per round that
+// hands d(state) on to the children and runs their elementwise part, then the weight gradients as
+// products over all rows.  The message flow of the batch must be a forest (every message read once).
+void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go) {
+  const CellSpec &c = *cell_;
+  union Slot {
+    const void *p;
+    long long i;
+  } a[CA_SLOTS];
+  std::memset(a, 0, sizeof a);
+  a[CA_POOL].p = pool_.get();
+  a[CA_CHILD].p = d_child_;
+  a[CA_PAIR].p = d_pair_;
+  a[CA_KIDS].p = d_kid_rows_;
+  a[CA_T2J].p = d_t2j_;
+  a[CA_ROWS].p = rows;
+  a[CA_XW].p = xW_.get();
+  a[CA_SV].p = gates_.get();
+  a[CA_ASRC].p = hlr_.get();
+  a[CA_GO].p = go;
+  a[CA_D].p = dxW_.get();
+  a[CA_DS].p = dc_.get();
+  a[CA_BT].p = UT_.get();
+  a[CA_COLSUM].p = cell_colsum_.get();
+  a[CA_OFF].i = off;
+  a[CA_N].i = n;
+  for (size_t i = 0; i < c.params.size(); i++) {
+    const Param &p = param(c.params[i].name);
+    a[CA_PARAM0 + i].p = p.w;
+    a[CA_PARAM0 + CA_MAX_PARAMS + i].p = p.g;
+  }
+  check(cavs_cell_launch(cell_module_, k, gx, gy, gz, block, a, sizeof a, stream_));
+  c_launches_ += 1;
+}
+
+void Engine::cell_forward() {
+  const CellSpec &c = *cell_;
+  const int N = N_, H = cfg_.H;
+  if (!forest_)
+    fail(CAVS_EUNSUPPORTED,
+         "the lowered vertex function needs the batch scheduler and a batch in which every message is read exactly once; "
+         "open the session without the fused path for other batches");
+  if (c.NX > 0) {
+    ProfScope ps(this, K_GEMM);
+    check(cavs_embed_pull_sgemm(xW_.get(), c.NX * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E_,
+                                param(c.params[c.W.param].name).w + c.W.offset, c.NX * H, c.NX * H, 0, 0, stream_));
+    c_gemm_flops_ += 2.0 * N * c.NX * H * E_;
+    c_launches_ += 1;
+  }
+  out_folded_ = true;  // the rounds write the pushed value by vertex id themselves
+  const unsigned block = 64u * c.waves;
+  for (const Round &r : sched_->rounds) {
+    if (leaf_round(r)) {
+      ProfScope ps(this, K_GATES);
+      cell_launch(CK_LEAVES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, fwd_out_);
+    } else {
+      ProfScope ps(this, K_ROUND);
+      cell_launch(CK_FWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, fwd_out_);
+      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+      c_gather_rows_ += (double)c.K * r.n;
+    }
+    c_scatter_rows_ += r.n;
+  }
+}
+
+void Engine::cell_backward() {
+  const CellSpec &c = *cell_;
+  const int N = N_, H = cfg_.H, lp = sched_->leaf_prefix;
+  const unsigned block = 64u * c.waves;
+  backward_prologue({}, c.NX > 0);
+  // a parameter F reads only parts of: the rest of its gradient is zero
+  {
+    std::vector<long> covered(c.params.size(), 0);
+    if (c.NX > 0) covered[c.W.param] += (long)E_ * c.NX * H;
+    for (const CellProduct &p : c.products) covered[p.B.param] += (long)p.terms.size() * H * H;
+    for (const CellBias &b : c.biases) covered[b.ref.param] += H;
+    for (size_t i = 0; i < c.params.size(); i++)
+      if (c.params[i].name != "Emb" && covered[i] < c.params[i].size) {
+        check(cavs_zero(param(c.params[i].name).g, (size_t)c.params[i].size * 4, stream_));
+        c_launches_ += 1;
+      }
+  }
+  {
+    ProfScope ps(this, K_OTHER);
+    cell_launch(CK_TRANSPOSE, H / 32, H / 32, c.terms(), 256, 0, 0, nullptr, d_dgo_);
+  }
+  if (n_orphans_ > 0) {
+    ProfScope ps(this, K_GATES);
+    cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
+  }
+  for (int k : sched_->bwd_rounds) {
+    const Round &r = sched_->rounds[k];
+    c_gather_rows_ += r.n;
+    if (leaf_round(r)) continue;
+    ProfScope ps(this, K_ROUND);
+    cell_launch(CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
+    c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+    c_scatter_rows_ += (double)c.K * r.n;
+  }
+  // the weight gradients, once over all rows: runs of terms whose operands, columns and gradient
+  // blocks are adjacent go as one product
+  const int ldd = c.ND * H, lda = (int)c.asrc.size() * H;
+  std::vector<cavs_gemm_desc> products;
+  if (c.NX > 0) {
+    float *W = param(c.params[c.W.param].name).w + c.W.offset, *dW = param(c.params[c.W.param].name).g + c.W.offset;
+    products.push_back({0, 1, N, E_, c.NX * H, 1.f, 0.f, dxW_.get(), ldd, W, c.NX * H, de_.get(), E_});
+    products.push_back({1, 0, E_, c.NX * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), ldd, dW, c.NX * H});
+  }
+  struct Run {
+    int asrc, dcol, param, ldb, width;
+    long view, brow, col;
+    long at() const { return view + brow * ldb + col; }
+  };
+  std::vector<Run> runs;
+  for (const CellProduct &p : c.products)
+    for (const CellTerm &t : p.terms) {
+      if (!runs.empty()) {
+        Run &q = runs.back();
+        if (q.asrc == t.asrc && q.param == p.B.param && q.view == p.B.offset && q.ldb == p.ldb && q.brow == t.brow &&
+            q.col + q.width == p.col && q.dcol + q.width / H == p.dcol) {
+          q.width += H;
+          continue;
+        }
+      }
+      runs.push_back({t.asrc, p.dcol, p.B.param, p.ldb, H, p.B.offset, t.brow, p.col});
+    }
+  // a block of weights that several products read collects their gradients one launch after the other
+  std::vector<std::vector<cavs_gemm_desc>> later;
+  if (N > lp)
+    for (size_t i = 0; i < runs.size(); i++) {
+      const Run &q = runs[i];
+      size_t before = 0;
+      for (size_t k = 0; k < i; k++)
+        if (runs[k].param == q.param && runs[k].at() == q.at()) {
+          if (runs[k].width != q.width || runs[k].ldb != q.ldb)
+            fail(CAVS_EUNSUPPORTED, "products of the lowered vertex function read overlapping but different blocks of one weight");
+          before++;
+        }
+      const cavs_gemm_desc d{1, 0, H, q.width, N - lp, 1.f, before ? 1.f : 0.f, hlr_.at((size_t)lp * lda + (size_t)q.asrc * H), lda,
+                             dxW_.at((size_t)lp * ldd + (size_t)q.dcol * H), ldd, param(c.params[q.param].name).g + q.at(), q.ldb};
+      if (!before) {
+        products.push_back(d);
+      } else {
+        if (later.size() < before) later.resize(before);
+        later[before - 1].push_back(d);
+      }
+    }
+  else
+    for (const Run &q : runs)  // a batch of single vertices: nothing was multiplied
+      for (int row = 0; row < H; row++) check(cavs_zero(param(c.params[q.param].name).g + q.at() + (size_t)row * q.ldb, (size_t)q.width * 4, stream_));
+  size_t at = 0;
+  if (c.NX > 0) {
+    const size_t take = std::min<size_t>(products.size(), 4);
+    gemm_group_embedding_backward(std::vector<cavs_gemm_desc>(products.begin(), products.begin() + take), E_);
+    at = take;
+  }
+  for (; at < products.size(); at += 4)
+    gemm_group(std::vector<cavs_gemm_desc>(products.begin() + at, products.begin() + std::min(products.size(), at + 4)));
+  for (const std::vector<cavs_gemm_desc> &wave : later)
+    for (size_t i = 0; i < wave.size(); i += 4)
+      gemm_group(std::vector<cavs_gemm_desc>(wave.begin() + i, wave.begin() + std::min(wave.size(), i + 4)));
+  if (!c.biases.empty()) {
+    colsum_fixed(cell_colsum_.get(), dxW_.get(), N, ldd);
+    ProfScope ps(this, K_OTHER);
+    cell_launch(CK_BIAS, (H + 255) / 256, 1, 1, 256, 0, 0, nullptr, d_dgo_);
   }
 }
 

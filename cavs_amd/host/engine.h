@@ -14,6 +14,7 @@
 #include <vector>
 
 #include "cavs_session.h"
+#include "cell.h"
 #include "device.h"
 #include "scheduler.h"
 
@@ -28,7 +29,8 @@ struct Param {
 class Engine {
  public:
   // external_stream: enqueue on the caller's stream instead of creating one
-  explicit Engine(const cavs_session_config &cfg, void *external_stream = nullptr);
+  // cell: the generated kernels of cfg.model == CAVS_MODEL_CELL
+  explicit Engine(const cavs_session_config &cfg, void *external_stream = nullptr, std::shared_ptr<const CellSpec> cell = nullptr);
   ~Engine();
 
   // Points a parameter and its gradient at device memory owned by the caller (the front
@@ -97,6 +99,10 @@ class Engine {
   void lstm_backward();
   void treefc_forward();
   void treefc_backward();
+  void cell_forward();
+  void cell_backward();
+  void model_forward();
+  void model_backward();
   void pop_ret(float *graph_out);
   void begin_step(const int *graph, int B, int maxlen);
   void head_forward_backward(bool backward);
@@ -349,6 +355,13 @@ class Engine {
   bool aux_pending_ = false;   // work on the side stream that the session's stream has not waited for yet
   DeviceArray<float> ws_aux_;  // its products' split-K workspace
   void aux_join();
+
+  // ---- a vertex function on generated kernels (CAVS_MODEL_CELL)
+  std::shared_ptr<const CellSpec> cell_;
+  void *cell_module_ = nullptr;
+  DeviceArray<float> cell_colsum_;
+  // one launch of kernel `k` of the module; `fill` sets the slots that differ from the step's common ones
+  void cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go);
 
   // counters of the last step
   double c_round_flops_ = 0;

@@ -10,6 +10,7 @@
 #include <string>
 #include <vector>
 
+#include "../midend/cell_gen.h"
 #include "../midend/executor.h"
 #include "../midend/fusion.h"
 #include "../midend/graph.h"
@@ -157,6 +158,23 @@ size_t C_DumpFusedGraph(char *buf, size_t cap) {
   return d.size() + 1;
 }
 
+size_t C_DumpCell(char *buf, size_t cap, int what) {
+  std::string d;
+  if (what == 0) {
+    d = cavs::mid::cell_host_source(cavs::mid::global_graph());
+  } else {
+    std::string why;
+    auto m = cavs::mid::match_cell(cavs::mid::global_graph(), &why);
+    d = m ? m->spec->source : "// not a cell: " + why + "\n";
+  }
+  if (buf && cap) {
+    size_t n = std::min(cap - 1, d.size());
+    std::memcpy(buf, d.data(), n);
+    buf[n] = 0;
+  }
+  return d.size() + 1;
+}
+
 void C_ResetGraph(void) { cavs::mid::reset_global_graph(); }
 
 int C_SetVariable(C_Session *s, const char *name, const float *data, size_t n) {
@@ -169,9 +187,9 @@ long C_ReadTensor(C_Session *s, const char *name, float *out, size_t cap) {
   return r;
 }
 
-int C_SessionUsesFusedPath(C_Session *s) { return s->exec.uses_fused_path() ? 1 : 0; }
+int C_SessionUsesFusedPath(C_Session *s) { return s->exec.fused_path_kind(); }
 int C_SessionGeneratedKernels(C_Session *s) { return s->exec.fused_kernel_count(); }
-void C_SessionAllowFusedPath(C_Session *s, int allow) { s->exec.allow_fused_path(allow != 0); }
+void C_SessionAllowFusedPath(C_Session *s, int allow) { s->exec.set_lowering_mode(allow < 0 ? 0 : allow > 2 ? 2 : allow); }
 void C_SessionSetPairing(C_Session *s, int pairing) { s->exec.set_pairing(pairing); }
 
 }  // extern "C"

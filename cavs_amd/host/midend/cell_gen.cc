@@ -1,0 +1,706 @@
+#include "cell_gen.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <set>
+#include <sstream>
+#include <tuple>
+
+#include "cavs/util/op_def_builder.h"
+
+namespace cavs {
+namespace mid {
+
+namespace {
+
+const char kTemplate[] =
+#include "cell_template.inc"
+    ;
+
+// ---------------------------------------------------------------- the elementwise part as a DAG
+// One node per value of one hidden unit of one vertex.  Nodes are created in evaluation order, so an
+// operand's id is below its user's; equal nodes are shared.
+enum Kind {
+  N_XW, N_HU, N_BIAS, N_CS,        // inputs of the forward part (i0, i1 index them)
+  N_DST, N_DRET, N_ZERO,           // seeds of the backward part, and "no gradient"
+  N_ADD, N_SUB, N_MUL, N_NEG, N_SIGM, N_TANH, N_RELU,
+  N_DSIGM, N_DTANH, N_DRELU        // a = gradient, b = the activation's output
+};
+
+struct ENode {
+  int kind, a, b, i0, i1;
+  float scale;
+};
+
+struct Dag {
+  std::vector<ENode> n;
+  std::map<std::tuple<int, int, int, int, int, uint32_t>, int> memo;
+  int make(int kind, int a = -1, int b = -1, int i0 = 0, int i1 = 0, float scale = 1.f) {
+    uint32_t bits;
+    std::memcpy(&bits, &scale, 4);
+    auto key = std::make_tuple(kind, a, b, i0, i1, bits);
+    auto it = memo.find(key);
+    if (it != memo.end()) return it->second;
+    n.push_back({kind, a, b, i0, i1, scale});
+    return memo[key] = (int)n.size() - 1;
+  }
+};
+
+std::string literal(float v) {
+  char buf[48];
+  std::snprintf(buf, sizeof buf, "%.9g", (double)v);
+  std::string s(buf);
+  if (s.find_first_of(".en") == std::string::npos) s += ".0";
+  return s + "f";
+}
+
+bool alias_op(const std::string &op) { return op == "Mirror" || op == "Reshape" || op == "Flatten" || op == "Expand_dims"; }
+
+struct Fail {
+  std::string why;
+};
+[[noreturn]] void no(const std::string &why) { throw Fail{why}; }
+
+// ---------------------------------------------------------------- reading F
+struct Reader {
+  const Graph &g;
+  const Scope *func;
+  CellSpec spec;
+  Dag dag;
+  std::map<const Edge *, std::vector<int>> val;  // H-wide blocks of a func-scope edge, as nodes
+  std::set<const Edge *> raw_x, emb_x;           // the pulled id; its embedding row
+  std::vector<int> st;                           // the scattered state blocks
+  int ret = -1;
+  std::map<std::string, int> param_of;           // Variable -> index in spec.params
+  std::map<std::string, std::string> roles;
+  std::map<std::string, CellSlot> slots;
+  std::map<std::pair<int, long>, int> bias_of;   // (param, offset) -> index in spec.biases
+  std::map<std::pair<int, int>, int> asrc_of;    // (mask, block) -> index in spec.asrc
+  bool have_xw = false;
+
+  explicit Reader(const Graph &graph) : g(graph), func(graph.func.get()) {}
+
+  int param_index(const Resolved &r, bool embedding) {
+    auto it = param_of.find(r.var);
+    if (it != param_of.end()) return it->second;
+    const Edge *ve = g.main.find(r.var);
+    if (!ve) no("no Variable edge " + r.var);
+    CellParam p;
+    p.name = embedding ? "Emb" : "P" + std::to_string(spec.params.size());
+    p.size = ve->width();
+    spec.params.push_back(p);
+    if ((int)spec.params.size() > CA_MAX_PARAMS) no("more than " + std::to_string(CA_MAX_PARAMS) + " Variables");
+    return param_of[r.var] = (int)spec.params.size() - 1;
+  }
+
+  // an operand that comes from the main scope: a view of a Variable, registered as a role
+  CellParamRef external(const Edge *e, long *count, bool embedding = false) {
+    Resolved r = resolve_external(e);
+    if (!r.ok) no("external input " + e->name + " is not a view of a Variable");
+    CellParamRef ref;
+    ref.param = param_index(r, embedding);
+    ref.offset = r.offset;
+    *count = r.count;
+    // the edge F consumes directly (the one the backward function returns a gradient for)
+    const Edge *direct = e;
+    while (direct->scope == func && direct->src && alias_op(direct->src->def.name())) direct = direct->src->in[0];
+    if (direct->scope == func) no("external input " + e->name + " is reshaped inside F in a way that is not a plain alias");
+    const std::string key = r.var + "@" + std::to_string(r.offset) + "+" + std::to_string(r.count);
+    auto it = roles.find(key);
+    if (it != roles.end() && it->second != direct->name) no("two main-scope edges view the same part of " + r.var);
+    roles[key] = direct->name;
+    slots[key] = {spec.params[ref.param].name, r.offset, r.count};
+    return ref;
+  }
+
+  bool is_external(const Edge *e) const {
+    while (e->scope == func && e->src && alias_op(e->src->def.name())) e = e->src->in[0];
+    return e->scope != func;
+  }
+
+  const std::vector<int> &blocks(const Edge *e) {
+    auto it = val.find(e);
+    if (it != val.end()) return it->second;
+    if (!is_external(e)) no("operand " + e->name + " is not made of H-wide blocks");
+    long count;
+    CellParamRef ref = external(e, &count);
+    const int H = spec.H;
+    if (count % H) no("external operand " + e->name + " is not a multiple of H wide");
+    std::vector<int> b;
+    for (long i = 0; i < count / H; i++) {
+      auto key = std::make_pair(ref.param, ref.offset + i * H);
+      if (!bias_of.count(key)) {
+        bias_of[key] = (int)spec.biases.size();
+        CellBias cb;
+        cb.ref.param = ref.param;
+        cb.ref.offset = ref.offset + i * H;
+        spec.biases.push_back(cb);
+      }
+      b.push_back(dag.make(N_BIAS, -1, -1, bias_of[key]));
+    }
+    return val[e] = b;
+  }
+
+  // the sum of state blocks of children that a product's left operand block is
+  int a_source(int node) {
+    int mask = 0, block = -1;
+    std::vector<int> todo{node};
+    while (!todo.empty()) {
+      const ENode &q = dag.n[todo.back()];
+      todo.pop_back();
+      if (q.kind == N_ADD) {
+        todo.push_back(q.a);
+        todo.push_back(q.b);
+      } else if (q.kind == N_CS) {
+        if (block >= 0 && block != q.i1) no("a product's left operand adds different state blocks");
+        if (mask & (1 << q.i0)) no("a product's left operand adds a child twice");
+        block = q.i1;
+        mask |= 1 << q.i0;
+      } else {
+        no("a product's left operand is not a sum of children's state blocks");
+      }
+    }
+    auto key = std::make_pair(mask, block);
+    if (!asrc_of.count(key)) {
+      asrc_of[key] = (int)spec.asrc.size();
+      spec.asrc.push_back({mask, block});
+    }
+    return asrc_of[key];
+  }
+
+  void read() {
+    if (!func) no("no vertex function");
+    CellSpec &s = spec;
+    for (auto &n : func->nodes)
+      if (n->def.name() == "Push") s.H = (int)n->in[0]->width();
+    if (s.H <= 0 || s.H % 32) no("the pushed value's width is not a multiple of 32");
+    const int H = s.H;
+    for (auto &np : func->nodes) {
+      const Node *n = np.get();
+      const OpDef &d = n->def;
+      const std::string &op = d.name();
+      const Edge *out = n->out.empty() ? nullptr : n->out[0];
+      if (op == "Gather") {
+        const int k = GetSingleArg<int>(d, "Child", 0);
+        const long w = out->width();
+        if (k < 0 || k > 1 || w % H) no("Gather of child " + std::to_string(k) + " with width " + std::to_string(w));
+        if (s.S && s.S != w / H) no("Gather widths differ");
+        s.S = (int)(w / H);
+        s.K = std::max(s.K, k + 1);
+        std::vector<int> b;
+        for (int m = 0; m < s.S; m++) b.push_back(dag.make(N_CS, -1, -1, k, m));
+        val[out] = b;
+      } else if (op == "Pull") {
+        if (out->width() != 1) no("Pull of a vertex input wider than one id");
+        raw_x.insert(out);
+      } else if (op == "EmbeddingLookup") {
+        if (!raw_x.count(n->in[0])) no("EmbeddingLookup of something other than the pulled id");
+        long count;
+        Resolved r = resolve_external(n->in[1]);
+        const Edge *table = n->in[1];
+        if (!r.ok || r.offset != 0 || table->shape.size() != 2) no("the embedding table is not a whole 2-D Variable");
+        external(table, &count, true);
+        s.V = table->shape[0];
+        s.E = table->shape[1];
+        emb_x.insert(out);
+      } else if (alias_op(op)) {
+        const Edge *in = n->in[0];
+        if (raw_x.count(in)) raw_x.insert(out);
+        else if (emb_x.count(in)) emb_x.insert(out);
+        else if (val.count(in)) val[out] = val[in];
+        // (an alias of an external edge is resolved where it is used)
+      } else if (op == "MatMul") {
+        const Edge *A = n->in[0], *B = n->in[1];
+        if (!is_external(B) || B->shape.size() != 2) no("MatMul whose right operand is not a 2-D view of a Variable");
+        const long rows = B->shape[0], cols = B->shape[1];
+        if (cols % H) no("MatMul output width is not a multiple of H");
+        long count;
+        CellParamRef ref = external(B, &count);
+        if (count != rows * cols) no("MatMul right operand view has the wrong size");
+        std::vector<int> b;
+        if (emb_x.count(A)) {
+          if (have_xw) no("more than one product with the vertex input");
+          if (rows != s.E) no("x * W: W has " + std::to_string(rows) + " rows, the embedding " + std::to_string(s.E));
+          have_xw = true;
+          s.W = ref;
+          s.NX = (int)(cols / H);
+          for (int i = 0; i < s.NX; i++) b.push_back(dag.make(N_XW, -1, -1, i));
+        } else {
+          const std::vector<int> &ab = blocks(A);
+          if ((long)ab.size() * H != rows) no("MatMul operand widths do not agree");
+          std::vector<int> src;
+          for (int node : ab) src.push_back(a_source(node));
+          for (long o = 0; o < cols / H; o++) {
+            CellProduct p;
+            for (size_t a = 0; a < src.size(); a++) p.terms.push_back({src[a], (long)a * H});
+            p.B = ref;
+            p.ldb = (int)cols;
+            p.col = o * H;
+            s.products.push_back(p);
+            b.push_back(dag.make(N_HU, -1, -1, (int)s.products.size() - 1));
+          }
+        }
+        val[out] = b;
+      } else if (op == "Slice") {
+        const std::vector<int> &in = blocks(n->in[0]);
+        const long w = (long)in.size() * H;
+        const long stride = d.find_attr("Split") ? w / GetSingleArg<int>(d, "Split") : GetSingleArg<int>(d, "Stride");
+        const long off = d.find_attr("Split") ? stride * GetSingleArg<int>(d, "Index") : GetSingleArg<int>(d, "Offset");
+        if (off % H || stride % H || off + stride > w) no("Slice that does not cut at multiples of H");
+        val[out] = std::vector<int>(in.begin() + off / H, in.begin() + (off + stride) / H);
+      } else if (op == "Concat") {
+        std::vector<int> b;
+        for (const Edge *e : n->in) {
+          const std::vector<int> &in = blocks(e);
+          b.insert(b.end(), in.begin(), in.end());
+        }
+        val[out] = b;
+      } else if (op == "Add" || op == "Sub" || op == "Mul") {
+        const std::vector<int> x = blocks(n->in[0]), y = blocks(n->in[1]);
+        if (x.size() != y.size()) no(op + " of operands of different widths");
+        const int kind = op == "Add" ? N_ADD : op == "Sub" ? N_SUB : N_MUL;
+        const float scale = op == "Mul" ? GetSingleArg<float>(d, "Scale", 1.f) : 1.f;
+        std::vector<int> b;
+        for (size_t i = 0; i < x.size(); i++) b.push_back(dag.make(kind, x[i], y[i], 0, 0, scale));
+        val[out] = b;
+      } else if (op == "Sigmoid" || op == "Tanh" || op == "Relu" || op == "Neg") {
+        const std::vector<int> x = blocks(n->in[0]);
+        const int kind = op == "Sigmoid" ? N_SIGM : op == "Tanh" ? N_TANH : op == "Relu" ? N_RELU : N_NEG;
+        std::vector<int> b;
+        for (int v : x) b.push_back(dag.make(kind, v));
+        val[out] = b;
+      } else if (op == "Scatter") {
+        st = blocks(n->in[0]);
+        if ((int)st.size() != s.S && s.S) no("the scattered message is not as wide as the gathered ones");
+        if (!s.S) s.S = (int)st.size();
+      } else if (op == "Push") {
+        const std::vector<int> &b = blocks(n->in[0]);
+        if (b.size() != 1) no("the pushed value is not H wide");
+        ret = b[0];
+      } else {
+        no("operator " + op + " inside F");
+      }
+    }
+    if (st.empty() || ret < 0) no("F has no Scatter or no Push");
+    if (s.K < 1) no("F gathers no child");
+    if (!raw_x.empty() && !have_xw) no("the vertex input is pulled but not multiplied");
+    if (s.products.empty()) no("F multiplies no child state");
+    if (s.products.size() > 16 || s.asrc.size() > 8 || s.NX > 16 || s.biases.size() > 32) no("too many products or operands");
+  }
+};
+
+// ---------------------------------------------------------------- the backward part
+struct Derived {
+  std::vector<int> dcols;                 // node of every block of a vertex's gradient row
+  std::vector<std::vector<int>> dcs;      // [k][m]: node of the elementwise gradient into child k's block m, or -1
+  std::vector<int> saved;                 // forward nodes the backward part reads, in sv order
+  bool reads_cs = false;
+  int ds_mask = 0;
+};
+
+Derived derive(Reader &r) {
+  Dag &dag = r.dag;
+  CellSpec &s = r.spec;
+  const int nfwd = (int)dag.n.size();
+  std::vector<std::vector<int>> adj(nfwd);
+  for (int m = 0; m < s.S; m++) adj[r.st[m]].push_back(dag.make(N_DST, -1, -1, m));
+  adj[r.ret].push_back(dag.make(N_DRET));
+  std::vector<int> grad(nfwd, -1);
+  for (int id = nfwd - 1; id >= 0; id--) {
+    if (adj[id].empty()) continue;
+    int gsum = adj[id][0];
+    for (size_t i = 1; i < adj[id].size(); i++) gsum = dag.make(N_ADD, gsum, adj[id][i]);
+    grad[id] = gsum;
+    const ENode q = dag.n[id];
+    switch (q.kind) {
+      case N_ADD: adj[q.a].push_back(gsum); adj[q.b].push_back(gsum); break;
+      case N_SUB: adj[q.a].push_back(gsum); adj[q.b].push_back(dag.make(N_NEG, gsum)); break;
+      case N_MUL:
+        adj[q.a].push_back(dag.make(N_MUL, gsum, q.b, 0, 0, q.scale));
+        adj[q.b].push_back(dag.make(N_MUL, gsum, q.a, 0, 0, q.scale));
+        break;
+      case N_NEG: adj[q.a].push_back(dag.make(N_NEG, gsum)); break;
+      case N_SIGM: adj[q.a].push_back(dag.make(N_DSIGM, gsum, id)); break;
+      case N_TANH: adj[q.a].push_back(dag.make(N_DTANH, gsum, id)); break;
+      case N_RELU: adj[q.a].push_back(dag.make(N_DRELU, gsum, id)); break;
+      default: break;  // inputs
+    }
+  }
+  Derived d;
+  const int zero = dag.make(N_ZERO);
+  auto input_grad = [&](int kind, int i0, int i1) {
+    for (int id = 0; id < nfwd; id++)
+      if (dag.n[id].kind == kind && dag.n[id].i0 == i0 && dag.n[id].i1 == i1) return grad[id];
+    return -1;
+  };
+  auto column_of = [&](int node) {
+    if (node < 0) node = zero;
+    return node;
+  };
+  // the blocks of d(x * W) first and in order: the weight gradient of W is one product over them
+  for (int i = 0; i < s.NX; i++) d.dcols.push_back(column_of(input_grad(N_XW, i, 0)));
+  auto shared_column = [&](int node) {
+    node = column_of(node);
+    for (size_t q = 0; q < d.dcols.size(); q++)
+      if (d.dcols[q] == node) return (int)q;
+    d.dcols.push_back(node);
+    return (int)d.dcols.size() - 1;
+  };
+  for (size_t p = 0; p < s.products.size(); p++) s.products[p].dcol = shared_column(input_grad(N_HU, (int)p, 0));
+  for (size_t i = 0; i < s.biases.size(); i++) s.biases[i].dcol = shared_column(input_grad(N_BIAS, (int)i, 0));
+  s.ND = (int)d.dcols.size();
+  d.dcs.assign(s.K, std::vector<int>(s.S, -1));
+  for (int k = 0; k < s.K; k++)
+    for (int m = 0; m < s.S; m++) {
+      d.dcs[k][m] = input_grad(N_CS, k, m);
+      if (d.dcs[k][m] >= 0) d.ds_mask |= 1 << m;
+    }
+  // forward values the backward part reads: children's states come from the pool, the rest is saved
+  std::set<int> seen;
+  std::vector<int> todo = d.dcols;
+  for (auto &row : d.dcs)
+    for (int v : row)
+      if (v >= 0) todo.push_back(v);
+  std::set<int> saved;
+  while (!todo.empty()) {
+    const int id = todo.back();
+    todo.pop_back();
+    if (!seen.insert(id).second) continue;
+    const ENode &q = dag.n[id];
+    if (id < nfwd) {
+      if (q.kind == N_CS) d.reads_cs = true;
+      else saved.insert(id);
+      continue;
+    }
+    if (q.a >= 0) todo.push_back(q.a);
+    if (q.b >= 0) todo.push_back(q.b);
+  }
+  d.saved.assign(saved.begin(), saved.end());
+  s.NSV = (int)d.saved.size();
+  return d;
+}
+
+// ---------------------------------------------------------------- writing the source
+struct Writer {
+  const Reader &r;
+  const Derived &dv;
+  const Dag &dag;
+  const CellSpec &s;
+  bool device;
+  std::ostringstream o;
+
+  Writer(const Reader &rd, const Derived &d, bool dev) : r(rd), dv(d), dag(rd.dag), s(rd.spec), device(dev) {}
+
+  std::string name(int id, bool backward, int nfwd) const {
+    const ENode &q = dag.n[id];
+    switch (q.kind) {
+      case N_XW: if (!backward) return "in.xw[" + std::to_string(q.i0) + "]"; break;
+      case N_HU: if (!backward) return "in.hu[" + std::to_string(q.i0) + "]"; break;
+      case N_BIAS: if (!backward) return "in.bias[" + std::to_string(q.i0) + "]"; break;
+      case N_CS: return "in.cs[" + std::to_string(q.i0) + "][" + std::to_string(q.i1) + "]";
+      case N_DST: return "in.dst[" + std::to_string(q.i0) + "]";
+      case N_DRET: return "in.dret";
+      case N_ZERO: return "0.f";
+      default: break;
+    }
+    if (backward && id < nfwd) {
+      auto it = std::find(dv.saved.begin(), dv.saved.end(), id);
+      return "in.sv[" + std::to_string(it - dv.saved.begin()) + "]";
+    }
+    return "v" + std::to_string(id);
+  }
+
+  std::string expr(int id, bool backward, int nfwd) const {
+    const ENode &q = dag.n[id];
+    auto A = [&] { return name(q.a, backward, nfwd); };
+    auto B = [&] { return name(q.b, backward, nfwd); };
+    switch (q.kind) {
+      case N_ADD: return A() + " + " + B();
+      case N_SUB: return A() + " - " + B();
+      case N_MUL: return A() + " * " + B() + (q.scale != 1.f ? " * " + literal(q.scale) : "");
+      case N_NEG: return "-" + A();
+      case N_SIGM: return "cell_sigm(" + A() + ")";
+      case N_TANH: return "cell_tanh(" + A() + ")";
+      case N_RELU: return "(" + A() + " > 0.f ? " + A() + " : 0.f)";
+      case N_DSIGM: return A() + " * (" + B() + " * (1.f - " + B() + "))";
+      case N_DTANH: return A() + " * (1.f - " + B() + " * " + B() + ")";
+      case N_DRELU: return "(" + B() + " > 0.f ? " + A() + " : 0.f)";
+      default: return name(id, backward, nfwd);
+    }
+  }
+
+  static bool computed(int kind) { return kind >= N_ADD; }
+
+  // statements for the nodes `roots` depend on, in evaluation order
+  void body(const std::vector<int> &roots, bool backward, int nfwd) {
+    std::set<int> need;
+    std::vector<int> todo = roots;
+    while (!todo.empty()) {
+      const int id = todo.back();
+      todo.pop_back();
+      if (id < 0 || !need.insert(id).second) continue;
+      if (backward && id < nfwd) continue;
+      const ENode &q = dag.n[id];
+      if (q.a >= 0) todo.push_back(q.a);
+      if (q.b >= 0) todo.push_back(q.b);
+    }
+    for (int id : need) {
+      if (backward && id < nfwd) continue;
+      if (!computed(dag.n[id].kind)) continue;
+      o << "  const float v" << id << " = " << expr(id, backward, nfwd) << ";\n";
+    }
+  }
+
+  void elementwise(int nfwd) {
+    const char *dev = device ? "static __device__ inline " : "static inline ";
+    o << "struct FwdIn { float xw[" << std::max(1, s.NX) << "], hu[" << s.products.size() << "], bias[" << std::max<size_t>(1, s.biases.size())
+      << "], cs[" << s.K << "][" << s.S << "]; };\n";
+    o << "struct FwdOut { float st[" << s.S << "], ret, sv[" << std::max(1, s.NSV) << "]; };\n";
+    o << "struct BwdIn { float dst[" << s.S << "], dret, sv[" << std::max(1, s.NSV) << "], cs[" << s.K << "][" << s.S << "]; };\n";
+    o << "struct BwdOut { float d[" << s.ND << "], dcs[" << s.K << "][" << s.S << "]; };\n";
+    if (device) {
+      // exp through v_exp_f32 and the reciprocal through v_rcp_f32 (1 ulp each); saturation comes out
+      // right without special cases
+      o << "static __device__ inline float cell_exp(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }\n"
+           "static __device__ inline float cell_sigm(float x) { return __builtin_amdgcn_rcpf(1.f + cell_exp(-x)); }\n"
+           "static __device__ inline float cell_tanh(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + cell_exp(2.f * x)); }\n";
+    } else {
+      o << "static inline float cell_sigm(float x) { return 1.f / (1.f + expf(-x)); }\n"
+           "static inline float cell_tanh(float x) { return tanhf(x); }\n";
+    }
+    o << dev << "void cell_forward(const FwdIn &in, FwdOut &out) {\n";
+    std::vector<int> roots = r.st;
+    roots.push_back(r.ret);
+    roots.insert(roots.end(), dv.saved.begin(), dv.saved.end());
+    body(roots, false, nfwd);
+    for (int m = 0; m < s.S; m++) o << "  out.st[" << m << "] = " << name(r.st[m], false, nfwd) << ";\n";
+    o << "  out.ret = " << name(r.ret, false, nfwd) << ";\n";
+    for (size_t t = 0; t < dv.saved.size(); t++) o << "  out.sv[" << t << "] = " << name(dv.saved[t], false, nfwd) << ";\n";
+    o << "}\n";
+    o << dev << "void cell_backward(const BwdIn &in, BwdOut &out) {\n";
+    roots = dv.dcols;
+    for (auto &row : dv.dcs)
+      for (int v : row)
+        if (v >= 0) roots.push_back(v);
+    body(roots, true, nfwd);
+    for (size_t q = 0; q < dv.dcols.size(); q++) o << "  out.d[" << q << "] = " << name(dv.dcols[q], true, nfwd) << ";\n";
+    for (int k = 0; k < s.K; k++)
+      for (int m = 0; m < s.S; m++)
+        o << "  out.dcs[" << k << "][" << m << "] = " << (dv.dcs[k][m] >= 0 ? name(dv.dcs[k][m], true, nfwd) : std::string("0.f")) << ";\n";
+    o << "}\n";
+  }
+
+  std::string param_ptr(const CellParamRef &ref, bool grad = false) const {
+    return "(a.p[" + std::to_string(ref.param + (grad ? CA_MAX_PARAMS : 0)) + "] + " + std::to_string(ref.offset) + "L)";
+  }
+
+  void kernels() {
+    const int H = s.H, NT = s.terms(), NP = (int)s.products.size(), NA = (int)s.asrc.size();
+    o << "#define CELL_H " << H << "\n#define CELL_K " << s.K << "\n#define CELL_S " << s.S << "\n#define CELL_MW " << s.S * H
+      << "\n#define CELL_NX " << s.NX << "\n#define CELL_NP " << NP << "\n#define CELL_NA " << NA << "\n#define CELL_NT " << NT
+      << "\n#define CELL_ND " << s.ND << "\n#define CELL_NSV " << s.NSV << "\n#define CELL_KS " << s.waves << "\n#define CELL_DS_MASK "
+      << dv.ds_mask << "\n#define CELL_BWD_CS " << (dv.reads_cs ? 1 : 0) << "\n";
+    o << "typedef float f4 __attribute__((ext_vector_type(4)));\n";
+    o << "struct CellArgs {\n  float *pool;\n  const int *child, *pair, *kids, *t2j, *rows;\n  const float *xw;\n"
+         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum;\n  long off, n;\n  float *p["
+      << 2 * CA_MAX_PARAMS << "];\n};\n";
+    o << "static __device__ inline f4 ld4(const float *p) { return *reinterpret_cast<const f4 *>(p); }\n";
+  }
+
+  void product_loops() {
+    const int H = s.H, NT = s.terms(), NP = (int)s.products.size(), NA = (int)s.asrc.size();
+    // biases and the saved left operands
+    o << "static __device__ inline void cell_load_bias(const CellArgs &a, int j, FwdIn &in) {\n";
+    for (size_t i = 0; i < s.biases.size(); i++) o << "  in.bias[" << i << "] = " << param_ptr(s.biases[i].ref) << "[j];\n";
+    o << "}\n";
+    o << "static __device__ inline void cell_store_asrc(float *dst, const FwdIn &in) {\n";
+    for (int q = 0; q < NA; q++) {
+      o << "  dst[" << (long)q * H << "] = ";
+      bool first = true;
+      for (int k = 0; k < s.K; k++)
+        if (s.asrc[q].mask >> k & 1) {
+          o << (first ? "" : " + ") << "in.cs[" << k << "][" << s.asrc[q].block << "]";
+          first = false;
+        }
+      o << ";\n";
+    }
+    o << "}\n";
+    o << "static __device__ inline void cell_add_products(float (&dst)[CELL_S], const float (&s)[CELL_NA], int k) {\n";
+    for (int k = 0; k < s.K; k++) {
+      o << "  if (k == " << k << ") {\n";
+      for (int q = 0; q < NA; q++)
+        if (s.asrc[q].mask >> k & 1) o << "    dst[" << s.asrc[q].block << "] += s[" << q << "];\n";
+      o << "  }\n";
+    }
+    o << "}\n";
+    // forward: B pointers, fragments, MFMAs
+    o << "static __device__ inline void cell_bptrs(const CellArgs &a, int slot, int jx, const float *(&bp)[CELL_NT]) {\n";
+    int t = 0;
+    std::vector<int> term_ld;
+    for (const CellProduct &p : s.products)
+      for (const CellTerm &tm : p.terms) {
+        o << "  bp[" << t << "] = " << param_ptr(p.B) << " + (long)(" << tm.brow << " + 4 * slot) * " << p.ldb << " + " << p.col << " + jx;\n";
+        term_ld.push_back(p.ldb);
+        t++;
+      }
+    o << "}\n";
+    o << "static __device__ inline const float *cell_term_block(const CellArgs &a, int t) {\n  switch (t) {\n";
+    t = 0;
+    for (const CellProduct &p : s.products)
+      for (const CellTerm &tm : p.terms) {
+        o << "    case " << t << ": return " << param_ptr(p.B) << " + " << tm.brow * p.ldb + p.col << "L;\n";
+        t++;
+      }
+    o << "  }\n  return nullptr;\n}\n";
+    o << "static __device__ inline int cell_term_ld(int t) {\n  switch (t) {\n";
+    for (int q = 0; q < NT; q++) o << "    case " << q << ": return " << term_ld[q] << ";\n";
+    o << "  }\n  return 0;\n}\n";
+    // which (child, block) rows the left operands read
+    std::set<std::pair<int, int>> raw;
+    for (const CellASrc &a : s.asrc)
+      for (int k = 0; k < s.K; k++)
+        if (a.mask >> k & 1) raw.insert({k, a.block});
+    o << "struct FFrag { f4 a[" << NA << "]; float b[" << NT << "][4]; };\n";
+    o << "static __device__ inline void cell_ffetch(FFrag &f, const float *const (&crow)[CELL_K], const bool (&has)[CELL_K], "
+         "const float *const (&bp)[CELL_NT], int kk) {\n  const f4 z = {0.f, 0.f, 0.f, 0.f};\n";
+    for (auto &kb : raw)
+      o << "  const f4 r" << kb.first << "_" << kb.second << " = has[" << kb.first << "] ? ld4(crow[" << kb.first << "] + "
+        << (long)kb.second * H << " + kk) : z;\n";
+    for (int q = 0; q < NA; q++) {
+      std::string e;
+      for (int k = 0; k < s.K; k++)
+        if (s.asrc[q].mask >> k & 1) {
+          const std::string v = "r" + std::to_string(k) + "_" + std::to_string(s.asrc[q].block);
+          e = e.empty() ? v : e + " + " + v;
+        }
+      o << "  f.a[" << q << "] = " << e << ";\n";
+    }
+    o << "#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
+    for (int q = 0; q < NT; q++) o << "    f.b[" << q << "][c] = bp[" << q << "][(long)(kk + c) * " << term_ld[q] << "];\n";
+    o << "  }\n}\n";
+    o << "static __device__ inline void cell_fmma(const FFrag &f, f4 (&acc)[CELL_NP]) {\n#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
+    t = 0;
+    for (int p = 0; p < NP; p++)
+      for (const CellTerm &tm : s.products[p].terms) {
+        o << "    acc[" << p << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << tm.asrc << "][c], f.b[" << t << "][c], acc[" << p
+          << "], 0, 0, 0);\n";
+        t++;
+      }
+    o << "  }\n}\n";
+    // backward: the left operands are blocks of the rows' own gradient rows
+    std::vector<int> dcols;
+    for (const CellProduct &p : s.products)
+      if (std::find(dcols.begin(), dcols.end(), p.dcol) == dcols.end()) dcols.push_back(p.dcol);
+    o << "struct BFrag { f4 a[" << dcols.size() << "]; float b[" << NT << "][4]; };\n";
+    o << "static __device__ inline void cell_bfetch(BFrag &f, const float *drow, const float *bt, int kk) {\n";
+    for (size_t q = 0; q < dcols.size(); q++) o << "  f.a[" << q << "] = ld4(drow + " << (long)dcols[q] * H << " + kk);\n";
+    o << "#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
+    for (int q = 0; q < NT; q++) o << "    f.b[" << q << "][c] = bt[" << (long)q * H * H << "L + (long)(kk + c) * " << H << "];\n";
+    o << "  }\n}\n";
+    o << "static __device__ inline void cell_bmma(const BFrag &f, f4 (&acc)[CELL_NA]) {\n#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
+    t = 0;
+    for (int p = 0; p < NP; p++) {
+      const int ai = (int)(std::find(dcols.begin(), dcols.end(), s.products[p].dcol) - dcols.begin());
+      for (const CellTerm &tm : s.products[p].terms) {
+        o << "    acc[" << tm.asrc << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << ai << "][c], f.b[" << t << "][c], acc[" << tm.asrc
+          << "], 0, 0, 0);\n";
+        t++;
+      }
+    }
+    o << "  }\n}\n";
+    // the bias gradients out of the column sums of the gradient rows
+    o << "extern \"C\" __global__ void cell_bias(CellArgs a) {\n  const int j = blockIdx.x * 256 + threadIdx.x;\n  if (j >= CELL_H) return;\n";
+    for (const CellBias &b : s.biases) o << "  " << param_ptr(b.ref, true) << "[j] = a.colsum[" << (long)b.dcol * H << " + j];\n";
+    o << "}\n";
+  }
+};
+
+struct Built {
+  Reader reader;
+  Derived derived;
+  int nfwd;
+  explicit Built(const Graph &g) : reader(g) {
+    reader.read();
+    nfwd = (int)reader.dag.n.size();
+    derived = derive(reader);
+  }
+};
+
+}  // namespace
+
+Resolved resolve_external(const Edge *e) {
+  Resolved r;
+  r.count = e->width();
+  long off = 0;
+  const Edge *cur = e;
+  while (cur && cur->src) {
+    const OpDef &d = cur->src->def;
+    const std::string &op = d.name();
+    if (op == "Variable") {
+      r.var = cur->name;
+      r.offset = off;
+      r.ok = true;
+      return r;
+    }
+    if (op == "Mirror" || op == "Reshape" || op == "Flatten" || op == "Expand_dims") {
+      cur = cur->src->in[0];
+    } else if (op == "Slice") {
+      const Edge *in = cur->src->in[0];
+      long stride = d.find_attr("Split") ? in->width() / GetSingleArg<int>(d, "Split") : GetSingleArg<int>(d, "Stride");
+      off += d.find_attr("Split") ? stride * GetSingleArg<int>(d, "Index") : GetSingleArg<int>(d, "Offset");
+      cur = in;
+    } else {
+      return r;
+    }
+  }
+  return r;
+}
+
+std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
+  try {
+    Built b(g);
+    CellSpec &s = b.reader.spec;
+    const int H = s.H;
+    s.waves = H % 128 == 0 ? 4 : H % 64 == 0 ? 2 : 1;
+    // the partial tiles of a workgroup must fit in LDS
+    const size_t lds = (size_t)s.waves * std::max(s.products.size(), s.asrc.size()) * 1024;
+    if (lds > 60 * 1024) no("too many accumulators for one workgroup");
+    Writer w(b.reader, b.derived, true);
+    w.kernels();
+    w.elementwise(b.nfwd);
+    w.product_loops();
+    w.o << kTemplate;
+    s.source = w.o.str();
+    // what decides the kernels, for sharing compiled modules between sessions
+    s.key = s.source;
+    auto m = std::make_unique<CellMatch>();
+    m->spec = std::make_shared<CellSpec>(s);
+    m->roles = b.reader.roles;
+    m->slots = b.reader.slots;
+    return m;
+  } catch (const Fail &f) {
+    if (why) *why = f.why;
+    return nullptr;
+  }
+}
+
+std::string cell_host_source(const Graph &g) {
+  try {
+    Built b(g);
+    Writer w(b.reader, b.derived, false);
+    w.o << "#include <math.h>\n";
+    w.elementwise(b.nfwd);
+    const CellSpec &s = b.reader.spec;
+    w.o << "// H=" << s.H << " K=" << s.K << " S=" << s.S << " NX=" << s.NX << " NP=" << s.products.size() << " NB=" << s.biases.size()
+        << " ND=" << s.ND << " NSV=" << s.NSV << "\n";
+    for (size_t p = 0; p < s.products.size(); p++) w.o << "// product " << p << " dcol " << s.products[p].dcol << "\n";
+    for (size_t i = 0; i < s.biases.size(); i++) w.o << "// bias " << i << " dcol " << s.biases[i].dcol << "\n";
+    return w.o.str();
+  } catch (const Fail &f) {
+    return "// not a cell: " + f.why + "\n";
+  }
+}
+
+}  // namespace mid
+}  // namespace cavs

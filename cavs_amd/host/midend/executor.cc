@@ -143,6 +143,10 @@ void Executor::compile() {
   pool_w_ = ret_w_ = arg_w_ = 0;
   lowered_ = false;
   lowering_.reset();
+  if (engine_) {  // (made for the program as it was)
+    check(cavs_stream_sync(stream_));
+    engine_.reset();
+  }
   if (g.func) {
     for (auto &n : g.func->nodes) {
       const std::string &op = n->def.name();
@@ -163,8 +167,8 @@ void Executor::compile() {
         arg_w_ = n->out[0]->width();
       }
     }
-    if (allow_fused_ && (opt_ & OPT_BATCHING)) {
-      lowering_ = match_vertex_function(g);
+    if (lowering_mode_ > 0 && (opt_ & OPT_BATCHING)) {
+      lowering_ = match_vertex_function(g, lowering_mode_);
       lowered_ = lowering_ != nullptr;
     }
   }

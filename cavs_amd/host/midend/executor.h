@@ -56,7 +56,8 @@ class Executor {
   long read_tensor(const std::string &name, float *out, size_t cap);
   bool uses_fused_path() const { return lowered_; }
   int fused_kernel_count() const { return fused_groups_; }
-  void allow_fused_path(bool a) { allow_fused_ = a; compiled_version_ = -1; }
+  int fused_path_kind() const;  // 0: F runs op by op; 1: hand-written round kernels; 2: generated ones
+  void set_lowering_mode(int m) { lowering_mode_ = m; compiled_version_ = -1; }
   void set_pairing(int p) { pairing_ = p; compiled_version_ = -1; }
 
  private:
@@ -87,7 +88,8 @@ class Executor {
   std::string name_;
   void *stream_ = nullptr;
   int compiled_version_ = -1;
-  bool allow_fused_ = true, lowered_ = false;
+  int lowering_mode_ = 1;  // 0: never lower F; 1: hand-written kernels, else generated ones; 2: generated ones only
+  bool lowered_ = false;
   int pairing_ = 0;
   std::map<std::string, std::unique_ptr<Tensor>> tensors_;
   std::map<std::string, FeedStage> feed_stages_;

@@ -3,51 +3,18 @@
 #include <algorithm>
 
 #include <functional>
+#include <set>
 #include <sstream>
 
 #include "cavs/frontend/cxx/graphsupport.h"
 #include "cavs/frontend/cxx/sym.h"
+#include "cell_gen.h"
 #include "executor.h"
 
 namespace cavs {
 namespace mid {
 
 namespace {
-
-// A main-scope edge traced back through aliasing ops to the Variable it views.
-struct Resolved {
-  std::string var;
-  long offset = 0, count = 0;
-  bool ok = false;
-};
-
-Resolved resolve_external(const Edge *e) {
-  Resolved r;
-  r.count = e->width();
-  long off = 0;
-  const Edge *cur = e;
-  while (cur && cur->src) {
-    const OpDef &d = cur->src->def;
-    const std::string &op = d.name();
-    if (op == "Variable") {
-      r.var = cur->name;
-      r.offset = off;
-      r.ok = true;
-      return r;
-    }
-    if (op == "Mirror" || op == "Reshape" || op == "Flatten" || op == "Expand_dims") {
-      cur = cur->src->in[0];
-    } else if (op == "Slice") {
-      const Edge *in = cur->src->in[0];
-      long stride = d.find_attr("Split") ? in->width() / GetSingleArg<int>(d, "Split") : GetSingleArg<int>(d, "Stride");
-      off += d.find_attr("Split") ? stride * GetSingleArg<int>(d, "Index") : GetSingleArg<int>(d, "Offset");
-      cur = in;
-    } else {
-      return r;
-    }
-  }
-  return r;
-}
 
 // Canonical text of the vertex function: the expressions feeding Scatter and Push, with
 // aliasing ops made transparent, shared sub-expressions numbered in traversal order and
@@ -262,7 +229,32 @@ struct RoleSlot {
 
 }  // namespace
 
-std::unique_ptr<Lowering> match_vertex_function(const Graph &g) {
+namespace {
+std::unique_ptr<Lowering> match_template(const Graph &g);
+}
+
+std::unique_ptr<Lowering> match_vertex_function(const Graph &g, int mode) {
+  if (!g.func) return nullptr;
+  if (mode == 1) {
+    auto lw = match_template(g);
+    if (lw) return lw;
+  }
+  std::unique_ptr<CellMatch> m = match_cell(g);
+  if (!m) return nullptr;
+  auto lw = std::make_unique<Lowering>();
+  lw->model = CAVS_MODEL_CELL;
+  lw->H = m->spec->H;
+  lw->E = m->spec->E;
+  lw->V = m->spec->V;
+  lw->use_x = m->spec->NX > 0;
+  lw->roles = m->roles;
+  lw->cell = m->spec;
+  lw->cell_slots = m->slots;
+  return lw;
+}
+
+namespace {
+std::unique_ptr<Lowering> match_template(const Graph &g) {
   if (!g.func) return nullptr;
   // cheap signature first: graph ops and the embedding table decide which template to try
   int gathers = 0, pulls = 0;
@@ -322,6 +314,8 @@ std::unique_ptr<Lowering> match_vertex_function(const Graph &g) {
   return lw;
 }
 
+}  // namespace
+
 // ------------------------------------------------------------------ running the lowered F
 namespace {
 struct Slot {
@@ -331,6 +325,10 @@ struct Slot {
 std::map<std::string, Slot> role_slots(const Lowering &lw) {
   const long H = lw.H, E = lw.E, V = lw.V;
   std::map<std::string, Slot> m;
+  if (lw.model == CAVS_MODEL_CELL) {
+    for (auto &kv : lw.cell_slots) m[kv.first] = {kv.second.param.c_str(), kv.second.offset, kv.second.count};
+    return m;
+  }
   if (lw.model == CAVS_MODEL_TREELSTM) {
     m["Emb"] = {"Emb", 0, V * E};
     m["W"] = {"W", 0, 4 * E * H};
@@ -354,6 +352,8 @@ std::map<std::string, Slot> role_slots(const Lowering &lw) {
 }
 }  // namespace
 
+int Executor::fused_path_kind() const { return !lowered_ ? 0 : lowering_->model == CAVS_MODEL_CELL ? 2 : 1; }
+
 void Executor::lowered_forward(const int32_t *graph, int B, int maxlen, float *) {
   const Lowering &lw = *lowering_;
   if (!engine_) {
@@ -367,15 +367,16 @@ void Executor::lowered_forward(const int32_t *graph, int B, int maxlen, float *)
     cfg.act = lw.act;
     cfg.use_bias = lw.use_bias;
     cfg.use_x = lw.use_x;
-    engine_ = std::make_unique<Engine>(cfg, stream_);
+    engine_ = std::make_unique<Engine>(cfg, stream_, lw.cell);
   }
   engine_->set_pairing(pairing_);
   // parameters live in the user's Variable tensors; the engine reads them in place
+  std::set<std::string> bound;
   for (auto &kv : role_slots(lw)) {
     const Slot &s = kv.second;
-    if (s.offset != 0) continue;  // the first view of each array carries its base address
+    if (!bound.insert(s.param).second) continue;  // every view of an array leads to its base address
     Tensor &t = tensor(lw.roles.at(kv.first));
-    engine_->bind_param(s.param, t.base, nullptr);
+    engine_->bind_param(s.param, t.base - s.offset, nullptr);
   }
   engine_->forward_only(graph, B, maxlen, func_arg_, nullptr);
   N_ = engine_->total_length();

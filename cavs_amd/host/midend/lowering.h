@@ -1,7 +1,8 @@
-// Recognition of the vertex functions the fused round kernels implement.  A user's F is
-// lowered onto cavs::Engine only when its operator graph is the same computation as one
-// of the templates (binary Tree-LSTM, chain LSTM, Tree-FC): same operators, same
-// wiring, same attributes -- everything else runs op by op.
+// Recognition of the vertex functions the engine runs on fused round kernels.  A user's F is
+// lowered onto cavs::Engine when its operator graph is the same computation as one of the
+// templates with hand-written kernels (binary Tree-LSTM, chain LSTM, Tree-FC: same operators, same
+// wiring, same attributes), or, failing that, when it has the general one-stage shape that
+// generated kernels cover (cell_gen.h) -- everything else runs op by op.
 #ifndef CAVS_HOST_MIDEND_LOWERING_H_
 #define CAVS_HOST_MIDEND_LOWERING_H_
 
@@ -9,6 +10,7 @@
 #include <memory>
 #include <string>
 
+#include "cell_gen.h"
 #include "graph.h"
 
 namespace cavs {
@@ -20,9 +22,13 @@ struct Lowering {
   int act = 0, use_bias = 0, use_x = 0;
   // role -> name of the main-scope edge that supplies it
   std::map<std::string, std::string> roles;
+  // model == CAVS_MODEL_CELL: the generated kernels and where each role lives in their parameters
+  std::shared_ptr<CellSpec> cell;
+  std::map<std::string, CellSlot> cell_slots;
 };
 
-std::unique_ptr<Lowering> match_vertex_function(const Graph &g);
+// mode 1: the hand-written templates first, then the general shape; 2: the general shape only
+std::unique_ptr<Lowering> match_vertex_function(const Graph &g, int mode = 1);
 
 }  // namespace mid
 }  // namespace cavs

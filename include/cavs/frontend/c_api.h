@@ -48,17 +48,23 @@ int C_SetVariable(C_Session *s, const char *name, const float *data, size_t n);
 /* Copies any tensor of the last run to host by edge name ("X" or "X_grad");
  * returns the element count, or the negative needed capacity, or 0 if unknown. */
 long C_ReadTensor(C_Session *s, const char *name, float *out, size_t cap);
-/* 1 if the vertex function was recognised and lowered onto the fused round kernels. */
+/* Whether the vertex function was lowered onto fused round kernels: 0 no (it runs op by op),
+ * 1 onto the hand-written kernels of a recognised function, 2 onto kernels generated for it. */
 int C_SessionUsesFusedPath(C_Session *s);
 /* Number of kernels the OPT_FUSION pass generated for the programs compiled so far. */
 int C_SessionGeneratedKernels(C_Session *s);
-/* 0 forbids that lowering (op-by-op execution of F, for A/B tests); default 1. */
+/* 0 forbids that lowering (op-by-op execution of F, for A/B tests); 1, the default, tries the
+ * hand-written kernels first and generated ones next; 2 goes for generated kernels only. */
 void C_SessionAllowFusedPath(C_Session *s, int allow);
 void C_SessionSetPairing(C_Session *s, int pairing); /* CAVS_PAIR_* of cavs_session.h */
 const char *C_LastError(void);
 /* Text dump of the declared program: forward ops, the vertex function, and the backward
  * programs the autograd pass derived.  Returns the length needed (including the NUL). */
 size_t C_DumpGraph(char *buf, size_t cap);
+/* The kernels generated for the declared vertex function when it has the general one-stage shape
+ * (what = 1), or its elementwise parts alone as host C++ (what = 0); a comment saying why not
+ * otherwise. */
+size_t C_DumpCell(char *buf, size_t cap, int what);
 /* The same programs after the OPT_FUSION pass, with the generated kernel sources. */
 size_t C_DumpFusedGraph(char *buf, size_t cap);
 

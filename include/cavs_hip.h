@@ -595,6 +595,17 @@ int cavs_fused_launch(void *handle, float *const *outs, int nouts, const float *
                       int nins, const int *out_counts, const int *in_counts, int n_elements,
                       void *stream);
 int cavs_fused_release(void *handle);
+/* The round kernels generated for a vertex function of the general one-stage shape (the reference
+ * fuses the elementwise operators of F into generated kernels, cavs/midend/runtime_compiler/
+ * code_generator.cc:104-185, and runs them through cavs/backend/op_impl_fused_kernel.cu:34-64; here
+ * the products of F are inside the generated kernels too).  `source` defines the extern "C" kernels
+ * cell_fwd, cell_leaves, cell_bwd, cell_bwd_rows, cell_transpose and cell_bias, each taking one
+ * struct of 8-byte slots by value; cavs_cell_launch passes `args` as that struct.  kernel: index in
+ * the order of the names above; block: threads per workgroup (a multiple of 64, at most 256). */
+int cavs_cell_compile(const char *source, void **handle);
+int cavs_cell_launch(void *handle, int kernel, unsigned grid_x, unsigned grid_y, unsigned grid_z,
+                     unsigned block, const void *args, size_t args_bytes, void *stream);
+int cavs_cell_release(void *handle);
 
 /* ------------------------------------------------------------------ device schedule
  * The level-wise ready frontier of BatchGraphScheduler::Initialize/ActivateNext

@@ -26,7 +26,10 @@ extern "C" {
 
 typedef struct cavs_session cavs_session;
 
-enum { CAVS_MODEL_TREELSTM = 0, CAVS_MODEL_LSTM = 1, CAVS_MODEL_TREEFC = 2 };
+enum { CAVS_MODEL_TREELSTM = 0, CAVS_MODEL_LSTM = 1, CAVS_MODEL_TREEFC = 2,
+       /* a vertex function lowered onto generated kernels: only the front end's sessions make
+        * one (its description does not fit this struct); cavs_session_create refuses it */
+       CAVS_MODEL_CELL = 3 };
 enum { CAVS_LOSS_SOFTMAX = 0, CAVS_LOSS_ROOT_SQ = 1, CAVS_LOSS_SUM_ABS = 2 };
 /* How the forward Scatter / backward Gather pair list entries with slab rows:
  * REFERENCE = b-th list entry with b-th slab row, exactly what the reference's
