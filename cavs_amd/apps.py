@@ -41,7 +41,7 @@ def libs():
 
 
 class App:
-    """model: treelstm | lstm | treefc | treefc_x.  opt: OPT_* bitmask, or -1 to only
+    """model: treelstm | lstm | treefc | treefc_x | treelstm2 | treegate.  opt: OPT_* bitmask, or -1 to only
     declare the program (no device)."""
 
     def __init__(self, model, *, B, maxlen, H, E=0, V=0, C_=0, opt=session.OPT_BATCHING, lr=0.0, clip=0.0,
@@ -110,7 +110,7 @@ class App:
                             loss.ctypes.data, loss.size, go.ctypes.data, go.size)
         if n < 0:
             raise hip.CavsError(f"cavs_app_step -> {n}")
-        nl = n if self.model in ("treelstm", "lstm") else 1
+        nl = n if not self.model.startswith("treefc") else 1  # (the Tree-FC apps end in one scalar loss)
         return loss[:nl].copy(), go[: n * self.H].reshape(n, self.H).copy()
 
     def grad(self, name, shape, grad=True):

@@ -83,9 +83,11 @@ enum CellArg {
   CA_ASRC,       // float*  [N, NA*H]
   CA_GO,         // float*  [N, H] by vertex id: the pushed value / its gradient
   CA_D,          // float*  [N, ND*H]
-  CA_DS,         // float*  [N, S*H] elementwise part of a vertex's message gradient
+  CA_DS,         // float*  [N, S*H] elementwise part of a vertex's message gradient by slab row; or, for
+                 //         cell_bwd_gates / cell_bwd_pool, [K * n, S*H] by row of the round and child
   CA_BT,         // float*  transposed H x H blocks of the products' terms
   CA_COLSUM,     // float*  [ND*H] column sums of D
+  CA_DPOOL,      // float*  gradient of the message pool [*, S*H] (batches whose message flow is no forest)
   CA_OFF,        // long    first slab row of the round
   CA_N,          // long    rows
   CA_PARAM0,     // float*  parameters, then their gradients, in CellSpec::params order
@@ -94,7 +96,7 @@ enum CellArg {
 };
 
 // kernels of a compiled cell, in the order cavs_cell_compile looks them up
-enum CellKernel { CK_FWD = 0, CK_LEAVES, CK_BWD, CK_BWD_ROWS, CK_TRANSPOSE, CK_BIAS, CK_COUNT };
+enum CellKernel { CK_FWD = 0, CK_LEAVES, CK_BWD, CK_BWD_ROWS, CK_TRANSPOSE, CK_BIAS, CK_BWD_GATES, CK_BWD_POOL, CK_COUNT };
 
 }  // namespace cavs
 #endif

@@ -1681,9 +1681,10 @@ void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned 
   a[CA_ASRC].p = hlr_.get();
   a[CA_GO].p = go;
   a[CA_D].p = dxW_.get();
-  a[CA_DS].p = dc_.get();
+  a[CA_DS].p = forest_ ? dc_.get() : r_dG_.get();
   a[CA_BT].p = UT_.get();
   a[CA_COLSUM].p = cell_colsum_.get();
+  a[CA_DPOOL].p = dpool_.get();
   a[CA_OFF].i = off;
   a[CA_N].i = n;
   for (size_t i = 0; i < c.params.size(); i++) {
@@ -1698,10 +1699,7 @@ void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned 
 void Engine::cell_forward() {
   const CellSpec &c = *cell_;
   const int N = N_, H = cfg_.H;
-  if (!forest_)
-    fail(CAVS_EUNSUPPORTED,
-         "the lowered vertex function needs the batch scheduler and a batch in which every message is read exactly once; "
-         "open the session without the fused path for other batches");
+  if (!sched_->batching) fail(CAVS_EUNSUPPORTED, "the lowered vertex function needs the batch scheduler (OPT_BATCHING)");
   if (c.NX > 0) {
     ProfScope ps(this, K_GEMM);
     check(cavs_embed_pull_sgemm(xW_.get(), c.NX * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E_,
@@ -1746,18 +1744,40 @@ void Engine::cell_backward() {
     ProfScope ps(this, K_OTHER);
     cell_launch(CK_TRANSPOSE, H / 32, H / 32, c.terms(), 256, 0, 0, nullptr, d_dgo_);
   }
-  if (n_orphans_ > 0) {
-    ProfScope ps(this, K_GATES);
-    cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
-  }
-  for (int k : sched_->bwd_rounds) {
-    const Round &r = sched_->rounds[k];
-    c_gather_rows_ += r.n;
-    if (leaf_round(r)) continue;
-    ProfScope ps(this, K_ROUND);
-    cell_launch(CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
-    c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
-    c_scatter_rows_ += (double)c.K * r.n;
+  if (forest_) {
+    // every message is read exactly once: a round's launch hands d(state) on to the children of its
+    // rows and runs their elementwise part at once; the vertices without a reader go first
+    if (n_orphans_ > 0) {
+      ProfScope ps(this, K_GATES);
+      cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
+    }
+    for (int k : sched_->bwd_rounds) {
+      const Round &r = sched_->rounds[k];
+      c_gather_rows_ += r.n;
+      if (leaf_round(r)) continue;
+      ProfScope ps(this, K_ROUND);
+      cell_launch(CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
+      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+      c_scatter_rows_ += (double)c.K * r.n;
+    }
+  } else {
+    // any other batch: two launches per round, with the message gradients going through the gradient
+    // of the message pool as in the reference (rows nobody wrote read as zero)
+    check(cavs_zero(dpool_.get(), (size_t)N * mw_ * 4, stream_));
+    c_launches_ += 1;
+    for (int k : sched_->bwd_rounds) {
+      const Round &r = sched_->rounds[k];
+      {
+        ProfScope ps(this, K_GATES);
+        cell_launch(CK_BWD_GATES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, d_dgo_);
+      }
+      c_gather_rows_ += r.n;
+      if (leaf_round(r)) continue;
+      ProfScope ps(this, K_ROUND);
+      cell_launch(CK_BWD_POOL, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
+      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+      c_scatter_rows_ += (double)c.K * r.n;
+    }
   }
   // the weight gradients, once over all rows: runs of terms whose operands, columns and gradient
   // blocks are adjacent go as one product

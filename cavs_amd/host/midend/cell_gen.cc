@@ -466,8 +466,8 @@ struct Writer {
            "static __device__ inline float cell_sigm(float x) { return __builtin_amdgcn_rcpf(1.f + cell_exp(-x)); }\n"
            "static __device__ inline float cell_tanh(float x) { return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + cell_exp(2.f * x)); }\n";
     } else {
-      o << "static inline float cell_sigm(float x) { return 1.f / (1.f + expf(-x)); }\n"
-           "static inline float cell_tanh(float x) { return tanhf(x); }\n";
+      o << "static inline float cell_sigm(float x) { return 1.f / (1.f + exp(-x)); }\n"
+           "static inline float cell_tanh(float x) { return tanh(x); }\n";
     }
     o << dev << "void cell_forward(const FwdIn &in, FwdOut &out) {\n";
     std::vector<int> roots = r.st;
@@ -503,7 +503,7 @@ struct Writer {
       << dv.ds_mask << "\n#define CELL_BWD_CS " << (dv.reads_cs ? 1 : 0) << "\n";
     o << "typedef float f4 __attribute__((ext_vector_type(4)));\n";
     o << "struct CellArgs {\n  float *pool;\n  const int *child, *pair, *kids, *t2j, *rows;\n  const float *xw;\n"
-         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum;\n  long off, n;\n  float *p["
+         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  long off, n;\n  float *p["
       << 2 * CA_MAX_PARAMS << "];\n};\n";
     o << "static __device__ inline f4 ld4(const float *p) { return *reinterpret_cast<const f4 *>(p); }\n";
   }

@@ -174,7 +174,13 @@ void ORF(treefc_bwd)(const real *dh_m, const real *dret, const real *h, real *dz
 enum {
   OR_MODEL_TREELSTM = 0, /* apps/paper/tree-lstm-cavs.cc */
   OR_MODEL_LSTM = 1,     /* apps/paper/seq-lstm-cavs.cc, seq-lstm-cavs-varLength.cc */
-  OR_MODEL_TREEFC = 2    /* apps/paper/tree-fc-cavs.cc */
+  OR_MODEL_TREEFC = 2,   /* apps/paper/tree-fc-cavs.cc */
+  /* Not one of the reference's applications: the Tree-LSTM of apps/paper/tree-lstm-cavs.cc:129-172 with
+   * a forget-gate matrix per child (U = [U_iou | U_fl | U_fr], 5*H*H) and the bias blocks in the
+   * order of the gate columns ([i|o|u|f]) -- a vertex function a user of the reference's API might
+   * declare, run through the same ops in the same order.  Pinned by the fp64 autograd formulation
+   * in tests/textbook.py. */
+  OR_MODEL_TREELSTM2 = 3
 };
 enum {
   OR_LOSS_SOFTMAX = 0,   /* FC head + softmax cross-entropy at every vertex */

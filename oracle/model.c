@@ -37,6 +37,7 @@ typedef struct {
   /* backward edges */
   real *dpool, *dmsg, *dret, *dxW, *dF, *dG, *dhlr, *dhf, *de;
   real *GO, *dGO;
+  real *bias; /* OR_MODEL_TREELSTM2: the bias in the block order the gate op reads ([i|f|u|o]) */
 } ctx;
 
 static real *zalloc(size_t n) { return (real *)calloc(n ? n : 1, sizeof(real)); }
@@ -93,7 +94,7 @@ static void fwd_round(ctx *c) {
   /* forward scatter: in row-id mode the slab row is list[b]; forward gather lists
    * are aligned with the job list in both modes. */
   int rowid = cfg->pairing == OR_PAIR_ROWID;
-  if (cfg->model == OR_MODEL_TREELSTM) {
+  if (cfg->model == OR_MODEL_TREELSTM || cfg->model == OR_MODEL_TREELSTM2) {
     do_gather(c, 0, 2, c->G, 2 * H, c->pool, 0);
     do_gather(c, 1, 2, c->G, 2 * H, c->pool, 0);
     real *G = c->G + (size_t)2 * off * 2 * H;
@@ -108,8 +109,13 @@ static void fwd_round(ctx *c) {
     real *hUf = c->hUf + (size_t)2 * off * H;
     ORF(sgemm)(0, 0, n, 4 * H, E, 1.f, e, E, p->W, 4 * H, 0.f, xW, 4 * H);               /* :146 */
     ORF(sgemm)(0, 0, n, 3 * H, H, 1.f, hlr, H, p->U, 3 * H, 0.f, hU, 3 * H);              /* :151 */
-    ORF(sgemm)(0, 0, 2 * n, H, H, 1.f, G, 2 * H, p->U + (size_t)3 * H * H, H, 0.f, hUf, H); /* :156-157 */
-    ORF(treelstm_gates_fwd)(xW, 4 * H, hU, hUf, G, p->Bv, c->gates + (size_t)off * 6 * H,
+    if (cfg->model == OR_MODEL_TREELSTM2) { /* rows 2b with U_fl, rows 2b+1 with U_fr */
+      ORF(sgemm)(0, 0, n, H, H, 1.f, G, 4 * H, p->U + (size_t)3 * H * H, H, 0.f, hUf, 2 * H);
+      ORF(sgemm)(0, 0, n, H, H, 1.f, G + 2 * H, 4 * H, p->U + (size_t)4 * H * H, H, 0.f, hUf + H, 2 * H);
+    } else {
+      ORF(sgemm)(0, 0, 2 * n, H, H, 1.f, G, 2 * H, p->U + (size_t)3 * H * H, H, 0.f, hUf, H); /* :156-157 */
+    }
+    ORF(treelstm_gates_fwd)(xW, 4 * H, hU, hUf, G, c->bias ? c->bias : p->Bv, c->gates + (size_t)off * 6 * H,
                           c->msg + (size_t)off * 2 * H, n, H);
     do_scatter(c, 0, 1, c->pool, 2 * H, c->msg, rowid);                                   /* :170 */
     ORF(copy_rows)(c->ret + (size_t)off * H, H, c->msg + (size_t)off * 2 * H, 2 * H, n, H); /* :171 Push */
@@ -152,7 +158,15 @@ static void weight_grads(ctx *c, int off, int n) {
   const or_config *cfg = c->cfg;
   ORF(grads) *g = c->g;
   int H = c->H, E = c->E;
-  if (cfg->model == OR_MODEL_TREELSTM) {
+  if (cfg->model == OR_MODEL_TREELSTM2) {
+    const real *dxW = c->dxW + (size_t)off * 4 * H;
+    const real *G = c->G + (size_t)2 * off * 2 * H, *dF = c->dF + (size_t)2 * off * H;
+    ORF(sgemm)(1, 0, E, 4 * H, n, 1.f, c->e + (size_t)off * E, E, dxW, 4 * H, 1.f, g->dW, 4 * H);
+    ORF(sgemm)(1, 0, H, 3 * H, n, 1.f, c->hlr + (size_t)off * H, H, dxW, 4 * H, 1.f, g->dU, 3 * H);
+    ORF(sgemm)(1, 0, H, H, n, 1.f, G, 4 * H, dF, 2 * H, 1.f, g->dU + (size_t)3 * H * H, H);
+    ORF(sgemm)(1, 0, H, H, n, 1.f, G + 2 * H, 4 * H, dF + H, 2 * H, 1.f, g->dU + (size_t)4 * H * H, H);
+    ORF(colsum)(g->dBv, dxW, 4 * H, n, 4 * H, 1); /* bias blocks in the order of the columns */
+  } else if (cfg->model == OR_MODEL_TREELSTM) {
     const real *dxW = c->dxW + (size_t)off * 4 * H;
     ORF(sgemm)(1, 0, E, 4 * H, n, 1.f, c->e + (size_t)off * E, E, dxW, 4 * H, 1.f, g->dW, 4 * H);
     ORF(sgemm)(1, 0, H, 3 * H, n, 1.f, c->hlr + (size_t)off * H, H, dxW, 4 * H, 1.f, g->dU, 3 * H);
@@ -189,14 +203,19 @@ static void bwd_round(ctx *c) {
   /* grad of Scatter is Gather(Child=0) on the swapped lists */
   do_gather(c, 0, 1, c->dmsg, mw, c->dpool, rowid);
   const real *dmsg = c->dmsg + (size_t)off * mw, *dret = c->dret + (size_t)off * H;
-  if (cfg->model == OR_MODEL_TREELSTM) {
+  if (cfg->model == OR_MODEL_TREELSTM || cfg->model == OR_MODEL_TREELSTM2) {
     real *dxW = c->dxW + (size_t)off * 4 * H, *dF = c->dF + (size_t)2 * off * H;
     real *dG = c->dG + (size_t)2 * off * 2 * H;
     const real *G = c->G + (size_t)2 * off * 2 * H;
     ORF(treelstm_gates_bwd)(dmsg, dret, c->gates + (size_t)off * 6 * H, G, dxW, 4 * H, dF, dG, n, H);
     real *dhlr = c->dhlr + (size_t)off * H, *dhf = c->dhf + (size_t)2 * off * H;
     ORF(sgemm)(0, 1, n, H, 3 * H, 1.f, dxW, 4 * H, p->U, 3 * H, 0.f, dhlr, H);
-    ORF(sgemm)(0, 1, 2 * n, H, H, 1.f, dF, H, p->U + (size_t)3 * H * H, H, 0.f, dhf, H);
+    if (cfg->model == OR_MODEL_TREELSTM2) {
+      ORF(sgemm)(0, 1, n, H, H, 1.f, dF, 2 * H, p->U + (size_t)3 * H * H, H, 0.f, dhf, 2 * H);
+      ORF(sgemm)(0, 1, n, H, H, 1.f, dF + H, 2 * H, p->U + (size_t)4 * H * H, H, 0.f, dhf + H, 2 * H);
+    } else {
+      ORF(sgemm)(0, 1, 2 * n, H, H, 1.f, dF, H, p->U + (size_t)3 * H * H, H, 0.f, dhf, H);
+    }
     for (int b = 0; b < 2 * n; b++) /* dh_l = dh_lr + d_fl*U_f^T (Mirror accumulate) */
       for (int j = 0; j < H; j++)
         dG[(size_t)b * 2 * H + j] = dhlr[(size_t)(b / 2) * H + j] + dhf[(size_t)b * H + j];
@@ -273,7 +292,12 @@ int ORF(model_step)(const or_config *cfg, const ORF(params) *p, const int *graph
     c.z = zalloc(R * H);
     c.dxW = zalloc(R * H);
   }
-  if (cfg->model == OR_MODEL_TREELSTM) {
+  if (cfg->model == OR_MODEL_TREELSTM2) {
+    static const int from[4] = {0, 3, 2, 1}; /* block k of [i|f|u|o] is block from[k] of [i|o|u|f] */
+    c.bias = zalloc((size_t)4 * H);
+    for (int k = 0; k < 4; k++) memcpy(c.bias + (size_t)k * H, p->Bv + (size_t)from[k] * H, sizeof(real) * (size_t)H);
+  }
+  if (cfg->model == OR_MODEL_TREELSTM || cfg->model == OR_MODEL_TREELSTM2) {
     c.hlr = zalloc(R * H);
     c.dhlr = zalloc(R * H);
     c.hU = zalloc(R * 3 * H);
@@ -352,9 +376,9 @@ int ORF(model_step)(const or_config *cfg, const ORF(params) *p, const int *graph
     } else if (cfg->use_bias) {
       memset(g->dBv, 0, sizeof(real) * (size_t)H);
     }
-    if (cfg->model == OR_MODEL_TREELSTM) {
+    if (cfg->model == OR_MODEL_TREELSTM || cfg->model == OR_MODEL_TREELSTM2) {
       memset(g->dW, 0, sizeof(real) * (size_t)E * 4 * H);
-      memset(g->dU, 0, sizeof(real) * (size_t)4 * H * H);
+      memset(g->dU, 0, sizeof(real) * (size_t)(cfg->model == OR_MODEL_TREELSTM2 ? 5 : 4) * H * H);
     } else if (cfg->model == OR_MODEL_LSTM) {
       memset(g->dW, 0, sizeof(real) * (size_t)8 * H * H);
     } else {
@@ -370,7 +394,7 @@ int ORF(model_step)(const or_config *cfg, const ORF(params) *p, const int *graph
   }
 
   real *all[] = {c.pool, c.dpool, c.G, c.dG, c.msg, c.dmsg, c.ret, c.dret, c.GO, c.dGO, c.xs,
-                  c.e, c.de, c.xW, c.dxW, c.gates, c.z, c.hlr, c.dhlr, c.hU, c.hUf, c.dF, c.dhf};
+                  c.e, c.de, c.xW, c.dxW, c.gates, c.z, c.hlr, c.dhlr, c.hU, c.hUf, c.dF, c.dhf, c.bias};
   for (size_t i = 0; i < sizeof all / sizeof all[0]; i++) free(all[i]);
   or_sched_free(c.s);
   return N;

@@ -12,7 +12,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_HERE, "libcavs_oracle.so")
 
-MODEL = {"treelstm": 0, "lstm": 1, "treefc": 2}
+MODEL = {"treelstm": 0, "lstm": 1, "treefc": 2, "treelstm2": 3}
 LOSS = {"softmax": 0, "root_sq": 1, "sum_abs": 2}
 PAIR = {"reference": 0, "rowid": 1}
 
@@ -252,9 +252,9 @@ def model_step(model, graph, x, labels, params, *, H, E=0, V=0, Cc=0, loss="soft
     pool = np.zeros((N, mw), dt)
     grads = {}
     if want_grads:
-        if model == "treelstm":
+        if model in ("treelstm", "treelstm2"):
             grads = dict(dEmb=np.zeros((V, Ee), dt), dW=np.zeros((Ee, 4 * H), dt),
-                         dU=np.zeros(4 * H * H, dt), dBv=np.zeros(4 * H, dt))
+                         dU=np.zeros((5 if model == "treelstm2" else 4) * H * H, dt), dBv=np.zeros(4 * H, dt))
         elif model == "lstm":
             grads = dict(dEmb=np.zeros((V, Ee), dt), dW=np.zeros(8 * H * H, dt),
                          dBv=np.zeros(4 * H, dt))

@@ -1,0 +1,118 @@
+"""Lowering of a vertex function of the general one-stage shape onto generated kernels, the parts
+that need no device: what the analysis of F accepts and refuses, and the elementwise part of the
+backward function it derives -- compiled for the host in double and held against central
+differences of the generated forward part (a wrong sign, a dropped term or a swapped operand of the
+derivation fails this)."""
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+
+from cavs_amd import apps
+
+
+def _dump(what):
+    _, h = apps.libs()
+    h.C_DumpCell.restype = C.c_size_t
+    h.C_DumpCell.argtypes = [C.c_char_p, C.c_size_t, C.c_int]
+    n = h.C_DumpCell(None, 0, what)
+    buf = C.create_string_buffer(n)
+    h.C_DumpCell(buf, n, what)
+    return buf.value.decode()
+
+
+def _declare(model, H=64):
+    return apps.App(model, B=3, maxlen=8, H=H, E=8, V=20, C_=4, opt=-1)
+
+
+HARNESS = r"""
+#include <math.h>
+#include <string.h>
+#define float double
+%s
+#undef float
+extern "C" {
+int sizes(int *s) { s[0] = sizeof(FwdIn) / 8; s[1] = sizeof(FwdOut) / 8; s[2] = sizeof(BwdIn) / 8; s[3] = sizeof(BwdOut) / 8; return 0; }
+void fwd(const double *in, double *out) { FwdIn i; FwdOut o; memcpy(&i, in, sizeof i); cell_forward(i, o); memcpy(out, &o, sizeof o); }
+void bwd(const double *in, double *out) { BwdIn i; BwdOut o; memcpy(&i, in, sizeof i); cell_backward(i, o); memcpy(out, &o, sizeof o); }
+}
+"""
+
+
+@pytest.mark.parametrize("model", ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"])
+def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, tmp_path):
+    a = _declare(model)
+    src = _dump(0)
+    a.close()
+    if model == "treefc_x":  # pulls a whole row of the vertex input: not the general shape
+        assert src.startswith("// not a cell")
+        return
+    dims = {k: int(v) for k, v in re.findall(r"(\w+)=(\d+)", [l for l in src.splitlines() if l.startswith("// H=")][0])}
+    K, S, NX, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "NX", "NP", "NB", "ND", "NSV"))
+    prod_col = [int(c) for c in re.findall(r"// product \d+ dcol (\d+)", src)]
+    bias_col = [int(c) for c in re.findall(r"// bias \d+ dcol (\d+)", src)]
+    assert len(prod_col) == NP and len(bias_col) == NB
+    cc = tmp_path / "cell.cc"
+    cc.write_text(HARNESS % src)
+    so = tmp_path / "cell.so"
+    subprocess.run(["g++", "-O1", "-shared", "-fPIC", "-o", str(so), str(cc)], check=True)
+    lib = C.CDLL(str(so))
+    sz = (C.c_int * 4)()
+    lib.sizes(sz)
+    nxm, nbm, nsvm = max(1, NX), max(1, NB), max(1, NSV)
+    assert list(sz) == [nxm + NP + nbm + K * S, S + 1 + nsvm, S + 1 + nsvm + K * S, ND + K * S]
+    dp = C.POINTER(C.c_double)
+
+    def fwd(x):
+        out = np.zeros(sz[1])
+        lib.fwd(np.ascontiguousarray(x).ctypes.data_as(dp), out.ctypes.data_as(dp))
+        return out
+
+    rng = np.random.default_rng(5)
+    for _ in range(20):
+        x = rng.normal(0, 0.8, sz[0])
+        seed = rng.normal(0, 1, S + 1)  # d st[0..S), d ret
+        out = fwd(x)
+        bin_ = np.concatenate([seed, out[S + 1:], x[nxm + NP + nbm:]])
+        bout = np.zeros(sz[3])
+        lib.bwd(bin_.ctypes.data_as(dp), bout.ctypes.data_as(dp))
+        num = np.zeros(sz[0])
+        eps = 1e-6
+        for i in range(sz[0]):
+            e = np.zeros(sz[0])
+            e[i] = eps
+            num[i] = (seed @ (fwd(x + e)[: S + 1] - fwd(x - e)[: S + 1])) / (2 * eps)
+        want = np.zeros(sz[0])
+        for i in range(NX):
+            want[i] = bout[i]
+        for p in range(NP):
+            want[nxm + p] = bout[prod_col[p]]
+        for i in range(NB):
+            want[nxm + NP + i] = bout[bias_col[i]]
+        want[nxm + NP + nbm:] = bout[ND:]
+        np.testing.assert_allclose(want, num, rtol=1e-6, atol=1e-8)
+
+
+def test_the_reference_tree_lstm_keeps_six_values_and_six_gradient_blocks_per_vertex():
+    """The same as the hand-written kernels keep: the five gates and tanh(c); d(x W) in four blocks
+    plus the two forget gates' own."""
+    a = _declare("treelstm")
+    src = _dump(0)
+    dev = _dump(1)
+    a.close()
+    assert "NX=4 NP=5 NB=4 ND=6 NSV=6" in src
+    assert "#define CELL_NA 3" in dev and "#define CELL_NT 5" in dev and "#define CELL_DS_MASK 2" in dev
+    assert dev.count("__builtin_amdgcn_mfma_f32_16x16x4f32") == 10  # five per direction and k step
+
+
+def test_what_is_not_of_the_general_shape_says_why():
+    a = _declare("treefc_x")
+    assert "Pull of a vertex input wider than one id" in _dump(1)
+    a.close()
+    a = _declare("treelstm", H=40)
+    assert "multiple of 32" in _dump(1)
+    a.close()

@@ -1,0 +1,111 @@
+"""Vertex functions lowered onto kernels generated for them (the general one-stage shape): the
+reference's three applications forced onto that path, a Tree-LSTM with a forget-gate matrix per
+child and a gated cell with one state block, against the oracle (or, for the gated cell, the fp64
+autograd formulation of tests/textbook.py) on the same seeded inputs."""
+import numpy as np
+import pytest
+
+import textbook
+from cavs_amd import apps, session, synth
+from test_oracle_models import small_workload
+from tolerance import close
+
+pytestmark = pytest.mark.gpu
+
+NAMES = {"treelstm": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treelstm2": ("Emb", "W", "U", "Bv", "Wfc", "bfc"),
+         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",)}
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _gpu():
+    import torch
+
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+
+
+def oracle_step(oracle, w, model, **kw):
+    return oracle.model_step(model, w["graph"], w["x"], w["labels"], w["params"], H=w["H"], E=w["E"], V=w["V"],
+                             Cc=w["C"], precise=True, threads=16, **kw)
+
+
+def run_generated(model, w, pairing, mode=2, lr=0.0):
+    B, maxlen = w["graph"].shape
+    a = apps.App(model, B=B, maxlen=maxlen, H=w["H"], E=w["E"], V=w["V"], C_=w["C"], opt=session.OPT_BATCHING, lr=lr,
+                 pairing=pairing, allow_fused=mode)
+    a.set_params({k: w["params"][k] for k in NAMES[model]})
+    print(f"[case] app={model} N={w['N']} H={w['H']} pairing={pairing} lowering mode={mode}", flush=True)
+    loss, go = a.step(w["graph"], w["x"], w["labels"], train=True)
+    grads = {"d" + k: a.grad(k, np.shape(w["params"][k])) for k in NAMES[model]}
+    kind = a.fused_kind
+    a.close()
+    return loss, go, grads, kind
+
+
+def compare(got, want):
+    loss, go, grads, _ = got
+    close(go, want["graph_out"], "graph_out")
+    close(loss, want["loss"], "loss")
+    for k, v in grads.items():
+        close(v, np.reshape(want["grads"][k], v.shape), k)
+
+
+@pytest.mark.parametrize("model,H", [("treelstm", 32), ("treelstm", 64), ("treelstm", 128), ("lstm", 64), ("treefc", 32), ("treefc", 128)])
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_the_reference_applications_on_generated_kernels(oracle, model, H, pairing):
+    """Lowering mode 2 skips the hand-written kernels: the same F, recognised by its shape alone.  The
+    batches are skewed, so under the reference's pairing the message flow is no forest and the
+    backward pass goes through the gradient of the message pool; under row-id pairing it is one."""
+    w = small_workload(model, 183, B=6, H=H, E=12, V=29, C=5)
+    kw = dict(loss="sum_abs", act=0) if model == "treefc" else {}
+    want = oracle_step(oracle, w, model, pairing=pairing, **kw)
+    got = run_generated(model, w, pairing)
+    assert got[3] == 2, "the vertex function was not lowered onto generated kernels"
+    compare(got, want)
+
+
+@pytest.mark.parametrize("H", [64, 128])
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_a_tree_lstm_with_a_forget_matrix_per_child(oracle, H, pairing):
+    """A fourth vertex function, which no hand-written kernel covers: lowered by the default mode."""
+    w = small_workload("treelstm2", 184, B=7, H=H, E=20, V=31, C=4)
+    want = oracle_step(oracle, w, "treelstm2", pairing=pairing)
+    got = run_generated("treelstm2", w, pairing, mode=1)
+    assert got[3] == 2
+    compare(got, want)
+    # and op by op, the way the reference would run it
+    compare(run_generated("treelstm2", w, pairing, mode=0), want)
+
+
+def test_a_gated_cell_with_one_state_block_against_fp64_autograd():
+    """Children's states enter through products (one of them over their concatenation) and
+    elementwise; the message has one block.  No oracle restatement: held to the per-sample fp64
+    formulation, which a batch under row-id pairing equals."""
+    w = small_workload("treegate", 185, B=6, H=64, E=12, V=29, C=5)
+    want = textbook.per_sample("treegate", w["graph"], w["x"], w["labels"], w["params"], w["H"])
+    got = run_generated("treegate", w, "rowid", mode=1)
+    assert got[3] == 2
+    compare(got, want)
+    compare(run_generated("treegate", w, "rowid", mode=0), want)
+
+
+def test_training_steps_on_generated_kernels_update_variables_like_the_oracle(oracle):
+    """Three SGD steps of the fourth vertex function through Session::Run({train})."""
+    H, E, V, C_ = 64, 10, 23, 4
+    w = small_workload("treelstm2", 187, B=5, H=H, E=E, V=V, C=C_)
+    B, maxlen = w["graph"].shape
+    lr = 0.25
+    a = apps.App("treelstm2", B=B, maxlen=maxlen, H=H, E=E, V=V, C_=C_, opt=session.OPT_BATCHING, lr=lr)
+    p = {k: np.array(w["params"][k], np.float32) for k in NAMES["treelstm2"]}
+    p["U"] = (p["U"] * np.float32(0.3)).astype(np.float32)
+    a.set_params(p)
+    for step in range(3):
+        print(f"[case] generated kernels, sgd step {step}", flush=True)
+        want = oracle_step(oracle, dict(w, params=p), "treelstm2")
+        loss, _ = a.step(w["graph"], w["x"], w["labels"], train=True)
+        assert a.fused_kind == 2
+        close(loss, want["loss"], f"loss at step {step}")
+        for k in NAMES["treelstm2"]:
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    close(a.grad("U", p["U"].shape, grad=False), p["U"], "U after 3 steps")
+    close(a.grad("Bv", p["Bv"].shape, grad=False), p["Bv"], "Bv after 3 steps")
+    a.close()

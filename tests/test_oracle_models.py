@@ -33,10 +33,14 @@ def small_workload(model, seed, B=5, H=12, E=10, V=37, C=5, skew=True):
             graph, leaves = synth.pack_graph([tree] * B, 15), [6] * B
         N = sum(2 * l - 1 for l in leaves)
     p = {}
-    if model == "treelstm":
+    if model in ("treelstm", "treelstm2"):  # (treelstm2: a forget-gate matrix per child, U = [U_iou | U_fl | U_fr])
         p = dict(Emb=rng.bulk_normal(V * E, 0, 0.5).reshape(V, E),
                  W=rng.bulk_uniform(E * 4 * H, -0.4, 0.4).reshape(E, 4 * H),
-                 U=rng.bulk_uniform(4 * H * H, -0.4, 0.4), Bv=rng.bulk_uniform(4 * H, -0.3, 0.3))
+                 U=rng.bulk_uniform((5 if model == "treelstm2" else 4) * H * H, -0.4, 0.4), Bv=rng.bulk_uniform(4 * H, -0.3, 0.3))
+        x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
+    elif model == "treegate":  # (textbook._treegate_cell: one state block, no oracle restatement)
+        p = dict(Emb=rng.bulk_normal(V * E, 0, 0.5).reshape(V, E), W=rng.bulk_uniform(E * 2 * H, -0.4, 0.4),
+                 U=rng.bulk_uniform(3 * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(2 * H, -0.3, 0.3))
         x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
     elif model == "lstm":
         p = dict(Emb=rng.bulk_normal(V * H, 0, 0.5).reshape(V, H),
@@ -68,7 +72,7 @@ def _compare(res, ref, grads=True):
 
 
 CASES = [("treelstm", dict()), ("lstm", dict()), ("treefc", dict(act=1, use_bias=True, use_x=True)),
-         ("treefc", dict(act=0))]
+         ("treefc", dict(act=0)), ("treelstm2", dict())]
 
 
 @pytest.mark.parametrize("model,kw", CASES)

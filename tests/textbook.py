@@ -62,6 +62,36 @@ def _treelstm_cell(P, H, xid, hl, cl, hr, cr):
     return o * torch.tanh(c), c
 
 
+def _treelstm2_cell(P, H, xid, hl, cl, hr, cr):
+    """Forget gates with a recurrent matrix per child; bias blocks in the order of the gate columns."""
+    W, U, Bv = P["W"], P["U"], P["Bv"]
+    U_iou = U[: 3 * H * H].reshape(H, 3 * H)
+    U_fl = U[3 * H * H : 4 * H * H].reshape(H, H)
+    U_fr = U[4 * H * H :].reshape(H, H)
+    xW = P["Emb"][xid] @ W
+    iou = xW[..., : 3 * H] + (hl + hr) @ U_iou + Bv[: 3 * H]
+    i, o, u = torch.sigmoid(iou[..., :H]), torch.sigmoid(iou[..., H : 2 * H]), torch.tanh(iou[..., 2 * H :])
+    fl = torch.sigmoid(xW[..., 3 * H :] + hl @ U_fl + Bv[3 * H :])
+    fr = torch.sigmoid(xW[..., 3 * H :] + hr @ U_fr + Bv[3 * H :])
+    c = i * u + fl * cl + fr * cr
+    return o * torch.tanh(c), c
+
+
+def _treegate_cell(P, H, xid, hl, hr):
+    """One state block: z = sigmoid(x W_z + (h_l + h_r) U_z + b_z), u = tanh(x W_u + [h_l, h_r] U_lr + b_u),
+    h = u z + g - z g with g = (h_l + h_r) sigmoid(h_l + h_r)."""
+    W, U, Bv = P["W"], P["U"], P["Bv"]
+    E = P["Emb"].shape[1]
+    U_z = U[: H * H].reshape(H, H)
+    U_lr = U[H * H :].reshape(2 * H, H)
+    xW = P["Emb"][xid] @ W.reshape(E, 2 * H)
+    hs = hl + hr
+    z = torch.sigmoid(xW[..., :H] + hs @ U_z + Bv[:H])
+    u = torch.tanh(xW[..., H:] + torch.cat([hl, hr], -1) @ U_lr + Bv[H:])
+    g = hs * torch.sigmoid(hs)
+    return u * z + g - z * g
+
+
 def _lstm_cell(P, H, xid, hp, cp):
     Wf = P["W"]
     Ux = Wf[: 4 * H * H].reshape(H, 4 * H)
@@ -102,10 +132,15 @@ def per_sample(model, graph, x, labels, params, H, loss="softmax", act=0, use_bi
                 stack.append(p)
     for v in order:
         ch = sorted(children[v])
-        if model == "treelstm":
+        if model in ("treelstm", "treelstm2"):
             hl, cl = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
-            hr, cr = (h[ch[1]], c[ch[1]]) if ch else (zero, zero)
-            h[v], c[v] = _treelstm_cell(P, H, int(xs[v]), hl, cl, hr, cr)
+            hr, cr = (h[ch[1]], c[ch[1]]) if len(ch) > 1 else (zero, zero)
+            cell = _treelstm_cell if model == "treelstm" else _treelstm2_cell
+            h[v], c[v] = cell(P, H, int(xs[v]), hl, cl, hr, cr)
+        elif model == "treegate":
+            hl = h[ch[0]] if ch else zero
+            hr = h[ch[1]] if len(ch) > 1 else zero
+            h[v] = _treegate_cell(P, H, int(xs[v]), hl, hr)
         elif model == "lstm":
             hp, cp = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
             h[v], c[v] = _lstm_cell(P, H, int(xs[v]), hp, cp)
@@ -140,9 +175,9 @@ def round_based(model, graph, trace, x, labels, params, H, loss="softmax", act=0
             if lst:
                 g = torch.cat([pool[lst], g[len(lst):]], 0)
             G.append(g)
-        if model == "treelstm":
-            hh, cc = _treelstm_cell(P, H, xs[jobs].long(), G[0][:, :H], G[0][:, H:], G[1][:, :H],
-                                    G[1][:, H:])
+        if model in ("treelstm", "treelstm2"):
+            cell = _treelstm_cell if model == "treelstm" else _treelstm2_cell
+            hh, cc = cell(P, H, xs[jobs].long(), G[0][:, :H], G[0][:, H:], G[1][:, :H], G[1][:, H:])
             msg = torch.cat([hh, cc], 1)
         elif model == "lstm":
             hh, cc = _lstm_cell(P, H, xs[jobs].long(), G[0][:, :H], G[0][:, H:])
