@@ -189,7 +189,7 @@ long C_ReadTensor(C_Session *s, const char *name, float *out, size_t cap) {
 
 int C_SessionUsesFusedPath(C_Session *s) { return s->exec.fused_path_kind(); }
 int C_SessionGeneratedKernels(C_Session *s) { return s->exec.fused_kernel_count(); }
-void C_SessionAllowFusedPath(C_Session *s, int allow) { s->exec.set_lowering_mode(allow < 0 ? 0 : allow > 2 ? 2 : allow); }
+void C_SessionAllowFusedPath(C_Session *s, int allow) { s->exec.set_lowering_mode(allow < 0 ? 0 : allow > 3 ? 3 : allow); }
 void C_SessionSetPairing(C_Session *s, int pairing) { s->exec.set_pairing(pairing); }
 
 }  // extern "C"

@@ -168,7 +168,7 @@ void Executor::compile() {
       }
     }
     if (lowering_mode_ > 0 && (opt_ & OPT_BATCHING)) {
-      lowering_ = match_vertex_function(g, lowering_mode_);
+      lowering_ = match_vertex_function(g, lowering_mode_ == 1 ? 1 : 2);
       lowered_ = lowering_ != nullptr;
     }
   }

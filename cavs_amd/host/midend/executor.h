@@ -88,7 +88,9 @@ class Executor {
   std::string name_;
   void *stream_ = nullptr;
   int compiled_version_ = -1;
-  int lowering_mode_ = 1;  // 0: never lower F; 1: hand-written kernels, else generated ones; 2: generated ones only
+  // 0: never lower F; 1: hand-written kernels, else generated ones; 2: generated ones only; 3: the same,
+  // with the backward rounds split as for a batch whose message flow is no forest
+  int lowering_mode_ = 1;
   bool lowered_ = false;
   int pairing_ = 0;
   std::map<std::string, std::unique_ptr<Tensor>> tensors_;

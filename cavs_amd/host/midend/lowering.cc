@@ -367,6 +367,7 @@ void Executor::lowered_forward(const int32_t *graph, int B, int maxlen, float *)
     cfg.act = lw.act;
     cfg.use_bias = lw.use_bias;
     cfg.use_x = lw.use_x;
+    cfg.split_backward_rounds = lowering_mode_ == 3;
     engine_ = std::make_unique<Engine>(cfg, stream_, lw.cell);
   }
   engine_->set_pairing(pairing_);

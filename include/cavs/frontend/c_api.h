@@ -54,7 +54,9 @@ int C_SessionUsesFusedPath(C_Session *s);
 /* Number of kernels the OPT_FUSION pass generated for the programs compiled so far. */
 int C_SessionGeneratedKernels(C_Session *s);
 /* 0 forbids that lowering (op-by-op execution of F, for A/B tests); 1, the default, tries the
- * hand-written kernels first and generated ones next; 2 goes for generated kernels only. */
+ * hand-written kernels first and generated ones next; 2 goes for generated kernels only; 3 does the
+ * same and runs the backward rounds the way a batch whose message flow is no forest needs them
+ * (two launches per round, message gradients through the gradient of the message pool). */
 void C_SessionAllowFusedPath(C_Session *s, int allow);
 void C_SessionSetPairing(C_Session *s, int pairing); /* CAVS_PAIR_* of cavs_session.h */
 const char *C_LastError(void);

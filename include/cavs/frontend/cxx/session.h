@@ -35,7 +35,7 @@ class Session {
   int GeneratedKernels() const { return C_SessionGeneratedKernels(s_); }
   int FusedPathKind() const { return C_SessionUsesFusedPath(s_); }  // 0 none, 1 hand-written, 2 generated
   void AllowFusedPath(bool allow) { C_SessionAllowFusedPath(s_, allow ? 1 : 0); }
-  void SetLoweringMode(int mode) { C_SessionAllowFusedPath(s_, mode); }  // 0 none, 1 any, 2 generated kernels only
+  void SetLoweringMode(int mode) { C_SessionAllowFusedPath(s_, mode); }  // 0 none, 1 any, 2 generated kernels only, 3 the same with split backward rounds
   void SetPairing(int pairing) { C_SessionSetPairing(s_, pairing); }
   C_Session *handle() const { return s_; }
 

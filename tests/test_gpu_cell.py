@@ -52,15 +52,16 @@ def compare(got, want):
 @pytest.mark.parametrize("model,H", [("treelstm", 32), ("treelstm", 64), ("treelstm", 128), ("lstm", 64), ("treefc", 32), ("treefc", 128)])
 @pytest.mark.parametrize("pairing", ["reference", "rowid"])
 def test_the_reference_applications_on_generated_kernels(oracle, model, H, pairing):
-    """Lowering mode 2 skips the hand-written kernels: the same F, recognised by its shape alone.  The
-    batches are skewed, so under the reference's pairing the message flow is no forest and the
-    backward pass goes through the gradient of the message pool; under row-id pairing it is one."""
+    """Lowering mode 2 skips the hand-written kernels: the same F, recognised by its shape alone.
+    Mode 3 also runs the backward rounds as a batch whose message flow is no forest needs them: two
+    launches per round, with the message gradients going through the gradient of the message pool."""
     w = small_workload(model, 183, B=6, H=H, E=12, V=29, C=5)
     kw = dict(loss="sum_abs", act=0) if model == "treefc" else {}
     want = oracle_step(oracle, w, model, pairing=pairing, **kw)
-    got = run_generated(model, w, pairing)
-    assert got[3] == 2, "the vertex function was not lowered onto generated kernels"
-    compare(got, want)
+    for mode in (2, 3):
+        got = run_generated(model, w, pairing, mode=mode)
+        assert got[3] == 2, "the vertex function was not lowered onto generated kernels"
+        compare(got, want)
 
 
 @pytest.mark.parametrize("H", [64, 128])
@@ -82,9 +83,10 @@ def test_a_gated_cell_with_one_state_block_against_fp64_autograd():
     formulation, which a batch under row-id pairing equals."""
     w = small_workload("treegate", 185, B=6, H=64, E=12, V=29, C=5)
     want = textbook.per_sample("treegate", w["graph"], w["x"], w["labels"], w["params"], w["H"])
-    got = run_generated("treegate", w, "rowid", mode=1)
-    assert got[3] == 2
-    compare(got, want)
+    for mode in (1, 3):
+        got = run_generated("treegate", w, "rowid", mode=mode)
+        assert got[3] == 2
+        compare(got, want)
     compare(run_generated("treegate", w, "rowid", mode=0), want)
 
 
