@@ -105,21 +105,30 @@ def cpu_baseline(w, budget_s=12.0):
 def front_end_modes(pool, steps=60, warmup=30):
     """The same training step through the reference's own API (Sym / GraphSupport / Session::Run with
     host feeds, one device synchronisation per Run, loss head and optimizer as ordinary ops), in the
-    three ways the session can execute F: lowered onto the fused round kernels, op by op with the
-    fusion pass's generated kernels, and plain op by op -- the reference's execution model on this GPU."""
+    ways the session can execute F: lowered onto the hand-written round kernels, lowered onto kernels
+    generated for it (its shape recognised, not its identity), op by op with the fusion pass's
+    generated kernels, and plain op by op -- the reference's execution model on this GPU.  For a
+    Tree-LSTM workload also a vertex function no hand-written kernel covers (a forget-gate matrix per
+    child, same sizes): lowered onto generated kernels against op by op with the fusion pass."""
     import torch
 
-    from cavs_amd import apps, session
+    from cavs_amd import apps, session, synth
 
     w = pool[0]
     B, maxlen = w["graph"].shape
+    H = w["H"]
     out = {}
-    for name, opt, lowered in (("lowered", session.OPT_BATCHING, True),
-                               ("op_by_op_fusion", session.OPT_BATCHING | session.OPT_FUSION, False),
-                               ("op_by_op", session.OPT_BATCHING, False)):
-        app = apps.App(w["model"], B=B, maxlen=maxlen, H=w["H"], E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=1e-3,
-                       allow_fused=lowered)
-        app.set_params(w["params"])
+    cases = [("lowered", w["model"], session.OPT_BATCHING, 1), ("lowered_generated", w["model"], session.OPT_BATCHING, 2),
+             ("op_by_op_fusion", w["model"], session.OPT_BATCHING | session.OPT_FUSION, 0), ("op_by_op", w["model"], session.OPT_BATCHING, 0)]
+    if w["model"] == "treelstm":
+        cases += [("fourth_function_lowered_generated", "treelstm2", session.OPT_BATCHING, 1),
+                  ("fourth_function_op_by_op_fusion", "treelstm2", session.OPT_BATCHING | session.OPT_FUSION, 0)]
+    for name, model, opt, lowered in cases:
+        app = apps.App(model, B=B, maxlen=maxlen, H=H, E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=1e-3, allow_fused=lowered)
+        params = dict(w["params"])
+        if model == "treelstm2":  # [U_iou | U_fl | U_fr]
+            params["U"] = np.concatenate([np.ravel(params["U"]), synth.SplitMix64(9).bulk_uniform(H * H, -0.1, 0.1)]).astype(np.float32)
+        app.set_params(params)
         # untimed: at least `warmup` steps and 150 ms of continuous work (steady clocks, as in measure())
         # the same pool of batch structures as the headline measurement, cycled the same way
         done, t0 = 0, time.perf_counter()
@@ -136,7 +145,8 @@ def front_end_modes(pool, steps=60, warmup=30):
         torch.cuda.synchronize()
         ms = 1e3 * (time.perf_counter() - t0) / n
         out[name] = {"ms_per_step": round(ms, 4), "value": round(B / ms * 1e3, 1), "unit": "samples/s", "steps": n,
-                     "generated_kernels": app.generated_kernels}
+                     "generated_kernels": app.generated_kernels, "vertex_function": model,
+                     "runs_on": ("operators", "hand-written round kernels", "generated round kernels")[app.fused_kind]}
         app.close()
     return out
 
