@@ -405,7 +405,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_mfma_kernel(GemmArgs g) {
 // one long launch.  Workgroup b belongs to product p with first[p] <= b < first[p+1] (each
 // product's share is padded to a multiple of 8, so that b % 8 is the XCD within the share as
 // well); within the share, tile = local % tiles[p] and K split = local / tiles[p].
-constexpr int kGroupMax = 4;
+constexpr int kGroupMax = 8;
 struct GemmGroup {
   GemmArgs g[kGroupMax];
   int first[kGroupMax + 1];

@@ -1830,17 +1830,18 @@ void Engine::cell_backward() {
   else
     for (const Run &q : runs)  // a batch of single vertices: nothing was multiplied
       for (int row = 0; row < H; row++) check(cavs_zero(param(c.params[q.param].name).g + q.at() + (size_t)row * q.ldb, (size_t)q.width * 4, stream_));
+  constexpr size_t kGroup = 8;  // products per cavs_sgemm_group launch
   size_t at = 0;
   if (c.NX > 0) {
-    const size_t take = std::min<size_t>(products.size(), 4);
+    const size_t take = std::min<size_t>(products.size(), kGroup);
     gemm_group_embedding_backward(std::vector<cavs_gemm_desc>(products.begin(), products.begin() + take), E_);
     at = take;
   }
-  for (; at < products.size(); at += 4)
-    gemm_group(std::vector<cavs_gemm_desc>(products.begin() + at, products.begin() + std::min(products.size(), at + 4)));
+  for (; at < products.size(); at += kGroup)
+    gemm_group(std::vector<cavs_gemm_desc>(products.begin() + at, products.begin() + std::min(products.size(), at + kGroup)));
   for (const std::vector<cavs_gemm_desc> &wave : later)
-    for (size_t i = 0; i < wave.size(); i += 4)
-      gemm_group(std::vector<cavs_gemm_desc>(wave.begin() + i, wave.begin() + std::min(wave.size(), i + 4)));
+    for (size_t i = 0; i < wave.size(); i += kGroup)
+      gemm_group(std::vector<cavs_gemm_desc>(wave.begin() + i, wave.begin() + std::min(wave.size(), i + kGroup)));
   if (!c.biases.empty()) {
     colsum_fixed(cell_colsum_.get(), dxW_.get(), N, ldd);
     ProfScope ps(this, K_OTHER);

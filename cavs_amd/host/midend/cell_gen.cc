@@ -664,8 +664,8 @@ std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
     const int H = s.H;
     s.waves = H % 128 == 0 ? 4 : H % 64 == 0 ? 2 : 1;
     // the partial tiles of a workgroup must fit in LDS
-    const size_t lds = (size_t)s.waves * std::max(s.products.size(), s.asrc.size()) * 1024;
-    if (lds > 60 * 1024) no("too many accumulators for one workgroup");
+    const size_t per_wave = std::max(s.products.size(), s.asrc.size()) * 1024;
+    if (s.waves * per_wave > 60 * 1024) no("too many accumulators for one workgroup");
     Writer w(b.reader, b.derived, true);
     w.kernels();
     w.elementwise(b.nfwd);

@@ -151,7 +151,7 @@ size_t cavs_sgemm_splitk_static_max_bytes(void);
 int cavs_sgemm_splitk_static(int transA, int transB, int M, int N, int K, float alpha, const float *A,
                              int lda, const float *B, int ldb, float beta, float *C, int ldc,
                              void *stream);
-/* Up to four independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
+/* Up to eight independent products C_p = alpha_p*op(A_p)*op(B_p) + beta_p*C_p in one launch
  * (plus one for the K splits): the once-per-step block of
  * cavs/midend/batch_weight_updater.h:12-84 -- the weight-gradient GEMMs -- and the embedding
  * gradient's product next to it.  Each of them alone gives every CU one round of workgroups

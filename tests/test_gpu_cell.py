@@ -49,7 +49,7 @@ def compare(got, want):
         close(v, np.reshape(want["grads"][k], v.shape), k)
 
 
-@pytest.mark.parametrize("model,H", [("treelstm", 32), ("treelstm", 64), ("treelstm", 128), ("lstm", 64), ("treefc", 32), ("treefc", 128)])
+@pytest.mark.parametrize("model,H", [("treelstm", 32), ("treelstm", 64), ("treelstm", 128), ("treelstm", 256), ("lstm", 64), ("treefc", 32), ("treefc", 128)])
 @pytest.mark.parametrize("pairing", ["reference", "rowid"])
 def test_the_reference_applications_on_generated_kernels(oracle, model, H, pairing):
     """Lowering mode 2 skips the hand-written kernels: the same F, recognised by its shape alone.

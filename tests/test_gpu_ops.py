@@ -286,8 +286,8 @@ def test_sgemm_group_matches_separate_products(g, oracle, name):
         close(got[:, :N], exact, f"product {p} vs fp64")
         if 2.0 * M * N * K < 2e9:  # the oracle's plain loops take seconds beyond this
             close(got[:, :N], oracle.sgemm(tA, tB, A, B, alpha=1.5, beta=beta, Cin=np.ascontiguousarray(C0[:, :N])), f"product {p} vs oracle")
-    with pytest.raises(hip.CavsError, match="at most 4"):
-        g.call("cavs_sgemm_group", 5, descs, g.P(ws), nbytes, g.stream())
+    with pytest.raises(hip.CavsError, match="at most 8"):
+        g.call("cavs_sgemm_group", 9, descs, g.P(ws), nbytes, g.stream())
     if nbytes:
         with pytest.raises(hip.CavsError, match="workspace"):
             g.call("cavs_sgemm_group", len(shapes), descs, g.P(ws), nbytes - 256, g.stream())
