@@ -1741,16 +1741,15 @@ void Engine::cell_backward() {
       }
   }
   {
+    // the transposed weight blocks and, when every message is read exactly once, the elementwise
+    // part of the vertices without a reader: one launch
     ProfScope ps(this, K_OTHER);
-    cell_launch(CK_TRANSPOSE, H / 32, H / 32, c.terms(), 256, 0, 0, nullptr, d_dgo_);
+    const unsigned tiles = (unsigned)c.terms() * (H / 32) * (H / 32);
+    const long rows = forest_ ? n_orphans_ : 0;
+    cell_launch(CK_TRANSPOSE, tiles + (unsigned)((rows * H + 255) / 256), 1, 1, 256, tiles, rows, d_orphans_, d_dgo_);
   }
   if (forest_) {
-    // every message is read exactly once: a round's launch hands d(state) on to the children of its
-    // rows and runs their elementwise part at once; the vertices without a reader go first
-    if (n_orphans_ > 0) {
-      ProfScope ps(this, K_GATES);
-      cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
-    }
+    // a round's launch hands d(state) on to the children of its rows and runs their elementwise part at once
     for (int k : sched_->bwd_rounds) {
       const Round &r = sched_->rounds[k];
       c_gather_rows_ += r.n;
