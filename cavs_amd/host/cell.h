@@ -52,7 +52,8 @@ struct CellParam {
 
 struct CellSpec {
   int H = 0, K = 0, S = 0;      // block width, children per vertex, state blocks per message
-  int E = 0, V = 0, NX = 0;     // embedding width, vocabulary, blocks of x * W (0: F reads no vertex input)
+  int E = 0, V = 0, NX = 0;     // embedding width, vocabulary, blocks of x * W (0: F looks no vertex input up)
+  int XD = 0;                   // H-wide blocks of the vertex input's row that F pulls and uses as they are
   CellParamRef W;               // [E, NX * H]
   std::vector<CellParam> params;
   std::vector<CellASrc> asrc;
@@ -88,6 +89,7 @@ enum CellArg {
   CA_BT,         // float*  transposed H x H blocks of the products' terms
   CA_COLSUM,     // float*  [ND*H] column sums of D
   CA_DPOOL,      // float*  gradient of the message pool [*, S*H] (batches whose message flow is no forest)
+  CA_X,          // float*  the vertex input by vertex id [*, XD*H]
   CA_OFF,        // long    first slab row of the round
   CA_N,          // long    rows
   CA_PARAM0,     // float*  parameters, then their gradients, in CellSpec::params order

@@ -777,7 +777,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
 void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_dev, float *graph_out) {
   state_epoch_++;
   begin_step(graph, B, maxlen);
-  const bool reads_x = cell_ ? cell_->NX > 0 : (cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x);
+  const bool reads_x = cell_ ? cell_->NX > 0 || cell_->XD > 0 : (cfg_.model != CAVS_MODEL_TREEFC || cfg_.use_x);
   if (reads_x && !x_dev) fail(CAVS_EINVAL, "vertex input feed is null");
   d_x_ = x_dev;
   check(cavs_event_record(ev_[0], stream_));
@@ -1685,6 +1685,7 @@ void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned 
   a[CA_BT].p = UT_.get();
   a[CA_COLSUM].p = cell_colsum_.get();
   a[CA_DPOOL].p = dpool_.get();
+  a[CA_X].p = d_x_;
   a[CA_OFF].i = off;
   a[CA_N].i = n;
   for (size_t i = 0; i < c.params.size(); i++) {

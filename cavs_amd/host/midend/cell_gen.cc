@@ -22,7 +22,7 @@ const char kTemplate[] =
 // One node per value of one hidden unit of one vertex.  Nodes are created in evaluation order, so an
 // operand's id is below its user's; equal nodes are shared.
 enum Kind {
-  N_XW, N_HU, N_BIAS, N_CS,        // inputs of the forward part (i0, i1 index them)
+  N_XW, N_HU, N_BIAS, N_CS, N_XD,  // inputs of the forward part (i0, i1 index them)
   N_DST, N_DRET, N_ZERO,           // seeds of the backward part, and "no gradient"
   N_ADD, N_SUB, N_MUL, N_NEG, N_SIGM, N_TANH, N_RELU,
   N_DSIGM, N_DTANH, N_DRELU        // a = gradient, b = the activation's output
@@ -192,8 +192,17 @@ struct Reader {
         for (int m = 0; m < s.S; m++) b.push_back(dag.make(N_CS, -1, -1, k, m));
         val[out] = b;
       } else if (op == "Pull") {
-        if (out->width() != 1) no("Pull of a vertex input wider than one id");
-        raw_x.insert(out);
+        const long w = out->width();
+        if (w == 1) {  // an id, to be looked up
+          raw_x.insert(out);
+        } else if (w % H == 0 && w / H <= 8 && !s.XD) {  // a row of the vertex input, used as it is
+          s.XD = (int)(w / H);
+          std::vector<int> b;
+          for (int i = 0; i < s.XD; i++) b.push_back(dag.make(N_XD, -1, -1, i));
+          val[out] = b;
+        } else {
+          no("Pull of a vertex input that is neither one id nor a few H-wide blocks");
+        }
       } else if (op == "EmbeddingLookup") {
         if (!raw_x.count(n->in[0])) no("EmbeddingLookup of something other than the pulled id");
         long count;
@@ -284,7 +293,7 @@ struct Reader {
     }
     if (st.empty() || ret < 0) no("F has no Scatter or no Push");
     if (s.K < 1) no("F gathers no child");
-    if (!raw_x.empty() && !have_xw) no("the vertex input is pulled but not multiplied");
+    if (!raw_x.empty() && !have_xw) no("the vertex input's id is pulled but not looked up and multiplied");
     if (s.products.empty()) no("F multiplies no child state");
     if (s.products.size() > 16 || s.asrc.size() > 8 || s.NX > 16 || s.biases.size() > 32) no("too many products or operands");
   }
@@ -398,6 +407,7 @@ struct Writer {
       case N_XW: if (!backward) return "in.xw[" + std::to_string(q.i0) + "]"; break;
       case N_HU: if (!backward) return "in.hu[" + std::to_string(q.i0) + "]"; break;
       case N_BIAS: if (!backward) return "in.bias[" + std::to_string(q.i0) + "]"; break;
+      case N_XD: if (!backward) return "in.xd[" + std::to_string(q.i0) + "]"; break;
       case N_CS: return "in.cs[" + std::to_string(q.i0) + "][" + std::to_string(q.i1) + "]";
       case N_DST: return "in.dst[" + std::to_string(q.i0) + "]";
       case N_DRET: return "in.dret";
@@ -455,7 +465,7 @@ struct Writer {
   void elementwise(int nfwd) {
     const char *dev = device ? "static __device__ inline " : "static inline ";
     o << "struct FwdIn { float xw[" << std::max(1, s.NX) << "], hu[" << s.products.size() << "], bias[" << std::max<size_t>(1, s.biases.size())
-      << "], cs[" << s.K << "][" << s.S << "]; };\n";
+      << "], cs[" << s.K << "][" << s.S << "], xd[" << std::max(1, s.XD) << "]; };\n";
     o << "struct FwdOut { float st[" << s.S << "], ret, sv[" << std::max(1, s.NSV) << "]; };\n";
     o << "struct BwdIn { float dst[" << s.S << "], dret, sv[" << std::max(1, s.NSV) << "], cs[" << s.K << "][" << s.S << "]; };\n";
     o << "struct BwdOut { float d[" << s.ND << "], dcs[" << s.K << "][" << s.S << "]; };\n";
@@ -498,12 +508,12 @@ struct Writer {
   void kernels() {
     const int H = s.H, NT = s.terms(), NP = (int)s.products.size(), NA = (int)s.asrc.size();
     o << "#define CELL_H " << H << "\n#define CELL_K " << s.K << "\n#define CELL_S " << s.S << "\n#define CELL_MW " << s.S * H
-      << "\n#define CELL_NX " << s.NX << "\n#define CELL_NP " << NP << "\n#define CELL_NA " << NA << "\n#define CELL_NT " << NT
+      << "\n#define CELL_NX " << s.NX << "\n#define CELL_XD " << s.XD << "\n#define CELL_NP " << NP << "\n#define CELL_NA " << NA << "\n#define CELL_NT " << NT
       << "\n#define CELL_ND " << s.ND << "\n#define CELL_NSV " << s.NSV << "\n#define CELL_KS " << s.waves << "\n#define CELL_DS_MASK "
       << dv.ds_mask << "\n#define CELL_BWD_CS " << (dv.reads_cs ? 1 : 0) << "\n";
     o << "typedef float f4 __attribute__((ext_vector_type(4)));\n";
     o << "struct CellArgs {\n  float *pool;\n  const int *child, *pair, *kids, *t2j, *rows;\n  const float *xw;\n"
-         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  long off, n;\n  float *p["
+         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  const float *x;\n  long off, n;\n  float *p["
       << 2 * CA_MAX_PARAMS << "];\n};\n";
     o << "static __device__ inline f4 ld4(const float *p) { return *reinterpret_cast<const f4 *>(p); }\n";
   }
@@ -692,7 +702,7 @@ std::string cell_host_source(const Graph &g) {
     w.o << "#include <math.h>\n";
     w.elementwise(b.nfwd);
     const CellSpec &s = b.reader.spec;
-    w.o << "// H=" << s.H << " K=" << s.K << " S=" << s.S << " NX=" << s.NX << " NP=" << s.products.size() << " NB=" << s.biases.size()
+    w.o << "// H=" << s.H << " K=" << s.K << " S=" << s.S << " NX=" << s.NX << " XD=" << s.XD << " NP=" << s.products.size() << " NB=" << s.biases.size()
         << " ND=" << s.ND << " NSV=" << s.NSV << "\n";
     for (size_t p = 0; p < s.products.size(); p++) w.o << "// product " << p << " dcol " << s.products[p].dcol << "\n";
     for (size_t i = 0; i < s.biases.size(); i++) w.o << "// bias " << i << " dcol " << s.biases[i].dcol << "\n";

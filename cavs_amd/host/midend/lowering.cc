@@ -246,7 +246,7 @@ std::unique_ptr<Lowering> match_vertex_function(const Graph &g, int mode) {
   lw->H = m->spec->H;
   lw->E = m->spec->E;
   lw->V = m->spec->V;
-  lw->use_x = m->spec->NX > 0;
+  lw->use_x = m->spec->NX > 0 || m->spec->XD > 0;
   lw->roles = m->roles;
   lw->cell = m->spec;
   lw->cell_slots = m->slots;

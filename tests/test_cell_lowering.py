@@ -48,11 +48,8 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
     a = _declare(model)
     src = _dump(0)
     a.close()
-    if model == "treefc_x":  # pulls a whole row of the vertex input: not the general shape
-        assert src.startswith("// not a cell")
-        return
     dims = {k: int(v) for k, v in re.findall(r"(\w+)=(\d+)", [l for l in src.splitlines() if l.startswith("// H=")][0])}
-    K, S, NX, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "NX", "NP", "NB", "ND", "NSV"))
+    K, S, NX, XD, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "NX", "XD", "NP", "NB", "ND", "NSV"))
     prod_col = [int(c) for c in re.findall(r"// product \d+ dcol (\d+)", src)]
     bias_col = [int(c) for c in re.findall(r"// bias \d+ dcol (\d+)", src)]
     assert len(prod_col) == NP and len(bias_col) == NB
@@ -63,8 +60,8 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
     lib = C.CDLL(str(so))
     sz = (C.c_int * 4)()
     lib.sizes(sz)
-    nxm, nbm, nsvm = max(1, NX), max(1, NB), max(1, NSV)
-    assert list(sz) == [nxm + NP + nbm + K * S, S + 1 + nsvm, S + 1 + nsvm + K * S, ND + K * S]
+    nxm, nbm, nsvm, xdm = max(1, NX), max(1, NB), max(1, NSV), max(1, XD)
+    assert list(sz) == [nxm + NP + nbm + K * S + xdm, S + 1 + nsvm, S + 1 + nsvm + K * S, ND + K * S]
     dp = C.POINTER(C.c_double)
 
     def fwd(x):
@@ -77,7 +74,7 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
         x = rng.normal(0, 0.8, sz[0])
         seed = rng.normal(0, 1, S + 1)  # d st[0..S), d ret
         out = fwd(x)
-        bin_ = np.concatenate([seed, out[S + 1:], x[nxm + NP + nbm:]])
+        bin_ = np.concatenate([seed, out[S + 1:], x[nxm + NP + nbm:nxm + NP + nbm + K * S]])
         bout = np.zeros(sz[3])
         lib.bwd(bin_.ctypes.data_as(dp), bout.ctypes.data_as(dp))
         num = np.zeros(sz[0])
@@ -93,8 +90,10 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
             want[nxm + p] = bout[prod_col[p]]
         for i in range(NB):
             want[nxm + NP + i] = bout[bias_col[i]]
-        want[nxm + NP + nbm:] = bout[ND:]
-        np.testing.assert_allclose(want, num, rtol=1e-6, atol=1e-8)
+        want[nxm + NP + nbm:nxm + NP + nbm + K * S] = bout[ND:]
+        live = np.ones(sz[0], bool)
+        live[nxm + NP + nbm + K * S:] = False  # the pulled vertex input is a feed: no gradient is derived for it
+        np.testing.assert_allclose(want[live], num[live], rtol=1e-6, atol=1e-8)
 
 
 def test_the_reference_tree_lstm_keeps_six_values_and_six_gradient_blocks_per_vertex():
@@ -104,15 +103,12 @@ def test_the_reference_tree_lstm_keeps_six_values_and_six_gradient_blocks_per_ve
     src = _dump(0)
     dev = _dump(1)
     a.close()
-    assert "NX=4 NP=5 NB=4 ND=6 NSV=6" in src
+    assert "NX=4 XD=0 NP=5 NB=4 ND=6 NSV=6" in src
     assert "#define CELL_NA 3" in dev and "#define CELL_NT 5" in dev and "#define CELL_DS_MASK 2" in dev
     assert dev.count("__builtin_amdgcn_mfma_f32_16x16x4f32") == 10  # five per direction and k step
 
 
 def test_what_is_not_of_the_general_shape_says_why():
-    a = _declare("treefc_x")
-    assert "Pull of a vertex input wider than one id" in _dump(1)
-    a.close()
     a = _declare("treelstm", H=40)
     assert "multiple of 32" in _dump(1)
     a.close()

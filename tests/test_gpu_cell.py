@@ -13,7 +13,7 @@ from tolerance import close
 pytestmark = pytest.mark.gpu
 
 NAMES = {"treelstm": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treelstm2": ("Emb", "W", "U", "Bv", "Wfc", "bfc"),
-         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",)}
+         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",), "treefc_x": ("W", "Bv")}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -28,13 +28,13 @@ def oracle_step(oracle, w, model, **kw):
                              Cc=w["C"], precise=True, threads=16, **kw)
 
 
-def run_generated(model, w, pairing, mode=2, lr=0.0):
+def run_generated(model, w, pairing, mode=2, lr=0.0, root_mask=None):
     B, maxlen = w["graph"].shape
     a = apps.App(model, B=B, maxlen=maxlen, H=w["H"], E=w["E"], V=w["V"], C_=w["C"], opt=session.OPT_BATCHING, lr=lr,
                  pairing=pairing, allow_fused=mode)
     a.set_params({k: w["params"][k] for k in NAMES[model]})
     print(f"[case] app={model} N={w['N']} H={w['H']} pairing={pairing} lowering mode={mode}", flush=True)
-    loss, go = a.step(w["graph"], w["x"], w["labels"], train=True)
+    loss, go = a.step(w["graph"], w["x"], w["labels"], train=True, root_mask=root_mask)
     grads = {"d" + k: a.grad(k, np.shape(w["params"][k])) for k in NAMES[model]}
     kind = a.fused_kind
     a.close()
@@ -61,6 +61,24 @@ def test_the_reference_applications_on_generated_kernels(oracle, model, H, pairi
     for mode in (2, 3):
         got = run_generated(model, w, pairing, mode=mode)
         assert got[3] == 2, "the vertex function was not lowered onto generated kernels"
+        compare(got, want)
+
+
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_a_pulled_row_of_the_vertex_input_on_generated_kernels(oracle, pairing):
+    """Tree-FC with tanh, a bias and the vertex's own input row added in: the row is read by vertex id
+    inside the round kernels (Pull folded in), the loss is the sum of squares at the roots."""
+    w = small_workload("treefc", 188, B=6, H=64)
+    want = oracle_step(oracle, w, "treefc", pairing=pairing, loss="root_sq", act=1, use_bias=True, use_x=True)
+    mask = np.zeros((w["N"], w["H"]), np.float32)
+    off = 0
+    for row in w["graph"]:
+        n = int(np.argmax(row == -1)) + 1
+        mask[off + n - 1] = 1
+        off += n
+    for mode in (2, 3):
+        got = run_generated("treefc_x", w, pairing, mode=mode, root_mask=mask)
+        assert got[3] == 2
         compare(got, want)
 
 
