@@ -102,7 +102,7 @@ def cpu_baseline(w, budget_s=12.0):
                                    sample=f"2 steps of the same batch in {el1:.1f} s"))
 
 
-def front_end_modes(pool, steps=60, warmup=30):
+def front_end_modes(pool, steps=60, warmup=30, only=None):
     """The same training step through the reference's own API (Sym / GraphSupport / Session::Run with
     host feeds, one device synchronisation per Run, loss head and optimizer as ordinary ops), in the
     ways the session can execute F: lowered onto the hand-written round kernels, lowered onto kernels
@@ -124,6 +124,8 @@ def front_end_modes(pool, steps=60, warmup=30):
         cases += [("fourth_function_lowered_generated", "treelstm2", session.OPT_BATCHING, 1),
                   ("fourth_function_op_by_op_fusion", "treelstm2", session.OPT_BATCHING | session.OPT_FUSION, 0)]
     for name, model, opt, lowered in cases:
+        if only and name != only:
+            continue
         app = apps.App(model, B=B, maxlen=maxlen, H=H, E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=1e-3, allow_fused=lowered)
         params = dict(w["params"])
         if model == "treelstm2":  # [U_iou | U_fl | U_fr]
@@ -361,6 +363,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-front-end", action="store_true",
                     help="skip the 'front_end' field (the step through Session::Run in its three execution modes)")
+    ap.add_argument("--front-end-case", default="",
+                    help="run only this entry of 'front_end' (e.g. fourth_function_lowered_generated) and print it: the command "
+                         "behind the kernel statistics of the generated round kernels")
     ap.add_argument("--no-schedule-modes", action="store_true",
                     help="skip 'schedule_modes' (the step with the schedule built on the host / on the GPU / from the plan cache)")
     ap.add_argument("--host-feeds", action="store_true",
@@ -381,6 +386,9 @@ def main():
     import torch
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
+    if a.front_end_case:
+        print(json.dumps({"front_end": front_end_modes(make_pool(a.workload, a.pool), only=a.front_end_case)}))
+        return
     res, w0 = measure(a, a.workload, a.steps, a.warmup, a.pool)
     out = {
         "metric": "train samples/sec (fwd+bwd) Tree-LSTM h=512 bs=64; % HBM/MFMA peak",
