@@ -22,7 +22,7 @@ constexpr int kFusedBlock = 256;
 // A vertex function's generated round kernels: one module, its kernels by a fixed order of names.
 constexpr int kCellKernels = 8;
 const char *const kCellKernelNames[kCellKernels] = {"cell_fwd",       "cell_leaves", "cell_bwd",       "cell_bwd_rows",
-                                                    "cell_transpose", "cell_bias",   "cell_bwd_gates", "cell_bwd_pool"};
+                                                    "cell_pack",      "cell_bias",   "cell_bwd_gates", "cell_bwd_pool"};
 struct CellModule {
   hipModule_t module = nullptr;
   hipFunction_t fn[kCellKernels] = {};

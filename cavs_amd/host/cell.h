@@ -69,6 +69,18 @@ struct CellSpec {
     for (const CellProduct &p : products) n += (int)p.terms.size();
     return n;
   }
+  // the distinct H x H weight blocks the terms read (a block may serve several terms)
+  int blocks() const {
+    std::vector<long> seen;  // (param, ldb, first element) triples
+    for (const CellProduct &p : products)
+      for (const CellTerm &t : p.terms) {
+        const long key[3] = {p.B.param, p.ldb, p.B.offset + t.brow * p.ldb + p.col};
+        bool found = false;
+        for (size_t i = 0; i + 2 < seen.size() && !found; i += 3) found = seen[i] == key[0] && seen[i + 1] == key[1] && seen[i + 2] == key[2];
+        if (!found) seen.insert(seen.end(), key, key + 3);
+      }
+    return (int)(seen.size() / 3);
+  }
 };
 
 // Order of the 8-byte argument slots of the generated kernels (struct CellArgs in their source).
@@ -86,7 +98,7 @@ enum CellArg {
   CA_D,          // float*  [N, ND*H]
   CA_DS,         // float*  [N, S*H] elementwise part of a vertex's message gradient by slab row; or, for
                  //         cell_bwd_gates / cell_bwd_pool, [K * n, S*H] by row of the round and child
-  CA_BT,         // float*  transposed H x H blocks of the products' terms
+  CA_BT,         // float*  tile-major copies of the weight blocks: as they are, then transposed
   CA_COLSUM,     // float*  [ND*H] column sums of D
   CA_DPOOL,      // float*  gradient of the message pool [*, S*H] (batches whose message flow is no forest)
   CA_X,          // float*  the vertex input by vertex id [*, XD*H]
@@ -98,7 +110,7 @@ enum CellArg {
 };
 
 // kernels of a compiled cell, in the order cavs_cell_compile looks them up
-enum CellKernel { CK_FWD = 0, CK_LEAVES, CK_BWD, CK_BWD_ROWS, CK_TRANSPOSE, CK_BIAS, CK_BWD_GATES, CK_BWD_POOL, CK_COUNT };
+enum CellKernel { CK_FWD = 0, CK_LEAVES, CK_BWD, CK_BWD_ROWS, CK_PACK, CK_BIAS, CK_BWD_GATES, CK_BWD_POOL, CK_COUNT };
 
 }  // namespace cavs
 #endif

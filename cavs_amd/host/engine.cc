@@ -394,7 +394,7 @@ void Engine::reserve_edges() {
     R(hlr_, cap * c.asrc.size() * H);                 // the products' left operands by slab row
     R(dxW_, cap * c.ND * H);                          // the gradient rows
     R(dc_, cap * mw);                                 // elementwise part of the message gradients
-    R(UT_, (size_t)c.terms() * H * H);
+    R(UT_, (size_t)2 * c.blocks() * H * H);  // the weight blocks tile-major, as they are and transposed
     R(cell_colsum_, (size_t)c.ND * H);
   } else if (cfg_.model != CAVS_MODEL_TREEFC) {
     R(xs_, cap);
@@ -1709,6 +1709,12 @@ void Engine::cell_forward() {
     c_launches_ += 1;
   }
   out_folded_ = true;  // the rounds write the pushed value by vertex id themselves
+  {
+    // the weights may have changed since the last step (the caller's optimizer writes them): both
+    // tile-major copies are rewritten, a few microseconds
+    ProfScope ps(this, K_OTHER);
+    cell_launch(CK_PACK, (unsigned)(((size_t)2 * c.blocks() * H * H / 4 + 255) / 256), 1, 1, 256, 0, 0, nullptr, fwd_out_);
+  }
   const unsigned block = 64u * c.waves;
   for (const Round &r : sched_->rounds) {
     if (leaf_round(r)) {
@@ -1741,16 +1747,13 @@ void Engine::cell_backward() {
         c_launches_ += 1;
       }
   }
-  {
-    // the transposed weight blocks and, when every message is read exactly once, the elementwise
-    // part of the vertices without a reader: one launch
-    ProfScope ps(this, K_OTHER);
-    const unsigned tiles = (unsigned)c.terms() * (H / 32) * (H / 32);
-    const long rows = forest_ ? n_orphans_ : 0;
-    cell_launch(CK_TRANSPOSE, tiles + (unsigned)((rows * H + 255) / 256), 1, 1, 256, tiles, rows, d_orphans_, d_dgo_);
-  }
   if (forest_) {
-    // a round's launch hands d(state) on to the children of its rows and runs their elementwise part at once
+    // every message is read exactly once: a round's launch hands d(state) on to the children of its
+    // rows and runs their elementwise part at once; the vertices without a reader go first
+    if (n_orphans_ > 0) {
+      ProfScope ps(this, K_GATES);
+      cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
+    }
     for (int k : sched_->bwd_rounds) {
       const Round &r = sched_->rounds[k];
       c_gather_rows_ += r.n;

@@ -519,7 +519,7 @@ struct Writer {
   }
 
   void product_loops() {
-    const int H = s.H, NT = s.terms(), NP = (int)s.products.size(), NA = (int)s.asrc.size();
+    const int H = s.H, NP = (int)s.products.size(), NA = (int)s.asrc.size();
     // biases and the saved left operands
     o << "static __device__ inline void cell_load_bias(const CellArgs &a, int j, FwdIn &in) {\n";
     for (size_t i = 0; i < s.biases.size(); i++) o << "  in.bias[" << i << "] = " << param_ptr(s.biases[i].ref) << "[j];\n";
@@ -544,36 +544,42 @@ struct Writer {
       o << "  }\n";
     }
     o << "}\n";
-    // forward: B pointers, fragments, MFMAs
-    o << "static __device__ inline void cell_bptrs(const CellArgs &a, int slot, int jx, const float *(&bp)[CELL_NT]) {\n";
-    int t = 0;
-    std::vector<int> term_ld;
+    // The weight blocks the terms read, each once (a block may serve several terms).  The round
+    // kernels read them from two tile-major copies that cell_pack writes before the forward rounds
+    // (for k-group g of 16 k and column tile t of 16 columns, 256 floats hold B[16g + 4s + c][16t + x]
+    // at [s][x][c]: a lane's four k are one 16-byte load and a wavefront's fragment one contiguous
+    // kilobyte): the blocks as they are for the forward products, transposed for the backward ones.
+    struct Blk {
+      int param, ldb;
+      long at;
+    };
+    std::vector<Blk> blks;
+    std::vector<int> term_blk;
     for (const CellProduct &p : s.products)
       for (const CellTerm &tm : p.terms) {
-        o << "  bp[" << t << "] = " << param_ptr(p.B) << " + (long)(" << tm.brow << " + 4 * slot) * " << p.ldb << " + " << p.col << " + jx;\n";
-        term_ld.push_back(p.ldb);
-        t++;
+        const Blk b{p.B.param, p.ldb, p.B.offset + tm.brow * p.ldb + p.col};
+        size_t q = 0;
+        while (q < blks.size() && !(blks[q].param == b.param && blks[q].ldb == b.ldb && blks[q].at == b.at)) q++;
+        if (q == blks.size()) blks.push_back(b);
+        term_blk.push_back((int)q);
       }
-    o << "}\n";
-    o << "static __device__ inline const float *cell_term_block(const CellArgs &a, int t) {\n  switch (t) {\n";
-    t = 0;
-    for (const CellProduct &p : s.products)
-      for (const CellTerm &tm : p.terms) {
-        o << "    case " << t << ": return " << param_ptr(p.B) << " + " << tm.brow * p.ldb + p.col << "L;\n";
-        t++;
-      }
+    const int NBK = (int)blks.size();
+    o << "#define CELL_NBK " << NBK << "\n";
+    o << "static __device__ inline const float *cell_block(const CellArgs &a, int q) {\n  switch (q) {\n";
+    for (int q = 0; q < NBK; q++) o << "    case " << q << ": return a.p[" << blks[q].param << "] + " << blks[q].at << "L;\n";
     o << "  }\n  return nullptr;\n}\n";
-    o << "static __device__ inline int cell_term_ld(int t) {\n  switch (t) {\n";
-    for (int q = 0; q < NT; q++) o << "    case " << q << ": return " << term_ld[q] << ";\n";
+    o << "static __device__ inline int cell_block_ld(int q) {\n  switch (q) {\n";
+    for (int q = 0; q < NBK; q++) o << "    case " << q << ": return " << blks[q].ldb << ";\n";
     o << "  }\n  return 0;\n}\n";
     // which (child, block) rows the left operands read
     std::set<std::pair<int, int>> raw;
     for (const CellASrc &a : s.asrc)
       for (int k = 0; k < s.K; k++)
         if (a.mask >> k & 1) raw.insert({k, a.block});
-    o << "struct FFrag { f4 a[" << NA << "]; float b[" << NT << "][4]; };\n";
+    const long kstep = (long)(H / 16) * 256;  // floats between the tiles of consecutive k-groups
+    o << "struct FFrag { f4 a[" << NA << "], b[" << NBK << "]; };\n";
     o << "static __device__ inline void cell_ffetch(FFrag &f, const float *const (&crow)[CELL_K], const bool (&has)[CELL_K], "
-         "const float *const (&bp)[CELL_NT], int kk) {\n  const f4 z = {0.f, 0.f, 0.f, 0.f};\n";
+         "const float *bpk, int kk) {\n  const f4 z = {0.f, 0.f, 0.f, 0.f};\n";
     for (auto &kb : raw)
       o << "  const f4 r" << kb.first << "_" << kb.second << " = has[" << kb.first << "] ? ld4(crow[" << kb.first << "] + "
         << (long)kb.second * H << " + kk) : z;\n";
@@ -586,14 +592,13 @@ struct Writer {
         }
       o << "  f.a[" << q << "] = " << e << ";\n";
     }
-    o << "#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
-    for (int q = 0; q < NT; q++) o << "    f.b[" << q << "][c] = bp[" << q << "][(long)(kk + c) * " << term_ld[q] << "];\n";
-    o << "  }\n}\n";
+    for (int q = 0; q < NBK; q++) o << "  f.b[" << q << "] = ld4(bpk + " << (long)q * H * H << "L + (long)(kk >> 4) * " << kstep << ");\n";
+    o << "}\n";
     o << "static __device__ inline void cell_fmma(const FFrag &f, f4 (&acc)[CELL_NP]) {\n#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
-    t = 0;
+    int t = 0;
     for (int p = 0; p < NP; p++)
       for (const CellTerm &tm : s.products[p].terms) {
-        o << "    acc[" << p << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << tm.asrc << "][c], f.b[" << t << "][c], acc[" << p
+        o << "    acc[" << p << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << tm.asrc << "][c], f.b[" << term_blk[t] << "][c], acc[" << p
           << "], 0, 0, 0);\n";
         t++;
       }
@@ -602,18 +607,17 @@ struct Writer {
     std::vector<int> dcols;
     for (const CellProduct &p : s.products)
       if (std::find(dcols.begin(), dcols.end(), p.dcol) == dcols.end()) dcols.push_back(p.dcol);
-    o << "struct BFrag { f4 a[" << dcols.size() << "]; float b[" << NT << "][4]; };\n";
-    o << "static __device__ inline void cell_bfetch(BFrag &f, const float *drow, const float *bt, int kk) {\n";
+    o << "struct BFrag { f4 a[" << dcols.size() << "], b[" << NBK << "]; };\n";
+    o << "static __device__ inline void cell_bfetch(BFrag &f, const float *drow, const float *btk, int kk) {\n";
     for (size_t q = 0; q < dcols.size(); q++) o << "  f.a[" << q << "] = ld4(drow + " << (long)dcols[q] * H << " + kk);\n";
-    o << "#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
-    for (int q = 0; q < NT; q++) o << "    f.b[" << q << "][c] = bt[" << (long)q * H * H << "L + (long)(kk + c) * " << H << "];\n";
-    o << "  }\n}\n";
+    for (int q = 0; q < NBK; q++) o << "  f.b[" << q << "] = ld4(btk + " << (long)q * H * H << "L + (long)(kk >> 4) * " << kstep << ");\n";
+    o << "}\n";
     o << "static __device__ inline void cell_bmma(const BFrag &f, f4 (&acc)[CELL_NA]) {\n#pragma unroll\n  for (int c = 0; c < 4; c++) {\n";
     t = 0;
     for (int p = 0; p < NP; p++) {
       const int ai = (int)(std::find(dcols.begin(), dcols.end(), s.products[p].dcol) - dcols.begin());
       for (const CellTerm &tm : s.products[p].terms) {
-        o << "    acc[" << tm.asrc << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << ai << "][c], f.b[" << t << "][c], acc[" << tm.asrc
+        o << "    acc[" << tm.asrc << "] = __builtin_amdgcn_mfma_f32_16x16x4f32(f.a[" << ai << "][c], f.b[" << term_blk[t] << "][c], acc[" << tm.asrc
           << "], 0, 0, 0);\n";
         t++;
       }

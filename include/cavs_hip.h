@@ -599,7 +599,7 @@ int cavs_fused_release(void *handle);
  * fuses the elementwise operators of F into generated kernels, cavs/midend/runtime_compiler/
  * code_generator.cc:104-185, and runs them through cavs/backend/op_impl_fused_kernel.cu:34-64; here
  * the products of F are inside the generated kernels too).  `source` defines the extern "C" kernels
- * cell_fwd, cell_leaves, cell_bwd, cell_bwd_rows, cell_transpose, cell_bias, cell_bwd_gates and
+ * cell_fwd, cell_leaves, cell_bwd, cell_bwd_rows, cell_pack, cell_bias, cell_bwd_gates and
  * cell_bwd_pool, each taking one
  * struct of 8-byte slots by value; cavs_cell_launch passes `args` as that struct.  kernel: index in
  * the order of the names above; block: threads per workgroup (a multiple of 64, at most 256). */
