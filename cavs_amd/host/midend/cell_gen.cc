@@ -580,9 +580,10 @@ struct Writer {
     o << "struct FFrag { f4 a[" << NA << "], b[" << NBK << "]; };\n";
     o << "static __device__ inline void cell_ffetch(FFrag &f, const float *const (&crow)[CELL_K], const bool (&has)[CELL_K], "
          "const float *bpk, int kk) {\n  const f4 z = {0.f, 0.f, 0.f, 0.f};\n";
+    // (a missing child reads row 0 of the pool and is masked afterwards: the loads are unconditional)
     for (auto &kb : raw)
-      o << "  const f4 r" << kb.first << "_" << kb.second << " = has[" << kb.first << "] ? ld4(crow[" << kb.first << "] + "
-        << (long)kb.second * H << " + kk) : z;\n";
+      o << "  f4 r" << kb.first << "_" << kb.second << " = ld4(crow[" << kb.first << "] + " << (long)kb.second * H << " + kk);\n"
+        << "  r" << kb.first << "_" << kb.second << " = has[" << kb.first << "] ? r" << kb.first << "_" << kb.second << " : z;\n";
     for (int q = 0; q < NA; q++) {
       std::string e;
       for (int k = 0; k < s.K; k++)
