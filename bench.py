@@ -128,6 +128,8 @@ def front_end_modes(pool, steps=60, warmup=30, only=None):
             continue
         app = apps.App(model, B=B, maxlen=maxlen, H=H, E=w["E"], V=w["V"], C_=w["C"], opt=opt, lr=1e-3, allow_fused=lowered)
         params = dict(w["params"])
+        if model == "treefc":  # (the reference's Tree-FC app has the one weight matrix)
+            params = {"W": params["W"]}
         if model == "treelstm2":  # [U_iou | U_fl | U_fr]
             params["U"] = np.concatenate([np.ravel(params["U"]), synth.SplitMix64(9).bulk_uniform(H * H, -0.1, 0.1)]).astype(np.float32)
         app.set_params(params)
