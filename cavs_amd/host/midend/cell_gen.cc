@@ -172,8 +172,15 @@ struct Reader {
   void read() {
     if (!func) no("no vertex function");
     CellSpec &s = spec;
-    for (auto &n : func->nodes)
-      if (n->def.name() == "Push") s.H = (int)n->in[0]->width();
+    int pushes = 0, scatters = 0;
+    for (auto &n : func->nodes) {
+      if (n->def.name() == "Push") {
+        s.H = (int)n->in[0]->width();
+        pushes++;
+      }
+      scatters += n->def.name() == "Scatter";
+    }
+    if (pushes != 1 || scatters != 1) no("F must end in one Scatter and one Push");
     if (s.H <= 0 || s.H % 32) no("the pushed value's width is not a multiple of 32");
     const int H = s.H;
     for (auto &np : func->nodes) {
