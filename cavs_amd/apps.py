@@ -31,6 +31,8 @@ def libs():
         a.cavs_app_read_param.restype = C.c_long
         a.cavs_app_read.argtypes = [C.c_char_p, C.c_void_p, C.c_size_t]
         a.cavs_app_read.restype = C.c_long
+        a.cavs_app_var_size.argtypes = [C.c_char_p]
+        a.cavs_app_var_size.restype = C.c_long
         _host.C_DumpGraph.restype = C.c_size_t
         _host.C_DumpGraph.argtypes = [C.c_char_p, C.c_size_t]
         _host.C_DumpFusedGraph.restype = C.c_size_t
@@ -41,7 +43,7 @@ def libs():
 
 
 class App:
-    """model: treelstm | lstm | treefc | treefc_x | treelstm2 | treegate.  opt: OPT_* bitmask, or -1 to only
+    """model: treelstm | lstm | treefc | treefc_x | treelstm2 | treegate | cell<seed>.  opt: OPT_* bitmask, or -1 to only
     declare the program (no device)."""
 
     def __init__(self, model, *, B, maxlen, H, E=0, V=0, C_=0, opt=session.OPT_BATCHING, lr=0.0, clip=0.0,
@@ -120,6 +122,14 @@ class App:
         if n != out.size:
             raise hip.CavsError(f"read_param({name}) -> {n}, expected {out.size}")
         return out
+
+    def var_size(self, name):
+        """Element count of a parameter (the seeded cell<seed> family sizes its weights by the seed)."""
+        a, _ = libs()
+        n = a.cavs_app_var_size(name.encode())
+        if n < 0:
+            raise hip.CavsError(f"var_size({name}) -> {n}")
+        return int(n)
 
     def read(self, edge, n):
         a, _ = libs()

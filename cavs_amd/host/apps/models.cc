@@ -228,6 +228,76 @@ class TreeFC : public GraphSupport {
   int H, variant_;
 };
 
+// A family of vertex functions of the general one-stage shape, one per seed, for testing the
+// lowering onto generated kernels beyond the handful of named cells: one or two children, one or
+// two state blocks, three or four gates, each gate with its own recurrent weights applied to the
+// first child's h, the last child's h, the sum or the concatenation of the children's h, sigmoid
+// or tanh per gate.  Every tensor that is used more than once goes through Mirror().
+class RandomCell : public GraphSupport {
+ public:
+  RandomCell(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d, unsigned seed)
+      : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H), K(1 + (seed & 1)), S(1 + ((seed >> 1) & 1)), NG(3 + ((seed >> 2) & 1)) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {NG * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    int usize = 0;
+    for (int g = 0; g < NG; g++) {
+      src[g] = (seed >> (3 + 2 * g)) & 3;
+      tanh_[g] = (seed >> (11 + g)) & 1;
+      rows[g] = (src[g] == 3 && K == 2) ? 2 * H : H;
+      usize += rows[g] * H;
+    }
+    U = Sym::Variable(DT_FLOAT, {usize}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {NG * H}, Sym::Zeros());
+    int at = 0;
+    for (int g = 0; g < NG; g++) {
+      Ug[g] = U.Slice(at, rows[g] * H).Reshape({rows[g], H});
+      bg[g] = B.Slice(g * H, H);
+      at += rows[g] * H;
+    }
+  }
+  void Node() override {
+    Sym h[2], c[2];
+    for (int k = 0; k < K; k++) {
+      if (S == 2) tie(h[k], c[k]) = Gather(k, {2 * H}).Split2();
+      else h[k] = Gather(k, {H});
+    }
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, NG * H}).Mirror()).Reshape({NG * H});
+    Sym gate[4];
+    for (int g = 0; g < NG; g++) {
+      Sym a;
+      if (K == 1 || src[g] == 0) a = h[0].Mirror();
+      else if (src[g] == 1) a = h[1].Mirror();
+      else if (src[g] == 2) a = h[0].Mirror() + h[1].Mirror();
+      else a = Sym::Concat({h[0].Mirror(), h[1].Mirror()});
+      Sym pre = xW.Slice(g * H, H) + Sym::MatMul(a.Reshape({1, rows[g]}), Ug[g].Mirror()).Reshape({H}) + bg[g].Mirror();
+      gate[g] = tanh_[g] ? pre.Tanh() : pre.Sigmoid();
+    }
+    Sym hn;
+    if (S == 2) {
+      Sym cn = gate[0].Mirror() * gate[1].Mirror() + gate[2].Mirror() * c[0].Mirror();
+      if (K == 2) cn = cn + gate[NG - 1].Mirror() * c[1].Mirror();
+      hn = gate[1].Mirror() * Sym::Tanh(cn.Mirror());
+      if (NG == 4 && K == 1) hn = hn + gate[3].Mirror() * gate[0].Mirror();
+      Scatter(Sym::Concat({hn.Mirror(), cn.Mirror()}));
+    } else {
+      hn = gate[0].Mirror() * gate[1].Mirror() + gate[2].Mirror() * h[0].Mirror();
+      if (K == 2) hn = hn - gate[NG - 1].Mirror() * h[1].Mirror();
+      else if (NG == 4) hn = hn + gate[3].Mirror();
+      Scatter(hn.Mirror());
+    }
+    Push(hn.Mirror());
+  }
+  Sym embedding, W, U, B;
+  int children() const { return K; }
+
+ private:
+  int E, H, K, S, NG;
+  int src[4], tanh_[4], rows[4];
+  Sym Ug[4], bg[4];
+};
+
 struct App {
   Dims d{};
   std::string model;
@@ -279,6 +349,10 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model == "treegate") {
       auto *m = new TreeGate(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model.rfind("cell", 0) == 0) {
+      auto *m = new RandomCell(app->graph, app->vertex, d, (unsigned)std::stoul(app->model.substr(4)));
       app->gs.reset(m);
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model == "lstm") {
@@ -397,6 +471,18 @@ long cavs_app_read_param(const char *name, int grad, float *out, size_t cap) {
 long cavs_app_read(const char *edge, float *out, size_t cap) {
   if (!g_app) return -1;
   return C_ReadTensor(g_app->sess->handle(), edge, out, cap);
+}
+
+// element count of a parameter by oracle name (the cells of the seeded family size theirs by the seed)
+long cavs_app_var_size(const char *name) {
+  if (!g_app) return -1;
+  for (auto &v : g_app->vars)
+    if (v.first == name) {
+      long n = 1;
+      for (int d : v.second.shape(0)) n *= d;
+      return n;
+    }
+  return -3;
 }
 
 int cavs_app_uses_fused_path(void) { return g_app ? g_app->sess->FusedPathKind() : 0; }

@@ -43,7 +43,12 @@ void bwd(const double *in, double *out) { BwdIn i; BwdOut o; memcpy(&i, in, size
 """
 
 
-@pytest.mark.parametrize("model", ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"])
+# the seeded family cell<seed> (cavs_amd/host/apps/models.cc: RandomCell): bits 0-2 choose the number of
+# children, state blocks and gates, the higher ones each gate's left operand and activation
+CELL_SEEDS = [(i & 7) | (((i * 2654435761) >> 7 & 0x1FFF) << 3) for i in range(16)]
+
+
+@pytest.mark.parametrize("model", ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"] + [f"cell{s}" for s in CELL_SEEDS])
 def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, tmp_path):
     a = _declare(model)
     src = _dump(0)

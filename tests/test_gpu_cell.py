@@ -7,6 +7,7 @@ import pytest
 
 import textbook
 from cavs_amd import apps, session, synth
+from test_cell_lowering import CELL_SEEDS
 from test_oracle_models import small_workload
 from tolerance import close
 
@@ -106,6 +107,37 @@ def test_a_gated_cell_with_one_state_block_against_fp64_autograd():
         assert got[3] == 2
         compare(got, want)
     compare(run_generated("treegate", w, "rowid", mode=0), want)
+
+
+@pytest.mark.parametrize("seed", CELL_SEEDS)
+def test_a_family_of_cells_lowered_and_op_by_op(seed):
+    """cell<seed>: one or two children, one or two state blocks, three or four gates over the first
+    child, the last child, the children's sum or their concatenation, sigmoid or tanh each.  No
+    restatement of these exists anywhere else: the generated kernels are held to the same program
+    run operator by operator (each operator of which the oracle pins), and the two backward forms
+    to each other."""
+    two = seed & 1
+    H, E, V, C_ = 64, 12, 29, 5
+    w = small_workload("treelstm" if two else "lstm", 190 + seed % 7, B=6, H=H, E=E, V=V, C=C_)
+    w = dict(w, E=E)  # (the chain workload sets E = H for its own model)
+    B, maxlen = w["graph"].shape
+    rng = synth.SplitMix64(seed)
+    res = {}
+    for mode in (1, 3, 0):
+        a = apps.App(f"cell{seed}", B=B, maxlen=maxlen, H=H, E=E, V=V, C_=C_, opt=session.OPT_BATCHING, lr=0.0, pairing="rowid",
+                     allow_fused=mode)
+        if mode == 1:
+            sizes = {k: a.var_size(k) for k in ("Emb", "W", "U", "Bv")}
+            p = {k: rng.bulk_uniform(n, -0.4, 0.4) for k, n in sizes.items()}
+            p["Wfc"], p["bfc"] = w["params"]["Wfc"], w["params"]["bfc"]
+        a.set_params(p)
+        print(f"[case] cell{seed} children={1 + two} N={w['N']} lowering mode={mode}", flush=True)
+        loss, go = a.step(w["graph"], w["x"], w["labels"], train=True)
+        assert a.fused_kind == (2 if mode else 0)
+        res[mode] = dict(loss=loss, graph_out=go, grads={"d" + k: a.grad(k, (np.size(v),)) for k, v in p.items()})
+        a.close()
+    for mode in (1, 3):
+        compare((res[mode]["loss"], res[mode]["graph_out"], res[mode]["grads"], 2), res[0])
 
 
 def test_training_steps_on_generated_kernels_update_variables_like_the_oracle(oracle):
