@@ -4,6 +4,8 @@
 // one the reference's generator emits and is valid HIP as is.
 #include <hip/hiprtc.h>
 
+#include <map>
+#include <mutex>
 #include <string>
 #include <vector>
 
@@ -26,7 +28,21 @@ const char *const kCellKernelNames[kCellKernels] = {"cell_fwd",       "cell_leav
 struct CellModule {
   hipModule_t module = nullptr;
   hipFunction_t fn[kCellKernels] = {};
+  int users = 0;
+  std::string source;
 };
+// Compiled modules by source: sessions that declare the same vertex function, at the same time or
+// one after the other, share one (a compile is about a second).  Guarded by a mutex; a module
+// without users stays loaded until more than kCellModulesKept are.
+constexpr size_t kCellModulesKept = 32;
+std::mutex &cell_mutex() {
+  static std::mutex m;
+  return m;
+}
+std::map<std::string, CellModule *> &cell_modules() {
+  static std::map<std::string, CellModule *> m;
+  return m;
+}
 
 // compiles `source` for gfx950 into `code`; the log of a failed compile goes into the error text
 int rtc_compile(const char *what, const char *source, std::vector<char> *code) {
@@ -127,6 +143,13 @@ int cavs_fused_release(void *handle) {
 int cavs_cell_compile(const char *source, void **handle) {
   CAVS_REQUIRE(source && handle, "cavs_cell_compile: null argument");
   *handle = nullptr;
+  std::lock_guard<std::mutex> lock(cell_mutex());
+  auto it = cell_modules().find(source);
+  if (it != cell_modules().end()) {
+    it->second->users++;
+    *handle = it->second;
+    return CAVS_OK;
+  }
   std::vector<char> code;
   if (int rc = rtc_compile("cell", source, &code)) return rc;
   CellModule *m = new CellModule;
@@ -137,6 +160,9 @@ int cavs_cell_compile(const char *source, void **handle) {
     delete m;
     return set_error(CAVS_EHIP, "loading the generated round kernels: %s", hipGetErrorString(e));
   }
+  m->users = 1;
+  m->source = source;
+  cell_modules()[m->source] = m;
   *handle = m;
   return CAVS_OK;
 }
@@ -167,6 +193,9 @@ int cavs_cell_launch(void *handle, int kernel, unsigned grid_x, unsigned grid_y,
 int cavs_cell_release(void *handle) {
   if (!handle) return CAVS_OK;
   CellModule *m = static_cast<CellModule *>(handle);
+  std::lock_guard<std::mutex> lock(cell_mutex());
+  if (--m->users > 0 || cell_modules().size() <= kCellModulesKept) return CAVS_OK;
+  cell_modules().erase(m->source);
   hipError_t e = hipModuleUnload(m->module);
   delete m;
   CAVS_HIP_TRY(e);
