@@ -62,8 +62,7 @@ struct CellSpec {
   int ND = 0;                   // blocks of a vertex's gradient row: d(x*W) blocks first, in order
   int NSV = 0;                  // blocks a vertex saves for the backward pass
   int waves = 0;                // wavefronts per workgroup of the round kernels (they split the k range)
-  std::string source;           // the kernels
-  std::string key;              // canonical text of the function (equal keys: equal kernels)
+  std::string source;           // the kernels (equal sources share a compiled module)
   int terms() const {
     int n = 0;
     for (const CellProduct &p : products) n += (int)p.terms.size();

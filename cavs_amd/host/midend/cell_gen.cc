@@ -694,8 +694,6 @@ std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
     w.product_loops();
     w.o << kTemplate;
     s.source = w.o.str();
-    // what decides the kernels, for sharing compiled modules between sessions
-    s.key = s.source;
     auto m = std::make_unique<CellMatch>();
     m->spec = std::make_shared<CellSpec>(s);
     m->roles = b.reader.roles;

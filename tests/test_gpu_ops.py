@@ -783,6 +783,45 @@ extern "C" __global__ void FusedKernel_1(float *S, float *Y, const float *X, con
         hip.call("cavs_fused_compile", b"k", b"this is not a kernel", C.byref(bad))
 
 
+def test_generated_cell_module_interface(g):
+    """cavs_cell_compile / cavs_cell_launch: a module that defines the eight kernels by name, each
+    taking one struct of 8-byte slots by value; the bytes passed are the struct.  A stand-in source
+    whose kernels write what they were given."""
+    names = ["cell_fwd", "cell_leaves", "cell_bwd", "cell_bwd_rows", "cell_pack", "cell_bias", "cell_bwd_gates", "cell_bwd_pool"]
+    src = "struct Args { float *out; long a, b; };\n" + "".join(
+        f'extern "C" __global__ void {n}(Args s) {{ if (threadIdx.x == 0) s.out[{k} * 8 + blockIdx.x + 2 * blockIdx.y] = '
+        f'{k} * 1000.f + s.a * 10.f + s.b + blockDim.x / 64; }}\n' for k, n in enumerate(names))
+    h = C.c_void_p()
+    hip.call("cavs_cell_compile", src.encode(), C.byref(h))
+    h2 = C.c_void_p()
+    hip.call("cavs_cell_compile", src.encode(), C.byref(h2))  # the same source: the same module
+    assert h2.value == h.value
+    out = g.zeros(64)
+
+    class Args(C.Structure):
+        _fields_ = [("out", C.c_void_p), ("a", C.c_long), ("b", C.c_long)]
+
+    for k in range(len(names)):
+        a = Args(g.P(out), 3 + k, 5)
+        hip.call("cavs_cell_launch", h, k, 2, 2, 1, 64 * (1 + k % 4), C.byref(a), C.sizeof(a), g.stream())
+    got = g.host(out).reshape(8, 8)
+    for k in range(len(names)):
+        np.testing.assert_array_equal(got[k, :4], k * 1000 + (3 + k) * 10 + 5 + (1 + k % 4))
+    a = Args(g.P(out), 0, 0)
+    with pytest.raises(hip.CavsError, match="no kernel"):
+        hip.call("cavs_cell_launch", h, 8, 1, 1, 1, 64, C.byref(a), C.sizeof(a), g.stream())
+    with pytest.raises(hip.CavsError, match="launch shape"):
+        hip.call("cavs_cell_launch", h, 0, 1, 1, 1, 96, C.byref(a), C.sizeof(a), g.stream())
+    hip.call("cavs_cell_launch", h, 0, 0, 1, 1, 64, C.byref(a), C.sizeof(a), g.stream())  # an empty grid is no launch
+    hip.call("cavs_cell_release", h)
+    hip.call("cavs_cell_release", h2)
+    bad = C.c_void_p()
+    with pytest.raises(hip.CavsError, match="compile"):
+        hip.call("cavs_cell_compile", b"this is not a kernel", C.byref(bad))
+    with pytest.raises(hip.CavsError, match="loading"):  # compiles, but a kernel is missing
+        hip.call("cavs_cell_compile", b'extern "C" __global__ void cell_fwd(int) {}', C.byref(bad))
+
+
 @pytest.mark.parametrize("kind,seed,B,lo,hi", [("tree", 1, 1, 2, 2), ("tree", 2, 7, 2, 30), ("tree", 3, 64, 2, 56),
                                                ("chain", 4, 9, 2, 40), ("tree", 5, 40, 32, 256)])
 def test_device_frontier_matches_host_schedule_bit_exact(g, oracle, kind, seed, B, lo, hi):
