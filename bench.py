@@ -368,6 +368,7 @@ def main():
     ap.add_argument("--front-end-case", default="",
                     help="run only this entry of 'front_end' (e.g. fourth_function_lowered_generated) and print it: the command "
                          "behind the kernel statistics of the generated round kernels")
+    ap.add_argument("--front-end-steps", type=int, default=60, help="timed steps of an op-by-op front-end case (a lowered one runs five times as many)")
     ap.add_argument("--no-schedule-modes", action="store_true",
                     help="skip 'schedule_modes' (the step with the schedule built on the host / on the GPU / from the plan cache)")
     ap.add_argument("--host-feeds", action="store_true",
@@ -389,7 +390,7 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs the MI355X"
     if a.front_end_case:
-        print(json.dumps({"front_end": front_end_modes(make_pool(a.workload, a.pool), only=a.front_end_case)}))
+        print(json.dumps({"front_end": front_end_modes(make_pool(a.workload, a.pool), steps=a.front_end_steps, warmup=min(30, a.front_end_steps), only=a.front_end_case)}))
         return
     res, w0 = measure(a, a.workload, a.steps, a.warmup, a.pool)
     out = {
