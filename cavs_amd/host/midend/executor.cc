@@ -1,6 +1,7 @@
 #include "executor.h"
 
 #include <algorithm>
+#include <cstdio>
 #include <cmath>
 #include <cstring>
 
@@ -169,6 +170,18 @@ void Executor::compile() {
     }
     if (lowering_mode_ > 0 && (opt_ & OPT_BATCHING)) {
       lowering_ = match_vertex_function(g, lowering_mode_ == 1 ? 1 : 2);
+      if (lowering_ && lowering_->cell) {
+        // the generated kernels must compile (the module stays cached for the engine); if they do
+        // not, F runs operator by operator like any function that is not of the shape
+        void *module = nullptr;
+        if (cavs_cell_compile(lowering_->cell->source.c_str(), &module) != CAVS_OK) {
+          std::fprintf(stderr, "cavs: the round kernels generated for the vertex function did not compile (%s); running it operator by operator\n",
+                       cavs_last_error());
+          lowering_.reset();
+        } else {
+          cavs_cell_release(module);
+        }
+      }
       lowered_ = lowering_ != nullptr;
     }
   }
