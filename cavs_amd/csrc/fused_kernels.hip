@@ -87,6 +87,7 @@ int cavs_fused_compile(const char *kernel_name, const char *source, void **handl
   if (e != hipSuccess) {
     if (k->module) (void)hipModuleUnload(k->module);
     delete k;
+    (void)hipGetLastError();  // reported here; not left behind for the next caller of the runtime
     return set_error(CAVS_EHIP, "loading fused kernel %s: %s", kernel_name, hipGetErrorString(e));
   }
   *handle = k;
@@ -158,6 +159,7 @@ int cavs_cell_compile(const char *source, void **handle) {
   if (e != hipSuccess) {
     if (m->module) (void)hipModuleUnload(m->module);
     delete m;
+    (void)hipGetLastError();  // reported here; not left behind for the next caller of the runtime
     return set_error(CAVS_EHIP, "loading the generated round kernels: %s", hipGetErrorString(e));
   }
   m->users = 1;

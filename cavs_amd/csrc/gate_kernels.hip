@@ -54,7 +54,8 @@ __global__ void treelstm_fwd_kernel(const float *__restrict__ xW, long ld_xw,
                                     const float *__restrict__ hU, const float *__restrict__ hUf,
                                     const float *__restrict__ G, const float *__restrict__ bias,
                                     float *__restrict__ gates, float *__restrict__ msg, int n,
-                                    int H) {
+                                    int H, float *pool = nullptr, const int *__restrict__ pair = nullptr,
+                                    float *__restrict__ graph_out = nullptr, const int *__restrict__ out_rows = nullptr) {
   const int hw = H / W;
   long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= (long)n * hw) return;
@@ -89,8 +90,17 @@ __global__ void treelstm_fwd_kernel(const float *__restrict__ xW, long ld_xw,
   float *g = gates + (long)r * 6 * H + j;
   vstore<W>(g, gi); vstore<W>(g + H, go); vstore<W>(g + 2 * H, gu);
   vstore<W>(g + 3 * H, gfl); vstore<W>(g + 4 * H, gfr); vstore<W>(g + 5 * H, gtc);
-  float *m = msg + (long)r * 2 * H + j;
-  vstore<W>(m, mh); vstore<W>(m + H, mc);
+  if (msg) {
+    float *m = msg + (long)r * 2 * H + j;
+    vstore<W>(m, mh); vstore<W>(m + H, mc);
+  }
+  // Scatter and Push / FunctionPopRet folded in: the message goes to the pool row the list names,
+  // the pushed value to its row of the graph output
+  if (pool) {
+    const int dst = pair[r];
+    if (dst >= 0) { vstore<W>(pool + (long)dst * 2 * H + j, mh); vstore<W>(pool + (long)dst * 2 * H + H + j, mc); }
+  }
+  if (graph_out) vstore<W>(graph_out + (long)out_rows[r] * H + j, mh);
 }
 
 template <int W>
@@ -271,9 +281,28 @@ int cavs_treelstm_gates_fwd(const float *xW, int ld_xw, const float *hU, const f
   CAVS_REQUIRE((hU && hUf && G) || (!hU && !hUf && !G), "cavs_treelstm_gates_fwd: hU, hUf and G must be all set or all null");
   hipStream_t st = as_stream(stream);
   if (H % 4 == 0 && ld_xw % 4 == 0 && all_aligned({xW, hU, hUf, G, bias, gates, msg}))
-    launch(treelstm_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
+    launch(treelstm_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H, (float *)nullptr,
+           (const int *)nullptr, (float *)nullptr, (const int *)nullptr);
   else
-    launch(treelstm_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H);
+    launch(treelstm_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H, (float *)nullptr,
+           (const int *)nullptr, (float *)nullptr, (const int *)nullptr);
+  CAVS_LAUNCH_CHECK();
+  return CAVS_OK;
+}
+
+int cavs_treelstm_gates_fwd_scatter(const float *xW, int ld_xw, const float *hU, const float *hUf, const float *G, const float *bias,
+                                    float *gates, float *msg, float *pool, const int *pair, float *graph_out, const int *out_rows,
+                                    int n, int H, void *stream) {
+  CAVS_REQUIRE(n >= 0 && H > 0 && ld_xw >= 4 * H, "cavs_treelstm_gates_fwd_scatter: bad shape n=%d H=%d ld=%d", n, H, ld_xw);
+  if (n == 0) return CAVS_OK;
+  CAVS_REQUIRE(xW && bias && gates && pool && pair, "cavs_treelstm_gates_fwd_scatter: null pointer");
+  CAVS_REQUIRE((hU && hUf && G) || (!hU && !hUf && !G), "cavs_treelstm_gates_fwd_scatter: hU, hUf and G must be all set or all null");
+  CAVS_REQUIRE(!graph_out || out_rows, "cavs_treelstm_gates_fwd_scatter: graph_out needs out_rows");
+  hipStream_t st = as_stream(stream);
+  if (H % 4 == 0 && ld_xw % 4 == 0 && all_aligned({xW, hU, hUf, G, bias, gates, msg, pool, graph_out}))
+    launch(treelstm_fwd_kernel<4>, GATE_GRID(n, H, 4), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H, pool, pair, graph_out, out_rows);
+  else
+    launch(treelstm_fwd_kernel<1>, GATE_GRID(n, H, 1), 0, st, xW, ld_xw, hU, hUf, G, bias, gates, msg, n, H, pool, pair, graph_out, out_rows);
   CAVS_LAUNCH_CHECK();
   return CAVS_OK;
 }

@@ -96,6 +96,7 @@ _SIGS = {
     "cavs_ew_unary": [_I, _P, _P, _Z, _I, _P],
     "cavs_scale": [_P, _P, _F, _Z, _P],
     "cavs_treelstm_gates_fwd": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _P],
+    "cavs_treelstm_gates_fwd_scatter": [_P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_treelstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _P],
     "cavs_lstm_gates_fwd": [_P, _I, _P, _P, _P, _P, _P, _I, _I, _P],
     "cavs_lstm_gates_bwd": [_P, _P, _P, _P, _P, _I, _P, _I, _I, _P],

@@ -1091,8 +1091,9 @@ void Engine::treelstm_forward() {
     check(cavs_zero(G_.get(), (size_t)N * 2 * 2 * H * 4, stream_));
     check(cavs_zero(hlr_.get(), (size_t)N * H * 4, stream_));
   }
-  // when every round runs fused, Push + FunctionPopRet ride along in the rounds' epilogues
-  out_folded_ = fused > 0 && sched_->max_round <= fused && fwd_out_ != nullptr;
+  // with the fused path on, Push + FunctionPopRet ride along in the rounds' epilogues (also in the
+  // gate launch of a round that runs its products as separate GEMMs)
+  out_folded_ = fused > 0 && fwd_out_ != nullptr;
   float *go = out_folded_ ? fwd_out_ : nullptr;
   // the last rounds, a few vertices each: one launch for all of them
   const size_t tail_from = (tail_.first >= 0 && any_packed) ? (size_t)tail_.first : sched_->rounds.size();
@@ -1117,7 +1118,7 @@ void Engine::treelstm_forward() {
     // the message slab is only read back by FunctionPopRet; when the rounds write the output
     // rows themselves nobody reads it and the fused launches skip it
     float *msg = out_folded_ ? nullptr : msg_.at(off * 2 * H);
-    if (leaf_round(r) && r.n <= fused) {
+    if (leaf_round(r) && fused > 0) {  // (elementwise: a round of any size)
       CAVS_TIMED(K_GATES, cavs_treelstm_round_leaves_fwd(pool_.get(), d_pair_ + off, xW_.at(off * 4 * H), 4 * H, Bv, gates_.at(off * 6 * H),
                                                          msg, go, d_t2j_ + off, r.n, H, stream_));
       c_scatter_rows_ += r.n;
@@ -1152,6 +1153,13 @@ void Engine::treelstm_forward() {
       c_launches_ += 1;
       gemm(0, 0, r.n, 3 * H, H, hlr, H, U, 3 * H, 0.f, r_hU_.get(), 3 * H);
       gemm(0, 0, 2 * r.n, H, H, G, 2 * H, U + (size_t)3 * H * H, H, 0.f, r_hUf_.get(), H);
+      if (fused > 0) {  // the gates with Scatter and Push / PopRet folded in
+        CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd_scatter(xW_.at(off * 4 * H), 4 * H, r_hU_.get(), r_hUf_.get(), G, Bv, gates_.at(off * 6 * H),
+                                                            msg, pool_.get(), d_pair_ + off, go, d_t2j_ + off, r.n, H, stream_));
+        c_scatter_rows_ += r.n;
+        c_launches_ += 1;
+        continue;
+      }
       CAVS_TIMED(K_GATES, cavs_treelstm_gates_fwd(xW_.at(off * 4 * H), 4 * H, r_hU_.get(), r_hUf_.get(), G, Bv,
                                     gates_.at(off * 6 * H), msg, r.n, H, stream_));
     }
@@ -1164,8 +1172,8 @@ void Engine::treelstm_backward() {
   const int N = N_, H = cfg_.H, E = E_;
   const float *W = param("W").w, *U = param("U").w;
   const int fused = fused_rows();
-  // grad of Push is Pull: read through the list by the fused gate kernels, or gathered up front
-  const bool dret_folded = fused > 0 && sched_->max_round <= fused;
+  // grad of Push is Pull: read through the list by the gate kernels of the fused path, or gathered up front
+  const bool dret_folded = fused > 0;
   if (!dret_folded && !forest_) gather(dret_.get(), H, d_dgo_, H, d_t2j_, N, H);
   if (!sched_->batching) check(cavs_zero(dF_.get(), (size_t)N * 2 * H * 4, stream_));
   // one launch per round when the message flow is a forest (below); then, if every such launch has
@@ -1246,6 +1254,30 @@ void Engine::treelstm_backward() {
         c_scatter_rows_ += 2.0 * r.n;
         c_launches_ += 1;
       }
+      continue;
+    }
+    if (fused > 0) {
+      // a round too large for the fused children launch: the same gate launch (it reads the message
+      // gradient through the scatter list and hands d c on to the children's pool rows), the two
+      // products as GEMMs, and the h halves scattered
+      const bool leaf = leaf_round(r);
+      float *dxW = dxW_.at(off * 4 * H), *dF = leaf ? nullptr : dF_.at(2 * off * H);
+      CAVS_TIMED(K_GATES, cavs_treelstm_round_bwd_gates(dpool_.get(), d_pair_ + off, leaf ? nullptr : d_child_ + 2 * off, d_dgo_, d_t2j_ + off,
+                                                        gates_.at(off * 6 * H), leaf ? nullptr : G_.at(2 * off * 2 * H), dxW, 4 * H, dF, r.n, H,
+                                                        stream_));
+      c_gather_rows_ += r.n;
+      c_launches_ += 1;
+      if (leaf) continue;
+      gemm(0, 1, r.n, H, 3 * H, dxW, 4 * H, U, 3 * H, 0.f, r_dhlr_.get(), H);
+      {
+        float *ws = workspace(cavs_sgemm_splitk_workspace(2 * r.n, H, H));
+        ProfScope ps(this, K_GEMM);
+        check(cavs_sgemm_addrows(0, 1, 2 * r.n, H, H, dF, H, U + (size_t)3 * H * H, H, r_dhlr_.get(), H, 1, r_dG_.get(), 2 * H, ws,
+                                 ws_.capacity() * 4, stream_));
+      }
+      c_gemm_flops_ += 2.0 * 2 * r.n * H * H;
+      c_launches_ += 1;
+      scatter(dpool_.get(), 2 * H, d_child_ + 2 * off, r_dG_.get(), 2 * H, 2 * r.n, H);
       continue;
     }
     // grad of Scatter is Gather on the recorded scatter list; rows without an entry read zero

@@ -286,6 +286,14 @@ int cavs_scale(float *out, const float *a, float s, size_t n, void *stream); /* 
 int cavs_treelstm_gates_fwd(const float *xW, int ld_xw, const float *hU, const float *hUf,
                             const float *G, const float *bias, float *gates, float *msg,
                             int n, int H, void *stream);
+/* The same with the Scatter that follows it (cavs/backend/op_impl_graphop.cu:128-190) and Push /
+ * FunctionPopRet (:214-318) folded in, for rounds that run their products as separate GEMMs: the
+ * message of row r also goes to row pair[r] of the message pool (-1: nowhere) and, if graph_out is
+ * given, its h to row out_rows[r] of the graph output.  msg may be NULL then. */
+int cavs_treelstm_gates_fwd_scatter(const float *xW, int ld_xw, const float *hU, const float *hUf,
+                                    const float *G, const float *bias, float *gates, float *msg,
+                                    float *pool, const int *pair, float *graph_out,
+                                    const int *out_rows, int n, int H, void *stream);
 /* dmsg [n,2H] gathered-back message gradient, dret [n,H] pulled d GraphOutput.
  * Writes dxW [n,4H] (ld_dxw) = [d_i|d_o|d_u|d_fl+d_fr]; for internal rounds also
  * dF [2n,H] = rows (d_fl, d_fr) and the c half of dG [2n,2H] (dc_l, dc_r); pass

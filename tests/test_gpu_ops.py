@@ -535,6 +535,27 @@ def test_treelstm_gates(g, oracle, n, H):
            g.P(gates), g.P(msg), n, H, g.stream())
     close(g.host(gates), gates_l, "leaf gates")
     close(g.host(msg), msg_l, "leaf msg")
+    # the same launch with Scatter and Push / PopRet folded in: bit for bit the gates and the message,
+    # the message also in the pool rows the list names (-1: nowhere), its h in the listed output rows
+    pair = np.arange(n, dtype=np.int32)[::-1] * 2
+    pair[::3] = -1
+    out_rows = (np.arange(n, dtype=np.int32) * 5 + 1) % n if n > 1 else np.zeros(1, np.int32)
+    out_rows = np.argsort(np.argsort(out_rows, kind="stable"), kind="stable").astype(np.int32)  # a permutation
+    for with_msg in (True, False):
+        gates2, msg2, pool, go = g.zeros(n, 6 * H), g.zeros(n, 2 * H), g.zeros(2 * n, 2 * H, fill=7.0), g.zeros(n, H)
+        g.call("cavs_treelstm_gates_fwd", g.P(g.devf(xW)), 4 * H, g.P(g.devf(hU)), g.P(g.devf(hUf)), g.P(dG_), g.P(g.devf(bias)), g.P(gates),
+               g.P(msg), n, H, g.stream())
+        g.call("cavs_treelstm_gates_fwd_scatter", g.P(g.devf(xW)), 4 * H, g.P(g.devf(hU)), g.P(g.devf(hUf)), g.P(dG_), g.P(g.devf(bias)),
+               g.P(gates2), g.P(msg2) if with_msg else None, g.P(pool), g.P(g.devi(pair)), g.P(go), g.P(g.devi(out_rows)), n, H, g.stream())
+        m = g.host(msg)
+        np.testing.assert_array_equal(g.host(gates2), g.host(gates))
+        np.testing.assert_array_equal(g.host(msg2), m if with_msg else 0 * m)
+        want_pool = np.full((2 * n, 2 * H), 7.0, np.float32)
+        want_pool[pair[pair >= 0]] = m[pair >= 0]
+        np.testing.assert_array_equal(g.host(pool), want_pool)
+        want_go = np.zeros((n, H), np.float32)
+        want_go[out_rows] = m[:, :H]
+        np.testing.assert_array_equal(g.host(go), want_go)
 
     dmsg = r.bulk_normal(n * 2 * H).reshape(n, 2 * H)
     dret = r.bulk_normal(n * H).reshape(n, H)
