@@ -11,6 +11,7 @@
 #ifndef CAVS_HOST_CELL_H_
 #define CAVS_HOST_CELL_H_
 
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -51,7 +52,8 @@ struct CellParam {
 };
 
 struct CellSpec {
-  int H = 0, K = 0, S = 0;      // block width, children per vertex, state blocks per message
+  int H = 0, K = 0, S = 0;      // block width, children per vertex, state blocks of the message it writes
+  int SI = 0;                   // state blocks of the rows it gathers (the children's messages; = S for a function of one stage)
   int E = 0, V = 0, NX = 0;     // embedding width, vocabulary, blocks of x * W (0: F looks no vertex input up)
   int XD = 0;                   // H-wide blocks of the vertex input's row that F pulls and uses as they are
   CellParamRef W;               // [E, NX * H]
@@ -63,6 +65,12 @@ struct CellSpec {
   int NSV = 0;                  // blocks a vertex saves for the backward pass
   int waves = 0;                // wavefronts per workgroup of the round kernels (they split the k range)
   std::string source;           // the kernels (equal sources share a compiled module)
+  // A vertex function of several stages -- a product whose left operand depends on another product
+  // of the same vertex -- runs as a chain of such cells: every cell but the last writes, per vertex,
+  // a row of intermediate blocks (the next stage's left operands and whatever later stages read of
+  // this one), which the next cell gathers as the state of its one "child", the vertex itself.
+  std::shared_ptr<CellSpec> next;
+  bool has_ret = true;          // the last cell of a chain pushes the return value
   int terms() const {
     int n = 0;
     for (const CellProduct &p : products) n += (int)p.terms.size();
@@ -84,7 +92,7 @@ struct CellSpec {
 
 // Order of the 8-byte argument slots of the generated kernels (struct CellArgs in their source).
 enum CellArg {
-  CA_POOL = 0,   // float*  message pool [*, S*H]
+  CA_POOL = 0,   // float*  the rows this cell's state goes to [*, S*H]
   CA_CHILD,      // int*    pool rows of the children by slab row [K * N]
   CA_PAIR,       // int*    pool row a slab row's message goes to [N]
   CA_KIDS,       // int*    slab rows of the children by slab row [K * N]
@@ -95,12 +103,14 @@ enum CellArg {
   CA_ASRC,       // float*  [N, NA*H]
   CA_GO,         // float*  [N, H] by vertex id: the pushed value / its gradient
   CA_D,          // float*  [N, ND*H]
-  CA_DS,         // float*  [N, S*H] elementwise part of a vertex's message gradient by slab row; or, for
-                 //         cell_bwd_gates / cell_bwd_pool, [K * n, S*H] by row of the round and child
+  CA_DS,         // float*  [N, SI*H] elementwise part of a vertex's message gradient by slab row; or, for
+                 //         cell_bwd_gates / cell_bwd_pool, [K * n, SI*H] by row of the round and child
   CA_BT,         // float*  tile-major copies of the weight blocks: as they are, then transposed
   CA_COLSUM,     // float*  [ND*H] column sums of D
-  CA_DPOOL,      // float*  gradient of the message pool [*, S*H] (batches whose message flow is no forest)
+  CA_DPOOL,      // float*  gradient of the rows this cell's state goes to [*, S*H] (cell_bwd_gates reads it)
   CA_X,          // float*  the vertex input by vertex id [*, XD*H]
+  CA_POOL_IN,    // float*  the rows this cell gathers its children's states from [*, SI*H] (a function of one stage: CA_POOL)
+  CA_DPOOL_IN,   // float*  gradient of those rows (cell_bwd_pool writes it; a function of one stage: CA_DPOOL)
   CA_OFF,        // long    first slab row of the round
   CA_N,          // long    rows
   CA_PARAM0,     // float*  parameters, then their gradients, in CellSpec::params order

@@ -1718,6 +1718,8 @@ void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned 
   a[CA_COLSUM].p = cell_colsum_.get();
   a[CA_DPOOL].p = dpool_.get();
   a[CA_X].p = d_x_;
+  a[CA_POOL_IN].p = pool_.get();
+  a[CA_DPOOL_IN].p = dpool_.get();
   a[CA_OFF].i = off;
   a[CA_N].i = n;
   for (size_t i = 0; i < c.params.size(); i++) {

@@ -192,11 +192,11 @@ struct Reader {
         const int k = GetSingleArg<int>(d, "Child", 0);
         const long w = out->width();
         if (k < 0 || k > 1 || w % H) no("Gather of child " + std::to_string(k) + " with width " + std::to_string(w));
-        if (s.S && s.S != w / H) no("Gather widths differ");
-        s.S = (int)(w / H);
+        if (s.SI && s.SI != w / H) no("Gather widths differ");
+        s.SI = (int)(w / H);
         s.K = std::max(s.K, k + 1);
         std::vector<int> b;
-        for (int m = 0; m < s.S; m++) b.push_back(dag.make(N_CS, -1, -1, k, m));
+        for (int m = 0; m < s.SI; m++) b.push_back(dag.make(N_CS, -1, -1, k, m));
         val[out] = b;
       } else if (op == "Pull") {
         const long w = out->width();
@@ -288,8 +288,8 @@ struct Reader {
         val[out] = b;
       } else if (op == "Scatter") {
         st = blocks(n->in[0]);
-        if ((int)st.size() != s.S && s.S) no("the scattered message is not as wide as the gathered ones");
-        if (!s.S) s.S = (int)st.size();
+        s.S = (int)st.size();
+        if (s.SI && s.S != s.SI) no("the scattered message is not as wide as the gathered ones");
       } else if (op == "Push") {
         const std::vector<int> &b = blocks(n->in[0]);
         if (b.size() != 1) no("the pushed value is not H wide");
@@ -321,7 +321,7 @@ Derived derive(Reader &r) {
   const int nfwd = (int)dag.n.size();
   std::vector<std::vector<int>> adj(nfwd);
   for (int m = 0; m < s.S; m++) adj[r.st[m]].push_back(dag.make(N_DST, -1, -1, m));
-  adj[r.ret].push_back(dag.make(N_DRET));
+  if (r.ret >= 0) adj[r.ret].push_back(dag.make(N_DRET));
   std::vector<int> grad(nfwd, -1);
   for (int id = nfwd - 1; id >= 0; id--) {
     if (adj[id].empty()) continue;
@@ -366,9 +366,9 @@ Derived derive(Reader &r) {
   for (size_t p = 0; p < s.products.size(); p++) s.products[p].dcol = shared_column(input_grad(N_HU, (int)p, 0));
   for (size_t i = 0; i < s.biases.size(); i++) s.biases[i].dcol = shared_column(input_grad(N_BIAS, (int)i, 0));
   s.ND = (int)d.dcols.size();
-  d.dcs.assign(s.K, std::vector<int>(s.S, -1));
+  d.dcs.assign(s.K, std::vector<int>(s.SI, -1));
   for (int k = 0; k < s.K; k++)
-    for (int m = 0; m < s.S; m++) {
+    for (int m = 0; m < s.SI; m++) {
       d.dcs[k][m] = input_grad(N_CS, k, m);
       if (d.dcs[k][m] >= 0) d.ds_mask |= 1 << m;
     }
@@ -472,10 +472,10 @@ struct Writer {
   void elementwise(int nfwd) {
     const char *dev = device ? "static __device__ inline " : "static inline ";
     o << "struct FwdIn { float xw[" << std::max(1, s.NX) << "], hu[" << s.products.size() << "], bias[" << std::max<size_t>(1, s.biases.size())
-      << "], cs[" << s.K << "][" << s.S << "], xd[" << std::max(1, s.XD) << "]; };\n";
+      << "], cs[" << s.K << "][" << s.SI << "], xd[" << std::max(1, s.XD) << "]; };\n";
     o << "struct FwdOut { float st[" << s.S << "], ret, sv[" << std::max(1, s.NSV) << "]; };\n";
-    o << "struct BwdIn { float dst[" << s.S << "], dret, sv[" << std::max(1, s.NSV) << "], cs[" << s.K << "][" << s.S << "]; };\n";
-    o << "struct BwdOut { float d[" << s.ND << "], dcs[" << s.K << "][" << s.S << "]; };\n";
+    o << "struct BwdIn { float dst[" << s.S << "], dret, sv[" << std::max(1, s.NSV) << "], cs[" << s.K << "][" << s.SI << "]; };\n";
+    o << "struct BwdOut { float d[" << s.ND << "], dcs[" << s.K << "][" << s.SI << "]; };\n";
     if (device) {
       // exp through v_exp_f32 and the reciprocal through v_rcp_f32 (1 ulp each); saturation comes out
       // right without special cases
@@ -488,11 +488,11 @@ struct Writer {
     }
     o << dev << "void cell_forward(const FwdIn &in, FwdOut &out) {\n";
     std::vector<int> roots = r.st;
-    roots.push_back(r.ret);
+    if (r.ret >= 0) roots.push_back(r.ret);
     roots.insert(roots.end(), dv.saved.begin(), dv.saved.end());
     body(roots, false, nfwd);
     for (int m = 0; m < s.S; m++) o << "  out.st[" << m << "] = " << name(r.st[m], false, nfwd) << ";\n";
-    o << "  out.ret = " << name(r.ret, false, nfwd) << ";\n";
+    o << "  out.ret = " << (r.ret >= 0 ? name(r.ret, false, nfwd) : std::string("0.f")) << ";\n";
     for (size_t t = 0; t < dv.saved.size(); t++) o << "  out.sv[" << t << "] = " << name(dv.saved[t], false, nfwd) << ";\n";
     o << "}\n";
     o << dev << "void cell_backward(const BwdIn &in, BwdOut &out) {\n";
@@ -503,7 +503,7 @@ struct Writer {
     body(roots, true, nfwd);
     for (size_t q = 0; q < dv.dcols.size(); q++) o << "  out.d[" << q << "] = " << name(dv.dcols[q], true, nfwd) << ";\n";
     for (int k = 0; k < s.K; k++)
-      for (int m = 0; m < s.S; m++)
+      for (int m = 0; m < s.SI; m++)
         o << "  out.dcs[" << k << "][" << m << "] = " << (dv.dcs[k][m] >= 0 ? name(dv.dcs[k][m], true, nfwd) : std::string("0.f")) << ";\n";
     o << "}\n";
   }
@@ -515,12 +515,13 @@ struct Writer {
   void kernels() {
     const int H = s.H, NT = s.terms(), NP = (int)s.products.size(), NA = (int)s.asrc.size();
     o << "#define CELL_H " << H << "\n#define CELL_K " << s.K << "\n#define CELL_S " << s.S << "\n#define CELL_MW " << s.S * H
+      << "\n#define CELL_SI " << s.SI << "\n#define CELL_MWI " << s.SI * H << "\n#define CELL_HAS_RET " << (s.has_ret ? 1 : 0)
       << "\n#define CELL_NX " << s.NX << "\n#define CELL_XD " << s.XD << "\n#define CELL_NP " << NP << "\n#define CELL_NA " << NA << "\n#define CELL_NT " << NT
       << "\n#define CELL_ND " << s.ND << "\n#define CELL_NSV " << s.NSV << "\n#define CELL_KS " << s.waves << "\n#define CELL_DS_MASK "
       << dv.ds_mask << "\n#define CELL_BWD_CS " << (dv.reads_cs ? 1 : 0) << "\n";
     o << "typedef float f4 __attribute__((ext_vector_type(4)));\n";
     o << "struct CellArgs {\n  float *pool;\n  const int *child, *pair, *kids, *t2j, *rows;\n  const float *xw;\n"
-         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  const float *x;\n  long off, n;\n  float *p["
+         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  const float *x;\n  float *pool_in, *dpool_in;\n  long off, n;\n  float *p["
       << 2 * CA_MAX_PARAMS << "];\n};\n";
     o << "static __device__ inline f4 ld4(const float *p) { return *reinterpret_cast<const f4 *>(p); }\n";
   }
@@ -543,7 +544,7 @@ struct Writer {
       o << ";\n";
     }
     o << "}\n";
-    o << "static __device__ inline void cell_add_products(float (&dst)[CELL_S], const float (&s)[CELL_NA], int k) {\n";
+    o << "static __device__ inline void cell_add_products(float (&dst)[CELL_SI], const float (&s)[CELL_NA], int k) {\n";
     for (int k = 0; k < s.K; k++) {
       o << "  if (k == " << k << ") {\n";
       for (int q = 0; q < NA; q++)
