@@ -228,6 +228,48 @@ class TreeFC : public GraphSupport {
   int H, variant_;
 };
 
+// A child-sum Tree-GRU: r = sigmoid(x W_r + hs U_r + b_r), z = sigmoid(x W_z + hs U_z + b_z) with
+// hs = h_l + h_r, candidate c = tanh(x W_c + (r * hs) U_c + b_c), h = z * hs + c - z * c.  The left
+// operand of the candidate's product depends on another product of the same vertex: a function of
+// two stages.
+class TreeGRU : public GraphSupport {
+ public:
+  TreeGRU(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {3 * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    U = Sym::Variable(DT_FLOAT, {3 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {3 * H}, Sym::Zeros());
+    U_r = U.Slice(0, H * H).Reshape({H, H});
+    U_z = U.Slice(H * H, H * H).Reshape({H, H});
+    U_c = U.Slice(2 * H * H, H * H).Reshape({H, H});
+    b_r = B.Slice(0, H);
+    b_z = B.Slice(H, H);
+    b_c = B.Slice(2 * H, H);
+  }
+  void Node() override {
+    Sym h_l = Gather(0, {H});
+    Sym h_r = Gather(1, {H});
+    Sym hs = h_l + h_r;
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, 3 * H}).Mirror()).Reshape({H * 3});
+    Sym xW_r, xW_z, xW_c;
+    tie(xW_r, xW_z, xW_c) = xW.Split3();
+    Sym r = (xW_r + Sym::MatMul(hs.Mirror().Reshape({1, H}), U_r.Mirror()).Reshape({H}) + b_r.Mirror()).Sigmoid();
+    Sym z = (xW_z + Sym::MatMul(hs.Mirror().Reshape({1, H}), U_z.Mirror()).Reshape({H}) + b_z.Mirror()).Sigmoid();
+    Sym rh = r * hs.Mirror();
+    Sym c = (xW_c + Sym::MatMul(rh.Reshape({1, H}), U_c.Mirror()).Reshape({H}) + b_c.Mirror()).Tanh();
+    Sym h = z.Mirror() * hs.Mirror() + c.Mirror() - z.Mirror() * c.Mirror();
+    Scatter(h.Mirror());
+    Push(h.Mirror());
+  }
+  Sym embedding, W, U, B;
+
+ private:
+  int E, H;
+  Sym U_r, U_z, U_c, b_r, b_z, b_c;
+};
+
 // A family of vertex functions of the general one-stage shape, one per seed, for testing the
 // lowering onto generated kernels beyond the handful of named cells: one or two children, one or
 // two state blocks, three or four gates, each gate with its own recurrent weights applied to the
@@ -349,6 +391,10 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model == "treegate") {
       auto *m = new TreeGate(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model == "treegru") {
+      auto *m = new TreeGRU(app->graph, app->vertex, d);
       app->gs.reset(m);
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model.rfind("cell", 0) == 0) {

@@ -44,6 +44,7 @@ struct CellProduct {
 struct CellBias {
   CellParamRef ref;  // H values
   int dcol = -1;     // block of the gradient rows whose column sums are its gradient
+  bool add = false;  // an earlier cell of the chain reads the same bias: this cell's share is added to that one's
 };
 
 struct CellParam {
@@ -57,6 +58,7 @@ struct CellSpec {
   int E = 0, V = 0, NX = 0;     // embedding width, vocabulary, blocks of x * W (0: F looks no vertex input up)
   int XD = 0;                   // H-wide blocks of the vertex input's row that F pulls and uses as they are
   CellParamRef W;               // [E, NX * H]
+  int xw_lo = 0, xw_hi = 0;     // the blocks of x * W this cell reads: [xw_lo, xw_hi) (the gradient rows' other x * W blocks are zero)
   std::vector<CellParam> params;
   std::vector<CellASrc> asrc;
   std::vector<CellProduct> products;

@@ -39,7 +39,10 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream, std::share
     if (cell_->H != cfg.H || cell_->K < 1 || cell_->K > 2 || (int)cell_->params.size() > CA_MAX_PARAMS)
       fail(CAVS_EINVAL, "the description of the lowered vertex function does not fit the session");
     E_ = ld_e_ = cell_->E;
-    mw_ = cell_->S * cfg.H;
+    const CellSpec *tail = cell_.get();
+    while (tail->next) tail = tail->next.get();
+    if (tail->S != cell_->SI) fail(CAVS_EINVAL, "the last cell of the chain does not write what the first one gathers");
+    mw_ = tail->S * cfg.H;
     nch_ = cell_->K;
   }
   const bool reads_x = cell_ ? cell_->NX > 0 : cfg.model != CAVS_MODEL_TREEFC;
@@ -68,7 +71,11 @@ Engine::Engine(const cavs_session_config &cfg, void *external_stream, std::share
       break;
     case CAVS_MODEL_CELL:
       for (const CellParam &p : cell_->params) add_param(p.name, (size_t)p.size);
-      check(cavs_cell_compile(cell_->source.c_str(), &cell_module_));
+      for (std::shared_ptr<const CellSpec> c = cell_; c; c = c->next) {
+        cells_.emplace_back();
+        cells_.back().spec = c;
+        check(cavs_cell_compile(c->source.c_str(), &cells_.back().module));
+      }
       break;
     default:
       add_param("W", 2 * H * H);
@@ -142,7 +149,7 @@ void Engine::tail_check() {
 
 Engine::~Engine() {
   cavs_stream_sync(stream_);
-  cavs_cell_release(cell_module_);
+  for (CellStage &st : cells_) cavs_cell_release(st.module);
   for (auto &e : ev_) cavs_event_destroy(e);
   for (auto &h : hlists_) {
     if (h.free_ev) cavs_event_destroy(h.free_ev);
@@ -390,12 +397,31 @@ void Engine::reserve_edges() {
       R(de_, cap * E_);
       R(xW_, cap * c.NX * H);
     }
-    R(gates_, cap * std::max(1, c.NSV) * H);          // what a vertex keeps for the backward pass
-    R(hlr_, cap * c.asrc.size() * H);                 // the products' left operands by slab row
-    R(dxW_, cap * c.ND * H);                          // the gradient rows
-    R(dc_, cap * mw);                                 // elementwise part of the message gradients
-    R(UT_, (size_t)2 * c.blocks() * H * H);  // the weight blocks tile-major, as they are and transposed
-    R(cell_colsum_, (size_t)c.ND * H);
+    for (size_t ci = 0; ci < cells_.size(); ci++) {
+      CellStage &st = cells_[ci];
+      const CellSpec &k = *st.spec;
+      R(st.sv, cap * std::max(1, k.NSV) * H);   // what a vertex keeps for the backward pass
+      R(st.asrc, cap * k.asrc.size() * H);      // the products' left operands by slab row
+      R(st.d, cap * k.ND * H);                  // the gradient rows
+      // elementwise part of the message gradients: by slab row (one launch per backward round), or
+      // by row of the round and child (two launches)
+      R(st.ds, std::max(cells_.size() == 1 ? cap * k.SI * H : (size_t)0, rc * k.K * k.SI * H));
+      R(st.bt, (size_t)2 * k.blocks() * H * H);  // the weight blocks tile-major, as they are and transposed
+      R(st.colsum, (size_t)k.ND * H);
+      if (ci + 1 < cells_.size()) {
+        R(st.rows, cap * k.S * H);
+        R(st.drows, cap * k.S * H);
+      }
+    }
+    if (cells_.size() > 1 && cell_iota_n_ < cap) {
+      std::vector<int> iota(cap);
+      for (size_t i = 0; i < cap; i++) iota[i] = (int)i;
+      check(cavs_stream_sync(stream_));
+      cell_iota_.reserve(cap);
+      check(cavs_memcpy_h2d(cell_iota_.get(), iota.data(), cap * 4, stream_));
+      check(cavs_stream_sync(stream_));
+      cell_iota_n_ = cap;
+    }
   } else if (cfg_.model != CAVS_MODEL_TREEFC) {
     R(xs_, cap);
     if (xs_prev_.capacity() < cap) {  // the list of dirty rows does not survive a reallocation
@@ -1691,35 +1717,41 @@ void Engine::treefc_backward() {
 }
 
 // ------------------------------------------------------------------ a vertex function on generated kernels
-// The general one-stage shape (cell.h): x * W for all vertices up front, one launch per round that
-// gathers, multiplies, runs the elementwise part and scatters; backward one launch per round that
-// hands d(state) on to the children and runs their elementwise part, then the weight gradients as
-// products over all rows.  The message flow of the batch must be a forest (every message read once).
-void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go) {
-  const CellSpec &c = *cell_;
+// The general shape (cell.h): x * W for all vertices up front, then per round one launch per cell of
+// the chain (a function of one stage is a chain of one) that gathers, multiplies, runs the
+// elementwise part and scatters.  Backward, a function of one stage over a batch whose message
+// flow is a forest takes one launch per round, which hands d(state) on to the children and runs
+// their elementwise part; anything else two launches per round and cell, with the message
+// gradients going through the gradients of the rows the cells write.  Then the weight gradients as
+// products over all rows.
+void Engine::cell_launch(int ci, int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go) {
+  CellStage &st = cells_[ci];
+  const CellSpec &c = *st.spec;
+  const bool first = ci == 0, last = ci + 1 == (int)cells_.size();
   union Slot {
     const void *p;
     long long i;
   } a[CA_SLOTS];
   std::memset(a, 0, sizeof a);
-  a[CA_POOL].p = pool_.get();
-  a[CA_CHILD].p = d_child_;
-  a[CA_PAIR].p = d_pair_;
+  // a cell in the middle of a chain gathers row v of the cell before and writes row v of its own
+  a[CA_POOL].p = last ? pool_.get() : st.rows.get();
+  a[CA_PAIR].p = last ? d_pair_ : cell_iota_.get();
+  a[CA_DPOOL].p = last ? dpool_.get() : st.drows.get();
+  a[CA_POOL_IN].p = first ? pool_.get() : cells_[ci - 1].rows.get();
+  a[CA_CHILD].p = first ? d_child_ : cell_iota_.get();
+  a[CA_DPOOL_IN].p = first ? dpool_.get() : cells_[ci - 1].drows.get();
   a[CA_KIDS].p = d_kid_rows_;
   a[CA_T2J].p = d_t2j_;
   a[CA_ROWS].p = rows;
   a[CA_XW].p = xW_.get();
-  a[CA_SV].p = gates_.get();
-  a[CA_ASRC].p = hlr_.get();
+  a[CA_SV].p = st.sv.get();
+  a[CA_ASRC].p = st.asrc.get();
   a[CA_GO].p = go;
-  a[CA_D].p = dxW_.get();
-  a[CA_DS].p = forest_ ? dc_.get() : r_dG_.get();
-  a[CA_BT].p = UT_.get();
-  a[CA_COLSUM].p = cell_colsum_.get();
-  a[CA_DPOOL].p = dpool_.get();
+  a[CA_D].p = st.d.get();
+  a[CA_DS].p = st.ds.get();
+  a[CA_BT].p = st.bt.get();
+  a[CA_COLSUM].p = st.colsum.get();
   a[CA_X].p = d_x_;
-  a[CA_POOL_IN].p = pool_.get();
-  a[CA_DPOOL_IN].p = dpool_.get();
   a[CA_OFF].i = off;
   a[CA_N].i = n;
   for (size_t i = 0; i < c.params.size(); i++) {
@@ -1727,163 +1759,227 @@ void Engine::cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned 
     a[CA_PARAM0 + i].p = p.w;
     a[CA_PARAM0 + CA_MAX_PARAMS + i].p = p.g;
   }
-  check(cavs_cell_launch(cell_module_, k, gx, gy, gz, block, a, sizeof a, stream_));
+  check(cavs_cell_launch(st.module, k, gx, gy, gz, block, a, sizeof a, stream_));
   c_launches_ += 1;
 }
 
 void Engine::cell_forward() {
-  const CellSpec &c = *cell_;
+  const CellSpec &c0 = *cells_[0].spec;
   const int N = N_, H = cfg_.H;
   if (!sched_->batching) fail(CAVS_EUNSUPPORTED, "the lowered vertex function needs the batch scheduler (OPT_BATCHING)");
-  if (c.NX > 0) {
+  if (c0.NX > 0) {
     ProfScope ps(this, K_GEMM);
-    check(cavs_embed_pull_sgemm(xW_.get(), c.NX * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E_,
-                                param(c.params[c.W.param].name).w + c.W.offset, c.NX * H, c.NX * H, 0, 0, stream_));
-    c_gemm_flops_ += 2.0 * N * c.NX * H * E_;
+    check(cavs_embed_pull_sgemm(xW_.get(), c0.NX * H, e_.get(), ld_e_, xs_.get(), d_x_, d_t2j_, param("Emb").w, N, E_,
+                                param(c0.params[c0.W.param].name).w + c0.W.offset, c0.NX * H, c0.NX * H, 0, 0, stream_));
+    c_gemm_flops_ += 2.0 * N * c0.NX * H * E_;
     c_launches_ += 1;
   }
   out_folded_ = true;  // the rounds write the pushed value by vertex id themselves
-  {
+  for (size_t ci = 0; ci < cells_.size(); ci++) {
     // the weights may have changed since the last step (the caller's optimizer writes them): both
     // tile-major copies are rewritten, a few microseconds
     ProfScope ps(this, K_OTHER);
-    cell_launch(CK_PACK, (unsigned)(((size_t)2 * c.blocks() * H * H / 4 + 255) / 256), 1, 1, 256, 0, 0, nullptr, fwd_out_);
+    const CellSpec &c = *cells_[ci].spec;
+    cell_launch((int)ci, CK_PACK, (unsigned)(((size_t)2 * c.blocks() * H * H / 4 + 255) / 256), 1, 1, 256, 0, 0, nullptr, fwd_out_);
   }
-  const unsigned block = 64u * c.waves;
-  for (const Round &r : sched_->rounds) {
-    if (leaf_round(r)) {
-      ProfScope ps(this, K_GATES);
-      cell_launch(CK_LEAVES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, fwd_out_);
-    } else {
-      ProfScope ps(this, K_ROUND);
-      cell_launch(CK_FWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, fwd_out_);
-      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
-      c_gather_rows_ += (double)c.K * r.n;
+  for (const Round &r : sched_->rounds)
+    for (size_t ci = 0; ci < cells_.size(); ci++) {
+      const CellSpec &c = *cells_[ci].spec;
+      if (ci == 0 && leaf_round(r)) {  // (a later cell's one child is the vertex itself: it always has it)
+        ProfScope ps(this, K_GATES);
+        cell_launch(0, CK_LEAVES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, fwd_out_);
+      } else {
+        ProfScope ps(this, K_ROUND);
+        cell_launch((int)ci, CK_FWD, H / 16, (r.n + 15) / 16, 1, 64u * c.waves, r.offset, r.n, nullptr, fwd_out_);
+        c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+        c_gather_rows_ += (double)c.K * r.n;
+      }
+      c_scatter_rows_ += r.n;
     }
-    c_scatter_rows_ += r.n;
-  }
 }
 
 void Engine::cell_backward() {
-  const CellSpec &c = *cell_;
+  const CellSpec &c0 = *cells_[0].spec;
   const int N = N_, H = cfg_.H, lp = sched_->leaf_prefix;
-  const unsigned block = 64u * c.waves;
-  backward_prologue({}, c.NX > 0);
+  const int L = (int)cells_.size();
+  backward_prologue({}, c0.NX > 0);
   // a parameter F reads only parts of: the rest of its gradient is zero
   {
-    std::vector<long> covered(c.params.size(), 0);
-    if (c.NX > 0) covered[c.W.param] += (long)E_ * c.NX * H;
-    for (const CellProduct &p : c.products) covered[p.B.param] += (long)p.terms.size() * H * H;
-    for (const CellBias &b : c.biases) covered[b.ref.param] += H;
-    for (size_t i = 0; i < c.params.size(); i++)
-      if (c.params[i].name != "Emb" && covered[i] < c.params[i].size) {
-        check(cavs_zero(param(c.params[i].name).g, (size_t)c.params[i].size * 4, stream_));
+    std::vector<long> covered(c0.params.size(), 0);
+    if (c0.NX > 0) covered[c0.W.param] += (long)E_ * c0.NX * H;
+    std::vector<std::pair<int, long>> seen;
+    for (const CellStage &st : cells_) {
+      for (const CellProduct &p : st.spec->products)
+        for (const CellTerm &t : p.terms) {
+          const auto key = std::make_pair(p.B.param, p.B.offset + t.brow * p.ldb + p.col);
+          if (std::find(seen.begin(), seen.end(), key) != seen.end()) continue;
+          seen.push_back(key);
+          covered[p.B.param] += (long)H * H;
+        }
+      for (const CellBias &b : st.spec->biases)
+        if (!b.add) covered[b.ref.param] += H;
+    }
+    for (size_t i = 0; i < c0.params.size(); i++)
+      if (c0.params[i].name != "Emb" && covered[i] < c0.params[i].size) {
+        check(cavs_zero(param(c0.params[i].name).g, (size_t)c0.params[i].size * 4, stream_));
         c_launches_ += 1;
       }
   }
-  if (forest_) {
+  if (forest_ && L == 1) {
     // every message is read exactly once: a round's launch hands d(state) on to the children of its
     // rows and runs their elementwise part at once; the vertices without a reader go first
+    const unsigned block = 64u * c0.waves;
     if (n_orphans_ > 0) {
       ProfScope ps(this, K_GATES);
-      cell_launch(CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
+      cell_launch(0, CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
     }
     for (int k : sched_->bwd_rounds) {
       const Round &r = sched_->rounds[k];
       c_gather_rows_ += r.n;
       if (leaf_round(r)) continue;
       ProfScope ps(this, K_ROUND);
-      cell_launch(CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
-      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
-      c_scatter_rows_ += (double)c.K * r.n;
+      cell_launch(0, CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
+      c_round_flops_ += 2.0 * r.n * c0.terms() * H * H;
+      c_scatter_rows_ += (double)c0.K * r.n;
     }
   } else {
-    // any other batch: two launches per round, with the message gradients going through the gradient
-    // of the message pool as in the reference (rows nobody wrote read as zero)
+    // any other batch, and every chain: two launches per round and cell, the message gradients
+    // going through the gradient of the rows the cells write, as in the reference (rows of the
+    // message pool nobody wrote read as zero)
     check(cavs_zero(dpool_.get(), (size_t)N * mw_ * 4, stream_));
     c_launches_ += 1;
     for (int k : sched_->bwd_rounds) {
       const Round &r = sched_->rounds[k];
-      {
-        ProfScope ps(this, K_GATES);
-        cell_launch(CK_BWD_GATES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, d_dgo_);
+      for (int ci = L - 1; ci >= 0; ci--) {
+        const CellSpec &c = *cells_[ci].spec;
+        {
+          ProfScope ps(this, K_GATES);
+          cell_launch(ci, CK_BWD_GATES, (unsigned)(((size_t)r.n * H + 255) / 256), 1, 1, 256, r.offset, r.n, nullptr, d_dgo_);
+        }
+        c_gather_rows_ += r.n;
+        if (ci == 0 && leaf_round(r)) continue;
+        ProfScope ps(this, K_ROUND);
+        cell_launch(ci, CK_BWD_POOL, H / 16, (r.n + 15) / 16, 1, 64u * c.waves, r.offset, r.n, nullptr, d_dgo_);
+        c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+        c_scatter_rows_ += (double)c.K * r.n;
       }
-      c_gather_rows_ += r.n;
-      if (leaf_round(r)) continue;
-      ProfScope ps(this, K_ROUND);
-      cell_launch(CK_BWD_POOL, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
-      c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
-      c_scatter_rows_ += (double)c.K * r.n;
     }
   }
-  // the weight gradients, once over all rows: runs of terms whose operands, columns and gradient
-  // blocks are adjacent go as one product
-  const int ldd = c.ND * H, lda = (int)c.asrc.size() * H;
-  std::vector<cavs_gemm_desc> products;
-  if (c.NX > 0) {
-    float *W = param(c.params[c.W.param].name).w + c.W.offset, *dW = param(c.params[c.W.param].name).g + c.W.offset;
-    products.push_back({0, 1, N, E_, c.NX * H, 1.f, 0.f, dxW_.get(), ldd, W, c.NX * H, de_.get(), E_});
-    products.push_back({1, 0, E_, c.NX * H, N, 1.f, 0.f, e_.get(), ld_e_, dxW_.get(), ldd, dW, c.NX * H});
-  }
-  struct Run {
-    int asrc, dcol, param, ldb, width;
-    long view, brow, col;
-    long at() const { return view + brow * ldb + col; }
+  // the weight gradients, once over all rows.  A product that writes where an earlier one of the
+  // list wrote adds to it, one launch later (a weight block several products read; d e of several
+  // cells); the rest go up to eight to a launch.
+  std::vector<std::vector<cavs_gemm_desc>> waves(1);
+  struct Written {
+    const float *first;
+    int n, ldc, times;
   };
-  std::vector<Run> runs;
-  for (const CellProduct &p : c.products)
-    for (const CellTerm &t : p.terms) {
-      if (!runs.empty()) {
-        Run &q = runs.back();
-        if (q.asrc == t.asrc && q.param == p.B.param && q.view == p.B.offset && q.ldb == p.ldb && q.brow == t.brow &&
-            q.col + q.width == p.col && q.dcol + q.width / H == p.dcol) {
-          q.width += H;
-          continue;
-        }
+  std::vector<Written> written;
+  auto add = [&](cavs_gemm_desc d) {
+    int before = 0;
+    bool known = false;
+    for (Written &w : written)
+      if (w.first == d.C) {
+        if (w.n != d.N || w.ldc != d.ldc)
+          fail(CAVS_EUNSUPPORTED, "products of the lowered vertex function read overlapping but different blocks of one weight");
+        before = w.times++;
+        known = true;
       }
-      runs.push_back({t.asrc, p.dcol, p.B.param, p.ldb, H, p.B.offset, t.brow, p.col});
+    if (!known) written.push_back({d.C, d.N, d.ldc, 1});
+    d.beta = before ? 1.f : 0.f;
+    if ((int)waves.size() <= before) waves.resize(before + 1);
+    waves[before].push_back(d);
+  };
+  if (c0.NX > 0) {
+    float *W = param(c0.params[c0.W.param].name).w + c0.W.offset, *dW = param(c0.params[c0.W.param].name).g + c0.W.offset;
+    // d e first: the launch that reduces the first group of a function of one stage also scatters it into the table's gradient
+    for (const CellStage &st : cells_) {
+      const CellSpec &c = *st.spec;
+      if (c.xw_hi <= c.xw_lo) continue;
+      const int w = (c.xw_hi - c.xw_lo) * H;
+      add({0, 1, N, E_, w, 1.f, 0.f, st.d.at((size_t)c.xw_lo * H), c.ND * H, W + (size_t)c.xw_lo * H, c.NX * H, de_.get(), E_});
     }
-  // a block of weights that several products read collects their gradients one launch after the other
-  std::vector<std::vector<cavs_gemm_desc>> later;
-  if (N > lp)
-    for (size_t i = 0; i < runs.size(); i++) {
-      const Run &q = runs[i];
-      size_t before = 0;
-      for (size_t k = 0; k < i; k++)
-        if (runs[k].param == q.param && runs[k].at() == q.at()) {
-          if (runs[k].width != q.width || runs[k].ldb != q.ldb)
-            fail(CAVS_EUNSUPPORTED, "products of the lowered vertex function read overlapping but different blocks of one weight");
-          before++;
+    for (const CellStage &st : cells_) {
+      const CellSpec &c = *st.spec;
+      if (c.xw_hi <= c.xw_lo) continue;
+      const int w = (c.xw_hi - c.xw_lo) * H;
+      add({1, 0, E_, w, N, 1.f, 0.f, e_.get(), ld_e_, st.d.at((size_t)c.xw_lo * H), c.ND * H, dW + (size_t)c.xw_lo * H, c.NX * H});
+    }
+  }
+  for (size_t ci = 0; ci < cells_.size(); ci++) {
+    const CellStage &st = cells_[ci];
+    const CellSpec &c = *st.spec;
+    const int ldd = c.ND * H, lda = (int)c.asrc.size() * H;
+    const int r0 = ci == 0 ? lp : 0;  // (the first cell's left operands are zero in the rows of leaves)
+    struct Run {
+      int asrc, dcol, param, ldb, width;
+      long view, brow, col;
+      long at() const { return view + brow * ldb + col; }
+    };
+    std::vector<Run> runs;  // terms whose operands, columns and gradient blocks are adjacent go as one product
+    for (const CellProduct &p : c.products)
+      for (const CellTerm &t : p.terms) {
+        if (!runs.empty()) {
+          Run &q = runs.back();
+          if (q.asrc == t.asrc && q.param == p.B.param && q.view == p.B.offset && q.ldb == p.ldb && q.brow == t.brow &&
+              q.col + q.width == p.col && q.dcol + q.width / H == p.dcol) {
+            q.width += H;
+            continue;
+          }
         }
-      const cavs_gemm_desc d{1, 0, H, q.width, N - lp, 1.f, before ? 1.f : 0.f, hlr_.at((size_t)lp * lda + (size_t)q.asrc * H), lda,
-                             dxW_.at((size_t)lp * ldd + (size_t)q.dcol * H), ldd, param(c.params[q.param].name).g + q.at(), q.ldb};
-      if (!before) {
-        products.push_back(d);
-      } else {
-        if (later.size() < before) later.resize(before);
-        later[before - 1].push_back(d);
+        runs.push_back({t.asrc, p.dcol, p.B.param, p.ldb, H, p.B.offset, t.brow, p.col});
+      }
+    for (const Run &q : runs) {
+      float *C = param(c.params[q.param].name).g + q.at();
+      if (N > r0) {
+        add({1, 0, H, q.width, N - r0, 1.f, 0.f, st.asrc.at((size_t)r0 * lda + (size_t)q.asrc * H), lda,
+             st.d.at((size_t)r0 * ldd + (size_t)q.dcol * H), ldd, C, q.ldb});
+      } else {  // a batch of single vertices: nothing was multiplied
+        for (int row = 0; row < H; row++) check(cavs_zero(C + (size_t)row * q.ldb, (size_t)q.width * 4, stream_));
       }
     }
-  else
-    for (const Run &q : runs)  // a batch of single vertices: nothing was multiplied
-      for (int row = 0; row < H; row++) check(cavs_zero(param(c.params[q.param].name).g + q.at() + (size_t)row * q.ldb, (size_t)q.width * 4, stream_));
+  }
+  // (overlapping but different blocks of one weight would need more than "the same first element")
   constexpr size_t kGroup = 8;  // products per cavs_sgemm_group launch
-  size_t at = 0;
-  if (c.NX > 0) {
-    const size_t take = std::min<size_t>(products.size(), kGroup);
-    gemm_group_embedding_backward(std::vector<cavs_gemm_desc>(products.begin(), products.begin() + take), E_);
-    at = take;
+  bool embedded = false;
+  for (size_t wv = 0; wv < waves.size(); wv++) {
+    const std::vector<cavs_gemm_desc> &w = waves[wv];
+    size_t at = 0;
+    if (wv == 0 && c0.NX > 0 && L == 1 && !w.empty()) {  // d e is complete after this launch
+      const size_t take = std::min(w.size(), kGroup);
+      gemm_group_embedding_backward(std::vector<cavs_gemm_desc>(w.begin(), w.begin() + take), E_);
+      at = take;
+      embedded = true;
+    }
+    for (; at < w.size(); at += kGroup) gemm_group(std::vector<cavs_gemm_desc>(w.begin() + at, w.begin() + std::min(w.size(), at + kGroup)));
   }
-  for (; at < products.size(); at += kGroup)
-    gemm_group(std::vector<cavs_gemm_desc>(products.begin() + at, products.begin() + std::min(products.size(), at + kGroup)));
-  for (const std::vector<cavs_gemm_desc> &wave : later)
-    for (size_t i = 0; i < wave.size(); i += kGroup)
-      gemm_group(std::vector<cavs_gemm_desc>(wave.begin() + i, wave.begin() + std::min(wave.size(), i + kGroup)));
-  if (!c.biases.empty()) {
-    colsum_fixed(cell_colsum_.get(), dxW_.get(), N, ldd);
+  if (c0.NX > 0 && !embedded) embedding_backward_rows();
+  for (size_t ci = 0; ci < cells_.size(); ci++) {
+    const CellStage &st = cells_[ci];
+    if (st.spec->biases.empty()) continue;
+    colsum_fixed(st.colsum.get(), st.d.get(), N, st.spec->ND * H);
     ProfScope ps(this, K_OTHER);
-    cell_launch(CK_BIAS, (H + 255) / 256, 1, 1, 256, 0, 0, nullptr, d_dgo_);
+    cell_launch((int)ci, CK_BIAS, (H + 255) / 256, 1, 1, 256, 0, 0, nullptr, d_dgo_);
   }
+}
+
+// EmbeddingLookup_grad as a launch of its own: rows of de_ added into the table's gradient.
+void Engine::embedding_backward_rows() {
+  Param &emb = param("Emb");
+  const bool owned = emb.g == emb.own_g.get();
+  if (emb_cleared_) {
+    emb_cleared_ = false;
+  } else if (owned && emb_sparse_valid_) {
+    if (emb_dirty_n_ > 0) check(cavs_embed_zero_rows(emb.g, xs_prev_.get(), emb_dirty_n_, E_, stream_));
+    c_launches_ += 1;
+  } else {
+    check(cavs_zero(emb.g, emb.n * 4, stream_));
+    c_launches_ += 1;
+  }
+  check(cavs_embed_bwd(emb.g, xs_.get(), de_.get(), E_, N_, E_, stream_));
+  c_launches_ += 1;
+  xs_.swap(xs_prev_);
+  emb_dirty_n_ = N_;
+  emb_sparse_valid_ = owned;
 }
 
 // ------------------------------------------------------------------ loss head

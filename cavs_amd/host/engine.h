@@ -11,6 +11,7 @@
 #include <map>
 #include <memory>
 #include <string>
+#include <deque>
 #include <vector>
 
 #include "cavs_session.h"
@@ -357,11 +358,21 @@ class Engine {
   void aux_join();
 
   // ---- a vertex function on generated kernels (CAVS_MODEL_CELL)
-  std::shared_ptr<const CellSpec> cell_;
-  void *cell_module_ = nullptr;
-  DeviceArray<float> cell_colsum_;
-  // one launch of kernel `k` of the module; `fill` sets the slots that differ from the step's common ones
-  void cell_launch(int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go);
+  // A function of several stages is a chain of cells (CellSpec::next); every cell has its module
+  // and its per-vertex rows.  A cell before the last writes `rows` by slab row, which the next one
+  // gathers through the identity list; `drows` is the gradient of those rows.
+  struct CellStage {
+    std::shared_ptr<const CellSpec> spec;
+    void *module = nullptr;
+    DeviceArray<float> sv, asrc, d, ds, bt, colsum, rows, drows;
+  };
+  std::shared_ptr<const CellSpec> cell_;  // the head of the chain
+  std::deque<CellStage> cells_;  // (the arrays do not move)
+  DeviceArray<int> cell_iota_;  // 0, 1, 2, ...: "the child of slab row v is slab row v"
+  size_t cell_iota_n_ = 0;
+  // one launch of kernel `k` of cell `ci`'s module
+  void cell_launch(int ci, int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go);
+  void embedding_backward_rows();
 
   // counters of the last step
   double c_round_flops_ = 0;

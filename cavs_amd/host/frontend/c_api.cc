@@ -160,12 +160,15 @@ size_t C_DumpFusedGraph(char *buf, size_t cap) {
 
 size_t C_DumpCell(char *buf, size_t cap, int what) {
   std::string d;
-  if (what == 0) {
-    d = cavs::mid::cell_host_source(cavs::mid::global_graph());
+  const int stage = what / 10;
+  if (what % 10 == 0) {
+    d = cavs::mid::cell_host_source(cavs::mid::global_graph(), stage);
   } else {
     std::string why;
     auto m = cavs::mid::match_cell(cavs::mid::global_graph(), &why);
-    d = m ? m->spec->source : "// not a cell: " + why + "\n";
+    std::shared_ptr<cavs::CellSpec> spec = m ? m->spec : nullptr;
+    for (int i = 0; i < stage && spec; i++) spec = spec->next;
+    d = spec ? spec->source : m ? std::string("// no such stage\n") : "// not a cell: " + why + "\n";
   }
   if (buf && cap) {
     size_t n = std::min(cap - 1, d.size());

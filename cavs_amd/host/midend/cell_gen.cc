@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstring>
+#include <functional>
 #include <set>
 #include <sstream>
 #include <tuple>
@@ -62,16 +63,33 @@ struct Fail {
 };
 [[noreturn]] void no(const std::string &why) { throw Fail{why}; }
 
-// ---------------------------------------------------------------- reading F
-struct Reader {
-  const Graph &g;
-  const Scope *func;
+// One cell: its description, its elementwise part, the nodes of its state blocks and of the value it pushes.
+struct Body {
   CellSpec spec;
   Dag dag;
+  std::vector<int> st;
+  int ret = -1;
+};
+
+// ---------------------------------------------------------------- reading F
+// A product as read: the nodes of its left operand's blocks, whatever they are.
+struct RawTerm {
+  int node;
+  long brow;
+};
+struct RawProduct {
+  std::vector<RawTerm> terms;
+  CellParamRef B;
+  int ldb = 0;
+  long col = 0;
+};
+
+struct Reader : Body {
+  const Graph &g;
+  const Scope *func;
   std::map<const Edge *, std::vector<int>> val;  // H-wide blocks of a func-scope edge, as nodes
   std::set<const Edge *> raw_x, emb_x;           // the pulled id; its embedding row
-  std::vector<int> st;                           // the scattered state blocks
-  int ret = -1;
+  std::vector<RawProduct> raw;                   // by the index of their N_HU node
   std::map<std::string, int> param_of;           // Variable -> index in spec.params
   std::map<std::string, std::string> roles;
   std::map<std::string, CellSlot> slots;
@@ -80,6 +98,7 @@ struct Reader {
   bool have_xw = false;
 
   explicit Reader(const Graph &graph) : g(graph), func(graph.func.get()) {}
+  std::map<std::pair<int, long>, int> &biases_seen() { return bias_of; }
 
   int param_index(const Resolved &r, bool embedding) {
     auto it = param_of.find(r.var);
@@ -142,8 +161,9 @@ struct Reader {
     return val[e] = b;
   }
 
-  // the sum of state blocks of children that a product's left operand block is
-  int a_source(int node) {
+  // whether a node is a plain sum of one state block of distinct children (what the first stage's
+  // products take as their left operand straight from the message pool)
+  bool child_sum(int node, int *mask_out, int *block_out) const {
     int mask = 0, block = -1;
     std::vector<int> todo{node};
     while (!todo.empty()) {
@@ -153,20 +173,16 @@ struct Reader {
         todo.push_back(q.a);
         todo.push_back(q.b);
       } else if (q.kind == N_CS) {
-        if (block >= 0 && block != q.i1) no("a product's left operand adds different state blocks");
-        if (mask & (1 << q.i0)) no("a product's left operand adds a child twice");
+        if ((block >= 0 && block != q.i1) || (mask & (1 << q.i0))) return false;
         block = q.i1;
         mask |= 1 << q.i0;
       } else {
-        no("a product's left operand is not a sum of children's state blocks");
+        return false;
       }
     }
-    auto key = std::make_pair(mask, block);
-    if (!asrc_of.count(key)) {
-      asrc_of[key] = (int)spec.asrc.size();
-      spec.asrc.push_back({mask, block});
-    }
-    return asrc_of[key];
+    *mask_out = mask;
+    *block_out = block;
+    return true;
   }
 
   void read() {
@@ -243,18 +259,16 @@ struct Reader {
           s.NX = (int)(cols / H);
           for (int i = 0; i < s.NX; i++) b.push_back(dag.make(N_XW, -1, -1, i));
         } else {
-          const std::vector<int> &ab = blocks(A);
+          const std::vector<int> ab = blocks(A);
           if ((long)ab.size() * H != rows) no("MatMul operand widths do not agree");
-          std::vector<int> src;
-          for (int node : ab) src.push_back(a_source(node));
           for (long o = 0; o < cols / H; o++) {
-            CellProduct p;
-            for (size_t a = 0; a < src.size(); a++) p.terms.push_back({src[a], (long)a * H});
+            RawProduct p;
+            for (size_t a = 0; a < ab.size(); a++) p.terms.push_back({ab[a], (long)a * H});
             p.B = ref;
             p.ldb = (int)cols;
             p.col = o * H;
-            s.products.push_back(p);
-            b.push_back(dag.make(N_HU, -1, -1, (int)s.products.size() - 1));
+            raw.push_back(p);
+            b.push_back(dag.make(N_HU, -1, -1, (int)raw.size() - 1));
           }
         }
         val[out] = b;
@@ -301,8 +315,8 @@ struct Reader {
     if (st.empty() || ret < 0) no("F has no Scatter or no Push");
     if (s.K < 1) no("F gathers no child");
     if (!raw_x.empty() && !have_xw) no("the vertex input's id is pulled but not looked up and multiplied");
-    if (s.products.empty()) no("F multiplies no child state");
-    if (s.products.size() > 16 || s.asrc.size() > 8 || s.NX > 16 || s.biases.size() > 32) no("too many products or operands");
+    if (raw.empty()) no("F multiplies no child state");
+    if (raw.size() > 32 || s.NX > 16 || s.biases.size() > 32) no("too many products or operands");
   }
 };
 
@@ -315,7 +329,7 @@ struct Derived {
   int ds_mask = 0;
 };
 
-Derived derive(Reader &r) {
+Derived derive(Body &r) {
   Dag &dag = r.dag;
   CellSpec &s = r.spec;
   const int nfwd = (int)dag.n.size();
@@ -399,14 +413,14 @@ Derived derive(Reader &r) {
 
 // ---------------------------------------------------------------- writing the source
 struct Writer {
-  const Reader &r;
+  const Body &r;
   const Derived &dv;
   const Dag &dag;
   const CellSpec &s;
   bool device;
   std::ostringstream o;
 
-  Writer(const Reader &rd, const Derived &d, bool dev) : r(rd), dv(d), dag(rd.dag), s(rd.spec), device(dev) {}
+  Writer(const Body &rd, const Derived &d, bool dev) : r(rd), dv(d), dag(rd.dag), s(rd.spec), device(dev) {}
 
   std::string name(int id, bool backward, int nfwd) const {
     const ENode &q = dag.n[id];
@@ -634,21 +648,193 @@ struct Writer {
     o << "  }\n}\n";
     // the bias gradients out of the column sums of the gradient rows
     o << "extern \"C\" __global__ void cell_bias(CellArgs a) {\n  const int j = blockIdx.x * 256 + threadIdx.x;\n  if (j >= CELL_H) return;\n";
-    for (const CellBias &b : s.biases) o << "  " << param_ptr(b.ref, true) << "[j] = a.colsum[" << (long)b.dcol * H << " + j];\n";
+    for (const CellBias &b : s.biases) o << "  " << param_ptr(b.ref, true) << "[j] " << (b.add ? "+=" : "=") << " a.colsum[" << (long)b.dcol * H << " + j];\n";
     o << "}\n";
   }
 };
 
-struct Built {
+// ---------------------------------------------------------------- stages
+// The stage of a value is the number of products on the longest way to it from the inputs.  A
+// function whose products are all of the first stage (left operands: plain sums of the children's
+// state blocks) is one cell.  Otherwise F is cut into a chain of cells, one per stage: cell s holds
+// the products of stage s and the elementwise values of that stage; what later stages read of it --
+// their products' left operands first of all -- becomes the blocks of a row it writes per vertex,
+// which the next cell gathers as the state of its one child, the vertex itself.
+struct Chain {
   Reader reader;
-  Derived derived;
-  int nfwd;
-  explicit Built(const Graph &g) : reader(g) {
+  std::vector<Body> cells;
+  std::vector<Derived> derived;
+  std::vector<int> nfwd;
+
+  explicit Chain(const Graph &g) : reader(g) {
     reader.read();
-    nfwd = (int)reader.dag.n.size();
-    derived = derive(reader);
+    const Dag &full = reader.dag;
+    const int n = (int)full.n.size();
+    // stages
+    std::vector<int> stage(n, 0);
+    int L = 0;
+    for (int id = 0; id < n; id++) {
+      const ENode &q = full.n[id];
+      if (q.kind == N_HU) {
+        int st = 1;
+        for (const RawTerm &t : reader.raw[q.i0].terms) {
+          int mask, block;
+          if (!reader.child_sum(t.node, &mask, &block)) st = std::max(st, 1 + std::max(1, stage[t.node]));
+        }
+        stage[id] = st;
+        L = std::max(L, st);
+      } else if (q.kind >= N_ADD) {
+        stage[id] = std::max(q.a >= 0 ? stage[q.a] : 0, q.b >= 0 ? stage[q.b] : 0);
+      }
+    }
+    if (L > 4) no("more than four stages of products");
+    bool first_stage = false;
+    for (int id = 0; id < n; id++) first_stage |= full.n[id].kind == N_HU && stage[id] == 1;
+    if (!first_stage) no("no product takes a sum of the children's state blocks as its left operand");
+    auto carried = [&](int id) { const int k = full.n[id].kind; return k != N_XW && k != N_BIAS && k != N_XD; };
+    // what each cell writes for the later ones: T[s] = blocks of the row cell s writes (s < L), found
+    // from the last cell backwards
+    std::vector<std::vector<int>> T(L + 1);
+    for (int sidx = L; sidx >= 2; sidx--) {
+      std::vector<int> &need = T[sidx - 1];
+      auto want = [&](int id) {
+        if (stage[id] < sidx && carried(id) && std::find(need.begin(), need.end(), id) == need.end()) need.push_back(id);
+      };
+      // left operands of this stage's products first: the next cell's products read them
+      for (int id = 0; id < n; id++)
+        if (full.n[id].kind == N_HU && stage[id] == sidx)
+          for (const RawTerm &t : reader.raw[full.n[id].i0].terms) want(t.node);
+      std::vector<int> roots = sidx == L ? reader.st : T[sidx];
+      if (sidx == L && reader.ret >= 0) roots.push_back(reader.ret);
+      std::set<int> seen;
+      while (!roots.empty()) {
+        const int id = roots.back();
+        roots.pop_back();
+        if (!seen.insert(id).second) continue;
+        if (stage[id] < sidx) {
+          want(id);
+          continue;
+        }
+        const ENode &q = full.n[id];
+        if (q.kind >= N_ADD) {
+          if (q.a >= 0) roots.push_back(q.a);
+          if (q.b >= 0) roots.push_back(q.b);
+        }
+      }
+      if (need.size() > 12) no("a stage hands more than twelve blocks on to the next");
+    }
+    // the cells
+    for (int sidx = 1; sidx <= L; sidx++) {
+      Body c;
+      CellSpec &cs = c.spec;
+      const CellSpec &rs = reader.spec;
+      cs.H = rs.H;
+      cs.E = rs.E;
+      cs.V = rs.V;
+      cs.NX = rs.NX;
+      cs.XD = rs.XD;
+      cs.W = rs.W;
+      cs.params = rs.params;
+      cs.K = sidx == 1 ? rs.K : 1;
+      cs.SI = sidx == 1 ? rs.SI : (int)T[sidx - 1].size();
+      cs.S = sidx == L ? rs.S : (int)T[sidx].size();
+      cs.has_ret = sidx == L;
+      std::map<int, int> memo, local_bias, local_product;
+      std::map<std::pair<int, int>, int> asrc_of;
+      auto a_source = [&](int mask, int block) {
+        auto key = std::make_pair(mask, block);
+        if (!asrc_of.count(key)) {
+          asrc_of[key] = (int)cs.asrc.size();
+          cs.asrc.push_back({mask, block});
+        }
+        return asrc_of[key];
+      };
+      std::function<int(int)> conv = [&](int old) -> int {
+        auto it = memo.find(old);
+        if (it != memo.end()) return it->second;
+        const ENode q = full.n[old];
+        int id;
+        if (q.kind == N_XW || q.kind == N_XD) {
+          id = c.dag.make(q.kind, -1, -1, q.i0);
+        } else if (q.kind == N_BIAS) {
+          if (!local_bias.count(q.i0)) {
+            local_bias[q.i0] = (int)cs.biases.size();
+            cs.biases.push_back(rs.biases[q.i0]);
+          }
+          id = c.dag.make(N_BIAS, -1, -1, local_bias[q.i0]);
+        } else if (sidx >= 2 && stage[old] < sidx) {  // written by the cell before: a block of this vertex's own row
+          const auto &row = T[sidx - 1];
+          id = c.dag.make(N_CS, -1, -1, 0, (int)(std::find(row.begin(), row.end(), old) - row.begin()));
+        } else if (q.kind == N_CS) {
+          id = c.dag.make(N_CS, -1, -1, q.i0, q.i1);
+        } else if (q.kind == N_HU) {
+          if (!local_product.count(q.i0)) {
+            const RawProduct &rp = reader.raw[q.i0];
+            CellProduct p;
+            p.B = rp.B;
+            p.ldb = rp.ldb;
+            p.col = rp.col;
+            for (const RawTerm &t : rp.terms) {
+              int mask = 1, block = 0;
+              if (sidx == 1) {
+                if (!reader.child_sum(t.node, &mask, &block)) no("internal: a first-stage product with another left operand");
+              } else {
+                const auto &row = T[sidx - 1];
+                block = (int)(std::find(row.begin(), row.end(), t.node) - row.begin());
+              }
+              p.terms.push_back({a_source(mask, block), t.brow});
+            }
+            local_product[q.i0] = (int)cs.products.size();
+            cs.products.push_back(p);
+          }
+          id = c.dag.make(N_HU, -1, -1, local_product[q.i0]);
+        } else {
+          const int a = q.a >= 0 ? conv(q.a) : -1, b = q.b >= 0 ? conv(q.b) : -1;
+          id = c.dag.make(q.kind, a, b, q.i0, q.i1, q.scale);
+        }
+        return memo[old] = id;
+      };
+      // (the products in their order of declaration, so that adjacent blocks of one MatMul stay adjacent)
+      for (int id = 0; id < n; id++)
+        if (full.n[id].kind == N_HU && stage[id] == sidx) conv(id);
+      for (int id : (sidx == L ? reader.st : T[sidx])) c.st.push_back(conv(id));
+      c.ret = sidx == L && reader.ret >= 0 ? conv(reader.ret) : -1;
+      if (cs.products.empty()) no("internal: a stage without products");
+      if (cs.products.size() > 16 || cs.asrc.size() > 8) no("too many products or operands in one stage");
+      cs.xw_lo = L == 1 ? 0 : cs.NX;
+      cs.xw_hi = L == 1 ? cs.NX : 0;
+      for (const ENode &q : c.dag.n)
+        if (q.kind == N_XW) {
+          cs.xw_lo = std::min(cs.xw_lo, q.i0);
+          cs.xw_hi = std::max(cs.xw_hi, q.i0 + 1);
+        }
+      for (CellBias &b : cs.biases)
+        for (const Body &before : cells)
+          for (const CellBias &e : before.spec.biases) b.add |= e.ref.param == b.ref.param && e.ref.offset == b.ref.offset;
+      cells.push_back(std::move(c));
+    }
+    for (Body &c : cells) {
+      nfwd.push_back((int)c.dag.n.size());
+      derived.push_back(derive(c));
+    }
   }
 };
+
+// the source of one cell's kernels
+void write_cell(Body &c, const Derived &d, int nfwd) {
+  CellSpec &s = c.spec;
+  const int H = s.H;
+  s.waves = H % 128 == 0 ? 4 : H % 64 == 0 ? 2 : 1;
+  // the partial tiles of a workgroup must fit in LDS
+  const size_t per_wave = std::max(s.products.size(), s.asrc.size()) * 1024;
+  if (s.waves * per_wave > 60 * 1024) no("too many accumulators for one workgroup");
+  Writer w(c, d, true);
+  w.kernels();
+  w.elementwise(nfwd);
+  w.product_loops();
+  w.o << kTemplate;
+  s.source = w.o.str();
+}
 
 }  // namespace
 
@@ -682,21 +868,17 @@ Resolved resolve_external(const Edge *e) {
 
 std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
   try {
-    Built b(g);
-    CellSpec &s = b.reader.spec;
-    const int H = s.H;
-    s.waves = H % 128 == 0 ? 4 : H % 64 == 0 ? 2 : 1;
-    // the partial tiles of a workgroup must fit in LDS
-    const size_t per_wave = std::max(s.products.size(), s.asrc.size()) * 1024;
-    if (s.waves * per_wave > 60 * 1024) no("too many accumulators for one workgroup");
-    Writer w(b.reader, b.derived, true);
-    w.kernels();
-    w.elementwise(b.nfwd);
-    w.product_loops();
-    w.o << kTemplate;
-    s.source = w.o.str();
+    Chain b(g);
+    std::shared_ptr<CellSpec> head, tail;
+    for (size_t i = 0; i < b.cells.size(); i++) {
+      write_cell(b.cells[i], b.derived[i], b.nfwd[i]);
+      auto spec = std::make_shared<CellSpec>(b.cells[i].spec);
+      if (tail) tail->next = spec;
+      else head = spec;
+      tail = spec;
+    }
     auto m = std::make_unique<CellMatch>();
-    m->spec = std::make_shared<CellSpec>(s);
+    m->spec = head;
     m->roles = b.reader.roles;
     m->slots = b.reader.slots;
     return m;
@@ -706,15 +888,17 @@ std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
   }
 }
 
-std::string cell_host_source(const Graph &g) {
+std::string cell_host_source(const Graph &g, int stage) {
   try {
-    Built b(g);
-    Writer w(b.reader, b.derived, false);
+    Chain b(g);
+    if (stage < 0 || stage >= (int)b.cells.size()) return "// no such stage\n";
+    Writer w(b.cells[stage], b.derived[stage], false);
     w.o << "#include <math.h>\n";
-    w.elementwise(b.nfwd);
-    const CellSpec &s = b.reader.spec;
-    w.o << "// H=" << s.H << " K=" << s.K << " S=" << s.S << " NX=" << s.NX << " XD=" << s.XD << " NP=" << s.products.size() << " NB=" << s.biases.size()
-        << " ND=" << s.ND << " NSV=" << s.NSV << "\n";
+    w.elementwise(b.nfwd[stage]);
+    const CellSpec &s = b.cells[stage].spec;
+    w.o << "// stages=" << b.cells.size() << "\n";
+    w.o << "// H=" << s.H << " K=" << s.K << " S=" << s.S << " SI=" << s.SI << " NX=" << s.NX << " XD=" << s.XD << " NP=" << s.products.size()
+        << " NB=" << s.biases.size() << " ND=" << s.ND << " NSV=" << s.NSV << "\n";
     for (size_t p = 0; p < s.products.size(); p++) w.o << "// product " << p << " dcol " << s.products[p].dcol << "\n";
     for (size_t i = 0; i < s.biases.size(); i++) w.o << "// bias " << i << " dcol " << s.biases[i].dcol << "\n";
     return w.o.str();

@@ -33,7 +33,8 @@ std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why = nullptr
 
 // The elementwise parts alone as host C++ (cell_forward / cell_backward over plain structs), for
 // checking the derived backward part against finite differences without a device.
-std::string cell_host_source(const Graph &g);
+// (stage: which cell of the chain a function of several stages is cut into; 0 for a function of one)
+std::string cell_host_source(const Graph &g, int stage = 0);
 
 // A main-scope edge traced back through aliasing ops to the Variable it views.
 struct Resolved {

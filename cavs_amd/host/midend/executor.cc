@@ -173,12 +173,14 @@ void Executor::compile() {
       if (lowering_ && lowering_->cell) {
         // the generated kernels must compile (the module stays cached for the engine); if they do
         // not, F runs operator by operator like any function that is not of the shape
-        void *module = nullptr;
-        if (cavs_cell_compile(lowering_->cell->source.c_str(), &module) != CAVS_OK) {
-          std::fprintf(stderr, "cavs: the round kernels generated for the vertex function did not compile (%s); running it operator by operator\n",
-                       cavs_last_error());
-          lowering_.reset();
-        } else {
+        for (std::shared_ptr<const CellSpec> c = lowering_->cell; c; c = c->next) {
+          void *module = nullptr;
+          if (cavs_cell_compile(c->source.c_str(), &module) != CAVS_OK) {
+            std::fprintf(stderr, "cavs: the round kernels generated for the vertex function did not compile (%s); running it operator by operator\n",
+                         cavs_last_error());
+            lowering_.reset();
+            break;
+          }
           cavs_cell_release(module);
         }
       }

@@ -63,9 +63,9 @@ const char *C_LastError(void);
 /* Text dump of the declared program: forward ops, the vertex function, and the backward
  * programs the autograd pass derived.  Returns the length needed (including the NUL). */
 size_t C_DumpGraph(char *buf, size_t cap);
-/* The kernels generated for the declared vertex function when it has the general one-stage shape
- * (what = 1), or its elementwise parts alone as host C++ (what = 0); a comment saying why not
- * otherwise. */
+/* The kernels generated for the declared vertex function when it has the general shape (what = 1),
+ * or its elementwise parts alone as host C++ (what = 0); a comment saying why not otherwise.  A
+ * function of several stages is a chain of cells: what + 10 * s names cell s of it. */
 size_t C_DumpCell(char *buf, size_t cap, int what);
 /* The same programs after the OPT_FUSION pass, with the generated kernel sources. */
 size_t C_DumpFusedGraph(char *buf, size_t cap);

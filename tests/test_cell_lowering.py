@@ -1,8 +1,8 @@
-"""Lowering of a vertex function of the general one-stage shape onto generated kernels, the parts
-that need no device: what the analysis of F accepts and refuses, and the elementwise part of the
-backward function it derives -- compiled for the host in double and held against central
-differences of the generated forward part (a wrong sign, a dropped term or a swapped operand of the
-derivation fails this)."""
+"""Lowering of a vertex function of the general shape onto generated kernels, the parts that need
+no device: what the analysis of F accepts and refuses, how it cuts a function of several stages
+into a chain of cells, and the elementwise part of the backward function it derives for every cell
+-- compiled for the host in double and held against central differences of the generated forward
+part (a wrong sign, a dropped term or a swapped operand of the derivation fails this)."""
 import ctypes as C
 import os
 import re
@@ -48,13 +48,18 @@ void bwd(const double *in, double *out) { BwdIn i; BwdOut o; memcpy(&i, in, size
 CELL_SEEDS = [(i & 7) | (((i * 2654435761) >> 7 & 0x1FFF) << 3) for i in range(16)]
 
 
-@pytest.mark.parametrize("model", ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"] + [f"cell{s}" for s in CELL_SEEDS])
-def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, tmp_path):
+# (model, cell of the chain it is cut into)
+FD_CASES = [(m, 0) for m in ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"] + [f"cell{s}" for s in CELL_SEEDS]]
+FD_CASES += [("treegru", 0), ("treegru", 1)]
+
+
+@pytest.mark.parametrize("model,stage", FD_CASES)
+def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, stage, tmp_path):
     a = _declare(model)
-    src = _dump(0)
+    src = _dump(10 * stage)
     a.close()
     dims = {k: int(v) for k, v in re.findall(r"(\w+)=(\d+)", [l for l in src.splitlines() if l.startswith("// H=")][0])}
-    K, S, NX, XD, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "NX", "XD", "NP", "NB", "ND", "NSV"))
+    K, S, SI, NX, XD, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "SI", "NX", "XD", "NP", "NB", "ND", "NSV"))
     prod_col = [int(c) for c in re.findall(r"// product \d+ dcol (\d+)", src)]
     bias_col = [int(c) for c in re.findall(r"// bias \d+ dcol (\d+)", src)]
     assert len(prod_col) == NP and len(bias_col) == NB
@@ -66,7 +71,7 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
     sz = (C.c_int * 4)()
     lib.sizes(sz)
     nxm, nbm, nsvm, xdm = max(1, NX), max(1, NB), max(1, NSV), max(1, XD)
-    assert list(sz) == [nxm + NP + nbm + K * S + xdm, S + 1 + nsvm, S + 1 + nsvm + K * S, ND + K * S]
+    assert list(sz) == [nxm + NP + nbm + K * SI + xdm, S + 1 + nsvm, S + 1 + nsvm + K * SI, ND + K * SI]
     dp = C.POINTER(C.c_double)
 
     def fwd(x):
@@ -79,7 +84,7 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
         x = rng.normal(0, 0.8, sz[0])
         seed = rng.normal(0, 1, S + 1)  # d st[0..S), d ret
         out = fwd(x)
-        bin_ = np.concatenate([seed, out[S + 1:], x[nxm + NP + nbm:nxm + NP + nbm + K * S]])
+        bin_ = np.concatenate([seed, out[S + 1:], x[nxm + NP + nbm:nxm + NP + nbm + K * SI]])
         bout = np.zeros(sz[3])
         lib.bwd(bin_.ctypes.data_as(dp), bout.ctypes.data_as(dp))
         num = np.zeros(sz[0])
@@ -95,9 +100,9 @@ def test_derived_backward_part_equals_central_differences_of_the_forward_part(mo
             want[nxm + p] = bout[prod_col[p]]
         for i in range(NB):
             want[nxm + NP + i] = bout[bias_col[i]]
-        want[nxm + NP + nbm:nxm + NP + nbm + K * S] = bout[ND:]
+        want[nxm + NP + nbm:nxm + NP + nbm + K * SI] = bout[ND:]
         live = np.ones(sz[0], bool)
-        live[nxm + NP + nbm + K * S:] = False  # the pulled vertex input is a feed: no gradient is derived for it
+        live[nxm + NP + nbm + K * SI:] = False  # the pulled vertex input is a feed: no gradient is derived for it
         np.testing.assert_allclose(want[live], num[live], rtol=1e-6, atol=1e-8)
 
 
@@ -117,3 +122,17 @@ def test_what_is_not_of_the_general_shape_says_why():
     a = _declare("treelstm", H=40)
     assert "multiple of 32" in _dump(1)
     a.close()
+
+
+def test_a_tree_gru_is_cut_into_two_cells():
+    """The candidate's product reads r * (h_l + h_r), which depends on the products behind r: the
+    first cell writes [r * hs, z, z * hs] per vertex, the second gathers that row as the state of
+    its one child, multiplies its first block and writes h."""
+    a = _declare("treegru")
+    first, second, none = _dump(0), _dump(10), _dump(20)
+    dev = _dump(11)
+    a.close()
+    assert "// stages=2" in first and "K=2 S=3 SI=1 NX=3 XD=0 NP=2 NB=2" in first
+    assert "// stages=2" in second and "K=1 S=1 SI=3 NX=3 XD=0 NP=1 NB=1" in second
+    assert "no such stage" in none
+    assert "#define CELL_HAS_RET 1" in dev and "#define CELL_K 1" in dev

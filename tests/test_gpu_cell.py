@@ -1,7 +1,8 @@
-"""Vertex functions lowered onto kernels generated for them (the general one-stage shape): the
-reference's three applications forced onto that path, a Tree-LSTM with a forget-gate matrix per
-child and a gated cell with one state block, against the oracle (or, for the gated cell, the fp64
-autograd formulation of tests/textbook.py) on the same seeded inputs."""
+"""Vertex functions lowered onto kernels generated for them: the reference's three applications
+forced onto that path, a Tree-LSTM with a forget-gate matrix per child, a gated cell with one state
+block and a tree GRU (two stages of products: a chain of two cells), against the oracle (or, where
+the oracle has no restatement, the fp64 autograd formulation of tests/textbook.py) on the same
+seeded inputs."""
 import numpy as np
 import pytest
 
@@ -14,7 +15,7 @@ from tolerance import close
 pytestmark = pytest.mark.gpu
 
 NAMES = {"treelstm": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treelstm2": ("Emb", "W", "U", "Bv", "Wfc", "bfc"),
-         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",), "treefc_x": ("W", "Bv")}
+         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treegru": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",), "treefc_x": ("W", "Bv")}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -107,6 +108,26 @@ def test_a_gated_cell_with_one_state_block_against_fp64_autograd():
         assert got[3] == 2
         compare(got, want)
     compare(run_generated("treegate", w, "rowid", mode=0), want)
+
+
+@pytest.mark.parametrize("H", [32, 64, 128])
+def test_a_tree_gru_runs_as_a_chain_of_two_cells_against_fp64_autograd(H):
+    """The candidate's product takes r * (h_l + h_r) as its left operand, which depends on the
+    products behind r: two launches per round forward, four backward.  Held to the per-sample fp64
+    formulation under row-id pairing, and to the same program run operator by operator under the
+    reference's pairing."""
+    w = small_workload("treegru", 186, B=6, H=H, E=12, V=29, C=5)
+    want = textbook.per_sample("treegru", w["graph"], w["x"], w["labels"], w["params"], w["H"])
+    for mode in (1, 3):
+        got = run_generated("treegru", w, "rowid", mode=mode)
+        assert got[3] == 2
+        compare(got, want)
+    by_op = run_generated("treegru", w, "rowid", mode=0)
+    compare(by_op, want)
+    ref_pairing = run_generated("treegru", w, "reference", mode=0)
+    got = run_generated("treegru", w, "reference", mode=1)
+    assert got[3] == 2
+    compare(got, dict(loss=ref_pairing[0], graph_out=ref_pairing[1], grads=ref_pairing[2]))
 
 
 @pytest.mark.parametrize("seed", CELL_SEEDS)

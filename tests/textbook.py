@@ -92,6 +92,21 @@ def _treegate_cell(P, H, xid, hl, hr):
     return u * z + g - z * g
 
 
+def _treegru_cell(P, H, xid, hl, hr):
+    """Child-sum tree GRU: r, z = sigmoid(x W_{r,z} + (h_l + h_r) U_{r,z} + b_{r,z}),
+    c = tanh(x W_c + (r (h_l + h_r)) U_c + b_c), h = z (h_l + h_r) + (1 - z) c.  The candidate's product
+    takes a left operand that depends on another product of the same vertex."""
+    W, U, Bv = P["W"], P["U"], P["Bv"]
+    E = P["Emb"].shape[1]
+    U_r, U_z, U_c = (U[i * H * H : (i + 1) * H * H].reshape(H, H) for i in range(3))
+    xW = P["Emb"][xid] @ W.reshape(E, 3 * H)
+    hs = hl + hr
+    r = torch.sigmoid(xW[..., :H] + hs @ U_r + Bv[:H])
+    z = torch.sigmoid(xW[..., H : 2 * H] + hs @ U_z + Bv[H : 2 * H])
+    c = torch.tanh(xW[..., 2 * H :] + (r * hs) @ U_c + Bv[2 * H :])
+    return z * hs + (1 - z) * c
+
+
 def _lstm_cell(P, H, xid, hp, cp):
     Wf = P["W"]
     Ux = Wf[: 4 * H * H].reshape(H, 4 * H)
@@ -141,6 +156,10 @@ def per_sample(model, graph, x, labels, params, H, loss="softmax", act=0, use_bi
             hl = h[ch[0]] if ch else zero
             hr = h[ch[1]] if len(ch) > 1 else zero
             h[v] = _treegate_cell(P, H, int(xs[v]), hl, hr)
+        elif model == "treegru":
+            hl = h[ch[0]] if ch else zero
+            hr = h[ch[1]] if len(ch) > 1 else zero
+            h[v] = _treegru_cell(P, H, int(xs[v]), hl, hr)
         elif model == "lstm":
             hp, cp = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
             h[v], c[v] = _lstm_cell(P, H, int(xs[v]), hp, cp)
