@@ -109,7 +109,9 @@ def front_end_modes(pool, steps=60, warmup=30, only=None):
     generated for it (its shape recognised, not its identity), op by op with the fusion pass's
     generated kernels, and plain op by op -- the reference's execution model on this GPU.  For a
     Tree-LSTM workload also a vertex function no hand-written kernel covers (a forget-gate matrix per
-    child, same sizes): lowered onto generated kernels against op by op with the fusion pass."""
+    child, same sizes) and one whose products come in two stages (a child-sum tree GRU, which runs
+    as a chain of two generated cells): lowered onto generated kernels against op by op with the
+    fusion pass."""
     import torch
 
     from cavs_amd import apps, session, synth
@@ -122,7 +124,9 @@ def front_end_modes(pool, steps=60, warmup=30, only=None):
              ("op_by_op_fusion", w["model"], session.OPT_BATCHING | session.OPT_FUSION, 0), ("op_by_op", w["model"], session.OPT_BATCHING, 0)]
     if w["model"] == "treelstm":
         cases += [("fourth_function_lowered_generated", "treelstm2", session.OPT_BATCHING, 1),
-                  ("fourth_function_op_by_op_fusion", "treelstm2", session.OPT_BATCHING | session.OPT_FUSION, 0)]
+                  ("fourth_function_op_by_op_fusion", "treelstm2", session.OPT_BATCHING | session.OPT_FUSION, 0),
+                  ("two_stage_function_lowered_generated", "treegru", session.OPT_BATCHING, 1),
+                  ("two_stage_function_op_by_op_fusion", "treegru", session.OPT_BATCHING | session.OPT_FUSION, 0)]
     for name, model, opt, lowered in cases:
         if only and name != only:
             continue
@@ -132,6 +136,9 @@ def front_end_modes(pool, steps=60, warmup=30, only=None):
             params = {"W": params["W"]}
         if model == "treelstm2":  # [U_iou | U_fl | U_fr]
             params["U"] = np.concatenate([np.ravel(params["U"]), synth.SplitMix64(9).bulk_uniform(H * H, -0.1, 0.1)]).astype(np.float32)
+        if model == "treegru":  # three gates instead of four, one state block
+            rng = synth.SplitMix64(10)
+            params.update({k: rng.bulk_uniform(app.var_size(k), -0.1, 0.1) for k in ("W", "U", "Bv")})
         app.set_params(params)
         # untimed: at least `warmup` steps and 150 ms of continuous work (steady clocks, as in measure())
         # the same pool of batch structures as the headline measurement, cycled the same way

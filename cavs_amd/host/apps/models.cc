@@ -270,6 +270,44 @@ class TreeGRU : public GraphSupport {
   Sym U_r, U_z, U_c, b_r, b_z, b_c;
 };
 
+// Three stages of products that share operands across the stages: the first and the third multiply by
+// the same weight block and read the same block of x * W, the first and the second add the same bias.
+//   a = sigmoid(xW_0 + hs U_1 + b_1),  m = tanh(xW_1 + (a hs) U_2 + b_1),  q = tanh(xW_0 + m U_1 + b_2),
+//   h = a q + hs - a hs                                        with hs = h_l + h_r
+class TreeDeep : public GraphSupport {
+ public:
+  TreeDeep(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d) : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H) {
+    embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
+    W = Sym::Variable(DT_FLOAT, {2 * E * H}, Sym::Uniform(-0.1f, 0.1f));
+    U = Sym::Variable(DT_FLOAT, {2 * H * H}, Sym::Uniform(-0.1f, 0.1f));
+    B = Sym::Variable(DT_FLOAT, {2 * H}, Sym::Zeros());
+    U_1 = U.Slice(0, H * H).Reshape({H, H});
+    U_2 = U.Slice(H * H, H * H).Reshape({H, H});
+    b_1 = B.Slice(0, H);
+    b_2 = B.Slice(H, H);
+  }
+  void Node() override {
+    Sym hs = Gather(0, {H}) + Gather(1, {H});
+    Sym x = Pull(0, {1});
+    x = x.EmbeddingLookup(embedding.Mirror());
+    Sym xW = Sym::MatMul(x, W.Reshape({E, 2 * H}).Mirror()).Reshape({H * 2});
+    Sym xW_0, xW_1;
+    tie(xW_0, xW_1) = xW.Split2();
+    Sym a = (xW_0.Mirror() + Sym::MatMul(hs.Mirror().Reshape({1, H}), U_1.Mirror()).Reshape({H}) + b_1.Mirror()).Sigmoid();
+    Sym ah = a.Mirror() * hs.Mirror();
+    Sym m = (xW_1 + Sym::MatMul(ah.Mirror().Reshape({1, H}), U_2.Mirror()).Reshape({H}) + b_1.Mirror()).Tanh();
+    Sym q = (xW_0.Mirror() + Sym::MatMul(m.Reshape({1, H}), U_1.Mirror()).Reshape({H}) + b_2.Mirror()).Tanh();
+    Sym h = a.Mirror() * q + hs.Mirror() - ah.Mirror();
+    Scatter(h.Mirror());
+    Push(h.Mirror());
+  }
+  Sym embedding, W, U, B;
+
+ private:
+  int E, H;
+  Sym U_1, U_2, b_1, b_2;
+};
+
 // A family of vertex functions of the general one-stage shape, one per seed, for testing the
 // lowering onto generated kernels beyond the handful of named cells: one or two children, one or
 // two state blocks, three or four gates, each gate with its own recurrent weights applied to the
@@ -395,6 +433,10 @@ int cavs_app_create(const char *model, int B, int maxlen, int V, int E, int H, i
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model == "treegru") {
       auto *m = new TreeGRU(app->graph, app->vertex, d);
+      app->gs.reset(m);
+      app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
+    } else if (app->model == "treedeep") {
+      auto *m = new TreeDeep(app->graph, app->vertex, d);
       app->gs.reset(m);
       app->vars = {{"Emb", m->embedding}, {"W", m->W}, {"U", m->U}, {"Bv", m->B}};
     } else if (app->model.rfind("cell", 0) == 0) {

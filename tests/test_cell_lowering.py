@@ -50,7 +50,7 @@ CELL_SEEDS = [(i & 7) | (((i * 2654435761) >> 7 & 0x1FFF) << 3) for i in range(1
 
 # (model, cell of the chain it is cut into)
 FD_CASES = [(m, 0) for m in ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"] + [f"cell{s}" for s in CELL_SEEDS]]
-FD_CASES += [("treegru", 0), ("treegru", 1)]
+FD_CASES += [("treegru", 0), ("treegru", 1), ("treedeep", 0), ("treedeep", 1), ("treedeep", 2)]
 
 
 @pytest.mark.parametrize("model,stage", FD_CASES)

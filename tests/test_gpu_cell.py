@@ -15,7 +15,7 @@ from tolerance import close
 pytestmark = pytest.mark.gpu
 
 NAMES = {"treelstm": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treelstm2": ("Emb", "W", "U", "Bv", "Wfc", "bfc"),
-         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treegru": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",), "treefc_x": ("W", "Bv")}
+         "treegate": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treegru": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "treedeep": ("Emb", "W", "U", "Bv", "Wfc", "bfc"), "lstm": ("Emb", "W", "Bv", "Wfc", "bfc"), "treefc": ("W",), "treefc_x": ("W", "Bv")}
 
 
 @pytest.fixture(scope="module", autouse=True)
@@ -128,6 +128,19 @@ def test_a_tree_gru_runs_as_a_chain_of_two_cells_against_fp64_autograd(H):
     got = run_generated("treegru", w, "reference", mode=1)
     assert got[3] == 2
     compare(got, dict(loss=ref_pairing[0], graph_out=ref_pairing[1], grads=ref_pairing[2]))
+
+
+@pytest.mark.parametrize("H", [32, 128])
+def test_three_stages_that_share_a_weight_block_a_block_of_xw_and_a_bias(H):
+    """A chain of three cells whose weight gradients meet: the first and the third cell multiply by
+    the same block (the second's share is added one launch later), read the same block of x W
+    (likewise for d W and d e), and the first two add the same bias."""
+    w = small_workload("treedeep", 189, B=6, H=H, E=12, V=29, C=5)
+    want = textbook.per_sample("treedeep", w["graph"], w["x"], w["labels"], w["params"], w["H"])
+    got = run_generated("treedeep", w, "rowid", mode=1)
+    assert got[3] == 2
+    compare(got, want)
+    compare(run_generated("treedeep", w, "rowid", mode=0), want)
 
 
 @pytest.mark.parametrize("seed", CELL_SEEDS)

@@ -42,9 +42,10 @@ def small_workload(model, seed, B=5, H=12, E=10, V=37, C=5, skew=True):
         p = dict(Emb=rng.bulk_normal(V * E, 0, 0.5).reshape(V, E), W=rng.bulk_uniform(E * 2 * H, -0.4, 0.4),
                  U=rng.bulk_uniform(3 * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(2 * H, -0.3, 0.3))
         x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
-    elif model == "treegru":  # (textbook._treegru_cell: two stages of products, no oracle restatement)
-        p = dict(Emb=rng.bulk_normal(V * E, 0, 0.5).reshape(V, E), W=rng.bulk_uniform(E * 3 * H, -0.4, 0.4),
-                 U=rng.bulk_uniform(3 * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(3 * H, -0.3, 0.3))
+    elif model in ("treegru", "treedeep"):  # (textbook._treegru_cell, _treedeep_cell: two and three stages of products, no oracle restatement)
+        g = 3 if model == "treegru" else 2
+        p = dict(Emb=rng.bulk_normal(V * E, 0, 0.5).reshape(V, E), W=rng.bulk_uniform(E * g * H, -0.4, 0.4),
+                 U=rng.bulk_uniform(g * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(g * H, -0.3, 0.3))
         x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
     elif model == "lstm":
         p = dict(Emb=rng.bulk_normal(V * H, 0, 0.5).reshape(V, H),

@@ -107,6 +107,21 @@ def _treegru_cell(P, H, xid, hl, hr):
     return z * hs + (1 - z) * c
 
 
+def _treedeep_cell(P, H, xid, hl, hr):
+    """Three stages of products sharing a weight block, a block of x W and a bias across stages:
+    a = sigmoid(xW_0 + hs U_1 + b_1), m = tanh(xW_1 + (a hs) U_2 + b_1), q = tanh(xW_0 + m U_1 + b_2),
+    h = a q + (1 - a) hs."""
+    W, U, Bv = P["W"], P["U"], P["Bv"]
+    E = P["Emb"].shape[1]
+    U_1, U_2 = (U[i * H * H : (i + 1) * H * H].reshape(H, H) for i in range(2))
+    xW = P["Emb"][xid] @ W.reshape(E, 2 * H)
+    hs = hl + hr
+    a = torch.sigmoid(xW[..., :H] + hs @ U_1 + Bv[:H])
+    m = torch.tanh(xW[..., H:] + (a * hs) @ U_2 + Bv[:H])
+    q = torch.tanh(xW[..., :H] + m @ U_1 + Bv[H:])
+    return a * q + (1 - a) * hs
+
+
 def _lstm_cell(P, H, xid, hp, cp):
     Wf = P["W"]
     Ux = Wf[: 4 * H * H].reshape(H, 4 * H)
@@ -156,10 +171,10 @@ def per_sample(model, graph, x, labels, params, H, loss="softmax", act=0, use_bi
             hl = h[ch[0]] if ch else zero
             hr = h[ch[1]] if len(ch) > 1 else zero
             h[v] = _treegate_cell(P, H, int(xs[v]), hl, hr)
-        elif model == "treegru":
+        elif model in ("treegru", "treedeep"):
             hl = h[ch[0]] if ch else zero
             hr = h[ch[1]] if len(ch) > 1 else zero
-            h[v] = _treegru_cell(P, H, int(xs[v]), hl, hr)
+            h[v] = (_treegru_cell if model == "treegru" else _treedeep_cell)(P, H, int(xs[v]), hl, hr)
         elif model == "lstm":
             hp, cp = (h[ch[0]], c[ch[0]]) if ch else (zero, zero)
             h[v], c[v] = _lstm_cell(P, H, int(xs[v]), hp, cp)
