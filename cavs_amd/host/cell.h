@@ -1,4 +1,5 @@
-// Description of a vertex function of the general one-stage shape
+// Description of a vertex function of the general shape (one stage of products; several stages are
+// a chain of such descriptions, see CellSpec::next)
 //
 //   state' , ret = f( x*W , sum_t A_t * B_t , bias , states of the children )      (f elementwise)
 //

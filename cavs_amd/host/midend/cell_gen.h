@@ -1,6 +1,7 @@
-// Lowering of a vertex function of the general one-stage shape onto generated round kernels:
+// Lowering of a vertex function of the general shape onto generated round kernels:
 // recognises  act(sum_i Gather_i * W_i + Pull * W + b)  with any elementwise tail over the
-// pre-activations and the children's states, derives the elementwise part of the backward
+// pre-activations and the children's states, cuts a function whose products depend on each other
+// into a chain of such cells, derives the elementwise part of each one's backward
 // function, and writes the kernels' source (the product loops for this function's operands plus
 // the two elementwise parts).  The counterpart of the reference's parser + code generator
 // (cavs/midend/runtime_compiler/parser.cc:73-139, code_generator.cc:104-185) for a whole F.

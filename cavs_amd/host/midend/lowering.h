@@ -1,7 +1,7 @@
 // Recognition of the vertex functions the engine runs on fused round kernels.  A user's F is
 // lowered onto cavs::Engine when its operator graph is the same computation as one of the
 // templates with hand-written kernels (binary Tree-LSTM, chain LSTM, Tree-FC: same operators, same
-// wiring, same attributes), or, failing that, when it has the general one-stage shape that
+// wiring, same attributes), or, failing that, when it has the general shape that
 // generated kernels cover (cell_gen.h) -- everything else runs op by op.
 #ifndef CAVS_HOST_MIDEND_LOWERING_H_
 #define CAVS_HOST_MIDEND_LOWERING_H_

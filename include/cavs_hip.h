@@ -603,7 +603,8 @@ int cavs_fused_launch(void *handle, float *const *outs, int nouts, const float *
                       int nins, const int *out_counts, const int *in_counts, int n_elements,
                       void *stream);
 int cavs_fused_release(void *handle);
-/* The round kernels generated for a vertex function of the general one-stage shape (the reference
+/* The round kernels generated for a vertex function of the general shape, or for one cell of the
+ * chain it is cut into (the reference
  * fuses the elementwise operators of F into generated kernels, cavs/midend/runtime_compiler/
  * code_generator.cc:104-185, and runs them through cavs/backend/op_impl_fused_kernel.cu:34-64; here
  * the products of F are inside the generated kernels too).  `source` defines the extern "C" kernels
