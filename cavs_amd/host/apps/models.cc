@@ -312,11 +312,14 @@ class TreeDeep : public GraphSupport {
 // lowering onto generated kernels beyond the handful of named cells: one or two children, one or
 // two state blocks, three or four gates, each gate with its own recurrent weights applied to the
 // first child's h, the last child's h, the sum or the concatenation of the children's h, sigmoid
-// or tanh per gate.  Every tensor that is used more than once goes through Mirror().
+// or tanh per gate.  Bits 16-17 of the seed add stages of products: the last gate then multiplies
+// the first gate times its operand (two stages), and the one before it the last gate times its
+// operand (three).  Every tensor that is used more than once goes through Mirror().
 class RandomCell : public GraphSupport {
  public:
   RandomCell(const Sym &graph_ph, const Sym &vertex_ph, const Dims &d, unsigned seed)
-      : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H), K(1 + (seed & 1)), S(1 + ((seed >> 1) & 1)), NG(3 + ((seed >> 2) & 1)) {
+      : GraphSupport(graph_ph, vertex_ph), E(d.E), H(d.H), K(1 + (seed & 1)), S(1 + ((seed >> 1) & 1)), NG(3 + ((seed >> 2) & 1)),
+        deep(std::min(2u, (seed >> 16) & 3)) {
     embedding = Sym::Variable(DT_FLOAT, {d.V, E}, Sym::Uniform(-0.1f, 0.1f));
     W = Sym::Variable(DT_FLOAT, {NG * E * H}, Sym::Uniform(-0.1f, 0.1f));
     int usize = 0;
@@ -345,12 +348,20 @@ class RandomCell : public GraphSupport {
     x = x.EmbeddingLookup(embedding.Mirror());
     Sym xW = Sym::MatMul(x, W.Reshape({E, NG * H}).Mirror()).Reshape({NG * H});
     Sym gate[4];
-    for (int g = 0; g < NG; g++) {
+    // the gates in the order of their stages: those over the children's states, then the last one
+    // (over the first gate times the states), then the one before it (over the last gate times them)
+    int order[4], scaled_by[4], n = 0;
+    for (int g = 0; g < NG - deep; g++) order[n] = g, scaled_by[n++] = -1;
+    if (deep >= 1) order[n] = NG - 1, scaled_by[n++] = 0;
+    if (deep >= 2) order[n] = NG - 2, scaled_by[n++] = NG - 1;
+    for (int i = 0; i < NG; i++) {
+      const int g = order[i], by = scaled_by[i];
+      auto part = [&](int k) { return by < 0 ? h[k].Mirror() : gate[by].Mirror() * h[k].Mirror(); };
       Sym a;
-      if (K == 1 || src[g] == 0) a = h[0].Mirror();
-      else if (src[g] == 1) a = h[1].Mirror();
-      else if (src[g] == 2) a = h[0].Mirror() + h[1].Mirror();
-      else a = Sym::Concat({h[0].Mirror(), h[1].Mirror()});
+      if (K == 1 || src[g] == 0) a = part(0);
+      else if (src[g] == 1) a = part(1);
+      else if (src[g] == 2) a = part(0) + part(1);
+      else a = Sym::Concat({part(0), part(1)});
       Sym pre = xW.Slice(g * H, H) + Sym::MatMul(a.Reshape({1, rows[g]}), Ug[g].Mirror()).Reshape({H}) + bg[g].Mirror();
       gate[g] = tanh_[g] ? pre.Tanh() : pre.Sigmoid();
     }
@@ -373,7 +384,7 @@ class RandomCell : public GraphSupport {
   int children() const { return K; }
 
  private:
-  int E, H, K, S, NG;
+  int E, H, K, S, NG, deep;
   int src[4], tanh_[4], rows[4];
   Sym Ug[4], bg[4];
 };

@@ -48,16 +48,27 @@ void bwd(const double *in, double *out) { BwdIn i; BwdOut o; memcpy(&i, in, size
 CELL_SEEDS = [(i & 7) | (((i * 2654435761) >> 7 & 0x1FFF) << 3) for i in range(16)]
 
 
-# (model, cell of the chain it is cut into)
-FD_CASES = [(m, 0) for m in ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x"] + [f"cell{s}" for s in CELL_SEEDS]]
-FD_CASES += [("treegru", 0), ("treegru", 1), ("treedeep", 0), ("treedeep", 1), ("treedeep", 2)]
+# members of the family with two or three stages of products (bits 16-17), which run as chains of cells
+CHAIN_SEEDS = [(1 + i % 2) << 16 | (i * 5 + 3) & 7 | (((i * 2246822519) >> 9 & 0x1FFF) << 3) for i in range(10)]
+FD_MODELS = ["treelstm", "treelstm2", "treegate", "lstm", "treefc", "treefc_x", "treegru", "treedeep"] + [f"cell{s}" for s in CELL_SEEDS + CHAIN_SEEDS]
 
 
-@pytest.mark.parametrize("model,stage", FD_CASES)
-def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, stage, tmp_path):
+@pytest.mark.parametrize("model", FD_MODELS)
+def test_derived_backward_part_equals_central_differences_of_the_forward_part(model, tmp_path):
+    """Every cell of the chain F is cut into (one cell for a function of one stage)."""
     a = _declare(model)
-    src = _dump(10 * stage)
+    srcs = [_dump(0)]
+    stages = int(re.search(r"// stages=(\d+)", srcs[0]).group(1))
+    srcs += [_dump(10 * st) for st in range(1, stages)]
     a.close()
+    want_stages = {"treegru": 2, "treedeep": 3}.get(model, 1 + (int(model[4:]) >> 16 & 3) if model.startswith("cell") else 1)
+    assert stages == want_stages
+    for st, src in enumerate(srcs):
+        _held_to_central_differences(src, tmp_path / str(st))
+
+
+def _held_to_central_differences(src, tmp_path):
+    tmp_path.mkdir()
     dims = {k: int(v) for k, v in re.findall(r"(\w+)=(\d+)", [l for l in src.splitlines() if l.startswith("// H=")][0])}
     K, S, SI, NX, XD, NP, NB, ND, NSV = (dims[k] for k in ("K", "S", "SI", "NX", "XD", "NP", "NB", "ND", "NSV"))
     prod_col = [int(c) for c in re.findall(r"// product \d+ dcol (\d+)", src)]

@@ -8,7 +8,7 @@ import pytest
 
 import textbook
 from cavs_amd import apps, session, synth
-from test_cell_lowering import CELL_SEEDS
+from test_cell_lowering import CELL_SEEDS, CHAIN_SEEDS
 from test_oracle_models import small_workload
 from tolerance import close
 
@@ -143,13 +143,14 @@ def test_three_stages_that_share_a_weight_block_a_block_of_xw_and_a_bias(H):
     compare(run_generated("treedeep", w, "rowid", mode=0), want)
 
 
-@pytest.mark.parametrize("seed", CELL_SEEDS)
+@pytest.mark.parametrize("seed", CELL_SEEDS + CHAIN_SEEDS)
 def test_a_family_of_cells_lowered_and_op_by_op(seed):
     """cell<seed>: one or two children, one or two state blocks, three or four gates over the first
-    child, the last child, the children's sum or their concatenation, sigmoid or tanh each.  No
-    restatement of these exists anywhere else: the generated kernels are held to the same program
-    run operator by operator (each operator of which the oracle pins), and the two backward forms
-    to each other."""
+    child, the last child, the children's sum or their concatenation, sigmoid or tanh each; for
+    the chain seeds one or two of the gates over another gate times those (two or three stages of
+    products).  No restatement of these exists anywhere else: the generated kernels are held to
+    the same program run operator by operator (each operator of which the oracle pins), and the
+    two backward forms to each other."""
     two = seed & 1
     H, E, V, C_ = 64, 12, 29, 5
     w = small_workload("treelstm" if two else "lstm", 190 + seed % 7, B=6, H=H, E=E, V=V, C=C_)
@@ -162,7 +163,11 @@ def test_a_family_of_cells_lowered_and_op_by_op(seed):
                      allow_fused=mode)
         if mode == 1:
             sizes = {k: a.var_size(k) for k in ("Emb", "W", "U", "Bv")}
-            p = {k: rng.bulk_uniform(n, -0.4, 0.4) for k, n in sizes.items()}
+            # (a chain's stages multiply one after the other: with +-0.4 at H = 64 the gain per stage is
+            # about 3 and the two paths' fp32 summation orders show, up to 5e-4 relative in single
+            # entries of one seed's gradients; with +-0.2 every tensor stays within 2 % of the tolerance)
+            amp = 0.2 if seed >> 16 else 0.4
+            p = {k: rng.bulk_uniform(n, -amp, amp) for k, n in sizes.items()}
             p["Wfc"], p["bfc"] = w["params"]["Wfc"], w["params"]["bfc"]
         a.set_params(p)
         print(f"[case] cell{seed} children={1 + two} N={w['N']} lowering mode={mode}", flush=True)
