@@ -114,6 +114,15 @@ enum CellArg {
   CA_X,          // float*  the vertex input by vertex id [*, XD*H]
   CA_POOL_IN,    // float*  the rows this cell gathers its children's states from [*, SI*H] (a function of one stage: CA_POOL)
   CA_DPOOL_IN,   // float*  gradient of those rows (cell_bwd_pool writes it; a function of one stage: CA_DPOOL)
+  // the cell whose rows this one gathers (itself for a function of one stage; in a chain the cell
+  // before, and for the first cell the last): cell_bwd runs the elementwise part of its backward
+  // function on the message gradients its products complete
+  CA_FT_SV,      // float*  that cell's kept values
+  CA_FT_D,       // float*  its gradient rows
+  CA_FT_DS,      // float*  elementwise part of the gradients of the rows it gathers, by slab row
+  CA_FT_POOL_IN, // float*  the rows it gathers
+  CA_FT_CHILD,   // int*    rows of those by slab row
+  CA_FT_KIDS,    // int*    slab rows of its children by slab row
   CA_OFF,        // long    first slab row of the round
   CA_N,          // long    rows
   CA_PARAM0,     // float*  parameters, then their gradients, in CellSpec::params order

@@ -405,7 +405,7 @@ void Engine::reserve_edges() {
       R(st.d, cap * k.ND * H);                  // the gradient rows
       // elementwise part of the message gradients: by slab row (one launch per backward round), or
       // by row of the round and child (two launches)
-      R(st.ds, std::max(cells_.size() == 1 ? cap * k.SI * H : (size_t)0, rc * k.K * k.SI * H));
+      R(st.ds, std::max(cap * k.SI * H, rc * k.K * k.SI * H));
       R(st.bt, (size_t)2 * k.blocks() * H * H);  // the weight blocks tile-major, as they are and transposed
       R(st.colsum, (size_t)k.ND * H);
       if (ci + 1 < cells_.size()) {
@@ -1740,7 +1740,18 @@ void Engine::cell_launch(int ci, int k, unsigned gx, unsigned gy, unsigned gz, u
   a[CA_POOL_IN].p = first ? pool_.get() : cells_[ci - 1].rows.get();
   a[CA_CHILD].p = first ? d_child_ : cell_iota_.get();
   a[CA_DPOOL_IN].p = first ? dpool_.get() : cells_[ci - 1].drows.get();
-  a[CA_KIDS].p = d_kid_rows_;
+  a[CA_KIDS].p = first ? d_kid_rows_ : cell_iota_.get();
+  {
+    // the cell whose rows this one gathers
+    const int pi = first ? (int)cells_.size() - 1 : ci - 1;
+    CellStage &ft = cells_[pi];
+    a[CA_FT_SV].p = ft.sv.get();
+    a[CA_FT_D].p = ft.d.get();
+    a[CA_FT_DS].p = ft.ds.get();
+    a[CA_FT_POOL_IN].p = pi == 0 ? pool_.get() : cells_[pi - 1].rows.get();
+    a[CA_FT_CHILD].p = pi == 0 ? d_child_ : cell_iota_.get();
+    a[CA_FT_KIDS].p = pi == 0 ? d_kid_rows_ : cell_iota_.get();
+  }
   a[CA_T2J].p = d_t2j_;
   a[CA_ROWS].p = rows;
   a[CA_XW].p = xW_.get();
@@ -1825,27 +1836,31 @@ void Engine::cell_backward() {
         c_launches_ += 1;
       }
   }
-  if (forest_ && L == 1) {
-    // every message is read exactly once: a round's launch hands d(state) on to the children of its
-    // rows and runs their elementwise part at once; the vertices without a reader go first
-    const unsigned block = 64u * c0.waves;
+  if (forest_) {
+    // every message is read exactly once: a cell's launch completes the gradient of the rows it
+    // gathered -- the states of the round's children for the first cell, the rows of the cell before
+    // for the others -- and runs the elementwise part of the cell that wrote them at once.  The
+    // vertices without a reader go first.
     if (n_orphans_ > 0) {
       ProfScope ps(this, K_GATES);
-      cell_launch(0, CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
+      cell_launch(L - 1, CK_BWD_ROWS, (unsigned)(((size_t)n_orphans_ * H + 255) / 256), 1, 1, 256, 0, n_orphans_, d_orphans_, d_dgo_);
     }
     for (int k : sched_->bwd_rounds) {
       const Round &r = sched_->rounds[k];
       c_gather_rows_ += r.n;
-      if (leaf_round(r)) continue;
-      ProfScope ps(this, K_ROUND);
-      cell_launch(0, CK_BWD, H / 16, (r.n + 15) / 16, 1, block, r.offset, r.n, nullptr, d_dgo_);
-      c_round_flops_ += 2.0 * r.n * c0.terms() * H * H;
-      c_scatter_rows_ += (double)c0.K * r.n;
+      for (int ci = L - 1; ci >= 0; ci--) {
+        if (ci == 0 && leaf_round(r)) continue;
+        const CellSpec &c = *cells_[ci].spec;
+        ProfScope ps(this, K_ROUND);
+        cell_launch(ci, CK_BWD, H / 16, (r.n + 15) / 16, 1, 64u * c.waves, r.offset, r.n, nullptr, d_dgo_);
+        c_round_flops_ += 2.0 * r.n * c.terms() * H * H;
+        c_scatter_rows_ += (double)c.K * r.n;
+      }
     }
   } else {
-    // any other batch, and every chain: two launches per round and cell, the message gradients
-    // going through the gradient of the rows the cells write, as in the reference (rows of the
-    // message pool nobody wrote read as zero)
+    // any other batch: two launches per round and cell, the message gradients going through the
+    // gradient of the rows the cells write, as in the reference (rows of the message pool nobody
+    // wrote read as zero)
     check(cavs_zero(dpool_.get(), (size_t)N * mw_ * 4, stream_));
     c_launches_ += 1;
     for (int k : sched_->bwd_rounds) {

@@ -535,7 +535,8 @@ struct Writer {
       << dv.ds_mask << "\n#define CELL_BWD_CS " << (dv.reads_cs ? 1 : 0) << "\n";
     o << "typedef float f4 __attribute__((ext_vector_type(4)));\n";
     o << "struct CellArgs {\n  float *pool;\n  const int *child, *pair, *kids, *t2j, *rows;\n  const float *xw;\n"
-         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  const float *x;\n  float *pool_in, *dpool_in;\n  long off, n;\n  float *p["
+         "  float *sv, *asrc, *go, *d, *ds, *bt, *colsum, *dpool;\n  const float *x;\n  float *pool_in, *dpool_in;\n"
+         "  float *ft_sv, *ft_d, *ft_ds;\n  const float *ft_pool_in;\n  const int *ft_child, *ft_kids;\n  long off, n;\n  float *p["
       << 2 * CA_MAX_PARAMS << "];\n};\n";
     o << "static __device__ inline f4 ld4(const float *p) { return *reinterpret_cast<const f4 *>(p); }\n";
   }
@@ -820,8 +821,9 @@ struct Chain {
   }
 };
 
-// the source of one cell's kernels
-void write_cell(Body &c, const Derived &d, int nfwd) {
+// the source of one cell's kernels; `ft`: the cell whose rows this one gathers, when it is another
+// one (a chain), with what was derived for it
+void write_cell(Body &c, const Derived &d, int nfwd, const Body *ft, const Derived *ftd, int ft_nfwd) {
   CellSpec &s = c.spec;
   const int H = s.H;
   s.waves = H % 128 == 0 ? 4 : H % 64 == 0 ? 2 : 1;
@@ -831,6 +833,21 @@ void write_cell(Body &c, const Derived &d, int nfwd) {
   Writer w(c, d, true);
   w.kernels();
   w.elementwise(nfwd);
+  if (ft) {
+    const CellSpec &f = ft->spec;
+    if (f.S != s.SI) no("internal: a cell gathers other rows than the cell before it writes");
+    w.o << "#define FT_K " << f.K << "\n#define FT_S " << f.S << "\n#define FT_SI " << f.SI << "\n#define FT_NSV " << f.NSV << "\n#define FT_ND " << f.ND
+        << "\n#define FT_DS_MASK " << ftd->ds_mask << "\n#define FT_BWD_CS " << (ftd->reads_cs ? 1 : 0) << "\n#define FT_HAS_RET " << (f.has_ret ? 1 : 0)
+        << "\nnamespace ft {\n";
+    Writer other(*ft, *ftd, true);
+    other.elementwise(ft_nfwd);
+    w.o << other.o.str() << "}  // namespace ft\n";
+  } else {
+    w.o << "#define FT_K CELL_K\n#define FT_S CELL_S\n#define FT_SI CELL_SI\n#define FT_NSV CELL_NSV\n#define FT_ND CELL_ND\n"
+           "#define FT_DS_MASK CELL_DS_MASK\n#define FT_BWD_CS CELL_BWD_CS\n#define FT_HAS_RET CELL_HAS_RET\n"
+           "namespace ft {\ntypedef ::BwdIn BwdIn;\ntypedef ::BwdOut BwdOut;\n"
+           "static __device__ inline void cell_backward(const BwdIn &in, BwdOut &out) { ::cell_backward(in, out); }\n}  // namespace ft\n";
+  }
   w.product_loops();
   w.o << kTemplate;
   s.source = w.o.str();
@@ -870,8 +887,10 @@ std::unique_ptr<CellMatch> match_cell(const Graph &g, std::string *why) {
   try {
     Chain b(g);
     std::shared_ptr<CellSpec> head, tail;
-    for (size_t i = 0; i < b.cells.size(); i++) {
-      write_cell(b.cells[i], b.derived[i], b.nfwd[i]);
+    const size_t L = b.cells.size();
+    for (size_t i = 0; i < L; i++) {
+      const size_t p = (i + L - 1) % L;  // whose rows cell i gathers
+      write_cell(b.cells[i], b.derived[i], b.nfwd[i], L > 1 ? &b.cells[p] : nullptr, L > 1 ? &b.derived[p] : nullptr, b.nfwd[p]);
       auto spec = std::make_shared<CellSpec>(b.cells[i].spec);
       if (tail) tail->next = spec;
       else head = spec;

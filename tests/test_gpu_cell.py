@@ -113,7 +113,8 @@ def test_a_gated_cell_with_one_state_block_against_fp64_autograd():
 @pytest.mark.parametrize("H", [32, 64, 128])
 def test_a_tree_gru_runs_as_a_chain_of_two_cells_against_fp64_autograd(H):
     """The candidate's product takes r * (h_l + h_r) as its left operand, which depends on the
-    products behind r: two launches per round forward, four backward.  Held to the per-sample fp64
+    products behind r: two launches per round and direction (four backward when the message flow
+    is no forest, which mode 3 forces).  Held to the per-sample fp64
     formulation under row-id pairing, and to the same program run operator by operator under the
     reference's pairing."""
     w = small_workload("treegru", 186, B=6, H=H, E=12, V=29, C=5)
@@ -137,9 +138,10 @@ def test_three_stages_that_share_a_weight_block_a_block_of_xw_and_a_bias(H):
     (likewise for d W and d e), and the first two add the same bias."""
     w = small_workload("treedeep", 189, B=6, H=H, E=12, V=29, C=5)
     want = textbook.per_sample("treedeep", w["graph"], w["x"], w["labels"], w["params"], w["H"])
-    got = run_generated("treedeep", w, "rowid", mode=1)
-    assert got[3] == 2
-    compare(got, want)
+    for mode in (1, 3):
+        got = run_generated("treedeep", w, "rowid", mode=mode)
+        assert got[3] == 2
+        compare(got, want)
     compare(run_generated("treedeep", w, "rowid", mode=0), want)
 
 
