@@ -202,3 +202,30 @@ def test_training_steps_on_generated_kernels_update_variables_like_the_oracle(or
     close(a.grad("U", p["U"].shape, grad=False), p["U"], "U after 3 steps")
     close(a.grad("Bv", p["Bv"].shape, grad=False), p["Bv"], "Bv after 3 steps")
     a.close()
+
+
+@pytest.mark.parametrize("model", ["treegru", "treedeep"])
+def test_training_steps_of_a_chain_of_cells_over_changing_batches(model):
+    """Three SGD steps, each on another batch (other trees, other words): what a step leaves behind
+    -- the rows of the embedding gradient it touched, bias and weight gradients that several cells
+    add their shares to -- must not show in the next one.  Held to fp64 autograd step by step."""
+    H, E, V, C_ = 64, 10, 23, 4
+    lr = 0.2
+    batches = [small_workload(model, 300 + i, B=5, H=H, E=E, V=V, C=C_) for i in range(3)]
+    B = max(b["graph"].shape[0] for b in batches)
+    maxlen = max(b["graph"].shape[1] for b in batches)
+    a = apps.App(model, B=B, maxlen=maxlen, H=H, E=E, V=V, C_=C_, opt=session.OPT_BATCHING, lr=lr, pairing="rowid")
+    p = {k: np.array(batches[0]["params"][k], np.float64) for k in NAMES[model]}
+    a.set_params({k: v.astype(np.float32) for k, v in p.items()})
+    for step, w in enumerate(batches):
+        assert w["graph"].shape == (B, maxlen)
+        print(f"[case] {model} on a chain of cells, sgd step {step}, N={w['N']}", flush=True)
+        want = textbook.per_sample(model, w["graph"], w["x"], w["labels"], {k: v.astype(np.float32) for k, v in p.items()}, H)
+        loss, _ = a.step(w["graph"], w["x"], w["labels"], train=True)
+        assert a.fused_kind == 2
+        close(loss, want["loss"], f"loss at step {step}")
+        for k in NAMES[model]:
+            p[k] = p[k] - lr * want["grads"]["d" + k].reshape(p[k].shape)
+    for k in NAMES[model]:
+        close(a.grad(k, p[k].shape, grad=False), p[k], f"{k} after 3 steps")
+    a.close()
