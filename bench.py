@@ -210,7 +210,7 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
     kw = model_kwargs(w0)
     s = session.Session(w0["model"], H=w0["H"], E=w0["E"], V=w0["V"], C_=w0["C"], pairing=a.pairing,
                         opt=session.OPT_BATCHING, fused_round_rows=a.fused_round_rows, schedule=schedule,
-                        plan_cache=plan_cache, tail_rows=a.tail_rows, graph_replay=graph_replay, **kw)
+                        plan_cache=plan_cache, tail_rows=a.tail_rows, graph_replay=graph_replay, head_chunks=a.head_chunks, **kw)
     s.set_params(w0["params"])
     feeds = []
     for w in pool:  # inputs resident in HBM before the timed region
@@ -385,6 +385,8 @@ def main():
     ap.add_argument("--tail-rows", type=int, default=0,
                     help="Tree-LSTM, H = 512: rounds whose rows can be dealt to eight groups with at most this many rows each run "
                          "inside one launch per direction (0: default limit, -1: one launch per round)")
+    ap.add_argument("--head-chunks", type=int, default=0,
+                    help="the loss head of a wide classifier (C4): 0 = in two chunks beside the backward rounds, 2..4 = in that many, negative = in one piece between the two passes")
     ap.add_argument("--also", default="C1,C2,C4,C5",
                     help="further workloads measured with few steps and reported under 'also' (C5 is the large "
                          "Tree-LSTM configuration, where rounds are GEMM-sized); 'none' to skip")

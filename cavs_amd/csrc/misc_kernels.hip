@@ -335,10 +335,15 @@ int cavs_bias_add_rows(float *out, const float *inp, const float *bias, int n, i
 
 int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const float *labels, int n,
                       int C, void *stream) {
-  CAVS_REQUIRE(n >= 0 && C > 0, "cavs_softmax_xent: bad shape n=%d C=%d", n, C);
+  return cavs_softmax_xent_part(loss, dlogits, logits, labels, n, C, n, stream);
+}
+
+int cavs_softmax_xent_part(float *loss, float *dlogits, const float *logits, const float *labels, int n,
+                           int C, int n_total, void *stream) {
+  CAVS_REQUIRE(n >= 0 && C > 0 && n_total >= n, "cavs_softmax_xent: bad shape n=%d of %d C=%d", n, n_total, C);
   if (n == 0) return CAVS_OK;
   CAVS_REQUIRE(logits && labels, "cavs_softmax_xent: null pointer");
-  const float inv_n = 1.f / (float)n;
+  const float inv_n = 1.f / (float)n_total;
   hipStream_t st = as_stream(stream);
   // wide rows: a workgroup per row with the row in registers; narrow ones: a wavefront per row
   if (C >= 512 && C % 4 == 0 && C <= 16384 && aligned16(logits) && (!dlogits || aligned16(dlogits))) {

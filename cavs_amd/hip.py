@@ -91,6 +91,7 @@ _SIGS = {
     "cavs_embed_bwd": [_P, _P, _P, _I, _I, _I, _P],
     "cavs_bias_add_rows": [_P, _P, _P, _I, _I, _P],
     "cavs_softmax_xent": [_P, _P, _P, _P, _I, _I, _P],
+    "cavs_softmax_xent_part": [_P, _P, _P, _P, _I, _I, _I, _P],
     "cavs_sgd": [_P, _P, _F, _Z, _P],
     "cavs_ew_binary": [_I, _P, _P, _Z, _P, _Z, _Z, _I, _P],
     "cavs_ew_unary": [_I, _P, _P, _Z, _I, _P],

@@ -166,6 +166,8 @@ Engine::~Engine() {
     cavs_event_destroy(aux_fork_ev_);
     cavs_event_destroy(aux_join_ev_);
   }
+  for (void *e : chunk_done_ev_)
+    if (e) cavs_event_destroy(e);
   for (auto &d : dsched_)
     if (d.free_ev) cavs_event_destroy(d.free_ev);
   if (own_stream_) cavs_stream_destroy(stream_);
@@ -363,6 +365,18 @@ void Engine::ensure(DeviceArray<float> &a, size_t n) {
   a.reserve(n);
 }
 
+// the identity list 0, 1, 2, ... of at least n entries
+void Engine::ensure_iota(size_t n) {
+  if (cell_iota_n_ >= n) return;
+  std::vector<int> iota(n);
+  for (size_t i = 0; i < n; i++) iota[i] = (int)i;
+  sync();
+  cell_iota_.reserve(n);
+  check(cavs_memcpy_h2d(cell_iota_.get(), iota.data(), n * 4, stream_));
+  check(cavs_stream_sync(stream_));
+  cell_iota_n_ = n;
+}
+
 // ------------------------------------------------------------------ memory manager
 // Every edge of F is a [rows, width] buffer in which round r lives at rows
 // [offset_r, offset_r + n_r): row index == tensor id for every edge, and forward
@@ -413,15 +427,7 @@ void Engine::reserve_edges() {
         R(st.drows, cap * k.S * H);
       }
     }
-    if (cells_.size() > 1 && cell_iota_n_ < cap) {
-      std::vector<int> iota(cap);
-      for (size_t i = 0; i < cap; i++) iota[i] = (int)i;
-      check(cavs_stream_sync(stream_));
-      cell_iota_.reserve(cap);
-      check(cavs_memcpy_h2d(cell_iota_.get(), iota.data(), cap * 4, stream_));
-      check(cavs_stream_sync(stream_));
-      cell_iota_n_ = cap;
-    }
+    if (cells_.size() > 1) ensure_iota(cap);
   } else if (cfg_.model != CAVS_MODEL_TREEFC) {
     R(xs_, cap);
     if (xs_prev_.capacity() < cap) {  // the list of dirty rows does not survive a reallocation
@@ -506,6 +512,7 @@ void Engine::upload_index_arena() {
   std::string err = build_index_lists(s, nch_, cfg_.pairing, t2j, pair, child, roots);
   if (!err.empty()) fail(CAVS_EUNSUPPORTED, err);
   forest_ = want_forest && build_forest_lists(s, nch_, fused_rows(), pair, child, roots + s.B, roots + s.B + (size_t)nch_ * N, &n_orphans_);
+  plan_head_chunks(roots + s.B + (size_t)nch_ * N);
   tail_ = TailPlan();
   int *tail_rows = roots + s.B + (size_t)N * (nch_ + 1);
   if (want_tail && forest_) build_tail_plan(roots + s.B, tail_rows);
@@ -751,6 +758,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
   c_round_flops_ = 0;
   c_tail_rounds_ = c_tail_launches_ = 0;
   bias_jobs_.clear();
+  head_chunks_.clear();  // (planned with the host scheduler's lists only)
   pending_tasks_.clear();  // (a step that failed half way may have left a job for a backward pass that never ran)
   wait_ms_ = 0.f;
   uint64_t hash = 0;
@@ -809,6 +817,7 @@ void Engine::forward_only(const int *graph, int B, int maxlen, const float *x_de
   check(cavs_event_record(ev_[0], stream_));
   fwd_out_ = graph_out ? graph_out : GO_.get();
   out_folded_ = false;
+  head_chunked_ = false;
   model_forward();
   pop_ret(fwd_out_);
   check(cavs_event_record(ev_[1], stream_));
@@ -825,6 +834,7 @@ void Engine::backward_only(const float *dgraph_out, bool settle_biases) {
   if (!dgraph_out || N_ == 0) fail(CAVS_EINVAL, "backward_only needs d graph_out of a forward pass");
   state_epoch_++;
   d_dgo_ = dgraph_out;
+  head_chunked_ = false;
   check(cavs_event_record(ev_[2], stream_));
   model_backward();
   if (settle_biases) settle_bias_jobs(0.f, nullptr);  // no update follows in here: the bias gradients are delivered now
@@ -838,6 +848,7 @@ void Engine::run_passes(bool backward) {
   if (!capturing_) check(cavs_event_record(ev_[0], stream_));
   fwd_out_ = GO_.get();
   out_folded_ = false;
+  head_chunked_ = backward && !head_chunks_.empty() && !profile_ && !capturing_ && cfg_.loss == CAVS_LOSS_SOFTMAX;
   model_forward();
   pop_ret(GO_.get());
   if (!capturing_) check(cavs_event_record(ev_[1], stream_));
@@ -1550,7 +1561,11 @@ void Engine::lstm_backward() {
     backward_prologue({}, true);
   }
   const bool folded = forest_;  // one launch per round, as in treelstm_backward
-  if (folded) {
+  // a wide head in chunks: d h comes in slab order, chunk by chunk, the last rounds' first
+  const float *dret = head_chunked_ ? dret_.get() : d_dgo_;
+  const int *dret_rows = head_chunked_ ? cell_iota_.get() : d_t2j_;
+  int chunk = head_chunked_ ? (int)head_chunks_.size() : 0;
+  if (folded && !head_chunked_) {
     CAVS_TIMED(K_GATES, cavs_lstm_bwd_gates_rows(d_orphans_, n_orphans_, d_dgo_, d_t2j_, gates_.get(), G_.get(), dxW_.get(), 4 * H,
                                                  dc_.get(), sched_->leaf_prefix, H, stream_));
     c_launches_ += 1;
@@ -1559,11 +1574,24 @@ void Engine::lstm_backward() {
     const Round &r = sched_->rounds[k];
     const size_t off = r.offset;
     float *da = dxW_.at(off * 4 * H);
+    while (head_chunked_ && chunk > 0 && (chunk == (int)head_chunks_.size() || k - 1 < head_chunks_[chunk].round0)) {
+      // a round's launch also runs the gate gradients of its rows' children, the rows of the round
+      // before: that round's chunk must have its d h.  Then the rows of the chunk nobody sends a
+      // gradient to.
+      chunk--;
+      const HeadChunk &h = head_chunks_[chunk];
+      check(cavs_stream_wait_event(stream_, chunk_done_ev_[chunk]));
+      if (h.orph1 > h.orph0) {
+        check(cavs_lstm_bwd_gates_rows(d_orphans_ + h.orph0, h.orph1 - h.orph0, dret, dret_rows, gates_.get(), G_.get(), dxW_.get(), 4 * H,
+                                       dc_.get(), sched_->leaf_prefix, H, stream_));
+        c_launches_ += 1;
+      }
+    }
     if (folded) {
       c_gather_rows_ += r.n;
       if (leaf_round(r)) continue;
       CAVS_TIMED(K_ROUND, (packed ? cavs_lstm_round_bwd_children_gates_packed : cavs_lstm_round_bwd_children_gates)(
-                              dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(), G_.get(), d_dgo_, d_t2j_, (int)off,
+                              dxW_.get(), 4 * H, dc_.get(), UT_.get(), d_kid_rows_ + off, gates_.get(), G_.get(), dret, dret_rows, (int)off,
                               r.n, sched_->leaf_prefix, H, stream_));
       c_round_flops_ += 2.0 * r.n * H * 4.0 * H;
       c_scatter_rows_ += r.n;
@@ -2000,6 +2028,10 @@ void Engine::embedding_backward_rows() {
 // ------------------------------------------------------------------ loss head
 void Engine::head_forward_backward(bool backward) {
   const int N = N_, H = cfg_.H, C = cfg_.C, B = sched_->B;
+  if (head_chunked_) {
+    head_in_chunks();
+    return;
+  }
   if (cfg_.loss == CAVS_LOSS_SOFTMAX) {
     // FullyConnected + SoftmaxEntropyLoss (cavs/backend/op_impl_fullyconnected_cublas.cc:71-79,
     // op_impl_softmax_entropy_logits_loss.cu:94-140) and their gradients (:150-163, :212-250)
@@ -2025,15 +2057,7 @@ void Engine::head_forward_backward(bool backward) {
     // The update writes the copy along with the weights (update_jobs); it is made here only
     // when somebody else has written them since.
     const bool wide = wide_head();
-    if (wide && !wfct_valid_) {
-      if (WfcT_.capacity() < (size_t)C * H) {
-        check(cavs_stream_sync(stream_));
-        WfcT_.reserve((size_t)C * H);
-      }
-      check(cavs_transpose(WfcT_.get(), Wfc.w, C, H, stream_));
-      c_launches_ += 1;
-      wfct_valid_ = Wfc.w == Wfc.own_w.get();
-    }
+    if (wide) ensure_wfct();
     {  // logits = GO * Wfc^T + bfc: the bias rides in the product's epilogue (row r adds D[r >> 30] = D[0])
       float *ws = workspace(cavs_sgemm_splitk_workspace(N, C, H));
       ProfScope ps(this, K_GEMM);
@@ -2055,16 +2079,8 @@ void Engine::head_forward_backward(bool backward) {
       if (wide && !profile_ && !cfg_.graph_replay) {
         // Only d GraphOutput is on the way of the backward rounds.  The weight and bias gradients are
         // wanted at the update: they run on the side stream, under the rounds.
-        if (!aux_stream_) {
-          check(cavs_stream_create(&aux_stream_));
-          check(cavs_event_create(&aux_fork_ev_));
-          check(cavs_event_create(&aux_join_ev_));
-        }
-        const size_t need = cavs_sgemm_group_workspace(1, &dWd);
-        if (ws_aux_.capacity() * 4 < need) {
-          check(cavs_stream_sync(aux_stream_));
-          ws_aux_.reserve(need / 4 + 1);
-        }
+        aux_open();
+        aux_workspace(cavs_sgemm_group_workspace(1, &dWd));
         // (forked behind the d GraphOutput product: side by side the two would only share the chip)
         gemm_group({dGd});
         check(cavs_event_record(aux_fork_ev_, stream_));
@@ -2109,6 +2125,117 @@ void Engine::head_forward_backward(bool backward) {
       c_launches_ += 1;
     }
   }
+}
+
+void Engine::ensure_wfct() {
+  if (wfct_valid_) return;
+  Param &Wfc = param("Wfc");
+  const size_t C = cfg_.C, H = cfg_.H;
+  if (WfcT_.capacity() < C * H) {
+    check(cavs_stream_sync(stream_));
+    WfcT_.reserve(C * H);
+  }
+  check(cavs_transpose(WfcT_.get(), Wfc.w, cfg_.C, cfg_.H, stream_));
+  c_launches_ += 1;
+  wfct_valid_ = Wfc.w == Wfc.own_w.get();
+}
+
+void Engine::aux_open() {
+  if (aux_stream_) return;
+  check(cavs_stream_create(&aux_stream_));
+  check(cavs_event_create(&aux_fork_ev_));
+  check(cavs_event_create(&aux_join_ev_));
+}
+
+float *Engine::aux_workspace(size_t bytes) {
+  if (ws_aux_.capacity() * 4 < bytes) {
+    check(cavs_stream_sync(aux_stream_));
+    ws_aux_.reserve(bytes / 4 + 1);
+  }
+  return ws_aux_.get();
+}
+
+// Which rounds go into which chunk of a wide head that runs beside the backward rounds: equal
+// shares of the rows, cut at round boundaries.  Two chunks by default -- measured on the 10 000-class
+// chain LSTM (7 000 rows, 99 rounds): 3.93 ms per step with two halves (3.99 / 4.03 with the cut at
+// 35 or 65 / 20 or 80 % of the rows), 4.04 with three chunks, 4.19 with four or with the head in
+// one piece between the passes: a chunk's products lose efficiency with their size, and the rounds
+// that run beside a product take two to three times as long.
+void Engine::plan_head_chunks(const int *orphans_host) {
+  head_chunks_.clear();
+  const Schedule &s = *sched_;
+  const int R = (int)s.rounds.size(), N = s.N;
+  if (cfg_.head_chunks < 0 || cfg_.model != CAVS_MODEL_LSTM || !wide_head() || !s.batching || !forest_ || cfg_.graph_replay || R < 8 ||
+      N < 256)
+    return;
+  const int K = cfg_.head_chunks > 0 ? std::min(cfg_.head_chunks, (int)kHeadChunks) : 2;
+  int k = 0;
+  for (int c = 0; c < K; c++) {
+    HeadChunk h;
+    h.round0 = k;
+    h.row0 = k < R ? s.rounds[k].offset : N;
+    const double upto = (double)(c + 1) / K;
+    while (k < R && (c == K - 1 || s.rounds[k].offset + s.rounds[k].n <= upto * N || k == h.round0)) k++;
+    h.round1 = k;
+    h.row1 = k < R ? s.rounds[k].offset : N;
+    if (h.round1 > h.round0) head_chunks_.push_back(h);
+  }
+  if (head_chunks_.size() < 2) {
+    head_chunks_.clear();
+    return;
+  }
+  for (HeadChunk &h : head_chunks_) {  // (the list is in ascending order of slab rows)
+    h.orph0 = (int)(std::lower_bound(orphans_host, orphans_host + n_orphans_, h.row0) - orphans_host);
+    h.orph1 = (int)(std::lower_bound(orphans_host, orphans_host + n_orphans_, h.row1) - orphans_host);
+  }
+}
+
+// Chunk k on the side stream: logits of its rows (h straight out of the message rows), loss and
+// d logits, d h.
+void Engine::head_chunk(int k) {
+  const HeadChunk &h = head_chunks_[k];
+  const int n = h.row1 - h.row0, H = cfg_.H, C = cfg_.C;
+  if (n > 0) {
+    const size_t r0 = h.row0;
+    float *ws = aux_workspace(cavs_sgemm_splitk_workspace(n, C, H));
+    check(cavs_sgemm_addrows(0, 0, n, C, H, msg_.at(r0 * mw_), (int)mw_, WfcT_.get(), C, param("bfc").w, C, 30, logits_.at(r0 * C), C, ws,
+                             ws_aux_.capacity() * 4, aux_stream_));
+    check(cavs_softmax_xent_part(loss_slab_.at(r0), dlogits_.at(r0 * C), logits_.at(r0 * C), labels_slab_.at(r0), n, C, N_, aux_stream_));
+    const cavs_gemm_desc dh{0, 1, n, H, C, 1.f, 0.f, dlogits_.at(r0 * C), C, WfcT_.get(), C, dret_.at(r0 * H), H};
+    ws = aux_workspace(cavs_sgemm_group_workspace(1, &dh));
+    check(cavs_sgemm_group_beside(1, &dh, ws, ws_aux_.capacity() * 4, aux_stream_));
+    c_gemm_flops_ += 4.0 * n * C * H;
+    c_launches_ += 3;
+  }
+  if (!chunk_done_ev_[k]) check(cavs_event_create(&chunk_done_ev_[k]));
+  check(cavs_event_record(chunk_done_ev_[k], aux_stream_));
+}
+
+// The whole head on the side stream, behind the forward rounds: the chunks last first (the backward
+// rounds start at the end), then what only the update and the caller wait for -- loss and d h by
+// vertex id, the head's weight and bias gradients.
+void Engine::head_in_chunks() {
+  const int N = N_, H = cfg_.H, C = cfg_.C;
+  ensure_wfct();
+  aux_open();
+  ensure_iota(cap_);
+  ensure(labels_slab_, grow((size_t)N, labels_slab_.capacity()));
+  ensure(loss_slab_, grow((size_t)N, loss_slab_.capacity()));
+  check(cavs_event_record(aux_fork_ev_, stream_));
+  check(cavs_stream_wait_event(aux_stream_, aux_fork_ev_));
+  check(cavs_gather_rows(labels_slab_.get(), 1, d_labels_, 1, d_t2j_, N, 1, aux_stream_));
+  for (int k = (int)head_chunks_.size() - 1; k >= 0; k--) head_chunk(k);
+  check(cavs_scatter_rows(loss_.get(), 1, d_t2j_, loss_slab_.get(), 1, N, 1, aux_stream_));
+  check(cavs_scatter_rows(dGO_.get(), H, d_t2j_, dret_.get(), H, N, H, aux_stream_));
+  Param &Wfc = param("Wfc");
+  const cavs_gemm_desc dWd{1, 0, C, H, N, 1.f, 0.f, dlogits_.get(), C, msg_.get(), (int)mw_, Wfc.g, H};
+  float *ws = aux_workspace(cavs_sgemm_group_workspace(1, &dWd));
+  check(cavs_sgemm_group_beside(1, &dWd, ws, ws_aux_.capacity() * 4, aux_stream_));
+  c_gemm_flops_ += 2.0 * dWd.M * dWd.N * dWd.K;
+  c_launches_ += 4;
+  bias_gradient("bfc", dlogits_.get(), N, C, head_bias_parts_, aux_stream_);
+  check(cavs_event_record(aux_join_ev_, aux_stream_));
+  aux_pending_ = true;
 }
 
 // The session's stream takes up what the side stream has been doing.
@@ -2187,6 +2314,7 @@ double Engine::counter(const std::string &key) const {
   if (key == "tail_lists_max") return (double)tail_.lists_max;
   if (key == "tail_tiles_max") return (double)tail_.tiles_max;
   if (key == "tail_vertices") return tail_.vertices;
+  if (key == "head_chunks") return head_chunked_ ? (double)head_chunks_.size() : 0.0;  // of the last step
   if (key == "graph_replays") return c_graph_replays_;
   if (key == "plan_hits") return c_plan_hits_;
   if (key == "plan_misses") return c_plan_misses_;

@@ -356,6 +356,33 @@ class Engine {
   bool aux_pending_ = false;   // work on the side stream that the session's stream has not waited for yet
   DeviceArray<float> ws_aux_;  // its products' split-K workspace
   void aux_join();
+  void aux_open();  // creates the side stream and its events
+  void ensure_wfct();  // the transposed copy of a wide head's weights, if somebody else wrote them since
+
+  // ---- a wide loss head in chunks (chain LSTM), beside the rounds
+  // The head of a wide classifier is three large products per vertex row, the rounds of a chain LSTM
+  // two hundred short dependent launches that leave most of the chip idle.  The head reads a vertex's
+  // h and hands back d h: nothing in it couples rows, so it runs on the side stream over chunks of
+  // slab rows (= ranges of rounds), last chunk first, so that the backward rounds, which start at
+  // the last round, can begin when the last chunk's d h is there and go on while the earlier chunks'
+  // is computed.  (Not under the forward rounds: their 512-thread workgroups find no room beside a
+  // large product's and a round then takes as long as the product.)  Rows are taken in slab order
+  // (h straight out of the message rows, labels gathered once, d h where the backward launches
+  // read it with the identity list).
+  struct HeadChunk {
+    int row0 = 0, row1 = 0;      // slab rows
+    int round0 = 0, round1 = 0;  // rounds [round0, round1)
+    int orph0 = 0, orph1 = 0;    // positions in the list of vertices nobody sends a gradient to
+  };
+  static constexpr int kHeadChunks = 4;
+  std::vector<HeadChunk> head_chunks_;  // of this step's schedule; empty: the head runs in one piece
+  bool head_chunked_ = false;           // this pass runs it in chunks
+  void *chunk_done_ev_[kHeadChunks] = {};
+  DeviceArray<float> labels_slab_, loss_slab_;
+  void plan_head_chunks(const int *orphans_host);
+  void head_chunk(int k);   // enqueues chunk k's logits, loss and d h on the side stream
+  void head_in_chunks();    // after the forward rounds: all chunks, then what only the update waits for
+  float *aux_workspace(size_t bytes);
 
   // ---- a vertex function on generated kernels (CAVS_MODEL_CELL)
   // A function of several stages is a chain of cells (CellSpec::next); every cell has its module
@@ -368,8 +395,9 @@ class Engine {
   };
   std::shared_ptr<const CellSpec> cell_;  // the head of the chain
   std::deque<CellStage> cells_;  // (the arrays do not move)
-  DeviceArray<int> cell_iota_;  // 0, 1, 2, ...: "the child of slab row v is slab row v"
+  DeviceArray<int> cell_iota_;  // 0, 1, 2, ...: "the child of slab row v is slab row v" (also: "d h of slab row v is row v")
   size_t cell_iota_n_ = 0;
+  void ensure_iota(size_t n);
   // one launch of kernel `k` of cell `ci`'s module
   void cell_launch(int ci, int k, unsigned gx, unsigned gy, unsigned gz, unsigned block, long off, long n, const int *rows, const float *go);
   void embedding_backward_rows();

@@ -23,7 +23,7 @@ PAIR = {"reference": 0, "rowid": 1}
 class _Config(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("model", "loss", "pairing", "opt", "V", "E", "H", "C", "act",
                                       "use_bias", "use_x", "device", "fused_round_rows", "split_backward_rounds",
-                                      "schedule_mode", "plan_cache", "tail_rows", "graph_replay")]
+                                      "schedule_mode", "plan_cache", "tail_rows", "graph_replay", "head_chunks")]
 
 
 _lib = None
@@ -175,12 +175,12 @@ class Session:
 
     def __init__(self, model, *, H, E=0, V=0, C_=0, loss="softmax", pairing="reference",
                  opt=OPT_BATCHING, act=0, use_bias=False, use_x=False, device=0, fused_round_rows=0,
-                 split_backward_rounds=False, schedule="host", plan_cache=0, tail_rows=0, graph_replay=False):
+                 split_backward_rounds=False, schedule="host", plan_cache=0, tail_rows=0, graph_replay=False, head_chunks=0):
         self.model, self.H, self.E, self.V, self.C, self.loss = model, H, (H if model == "lstm" else E), V, C_, loss
         self.mw = H if model == "treefc" else 2 * H
         cfg = _Config(MODEL[model], LOSS[loss], PAIR[pairing], opt, V, E, H, C_, int(act), int(use_bias),
                       int(use_x), device, int(fused_round_rows), int(split_backward_rounds),
-                      {"host": 0, "device": 1}[schedule], int(plan_cache), int(tail_rows), int(graph_replay))
+                      {"host": 0, "device": 1}[schedule], int(plan_cache), int(tail_rows), int(graph_replay), int(head_chunks))
         self._h = C.c_void_p()
         _check(lib().cavs_session_create(C.byref(cfg), C.byref(self._h)), "cavs_session_create")
         self._keep = None

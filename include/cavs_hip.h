@@ -244,6 +244,11 @@ int cavs_bias_add_rows(float *out, const float *inp, const float *bias, int n, i
  * Either output may be NULL. */
 int cavs_softmax_xent(float *loss, float *dlogits, const float *logits, const float *labels,
                       int n, int C, void *stream);
+/* The same for n rows out of a batch of n_total (dlogits = (softmax - onehot)/n_total): a loss head
+ * that runs chunk by chunk, under the rounds that produce the next chunk's rows.  Row for row the
+ * values of the call over the whole batch. */
+int cavs_softmax_xent_part(float *loss, float *dlogits, const float *logits, const float *labels,
+                           int n, int C, int n_total, void *stream);
 /* SGD (cavs/backend/op_impl_sgd.cu): w -= lr * g */
 int cavs_sgd(float *w, const float *g, float lr, size_t n, void *stream);
 

@@ -85,6 +85,14 @@ typedef struct {
    * the next step an ordinary one.  Replayed steps have no "RNNForward" / "RNNBackward" timings.
    * The counter "graph_replays" counts them.  0 = off. */
   int graph_replay;
+  /* Chain LSTM with a wide classifier head (head weights of at least 2^18 elements), host
+   * scheduler, message flow a forest: the head runs over chunks of the rounds on a second stream
+   * beside the backward rounds (cavs/midend/statement.cc:69-76,106-111 run them one
+   * after the other): the chunks last first, each one's d h releasing the backward rounds of its
+   * rows while the next chunk's is computed.  0 = default (two chunks), 2..4 = that many, negative =
+   * off: the head in one piece between the two passes.  The counter "head_chunks" says in how many
+   * chunks the last step's head ran (0: in one piece). */
+  int head_chunks;
 } cavs_session_config;
 
 const char *cavs_session_error(void);

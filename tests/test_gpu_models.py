@@ -547,6 +547,45 @@ def test_the_transposed_copy_of_a_wide_heads_weights_follows_every_writer(oracle
     s.close()
 
 
+@pytest.mark.parametrize("pairing", ["reference", "rowid"])
+def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
+    """Chain LSTM with a wide classifier: the head runs on a second stream over chunks of the rounds,
+    last chunk first, while the backward rounds of the chunks already done run.  Sequences of 4..30
+    steps end in every chunk (the vertices nobody sends a gradient to are handled chunk by chunk).
+    Three training steps on changing batches against the oracle: two chunks (the default), four,
+    and the head in one piece."""
+    model, H, V, C_ = "lstm", 64, 41, 4096
+    rng = synth.SplitMix64(91)
+    p = dict(Emb=rng.bulk_normal(V * H, 0, 0.5).reshape(V, H), W=rng.bulk_uniform(8 * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(4 * H, -0.3, 0.3),
+             Wfc=rng.bulk_uniform(C_ * H, -0.3, 0.3).reshape(C_, H), bfc=rng.bulk_uniform(C_, -0.2, 0.2))
+    p = {k: np.asarray(v, np.float32) for k, v in p.items()}
+    lr = 0.2
+    sessions = {hc: session.Session(model, H=H, E=H, V=V, C_=C_, pairing=pairing, head_chunks=hc) for hc in (0, 4, -1)}
+    for s in sessions.values():
+        s.set_params(p)
+    for step in range(3):
+        graph, lens, _ = synth.chain_batch(500 + step, 40, 4, 30, 30)
+        N = sum(lens)
+        x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
+        labels = np.floor(rng.bulk_uniform(N) * C_).astype(np.float32)
+        want = oracle.model_step(model, graph, x, labels, p, H=H, E=H, V=V, Cc=C_, pairing=pairing, precise=True, threads=16)
+        for hc, s in sessions.items():
+            print(f"[case] wide head, head_chunks={hc}, step {step}, N={N}, pairing={pairing}", flush=True)
+            s.step(graph, x, labels, backward=True, lr=lr)
+            assert s.counter("head_chunks") == {0: 2, 4: 4, -1: 0}[hc]
+            for k in ("loss", "graph_out", "dgraph_out"):
+                close(s.fetch(k), want[k], f"{k} at step {step}", scaled=False)
+            got = s.grads()
+            for k in p:
+                close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", scaled=False)
+        for k in p:
+            p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    for s in sessions.values():
+        close(s.param("Wfc", p["Wfc"].shape), p["Wfc"], "Wfc after the steps")
+        close(s.param("W", p["W"].shape), p["W"], "W after the steps")
+        s.close()
+
+
 @pytest.mark.parametrize("kind", ["trees", "tokens"])
 def test_training_step_on_reader_batches(oracle, kind):
     """The text readers (cavs_amd/data.py) feed the session directly: the fixture corpora

@@ -673,6 +673,24 @@ def test_softmax_xent_bias_sgd(g, oracle, n, C_):
     np.testing.assert_array_equal(g.host(w), logits - np.float32(0.5) * grad)
 
 
+@pytest.mark.parametrize("n,C_", [(40, 10000), (23, 600), (9, 7)])
+def test_softmax_xent_of_a_batch_in_parts_is_the_whole_row_for_row(g, n, C_):
+    """The loss head of a wide classifier runs chunk by chunk: a part's rows come out bit for bit as
+    in the call over the whole batch (the gradient's 1/n is the batch's)."""
+    r = rng(n * 3 + C_)
+    logits = g.devf(3 * r.bulk_normal(n * C_).reshape(n, C_))
+    labels = g.devf(np.floor(r.bulk_uniform(n) * C_).astype(np.float32))
+    loss, d = g.zeros(n), g.zeros(n, C_)
+    g.call("cavs_softmax_xent", g.P(loss), g.P(d), g.P(logits), g.P(labels), n, C_, g.stream())
+    loss2, d2 = g.zeros(n), g.zeros(n, C_)
+    cut = [0, n // 3, n // 3, n - 2, n]  # (one part is empty)
+    for a, b in zip(cut[:-1], cut[1:]):
+        g.call("cavs_softmax_xent_part", g.P(loss2) + 4 * a, g.P(d2) + 4 * a * C_, g.P(logits) + 4 * a * C_, g.P(labels) + 4 * a, b - a, C_, n,
+               g.stream())
+    np.testing.assert_array_equal(g.host(loss2), g.host(loss))
+    np.testing.assert_array_equal(g.host(d2), g.host(d))
+
+
 def test_elementwise_family(g):
     r = rng(3)
     n, w = 37, 20
