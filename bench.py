@@ -28,9 +28,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 FP32_MFMA_PEAK_TF = 157.3  # MI355X dense FP32 matrix
 # (workload, kernel class) -> HBM bytes per dispatch, from profiles/bench_<workload>_hbm_traffic_pmc.txt
-PMC_TRAFFIC_BYTES = {("C3", "gemm"): 82.06e6, ("C3", "round"): 98.58e6, ("C1", "gemm"): 3.35e6, ("C1", "round"): 0.96e6,
-                     ("C2", "gemm"): 17.11e6, ("C2", "round"): 4.05e6, ("C4", "gemm"): 328.8e6, ("C4", "round"): 10.55e6,
-                     ("C5", "gemm"): 921.3e6, ("C5", "round"): 125.4e6}
+PMC_TRAFFIC_BYTES = {("C3", "gemm"): 82.05e6, ("C3", "round"): 98.59e6, ("C1", "gemm"): 3.35e6, ("C1", "round"): 0.96e6,
+                     ("C2", "gemm"): 17.11e6, ("C2", "round"): 4.05e6, ("C4", "gemm"): 299.6e6, ("C4", "round"): 10.55e6,
+                     ("C5", "gemm"): 918.6e6, ("C5", "round"): 125.4e6}
 # a constant taken from the profile named, not a counter read during this run
 PMC_TRAFFIC_SOURCE = {k: f"profiles/bench_{k[0]}_hbm_traffic_pmc.txt (two rocprofv3 --pmc runs of this command, FETCH_SIZE and "
                          "WRITE_SIZE per dispatch of the class; a constant copied from there, not read in this run)"
