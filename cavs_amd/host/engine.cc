@@ -582,6 +582,7 @@ void Engine::remember_plan(const int *graph, int B, int maxlen, uint64_t hash) {
   p->forest = forest_;
   p->last_used = ++plan_clock_;
   p->tail = tail_;
+  p->head_chunks = head_chunks_;
   p->lists.reserve(2 * N + 2 * nk + B + N + N);
   int *base = p->lists.get();
   const bool kids = d_kid_rows_ != nullptr;
@@ -789,6 +790,7 @@ void Engine::begin_step(const int *graph, int B, int maxlen) {
     d_orphans_ = base + 2 * N + 2 * nk + B;
     d_tail_rows_ = base + 3 * N + 2 * nk + B;
     tail_ = (forest_ && tail_limit() > 0) ? hit->tail : TailPlan();
+    if (forest_ && !cfg_.graph_replay) head_chunks_ = hit->head_chunks;
     sched_ms_ = 0.f;
   } else {
     tail_ = TailPlan();  // (the host-built lists bring a new one)

@@ -249,6 +249,12 @@ class Engine {
   uint64_t state_epoch_ = 0;  // bumped by every call other than step() that changes what a step enqueues
   double c_graph_replays_ = 0;
 
+  // a chunk of the loss head of a wide classifier that runs beside the backward rounds (below)
+  struct HeadChunk {
+    int row0 = 0, row1 = 0;      // slab rows
+    int round0 = 0, round1 = 0;  // rounds [round0, round1)
+    int orph0 = 0, orph1 = 0;    // positions in the list of vertices nobody sends a gradient to
+  };
   struct Plan {
     ~Plan() { drop_graphs(); }
     void drop_graphs() {
@@ -269,6 +275,7 @@ class Engine {
     int n_orphans = 0;
     bool forest = false;
     TailPlan tail;
+    std::vector<HeadChunk> head_chunks;
     uint64_t last_used = 0;
   };
   std::vector<std::unique_ptr<Plan>> plans_;
@@ -369,11 +376,6 @@ class Engine {
   // large product's and a round then takes as long as the product.)  Rows are taken in slab order
   // (h straight out of the message rows, labels gathered once, d h where the backward launches
   // read it with the identity list).
-  struct HeadChunk {
-    int row0 = 0, row1 = 0;      // slab rows
-    int round0 = 0, round1 = 0;  // rounds [round0, round1)
-    int orph0 = 0, orph1 = 0;    // positions in the list of vertices nobody sends a gradient to
-  };
   static constexpr int kHeadChunks = 4;
   std::vector<HeadChunk> head_chunks_;  // of this step's schedule; empty: the head runs in one piece
   bool head_chunked_ = false;           // this pass runs it in chunks

@@ -552,8 +552,9 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
     """Chain LSTM with a wide classifier: the head runs on a second stream over chunks of the rounds,
     last chunk first, while the backward rounds of the chunks already done run.  Sequences of 4..30
     steps end in every chunk (the vertices nobody sends a gradient to are handled chunk by chunk).
-    Three training steps on changing batches against the oracle: two chunks (the default), four,
-    and the head in one piece."""
+    Five training steps on changing batches (two of them met before) against the oracle: two chunks
+    (the default), four, two with a plan cache (the chunks of a structure met again come out of the
+    cache), and the head in one piece."""
     model, H, V, C_ = "lstm", 64, 41, 4096
     rng = synth.SplitMix64(91)
     p = dict(Emb=rng.bulk_normal(V * H, 0, 0.5).reshape(V, H), W=rng.bulk_uniform(8 * H * H, -0.3, 0.3), Bv=rng.bulk_uniform(4 * H, -0.3, 0.3),
@@ -561,10 +562,11 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
     p = {k: np.asarray(v, np.float32) for k, v in p.items()}
     lr = 0.2
     sessions = {hc: session.Session(model, H=H, E=H, V=V, C_=C_, pairing=pairing, head_chunks=hc) for hc in (0, 4, -1)}
+    sessions["cache"] = session.Session(model, H=H, E=H, V=V, C_=C_, pairing=pairing, plan_cache=4)
     for s in sessions.values():
         s.set_params(p)
-    for step in range(3):
-        graph, lens, _ = synth.chain_batch(500 + step, 40, 4, 30, 30)
+    for step, seed in enumerate([500, 501, 500, 502, 501]):
+        graph, lens, _ = synth.chain_batch(seed, 40, 4, 30, 30)
         N = sum(lens)
         x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
         labels = np.floor(rng.bulk_uniform(N) * C_).astype(np.float32)
@@ -572,7 +574,7 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
         for hc, s in sessions.items():
             print(f"[case] wide head, head_chunks={hc}, step {step}, N={N}, pairing={pairing}", flush=True)
             s.step(graph, x, labels, backward=True, lr=lr)
-            assert s.counter("head_chunks") == {0: 2, 4: 4, -1: 0}[hc]
+            assert s.counter("head_chunks") == {0: 2, 4: 4, -1: 0, "cache": 2}[hc]
             for k in ("loss", "graph_out", "dgraph_out"):
                 close(s.fetch(k), want[k], f"{k} at step {step}", scaled=False)
             got = s.grads()
@@ -580,6 +582,7 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
                 close(got["d" + k], want["grads"]["d" + k], f"d{k} at step {step}", scaled=False)
         for k in p:
             p[k] = (p[k] - np.float32(lr) * want["grads"]["d" + k].reshape(p[k].shape)).astype(np.float32)
+    assert sessions["cache"].counter("plan_hits") == 2
     for s in sessions.values():
         close(s.param("Wfc", p["Wfc"].shape), p["Wfc"], "Wfc after the steps")
         close(s.param("W", p["W"].shape), p["W"], "W after the steps")
