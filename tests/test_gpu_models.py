@@ -552,7 +552,8 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
     """Chain LSTM with a wide classifier: the head runs on a second stream over chunks of the rounds,
     last chunk first, while the backward rounds of the chunks already done run.  Sequences of 4..30
     steps end in every chunk (the vertices nobody sends a gradient to are handled chunk by chunk).
-    Five training steps on changing batches (two of them met before) against the oracle: two chunks
+    Six training steps on changing batches (two of them met before, the last one larger than the
+    buffers) against the oracle: two chunks
     (the default), four, two with a plan cache (the chunks of a structure met again come out of the
     cache), and the head in one piece."""
     model, H, V, C_ = "lstm", 64, 41, 4096
@@ -565,8 +566,9 @@ def test_a_wide_head_in_chunks_beside_the_rounds(oracle, pairing):
     sessions["cache"] = session.Session(model, H=H, E=H, V=V, C_=C_, pairing=pairing, plan_cache=4)
     for s in sessions.values():
         s.set_params(p)
-    for step, seed in enumerate([500, 501, 500, 502, 501]):
-        graph, lens, _ = synth.chain_batch(seed, 40, 4, 30, 30)
+    for step, seed in enumerate([500, 501, 500, 502, 501, 503]):
+        # (the last batch is half as large again: every per-vertex buffer is reallocated)
+        graph, lens, _ = synth.chain_batch(seed, 40, 22 if seed == 503 else 4, 30, 30)
         N = sum(lens)
         x = np.floor(rng.bulk_uniform(N) * V).astype(np.float32)
         labels = np.floor(rng.bulk_uniform(N) * C_).astype(np.float32)
