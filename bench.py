@@ -271,6 +271,7 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
         torch.cuda.empty_cache()
         return out, w0
 
+    head_chunks = s.counter("head_chunks")  # (of the last timed step; the pass below runs the head in one piece)
     # Roofline of the dominant kernel: the same steps again with the kernels of every entry point
     # stamping a start and a stop event themselves (the interval a kernel trace reports) on the
     # session's own stream; kept out of the throughput figure above.
@@ -324,7 +325,7 @@ def measure(a, workload, steps, warmup, n_pool, schedule="host", plan_cache=0, p
                                f"N~{w0['N']} vertices/batch, {len(pool)} seeded batches cycled",
                    "step": "schedule+fwd+loss+bwd+sgd", "pairing": a.pairing,
                    "feeds": "pageable host memory, copied every step" if a.host_feeds else "resident in HBM",
-                   "rounds_last_batch": rounds, "launches_last_batch": launches,
+                   "rounds_last_batch": rounds, "launches_last_batch": launches, "loss_head_chunks": head_chunks,
                    "untimed_settle_steps": settle},
         "roofline": {"bound": "mfma", "achieved": round(dom["tf"], 3), "peak": FP32_MFMA_PEAK_TF,
                      "unit": "TFLOP/s", "frac": round(dom["tf"] / FP32_MFMA_PEAK_TF, 5), "traffic": traffic,
